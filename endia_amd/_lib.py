@@ -1,0 +1,127 @@
+"""ctypes binding of libendia_hip.so (the C ABI declared in include/endia_hip.h).
+
+There is no CPU fallback: if the library is missing, or no gfx950 device can be initialised, every
+entry point raises. `lib()` loads the shared object (possible without a GPU, e.g. to check the
+exported symbols); `ensure_init()` additionally creates the device context.
+"""
+import ctypes
+import os
+from ctypes import POINTER, c_char_p, c_float, c_int32, c_int64, c_uint32, c_void_p
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "libendia_hip.so")
+
+# enums of include/endia_hip.h
+OP_RELU, OP_TANH, OP_SIN, OP_COS, OP_NEG, OP_SQUARE, OP_SQRT, OP_ABS, OP_IDENTITY, OP_GREATER0 = range(10)
+BIN_ADD, BIN_SUB, BIN_MUL, BIN_DIV, BIN_GREATER = range(5)
+EPI_NONE, EPI_BIAS, EPI_BIAS_ACT, EPI_ACT_GRAD = range(4)
+ACT_FROM_OUTPUT = 0x100
+GEMM_ACCUMULATE = 0x200
+CGEMM_4M, CGEMM_3M = 0, 1
+
+ERR_INVALID, ERR_NOT_INIT, ERR_RUNTIME, ERR_NOMEM, ERR_UNSUPPORTED = -1, -2, -3, -4, -5
+
+
+class EndiaHipError(RuntimeError):
+    def __init__(self, code, message):
+        super().__init__("libendia_hip: error %d: %s" % (code, message))
+        self.code = code
+
+
+class Conv2dDesc(ctypes.Structure):
+    _fields_ = [(n, c_int64) for n in (
+        "N", "C", "H", "W", "K", "R", "S",
+        "stride_h", "stride_w", "pad_h", "pad_w", "dil_h", "dil_w", "groups")]
+
+
+_fp = c_void_p  # device pointers travel as plain addresses
+_i64p = POINTER(c_int64)
+
+SIGNATURES = {
+    "endia_hip_init": [c_int32],
+    "endia_hip_shutdown": [],
+    "endia_hip_sync": [],
+    "endia_hip_device_info": [c_char_p, c_int64, POINTER(c_int32), POINTER(c_int32)],
+    "endia_hip_malloc": [c_int64, POINTER(c_void_p)],
+    "endia_hip_free": [c_void_p],
+    "endia_hip_memcpy_h2d": [c_void_p, c_void_p, c_int64],
+    "endia_hip_memcpy_d2h": [c_void_p, c_void_p, c_int64],
+    "endia_hip_memcpy_d2d": [c_void_p, c_void_p, c_int64],
+    "endia_hip_memset0": [c_void_p, c_int64],
+    "endia_hip_fill": [_fp, c_int64, c_float],
+    "endia_hip_pool_stats": [_i64p, _i64p, _i64p],
+    "endia_hip_pool_trim": [],
+    "endia_hip_timer_start": [c_int32],
+    "endia_hip_timer_stop": [c_int32],
+    "endia_hip_timer_elapsed_ms": [c_int32, POINTER(c_float)],
+    "endia_hip_strided_copy": [c_int32, _i64p, _i64p, c_int64, _fp, _fp, c_int32],
+    "endia_hip_sgemm": [c_int32, c_int32, c_int64, c_int64, c_int64, _fp, c_int64, _fp, c_int64, _fp, c_int64,
+                        c_int64, c_int64, c_int64, c_int64, c_int32, c_int32, _fp, _fp, _fp],
+    "endia_hip_cgemm": [c_int32, c_int32, c_int32, c_int32, c_int64, c_int64, c_int64, _fp, c_int64, _fp, c_int64,
+                        _fp, c_int64, c_int64, c_int64, c_int64, c_int64, c_int32, c_int32],
+    "endia_hip_unary_fwd": [c_int32, c_int64, _fp, _fp, c_int32],
+    "endia_hip_unary_vjp": [c_int32, c_int64, _fp, _fp, _fp, c_int32],
+    "endia_hip_binary": [c_int32, c_int32, _i64p, _i64p, _i64p, _fp, _fp, _fp, c_int32],
+    "endia_hip_axpby": [c_int64, c_float, _fp, c_float, _fp, _fp],
+    "endia_hip_reduce_add": [c_int32, _i64p, c_uint32, _fp, _fp, c_float, c_int32],
+    "endia_hip_mse_fwd_bwd": [c_int64, _fp, _fp, _fp, _fp],
+    "endia_hip_conv2d_out_shape": [POINTER(Conv2dDesc), _i64p, _i64p],
+    "endia_hip_conv2d_fwd": [POINTER(Conv2dDesc), _fp, _fp, _fp, _fp, c_int32],
+    "endia_hip_conv2d_bwd_data": [POINTER(Conv2dDesc), _fp, _fp, _fp],
+    "endia_hip_conv2d_bwd_weight": [POINTER(Conv2dDesc), _fp, _fp, _fp],
+    "endia_hip_conv2d_bwd_bias": [POINTER(Conv2dDesc), _fp, _fp],
+    "endia_hip_sgd_step": [c_int64, _fp, _fp, c_float],
+    "endia_hip_adam_step": [c_int64, _fp, _fp, _fp, _fp, c_float, c_float, c_float, c_float, c_float],
+}
+
+_lib = None
+_ready = False
+
+
+def lib():
+    """Load libendia_hip.so and attach argument types. Raises if the library has not been built."""
+    global _lib
+    if _lib is None:
+        if not os.path.exists(LIB_PATH):
+            raise ImportError(
+                "%s is missing: build it with `python -m endia_amd.build` (there is no CPU fallback)" % LIB_PATH)
+        handle = ctypes.CDLL(LIB_PATH)
+        for name, argtypes in SIGNATURES.items():
+            fn = getattr(handle, name)
+            fn.argtypes = argtypes
+            fn.restype = c_int32
+        handle.endia_hip_last_error.argtypes = []
+        handle.endia_hip_last_error.restype = c_char_p
+        _lib = handle
+    return _lib
+
+
+def check(code):
+    if code != 0:
+        raise EndiaHipError(code, lib().endia_hip_last_error().decode("utf-8", "replace"))
+
+
+def ensure_init(device=0):
+    """Create the device context once. Raises EndiaHipError when no gfx950 device is usable."""
+    global _ready
+    if not _ready:
+        check(lib().endia_hip_init(device))
+        _ready = True
+    return lib()
+
+
+def call(name, *args):
+    """Call an entry point on the initialised library and raise on a non-zero status."""
+    check(getattr(ensure_init(), name)(*args))
+
+
+def i64_array(values):
+    values = list(values)
+    return (c_int64 * max(len(values), 1))(*values)
+
+
+def device_info():
+    buf = ctypes.create_string_buffer(256)
+    cu, mhz = c_int32(), c_int32()
+    call("endia_hip_device_info", buf, 256, ctypes.byref(cu), ctypes.byref(mhz))
+    return buf.value.decode(), cu.value, mhz.value

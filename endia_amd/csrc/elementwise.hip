@@ -1,0 +1,539 @@
+// Streaming (HBM-bound) kernels: fills, unary forward / VJP, broadcasting binary ops, axpby and the
+// strided gather copy. Each replaces a run of full-tensor passes in the reference
+// (execute_unary_op, endia/functional/unary_ops/_utils.mojo:77-134; execute_binary_op,
+// endia/functional/binary_ops/_utils.mojo:93-177; execute_copy_raw, endia/functional/_utils.mojo:79-163)
+// with ONE coalesced pass: every lane moves 16 bytes per access, a wave covers 1 KiB of
+// consecutive addresses, and the grid is a few work-groups per CU walking the tensor with a
+// grid stride.
+#include "common.h"
+
+namespace {
+
+constexpr int TPB = 256;
+
+inline int stream_grid(int64_t nvec) {
+  int64_t blocks = ceil_div64(nvec, TPB);
+  int64_t cap = (int64_t)endia::ctx().cu_count * 8;
+  if (cap < 256) cap = 2048;
+  if (blocks > cap) blocks = cap;
+  if (blocks < 1) blocks = 1;
+  return (int)blocks;
+}
+
+inline bool al16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; }
+
+// ---- fill -----------------------------------------------------------------------------------
+__global__ __launch_bounds__(TPB) void fill_kernel(float* __restrict__ p, int64_t n, float v) {
+  int64_t i = (int64_t)blockIdx.x * TPB + threadIdx.x;
+  int64_t stride = (int64_t)gridDim.x * TPB;
+  int64_t n4 = n >> 2;
+  float4 v4 = make_float4(v, v, v, v);
+  float4* p4 = reinterpret_cast<float4*>(p);
+  for (int64_t j = i; j < n4; j += stride) p4[j] = v4;
+  for (int64_t j = (n4 << 2) + i; j < n; j += stride) p[j] = v;
+}
+
+__global__ __launch_bounds__(TPB) void fill_scalar_kernel(float* __restrict__ p, int64_t n, float v) {
+  int64_t i = (int64_t)blockIdx.x * TPB + threadIdx.x;
+  int64_t stride = (int64_t)gridDim.x * TPB;
+  for (int64_t j = i; j < n; j += stride) p[j] = v;
+}
+
+// ---- unary ----------------------------------------------------------------------------------
+template <int OP>
+__device__ __forceinline__ float unary_real(float x) {
+  switch (OP) {
+    case ENDIA_OP_RELU: return x > 0.f ? x : 0.f;
+    case ENDIA_OP_TANH: return tanhf(x);
+    case ENDIA_OP_SIN: return sinf(x);
+    case ENDIA_OP_COS: return cosf(x);
+    case ENDIA_OP_NEG: return -x;
+    case ENDIA_OP_SQUARE: return x * x;
+    case ENDIA_OP_SQRT: return sqrtf((fabsf(x) + x) * 0.5f);  // 0 for negative x, as the reference
+    case ENDIA_OP_ABS: return fabsf(x);
+    case ENDIA_OP_GREATER0: return x > 0.f ? 1.f : 0.f;
+    default: return x;
+  }
+}
+
+// g * d(op)/dx at x
+template <int OP>
+__device__ __forceinline__ float unary_vjp_real(float x, float g) {
+  switch (OP) {
+    case ENDIA_OP_RELU: return x > 0.f ? g : 0.f;
+    case ENDIA_OP_TANH: { float t = tanhf(x); return (1.f - t * t) * g; }
+    case ENDIA_OP_SIN: return cosf(x) * g;
+    case ENDIA_OP_COS: return -sinf(x) * g;
+    case ENDIA_OP_NEG: return -g;
+    case ENDIA_OP_SQUARE: return 2.f * x * g;
+    case ENDIA_OP_SQRT: return g / (2.f * sqrtf((fabsf(x) + x) * 0.5f));
+    case ENDIA_OP_ABS: return (x > 0.f ? 1.f : (x < 0.f ? -1.f : 0.f)) * g;
+    case ENDIA_OP_GREATER0: return 0.f;
+    default: return g;
+  }
+}
+
+template <int OP, bool VEC>
+__global__ __launch_bounds__(TPB) void unary_fwd_kernel(const float* __restrict__ x, float* __restrict__ y, int64_t n) {
+  int64_t i = (int64_t)blockIdx.x * TPB + threadIdx.x;
+  int64_t stride = (int64_t)gridDim.x * TPB;
+  if (VEC) {
+    int64_t n4 = n >> 2;
+    const float4* x4 = reinterpret_cast<const float4*>(x);
+    float4* y4 = reinterpret_cast<float4*>(y);
+    for (int64_t j = i; j < n4; j += stride) {
+      float4 a = x4[j];
+      y4[j] = make_float4(unary_real<OP>(a.x), unary_real<OP>(a.y), unary_real<OP>(a.z), unary_real<OP>(a.w));
+    }
+    for (int64_t j = (n4 << 2) + i; j < n; j += stride) y[j] = unary_real<OP>(x[j]);
+  } else {
+    for (int64_t j = i; j < n; j += stride) y[j] = unary_real<OP>(x[j]);
+  }
+}
+
+template <int OP, bool VEC>
+__global__ __launch_bounds__(TPB) void unary_vjp_kernel(const float* __restrict__ x, const float* __restrict__ g,
+                                                        float* __restrict__ dx, int64_t n) {
+  int64_t i = (int64_t)blockIdx.x * TPB + threadIdx.x;
+  int64_t stride = (int64_t)gridDim.x * TPB;
+  if (VEC) {
+    int64_t n4 = n >> 2;
+    const float4* x4 = reinterpret_cast<const float4*>(x);
+    const float4* g4 = reinterpret_cast<const float4*>(g);
+    float4* d4 = reinterpret_cast<float4*>(dx);
+    for (int64_t j = i; j < n4; j += stride) {
+      float4 a = x4[j], b = g4[j];
+      d4[j] = make_float4(unary_vjp_real<OP>(a.x, b.x), unary_vjp_real<OP>(a.y, b.y),
+                          unary_vjp_real<OP>(a.z, b.z), unary_vjp_real<OP>(a.w, b.w));
+    }
+    for (int64_t j = (n4 << 2) + i; j < n; j += stride) dx[j] = unary_vjp_real<OP>(x[j], g[j]);
+  } else {
+    for (int64_t j = i; j < n; j += stride) dx[j] = unary_vjp_real<OP>(x[j], g[j]);
+  }
+}
+
+// complex forward: one complex element (8 bytes) per lane access
+__global__ __launch_bounds__(TPB) void unary_fwd_complex_kernel(int op, const float2* __restrict__ x,
+                                                                float* __restrict__ y, int64_t n) {
+  int64_t i = (int64_t)blockIdx.x * TPB + threadIdx.x;
+  int64_t stride = (int64_t)gridDim.x * TPB;
+  float2* y2 = reinterpret_cast<float2*>(y);
+  for (int64_t j = i; j < n; j += stride) {
+    float2 z = x[j];
+    switch (op) {
+      case ENDIA_OP_NEG: y2[j] = make_float2(-z.x, -z.y); break;
+      case ENDIA_OP_SQUARE: y2[j] = make_float2(z.x * z.x - z.y * z.y, 2.f * z.x * z.y); break;
+      case ENDIA_OP_ABS: y[j] = sqrtf(z.x * z.x + z.y * z.y); break;
+      default: y2[j] = z; break;
+    }
+  }
+}
+
+// complex VJPs under the reference's rules (no conjugation: mul_op.mojo:125-128)
+__global__ __launch_bounds__(TPB) void unary_vjp_complex_kernel(int op, const float2* __restrict__ x,
+                                                                const float* __restrict__ g,
+                                                                float2* __restrict__ dx, int64_t n) {
+  int64_t i = (int64_t)blockIdx.x * TPB + threadIdx.x;
+  int64_t stride = (int64_t)gridDim.x * TPB;
+  const float2* g2 = reinterpret_cast<const float2*>(g);
+  for (int64_t j = i; j < n; j += stride) {
+    float2 z = x[j];
+    switch (op) {
+      case ENDIA_OP_NEG: { float2 c = g2[j]; dx[j] = make_float2(-c.x, -c.y); break; }
+      case ENDIA_OP_SQUARE: {  // 2 * z * g, square_op.mojo:96
+        float2 c = g2[j];
+        dx[j] = make_float2(2.f * (z.x * c.x - z.y * c.y), 2.f * (z.x * c.y + z.y * c.x));
+        break;
+      }
+      case ENDIA_OP_ABS: {  // sign(z) * g with real g: abs_op.mojo:93, sign_op.mojo:78-81, real_op.mojo:74-77
+        float r = sqrtf(z.x * z.x + z.y * z.y);
+        float c = g[j];
+        dx[j] = make_float2(z.x / r * c, z.y / r * c);
+        break;
+      }
+      default: dx[j] = g2[j]; break;
+    }
+  }
+}
+
+// ---- binary with broadcast -------------------------------------------------------------------
+struct BinDesc {
+  int ndim;
+  int64_t shape[8];
+  int64_t as[8];
+  int64_t bs[8];
+};
+
+template <int OP>
+__device__ __forceinline__ float bin_real(float a, float b) {
+  switch (OP) {
+    case ENDIA_BIN_ADD: return a + b;
+    case ENDIA_BIN_SUB: return a - b;
+    case ENDIA_BIN_MUL: return a * b;
+    case ENDIA_BIN_DIV: return a / b;
+    default: return a > b ? 1.f : 0.f;
+  }
+}
+
+template <int OP>
+__device__ __forceinline__ float2 bin_complex(float2 a, float2 b) {
+  switch (OP) {
+    case ENDIA_BIN_ADD: return make_float2(a.x + b.x, a.y + b.y);
+    case ENDIA_BIN_SUB: return make_float2(a.x - b.x, a.y - b.y);
+    case ENDIA_BIN_MUL: return make_float2(a.x * b.x - a.y * b.y, a.x * b.y + a.y * b.x);  // mul_op.mojo:152-155
+    default: {  // div_op.mojo:117-142
+      float d = b.x * b.x + b.y * b.y;
+      return make_float2((a.x * b.x + a.y * b.y) / d, (a.y * b.x - a.x * b.y) / d);
+    }
+  }
+}
+
+// Same-shape contiguous operands.
+template <int OP>
+__global__ __launch_bounds__(TPB) void bin_flat_kernel(const float* __restrict__ a, const float* __restrict__ b,
+                                                       float* __restrict__ o, int64_t n) {
+  int64_t i = (int64_t)blockIdx.x * TPB + threadIdx.x;
+  int64_t stride = (int64_t)gridDim.x * TPB;
+  int64_t n4 = n >> 2;
+  const float4* a4 = reinterpret_cast<const float4*>(a);
+  const float4* b4 = reinterpret_cast<const float4*>(b);
+  float4* o4 = reinterpret_cast<float4*>(o);
+  for (int64_t j = i; j < n4; j += stride) {
+    float4 x = a4[j], y = b4[j];
+    o4[j] = make_float4(bin_real<OP>(x.x, y.x), bin_real<OP>(x.y, y.y), bin_real<OP>(x.z, y.z), bin_real<OP>(x.w, y.w));
+  }
+  for (int64_t j = (n4 << 2) + i; j < n; j += stride) o[j] = bin_real<OP>(a[j], b[j]);
+}
+
+// [rows, cols] op with one operand a row vector [cols] (bias add and friends) or a scalar.
+// amode/bmode: 0 = full, 1 = row vector (index = col), 2 = scalar (index 0).
+template <int OP>
+__global__ __launch_bounds__(TPB) void bin_rowvec_kernel(const float* __restrict__ a, const float* __restrict__ b,
+                                                         float* __restrict__ o, int64_t n, int64_t cols,
+                                                         int amode, int bmode) {
+  int64_t i = (int64_t)blockIdx.x * TPB + threadIdx.x;
+  int64_t stride = (int64_t)gridDim.x * TPB;
+  for (int64_t j = i; j < n; j += stride) {
+    int64_t c = j % cols;
+    float x = a[amode == 0 ? j : (amode == 1 ? c : 0)];
+    float y = b[bmode == 0 ? j : (bmode == 1 ? c : 0)];
+    o[j] = bin_real<OP>(x, y);
+  }
+}
+
+template <int OP, bool CPLX>
+__global__ __launch_bounds__(TPB) void bin_general_kernel(BinDesc d, const float* __restrict__ a,
+                                                          const float* __restrict__ b, float* __restrict__ o,
+                                                          int64_t n) {
+  int64_t i = (int64_t)blockIdx.x * TPB + threadIdx.x;
+  int64_t stride = (int64_t)gridDim.x * TPB;
+  for (int64_t j = i; j < n; j += stride) {
+    int64_t r = j, ia = 0, ib = 0;
+    for (int k = d.ndim - 1; k >= 0; --k) {
+      int64_t q = r / d.shape[k];
+      int64_t c = r - q * d.shape[k];
+      ia += c * d.as[k];
+      ib += c * d.bs[k];
+      r = q;
+    }
+    if (CPLX) {
+      float2 x = reinterpret_cast<const float2*>(a)[ia];
+      float2 y = reinterpret_cast<const float2*>(b)[ib];
+      reinterpret_cast<float2*>(o)[j] = bin_complex<OP>(x, y);
+    } else {
+      o[j] = bin_real<OP>(a[ia], b[ib]);
+    }
+  }
+}
+
+__global__ __launch_bounds__(TPB) void axpby_kernel(int64_t n, float alpha, const float* __restrict__ a, float beta,
+                                                    const float* __restrict__ b, float* __restrict__ o, int vec) {
+  int64_t i = (int64_t)blockIdx.x * TPB + threadIdx.x;
+  int64_t stride = (int64_t)gridDim.x * TPB;
+  if (vec) {
+    int64_t n4 = n >> 2;
+    const float4* a4 = reinterpret_cast<const float4*>(a);
+    const float4* b4 = reinterpret_cast<const float4*>(b);
+    float4* o4 = reinterpret_cast<float4*>(o);
+    for (int64_t j = i; j < n4; j += stride) {
+      float4 x = a4[j];
+      float4 r = make_float4(alpha * x.x, alpha * x.y, alpha * x.z, alpha * x.w);
+      if (b) {
+        float4 y = b4[j];
+        r.x += beta * y.x; r.y += beta * y.y; r.z += beta * y.z; r.w += beta * y.w;
+      }
+      o4[j] = r;
+    }
+    for (int64_t j = (n4 << 2) + i; j < n; j += stride) o[j] = alpha * a[j] + (b ? beta * b[j] : 0.f);
+  } else {
+    for (int64_t j = i; j < n; j += stride) o[j] = alpha * a[j] + (b ? beta * b[j] : 0.f);
+  }
+}
+
+// ---- strided gather copy ---------------------------------------------------------------------
+struct CopyDesc {
+  int ndim;
+  int64_t shape[8];
+  int64_t st[8];
+  int64_t offset;
+};
+
+template <bool CPLX>
+__global__ __launch_bounds__(TPB) void strided_copy_kernel(CopyDesc d, const float* __restrict__ src,
+                                                           float* __restrict__ dst, int64_t n) {
+  int64_t i = (int64_t)blockIdx.x * TPB + threadIdx.x;
+  int64_t stride = (int64_t)gridDim.x * TPB;
+  for (int64_t j = i; j < n; j += stride) {
+    int64_t r = j, is = d.offset;
+    for (int k = d.ndim - 1; k >= 0; --k) {
+      int64_t q = r / d.shape[k];
+      is += (r - q * d.shape[k]) * d.st[k];
+      r = q;
+    }
+    if (CPLX) reinterpret_cast<float2*>(dst)[j] = reinterpret_cast<const float2*>(src)[is];
+    else dst[j] = src[is];
+  }
+}
+
+// 2-D transpose through LDS: dst[r][c] = src[c*ld + r]; both sides coalesced.
+__global__ __launch_bounds__(256) void transpose_kernel(const float* __restrict__ src, float* __restrict__ dst,
+                                                        int64_t rows, int64_t cols, int64_t ld, int64_t off) {
+  __shared__ float t[32][33];
+  int64_t c0 = (int64_t)blockIdx.x * 32, r0 = (int64_t)blockIdx.y * 32;
+  int tx = threadIdx.x & 31, ty = threadIdx.x >> 5;
+  for (int k = ty; k < 32; k += 8) {
+    int64_t c = c0 + k, r = r0 + tx;  // read src row c (contiguous in r)
+    t[k][tx] = (c < cols && r < rows) ? src[off + c * ld + r] : 0.f;
+  }
+  __syncthreads();
+  for (int k = ty; k < 32; k += 8) {
+    int64_t r = r0 + k, c = c0 + tx;
+    if (r < rows && c < cols) dst[r * cols + c] = t[tx][k];
+  }
+}
+
+template <typename F>
+int32_t dispatch_unary(int op, F&& f) {
+  switch (op) {
+    case ENDIA_OP_RELU: f(std::integral_constant<int, ENDIA_OP_RELU>()); break;
+    case ENDIA_OP_TANH: f(std::integral_constant<int, ENDIA_OP_TANH>()); break;
+    case ENDIA_OP_SIN: f(std::integral_constant<int, ENDIA_OP_SIN>()); break;
+    case ENDIA_OP_COS: f(std::integral_constant<int, ENDIA_OP_COS>()); break;
+    case ENDIA_OP_NEG: f(std::integral_constant<int, ENDIA_OP_NEG>()); break;
+    case ENDIA_OP_SQUARE: f(std::integral_constant<int, ENDIA_OP_SQUARE>()); break;
+    case ENDIA_OP_SQRT: f(std::integral_constant<int, ENDIA_OP_SQRT>()); break;
+    case ENDIA_OP_ABS: f(std::integral_constant<int, ENDIA_OP_ABS>()); break;
+    case ENDIA_OP_IDENTITY: f(std::integral_constant<int, ENDIA_OP_IDENTITY>()); break;
+    case ENDIA_OP_GREATER0: f(std::integral_constant<int, ENDIA_OP_GREATER0>()); break;
+    default: return -1;
+  }
+  return 0;
+}
+
+template <typename F>
+int32_t dispatch_binary(int op, F&& f) {
+  switch (op) {
+    case ENDIA_BIN_ADD: f(std::integral_constant<int, ENDIA_BIN_ADD>()); break;
+    case ENDIA_BIN_SUB: f(std::integral_constant<int, ENDIA_BIN_SUB>()); break;
+    case ENDIA_BIN_MUL: f(std::integral_constant<int, ENDIA_BIN_MUL>()); break;
+    case ENDIA_BIN_DIV: f(std::integral_constant<int, ENDIA_BIN_DIV>()); break;
+    case ENDIA_BIN_GREATER: f(std::integral_constant<int, ENDIA_BIN_GREATER>()); break;
+    default: return -1;
+  }
+  return 0;
+}
+
+}  // namespace
+
+using namespace endia;
+
+extern "C" {
+
+int32_t endia_hip_fill(float* p, int64_t n, float value) {
+  ENDIA_REQUIRE_INIT();
+  ENDIA_CHECK_ARG(n >= 0, "endia_hip_fill: negative n");
+  if (n == 0) return ENDIA_HIP_OK;
+  ENDIA_CHECK_ARG(p != nullptr, "endia_hip_fill: null pointer");
+  if (al16(p))
+    hipLaunchKernelGGL(fill_kernel, dim3(stream_grid((n + 3) / 4)), dim3(TPB), 0, ctx().stream, p, n, value);
+  else
+    hipLaunchKernelGGL(fill_scalar_kernel, dim3(stream_grid(n)), dim3(TPB), 0, ctx().stream, p, n, value);
+  ENDIA_LAUNCH_CHECK();
+  return ENDIA_HIP_OK;
+}
+
+// A fill kernel rather than hipMemsetAsync, so that a caller may record it into a HIP graph.
+int32_t endia_hip_memset0(void* p, int64_t bytes) {
+  ENDIA_REQUIRE_INIT();
+  ENDIA_CHECK_ARG(bytes >= 0 && bytes % 4 == 0, "endia_hip_memset0: size %lld is not a multiple of 4", (long long)bytes);
+  return endia_hip_fill(static_cast<float*>(p), bytes / 4, 0.f);
+}
+
+int32_t endia_hip_unary_fwd(int32_t op, int64_t n, const float* x, float* y, int32_t is_complex) {
+  ENDIA_REQUIRE_INIT();
+  ENDIA_CHECK_ARG(n >= 0, "endia_hip_unary_fwd: negative n");
+  if (n == 0) return ENDIA_HIP_OK;
+  ENDIA_CHECK_ARG(x && y, "endia_hip_unary_fwd: null pointer");
+  hipStream_t s = ctx().stream;
+  if (is_complex) {
+    if (!(op == ENDIA_OP_NEG || op == ENDIA_OP_SQUARE || op == ENDIA_OP_ABS || op == ENDIA_OP_IDENTITY))
+      return fail(ENDIA_HIP_ERR_UNSUPPORTED, "endia_hip_unary_fwd: op %d has no complex form here", op);
+    hipLaunchKernelGGL(unary_fwd_complex_kernel, dim3(stream_grid(n)), dim3(TPB), 0, s, op,
+                       reinterpret_cast<const float2*>(x), y, n);
+  } else {
+    bool vec = al16(x) && al16(y);
+    int grid = stream_grid(vec ? (n + 3) / 4 : n);
+    int rc = dispatch_unary(op, [&](auto tag) {
+      constexpr int OP = decltype(tag)::value;
+      if (vec) hipLaunchKernelGGL((unary_fwd_kernel<OP, true>), dim3(grid), dim3(TPB), 0, s, x, y, n);
+      else hipLaunchKernelGGL((unary_fwd_kernel<OP, false>), dim3(grid), dim3(TPB), 0, s, x, y, n);
+    });
+    ENDIA_CHECK_ARG(rc == 0, "endia_hip_unary_fwd: unknown op %d", op);
+  }
+  ENDIA_LAUNCH_CHECK();
+  return ENDIA_HIP_OK;
+}
+
+int32_t endia_hip_unary_vjp(int32_t op, int64_t n, const float* x, const float* g, float* dx, int32_t is_complex) {
+  ENDIA_REQUIRE_INIT();
+  ENDIA_CHECK_ARG(n >= 0, "endia_hip_unary_vjp: negative n");
+  if (n == 0) return ENDIA_HIP_OK;
+  ENDIA_CHECK_ARG(x && g && dx, "endia_hip_unary_vjp: null pointer");
+  hipStream_t s = ctx().stream;
+  if (is_complex) {
+    if (!(op == ENDIA_OP_NEG || op == ENDIA_OP_SQUARE || op == ENDIA_OP_ABS || op == ENDIA_OP_IDENTITY))
+      return fail(ENDIA_HIP_ERR_UNSUPPORTED, "endia_hip_unary_vjp: op %d has no complex form here", op);
+    hipLaunchKernelGGL(unary_vjp_complex_kernel, dim3(stream_grid(n)), dim3(TPB), 0, s, op,
+                       reinterpret_cast<const float2*>(x), g, reinterpret_cast<float2*>(dx), n);
+  } else {
+    bool vec = al16(x) && al16(g) && al16(dx);
+    int grid = stream_grid(vec ? (n + 3) / 4 : n);
+    int rc = dispatch_unary(op, [&](auto tag) {
+      constexpr int OP = decltype(tag)::value;
+      if (vec) hipLaunchKernelGGL((unary_vjp_kernel<OP, true>), dim3(grid), dim3(TPB), 0, s, x, g, dx, n);
+      else hipLaunchKernelGGL((unary_vjp_kernel<OP, false>), dim3(grid), dim3(TPB), 0, s, x, g, dx, n);
+    });
+    ENDIA_CHECK_ARG(rc == 0, "endia_hip_unary_vjp: unknown op %d", op);
+  }
+  ENDIA_LAUNCH_CHECK();
+  return ENDIA_HIP_OK;
+}
+
+int32_t endia_hip_binary(int32_t op, int32_t ndim, const int64_t* shape, const int64_t* a_strides,
+                         const int64_t* b_strides, const float* a, const float* b, float* out, int32_t is_complex) {
+  ENDIA_REQUIRE_INIT();
+  ENDIA_CHECK_ARG(ndim >= 0 && ndim <= 8, "endia_hip_binary: ndim %d out of [0,8]", ndim);
+  ENDIA_CHECK_ARG(ndim == 0 || (shape && a_strides && b_strides), "endia_hip_binary: null descriptor");
+  ENDIA_CHECK_ARG(op >= ENDIA_BIN_ADD && op <= ENDIA_BIN_GREATER, "endia_hip_binary: unknown op %d", op);
+  ENDIA_CHECK_ARG(!(is_complex && op == ENDIA_BIN_GREATER), "endia_hip_binary: greater is not defined for complex");
+  int64_t n = 1;
+  for (int i = 0; i < ndim; ++i) {
+    ENDIA_CHECK_ARG(shape[i] >= 0 && a_strides[i] >= 0 && b_strides[i] >= 0, "endia_hip_binary: negative extent or stride");
+    n *= shape[i];
+  }
+  if (n == 0) return ENDIA_HIP_OK;
+  ENDIA_CHECK_ARG(a && b && out, "endia_hip_binary: null pointer");
+  hipStream_t s = ctx().stream;
+
+  // classify each operand: contiguous-full, row vector along the last axis, scalar, or general
+  auto classify = [&](const int64_t* st) {
+    bool full = true, rowvec = ndim >= 1, scalar = true;
+    int64_t expect = 1;
+    for (int i = ndim - 1; i >= 0; --i) {
+      if (shape[i] != 1) {
+        if (st[i] != expect) full = false;
+        if (st[i] != 0) scalar = false;
+        if (i == ndim - 1) { if (st[i] != 1) rowvec = false; }
+        else if (st[i] != 0) rowvec = false;
+      }
+      expect *= shape[i];
+    }
+    return full ? 0 : (scalar ? 2 : (rowvec ? 1 : 3));
+  };
+  int am = classify(a_strides), bm = classify(b_strides);
+  int rc = 0;
+  if (!is_complex && am == 0 && bm == 0 && al16(a) && al16(b) && al16(out)) {
+    rc = dispatch_binary(op, [&](auto tag) {
+      constexpr int OP = decltype(tag)::value;
+      hipLaunchKernelGGL((bin_flat_kernel<OP>), dim3(stream_grid((n + 3) / 4)), dim3(TPB), 0, s, a, b, out, n);
+    });
+  } else if (!is_complex && am != 3 && bm != 3) {
+    int64_t cols = ndim ? shape[ndim - 1] : 1;
+    rc = dispatch_binary(op, [&](auto tag) {
+      constexpr int OP = decltype(tag)::value;
+      hipLaunchKernelGGL((bin_rowvec_kernel<OP>), dim3(stream_grid(n)), dim3(TPB), 0, s, a, b, out, n, cols, am, bm);
+    });
+  } else {
+    BinDesc d;
+    d.ndim = ndim;
+    for (int i = 0; i < 8; ++i) {
+      d.shape[i] = i < ndim ? shape[i] : 1;
+      d.as[i] = i < ndim ? a_strides[i] : 0;
+      d.bs[i] = i < ndim ? b_strides[i] : 0;
+    }
+    rc = dispatch_binary(op, [&](auto tag) {
+      constexpr int OP = decltype(tag)::value;
+      if (is_complex) {
+        if constexpr (OP != ENDIA_BIN_GREATER)
+          hipLaunchKernelGGL((bin_general_kernel<OP, true>), dim3(stream_grid(n)), dim3(TPB), 0, s, d, a, b, out, n);
+      } else {
+        hipLaunchKernelGGL((bin_general_kernel<OP, false>), dim3(stream_grid(n)), dim3(TPB), 0, s, d, a, b, out, n);
+      }
+    });
+  }
+  ENDIA_CHECK_ARG(rc == 0, "endia_hip_binary: unknown op %d", op);
+  ENDIA_LAUNCH_CHECK();
+  return ENDIA_HIP_OK;
+}
+
+int32_t endia_hip_axpby(int64_t n, float alpha, const float* a, float beta, const float* b, float* out) {
+  ENDIA_REQUIRE_INIT();
+  ENDIA_CHECK_ARG(n >= 0, "endia_hip_axpby: negative n");
+  if (n == 0) return ENDIA_HIP_OK;
+  ENDIA_CHECK_ARG(a && out, "endia_hip_axpby: null pointer");
+  int vec = al16(a) && al16(out) && (!b || al16(b));
+  hipLaunchKernelGGL(axpby_kernel, dim3(stream_grid(vec ? (n + 3) / 4 : n)), dim3(TPB), 0, ctx().stream, n, alpha, a,
+                     beta, b, out, vec);
+  ENDIA_LAUNCH_CHECK();
+  return ENDIA_HIP_OK;
+}
+
+int32_t endia_hip_strided_copy(int32_t ndim, const int64_t* shape, const int64_t* src_strides, int64_t src_offset,
+                               const float* src, float* dst, int32_t is_complex) {
+  ENDIA_REQUIRE_INIT();
+  ENDIA_CHECK_ARG(ndim >= 0 && ndim <= 8, "endia_hip_strided_copy: ndim %d out of [0,8]", ndim);
+  ENDIA_CHECK_ARG(ndim == 0 || (shape && src_strides), "endia_hip_strided_copy: null descriptor");
+  ENDIA_CHECK_ARG(src_offset >= 0, "endia_hip_strided_copy: negative offset");
+  int64_t n = 1;
+  for (int i = 0; i < ndim; ++i) {
+    ENDIA_CHECK_ARG(shape[i] >= 0 && src_strides[i] >= 0, "endia_hip_strided_copy: negative extent or stride");
+    n *= shape[i];
+  }
+  if (n == 0) return ENDIA_HIP_OK;
+  ENDIA_CHECK_ARG(src && dst, "endia_hip_strided_copy: null pointer");
+  hipStream_t s = ctx().stream;
+  // plain 2-D transpose (the .T() of a contiguous matrix) goes through LDS so both sides coalesce
+  if (!is_complex && ndim == 2 && src_strides[0] == 1 && src_strides[1] >= shape[0] && shape[0] > 1 && shape[1] > 1) {
+    dim3 grid((unsigned)ceil_div64(shape[1], 32), (unsigned)ceil_div64(shape[0], 32));
+    if (grid.y <= 65535) {
+      hipLaunchKernelGGL(transpose_kernel, grid, dim3(256), 0, s, src, dst, shape[0], shape[1], src_strides[1], src_offset);
+      ENDIA_LAUNCH_CHECK();
+      return ENDIA_HIP_OK;
+    }
+  }
+  CopyDesc d;
+  d.ndim = ndim;
+  d.offset = src_offset;
+  for (int i = 0; i < 8; ++i) {
+    d.shape[i] = i < ndim ? shape[i] : 1;
+    d.st[i] = i < ndim ? src_strides[i] : 0;
+  }
+  if (is_complex)
+    hipLaunchKernelGGL((strided_copy_kernel<true>), dim3(stream_grid(n)), dim3(TPB), 0, s, d, src, dst, n);
+  else
+    hipLaunchKernelGGL((strided_copy_kernel<false>), dim3(stream_grid(n)), dim3(TPB), 0, s, d, src, dst, n);
+  ENDIA_LAUNCH_CHECK();
+  return ENDIA_HIP_OK;
+}
+
+}  // extern "C"

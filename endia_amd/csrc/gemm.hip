@@ -1,0 +1,393 @@
+// fp32 GEMM on the CDNA4 matrix cores: matmul_fwd and both products of matmul_vjp
+// (endia/functional/binary_ops/matmul_op.mojo:93-254, 278-283) as ONE kernel family.
+//
+// The reference makes the left operand contiguous, materialises a transposed copy of the right
+// operand and then runs one dot product per output element (matmul_op.mojo:107-199). Here a
+// transposed operand is only a different global->LDS path, selected by transA/transB, and the
+// products run on v_mfma_f32_32x32x2_f32.
+//
+// Tiling: a 256-thread work-group (four 64-lane waves, 2 x 2) owns a 128 x 128 tile of C; each
+// wave owns 64 x 64 as 2 x 2 MFMA blocks of 32 x 32 (64 accumulator registers per lane). The K
+// loop advances 32 at a time: the next tile's global loads are issued into registers before the
+// MFMAs of the current tile and written to LDS after them.
+//
+// LDS layouts. An operand whose K index is contiguous in memory ("K-major": A when transA = 0,
+// B when transB = 1) is stored [row][32 + 4] and fetched with one 128-bit read per four MFMA
+// steps; an operand whose M (or N) index is contiguous ("MN-major") is stored [k][128 + 8] and
+// fetched with 32-bit reads. The MFMA takes K in pairs (lanes 0-31 hold k, lanes 32-63 hold
+// k + 1); because a sum over k may be taken in any order, step s = 4j + i of a tile uses
+// k = 8j + 4h + i for half-wave h, which is what makes the 128-bit fetch possible. Both
+// operands use the same mapping.
+#include "common.h"
+
+typedef float floatx16 __attribute__((ext_vector_type(16)));
+
+namespace {
+
+constexpr int BM = 128, BN = 128, BK = 32;
+constexpr int LDK = BK + 4;   // row stride of a K-major tile (floats)
+constexpr int LDM = BM + 8;   // row stride of an MN-major tile (floats)
+constexpr int NTHREADS = 256;
+
+struct GemmArgs {
+  const float* A;
+  const float* B;
+  float* C;
+  const float* bias;
+  const float* aux_in;
+  float* aux_out;
+  int64_t lda, ldb, ldc;
+  int64_t sA, sB, sC;
+  int M, N, K;
+  int tiles_m, tiles_n;
+  int act;        // endia_hip_unary_op
+  int from_out;   // activation gradient from stored output instead of pre-activation
+  int accumulate;
+};
+
+__device__ __forceinline__ float act_fwd(int act, float z) {
+  switch (act) {
+    case ENDIA_OP_RELU: return z > 0.f ? z : 0.f;
+    case ENDIA_OP_TANH: return tanhf(z);
+    case ENDIA_OP_SIN: return sinf(z);
+    default: return z;
+  }
+}
+
+__device__ __forceinline__ float act_grad(int act, int from_out, float aux) {
+  switch (act) {
+    case ENDIA_OP_RELU: return aux > 0.f ? 1.f : 0.f;
+    case ENDIA_OP_TANH: {
+      float a = from_out ? aux : tanhf(aux);
+      return 1.f - a * a;
+    }
+    case ENDIA_OP_SIN: return cosf(aux);
+    default: return 1.f;
+  }
+}
+
+template <int EPI>
+__device__ __forceinline__ void epilogue_store(const GemmArgs& p, float* __restrict__ C,
+                                               const float* __restrict__ aux_in,
+                                               float* __restrict__ aux_out, int row, int col, float v) {
+  int64_t off = (int64_t)row * p.ldc + col;
+  if (EPI == ENDIA_EPI_BIAS) {
+    v += p.bias[col];
+  } else if (EPI == ENDIA_EPI_BIAS_ACT) {
+    v += p.bias[col];
+    if (aux_out) aux_out[off] = v;
+    v = act_fwd(p.act, v);
+  } else if (EPI == ENDIA_EPI_ACT_GRAD) {
+    v *= act_grad(p.act, p.from_out, aux_in[off]);
+  }
+  if (p.accumulate) v += C[off];
+  C[off] = v;
+}
+
+// Map the linear work-group id to a tile. Work-groups are dealt round-robin to the 8 XCDs, each
+// with a private L2, so first give every XCD a contiguous range of tile ids, then walk that range
+// in column-major order inside bands of 8 tile-rows so that concurrently resident tiles share
+// A-rows and B-columns.
+__device__ __forceinline__ void tile_of_block(int bid, int nblocks, int tiles_m, int tiles_n, int& tm,
+                                              int& tn) {
+  int lid = bid;
+  if ((nblocks & 7) == 0) {
+    int per = nblocks >> 3;
+    lid = (bid & 7) * per + (bid >> 3);
+  }
+  const int GM = 8;
+  int band = GM * tiles_n;
+  int g = lid / band;
+  int first_m = g * GM;
+  int gsz = tiles_m - first_m < GM ? tiles_m - first_m : GM;
+  int r = lid - g * band;
+  tm = first_m + r % gsz;
+  tn = r / gsz;
+}
+
+template <bool A_KMAJOR, bool B_KMAJOR, int EPI>
+__global__ __launch_bounds__(NTHREADS, 2) void sgemm_mfma_kernel(GemmArgs p) {
+  __shared__ __attribute__((aligned(16))) float As[A_KMAJOR ? BM * LDK : BK * LDM];
+  __shared__ __attribute__((aligned(16))) float Bs[B_KMAJOR ? BN * LDK : BK * LDM];
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = tid >> 6;
+  const int wm = wave >> 1, wn = wave & 1;
+  const int l32 = lane & 31, h = lane >> 5;
+
+  int tm, tn;
+  tile_of_block(blockIdx.x, gridDim.x, p.tiles_m, p.tiles_n, tm, tn);
+  const int m0 = tm * BM, n0 = tn * BN;
+  const int64_t bz = blockIdx.y;
+  const float* __restrict__ A = p.A + bz * p.sA;
+  const float* __restrict__ B = p.B + bz * p.sB;
+  float* __restrict__ C = p.C + bz * p.sC;
+  const float* __restrict__ aux_in = p.aux_in ? p.aux_in + bz * p.sC : nullptr;
+  float* __restrict__ aux_out = p.aux_out ? p.aux_out + bz * p.sC : nullptr;
+
+  // ---- global -> register staging ---------------------------------------------------------
+  // K-major tile: thread covers rows r0 + 32*i (i < 4), floats [kq*4, kq*4+4) of the 32-wide slab.
+  // MN-major tile: thread covers k rows k0 + 8*i (i < 4), floats [mq*4, mq*4+4) of the 128-wide row.
+  float4 ra[4], rb[4];
+  const int a_r = A_KMAJOR ? (tid >> 3) : (tid >> 5);
+  const int a_c = A_KMAJOR ? (tid & 7) * 4 : (tid & 31) * 4;
+  const int b_r = B_KMAJOR ? (tid >> 3) : (tid >> 5);
+  const int b_c = B_KMAJOR ? (tid & 7) * 4 : (tid & 31) * 4;
+
+  auto load_tiles = [&](int k0) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      if (A_KMAJOR) {
+        int m = m0 + a_r + 32 * i, k = k0 + a_c;
+        ra[i] = (m < p.M && k < p.K) ? *reinterpret_cast<const float4*>(A + (int64_t)m * p.lda + k)
+                                     : make_float4(0.f, 0.f, 0.f, 0.f);
+      } else {
+        int k = k0 + a_r + 8 * i, m = m0 + a_c;
+        ra[i] = (k < p.K && m < p.M) ? *reinterpret_cast<const float4*>(A + (int64_t)k * p.lda + m)
+                                     : make_float4(0.f, 0.f, 0.f, 0.f);
+      }
+      if (B_KMAJOR) {
+        int n = n0 + b_r + 32 * i, k = k0 + b_c;
+        rb[i] = (n < p.N && k < p.K) ? *reinterpret_cast<const float4*>(B + (int64_t)n * p.ldb + k)
+                                     : make_float4(0.f, 0.f, 0.f, 0.f);
+      } else {
+        int k = k0 + b_r + 8 * i, n = n0 + b_c;
+        rb[i] = (k < p.K && n < p.N) ? *reinterpret_cast<const float4*>(B + (int64_t)k * p.ldb + n)
+                                     : make_float4(0.f, 0.f, 0.f, 0.f);
+      }
+    }
+  };
+  auto store_tiles = [&]() {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      if (A_KMAJOR)
+        *reinterpret_cast<float4*>(&As[(a_r + 32 * i) * LDK + a_c]) = ra[i];
+      else
+        *reinterpret_cast<float4*>(&As[(a_r + 8 * i) * LDM + a_c]) = ra[i];
+      if (B_KMAJOR)
+        *reinterpret_cast<float4*>(&Bs[(b_r + 32 * i) * LDK + b_c]) = rb[i];
+      else
+        *reinterpret_cast<float4*>(&Bs[(b_r + 8 * i) * LDM + b_c]) = rb[i];
+    }
+  };
+
+  floatx16 acc[2][2];
+#pragma unroll
+  for (int i = 0; i < 2; ++i)
+#pragma unroll
+    for (int j = 0; j < 2; ++j)
+#pragma unroll
+      for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.f;
+
+  const int a_row = wm * 64 + l32;  // + 32*fm
+  const int b_col = wn * 64 + l32;  // + 32*fn
+
+  load_tiles(0);
+  store_tiles();
+  __syncthreads();
+
+  for (int k0 = 0; k0 < p.K; k0 += BK) {
+    const bool more = k0 + BK < p.K;
+    if (more) load_tiles(k0 + BK);
+
+#pragma unroll
+    for (int j = 0; j < BK / 8; ++j) {
+      float af[2][4], bf[2][4];
+#pragma unroll
+      for (int f = 0; f < 2; ++f) {
+        if (A_KMAJOR) {
+          float4 t = *reinterpret_cast<const float4*>(&As[(a_row + 32 * f) * LDK + 8 * j + 4 * h]);
+          af[f][0] = t.x; af[f][1] = t.y; af[f][2] = t.z; af[f][3] = t.w;
+        } else {
+#pragma unroll
+          for (int i = 0; i < 4; ++i) af[f][i] = As[(8 * j + 4 * h + i) * LDM + a_row + 32 * f];
+        }
+        if (B_KMAJOR) {
+          float4 t = *reinterpret_cast<const float4*>(&Bs[(b_col + 32 * f) * LDK + 8 * j + 4 * h]);
+          bf[f][0] = t.x; bf[f][1] = t.y; bf[f][2] = t.z; bf[f][3] = t.w;
+        } else {
+#pragma unroll
+          for (int i = 0; i < 4; ++i) bf[f][i] = Bs[(8 * j + 4 * h + i) * LDM + b_col + 32 * f];
+        }
+      }
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int fm = 0; fm < 2; ++fm)
+#pragma unroll
+          for (int fn = 0; fn < 2; ++fn)
+            acc[fm][fn] = __builtin_amdgcn_mfma_f32_32x32x2f32(af[fm][i], bf[fn][i], acc[fm][fn], 0, 0, 0);
+    }
+
+    if (more) {
+      __syncthreads();
+      store_tiles();
+      __syncthreads();
+    }
+  }
+
+  // ---- epilogue: lane holds rows 8*(v/4) + 4*h + v%4 and column l32 of each 32 x 32 block ----
+#pragma unroll
+  for (int fm = 0; fm < 2; ++fm)
+#pragma unroll
+    for (int fn = 0; fn < 2; ++fn) {
+      int col = n0 + wn * 64 + fn * 32 + l32;
+      if (col >= p.N) continue;
+#pragma unroll
+      for (int v = 0; v < 16; ++v) {
+        int row = m0 + wm * 64 + fm * 32 + 8 * (v >> 2) + 4 * h + (v & 3);
+        if (row < p.M) epilogue_store<EPI>(p, C, aux_in, aux_out, row, col, acc[fm][fn][v]);
+      }
+    }
+}
+
+// Fallback for operands the vector path cannot take (leading dimensions, sizes or pointers that are
+// not multiples of 4 floats, e.g. the 1-wide first and last layers of the reference's sine-fit
+// MLP, benchmarks/mlp_benchmarks/mlp_imp.mojo:35-37). 64 x 64 tile, 16 x 16 threads, 4 x 4 each.
+template <int EPI>
+__global__ __launch_bounds__(256) void sgemm_generic_kernel(GemmArgs p, int transA, int transB) {
+  constexpr int T = 64, TK = 16;
+  __shared__ float As[TK][T + 1];
+  __shared__ float Bs[TK][T + 1];
+  const int tid = threadIdx.x;
+  const int tx = tid & 15, ty = tid >> 4;
+  const int m0 = blockIdx.y * T, n0 = blockIdx.x * T;
+  const int64_t bz = blockIdx.z;
+  const float* __restrict__ A = p.A + bz * p.sA;
+  const float* __restrict__ B = p.B + bz * p.sB;
+  float* __restrict__ C = p.C + bz * p.sC;
+  const float* __restrict__ aux_in = p.aux_in ? p.aux_in + bz * p.sC : nullptr;
+  float* __restrict__ aux_out = p.aux_out ? p.aux_out + bz * p.sC : nullptr;
+  float acc[4][4] = {};
+  for (int k0 = 0; k0 < p.K; k0 += TK) {
+    for (int e = tid; e < T * TK; e += 256) {
+      int kk, mm;
+      if (transA) { kk = e / T; mm = e % T; } else { mm = e / TK; kk = e % TK; }
+      int m = m0 + mm, k = k0 + kk;
+      float v = 0.f;
+      if (m < p.M && k < p.K) v = transA ? A[(int64_t)k * p.lda + m] : A[(int64_t)m * p.lda + k];
+      As[kk][mm] = v;
+      int nn;
+      if (transB) { nn = e / TK; kk = e % TK; } else { kk = e / T; nn = e % T; }
+      int n = n0 + nn;
+      k = k0 + kk;
+      v = 0.f;
+      if (n < p.N && k < p.K) v = transB ? B[(int64_t)n * p.ldb + k] : B[(int64_t)k * p.ldb + n];
+      Bs[kk][nn] = v;
+    }
+    __syncthreads();
+#pragma unroll
+    for (int kk = 0; kk < TK; ++kk) {
+      float a[4], b[4];
+#pragma unroll
+      for (int i = 0; i < 4; ++i) { a[i] = As[kk][ty + 16 * i]; b[i] = Bs[kk][tx + 16 * i]; }
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) acc[i][j] = fmaf(a[i], b[j], acc[i][j]);
+    }
+    __syncthreads();
+  }
+#pragma unroll
+  for (int i = 0; i < 4; ++i)
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      int row = m0 + ty + 16 * i, col = n0 + tx + 16 * j;
+      if (row < p.M && col < p.N) epilogue_store<EPI>(p, C, aux_in, aux_out, row, col, acc[i][j]);
+    }
+}
+
+template <int EPI>
+void launch_mfma(const GemmArgs& p, int transA, int transB, dim3 grid, hipStream_t s) {
+  const bool ak = !transA, bk = transB != 0;
+  if (ak && bk) hipLaunchKernelGGL((sgemm_mfma_kernel<true, true, EPI>), grid, dim3(NTHREADS), 0, s, p);
+  else if (ak && !bk) hipLaunchKernelGGL((sgemm_mfma_kernel<true, false, EPI>), grid, dim3(NTHREADS), 0, s, p);
+  else if (!ak && bk) hipLaunchKernelGGL((sgemm_mfma_kernel<false, true, EPI>), grid, dim3(NTHREADS), 0, s, p);
+  else hipLaunchKernelGGL((sgemm_mfma_kernel<false, false, EPI>), grid, dim3(NTHREADS), 0, s, p);
+}
+
+inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; }
+
+}  // namespace
+
+namespace endia {
+
+// Shared by endia_hip_sgemm and the complex and convolution front ends.
+int32_t sgemm_impl(int transA, int transB, int64_t M, int64_t N, int64_t K, const float* A, int64_t lda,
+                   const float* B, int64_t ldb, float* C, int64_t ldc, int64_t batch, int64_t sA,
+                   int64_t sB, int64_t sC, int epi_flags, int act_flags, const float* bias,
+                   const float* aux_in, float* aux_out) {
+  const int epi = epi_flags & 0xff;
+  const int accumulate = (epi_flags & ENDIA_GEMM_ACCUMULATE) ? 1 : 0;
+  const int act = act_flags & 0xff;
+  const int from_out = (act_flags & ENDIA_ACT_FROM_OUTPUT) ? 1 : 0;
+  ENDIA_CHECK_ARG(M >= 0 && N >= 0 && K >= 0 && batch >= 0, "sgemm: negative dimension (M=%lld N=%lld K=%lld batch=%lld)",
+                  (long long)M, (long long)N, (long long)K, (long long)batch);
+  ENDIA_CHECK_ARG(M < (1ll << 31) && N < (1ll << 31) && K < (1ll << 31) && batch <= 65535,
+                  "sgemm: dimension too large");
+  ENDIA_CHECK_ARG(epi >= ENDIA_EPI_NONE && epi <= ENDIA_EPI_ACT_GRAD, "sgemm: unknown epilogue %d", epi);
+  ENDIA_CHECK_ARG((epi_flags & ~(0xff | ENDIA_GEMM_ACCUMULATE)) == 0, "sgemm: unknown epilogue flag bits 0x%x", epi_flags);
+  ENDIA_CHECK_ARG(act == ENDIA_OP_RELU || act == ENDIA_OP_TANH || act == ENDIA_OP_SIN || act == ENDIA_OP_IDENTITY,
+                  "sgemm: activation %d is not one of relu/tanh/sin/identity", act);
+  ENDIA_CHECK_ARG(!(from_out && act == ENDIA_OP_SIN), "sgemm: sin gradient needs the pre-activation, not the output");
+  if (M == 0 || N == 0 || batch == 0) return ENDIA_HIP_OK;
+  ENDIA_CHECK_ARG(C != nullptr, "sgemm: C is null");
+  ENDIA_CHECK_ARG(K == 0 || (A != nullptr && B != nullptr), "sgemm: A or B is null");
+  ENDIA_CHECK_ARG(lda >= (transA ? M : K) && ldb >= (transB ? K : N) && ldc >= N,
+                  "sgemm: leading dimension too small (lda=%lld ldb=%lld ldc=%lld)", (long long)lda,
+                  (long long)ldb, (long long)ldc);
+  ENDIA_CHECK_ARG(sA >= 0 && sB >= 0 && sC >= 0, "sgemm: negative batch stride");
+  ENDIA_CHECK_ARG(batch == 1 || sC >= (M - 1) * ldc + N, "sgemm: batch stride of C overlaps");
+  if (epi == ENDIA_EPI_BIAS || epi == ENDIA_EPI_BIAS_ACT) ENDIA_CHECK_ARG(bias != nullptr, "sgemm: epilogue needs bias");
+  if (epi == ENDIA_EPI_ACT_GRAD) ENDIA_CHECK_ARG(aux_in != nullptr, "sgemm: ACT_GRAD epilogue needs aux_in");
+
+  GemmArgs p;
+  p.A = A; p.B = B; p.C = C; p.bias = bias; p.aux_in = aux_in;
+  p.aux_out = (epi == ENDIA_EPI_BIAS_ACT) ? aux_out : nullptr;
+  p.lda = lda; p.ldb = ldb; p.ldc = ldc; p.sA = sA; p.sB = sB; p.sC = sC;
+  p.M = (int)M; p.N = (int)N; p.K = (int)K;
+  p.act = act; p.from_out = from_out; p.accumulate = accumulate;
+  hipStream_t s = ctx().stream;
+
+  // The vector path loads 4 floats at a time along the contiguous index of each operand.
+  const bool a_ok = aligned16(A) && lda % 4 == 0 && sA % 4 == 0 && (transA ? M % 4 == 0 : K % 4 == 0);
+  const bool b_ok = aligned16(B) && ldb % 4 == 0 && sB % 4 == 0 && (transB ? K % 4 == 0 : N % 4 == 0);
+  const bool big = M * N >= 64 * 64 && K >= 8;
+  if (a_ok && b_ok && big) {
+    p.tiles_m = (int)ceil_div64(M, BM);
+    p.tiles_n = (int)ceil_div64(N, BN);
+    dim3 grid((unsigned)(p.tiles_m * p.tiles_n), (unsigned)batch);
+    switch (epi) {
+      case ENDIA_EPI_NONE: launch_mfma<ENDIA_EPI_NONE>(p, transA, transB, grid, s); break;
+      case ENDIA_EPI_BIAS: launch_mfma<ENDIA_EPI_BIAS>(p, transA, transB, grid, s); break;
+      case ENDIA_EPI_BIAS_ACT: launch_mfma<ENDIA_EPI_BIAS_ACT>(p, transA, transB, grid, s); break;
+      default: launch_mfma<ENDIA_EPI_ACT_GRAD>(p, transA, transB, grid, s); break;
+    }
+  } else {
+    p.tiles_m = (int)ceil_div64(M, 64);
+    p.tiles_n = (int)ceil_div64(N, 64);
+    ENDIA_CHECK_ARG(p.tiles_m <= 65535, "sgemm: M too large for the unaligned path");
+    dim3 grid((unsigned)p.tiles_n, (unsigned)p.tiles_m, (unsigned)batch);
+    switch (epi) {
+      case ENDIA_EPI_NONE: hipLaunchKernelGGL((sgemm_generic_kernel<ENDIA_EPI_NONE>), grid, dim3(256), 0, s, p, transA, transB); break;
+      case ENDIA_EPI_BIAS: hipLaunchKernelGGL((sgemm_generic_kernel<ENDIA_EPI_BIAS>), grid, dim3(256), 0, s, p, transA, transB); break;
+      case ENDIA_EPI_BIAS_ACT: hipLaunchKernelGGL((sgemm_generic_kernel<ENDIA_EPI_BIAS_ACT>), grid, dim3(256), 0, s, p, transA, transB); break;
+      default: hipLaunchKernelGGL((sgemm_generic_kernel<ENDIA_EPI_ACT_GRAD>), grid, dim3(256), 0, s, p, transA, transB); break;
+    }
+  }
+  ENDIA_LAUNCH_CHECK();
+  return ENDIA_HIP_OK;
+}
+
+}  // namespace endia
+
+extern "C" int32_t endia_hip_sgemm(int32_t transA, int32_t transB, int64_t M, int64_t N, int64_t K,
+                                   const float* A, int64_t lda, const float* B, int64_t ldb, float* C,
+                                   int64_t ldc, int64_t batch, int64_t strideA, int64_t strideB,
+                                   int64_t strideC, int32_t epilogue, int32_t act, const float* bias,
+                                   const float* aux_in, float* aux_out) {
+  ENDIA_REQUIRE_INIT();
+  return endia::sgemm_impl(transA, transB, M, N, K, A, lda, B, ldb, C, ldc, batch, strideA, strideB,
+                           strideC, epilogue, act, bias, aux_in, aux_out);
+}

@@ -1,0 +1,124 @@
+// Fused optimizer steps. The reference builds each update from ~3 (SGD, endia/optim/sgd.mojo:61-62)
+// or ~14 (Adam, endia/optim/adam.mojo:47-65) separate full-tensor Array ops with temporaries and a raw
+// copy back into the parameter (endia/_array/_array.mojo:998-1006). Here each is ONE pass: SGD moves
+// 12 bytes per parameter (read p, g; write p), Adam 28 (read p, g, m, v; write p, m, v).
+//
+// Every intermediate of the reference is an fp32 Array, so each arithmetic step rounds to fp32. The
+// kernels keep that: products and sums are written with the round-to-nearest intrinsics so the
+// compiler cannot contract them into fused multiply-adds.
+#include "common.h"
+
+#include <math.h>
+
+namespace {
+
+constexpr int TPB = 256;
+
+struct AdamK {
+  float lr, b1, b2, eps, omb1, omb2, c1, c2;  // c1 = 1 - b1^t, c2 = 1 - b2^t
+};
+
+__device__ __forceinline__ void adam_one(float& p, float g, float& m, float& v, const AdamK& k) {
+  m = __fadd_rn(__fmul_rn(k.b1, m), __fmul_rn(k.omb1, g));
+  v = __fadd_rn(__fmul_rn(k.b2, v), __fmul_rn(__fmul_rn(k.omb2, g), g));
+  float mh = __fdiv_rn(m, k.c1);
+  float vh = __fdiv_rn(v, k.c2);
+  // the reference's real sqrt is sqrt((|x|+x)/2) (sqrt_op.mojo:111-114): equal to sqrt(x) for x >= 0
+  float den = __fadd_rn(__fsqrt_rn(__fmul_rn(__fadd_rn(fabsf(vh), vh), 0.5f)), k.eps);
+  p = __fsub_rn(p, __fdiv_rn(__fmul_rn(k.lr, mh), den));
+}
+
+__global__ __launch_bounds__(TPB) void adam_kernel(int64_t n, float* __restrict__ p, const float* __restrict__ g,
+                                                   float* __restrict__ m, float* __restrict__ v, AdamK k, int vec) {
+  int64_t i = (int64_t)blockIdx.x * TPB + threadIdx.x;
+  int64_t stride = (int64_t)gridDim.x * TPB;
+  if (vec) {
+    int64_t n4 = n >> 2;
+    float4* p4 = reinterpret_cast<float4*>(p);
+    const float4* g4 = reinterpret_cast<const float4*>(g);
+    float4* m4 = reinterpret_cast<float4*>(m);
+    float4* v4 = reinterpret_cast<float4*>(v);
+    for (int64_t j = i; j < n4; j += stride) {
+      float4 P = p4[j], G = g4[j], M = m4[j], V = v4[j];
+      adam_one(P.x, G.x, M.x, V.x, k);
+      adam_one(P.y, G.y, M.y, V.y, k);
+      adam_one(P.z, G.z, M.z, V.z, k);
+      adam_one(P.w, G.w, M.w, V.w, k);
+      p4[j] = P; m4[j] = M; v4[j] = V;
+    }
+    for (int64_t j = (n4 << 2) + i; j < n; j += stride) adam_one(p[j], g[j], m[j], v[j], k);
+  } else {
+    for (int64_t j = i; j < n; j += stride) adam_one(p[j], g[j], m[j], v[j], k);
+  }
+}
+
+__global__ __launch_bounds__(TPB) void sgd_kernel(int64_t n, float* __restrict__ p, const float* __restrict__ g, float lr,
+                                                  int vec) {
+  int64_t i = (int64_t)blockIdx.x * TPB + threadIdx.x;
+  int64_t stride = (int64_t)gridDim.x * TPB;
+  if (vec) {
+    int64_t n4 = n >> 2;
+    float4* p4 = reinterpret_cast<float4*>(p);
+    const float4* g4 = reinterpret_cast<const float4*>(g);
+    for (int64_t j = i; j < n4; j += stride) {
+      float4 P = p4[j], G = g4[j];
+      P.x = __fsub_rn(P.x, __fmul_rn(lr, G.x));
+      P.y = __fsub_rn(P.y, __fmul_rn(lr, G.y));
+      P.z = __fsub_rn(P.z, __fmul_rn(lr, G.z));
+      P.w = __fsub_rn(P.w, __fmul_rn(lr, G.w));
+      p4[j] = P;
+    }
+    for (int64_t j = (n4 << 2) + i; j < n; j += stride) p[j] = __fsub_rn(p[j], __fmul_rn(lr, g[j]));
+  } else {
+    for (int64_t j = i; j < n; j += stride) p[j] = __fsub_rn(p[j], __fmul_rn(lr, g[j]));
+  }
+}
+
+inline bool al16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; }
+
+inline int stream_grid(int64_t nvec) {
+  int64_t blocks = ceil_div64(nvec, TPB);
+  int64_t cap = (int64_t)endia::ctx().cu_count * 8;
+  if (blocks > cap) blocks = cap;
+  if (blocks < 1) blocks = 1;
+  return (int)blocks;
+}
+
+}  // namespace
+
+using namespace endia;
+
+extern "C" {
+
+int32_t endia_hip_sgd_step(int64_t n, float* p, const float* g, float lr) {
+  ENDIA_REQUIRE_INIT();
+  ENDIA_CHECK_ARG(n >= 0, "endia_hip_sgd_step: negative n");
+  if (n == 0) return ENDIA_HIP_OK;
+  ENDIA_CHECK_ARG(p && g, "endia_hip_sgd_step: null pointer");
+  int vec = al16(p) && al16(g);
+  hipLaunchKernelGGL(sgd_kernel, dim3(stream_grid(vec ? (n + 3) / 4 : n)), dim3(TPB), 0, ctx().stream, n, p, g, lr, vec);
+  ENDIA_LAUNCH_CHECK();
+  return ENDIA_HIP_OK;
+}
+
+int32_t endia_hip_adam_step(int64_t n, float* p, const float* g, float* m, float* v, float lr, float beta1, float beta2,
+                            float eps, float t) {
+  ENDIA_REQUIRE_INIT();
+  ENDIA_CHECK_ARG(n >= 0, "endia_hip_adam_step: negative n");
+  ENDIA_CHECK_ARG(t >= 1.0f, "endia_hip_adam_step: step counter t = %g must start at 1", (double)t);
+  if (n == 0) return ENDIA_HIP_OK;
+  ENDIA_CHECK_ARG(p && g && m && v, "endia_hip_adam_step: null pointer");
+  AdamK k;
+  k.lr = lr; k.b1 = beta1; k.b2 = beta2; k.eps = eps;
+  k.omb1 = 1.0f - beta1;
+  k.omb2 = 1.0f - beta2;
+  k.c1 = 1.0f - powf(beta1, t);
+  k.c2 = 1.0f - powf(beta2, t);
+  int vec = al16(p) && al16(g) && al16(m) && al16(v);
+  hipLaunchKernelGGL(adam_kernel, dim3(stream_grid(vec ? (n + 3) / 4 : n)), dim3(TPB), 0, ctx().stream, n, p, g, m, v, k,
+                     vec);
+  ENDIA_LAUNCH_CHECK();
+  return ENDIA_HIP_OK;
+}
+
+}  // extern "C"

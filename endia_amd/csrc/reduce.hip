@@ -1,0 +1,348 @@
+// Sum reductions: ReduceAdd.__call__ (endia/functional/reduce_ops/reduce_add_op.mojo:65-210), which
+// is also Expand.vjp, the bias gradient db = 1^T dZ (endia/functional/view_ops/expand_op.mojo:121-126),
+// sum and mean (sum_op.mojo:35-62, mean_op.mojo:35-65), and the fused MSE loss + gradient
+// (endia/functional/loss_ops/mse_op.mojo:17-20).
+//
+// The reference accumulates sequentially in fp32 into a zeroed output. Here every reduction is two
+// stages with a fixed shape (so results are run-to-run identical): stage 1 spreads the input over
+// enough work-groups to fill the chip, each wave reading 1 KiB of consecutive addresses per access
+// and combining lanes with wave shuffles; stage 2 adds the per-group partials in index order.
+#include "common.h"
+
+namespace {
+
+constexpr int TPB = 256;
+
+__device__ __forceinline__ float wave_sum(float v) {
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) v += __shfl_down(v, off, 64);
+  return v;
+}
+
+// all 256 threads call; result valid in thread 0
+__device__ __forceinline__ float block_sum(float v, float* red /* >= 4 floats */) {
+  v = wave_sum(v);
+  int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
+  __syncthreads();
+  if (lane == 0) red[w] = v;
+  __syncthreads();
+  return red[0] + red[1] + red[2] + red[3];
+}
+
+// ---- column reduction: x[batch][R][C] -> out[batch][C] (sum over R) --------------------------
+// grid (ceil(C/256), S, batch). A wave reads 256 consecutive columns of one row per access (float4
+// per lane); the four waves of a group take rows r, r+1, r+2, r+3 (mod 4) of the group's row range.
+__global__ __launch_bounds__(TPB) void col_reduce_vec_kernel(const float* __restrict__ x, float* __restrict__ part,
+                                                             int64_t R, int64_t C, int64_t rows_per_split) {
+  __shared__ float4 red[4][64];
+  const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
+  const int64_t c = ((int64_t)blockIdx.x * 64 + lane) * 4;
+  const int64_t b = blockIdx.z;
+  const int64_t r0 = (int64_t)blockIdx.y * rows_per_split;
+  int64_t r1 = r0 + rows_per_split;
+  if (r1 > R) r1 = R;
+  float4 acc = make_float4(0.f, 0.f, 0.f, 0.f);
+  if (c < C) {
+    const float* base = x + b * R * C + c;
+    for (int64_t r = r0 + w; r < r1; r += 4) {
+      float4 v = *reinterpret_cast<const float4*>(base + r * C);
+      acc.x += v.x; acc.y += v.y; acc.z += v.z; acc.w += v.w;
+    }
+  }
+  red[w][lane] = acc;
+  __syncthreads();
+  if (w == 0 && c < C) {
+    float4 a = red[0][lane], b1 = red[1][lane], c1 = red[2][lane], d = red[3][lane];
+    float4 s = make_float4((a.x + b1.x) + (c1.x + d.x), (a.y + b1.y) + (c1.y + d.y),
+                           (a.z + b1.z) + (c1.z + d.z), (a.w + b1.w) + (c1.w + d.w));
+    *reinterpret_cast<float4*>(part + ((b * gridDim.y + blockIdx.y) * C + c)) = s;
+  }
+}
+
+// scalar variant for C not a multiple of 4 or unaligned: thread per column, 256 columns per group
+__global__ __launch_bounds__(TPB) void col_reduce_scalar_kernel(const float* __restrict__ x, float* __restrict__ part,
+                                                                int64_t R, int64_t C, int64_t rows_per_split) {
+  const int64_t c = (int64_t)blockIdx.x * TPB + threadIdx.x;
+  const int64_t b = blockIdx.z;
+  const int64_t r0 = (int64_t)blockIdx.y * rows_per_split;
+  int64_t r1 = r0 + rows_per_split;
+  if (r1 > R) r1 = R;
+  if (c >= C) return;
+  float acc = 0.f;
+  const float* base = x + b * R * C + c;
+  for (int64_t r = r0; r < r1; ++r) acc += base[r * C];
+  part[(b * gridDim.y + blockIdx.y) * C + c] = acc;
+}
+
+// stage 2: out[b][c] = scale * sum_s part[b][s][c]
+__global__ __launch_bounds__(TPB) void col_reduce_final_kernel(const float* __restrict__ part, float* __restrict__ out,
+                                                               int64_t S, int64_t C, int64_t batch, float scale) {
+  int64_t i = (int64_t)blockIdx.x * TPB + threadIdx.x;
+  if (i >= batch * C) return;
+  int64_t b = i / C, c = i - b * C;
+  float acc = 0.f;
+  for (int64_t s = 0; s < S; ++s) acc += part[(b * S + s) * C + c];
+  out[i] = acc * scale;
+}
+
+// ---- row reduction: x[R][C] -> out[R] (sum over C) --------------------------------------------
+// grid (S, R). Each group sums a contiguous chunk of one row; partials [R][S].
+__global__ __launch_bounds__(TPB) void row_reduce_kernel(const float* __restrict__ x, float* __restrict__ part,
+                                                         int64_t C, int64_t chunk, int vec) {
+  __shared__ float red[4];
+  const int64_t r = blockIdx.y;
+  const int64_t c0 = (int64_t)blockIdx.x * chunk;
+  int64_t c1 = c0 + chunk;
+  if (c1 > C) c1 = C;
+  const float* row = x + r * C;
+  float acc = 0.f;
+  if (vec) {  // chunk % 4 == 0, row base 16-byte aligned
+    int64_t n4 = (c1 - c0) >> 2;
+    const float4* p4 = reinterpret_cast<const float4*>(row + c0);
+    for (int64_t j = threadIdx.x; j < n4; j += TPB) {
+      float4 v = p4[j];
+      acc += (v.x + v.y) + (v.z + v.w);
+    }
+    for (int64_t j = c0 + (n4 << 2) + threadIdx.x; j < c1; j += TPB) acc += row[j];
+  } else {
+    for (int64_t j = c0 + threadIdx.x; j < c1; j += TPB) acc += row[j];
+  }
+  float s = block_sum(acc, red);
+  if (threadIdx.x == 0) part[r * gridDim.x + blockIdx.x] = s;
+}
+
+// stage 2: out[r] = scale * sum_s part[r][s]; one wave per row
+__global__ __launch_bounds__(TPB) void row_reduce_final_kernel(const float* __restrict__ part, float* __restrict__ out,
+                                                               int64_t R, int64_t S, float scale) {
+  const int lane = threadIdx.x & 63;
+  const int64_t r = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (r >= R) return;
+  float acc = 0.f;
+  for (int64_t s = lane; s < S; s += 64) acc += part[r * S + s];
+  acc = wave_sum(acc);
+  if (lane == 0) out[r] = acc * scale;
+}
+
+// ---- any mask: one work-group per output element ----------------------------------------------
+struct RedDesc {
+  int nk, nr;            // number of kept / reduced axes
+  int64_t kshape[8], kstride[8];
+  int64_t rshape[8], rstride[8];
+};
+
+__global__ __launch_bounds__(TPB) void generic_reduce_kernel(RedDesc d, const float* __restrict__ x,
+                                                             float* __restrict__ out, int64_t nred, float scale) {
+  __shared__ float red[4];
+  int64_t o = blockIdx.x, rem = o, base = 0;
+  for (int k = d.nk - 1; k >= 0; --k) {
+    int64_t q = rem / d.kshape[k];
+    base += (rem - q * d.kshape[k]) * d.kstride[k];
+    rem = q;
+  }
+  float acc = 0.f;
+  for (int64_t j = threadIdx.x; j < nred; j += TPB) {
+    int64_t r = j, off = base;
+    for (int k = d.nr - 1; k >= 0; --k) {
+      int64_t q = r / d.rshape[k];
+      off += (r - q * d.rshape[k]) * d.rstride[k];
+      r = q;
+    }
+    acc += x[off];
+  }
+  float s = block_sum(acc, red);
+  if (threadIdx.x == 0) out[o] = s * scale;
+}
+
+// ---- MSE ------------------------------------------------------------------------------------
+// One pass: dpred = 2 (p - t) / n and per-group partial sums of (p - t)^2.
+__global__ __launch_bounds__(TPB) void mse_kernel(const float* __restrict__ p, const float* __restrict__ t,
+                                                  float* __restrict__ dp, float* __restrict__ part, int64_t n,
+                                                  float two_over_n, int vec) {
+  __shared__ float red[4];
+  int64_t i = (int64_t)blockIdx.x * TPB + threadIdx.x;
+  int64_t stride = (int64_t)gridDim.x * TPB;
+  float acc = 0.f;
+  if (vec) {
+    int64_t n4 = n >> 2;
+    const float4* p4 = reinterpret_cast<const float4*>(p);
+    const float4* t4 = reinterpret_cast<const float4*>(t);
+    float4* d4 = reinterpret_cast<float4*>(dp);
+    for (int64_t j = i; j < n4; j += stride) {
+      float4 a = p4[j], b = t4[j];
+      float4 d = make_float4(a.x - b.x, a.y - b.y, a.z - b.z, a.w - b.w);
+      acc += (d.x * d.x + d.y * d.y) + (d.z * d.z + d.w * d.w);
+      if (dp) d4[j] = make_float4(d.x * two_over_n, d.y * two_over_n, d.z * two_over_n, d.w * two_over_n);
+    }
+    for (int64_t j = (n4 << 2) + i; j < n; j += stride) {
+      float d = p[j] - t[j];
+      acc += d * d;
+      if (dp) dp[j] = d * two_over_n;
+    }
+  } else {
+    for (int64_t j = i; j < n; j += stride) {
+      float d = p[j] - t[j];
+      acc += d * d;
+      if (dp) dp[j] = d * two_over_n;
+    }
+  }
+  float s = block_sum(acc, red);
+  if (part && threadIdx.x == 0) part[blockIdx.x] = s;
+}
+
+__global__ __launch_bounds__(TPB) void sum_partials_kernel(const float* __restrict__ part, float* __restrict__ out,
+                                                           int64_t S, float scale) {
+  __shared__ float red[4];
+  float acc = 0.f;
+  for (int64_t j = threadIdx.x; j < S; j += TPB) acc += part[j];
+  float s = block_sum(acc, red);
+  if (threadIdx.x == 0) out[0] = s * scale;
+}
+
+inline bool al16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; }
+
+}  // namespace
+
+namespace endia {
+
+// out[b][c] = scale * sum_r x[b][r][c]
+int32_t col_reduce(int64_t batch, int64_t R, int64_t C, const float* x, float* out, float scale) {
+  hipStream_t s = ctx().stream;
+  const bool vec = (C % 4 == 0) && al16(x);
+  const int64_t col_tiles = ceil_div64(C, 256);
+  if (col_tiles * 1 > 2147483647ll || batch > 65535)
+    return fail(ENDIA_HIP_ERR_UNSUPPORTED, "col_reduce: extent too large");
+  // enough row splits for ~4 groups per CU, at least 16 rows each
+  int64_t want = (int64_t)ctx().cu_count * 4;
+  int64_t S = want / (col_tiles * batch);
+  if (S < 1) S = 1;
+  int64_t max_s = ceil_div64(R, 16);
+  if (S > max_s) S = max_s;
+  if (S > 1024) S = 1024;
+  int64_t rows_per_split = ceil_div64(R, S);
+  S = ceil_div64(R, rows_per_split);
+  void* ws = nullptr;
+  int32_t rc = workspace(batch * S * C * (int64_t)sizeof(float), &ws);
+  if (rc) return rc;
+  float* part = static_cast<float*>(ws);
+  dim3 grid((unsigned)col_tiles, (unsigned)S, (unsigned)batch);
+  if (vec) hipLaunchKernelGGL(col_reduce_vec_kernel, grid, dim3(TPB), 0, s, x, part, R, C, rows_per_split);
+  else hipLaunchKernelGGL(col_reduce_scalar_kernel, grid, dim3(TPB), 0, s, x, part, R, C, rows_per_split);
+  ENDIA_LAUNCH_CHECK();
+  hipLaunchKernelGGL(col_reduce_final_kernel, dim3((unsigned)ceil_div64(batch * C, TPB)), dim3(TPB), 0, s, part, out, S,
+                     C, batch, scale);
+  ENDIA_LAUNCH_CHECK();
+  return ENDIA_HIP_OK;
+}
+
+// out[r] = scale * sum_c x[r][c]
+int32_t row_reduce(int64_t R, int64_t C, const float* x, float* out, float scale) {
+  hipStream_t s = ctx().stream;
+  if (R > 65535) return fail(ENDIA_HIP_ERR_UNSUPPORTED, "row_reduce: more than 65535 rows");
+  int64_t want = (int64_t)ctx().cu_count * 8;
+  int64_t S = want / R;
+  if (S < 1) S = 1;
+  int64_t max_s = ceil_div64(C, 4096);
+  if (S > max_s) S = max_s;
+  int64_t chunk = ceil_div64(ceil_div64(C, S), 4) * 4;
+  S = ceil_div64(C, chunk);
+  const int vec = (C % 4 == 0) && al16(x);
+  void* ws = nullptr;
+  int32_t rc = workspace(R * S * (int64_t)sizeof(float), &ws);
+  if (rc) return rc;
+  float* part = static_cast<float*>(ws);
+  hipLaunchKernelGGL(row_reduce_kernel, dim3((unsigned)S, (unsigned)R), dim3(TPB), 0, s, x, part, C, chunk, vec);
+  ENDIA_LAUNCH_CHECK();
+  hipLaunchKernelGGL(row_reduce_final_kernel, dim3((unsigned)ceil_div64(R, 4)), dim3(TPB), 0, s, part, out, R, S, scale);
+  ENDIA_LAUNCH_CHECK();
+  return ENDIA_HIP_OK;
+}
+
+}  // namespace endia
+
+using namespace endia;
+
+extern "C" {
+
+int32_t endia_hip_reduce_add(int32_t ndim, const int64_t* shape, uint32_t reduce_mask, const float* x, float* out,
+                             float scale, int32_t is_complex) {
+  ENDIA_REQUIRE_INIT();
+  ENDIA_CHECK_ARG(ndim >= 0 && ndim <= 8, "endia_hip_reduce_add: ndim %d out of [0,8]", ndim);
+  ENDIA_CHECK_ARG(ndim == 0 || shape, "endia_hip_reduce_add: null shape");
+  ENDIA_CHECK_ARG(ndim == 8 ? true : (reduce_mask >> ndim) == 0, "endia_hip_reduce_add: mask 0x%x names an axis >= ndim", reduce_mask);
+  ENDIA_CHECK_ARG(!(is_complex && ndim == 8), "endia_hip_reduce_add: complex needs ndim <= 7");
+  // collapse neighbouring axes with the same status into groups; size-1 axes join either side
+  int64_t gshape[9];
+  int gred[9];
+  int ng = 0;
+  int64_t total = 1, nout = 1;
+  for (int i = 0; i < ndim; ++i) {
+    ENDIA_CHECK_ARG(shape[i] >= 0, "endia_hip_reduce_add: negative extent");
+    total *= shape[i];
+    int red = (reduce_mask >> i) & 1;
+    if (!red) nout *= shape[i];
+    if (shape[i] == 1) continue;
+    if (ng && gred[ng - 1] == red) gshape[ng - 1] *= shape[i];
+    else { gshape[ng] = shape[i]; gred[ng] = red; ++ng; }
+  }
+  if (is_complex) {  // trailing kept axis of the (re, im) pair
+    if (ng && gred[ng - 1] == 0) gshape[ng - 1] *= 2;
+    else { gshape[ng] = 2; gred[ng] = 0; ++ng; }
+    nout *= 2;
+  }
+  if (nout == 0) return ENDIA_HIP_OK;
+  ENDIA_CHECK_ARG(out != nullptr, "endia_hip_reduce_add: out is null");
+  if (total == 0) return endia_hip_fill(out, nout, 0.f);  // empty sum
+  ENDIA_CHECK_ARG(x != nullptr, "endia_hip_reduce_add: x is null");
+
+  if (ng == 0) return endia_hip_axpby(1, scale, x, 0.f, nullptr, out);
+  if (ng == 1 && !gred[0]) return endia_hip_axpby(gshape[0], scale, x, 0.f, nullptr, out);
+  if (ng == 1 && gred[0]) return row_reduce(1, gshape[0], x, out, scale);
+  if (ng == 2 && gred[0] && !gred[1]) return col_reduce(1, gshape[0], gshape[1], x, out, scale);
+  if (ng == 2 && !gred[0] && gred[1] && gshape[0] <= 65535) return row_reduce(gshape[0], gshape[1], x, out, scale);
+  if (ng == 3 && !gred[0] && gred[1] && !gred[2] && gshape[0] <= 65535)
+    return col_reduce(gshape[0], gshape[1], gshape[2], x, out, scale);
+
+  // everything else (e.g. N,C,H,W -> C): one work-group per output element
+  RedDesc d;
+  d.nk = d.nr = 0;
+  int64_t st = 1, nred = 1;
+  int64_t strides[9];
+  for (int g = ng - 1; g >= 0; --g) { strides[g] = st; st *= gshape[g]; }
+  for (int g = 0; g < ng; ++g) {
+    if (gred[g]) { d.rshape[d.nr] = gshape[g]; d.rstride[d.nr] = strides[g]; ++d.nr; nred *= gshape[g]; }
+    else { d.kshape[d.nk] = gshape[g]; d.kstride[d.nk] = strides[g]; ++d.nk; }
+  }
+  ENDIA_CHECK_ARG(nout <= 2147483647ll, "endia_hip_reduce_add: too many outputs for the general path");
+  hipLaunchKernelGGL(generic_reduce_kernel, dim3((unsigned)nout), dim3(TPB), 0, ctx().stream, d, x, out, nred, scale);
+  ENDIA_LAUNCH_CHECK();
+  return ENDIA_HIP_OK;
+}
+
+int32_t endia_hip_mse_fwd_bwd(int64_t n, const float* pred, const float* target, float* loss, float* dpred) {
+  ENDIA_REQUIRE_INIT();
+  ENDIA_CHECK_ARG(n > 0, "endia_hip_mse_fwd_bwd: n must be positive (got %lld)", (long long)n);
+  ENDIA_CHECK_ARG(pred && target, "endia_hip_mse_fwd_bwd: null input");
+  ENDIA_CHECK_ARG(loss || dpred, "endia_hip_mse_fwd_bwd: nothing to compute");
+  hipStream_t s = ctx().stream;
+  const int vec = al16(pred) && al16(target) && (!dpred || al16(dpred));
+  int64_t blocks = ceil_div64(vec ? (n + 3) / 4 : n, TPB);
+  int64_t cap = (int64_t)ctx().cu_count * 8;
+  if (blocks > cap) blocks = cap;
+  float* part = nullptr;
+  if (loss) {
+    void* ws = nullptr;
+    int32_t rc = workspace(blocks * (int64_t)sizeof(float), &ws);
+    if (rc) return rc;
+    part = static_cast<float*>(ws);
+  }
+  const float inv_n = 1.0f / (float)n;
+  hipLaunchKernelGGL(mse_kernel, dim3((unsigned)blocks), dim3(TPB), 0, s, pred, target, dpred, part, n, 2.0f * inv_n, vec);
+  ENDIA_LAUNCH_CHECK();
+  if (loss) {
+    hipLaunchKernelGGL(sum_partials_kernel, dim3(1), dim3(TPB), 0, s, part, loss, blocks, inv_n);
+    ENDIA_LAUNCH_CHECK();
+  }
+  return ENDIA_HIP_OK;
+}
+
+}  // extern "C"

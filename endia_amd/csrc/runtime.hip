@@ -1,0 +1,268 @@
+// Context, buffer pool, copies and timers of libendia_hip.so.
+//
+// The reference allocates and zero-fills a fresh heap buffer for every op output
+// (endia/functional/_utils.mojo:319-327) and frees it when the node dies
+// (endia/_array/_array.mojo:177-179). Here the same two calls hit a size-bucketed pool of device
+// buffers, so a training step runs without hipMalloc after its first iteration, and buffers
+// that a kernel overwrites completely are never memset.
+#include "common.h"
+
+#include <map>
+#include <string.h>
+#include <unordered_map>
+#include <vector>
+
+namespace endia {
+
+static Context g_ctx;
+Context& ctx() { return g_ctx; }
+
+static thread_local char g_err[512] = "";
+
+int32_t fail(int32_t code, const char* fmt, ...) {
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(g_err, sizeof(g_err), fmt, ap);
+  va_end(ap);
+  return code;
+}
+
+// ---- pool ---------------------------------------------------------------------------------
+// Sizes round up to 512 B below 1 MiB and to 2 MiB above, so the activations of one layer
+// shape all land in one bucket.
+static int64_t bucket_of(int64_t bytes) {
+  if (bytes <= 0) bytes = 1;
+  const int64_t small = 512, large = 2ll << 20;
+  if (bytes <= (1ll << 20)) return (bytes + small - 1) / small * small;
+  return (bytes + large - 1) / large * large;
+}
+
+struct Pool {
+  std::multimap<int64_t, void*> free_by_size;
+  std::unordered_map<void*, int64_t> live;    // pointer -> bucket size, handed out
+  std::unordered_map<void*, int64_t> owned;   // every pointer obtained from hipMalloc
+  int64_t in_use = 0, cached = 0, n_allocs = 0;
+};
+static Pool g_pool;
+
+static void* g_ws = nullptr;
+static int64_t g_ws_bytes = 0;
+
+int32_t workspace(int64_t bytes, void** out) {
+  if (bytes > g_ws_bytes) {
+    if (g_ws) (void)hipFree(g_ws);
+    g_ws = nullptr;
+    g_ws_bytes = 0;
+    int64_t want = bucket_of(bytes);
+    hipError_t e = hipMalloc(&g_ws, (size_t)want);
+    if (e != hipSuccess)
+      return fail(ENDIA_HIP_ERR_NOMEM, "workspace: hipMalloc(%lld) failed: %s", (long long)want,
+                  hipGetErrorString(e));
+    g_ws_bytes = want;
+  }
+  *out = g_ws;
+  return ENDIA_HIP_OK;
+}
+
+static const int kTimerSlots = 64;
+static hipEvent_t g_ev_start[kTimerSlots], g_ev_stop[kTimerSlots];
+static bool g_ev_made = false;
+
+}  // namespace endia
+
+using namespace endia;
+
+extern "C" {
+
+const char* endia_hip_last_error(void) { return g_err; }
+
+int32_t endia_hip_init(int32_t device) {
+  if (g_ctx.ready) {
+    if (g_ctx.device == device) return ENDIA_HIP_OK;
+    return fail(ENDIA_HIP_ERR_INVALID, "endia_hip_init: already initialised on device %d", g_ctx.device);
+  }
+  int count = 0;
+  hipError_t e = hipGetDeviceCount(&count);
+  if (e != hipSuccess || count == 0)
+    return fail(ENDIA_HIP_ERR_RUNTIME, "endia_hip_init: no HIP device visible (%s)",
+                e == hipSuccess ? "count = 0" : hipGetErrorString(e));
+  ENDIA_CHECK_ARG(device >= 0 && device < count, "endia_hip_init: device %d out of range [0,%d)", device, count);
+  ENDIA_HIP_CALL(hipSetDevice(device));
+  hipDeviceProp_t prop;
+  ENDIA_HIP_CALL(hipGetDeviceProperties(&prop, device));
+  if (strncmp(prop.gcnArchName, "gfx950", 6) != 0)
+    return fail(ENDIA_HIP_ERR_UNSUPPORTED, "endia_hip_init: device is %s; this library holds gfx950 code only",
+                prop.gcnArchName);
+  ENDIA_HIP_CALL(hipStreamCreateWithFlags(&g_ctx.stream, hipStreamNonBlocking));
+  if (!g_ev_made) {
+    for (int i = 0; i < kTimerSlots; ++i) {
+      ENDIA_HIP_CALL(hipEventCreate(&g_ev_start[i]));
+      ENDIA_HIP_CALL(hipEventCreate(&g_ev_stop[i]));
+    }
+    g_ev_made = true;
+  }
+  g_ctx.device = device;
+  g_ctx.cu_count = prop.multiProcessorCount;
+  g_ctx.clock_mhz = prop.clockRate / 1000;
+  g_ctx.ready = true;
+  return ENDIA_HIP_OK;
+}
+
+int32_t endia_hip_shutdown(void) {
+  if (!g_ctx.ready) return ENDIA_HIP_OK;
+  (void)hipStreamSynchronize(g_ctx.stream);
+  for (auto& kv : g_pool.owned) (void)hipFree(kv.first);
+  g_pool = Pool();
+  if (g_ws) (void)hipFree(g_ws);
+  g_ws = nullptr;
+  g_ws_bytes = 0;
+  (void)hipStreamDestroy(g_ctx.stream);
+  g_ctx = Context();
+  return ENDIA_HIP_OK;
+}
+
+int32_t endia_hip_sync(void) {
+  ENDIA_REQUIRE_INIT();
+  ENDIA_HIP_CALL(hipStreamSynchronize(g_ctx.stream));
+  return ENDIA_HIP_OK;
+}
+
+int32_t endia_hip_device_info(char* buf, int64_t buf_bytes, int32_t* cu_count, int32_t* clock_mhz) {
+  ENDIA_REQUIRE_INIT();
+  hipDeviceProp_t prop;
+  ENDIA_HIP_CALL(hipGetDeviceProperties(&prop, g_ctx.device));
+  if (buf && buf_bytes > 0)
+    snprintf(buf, (size_t)buf_bytes, "%s %s, %d CUs, %d MHz, %.1f GiB", prop.name, prop.gcnArchName,
+             prop.multiProcessorCount, prop.clockRate / 1000, prop.totalGlobalMem / 1073741824.0);
+  if (cu_count) *cu_count = prop.multiProcessorCount;
+  if (clock_mhz) *clock_mhz = prop.clockRate / 1000;
+  return ENDIA_HIP_OK;
+}
+
+int32_t endia_hip_malloc(int64_t bytes, void** out) {
+  ENDIA_REQUIRE_INIT();
+  ENDIA_CHECK_ARG(out != nullptr, "endia_hip_malloc: out is null");
+  ENDIA_CHECK_ARG(bytes >= 0, "endia_hip_malloc: negative size %lld", (long long)bytes);
+  int64_t b = bucket_of(bytes);
+  auto it = g_pool.free_by_size.find(b);
+  void* p = nullptr;
+  if (it != g_pool.free_by_size.end()) {
+    p = it->second;
+    g_pool.free_by_size.erase(it);
+    g_pool.cached -= b;
+  } else {
+    hipError_t e = hipMalloc(&p, (size_t)b);
+    if (e != hipSuccess) {
+      // give cached buffers back to the driver and retry once
+      (void)hipStreamSynchronize(g_ctx.stream);
+      for (auto& kv : g_pool.free_by_size) {
+        (void)hipFree(kv.second);
+        g_pool.owned.erase(kv.second);
+      }
+      g_pool.free_by_size.clear();
+      g_pool.cached = 0;
+      (void)hipGetLastError();
+      e = hipMalloc(&p, (size_t)b);
+      if (e != hipSuccess) {
+        (void)hipGetLastError();
+        *out = nullptr;
+        return fail(ENDIA_HIP_ERR_NOMEM, "endia_hip_malloc: hipMalloc(%lld) failed: %s", (long long)b,
+                    hipGetErrorString(e));
+      }
+    }
+    g_pool.owned[p] = b;
+    g_pool.n_allocs++;
+  }
+  g_pool.live[p] = b;
+  g_pool.in_use += b;
+  *out = p;
+  return ENDIA_HIP_OK;
+}
+
+int32_t endia_hip_free(void* p) {
+  ENDIA_REQUIRE_INIT();
+  if (!p) return ENDIA_HIP_OK;
+  auto it = g_pool.live.find(p);
+  ENDIA_CHECK_ARG(it != g_pool.live.end(), "endia_hip_free: %p was not handed out by endia_hip_malloc", p);
+  int64_t b = it->second;
+  g_pool.live.erase(it);
+  g_pool.in_use -= b;
+  g_pool.free_by_size.emplace(b, p);
+  g_pool.cached += b;
+  return ENDIA_HIP_OK;
+}
+
+int32_t endia_hip_pool_stats(int64_t* bytes_in_use, int64_t* bytes_cached, int64_t* n_device_allocs) {
+  ENDIA_REQUIRE_INIT();
+  if (bytes_in_use) *bytes_in_use = g_pool.in_use;
+  if (bytes_cached) *bytes_cached = g_pool.cached;
+  if (n_device_allocs) *n_device_allocs = g_pool.n_allocs;
+  return ENDIA_HIP_OK;
+}
+
+int32_t endia_hip_pool_trim(void) {
+  ENDIA_REQUIRE_INIT();
+  ENDIA_HIP_CALL(hipStreamSynchronize(g_ctx.stream));
+  for (auto& kv : g_pool.free_by_size) {
+    (void)hipFree(kv.second);
+    g_pool.owned.erase(kv.second);
+  }
+  g_pool.free_by_size.clear();
+  g_pool.cached = 0;
+  return ENDIA_HIP_OK;
+}
+
+int32_t endia_hip_memcpy_h2d(void* dst, const void* src, int64_t bytes) {
+  ENDIA_REQUIRE_INIT();
+  ENDIA_CHECK_ARG(bytes >= 0, "endia_hip_memcpy_h2d: negative size");
+  if (bytes == 0) return ENDIA_HIP_OK;
+  ENDIA_CHECK_ARG(dst && src, "endia_hip_memcpy_h2d: null pointer");
+  // pageable host memory: the copy is staged by the runtime and the host buffer may be reused on return
+  ENDIA_HIP_CALL(hipMemcpyAsync(dst, src, (size_t)bytes, hipMemcpyHostToDevice, g_ctx.stream));
+  ENDIA_HIP_CALL(hipStreamSynchronize(g_ctx.stream));
+  return ENDIA_HIP_OK;
+}
+
+int32_t endia_hip_memcpy_d2h(void* dst, const void* src, int64_t bytes) {
+  ENDIA_REQUIRE_INIT();
+  ENDIA_CHECK_ARG(bytes >= 0, "endia_hip_memcpy_d2h: negative size");
+  if (bytes == 0) return ENDIA_HIP_OK;
+  ENDIA_CHECK_ARG(dst && src, "endia_hip_memcpy_d2h: null pointer");
+  ENDIA_HIP_CALL(hipMemcpyAsync(dst, src, (size_t)bytes, hipMemcpyDeviceToHost, g_ctx.stream));
+  ENDIA_HIP_CALL(hipStreamSynchronize(g_ctx.stream));
+  return ENDIA_HIP_OK;
+}
+
+int32_t endia_hip_memcpy_d2d(void* dst, const void* src, int64_t bytes) {
+  ENDIA_REQUIRE_INIT();
+  ENDIA_CHECK_ARG(bytes >= 0, "endia_hip_memcpy_d2d: negative size");
+  if (bytes == 0) return ENDIA_HIP_OK;
+  ENDIA_CHECK_ARG(dst && src, "endia_hip_memcpy_d2d: null pointer");
+  ENDIA_HIP_CALL(hipMemcpyAsync(dst, src, (size_t)bytes, hipMemcpyDeviceToDevice, g_ctx.stream));
+  return ENDIA_HIP_OK;
+}
+
+int32_t endia_hip_timer_start(int32_t slot) {
+  ENDIA_REQUIRE_INIT();
+  ENDIA_CHECK_ARG(slot >= 0 && slot < kTimerSlots, "endia_hip_timer_start: slot %d out of range", slot);
+  ENDIA_HIP_CALL(hipEventRecord(g_ev_start[slot], g_ctx.stream));
+  return ENDIA_HIP_OK;
+}
+
+int32_t endia_hip_timer_stop(int32_t slot) {
+  ENDIA_REQUIRE_INIT();
+  ENDIA_CHECK_ARG(slot >= 0 && slot < kTimerSlots, "endia_hip_timer_stop: slot %d out of range", slot);
+  ENDIA_HIP_CALL(hipEventRecord(g_ev_stop[slot], g_ctx.stream));
+  return ENDIA_HIP_OK;
+}
+
+int32_t endia_hip_timer_elapsed_ms(int32_t slot, float* ms) {
+  ENDIA_REQUIRE_INIT();
+  ENDIA_CHECK_ARG(slot >= 0 && slot < kTimerSlots, "endia_hip_timer_elapsed_ms: slot %d out of range", slot);
+  ENDIA_CHECK_ARG(ms != nullptr, "endia_hip_timer_elapsed_ms: ms is null");
+  ENDIA_HIP_CALL(hipEventSynchronize(g_ev_stop[slot]));
+  ENDIA_HIP_CALL(hipEventElapsedTime(ms, g_ev_start[slot], g_ev_stop[slot]));
+  return ENDIA_HIP_OK;
+}
+
+}  // extern "C"

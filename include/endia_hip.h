@@ -1,0 +1,197 @@
+/*
+ * endia_hip.h -- C ABI of libendia_hip.so: the MI355X (gfx950) implementation of
+ * Endia's reverse-mode dense-layer training step.
+ *
+ * Conventions (they mirror the data contract of the reference's op plug-in seam,
+ * endia/functional/_utils.mojo:208-327 and endia/_array/_array.mojo:523-536):
+ *   - every tensor is fp32, row-major; a complex64 tensor is interleaved (re, im) fp32 pairs;
+ *   - every data pointer is a DEVICE pointer obtained from endia_hip_malloc (or any
+ *     hipMalloc'ed memory of the current device); host pointers appear only in the
+ *     memcpy calls and in small descriptor arrays (shapes, strides);
+ *   - sizes, leading dimensions and strides are int64 counts of ELEMENTS (complex: of
+ *     complex elements), never bytes, except where the name says "bytes";
+ *   - every call returns 0 on success or a negative endia_hip_status; the text of the last
+ *     failure on the calling thread is returned by endia_hip_last_error();
+ *   - work is enqueued on one internal HIP stream in call order and is asynchronous to the
+ *     host; endia_hip_sync() (and the d2h copy) block until it has drained;
+ *   - the library keeps one global context and is not thread-safe, like the reference,
+ *     whose hot path is single-threaded (matmul_op.mojo:168-169).
+ */
+#ifndef ENDIA_HIP_H
+#define ENDIA_HIP_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define ENDIA_API __attribute__((visibility("default")))
+
+typedef enum {
+  ENDIA_HIP_OK = 0,
+  ENDIA_HIP_ERR_INVALID = -1,     /* bad argument: null pointer, negative size, bad enum, bad shape */
+  ENDIA_HIP_ERR_NOT_INIT = -2,    /* endia_hip_init has not succeeded */
+  ENDIA_HIP_ERR_RUNTIME = -3,     /* a HIP runtime call failed */
+  ENDIA_HIP_ERR_NOMEM = -4,       /* device allocation failed */
+  ENDIA_HIP_ERR_UNSUPPORTED = -5  /* valid request outside what this build implements */
+} endia_hip_status;
+
+/* Unary operators. Replaces the per-op forward bodies and VJP rules of
+ * endia/functional/unary_ops/{relu,tanh,sin,cos,neg,square,sqrt,abs}_op.mojo. */
+typedef enum {
+  ENDIA_OP_RELU = 0,   /* relu_op.mojo:115-117 ; vjp greater(x,0)*g  relu_op.mojo:95  */
+  ENDIA_OP_TANH = 1,   /* tanh_op.mojo:112-115 ; vjp (1-tanh(x)^2)*g tanh_op.mojo:92  */
+  ENDIA_OP_SIN = 2,    /* sin_op.mojo:112-114  ; vjp cos(x)*g        sin_op.mojo:92   */
+  ENDIA_OP_COS = 3,    /* cos_op.mojo:113-115  ; vjp -sin(x)*g       cos_op.mojo:93   */
+  ENDIA_OP_NEG = 4,    /* neg_op.mojo:111-113  ; vjp -g              neg_op.mojo:91   */
+  ENDIA_OP_SQUARE = 5, /* square_op.mojo:117-119; vjp 2*x*g          square_op.mojo:96 */
+  ENDIA_OP_SQRT = 6,   /* sqrt_op.mojo:111-114 (0 for x<0) ; vjp g/(2*sqrt(x)) sqrt_op.mojo:91 */
+  ENDIA_OP_ABS = 7,    /* abs_op.mojo:114-115,157 ; vjp sign(x)*g    abs_op.mojo:93   */
+  ENDIA_OP_IDENTITY = 8,
+  ENDIA_OP_GREATER0 = 9 /* 1.0 where x > 0 else 0.0: greater_op.mojo:46-60 against a zero operand */
+} endia_hip_unary_op;
+
+/* Binary operators: endia/functional/binary_ops/{add,sub,mul,div}_op.mojo. */
+typedef enum {
+  ENDIA_BIN_ADD = 0,
+  ENDIA_BIN_SUB = 1,
+  ENDIA_BIN_MUL = 2,
+  ENDIA_BIN_DIV = 3,
+  ENDIA_BIN_GREATER = 4 /* 1.0 where a > b else 0.0 (real only): greater_op.mojo:46-60 */
+} endia_hip_binary_op;
+
+/* GEMM epilogues (what is applied to the accumulator tile before it is stored). */
+typedef enum {
+  ENDIA_EPI_NONE = 0,      /* C = AB */
+  ENDIA_EPI_BIAS = 1,      /* C = AB + bias[n]                       (x @ W + b, _mlp.mojo:50) */
+  ENDIA_EPI_BIAS_ACT = 2,  /* Z = AB + bias[n]; aux_out = Z if non-null; C = act(Z)   (_mlp.mojo:50-52) */
+  ENDIA_EPI_ACT_GRAD = 3   /* C = (AB) * act'(aux_in)  -- activation VJP fused into dX = dZ W^T.
+                              aux_in is the PRE-activation Z unless ENDIA_ACT_FROM_OUTPUT is or'ed into
+                              `act`, in which case it is the stored activation output A = act(Z)
+                              (valid for relu and tanh only). */
+} endia_hip_epilogue;
+#define ENDIA_ACT_FROM_OUTPUT 0x100
+#define ENDIA_GEMM_ACCUMULATE 0x200 /* or'ed into `epilogue`: C += result instead of C = result */
+
+typedef enum { ENDIA_CGEMM_4M = 0, ENDIA_CGEMM_3M = 1 } endia_hip_cgemm_algo;
+
+/* ---- context ------------------------------------------------------------------------------- */
+/* No counterpart in the reference (it has no device); creates the stream and buffer pool. */
+ENDIA_API int32_t endia_hip_init(int32_t device);
+ENDIA_API int32_t endia_hip_shutdown(void);
+ENDIA_API const char* endia_hip_last_error(void);
+ENDIA_API int32_t endia_hip_sync(void);
+/* Writes a short description of the device ("gfx950 ... CUs ... MHz") into buf. */
+ENDIA_API int32_t endia_hip_device_info(char* buf, int64_t buf_bytes, int32_t* cu_count, int32_t* clock_mhz);
+
+/* ---- memory: replaces Node buffer allocation, setup_shape_and_data (functional/_utils.mojo:319-327)
+ *      and Node.__del__ (_array.mojo:177-179). Buffers come from a size-bucketed pool, so a freed
+ *      buffer is reused by later calls without hipMalloc. malloc does NOT zero the buffer. */
+ENDIA_API int32_t endia_hip_malloc(int64_t bytes, void** out);
+ENDIA_API int32_t endia_hip_free(void* p);
+ENDIA_API int32_t endia_hip_memcpy_h2d(void* dst, const void* src, int64_t bytes);
+ENDIA_API int32_t endia_hip_memcpy_d2h(void* dst, const void* src, int64_t bytes); /* blocks */
+ENDIA_API int32_t endia_hip_memcpy_d2d(void* dst, const void* src, int64_t bytes);
+ENDIA_API int32_t endia_hip_memset0(void* p, int64_t bytes);
+ENDIA_API int32_t endia_hip_fill(float* p, int64_t n, float value); /* init_ops.mojo full/ones/zeros */
+ENDIA_API int32_t endia_hip_pool_stats(int64_t* bytes_in_use, int64_t* bytes_cached, int64_t* n_device_allocs);
+ENDIA_API int32_t endia_hip_pool_trim(void);
+
+/* ---- timing on the library's stream (hipEvent pairs); slots 0..63 ---------------------------- */
+ENDIA_API int32_t endia_hip_timer_start(int32_t slot);
+ENDIA_API int32_t endia_hip_timer_stop(int32_t slot);
+ENDIA_API int32_t endia_hip_timer_elapsed_ms(int32_t slot, float* ms); /* blocks until the stop event */
+
+/* ---- strided gather copy: execute_copy_raw / contiguous (functional/_utils.mojo:79-205).
+ *      dst is contiguous row-major of `shape`; src element (i0..i_{r-1}) is at
+ *      src[offset + sum i_d*stride_d]; stride 0 broadcasts. ndim <= 8. is_complex copies pairs. */
+ENDIA_API int32_t endia_hip_strided_copy(int32_t ndim, const int64_t* shape, const int64_t* src_strides,
+                               int64_t src_offset, const float* src, float* dst, int32_t is_complex);
+
+/* ---- fp32 GEMM: matmul_fwd (binary_ops/matmul_op.mojo:93-254) and both products of matmul_vjp
+ *      (matmul_op.mojo:278-283). C[b] = opA(A[b]) . opB(B[b]), C is M x N with row stride ldc.
+ *      transA = 0: A is M x K, element (m,k) at A[m*lda + k];  transA = 1: A is stored K x M, element
+ *      (m,k) at A[k*lda + m]. Same for B (K x N, or stored N x K when transB = 1). The transposed
+ *      forms replace the reference's materialised .T() copies (matmul_op.mojo:111-136).
+ *      batch >= 1; a batch stride of 0 broadcasts that operand (matmul_op.mojo:162-165).
+ *      epilogue: endia_hip_epilogue, optionally | ENDIA_GEMM_ACCUMULATE.
+ *      act: endia_hip_unary_op in {RELU,TANH,SIN,IDENTITY}, optionally | ENDIA_ACT_FROM_OUTPUT.
+ *      bias: N floats (BIAS, BIAS_ACT) else null.  aux_in: M x N, row stride ldc (ACT_GRAD) else null.
+ *      aux_out: M x N, row stride ldc, or null (BIAS_ACT only). */
+ENDIA_API int32_t endia_hip_sgemm(int32_t transA, int32_t transB, int64_t M, int64_t N, int64_t K,
+                        const float* A, int64_t lda, const float* B, int64_t ldb, float* C, int64_t ldc,
+                        int64_t batch, int64_t strideA, int64_t strideB, int64_t strideC,
+                        int32_t epilogue, int32_t act, const float* bias, const float* aux_in,
+                        float* aux_out);
+
+/* ---- complex64 GEMM: the complex branch of matmul_fwd (matmul_op.mojo:201-238). Interleaved
+ *      operands; lda/ldb/ldc and strides count complex elements. conjA/conjB conjugate the operand
+ *      (the reference's VJP does not conjugate, matmul_op.mojo:278-283; the Wirtinger convention does).
+ *      algo 4M forms the four real products of matmul_op.mojo:216-217; 3M uses three. */
+ENDIA_API int32_t endia_hip_cgemm(int32_t transA, int32_t conjA, int32_t transB, int32_t conjB, int64_t M,
+                        int64_t N, int64_t K, const float* A, int64_t lda, const float* B, int64_t ldb,
+                        float* C, int64_t ldc, int64_t batch, int64_t strideA, int64_t strideB,
+                        int64_t strideC, int32_t algo, int32_t accumulate);
+
+/* ---- elementwise: execute_unary_op (unary_ops/_utils.mojo:77-134) and the VJP rules listed at
+ *      endia_hip_unary_op. n counts elements (complex: complex elements). In-place (y == x) allowed.
+ *      Complex forward is implemented for NEG, SQUARE, IDENTITY; ABS with is_complex writes n REAL
+ *      values |z| (abs_op.mojo:114-115,157). */
+ENDIA_API int32_t endia_hip_unary_fwd(int32_t op, int64_t n, const float* x, float* y, int32_t is_complex);
+/* dx = g * op'(x). For ABS with is_complex: g is real (n floats), x and dx complex: dx = g*z/|z|. */
+ENDIA_API int32_t endia_hip_unary_vjp(int32_t op, int64_t n, const float* x, const float* g, float* dx,
+                            int32_t is_complex);
+
+/* ---- broadcasting binary op: binary_op_array + execute_binary_op (binary_ops/_utils.mojo:57-177).
+ *      out is contiguous row-major of `shape`; a and b are addressed through element strides
+ *      (0 = broadcast axis) so the reference's materialised expand copies are never made. ndim <= 8. */
+ENDIA_API int32_t endia_hip_binary(int32_t op, int32_t ndim, const int64_t* shape, const int64_t* a_strides,
+                         const int64_t* b_strides, const float* a, const float* b, float* out,
+                         int32_t is_complex);
+/* out[i] = alpha * a[i] + beta * b[i]  (gradient accumulation `add`, autograd/functional.mojo:55-57,
+ * and scalar scaling such as Div by a full([1], n) operand, _array.mojo:1041-1043). b may be null. */
+ENDIA_API int32_t endia_hip_axpby(int64_t n, float alpha, const float* a, float beta, const float* b, float* out);
+
+/* ---- reductions: ReduceAdd.__call__ (reduce_ops/reduce_add_op.mojo:65-210) -- also Expand.vjp, the
+ *      bias gradient (view_ops/expand_op.mojo:121-126) -- and sum / mean (sum_op.mojo:35-62,
+ *      mean_op.mojo:35-65). x is contiguous row-major of `shape`; axes with reduce_mask bit d set are
+ *      summed and kept as size 1; out is contiguous of the reduced shape. scale multiplies the result
+ *      (1/count for mean). ndim <= 8. is_complex reduces pairs. */
+ENDIA_API int32_t endia_hip_reduce_add(int32_t ndim, const int64_t* shape, uint32_t reduce_mask, const float* x,
+                             float* out, float scale, int32_t is_complex);
+
+/* ---- loss: mse (loss_ops/mse_op.mojo:17-20) and its gradient 2(p-t)/n as produced by the
+ *      sub/mul/sum/div VJP chain. loss is one device float; dpred may be null (forward only);
+ *      loss may be null (gradient only). */
+ENDIA_API int32_t endia_hip_mse_fwd_bwd(int64_t n, const float* pred, const float* target, float* loss,
+                              float* dpred);
+
+/* ---- conv2d, NCHW, groups = 1: Conv2d.__call__ (spacial_ops/conv2d_op.mojo:88-196), output shape
+ *      rule conv2d_op.mojo:31-85. The three gradients have no counterpart in the reference, whose
+ *      Conv2d.vjp is default_vjp (conv2d_op.mojo:198-200); they are the adjoints of that forward loop.
+ *      x [N,C,H,W], w [K,C,R,S], bias [K] or null, y/dy [N,K,P,Q]. */
+typedef struct {
+  int64_t N, C, H, W, K, R, S;
+  int64_t stride_h, stride_w, pad_h, pad_w, dil_h, dil_w, groups;
+} endia_hip_conv2d_desc;
+ENDIA_API int32_t endia_hip_conv2d_out_shape(const endia_hip_conv2d_desc* d, int64_t* P, int64_t* Q);
+/* act in {IDENTITY, RELU}: y = act(conv(x,w)+bias). */
+ENDIA_API int32_t endia_hip_conv2d_fwd(const endia_hip_conv2d_desc* d, const float* x, const float* w,
+                             const float* bias, float* y, int32_t act);
+ENDIA_API int32_t endia_hip_conv2d_bwd_data(const endia_hip_conv2d_desc* d, const float* dy, const float* w,
+                                  float* dx);
+ENDIA_API int32_t endia_hip_conv2d_bwd_weight(const endia_hip_conv2d_desc* d, const float* x, const float* dy,
+                                    float* dw);
+ENDIA_API int32_t endia_hip_conv2d_bwd_bias(const endia_hip_conv2d_desc* d, const float* dy, float* db);
+
+/* ---- optimizers: SGD.step plain path (optim/sgd.mojo:61-62) and Adam.step (optim/adam.mojo:47-65),
+ *      each as one pass over the parameter. t is Adam's fp32 step counter (starts at 1, adam.mojo:40). */
+ENDIA_API int32_t endia_hip_sgd_step(int64_t n, float* p, const float* g, float lr);
+ENDIA_API int32_t endia_hip_adam_step(int64_t n, float* p, const float* g, float* m, float* v, float lr,
+                            float beta1, float beta2, float eps, float t);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* ENDIA_HIP_H */
