@@ -1,0 +1,208 @@
+#!/usr/bin/env python3
+"""Benchmark of the dense-layer training step on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload wide_mlp|sine_mlp]
+
+Default workload (the one the headline metric is quoted on): 8 Linear layers 4096 -> 4096 with bias,
+tanh between, MSE against N(0,1) targets, batch 4096, Adam(lr 1e-3, betas 0.9/0.999, eps 1e-8),
+x ~ N(0,1), W ~ N(0, 1/4096), b ~ N(0, 1/4096); synthetic data, random-init weights. One step is
+forward + loss + backward + Adam + zero_grad, the loop of the reference's MLP benchmark
+(benchmarks/mlp_benchmarks/mlp_imp.mojo:47-75), with inputs resident in HBM before the timed region.
+
+Prints ONE JSON line. `value` is train steps/s. `roofline` describes the dominant kernel (the fp32 MFMA
+GEMM): algorithmic 2*M*N*K flops per launch over the average launch duration, measured with HIP event
+pairs around every GEMM launch inside the timed region, against the 157.3 TFLOP/s dense fp32 matrix
+peak. `cpu_baseline` times the single-threaded CPU restatement of the reference's algorithms
+(oracle/) on a bounded sample of the same workload and extrapolates to one step.
+"""
+import argparse
+import ctypes
+import json
+import os
+import sys
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+FP32_MFMA_PEAK_TFLOPS = 157.3
+HBM_PEAK_GBS = 8000.0
+
+
+def build_wide_mlp(nd, width=4096, layers=8, batch=4096, seed=2):
+    rng = np.random.default_rng(seed)
+    std = 1.0 / np.sqrt(width)
+    mlp = nd.nn.MLP([width] * (layers + 1), compute_backward=True, activation="tanh", fused=True)
+    for i in range(layers):
+        mlp.weights[i] = nd.array((rng.standard_normal((width, width)) * std).astype(np.float32), requires_grad=True)
+        mlp.biases[i] = nd.array((rng.standard_normal(width) * std).astype(np.float32), requires_grad=True)
+    x = nd.array(rng.standard_normal((batch, width)).astype(np.float32))
+    y = nd.array(rng.standard_normal((batch, width)).astype(np.float32))
+    opt = nd.optim.Adam(mlp.params(), lr=1e-3, beta1=0.9, beta2=0.999, eps=1e-8)
+    return mlp, opt, x, y
+
+
+def build_sine_mlp(nd, seed=0):
+    rng = np.random.default_rng(seed)
+    widths = [1, 32, 64, 128, 128, 128, 64, 32, 1]
+    mlp = nd.nn.MLP(widths, compute_backward=True, activation="relu", fused=True)
+    for i in range(8):
+        s = np.sqrt(2.0 / widths[i])
+        mlp.weights[i] = nd.array((rng.standard_normal((widths[i], widths[i + 1])) * s).astype(np.float32), requires_grad=True)
+        mlp.biases[i] = nd.array((rng.standard_normal(widths[i + 1]) * s).astype(np.float32), requires_grad=True)
+    xb = rng.uniform(0, 1, (128, 1)).astype(np.float32)
+    x, y = nd.array(xb), nd.array(np.sin(2 * np.pi * xb).astype(np.float32))
+    opt = nd.optim.SGD(mlp.params(), lr=1e-3)
+    return mlp, opt, x, y
+
+
+def train_step(nd, mlp, opt, x, y):
+    pred = mlp.forward(x)
+    loss = nd.mse(pred, y)
+    loss.backward()
+    opt.step()
+    loss.zero_grad()
+    return loss
+
+
+def cpu_baseline_wide(width=4096, layers=8, batch=4096, rows=None, target_seconds=15.0):
+    """Single-threaded ref-order restatement, timed on row slices of the real shapes and composed by op
+    count: one step = 8 NN + 7 NT + 8 TN GEMMs, 7 tanh forward + 7 tanh VJPs, 8 bias adds, 8 column sums,
+    1 MSE, Adam over 8 weight matrices (biases are 0.02 % of the work and are ignored)."""
+    from oracle import endia_ref as R
+    rng = np.random.default_rng(0)
+    t_all0 = time.perf_counter()
+    X = rng.standard_normal((batch, width)).astype(np.float32)
+    W = (rng.standard_normal((width, width)) / 64).astype(np.float32)
+    if rows is None:
+        # size the sample to about target_seconds of CPU work: a 64-row probe of the NN GEMM sets the rate
+        t0 = time.perf_counter()
+        R.matmul(X[:64], W)
+        per_row = (time.perf_counter() - t0) / 64
+        rows = int(target_seconds / (3.3 * per_row)) // 64 * 64
+        rows = max(64, min(rows, batch))
+    scale = batch / rows
+
+    def timed(fn):
+        t0 = time.perf_counter()
+        fn()
+        return time.perf_counter() - t0
+
+    t_nn = timed(lambda: R.matmul(X[:rows], W)) * scale              # Z = A W          (rows of the batch)
+    t_nt = timed(lambda: R.matmul(X[:rows], W.T)) * scale            # dA = dZ W^T
+    t_tn = timed(lambda: R.matmul(X[:, :rows].T, X)) * (width / rows)  # dW = A^T dZ    (rows of dW)
+    Z = X[:rows]
+    t_tanh = timed(lambda: R.unary("tanh", Z)) * scale
+    t_tanh_vjp = timed(lambda: R.unary_vjp("tanh", Z, Z)) * scale
+    t_bias = timed(lambda: R.binary("add", Z, W[0])) * scale
+    t_col = timed(lambda: R.reduce_add(Z, [0])) * scale
+    t_mse = timed(lambda: R.mse(Z, Z)) * scale
+    Wp = W[:rows].copy()
+    t_adam = timed(lambda: R.adam(Wp, Wp, Wp, Wp)) * (width / rows)
+    step = (layers * t_nn + (layers - 1) * t_nt + layers * t_tn + (layers - 1) * (t_tanh + t_tanh_vjp) +
+            layers * (t_bias + t_col) + t_mse + layers * t_adam)
+    return {
+        "value": 1.0 / step, "unit": "steps/s", "cores": 1, "kind": "port",
+        "host_cores_available": os.cpu_count(),
+        "sample": "ref-order CPU restatement (oracle/endia_ref.c, 1 thread): %d-row slices of each of the three "
+                  "4096^3 GEMM modes and of each streaming op, extrapolated to full size and composed by op count "
+                  "(8 NN + 7 NT + 8 TN GEMMs, 14 tanh passes, 8 bias adds, 8 column sums, MSE, Adam); "
+                  "%.1f s of CPU work" % (rows, time.perf_counter() - t_all0),
+        "seconds_per_step": step,
+        "gemm_seconds_per_step": layers * t_nn + (layers - 1) * t_nt + layers * t_tn,
+    }
+
+
+def cpu_baseline_sine(steps=200):
+    from oracle import endia_ref as R
+    rng = np.random.default_rng(0)
+    widths = [1, 32, 64, 128, 128, 128, 64, 32, 1]
+    Ws = [(rng.standard_normal((widths[i], widths[i + 1])) * np.sqrt(2.0 / widths[i])).astype(np.float32) for i in range(8)]
+    bs = [(rng.standard_normal(widths[i + 1]) * np.sqrt(2.0 / widths[i])).astype(np.float32) for i in range(8)]
+    xb = rng.uniform(0, 1, (128, 1)).astype(np.float32)
+    yb = np.sin(2 * np.pi * xb).astype(np.float32)
+    R.mlp_step(widths, "relu", xb, yb, Ws, bs, opt="sgd", lr=1e-3)
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        R.mlp_step(widths, "relu", xb, yb, Ws, bs, opt="sgd", lr=1e-3)
+    dt = time.perf_counter() - t0
+    return {"value": steps / dt, "unit": "steps/s", "cores": 1, "kind": "port", "host_cores_available": os.cpu_count(),
+            "sample": "%d full fwd+bwd+SGD steps of the ref-order CPU restatement, 1 thread" % steps}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--workload", default="wide_mlp", choices=["wide_mlp", "sine_mlp"])
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py: this build runs on ONE GPU (no collectives, no sharding); --gpus %d is not supported. "
+                 "`value` is one GPU's throughput." % args.gpus)
+
+    import endia_amd as nd
+    from endia_amd import _lib as L
+    L.ensure_init(0)
+    dev_name, cus, mhz = L.device_info()
+
+    if args.workload == "wide_mlp":
+        mlp, opt, x, y = build_wide_mlp(nd)
+        width, layers, batch = 4096, 8, 4096
+        gemm_flops_step = (layers + layers + layers - 1) * 2.0 * batch * width * width
+        config = {"workload": "wide_mlp: 8 x Linear(4096->4096)+bias, tanh, MSE, Adam, batch 4096, fp32",
+                  "batch": batch, "width": width, "layers": layers, "optimizer": "adam"}
+    else:
+        mlp, opt, x, y = build_sine_mlp(nd)
+        w = [1, 32, 64, 128, 128, 128, 64, 32, 1]
+        kn = sum(w[i] * w[i + 1] for i in range(8))
+        gemm_flops_step = 2.0 * 128 * (3 * kn - w[0] * w[1])
+        config = {"workload": "sine_mlp: widths 1-32-64-128-128-128-64-32-1, relu, MSE, SGD 1e-3, batch 128, fp32",
+                  "batch": 128, "optimizer": "sgd"}
+
+    for _ in range(args.warmup):
+        train_step(nd, mlp, opt, x, y)
+    nd.synchronize()
+
+    L.call("endia_hip_gemm_timing_begin")
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        loss = train_step(nd, mlp, opt, x, y)
+    nd.synchronize()
+    elapsed = time.perf_counter() - t0
+    launches, g_ms, g_flops = ctypes.c_int64(), ctypes.c_double(), ctypes.c_double()
+    L.call("endia_hip_gemm_timing_end", ctypes.byref(launches), ctypes.byref(g_ms), ctypes.byref(g_flops))
+    final_loss = float(loss.item())
+
+    ms_per_step = 1e3 * elapsed / args.steps
+    steps_per_s = args.steps / elapsed
+    out = {
+        "metric": "fwd+bwd train steps/s + MFMA util %, 8-layer 4096-wide fp32 MLP, batch 4096"
+                  if args.workload == "wide_mlp" else "fwd+bwd+SGD train steps/s, sine-fit MLP",
+        "value": steps_per_s, "unit": "steps/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": ms_per_step, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "f32", "data": "synthetic", "config": config,
+        "device": dev_name, "final_loss": final_loss,
+        "gemm_tflops_whole_step": gemm_flops_step / (ms_per_step * 1e-3) / 1e12,
+    }
+    if launches.value:
+        avg_ms = g_ms.value / launches.value
+        flops_per_launch = g_flops.value / launches.value
+        achieved = flops_per_launch / (avg_ms * 1e-3) / 1e12
+        out["roofline"] = {
+            "bound": "mfma", "kernel": "sgemm_mfma_kernel (fp32 v_mfma_f32_32x32x2, 128x128x32 tiles)",
+            "achieved": achieved, "peak": FP32_MFMA_PEAK_TFLOPS, "unit": "TFLOP/s", "frac": achieved / FP32_MFMA_PEAK_TFLOPS,
+            "traffic": None, "launches": launches.value, "avg_launch_ms": avg_ms,
+            "flops_per_launch": flops_per_launch, "gemm_share_of_step": g_ms.value / (1e3 * elapsed),
+        }
+        out["mfma_util_pct"] = 100.0 * achieved / FP32_MFMA_PEAK_TFLOPS
+    if not args.no_cpu_baseline:
+        out["cpu_baseline"] = cpu_baseline_wide() if args.workload == "wide_mlp" else cpu_baseline_sine()
+    print(json.dumps(out))
+
+
+if __name__ == "__main__":
+    main()

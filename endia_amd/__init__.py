@@ -1,0 +1,26 @@
+"""endia_amd: Endia's reverse-mode training-step path on one AMD MI355X (gfx950).
+
+The public names mirror the reference's `endia` package (endia/__init__.mojo,
+endia/functional/__init__.mojo): `Array` / `Tensor` / `ndarray`, the functional ops, `backward` /
+`grad` / `jacobian` / `hessian` / `value_and_grad`, `nn.MLP`, `optim.SGD` / `optim.Adam`. All
+arithmetic runs in libendia_hip.so (hand-written HIP kernels behind the C ABI of
+include/endia_hip.h); importing this package without that library raises.
+"""
+from . import _lib
+
+_lib.lib()  # fail loudly when the HIP library has not been built
+
+from ._array import Array, Tensor, ndarray  # noqa: E402
+from .functional import (  # noqa: E402,F401
+    abs, add, arange, array, complex, conj, contiguous, conv2d, cos, detach, div, expand, eye, full, greater, imag,
+    linear, matmul, mean, mse, mul, neg, ones, permute, rand_he_normal, randn, randn_complex, randu, real, reduce_add,
+    relu, reshape, seed, set_complex_matmul_algorithm, sign, sin, sqrt, square, squeeze, sub, sum, tanh, unsqueeze,
+    zeros,
+)
+from .autograd.functional import backward, grad, hessian, jacobian, value_and_grad  # noqa: E402,F401
+from . import autograd, nn, optim, utils  # noqa: E402,F401
+
+
+def synchronize():
+    """Block until every kernel enqueued so far has finished."""
+    _lib.call("endia_hip_sync")

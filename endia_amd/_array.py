@@ -1,0 +1,276 @@
+"""Device-resident Array: the host-side mirror of endia/_array/_array.mojo.
+
+An Array is a handle on a node: a (possibly shared) device buffer, a shape / element-stride / offset
+triple, and the autograd fields of the reference's Node (`requires_grad`, the stored gradient, the
+argument list and the VJP rule: _array.mojo:55-179). Views (permute, expand, squeeze, reshape, real)
+share the buffer of their base, as in the reference. Storage is fp32, row-major; complex arrays are
+interleaved (re, im) pairs (_array.mojo:126,528-536) and `is_complex` arrays count COMPLEX elements in
+their shape and strides.
+
+All arithmetic happens in libendia_hip.so; numpy appears only where data crosses the host boundary.
+"""
+import ctypes
+
+import numpy as np
+
+from . import _lib as L
+
+
+class Buffer:
+    """One allocation from the library's pool; returned to the pool when the last view dies."""
+
+    __slots__ = ("ptr", "nbytes")
+
+    def __init__(self, nbytes):
+        p = ctypes.c_void_p()
+        L.call("endia_hip_malloc", int(nbytes), ctypes.byref(p))
+        self.ptr = p.value or 0
+        self.nbytes = int(nbytes)
+
+    def __del__(self):
+        if getattr(self, "ptr", 0):
+            try:
+                L.lib().endia_hip_free(ctypes.c_void_p(self.ptr))
+            except Exception:
+                pass
+            self.ptr = 0
+
+
+def contiguous_strides(shape):
+    st, acc = [], 1
+    for s in reversed(shape):
+        st.append(acc)
+        acc *= s
+    return tuple(reversed(st))
+
+
+def _prod(shape):
+    n = 1
+    for s in shape:
+        n *= int(s)
+    return n
+
+
+class Array:
+    """`Array(shape)` gives a zero-filled array like the reference's constructor (_array.mojo:198-214)."""
+
+    def __init__(self, shape=None, requires_grad=False, is_complex=False, _buffer=None, _strides=None, _offset=0,
+                 _zero=True):
+        if isinstance(shape, np.ndarray):
+            raise TypeError("use endia_amd.array(ndarray) / Array.from_numpy to upload host data")
+        if isinstance(shape, int):
+            shape = [shape]
+        shape = tuple(int(s) for s in (shape if shape is not None else (0,)))
+        self._shape = shape
+        self._strides = tuple(_strides) if _strides is not None else contiguous_strides(shape)
+        self._offset = int(_offset)
+        self.is_complex_ = bool(is_complex)
+        if _buffer is None:
+            n = _prod(shape) * (2 if is_complex else 1)
+            _buffer = Buffer(4 * n)
+            if _zero and n:
+                L.call("endia_hip_fill", _buffer.ptr, n, 0.0)
+        self._buf = _buffer
+        self._requires_grad = bool(requires_grad)
+        self._grad = None
+        self._args = []
+        self._vjp = None
+        self._name = "arg"
+        self._meta = None
+        self._id = -1
+        self._consumers = 0
+        self._is_seed = False
+        self._act_applied = False  # a gradient that already carries the producer's activation derivative
+
+    # ---- construction / host transfer ---------------------------------------------------------
+    @staticmethod
+    def empty(shape, is_complex=False):
+        return Array(shape, is_complex=is_complex, _zero=False)
+
+    @staticmethod
+    def from_numpy(a, requires_grad=False):
+        a = np.asarray(a)
+        cplx = np.iscomplexobj(a)
+        a = np.ascontiguousarray(a, dtype=np.complex64 if cplx else np.float32)
+        shape = a.shape if a.ndim else (1,)
+        out = Array(shape, requires_grad=requires_grad, is_complex=cplx, _zero=False)
+        if a.size:
+            L.call("endia_hip_memcpy_h2d", out._buf.ptr, a.ctypes.data, a.nbytes)
+        return out
+
+    def to_numpy(self):
+        c = self if self.is_contiguous() else _contiguous_copy(self)
+        out = np.empty(self._shape, dtype=np.complex64 if self.is_complex_ else np.float32)
+        if out.size:
+            L.call("endia_hip_memcpy_d2h", out.ctypes.data, c.data_ptr(), out.nbytes)
+        return out
+
+    # ---- shape queries (names follow the reference) ---------------------------------------------
+    def shape(self):
+        return list(self._shape)
+
+    def stride(self):
+        return list(self._strides)
+
+    def storage_offset(self):
+        return self._offset
+
+    def ndim(self):
+        return len(self._shape)
+
+    def size(self):
+        return _prod(self._shape)
+
+    def is_complex(self):
+        return self.is_complex_
+
+    def is_contiguous(self):
+        expect = 1
+        for s, st in zip(reversed(self._shape), reversed(self._strides)):
+            if s != 1 and st != expect:
+                return False
+            expect *= s
+        return True
+
+    def data_ptr(self):
+        """Device address of element 0 of this view."""
+        return self._buf.ptr + 4 * self._offset * (2 if self.is_complex_ else 1)
+
+    def load(self, i):
+        return self.to_numpy().reshape(-1)[i]
+
+    def item(self):
+        return self.to_numpy().reshape(-1)[0]
+
+    # ---- autograd fields ------------------------------------------------------------------------
+    def requires_grad(self):
+        return self._requires_grad
+
+    def requires_grad_(self, flag=True):
+        self._requires_grad = bool(flag)
+        return self
+
+    def has_grad(self):
+        return self._grad is not None
+
+    def grad_(self, g):
+        self._grad = g
+
+    def grad(self):
+        if self._grad is None:
+            return Array(self._shape, is_complex=self.is_complex_)
+        return self._grad
+
+    def remove_grad(self):
+        self._grad = None
+
+    def args(self):
+        return list(self._args)
+
+    def clear_args(self):
+        self._args = []
+        self._vjp = None
+
+    def name(self):
+        return self._name
+
+    def backward(self, create_graph=False):
+        from .autograd.functional import backward
+        backward(self, create_graph)
+
+    def zero_grad(self):
+        from .autograd.functional import zero_grad_rec
+        zero_grad_rec(self)
+
+    # ---- operators (endia/_array/_array.mojo:791-1099) ---------------------------------------------
+    def T(self):
+        from . import functional as F
+        if self.ndim() == 1:
+            return self
+        return F.permute(self, [-1, -2])
+
+    def reshape(self, shape):
+        from . import functional as F
+        return F.reshape(self, shape)
+
+    def _bin(self, other, fn, reverse=False):
+        from . import functional as F
+        if not isinstance(other, Array):
+            # scalars become a one-row `full` operand and broadcast (_array.mojo:1014-1016)
+            last = self._shape[-1] if self._shape else 1
+            other = F.full([last], float(other))
+        return fn(other, self) if reverse else fn(self, other)
+
+    def __add__(self, o):
+        from . import functional as F
+        return self._bin(o, F.add)
+
+    __radd__ = __add__
+
+    def __sub__(self, o):
+        from . import functional as F
+        return self._bin(o, F.sub)
+
+    def __rsub__(self, o):
+        from . import functional as F
+        return self._bin(o, F.sub, reverse=True)
+
+    def __mul__(self, o):
+        from . import functional as F
+        return self._bin(o, F.mul)
+
+    __rmul__ = __mul__
+
+    def __truediv__(self, o):
+        from . import functional as F
+        return self._bin(o, F.div)
+
+    def __rtruediv__(self, o):
+        from . import functional as F
+        return self._bin(o, F.div, reverse=True)
+
+    def __matmul__(self, o):
+        from . import functional as F
+        return F.matmul(self, o)
+
+    def __neg__(self):
+        from . import functional as F
+        return F.neg(self)
+
+    def __pow__(self, p):
+        from . import functional as F
+        return F.pow_int(self, p)
+
+    # in-place updates write through to the existing buffer (execute_copy_raw, _array.mojo:998-1006)
+    def _assign_from(self, other):
+        assert other.size() == self.size() and other.is_complex_ == self.is_complex_
+        src = other if other.is_contiguous() else _contiguous_copy(other)
+        assert self.is_contiguous()
+        L.call("endia_hip_memcpy_d2d", self.data_ptr(), src.data_ptr(), 4 * self.size() * (2 if self.is_complex_ else 1))
+
+    def __isub__(self, o):
+        self._assign_from(self - o)
+        return self
+
+    def __iadd__(self, o):
+        self._assign_from(self + o)
+        return self
+
+    def __repr__(self):
+        return "Array(shape=%s%s, requires_grad=%s)" % (list(self._shape), ", complex" if self.is_complex_ else "",
+                                                        self._requires_grad)
+
+    def __str__(self):
+        return str(self.to_numpy())
+
+
+def _contiguous_copy(x):
+    out = Array.empty(x._shape, x.is_complex_)
+    if x.size():
+        L.call("endia_hip_strided_copy", x.ndim(), L.i64_array(x._shape), L.i64_array(x._strides), x._offset,
+               x._buf.ptr, out._buf.ptr, 1 if x.is_complex_ else 0)
+    return out
+
+
+Tensor = Array
+ndarray = Array

@@ -6,7 +6,7 @@ exported symbols); `ensure_init()` additionally creates the device context.
 """
 import ctypes
 import os
-from ctypes import POINTER, c_char_p, c_float, c_int32, c_int64, c_uint32, c_void_p
+from ctypes import POINTER, c_char_p, c_double, c_float, c_int32, c_int64, c_uint32, c_void_p
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libendia_hip.so")
@@ -54,6 +54,8 @@ SIGNATURES = {
     "endia_hip_timer_start": [c_int32],
     "endia_hip_timer_stop": [c_int32],
     "endia_hip_timer_elapsed_ms": [c_int32, POINTER(c_float)],
+    "endia_hip_gemm_timing_begin": [],
+    "endia_hip_gemm_timing_end": [_i64p, POINTER(c_double), POINTER(c_double)],
     "endia_hip_strided_copy": [c_int32, _i64p, _i64p, c_int64, _fp, _fp, c_int32],
     "endia_hip_sgemm": [c_int32, c_int32, c_int64, c_int64, c_int64, _fp, c_int64, _fp, c_int64, _fp, c_int64,
                         c_int64, c_int64, c_int64, c_int64, c_int32, c_int32, _fp, _fp, _fp],
@@ -61,8 +63,10 @@ SIGNATURES = {
                         _fp, c_int64, c_int64, c_int64, c_int64, c_int64, c_int32, c_int32],
     "endia_hip_unary_fwd": [c_int32, c_int64, _fp, _fp, c_int32],
     "endia_hip_unary_vjp": [c_int32, c_int64, _fp, _fp, _fp, c_int32],
+    "endia_hip_unary_vjp_from_output": [c_int32, c_int64, _fp, _fp, _fp],
     "endia_hip_binary": [c_int32, c_int32, _i64p, _i64p, _i64p, _fp, _fp, _fp, c_int32],
     "endia_hip_axpby": [c_int64, c_float, _fp, c_float, _fp, _fp],
+    "endia_hip_complex_pack": [c_int64, _fp, _fp, _fp],
     "endia_hip_reduce_add": [c_int32, _i64p, c_uint32, _fp, _fp, c_float, c_int32],
     "endia_hip_mse_fwd_bwd": [c_int64, _fp, _fp, _fp, _fp],
     "endia_hip_conv2d_out_shape": [POINTER(Conv2dDesc), _i64p, _i64p],
@@ -84,7 +88,7 @@ def lib():
     if _lib is None:
         if not os.path.exists(LIB_PATH):
             raise ImportError(
-                "%s is missing: build it with `python -m endia_amd.build` (there is no CPU fallback)" % LIB_PATH)
+                "%s is missing: build it with `python endia_amd/csrc/build.py` (there is no CPU fallback)" % LIB_PATH)
         handle = ctypes.CDLL(LIB_PATH)
         for name, argtypes in SIGNATURES.items():
             fn = getattr(handle, name)

@@ -1,0 +1,187 @@
+"""Reverse-mode driver: the host-side mirror of endia/autograd/functional.mojo.
+
+`jacrev` follows the reference's walk (functional.mojo:26-67): depth-first post-order over the
+argument lists (endia/utils/general.mojo:18-32), a seed of ones(1) for a scalar output or an identity
+Jacobian seed otherwise (:34-38), then the trace in reverse, calling each node's VJP rule and
+accumulating with an `add` op where a tensor has several consumers (:51-57). Unless
+`create_graph=True`, every stored gradient is cut from the graph that produced it (:63-65).
+
+The functional wrappers (grad / jacobian / hessian / value_and_grad over a Python callable) follow the
+non-JIT branch of Callable.__call__ (endia/compile/callable.mojo:100-197): repeated
+backward(create_graph=True) passes, then detached copies of the results.
+"""
+from .. import functional as F
+from .._array import Array
+
+_building_graph = [False]
+
+
+def building_graph():
+    """True while a backward pass runs with create_graph=True. Fused ops consult it to pick between
+    their single-kernel first-order rule and a rule rebuilt from differentiable ops."""
+    return _building_graph[0]
+
+
+def top_order(out):
+    """Post-order DFS over args (general.mojo:26-32), iterative so deep graphs do not hit the
+    interpreter's recursion limit."""
+    trace, seen = [], set()
+    stack = [(out, 0)]
+    seen.add(id(out))
+    while stack:
+        node, i = stack[-1]
+        if i < len(node._args):
+            stack[-1] = (node, i + 1)
+            child = node._args[i]
+            if id(child) not in seen:
+                seen.add(id(child))
+                stack.append((child, 0))
+        else:
+            stack.pop()
+            trace.append(node)
+    return trace
+
+
+def backward(arg, create_graph=False):
+    jacrev(arg, create_graph)
+
+
+def jacrev(arg, create_graph=False):
+    out = arg
+    trace = top_order(out)
+    for node in trace:
+        node._consumers = 0
+    for node in trace:
+        for a in node._args:
+            a._consumers += 1
+
+    dims = out._shape[-1] if out._shape else 1
+    if out.ndim() != 1 or dims != 1:
+        n = out.size()
+        seed = F.reshape(F.eye(n), out.shape() + out.shape())
+    else:
+        seed = F.ones([dims])
+        seed._is_seed = True
+    out.grad_(seed)
+
+    prev = _building_graph[0]
+    _building_graph[0] = bool(create_graph)
+    try:
+        for curr in reversed(trace):
+            primals = curr._args
+            if not primals or curr._vjp is None:
+                continue
+            grad = curr.grad()
+            primals_grads = curr._vjp(primals, grad, curr)
+            for primal, pg in zip(primals, primals_grads):
+                if not primal._requires_grad or pg is None:
+                    continue
+                if primal.has_grad():
+                    if pg._act_applied or primal._grad._act_applied:
+                        raise RuntimeError("internal: a fused activation gradient met an accumulated gradient")
+                    pg = F.add(pg, primal._grad)
+                primal.grad_(pg)
+                if not create_graph:
+                    pg.clear_args()
+    finally:
+        _building_graph[0] = prev
+
+
+def _visit_all(out, fn):
+    for node in top_order(out):
+        fn(node)
+
+
+def zero_grad_rec(out):
+    """Array.zero_grad: drop the gradient of every node reachable from `out` (general.mojo:35-47)."""
+    _visit_all(out, lambda n: n.remove_grad())
+
+
+remove_grad_rec = zero_grad_rec
+
+
+def grad(outs=None, inputs=None, retain_grads=True, create_graph=False, argnums=None):
+    """Two forms, as in the reference:
+
+    grad(outs=[...], inputs=[...]) -> list of gradients (functional.mojo:70-97);
+    grad(f, argnums=...)           -> Callable computing the gradient of f (functional.mojo:100-128).
+    """
+    if isinstance(outs, Callable):
+        f = outs
+        return Callable(f.func, f.argnums + [argnums if argnums is not None else [-1]], f.order + 1, False)
+    if callable(outs) and not isinstance(outs, Array):
+        return Callable(outs, [argnums if argnums is not None else [-1]], 1, False)
+    single = isinstance(inputs, Array)
+    outs = [outs] if isinstance(outs, Array) else list(outs)
+    inputs = [inputs] if single else list(inputs)
+    for o in outs:
+        remove_grad_rec(o)
+    for i in inputs:
+        remove_grad_rec(i)
+    for o in outs:
+        o.backward(create_graph=create_graph)
+    res = []
+    for i in inputs:
+        g = i.grad()
+        if not create_graph:
+            g.clear_args()
+            g.remove_grad()
+        if not retain_grads:
+            i.remove_grad()
+        res.append(g)
+    return res
+
+
+class Callable:
+    """grad(f) / jacobian(f) / hessian(f): endia/compile/callable.mojo:60-197, non-JIT branch."""
+
+    def __init__(self, func, argnums, order, keep_outs):
+        self.func = func
+        self.argnums = [list(a) if isinstance(a, (list, tuple)) else [a] for a in argnums]
+        self.order = order
+        self.keep_outs = keep_outs
+
+    def __call__(self, *args):
+        single = len(args) == 1 and isinstance(args[0], Array)
+        arrs = list(args[0]) if (len(args) == 1 and not single) else list(args)
+        # fresh leaves, so that repeated calls never see stale graphs (callable.mojo:100-112)
+        leaves = [F.detach(a) for a in arrs]
+        chosen = self.argnums[0]
+        idx = list(range(len(leaves))) if chosen == [-1] else chosen
+        for i in idx:
+            leaves[i].requires_grad_(True)
+        res = self.func(leaves[0]) if single else self.func(leaves)
+        outs = [res]
+        value = res
+        for o in range(self.order):
+            nxt = []
+            last = o == self.order - 1
+            for arr in outs:
+                remove_grad_rec(arr)
+                arr.backward(create_graph=not last)
+                for i in idx:
+                    nxt.append(leaves[i].grad())
+                for i in idx:
+                    leaves[i].remove_grad()
+            outs = nxt
+        # detach by copy (callable.mojo:165-176)
+        final = [F.array(g.to_numpy()) for g in outs]
+        if self.keep_outs:
+            final = [F.array(value.to_numpy())] + final
+        if len(final) == 1:
+            return final[0]
+        return final
+
+
+def jacobian(f, argnums=None):
+    return grad(f, argnums=argnums)
+
+
+def hessian(f, argnums=None):
+    return grad(grad(f, argnums=argnums), argnums=argnums)
+
+
+def value_and_grad(f, argnums=None):
+    if isinstance(f, Callable):
+        return Callable(f.func, f.argnums + [argnums if argnums is not None else [-1]], f.order + 1, True)
+    return Callable(f, [argnums if argnums is not None else [-1]], 1, True)

@@ -1,6 +1,9 @@
 """Build libendia_hip.so (gfx950 only) in-tree with hipcc.
 
-    python -m endia_amd.build            # compile every csrc/*.hip, link endia_amd/libendia_hip.so
+    python endia_amd/csrc/build.py       # compile every csrc/*.hip, link endia_amd/libendia_hip.so
+
+It is run as a script (or loaded by path), never through `import endia_amd`, because importing the
+package requires the library this script produces.
 
 The library has no dependency beyond the HIP runtime; nothing here needs a GPU.
 """
@@ -9,10 +12,9 @@ import os
 import subprocess
 import sys
 
-HERE = os.path.dirname(os.path.abspath(__file__))
-CSRC = os.path.join(HERE, "csrc")
-OBJ_DIR = os.path.join(HERE, "csrc", "build")
-LIB_PATH = os.path.join(HERE, "libendia_hip.so")
+CSRC = os.path.dirname(os.path.abspath(__file__))
+OBJ_DIR = os.path.join(CSRC, "build")
+LIB_PATH = os.path.join(os.path.dirname(CSRC), "libendia_hip.so")
 
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 # packed fp32 instructions are switched off for every device translation unit

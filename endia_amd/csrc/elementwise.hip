@@ -112,6 +112,23 @@ __global__ __launch_bounds__(TPB) void unary_vjp_kernel(const float* __restrict_
   }
 }
 
+__global__ __launch_bounds__(TPB) void vjp_from_output_kernel(int op, const float* __restrict__ y,
+                                                              const float* __restrict__ g, float* __restrict__ dx,
+                                                              int64_t n) {
+  int64_t stride = (int64_t)gridDim.x * TPB;
+  for (int64_t j = (int64_t)blockIdx.x * TPB + threadIdx.x; j < n; j += stride) {
+    float a = y[j], c = g[j];
+    float r;
+    switch (op) {
+      case ENDIA_OP_RELU: r = a > 0.f ? c : 0.f; break;
+      case ENDIA_OP_TANH: r = (1.f - a * a) * c; break;
+      case ENDIA_OP_SQRT: r = c / (2.f * a); break;
+      default: r = c; break;
+    }
+    dx[j] = r;
+  }
+}
+
 // complex forward: one complex element (8 bytes) per lane access
 __global__ __launch_bounds__(TPB) void unary_fwd_complex_kernel(int op, const float2* __restrict__ x,
                                                                 float* __restrict__ y, int64_t n) {
@@ -270,6 +287,13 @@ __global__ __launch_bounds__(TPB) void axpby_kernel(int64_t n, float alpha, cons
   }
 }
 
+__global__ __launch_bounds__(TPB) void complex_pack_kernel(int64_t n, const float* __restrict__ re,
+                                                           const float* __restrict__ im, float2* __restrict__ out) {
+  int64_t stride = (int64_t)gridDim.x * TPB;
+  for (int64_t j = (int64_t)blockIdx.x * TPB + threadIdx.x; j < n; j += stride)
+    out[j] = make_float2(re[j], im ? im[j] : 0.f);
+}
+
 // ---- strided gather copy ---------------------------------------------------------------------
 struct CopyDesc {
   int ndim;
@@ -419,6 +443,18 @@ int32_t endia_hip_unary_vjp(int32_t op, int64_t n, const float* x, const float* 
   return ENDIA_HIP_OK;
 }
 
+int32_t endia_hip_unary_vjp_from_output(int32_t op, int64_t n, const float* y, const float* g, float* dx) {
+  ENDIA_REQUIRE_INIT();
+  ENDIA_CHECK_ARG(n >= 0, "endia_hip_unary_vjp_from_output: negative n");
+  ENDIA_CHECK_ARG(op == ENDIA_OP_RELU || op == ENDIA_OP_TANH || op == ENDIA_OP_SQRT || op == ENDIA_OP_IDENTITY,
+                  "endia_hip_unary_vjp_from_output: op %d cannot be differentiated from its output", op);
+  if (n == 0) return ENDIA_HIP_OK;
+  ENDIA_CHECK_ARG(y && g && dx, "endia_hip_unary_vjp_from_output: null pointer");
+  hipLaunchKernelGGL(vjp_from_output_kernel, dim3(stream_grid(n)), dim3(TPB), 0, ctx().stream, op, y, g, dx, n);
+  ENDIA_LAUNCH_CHECK();
+  return ENDIA_HIP_OK;
+}
+
 int32_t endia_hip_binary(int32_t op, int32_t ndim, const int64_t* shape, const int64_t* a_strides,
                          const int64_t* b_strides, const float* a, const float* b, float* out, int32_t is_complex) {
   ENDIA_REQUIRE_INIT();
@@ -494,6 +530,17 @@ int32_t endia_hip_axpby(int64_t n, float alpha, const float* a, float beta, cons
   int vec = al16(a) && al16(out) && (!b || al16(b));
   hipLaunchKernelGGL(axpby_kernel, dim3(stream_grid(vec ? (n + 3) / 4 : n)), dim3(TPB), 0, ctx().stream, n, alpha, a,
                      beta, b, out, vec);
+  ENDIA_LAUNCH_CHECK();
+  return ENDIA_HIP_OK;
+}
+
+int32_t endia_hip_complex_pack(int64_t n, const float* re, const float* im, float* out) {
+  ENDIA_REQUIRE_INIT();
+  ENDIA_CHECK_ARG(n >= 0, "endia_hip_complex_pack: negative n");
+  if (n == 0) return ENDIA_HIP_OK;
+  ENDIA_CHECK_ARG(re && out, "endia_hip_complex_pack: null pointer");
+  hipLaunchKernelGGL(complex_pack_kernel, dim3(stream_grid(n)), dim3(TPB), 0, ctx().stream, n, re, im,
+                     reinterpret_cast<float2*>(out));
   ENDIA_LAUNCH_CHECK();
   return ENDIA_HIP_OK;
 }

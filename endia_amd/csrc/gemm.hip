@@ -20,6 +20,8 @@
 // operands use the same mapping.
 #include "common.h"
 
+#include <vector>
+
 typedef float floatx16 __attribute__((ext_vector_type(16)));
 
 namespace {
@@ -311,6 +313,17 @@ inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 
 
 }  // namespace
 
+namespace {
+// per-launch event pairs for endia_hip_gemm_timing_*
+struct GemmTiming {
+  bool on = false;
+  std::vector<hipEvent_t> start, stop;
+  size_t used = 0;
+  double flops = 0.0;
+};
+GemmTiming g_timing;
+}  // namespace
+
 namespace endia {
 
 // Shared by endia_hip_sgemm and the complex and convolution front ends.
@@ -358,11 +371,27 @@ int32_t sgemm_impl(int transA, int transB, int64_t M, int64_t N, int64_t K, cons
     p.tiles_m = (int)ceil_div64(M, BM);
     p.tiles_n = (int)ceil_div64(N, BN);
     dim3 grid((unsigned)(p.tiles_m * p.tiles_n), (unsigned)batch);
+    const bool timed = g_timing.on;
+    if (timed) {
+      if (g_timing.used == g_timing.start.size()) {
+        hipEvent_t a, b;
+        ENDIA_HIP_CALL(hipEventCreate(&a));
+        ENDIA_HIP_CALL(hipEventCreate(&b));
+        g_timing.start.push_back(a);
+        g_timing.stop.push_back(b);
+      }
+      ENDIA_HIP_CALL(hipEventRecord(g_timing.start[g_timing.used], s));
+    }
     switch (epi) {
       case ENDIA_EPI_NONE: launch_mfma<ENDIA_EPI_NONE>(p, transA, transB, grid, s); break;
       case ENDIA_EPI_BIAS: launch_mfma<ENDIA_EPI_BIAS>(p, transA, transB, grid, s); break;
       case ENDIA_EPI_BIAS_ACT: launch_mfma<ENDIA_EPI_BIAS_ACT>(p, transA, transB, grid, s); break;
       default: launch_mfma<ENDIA_EPI_ACT_GRAD>(p, transA, transB, grid, s); break;
+    }
+    if (timed) {
+      ENDIA_HIP_CALL(hipEventRecord(g_timing.stop[g_timing.used], s));
+      g_timing.used++;
+      g_timing.flops += 2.0 * (double)M * (double)N * (double)K * (double)batch;
     }
   } else {
     p.tiles_m = (int)ceil_div64(M, 64);
@@ -390,4 +419,28 @@ extern "C" int32_t endia_hip_sgemm(int32_t transA, int32_t transB, int64_t M, in
   ENDIA_REQUIRE_INIT();
   return endia::sgemm_impl(transA, transB, M, N, K, A, lda, B, ldb, C, ldc, batch, strideA, strideB,
                            strideC, epilogue, act, bias, aux_in, aux_out);
+}
+
+extern "C" int32_t endia_hip_gemm_timing_begin(void) {
+  ENDIA_REQUIRE_INIT();
+  g_timing.on = true;
+  g_timing.used = 0;
+  g_timing.flops = 0.0;
+  return ENDIA_HIP_OK;
+}
+
+extern "C" int32_t endia_hip_gemm_timing_end(int64_t* launches, double* total_ms, double* total_flops) {
+  ENDIA_REQUIRE_INIT();
+  g_timing.on = false;
+  ENDIA_HIP_CALL(hipStreamSynchronize(endia::ctx().stream));
+  double ms = 0.0;
+  for (size_t i = 0; i < g_timing.used; ++i) {
+    float t = 0.f;
+    ENDIA_HIP_CALL(hipEventElapsedTime(&t, g_timing.start[i], g_timing.stop[i]));
+    ms += t;
+  }
+  if (launches) *launches = (int64_t)g_timing.used;
+  if (total_ms) *total_ms = ms;
+  if (total_flops) *total_flops = g_timing.flops;
+  return ENDIA_HIP_OK;
 }

@@ -4,11 +4,13 @@
 // 12 bytes per parameter (read p, g; write p), Adam 28 (read p, g, m, v; write p, m, v).
 //
 // Every intermediate of the reference is an fp32 Array, so each arithmetic step rounds to fp32. The
-// kernels keep that: products and sums are written with the round-to-nearest intrinsics so the
-// compiler cannot contract them into fused multiply-adds.
+// kernels keep that: floating-point contraction is switched off for this file, so no product-sum
+// pair is fused into an fma and the results equal the reference's op-by-op arithmetic bit for bit.
 #include "common.h"
 
 #include <math.h>
+
+#pragma clang fp contract(off)
 
 namespace {
 
@@ -18,14 +20,26 @@ struct AdamK {
   float lr, b1, b2, eps, omb1, omb2, c1, c2;  // c1 = 1 - b1^t, c2 = 1 - b2^t
 };
 
+// Plain operators, not the __f*_rn helpers: those are inline functions of a header compiled with
+// contraction allowed, and would carry that permission into this file after inlining.
 __device__ __forceinline__ void adam_one(float& p, float g, float& m, float& v, const AdamK& k) {
-  m = __fadd_rn(__fmul_rn(k.b1, m), __fmul_rn(k.omb1, g));
-  v = __fadd_rn(__fmul_rn(k.b2, v), __fmul_rn(__fmul_rn(k.omb2, g), g));
-  float mh = __fdiv_rn(m, k.c1);
-  float vh = __fdiv_rn(v, k.c2);
+  float a = k.b1 * m, b = k.omb1 * g;
+  m = a + b;
+  float c = k.b2 * v, e = k.omb2 * g;
+  e = e * g;
+  v = c + e;
+  float mh = m / k.c1;
+  float vh = v / k.c2;
   // the reference's real sqrt is sqrt((|x|+x)/2) (sqrt_op.mojo:111-114): equal to sqrt(x) for x >= 0
-  float den = __fadd_rn(__fsqrt_rn(__fmul_rn(__fadd_rn(fabsf(vh), vh), 0.5f)), k.eps);
-  p = __fsub_rn(p, __fdiv_rn(__fmul_rn(k.lr, mh), den));
+  float r = (fabsf(vh) + vh) * 0.5f;
+  float den = __builtin_sqrtf(r) + k.eps;
+  float num = k.lr * mh;
+  p = p - num / den;
+}
+
+__device__ __forceinline__ float sgd_one(float p, float g, float lr) {
+  float u = lr * g;
+  return p - u;
 }
 
 __global__ __launch_bounds__(TPB) void adam_kernel(int64_t n, float* __restrict__ p, const float* __restrict__ g,
@@ -62,15 +76,15 @@ __global__ __launch_bounds__(TPB) void sgd_kernel(int64_t n, float* __restrict__
     const float4* g4 = reinterpret_cast<const float4*>(g);
     for (int64_t j = i; j < n4; j += stride) {
       float4 P = p4[j], G = g4[j];
-      P.x = __fsub_rn(P.x, __fmul_rn(lr, G.x));
-      P.y = __fsub_rn(P.y, __fmul_rn(lr, G.y));
-      P.z = __fsub_rn(P.z, __fmul_rn(lr, G.z));
-      P.w = __fsub_rn(P.w, __fmul_rn(lr, G.w));
+      P.x = sgd_one(P.x, G.x, lr);
+      P.y = sgd_one(P.y, G.y, lr);
+      P.z = sgd_one(P.z, G.z, lr);
+      P.w = sgd_one(P.w, G.w, lr);
       p4[j] = P;
     }
-    for (int64_t j = (n4 << 2) + i; j < n; j += stride) p[j] = __fsub_rn(p[j], __fmul_rn(lr, g[j]));
+    for (int64_t j = (n4 << 2) + i; j < n; j += stride) p[j] = sgd_one(p[j], g[j], lr);
   } else {
-    for (int64_t j = i; j < n; j += stride) p[j] = __fsub_rn(p[j], __fmul_rn(lr, g[j]));
+    for (int64_t j = i; j < n; j += stride) p[j] = sgd_one(p[j], g[j], lr);
   }
 }
 

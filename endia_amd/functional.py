@@ -1,0 +1,751 @@
+"""Functional ops: forward kernels and VJP rules, the host-side mirror of endia/functional/.
+
+Each op is registered the way the reference's `op_array` does it
+(endia/functional/_utils.mojo:208-316): the forward body runs eagerly, and when any argument
+requires a gradient the output keeps its arguments and its `vjp(primals, grad, out)` rule. VJP rules
+are written in terms of these same ops, so a gradient built with `create_graph=True` is itself a
+differentiable graph, which is the reference's whole higher-order mechanism
+(endia/autograd/functional.mojo:63-65). A primal that does not require a gradient gets `None`, the
+counterpart of the reference's `Array(0)` placeholder.
+
+Every forward body is one or two calls into libendia_hip.so.
+"""
+import numpy as np
+
+from . import _lib as L
+from ._array import Array, _contiguous_copy, _prod, contiguous_strides
+
+
+# --------------------------------------------------------------------------------------------------
+# registration
+# --------------------------------------------------------------------------------------------------
+def _register(out, args, name, vjp, meta=None):
+    out._name = name
+    if any(a._requires_grad for a in args):
+        out._requires_grad = True
+        out._args = list(args)
+        out._vjp = vjp
+        out._meta = meta
+    return out
+
+
+def _view(base, shape, strides, offset, args, name, vjp, meta=None, is_complex=None):
+    out = Array(shape, is_complex=base.is_complex_ if is_complex is None else is_complex, _buffer=base._buf,
+                _strides=strides, _offset=offset)
+    return _register(out, args, name, vjp, meta)
+
+
+def contiguous(x):
+    """contiguous(): functional/_utils.mojo:201-205 (a strided gather copy when x is a view)."""
+    return x if x.is_contiguous() else _contiguous_copy(x)
+
+
+def detach(x):
+    return Array(x._shape, is_complex=x.is_complex_, _buffer=x._buf, _strides=x._strides, _offset=x._offset)
+
+
+# --------------------------------------------------------------------------------------------------
+# creation (init_ops.mojo). Random data is generated on the host with a seeded numpy Generator: the
+# reference's generators are time-seeded (init_ops.mojo:230,260) and cannot be reproduced.
+# --------------------------------------------------------------------------------------------------
+_rng = np.random.default_rng(0)
+
+
+def seed(s):
+    global _rng
+    _rng = np.random.default_rng(s)
+
+
+def array(data, requires_grad=False):
+    return Array.from_numpy(np.asarray(data), requires_grad=requires_grad)
+
+
+def zeros(shape, requires_grad=False, is_complex=False):
+    return Array(shape, requires_grad=requires_grad, is_complex=is_complex)
+
+
+def full(shape, value, requires_grad=False):
+    out = Array.empty(shape)
+    L.call("endia_hip_fill", out.data_ptr(), out.size(), float(value))
+    out._requires_grad = requires_grad
+    return out
+
+
+def ones(shape, requires_grad=False):
+    return full(shape, 1.0, requires_grad)
+
+
+def eye(n, requires_grad=False):
+    return array(np.eye(n, dtype=np.float32), requires_grad)
+
+
+def arange(start, end, step=1.0, requires_grad=False):
+    return array(np.arange(start, end, step, dtype=np.float32), requires_grad)
+
+
+def randn(shape, mean=0.0, std=1.0, requires_grad=False):
+    return array((_rng.standard_normal(tuple(shape)) * std + mean).astype(np.float32), requires_grad)
+
+
+def randu(shape, min=0.0, max=1.0, requires_grad=False):
+    return array(_rng.uniform(min, max, tuple(shape)).astype(np.float32), requires_grad)
+
+
+def randn_complex(shape, requires_grad=False):
+    z = _rng.standard_normal(tuple(shape)) + 1j * _rng.standard_normal(tuple(shape))
+    return array(z.astype(np.complex64), requires_grad)
+
+
+def rand_he_normal(shape, fan_in, requires_grad=False):
+    """He-normal init, std = sqrt(2 / fan_in): init_ops.mojo:285-287."""
+    return randn(shape, 0.0, float(np.sqrt(2.0 / fan_in)), requires_grad)
+
+
+def complex(real, imag=None):
+    """complex(real, imag): init_ops.mojo:419-433."""
+    r = contiguous(real)
+    i = contiguous(imag) if imag is not None else None
+    out = Array.empty(r._shape, is_complex=True)
+    L.call("endia_hip_complex_pack", r.size(), r.data_ptr(), i.data_ptr() if i is not None else None, out.data_ptr())
+
+    def vjp(primals, grad, out_):
+        return [real_part(grad) if primals[0]._requires_grad else None] + (
+            [imag_part(grad) if primals[1]._requires_grad else None] if len(primals) > 1 else [])
+
+    return _register(out, [real] + ([imag] if imag is not None else []), "complex", vjp)
+
+
+# --------------------------------------------------------------------------------------------------
+# view ops (endia/functional/view_ops)
+# --------------------------------------------------------------------------------------------------
+def _norm_axes(axes, ndim):
+    return [a + ndim if a < 0 else a for a in axes]
+
+
+def expand(x, shape, ignore_axes=()):
+    """Broadcast view with stride 0 on expanded axes (expand_op.mojo:36-199). Its VJP is the sum over
+    those axes, KEPT as size 1 (expand_op.mojo:121-126): this is the bias gradient."""
+    shape = list(shape)
+    ign = _norm_axes(list(ignore_axes), x.ndim())
+    if x.ndim() == len(shape) and all(i in ign or x._shape[i] == shape[i] for i in range(x.ndim())):
+        return x
+    diff = len(shape) - x.ndim()
+    if diff < 0:
+        raise ValueError("expand: source has more dimensions than the target")
+    new_shape = list(shape[:diff])
+    new_strides = [0] * diff
+    for i in range(x.ndim()):
+        if i in ign:
+            new_shape.append(x._shape[i])
+            new_strides.append(x._strides[i])
+        elif x._shape[i] == shape[i + diff]:
+            new_shape.append(x._shape[i])
+            new_strides.append(x._strides[i])
+        elif x._shape[i] == 1:
+            new_shape.append(shape[i + diff])
+            new_strides.append(0)
+        else:
+            raise ValueError("expand: cannot broadcast %s to %s" % (x.shape(), shape))
+
+    def vjp(primals, grad, out):
+        lead = grad.ndim() - out.ndim()
+        axes = [i + lead for i in range(out.ndim()) if out._strides[i] == 0 and out._shape[i] != 1]
+        return [reduce_add(grad, axes) if axes else grad]
+
+    return _view(x, new_shape, new_strides, x._offset, [x], "brdcst", vjp)
+
+
+def permute(x, axes):
+    """permute_op.mojo:35-143. Given fewer axes than dimensions, they permute the trailing ones."""
+    nd = x.ndim()
+    axes = list(axes)
+    if len(axes) < nd:
+        k = len(axes)
+        axes = list(range(nd - k)) + [nd + a if a < 0 else nd - k + a for a in axes]
+    else:
+        axes = _norm_axes(axes, nd)
+    if sorted(axes) != list(range(nd)):
+        raise ValueError("permute: bad axes %s" % axes)
+    shape = [x._shape[a] for a in axes]
+    strides = [x._strides[a] for a in axes]
+
+    def vjp(primals, grad, out):
+        lead = grad.ndim() - nd
+        inv = [0] * nd
+        for i, a in enumerate(axes):
+            inv[a] = i
+        return [permute(grad, list(range(lead)) + [lead + i for i in inv])]
+
+    return _view(x, shape, strides, x._offset, [x], "permute", vjp)
+
+
+def squeeze(x):
+    """Drop every size-1 axis, keeping one if all are (squeeze_op.mojo:31-60)."""
+    ax = [i for i, s in enumerate(x._shape) if s == 1]
+    if len(ax) == x.ndim() and ax:
+        ax.pop()
+    if not ax:
+        return x
+    shape = [s for i, s in enumerate(x._shape) if i not in ax]
+    strides = [s for i, s in enumerate(x._strides) if i not in ax]
+    in_shape = list(x._shape)
+
+    def vjp(primals, grad, out):
+        lead = grad.ndim() - out.ndim()
+        return [reshape(grad, list(grad._shape[:lead]) + in_shape)]
+
+    return _view(x, shape, strides, x._offset, [x], "squeeze", vjp)
+
+
+def unsqueeze(x, axes):
+    axes = sorted(_norm_axes(list(axes), x.ndim() + len(axes)))
+    shape, strides = list(x._shape), list(x._strides)
+    for a in axes:
+        shape.insert(a, 1)
+        strides.insert(a, 0)
+    in_shape = list(x._shape)
+
+    def vjp(primals, grad, out):
+        lead = grad.ndim() - out.ndim()
+        return [reshape(grad, list(grad._shape[:lead]) + in_shape)]
+
+    return _view(x, shape, strides, x._offset, [x], "unsqueeze", vjp)
+
+
+def reshape(x, shape):
+    """view_op.mojo:33-141: a view when x is contiguous, otherwise a copy first."""
+    shape = list(shape)
+    if -1 in shape:
+        known = _prod([s for s in shape if s != -1])
+        shape[shape.index(-1)] = x.size() // max(known, 1)
+    if _prod(shape) != x.size():
+        raise ValueError("reshape: %s -> %s changes the element count" % (x.shape(), shape))
+    src = x if x.is_contiguous() else _contiguous_copy(x)
+    in_shape = list(x._shape)
+
+    def vjp(primals, grad, out):
+        lead = grad.ndim() - out.ndim()
+        return [reshape(grad, list(grad._shape[:lead]) + in_shape)]
+
+    return _view(src, shape, contiguous_strides(shape), src._offset, [x], "reshape", vjp)
+
+
+def real_part(x):
+    """real(): stride-2 fp32 view of a complex array (real_op.mojo:43-52); VJP complex(g, 0) (:74-77)."""
+    if not x.is_complex_:
+        return x
+
+    def vjp(primals, grad, out):
+        return [complex(grad)]
+
+    return _view(x, x._shape, [2 * s for s in x._strides], 2 * x._offset, [x], "real", vjp, is_complex=False)
+
+
+def imag_part(x):
+    if not x.is_complex_:
+        return zeros(x._shape)
+    return _view(x, x._shape, [2 * s for s in x._strides], 2 * x._offset + 1, [x], "imag", None, is_complex=False)
+
+
+real = real_part
+imag = imag_part
+
+
+# --------------------------------------------------------------------------------------------------
+# binary elementwise ops (endia/functional/binary_ops)
+# --------------------------------------------------------------------------------------------------
+def _broadcast_shape(a, b):
+    sa, sb = list(a._shape), list(b._shape)
+    n = max(len(sa), len(sb))
+    sa = [1] * (n - len(sa)) + sa
+    sb = [1] * (n - len(sb)) + sb
+    out = []
+    for x, y in zip(sa, sb):
+        if x == y or y == 1:
+            out.append(x)
+        elif x == 1:
+            out.append(y)
+        else:
+            raise ValueError("cannot broadcast %s with %s" % (a.shape(), b.shape()))
+    return out
+
+
+def _binary(op, name, a, b, vjp):
+    if a.is_complex_ != b.is_complex_:
+        a = a if a.is_complex_ else complex(a)
+        b = b if b.is_complex_ else complex(b)
+    shape = _broadcast_shape(a, b)
+    # binary_op_array expands both operands to the broadcast shape (binary_ops/_utils.mojo:83-86); the
+    # expanded views take part in autograd, so broadcast axes are summed on the way back
+    ea, eb = expand(a, shape), expand(b, shape)
+    out = Array.empty(shape, is_complex=a.is_complex_)
+    if len(shape) > 8:
+        raise ValueError("more than 8 dimensions")
+    if out.size():
+        L.call("endia_hip_binary", op, len(shape), L.i64_array(shape), L.i64_array(ea._strides), L.i64_array(eb._strides),
+               ea.data_ptr(), eb.data_ptr(), out.data_ptr(), 1 if out.is_complex_ else 0)
+    return _register(out, [ea, eb], name, vjp)
+
+
+def add(a, b):
+    def vjp(primals, grad, out):  # add_op.mojo:107-110
+        return [grad if primals[0]._requires_grad else None, grad if primals[1]._requires_grad else None]
+    return _binary(L.BIN_ADD, "add", a, b, vjp)
+
+
+def sub(a, b):
+    def vjp(primals, grad, out):  # sub_op.mojo:109-112
+        return [grad if primals[0]._requires_grad else None, neg(grad) if primals[1]._requires_grad else None]
+    return _binary(L.BIN_SUB, "sub", a, b, vjp)
+
+
+def mul(a, b):
+    def vjp(primals, grad, out):  # mul_op.mojo:125-128 (no conjugation for complex operands)
+        return [mul(primals[1], grad) if primals[0]._requires_grad else None,
+                mul(primals[0], grad) if primals[1]._requires_grad else None]
+    return _binary(L.BIN_MUL, "mul", a, b, vjp)
+
+
+def div(a, b):
+    def vjp(primals, grad, out):  # div_op.mojo:108-114
+        lhs = div(grad, primals[1]) if primals[0]._requires_grad else None
+        rhs = div(mul(neg(grad), primals[0]), mul(primals[1], primals[1])) if primals[1]._requires_grad else None
+        return [lhs, rhs]
+    return _binary(L.BIN_DIV, "div", a, b, vjp)
+
+
+def greater(a, b):
+    """1.0 where a > b, else 0.0; not differentiable (greater_op.mojo:46-60)."""
+    out = _binary(L.BIN_GREATER, "greater", detach(a), detach(b), None)
+    return out
+
+
+def pow_int(x, p):
+    """x ** p for a small non-negative integer p, as repeated products (x ** 2 is `square`)."""
+    if int(p) != p or p < 0:
+        raise ValueError("only non-negative integer powers are implemented")
+    p = int(p)
+    if p == 0:
+        return ones(x._shape)
+    if p == 2:
+        return square(x)
+    out = x
+    for _ in range(p - 1):
+        out = mul(out, x)
+    return out
+
+
+# --------------------------------------------------------------------------------------------------
+# unary elementwise ops (endia/functional/unary_ops)
+# --------------------------------------------------------------------------------------------------
+def _unary(op, name, x, vjp):
+    src = contiguous(x)
+    out = Array.empty(x._shape, is_complex=x.is_complex_)
+    if out.size():
+        L.call("endia_hip_unary_fwd", op, src.size(), src.data_ptr(), out.data_ptr(), 1 if x.is_complex_ else 0)
+    return _register(out, [x], name, vjp)
+
+
+def relu(x):
+    if x.is_complex_:
+        raise ValueError("relu is not defined for complex arrays")  # relu_op.mojo:51-52
+
+    def vjp(primals, grad, out):  # greater(x, zeros) * g : relu_op.mojo:95
+        return [mul(greater(primals[0], zeros([primals[0]._shape[-1]])), grad)]
+    return _unary(L.OP_RELU, "relu", x, vjp)
+
+
+def tanh(x):
+    def vjp(primals, grad, out):  # (1 - square(tanh(x))) * g, recomputed from the input: tanh_op.mojo:92
+        return [mul(1 - square(tanh(primals[0])), grad)]
+    return _unary(L.OP_TANH, "tanh", x, vjp)
+
+
+def sin(x):
+    def vjp(primals, grad, out):  # sin_op.mojo:92
+        return [mul(cos(primals[0]), grad)]
+    return _unary(L.OP_SIN, "sin", x, vjp)
+
+
+def cos(x):
+    def vjp(primals, grad, out):  # cos_op.mojo:93
+        return [mul(neg(sin(primals[0])), grad)]
+    return _unary(L.OP_COS, "cos", x, vjp)
+
+
+def neg(x):
+    def vjp(primals, grad, out):  # neg_op.mojo:91
+        return [neg(grad)]
+    return _unary(L.OP_NEG, "neg", x, vjp)
+
+
+def square(x):
+    def vjp(primals, grad, out):  # 2 * x * g : square_op.mojo:96
+        return [mul(2 * primals[0], grad)]
+    return _unary(L.OP_SQUARE, "square", x, vjp)
+
+
+def sqrt(x):
+    def vjp(primals, grad, out):  # g / (2 * sqrt(x)) : sqrt_op.mojo:91
+        return [div(grad, 2 * sqrt(primals[0]))]
+    return _unary(L.OP_SQRT, "sqrt", x, vjp)
+
+
+def sign(x):
+    """z / |z| (sign_op.mojo:78-81); used by the VJP of abs."""
+    if x.is_complex_:
+        return div(x, complex(_abs_raw(x)))
+    return div(x, _abs_raw(x))
+
+
+def _abs_raw(x):
+    src = contiguous(x)
+    out = Array.empty(x._shape)
+    if out.size():
+        L.call("endia_hip_unary_fwd", L.OP_ABS, src.size(), src.data_ptr(), out.data_ptr(), 1 if x.is_complex_ else 0)
+    return out
+
+
+def abs(x):
+    """to_abs: |x| as a real array (abs_op.mojo:114-115,157); VJP sign(x) * g (abs_op.mojo:93), where for a
+    complex x the real cotangent first becomes complex(g, 0) (real_op.mojo:74-77)."""
+    out = _abs_raw(x)
+
+    def vjp(primals, grad, out_):
+        z = primals[0]
+        if z.is_complex_:
+            return [mul(sign(z), complex(grad))]
+        return [mul(sign(z), grad)]
+
+    return _register(out, [x], "abs", vjp)
+
+
+# --------------------------------------------------------------------------------------------------
+# reductions (endia/functional/reduce_ops)
+# --------------------------------------------------------------------------------------------------
+def reduce_add(x, axes, _scale=1.0):
+    """Sum over `axes`, keeping them as size 1 (reduce_add_op.mojo:57-61,65-210); VJP = expand (:234)."""
+    axes = sorted(set(_norm_axes(list(axes), x.ndim())))
+    src = contiguous(x)
+    oshape = [1 if i in axes else s for i, s in enumerate(x._shape)]
+    out = Array.empty(oshape, is_complex=x.is_complex_)
+    mask = 0
+    for a in axes:
+        mask |= 1 << a
+    if x.ndim() > 8:
+        raise ValueError("more than 8 dimensions")
+    if out.size():
+        L.call("endia_hip_reduce_add", x.ndim(), L.i64_array(x._shape), mask, src.data_ptr(), out.data_ptr(),
+               float(_scale), 1 if x.is_complex_ else 0)
+    in_shape = list(x._shape)
+
+    def vjp(primals, grad, out_):
+        lead = grad.ndim() - out_.ndim()
+        return [expand(grad, list(grad._shape[:lead]) + in_shape)]
+
+    return _register(out, [x], "reduce_add", vjp)
+
+
+def sum(x):
+    """Sum over all axes, shape [1] (sum_op.mojo:35-62)."""
+    return squeeze(reduce_add(x, list(range(x.ndim()))))
+
+
+def mean(x, axes=None, keepdims=False):
+    """mean_op.mojo:35-65: reduce_add divided by the number of reduced elements."""
+    axes = list(range(x.ndim())) if axes is None else axes
+    res = reduce_add(x, axes)
+    divisor = float(x.size() // max(res.size(), 1))
+    out = res / divisor
+    return out if keepdims else squeeze(out)
+
+
+# --------------------------------------------------------------------------------------------------
+# matmul (endia/functional/binary_ops/matmul_op.mojo)
+# --------------------------------------------------------------------------------------------------
+def _gemm_operand(x):
+    """Describe the last two axes of x for the GEMM: (array, trans, ld, batch_stride).
+
+    A row-major matrix (unit column stride) is passed as is; its transpose view (unit row stride) is
+    passed with the transpose flag, so `.T()` never costs a copy (the reference copies:
+    matmul_op.mojo:111-136). Leading axes must collapse to one batch stride; otherwise x is copied.
+    """
+    def describe(a):
+        rows, cols = a._shape[-2], a._shape[-1]
+        rs, cs = a._strides[-2], a._strides[-1]
+        if (cs == 1 or cols == 1) and (rs >= cols or rows == 1):
+            trans, ld = 0, (rs if rows > 1 else max(cols, 1))
+        elif (rs == 1 or rows == 1) and (cs >= rows or cols == 1):
+            trans, ld = 1, (cs if cols > 1 else max(rows, 1))
+        else:
+            return None
+        # collapse the batch axes
+        bshape = [s for s in a._shape[:-2]]
+        bstr = [s for s in a._strides[:-2]]
+        dims = [(s, st) for s, st in zip(bshape, bstr) if s != 1]
+        if not dims:
+            return a, trans, ld, 0
+        if all(st == 0 for _, st in dims):
+            return a, trans, ld, 0
+        ok = all(dims[i][1] == dims[i + 1][1] * dims[i + 1][0] for i in range(len(dims) - 1))
+        if ok:
+            return a, trans, ld, dims[-1][1]
+        return None
+
+    d = describe(x)
+    if d is None:
+        d = describe(_contiguous_copy(x))
+    return d
+
+
+def matmul(a, b, _conj_vjp=False):
+    """Batched matrix product with broadcast batch axes (matmul_op.mojo:36-90,309-346).
+
+    VJP (matmul_op.mojo:278-283): dA = g @ B.T(), dB = A.T() @ g -- for complex operands WITHOUT
+    conjugation, exactly as the reference codes it. `_conj_vjp=True` selects the Wirtinger rule
+    (g @ B^H, A^H @ g) that PyTorch uses.
+    """
+    if a.ndim() < 2 or b.ndim() < 2:
+        raise ValueError("Invalid shapes for matmul, i.e. ndim < 2")
+    if a._shape[-1] != b._shape[-2]:
+        raise ValueError("Invalid shapes for matmul, i.e. shapes are not compatible for matmul")
+    if a.is_complex_ != b.is_complex_:
+        a = a if a.is_complex_ else complex(a)
+        b = b if b.is_complex_ else complex(b)
+    ba, bb = list(a._shape[:-2]), list(b._shape[:-2])
+    n = max(len(ba), len(bb))
+    ba_p = [1] * (n - len(ba)) + ba
+    bb_p = [1] * (n - len(bb)) + bb
+    bshape = []
+    for x, y in zip(ba_p, bb_p):
+        if x == y or y == 1:
+            bshape.append(x)
+        elif x == 1:
+            bshape.append(y)
+        else:
+            raise ValueError("Error: matmul Incompatible shapes for broadcasting")
+    M, K, N = a._shape[-2], a._shape[-1], b._shape[-1]
+    out_shape = bshape + [M, N]
+    ea = expand(a, bshape + [M, K], [-2, -1])
+    eb = expand(b, bshape + [K, N], [-2, -1])
+    A_, ta, lda, sa = _gemm_operand(ea)
+    B_, tb, ldb, sb = _gemm_operand(eb)
+    out = Array.empty(out_shape, is_complex=a.is_complex_)
+    batch = _prod(bshape)
+    if out.size():
+        if a.is_complex_:
+            L.call("endia_hip_cgemm", ta, 0, tb, 0, M, N, K, A_.data_ptr(), lda, B_.data_ptr(), ldb, out.data_ptr(), N,
+                   batch, sa, sb, M * N, _cgemm_algo[0], 0)
+        else:
+            L.call("endia_hip_sgemm", ta, tb, M, N, K, A_.data_ptr(), lda, B_.data_ptr(), ldb, out.data_ptr(), N, batch,
+                   sa, sb, M * N, L.EPI_NONE, L.OP_IDENTITY, None, None, None)
+
+    def vjp(primals, grad, out_):
+        p0, p1 = primals
+        if _conj_vjp and p0.is_complex_:
+            lhs = matmul(grad, conj(p1).T(), True) if p0._requires_grad else None
+            rhs = matmul(conj(p0).T(), grad, True) if p1._requires_grad else None
+        else:
+            lhs = matmul(grad, p1.T()) if p0._requires_grad else None
+            rhs = matmul(p0.T(), grad) if p1._requires_grad else None
+        return [lhs, rhs]
+
+    return _register(out, [ea, eb], "matmul", vjp)
+
+
+_cgemm_algo = [L.CGEMM_4M]
+
+
+def set_complex_matmul_algorithm(name):
+    """'4m' (the reference's four real products, default) or '3m' (three products, larger rounding error)."""
+    _cgemm_algo[0] = {"4m": L.CGEMM_4M, "3m": L.CGEMM_3M}[name.lower()]
+
+
+def conj(x):
+    """conj_op.mojo:44,54: (re, -im); VJP conj(g)."""
+    if not x.is_complex_:
+        return x
+    out = complex(real_part(x), neg(contiguous(imag_part(x))))
+    out._args, out._vjp = [], None
+
+    def vjp(primals, grad, out_):
+        return [conj(grad)]
+
+    return _register(out, [x], "conj", vjp)
+
+
+# --------------------------------------------------------------------------------------------------
+# loss (endia/functional/loss_ops/mse_op.mojo)
+# --------------------------------------------------------------------------------------------------
+def mse(pred, target):
+    """mse = sum((pred - target) * (pred - target)) / pred.size()  (mse_op.mojo:17-20), as ONE kernel
+    that also writes the gradient 2 (pred - target) / n which the reference's VJP chain
+    (div -> sum -> mul(d, d) -> sub) arrives at. Under create_graph=True the VJP is rebuilt from
+    differentiable ops instead, so higher-order derivatives see the same graph as the reference."""
+    if pred.is_complex_ or target.is_complex_ or pred._shape != target._shape:
+        diff = sub(pred, target)
+        return sum(mul(diff, diff)) / float(pred.size())
+    p, t = contiguous(pred), contiguous(target)
+    loss = Array.empty([1])
+    need_grad = pred._requires_grad
+    dpred = Array.empty(pred._shape) if need_grad else None
+    L.call("endia_hip_mse_fwd_bwd", p.size(), p.data_ptr(), t.data_ptr(), loss.data_ptr(),
+           dpred.data_ptr() if need_grad else None)
+    n = float(pred.size())
+
+    def vjp(primals, grad, out_):
+        from .autograd.functional import building_graph
+        pr, tg = primals
+        if building_graph() or tg._requires_grad or not grad._is_seed:
+            d = sub(pr, tg)
+            g = (d * 2.0) * (grad / n)
+            return [g if pr._requires_grad else None, neg(g) if tg._requires_grad else None]
+        return [dpred, None]
+
+    return _register(loss, [pred, target], "mse", vjp)
+
+
+# --------------------------------------------------------------------------------------------------
+# conv2d (endia/functional/spacial_ops/conv2d_op.mojo)
+# --------------------------------------------------------------------------------------------------
+def _pair(v):
+    return (int(v), int(v)) if np.isscalar(v) else (int(v[0]), int(v[1]))
+
+
+def conv2d(x, kernel, bias=None, stride=1, padding=0, dilation=1, groups=1, _act=None):
+    """NCHW cross-correlation (conv2d_op.mojo:88-196; tuple order is (height, width)). The reference has
+    no backward rule for it (conv2d_op.mojo:198-200); the VJP here is the adjoint of its forward loop."""
+    if x.ndim() != 4:
+        raise ValueError("Input must be 4-dimensional (batch_size, in_channels, height, width) for 2D convolution!")
+    if x._shape[1] != kernel._shape[1]:
+        raise ValueError("Input channels must match kernel channels for 2D convolution!")
+    if x.is_complex_ or kernel.is_complex_:
+        raise ValueError("conv2d is not defined for complex arrays")  # conv2d_op.mojo:216-217
+    (sh, sw), (ph, pw), (dh, dw) = _pair(stride), _pair(padding), _pair(dilation)
+    N, C, H, W = x._shape
+    K, _, R, S = kernel._shape
+    desc = L.Conv2dDesc(N, C, H, W, K, R, S, sh, sw, ph, pw, dh, dw, groups)
+    import ctypes
+    P, Q = ctypes.c_int64(), ctypes.c_int64()
+    L.call("endia_hip_conv2d_out_shape", ctypes.byref(desc), ctypes.byref(P), ctypes.byref(Q))
+    xs, ks = contiguous(x), contiguous(kernel)
+    bsrc = contiguous(bias) if bias is not None else None
+    out = Array.empty([N, K, P.value, Q.value])
+    act = L.OP_RELU if _act == "relu" else L.OP_IDENTITY
+    L.call("endia_hip_conv2d_fwd", ctypes.byref(desc), xs.data_ptr(), ks.data_ptr(),
+           bsrc.data_ptr() if bsrc is not None else None, out.data_ptr(), act)
+
+    def vjp(primals, grad, out_):
+        from .autograd.functional import building_graph
+        if building_graph():
+            raise NotImplementedError("conv2d has no second-order rule")
+        g = contiguous(grad)
+        if _act == "relu":
+            g = mul(greater(out_, zeros([out_._shape[-1]])), g)
+        res = []
+        if primals[0]._requires_grad:
+            dx = Array.empty(primals[0]._shape)
+            L.call("endia_hip_conv2d_bwd_data", ctypes.byref(desc), g.data_ptr(), ks.data_ptr(), dx.data_ptr())
+            res.append(dx)
+        else:
+            res.append(None)
+        if primals[1]._requires_grad:
+            dw = Array.empty(primals[1]._shape)
+            L.call("endia_hip_conv2d_bwd_weight", ctypes.byref(desc), xs.data_ptr(), g.data_ptr(), dw.data_ptr())
+            res.append(dw)
+        else:
+            res.append(None)
+        if len(primals) > 2:
+            if primals[2]._requires_grad:
+                db = Array.empty(primals[2]._shape)
+                L.call("endia_hip_conv2d_bwd_bias", ctypes.byref(desc), g.data_ptr(), db.data_ptr())
+                res.append(db)
+            else:
+                res.append(None)
+        return res
+
+    args = [x, kernel] + ([bias] if bias is not None else [])
+    return _register(out, args, "conv2d", vjp)
+
+
+# --------------------------------------------------------------------------------------------------
+# fused dense layer: act(x @ W + b) as one GEMM with an epilogue (nn/modules/_mlp.mojo:50-52)
+# --------------------------------------------------------------------------------------------------
+_ACT = {None: L.OP_IDENTITY, "identity": L.OP_IDENTITY, "relu": L.OP_RELU, "tanh": L.OP_TANH, "sin": L.OP_SIN}
+_ACT_FN = {"relu": relu, "tanh": tanh, "sin": sin}
+
+
+def linear(x, W, b, act=None):
+    """out = act(x @ W + b) with W [in, out] (no transpose: _mlp.mojo:50).
+
+    Forward: one MFMA GEMM whose epilogue adds the bias row and applies the activation. Backward of a
+    first-order pass: dW = x^T g' (TN GEMM), db = column sum of g', dx = g' W^T (NT GEMM) where
+    g' = g * act'(.). When x is itself the output of a fused layer with a single consumer, that
+    layer's activation derivative is applied in the epilogue of THIS layer's dx GEMM and the gradient
+    is handed over marked as already carrying it. With create_graph=True the rule is rebuilt from
+    matmul / add / activation ops so that the result is differentiable again.
+    """
+    if x.ndim() != 2 or x.is_complex_ or W.is_complex_ or act not in _ACT:
+        z = add(matmul(x, W), b)
+        return _ACT_FN[act](z) if act in _ACT_FN else z
+    xs, Ws, bs_ = contiguous(x), contiguous(W), contiguous(b)
+    B, K = xs._shape
+    N = Ws._shape[1]
+    out = Array.empty([B, N])
+    keep_z = act == "sin" and (x._requires_grad or W._requires_grad or b._requires_grad)
+    z = Array.empty([B, N]) if keep_z else None
+    epi = L.EPI_BIAS if _ACT[act] == L.OP_IDENTITY else L.EPI_BIAS_ACT
+    L.call("endia_hip_sgemm", 0, 0, B, N, K, xs.data_ptr(), K, Ws.data_ptr(), N, out.data_ptr(), N, 1, 0, 0, 0, epi,
+           _ACT[act], bs_.data_ptr(), None, z.data_ptr() if keep_z else None)
+    meta = {"act": act, "z": z}
+
+    def vjp(primals, grad, out_):
+        from .autograd.functional import building_graph
+        px, pW, pb = primals
+        if building_graph():
+            zz = add(matmul(px, pW), pb)
+            if act in _ACT_FN:
+                # the activation's own rule, applied to a re-built pre-activation
+                a = _ACT_FN[act](zz)
+                g = a._vjp(a._args, grad, a)[0]
+            else:
+                g = grad
+            return [matmul(g, pW.T()) if px._requires_grad else None,
+                    matmul(px.T(), g) if pW._requires_grad else None,
+                    reduce_add(g, [0]) if pb._requires_grad else None]
+        g = contiguous(grad)
+        if act in _ACT_FN and not grad._act_applied:
+            gp = Array.empty([B, N])
+            if act == "sin":
+                L.call("endia_hip_unary_vjp", L.OP_SIN, B * N, z.data_ptr(), g.data_ptr(), gp.data_ptr(), 0)
+            else:  # relu and tanh derivatives from the stored output
+                L.call("endia_hip_unary_vjp_from_output", _ACT[act], B * N, out_.data_ptr(), g.data_ptr(), gp.data_ptr())
+            g = gp
+        res = [None, None, None]
+        if pW._requires_grad:
+            dW = Array.empty([K, N])
+            L.call("endia_hip_sgemm", 1, 0, K, N, B, xs.data_ptr(), K, g.data_ptr(), N, dW.data_ptr(), N, 1, 0, 0, 0,
+                   L.EPI_NONE, L.OP_IDENTITY, None, None, None)
+            res[1] = dW
+        if pb._requires_grad:
+            db = Array.empty([1, N])  # kept leading axis, like Expand.vjp (expand_op.mojo:121-126)
+            L.call("endia_hip_reduce_add", 2, L.i64_array([B, N]), 1, g.data_ptr(), db.data_ptr(), 1.0, 0)
+            res[2] = db
+        if px._requires_grad:
+            dx = Array.empty([B, K])
+            single_use = px._consumers == 1 and not px.has_grad()
+            pm = px._meta if (px._name == "linear" and single_use and px._meta) else None
+            if pm and pm["act"] in _ACT_FN:
+                a = pm["act"]
+                aux = pm["z"] if a == "sin" else px
+                flags = _ACT[a] | (0 if a == "sin" else L.ACT_FROM_OUTPUT)
+                L.call("endia_hip_sgemm", 0, 1, B, K, N, g.data_ptr(), N, Ws.data_ptr(), N, dx.data_ptr(), K, 1, 0, 0, 0,
+                       L.EPI_ACT_GRAD, flags, None, contiguous(aux).data_ptr(), None)
+                dx._act_applied = True
+            else:
+                L.call("endia_hip_sgemm", 0, 1, B, K, N, g.data_ptr(), N, Ws.data_ptr(), N, dx.data_ptr(), K, 1, 0, 0, 0,
+                       L.EPI_NONE, L.OP_IDENTITY, None, None, None)
+            res[0] = dx
+        return res
+
+    return _register(out, [x, W, b], "linear", vjp, meta)

@@ -1,0 +1,58 @@
+"""SGD and Adam: the host-side mirror of endia/optim/sgd.mojo and endia/optim/adam.mojo.
+
+The reference builds every update from separate Array ops; here `step()` is one fused kernel per
+parameter tensor, writing the parameter (and the moments) in place, which is what the reference's
+`-=` does through a raw copy (endia/_array/_array.mojo:998-1006). A gradient may carry a kept leading
+axis ([1, N] for an [N] bias: view_ops/expand_op.mojo:121-126); only the element count must match.
+"""
+import numpy as np
+
+from . import _lib as L
+from . import functional as F
+from ._array import Array
+
+
+def _flat_grad(p):
+    if not p.has_grad():
+        raise ValueError("optimizer.step(): a parameter has no gradient")
+    g = F.contiguous(p.grad())
+    if g.size() != p.size():
+        raise ValueError("gradient of shape %s does not match parameter %s" % (g.shape(), p.shape()))
+    return g
+
+
+class SGD:
+    """Plain path `p -= lr * p.grad()` (sgd.mojo:61-62). Momentum and weight decay are not built."""
+
+    def __init__(self, params, lr=0.01, momentum=0.0, weight_decay=0.0):
+        if momentum != 0 or weight_decay != 0:
+            raise NotImplementedError("SGD momentum / weight decay variants (sgd.mojo:42-60) are out of scope")
+        self.params = list(params)
+        self.lr = float(np.float32(lr))
+
+    def step(self):
+        for p in self.params:
+            g = _flat_grad(p)
+            assert p.is_contiguous()
+            L.call("endia_hip_sgd_step", p.size(), p.data_ptr(), g.data_ptr(), self.lr)
+            p.clear_args()
+
+
+class Adam:
+    """adam.mojo:14-65. `t` is an fp32 counter that starts at 1 and grows by one per step()."""
+
+    def __init__(self, params, lr=0.001, beta1=0.9, beta2=0.999, eps=1e-8):
+        self.params = list(params)
+        self.lr, self.beta1, self.beta2, self.eps = (float(np.float32(v)) for v in (lr, beta1, beta2, eps))
+        self.t = 1.0
+        self.m = [Array(p.shape()) for p in self.params]
+        self.v = [Array(p.shape()) for p in self.params]
+
+    def step(self):
+        for p, m, v in zip(self.params, self.m, self.v):
+            g = _flat_grad(p)
+            assert p.is_contiguous()
+            L.call("endia_hip_adam_step", p.size(), p.data_ptr(), g.data_ptr(), m.data_ptr(), v.data_ptr(), self.lr,
+                   self.beta1, self.beta2, self.eps, self.t)
+            p.clear_args()
+        self.t += 1.0

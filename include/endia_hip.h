@@ -103,6 +103,13 @@ ENDIA_API int32_t endia_hip_timer_start(int32_t slot);
 ENDIA_API int32_t endia_hip_timer_stop(int32_t slot);
 ENDIA_API int32_t endia_hip_timer_elapsed_ms(int32_t slot, float* ms); /* blocks until the stop event */
 
+/* ---- per-launch timing of the MFMA GEMM kernel. Between begin and end every launch of the tiled
+ *      fp32 GEMM kernel is bracketed by a pair of HIP events on the library's stream; end blocks, then
+ *      reports the number of launches, the sum of their durations and of their 2*M*N*K*batch flops.
+ *      Used by the benchmark to state achieved TFLOP/s of the dominant kernel inside the timed region. */
+ENDIA_API int32_t endia_hip_gemm_timing_begin(void);
+ENDIA_API int32_t endia_hip_gemm_timing_end(int64_t* launches, double* total_ms, double* total_flops);
+
 /* ---- strided gather copy: execute_copy_raw / contiguous (functional/_utils.mojo:79-205).
  *      dst is contiguous row-major of `shape`; src element (i0..i_{r-1}) is at
  *      src[offset + sum i_d*stride_d]; stride 0 broadcasts. ndim <= 8. is_complex copies pairs. */
@@ -143,6 +150,11 @@ ENDIA_API int32_t endia_hip_unary_fwd(int32_t op, int64_t n, const float* x, flo
 ENDIA_API int32_t endia_hip_unary_vjp(int32_t op, int64_t n, const float* x, const float* g, float* dx,
                             int32_t is_complex);
 
+/* dx = g * op'(x) computed from the stored OUTPUT y = op(x) instead of x: RELU (y > 0), TANH (1 - y^2),
+ * SQRT (1 / (2y)), IDENTITY. Equal to endia_hip_unary_vjp where the reference recomputes the forward
+ * (tanh_op.mojo:92) but without the second transcendental pass. Real only. */
+ENDIA_API int32_t endia_hip_unary_vjp_from_output(int32_t op, int64_t n, const float* y, const float* g, float* dx);
+
 /* ---- broadcasting binary op: binary_op_array + execute_binary_op (binary_ops/_utils.mojo:57-177).
  *      out is contiguous row-major of `shape`; a and b are addressed through element strides
  *      (0 = broadcast axis) so the reference's materialised expand copies are never made. ndim <= 8. */
@@ -152,6 +164,10 @@ ENDIA_API int32_t endia_hip_binary(int32_t op, int32_t ndim, const int64_t* shap
 /* out[i] = alpha * a[i] + beta * b[i]  (gradient accumulation `add`, autograd/functional.mojo:55-57,
  * and scalar scaling such as Div by a full([1], n) operand, _array.mojo:1041-1043). b may be null. */
 ENDIA_API int32_t endia_hip_axpby(int64_t n, float alpha, const float* a, float beta, const float* b, float* out);
+
+/* out[i] = (re[i], im[i]) as interleaved complex; im may be null (imaginary part 0). Replaces
+ * complex(real, imag) (init_ops.mojo:419-433), which Real.vjp uses (view_ops/real_op.mojo:74-77). */
+ENDIA_API int32_t endia_hip_complex_pack(int64_t n, const float* re, const float* im, float* out);
 
 /* ---- reductions: ReduceAdd.__call__ (reduce_ops/reduce_add_op.mojo:65-210) -- also Expand.vjp, the
  *      bias gradient (view_ops/expand_op.mojo:121-126) -- and sum / mean (sum_op.mojo:35-62,

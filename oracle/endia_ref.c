@@ -1,0 +1,497 @@
+/*
+ * endia_ref.c -- TEST INFRASTRUCTURE, not product code.
+ *
+ * A single-threaded CPU restatement, in plain C, of the algorithms on Endia's dense-layer training
+ * path, written from the text of the reference (Mojo 24.5, which cannot be built in this image).
+ * It keeps the reference's loop structure, its fp32 storage of every intermediate and its
+ * accumulation order ("ref order"), so that it serves both as the parity checker of the HIP
+ * kernels and as the timed "Endia CPU path" stand-in. Only tests, the smoke check and the
+ * cpu_baseline leg of the benchmark may call it; nothing shipped links against it.
+ *
+ * Build: see oracle/Makefile (-O3, -ffp-contract=off so that no product-sum is fused).
+ *
+ * How each function is pinned (tests/test_oracle.py, no GPU needed):
+ *   matmul (real, complex), binary ops + broadcast, unary ops and their VJPs, reduce_add, mse,
+ *   conv2d forward, SGD, Adam and the full MLP step are compared with PyTorch float64 -- the oracle
+ *   the reference's own tests use (tests/test_endia/.../test_matmul_op.mojo:18-59 and siblings,
+ *   metric endia/utils/array_conversions.mojo:63-135) -- with the doc known-answers
+ *   (README.md:74-76,106-108; examples/custom_ops_examples/custom_mul.mojo:64-71) and with
+ *   invariants (adjoint identities for the conv2d gradients, which the reference does not have).
+ *   Parity unpinned by any reference test: complex matmul VJP without conjugation (pinned by
+ *   reading matmul_op.mojo:278-283 only) and the conv2d gradients (absent from the reference,
+ *   conv2d_op.mojo:198-200).
+ */
+#include <math.h>
+#include <stdint.h>
+#include <stdlib.h>
+#include <string.h>
+
+/* nelts = 2 * simdwidthof[float32] (endia/utils/aliases.mojo:20-21); 8-lane AVX2 host assumed */
+#define NELTS 16
+
+enum { OP_RELU, OP_TANH, OP_SIN, OP_COS, OP_NEG, OP_SQUARE, OP_SQRT, OP_ABS, OP_IDENTITY, OP_GREATER0 };
+enum { BIN_ADD, BIN_SUB, BIN_MUL, BIN_DIV, BIN_GREATER };
+
+/* Every op output is a freshly allocated, zero-filled buffer: functional/_utils.mojo:319-324 */
+static float* fresh(int64_t n) { return (float*)calloc((size_t)(n > 0 ? n : 1), sizeof(float)); }
+
+/* SIMD reduce_add: pairwise halving of the lane vector */
+static float lanes_reduce(float* v, int n) {
+  for (int w = n / 2; w >= 1; w /= 2)
+    for (int i = 0; i < w; ++i) v[i] = v[i] + v[i + w];
+  return v[0];
+}
+
+/* ---- execute_copy_raw / contiguous: functional/_utils.mojo:79-205 ----------------------------- */
+void ref_strided_copy(int32_t ndim, const int64_t* shape, const int64_t* strides, int64_t offset,
+                      const float* src, float* dst, int32_t is_complex) {
+  int64_t n = 1;
+  for (int i = 0; i < ndim; ++i) n *= shape[i];
+  for (int64_t j = 0; j < n; ++j) {
+    int64_t r = j, is = offset;
+    for (int k = ndim - 1; k >= 0; --k) {
+      is += (r % shape[k]) * strides[k];
+      r /= shape[k];
+    }
+    if (is_complex) {
+      dst[2 * j] = src[2 * is];
+      dst[2 * j + 1] = src[2 * is + 1];
+    } else {
+      dst[j] = src[is];
+    }
+  }
+}
+
+/* ---- matmul_fwd: binary_ops/matmul_op.mojo:93-254 ---------------------------------------------
+ * A is addressed as A[b*a_bs + m*a_rs + k*a_cs], B as B[b*b_bs + k*b_rs + n*b_cs] (element strides, so
+ * a .T() view is a_rs/a_cs swapped). Step 1: contiguous copy of the LHS (:107). Step 2: contiguous
+ * TRANSPOSED copy of the RHS, [N][K] (:111-136; the square-matrix shortcut of :121-129 is not
+ * reproduced -- the documented semantics are). Step 3: one dot product per output element with NELTS
+ * partial sums, a horizontal add, then a scalar tail (:181-199). */
+void ref_matmul(int64_t batch, int64_t M, int64_t N, int64_t K, const float* A, int64_t a_bs, int64_t a_rs,
+                int64_t a_cs, const float* B, int64_t b_bs, int64_t b_rs, int64_t b_cs, float* C) {
+  float* lhs = fresh(M * K);
+  float* rhs = fresh(N * K);
+  for (int64_t b = 0; b < batch; ++b) {
+    for (int64_t m = 0; m < M; ++m)
+      for (int64_t k = 0; k < K; ++k) lhs[m * K + k] = A[b * a_bs + m * a_rs + k * a_cs];
+    for (int64_t n = 0; n < N; ++n)
+      for (int64_t k = 0; k < K; ++k) rhs[n * K + k] = B[b * b_bs + k * b_rs + n * b_cs];
+    int64_t k_end = K - (K % NELTS);
+    float* Cb = C + b * M * N;
+    for (int64_t m = 0; m < M; ++m) {
+      const float* l = lhs + m * K;
+      for (int64_t n = 0; n < N; ++n) {
+        const float* r = rhs + n * K;
+        float sum[NELTS];
+        for (int i = 0; i < NELTS; ++i) sum[i] = 0.f;
+        for (int64_t k = 0; k < k_end; k += NELTS)
+          for (int i = 0; i < NELTS; ++i) sum[i] = sum[i] + l[k + i] * r[k + i];
+        float s = lanes_reduce(sum, NELTS);
+        for (int64_t k = k_end; k < K; ++k) s = s + l[k] * r[k];
+        Cb[m * N + n] = s;
+      }
+    }
+  }
+  free(lhs);
+  free(rhs);
+}
+
+/* complex branch: matmul_op.mojo:201-238. Interleaved operands, strides in complex elements. */
+void ref_cmatmul(int64_t batch, int64_t M, int64_t N, int64_t K, const float* A, int64_t a_bs, int64_t a_rs,
+                 int64_t a_cs, const float* B, int64_t b_bs, int64_t b_rs, int64_t b_cs, float* C) {
+  float* lhs = fresh(2 * M * K);
+  float* rhs = fresh(2 * N * K);
+  for (int64_t b = 0; b < batch; ++b) {
+    for (int64_t m = 0; m < M; ++m)
+      for (int64_t k = 0; k < K; ++k) {
+        int64_t s = b * a_bs + m * a_rs + k * a_cs;
+        lhs[2 * (m * K + k)] = A[2 * s];
+        lhs[2 * (m * K + k) + 1] = A[2 * s + 1];
+      }
+    for (int64_t n = 0; n < N; ++n)
+      for (int64_t k = 0; k < K; ++k) {
+        int64_t s = b * b_bs + k * b_rs + n * b_cs;
+        rhs[2 * (n * K + k)] = B[2 * s];
+        rhs[2 * (n * K + k) + 1] = B[2 * s + 1];
+      }
+    int64_t k_end = K - (K % NELTS);
+    float* Cb = C + 2 * b * M * N;
+    for (int64_t m = 0; m < M; ++m) {
+      const float* l = lhs + 2 * m * K;
+      for (int64_t n = 0; n < N; ++n) {
+        const float* r = rhs + 2 * n * K;
+        float sr[NELTS], si[NELTS];
+        for (int i = 0; i < NELTS; ++i) sr[i] = si[i] = 0.f;
+        for (int64_t k = 0; k < k_end; k += NELTS)
+          for (int i = 0; i < NELTS; ++i) {
+            float lr = l[2 * (k + i)], li = l[2 * (k + i) + 1], rr = r[2 * (k + i)], ri = r[2 * (k + i) + 1];
+            sr[i] = sr[i] + (lr * rr - li * ri);
+            si[i] = si[i] + (lr * ri + li * rr);
+          }
+        float re = lanes_reduce(sr, NELTS), im = lanes_reduce(si, NELTS);
+        for (int64_t k = k_end; k < K; ++k) {
+          float lr = l[2 * k], li = l[2 * k + 1], rr = r[2 * k], ri = r[2 * k + 1];
+          re = re + (lr * rr - li * ri);
+          im = im + (lr * ri + li * rr);
+        }
+        Cb[2 * (m * N + n)] = re;
+        Cb[2 * (m * N + n) + 1] = im;
+      }
+    }
+  }
+  free(lhs);
+  free(rhs);
+}
+
+/* ---- unary forward bodies (real path = complex SIMD body with imag = 0) ------------------------ */
+static float unary_real(int op, float x) {
+  switch (op) {
+    case OP_RELU: return x > 0.f ? x : 0.f;                          /* relu_op.mojo:115-117 */
+    case OP_TANH: return sinhf(2.f * x) / (coshf(2.f * x) + cosf(0.f)); /* tanh_op.mojo:112-115 */
+    case OP_SIN: return sinf(x) * coshf(0.f);                        /* sin_op.mojo:112-114 */
+    case OP_COS: return cosf(x) * coshf(0.f);                        /* cos_op.mojo:113-115 */
+    case OP_NEG: return -x;                                          /* neg_op.mojo:111-113 */
+    case OP_SQUARE: return x * x - 0.f * 0.f;                        /* square_op.mojo:117-119 */
+    case OP_SQRT: {                                                  /* sqrt_op.mojo:111-114 */
+      float r = sqrtf(x * x + 0.f);
+      return sqrtf((r + x) / 2.f);
+    }
+    case OP_ABS: return sqrtf(x * x + 0.f);                          /* abs_op.mojo:114-115 */
+    case OP_GREATER0: return x > 0.f ? 1.f : 0.f;                    /* greater_op.mojo:46-60 */
+    default: return x;
+  }
+}
+
+/* execute_unary_op: unary_ops/_utils.mojo:77-134 */
+void ref_unary(int32_t op, int64_t n, const float* x, float* y) {
+  for (int64_t i = 0; i < n; ++i) y[i] = unary_real(op, x[i]);
+}
+
+/* flat binary op on materialised operands: binary_ops/_utils.mojo:93-177 */
+static void binary_flat(int op, int64_t n, const float* a, const float* b, float* o) {
+  switch (op) {
+    case BIN_ADD: for (int64_t i = 0; i < n; ++i) o[i] = a[i] + b[i]; break;
+    case BIN_SUB: for (int64_t i = 0; i < n; ++i) o[i] = a[i] - b[i]; break;
+    case BIN_MUL: for (int64_t i = 0; i < n; ++i) o[i] = a[i] * b[i]; break;
+    case BIN_DIV: for (int64_t i = 0; i < n; ++i) o[i] = a[i] / b[i]; break;
+    default: for (int64_t i = 0; i < n; ++i) o[i] = a[i] > b[i] ? 1.f : 0.f; break;
+  }
+}
+
+static void binary_flat_complex(int op, int64_t n, const float* a, const float* b, float* o) {
+  for (int64_t i = 0; i < n; ++i) {
+    float ar = a[2 * i], ai = a[2 * i + 1], br = b[2 * i], bi = b[2 * i + 1];
+    switch (op) {
+      case BIN_ADD: o[2 * i] = ar + br; o[2 * i + 1] = ai + bi; break;      /* add_op.mojo:134 */
+      case BIN_SUB: o[2 * i] = ar - br; o[2 * i + 1] = ai - bi; break;      /* sub_op.mojo:136 */
+      case BIN_MUL: o[2 * i] = ar * br - ai * bi; o[2 * i + 1] = ar * bi + ai * br; break; /* mul_op.mojo:152-155 */
+      default: {                                                            /* div_op.mojo:117-142 */
+        float d = br * br + bi * bi;
+        o[2 * i] = (ar * br + ai * bi) / d;
+        o[2 * i + 1] = (ai * br - ar * bi) / d;
+      }
+    }
+  }
+}
+
+/* binary_op_array + execute_binary_op: both operands are expanded to the broadcast shape (stride-0
+ * views, binary_ops/_utils.mojo:83-86) and then made contiguous, i.e. materialised (:95-96). */
+void ref_binary(int32_t op, int32_t ndim, const int64_t* shape, const int64_t* a_strides, const int64_t* b_strides,
+                const float* a, const float* b, float* out, int32_t is_complex) {
+  int64_t n = 1;
+  for (int i = 0; i < ndim; ++i) n *= shape[i];
+  int w = is_complex ? 2 : 1;
+  float* am = fresh(n * w);
+  float* bm = fresh(n * w);
+  ref_strided_copy(ndim, shape, a_strides, 0, a, am, is_complex);
+  ref_strided_copy(ndim, shape, b_strides, 0, b, bm, is_complex);
+  if (is_complex) binary_flat_complex(op, n, am, bm, out);
+  else binary_flat(op, n, am, bm, out);
+  free(am);
+  free(bm);
+}
+
+/* VJP rules, composed from the same ops the reference composes them from */
+void ref_unary_vjp(int32_t op, int64_t n, const float* x, const float* g, float* dx) {
+  float* t = fresh(n);
+  float* u = fresh(n);
+  switch (op) {
+    case OP_RELU: /* greater(x, zeros) * g : relu_op.mojo:95 */
+      for (int64_t i = 0; i < n; ++i) t[i] = x[i] > 0.f ? 1.f : 0.f;
+      binary_flat(BIN_MUL, n, t, g, dx);
+      break;
+    case OP_TANH: /* (1 - square(tanh(x))) * g : tanh_op.mojo:92 */
+      ref_unary(OP_TANH, n, x, t);
+      ref_unary(OP_SQUARE, n, t, u);
+      for (int64_t i = 0; i < n; ++i) t[i] = 1.f - u[i];
+      binary_flat(BIN_MUL, n, t, g, dx);
+      break;
+    case OP_SIN: /* cos(x) * g : sin_op.mojo:92 */
+      ref_unary(OP_COS, n, x, t);
+      binary_flat(BIN_MUL, n, t, g, dx);
+      break;
+    case OP_COS: /* -sin(x) * g : cos_op.mojo:93 */
+      ref_unary(OP_SIN, n, x, t);
+      ref_unary(OP_NEG, n, t, u);
+      binary_flat(BIN_MUL, n, u, g, dx);
+      break;
+    case OP_NEG: /* -g : neg_op.mojo:91 */
+      ref_unary(OP_NEG, n, g, dx);
+      break;
+    case OP_SQUARE: /* 2 * x * g : square_op.mojo:96 */
+      for (int64_t i = 0; i < n; ++i) t[i] = 2.f * x[i];
+      binary_flat(BIN_MUL, n, t, g, dx);
+      break;
+    case OP_SQRT: /* g / (2 * sqrt(x)) : sqrt_op.mojo:91 */
+      ref_unary(OP_SQRT, n, x, t);
+      for (int64_t i = 0; i < n; ++i) u[i] = 2.f * t[i];
+      binary_flat(BIN_DIV, n, g, u, dx);
+      break;
+    case OP_ABS: /* sign(x) * g, sign = x / |x| : abs_op.mojo:93, sign_op.mojo:78-81 (NaN at 0) */
+      for (int64_t i = 0; i < n; ++i) t[i] = x[i] / sqrtf(x[i] * x[i] + 0.f);
+      binary_flat(BIN_MUL, n, t, g, dx);
+      break;
+    default:
+      memcpy(dx, g, (size_t)n * sizeof(float));
+  }
+  free(t);
+  free(u);
+}
+
+/* complex |z| forward (n real outputs) and its VJP sign(z)*complex(g,0): abs_op.mojo:93,114-115,157;
+ * sign_op.mojo:78-81; real_op.mojo:74-77 */
+void ref_cabs(int64_t n, const float* z, float* y) {
+  for (int64_t i = 0; i < n; ++i) y[i] = sqrtf(z[2 * i] * z[2 * i] + z[2 * i + 1] * z[2 * i + 1]);
+}
+void ref_cabs_vjp(int64_t n, const float* z, const float* g, float* dz) {
+  for (int64_t i = 0; i < n; ++i) {
+    float norm = sqrtf(z[2 * i] * z[2 * i] + z[2 * i + 1] * z[2 * i + 1]);
+    float sr = z[2 * i] / norm, si = z[2 * i + 1] / norm;
+    dz[2 * i] = sr * g[i] - si * 0.f;
+    dz[2 * i + 1] = sr * 0.f + si * g[i];
+  }
+}
+
+/* ---- ReduceAdd.__call__: reduce_ops/reduce_add_op.mojo:65-210. Axes with mask bit set are summed and
+ * kept as size 1. The output is zero-initialised and every input element is added to its target in
+ * row-major input order (:112-159); the rank-1 full reduction adds one NELTS-wide horizontal sum
+ * per step and then a scalar tail (:160-190). */
+void ref_reduce_add(int32_t ndim, const int64_t* shape, uint32_t mask, const float* x, float* out, int32_t is_complex) {
+  int64_t n = 1, nout = 1, tstride[8];
+  for (int i = 0; i < ndim; ++i) n *= shape[i];
+  for (int i = ndim - 1; i >= 0; --i) {
+    int red = (mask >> i) & 1;
+    tstride[i] = red ? 0 : nout;
+    if (!red) nout *= shape[i];
+  }
+  int w = is_complex ? 2 : 1;
+  for (int64_t i = 0; i < nout * w; ++i) out[i] = 0.f;
+  if (ndim == 1 && (mask & 1) && !is_complex) {
+    int64_t end = n - n % NELTS;
+    for (int64_t i = 0; i < end; i += NELTS) {
+      float v[NELTS];
+      for (int k = 0; k < NELTS; ++k) v[k] = x[i + k];
+      out[0] = out[0] + lanes_reduce(v, NELTS);
+    }
+    for (int64_t i = end; i < n; ++i) out[0] = out[0] + x[i];
+    return;
+  }
+  for (int64_t j = 0; j < n; ++j) {
+    int64_t r = j, t = 0;
+    for (int k = ndim - 1; k >= 0; --k) {
+      t += (r % shape[k]) * tstride[k];
+      r /= shape[k];
+    }
+    if (is_complex) {
+      out[2 * t] = out[2 * t] + x[2 * j];
+      out[2 * t + 1] = out[2 * t + 1] + x[2 * j + 1];
+    } else {
+      out[t] = out[t] + x[j];
+    }
+  }
+}
+
+/* ---- mse: loss_ops/mse_op.mojo:17-20 = sum((p - t) * (p - t)) / n, and the gradient its VJP chain
+ * yields: Div.vjp g/n (div_op.mojo:108-110), ReduceAdd.vjp expand (reduce_add_op.mojo:234), Mul.vjp
+ * returns diff*g for both operands, which land on the same tensor and are added
+ * (mul_op.mojo:125-128, autograd/functional.mojo:55-57), Sub.vjp passes g to pred (sub_op.mojo:109-112). */
+void ref_mse(int64_t n, const float* pred, const float* target, float* loss, float* dpred) {
+  float* diff = fresh(n);
+  float* sq = fresh(n);
+  binary_flat(BIN_SUB, n, pred, target, diff);
+  binary_flat(BIN_MUL, n, diff, diff, sq);
+  float s = 0.f;
+  for (int64_t i = 0; i < n; ++i) s = s + sq[i];
+  float nf = (float)n;
+  if (loss) *loss = s / nf;
+  if (dpred) {
+    float g = 1.f / nf;
+    for (int64_t i = 0; i < n; ++i) {
+      float a = diff[i] * g;
+      dpred[i] = a + a;
+    }
+  }
+  free(diff);
+  free(sq);
+}
+
+/* ---- Conv2d.__call__: spacial_ops/conv2d_op.mojo:88-196 (groups = 1) -------------------------- */
+typedef struct {
+  int64_t N, C, H, W, K, R, S;
+  int64_t stride_h, stride_w, pad_h, pad_w, dil_h, dil_w, groups;
+} conv_desc;
+
+static void conv_out(const conv_desc* d, int64_t* P, int64_t* Q) {
+  *P = (d->H + 2 * d->pad_h - d->dil_h * (d->R - 1) - 1) / d->stride_h + 1; /* conv2d_op.mojo:65-84 */
+  *Q = (d->W + 2 * d->pad_w - d->dil_w * (d->S - 1) - 1) / d->stride_w + 1;
+}
+
+void ref_conv2d_fwd(const conv_desc* d, const float* x, const float* w, const float* bias, float* y) {
+  int64_t P, Q;
+  conv_out(d, &P, &Q);
+  for (int64_t n = 0; n < d->N; ++n)
+    for (int64_t k = 0; k < d->K; ++k)
+      for (int64_t p = 0; p < P; ++p) {
+        int64_t h0 = p * d->stride_h - d->pad_h;
+        for (int64_t q = 0; q < Q; ++q) {
+          float value = 0.f;
+          int64_t w0 = q * d->stride_w - d->pad_w;
+          for (int64_t c = 0; c < d->C; ++c)
+            for (int64_t r = 0; r < d->R; ++r) {
+              int64_t h = h0 + r * d->dil_h;
+              if (h < 0 || h >= d->H) continue;
+              for (int64_t s = 0; s < d->S; ++s) {
+                int64_t ww = w0 + s * d->dil_w;
+                if (ww < 0 || ww >= d->W) continue;
+                value = value + x[((n * d->C + c) * d->H + h) * d->W + ww] * w[((k * d->C + c) * d->R + r) * d->S + s];
+              }
+            }
+          y[((n * d->K + k) * P + p) * Q + q] = value + (bias ? bias[k] : 0.f);
+        }
+      }
+}
+
+/* Adjoints of the loop above (not in the reference: Conv2d.vjp is default_vjp, conv2d_op.mojo:198-200).
+ * Brute force: every (output element, tap) pair of the forward loop scatters its contribution. */
+void ref_conv2d_bwd(const conv_desc* d, const float* x, const float* w, const float* dy, float* dx, float* dw, float* db) {
+  int64_t P, Q;
+  conv_out(d, &P, &Q);
+  if (dx) memset(dx, 0, sizeof(float) * (size_t)(d->N * d->C * d->H * d->W));
+  if (dw) memset(dw, 0, sizeof(float) * (size_t)(d->K * d->C * d->R * d->S));
+  if (db) memset(db, 0, sizeof(float) * (size_t)d->K);
+  for (int64_t n = 0; n < d->N; ++n)
+    for (int64_t k = 0; k < d->K; ++k)
+      for (int64_t p = 0; p < P; ++p)
+        for (int64_t q = 0; q < Q; ++q) {
+          float g = dy[((n * d->K + k) * P + p) * Q + q];
+          if (db) db[k] = db[k] + g;
+          int64_t h0 = p * d->stride_h - d->pad_h, w0 = q * d->stride_w - d->pad_w;
+          for (int64_t c = 0; c < d->C; ++c)
+            for (int64_t r = 0; r < d->R; ++r) {
+              int64_t h = h0 + r * d->dil_h;
+              if (h < 0 || h >= d->H) continue;
+              for (int64_t s = 0; s < d->S; ++s) {
+                int64_t ww = w0 + s * d->dil_w;
+                if (ww < 0 || ww >= d->W) continue;
+                int64_t xi = ((n * d->C + c) * d->H + h) * d->W + ww, wi = ((k * d->C + c) * d->R + r) * d->S + s;
+                if (dx) dx[xi] = dx[xi] + g * w[wi];
+                if (dw) dw[wi] = dw[wi] + g * x[xi];
+              }
+            }
+        }
+}
+
+/* ---- optimizers ------------------------------------------------------------------------------
+ * SGD plain path: p -= lr * g (optim/sgd.mojo:61-62). Adam: optim/adam.mojo:47-65, one fp32 Array op
+ * at a time. Scalars are fp32 (adam.mojo:19-23); t starts at 1 and is incremented by the caller. */
+void ref_sgd(int64_t n, float* p, const float* g, float lr) {
+  for (int64_t i = 0; i < n; ++i) {
+    float u = lr * g[i];
+    p[i] = p[i] - u;
+  }
+}
+
+void ref_adam(int64_t n, float* p, const float* g, float* m, float* v, float lr, float b1, float b2, float eps, float t) {
+  float omb1 = 1.f - b1, omb2 = 1.f - b2;
+  float c1 = 1.f - powf(b1, t), c2 = 1.f - powf(b2, t);
+  for (int64_t i = 0; i < n; ++i) {
+    float a = b1 * m[i], b = omb1 * g[i];
+    m[i] = a + b;
+    float c = b2 * v[i], e = omb2 * g[i];
+    e = e * g[i];
+    v[i] = c + e;
+    float mh = m[i] / c1, vh = v[i] / c2;
+    float num = lr * mh;
+    float den = unary_real(OP_SQRT, vh) + eps;
+    float q = num / den;
+    p[i] = p[i] - q;
+  }
+}
+
+/* ---- one imperative training step: benchmarks/mlp_benchmarks/mlp_imp.mojo:47-75 -----------------
+ * forward (nn/modules/_mlp.mojo:47-53): pred = act(pred @ W_i + b_i), no activation after the last layer;
+ * loss = mse(pred, y); backward in jacrev order (autograd/functional.mojo:40-65); optimizer step.
+ * W_i is [widths[i], widths[i+1]], b_i [widths[i+1]]. opt: 0 = none, 1 = SGD, 2 = Adam.
+ * Gradients are written to dW[i], db[i] (caller-allocated). Returns the loss. */
+float ref_mlp_step(int32_t L, const int64_t* widths, int64_t batch, int32_t act, const float* x, const float* target,
+                   float** W, float** b, float** dW, float** db, int32_t opt, float lr, float b1, float b2, float eps,
+                   float t, float** mW, float** vW, float** mb, float** vb) {
+  float** Z = (float**)calloc((size_t)L, sizeof(float*));
+  float** A = (float**)calloc((size_t)L + 1, sizeof(float*));
+  A[0] = (float*)x;
+  for (int l = 0; l < L; ++l) {
+    int64_t K = widths[l], N = widths[l + 1];
+    float* mm = fresh(batch * N);
+    ref_matmul(1, batch, N, K, A[l], 0, K, 1, W[l], 0, N, 1, mm);
+    Z[l] = fresh(batch * N);
+    int64_t shape[2] = {batch, N}, fs[2] = {N, 1}, bs[2] = {0, 1};
+    ref_binary(BIN_ADD, 2, shape, fs, bs, mm, b[l], Z[l], 0);
+    free(mm);
+    if (l < L - 1) {
+      A[l + 1] = fresh(batch * N);
+      ref_unary(act, batch * N, Z[l], A[l + 1]);
+    } else {
+      A[l + 1] = Z[l];
+    }
+  }
+  int64_t n_out = batch * widths[L];
+  float loss = 0.f;
+  float* delta = fresh(n_out);
+  ref_mse(n_out, A[L], target, &loss, delta);
+  for (int l = L - 1; l >= 0; --l) {
+    int64_t K = widths[l], N = widths[l + 1];
+    /* Expand.vjp: reduce_add over the broadcast axis (expand_op.mojo:121-126) -> db [1, N] */
+    int64_t shape[2] = {batch, N};
+    ref_reduce_add(2, shape, 1u, delta, db[l], 0);
+    /* matmul_vjp (matmul_op.mojo:278-283): dW = A^T @ delta, dA = delta @ W^T (skipped for the input) */
+    ref_matmul(1, K, N, batch, A[l], 0, 1, K, delta, 0, N, 1, dW[l]);
+    if (l > 0) {
+      float* dA = fresh(batch * K);
+      ref_matmul(1, batch, K, N, delta, 0, N, 1, W[l], 0, 1, N, dA);
+      float* nd = fresh(batch * K);
+      ref_unary_vjp(act, batch * K, Z[l - 1], dA, nd);
+      free(dA);
+      free(delta);
+      delta = nd;
+    }
+  }
+  free(delta);
+  for (int l = 0; l < L; ++l) {
+    int64_t nW = widths[l] * widths[l + 1], nb = widths[l + 1];
+    if (opt == 1) {
+      ref_sgd(nW, W[l], dW[l], lr);
+      ref_sgd(nb, b[l], db[l], lr);
+    } else if (opt == 2) {
+      ref_adam(nW, W[l], dW[l], mW[l], vW[l], lr, b1, b2, eps, t);
+      ref_adam(nb, b[l], db[l], mb[l], vb[l], lr, b1, b2, eps, t);
+    }
+  }
+  for (int l = 0; l < L; ++l) {
+    free(Z[l]);
+    if (l > 0 && l < L) free(A[l]);
+  }
+  free(Z);
+  free(A);
+  return loss;
+}

@@ -1,0 +1,236 @@
+"""Writes the golden fixtures of this directory with PyTorch float64 on the CPU.
+
+PyTorch float64 is the oracle of the reference's own tests (every test converts to float64 torch
+tensors and compares: endia/utils/array_conversions.mojo:41-135, e.g.
+tests/test_endia/test_functional/test_binary_ops/test_matmul_op.mojo:18-59); the reference itself is
+Mojo and cannot run here, and it ships no fixture files. Inputs are seeded, shapes follow the
+reference's tests ((2,30,40) @ (40,50), ...). Run:  python tests/golden/make_golden.py
+"""
+import os
+
+import numpy as np
+import torch
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+torch.manual_seed(0)
+rng = np.random.default_rng(1234)
+
+
+def f32(*shape, scale=1.0):
+    return (rng.standard_normal(shape) * scale).astype(np.float32)
+
+
+def c64(*shape):
+    return (rng.standard_normal(shape) + 1j * rng.standard_normal(shape)).astype(np.complex64)
+
+
+def t64(a, grad=False):
+    dt = torch.complex128 if np.iscomplexobj(a) else torch.float64
+    return torch.tensor(a, dtype=dt, requires_grad=grad)
+
+
+def save(name, **arrays):
+    # expected values are stored rounded to fp32 / complex64: 6e-8 relative, far below the 1e-4 gate
+    arrays = {k: (v.astype(np.complex64) if np.iscomplexobj(v) else v.astype(np.float32)) if v.size > 1 else v
+              for k, v in arrays.items()}
+    np.savez_compressed(os.path.join(HERE, name + ".npz"), **arrays)
+    print("wrote", name, {k: v.shape for k, v in arrays.items()})
+
+
+# ---- matmul: forward, gradients of sum(matmul) (test_matmul_op.mojo:18-75) ------------------------
+a, b = f32(2, 30, 40), f32(40, 50)
+ta, tb = t64(a, True), t64(b, True)
+out = torch.matmul(ta, tb)
+out.sum().backward()
+ca, cb = c64(2, 30, 40), c64(40, 50)
+cout = torch.matmul(t64(ca), t64(cb))
+# square case (the shape class of dX = dY W^T in the MLP configs)
+sa, sb, sg = f32(64, 64), f32(64, 64), f32(64, 64)
+tsa, tsb = t64(sa, True), t64(sb, True)
+(torch.matmul(tsa, tsb) * t64(sg)).sum().backward()
+save("matmul", a=a, b=b, out=out.detach().numpy(), da=ta.grad.numpy(), db=tb.grad.numpy(), ca=ca, cb=cb,
+     cout=cout.numpy(), sa=sa, sb=sb, sg=sg, dsa=tsa.grad.numpy(), dsb=tsb.grad.numpy())
+
+# ---- complex matmul gradients under the Wirtinger-conjugate convention (what torch computes) -------
+za, zb = c64(6, 10), c64(10, 8)
+tza, tzb = t64(za, True), t64(zb, True)
+(torch.matmul(tza, tzb).abs() ** 2).sum().backward()
+save("cmatmul_grad", za=za, zb=zb, dza=tza.grad.numpy(), dzb=tzb.grad.numpy())
+
+# ---- elementwise: forward and gradient of sum(op(x)) (test_relu_op.mojo, test_tanh_op.mojo, ...) ----
+x = f32(2, 30, 40)
+xp = np.abs(x) + 0.1
+d = {"x": x, "xp": xp}
+for name, fn, src in [("relu", torch.relu, x), ("tanh", torch.tanh, x), ("sin", torch.sin, x), ("cos", torch.cos, x),
+                      ("neg", torch.neg, x), ("square", torch.square, x), ("sqrt", torch.sqrt, xp),
+                      ("abs", torch.abs, x)]:
+    t = t64(src, True)
+    y = fn(t)
+    y.sum().backward()
+    d[name] = y.detach().numpy()
+    d["d" + name] = t.grad.numpy()
+save("unary", **d)
+
+# ---- binary with broadcasting and their gradients (test_add_op.mojo:34-60, test_mul_op.mojo:34-59) ---
+a, b = f32(2, 30, 40), f32(30, 40)
+b2 = np.abs(b) + 0.5
+d = {"a": a, "b": b, "b2": b2}
+for name, fn, rhs in [("add", torch.add, b), ("sub", torch.sub, b), ("mul", torch.mul, b), ("div", torch.div, b2)]:
+    ta, tb = t64(a, True), t64(rhs, True)
+    y = fn(ta, tb)
+    torch.sin(y).sum().backward()
+    d[name] = y.detach().numpy()
+    d[name + "_da"] = ta.grad.numpy()
+    d[name + "_db"] = tb.grad.numpy()
+ca, cb = c64(3, 5), c64(5)
+d.update(ca=ca, cb=cb, cmul=(t64(ca) * t64(cb)).numpy(), cdiv=(t64(ca) / t64(cb)).numpy(),
+         cadd=(t64(ca) + t64(cb)).numpy())
+save("binary", **d)
+
+# ---- reductions (test_reduce_add_op.mojo:18-55, test_mean_op.mojo:18-55, test_expand_op.mojo:18-52) ---
+x = f32(2, 30, 40)
+t = t64(x, True)
+r = torch.sum(t, dim=(0, 2), keepdim=True)
+torch.sin(r).sum().backward()
+t2 = t64(x, True)
+m = torch.mean(t2, dim=(1,))
+torch.sin(m).sum().backward()
+bsrc = f32(40)
+t3 = t64(bsrc, True)
+e = t3.expand(2, 30, 40)
+(e * t64(x)).sum().backward()
+save("reduce", x=x, sum02=r.detach().numpy(), dsum02=t.grad.numpy(), mean1=m.detach().numpy(), dmean1=t2.grad.numpy(),
+     total=np.array([x.astype(np.float64).sum()]), bsrc=bsrc, dexpand=t3.grad.numpy())
+
+# ---- mse + gradient (loss_ops/mse_op.mojo:17-20; no reference test) ----------------------------------
+p, tg = f32(16, 8), f32(16, 8)
+tp = t64(p, True)
+loss = torch.nn.functional.mse_loss(tp, t64(tg))
+loss.backward()
+save("mse", pred=p, target=tg, loss=np.array([loss.item()]), dpred=tp.grad.numpy())
+
+# ---- conv2d forward (test_conv2d_op.mojo:18-67: stride 2, pad 1) and gradients ------------------------
+x, w, bb = f32(2, 3, 9, 10), f32(4, 3, 3, 2), f32(4)
+d = {"x": x, "w": w, "b": bb}
+for tag, st, pd, dl in [("s2p1", (2, 2), (1, 1), (1, 1)), ("s1p1", (1, 1), (1, 1), (1, 1)), ("s2p2d2", (2, 1), (2, 0), (2, 1))]:
+    tx, tw, tb = t64(x, True), t64(w, True), t64(bb, True)
+    y = torch.nn.functional.conv2d(tx, tw, tb, stride=st, padding=pd, dilation=dl)
+    g = f32(*y.shape)
+    (y * t64(g)).sum().backward()
+    d.update({tag + "_y": y.detach().numpy(), tag + "_g": g, tag + "_dx": tx.grad.numpy(), tag + "_dw": tw.grad.numpy(),
+              tag + "_db": tb.grad.numpy()})
+save("conv2d", **d)
+
+# ---- optimizers against torch.optim (optim/sgd.mojo:61-62, optim/adam.mojo:47-65; no reference test) ----
+p0 = f32(50, 7)
+gs = [f32(50, 7, scale=0.1) for _ in range(3)]
+d = {"p0": p0, "g0": gs[0], "g1": gs[1], "g2": gs[2]}
+for name, mk in [("sgd", lambda q: torch.optim.SGD([q], lr=1e-3)),
+                 ("adam", lambda q: torch.optim.Adam([q], lr=1e-3, betas=(0.9, 0.999), eps=1e-8))]:
+    q = t64(p0, True)
+    opt = mk(q)
+    for i, g in enumerate(gs):
+        q.grad = t64(g)
+        opt.step()
+        d["%s_p%d" % (name, i + 1)] = q.detach().numpy().copy()
+save("optim", **d)
+
+# ---- the reference's sine-fit MLP, three SGD steps (benchmarks/mlp_benchmarks/mlp_imp.mojo:25-75) -----
+widths = [1, 32, 64, 128, 128, 128, 64, 32, 1]
+xb = rng.uniform(0, 1, (128, 1)).astype(np.float32)
+yb = np.sin(2 * np.pi * xb).astype(np.float32)
+Ws = [f32(widths[i], widths[i + 1], scale=np.sqrt(2.0 / widths[i])) for i in range(8)]
+bs = [f32(widths[i + 1], scale=np.sqrt(2.0 / widths[i])) for i in range(8)]
+d = {"x": xb, "y": yb}
+for i in range(8):
+    d["W%d" % i], d["b%d" % i] = Ws[i], bs[i]
+tW = [t64(W, True) for W in Ws]
+tb_ = [t64(b, True) for b in bs]
+opt = torch.optim.SGD(tW + tb_, lr=1e-3)
+for step in range(3):
+    h = t64(xb)
+    for i in range(8):
+        h = h @ tW[i] + tb_[i]
+        if i < 7:
+            h = torch.relu(h)
+    loss = torch.nn.functional.mse_loss(h, t64(yb))
+    opt.zero_grad()
+    loss.backward()
+    if step == 0:
+        for i in range(8):
+            d["dW%d" % i], d["db%d" % i] = tW[i].grad.numpy().copy(), tb_[i].grad.numpy().copy()
+    d["loss%d" % step] = np.array([loss.item()])
+    opt.step()
+for i in range(8):
+    d["W%d_after" % i], d["b%d_after" % i] = tW[i].detach().numpy(), tb_[i].detach().numpy()
+save("mlp_sine", **d)
+
+# ---- tanh MLP + Adam, small cousin of the wide config (batch 32, 3 layers of 48) ----------------------
+B, H, Lyr = 32, 48, 3
+xb, yb = f32(B, H), f32(B, H)
+Ws = [f32(H, H, scale=1 / np.sqrt(H)) for _ in range(Lyr)]
+bs = [f32(H, scale=1 / np.sqrt(H)) for _ in range(Lyr)]
+d = {"x": xb, "y": yb}
+for i in range(Lyr):
+    d["W%d" % i], d["b%d" % i] = Ws[i], bs[i]
+tW = [t64(W, True) for W in Ws]
+tb_ = [t64(b, True) for b in bs]
+opt = torch.optim.Adam(tW + tb_, lr=1e-3, betas=(0.9, 0.999), eps=1e-8)
+for step in range(2):
+    h = t64(xb)
+    for i in range(Lyr):
+        h = h @ tW[i] + tb_[i]
+        if i < Lyr - 1:
+            h = torch.tanh(h)
+    loss = torch.nn.functional.mse_loss(h, t64(yb))
+    opt.zero_grad()
+    loss.backward()
+    if step == 0:
+        for i in range(Lyr):
+            d["dW%d" % i], d["db%d" % i] = tW[i].grad.numpy().copy(), tb_[i].grad.numpy().copy()
+    d["loss%d" % step] = np.array([loss.item()])
+    opt.step()
+for i in range(Lyr):
+    d["W%d_after" % i], d["b%d_after" % i] = tW[i].detach().numpy(), tb_[i].detach().numpy()
+save("mlp_tanh_adam", **d)
+
+# ---- Hessian-vector product by double backward: sin MLP, loss = sum(out^2) (README.md:69-71 pattern) ----
+B, H, Lyr = 16, 24, 3
+xb = f32(B, H)
+Ws = [f32(H, H, scale=1 / np.sqrt(H)) for _ in range(Lyr)]
+bs = [f32(H, scale=1 / np.sqrt(H)) for _ in range(Lyr)]
+vW = [f32(H, H) for _ in range(Lyr)]
+vb = [f32(H) for _ in range(Lyr)]
+tW = [t64(W, True) for W in Ws]
+tb_ = [t64(b, True) for b in bs]
+h = t64(xb)
+for i in range(Lyr):
+    h = h @ tW[i] + tb_[i]
+    if i < Lyr - 1:
+        h = torch.sin(h)
+loss = (h * h).sum()
+params = tW + tb_
+grads = torch.autograd.grad(loss, params, create_graph=True)
+s = sum((g * t64(v)).sum() for g, v in zip(grads, vW + vb))
+hv = torch.autograd.grad(s, params)
+d = {"x": xb, "loss": np.array([loss.item()])}
+for i in range(Lyr):
+    d["W%d" % i], d["b%d" % i], d["vW%d" % i], d["vb%d" % i] = Ws[i], bs[i], vW[i], vb[i]
+    d["gW%d" % i], d["gb%d" % i] = grads[i].detach().numpy(), grads[Lyr + i].detach().numpy()
+    d["hW%d" % i], d["hb%d" % i] = hv[i].numpy(), hv[Lyr + i].numpy()
+save("hvp_sin", **d)
+
+# ---- complex MLP, identity layers, loss = sum |out|^2: Wirtinger-conjugate gradients (torch) -----------
+B, H, Lyr = 8, 12, 3
+zb = c64(B, H)
+Ws = [(c64(H, H) / np.sqrt(2 * H)).astype(np.complex64) for _ in range(Lyr)]
+tW = [t64(W, True) for W in Ws]
+h = t64(zb)
+for i in range(Lyr):
+    h = h @ tW[i]
+loss = (h.abs() ** 2).sum()
+loss.backward()
+d = {"z": zb, "loss": np.array([loss.item()]), "out": h.detach().numpy()}
+for i in range(Lyr):
+    d["W%d" % i], d["dW%d" % i] = Ws[i], tW[i].grad.numpy()
+save("complex_mlp", **d)

@@ -1,0 +1,323 @@
+"""The host-side mirror of the reference API (Array / backward() / grad(), nn.MLP, optim) running on
+the HIP library, checked against the PyTorch-float64 golden fixtures and the CPU oracle. The tests
+follow the shape of the reference's own (tests/test_endia/test_functional/...): forward, gradient of
+sum(op(x)), complex forward. Tolerance 1e-4 relative per tensor."""
+import numpy as np
+import pytest
+
+from conftest import assert_close, mean_rel
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def nd():
+    import endia_amd
+    return endia_amd
+
+
+def test_matmul_and_grad(nd, golden):  # test_matmul_op.mojo:18-59
+    g = golden("matmul")
+    a, b = nd.array(g["a"], requires_grad=True), nd.array(g["b"], requires_grad=True)
+    res = nd.matmul(a, b)
+    assert_close(res.to_numpy(), g["out"], what="matmul")
+    assert nd.utils.is_close(res, g["out"])
+    nd.sum(res).backward()
+    assert_close(a.grad().to_numpy(), g["da"], what="grad0")
+    assert_close(b.grad().to_numpy(), g["db"], what="grad1")  # shape [1,40,50]: kept broadcast axis
+    assert mean_rel(b.grad().to_numpy().reshape(40, 50), g["db"]) <= 1e-4
+
+
+def test_matmul_square_transposed_views(nd, golden):
+    # dX = g W^T with a SQUARE W: the documented semantics, not the reference's contiguity-shortcut defect
+    g = golden("matmul")
+    a, b = nd.array(g["sa"], requires_grad=True), nd.array(g["sb"], requires_grad=True)
+    nd.sum(nd.matmul(a, b) * nd.array(g["sg"])).backward()
+    assert_close(a.grad().to_numpy(), g["dsa"], what="dA")
+    assert_close(b.grad().to_numpy(), g["dsb"], what="dB")
+
+
+def test_matmul_complex(nd, golden):  # test_matmul_op.mojo:62-75
+    g = golden("matmul")
+    res = nd.matmul(nd.array(g["ca"]), nd.array(g["cb"]))
+    assert res.is_complex()
+    assert_close(res.to_numpy(), g["cout"], what="complex matmul")
+
+
+@pytest.mark.parametrize("op", ["relu", "tanh", "sin", "cos", "neg", "square", "sqrt", "abs"])
+def test_unary_grad(nd, golden, op):  # test_relu_op.mojo:32-49 and siblings
+    g = golden("unary")
+    x = nd.array(g["xp"] if op == "sqrt" else g["x"], requires_grad=True)
+    y = getattr(nd, op)(x)
+    assert_close(y.to_numpy(), g[op], what=op)
+    nd.sum(y).backward()
+    assert_close(x.grad().to_numpy(), g["d" + op], what="grad " + op)
+
+
+@pytest.mark.parametrize("op", ["add", "sub", "mul", "div"])
+def test_binary_grad(nd, golden, op):  # test_add_op.mojo:34-60, test_mul_op.mojo:34-59
+    g = golden("binary")
+    a = nd.array(g["a"], requires_grad=True)
+    b = nd.array(g["b2"] if op == "div" else g["b"], requires_grad=True)
+    y = getattr(nd, op)(a, b)
+    assert_close(y.to_numpy(), g[op], what=op)
+    nd.sum(nd.sin(y)).backward(create_graph=True)  # the reference's add/mul tests build the graph too
+    assert_close(a.grad().to_numpy(), g[op + "_da"], what="dA")
+    assert_close(b.grad().to_numpy(), g[op + "_db"], what="dB")
+
+
+def test_reduce_mean_expand_grad(nd, golden):  # test_reduce_add_op / test_mean_op / test_expand_op
+    g = golden("reduce")
+    x = nd.array(g["x"], requires_grad=True)
+    r = nd.reduce_add(x, [0, 2])
+    assert r.shape() == [1, 30, 1]
+    assert_close(r.to_numpy(), g["sum02"], what="reduce_add")
+    nd.sum(nd.sin(r)).backward()
+    assert_close(x.grad().to_numpy(), g["dsum02"], what="d reduce_add")
+    x2 = nd.array(g["x"], requires_grad=True)
+    m = nd.mean(x2, [1])
+    assert m.shape() == [2, 40]
+    assert_close(m.to_numpy(), g["mean1"], what="mean")
+    nd.sum(nd.sin(m)).backward()
+    assert_close(x2.grad().to_numpy(), g["dmean1"], what="d mean")
+    b = nd.array(g["bsrc"], requires_grad=True)
+    e = nd.expand(b, [2, 30, 40])
+    nd.sum(e * nd.array(g["x"])).backward()
+    assert b.grad().shape() == [1, 1, 40]  # kept axes, as Expand.vjp leaves them
+    assert_close(b.grad().to_numpy(), g["dexpand"], what="d expand")
+
+
+def test_permute_reshape_views(nd):
+    rng = np.random.default_rng(0)
+    a = rng.standard_normal((2, 3, 4)).astype(np.float32)
+    x = nd.array(a, requires_grad=True)
+    p = nd.permute(x, [2, 0, 1])
+    np.testing.assert_array_equal(p.to_numpy(), a.transpose(2, 0, 1))
+    np.testing.assert_array_equal(x.T().to_numpy(), np.swapaxes(a, -1, -2))
+    w = rng.standard_normal((4, 2, 3)).astype(np.float32)
+    nd.sum(p * nd.array(w)).backward()
+    assert_close(x.grad().to_numpy(), w.transpose(1, 2, 0), what="permute vjp")
+    np.testing.assert_array_equal(nd.reshape(x.T(), [6, 4]).to_numpy(), np.swapaxes(a, -1, -2).reshape(6, 4))
+
+
+def test_doc_example_second_order(nd):  # README.md:56-76
+    x = nd.arange(1.0, 4.0, requires_grad=True)
+    y = nd.sum(x ** 2)
+    y.backward(create_graph=True)
+    dy_dx = x.grad()
+    d2y = nd.grad(outs=nd.sum(dy_dx), inputs=x)[0]
+    assert y.item() == 14.0
+    np.testing.assert_array_equal(dy_dx.to_numpy(), [2, 4, 6])
+    np.testing.assert_array_equal(d2y.to_numpy(), [2, 2, 2])
+
+
+def test_doc_example_functional(nd):  # README.md:92-108
+    def foo(x):
+        return nd.sum(x ** 2)
+    foo_jac = nd.grad(foo)
+    foo_hes = nd.jacobian(foo_jac)
+    x = nd.arange(1.0, 4.0)
+    np.testing.assert_array_equal(foo_jac(x).to_numpy(), [2, 4, 6])
+    np.testing.assert_array_equal(foo_hes(x).to_numpy(), 2 * np.eye(3, dtype=np.float32))
+    v, gr = nd.value_and_grad(foo)(x)
+    assert v.item() == 14.0
+    np.testing.assert_array_equal(gr.to_numpy(), [2, 4, 6])
+
+
+def test_custom_op_example(nd):  # examples/custom_ops_examples/custom_mul.mojo:64-71
+    a = nd.array([1.0, 2.0, 3.0], requires_grad=True)
+    b = nd.array([4.0, 5.0, 6.0], requires_grad=True)
+    c = nd.sum(nd.mul(a, b))
+    c.backward()
+    assert c.item() == 32.0
+    np.testing.assert_array_equal(a.grad().to_numpy(), [4, 5, 6])
+    np.testing.assert_array_equal(b.grad().to_numpy(), [1, 2, 3])
+
+
+def test_gradient_accumulation_multi_use(nd):
+    # x used twice: the two cotangents are added by an `add` op (autograd/functional.mojo:55-57)
+    x = nd.array([0.5, -1.0, 2.0], requires_grad=True)
+    y = nd.sum(nd.sin(x) * x)
+    y.backward()
+    v = np.array([0.5, -1.0, 2.0])
+    assert_close(x.grad().to_numpy(), np.cos(v) * v + np.sin(v), what="product rule")
+    y.zero_grad()
+    assert not x.has_grad()
+
+
+def test_mse_fused_matches_composed(nd, golden):
+    g = golden("mse")
+    p = nd.array(g["pred"], requires_grad=True)
+    loss = nd.mse(p, nd.array(g["target"]))
+    loss.backward()
+    assert_close([loss.item()], g["loss"], what="mse")
+    assert_close(p.grad().to_numpy(), g["dpred"], what="mse grad")
+    p2 = nd.array(g["pred"], requires_grad=True)
+    d = nd.sub(p2, nd.array(g["target"]))
+    loss2 = nd.sum(d * d) / float(p2.size())  # mse_op.mojo:17-20 verbatim
+    loss2.backward()
+    assert_close([loss2.item()], g["loss"], what="composed mse")
+    assert_close(p2.grad().to_numpy(), g["dpred"], what="composed mse grad")
+
+
+def _load_mlp(nd, g, n_layers, act, fused):
+    widths = [g["W0"].shape[0]] + [g["W%d" % i].shape[1] for i in range(n_layers)]
+    mlp = nd.nn.MLP(widths, compute_backward=True, activation=act, fused=fused)
+    for i in range(n_layers):
+        mlp.weights[i] = nd.array(g["W%d" % i], requires_grad=True)
+        mlp.biases[i] = nd.array(g["b%d" % i], requires_grad=True)
+    return mlp, widths
+
+
+@pytest.mark.parametrize("fused", [True, False])
+def test_mlp_sine_sgd(nd, golden, fused):
+    """The reference's benchmark model (mlp_imp.mojo:25-75) for three SGD steps, against torch float64
+    and against the CPU oracle's restatement of the same tape."""
+    from oracle import endia_ref as R
+    g = golden("mlp_sine")
+    mlp, widths = _load_mlp(nd, g, 8, "relu", fused)
+    opt = nd.optim.SGD(mlp.params(), lr=1e-3)
+    x, y = nd.array(g["x"]), nd.array(g["y"])
+    Wr = [np.ascontiguousarray(g["W%d" % i]) for i in range(8)]
+    br = [np.ascontiguousarray(g["b%d" % i]) for i in range(8)]
+    for step in range(3):
+        pred = mlp.forward(x)
+        loss = nd.mse(pred, y)
+        loss.backward()
+        loss_ref, dWr, dbr = R.mlp_step(widths, "relu", g["x"], g["y"], Wr, br, opt="sgd", lr=1e-3)
+        assert_close([loss.item()], g["loss%d" % step], what="loss %d" % step)
+        assert_close([loss.item()], [loss_ref], what="loss %d vs oracle" % step)
+        for i in range(8):
+            assert_close(mlp.weights[i].grad().to_numpy(), dWr[i], what="dW%d step %d vs oracle" % (i, step))
+            assert_close(mlp.biases[i].grad().to_numpy(), dbr[i], what="db%d step %d vs oracle" % (i, step))
+            if step == 0:
+                assert_close(mlp.weights[i].grad().to_numpy(), g["dW%d" % i], what="dW%d" % i)
+                assert_close(mlp.biases[i].grad().to_numpy(), g["db%d" % i], what="db%d" % i)
+        opt.step()
+        loss.zero_grad()
+    for i in range(8):
+        assert_close(mlp.weights[i].to_numpy(), g["W%d_after" % i], what="W%d after" % i)
+        assert_close(mlp.biases[i].to_numpy(), g["b%d_after" % i], what="b%d after" % i)
+
+
+@pytest.mark.parametrize("fused", [True, False])
+def test_mlp_tanh_adam(nd, golden, fused):
+    g = golden("mlp_tanh_adam")
+    mlp, widths = _load_mlp(nd, g, 3, "tanh", fused)
+    opt = nd.optim.Adam(mlp.params(), lr=1e-3, beta1=0.9, beta2=0.999, eps=1e-8)
+    x, y = nd.array(g["x"]), nd.array(g["y"])
+    for step in range(2):
+        loss = nd.mse(mlp.forward(x), y)
+        loss.backward()
+        assert_close([loss.item()], g["loss%d" % step], what="loss")
+        if step == 0:
+            for i in range(3):
+                assert_close(mlp.weights[i].grad().to_numpy(), g["dW%d" % i], what="dW%d" % i)
+                assert_close(mlp.biases[i].grad().to_numpy(), g["db%d" % i], what="db%d" % i)
+        opt.step()
+        loss.zero_grad()
+    for i in range(3):
+        assert_close(mlp.weights[i].to_numpy(), g["W%d_after" % i], what="W%d after Adam" % i)
+        assert_close(mlp.biases[i].to_numpy(), g["b%d_after" % i], what="b%d after Adam" % i)
+
+
+@pytest.mark.parametrize("fused", [True, False])
+def test_hvp_double_backward(nd, golden, fused):
+    """Hessian-vector product by create_graph=True double backward (README.md:69-71 pattern) on a sin MLP
+    with loss = sum(out^2); also <u, Hv> = <v, Hu>."""
+    g = golden("hvp_sin")
+    mlp, _ = _load_mlp(nd, g, 3, "sin", fused)
+    x = nd.array(g["x"])
+
+    def hvp(vs):
+        out = mlp.forward(x)
+        loss = nd.sum(out * out)
+        loss.backward(create_graph=True)
+        s = None
+        for p, v in zip(mlp.params(), vs):
+            term = nd.sum(p.grad() * nd.reshape(nd.array(v), p.grad().shape()))
+            s = term if s is None else s + term
+        grads = [p.grad().to_numpy() for p in mlp.params()]
+        hv = nd.grad(outs=s, inputs=mlp.params())
+        res = [h.to_numpy() for h in hv]
+        loss.zero_grad()
+        return float(loss.item()), grads, res
+
+    vs = []
+    for i in range(3):
+        vs += [g["vW%d" % i], g["vb%d" % i]]
+    loss, grads, hv = hvp(vs)
+    assert_close([loss], g["loss"], what="loss")
+    for i in range(3):
+        assert_close(grads[2 * i], g["gW%d" % i], what="gW%d" % i)
+        assert_close(grads[2 * i + 1], g["gb%d" % i], what="gb%d" % i)
+        assert_close(hv[2 * i], g["hW%d" % i], what="HvW%d" % i)
+        assert_close(hv[2 * i + 1], g["hb%d" % i], what="Hvb%d" % i)
+    rng = np.random.default_rng(5)
+    us = [rng.standard_normal(v.shape).astype(np.float32) for v in vs]
+    _, _, hu = hvp(us)
+    uHv = sum(float(np.vdot(u.astype(np.float64), h.reshape(u.shape))) for u, h in zip(us, hv))
+    vHu = sum(float(np.vdot(v.astype(np.float64), h.reshape(v.shape))) for v, h in zip(vs, hu))
+    assert abs(uHv - vHu) <= 1e-4 * max(abs(uHv), abs(vHu))
+
+
+def test_complex_mlp_both_conventions(nd, golden):
+    """Identity complex layers, loss = sum |out|^2. `_conj_vjp=True` gives the Wirtinger-conjugate
+    gradients (equal to torch); the default follows the reference's coded rule without conjugation
+    (matmul_op.mojo:278-283), checked against the oracle's composition of the same products."""
+    from oracle import endia_ref as R
+    g = golden("complex_mlp")
+    for conj in (True, False):
+        Ws = [nd.array(g["W%d" % i], requires_grad=True) for i in range(3)]
+        h = nd.array(g["z"])
+        for W in Ws:
+            h = nd.matmul(h, W, _conj_vjp=conj)
+        loss = nd.sum(nd.square(nd.abs(h)))
+        assert_close(h.to_numpy(), g["out"], what="forward")
+        assert_close([loss.item()], g["loss"], what="loss")
+        loss.backward()
+        if conj:
+            for i in range(3):
+                assert_close(Ws[i].grad().to_numpy(), g["dW%d" % i], what="Wirtinger dW%d" % i)
+        else:
+            acts = [g["z"]]
+            for i in range(3):
+                acts.append(R.matmul(acts[-1], g["W%d" % i]))
+            delta = 2 * acts[-1]
+            for i in (2, 1, 0):
+                assert_close(Ws[i].grad().to_numpy(), R.matmul(acts[i].T, delta), what="reference-rule dW%d" % i)
+                delta = R.matmul(delta, g["W%d" % i].T)
+
+
+def test_conv2d_autograd(nd, golden):
+    g = golden("conv2d")
+    x, w, b = (nd.array(g[k], requires_grad=True) for k in ("x", "w", "b"))
+    y = nd.conv2d(x, w, b, stride=2, padding=1)  # the reference's forward test: test_conv2d_op.mojo:54-62
+    assert_close(y.to_numpy(), g["s2p1_y"], what="conv2d")
+    nd.sum(y * nd.array(g["s2p1_g"])).backward()
+    assert_close(x.grad().to_numpy(), g["s2p1_dx"], what="dx")
+    assert_close(w.grad().to_numpy(), g["s2p1_dw"], what="dw")
+    assert_close(b.grad().to_numpy(), g["s2p1_db"], what="db")
+    # relu + mean loss, the benchmark configuration's head
+    x2, w2, b2 = (nd.array(g[k], requires_grad=True) for k in ("x", "w", "b"))
+    loss = nd.mean(nd.relu(nd.conv2d(x2, w2, b2, stride=1, padding=1)))
+    loss.backward()
+    import torch
+    tx, tw, tb = (torch.tensor(g[k], dtype=torch.float64, requires_grad=True) for k in ("x", "w", "b"))
+    tl = torch.relu(torch.nn.functional.conv2d(tx, tw, tb, stride=1, padding=1)).mean()
+    tl.backward()
+    assert_close([loss.item()], [tl.item()], what="loss")
+    assert_close(w2.grad().to_numpy(), tw.grad.numpy(), what="dw")
+    assert_close(b2.grad().to_numpy(), tb.grad.numpy(), what="db")
+    assert_close(x2.grad().to_numpy(), tx.grad.numpy(), what="dx")
+
+
+def test_shape_errors(nd):
+    with pytest.raises(ValueError, match="ndim < 2"):
+        nd.matmul(nd.zeros([3]), nd.zeros([3, 3]))
+    with pytest.raises(ValueError, match="not compatible"):
+        nd.matmul(nd.zeros([2, 3]), nd.zeros([4, 3]))
+    with pytest.raises(ValueError, match="complex"):
+        nd.relu(nd.zeros([2], is_complex=True))
+    with pytest.raises(ValueError, match="4-dimensional"):
+        nd.conv2d(nd.zeros([3, 3]), nd.zeros([1, 1, 1, 1]))

@@ -1,0 +1,165 @@
+"""fp32 and complex64 GEMM through the C ABI against the CPU oracle and float64.
+
+Tolerance 1e-4 relative per tensor (fp32; the accumulation order differs from the reference's
+lane-strided dot product, matmul_op.mojo:181-199: MFMA sums K in pairs, tile by tile)."""
+import numpy as np
+import pytest
+
+from conftest import assert_close
+from endia_amd import _lib as L
+from oracle import endia_ref as R
+
+pytestmark = pytest.mark.gpu
+
+
+def run_sgemm(dev, A, B, ta, tb, M, N, K, epi=L.EPI_NONE, act=L.OP_IDENTITY, bias=None, aux=None, want_z=False,
+              C0=None, batch=1, sA=0, sB=0):
+    dA, dB = dev.put(A), dev.put(B)
+    dC = dev.put(C0) if C0 is not None else dev.alloc(max(batch * M * N * 4, 4))
+    dbias = dev.put(bias) if bias is not None else None
+    daux = dev.put(aux) if aux is not None else None
+    dz = dev.alloc(max(M * N * 4, 4)) if want_z else None
+    lda = A.shape[-1] if A.ndim >= 2 else 1
+    ldb = B.shape[-1] if B.ndim >= 2 else 1
+    dev.call("endia_hip_sgemm", ta, tb, M, N, K, dA, lda, dB, ldb, dC, N, batch, sA, sB, M * N, epi, act, dbias, daux, dz)
+    C = dev.get(dC, (batch, M, N) if batch > 1 else (M, N))
+    return (C, dev.get(dz, (M, N))) if want_z else C
+
+
+SHAPES = [(128, 128, 32), (256, 384, 72), (132, 260, 100), (37, 53, 19), (4, 4, 4), (1, 1, 1), (128, 1, 32),
+          (1, 32, 128), (300, 200, 8), (64, 64, 1024)]
+
+
+@pytest.mark.parametrize("ta,tb", [(0, 0), (0, 1), (1, 0), (1, 1)])
+@pytest.mark.parametrize("M,N,K", SHAPES)
+def test_sgemm_modes_vs_oracle(dev, M, N, K, ta, tb):
+    rng = np.random.default_rng(M * 7 + N * 3 + K + ta * 2 + tb)
+    A = rng.standard_normal((K, M) if ta else (M, K)).astype(np.float32)
+    B = rng.standard_normal((N, K) if tb else (K, N)).astype(np.float32)
+    C = run_sgemm(dev, A, B, ta, tb, M, N, K)
+    opA, opB = (A.T if ta else A), (B.T if tb else B)
+    assert_close(C, R.matmul(opA, opB), what="vs oracle")
+    assert_close(C, opA.astype(np.float64) @ opB.astype(np.float64), what="vs float64")
+
+
+def test_sgemm_golden(dev, golden):
+    g = golden("matmul")
+    a, b = g["a"], g["b"]
+    # (2,30,40) @ (40,50): batch of 2 with a broadcast right operand (batch stride 0)
+    C = run_sgemm(dev, a, b, 0, 0, 30, 50, 40, batch=2, sA=30 * 40, sB=0)
+    assert_close(C, g["out"], what="batched forward")
+    # the square VJP pair: dA = G B^T (NT), dB = A^T G (TN)
+    assert_close(run_sgemm(dev, g["sg"], g["sb"], 0, 1, 64, 64, 64), g["dsa"], what="dA")
+    assert_close(run_sgemm(dev, g["sa"], g["sg"], 1, 0, 64, 64, 64), g["dsb"], what="dB")
+
+
+@pytest.mark.parametrize("M,N,K", [(256, 256, 64), (50, 30, 7), (130, 70, 36)])
+@pytest.mark.parametrize("act", ["relu", "tanh", "sin", "identity"])
+def test_sgemm_epilogues(dev, M, N, K, act):
+    rng = np.random.default_rng(5)
+    A = rng.standard_normal((M, K)).astype(np.float32)
+    B = (rng.standard_normal((K, N)) / np.sqrt(K)).astype(np.float32)
+    bias = rng.standard_normal(N).astype(np.float32)
+    aux = rng.standard_normal((M, N)).astype(np.float32)
+    code = {"relu": L.OP_RELU, "tanh": L.OP_TANH, "sin": L.OP_SIN, "identity": L.OP_IDENTITY}[act]
+    z_ref = R.binary("add", R.matmul(A, B), bias)
+    # x @ W + b
+    assert_close(run_sgemm(dev, A, B, 0, 0, M, N, K, L.EPI_BIAS, L.OP_IDENTITY, bias=bias), z_ref, what="bias")
+    # act(x @ W + b), also storing the pre-activation
+    C, Z = run_sgemm(dev, A, B, 0, 0, M, N, K, L.EPI_BIAS_ACT, code, bias=bias, want_z=True)
+    assert_close(Z, z_ref, what="stored pre-activation")
+    assert_close(C, R.unary(act, z_ref), what="bias+act")
+    # (dZ W^T) * act'(aux) with aux = pre-activation
+    g_ref = R.unary_vjp(act, aux, R.matmul(A, B))
+    assert_close(run_sgemm(dev, A, B, 0, 0, M, N, K, L.EPI_ACT_GRAD, code, aux=aux), g_ref, what="act grad from input")
+    if act in ("relu", "tanh"):
+        out = R.unary(act, aux)
+        assert_close(run_sgemm(dev, A, B, 0, 0, M, N, K, L.EPI_ACT_GRAD, code | L.ACT_FROM_OUTPUT, aux=out), g_ref,
+                     what="act grad from output")
+    # accumulate into C
+    C0 = rng.standard_normal((M, N)).astype(np.float32)
+    assert_close(run_sgemm(dev, A, B, 0, 0, M, N, K, L.EPI_NONE | L.GEMM_ACCUMULATE, C0=C0),
+                 C0 + R.matmul(A, B), what="accumulate")
+
+
+def test_sgemm_edge_cases(dev):
+    A = np.ones((4, 4), np.float32)
+    # K = 0: the empty sum
+    C = run_sgemm(dev, np.zeros((4, 0), np.float32), np.zeros((0, 4), np.float32), 0, 0, 4, 4, 0,
+                  C0=np.full((4, 4), 7, np.float32))
+    np.testing.assert_array_equal(C, np.zeros((4, 4), np.float32))
+    # M = 0 / N = 0: nothing to do, no error
+    dev.call("endia_hip_sgemm", 0, 0, 0, 4, 4, None, 4, None, 4, None, 4, 1, 0, 0, 0, 0, L.OP_IDENTITY, None, None, None)
+    # errors are reported, not executed
+    lib = L.lib()
+    dA = dev.put(A)
+    assert lib.endia_hip_sgemm(0, 0, 4, 4, 4, dA, 2, dA, 4, dA, 4, 1, 0, 0, 0, 0, L.OP_IDENTITY, None, None, None) == L.ERR_INVALID
+    assert b"leading dimension" in lib.endia_hip_last_error()
+    assert lib.endia_hip_sgemm(0, 0, 4, 4, 4, None, 4, dA, 4, dA, 4, 1, 0, 0, 0, 0, L.OP_IDENTITY, None, None, None) == L.ERR_INVALID
+    assert lib.endia_hip_sgemm(0, 0, -1, 4, 4, dA, 4, dA, 4, dA, 4, 1, 0, 0, 0, 0, L.OP_IDENTITY, None, None, None) == L.ERR_INVALID
+    assert lib.endia_hip_sgemm(0, 0, 4, 4, 4, dA, 4, dA, 4, dA, 4, 1, 0, 0, 0, L.EPI_BIAS, L.OP_IDENTITY, None, None, None) == L.ERR_INVALID
+    assert lib.endia_hip_sgemm(0, 0, 4, 4, 4, dA, 4, dA, 4, dA, 4, 1, 0, 0, 0, 0, L.OP_COS, None, None, None) == L.ERR_INVALID
+
+
+def test_sgemm_unaligned_views(dev):
+    # operands that start in the middle of a buffer with odd leading dimensions take the unaligned path
+    rng = np.random.default_rng(9)
+    big = rng.standard_normal((70, 67)).astype(np.float32)
+    dbig = dev.put(big)
+    A = big[3:3 + 40, 5:5 + 33]
+    B = rng.standard_normal((33, 21)).astype(np.float32)
+    dB = dev.put(B)
+    dC = dev.alloc(40 * 21 * 4)
+    dev.call("endia_hip_sgemm", 0, 0, 40, 21, 33, dbig + 4 * (3 * 67 + 5), 67, dB, 21, dC, 21, 1, 0, 0, 0, 0,
+             L.OP_IDENTITY, None, None, None)
+    assert_close(dev.get(dC, (40, 21)), R.matmul(A, B), what="strided view")
+
+
+@pytest.mark.parametrize("algo,tol", [(L.CGEMM_4M, 1e-4), (L.CGEMM_3M, 1e-4)])
+@pytest.mark.parametrize("ta,ca,tb,cb", [(0, 0, 0, 0), (0, 0, 1, 0), (1, 0, 0, 0), (0, 0, 1, 1), (1, 1, 0, 0)])
+def test_cgemm(dev, algo, tol, ta, ca, tb, cb):
+    rng = np.random.default_rng(11)
+    M, N, K = 96, 72, 40
+    A = (rng.standard_normal((K, M) if ta else (M, K)) + 1j * rng.standard_normal((K, M) if ta else (M, K))).astype(np.complex64)
+    B = (rng.standard_normal((N, K) if tb else (K, N)) + 1j * rng.standard_normal((N, K) if tb else (K, N))).astype(np.complex64)
+    dA, dB, dC = dev.put(A), dev.put(B), dev.alloc(M * N * 8)
+    dev.call("endia_hip_cgemm", ta, ca, tb, cb, M, N, K, dA, A.shape[1], dB, B.shape[1], dC, N, 1, 0, 0, 0, algo, 0)
+    C = dev.get(dC, (M, N), np.complex64)
+    opA = (A.T if ta else A)
+    opB = (B.T if tb else B)
+    opA = np.conj(opA) if ca else opA
+    opB = np.conj(opB) if cb else opB
+    assert_close(C, R.matmul(opA, opB), tol, what="vs oracle")
+    assert_close(C, opA.astype(np.complex128) @ opB.astype(np.complex128), tol, what="vs complex128")
+
+
+def test_cgemm_golden_and_accumulate(dev, golden):
+    g = golden("matmul")
+    ca, cb = g["ca"], g["cb"]
+    dA, dB, dC = dev.put(ca), dev.put(cb), dev.alloc(2 * 30 * 50 * 8)
+    dev.call("endia_hip_cgemm", 0, 0, 0, 0, 30, 50, 40, dA, 40, dB, 50, dC, 50, 2, 30 * 40, 0, 30 * 50, L.CGEMM_4M, 0)
+    out = dev.get(dC, (2, 30, 50), np.complex64)
+    assert_close(out, g["cout"], what="complex batched forward")
+    dev.call("endia_hip_cgemm", 0, 0, 0, 0, 30, 50, 40, dA, 40, dB, 50, dC, 50, 2, 30 * 40, 0, 30 * 50, L.CGEMM_4M, 1)
+    assert_close(dev.get(dC, (2, 30, 50), np.complex64), 2 * g["cout"], what="accumulate")
+
+
+def test_sgemm_large_properties(dev):
+    """Full-size check (4096^3, the wide-MLP shape) through properties that need no CPU GEMM:
+    linearity in A, and agreement of row/column probes with float64 dot products."""
+    rng = np.random.default_rng(21)
+    n = 4096
+    A = rng.standard_normal((n, n)).astype(np.float32)
+    B = (rng.standard_normal((n, n)) / 64).astype(np.float32)
+    for ta, tb in [(0, 0), (0, 1), (1, 0)]:
+        C = run_sgemm(dev, A, B, ta, tb, n, n, n)
+        opA, opB = (A.T if ta else A), (B.T if tb else B)
+        rows = [0, 1, 127, 128, 2049, 4095]
+        cols = [0, 31, 32, 1000, 4095]
+        ref = opA[rows].astype(np.float64) @ opB[:, cols].astype(np.float64)
+        assert_close(C[np.ix_(rows, cols)], ref, what="probes ta=%d tb=%d" % (ta, tb))
+        # checksum of checksums: 1^T C 1 = (1^T A)(B 1)
+        total = opA.astype(np.float64).sum(0) @ opB.astype(np.float64).sum(1)
+        got = C.astype(np.float64).sum()
+        assert abs(got - total) <= 1e-4 * np.abs(opA).astype(np.float64).sum(0) @ np.abs(opB).astype(np.float64).sum(1)
+        dev.release()

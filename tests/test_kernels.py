@@ -1,0 +1,283 @@
+"""Streaming, reduction, loss, optimizer and conv2d kernels through the C ABI against the CPU oracle
+and the PyTorch-float64 golden fixtures. Tolerance 1e-4 relative per tensor unless a test says
+otherwise (optimizer steps are checked much tighter: they do the reference's arithmetic exactly)."""
+import ctypes
+
+import numpy as np
+import pytest
+
+from conftest import assert_close
+from endia_amd import _lib as L
+from oracle import endia_ref as R
+
+pytestmark = pytest.mark.gpu
+
+OPS = {"relu": L.OP_RELU, "tanh": L.OP_TANH, "sin": L.OP_SIN, "cos": L.OP_COS, "neg": L.OP_NEG, "square": L.OP_SQUARE,
+       "sqrt": L.OP_SQRT, "abs": L.OP_ABS}
+
+
+@pytest.mark.parametrize("op", sorted(OPS))
+@pytest.mark.parametrize("n", [1, 5, 1024, 30 * 40 * 2 + 3])
+def test_unary_fwd_and_vjp(dev, golden, op, n):
+    g = golden("unary")
+    x = (g["xp"] if op == "sqrt" else g["x"]).reshape(-1)
+    x = np.resize(x, n).astype(np.float32)
+    gr = np.resize(g["x"].reshape(-1)[::-1], n).astype(np.float32)
+    dx_, dg = dev.put(x), dev.put(gr)
+    dy, dd = dev.alloc(4 * n), dev.alloc(4 * n)
+    dev.call("endia_hip_unary_fwd", OPS[op], n, dx_, dy, 0)
+    dev.call("endia_hip_unary_vjp", OPS[op], n, dx_, dg, dd, 0)
+    y, d = dev.get(dy, (n,)), dev.get(dd, (n,))
+    assert_close(y, R.unary(op, x), what=op)
+    assert_close(d, R.unary_vjp(op, x, gr), what="vjp " + op)
+    if n == 2403:
+        full = g["xp"] if op == "sqrt" else g["x"]
+        assert_close(y[:2400], g[op].reshape(-1), what=op + " vs torch")
+
+
+def test_unary_special_values(dev):
+    x = np.array([0.0, -0.0, 1e-30, -1.0, 60.0, -60.0], np.float32)
+    dx_, dg = dev.put(x), dev.put(np.ones(6, np.float32))
+    dy = dev.alloc(24)
+    dev.call("endia_hip_unary_vjp", L.OP_RELU, 6, dx_, dg, dy, 0)
+    np.testing.assert_array_equal(dev.get(dy, (6,)), [0, 0, 1, 0, 1, 0])  # strict >, greater_op.mojo:57-59
+    dev.call("endia_hip_unary_fwd", L.OP_SQRT, 6, dx_, dy, 0)
+    assert dev.get(dy, (6,))[3] == 0.0  # sqrt of a negative is 0 (sqrt_op.mojo:111-114)
+    # tanh stays finite where the reference's sinh/cosh form overflows to NaN (tanh_op.mojo:112-115)
+    dev.call("endia_hip_unary_fwd", L.OP_TANH, 6, dx_, dy, 0)
+    np.testing.assert_array_equal(dev.get(dy, (6,))[4:], [1.0, -1.0])
+
+
+def test_unary_from_output(dev):
+    rng = np.random.default_rng(0)
+    x = rng.standard_normal(1000).astype(np.float32)
+    g = rng.standard_normal(1000).astype(np.float32)
+    for op in ("relu", "tanh"):
+        y = R.unary(op, x)
+        dy, dg, dd = dev.put(y), dev.put(g), dev.alloc(4000)
+        dev.call("endia_hip_unary_vjp_from_output", OPS[op], 1000, dy, dg, dd)
+        assert_close(dev.get(dd, (1000,)), R.unary_vjp(op, x, g), what=op)
+
+
+def test_complex_unary(dev):
+    rng = np.random.default_rng(1)
+    z = (rng.standard_normal(300) + 1j * rng.standard_normal(300)).astype(np.complex64)
+    g = rng.standard_normal(300).astype(np.float32)
+    dz, dg = dev.put(z), dev.put(g)
+    dy, dd = dev.alloc(1200), dev.alloc(2400)
+    dev.call("endia_hip_unary_fwd", L.OP_ABS, 300, dz, dy, 1)
+    assert_close(dev.get(dy, (300,)), R.cabs(z), what="|z|")
+    dev.call("endia_hip_unary_vjp", L.OP_ABS, 300, dz, dg, dd, 1)
+    assert_close(dev.get(dd, (300,), np.complex64), R.cabs_vjp(z, g), what="abs vjp")
+    dev.call("endia_hip_complex_pack", 300, dg, None, dd)
+    np.testing.assert_array_equal(dev.get(dd, (300,), np.complex64), g.astype(np.complex64))
+
+
+def _binary(dev, op, a, b):
+    cplx = np.iscomplexobj(a)
+    shape = np.broadcast_shapes(a.shape, b.shape)
+    isz = a.itemsize
+    av, bv = np.broadcast_to(a, shape), np.broadcast_to(b, shape)
+    da, db = dev.put(a), dev.put(b)
+    n = int(np.prod(shape))
+    do = dev.alloc(max(n * isz, 4))
+    dev.call("endia_hip_binary", op, len(shape), L.i64_array(shape), L.i64_array([s // isz for s in av.strides]),
+             L.i64_array([s // isz for s in bv.strides]), da, db, do, 1 if cplx else 0)
+    return dev.get(do, shape, a.dtype)
+
+
+@pytest.mark.parametrize("name", ["add", "sub", "mul", "div", "greater"])
+def test_binary_broadcast(dev, golden, name):
+    g = golden("binary")
+    code = dict(add=L.BIN_ADD, sub=L.BIN_SUB, mul=L.BIN_MUL, div=L.BIN_DIV, greater=L.BIN_GREATER)[name]
+    b = g["b2"] if name == "div" else g["b"]
+    out = _binary(dev, code, g["a"], b)
+    assert_close(out, R.binary(name, g["a"], b), tol=1e-6, what=name)
+    if name != "greater":
+        assert_close(out, g[name], what=name + " vs torch")
+    rng = np.random.default_rng(3)
+    # bias row, scalar, middle-axis broadcast, same shape
+    for sa, sb in [((64, 48), (48,)), ((7, 5), (1,)), ((4, 1, 6), (1, 3, 1)), ((33, 9), (33, 9)), ((5,), (3, 5))]:
+        a = rng.standard_normal(sa).astype(np.float32)
+        bb = (np.abs(rng.standard_normal(sb)) + 0.5).astype(np.float32)
+        assert_close(_binary(dev, code, a, bb), R.binary(name, a, bb), tol=1e-6, what="%s %s%s" % (name, sa, sb))
+
+
+def test_binary_complex(dev, golden):
+    g = golden("binary")
+    for name, code in [("add", L.BIN_ADD), ("mul", L.BIN_MUL), ("div", L.BIN_DIV)]:
+        assert_close(_binary(dev, code, g["ca"], g["cb"]), g["c" + name], what="complex " + name)
+
+
+def test_axpby_fill_copy(dev):
+    rng = np.random.default_rng(4)
+    a, b = rng.standard_normal(1001).astype(np.float32), rng.standard_normal(1001).astype(np.float32)
+    da, db, do = dev.put(a), dev.put(b), dev.alloc(4004)
+    dev.call("endia_hip_axpby", 1001, 2.0, da, -0.5, db, do)
+    assert_close(dev.get(do, (1001,)), 2 * a - 0.5 * b, tol=1e-6, what="axpby")
+    dev.call("endia_hip_fill", do, 1001, 3.25)
+    np.testing.assert_array_equal(dev.get(do, (1001,)), np.full(1001, 3.25, np.float32))
+    dev.call("endia_hip_memset0", do, 4004)
+    np.testing.assert_array_equal(dev.get(do, (1001,)), np.zeros(1001, np.float32))
+    # strided gather: transpose, broadcast, offset
+    m = rng.standard_normal((37, 50)).astype(np.float32)
+    dm, dt = dev.put(m), dev.alloc(37 * 50 * 4)
+    dev.call("endia_hip_strided_copy", 2, L.i64_array([50, 37]), L.i64_array([1, 50]), 0, dm, dt, 0)
+    np.testing.assert_array_equal(dev.get(dt, (50, 37)), m.T)
+    dev.call("endia_hip_strided_copy", 3, L.i64_array([2, 5, 7]), L.i64_array([0, 50, 2]), 3, dm, dt, 0)
+    np.testing.assert_array_equal(dev.get(dt, (2, 5, 7)), np.broadcast_to(m[:5, 3:17:2], (2, 5, 7)))
+
+
+CASES = [((2, 30, 40), [0, 2]), ((2, 30, 40), [0, 1, 2]), ((2, 30, 40), [1]), ((2, 30, 40), [2]), ((2, 30, 40), [0, 1]),
+         ((4096, 256), [0]), ((1003,), [0]), ((6, 5, 4, 3), [0, 2, 3]), ((3, 1, 7), [1]), ((8, 16, 12, 12), [0, 2, 3]),
+         ((5, 6, 7, 8), [1, 3])]
+
+
+@pytest.mark.parametrize("shape,axes", CASES)
+def test_reduce_add(dev, shape, axes):
+    rng = np.random.default_rng(sum(shape))
+    x = rng.standard_normal(shape).astype(np.float32)
+    mask = 0
+    for a in axes:
+        mask |= 1 << a
+    oshape = tuple(1 if i in axes else s for i, s in enumerate(shape))
+    dx_, do = dev.put(x), dev.alloc(4 * int(np.prod(oshape)))
+    dev.call("endia_hip_reduce_add", len(shape), L.i64_array(shape), mask, dx_, do, 1.0, 0)
+    out = dev.get(do, oshape)
+    ref64 = x.astype(np.float64).sum(axis=tuple(axes), keepdims=True)
+    # compared on the scale of sum |x|: a sum that cancels has no meaningful relative error
+    scale = np.abs(x).astype(np.float64).sum(axis=tuple(axes), keepdims=True)
+    assert np.all(np.abs(out - ref64) <= 1e-5 * scale + 1e-30)
+    assert np.all(np.abs(out - R.reduce_add(x, axes)) <= 2e-5 * scale + 1e-30)
+
+
+def test_reduce_golden_scale_complex_empty(dev, golden):
+    g = golden("reduce")
+    x = g["x"]
+    dx_, do = dev.put(x), dev.alloc(4 * 80)
+    dev.call("endia_hip_reduce_add", 3, L.i64_array([2, 30, 40]), 0b010, dx_, do, 1.0 / 30.0, 0)
+    assert_close(dev.get(do, (2, 40)), g["mean1"], what="mean over axis 1")
+    dev.call("endia_hip_reduce_add", 3, L.i64_array([2, 30, 40]), 0b011, dx_, do, 1.0, 0)
+    assert_close(dev.get(do, (40,)), g["dexpand"], what="bias-gradient reduction")
+    z = (x[0] + 1j * x[1]).astype(np.complex64)
+    dz = dev.put(z)
+    dev.call("endia_hip_reduce_add", 2, L.i64_array([30, 40]), 0b01, dz, do, 1.0, 1)
+    assert_close(dev.get(do, (40,), np.complex64), R.reduce_add(z, [0]).reshape(-1), what="complex column sum")
+    dev.call("endia_hip_reduce_add", 2, L.i64_array([30, 40]), 0b10, dz, do, 1.0, 1)
+    assert_close(dev.get(do, (30,), np.complex64), R.reduce_add(z, [1]).reshape(-1), what="complex row sum")
+    dev.call("endia_hip_fill", do, 8, 5.0)
+    dev.call("endia_hip_reduce_add", 2, L.i64_array([0, 8]), 0b01, None, do, 1.0, 0)
+    np.testing.assert_array_equal(dev.get(do, (8,)), np.zeros(8, np.float32))  # empty sum
+
+
+@pytest.mark.parametrize("n", [1, 128, 16 * 8, 100003])
+def test_mse(dev, golden, n):
+    g = golden("mse")
+    p = np.resize(g["pred"].reshape(-1), n).astype(np.float32)
+    t = np.resize(g["target"].reshape(-1)[::-1], n).astype(np.float32)
+    dp, dt, dl, dg = dev.put(p), dev.put(t), dev.alloc(4), dev.alloc(4 * n)
+    dev.call("endia_hip_mse_fwd_bwd", n, dp, dt, dl, dg)
+    loss_ref, grad_ref = R.mse(p, t)
+    assert_close(dev.get(dl, (1,)), [((p.astype(np.float64) - t) ** 2).mean()], tol=1e-5, what="loss vs float64")
+    assert_close(dev.get(dl, (1,)), [loss_ref], what="loss vs oracle")
+    assert_close(dev.get(dg, (n,)), grad_ref, tol=1e-6, what="gradient")
+
+
+def test_mse_golden_and_errors(dev, golden):
+    g = golden("mse")
+    dp, dt, dl, dg = dev.put(g["pred"]), dev.put(g["target"]), dev.alloc(4), dev.alloc(4 * 128)
+    dev.call("endia_hip_mse_fwd_bwd", 128, dp, dt, dl, dg)
+    assert_close(dev.get(dl, (1,)), g["loss"], what="loss")
+    assert_close(dev.get(dg, (16, 8)), g["dpred"], what="dpred")
+    assert L.lib().endia_hip_mse_fwd_bwd(0, dp, dt, dl, dg) == L.ERR_INVALID
+    assert L.lib().endia_hip_mse_fwd_bwd(4, dp, dt, None, None) == L.ERR_INVALID
+
+
+def test_optimizers_bit_exact_vs_oracle(dev, golden):
+    """The fused steps perform the reference's op chain with the same fp32 roundings, so they must agree
+    with the oracle to the last bit (powf of the two betas is evaluated on the host in both)."""
+    g = golden("optim")
+    p_ref = g["p0"]
+    dp = dev.put(g["p0"])
+    for i in range(3):
+        dg = dev.put(g["g%d" % i])
+        dev.call("endia_hip_sgd_step", 350, dp, dg, 1e-3)
+        p_ref = R.sgd(p_ref, g["g%d" % i], 1e-3)
+        got = dev.get(dp, (50, 7))
+        np.testing.assert_array_equal(got, p_ref)
+        assert_close(got, g["sgd_p%d" % (i + 1)], tol=1e-6, what="sgd vs torch")
+    p_ref, m_ref, v_ref = g["p0"], np.zeros((50, 7), np.float32), np.zeros((50, 7), np.float32)
+    dp, dm, dv = dev.put(g["p0"]), dev.put(m_ref), dev.put(v_ref)
+    for i in range(3):
+        dg = dev.put(g["g%d" % i])
+        dev.call("endia_hip_adam_step", 350, dp, dg, dm, dv, 1e-3, 0.9, 0.999, 1e-8, float(i + 1))
+        p_ref, m_ref, v_ref = R.adam(p_ref, g["g%d" % i], m_ref, v_ref, 1e-3, 0.9, 0.999, 1e-8, float(i + 1))
+        np.testing.assert_array_equal(dev.get(dp, (50, 7)), p_ref)
+        np.testing.assert_array_equal(dev.get(dm, (50, 7)), m_ref)
+        np.testing.assert_array_equal(dev.get(dv, (50, 7)), v_ref)
+        assert_close(dev.get(dp, (50, 7)), g["adam_p%d" % (i + 1)], tol=1e-6, what="adam vs torch")
+    assert L.lib().endia_hip_adam_step(350, dp, dg, dm, dv, 1e-3, 0.9, 0.999, 1e-8, ctypes.c_float(0.0)) == L.ERR_INVALID
+
+
+def _desc(x, w, st, pd, dl):
+    N, C, H, W = x.shape
+    K, _, Rr, S = w.shape
+    return L.Conv2dDesc(N, C, H, W, K, Rr, S, st[0], st[1], pd[0], pd[1], dl[0], dl[1], 1)
+
+
+@pytest.mark.parametrize("tag,st,pd,dl", [("s2p1", (2, 2), (1, 1), (1, 1)), ("s1p1", (1, 1), (1, 1), (1, 1)),
+                                         ("s2p2d2", (2, 1), (2, 0), (2, 1))])
+def test_conv2d_golden(dev, golden, tag, st, pd, dl):
+    g = golden("conv2d")
+    x, w, b, gy = g["x"], g["w"], g["b"], g[tag + "_g"]
+    d = _desc(x, w, st, pd, dl)
+    dx_, dw_, db_, dg = dev.put(x), dev.put(w), dev.put(b), dev.put(gy)
+    dy = dev.alloc(gy.nbytes)
+    dev.call("endia_hip_conv2d_fwd", ctypes.byref(d), dx_, dw_, db_, dy, L.OP_IDENTITY)
+    assert_close(dev.get(dy, gy.shape), g[tag + "_y"], what="fwd")
+    assert_close(dev.get(dy, gy.shape), R.conv2d(x, w, b, st, pd, dl), tol=1e-5, what="fwd vs oracle")
+    ddx, ddw, ddb = dev.alloc(x.nbytes), dev.alloc(w.nbytes), dev.alloc(b.nbytes)
+    dev.call("endia_hip_conv2d_bwd_data", ctypes.byref(d), dg, dw_, ddx)
+    dev.call("endia_hip_conv2d_bwd_weight", ctypes.byref(d), dx_, dg, ddw)
+    dev.call("endia_hip_conv2d_bwd_bias", ctypes.byref(d), dg, ddb)
+    assert_close(dev.get(ddx, x.shape), g[tag + "_dx"], what="dx")
+    assert_close(dev.get(ddw, w.shape), g[tag + "_dw"], what="dw")
+    assert_close(dev.get(ddb, b.shape), g[tag + "_db"], what="db")
+    # relu epilogue
+    dev.call("endia_hip_conv2d_fwd", ctypes.byref(d), dx_, dw_, db_, dy, L.OP_RELU)
+    assert_close(dev.get(dy, gy.shape), np.maximum(g[tag + "_y"], 0), what="fwd+relu")
+
+
+def test_conv2d_medium_vs_oracle(dev):
+    # a slice of the benchmark configuration (64 -> 128 channels, 3x3, pad 1) small enough for the CPU loop
+    rng = np.random.default_rng(6)
+    x = rng.standard_normal((2, 16, 14, 14)).astype(np.float32)
+    w = (rng.standard_normal((24, 16, 3, 3)) * np.sqrt(2 / (16 * 9))).astype(np.float32)
+    b = rng.standard_normal(24).astype(np.float32)
+    d = _desc(x, w, (1, 1), (1, 1), (1, 1))
+    y_ref = R.conv2d(x, w, b, (1, 1), (1, 1), (1, 1))
+    gy = rng.standard_normal(y_ref.shape).astype(np.float32)
+    dx_ref, dw_ref, db_ref = R.conv2d_bwd(x, w, gy, (1, 1), (1, 1), (1, 1))
+    dx_, dw_, db_, dg = dev.put(x), dev.put(w), dev.put(b), dev.put(gy)
+    dy, ddx, ddw, ddb = dev.alloc(gy.nbytes), dev.alloc(x.nbytes), dev.alloc(w.nbytes), dev.alloc(b.nbytes)
+    dev.call("endia_hip_conv2d_fwd", ctypes.byref(d), dx_, dw_, db_, dy, L.OP_IDENTITY)
+    dev.call("endia_hip_conv2d_bwd_data", ctypes.byref(d), dg, dw_, ddx)
+    dev.call("endia_hip_conv2d_bwd_weight", ctypes.byref(d), dx_, dg, ddw)
+    dev.call("endia_hip_conv2d_bwd_bias", ctypes.byref(d), dg, ddb)
+    assert_close(dev.get(dy, gy.shape), y_ref, what="fwd")
+    assert_close(dev.get(ddx, x.shape), dx_ref, what="dx")
+    assert_close(dev.get(ddw, w.shape), dw_ref, what="dw")
+    assert_close(dev.get(ddb, b.shape), db_ref, what="db")
+
+
+def test_pool_reuses_buffers(dev):
+    u, c, n0 = ctypes.c_int64(), ctypes.c_int64(), ctypes.c_int64()
+    p = dev.alloc(1 << 20)
+    dev.call("endia_hip_free", p)
+    dev._live.remove(p)
+    dev.call("endia_hip_pool_stats", ctypes.byref(u), ctypes.byref(c), ctypes.byref(n0))
+    q = dev.alloc(1 << 20)
+    n1 = ctypes.c_int64()
+    dev.call("endia_hip_pool_stats", ctypes.byref(u), ctypes.byref(c), ctypes.byref(n1))
+    assert q == p and n1.value == n0.value  # same buffer, no new device allocation
+    assert L.lib().endia_hip_free(ctypes.c_void_p(12345)) == L.ERR_INVALID
