@@ -132,12 +132,78 @@ def cpu_baseline_sine(steps=200):
             "sample": "%d full fwd+bwd+SGD steps of the ref-order CPU restatement, 1 thread" % steps}
 
 
+def kernel_table(reps=10):
+    """Times each hot kernel alone at the wide-MLP shape with HIP events on the library's stream and
+    prices it against its roofline (fp32 MFMA peak for the GEMMs, HBM peak for the rest). Algorithmic
+    bytes: every operand read once, every result written once. The `copy` row (out = 1.0 * a, 64 MiB in,
+    64 MiB out) is the known-size kernel that scales the FETCH_SIZE / WRITE_SIZE counters."""
+    from endia_amd import _lib as L
+    L.ensure_init(0)
+    n = 4096
+    nn = n * n
+
+    def dmalloc(nbytes):
+        p = ctypes.c_void_p()
+        L.call("endia_hip_malloc", nbytes, ctypes.byref(p))
+        return p.value
+
+    rng = np.random.default_rng(0)
+    host = (rng.standard_normal(nn) / 64).astype(np.float32)
+    bufs = [dmalloc(4 * nn) for _ in range(5)]
+    for b in bufs:
+        L.call("endia_hip_memcpy_h2d", b, host.ctypes.data, host.nbytes)
+    A, B, C, D, E = bufs
+    bias = dmalloc(4 * n)
+    L.call("endia_hip_memcpy_h2d", bias, host.ctypes.data, 4 * n)
+    loss = dmalloc(4)
+    I = L.OP_IDENTITY
+
+    def gemm(ta, tb, epi=L.EPI_NONE, act=I, aux=None):
+        return lambda: L.call("endia_hip_sgemm", ta, tb, n, n, n, A, n, B, n, C, n, 1, 0, 0, 0, epi, act, bias, aux, None)
+
+    gflop = 2.0 * n * n * n
+    cases = [
+        ("sgemm_nn  Z = A W", gemm(0, 0), gflop, "mfma"),
+        ("sgemm_nn  tanh(A W + b) epilogue", gemm(0, 0, L.EPI_BIAS_ACT, L.OP_TANH), gflop, "mfma"),
+        ("sgemm_nt  dA = dZ W^T", gemm(0, 1), gflop, "mfma"),
+        ("sgemm_nt  (dZ W^T) * tanh' epilogue", gemm(0, 1, L.EPI_ACT_GRAD, L.OP_TANH | L.ACT_FROM_OUTPUT, D), gflop, "mfma"),
+        ("sgemm_tn  dW = A^T dZ", gemm(1, 0), gflop, "mfma"),
+        ("copy      out = a (64 MiB)", lambda: L.call("endia_hip_axpby", nn, 1.0, A, 0.0, None, C), 8.0 * nn, "hbm"),
+        ("col_reduce  db = 1^T dZ", lambda: L.call("endia_hip_reduce_add", 2, L.i64_array([n, n]), 1, A, bias, 1.0, 0),
+         4.0 * nn + 4.0 * n, "hbm"),
+        ("mse_fwd_bwd", lambda: L.call("endia_hip_mse_fwd_bwd", nn, A, B, loss, C), 12.0 * nn, "hbm"),
+        ("adam_step (one 4096^2 weight)", lambda: L.call("endia_hip_adam_step", nn, C, A, D, E, 1e-3, 0.9, 0.999, 1e-8, 1.0),
+         28.0 * nn, "hbm"),
+        ("sgd_step", lambda: L.call("endia_hip_sgd_step", nn, C, A, 1e-3), 12.0 * nn, "hbm"),
+        ("tanh_fwd", lambda: L.call("endia_hip_unary_fwd", L.OP_TANH, nn, A, C, 0), 8.0 * nn, "hbm"),
+        ("tanh_vjp", lambda: L.call("endia_hip_unary_vjp", L.OP_TANH, nn, A, B, C, 0), 12.0 * nn, "hbm"),
+    ]
+    rows = []
+    ms = ctypes.c_float()
+    for name, fn, work, bound in cases:
+        for _ in range(2):
+            fn()
+        L.call("endia_hip_timer_start", 0)
+        for _ in range(reps):
+            fn()
+        L.call("endia_hip_timer_stop", 0)
+        L.call("endia_hip_timer_elapsed_ms", 0, ctypes.byref(ms))
+        t = ms.value / reps
+        if bound == "mfma":
+            ach, peak, unit = work / (t * 1e-3) / 1e12, FP32_MFMA_PEAK_TFLOPS, "TFLOP/s"
+        else:
+            ach, peak, unit = work / (t * 1e-3) / 1e9, HBM_PEAK_GBS, "GB/s"
+        rows.append({"kernel": name, "ms": t, "bound": bound, "achieved": ach, "peak": peak, "unit": unit,
+                     "frac": ach / peak, "algorithmic_work": work})
+    return rows
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=3)
-    ap.add_argument("--workload", default="wide_mlp", choices=["wide_mlp", "sine_mlp"])
+    ap.add_argument("--workload", default="wide_mlp", choices=["wide_mlp", "sine_mlp", "kernels"])
     ap.add_argument("--no-cpu-baseline", action="store_true")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -148,6 +214,12 @@ def main():
     from endia_amd import _lib as L
     L.ensure_init(0)
     dev_name, cus, mhz = L.device_info()
+
+    if args.workload == "kernels":
+        rows = kernel_table(max(args.steps, 1))
+        print(json.dumps({"metric": "per-kernel roofline at the wide-MLP shape (4096 x 4096 operands)", "device": dev_name,
+                          "reps": max(args.steps, 1), "kernels": rows}))
+        return
 
     if args.workload == "wide_mlp":
         mlp, opt, x, y = build_wide_mlp(nd)
