@@ -181,7 +181,59 @@ def kernel_table(reps=10):
     rows = []
     ms = ctypes.c_float()
     for name, fn, work, bound in cases:
-        for _ in range(2):
+        for _ in range(5):
+            fn()
+        L.call("endia_hip_timer_start", 0)
+        for _ in range(reps):
+            fn()
+        L.call("endia_hip_timer_stop", 0)
+        L.call("endia_hip_timer_elapsed_ms", 0, ctypes.byref(ms))
+        t = ms.value / reps
+        if bound == "mfma":
+            ach, peak, unit = work / (t * 1e-3) / 1e12, FP32_MFMA_PEAK_TFLOPS, "TFLOP/s"
+        else:
+            ach, peak, unit = work / (t * 1e-3) / 1e9, HBM_PEAK_GBS, "GB/s"
+        rows.append({"kernel": name, "ms": t, "bound": bound, "achieved": ach, "peak": peak, "unit": unit,
+                     "frac": ach / peak, "algorithmic_work": work})
+    return rows
+
+
+def conv_table(reps=10):
+    """conv2d at the benchmark configuration: x [64,64,56,56], w [128,64,3,3], stride 1, pad 1 (fp32, NCHW).
+    Algorithmic flops per pass: 2*N*K*C*R*S*P*Q = 29.6 GFLOP for each of forward, data and weight gradient."""
+    from endia_amd import _lib as L
+    L.ensure_init(0)
+    N, C, H, W, K, R, S = 64, 64, 56, 56, 128, 3, 3
+    d = L.Conv2dDesc(N, C, H, W, K, R, S, 1, 1, 1, 1, 1, 1, 1)
+    P = Q = 56
+    rng = np.random.default_rng(5)
+
+    def put(a):
+        p = ctypes.c_void_p()
+        L.call("endia_hip_malloc", a.nbytes, ctypes.byref(p))
+        L.call("endia_hip_memcpy_h2d", p.value, a.ctypes.data, a.nbytes)
+        return p.value
+
+    x = put(rng.standard_normal((N, C, H, W)).astype(np.float32))
+    w = put((rng.standard_normal((K, C, R, S)) * np.sqrt(2.0 / (C * R * S))).astype(np.float32))
+    b = put(rng.standard_normal(K).astype(np.float32))
+    dy = put(rng.standard_normal((N, K, P, Q)).astype(np.float32))
+    y = put(np.zeros((N, K, P, Q), np.float32))
+    dx = put(np.zeros((N, C, H, W), np.float32))
+    dw = put(np.zeros((K, C, R, S), np.float32))
+    db = put(np.zeros(K, np.float32))
+    flop = 2.0 * N * K * C * R * S * P * Q
+    ref = ctypes.byref(d)
+    cases = [
+        ("conv2d_fwd (+bias, relu)", lambda: L.call("endia_hip_conv2d_fwd", ref, x, w, b, y, L.OP_RELU), flop, "mfma"),
+        ("conv2d_bwd_data", lambda: L.call("endia_hip_conv2d_bwd_data", ref, dy, w, dx), flop, "mfma"),
+        ("conv2d_bwd_weight", lambda: L.call("endia_hip_conv2d_bwd_weight", ref, x, dy, dw), flop, "mfma"),
+        ("conv2d_bwd_bias", lambda: L.call("endia_hip_conv2d_bwd_bias", ref, dy, db), 4.0 * N * K * P * Q, "hbm"),
+    ]
+    rows = []
+    ms = ctypes.c_float()
+    for name, fn, work, bound in cases:
+        for _ in range(3):
             fn()
         L.call("endia_hip_timer_start", 0)
         for _ in range(reps):
@@ -203,7 +255,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=3)
-    ap.add_argument("--workload", default="wide_mlp", choices=["wide_mlp", "sine_mlp", "kernels"])
+    ap.add_argument("--workload", default="wide_mlp", choices=["wide_mlp", "sine_mlp", "kernels", "conv2d"])
     ap.add_argument("--no-cpu-baseline", action="store_true")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -215,6 +267,11 @@ def main():
     L.ensure_init(0)
     dev_name, cus, mhz = L.device_info()
 
+    if args.workload == "conv2d":
+        rows = conv_table(max(args.steps, 1))
+        print(json.dumps({"metric": "conv2d fwd + VJPs, batch 64, 64->128 channels, 3x3, stride 1, pad 1, 56x56, fp32",
+                          "device": dev_name, "reps": max(args.steps, 1), "kernels": rows}))
+        return
     if args.workload == "kernels":
         rows = kernel_table(max(args.steps, 1))
         print(json.dumps({"metric": "per-kernel roofline at the wide-MLP shape (4096 x 4096 operands)", "device": dev_name,

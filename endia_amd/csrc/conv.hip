@@ -1,12 +1,24 @@
-// conv2d (NCHW, cross-correlation, groups = 1): forward as in Conv2d.__call__
-// (endia/functional/spacial_ops/conv2d_op.mojo:88-196; output shape rule conv2d_op.mojo:31-85) and the
-// three adjoints of that loop. The reference registers no backward rule for conv2d
-// (Conv2d.vjp = default_vjp, conv2d_op.mojo:198-200), so the gradients are defined here as
+// conv2d (NCHW, cross-correlation, groups = 1) as implicit GEMMs on the fp32 matrix cores.
+//
+// Forward follows Conv2d.__call__ (endia/functional/spacial_ops/conv2d_op.mojo:88-196; output shape rule
+// conv2d_op.mojo:31-85):
+//   y[n,k,p,q] = b[k] + sum_{c,r,s} x[n,c, p*sh - ph + r*dh, q*sw - pw + s*dw] * w[k,c,r,s]
+// with out-of-range taps contributing zero. The reference registers no backward rule for conv2d
+// (Conv2d.vjp = default_vjp, conv2d_op.mojo:198-200); the gradients here are the adjoints of that loop:
 //   db[k]       = sum_{n,p,q} dy[n,k,p,q]
 //   dw[k,c,r,s] = sum_{n,p,q} dy[n,k,p,q] * x[n,c, p*sh - ph + r*dh, q*sw - pw + s*dw]
 //   dx[n,c,h,w] = sum_{k,r,s} dy[n,k,p,q] * w[k,c,r,s]  over (p,q) with p*sh - ph + r*dh = h, q*sw - pw + s*dw = w
-// with out-of-range taps contributing zero, exactly as the forward loop skips them.
+//
+// GEMM views (no im2col matrix is ever written; the gather happens on the way into LDS):
+//   forward   C[K, N*P*Q]   = Wp[K, C*R*S]    . col(x)[C*R*S, N*P*Q]
+//   data grad C[C, N*H*W]   = WpT[C, K*R*S]   . col'(dy)[K*R*S, N*H*W]      (transposed convolution)
+//   weight    C[K, C*R*S]   = dy[K, N*P*Q]    . col(x)[C*R*S, N*P*Q]^T      (split over N*P*Q, partials
+//                                                                            summed in a fixed order)
+// Wp / WpT are the weights repacked once per call into a row-padded matrix (a few hundred KiB).
+// The 7-deep scalar loop of the reference becomes: K tile of 32, 128 x 128 (or 64 x 128) tile of C per
+// work-group, v_mfma_f32_32x32x2_f32, the same LDS layouts as the dense GEMM.
 #include "common.h"
+#include "mfma_tile.h"
 
 namespace endia {
 int32_t col_reduce(int64_t batch, int64_t R, int64_t C, const float* x, float* out, float scale);
@@ -15,113 +27,371 @@ int32_t row_reduce(int64_t R, int64_t C, const float* x, float* out, float scale
 
 namespace {
 
+using namespace mfma;
+
 constexpr int TPB = 256;
+constexpr int FAR = -(1 << 28);  // coordinate that fails every bounds test
 
 struct ConvP {
   int N, C, H, W, K, R, S, P, Q;
   int sh, sw, ph, pw, dh, dw;
 };
 
-__device__ __forceinline__ float wave_sum(float v) {
-#pragma unroll
-  for (int off = 32; off > 0; off >>= 1) v += __shfl_down(v, off, 64);
-  return v;
-}
+enum { MODE_FWD = 0, MODE_BWD_DATA = 1 };
 
-// one lane per output element; consecutive lanes walk q, so x reads and y writes coalesce
-__global__ __launch_bounds__(TPB) void conv_fwd_direct_kernel(ConvP p, const float* __restrict__ x,
-                                                              const float* __restrict__ w, const float* __restrict__ bias,
-                                                              float* __restrict__ y, int relu) {
-  int64_t total = (int64_t)p.N * p.K * p.P * p.Q;
-  int64_t stride = (int64_t)gridDim.x * TPB;
-  for (int64_t idx = (int64_t)blockIdx.x * TPB + threadIdx.x; idx < total; idx += stride) {
-    int q = (int)(idx % p.Q);
-    int64_t t = idx / p.Q;
-    int pp = (int)(t % p.P);
-    t /= p.P;
-    int k = (int)(t % p.K);
-    int n = (int)(t / p.K);
-    float acc = 0.f;
-    const int h0 = pp * p.sh - p.ph, w0 = q * p.sw - p.pw;
-    for (int c = 0; c < p.C; ++c) {
-      const float* xc = x + ((int64_t)n * p.C + c) * p.H * p.W;
-      const float* wc = w + ((int64_t)k * p.C + c) * p.R * p.S;
-      for (int r = 0; r < p.R; ++r) {
-        int h = h0 + r * p.dh;
-        if (h < 0 || h >= p.H) continue;
-        for (int s = 0; s < p.S; ++s) {
-          int ww = w0 + s * p.dw;
-          if (ww < 0 || ww >= p.W) continue;
-          acc = fmaf(xc[(int64_t)h * p.W + ww], wc[r * p.S + s], acc);
+// ---- forward and data gradient ------------------------------------------------------------------
+struct IgemmArgs {
+  const float* src;   // fwd: x [N,C,H,W]; data grad: dy [N,K,P,Q]
+  const float* wp;    // packed weights [Mrows, Kd_pad]
+  const float* bias;  // fwd: [K] or null
+  float* out;         // fwd: y; data grad: dx
+  int Mrows, Cred;    // output channels of this GEMM; channels reduced over
+  int SH, SW, OH, OW; // source and output spatial extents
+  int Kd, Kd_pad;     // Cred*R*S and its multiple-of-4 padding
+  int Ncols;          // N*OH*OW
+  int R, S, sh, sw, ph, pw, dh, dw;
+  FastDiv d_rs, d_s, d_ohw, d_ow, d_sh, d_sw;
+  int tiles_m, tiles_n, relu;
+  int64_t src_bytes;
+};
+
+// B operand: rows = reduction index t = (ch, r, s), columns = output pixels j = (n, oy, ox).
+// A lane owns 4 consecutive columns for the whole kernel (decoded once) and PASSES rows per K tile.
+template <int MODE, int BN, int NT>
+struct GatherColsLoader {
+  static constexpr int F4_PER_ROW = BN / 4;
+  static constexpr int ROWS_PER_PASS = NT / F4_PER_ROW;
+  static constexpr int PASSES = BK / ROWS_PER_PASS;
+  static constexpr int LD = TileShape<false, BN>::LD;
+  int base[4], y0[4], x0[4];
+  int r, lds_off;
+  float reg[PASSES][4];
+
+  __device__ __forceinline__ void init(const IgemmArgs& a, int n0, int tid) {
+    r = tid / F4_PER_ROW;
+    const int c4 = (tid % F4_PER_ROW) * 4;
+    lds_off = r * LD + c4;
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      int j = n0 + c4 + e;
+      if (j < a.Ncols) {
+        int n = (int)fdiv((uint32_t)j, a.d_ohw);
+        int rem = j - n * a.OH * a.OW;
+        int oy = (int)fdiv((uint32_t)rem, a.d_ow);
+        int ox = rem - oy * a.OW;
+        base[e] = n * a.Cred * a.SH * a.SW;
+        y0[e] = MODE == MODE_FWD ? oy * a.sh - a.ph : oy + a.ph;
+        x0[e] = MODE == MODE_FWD ? ox * a.sw - a.pw : ox + a.pw;
+      } else {
+        base[e] = 0;
+        y0[e] = FAR;
+        x0[e] = 0;
+      }
+    }
+  }
+  __device__ __forceinline__ void load(const IgemmArgs& a, int k0) {
+    __amdgpu_buffer_rsrc_t rs = make_rsrc(a.src, a.src_bytes);
+#pragma unroll
+    for (int i = 0; i < PASSES; ++i) {
+      int t = k0 + r + i * ROWS_PER_PASS;
+      int ch = (int)fdiv((uint32_t)t, a.d_rs);
+      int rem = t - ch * a.R * a.S;
+      int rr = (int)fdiv((uint32_t)rem, a.d_s);
+      int ss = rem - rr * a.S;
+      int roff = ch * a.SH * a.SW;
+      int dyv = t < a.Kd ? rr * a.dh : (MODE == MODE_FWD ? FAR : -FAR);
+      int dxv = ss * a.dw;
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        int iy, ix;
+        bool ok;
+        if (MODE == MODE_FWD) {
+          iy = y0[e] + dyv;
+          ix = x0[e] + dxv;
+          ok = (unsigned)iy < (unsigned)a.SH && (unsigned)ix < (unsigned)a.SW;
+        } else {
+          int ty = y0[e] - dyv, tx = x0[e] - dxv;
+          if (a.sh == 1 && a.sw == 1) {
+            iy = ty;
+            ix = tx;
+            ok = (unsigned)iy < (unsigned)a.SH && (unsigned)ix < (unsigned)a.SW;
+          } else {
+            ok = ty >= 0 && tx >= 0;
+            iy = (int)fdiv((uint32_t)(ok ? ty : 0), a.d_sh);
+            ix = (int)fdiv((uint32_t)(ok ? tx : 0), a.d_sw);
+            ok = ok && iy * a.sh == ty && ix * a.sw == tx && iy < a.SH && ix < a.SW;
+          }
+        }
+        uint32_t off = ok ? (uint32_t)(base[e] + roff + iy * a.SW + ix) * 4u : OOB_OFFSET;
+        reg[i][e] = buffer_load_f1(rs, off);
+      }
+    }
+  }
+  __device__ __forceinline__ void store(float* lds) {
+#pragma unroll
+    for (int i = 0; i < PASSES; ++i)
+      *reinterpret_cast<float4*>(&lds[lds_off + i * ROWS_PER_PASS * LD]) = make_float4(reg[i][0], reg[i][1], reg[i][2], reg[i][3]);
+  }
+};
+
+template <int MODE, int WGM, int WGN, int FM, int FN>
+__global__ __launch_bounds__(WGM* WGN * 64, 3) void conv_igemm_kernel(IgemmArgs a) {
+  constexpr int NT = WGM * WGN * 64, BM = WGM * FM * 32, BN = WGN * FN * 32;
+  using LA = MatrixTileLoader<true, BM, NT>;
+  using LB = GatherColsLoader<MODE, BN, NT>;
+  __shared__ __attribute__((aligned(16))) float As[TileShape<true, BM>::FLOATS];
+  __shared__ __attribute__((aligned(16))) float Bs[TileShape<false, BN>::FLOATS];
+
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int wm = wave / WGN, wn = wave % WGN;
+  const int l32 = lane & 31, h = lane >> 5;
+  int tm, tn;
+  tile_of_block(blockIdx.x, gridDim.x, a.tiles_m, a.tiles_n, tm, tn);
+  const int m0 = tm * BM, n0 = tn * BN;
+
+  LA la;
+  LB lb;
+  la.init(a.wp, a.Kd_pad, m0, a.Mrows, a.Kd_pad, tid);
+  lb.init(a, n0, tid);
+
+  floatx16 acc[FM][FN];
+  zero_acc<FM, FN>(acc);
+
+  la.load(a.Kd_pad);
+  lb.load(a, 0);
+  la.store(As);
+  lb.store(Bs);
+  __syncthreads();
+
+  for (int k0 = 0; k0 < a.Kd_pad; k0 += BK) {
+    const bool more = k0 + BK < a.Kd_pad;
+    if (more) {
+      la.advance();
+      la.load(a.Kd_pad - k0 - BK);
+      lb.load(a, k0 + BK);
+    }
+    compute_ktile<true, false, FM, FN, BM, BN>(As, Bs, wm * FM * 32 + l32, wn * FN * 32 + l32, h, acc);
+    if (more) {
+      __syncthreads();
+      la.store(As);
+      lb.store(Bs);
+      __syncthreads();
+    }
+  }
+
+  const int64_t ohw = (int64_t)a.OH * a.OW;
+#pragma unroll
+  for (int fn = 0; fn < FN; ++fn) {
+    int j = n0 + wn * FN * 32 + fn * 32 + l32;
+    if (j >= a.Ncols) continue;
+    int n = (int)fdiv((uint32_t)j, a.d_ohw);
+    int64_t col_off = (int64_t)n * a.Mrows * ohw + (j - (int64_t)n * ohw);
+#pragma unroll
+    for (int fm = 0; fm < FM; ++fm)
+#pragma unroll
+      for (int v = 0; v < 16; ++v) {
+        int m = m0 + wm * FM * 32 + fm * 32 + acc_row(v, h);
+        if (m < a.Mrows) {
+          float val = acc[fm][fn][v];
+          if (MODE == MODE_FWD) {
+            if (a.bias) val += a.bias[m];
+            if (a.relu) val = val > 0.f ? val : 0.f;
+          }
+          a.out[col_off + m * ohw] = val;
         }
       }
-    }
-    if (bias) acc += bias[k];
-    if (relu) acc = acc > 0.f ? acc : 0.f;
-    y[idx] = acc;
   }
 }
 
-// one lane per input element: gather form of the transposed convolution
-__global__ __launch_bounds__(TPB) void conv_bwd_data_direct_kernel(ConvP p, const float* __restrict__ dy,
-                                                                   const float* __restrict__ w, float* __restrict__ dx) {
-  int64_t total = (int64_t)p.N * p.C * p.H * p.W;
-  int64_t stride = (int64_t)gridDim.x * TPB;
-  for (int64_t idx = (int64_t)blockIdx.x * TPB + threadIdx.x; idx < total; idx += stride) {
-    int ww = (int)(idx % p.W);
-    int64_t t = idx / p.W;
-    int h = (int)(t % p.H);
-    t /= p.H;
-    int c = (int)(t % p.C);
-    int n = (int)(t / p.C);
-    float acc = 0.f;
-    for (int r = 0; r < p.R; ++r) {
-      int hn = h + p.ph - r * p.dh;
-      if (hn < 0 || hn % p.sh) continue;
-      int pp = hn / p.sh;
-      if (pp >= p.P) continue;
-      for (int s = 0; s < p.S; ++s) {
-        int wn = ww + p.pw - s * p.dw;
-        if (wn < 0 || wn % p.sw) continue;
-        int q = wn / p.sw;
-        if (q >= p.Q) continue;
-        const float* dyp = dy + ((int64_t)n * p.K * p.P + pp) * p.Q + q;
-        const float* wp = w + ((int64_t)c * p.R + r) * p.S + s;
-        for (int k = 0; k < p.K; ++k)
-          acc = fmaf(dyp[(int64_t)k * p.P * p.Q], wp[(int64_t)k * p.C * p.R * p.S], acc);
+// ---- weight gradient ------------------------------------------------------------------------------
+struct WgradArgs {
+  const float* x;
+  const float* dy;
+  float* part;  // [splits][K][Kd]
+  int N, C, H, W, K, R, S, P, Q, sh, sw, ph, pw, dh, dw;
+  int Kd;
+  int total_j, chunk;  // N*P*Q and the slice of it one split reduces over (multiple of 32)
+  FastDiv d_pq, d_q, d_rs, d_s;
+  int tiles_m, tiles_n;
+  int64_t x_bytes, dy_bytes;
+};
+
+// dy as the A operand: rows = output channel k, 32 consecutive j = (n, p, q) per tile.
+template <int BM, int NT>
+struct DyRowsLoader {
+  static constexpr int ROWS_PER_PASS = NT / 8;
+  static constexpr int PASSES = BM / ROWS_PER_PASS;
+  int rowoff[PASSES];  // k * P*Q, or -1 for rows past K
+  int c4, lds_off;
+  float reg[PASSES][4];
+  __device__ __forceinline__ void init(const WgradArgs& a, int m0, int tid) {
+    const int r = tid / 8;
+    c4 = (tid % 8) * 4;
+    lds_off = r * LDK + c4;
+#pragma unroll
+    for (int i = 0; i < PASSES; ++i) {
+      int m = m0 + r + i * ROWS_PER_PASS;
+      rowoff[i] = m < a.K ? m * a.P * a.Q : -1;
+    }
+  }
+  __device__ __forceinline__ void load(const WgradArgs& a, int jt, int j_end) {
+    __amdgpu_buffer_rsrc_t rs = make_rsrc(a.dy, a.dy_bytes);
+    const int pq_n = a.P * a.Q;
+    int j = jt + c4;
+    int n = (int)fdiv((uint32_t)j, a.d_pq);
+    int pq = j - n * pq_n;
+    int off[4];
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      off[e] = (j + e < j_end) ? n * a.K * pq_n + pq : -1;
+      if (++pq == pq_n) { pq = 0; ++n; }
+    }
+#pragma unroll
+    for (int i = 0; i < PASSES; ++i)
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        bool ok = rowoff[i] >= 0 && off[e] >= 0;
+        reg[i][e] = buffer_load_f1(rs, ok ? (uint32_t)(off[e] + rowoff[i]) * 4u : OOB_OFFSET);
       }
+  }
+  __device__ __forceinline__ void store(float* lds) {
+#pragma unroll
+    for (int i = 0; i < PASSES; ++i)
+      *reinterpret_cast<float4*>(&lds[lds_off + i * ROWS_PER_PASS * LDK]) = make_float4(reg[i][0], reg[i][1], reg[i][2], reg[i][3]);
+  }
+};
+
+// col(x) as the B operand: rows = filter tap t = (c, r, s), 32 consecutive j per tile.
+template <int BN, int NT>
+struct TapRowsLoader {
+  static constexpr int ROWS_PER_PASS = NT / 8;
+  static constexpr int PASSES = BN / ROWS_PER_PASS;
+  int roff[PASSES], dyv[PASSES], dxv[PASSES];
+  int c4, lds_off;
+  float reg[PASSES][4];
+  __device__ __forceinline__ void init(const WgradArgs& a, int n0, int tid) {
+    const int r = tid / 8;
+    c4 = (tid % 8) * 4;
+    lds_off = r * LDK + c4;
+#pragma unroll
+    for (int i = 0; i < PASSES; ++i) {
+      int t = n0 + r + i * ROWS_PER_PASS;
+      int ch = (int)fdiv((uint32_t)t, a.d_rs);
+      int rem = t - ch * a.R * a.S;
+      int rr = (int)fdiv((uint32_t)rem, a.d_s);
+      int ss = rem - rr * a.S;
+      roff[i] = ch * a.H * a.W;
+      dyv[i] = t < a.Kd ? rr * a.dh - a.ph : FAR;
+      dxv[i] = ss * a.dw - a.pw;
     }
-    dx[idx] = acc;
+  }
+  __device__ __forceinline__ void load(const WgradArgs& a, int jt, int j_end) {
+    __amdgpu_buffer_rsrc_t rs = make_rsrc(a.x, a.x_bytes);
+    int j = jt + c4;
+    int n = (int)fdiv((uint32_t)j, a.d_pq);
+    int rem = j - n * a.P * a.Q;
+    int p = (int)fdiv((uint32_t)rem, a.d_q);
+    int q = rem - p * a.Q;
+    int base[4], ye[4], xe[4];
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      base[e] = n * a.C * a.H * a.W;
+      ye[e] = (j + e < j_end) ? p * a.sh : FAR;
+      xe[e] = q * a.sw;
+      if (++q == a.Q) { q = 0; if (++p == a.P) { p = 0; ++n; } }
+    }
+#pragma unroll
+    for (int i = 0; i < PASSES; ++i)
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        int iy = ye[e] + dyv[i], ix = xe[e] + dxv[i];
+        bool ok = (unsigned)iy < (unsigned)a.H && (unsigned)ix < (unsigned)a.W;
+        reg[i][e] = buffer_load_f1(rs, ok ? (uint32_t)(base[e] + roff[i] + iy * a.W + ix) * 4u : OOB_OFFSET);
+      }
+  }
+  __device__ __forceinline__ void store(float* lds) {
+#pragma unroll
+    for (int i = 0; i < PASSES; ++i)
+      *reinterpret_cast<float4*>(&lds[lds_off + i * ROWS_PER_PASS * LDK]) = make_float4(reg[i][0], reg[i][1], reg[i][2], reg[i][3]);
+  }
+};
+
+template <int WGM, int WGN, int FM, int FN>
+__global__ __launch_bounds__(WGM* WGN * 64, 2) void conv_wgrad_kernel(WgradArgs a) {
+  constexpr int NT = WGM * WGN * 64, BM = WGM * FM * 32, BN = WGN * FN * 32;
+  using LA = DyRowsLoader<BM, NT>;
+  using LB = TapRowsLoader<BN, NT>;
+  __shared__ __attribute__((aligned(16))) float As[TileShape<true, BM>::FLOATS];
+  __shared__ __attribute__((aligned(16))) float Bs[TileShape<true, BN>::FLOATS];
+
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int wm = wave / WGN, wn = wave % WGN;
+  const int l32 = lane & 31, h = lane >> 5;
+  const int tm = blockIdx.x / a.tiles_n, tn = blockIdx.x % a.tiles_n;
+  const int m0 = tm * BM, n0 = tn * BN;
+  const int split = blockIdx.y;
+  const int j_begin = split * a.chunk;
+  const int j_end = j_begin + a.chunk < a.total_j ? j_begin + a.chunk : a.total_j;
+
+  LA la;
+  LB lb;
+  la.init(a, m0, tid);
+  lb.init(a, n0, tid);
+  floatx16 acc[FM][FN];
+  zero_acc<FM, FN>(acc);
+
+  la.load(a, j_begin, j_end);
+  lb.load(a, j_begin, j_end);
+  la.store(As);
+  lb.store(Bs);
+  __syncthreads();
+  for (int jt = j_begin; jt < j_end; jt += BK) {
+    const bool more = jt + BK < j_end;
+    if (more) {
+      la.load(a, jt + BK, j_end);
+      lb.load(a, jt + BK, j_end);
+    }
+    compute_ktile<true, true, FM, FN, BM, BN>(As, Bs, wm * FM * 32 + l32, wn * FN * 32 + l32, h, acc);
+    if (more) {
+      __syncthreads();
+      la.store(As);
+      lb.store(Bs);
+      __syncthreads();
+    }
+  }
+
+  float* out = a.part + (int64_t)split * a.K * a.Kd;
+#pragma unroll
+  for (int fn = 0; fn < FN; ++fn) {
+    int t = n0 + wn * FN * 32 + fn * 32 + l32;
+    if (t >= a.Kd) continue;
+#pragma unroll
+    for (int fm = 0; fm < FM; ++fm)
+#pragma unroll
+      for (int v = 0; v < 16; ++v) {
+        int m = m0 + wm * FM * 32 + fm * 32 + acc_row(v, h);
+        if (m < a.K) out[(int64_t)m * a.Kd + t] = acc[fm][fn][v];
+      }
   }
 }
 
-// one work-group per filter tap (k,c,r,s): lanes stride over (n,p,q)
-__global__ __launch_bounds__(TPB) void conv_bwd_weight_direct_kernel(ConvP p, const float* __restrict__ x,
-                                                                     const float* __restrict__ dy, float* __restrict__ dw) {
-  __shared__ float red[4];
-  int64_t tap = blockIdx.x;
-  int s = (int)(tap % p.S);
-  int64_t t = tap / p.S;
-  int r = (int)(t % p.R);
-  t /= p.R;
-  int c = (int)(t % p.C);
-  int k = (int)(t / p.C);
-  const int64_t PQ = (int64_t)p.P * p.Q;
-  const int64_t total = (int64_t)p.N * PQ;
-  float acc = 0.f;
-  for (int64_t j = threadIdx.x; j < total; j += TPB) {
-    int n = (int)(j / PQ);
-    int rem = (int)(j - (int64_t)n * PQ);
-    int pp = rem / p.Q, q = rem - pp * p.Q;
-    int h = pp * p.sh - p.ph + r * p.dh, ww = q * p.sw - p.pw + s * p.dw;
-    if (h < 0 || h >= p.H || ww < 0 || ww >= p.W) continue;
-    acc = fmaf(dy[((int64_t)n * p.K + k) * PQ + rem], x[(((int64_t)n * p.C + c) * p.H + h) * p.W + ww], acc);
+// ---- weight repacking -------------------------------------------------------------------------------
+// fwd:  wp[k][t]        = w[k][t]                       t = (c, r, s), rows padded to Kd_pad with zeros
+// data: wp[c][(k,r,s)]  = w[k][c][r][s]
+__global__ __launch_bounds__(TPB) void pack_weights_kernel(const float* __restrict__ w, float* __restrict__ wp, int K, int C,
+                                                           int RS, int Kd_pad, int transpose) {
+  const int rows = transpose ? C : K;
+  const int64_t total = (int64_t)rows * Kd_pad;
+  const int kd = (transpose ? K : C) * RS;
+  for (int64_t i = (int64_t)blockIdx.x * TPB + threadIdx.x; i < total; i += (int64_t)gridDim.x * TPB) {
+    int m = (int)(i / Kd_pad), t = (int)(i - (int64_t)m * Kd_pad);
+    float v = 0.f;
+    if (t < kd) {
+      if (!transpose) v = w[(int64_t)m * kd + t];
+      else { int k = t / RS, rs = t - k * RS; v = w[((int64_t)k * C + m) * RS + rs]; }
+    }
+    wp[i] = v;
   }
-  acc = wave_sum(acc);
-  int lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
-  if (lane == 0) red[wv] = acc;
-  __syncthreads();
-  if (threadIdx.x == 0) dw[tap] = (red[0] + red[1]) + (red[2] + red[3]);
 }
 
 int32_t make_params(const endia_hip_conv2d_desc* d, ConvP& p) {
@@ -132,13 +402,14 @@ int32_t make_params(const endia_hip_conv2d_desc* d, ConvP& p) {
     return endia::fail(ENDIA_HIP_ERR_INVALID, "conv2d: bad stride, dilation or padding");
   if (d->groups != 1)
     return endia::fail(ENDIA_HIP_ERR_UNSUPPORTED, "conv2d: groups = %lld; only groups = 1 is implemented", (long long)d->groups);
-  int64_t P = (d->H + 2 * d->pad_h - d->dil_h * (d->R - 1) - 1) / d->stride_h + 1;
-  int64_t Q = (d->W + 2 * d->pad_w - d->dil_w * (d->S - 1) - 1) / d->stride_w + 1;
-  if (d->H + 2 * d->pad_h - d->dil_h * (d->R - 1) - 1 < 0 || d->W + 2 * d->pad_w - d->dil_w * (d->S - 1) - 1 < 0)
-    return endia::fail(ENDIA_HIP_ERR_INVALID, "conv2d: kernel larger than padded input");
-  const int64_t lim = 1ll << 31;
-  if (d->N * d->C * d->H * d->W >= lim * 4 || d->N * d->K * P * Q >= lim * 4 || d->K * d->C * d->R * d->S >= lim)
-    return endia::fail(ENDIA_HIP_ERR_UNSUPPORTED, "conv2d: tensor too large");
+  int64_t eh = d->H + 2 * d->pad_h - d->dil_h * (d->R - 1) - 1, ew = d->W + 2 * d->pad_w - d->dil_w * (d->S - 1) - 1;
+  if (eh < 0 || ew < 0) return endia::fail(ENDIA_HIP_ERR_INVALID, "conv2d: kernel larger than padded input");
+  int64_t P = eh / d->stride_h + 1, Q = ew / d->stride_w + 1;
+  // element offsets are 32-bit with 4-byte scaling inside the gathers: every tensor must stay below 2^29 elements
+  const int64_t lim = 1ll << 29;
+  if (d->N * d->C * d->H * d->W >= lim || d->N * d->K * P * Q >= lim || d->K * d->C * d->R * d->S >= lim ||
+      d->pad_h >= (1 << 20) || d->pad_w >= (1 << 20) || d->dil_h * d->R >= (1 << 20) || d->dil_w * d->S >= (1 << 20))
+    return endia::fail(ENDIA_HIP_ERR_UNSUPPORTED, "conv2d: tensor has 2^29 elements or more");
   p.N = (int)d->N; p.C = (int)d->C; p.H = (int)d->H; p.W = (int)d->W; p.K = (int)d->K; p.R = (int)d->R; p.S = (int)d->S;
   p.P = (int)P; p.Q = (int)Q;
   p.sh = (int)d->stride_h; p.sw = (int)d->stride_w; p.ph = (int)d->pad_h; p.pw = (int)d->pad_w;
@@ -146,10 +417,55 @@ int32_t make_params(const endia_hip_conv2d_desc* d, ConvP& p) {
   return ENDIA_HIP_OK;
 }
 
-inline int grid_for(int64_t n) {
-  int64_t b = ceil_div64(n, TPB), cap = (int64_t)endia::ctx().cu_count * 16;
-  if (b > cap) b = cap;
-  return (int)(b < 1 ? 1 : b);
+struct PoolBuf {  // scratch from the library's pool, returned on scope exit (stream-ordered reuse)
+  void* p = nullptr;
+  ~PoolBuf() { if (p) endia_hip_free(p); }
+};
+
+int32_t run_igemm(int mode, const ConvP& p, const float* src, const float* w, const float* bias, float* out, int relu) {
+  hipStream_t s = endia::ctx().stream;
+  IgemmArgs a;
+  const bool fwd = mode == MODE_FWD;
+  a.src = src; a.bias = bias; a.out = out; a.relu = relu;
+  a.Mrows = fwd ? p.K : p.C;
+  a.Cred = fwd ? p.C : p.K;
+  a.SH = fwd ? p.H : p.P; a.SW = fwd ? p.W : p.Q;
+  a.OH = fwd ? p.P : p.H; a.OW = fwd ? p.Q : p.W;
+  a.Kd = a.Cred * p.R * p.S;
+  a.Kd_pad = (a.Kd + 3) / 4 * 4;
+  a.Ncols = p.N * a.OH * a.OW;
+  a.R = p.R; a.S = p.S; a.sh = p.sh; a.sw = p.sw; a.ph = p.ph; a.pw = p.pw; a.dh = p.dh; a.dw = p.dw;
+  a.d_rs = make_fastdiv(p.R * p.S); a.d_s = make_fastdiv(p.S);
+  a.d_ohw = make_fastdiv(a.OH * a.OW); a.d_ow = make_fastdiv(a.OW);
+  a.d_sh = make_fastdiv(p.sh); a.d_sw = make_fastdiv(p.sw);
+  a.src_bytes = (int64_t)p.N * a.Cred * a.SH * a.SW * 4;
+
+  PoolBuf wp;
+  int32_t rc = endia_hip_malloc((int64_t)a.Mrows * a.Kd_pad * 4, &wp.p);
+  if (rc) return rc;
+  {
+    int64_t total = (int64_t)a.Mrows * a.Kd_pad;
+    int blocks = (int)((total + TPB - 1) / TPB);
+    if (blocks > 2048) blocks = 2048;
+    hipLaunchKernelGGL(pack_weights_kernel, dim3(blocks), dim3(TPB), 0, s, w, static_cast<float*>(wp.p), p.K, p.C,
+                       p.R * p.S, a.Kd_pad, fwd ? 0 : 1);
+    ENDIA_LAUNCH_CHECK();
+  }
+  a.wp = static_cast<const float*>(wp.p);
+  a.tiles_n = (a.Ncols + 127) / 128;
+  if (a.Mrows > 64) {
+    a.tiles_m = (a.Mrows + 127) / 128;
+    dim3 grid((unsigned)(a.tiles_m * a.tiles_n));
+    if (fwd) hipLaunchKernelGGL((conv_igemm_kernel<MODE_FWD, 2, 2, 2, 2>), grid, dim3(256), 0, s, a);
+    else hipLaunchKernelGGL((conv_igemm_kernel<MODE_BWD_DATA, 2, 2, 2, 2>), grid, dim3(256), 0, s, a);
+  } else {  // up to 64 output channels: a 64 x 128 tile wastes no MFMA rows
+    a.tiles_m = 1;
+    dim3 grid((unsigned)a.tiles_n);
+    if (fwd) hipLaunchKernelGGL((conv_igemm_kernel<MODE_FWD, 1, 4, 2, 1>), grid, dim3(256), 0, s, a);
+    else hipLaunchKernelGGL((conv_igemm_kernel<MODE_BWD_DATA, 1, 4, 2, 1>), grid, dim3(256), 0, s, a);
+  }
+  ENDIA_LAUNCH_CHECK();
+  return ENDIA_HIP_OK;
 }
 
 }  // namespace
@@ -175,13 +491,9 @@ int32_t endia_hip_conv2d_fwd(const endia_hip_conv2d_desc* d, const float* x, con
   int32_t rc = make_params(d, p);
   if (rc) return rc;
   ENDIA_CHECK_ARG(act == ENDIA_OP_IDENTITY || act == ENDIA_OP_RELU, "endia_hip_conv2d_fwd: activation must be identity or relu");
-  int64_t total = (int64_t)p.N * p.K * p.P * p.Q;
-  if (total == 0) return ENDIA_HIP_OK;
+  if ((int64_t)p.N * p.K * p.P * p.Q == 0) return ENDIA_HIP_OK;
   ENDIA_CHECK_ARG(x && w && y, "endia_hip_conv2d_fwd: null pointer");
-  hipLaunchKernelGGL(conv_fwd_direct_kernel, dim3(grid_for(total)), dim3(TPB), 0, ctx().stream, p, x, w, bias, y,
-                     act == ENDIA_OP_RELU ? 1 : 0);
-  ENDIA_LAUNCH_CHECK();
-  return ENDIA_HIP_OK;
+  return run_igemm(MODE_FWD, p, x, w, bias, y, act == ENDIA_OP_RELU ? 1 : 0);
 }
 
 int32_t endia_hip_conv2d_bwd_data(const endia_hip_conv2d_desc* d, const float* dy, const float* w, float* dx) {
@@ -191,10 +503,10 @@ int32_t endia_hip_conv2d_bwd_data(const endia_hip_conv2d_desc* d, const float* d
   if (rc) return rc;
   int64_t total = (int64_t)p.N * p.C * p.H * p.W;
   if (total == 0) return ENDIA_HIP_OK;
-  ENDIA_CHECK_ARG(dy && w && dx, "endia_hip_conv2d_bwd_data: null pointer");
-  hipLaunchKernelGGL(conv_bwd_data_direct_kernel, dim3(grid_for(total)), dim3(TPB), 0, ctx().stream, p, dy, w, dx);
-  ENDIA_LAUNCH_CHECK();
-  return ENDIA_HIP_OK;
+  ENDIA_CHECK_ARG(dx != nullptr, "endia_hip_conv2d_bwd_data: dx is null");
+  if ((int64_t)p.P * p.Q == 0) return endia_hip_fill(dx, total, 0.f);
+  ENDIA_CHECK_ARG(dy && w, "endia_hip_conv2d_bwd_data: null pointer");
+  return run_igemm(MODE_BWD_DATA, p, dy, w, nullptr, dx, 0);
 }
 
 int32_t endia_hip_conv2d_bwd_weight(const endia_hip_conv2d_desc* d, const float* x, const float* dy, float* dw) {
@@ -202,12 +514,49 @@ int32_t endia_hip_conv2d_bwd_weight(const endia_hip_conv2d_desc* d, const float*
   ConvP p;
   int32_t rc = make_params(d, p);
   if (rc) return rc;
-  int64_t taps = (int64_t)p.K * p.C * p.R * p.S;
+  const int Kd = p.C * p.R * p.S;
+  const int64_t taps = (int64_t)p.K * Kd;
   ENDIA_CHECK_ARG(dw != nullptr, "endia_hip_conv2d_bwd_weight: dw is null");
-  if ((int64_t)p.N * p.P * p.Q == 0) return endia_hip_fill(dw, taps, 0.f);
+  const int64_t total_j = (int64_t)p.N * p.P * p.Q;
+  if (total_j == 0) return endia_hip_fill(dw, taps, 0.f);
   ENDIA_CHECK_ARG(x && dy, "endia_hip_conv2d_bwd_weight: null pointer");
-  hipLaunchKernelGGL(conv_bwd_weight_direct_kernel, dim3((unsigned)taps), dim3(TPB), 0, ctx().stream, p, x, dy, dw);
+  hipStream_t s = ctx().stream;
+
+  WgradArgs a;
+  a.x = x; a.dy = dy;
+  a.N = p.N; a.C = p.C; a.H = p.H; a.W = p.W; a.K = p.K; a.R = p.R; a.S = p.S; a.P = p.P; a.Q = p.Q;
+  a.sh = p.sh; a.sw = p.sw; a.ph = p.ph; a.pw = p.pw; a.dh = p.dh; a.dw = p.dw;
+  a.Kd = Kd;
+  a.total_j = (int)total_j;
+  a.d_pq = make_fastdiv(p.P * p.Q); a.d_q = make_fastdiv(p.Q);
+  a.d_rs = make_fastdiv(p.R * p.S); a.d_s = make_fastdiv(p.S);
+  a.x_bytes = (int64_t)p.N * p.C * p.H * p.W * 4;
+  a.dy_bytes = (int64_t)p.N * p.K * p.P * p.Q * 4;
+  a.tiles_m = (p.K + 127) / 128;
+  a.tiles_n = (Kd + 127) / 128;
+  // split the N*P*Q reduction so that about 4 work-groups per CU exist; every split reduces >= 256 columns
+  int64_t tiles = (int64_t)a.tiles_m * a.tiles_n;
+  int64_t splits = ((int64_t)ctx().cu_count * 4 + tiles - 1) / tiles;
+  int64_t max_splits = (total_j + 255) / 256;
+  if (splits > max_splits) splits = max_splits;
+  if (splits > 1024) splits = 1024;
+  if (splits < 1) splits = 1;
+  int64_t chunk = ((total_j + splits - 1) / splits + 31) / 32 * 32;
+  splits = (total_j + chunk - 1) / chunk;
+  a.chunk = (int)chunk;
+
+  PoolBuf part;
+  if (splits > 1) {
+    rc = endia_hip_malloc(splits * taps * 4, &part.p);
+    if (rc) return rc;
+    a.part = static_cast<float*>(part.p);
+  } else {
+    a.part = dw;
+  }
+  dim3 grid((unsigned)tiles, (unsigned)splits);
+  hipLaunchKernelGGL((conv_wgrad_kernel<2, 2, 2, 2>), grid, dim3(256), 0, s, a);
   ENDIA_LAUNCH_CHECK();
+  if (splits > 1) return col_reduce(1, splits, taps, a.part, dw, 1.f);  // partials added in split order
   return ENDIA_HIP_OK;
 }
 
@@ -222,12 +571,11 @@ int32_t endia_hip_conv2d_bwd_bias(const endia_hip_conv2d_desc* d, const float* d
   ENDIA_CHECK_ARG(dy != nullptr, "endia_hip_conv2d_bwd_bias: dy is null");
   ENDIA_CHECK_ARG(rows <= 65535, "endia_hip_conv2d_bwd_bias: N*K = %lld exceeds 65535", (long long)rows);
   // [N*K, P*Q] -> [N*K] with wave-shuffle row sums, then [N, K] -> [K]
-  void* tmp = nullptr;
-  rc = endia_hip_malloc(rows * (int64_t)sizeof(float), &tmp);
+  PoolBuf tmp;
+  rc = endia_hip_malloc(rows * (int64_t)sizeof(float), &tmp.p);
   if (rc) return rc;
-  rc = row_reduce(rows, PQ, dy, static_cast<float*>(tmp), 1.f);
-  if (!rc) rc = col_reduce(1, p.N, p.K, static_cast<float*>(tmp), db, 1.f);
-  endia_hip_free(tmp);  // stream-ordered: later users of the buffer run after the kernels above
+  rc = row_reduce(rows, PQ, dy, static_cast<float*>(tmp.p), 1.f);
+  if (!rc) rc = col_reduce(1, p.N, p.K, static_cast<float*>(tmp.p), db, 1.f);
   return rc;
 }
 

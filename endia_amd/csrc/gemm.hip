@@ -8,8 +8,9 @@
 //
 // Tiling: a 256-thread work-group (four 64-lane waves, 2 x 2) owns a 128 x 128 tile of C; each
 // wave owns 64 x 64 as 2 x 2 MFMA blocks of 32 x 32 (64 accumulator registers per lane). The K
-// loop advances 32 at a time: the next tile's global loads are issued into registers before the
-// MFMAs of the current tile and written to LDS after them.
+// loop advances 32 at a time: the next tile's global loads (buffer loads, bounds-checked by their
+// descriptor) are issued into registers before the MFMAs of the current tile and written to LDS
+// after them. 128 registers per lane and 36 KiB of LDS per group give 4 groups per CU.
 //
 // LDS layouts. An operand whose K index is contiguous in memory ("K-major": A when transA = 0,
 // B when transB = 1) is stored [row][32 + 4] and fetched with one 128-bit read per four MFMA
@@ -19,16 +20,15 @@
 // k = 8j + 4h + i for half-wave h, which is what makes the 128-bit fetch possible. Both
 // operands use the same mapping.
 #include "common.h"
+#include "mfma_tile.h"
 
 #include <vector>
 
-typedef float floatx16 __attribute__((ext_vector_type(16)));
-
 namespace {
 
-constexpr int BM = 128, BN = 128, BK = 32;
-constexpr int LDK = BK + 4;   // row stride of a K-major tile (floats)
-constexpr int LDM = BM + 8;   // row stride of an MN-major tile (floats)
+using namespace mfma;
+
+constexpr int BM = 128, BN = 128;
 constexpr int NTHREADS = 256;
 
 struct GemmArgs {
@@ -86,31 +86,12 @@ __device__ __forceinline__ void epilogue_store(const GemmArgs& p, float* __restr
   C[off] = v;
 }
 
-// Map the linear work-group id to a tile. Work-groups are dealt round-robin to the 8 XCDs, each
-// with a private L2, so first give every XCD a contiguous range of tile ids, then walk that range
-// in column-major order inside bands of 8 tile-rows so that concurrently resident tiles share
-// A-rows and B-columns.
-__device__ __forceinline__ void tile_of_block(int bid, int nblocks, int tiles_m, int tiles_n, int& tm,
-                                              int& tn) {
-  int lid = bid;
-  if ((nblocks & 7) == 0) {
-    int per = nblocks >> 3;
-    lid = (bid & 7) * per + (bid >> 3);
-  }
-  const int GM = 8;
-  int band = GM * tiles_n;
-  int g = lid / band;
-  int first_m = g * GM;
-  int gsz = tiles_m - first_m < GM ? tiles_m - first_m : GM;
-  int r = lid - g * band;
-  tm = first_m + r % gsz;
-  tn = r / gsz;
-}
-
 template <bool A_KMAJOR, bool B_KMAJOR, int EPI>
-__global__ __launch_bounds__(NTHREADS, 2) void sgemm_mfma_kernel(GemmArgs p) {
-  __shared__ __attribute__((aligned(16))) float As[A_KMAJOR ? BM * LDK : BK * LDM];
-  __shared__ __attribute__((aligned(16))) float Bs[B_KMAJOR ? BN * LDK : BK * LDM];
+__global__ __launch_bounds__(NTHREADS, 4) void sgemm_mfma_kernel(GemmArgs p) {
+  using LA = MatrixTileLoader<A_KMAJOR, BM, NTHREADS>;
+  using LB = MatrixTileLoader<B_KMAJOR, BN, NTHREADS>;
+  __shared__ __attribute__((aligned(16))) float As[TileShape<A_KMAJOR, BM>::FLOATS];
+  __shared__ __attribute__((aligned(16))) float Bs[TileShape<B_KMAJOR, BN>::FLOATS];
 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
@@ -122,114 +103,41 @@ __global__ __launch_bounds__(NTHREADS, 2) void sgemm_mfma_kernel(GemmArgs p) {
   tile_of_block(blockIdx.x, gridDim.x, p.tiles_m, p.tiles_n, tm, tn);
   const int m0 = tm * BM, n0 = tn * BN;
   const int64_t bz = blockIdx.y;
-  const float* __restrict__ A = p.A + bz * p.sA;
-  const float* __restrict__ B = p.B + bz * p.sB;
   float* __restrict__ C = p.C + bz * p.sC;
   const float* __restrict__ aux_in = p.aux_in ? p.aux_in + bz * p.sC : nullptr;
   float* __restrict__ aux_out = p.aux_out ? p.aux_out + bz * p.sC : nullptr;
 
-  // ---- global -> register staging ---------------------------------------------------------
-  // K-major tile: thread covers rows r0 + 32*i (i < 4), floats [kq*4, kq*4+4) of the 32-wide slab.
-  // MN-major tile: thread covers k rows k0 + 8*i (i < 4), floats [mq*4, mq*4+4) of the 128-wide row.
-  float4 ra[4], rb[4];
-  const int a_r = A_KMAJOR ? (tid >> 3) : (tid >> 5);
-  const int a_c = A_KMAJOR ? (tid & 7) * 4 : (tid & 31) * 4;
-  const int b_r = B_KMAJOR ? (tid >> 3) : (tid >> 5);
-  const int b_c = B_KMAJOR ? (tid & 7) * 4 : (tid & 31) * 4;
-
-  auto load_tiles = [&](int k0) {
-#pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      if (A_KMAJOR) {
-        int m = m0 + a_r + 32 * i, k = k0 + a_c;
-        ra[i] = (m < p.M && k < p.K) ? *reinterpret_cast<const float4*>(A + (int64_t)m * p.lda + k)
-                                     : make_float4(0.f, 0.f, 0.f, 0.f);
-      } else {
-        int k = k0 + a_r + 8 * i, m = m0 + a_c;
-        ra[i] = (k < p.K && m < p.M) ? *reinterpret_cast<const float4*>(A + (int64_t)k * p.lda + m)
-                                     : make_float4(0.f, 0.f, 0.f, 0.f);
-      }
-      if (B_KMAJOR) {
-        int n = n0 + b_r + 32 * i, k = k0 + b_c;
-        rb[i] = (n < p.N && k < p.K) ? *reinterpret_cast<const float4*>(B + (int64_t)n * p.ldb + k)
-                                     : make_float4(0.f, 0.f, 0.f, 0.f);
-      } else {
-        int k = k0 + b_r + 8 * i, n = n0 + b_c;
-        rb[i] = (k < p.K && n < p.N) ? *reinterpret_cast<const float4*>(B + (int64_t)k * p.ldb + n)
-                                     : make_float4(0.f, 0.f, 0.f, 0.f);
-      }
-    }
-  };
-  auto store_tiles = [&]() {
-#pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      if (A_KMAJOR)
-        *reinterpret_cast<float4*>(&As[(a_r + 32 * i) * LDK + a_c]) = ra[i];
-      else
-        *reinterpret_cast<float4*>(&As[(a_r + 8 * i) * LDM + a_c]) = ra[i];
-      if (B_KMAJOR)
-        *reinterpret_cast<float4*>(&Bs[(b_r + 32 * i) * LDK + b_c]) = rb[i];
-      else
-        *reinterpret_cast<float4*>(&Bs[(b_r + 8 * i) * LDM + b_c]) = rb[i];
-    }
-  };
+  LA la;
+  LB lb;
+  la.init(p.A + bz * p.sA, p.lda, m0, p.M, p.K, tid);
+  lb.init(p.B + bz * p.sB, p.ldb, n0, p.N, p.K, tid);
 
   floatx16 acc[2][2];
-#pragma unroll
-  for (int i = 0; i < 2; ++i)
-#pragma unroll
-    for (int j = 0; j < 2; ++j)
-#pragma unroll
-      for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.f;
+  zero_acc<2, 2>(acc);
 
-  const int a_row = wm * 64 + l32;  // + 32*fm
-  const int b_col = wn * 64 + l32;  // + 32*fn
-
-  load_tiles(0);
-  store_tiles();
+  la.load(p.K);
+  lb.load(p.K);
+  la.store(As);
+  lb.store(Bs);
   __syncthreads();
 
   for (int k0 = 0; k0 < p.K; k0 += BK) {
     const bool more = k0 + BK < p.K;
-    if (more) load_tiles(k0 + BK);
-
-#pragma unroll
-    for (int j = 0; j < BK / 8; ++j) {
-      float af[2][4], bf[2][4];
-#pragma unroll
-      for (int f = 0; f < 2; ++f) {
-        if (A_KMAJOR) {
-          float4 t = *reinterpret_cast<const float4*>(&As[(a_row + 32 * f) * LDK + 8 * j + 4 * h]);
-          af[f][0] = t.x; af[f][1] = t.y; af[f][2] = t.z; af[f][3] = t.w;
-        } else {
-#pragma unroll
-          for (int i = 0; i < 4; ++i) af[f][i] = As[(8 * j + 4 * h + i) * LDM + a_row + 32 * f];
-        }
-        if (B_KMAJOR) {
-          float4 t = *reinterpret_cast<const float4*>(&Bs[(b_col + 32 * f) * LDK + 8 * j + 4 * h]);
-          bf[f][0] = t.x; bf[f][1] = t.y; bf[f][2] = t.z; bf[f][3] = t.w;
-        } else {
-#pragma unroll
-          for (int i = 0; i < 4; ++i) bf[f][i] = Bs[(8 * j + 4 * h + i) * LDM + b_col + 32 * f];
-        }
-      }
-#pragma unroll
-      for (int i = 0; i < 4; ++i)
-#pragma unroll
-        for (int fm = 0; fm < 2; ++fm)
-#pragma unroll
-          for (int fn = 0; fn < 2; ++fn)
-            acc[fm][fn] = __builtin_amdgcn_mfma_f32_32x32x2f32(af[fm][i], bf[fn][i], acc[fm][fn], 0, 0, 0);
+    if (more) {  // next tile: global -> registers, in flight during this tile's MFMAs
+      la.advance();
+      lb.advance();
+      la.load(p.K - k0 - BK);
+      lb.load(p.K - k0 - BK);
     }
-
+    compute_ktile<A_KMAJOR, B_KMAJOR, 2, 2, BM, BN>(As, Bs, wm * 64 + l32, wn * 64 + l32, h, acc);
     if (more) {
       __syncthreads();
-      store_tiles();
+      la.store(As);
+      lb.store(Bs);
       __syncthreads();
     }
   }
 
-  // ---- epilogue: lane holds rows 8*(v/4) + 4*h + v%4 and column l32 of each 32 x 32 block ----
 #pragma unroll
   for (int fm = 0; fm < 2; ++fm)
 #pragma unroll
@@ -238,7 +146,7 @@ __global__ __launch_bounds__(NTHREADS, 2) void sgemm_mfma_kernel(GemmArgs p) {
       if (col >= p.N) continue;
 #pragma unroll
       for (int v = 0; v < 16; ++v) {
-        int row = m0 + wm * 64 + fm * 32 + 8 * (v >> 2) + 4 * h + (v & 3);
+        int row = m0 + wm * 64 + fm * 32 + acc_row(v, h);
         if (row < p.M) epilogue_store<EPI>(p, C, aux_in, aux_out, row, col, acc[fm][fn][v]);
       }
     }
@@ -366,7 +274,7 @@ int32_t sgemm_impl(int transA, int transB, int64_t M, int64_t N, int64_t K, cons
   // The vector path loads 4 floats at a time along the contiguous index of each operand.
   const bool a_ok = aligned16(A) && lda % 4 == 0 && sA % 4 == 0 && (transA ? M % 4 == 0 : K % 4 == 0);
   const bool b_ok = aligned16(B) && ldb % 4 == 0 && sB % 4 == 0 && (transB ? K % 4 == 0 : N % 4 == 0);
-  const bool big = M * N >= 64 * 64 && K >= 8;
+  const bool big = M * N >= 64 * 64 && K >= 8 && lda < (1ll << 22) && ldb < (1ll << 22);  // 32-bit tile offsets
   if (a_ok && b_ok && big) {
     p.tiles_m = (int)ceil_div64(M, BM);
     p.tiles_n = (int)ceil_div64(N, BN);

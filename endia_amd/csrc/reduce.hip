@@ -74,15 +74,20 @@ __global__ __launch_bounds__(TPB) void col_reduce_scalar_kernel(const float* __r
   part[(b * gridDim.y + blockIdx.y) * C + c] = acc;
 }
 
-// stage 2: out[b][c] = scale * sum_s part[b][s][c]
+// stage 2: out[b][c] = scale * sum_s part[b][s][c]. 64 columns per group; the four waves take
+// s = w, w+4, ... and are combined through LDS in wave order, so the result does not depend on timing.
 __global__ __launch_bounds__(TPB) void col_reduce_final_kernel(const float* __restrict__ part, float* __restrict__ out,
                                                                int64_t S, int64_t C, int64_t batch, float scale) {
-  int64_t i = (int64_t)blockIdx.x * TPB + threadIdx.x;
-  if (i >= batch * C) return;
-  int64_t b = i / C, c = i - b * C;
+  __shared__ float red[4][64];
+  const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
+  const int64_t c = (int64_t)blockIdx.x * 64 + lane;
+  const int64_t b = blockIdx.y;
   float acc = 0.f;
-  for (int64_t s = 0; s < S; ++s) acc += part[(b * S + s) * C + c];
-  out[i] = acc * scale;
+  if (c < C)
+    for (int64_t s = w; s < S; s += 4) acc += part[(b * S + s) * C + c];
+  red[w][lane] = acc;
+  __syncthreads();
+  if (w == 0 && c < C) out[b * C + c] = ((red[0][lane] + red[1][lane]) + (red[2][lane] + red[3][lane])) * scale;
 }
 
 // ---- row reduction: x[R][C] -> out[R] (sum over C) --------------------------------------------
@@ -214,6 +219,7 @@ int32_t col_reduce(int64_t batch, int64_t R, int64_t C, const float* x, float* o
   // enough row splits for ~4 groups per CU, at least 16 rows each
   int64_t want = (int64_t)ctx().cu_count * 4;
   int64_t S = want / (col_tiles * batch);
+  if (S > 32) S = 32;
   if (S < 1) S = 1;
   int64_t max_s = ceil_div64(R, 16);
   if (S > max_s) S = max_s;
@@ -228,8 +234,8 @@ int32_t col_reduce(int64_t batch, int64_t R, int64_t C, const float* x, float* o
   if (vec) hipLaunchKernelGGL(col_reduce_vec_kernel, grid, dim3(TPB), 0, s, x, part, R, C, rows_per_split);
   else hipLaunchKernelGGL(col_reduce_scalar_kernel, grid, dim3(TPB), 0, s, x, part, R, C, rows_per_split);
   ENDIA_LAUNCH_CHECK();
-  hipLaunchKernelGGL(col_reduce_final_kernel, dim3((unsigned)ceil_div64(batch * C, TPB)), dim3(TPB), 0, s, part, out, S,
-                     C, batch, scale);
+  hipLaunchKernelGGL(col_reduce_final_kernel, dim3((unsigned)ceil_div64(C, 64), (unsigned)batch), dim3(TPB), 0, s, part,
+                     out, S, C, batch, scale);
   ENDIA_LAUNCH_CHECK();
   return ENDIA_HIP_OK;
 }
