@@ -250,12 +250,87 @@ def conv_table(reps=10):
     return rows
 
 
+def run_hvp(nd, steps, warmup):
+    """Hessian-vector product by create_graph=True double backward: 4 Linear layers 2048 wide, sin
+    between, batch 1024, loss = sum(out^2), v ~ N(0,1) per parameter. Algorithmic GEMM work of the
+    reference's decomposition: 31 products of 2*1024*2048^2 flops (4 forward, 7 first backward, 20 second)."""
+    rng = np.random.default_rng(3)
+    B, Wd, Ly = 1024, 2048, 4
+    mlp = nd.nn.MLP([Wd] * (Ly + 1), compute_backward=True, activation="sin", fused=True)
+    vs = []
+    for i in range(Ly):
+        mlp.weights[i] = nd.array((rng.standard_normal((Wd, Wd)) / np.sqrt(Wd)).astype(np.float32), requires_grad=True)
+        mlp.biases[i] = nd.array((rng.standard_normal(Wd) / np.sqrt(Wd)).astype(np.float32), requires_grad=True)
+        vs += [nd.array(rng.standard_normal((Wd, Wd)).astype(np.float32)), nd.array(rng.standard_normal((1, Wd)).astype(np.float32))]
+    x = nd.array(rng.standard_normal((B, Wd)).astype(np.float32))
+
+    def step():
+        out = mlp.forward(x)
+        loss = nd.sum(out * out)
+        loss.backward(create_graph=True)
+        s = None
+        for p, v in zip(mlp.params(), vs):
+            term = nd.sum(p.grad() * v)
+            s = term if s is None else s + term
+        hv = nd.grad(outs=s, inputs=mlp.params())
+        loss.zero_grad()
+        return hv
+
+    for _ in range(warmup):
+        step()
+    nd.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        hv = step()
+    nd.synchronize()
+    dt = (time.perf_counter() - t0) / steps
+    flops = 31 * 2.0 * B * Wd * Wd
+    return {"metric": "Hessian-vector products/s, 4 x 2048 sin MLP, batch 1024 (double backward)", "value": 1.0 / dt,
+            "unit": "HVP/s", "ms_per_step": dt * 1e3, "algorithmic_gemm_tflops": flops / dt / 1e12,
+            "frac_of_fp32_mfma_peak": flops / dt / 1e12 / FP32_MFMA_PEAK_TFLOPS, "steps": steps, "warmup": warmup,
+            "dtype": "f32", "data": "synthetic"}
+
+
+def run_complex(nd, steps, warmup, algo):
+    """complex64 MLP: 4 complex Linear layers 2048 -> 2048 (identity activation), batch 2048, loss =
+    sum |out|^2, backward with the reference's rule (no conjugation). 11 complex GEMMs of 8*2048^3 flops."""
+    rng = np.random.default_rng(4)
+    n, Ly = 2048, 4
+    nd.set_complex_matmul_algorithm(algo)
+    Ws = [nd.array(((rng.standard_normal((n, n)) + 1j * rng.standard_normal((n, n))) / np.sqrt(2 * n)).astype(np.complex64),
+                   requires_grad=True) for _ in range(Ly)]
+    z = nd.array((rng.standard_normal((n, n)) + 1j * rng.standard_normal((n, n))).astype(np.complex64))
+
+    def step():
+        h = z
+        for W in Ws:
+            h = nd.matmul(h, W)
+        loss = nd.sum(nd.square(nd.abs(h)))
+        loss.backward()
+        loss.zero_grad()
+        return loss
+
+    for _ in range(warmup):
+        step()
+    nd.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        step()
+    nd.synchronize()
+    dt = (time.perf_counter() - t0) / steps
+    flops = 11 * 8.0 * n * n * n
+    return {"metric": "fwd+bwd steps/s, complex64 MLP 4 x 2048, batch 2048, algorithm " + algo, "value": 1.0 / dt,
+            "unit": "steps/s", "ms_per_step": dt * 1e3, "algorithmic_gemm_tflops": flops / dt / 1e12,
+            "frac_of_fp32_mfma_peak": flops / dt / 1e12 / FP32_MFMA_PEAK_TFLOPS, "steps": steps, "warmup": warmup,
+            "dtype": "c64 (f32 pairs)", "data": "synthetic"}
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=3)
-    ap.add_argument("--workload", default="wide_mlp", choices=["wide_mlp", "sine_mlp", "kernels", "conv2d"])
+    ap.add_argument("--workload", default="wide_mlp", choices=["wide_mlp", "sine_mlp", "kernels", "conv2d", "hvp", "complex_mlp", "complex_mlp_3m"])
     ap.add_argument("--no-cpu-baseline", action="store_true")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -267,6 +342,12 @@ def main():
     L.ensure_init(0)
     dev_name, cus, mhz = L.device_info()
 
+    if args.workload == "hvp":
+        print(json.dumps(run_hvp(nd, args.steps, args.warmup)))
+        return
+    if args.workload.startswith("complex_mlp"):
+        print(json.dumps(run_complex(nd, args.steps, args.warmup, "3m" if args.workload.endswith("3m") else "4m")))
+        return
     if args.workload == "conv2d":
         rows = conv_table(max(args.steps, 1))
         print(json.dumps({"metric": "conv2d fwd + VJPs, batch 64, 64->128 channels, 3x3, stride 1, pad 1, 56x56, fp32",

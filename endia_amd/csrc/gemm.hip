@@ -7,7 +7,8 @@
 // products run on v_mfma_f32_32x32x2_f32.
 //
 // Tiling: a 256-thread work-group (four 64-lane waves, 2 x 2) owns a 128 x 128 tile of C; each
-// wave owns 64 x 64 as 2 x 2 MFMA blocks of 32 x 32 (64 accumulator registers per lane). The K
+// wave owns 64 x 64 as 2 x 2 MFMA blocks of 32 x 32 (64 accumulator registers per lane). Products
+// too small to give every CU work at that size use 64 x 64 tiles (one MFMA block per wave). The K
 // loop advances 32 at a time: the next tile's global loads (buffer loads, bounds-checked by their
 // descriptor) are issued into registers before the MFMAs of the current tile and written to LDS
 // after them. 128 registers per lane and 36 KiB of LDS per group give 4 groups per CU.
@@ -28,8 +29,7 @@ namespace {
 
 using namespace mfma;
 
-constexpr int BM = 128, BN = 128;
-constexpr int NTHREADS = 256;
+constexpr int NTHREADS = 256;  // four waves, 2 x 2
 
 struct GemmArgs {
   const float* A;
@@ -86,8 +86,11 @@ __device__ __forceinline__ void epilogue_store(const GemmArgs& p, float* __restr
   C[off] = v;
 }
 
-template <bool A_KMAJOR, bool B_KMAJOR, int EPI>
+// F = MFMA blocks per wave in each direction: F = 2 gives the 128 x 128 tile, F = 1 the 64 x 64 tile
+// used when the larger one would leave CUs without work.
+template <bool A_KMAJOR, bool B_KMAJOR, int EPI, int F>
 __global__ __launch_bounds__(NTHREADS, 4) void sgemm_mfma_kernel(GemmArgs p) {
+  constexpr int BM = 64 * F, BN = 64 * F;
   using LA = MatrixTileLoader<A_KMAJOR, BM, NTHREADS>;
   using LB = MatrixTileLoader<B_KMAJOR, BN, NTHREADS>;
   __shared__ __attribute__((aligned(16))) float As[TileShape<A_KMAJOR, BM>::FLOATS];
@@ -112,8 +115,8 @@ __global__ __launch_bounds__(NTHREADS, 4) void sgemm_mfma_kernel(GemmArgs p) {
   la.init(p.A + bz * p.sA, p.lda, m0, p.M, p.K, tid);
   lb.init(p.B + bz * p.sB, p.ldb, n0, p.N, p.K, tid);
 
-  floatx16 acc[2][2];
-  zero_acc<2, 2>(acc);
+  floatx16 acc[F][F];
+  zero_acc<F, F>(acc);
 
   la.load(p.K);
   lb.load(p.K);
@@ -129,7 +132,7 @@ __global__ __launch_bounds__(NTHREADS, 4) void sgemm_mfma_kernel(GemmArgs p) {
       la.load(p.K - k0 - BK);
       lb.load(p.K - k0 - BK);
     }
-    compute_ktile<A_KMAJOR, B_KMAJOR, 2, 2, BM, BN>(As, Bs, wm * 64 + l32, wn * 64 + l32, h, acc);
+    compute_ktile<A_KMAJOR, B_KMAJOR, F, F, BM, BN>(As, Bs, wm * 32 * F + l32, wn * 32 * F + l32, h, acc);
     if (more) {
       __syncthreads();
       la.store(As);
@@ -139,14 +142,14 @@ __global__ __launch_bounds__(NTHREADS, 4) void sgemm_mfma_kernel(GemmArgs p) {
   }
 
 #pragma unroll
-  for (int fm = 0; fm < 2; ++fm)
+  for (int fm = 0; fm < F; ++fm)
 #pragma unroll
-    for (int fn = 0; fn < 2; ++fn) {
-      int col = n0 + wn * 64 + fn * 32 + l32;
+    for (int fn = 0; fn < F; ++fn) {
+      int col = n0 + wn * 32 * F + fn * 32 + l32;
       if (col >= p.N) continue;
 #pragma unroll
       for (int v = 0; v < 16; ++v) {
-        int row = m0 + wm * 64 + fm * 32 + acc_row(v, h);
+        int row = m0 + wm * 32 * F + fm * 32 + acc_row(v, h);
         if (row < p.M) epilogue_store<EPI>(p, C, aux_in, aux_out, row, col, acc[fm][fn][v]);
       }
     }
@@ -208,13 +211,23 @@ __global__ __launch_bounds__(256) void sgemm_generic_kernel(GemmArgs p, int tran
     }
 }
 
-template <int EPI>
+template <int EPI, int F>
 void launch_mfma(const GemmArgs& p, int transA, int transB, dim3 grid, hipStream_t s) {
   const bool ak = !transA, bk = transB != 0;
-  if (ak && bk) hipLaunchKernelGGL((sgemm_mfma_kernel<true, true, EPI>), grid, dim3(NTHREADS), 0, s, p);
-  else if (ak && !bk) hipLaunchKernelGGL((sgemm_mfma_kernel<true, false, EPI>), grid, dim3(NTHREADS), 0, s, p);
-  else if (!ak && bk) hipLaunchKernelGGL((sgemm_mfma_kernel<false, true, EPI>), grid, dim3(NTHREADS), 0, s, p);
-  else hipLaunchKernelGGL((sgemm_mfma_kernel<false, false, EPI>), grid, dim3(NTHREADS), 0, s, p);
+  if (ak && bk) hipLaunchKernelGGL((sgemm_mfma_kernel<true, true, EPI, F>), grid, dim3(NTHREADS), 0, s, p);
+  else if (ak && !bk) hipLaunchKernelGGL((sgemm_mfma_kernel<true, false, EPI, F>), grid, dim3(NTHREADS), 0, s, p);
+  else if (!ak && bk) hipLaunchKernelGGL((sgemm_mfma_kernel<false, true, EPI, F>), grid, dim3(NTHREADS), 0, s, p);
+  else hipLaunchKernelGGL((sgemm_mfma_kernel<false, false, EPI, F>), grid, dim3(NTHREADS), 0, s, p);
+}
+
+template <int F>
+void launch_mfma_epi(const GemmArgs& p, int epi, int transA, int transB, dim3 grid, hipStream_t s) {
+  switch (epi) {
+    case ENDIA_EPI_NONE: launch_mfma<ENDIA_EPI_NONE, F>(p, transA, transB, grid, s); break;
+    case ENDIA_EPI_BIAS: launch_mfma<ENDIA_EPI_BIAS, F>(p, transA, transB, grid, s); break;
+    case ENDIA_EPI_BIAS_ACT: launch_mfma<ENDIA_EPI_BIAS_ACT, F>(p, transA, transB, grid, s); break;
+    default: launch_mfma<ENDIA_EPI_ACT_GRAD, F>(p, transA, transB, grid, s); break;
+  }
 }
 
 inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; }
@@ -276,8 +289,10 @@ int32_t sgemm_impl(int transA, int transB, int64_t M, int64_t N, int64_t K, cons
   const bool b_ok = aligned16(B) && ldb % 4 == 0 && sB % 4 == 0 && (transB ? K % 4 == 0 : N % 4 == 0);
   const bool big = M * N >= 64 * 64 && K >= 8 && lda < (1ll << 22) && ldb < (1ll << 22);  // 32-bit tile offsets
   if (a_ok && b_ok && big) {
-    p.tiles_m = (int)ceil_div64(M, BM);
-    p.tiles_n = (int)ceil_div64(N, BN);
+    // 128 x 128 tiles when they give every CU about four work-groups, else 64 x 64 tiles
+    const int F = ceil_div64(M, 128) * ceil_div64(N, 128) * batch >= 3 * (int64_t)ctx().cu_count ? 2 : 1;
+    p.tiles_m = (int)ceil_div64(M, 64 * F);
+    p.tiles_n = (int)ceil_div64(N, 64 * F);
     dim3 grid((unsigned)(p.tiles_m * p.tiles_n), (unsigned)batch);
     const bool timed = g_timing.on;
     if (timed) {
@@ -290,12 +305,8 @@ int32_t sgemm_impl(int transA, int transB, int64_t M, int64_t N, int64_t K, cons
       }
       ENDIA_HIP_CALL(hipEventRecord(g_timing.start[g_timing.used], s));
     }
-    switch (epi) {
-      case ENDIA_EPI_NONE: launch_mfma<ENDIA_EPI_NONE>(p, transA, transB, grid, s); break;
-      case ENDIA_EPI_BIAS: launch_mfma<ENDIA_EPI_BIAS>(p, transA, transB, grid, s); break;
-      case ENDIA_EPI_BIAS_ACT: launch_mfma<ENDIA_EPI_BIAS_ACT>(p, transA, transB, grid, s); break;
-      default: launch_mfma<ENDIA_EPI_ACT_GRAD>(p, transA, transB, grid, s); break;
-    }
+    if (F == 2) launch_mfma_epi<2>(p, epi, transA, transB, grid, s);
+    else launch_mfma_epi<1>(p, epi, transA, transB, grid, s);
     if (timed) {
       ENDIA_HIP_CALL(hipEventRecord(g_timing.stop[g_timing.used], s));
       g_timing.used++;
