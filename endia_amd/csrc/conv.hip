@@ -375,6 +375,240 @@ __global__ __launch_bounds__(WGM* WGN * 64, 2) void conv_wgrad_kernel(WgradArgs 
   }
 }
 
+// ---- fast path: unit stride along the row, output width a multiple of 4, padded source ------------
+// The source tensor is first copied into a zero-padded tensor, so no tap is ever out of range, and a
+// table gives every reduction index t its byte offset inside one padded image. A lane's four
+// consecutive output pixels then read four consecutive source floats: ONE 16-byte buffer load at
+// colbase(j) + table[t], and the whole gather is one integer add per load.
+struct VecArgs {
+  const float* src;   // padded source [N, Cred, Hp, Wp]
+  const float* wp;    // packed weights [Mrows, Kd_pad]
+  const int* table;   // [Kd_pad] byte offset of reduction index t inside an image; OOB_OFFSET for padding rows
+  const float* bias;
+  float* out;
+  int Mrows, OH, OW, Ncols, Kd_pad;
+  int img_floats, Wp, sh;  // floats per padded image, padded row length, stride along rows
+  FastDiv d_ohw, d_ow;
+  int tiles_m, tiles_n, relu;
+  int64_t src_bytes;
+};
+
+template <int WGM, int WGN, int FM, int FN, bool FWD>
+__global__ __launch_bounds__(WGM* WGN * 64, 4) void conv_igemm_vec_kernel(VecArgs a) {
+  constexpr int NT = WGM * WGN * 64, BM = WGM * FM * 32, BN = WGN * FN * 32;
+  constexpr int F4_PER_ROW = BN / 4, ROWS_PER_PASS = NT / F4_PER_ROW, PASSES = BK / ROWS_PER_PASS;
+  constexpr int LDB = TileShape<false, BN>::LD;
+  using LA = MatrixTileLoader<true, BM, NT>;
+  __shared__ __attribute__((aligned(16))) float As[TileShape<true, BM>::FLOATS];
+  __shared__ __attribute__((aligned(16))) float Bs[TileShape<false, BN>::FLOATS];
+  extern __shared__ int tab[];
+
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int wm = wave / WGN, wn = wave % WGN;
+  const int l32 = lane & 31, h = lane >> 5;
+  int tm, tn;
+  tile_of_block(blockIdx.x, gridDim.x, a.tiles_m, a.tiles_n, tm, tn);
+  const int m0 = tm * BM, n0 = tn * BN;
+
+  for (int i = tid; i < a.Kd_pad; i += NT) tab[i] = a.table[i];
+
+  LA la;
+  la.init(a.wp, a.Kd_pad, m0, a.Mrows, a.Kd_pad, tid);
+  const int r = tid / F4_PER_ROW, c4 = (tid % F4_PER_ROW) * 4;
+  const int lds_off = r * LDB + c4;
+  uint32_t colbase = OOB_OFFSET;
+  {
+    int j = n0 + c4;
+    if (j < a.Ncols) {
+      int n = (int)fdiv((uint32_t)j, a.d_ohw);
+      int rem = j - n * a.OH * a.OW;
+      int oy = (int)fdiv((uint32_t)rem, a.d_ow);
+      int ox = rem - oy * a.OW;
+      colbase = (uint32_t)(n * a.img_floats + oy * a.sh * a.Wp + ox) * 4u;
+    }
+  }
+  const __amdgpu_buffer_rsrc_t rs = make_rsrc(a.src, a.src_bytes);
+  float4 breg[PASSES];
+  __syncthreads();  // table visible
+
+  auto load_b = [&](int k0) {
+#pragma unroll
+    for (int i = 0; i < PASSES; ++i) breg[i] = buffer_load_f4(rs, colbase + (uint32_t)tab[k0 + r + i * ROWS_PER_PASS]);
+  };
+  auto store_b = [&]() {
+#pragma unroll
+    for (int i = 0; i < PASSES; ++i) *reinterpret_cast<float4*>(&Bs[lds_off + i * ROWS_PER_PASS * LDB]) = breg[i];
+  };
+
+  floatx16 acc[FM][FN];
+  zero_acc<FM, FN>(acc);
+  la.load(a.Kd_pad);
+  load_b(0);
+  la.store(As);
+  store_b();
+  __syncthreads();
+  for (int k0 = 0; k0 < a.Kd_pad; k0 += BK) {
+    const bool more = k0 + BK < a.Kd_pad;
+    if (more) {
+      la.advance();
+      la.load(a.Kd_pad - k0 - BK);
+      load_b(k0 + BK);
+    }
+    compute_ktile<true, false, FM, FN, BM, BN>(As, Bs, wm * FM * 32 + l32, wn * FN * 32 + l32, h, acc);
+    if (more) {
+      __syncthreads();
+      la.store(As);
+      store_b();
+      __syncthreads();
+    }
+  }
+
+  const int64_t ohw = (int64_t)a.OH * a.OW;
+#pragma unroll
+  for (int fn = 0; fn < FN; ++fn) {
+    int j = n0 + wn * FN * 32 + fn * 32 + l32;
+    if (j >= a.Ncols) continue;
+    int n = (int)fdiv((uint32_t)j, a.d_ohw);
+    int64_t col_off = (int64_t)n * a.Mrows * ohw + (j - (int64_t)n * ohw);
+#pragma unroll
+    for (int fm = 0; fm < FM; ++fm)
+#pragma unroll
+      for (int v = 0; v < 16; ++v) {
+        int m = m0 + wm * FM * 32 + fm * 32 + acc_row(v, h);
+        if (m < a.Mrows) {
+          float val = acc[fm][fn][v];
+          if (FWD) {
+            if (a.bias) val += a.bias[m];
+            if (a.relu) val = val > 0.f ? val : 0.f;
+          }
+          a.out[col_off + m * ohw] = val;
+        }
+      }
+  }
+}
+
+struct WgradVecArgs {
+  const float* xpad;  // [N, C, Hp, Wp]
+  const float* dy;    // [N, K, P, Q], Q % 4 == 0
+  const int* table;   // [tiles_n * BN] byte offset of tap t inside a padded image; OOB_OFFSET past Kd
+  float* part;
+  int K, Kd, PQ, Q, sh, Wp, img_floats;
+  int total_j, chunk;
+  FastDiv d_pq, d_q;
+  int tiles_m, tiles_n;
+  int64_t x_bytes, dy_bytes;
+};
+
+template <int WGM, int WGN, int FM, int FN>
+__global__ __launch_bounds__(WGM* WGN * 64, 4) void conv_wgrad_vec_kernel(WgradVecArgs a) {
+  constexpr int NT = WGM * WGN * 64, BM = WGM * FM * 32, BN = WGN * FN * 32;
+  constexpr int ROWS_PER_PASS = NT / 8, PA = BM / ROWS_PER_PASS, PB = BN / ROWS_PER_PASS;
+  __shared__ __attribute__((aligned(16))) float As[TileShape<true, BM>::FLOATS];
+  __shared__ __attribute__((aligned(16))) float Bs[TileShape<true, BN>::FLOATS];
+
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int wm = wave / WGN, wn = wave % WGN;
+  const int l32 = lane & 31, h = lane >> 5;
+  const int tm = blockIdx.x / a.tiles_n, tn = blockIdx.x % a.tiles_n;
+  const int m0 = tm * BM, n0 = tn * BN;
+  const int split = blockIdx.y;
+  const int j_begin = split * a.chunk;
+  const int j_end = j_begin + a.chunk < a.total_j ? j_begin + a.chunk : a.total_j;
+
+  const int r = tid / 8, c4 = (tid % 8) * 4;
+  const int lds_off = r * LDK + c4;
+  uint32_t rowa[PA], rowb[PB];
+#pragma unroll
+  for (int i = 0; i < PA; ++i) {
+    int m = m0 + r + i * ROWS_PER_PASS;
+    rowa[i] = m < a.K ? (uint32_t)(m * a.PQ) * 4u : OOB_OFFSET;
+  }
+#pragma unroll
+  for (int i = 0; i < PB; ++i) rowb[i] = (uint32_t)a.table[n0 + r + i * ROWS_PER_PASS];
+  const __amdgpu_buffer_rsrc_t rs_dy = make_rsrc(a.dy, a.dy_bytes);
+  const __amdgpu_buffer_rsrc_t rs_x = make_rsrc(a.xpad, a.x_bytes);
+  float4 ra[PA], rb[PB];
+
+  auto load = [&](int jt) {
+    int j = jt + c4;
+    uint32_t ca = OOB_OFFSET, cb = OOB_OFFSET;
+    if (j < j_end) {
+      int n = (int)fdiv((uint32_t)j, a.d_pq);
+      int pq = j - n * a.PQ;
+      int p = (int)fdiv((uint32_t)pq, a.d_q);
+      int q = pq - p * a.Q;
+      ca = (uint32_t)(n * a.K * a.PQ + pq) * 4u;
+      cb = (uint32_t)(n * a.img_floats + p * a.sh * a.Wp + q) * 4u;
+    }
+#pragma unroll
+    for (int i = 0; i < PA; ++i) ra[i] = buffer_load_f4(rs_dy, ca + rowa[i]);
+#pragma unroll
+    for (int i = 0; i < PB; ++i) rb[i] = buffer_load_f4(rs_x, cb + rowb[i]);
+  };
+  auto store = [&]() {
+#pragma unroll
+    for (int i = 0; i < PA; ++i) *reinterpret_cast<float4*>(&As[lds_off + i * ROWS_PER_PASS * LDK]) = ra[i];
+#pragma unroll
+    for (int i = 0; i < PB; ++i) *reinterpret_cast<float4*>(&Bs[lds_off + i * ROWS_PER_PASS * LDK]) = rb[i];
+  };
+
+  floatx16 acc[FM][FN];
+  zero_acc<FM, FN>(acc);
+  load(j_begin);
+  store();
+  __syncthreads();
+  for (int jt = j_begin; jt < j_end; jt += BK) {
+    const bool more = jt + BK < j_end;
+    if (more) load(jt + BK);
+    compute_ktile<true, true, FM, FN, BM, BN>(As, Bs, wm * FM * 32 + l32, wn * FN * 32 + l32, h, acc);
+    if (more) {
+      __syncthreads();
+      store();
+      __syncthreads();
+    }
+  }
+
+  float* out = a.part + (int64_t)split * a.K * a.Kd;
+#pragma unroll
+  for (int fn = 0; fn < FN; ++fn) {
+    int t = n0 + wn * FN * 32 + fn * 32 + l32;
+    if (t >= a.Kd) continue;
+#pragma unroll
+    for (int fm = 0; fm < FM; ++fm)
+#pragma unroll
+      for (int v = 0; v < 16; ++v) {
+        int m = m0 + wm * FM * 32 + fm * 32 + acc_row(v, h);
+        if (m < a.K) out[(int64_t)m * a.Kd + t] = acc[fm][fn][v];
+      }
+  }
+}
+
+// Zero-padded copy: dst[n][c][y][x] = src[n][c][y - py][x - px] where in range, else 0.
+__global__ __launch_bounds__(TPB) void pad_kernel(const float* __restrict__ src, float* __restrict__ dst, int64_t planes,
+                                                  int H, int W, int Hp, int Wp, int py, int px) {
+  const int64_t total = planes * Hp * Wp;
+  for (int64_t i = (int64_t)blockIdx.x * TPB + threadIdx.x; i < total; i += (int64_t)gridDim.x * TPB) {
+    int x = (int)(i % Wp);
+    int64_t t = i / Wp;
+    int y = (int)(t % Hp);
+    int64_t pl = t / Hp;
+    int sy = y - py, sx = x - px;
+    dst[i] = ((unsigned)sy < (unsigned)H && (unsigned)sx < (unsigned)W) ? src[(pl * H + sy) * W + sx] : 0.f;
+  }
+}
+
+// table[t] for t = (ch, r, s): byte offset (ch*Hp + r_eff*dh)*Wp + s_eff*dw inside a padded image, where the
+// data gradient walks the taps in reverse (r_eff = R-1-r). Entries past Kd get OOB_OFFSET.
+__global__ __launch_bounds__(TPB) void tap_table_kernel(int* __restrict__ table, int n, int Kd, int R, int S, int Hp, int Wp,
+                                                        int dh, int dw, int flip) {
+  int t = blockIdx.x * TPB + threadIdx.x;
+  if (t >= n) return;
+  if (t >= Kd) { table[t] = (int)OOB_OFFSET; return; }
+  int ch = t / (R * S), rem = t - ch * R * S, r = rem / S, s = rem - r * S;
+  if (flip) { r = R - 1 - r; s = S - 1 - s; }
+  table[t] = ((ch * Hp + r * dh) * Wp + s * dw) * 4;
+}
+
 // ---- weight repacking -------------------------------------------------------------------------------
 // fwd:  wp[k][t]        = w[k][t]                       t = (c, r, s), rows padded to Kd_pad with zeros
 // data: wp[c][(k,r,s)]  = w[k][c][r][s]
@@ -422,7 +656,100 @@ struct PoolBuf {  // scratch from the library's pool, returned on scope exit (st
   ~PoolBuf() { if (p) endia_hip_free(p); }
 };
 
+inline int grid_for(int64_t n) {
+  int64_t b = (n + TPB - 1) / TPB, cap = (int64_t)endia::ctx().cu_count * 16;
+  if (b > cap) b = cap;
+  return (int)(b < 1 ? 1 : b);
+}
+
+// Padded copy of a [planes, H, W] tensor with (py, px) zeros on every side.
+int32_t make_padded(const float* src, int64_t planes, int H, int W, int py, int px, PoolBuf& buf) {
+  const int Hp = H + 2 * py, Wp = W + 2 * px;
+  int32_t rc = endia_hip_malloc(planes * Hp * Wp * 4, &buf.p);
+  if (rc) return rc;
+  hipLaunchKernelGGL(pad_kernel, dim3(grid_for(planes * Hp * Wp)), dim3(TPB), 0, endia::ctx().stream, src,
+                     static_cast<float*>(buf.p), planes, H, W, Hp, Wp, py, px);
+  ENDIA_LAUNCH_CHECK();
+  return ENDIA_HIP_OK;
+}
+
+int32_t make_table(int n, int Kd, int R, int S, int Hp, int Wp, int dh, int dw, int flip, PoolBuf& buf) {
+  int32_t rc = endia_hip_malloc((int64_t)n * 4, &buf.p);
+  if (rc) return rc;
+  hipLaunchKernelGGL(tap_table_kernel, dim3((n + TPB - 1) / TPB), dim3(TPB), 0, endia::ctx().stream,
+                     static_cast<int*>(buf.p), n, Kd, R, S, Hp, Wp, dh, dw, flip);
+  ENDIA_LAUNCH_CHECK();
+  return ENDIA_HIP_OK;
+}
+
+int32_t pack_weights(const ConvP& p, const float* w, int transpose, int Kd_pad, PoolBuf& buf) {
+  const int rows = transpose ? p.C : p.K;
+  int32_t rc = endia_hip_malloc((int64_t)rows * Kd_pad * 4, &buf.p);
+  if (rc) return rc;
+  int64_t total = (int64_t)rows * Kd_pad;
+  int blocks = (int)((total + TPB - 1) / TPB);
+  if (blocks > 2048) blocks = 2048;
+  hipLaunchKernelGGL(pack_weights_kernel, dim3(blocks), dim3(TPB), 0, endia::ctx().stream, w, static_cast<float*>(buf.p),
+                     p.K, p.C, p.R * p.S, Kd_pad, transpose);
+  ENDIA_LAUNCH_CHECK();
+  return ENDIA_HIP_OK;
+}
+
+// Fast path of forward / data gradient (see VecArgs). Returns 1 when the shape does not qualify.
+int32_t run_igemm_vec(int mode, const ConvP& p, const float* src, const float* w, const float* bias, float* out, int relu) {
+  const bool fwd = mode == MODE_FWD;
+  const int OW = fwd ? p.Q : p.W, OH = fwd ? p.P : p.H;
+  const int SH = fwd ? p.H : p.P, SW = fwd ? p.W : p.Q;
+  const int Cred = fwd ? p.C : p.K, Mrows = fwd ? p.K : p.C;
+  int py, px, row_stride;
+  if (fwd) {
+    if (p.sw != 1 || OW % 4) return 1;
+    py = p.ph; px = p.pw; row_stride = p.sh;
+  } else {  // transposed convolution with unit strides: pad by (R-1)*d - p
+    if (p.sh != 1 || p.sw != 1 || OW % 4) return 1;
+    py = (p.R - 1) * p.dh - p.ph; px = (p.S - 1) * p.dw - p.pw; row_stride = 1;
+    if (py < 0 || px < 0) return 1;
+  }
+  const int Hp = SH + 2 * py, Wp = SW + 2 * px;
+  const int Kd = Cred * p.R * p.S, Kd_pad = (Kd + 31) / 32 * 32;
+  if ((int64_t)p.N * Cred * Hp * Wp >= (1ll << 29) || Kd_pad > 8192) return 1;
+  // the last reads of a row group must stay inside the padded image rows: ox + 3 + (S-1)*dw <= Wp - 1 holds because
+  // OW - 1 + (S-1)*dw <= Wp - 1 by the output-size rule; nothing else to check.
+  PoolBuf spad, wp, table;
+  int32_t rc = make_padded(src, (int64_t)p.N * Cred, SH, SW, py, px, spad);
+  if (rc) return rc;
+  if ((rc = pack_weights(p, w, fwd ? 0 : 1, Kd_pad, wp))) return rc;
+  if ((rc = make_table(Kd_pad, Kd, p.R, p.S, Hp, Wp, p.dh, p.dw, fwd ? 0 : 1, table))) return rc;
+  VecArgs a;
+  a.src = static_cast<const float*>(spad.p); a.wp = static_cast<const float*>(wp.p);
+  a.table = static_cast<const int*>(table.p); a.bias = bias; a.out = out; a.relu = relu;
+  a.Mrows = Mrows; a.OH = OH; a.OW = OW; a.Ncols = p.N * OH * OW; a.Kd_pad = Kd_pad;
+  a.img_floats = Cred * Hp * Wp; a.Wp = Wp; a.sh = row_stride;
+  a.d_ohw = make_fastdiv(OH * OW); a.d_ow = make_fastdiv(OW);
+  a.src_bytes = (int64_t)p.N * Cred * Hp * Wp * 4;
+  a.tiles_n = (a.Ncols + 127) / 128;
+  hipStream_t s = endia::ctx().stream;
+  const size_t dyn = (size_t)Kd_pad * 4;
+  if (Mrows > 64) {
+    a.tiles_m = (Mrows + 127) / 128;
+    dim3 grid((unsigned)(a.tiles_m * a.tiles_n));
+    if (fwd) hipLaunchKernelGGL((conv_igemm_vec_kernel<2, 2, 2, 2, true>), grid, dim3(256), dyn, s, a);
+    else hipLaunchKernelGGL((conv_igemm_vec_kernel<2, 2, 2, 2, false>), grid, dim3(256), dyn, s, a);
+  } else {
+    a.tiles_m = 1;
+    dim3 grid((unsigned)a.tiles_n);
+    if (fwd) hipLaunchKernelGGL((conv_igemm_vec_kernel<1, 4, 2, 1, true>), grid, dim3(256), dyn, s, a);
+    else hipLaunchKernelGGL((conv_igemm_vec_kernel<1, 4, 2, 1, false>), grid, dim3(256), dyn, s, a);
+  }
+  ENDIA_LAUNCH_CHECK();
+  return ENDIA_HIP_OK;
+}
+
 int32_t run_igemm(int mode, const ConvP& p, const float* src, const float* w, const float* bias, float* out, int relu) {
+  {
+    int32_t rc = run_igemm_vec(mode, p, src, w, bias, out, relu);
+    if (rc != 1) return rc;
+  }
   hipStream_t s = endia::ctx().stream;
   IgemmArgs a;
   const bool fwd = mode == MODE_FWD;
@@ -441,16 +768,8 @@ int32_t run_igemm(int mode, const ConvP& p, const float* src, const float* w, co
   a.src_bytes = (int64_t)p.N * a.Cred * a.SH * a.SW * 4;
 
   PoolBuf wp;
-  int32_t rc = endia_hip_malloc((int64_t)a.Mrows * a.Kd_pad * 4, &wp.p);
+  int32_t rc = pack_weights(p, w, fwd ? 0 : 1, a.Kd_pad, wp);
   if (rc) return rc;
-  {
-    int64_t total = (int64_t)a.Mrows * a.Kd_pad;
-    int blocks = (int)((total + TPB - 1) / TPB);
-    if (blocks > 2048) blocks = 2048;
-    hipLaunchKernelGGL(pack_weights_kernel, dim3(blocks), dim3(TPB), 0, s, w, static_cast<float*>(wp.p), p.K, p.C,
-                       p.R * p.S, a.Kd_pad, fwd ? 0 : 1);
-    ENDIA_LAUNCH_CHECK();
-  }
   a.wp = static_cast<const float*>(wp.p);
   a.tiles_n = (a.Ncols + 127) / 128;
   if (a.Mrows > 64) {
@@ -554,7 +873,23 @@ int32_t endia_hip_conv2d_bwd_weight(const endia_hip_conv2d_desc* d, const float*
     a.part = dw;
   }
   dim3 grid((unsigned)tiles, (unsigned)splits);
-  hipLaunchKernelGGL((conv_wgrad_kernel<2, 2, 2, 2>), grid, dim3(256), 0, s, a);
+  const int Hp = p.H + 2 * p.ph, Wp = p.W + 2 * p.pw;
+  const bool vec = p.sw == 1 && p.Q % 4 == 0 && (int64_t)p.N * p.C * Hp * Wp < (1ll << 29) &&
+                   (reinterpret_cast<uintptr_t>(dy) & 15) == 0;
+  if (vec) {
+    PoolBuf xpad, table;
+    if ((rc = make_padded(x, (int64_t)p.N * p.C, p.H, p.W, p.ph, p.pw, xpad))) return rc;
+    if ((rc = make_table(a.tiles_n * 128, Kd, p.R, p.S, Hp, Wp, p.dh, p.dw, 0, table))) return rc;
+    WgradVecArgs v;
+    v.xpad = static_cast<const float*>(xpad.p); v.dy = dy; v.table = static_cast<const int*>(table.p); v.part = a.part;
+    v.K = p.K; v.Kd = Kd; v.PQ = p.P * p.Q; v.Q = p.Q; v.sh = p.sh; v.Wp = Wp; v.img_floats = p.C * Hp * Wp;
+    v.total_j = a.total_j; v.chunk = a.chunk; v.d_pq = a.d_pq; v.d_q = a.d_q;
+    v.tiles_m = a.tiles_m; v.tiles_n = a.tiles_n;
+    v.x_bytes = (int64_t)p.N * p.C * Hp * Wp * 4; v.dy_bytes = a.dy_bytes;
+    hipLaunchKernelGGL((conv_wgrad_vec_kernel<2, 2, 2, 2>), grid, dim3(256), 0, s, v);
+  } else {
+    hipLaunchKernelGGL((conv_wgrad_kernel<2, 2, 2, 2>), grid, dim3(256), 0, s, a);
+  }
   ENDIA_LAUNCH_CHECK();
   if (splits > 1) return col_reduce(1, splits, taps, a.part, dw, 1.f);  // partials added in split order
   return ENDIA_HIP_OK;

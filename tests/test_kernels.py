@@ -270,6 +270,76 @@ def test_conv2d_medium_vs_oracle(dev):
     assert_close(dev.get(ddb, b.shape), db_ref, what="db")
 
 
+FAST_CASES = [
+    # (x shape, w shape, stride, pad, dilation): unit stride along rows and an output width that is a multiple
+    # of 4 take the padded-source path with 16-byte gathers; the others take the general gather
+    ((2, 5, 12, 16), (7, 5, 3, 3), (1, 1), (1, 1), (1, 1)),
+    ((3, 4, 9, 10), (70, 4, 3, 3), (2, 1), (1, 2), (1, 2)),
+    ((2, 6, 8, 8), (5, 6, 1, 1), (1, 1), (0, 0), (1, 1)),
+    ((1, 3, 10, 20), (4, 3, 5, 5), (1, 1), (2, 2), (1, 1)),
+    ((2, 8, 7, 12), (130, 8, 3, 3), (1, 1), (1, 1), (1, 1)),
+    ((2, 3, 9, 9), (4, 3, 3, 3), (1, 1), (0, 0), (1, 1)),      # output width 7: general path
+    ((2, 3, 11, 13), (4, 3, 3, 3), (2, 2), (1, 1), (1, 1)),    # strided data gradient: general path
+]
+
+
+@pytest.mark.parametrize("xs,ws,st,pd,dl", FAST_CASES)
+def test_conv2d_paths_vs_oracle(dev, xs, ws, st,pd, dl):
+    rng = np.random.default_rng(sum(xs) + sum(ws))
+    x = rng.standard_normal(xs).astype(np.float32)
+    w = (rng.standard_normal(ws) * 0.3).astype(np.float32)
+    b = rng.standard_normal(ws[0]).astype(np.float32)
+    d = _desc(x, w, st, pd, dl)
+    y_ref = R.conv2d(x, w, b, st, pd, dl)
+    gy = rng.standard_normal(y_ref.shape).astype(np.float32)
+    dx_ref, dw_ref, db_ref = R.conv2d_bwd(x, w, gy, st, pd, dl)
+    dx_, dw_, db_, dg = dev.put(x), dev.put(w), dev.put(b), dev.put(gy)
+    dy, ddx, ddw, ddb = dev.alloc(gy.nbytes), dev.alloc(x.nbytes), dev.alloc(w.nbytes), dev.alloc(b.nbytes)
+    dev.call("endia_hip_conv2d_fwd", ctypes.byref(d), dx_, dw_, db_, dy, L.OP_IDENTITY)
+    dev.call("endia_hip_conv2d_bwd_data", ctypes.byref(d), dg, dw_, ddx)
+    dev.call("endia_hip_conv2d_bwd_weight", ctypes.byref(d), dx_, dg, ddw)
+    dev.call("endia_hip_conv2d_bwd_bias", ctypes.byref(d), dg, ddb)
+    assert_close(dev.get(dy, gy.shape), y_ref, what="fwd")
+    assert_close(dev.get(ddx, x.shape), dx_ref, what="dx")
+    assert_close(dev.get(ddw, w.shape), dw_ref, what="dw")
+    assert_close(dev.get(ddb, b.shape), db_ref, what="db")
+    import torch
+    tx, tw, tb = (torch.tensor(v, dtype=torch.float64, requires_grad=True) for v in (x, w, b))
+    ty = torch.nn.functional.conv2d(tx, tw, tb, stride=st, padding=pd, dilation=dl)
+    (ty * torch.tensor(gy, dtype=torch.float64)).sum().backward()
+    assert_close(dev.get(dy, gy.shape), ty.detach().numpy(), what="fwd vs torch")
+    assert_close(dev.get(ddx, x.shape), tx.grad.numpy(), what="dx vs torch")
+    assert_close(dev.get(ddw, w.shape), tw.grad.numpy(), what="dw vs torch")
+
+
+def test_conv2d_full_size_properties(dev):
+    """The benchmark configuration (64 x 64 x 56 x 56 input, 128 filters 3 x 3, pad 1) is too large for the
+    CPU loop; check it through the adjoint identities <conv(x,w), dy> = <x, dX> = <w, dW>, through db
+    against a float64 sum, and through output probes against float64 dot products."""
+    rng = np.random.default_rng(7)
+    N, C, H, W, K = 64, 64, 56, 56, 128
+    x = rng.standard_normal((N, C, H, W)).astype(np.float32)
+    w = (rng.standard_normal((K, C, 3, 3)) * np.sqrt(2.0 / (C * 9))).astype(np.float32)
+    gy = rng.standard_normal((N, K, H, W)).astype(np.float32)
+    d = _desc(x, w, (1, 1), (1, 1), (1, 1))
+    dx_, dw_, dg = dev.put(x), dev.put(w), dev.put(gy)
+    dy, ddx, ddw, ddb = dev.alloc(gy.nbytes), dev.alloc(x.nbytes), dev.alloc(w.nbytes), dev.alloc(4 * K)
+    dev.call("endia_hip_conv2d_fwd", ctypes.byref(d), dx_, dw_, None, dy, L.OP_IDENTITY)
+    dev.call("endia_hip_conv2d_bwd_data", ctypes.byref(d), dg, dw_, ddx)
+    dev.call("endia_hip_conv2d_bwd_weight", ctypes.byref(d), dx_, dg, ddw)
+    dev.call("endia_hip_conv2d_bwd_bias", ctypes.byref(d), dg, ddb)
+    y = dev.get(dy, gy.shape)
+    lhs = float(np.vdot(y.astype(np.float64), gy))
+    scale = float(np.linalg.norm(y.astype(np.float64)) * np.linalg.norm(gy.astype(np.float64)))
+    assert abs(lhs - float(np.vdot(x.astype(np.float64), dev.get(ddx, x.shape)))) <= 1e-5 * scale
+    assert abs(lhs - float(np.vdot(w.astype(np.float64), dev.get(ddw, w.shape)))) <= 1e-5 * scale
+    assert_close(dev.get(ddb, (K,)), gy.astype(np.float64).sum(axis=(0, 2, 3)), what="db")
+    xp = np.pad(x.astype(np.float64), ((0, 0), (0, 0), (1, 1), (1, 1)))
+    for (n, k, p, q) in [(0, 0, 0, 0), (63, 127, 55, 55), (17, 5, 0, 31), (40, 99, 28, 0), (1, 64, 55, 3)]:
+        ref = float((xp[n, :, p:p + 3, q:q + 3] * w[k].astype(np.float64)).sum())
+        assert abs(y[n, k, p, q] - ref) <= 1e-4 * max(1.0, abs(ref))
+
+
 def test_pool_reuses_buffers(dev):
     u, c, n0 = ctypes.c_int64(), ctypes.c_int64(), ctypes.c_int64()
     p = dev.alloc(1 << 20)
