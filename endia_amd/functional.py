@@ -682,8 +682,9 @@ def linear(x, W, b, act=None):
     first-order pass: dW = x^T g' (TN GEMM), db = column sum of g', dx = g' W^T (NT GEMM) where
     g' = g * act'(.). When x is itself the output of a fused layer with a single consumer, that
     layer's activation derivative is applied in the epilogue of THIS layer's dx GEMM and the gradient
-    is handed over marked as already carrying it. With create_graph=True the rule is rebuilt from
-    matmul / add / activation ops so that the result is differentiable again.
+    is handed over marked as already carrying it. With create_graph=True the rules are written in
+    differentiable ops instead: relu and tanh through the layer's own output, sin through the stored
+    pre-activation, which for that purpose is a node of its own (the kernel writes both z and sin(z)).
     """
     if x.ndim() != 2 or x.is_complex_ or W.is_complex_ or act not in _ACT:
         z = add(matmul(x, W), b)
@@ -697,29 +698,60 @@ def linear(x, W, b, act=None):
     epi = L.EPI_BIAS if _ACT[act] == L.OP_IDENTITY else L.EPI_BIAS_ACT
     L.call("endia_hip_sgemm", 0, 0, B, N, K, xs.data_ptr(), K, Ws.data_ptr(), N, out.data_ptr(), N, 1, 0, 0, 0, epi,
            _ACT[act], bs_.data_ptr(), None, z.data_ptr() if keep_z else None)
-    meta = {"act": act, "z": z}
+    if keep_z:
+        zz = _linear_node(z, x, W, b, xs, Ws, None)
+        return _sin_of_linear_node(out, zz)
+    return _linear_node(out, x, W, b, xs, Ws, act)
+
+
+def _fused_act_of(px):
+    """The activation a gradient may absorb on its way to px: px is the output of a fused layer (or the
+    fused sin node on top of one), nothing else consumes it and it holds no earlier gradient."""
+    m = px._meta
+    if not m or m.get("act") not in _ACT_FN or px._consumers != 1 or px.has_grad():
+        return None
+    return m
+
+
+def _sin_of_linear_node(out, zz):
+    n = out.size()
+
+    def vjp(primals, grad, out_):
+        from .autograd.functional import building_graph
+        z = primals[0]
+        if building_graph():
+            return [mul(cos(z), grad)]  # sin_op.mojo:92
+        if grad._act_applied:
+            return [grad]
+        g = contiguous(grad)
+        gz = Array.empty(out_._shape)
+        L.call("endia_hip_unary_vjp", L.OP_SIN, n, z.data_ptr(), g.data_ptr(), gz.data_ptr(), 0)
+        return [gz]
+
+    return _register(out, [zz], "sin", vjp, {"act": "sin", "aux": zz, "from_output": False})
+
+
+def _linear_node(out, x, W, b, xs, Ws, act):
+    B, K = xs._shape
+    N = Ws._shape[1]
 
     def vjp(primals, grad, out_):
         from .autograd.functional import building_graph
         px, pW, pb = primals
         if building_graph():
-            zz = add(matmul(px, pW), pb)
-            if act in _ACT_FN:
-                # the activation's own rule, applied to a re-built pre-activation
-                a = _ACT_FN[act](zz)
-                g = a._vjp(a._args, grad, a)[0]
+            if act == "tanh":
+                g = mul(1 - square(out_), grad)                      # tanh_op.mojo:92 with tanh(z) = out
+            elif act == "relu":
+                g = mul(greater(out_, zeros([N])), grad)             # relu_op.mojo:95; out > 0 iff z > 0
             else:
                 g = grad
             return [matmul(g, pW.T()) if px._requires_grad else None,
                     matmul(px.T(), g) if pW._requires_grad else None,
                     reduce_add(g, [0]) if pb._requires_grad else None]
         g = contiguous(grad)
-        if act in _ACT_FN and not grad._act_applied:
+        if act in _ACT_FN and not grad._act_applied:  # relu and tanh derivatives from the stored output
             gp = Array.empty([B, N])
-            if act == "sin":
-                L.call("endia_hip_unary_vjp", L.OP_SIN, B * N, z.data_ptr(), g.data_ptr(), gp.data_ptr(), 0)
-            else:  # relu and tanh derivatives from the stored output
-                L.call("endia_hip_unary_vjp_from_output", _ACT[act], B * N, out_.data_ptr(), g.data_ptr(), gp.data_ptr())
+            L.call("endia_hip_unary_vjp_from_output", _ACT[act], B * N, out_.data_ptr(), g.data_ptr(), gp.data_ptr())
             g = gp
         res = [None, None, None]
         if pW._requires_grad:
@@ -733,14 +765,11 @@ def linear(x, W, b, act=None):
             res[2] = db
         if px._requires_grad:
             dx = Array.empty([B, K])
-            single_use = px._consumers == 1 and not px.has_grad()
-            pm = px._meta if (px._name == "linear" and single_use and px._meta) else None
-            if pm and pm["act"] in _ACT_FN:
-                a = pm["act"]
-                aux = pm["z"] if a == "sin" else px
-                flags = _ACT[a] | (0 if a == "sin" else L.ACT_FROM_OUTPUT)
+            pm = _fused_act_of(px)
+            if pm:
+                flags = _ACT[pm["act"]] | (L.ACT_FROM_OUTPUT if pm["from_output"] else 0)
                 L.call("endia_hip_sgemm", 0, 1, B, K, N, g.data_ptr(), N, Ws.data_ptr(), N, dx.data_ptr(), K, 1, 0, 0, 0,
-                       L.EPI_ACT_GRAD, flags, None, contiguous(aux).data_ptr(), None)
+                       L.EPI_ACT_GRAD, flags, None, contiguous(pm["aux"]).data_ptr(), None)
                 dx._act_applied = True
             else:
                 L.call("endia_hip_sgemm", 0, 1, B, K, N, g.data_ptr(), N, Ws.data_ptr(), N, dx.data_ptr(), K, 1, 0, 0, 0,
@@ -748,4 +777,5 @@ def linear(x, W, b, act=None):
             res[0] = dx
         return res
 
+    meta = {"act": act, "aux": out, "from_output": True} if act in _ACT_FN else {"act": None}
     return _register(out, [x, W, b], "linear", vjp, meta)
