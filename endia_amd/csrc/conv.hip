@@ -583,17 +583,22 @@ __global__ __launch_bounds__(WGM* WGN * 64, 4) void conv_wgrad_vec_kernel(WgradV
   }
 }
 
-// Zero-padded copy: dst[n][c][y][x] = src[n][c][y - py][x - px] where in range, else 0.
-__global__ __launch_bounds__(TPB) void pad_kernel(const float* __restrict__ src, float* __restrict__ dst, int64_t planes,
+// Zero-padded copy: dst[pl][y][x] = src[pl][y - py][x - px] where in range, else 0. One wave per padded row
+// (rows are short: the walk over x needs no division, and reads and writes stay contiguous).
+__global__ __launch_bounds__(TPB) void pad_kernel(const float* __restrict__ src, float* __restrict__ dst, int64_t rows_total,
                                                   int H, int W, int Hp, int Wp, int py, int px) {
-  const int64_t total = planes * Hp * Wp;
-  for (int64_t i = (int64_t)blockIdx.x * TPB + threadIdx.x; i < total; i += (int64_t)gridDim.x * TPB) {
-    int x = (int)(i % Wp);
-    int64_t t = i / Wp;
-    int y = (int)(t % Hp);
-    int64_t pl = t / Hp;
-    int sy = y - py, sx = x - px;
-    dst[i] = ((unsigned)sy < (unsigned)H && (unsigned)sx < (unsigned)W) ? src[(pl * H + sy) * W + sx] : 0.f;
+  const int lane = threadIdx.x & 63;
+  const int64_t waves = (int64_t)gridDim.x * (TPB / 64);
+  for (int64_t row = (int64_t)blockIdx.x * (TPB / 64) + (threadIdx.x >> 6); row < rows_total; row += waves) {
+    const int64_t pl = row / Hp;
+    const int y = (int)(row - pl * Hp), sy = y - py;
+    const bool row_ok = (unsigned)sy < (unsigned)H;
+    const float* s = src + (pl * H + (row_ok ? sy : 0)) * W;
+    float* d = dst + row * Wp;
+    for (int x = lane; x < Wp; x += 64) {
+      int sx = x - px;
+      d[x] = (row_ok && (unsigned)sx < (unsigned)W) ? s[sx] : 0.f;
+    }
   }
 }
 
@@ -667,8 +672,11 @@ int32_t make_padded(const float* src, int64_t planes, int H, int W, int py, int 
   const int Hp = H + 2 * py, Wp = W + 2 * px;
   int32_t rc = endia_hip_malloc(planes * Hp * Wp * 4, &buf.p);
   if (rc) return rc;
-  hipLaunchKernelGGL(pad_kernel, dim3(grid_for(planes * Hp * Wp)), dim3(TPB), 0, endia::ctx().stream, src,
-                     static_cast<float*>(buf.p), planes, H, W, Hp, Wp, py, px);
+  const int64_t rows = planes * Hp;
+  int64_t blocks = (rows + 3) / 4, cap = (int64_t)endia::ctx().cu_count * 64;
+  if (blocks > cap) blocks = cap;
+  hipLaunchKernelGGL(pad_kernel, dim3((unsigned)blocks), dim3(TPB), 0, endia::ctx().stream, src,
+                     static_cast<float*>(buf.p), rows, H, W, Hp, Wp, py, px);
   ENDIA_LAUNCH_CHECK();
   return ENDIA_HIP_OK;
 }

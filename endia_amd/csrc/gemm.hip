@@ -42,6 +42,7 @@ struct GemmArgs {
   int64_t sA, sB, sC;
   int M, N, K;
   int tiles_m, tiles_n;
+  int k_split;    // > 0: grid.y indexes slices of K of this length instead of batch entries
   int act;        // endia_hip_unary_op
   int from_out;   // activation gradient from stored output instead of pre-activation
   int accumulate;
@@ -110,27 +111,29 @@ __global__ __launch_bounds__(NTHREADS, 4) void sgemm_mfma_kernel(GemmArgs p) {
   const float* __restrict__ aux_in = p.aux_in ? p.aux_in + bz * p.sC : nullptr;
   float* __restrict__ aux_out = p.aux_out ? p.aux_out + bz * p.sC : nullptr;
 
+  // split-K: this group reduces k in [bz * k_split, bz * k_split + K) and writes slice bz of the partials
+  const int K = p.k_split ? (p.K - (int)bz * p.k_split < p.k_split ? p.K - (int)bz * p.k_split : p.k_split) : p.K;
   LA la;
   LB lb;
-  la.init(p.A + bz * p.sA, p.lda, m0, p.M, p.K, tid);
-  lb.init(p.B + bz * p.sB, p.ldb, n0, p.N, p.K, tid);
+  la.init(p.A + bz * p.sA, p.lda, m0, p.M, K, tid);
+  lb.init(p.B + bz * p.sB, p.ldb, n0, p.N, K, tid);
 
   floatx16 acc[F][F];
   zero_acc<F, F>(acc);
 
-  la.load(p.K);
-  lb.load(p.K);
+  la.load(K);
+  lb.load(K);
   la.store(As);
   lb.store(Bs);
   __syncthreads();
 
-  for (int k0 = 0; k0 < p.K; k0 += BK) {
-    const bool more = k0 + BK < p.K;
+  for (int k0 = 0; k0 < K; k0 += BK) {
+    const bool more = k0 + BK < K;
     if (more) {  // next tile: global -> registers, in flight during this tile's MFMAs
       la.advance();
       lb.advance();
-      la.load(p.K - k0 - BK);
-      lb.load(p.K - k0 - BK);
+      la.load(K - k0 - BK);
+      lb.load(K - k0 - BK);
     }
     compute_ktile<A_KMAJOR, B_KMAJOR, F, F, BM, BN>(As, Bs, wm * 32 * F + l32, wn * 32 * F + l32, h, acc);
     if (more) {
@@ -234,7 +237,16 @@ inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 
 
 }  // namespace
 
+namespace endia {
+int32_t col_reduce(int64_t batch, int64_t R, int64_t C, const float* x, float* out, float scale);
+}
+
 namespace {
+struct PoolBuf {  // scratch from the library's pool, handed back on scope exit (reuse is stream-ordered)
+  void* p = nullptr;
+  ~PoolBuf() { if (p) endia_hip_free(p); }
+};
+
 // per-launch event pairs for endia_hip_gemm_timing_*
 struct GemmTiming {
   bool on = false;
@@ -289,11 +301,39 @@ int32_t sgemm_impl(int transA, int transB, int64_t M, int64_t N, int64_t K, cons
   const bool b_ok = aligned16(B) && ldb % 4 == 0 && sB % 4 == 0 && (transB ? K % 4 == 0 : N % 4 == 0);
   const bool big = M * N >= 64 * 64 && K >= 8 && lda < (1ll << 22) && ldb < (1ll << 22);  // 32-bit tile offsets
   if (a_ok && b_ok && big) {
-    // 128 x 128 tiles when they give every CU about four work-groups, else 64 x 64 tiles
-    const int F = ceil_div64(M, 128) * ceil_div64(N, 128) * batch >= 3 * (int64_t)ctx().cu_count ? 2 : 1;
+    // 128 x 128 tiles when they give every CU about four work-groups and do not pad M or N by more than
+    // a quarter, else 64 x 64 tiles
+    const int64_t cus = ctx().cu_count;
+    const int64_t t128 = ceil_div64(M, 128) * ceil_div64(N, 128);
+    const bool fits128 = (double)(ceil_div64(M, 128) * 128) * (double)(ceil_div64(N, 128) * 128) <= 1.25 * (double)M * (double)N;
+    const int F = (t128 * batch >= 3 * cus && fits128) ? 2 : 1;
     p.tiles_m = (int)ceil_div64(M, 64 * F);
     p.tiles_n = (int)ceil_div64(N, 64 * F);
-    dim3 grid((unsigned)(p.tiles_m * p.tiles_n), (unsigned)batch);
+    const int64_t tiles = (int64_t)p.tiles_m * p.tiles_n;
+    // A long reduction with few output tiles (dW of a narrow layer over a large batch) is split along K:
+    // slices write partial products that are then added in slice order.
+    int64_t splits = 1;
+    if (batch == 1 && epi == ENDIA_EPI_NONE && !accumulate && ldc == N && tiles * 2 <= cus && K >= 2048) {
+      splits = (4 * cus + tiles - 1) / tiles;
+      if (splits > K / 256) splits = K / 256;
+      if (splits > 1024) splits = 1024;
+    }
+    PoolBuf part;
+    float* const C_final = C;
+    p.k_split = 0;
+    if (splits > 1) {
+      int64_t chunk = ceil_div64(ceil_div64(K, splits), BK) * BK;
+      splits = ceil_div64(K, chunk);
+      int32_t rc = endia_hip_malloc(splits * M * N * 4, &part.p);
+      if (rc) return rc;
+      p.k_split = (int)chunk;
+      p.sA = chunk * (transA ? lda : 1);
+      p.sB = chunk * (transB ? 1 : ldb);
+      p.C = static_cast<float*>(part.p);
+      p.ldc = N;
+      p.sC = M * N;
+    }
+    dim3 grid((unsigned)tiles, (unsigned)(splits > 1 ? splits : batch));
     const bool timed = g_timing.on;
     if (timed) {
       if (g_timing.used == g_timing.start.size()) {
@@ -312,7 +352,12 @@ int32_t sgemm_impl(int transA, int transB, int64_t M, int64_t N, int64_t K, cons
       g_timing.used++;
       g_timing.flops += 2.0 * (double)M * (double)N * (double)K * (double)batch;
     }
+    if (splits > 1) {
+      ENDIA_LAUNCH_CHECK();
+      return col_reduce(1, splits, M * N, p.C, C_final, 1.f);  // partials added in slice order
+    }
   } else {
+    p.k_split = 0;
     p.tiles_m = (int)ceil_div64(M, 64);
     p.tiles_n = (int)ceil_div64(N, 64);
     ENDIA_CHECK_ARG(p.tiles_m <= 65535, "sgemm: M too large for the unaligned path");

@@ -219,7 +219,7 @@ int32_t col_reduce(int64_t batch, int64_t R, int64_t C, const float* x, float* o
   // enough row splits for ~4 groups per CU, at least 16 rows each
   int64_t want = (int64_t)ctx().cu_count * 4;
   int64_t S = want / (col_tiles * batch);
-  if (S > 32) S = 32;
+  if (S > 64) S = 64;
   if (S < 1) S = 1;
   int64_t max_s = ceil_div64(R, 16);
   if (S > max_s) S = max_s;

@@ -27,7 +27,7 @@ def run_sgemm(dev, A, B, ta, tb, M, N, K, epi=L.EPI_NONE, act=L.OP_IDENTITY, bia
 
 
 SHAPES = [(128, 128, 32), (256, 384, 72), (132, 260, 100), (37, 53, 19), (4, 4, 4), (1, 1, 1), (128, 1, 32),
-          (1, 32, 128), (300, 200, 8), (64, 64, 1024)]
+          (1, 32, 128), (300, 200, 8), (64, 64, 1024), (64, 96, 8192), (128, 200, 5000), (72, 64, 2052)]
 
 
 @pytest.mark.parametrize("ta,tb", [(0, 0), (0, 1), (1, 0), (1, 1)])
