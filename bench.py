@@ -29,6 +29,11 @@ sys.path.insert(0, ROOT)
 
 FP32_MFMA_PEAK_TFLOPS = 157.3
 HBM_PEAK_GBS = 8000.0
+# HBM-side bytes per 4096^3 GEMM launch, averaged over the launch mix of one training step (8 NN with the bias /
+# bias+tanh epilogue, 7 NT with the tanh' epilogue, 8 TN). It cannot be read while the benchmark runs: it comes
+# from two rocprofv3 --pmc runs (FETCH_SIZE, WRITE_SIZE in KiB per dispatch), each scaled by what the same counter
+# reads for a 64 MiB copy kernel (x1.999 and x1.000); the per-kernel table is in profiles/.
+GEMM_TRAFFIC_BYTES = int((8 * 802.7 + 7 * 1364.9 + 8 * 752.5) / 23 * 1024 * 1024)
 
 
 def build_wide_mlp(nd, width=4096, layers=8, batch=4096, seed=2):
@@ -405,7 +410,10 @@ def main():
         out["roofline"] = {
             "bound": "mfma", "kernel": "sgemm_mfma_kernel (fp32 v_mfma_f32_32x32x2, 128x128x32 tiles)",
             "achieved": achieved, "peak": FP32_MFMA_PEAK_TFLOPS, "unit": "TFLOP/s", "frac": achieved / FP32_MFMA_PEAK_TFLOPS,
-            "traffic": None, "launches": launches.value, "avg_launch_ms": avg_ms,
+            "traffic": GEMM_TRAFFIC_BYTES if args.workload == "wide_mlp" else None,
+            "traffic_source": "rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, see profiles/kernels_wide_mlp_counters.md",
+            "algorithmic_bytes": 3 * 4096 * 4096 * 4 if args.workload == "wide_mlp" else None,
+            "launches": launches.value, "avg_launch_ms": avg_ms,
             "flops_per_launch": flops_per_launch, "gemm_share_of_step": g_ms.value / (1e3 * elapsed),
         }
         out["mfma_util_pct"] = 100.0 * achieved / FP32_MFMA_PEAK_TFLOPS

@@ -75,6 +75,9 @@ SIGNATURES = {
     "endia_hip_conv2d_bwd_weight": [POINTER(Conv2dDesc), _fp, _fp, _fp],
     "endia_hip_conv2d_bwd_bias": [POINTER(Conv2dDesc), _fp, _fp],
     "endia_hip_sgd_step": [c_int64, _fp, _fp, c_float],
+    "endia_hip_sgd_momentum_step": [c_int64, _fp, _fp, _fp, c_float, c_float, c_float],
+    "endia_hip_adagrad_step": [c_int64, _fp, _fp, _fp, c_float, c_float],
+    "endia_hip_rmsprop_step": [c_int64, _fp, _fp, _fp, c_float, c_float, c_float],
     "endia_hip_adam_step": [c_int64, _fp, _fp, _fp, _fp, c_float, c_float, c_float, c_float, c_float],
 }
 

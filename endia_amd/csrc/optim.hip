@@ -88,6 +88,74 @@ __global__ __launch_bounds__(TPB) void sgd_kernel(int64_t n, float* __restrict__
   }
 }
 
+// kind: 0 = SGD with momentum / weight decay, 1 = Adagrad, 2 = RMSprop. `s` is the state tensor (velocity or cache).
+struct OptK {
+  int kind;
+  float lr, a, b, eps;  // SGD: a = momentum, b = weight decay; RMSprop: a = alpha, b = 1 - alpha
+};
+
+__device__ __forceinline__ void opt_one(float& p, float g, float& s, const OptK& k, bool has_state) {
+  if (k.kind == 0) {
+    float c = g;
+    if (k.b > 0.f) { float w = k.b * p; c = g + w; }
+    float d = k.lr * c;
+    if (k.a > 0.f && has_state) {
+      float m = k.a * s;
+      s = m - d;
+      p = p + s;
+    } else {
+      p = p - d;
+    }
+  } else {
+    float gg;
+    if (k.kind == 1) {
+      gg = g * g;
+      s = s + gg;
+    } else {
+      float x = k.a * s, y = k.b * g;
+      y = y * g;
+      s = x + y;
+    }
+    float r = (fabsf(s) + s) * 0.5f;  // the reference's real sqrt, sqrt_op.mojo:111-114
+    float den = __builtin_sqrtf(r) + k.eps;
+    float num = k.lr * g;
+    p = p - num / den;
+  }
+}
+
+__global__ __launch_bounds__(TPB) void opt_kernel(int64_t n, float* __restrict__ p, const float* __restrict__ g,
+                                                  float* __restrict__ s, OptK k, int vec) {
+  int64_t i = (int64_t)blockIdx.x * TPB + threadIdx.x;
+  int64_t stride = (int64_t)gridDim.x * TPB;
+  const bool hs = s != nullptr;
+  if (vec) {
+    int64_t n4 = n >> 2;
+    float4* p4 = reinterpret_cast<float4*>(p);
+    const float4* g4 = reinterpret_cast<const float4*>(g);
+    float4* s4 = reinterpret_cast<float4*>(s);
+    for (int64_t j = i; j < n4; j += stride) {
+      float4 P = p4[j], G = g4[j], S = hs ? s4[j] : make_float4(0.f, 0.f, 0.f, 0.f);
+      opt_one(P.x, G.x, S.x, k, hs);
+      opt_one(P.y, G.y, S.y, k, hs);
+      opt_one(P.z, G.z, S.z, k, hs);
+      opt_one(P.w, G.w, S.w, k, hs);
+      p4[j] = P;
+      if (hs) s4[j] = S;
+    }
+    for (int64_t j = (n4 << 2) + i; j < n; j += stride) {
+      float S = hs ? s[j] : 0.f;
+      opt_one(p[j], g[j], S, k, hs);
+      if (hs) s[j] = S;
+    }
+  } else {
+    for (int64_t j = i; j < n; j += stride) {
+      float S = hs ? s[j] : 0.f;
+      opt_one(p[j], g[j], S, k, hs);
+      if (hs) s[j] = S;
+    }
+  }
+}
+
 inline bool al16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; }
 
 inline int stream_grid(int64_t nvec) {
@@ -113,6 +181,37 @@ int32_t endia_hip_sgd_step(int64_t n, float* p, const float* g, float lr) {
   hipLaunchKernelGGL(sgd_kernel, dim3(stream_grid(vec ? (n + 3) / 4 : n)), dim3(TPB), 0, ctx().stream, n, p, g, lr, vec);
   ENDIA_LAUNCH_CHECK();
   return ENDIA_HIP_OK;
+}
+
+static int32_t launch_opt(const char* who, int64_t n, float* p, const float* g, float* s, const OptK& k, bool need_state) {
+  ENDIA_REQUIRE_INIT();
+  if (n < 0) return fail(ENDIA_HIP_ERR_INVALID, "%s: negative n", who);
+  if (n == 0) return ENDIA_HIP_OK;
+  if (!p || !g || (need_state && !s)) return fail(ENDIA_HIP_ERR_INVALID, "%s: null pointer", who);
+  int vec = al16(p) && al16(g) && (!s || al16(s));
+  hipLaunchKernelGGL(opt_kernel, dim3(stream_grid(vec ? (n + 3) / 4 : n)), dim3(TPB), 0, ctx().stream, n, p, g, s, k, vec);
+  ENDIA_LAUNCH_CHECK();
+  return ENDIA_HIP_OK;
+}
+
+int32_t endia_hip_sgd_momentum_step(int64_t n, float* p, const float* g, float* vel, float lr, float momentum,
+                                    float weight_decay) {
+  ENDIA_CHECK_ARG(momentum >= 0.f && weight_decay >= 0.f, "endia_hip_sgd_momentum_step: negative momentum or weight decay");
+  OptK k;
+  k.kind = 0; k.lr = lr; k.a = momentum; k.b = weight_decay; k.eps = 0.f;
+  return launch_opt("endia_hip_sgd_momentum_step", n, p, g, momentum > 0.f ? vel : nullptr, k, momentum > 0.f);
+}
+
+int32_t endia_hip_adagrad_step(int64_t n, float* p, const float* g, float* cache, float lr, float eps) {
+  OptK k;
+  k.kind = 1; k.lr = lr; k.a = 0.f; k.b = 0.f; k.eps = eps;
+  return launch_opt("endia_hip_adagrad_step", n, p, g, cache, k, true);
+}
+
+int32_t endia_hip_rmsprop_step(int64_t n, float* p, const float* g, float* cache, float lr, float alpha, float eps) {
+  OptK k;
+  k.kind = 2; k.lr = lr; k.a = alpha; k.b = 1.0f - alpha; k.eps = eps;
+  return launch_opt("endia_hip_rmsprop_step", n, p, g, cache, k, true);
 }
 
 int32_t endia_hip_adam_step(int64_t n, float* p, const float* g, float* m, float* v, float lr, float beta1, float beta2,

@@ -1,4 +1,4 @@
-"""SGD and Adam: the host-side mirror of endia/optim/sgd.mojo and endia/optim/adam.mojo.
+"""SGD, Adam, Adagrad and RMSprop: the host-side mirror of endia/optim/{sgd,adam,adagrad,rmsprop}.mojo.
 
 The reference builds every update from separate Array ops; here `step()` is one fused kernel per
 parameter tensor, writing the parameter (and the moments) in place, which is what the reference's
@@ -22,19 +22,56 @@ def _flat_grad(p):
 
 
 class SGD:
-    """Plain path `p -= lr * p.grad()` (sgd.mojo:61-62). Momentum and weight decay are not built."""
+    """sgd.mojo:14-63: plain `p -= lr * p.grad()`, or with momentum (velocity = momentum * velocity - lr * (grad +
+    weight_decay * p); p += velocity) and / or weight decay."""
 
     def __init__(self, params, lr=0.01, momentum=0.0, weight_decay=0.0):
-        if momentum != 0 or weight_decay != 0:
-            raise NotImplementedError("SGD momentum / weight decay variants (sgd.mojo:42-60) are out of scope")
         self.params = list(params)
-        self.lr = float(np.float32(lr))
+        self.lr, self.momentum, self.weight_decay = (float(np.float32(v)) for v in (lr, momentum, weight_decay))
+        self.velocity = [Array(p.shape()) for p in self.params] if self.momentum > 0 else []
 
     def step(self):
-        for p in self.params:
+        for i, p in enumerate(self.params):
             g = _flat_grad(p)
             assert p.is_contiguous()
-            L.call("endia_hip_sgd_step", p.size(), p.data_ptr(), g.data_ptr(), self.lr)
+            if self.momentum > 0 or self.weight_decay > 0:
+                vel = self.velocity[i].data_ptr() if self.momentum > 0 else None
+                L.call("endia_hip_sgd_momentum_step", p.size(), p.data_ptr(), g.data_ptr(), vel, self.lr, self.momentum,
+                       self.weight_decay)
+            else:
+                L.call("endia_hip_sgd_step", p.size(), p.data_ptr(), g.data_ptr(), self.lr)
+            p.clear_args()
+
+
+class Adagrad:
+    """adagrad.mojo:14-45."""
+
+    def __init__(self, params, lr=0.01, eps=1e-8):
+        self.params = list(params)
+        self.lr, self.eps = float(np.float32(lr)), float(np.float32(eps))
+        self.cache = [Array(p.shape()) for p in self.params]
+
+    def step(self):
+        for p, c in zip(self.params, self.cache):
+            g = _flat_grad(p)
+            assert p.is_contiguous()
+            L.call("endia_hip_adagrad_step", p.size(), p.data_ptr(), g.data_ptr(), c.data_ptr(), self.lr, self.eps)
+            p.clear_args()
+
+
+class RMSprop:
+    """rmsprop.mojo:14-53."""
+
+    def __init__(self, params, lr=0.01, alpha=0.99, eps=1e-8):
+        self.params = list(params)
+        self.lr, self.alpha, self.eps = (float(np.float32(v)) for v in (lr, alpha, eps))
+        self.cache = [Array(p.shape()) for p in self.params]
+
+    def step(self):
+        for p, c in zip(self.params, self.cache):
+            g = _flat_grad(p)
+            assert p.is_contiguous()
+            L.call("endia_hip_rmsprop_step", p.size(), p.data_ptr(), g.data_ptr(), c.data_ptr(), self.lr, self.alpha, self.eps)
             p.clear_args()
 
 

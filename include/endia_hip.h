@@ -204,6 +204,14 @@ ENDIA_API int32_t endia_hip_conv2d_bwd_bias(const endia_hip_conv2d_desc* d, cons
 /* ---- optimizers: SGD.step plain path (optim/sgd.mojo:61-62) and Adam.step (optim/adam.mojo:47-65),
  *      each as one pass over the parameter. t is Adam's fp32 step counter (starts at 1, adam.mojo:40). */
 ENDIA_API int32_t endia_hip_sgd_step(int64_t n, float* p, const float* g, float lr);
+/* SGD with momentum and / or weight decay (optim/sgd.mojo:42-60): vel = momentum*vel - lr*(g + wd*p); p += vel
+ * (without momentum: p -= lr*(g + wd*p); vel may then be null). Adagrad (optim/adagrad.mojo:36-45):
+ * cache += g*g; p -= lr*g / (sqrt(cache) + eps). RMSprop (optim/rmsprop.mojo:39-53):
+ * cache = alpha*cache + (1-alpha)*g*g; p -= lr*g / (sqrt(cache) + eps). One pass each. */
+ENDIA_API int32_t endia_hip_sgd_momentum_step(int64_t n, float* p, const float* g, float* vel, float lr, float momentum,
+                                    float weight_decay);
+ENDIA_API int32_t endia_hip_adagrad_step(int64_t n, float* p, const float* g, float* cache, float lr, float eps);
+ENDIA_API int32_t endia_hip_rmsprop_step(int64_t n, float* p, const float* g, float* cache, float lr, float alpha, float eps);
 ENDIA_API int32_t endia_hip_adam_step(int64_t n, float* p, const float* g, float* m, float* v, float lr,
                             float beta1, float beta2, float eps, float t);
 

@@ -429,6 +429,47 @@ void ref_adam(int64_t n, float* p, const float* g, float* m, float* v, float lr,
   }
 }
 
+/* SGD with momentum / weight decay (optim/sgd.mojo:42-60), Adagrad (optim/adagrad.mojo:36-45), RMSprop
+ * (optim/rmsprop.mojo:39-53), one fp32 Array op at a time. vel may be NULL when momentum == 0. */
+void ref_sgd_momentum(int64_t n, float* p, const float* g, float* vel, float lr, float momentum, float wd) {
+  for (int64_t i = 0; i < n; ++i) {
+    float c = g[i];
+    if (wd > 0.f) { float w = wd * p[i]; c = g[i] + w; }
+    float d = lr * c;
+    if (momentum > 0.f) {
+      float m = momentum * vel[i];
+      vel[i] = m - d;
+      p[i] = p[i] + vel[i];
+    } else {
+      p[i] = p[i] - d;
+    }
+  }
+}
+
+void ref_adagrad(int64_t n, float* p, const float* g, float* cache, float lr, float eps) {
+  for (int64_t i = 0; i < n; ++i) {
+    float gg = g[i] * g[i];
+    cache[i] = cache[i] + gg;
+    float num = lr * g[i];
+    float den = unary_real(OP_SQRT, cache[i]) + eps;
+    float q = num / den;
+    p[i] = p[i] - q;
+  }
+}
+
+void ref_rmsprop(int64_t n, float* p, const float* g, float* cache, float lr, float alpha, float eps) {
+  float oma = 1.f - alpha;
+  for (int64_t i = 0; i < n; ++i) {
+    float x = alpha * cache[i], y = oma * g[i];
+    y = y * g[i];
+    cache[i] = x + y;
+    float num = lr * g[i];
+    float den = unary_real(OP_SQRT, cache[i]) + eps;
+    float q = num / den;
+    p[i] = p[i] - q;
+  }
+}
+
 /* ---- one imperative training step: benchmarks/mlp_benchmarks/mlp_imp.mojo:47-75 -----------------
  * forward (nn/modules/_mlp.mojo:47-53): pred = act(pred @ W_i + b_i), no activation after the last layer;
  * loss = mse(pred, y); backward in jacrev order (autograd/functional.mojo:40-65); optimizer step.

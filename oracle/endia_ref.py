@@ -199,6 +199,27 @@ def adam(p, g, m, v, lr=1e-3, b1=0.9, b2=0.999, eps=1e-8, t=1.0):
     return p, m, v
 
 
+def sgd_momentum(p, g, vel, lr, momentum=0.0, weight_decay=0.0):
+    p, vel = _f32(p).copy(), _f32(vel).copy()
+    g = _f32(g)
+    lib().ref_sgd_momentum(c_int64(p.size), _ptr(p), _ptr(g), _ptr(vel), c_float(lr), c_float(momentum), c_float(weight_decay))
+    return p, vel
+
+
+def adagrad(p, g, cache, lr=0.01, eps=1e-8):
+    p, cache = _f32(p).copy(), _f32(cache).copy()
+    g = _f32(g)
+    lib().ref_adagrad(c_int64(p.size), _ptr(p), _ptr(g), _ptr(cache), c_float(lr), c_float(eps))
+    return p, cache
+
+
+def rmsprop(p, g, cache, lr=0.01, alpha=0.99, eps=1e-8):
+    p, cache = _f32(p).copy(), _f32(cache).copy()
+    g = _f32(g)
+    lib().ref_rmsprop(c_int64(p.size), _ptr(p), _ptr(g), _ptr(cache), c_float(lr), c_float(alpha), c_float(eps))
+    return p, cache
+
+
 def mlp_step(widths, act, x, target, Ws, bs, opt="none", lr=1e-3, b1=0.9, b2=0.999, eps=1e-8, t=1.0, state=None):
     """One fwd + bwd (+ optimizer) step. Ws/bs are updated IN PLACE when opt != "none".
 

@@ -133,6 +133,17 @@ for name, mk in [("sgd", lambda q: torch.optim.SGD([q], lr=1e-3)),
         q.grad = t64(g)
         opt.step()
         d["%s_p%d" % (name, i + 1)] = q.detach().numpy().copy()
+for name, mk in [("sgdm", lambda q: torch.optim.SGD([q], lr=1e-2, momentum=0.9)),
+                 ("sgdmw", lambda q: torch.optim.SGD([q], lr=1e-2, momentum=0.9, weight_decay=0.05)),
+                 ("sgdw", lambda q: torch.optim.SGD([q], lr=1e-2, weight_decay=0.05)),
+                 ("adagrad", lambda q: torch.optim.Adagrad([q], lr=1e-2, eps=1e-8)),
+                 ("rmsprop", lambda q: torch.optim.RMSprop([q], lr=1e-2, alpha=0.99, eps=1e-8))]:
+    q = t64(p0, True)
+    opt = mk(q)
+    for i, g in enumerate(gs):
+        q.grad = t64(g)
+        opt.step()
+        d["%s_p%d" % (name, i + 1)] = q.detach().numpy().copy()
 save("optim", **d)
 
 # ---- the reference's sine-fit MLP, three SGD steps (benchmarks/mlp_benchmarks/mlp_imp.mojo:25-75) -----

@@ -261,6 +261,26 @@ def test_hvp_double_backward(nd, golden, fused):
     assert abs(uHv - vHu) <= 1e-4 * max(abs(uHv), abs(vHu))
 
 
+def test_optimizer_classes(nd, golden):
+    g = golden("optim")
+    makers = {
+        "sgdm": lambda ps: nd.optim.SGD(ps, lr=1e-2, momentum=0.9),
+        "sgdmw": lambda ps: nd.optim.SGD(ps, lr=1e-2, momentum=0.9, weight_decay=0.05),
+        "sgdw": lambda ps: nd.optim.SGD(ps, lr=1e-2, weight_decay=0.05),
+        "adagrad": lambda ps: nd.optim.Adagrad(ps, lr=1e-2, eps=1e-8),
+        "rmsprop": lambda ps: nd.optim.RMSprop(ps, lr=1e-2, alpha=0.99, eps=1e-8),
+        "adam": lambda ps: nd.optim.Adam(ps, lr=1e-3),
+        "sgd": lambda ps: nd.optim.SGD(ps, lr=1e-3),
+    }
+    for name, mk in makers.items():
+        p = nd.array(g["p0"], requires_grad=True)
+        opt = mk([p])
+        for i in range(3):
+            p.grad_(nd.array(g["g%d" % i]))
+            opt.step()
+            assert_close(p.to_numpy(), g["%s_p%d" % (name, i + 1)], tol=2e-6, what="%s step %d" % (name, i))
+
+
 def test_complex_mlp_both_conventions(nd, golden):
     """Identity complex layers, loss = sum |out|^2. `_conj_vjp=True` gives the Wirtinger-conjugate
     gradients (equal to torch); the default follows the reference's coded rule without conjugation

@@ -219,6 +219,34 @@ def test_optimizers_bit_exact_vs_oracle(dev, golden):
     assert L.lib().endia_hip_adam_step(350, dp, dg, dm, dv, 1e-3, 0.9, 0.999, 1e-8, ctypes.c_float(0.0)) == L.ERR_INVALID
 
 
+def test_more_optimizers_bit_exact_vs_oracle(dev, golden):
+    g = golden("optim")
+    n = g["p0"].size
+    cases = {
+        "sgdm": ("endia_hip_sgd_momentum_step", (1e-2, 0.9, 0.0), lambda p, gr, st: R.sgd_momentum(p, gr, st, 1e-2, 0.9, 0.0)),
+        "sgdmw": ("endia_hip_sgd_momentum_step", (1e-2, 0.9, 0.05), lambda p, gr, st: R.sgd_momentum(p, gr, st, 1e-2, 0.9, 0.05)),
+        "sgdw": ("endia_hip_sgd_momentum_step", (1e-2, 0.0, 0.05), lambda p, gr, st: R.sgd_momentum(p, gr, st, 1e-2, 0.0, 0.05)),
+        "adagrad": ("endia_hip_adagrad_step", (1e-2, 1e-8), lambda p, gr, st: R.adagrad(p, gr, st, 1e-2, 1e-8)),
+        "rmsprop": ("endia_hip_rmsprop_step", (1e-2, 0.99, 1e-8), lambda p, gr, st: R.rmsprop(p, gr, st, 1e-2, 0.99, 1e-8)),
+    }
+    for name, (entry, hyper, ref) in cases.items():
+        p_ref, st_ref = g["p0"], np.zeros_like(g["p0"])
+        dp, ds = dev.put(g["p0"]), dev.put(st_ref)
+        for i in range(3):
+            dg = dev.put(g["g%d" % i])
+            dev.call(entry, n, dp, dg, ds, *hyper)
+            p_ref, st_ref = ref(p_ref, g["g%d" % i], st_ref)
+            np.testing.assert_array_equal(dev.get(dp, (50, 7)), p_ref, err_msg=name)
+            if name != "sgdw":
+                np.testing.assert_array_equal(dev.get(ds, (50, 7)), st_ref, err_msg=name + " state")
+            assert_close(dev.get(dp, (50, 7)), g["%s_p%d" % (name, i + 1)], tol=2e-6, what=name + " vs torch")
+    # weight decay without momentum needs no velocity buffer
+    dp, dg = dev.put(g["p0"]), dev.put(g["g0"])
+    dev.call("endia_hip_sgd_momentum_step", n, dp, dg, None, 1e-2, 0.0, 0.05)
+    np.testing.assert_array_equal(dev.get(dp, (50, 7)), R.sgd_momentum(g["p0"], g["g0"], np.zeros_like(g["p0"]), 1e-2, 0.0, 0.05)[0])
+    assert L.lib().endia_hip_sgd_momentum_step(n, dp, dg, None, ctypes.c_float(1e-2), ctypes.c_float(0.9), ctypes.c_float(0.0)) == L.ERR_INVALID
+
+
 def _desc(x, w, st, pd, dl):
     N, C, H, W = x.shape
     K, _, Rr, S = w.shape

@@ -161,6 +161,24 @@ def test_optimizers_golden(golden):
                      what="adam update %d" % i)
 
 
+def test_more_optimizers_golden(golden):
+    """SGD momentum / weight decay, Adagrad, RMSprop (optim/sgd.mojo:42-60, adagrad.mojo:36-45, rmsprop.mojo:39-53)
+    against torch.optim, three steps each. The reference stores velocity = -lr * (torch's momentum buffer)."""
+    g = golden("optim")
+    cases = {
+        "sgdm": lambda p, gr, st: R.sgd_momentum(p, gr, st, 1e-2, 0.9, 0.0),
+        "sgdmw": lambda p, gr, st: R.sgd_momentum(p, gr, st, 1e-2, 0.9, 0.05),
+        "sgdw": lambda p, gr, st: R.sgd_momentum(p, gr, st, 1e-2, 0.0, 0.05),
+        "adagrad": lambda p, gr, st: R.adagrad(p, gr, st, 1e-2, 1e-8),
+        "rmsprop": lambda p, gr, st: R.rmsprop(p, gr, st, 1e-2, 0.99, 1e-8),
+    }
+    for name, fn in cases.items():
+        p, st = g["p0"], np.zeros_like(g["p0"])
+        for i in range(3):
+            p, st = fn(p, g["g%d" % i], st)
+            assert_close(p, g["%s_p%d" % (name, i + 1)], tol=2e-6, what="%s step %d" % (name, i))
+
+
 def _mlp_case(g, n_layers):
     Ws = [np.ascontiguousarray(g["W%d" % i]) for i in range(n_layers)]
     bs = [np.ascontiguousarray(g["b%d" % i]) for i in range(n_layers)]
