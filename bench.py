@@ -337,6 +337,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--workload", default="wide_mlp", choices=["wide_mlp", "sine_mlp", "kernels", "conv2d", "hvp", "complex_mlp", "complex_mlp_3m"])
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--eager", action="store_true", help="sine_mlp: issue every kernel from the host instead of replaying a graph")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build runs on ONE GPU (no collectives, no sharding); --gpus %d is not supported. "
@@ -382,10 +383,15 @@ def main():
         train_step(nd, mlp, opt, x, y)
     nd.synchronize()
 
+    captured = None
+    if args.workload == "sine_mlp" and not args.eager:
+        # launch-latency bound: replay the step as one HIP graph (same kernels, same results)
+        captured = nd.capture(lambda: train_step(nd, mlp, opt, x, y))
+        config["execution"] = "HIP graph replay of the eager step"
     L.call("endia_hip_gemm_timing_begin")
     t0 = time.perf_counter()
     for _ in range(args.steps):
-        loss = train_step(nd, mlp, opt, x, y)
+        loss = captured.replay() if captured else train_step(nd, mlp, opt, x, y)
     nd.synchronize()
     elapsed = time.perf_counter() - t0
     launches, g_ms, g_flops = ctypes.c_int64(), ctypes.c_double(), ctypes.c_double()

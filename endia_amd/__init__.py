@@ -18,7 +18,8 @@ from .functional import (  # noqa: E402,F401
     zeros,
 )
 from .autograd.functional import backward, grad, hessian, jacobian, value_and_grad  # noqa: E402,F401
-from . import autograd, nn, optim, utils  # noqa: E402,F401
+from . import autograd, graph, nn, optim, utils  # noqa: E402,F401
+from .graph import capture  # noqa: E402,F401
 
 
 def synchronize():

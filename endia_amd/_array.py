@@ -98,6 +98,15 @@ class Array:
             L.call("endia_hip_memcpy_h2d", out._buf.ptr, a.ctypes.data, a.nbytes)
         return out
 
+    def copy_from_numpy(self, a):
+        """Overwrite this (contiguous) array's buffer in place, e.g. to feed a captured step its next batch."""
+        a = np.ascontiguousarray(a, dtype=np.complex64 if self.is_complex_ else np.float32)
+        if a.size != self.size() or not self.is_contiguous():
+            raise ValueError("copy_from_numpy: need a contiguous destination of the same element count")
+        if a.size:
+            L.call("endia_hip_memcpy_h2d", self.data_ptr(), a.ctypes.data, a.nbytes)
+        return self
+
     def to_numpy(self):
         c = self if self.is_contiguous() else _contiguous_copy(self)
         out = np.empty(self._shape, dtype=np.complex64 if self.is_complex_ else np.float32)

@@ -54,6 +54,10 @@ SIGNATURES = {
     "endia_hip_timer_start": [c_int32],
     "endia_hip_timer_stop": [c_int32],
     "endia_hip_timer_elapsed_ms": [c_int32, POINTER(c_float)],
+    "endia_hip_graph_begin": [],
+    "endia_hip_graph_end": [_i64p],
+    "endia_hip_graph_launch": [c_int64],
+    "endia_hip_graph_destroy": [c_int64],
     "endia_hip_gemm_timing_begin": [],
     "endia_hip_gemm_timing_end": [_i64p, POINTER(c_double), POINTER(c_double)],
     "endia_hip_strided_copy": [c_int32, _i64p, _i64p, c_int64, _fp, _fp, c_int32],
@@ -83,6 +87,7 @@ SIGNATURES = {
 
 _lib = None
 _ready = False
+capturing = False  # set by endia_amd.graph while a step is being recorded
 
 
 def lib():

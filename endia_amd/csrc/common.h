@@ -11,6 +11,7 @@ namespace endia {
 
 struct Context {
   bool ready = false;
+  bool capturing = false;  // between endia_hip_graph_begin and endia_hip_graph_end
   int device = -1;
   hipStream_t stream = nullptr;
   int cu_count = 0;

@@ -334,7 +334,7 @@ int32_t sgemm_impl(int transA, int transB, int64_t M, int64_t N, int64_t K, cons
       p.sC = M * N;
     }
     dim3 grid((unsigned)tiles, (unsigned)(splits > 1 ? splits : batch));
-    const bool timed = g_timing.on;
+    const bool timed = g_timing.on && !ctx().capturing;
     if (timed) {
       if (g_timing.used == g_timing.start.size()) {
         hipEvent_t a, b;

@@ -37,19 +37,36 @@ static int64_t bucket_of(int64_t bytes) {
   return (bytes + large - 1) / large * large;
 }
 
+struct Live {
+  int64_t bucket;
+  int64_t graph;  // 0, or the captured graph during whose capture the buffer was handed out
+};
+
 struct Pool {
   std::multimap<int64_t, void*> free_by_size;
-  std::unordered_map<void*, int64_t> live;    // pointer -> bucket size, handed out
+  std::unordered_map<void*, Live> live;       // handed out
   std::unordered_map<void*, int64_t> owned;   // every pointer obtained from hipMalloc
   int64_t in_use = 0, cached = 0, n_allocs = 0;
 };
 static Pool g_pool;
+
+// A captured step keeps every buffer that was handed out while it was being captured: its kernels hold
+// those addresses, so the buffers go back to the pool only when the graph is destroyed.
+struct Graph {
+  hipGraph_t graph = nullptr;
+  hipGraphExec_t exec = nullptr;
+  std::vector<std::pair<void*, int64_t>> retained;  // released by their holders, kept for replays
+};
+static std::unordered_map<int64_t, Graph> g_graphs;
+static int64_t g_next_graph = 1, g_capture_id = 0;
 
 static void* g_ws = nullptr;
 static int64_t g_ws_bytes = 0;
 
 int32_t workspace(int64_t bytes, void** out) {
   if (bytes > g_ws_bytes) {
+    if (g_ctx.capturing)
+      return fail(ENDIA_HIP_ERR_UNSUPPORTED, "workspace: would have to grow during capture; run the step once eagerly first");
     if (g_ws) (void)hipFree(g_ws);
     g_ws = nullptr;
     g_ws_bytes = 0;
@@ -71,6 +88,8 @@ static bool g_ev_made = false;
 }  // namespace endia
 
 using namespace endia;
+
+static void release_graph(int64_t id);
 
 extern "C" {
 
@@ -111,6 +130,7 @@ int32_t endia_hip_init(int32_t device) {
 int32_t endia_hip_shutdown(void) {
   if (!g_ctx.ready) return ENDIA_HIP_OK;
   (void)hipStreamSynchronize(g_ctx.stream);
+  while (!g_graphs.empty()) release_graph(g_graphs.begin()->first);
   for (auto& kv : g_pool.owned) (void)hipFree(kv.first);
   g_pool = Pool();
   if (g_ws) (void)hipFree(g_ws);
@@ -123,6 +143,7 @@ int32_t endia_hip_shutdown(void) {
 
 int32_t endia_hip_sync(void) {
   ENDIA_REQUIRE_INIT();
+  if (g_ctx.capturing) return fail(ENDIA_HIP_ERR_UNSUPPORTED, "%s: not allowed while a step is being captured", __func__);
   ENDIA_HIP_CALL(hipStreamSynchronize(g_ctx.stream));
   return ENDIA_HIP_OK;
 }
@@ -173,7 +194,7 @@ int32_t endia_hip_malloc(int64_t bytes, void** out) {
     g_pool.owned[p] = b;
     g_pool.n_allocs++;
   }
-  g_pool.live[p] = b;
+  g_pool.live[p] = Live{b, g_ctx.capturing ? g_capture_id : 0};
   g_pool.in_use += b;
   *out = p;
   return ENDIA_HIP_OK;
@@ -184,9 +205,15 @@ int32_t endia_hip_free(void* p) {
   if (!p) return ENDIA_HIP_OK;
   auto it = g_pool.live.find(p);
   ENDIA_CHECK_ARG(it != g_pool.live.end(), "endia_hip_free: %p was not handed out by endia_hip_malloc", p);
-  int64_t b = it->second;
+  int64_t b = it->second.bucket;
+  int64_t owner = it->second.graph;
   g_pool.live.erase(it);
   g_pool.in_use -= b;
+  auto g = owner ? g_graphs.find(owner) : g_graphs.end();
+  if (g != g_graphs.end()) {
+    g->second.retained.emplace_back(p, b);  // still written by replays of that graph
+    return ENDIA_HIP_OK;
+  }
   g_pool.free_by_size.emplace(b, p);
   g_pool.cached += b;
   return ENDIA_HIP_OK;
@@ -202,6 +229,7 @@ int32_t endia_hip_pool_stats(int64_t* bytes_in_use, int64_t* bytes_cached, int64
 
 int32_t endia_hip_pool_trim(void) {
   ENDIA_REQUIRE_INIT();
+  if (g_ctx.capturing) return fail(ENDIA_HIP_ERR_UNSUPPORTED, "%s: not allowed while a step is being captured", __func__);
   ENDIA_HIP_CALL(hipStreamSynchronize(g_ctx.stream));
   for (auto& kv : g_pool.free_by_size) {
     (void)hipFree(kv.second);
@@ -214,6 +242,7 @@ int32_t endia_hip_pool_trim(void) {
 
 int32_t endia_hip_memcpy_h2d(void* dst, const void* src, int64_t bytes) {
   ENDIA_REQUIRE_INIT();
+  if (g_ctx.capturing) return fail(ENDIA_HIP_ERR_UNSUPPORTED, "%s: not allowed while a step is being captured", __func__);
   ENDIA_CHECK_ARG(bytes >= 0, "endia_hip_memcpy_h2d: negative size");
   if (bytes == 0) return ENDIA_HIP_OK;
   ENDIA_CHECK_ARG(dst && src, "endia_hip_memcpy_h2d: null pointer");
@@ -225,6 +254,7 @@ int32_t endia_hip_memcpy_h2d(void* dst, const void* src, int64_t bytes) {
 
 int32_t endia_hip_memcpy_d2h(void* dst, const void* src, int64_t bytes) {
   ENDIA_REQUIRE_INIT();
+  if (g_ctx.capturing) return fail(ENDIA_HIP_ERR_UNSUPPORTED, "%s: not allowed while a step is being captured", __func__);
   ENDIA_CHECK_ARG(bytes >= 0, "endia_hip_memcpy_d2h: negative size");
   if (bytes == 0) return ENDIA_HIP_OK;
   ENDIA_CHECK_ARG(dst && src, "endia_hip_memcpy_d2h: null pointer");
@@ -244,6 +274,7 @@ int32_t endia_hip_memcpy_d2d(void* dst, const void* src, int64_t bytes) {
 
 int32_t endia_hip_timer_start(int32_t slot) {
   ENDIA_REQUIRE_INIT();
+  if (g_ctx.capturing) return fail(ENDIA_HIP_ERR_UNSUPPORTED, "%s: not allowed while a step is being captured", __func__);
   ENDIA_CHECK_ARG(slot >= 0 && slot < kTimerSlots, "endia_hip_timer_start: slot %d out of range", slot);
   ENDIA_HIP_CALL(hipEventRecord(g_ev_start[slot], g_ctx.stream));
   return ENDIA_HIP_OK;
@@ -251,6 +282,7 @@ int32_t endia_hip_timer_start(int32_t slot) {
 
 int32_t endia_hip_timer_stop(int32_t slot) {
   ENDIA_REQUIRE_INIT();
+  if (g_ctx.capturing) return fail(ENDIA_HIP_ERR_UNSUPPORTED, "%s: not allowed while a step is being captured", __func__);
   ENDIA_CHECK_ARG(slot >= 0 && slot < kTimerSlots, "endia_hip_timer_stop: slot %d out of range", slot);
   ENDIA_HIP_CALL(hipEventRecord(g_ev_stop[slot], g_ctx.stream));
   return ENDIA_HIP_OK;
@@ -262,6 +294,75 @@ int32_t endia_hip_timer_elapsed_ms(int32_t slot, float* ms) {
   ENDIA_CHECK_ARG(ms != nullptr, "endia_hip_timer_elapsed_ms: ms is null");
   ENDIA_HIP_CALL(hipEventSynchronize(g_ev_stop[slot]));
   ENDIA_HIP_CALL(hipEventElapsedTime(ms, g_ev_start[slot], g_ev_stop[slot]));
+  return ENDIA_HIP_OK;
+}
+
+// ---- captured steps --------------------------------------------------------------------------
+// Everything enqueued between begin and end is recorded into a HIP graph instead of being executed.
+// Launch-latency-bound steps (the reference's 1-32-64-128-128-128-64-32-1 sine-fit MLP issues ~60
+// kernels of a few microseconds each) are then replayed with one launch.
+int32_t endia_hip_graph_begin(void) {
+  ENDIA_REQUIRE_INIT();
+  ENDIA_CHECK_ARG(!g_ctx.capturing, "endia_hip_graph_begin: a capture is already in progress");
+  ENDIA_HIP_CALL(hipStreamSynchronize(g_ctx.stream));
+  g_capture_id = g_next_graph++;
+  g_graphs[g_capture_id] = Graph();
+  hipError_t e = hipStreamBeginCapture(g_ctx.stream, hipStreamCaptureModeRelaxed);
+  if (e != hipSuccess) {
+    g_graphs.erase(g_capture_id);
+    return fail(ENDIA_HIP_ERR_RUNTIME, "endia_hip_graph_begin: hipStreamBeginCapture failed: %s", hipGetErrorString(e));
+  }
+  g_ctx.capturing = true;
+  return ENDIA_HIP_OK;
+}
+
+static void release_graph(int64_t id) {
+  auto it = g_graphs.find(id);
+  if (it == g_graphs.end()) return;
+  if (it->second.exec) (void)hipGraphExecDestroy(it->second.exec);
+  if (it->second.graph) (void)hipGraphDestroy(it->second.graph);
+  for (auto& pb : it->second.retained) {
+    g_pool.free_by_size.emplace(pb.second, pb.first);
+    g_pool.cached += pb.second;
+  }
+  g_graphs.erase(it);
+  // buffers of this graph that are still held elsewhere become ordinary buffers
+  for (auto& kv : g_pool.live)
+    if (kv.second.graph == id) kv.second.graph = 0;
+}
+
+int32_t endia_hip_graph_end(int64_t* handle) {
+  ENDIA_REQUIRE_INIT();
+  ENDIA_CHECK_ARG(g_ctx.capturing, "endia_hip_graph_end: no capture in progress");
+  g_ctx.capturing = false;
+  const int64_t id = g_capture_id;
+  Graph& g = g_graphs[id];
+  hipError_t e = hipStreamEndCapture(g_ctx.stream, &g.graph);
+  if (e == hipSuccess) e = hipGraphInstantiate(&g.exec, g.graph, nullptr, nullptr, 0);
+  if (e != hipSuccess || !handle) {
+    (void)hipGetLastError();
+    release_graph(id);
+    if (!handle) return fail(ENDIA_HIP_ERR_INVALID, "endia_hip_graph_end: handle is null");
+    return fail(ENDIA_HIP_ERR_RUNTIME, "endia_hip_graph_end: capture failed: %s", hipGetErrorString(e));
+  }
+  *handle = id;
+  return ENDIA_HIP_OK;
+}
+
+int32_t endia_hip_graph_launch(int64_t handle) {
+  ENDIA_REQUIRE_INIT();
+  ENDIA_CHECK_ARG(!g_ctx.capturing, "endia_hip_graph_launch: not allowed while a step is being captured");
+  auto it = g_graphs.find(handle);
+  ENDIA_CHECK_ARG(it != g_graphs.end() && it->second.exec, "endia_hip_graph_launch: unknown graph %lld", (long long)handle);
+  ENDIA_HIP_CALL(hipGraphLaunch(it->second.exec, g_ctx.stream));
+  return ENDIA_HIP_OK;
+}
+
+int32_t endia_hip_graph_destroy(int64_t handle) {
+  ENDIA_REQUIRE_INIT();
+  ENDIA_CHECK_ARG(g_graphs.count(handle), "endia_hip_graph_destroy: unknown graph %lld", (long long)handle);
+  ENDIA_HIP_CALL(hipStreamSynchronize(g_ctx.stream));
+  release_graph(handle);
   return ENDIA_HIP_OK;
 }
 

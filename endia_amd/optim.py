@@ -86,6 +86,9 @@ class Adam:
         self.v = [Array(p.shape()) for p in self.params]
 
     def step(self):
+        if L.capturing:
+            raise NotImplementedError("Adam inside a captured step: its bias correction 1 - beta^t changes every step, "
+                                      "but a captured kernel's scalar arguments are frozen")
         for p, m, v in zip(self.params, self.m, self.v):
             g = _flat_grad(p)
             assert p.is_contiguous()

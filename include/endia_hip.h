@@ -103,6 +103,17 @@ ENDIA_API int32_t endia_hip_timer_start(int32_t slot);
 ENDIA_API int32_t endia_hip_timer_stop(int32_t slot);
 ENDIA_API int32_t endia_hip_timer_elapsed_ms(int32_t slot, float* ms); /* blocks until the stop event */
 
+/* ---- captured steps (HIP graphs). No counterpart in the reference. Calls made between begin and end are
+ *      recorded, not executed; endia_hip_graph_launch replays them on the library's stream with one launch.
+ *      While capturing, host<->device copies, endia_hip_sync and the timers return ENDIA_HIP_ERR_UNSUPPORTED.
+ *      Buffers handed out during the capture stay reserved for the graph until endia_hip_graph_destroy, even
+ *      after their holders free them, because the recorded kernels keep their addresses. Scalar arguments
+ *      (learning rate, Adam's step counter) are frozen at capture time. */
+ENDIA_API int32_t endia_hip_graph_begin(void);
+ENDIA_API int32_t endia_hip_graph_end(int64_t* handle);
+ENDIA_API int32_t endia_hip_graph_launch(int64_t handle);
+ENDIA_API int32_t endia_hip_graph_destroy(int64_t handle);
+
 /* ---- per-launch timing of the MFMA GEMM kernel. Between begin and end every launch of the tiled
  *      fp32 GEMM kernel is bracketed by a pair of HIP events on the library's stream; end blocks, then
  *      reports the number of launches, the sum of their durations and of their 2*M*N*K*batch flops.

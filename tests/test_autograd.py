@@ -332,6 +332,59 @@ def test_conv2d_autograd(nd, golden):
     assert_close(x2.grad().to_numpy(), tx.grad.numpy(), what="dx")
 
 
+def test_captured_step_matches_eager(nd, golden):
+    """The sine-fit MLP step recorded into a HIP graph: every replay must leave exactly the parameters the
+    eager step leaves. Replays are interleaved with eager work and synchronisations."""
+    g = golden("mlp_sine")
+
+    def build():
+        mlp, _ = _load_mlp(nd, g, 8, "relu", True)
+        opt = nd.optim.SGD(mlp.params(), lr=1e-3, momentum=0.9)
+        x, y = nd.array(g["x"]), nd.array(g["y"])
+
+        def step():
+            loss = nd.mse(mlp.forward(x), y)
+            loss.backward()
+            opt.step()
+            loss.zero_grad()
+            return loss
+        return mlp, step, x
+
+    mlp_e, step_e, _ = build()
+    mlp_c, step_c, x_c = build()
+    step_e()
+    step_c()                                  # warm-up: pool and workspace sized
+    captured = nd.capture(step_c)             # recorded, not executed
+    scratch = nd.randn([300, 70])
+    for it in range(4):
+        loss_e = step_e()
+        loss_c = captured.replay()
+        nd.synchronize()
+        scratch = nd.tanh(scratch @ nd.randn([70, 70]))   # eager work between replays reuses pool buffers
+        assert loss_c.item() == loss_e.item(), "replay %d" % it
+        for pe, pc in zip(mlp_e.params(), mlp_c.params()):
+            np.testing.assert_array_equal(pc.to_numpy(), pe.to_numpy())
+    # new input through the fixed buffer
+    xb = np.linspace(0, 1, 128, dtype=np.float32).reshape(128, 1)
+    x_c.copy_from_numpy(xb)
+    before = mlp_c.weights[3].to_numpy()
+    captured.replay()
+    assert not np.array_equal(mlp_c.weights[3].to_numpy(), before)
+    captured.close()
+    with pytest.raises(RuntimeError):
+        captured.replay()
+    # host reads and Adam are refused inside a capture, and the failed capture leaves the library usable
+    with pytest.raises(nd._lib.EndiaHipError, match="captured"):
+        nd.capture(lambda: scratch.to_numpy())
+    mlp_a, _ = _load_mlp(nd, g, 8, "relu", True)
+    adam = nd.optim.Adam(mlp_a.params())
+    for p in mlp_a.params():
+        p.grad_(nd.zeros(p.shape()))
+    with pytest.raises(NotImplementedError):
+        nd.capture(adam.step)
+    assert nd.sum(nd.ones([5])).item() == 5.0
+
+
 def test_shape_errors(nd):
     with pytest.raises(ValueError, match="ndim < 2"):
         nd.matmul(nd.zeros([3]), nd.zeros([3, 3]))
