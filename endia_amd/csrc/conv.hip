@@ -738,14 +738,22 @@ int32_t run_igemm_vec(int mode, const ConvP& p, const float* src, const float* w
   a.tiles_n = (a.Ncols + 127) / 128;
   hipStream_t s = endia::ctx().stream;
   const size_t dyn = (size_t)Kd_pad * 4;
-  if (Mrows > 64) {
+  // 128-row tiles, or 64-row tiles when they waste fewer MFMA rows or spread more evenly over the CUs
+  // (the busiest CU sets the time: ceil(tiles / CUs) against tiles / CUs)
+  const double cus = (double)endia::ctx().cu_count;
+  auto cost = [&](int bm) {
+    double tm = (double)((Mrows + bm - 1) / bm), t = tm * a.tiles_n;
+    double rounds = t >= cus ? ((int64_t)((t + cus - 1) / cus)) / (t / cus) : 1.0;
+    return rounds * (tm * bm) / (double)Mrows;
+  };
+  if (cost(128) <= cost(64) * 0.97) {
     a.tiles_m = (Mrows + 127) / 128;
     dim3 grid((unsigned)(a.tiles_m * a.tiles_n));
     if (fwd) hipLaunchKernelGGL((conv_igemm_vec_kernel<2, 2, 2, 2, true>), grid, dim3(256), dyn, s, a);
     else hipLaunchKernelGGL((conv_igemm_vec_kernel<2, 2, 2, 2, false>), grid, dim3(256), dyn, s, a);
   } else {
-    a.tiles_m = 1;
-    dim3 grid((unsigned)a.tiles_n);
+    a.tiles_m = (Mrows + 63) / 64;
+    dim3 grid((unsigned)(a.tiles_m * a.tiles_n));
     if (fwd) hipLaunchKernelGGL((conv_igemm_vec_kernel<1, 4, 2, 1, true>), grid, dim3(256), dyn, s, a);
     else hipLaunchKernelGGL((conv_igemm_vec_kernel<1, 4, 2, 1, false>), grid, dim3(256), dyn, s, a);
   }
@@ -859,8 +867,13 @@ int32_t endia_hip_conv2d_bwd_weight(const endia_hip_conv2d_desc* d, const float*
   a.d_rs = make_fastdiv(p.R * p.S); a.d_s = make_fastdiv(p.S);
   a.x_bytes = (int64_t)p.N * p.C * p.H * p.W * 4;
   a.dy_bytes = (int64_t)p.N * p.K * p.P * p.Q * 4;
+  const int Hp = p.H + 2 * p.ph, Wp = p.W + 2 * p.pw;
+  const bool vec = p.sw == 1 && p.Q % 4 == 0 && (int64_t)p.N * p.C * Hp * Wp < (1ll << 29) &&
+                   (reinterpret_cast<uintptr_t>(dy) & 15) == 0;
+  // 64-wide tiles over the taps when the last 128-wide tile would be at most half full
+  const int bn = (vec && Kd % 128 != 0 && Kd % 128 <= 64) ? 64 : 128;
   a.tiles_m = (p.K + 127) / 128;
-  a.tiles_n = (Kd + 127) / 128;
+  a.tiles_n = (Kd + bn - 1) / bn;
   // split the N*P*Q reduction so that about 4 work-groups per CU exist; every split reduces >= 256 columns
   int64_t tiles = (int64_t)a.tiles_m * a.tiles_n;
   int64_t splits = ((int64_t)ctx().cu_count * 4 + tiles - 1) / tiles;
@@ -881,20 +894,18 @@ int32_t endia_hip_conv2d_bwd_weight(const endia_hip_conv2d_desc* d, const float*
     a.part = dw;
   }
   dim3 grid((unsigned)tiles, (unsigned)splits);
-  const int Hp = p.H + 2 * p.ph, Wp = p.W + 2 * p.pw;
-  const bool vec = p.sw == 1 && p.Q % 4 == 0 && (int64_t)p.N * p.C * Hp * Wp < (1ll << 29) &&
-                   (reinterpret_cast<uintptr_t>(dy) & 15) == 0;
   if (vec) {
     PoolBuf xpad, table;
     if ((rc = make_padded(x, (int64_t)p.N * p.C, p.H, p.W, p.ph, p.pw, xpad))) return rc;
-    if ((rc = make_table(a.tiles_n * 128, Kd, p.R, p.S, Hp, Wp, p.dh, p.dw, 0, table))) return rc;
+    if ((rc = make_table(a.tiles_n * bn, Kd, p.R, p.S, Hp, Wp, p.dh, p.dw, 0, table))) return rc;
     WgradVecArgs v;
     v.xpad = static_cast<const float*>(xpad.p); v.dy = dy; v.table = static_cast<const int*>(table.p); v.part = a.part;
     v.K = p.K; v.Kd = Kd; v.PQ = p.P * p.Q; v.Q = p.Q; v.sh = p.sh; v.Wp = Wp; v.img_floats = p.C * Hp * Wp;
     v.total_j = a.total_j; v.chunk = a.chunk; v.d_pq = a.d_pq; v.d_q = a.d_q;
     v.tiles_m = a.tiles_m; v.tiles_n = a.tiles_n;
     v.x_bytes = (int64_t)p.N * p.C * Hp * Wp * 4; v.dy_bytes = a.dy_bytes;
-    hipLaunchKernelGGL((conv_wgrad_vec_kernel<2, 2, 2, 2>), grid, dim3(256), 0, s, v);
+    if (bn == 128) hipLaunchKernelGGL((conv_wgrad_vec_kernel<2, 2, 2, 2>), grid, dim3(256), 0, s, v);
+    else hipLaunchKernelGGL((conv_wgrad_vec_kernel<2, 2, 2, 1>), grid, dim3(256), 0, s, v);
   } else {
     hipLaunchKernelGGL((conv_wgrad_kernel<2, 2, 2, 2>), grid, dim3(256), 0, s, a);
   }
