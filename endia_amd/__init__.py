@@ -12,13 +12,15 @@ _lib.lib()  # fail loudly when the HIP library has not been built
 
 from ._array import Array, Tensor, ndarray  # noqa: E402
 from .functional import (  # noqa: E402,F401
-    abs, add, arange, array, complex, conj, contiguous, conv2d, cos, detach, div, expand, eye, full, greater, imag,
-    linear, matmul, mean, mse, mul, neg, ones, permute, rand_he_normal, randn, randn_complex, randu, real, reduce_add,
-    relu, reshape, seed, set_complex_matmul_algorithm, sign, sin, sqrt, square, squeeze, sub, sum, tanh, unsqueeze,
-    zeros,
+    abs, acos, add, arange, array, asin, atan, complex, conj, contiguous, conv2d, cos, cosh, detach, div, equal, exp,
+    expand, eye, full, greater, greater_equal, imag, less, less_equal, linear, log, matmul, mean, mse, mul, neg,
+    not_equal, ones, permute, pow, pow_to, rand_he_normal, randn, randn_complex, randu, real, reciprocal, reduce_add,
+    relu, reshape, seed, set_complex_matmul_algorithm, sigmoid, sign, sin, sinh, sqrt, square, squeeze, sub, sum, tan,
+    tanh, unsqueeze, zeros,
 )
 from .autograd.functional import backward, grad, hessian, jacobian, value_and_grad  # noqa: E402,F401
-from . import autograd, graph, nn, optim, utils  # noqa: E402,F401
+from . import autograd, fusion, graph, nn, optim, utils  # noqa: E402,F401
+from .fusion import fuse  # noqa: E402,F401
 from .graph import capture  # noqa: E402,F401
 
 

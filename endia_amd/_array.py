@@ -246,9 +246,13 @@ class Array:
         from . import functional as F
         return F.neg(self)
 
-    def __pow__(self, p):
+    def __pow__(self, o):  # pow_to, with a scalar spread over the last axis (_array.mojo:1074-1079)
         from . import functional as F
-        return F.pow_int(self, p)
+        return self._bin(o, F.pow)
+
+    def __rpow__(self, o):
+        from . import functional as F
+        return self._bin(o, F.pow, reverse=True)
 
     # in-place updates write through to the existing buffer (execute_copy_raw, _array.mojo:998-1006)
     def _assign_from(self, other):

@@ -12,8 +12,14 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libendia_hip.so")
 
 # enums of include/endia_hip.h
-OP_RELU, OP_TANH, OP_SIN, OP_COS, OP_NEG, OP_SQUARE, OP_SQRT, OP_ABS, OP_IDENTITY, OP_GREATER0 = range(10)
-BIN_ADD, BIN_SUB, BIN_MUL, BIN_DIV, BIN_GREATER = range(5)
+(OP_RELU, OP_TANH, OP_SIN, OP_COS, OP_NEG, OP_SQUARE, OP_SQRT, OP_ABS, OP_IDENTITY, OP_GREATER0, OP_EXP, OP_LOG,
+ OP_SIGMOID, OP_SINH, OP_COSH, OP_TAN, OP_ASIN, OP_ACOS, OP_ATAN, OP_RECIPROCAL, OP_SIGN) = range(21)
+(BIN_ADD, BIN_SUB, BIN_MUL, BIN_DIV, BIN_GREATER, BIN_POW, BIN_GREATER_EQUAL, BIN_LESS, BIN_LESS_EQUAL, BIN_EQUAL,
+ BIN_NOT_EQUAL) = range(11)
+EW_LOAD, EW_UNARY, EW_BINARY, EW_RBINARY, EW_SAVE, EW_STORE = range(6)
+EW_SRC_INPUT, EW_SRC_SLOT, EW_SRC_IMM = range(3)
+EW_FULL, EW_ROW_VECTOR, EW_SCALAR = range(3)
+EW_MAX_INPUTS, EW_MAX_OUTPUTS, EW_MAX_SLOTS, EW_MAX_STEPS = 8, 4, 4, 48
 EPI_NONE, EPI_BIAS, EPI_BIAS_ACT, EPI_ACT_GRAD = range(4)
 ACT_FROM_OUTPUT = 0x100
 GEMM_ACCUMULATE = 0x200
@@ -32,6 +38,10 @@ class Conv2dDesc(ctypes.Structure):
     _fields_ = [(n, c_int64) for n in (
         "N", "C", "H", "W", "K", "R", "S",
         "stride_h", "stride_w", "pad_h", "pad_w", "dil_h", "dil_w", "groups")]
+
+
+class EwStep(ctypes.Structure):
+    _fields_ = [("kind", c_int32), ("op", c_int32), ("src_kind", c_int32), ("src_index", c_int32), ("imm", c_float)]
 
 
 _fp = c_void_p  # device pointers travel as plain addresses
@@ -69,6 +79,8 @@ SIGNATURES = {
     "endia_hip_unary_vjp": [c_int32, c_int64, _fp, _fp, _fp, c_int32],
     "endia_hip_unary_vjp_from_output": [c_int32, c_int64, _fp, _fp, _fp],
     "endia_hip_binary": [c_int32, c_int32, _i64p, _i64p, _i64p, _fp, _fp, _fp, c_int32],
+    "endia_hip_ew_program": [c_int64, c_int64, c_int32, POINTER(c_void_p), POINTER(c_int32), c_int32, POINTER(c_void_p),
+                             c_int32, POINTER(EwStep)],
     "endia_hip_axpby": [c_int64, c_float, _fp, c_float, _fp, _fp],
     "endia_hip_complex_pack": [c_int64, _fp, _fp, _fp],
     "endia_hip_reduce_add": [c_int32, _i64p, c_uint32, _fp, _fp, c_float, c_int32],

@@ -6,8 +6,17 @@
 // consecutive addresses, and the grid is a few work-groups per CU walking the tensor with a
 // grid stride.
 #include "common.h"
+#include "ew_ops.h"
+
+#include <utility>
 
 namespace {
+
+using endia::bin_complex;
+using endia::bin_real;
+using endia::unary_complex;
+using endia::unary_real;
+using endia::unary_vjp_real;
 
 constexpr int TPB = 256;
 
@@ -40,39 +49,6 @@ __global__ __launch_bounds__(TPB) void fill_scalar_kernel(float* __restrict__ p,
 }
 
 // ---- unary ----------------------------------------------------------------------------------
-template <int OP>
-__device__ __forceinline__ float unary_real(float x) {
-  switch (OP) {
-    case ENDIA_OP_RELU: return x > 0.f ? x : 0.f;
-    case ENDIA_OP_TANH: return tanhf(x);
-    case ENDIA_OP_SIN: return sinf(x);
-    case ENDIA_OP_COS: return cosf(x);
-    case ENDIA_OP_NEG: return -x;
-    case ENDIA_OP_SQUARE: return x * x;
-    case ENDIA_OP_SQRT: return sqrtf((fabsf(x) + x) * 0.5f);  // 0 for negative x, as the reference
-    case ENDIA_OP_ABS: return fabsf(x);
-    case ENDIA_OP_GREATER0: return x > 0.f ? 1.f : 0.f;
-    default: return x;
-  }
-}
-
-// g * d(op)/dx at x
-template <int OP>
-__device__ __forceinline__ float unary_vjp_real(float x, float g) {
-  switch (OP) {
-    case ENDIA_OP_RELU: return x > 0.f ? g : 0.f;
-    case ENDIA_OP_TANH: { float t = tanhf(x); return (1.f - t * t) * g; }
-    case ENDIA_OP_SIN: return cosf(x) * g;
-    case ENDIA_OP_COS: return -sinf(x) * g;
-    case ENDIA_OP_NEG: return -g;
-    case ENDIA_OP_SQUARE: return 2.f * x * g;
-    case ENDIA_OP_SQRT: return g / (2.f * sqrtf((fabsf(x) + x) * 0.5f));
-    case ENDIA_OP_ABS: return (x > 0.f ? 1.f : (x < 0.f ? -1.f : 0.f)) * g;
-    case ENDIA_OP_GREATER0: return 0.f;
-    default: return g;
-  }
-}
-
 template <int OP, bool VEC>
 __global__ __launch_bounds__(TPB) void unary_fwd_kernel(const float* __restrict__ x, float* __restrict__ y, int64_t n) {
   int64_t i = (int64_t)blockIdx.x * TPB + threadIdx.x;
@@ -83,11 +59,11 @@ __global__ __launch_bounds__(TPB) void unary_fwd_kernel(const float* __restrict_
     float4* y4 = reinterpret_cast<float4*>(y);
     for (int64_t j = i; j < n4; j += stride) {
       float4 a = x4[j];
-      y4[j] = make_float4(unary_real<OP>(a.x), unary_real<OP>(a.y), unary_real<OP>(a.z), unary_real<OP>(a.w));
+      y4[j] = make_float4(unary_real(OP, a.x), unary_real(OP, a.y), unary_real(OP, a.z), unary_real(OP, a.w));
     }
-    for (int64_t j = (n4 << 2) + i; j < n; j += stride) y[j] = unary_real<OP>(x[j]);
+    for (int64_t j = (n4 << 2) + i; j < n; j += stride) y[j] = unary_real(OP, x[j]);
   } else {
-    for (int64_t j = i; j < n; j += stride) y[j] = unary_real<OP>(x[j]);
+    for (int64_t j = i; j < n; j += stride) y[j] = unary_real(OP, x[j]);
   }
 }
 
@@ -103,12 +79,12 @@ __global__ __launch_bounds__(TPB) void unary_vjp_kernel(const float* __restrict_
     float4* d4 = reinterpret_cast<float4*>(dx);
     for (int64_t j = i; j < n4; j += stride) {
       float4 a = x4[j], b = g4[j];
-      d4[j] = make_float4(unary_vjp_real<OP>(a.x, b.x), unary_vjp_real<OP>(a.y, b.y),
-                          unary_vjp_real<OP>(a.z, b.z), unary_vjp_real<OP>(a.w, b.w));
+      d4[j] = make_float4(unary_vjp_real(OP, a.x, b.x), unary_vjp_real(OP, a.y, b.y),
+                          unary_vjp_real(OP, a.z, b.z), unary_vjp_real(OP, a.w, b.w));
     }
-    for (int64_t j = (n4 << 2) + i; j < n; j += stride) dx[j] = unary_vjp_real<OP>(x[j], g[j]);
+    for (int64_t j = (n4 << 2) + i; j < n; j += stride) dx[j] = unary_vjp_real(OP, x[j], g[j]);
   } else {
-    for (int64_t j = i; j < n; j += stride) dx[j] = unary_vjp_real<OP>(x[j], g[j]);
+    for (int64_t j = i; j < n; j += stride) dx[j] = unary_vjp_real(OP, x[j], g[j]);
   }
 }
 
@@ -116,17 +92,8 @@ __global__ __launch_bounds__(TPB) void vjp_from_output_kernel(int op, const floa
                                                               const float* __restrict__ g, float* __restrict__ dx,
                                                               int64_t n) {
   int64_t stride = (int64_t)gridDim.x * TPB;
-  for (int64_t j = (int64_t)blockIdx.x * TPB + threadIdx.x; j < n; j += stride) {
-    float a = y[j], c = g[j];
-    float r;
-    switch (op) {
-      case ENDIA_OP_RELU: r = a > 0.f ? c : 0.f; break;
-      case ENDIA_OP_TANH: r = (1.f - a * a) * c; break;
-      case ENDIA_OP_SQRT: r = c / (2.f * a); break;
-      default: r = c; break;
-    }
-    dx[j] = r;
-  }
+  for (int64_t j = (int64_t)blockIdx.x * TPB + threadIdx.x; j < n; j += stride)
+    dx[j] = endia::unary_vjp_from_output(op, y[j], g[j]);
 }
 
 // complex forward: one complex element (8 bytes) per lane access
@@ -137,12 +104,8 @@ __global__ __launch_bounds__(TPB) void unary_fwd_complex_kernel(int op, const fl
   float2* y2 = reinterpret_cast<float2*>(y);
   for (int64_t j = i; j < n; j += stride) {
     float2 z = x[j];
-    switch (op) {
-      case ENDIA_OP_NEG: y2[j] = make_float2(-z.x, -z.y); break;
-      case ENDIA_OP_SQUARE: y2[j] = make_float2(z.x * z.x - z.y * z.y, 2.f * z.x * z.y); break;
-      case ENDIA_OP_ABS: y[j] = sqrtf(z.x * z.x + z.y * z.y); break;
-      default: y2[j] = z; break;
-    }
+    if (op == ENDIA_OP_ABS) y[j] = sqrtf(z.x * z.x + z.y * z.y);
+    else y2[j] = unary_complex(op, z);
   }
 }
 
@@ -181,30 +144,6 @@ struct BinDesc {
   int64_t bs[8];
 };
 
-template <int OP>
-__device__ __forceinline__ float bin_real(float a, float b) {
-  switch (OP) {
-    case ENDIA_BIN_ADD: return a + b;
-    case ENDIA_BIN_SUB: return a - b;
-    case ENDIA_BIN_MUL: return a * b;
-    case ENDIA_BIN_DIV: return a / b;
-    default: return a > b ? 1.f : 0.f;
-  }
-}
-
-template <int OP>
-__device__ __forceinline__ float2 bin_complex(float2 a, float2 b) {
-  switch (OP) {
-    case ENDIA_BIN_ADD: return make_float2(a.x + b.x, a.y + b.y);
-    case ENDIA_BIN_SUB: return make_float2(a.x - b.x, a.y - b.y);
-    case ENDIA_BIN_MUL: return make_float2(a.x * b.x - a.y * b.y, a.x * b.y + a.y * b.x);  // mul_op.mojo:152-155
-    default: {  // div_op.mojo:117-142
-      float d = b.x * b.x + b.y * b.y;
-      return make_float2((a.x * b.x + a.y * b.y) / d, (a.y * b.x - a.x * b.y) / d);
-    }
-  }
-}
-
 // Same-shape contiguous operands.
 template <int OP>
 __global__ __launch_bounds__(TPB) void bin_flat_kernel(const float* __restrict__ a, const float* __restrict__ b,
@@ -217,9 +156,9 @@ __global__ __launch_bounds__(TPB) void bin_flat_kernel(const float* __restrict__
   float4* o4 = reinterpret_cast<float4*>(o);
   for (int64_t j = i; j < n4; j += stride) {
     float4 x = a4[j], y = b4[j];
-    o4[j] = make_float4(bin_real<OP>(x.x, y.x), bin_real<OP>(x.y, y.y), bin_real<OP>(x.z, y.z), bin_real<OP>(x.w, y.w));
+    o4[j] = make_float4(bin_real(OP, x.x, y.x), bin_real(OP, x.y, y.y), bin_real(OP, x.z, y.z), bin_real(OP, x.w, y.w));
   }
-  for (int64_t j = (n4 << 2) + i; j < n; j += stride) o[j] = bin_real<OP>(a[j], b[j]);
+  for (int64_t j = (n4 << 2) + i; j < n; j += stride) o[j] = bin_real(OP, a[j], b[j]);
 }
 
 // [rows, cols] op with one operand a row vector [cols] (bias add and friends) or a scalar.
@@ -234,7 +173,7 @@ __global__ __launch_bounds__(TPB) void bin_rowvec_kernel(const float* __restrict
     int64_t c = j % cols;
     float x = a[amode == 0 ? j : (amode == 1 ? c : 0)];
     float y = b[bmode == 0 ? j : (bmode == 1 ? c : 0)];
-    o[j] = bin_real<OP>(x, y);
+    o[j] = bin_real(OP, x, y);
   }
 }
 
@@ -256,9 +195,9 @@ __global__ __launch_bounds__(TPB) void bin_general_kernel(BinDesc d, const float
     if (CPLX) {
       float2 x = reinterpret_cast<const float2*>(a)[ia];
       float2 y = reinterpret_cast<const float2*>(b)[ib];
-      reinterpret_cast<float2*>(o)[j] = bin_complex<OP>(x, y);
+      reinterpret_cast<float2*>(o)[j] = bin_complex(OP, x, y);
     } else {
-      o[j] = bin_real<OP>(a[ia], b[ib]);
+      o[j] = bin_real(OP, a[ia], b[ib]);
     }
   }
 }
@@ -336,35 +275,19 @@ __global__ __launch_bounds__(256) void transpose_kernel(const float* __restrict_
   }
 }
 
+template <int... I, typename F>
+bool dispatch_seq(int op, std::integer_sequence<int, I...>, F&& f) {
+  return ((op == I ? (f(std::integral_constant<int, I>()), true) : false) || ...);
+}
+
 template <typename F>
 int32_t dispatch_unary(int op, F&& f) {
-  switch (op) {
-    case ENDIA_OP_RELU: f(std::integral_constant<int, ENDIA_OP_RELU>()); break;
-    case ENDIA_OP_TANH: f(std::integral_constant<int, ENDIA_OP_TANH>()); break;
-    case ENDIA_OP_SIN: f(std::integral_constant<int, ENDIA_OP_SIN>()); break;
-    case ENDIA_OP_COS: f(std::integral_constant<int, ENDIA_OP_COS>()); break;
-    case ENDIA_OP_NEG: f(std::integral_constant<int, ENDIA_OP_NEG>()); break;
-    case ENDIA_OP_SQUARE: f(std::integral_constant<int, ENDIA_OP_SQUARE>()); break;
-    case ENDIA_OP_SQRT: f(std::integral_constant<int, ENDIA_OP_SQRT>()); break;
-    case ENDIA_OP_ABS: f(std::integral_constant<int, ENDIA_OP_ABS>()); break;
-    case ENDIA_OP_IDENTITY: f(std::integral_constant<int, ENDIA_OP_IDENTITY>()); break;
-    case ENDIA_OP_GREATER0: f(std::integral_constant<int, ENDIA_OP_GREATER0>()); break;
-    default: return -1;
-  }
-  return 0;
+  return dispatch_seq(op, std::make_integer_sequence<int, ENDIA_OP_COUNT>(), f) ? 0 : -1;
 }
 
 template <typename F>
 int32_t dispatch_binary(int op, F&& f) {
-  switch (op) {
-    case ENDIA_BIN_ADD: f(std::integral_constant<int, ENDIA_BIN_ADD>()); break;
-    case ENDIA_BIN_SUB: f(std::integral_constant<int, ENDIA_BIN_SUB>()); break;
-    case ENDIA_BIN_MUL: f(std::integral_constant<int, ENDIA_BIN_MUL>()); break;
-    case ENDIA_BIN_DIV: f(std::integral_constant<int, ENDIA_BIN_DIV>()); break;
-    case ENDIA_BIN_GREATER: f(std::integral_constant<int, ENDIA_BIN_GREATER>()); break;
-    default: return -1;
-  }
-  return 0;
+  return dispatch_seq(op, std::make_integer_sequence<int, ENDIA_BIN_COUNT>(), f) ? 0 : -1;
 }
 
 }  // namespace
@@ -400,8 +323,9 @@ int32_t endia_hip_unary_fwd(int32_t op, int64_t n, const float* x, float* y, int
   ENDIA_CHECK_ARG(x && y, "endia_hip_unary_fwd: null pointer");
   hipStream_t s = ctx().stream;
   if (is_complex) {
-    if (!(op == ENDIA_OP_NEG || op == ENDIA_OP_SQUARE || op == ENDIA_OP_ABS || op == ENDIA_OP_IDENTITY))
-      return fail(ENDIA_HIP_ERR_UNSUPPORTED, "endia_hip_unary_fwd: op %d has no complex form here", op);
+    ENDIA_CHECK_ARG(op >= 0 && op < ENDIA_OP_COUNT, "endia_hip_unary_fwd: unknown op %d", op);
+    if (!endia::unary_has_complex_form(op))
+      return fail(ENDIA_HIP_ERR_UNSUPPORTED, "endia_hip_unary_fwd: op %d has no complex form", op);
     hipLaunchKernelGGL(unary_fwd_complex_kernel, dim3(stream_grid(n)), dim3(TPB), 0, s, op,
                        reinterpret_cast<const float2*>(x), y, n);
   } else {
@@ -446,7 +370,7 @@ int32_t endia_hip_unary_vjp(int32_t op, int64_t n, const float* x, const float* 
 int32_t endia_hip_unary_vjp_from_output(int32_t op, int64_t n, const float* y, const float* g, float* dx) {
   ENDIA_REQUIRE_INIT();
   ENDIA_CHECK_ARG(n >= 0, "endia_hip_unary_vjp_from_output: negative n");
-  ENDIA_CHECK_ARG(op == ENDIA_OP_RELU || op == ENDIA_OP_TANH || op == ENDIA_OP_SQRT || op == ENDIA_OP_IDENTITY,
+  ENDIA_CHECK_ARG(endia::unary_has_output_rule(op),
                   "endia_hip_unary_vjp_from_output: op %d cannot be differentiated from its output", op);
   if (n == 0) return ENDIA_HIP_OK;
   ENDIA_CHECK_ARG(y && g && dx, "endia_hip_unary_vjp_from_output: null pointer");
@@ -460,8 +384,8 @@ int32_t endia_hip_binary(int32_t op, int32_t ndim, const int64_t* shape, const i
   ENDIA_REQUIRE_INIT();
   ENDIA_CHECK_ARG(ndim >= 0 && ndim <= 8, "endia_hip_binary: ndim %d out of [0,8]", ndim);
   ENDIA_CHECK_ARG(ndim == 0 || (shape && a_strides && b_strides), "endia_hip_binary: null descriptor");
-  ENDIA_CHECK_ARG(op >= ENDIA_BIN_ADD && op <= ENDIA_BIN_GREATER, "endia_hip_binary: unknown op %d", op);
-  ENDIA_CHECK_ARG(!(is_complex && op == ENDIA_BIN_GREATER), "endia_hip_binary: greater is not defined for complex");
+  ENDIA_CHECK_ARG(op >= 0 && op < ENDIA_BIN_COUNT, "endia_hip_binary: unknown op %d", op);
+  ENDIA_CHECK_ARG(!(is_complex && !endia::binary_has_complex_form(op)), "endia_hip_binary: comparisons are real only (op %d)", op);
   int64_t n = 1;
   for (int i = 0; i < ndim; ++i) {
     ENDIA_CHECK_ARG(shape[i] >= 0 && a_strides[i] >= 0 && b_strides[i] >= 0, "endia_hip_binary: negative extent or stride");
@@ -510,7 +434,7 @@ int32_t endia_hip_binary(int32_t op, int32_t ndim, const int64_t* shape, const i
     rc = dispatch_binary(op, [&](auto tag) {
       constexpr int OP = decltype(tag)::value;
       if (is_complex) {
-        if constexpr (OP != ENDIA_BIN_GREATER)
+        if constexpr (endia::binary_has_complex_form(OP))
           hipLaunchKernelGGL((bin_general_kernel<OP, true>), dim3(stream_grid(n)), dim3(TPB), 0, s, d, a, b, out, n);
       } else {
         hipLaunchKernelGGL((bin_general_kernel<OP, false>), dim3(stream_grid(n)), dim3(TPB), 0, s, d, a, b, out, n);

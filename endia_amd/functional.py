@@ -40,7 +40,12 @@ def contiguous(x):
     return x if x.is_contiguous() else _contiguous_copy(x)
 
 
+_fusion = None  # set by endia_amd.fusion: while it traces a function, ops on its symbols build an expression
+
+
 def detach(x):
+    if _fusion is not None and _fusion.tracing(x):
+        return x
     return Array(x._shape, is_complex=x.is_complex_, _buffer=x._buf, _strides=x._strides, _offset=x._offset)
 
 
@@ -271,6 +276,8 @@ def _broadcast_shape(a, b):
 
 
 def _binary(op, name, a, b, vjp):
+    if _fusion is not None and _fusion.tracing(a, b):
+        return _fusion.sym_binary(op, name, a, b, vjp)
     if a.is_complex_ != b.is_complex_:
         a = a if a.is_complex_ else complex(a)
         b = b if b.is_complex_ else complex(b)
@@ -314,10 +321,52 @@ def div(a, b):
     return _binary(L.BIN_DIV, "div", a, b, vjp)
 
 
+def pow(a, b):
+    """Elementwise a ** b as exp(log|a| * b) * cos(arg(a) * b) (pow_op.mojo:139-146); broadcasting."""
+    def vjp(primals, grad, out):  # pow_op.mojo:109-115
+        lhs = mul(mul(grad, primals[1]), div(out, primals[0])) if primals[0]._requires_grad else None
+        rhs = mul(mul(grad, out), log(primals[0])) if primals[1]._requires_grad else None
+        return [lhs, rhs]
+    return _binary(L.BIN_POW, "pow", a, b, vjp)
+
+
+pow_to = pow
+
+
+def _comparison(op, name, a, b):
+    if a.is_complex_ or b.is_complex_:
+        raise ValueError("%s is implemented for real arrays only" % name)
+    return _binary(op, name, detach(a), detach(b), None)
+
+
 def greater(a, b):
     """1.0 where a > b, else 0.0; not differentiable (greater_op.mojo:46-60)."""
-    out = _binary(L.BIN_GREATER, "greater", detach(a), detach(b), None)
-    return out
+    return _comparison(L.BIN_GREATER, "greater", a, b)
+
+
+def greater_equal(a, b):
+    """1.0 where a >= b (comparison_ops/greater_equal_op.mojo)."""
+    return _comparison(L.BIN_GREATER_EQUAL, "greater_equal", a, b)
+
+
+def less(a, b):
+    """1.0 where a < b (comparison_ops/less_op.mojo)."""
+    return _comparison(L.BIN_LESS, "less", a, b)
+
+
+def less_equal(a, b):
+    """1.0 where a <= b (comparison_ops/less_equal_op.mojo)."""
+    return _comparison(L.BIN_LESS_EQUAL, "less_equal", a, b)
+
+
+def equal(a, b):
+    """1.0 where a == b (comparison_ops/equal_op.mojo)."""
+    return _comparison(L.BIN_EQUAL, "equal", a, b)
+
+
+def not_equal(a, b):
+    """1.0 where a != b (comparison_ops/not_equal_op.mojo)."""
+    return _comparison(L.BIN_NOT_EQUAL, "not_equal", a, b)
 
 
 def pow_int(x, p):
@@ -339,6 +388,8 @@ def pow_int(x, p):
 # unary elementwise ops (endia/functional/unary_ops)
 # --------------------------------------------------------------------------------------------------
 def _unary(op, name, x, vjp):
+    if _fusion is not None and _fusion.tracing(x):
+        return _fusion.sym_unary(op, name, x, vjp)
     src = contiguous(x)
     out = Array.empty(x._shape, is_complex=x.is_complex_)
     if out.size():
@@ -392,10 +443,86 @@ def sqrt(x):
 
 
 def sign(x):
-    """z / |z| (sign_op.mojo:78-81); used by the VJP of abs."""
+    """z / |z| (sign_op.mojo:78-81); used by the VJP of abs. Its own VJP hands the gradient on (sign_op.mojo:58)."""
+    def vjp(primals, grad, out):
+        return [grad]
+    return _unary(L.OP_SIGN, "sign", x, vjp)
+
+
+def exp(x):
+    def vjp(primals, grad, out):  # exp_op.mojo:92
+        return [mul(exp(primals[0]), grad)]
+    return _unary(L.OP_EXP, "exp", x, vjp)
+
+
+def log(x):
+    """log of the modulus for real x (log_op.mojo:111-113)."""
+    def vjp(primals, grad, out):  # log_op.mojo:91
+        return [div(grad, primals[0])]
+    return _unary(L.OP_LOG, "log", x, vjp)
+
+
+def _real_only(x, name):
     if x.is_complex_:
-        return div(x, complex(_abs_raw(x)))
-    return div(x, _abs_raw(x))
+        raise ValueError("%s is implemented for real arrays only" % name)
+
+
+def sigmoid(x):
+    _real_only(x, "sigmoid")
+
+    def vjp(primals, grad, out):  # out * (1 - out) * grad : sigmoid_op.mojo:98
+        return [mul(mul(out, 1 - out), grad)]
+    return _unary(L.OP_SIGMOID, "sigmoid", x, vjp)
+
+
+def sinh(x):
+    def vjp(primals, grad, out):  # sinh_op.mojo:88
+        return [mul(cosh(primals[0]), grad)]
+    return _unary(L.OP_SINH, "sinh", x, vjp)
+
+
+def cosh(x):
+    def vjp(primals, grad, out):  # cosh_op.mojo:89
+        return [mul(sinh(primals[0]), grad)]
+    return _unary(L.OP_COSH, "cosh", x, vjp)
+
+
+def tan(x):
+    _real_only(x, "tan")
+
+    def vjp(primals, grad, out):  # grad * (1 + square(out)) : tan_op.mojo:81
+        return [mul(grad, 1 + square(out))]
+    return _unary(L.OP_TAN, "tan", x, vjp)
+
+
+def asin(x):
+    _real_only(x, "asin")
+
+    def vjp(primals, grad, out):  # grad / sqrt(1 - x ** 2) : asin_op.mojo:83
+        return [div(grad, sqrt(1 - primals[0] ** 2))]
+    return _unary(L.OP_ASIN, "asin", x, vjp)
+
+
+def acos(x):
+    _real_only(x, "acos")
+
+    def vjp(primals, grad, out):  # -1 / sqrt(1 - x ** 2) * grad : acos_op.mojo:91
+        return [mul(-1 / sqrt(1 - primals[0] ** 2), grad)]
+    return _unary(L.OP_ACOS, "acos", x, vjp)
+
+
+def atan(x):
+    _real_only(x, "atan")
+
+    def vjp(primals, grad, out):  # grad / (1 + square(x)) : atan_op.mojo:85
+        return [div(grad, 1 + square(primals[0]))]
+    return _unary(L.OP_ATAN, "atan", x, vjp)
+
+
+def reciprocal(x):
+    def vjp(primals, grad, out):  # -grad / square(x) : reciprocal_op.mojo:95
+        return [div(neg(grad), square(primals[0]))]
+    return _unary(L.OP_RECIPROCAL, "reciprocal", x, vjp)
 
 
 def _abs_raw(x):
@@ -409,15 +536,15 @@ def _abs_raw(x):
 def abs(x):
     """to_abs: |x| as a real array (abs_op.mojo:114-115,157); VJP sign(x) * g (abs_op.mojo:93), where for a
     complex x the real cotangent first becomes complex(g, 0) (real_op.mojo:74-77)."""
-    out = _abs_raw(x)
-
     def vjp(primals, grad, out_):
         z = primals[0]
         if z.is_complex_:
             return [mul(sign(z), complex(grad))]
         return [mul(sign(z), grad)]
 
-    return _register(out, [x], "abs", vjp)
+    if _fusion is not None and _fusion.tracing(x):
+        return _fusion.sym_unary(L.OP_ABS, "abs", x, vjp)
+    return _register(_abs_raw(x), [x], "abs", vjp)
 
 
 # --------------------------------------------------------------------------------------------------

@@ -38,7 +38,8 @@ typedef enum {
 } endia_hip_status;
 
 /* Unary operators. Replaces the per-op forward bodies and VJP rules of
- * endia/functional/unary_ops/{relu,tanh,sin,cos,neg,square,sqrt,abs}_op.mojo. */
+ * endia/functional/unary_ops/<name>_op.mojo. Real arrays take the reference's complex body at
+ * imag = 0 (unary_ops/_utils.mojo:113-118), which is why LOG is log|x| and SQRT is 0 for x < 0. */
 typedef enum {
   ENDIA_OP_RELU = 0,   /* relu_op.mojo:115-117 ; vjp greater(x,0)*g  relu_op.mojo:95  */
   ENDIA_OP_TANH = 1,   /* tanh_op.mojo:112-115 ; vjp (1-tanh(x)^2)*g tanh_op.mojo:92  */
@@ -49,17 +50,37 @@ typedef enum {
   ENDIA_OP_SQRT = 6,   /* sqrt_op.mojo:111-114 (0 for x<0) ; vjp g/(2*sqrt(x)) sqrt_op.mojo:91 */
   ENDIA_OP_ABS = 7,    /* abs_op.mojo:114-115,157 ; vjp sign(x)*g    abs_op.mojo:93   */
   ENDIA_OP_IDENTITY = 8,
-  ENDIA_OP_GREATER0 = 9 /* 1.0 where x > 0 else 0.0: greater_op.mojo:46-60 against a zero operand */
+  ENDIA_OP_GREATER0 = 9, /* 1.0 where x > 0 else 0.0: greater_op.mojo:46-60 against a zero operand */
+  ENDIA_OP_EXP = 10,     /* exp_op.mojo:113-114 ; vjp exp(x)*g            exp_op.mojo:92     */
+  ENDIA_OP_LOG = 11,     /* log_op.mojo:111-114 (log|x|) ; vjp g/x        log_op.mojo:91     */
+  ENDIA_OP_SIGMOID = 12, /* sigmoid_op.mojo:118-121 ; vjp out*(1-out)*g   sigmoid_op.mojo:98 */
+  ENDIA_OP_SINH = 13,    /* sinh_op.mojo:108-109 ; vjp cosh(x)*g          sinh_op.mojo:88    */
+  ENDIA_OP_COSH = 14,    /* cosh_op.mojo:109-110 ; vjp sinh(x)*g          cosh_op.mojo:89    */
+  ENDIA_OP_TAN = 15,     /* tan_op.mojo (real) ; vjp g*(1+out^2)          tan_op.mojo:81     */
+  ENDIA_OP_ASIN = 16,    /* asin_op.mojo:103 ; vjp g/sqrt(1-x^2)          asin_op.mojo:83    */
+  ENDIA_OP_ACOS = 17,    /* acos_op.mojo:111 ; vjp -1/sqrt(1-x^2)*g       acos_op.mojo:91    */
+  ENDIA_OP_ATAN = 18,    /* atan_op.mojo:105 ; vjp g/(1+x^2)              atan_op.mojo:85    */
+  ENDIA_OP_RECIPROCAL = 19, /* reciprocal_op.mojo:115-117 (x/x^2) ; vjp -g/x^2  reciprocal_op.mojo:95 */
+  ENDIA_OP_SIGN = 20     /* sign_op.mojo:78-81 (x/|x|, NaN at 0) ; vjp passes g on (sign_op.mojo:58) */
 } endia_hip_unary_op;
+#define ENDIA_OP_COUNT 21
 
-/* Binary operators: endia/functional/binary_ops/{add,sub,mul,div}_op.mojo. */
+/* Binary operators: endia/functional/binary_ops/{add,sub,mul,div,pow}_op.mojo and the comparisons of
+ * endia/functional/comparison_ops (1.0 / 0.0 results, real only, not differentiable). */
 typedef enum {
   ENDIA_BIN_ADD = 0,
   ENDIA_BIN_SUB = 1,
   ENDIA_BIN_MUL = 2,
   ENDIA_BIN_DIV = 3,
-  ENDIA_BIN_GREATER = 4 /* 1.0 where a > b else 0.0 (real only): greater_op.mojo:46-60 */
+  ENDIA_BIN_GREATER = 4,       /* greater_op.mojo:46-60 */
+  ENDIA_BIN_POW = 5,           /* exp(log|a|*b) * cos(arg(a)*b), complex form likewise: pow_op.mojo:139-146 */
+  ENDIA_BIN_GREATER_EQUAL = 6, /* greater_equal_op.mojo */
+  ENDIA_BIN_LESS = 7,          /* less_op.mojo */
+  ENDIA_BIN_LESS_EQUAL = 8,    /* less_equal_op.mojo */
+  ENDIA_BIN_EQUAL = 9,         /* equal_op.mojo */
+  ENDIA_BIN_NOT_EQUAL = 10     /* not_equal_op.mojo */
 } endia_hip_binary_op;
+#define ENDIA_BIN_COUNT 11
 
 /* GEMM epilogues (what is applied to the accumulator tile before it is stored). */
 typedef enum {
@@ -154,17 +175,47 @@ ENDIA_API int32_t endia_hip_cgemm(int32_t transA, int32_t conjA, int32_t transB,
 
 /* ---- elementwise: execute_unary_op (unary_ops/_utils.mojo:77-134) and the VJP rules listed at
  *      endia_hip_unary_op. n counts elements (complex: complex elements). In-place (y == x) allowed.
- *      Complex forward is implemented for NEG, SQUARE, IDENTITY; ABS with is_complex writes n REAL
- *      values |z| (abs_op.mojo:114-115,157). */
+ *      Complex forward is implemented for NEG, SQUARE, IDENTITY, SIN, COS, TANH, EXP, LOG, SINH, COSH,
+ *      SQRT, RECIPROCAL and SIGN; ABS with is_complex writes n REAL values |z| (abs_op.mojo:114-115,157). */
 ENDIA_API int32_t endia_hip_unary_fwd(int32_t op, int64_t n, const float* x, float* y, int32_t is_complex);
-/* dx = g * op'(x). For ABS with is_complex: g is real (n floats), x and dx complex: dx = g*z/|z|. */
+/* dx = g * op'(x). Complex: NEG, SQUARE, IDENTITY, and ABS, for which g is real (n floats) and x and dx
+ * are complex: dx = g*z/|z|. */
 ENDIA_API int32_t endia_hip_unary_vjp(int32_t op, int64_t n, const float* x, const float* g, float* dx,
                             int32_t is_complex);
 
 /* dx = g * op'(x) computed from the stored OUTPUT y = op(x) instead of x: RELU (y > 0), TANH (1 - y^2),
- * SQRT (1 / (2y)), IDENTITY. Equal to endia_hip_unary_vjp where the reference recomputes the forward
+ * SQRT (1 / (2y)), EXP (y), SIGMOID (y(1-y)), TAN (1 + y^2), IDENTITY. Equal to endia_hip_unary_vjp where the reference recomputes the forward
  * (tanh_op.mojo:92) but without the second transcendental pass. Real only. */
 ENDIA_API int32_t endia_hip_unary_vjp_from_output(int32_t op, int64_t n, const float* y, const float* g, float* dx);
+
+/* ---- fused elementwise program: a run of elementwise ops in one pass over memory. Replaces the
+ *      reference's fused unary runs (simd_op_list + execute_fwds, endia/_array/_array.mojo:90-101,756-782)
+ *      and stands in for its JIT-compiled elementwise subgraphs (endia/compile/fx.mojo:105-159).
+ *      Every lane interprets `steps` on an accumulator `acc` (0 at the start) and 4 save slots:
+ *        LOAD     acc = operand            UNARY    acc = op(acc)           (endia_hip_unary_op)
+ *        BINARY   acc = op(acc, operand)   RBINARY  acc = op(operand, acc)  (endia_hip_binary_op)
+ *        SAVE     slot[src_index] = acc    STORE    outputs[src_index][i] = acc
+ *      An operand is input `src_index` (src_kind INPUT), slot `src_index` (SLOT) or `imm` (IMM).
+ *      Inputs are real fp32: FULL = [rows*cols] contiguous, ROW_VECTOR = [cols] broadcast over rows,
+ *      SCALAR = one element. Outputs are [rows*cols]; every output must be stored by some step. */
+typedef enum { ENDIA_EW_LOAD = 0, ENDIA_EW_UNARY = 1, ENDIA_EW_BINARY = 2, ENDIA_EW_RBINARY = 3, ENDIA_EW_SAVE = 4,
+               ENDIA_EW_STORE = 5 } endia_hip_ew_kind;
+typedef enum { ENDIA_EW_SRC_INPUT = 0, ENDIA_EW_SRC_SLOT = 1, ENDIA_EW_SRC_IMM = 2 } endia_hip_ew_src;
+typedef enum { ENDIA_EW_FULL = 0, ENDIA_EW_ROW_VECTOR = 1, ENDIA_EW_SCALAR = 2 } endia_hip_ew_mode;
+typedef struct endia_hip_ew_step {
+  int32_t kind;      /* endia_hip_ew_kind */
+  int32_t op;        /* unary or binary op code, for UNARY / BINARY / RBINARY */
+  int32_t src_kind;  /* endia_hip_ew_src, for LOAD / BINARY / RBINARY */
+  int32_t src_index; /* input, slot or output index */
+  float imm;
+} endia_hip_ew_step;
+#define ENDIA_EW_MAX_INPUTS 8
+#define ENDIA_EW_MAX_OUTPUTS 4
+#define ENDIA_EW_MAX_SLOTS 4
+#define ENDIA_EW_MAX_STEPS 48
+ENDIA_API int32_t endia_hip_ew_program(int64_t rows, int64_t cols, int32_t n_inputs, const float* const* inputs,
+                             const int32_t* input_modes, int32_t n_outputs, float* const* outputs,
+                             int32_t n_steps, const endia_hip_ew_step* steps);
 
 /* ---- broadcasting binary op: binary_op_array + execute_binary_op (binary_ops/_utils.mojo:57-177).
  *      out is contiguous row-major of `shape`; a and b are addressed through element strides

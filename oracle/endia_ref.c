@@ -29,8 +29,10 @@
 /* nelts = 2 * simdwidthof[float32] (endia/utils/aliases.mojo:20-21); 8-lane AVX2 host assumed */
 #define NELTS 16
 
-enum { OP_RELU, OP_TANH, OP_SIN, OP_COS, OP_NEG, OP_SQUARE, OP_SQRT, OP_ABS, OP_IDENTITY, OP_GREATER0 };
-enum { BIN_ADD, BIN_SUB, BIN_MUL, BIN_DIV, BIN_GREATER };
+enum { OP_RELU, OP_TANH, OP_SIN, OP_COS, OP_NEG, OP_SQUARE, OP_SQRT, OP_ABS, OP_IDENTITY, OP_GREATER0, OP_EXP, OP_LOG,
+       OP_SIGMOID, OP_SINH, OP_COSH, OP_TAN, OP_ASIN, OP_ACOS, OP_ATAN, OP_RECIPROCAL, OP_SIGN };
+enum { BIN_ADD, BIN_SUB, BIN_MUL, BIN_DIV, BIN_GREATER, BIN_POW, BIN_GREATER_EQUAL, BIN_LESS, BIN_LESS_EQUAL, BIN_EQUAL,
+       BIN_NOT_EQUAL };
 
 /* Every op output is a freshly allocated, zero-filled buffer: functional/_utils.mojo:319-324 */
 static float* fresh(int64_t n) { return (float*)calloc((size_t)(n > 0 ? n : 1), sizeof(float)); }
@@ -159,6 +161,17 @@ static float unary_real(int op, float x) {
     }
     case OP_ABS: return sqrtf(x * x + 0.f);                          /* abs_op.mojo:114-115 */
     case OP_GREATER0: return x > 0.f ? 1.f : 0.f;                    /* greater_op.mojo:46-60 */
+    case OP_EXP: return expf(x) * cosf(0.f);                         /* exp_op.mojo:113 */
+    case OP_LOG: return logf(sqrtf(x * x + 0.f));                    /* log_op.mojo:111-113 */
+    case OP_SIGMOID: return 1.f / (1.f + expf(-x));                  /* sigmoid_op.mojo:120 */
+    case OP_SINH: return sinhf(x) * cosf(0.f);                       /* sinh_op.mojo:108 */
+    case OP_COSH: return coshf(x) * cosf(0.f);                       /* cosh_op.mojo:109 */
+    case OP_TAN: return tanf(x);                                     /* tan_op.mojo (real body) */
+    case OP_ASIN: return asinf(x) * coshf(0.f);                      /* asin_op.mojo:103 */
+    case OP_ACOS: return acosf(x);                                   /* acos_op.mojo:111 */
+    case OP_ATAN: return atanf(x);                                   /* atan_op.mojo:105 */
+    case OP_RECIPROCAL: return x / (x * x + 0.f);                    /* reciprocal_op.mojo:115-116 */
+    case OP_SIGN: return x / sqrtf(x * x + 0.f);                     /* sign_op.mojo:78-79 */
     default: return x;
   }
 }
@@ -175,6 +188,20 @@ static void binary_flat(int op, int64_t n, const float* a, const float* b, float
     case BIN_SUB: for (int64_t i = 0; i < n; ++i) o[i] = a[i] - b[i]; break;
     case BIN_MUL: for (int64_t i = 0; i < n; ++i) o[i] = a[i] * b[i]; break;
     case BIN_DIV: for (int64_t i = 0; i < n; ++i) o[i] = a[i] / b[i]; break;
+    case BIN_POW: /* pow_op.mojo:139-146 with zero imaginary parts */
+      for (int64_t i = 0; i < n; ++i) {
+        float log_mag = logf(sqrtf(a[i] * a[i] + 0.f));
+        float arg = atan2f(0.f, a[i]);
+        float u = expf(log_mag * b[i] - arg * 0.f);
+        float v = log_mag * 0.f + arg * b[i];
+        o[i] = u * cosf(v);
+      }
+      break;
+    case BIN_GREATER_EQUAL: for (int64_t i = 0; i < n; ++i) o[i] = a[i] >= b[i] ? 1.f : 0.f; break;
+    case BIN_LESS: for (int64_t i = 0; i < n; ++i) o[i] = a[i] < b[i] ? 1.f : 0.f; break;
+    case BIN_LESS_EQUAL: for (int64_t i = 0; i < n; ++i) o[i] = a[i] <= b[i] ? 1.f : 0.f; break;
+    case BIN_EQUAL: for (int64_t i = 0; i < n; ++i) o[i] = a[i] == b[i] ? 1.f : 0.f; break;
+    case BIN_NOT_EQUAL: for (int64_t i = 0; i < n; ++i) o[i] = a[i] != b[i] ? 1.f : 0.f; break;
     default: for (int64_t i = 0; i < n; ++i) o[i] = a[i] > b[i] ? 1.f : 0.f; break;
   }
 }
@@ -186,6 +213,15 @@ static void binary_flat_complex(int op, int64_t n, const float* a, const float* 
       case BIN_ADD: o[2 * i] = ar + br; o[2 * i + 1] = ai + bi; break;      /* add_op.mojo:134 */
       case BIN_SUB: o[2 * i] = ar - br; o[2 * i + 1] = ai - bi; break;      /* sub_op.mojo:136 */
       case BIN_MUL: o[2 * i] = ar * br - ai * bi; o[2 * i + 1] = ar * bi + ai * br; break; /* mul_op.mojo:152-155 */
+      case BIN_POW: {                                                       /* pow_op.mojo:139-146 */
+        float log_mag = logf(sqrtf(ar * ar + ai * ai));
+        float arg = atan2f(ai, ar);
+        float u = expf(log_mag * br - arg * bi);
+        float v = log_mag * bi + arg * br;
+        o[2 * i] = u * cosf(v);
+        o[2 * i + 1] = u * sinf(v);
+        break;
+      }
       default: {                                                            /* div_op.mojo:117-142 */
         float d = br * br + bi * bi;
         o[2 * i] = (ar * br + ai * bi) / d;
@@ -252,11 +288,93 @@ void ref_unary_vjp(int32_t op, int64_t n, const float* x, const float* g, float*
       for (int64_t i = 0; i < n; ++i) t[i] = x[i] / sqrtf(x[i] * x[i] + 0.f);
       binary_flat(BIN_MUL, n, t, g, dx);
       break;
-    default:
+    case OP_EXP: /* exp(x) * g : exp_op.mojo:92 */
+      ref_unary(OP_EXP, n, x, t);
+      binary_flat(BIN_MUL, n, t, g, dx);
+      break;
+    case OP_LOG: /* g / x : log_op.mojo:91 */
+      binary_flat(BIN_DIV, n, g, x, dx);
+      break;
+    case OP_SIGMOID: /* out * (1 - out) * g : sigmoid_op.mojo:98 */
+      ref_unary(OP_SIGMOID, n, x, t);
+      for (int64_t i = 0; i < n; ++i) u[i] = 1.f - t[i];
+      binary_flat(BIN_MUL, n, t, u, u);
+      binary_flat(BIN_MUL, n, u, g, dx);
+      break;
+    case OP_SINH: /* cosh(x) * g : sinh_op.mojo:88 */
+      ref_unary(OP_COSH, n, x, t);
+      binary_flat(BIN_MUL, n, t, g, dx);
+      break;
+    case OP_COSH: /* sinh(x) * g : cosh_op.mojo:89 */
+      ref_unary(OP_SINH, n, x, t);
+      binary_flat(BIN_MUL, n, t, g, dx);
+      break;
+    case OP_TAN: /* g * (1 + square(out)) : tan_op.mojo:81 */
+      ref_unary(OP_TAN, n, x, t);
+      ref_unary(OP_SQUARE, n, t, u);
+      for (int64_t i = 0; i < n; ++i) t[i] = 1.f + u[i];
+      binary_flat(BIN_MUL, n, g, t, dx);
+      break;
+    case OP_ASIN: /* g / sqrt(1 - x ** 2) : asin_op.mojo:83 */
+    case OP_ACOS: /* -1 / sqrt(1 - x ** 2) * g : acos_op.mojo:91 */
+      for (int64_t i = 0; i < n; ++i) u[i] = 2.f;
+      binary_flat(BIN_POW, n, x, u, t);
+      for (int64_t i = 0; i < n; ++i) u[i] = 1.f - t[i];
+      ref_unary(OP_SQRT, n, u, t);
+      if (op == OP_ASIN) {
+        binary_flat(BIN_DIV, n, g, t, dx);
+      } else {
+        for (int64_t i = 0; i < n; ++i) u[i] = -1.f / t[i];
+        binary_flat(BIN_MUL, n, u, g, dx);
+      }
+      break;
+    case OP_ATAN: /* g / (1 + square(x)) : atan_op.mojo:85 */
+      ref_unary(OP_SQUARE, n, x, t);
+      for (int64_t i = 0; i < n; ++i) u[i] = 1.f + t[i];
+      binary_flat(BIN_DIV, n, g, u, dx);
+      break;
+    case OP_RECIPROCAL: /* -g / square(x) : reciprocal_op.mojo:95 */
+      ref_unary(OP_NEG, n, g, t);
+      ref_unary(OP_SQUARE, n, x, u);
+      binary_flat(BIN_DIV, n, t, u, dx);
+      break;
+    default: /* identity; sign hands the gradient on (default_vjp, sign_op.mojo:58, _array.mojo:43-47) */
       memcpy(dx, g, (size_t)n * sizeof(float));
   }
   free(t);
   free(u);
+}
+
+/* complex -> complex forward bodies, interleaved in and out */
+void ref_unary_complex(int32_t op, int64_t n, const float* z, float* y) {
+  for (int64_t i = 0; i < n; ++i) {
+    float a = z[2 * i], b = z[2 * i + 1], re = a, im = b;
+    switch (op) {
+      case OP_NEG: re = -a; im = -b; break;                                             /* neg_op.mojo:111-113 */
+      case OP_SQUARE: re = a * a - b * b; im = 2.f * a * b; break;                      /* square_op.mojo:117-119 */
+      case OP_SIN: re = sinf(a) * coshf(b); im = cosf(a) * sinhf(b); break;             /* sin_op.mojo:112-113 */
+      case OP_COS: re = cosf(a) * coshf(b); im = -sinf(a) * sinhf(b); break;            /* cos_op.mojo:113-114 */
+      case OP_TANH: {                                                                   /* tanh_op.mojo:112-115 */
+        float d = coshf(2.f * a) + cosf(2.f * b);
+        re = sinhf(2.f * a) / d; im = sinf(2.f * b) / d;
+        break;
+      }
+      case OP_EXP: re = expf(a) * cosf(b); im = expf(a) * sinf(b); break;               /* exp_op.mojo:113-114 */
+      case OP_LOG: re = logf(sqrtf(a * a + b * b)); im = atan2f(b, a); break;           /* log_op.mojo:111-114 */
+      case OP_SINH: re = sinhf(a) * cosf(b); im = coshf(a) * sinf(b); break;            /* sinh_op.mojo:108-109 */
+      case OP_COSH: re = coshf(a) * cosf(b); im = sinhf(a) * sinf(b); break;            /* cosh_op.mojo:109-110 */
+      case OP_SQRT: {                                                                   /* sqrt_op.mojo:111-113 */
+        float r = sqrtf(a * a + b * b);
+        re = sqrtf((r + a) / 2.f); im = copysignf(sqrtf((r - a) / 2.f), b);
+        break;
+      }
+      case OP_RECIPROCAL: { float d = a * a + b * b; re = a / d; im = -b / d; break; }  /* reciprocal_op.mojo:115-117 */
+      case OP_SIGN: { float r = sqrtf(a * a + b * b); re = a / r; im = b / r; break; }  /* sign_op.mojo:78-80 */
+      default: break;
+    }
+    y[2 * i] = re;
+    y[2 * i + 1] = im;
+  }
 }
 
 /* complex |z| forward (n real outputs) and its VJP sign(z)*complex(g,0): abs_op.mojo:93,114-115,157;

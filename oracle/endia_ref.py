@@ -14,8 +14,9 @@ import numpy as np
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libendia_ref.so")
 
-OP = dict(relu=0, tanh=1, sin=2, cos=3, neg=4, square=5, sqrt=6, abs=7, identity=8, greater0=9)
-BIN = dict(add=0, sub=1, mul=2, div=3, greater=4)
+OP = dict(relu=0, tanh=1, sin=2, cos=3, neg=4, square=5, sqrt=6, abs=7, identity=8, greater0=9, exp=10, log=11,
+          sigmoid=12, sinh=13, cosh=14, tan=15, asin=16, acos=17, atan=18, reciprocal=19, sign=20)
+BIN = dict(add=0, sub=1, mul=2, div=3, greater=4, pow=5, greater_equal=6, less=7, less_equal=8, equal=9, not_equal=10)
 
 
 def build():
@@ -98,6 +99,14 @@ def unary_vjp(op, x, g):
     return dx
 
 
+def unary_complex(op, z):
+    """complex -> complex forward body of a unary op."""
+    z = np.ascontiguousarray(z, dtype=np.complex64)
+    y = np.empty_like(z)
+    lib().ref_unary_complex(c_int32(OP[op]), c_int64(z.size), _ptr(z), _ptr(y))
+    return y
+
+
 def cabs(z):
     z = np.ascontiguousarray(z, dtype=np.complex64)
     y = np.empty(z.shape, dtype=np.float32)
@@ -114,7 +123,7 @@ def cabs_vjp(z, g):
 
 
 def binary(op, a, b):
-    """Broadcasting elementwise op (add, sub, mul, div, greater)."""
+    """Broadcasting elementwise op (add, sub, mul, div, pow and the comparisons)."""
     cplx = np.iscomplexobj(a) or np.iscomplexobj(b)
     dt = np.complex64 if cplx else np.float32
     a = np.ascontiguousarray(a, dtype=dt)

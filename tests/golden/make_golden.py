@@ -4,9 +4,11 @@ PyTorch float64 is the oracle of the reference's own tests (every test converts 
 tensors and compares: endia/utils/array_conversions.mojo:41-135, e.g.
 tests/test_endia/test_functional/test_binary_ops/test_matmul_op.mojo:18-59); the reference itself is
 Mojo and cannot run here, and it ships no fixture files. Inputs are seeded, shapes follow the
-reference's tests ((2,30,40) @ (40,50), ...). Run:  python tests/golden/make_golden.py
+reference's tests ((2,30,40) @ (40,50), ...). Run:  python tests/golden/make_golden.py [fixture names]
+(every fixture is always computed, so the random stream is the same; only the named ones are written).
 """
 import os
+import sys
 
 import numpy as np
 import torch
@@ -30,6 +32,8 @@ def t64(a, grad=False):
 
 
 def save(name, **arrays):
+    if len(sys.argv) > 1 and name not in sys.argv[1:]:
+        return
     # expected values are stored rounded to fp32 / complex64: 6e-8 relative, far below the 1e-4 gate
     arrays = {k: (v.astype(np.complex64) if np.iscomplexobj(v) else v.astype(np.float32)) if v.size > 1 else v
               for k, v in arrays.items()}
@@ -245,3 +249,45 @@ d = {"z": zb, "loss": np.array([loss.item()]), "out": h.detach().numpy()}
 for i in range(Lyr):
     d["W%d" % i], d["dW%d" % i] = Ws[i], tW[i].grad.numpy()
 save("complex_mlp", **d)
+
+# ---- the rest of the unary ops: forward and gradient of sum(op(x)) (test_exp_op.mojo, test_log_op.mojo, ...) ----
+x = f32(2, 30, 40)
+xp = np.abs(x) + 0.1                       # positive: log, reciprocal, sign
+xu = (np.tanh(x) * 0.95).astype(np.float32)  # inside (-1, 1): asin, acos
+d = {"x": x, "xp": xp, "xu": xu}
+for name, fn, src in [("exp", torch.exp, x), ("log", torch.log, xp), ("sigmoid", torch.sigmoid, x),
+                      ("sinh", torch.sinh, x), ("cosh", torch.cosh, x), ("tan", torch.tan, xu),
+                      ("asin", torch.asin, xu), ("acos", torch.acos, xu), ("atan", torch.atan, x),
+                      ("reciprocal", torch.reciprocal, xp)]:
+    t = t64(src, True)
+    y = fn(t)
+    y.sum().backward()
+    d[name] = y.detach().numpy()
+    d["d" + name] = t.grad.numpy()
+d["sign"] = np.sign(xp.astype(np.float64)) * 1.0
+# complex forward bodies (the reference's tests run most unary ops on complex inputs too)
+z = c64(2, 30, 40)
+d["z"] = z
+tz = t64(z)
+for name, fn in [("sin", torch.sin), ("cos", torch.cos), ("tanh", torch.tanh), ("exp", torch.exp), ("log", torch.log),
+                 ("sinh", torch.sinh), ("cosh", torch.cosh), ("sqrt", torch.sqrt), ("reciprocal", torch.reciprocal),
+                 ("sign", torch.sgn)]:
+    d["c" + name] = fn(tz).numpy()
+save("unary_more", **d)
+
+# ---- pow with broadcasting and its gradients (test_pow_op.mojo), comparisons (comparison_ops) -------------
+a, b = (np.abs(f32(2, 30, 40)) + 0.2).astype(np.float32), f32(30, 40)
+ta, tb = t64(a, True), t64(b, True)
+y = torch.pow(ta, tb)
+y.sum().backward()
+an = f32(2, 30, 40)                         # negative bases with integer exponents
+ei = rng.integers(0, 4, size=(30, 40)).astype(np.float32)
+yn = torch.pow(t64(an), t64(ei))
+ca, cb = f32(2, 30, 40).round(), f32(30, 40).round()   # many ties, so == and != see both outcomes
+d = {"a": a, "b": b, "pow": y.detach().numpy(), "dpow_a": ta.grad.numpy(), "dpow_b": tb.grad.numpy(),
+     "an": an, "ei": ei, "pow_neg": yn.numpy(), "ca": ca, "cb": cb}
+tca, tcb = t64(ca), t64(cb)
+for name, fn in [("greater", torch.gt), ("greater_equal", torch.ge), ("less", torch.lt), ("less_equal", torch.le),
+                 ("equal", torch.eq), ("not_equal", torch.ne)]:
+    d[name] = fn(tca, tcb).numpy().astype(np.float32)
+save("binary_more", **d)

@@ -54,6 +54,123 @@ def test_unary_grad(nd, golden, op):  # test_relu_op.mojo:32-49 and siblings
     assert_close(x.grad().to_numpy(), g["d" + op], what="grad " + op)
 
 
+MORE_UNARY = ["exp", "log", "sigmoid", "sinh", "cosh", "tan", "asin", "acos", "atan", "reciprocal"]
+
+
+def _more_src(g, op):
+    return g["xp"] if op in ("log", "reciprocal") else (g["xu"] if op in ("tan", "asin", "acos") else g["x"])
+
+
+@pytest.mark.parametrize("op", MORE_UNARY)
+def test_unary_more_grad(nd, golden, op):  # test_exp_op.mojo, test_log_op.mojo, ... : forward and grad of sum(op(x))
+    g = golden("unary_more")
+    x = nd.array(_more_src(g, op), requires_grad=True)
+    y = getattr(nd, op)(x)
+    assert_close(y.to_numpy(), g[op], what=op)
+    nd.sum(y).backward()
+    assert_close(x.grad().to_numpy(), g["d" + op], what="grad " + op)
+
+
+def test_pow_grad_and_comparisons(nd, golden):  # test_pow_op.mojo
+    g = golden("binary_more")
+    a, b = nd.array(g["a"], requires_grad=True), nd.array(g["b"], requires_grad=True)
+    y = nd.pow(a, b)
+    assert_close(y.to_numpy(), g["pow"], what="pow")
+    nd.sum(y).backward()
+    assert_close(a.grad().to_numpy(), g["dpow_a"], what="dpow/da")
+    assert_close(b.grad().to_numpy(), g["dpow_b"], what="dpow/db")
+    ca, cb = nd.array(g["ca"]), nd.array(g["cb"])
+    for name in ("greater", "greater_equal", "less", "less_equal", "equal", "not_equal"):
+        np.testing.assert_array_equal(getattr(nd, name)(ca, cb).to_numpy(), g[name], err_msg=name)
+    x = nd.array(np.array([1.5, -2.0, 3.0], np.float32), requires_grad=True)
+    np.testing.assert_allclose((x ** 3).to_numpy(), [3.375, -8.0, 27.0], rtol=1e-5)
+    np.testing.assert_allclose((2.0 ** x).to_numpy(), [2 ** 1.5, 0.25, 8.0], rtol=1e-5)
+
+
+def test_fused_expression_forward_and_gradients(nd, golden):
+    """A fused expression must equal the same ops run one by one, in value and in every gradient, with
+    full, row-vector and one-element inputs; and both must equal float64."""
+    g = golden("binary")
+    a_np, b_np = g["a"], g["b2"][0]          # [2,30,40], [40]
+    s_np = np.array([0.7], np.float32)
+
+    def expr(a, b, s):
+        return nd.sigmoid(a * b + 1.0) * nd.tanh(a - s) / (nd.square(b) + 2.0)
+
+    fused = nd.fuse(expr)
+    outs = []
+    for f in (fused, expr):
+        a, b, s = (nd.array(v, requires_grad=True) for v in (a_np, b_np, s_np))
+        y = f(a, b, s)
+        nd.sum(nd.sin(y)).backward()
+        outs.append([y.to_numpy(), a.grad().to_numpy(), b.grad().to_numpy(), s.grad().to_numpy()])
+    for got, want, what in zip(outs[0], outs[1], ["value", "da", "db", "ds"]):
+        assert got.shape == want.shape, what
+        assert_close(got, want, tol=1e-5, what="fused vs op by op: " + what)
+    import torch
+    ta, tb, ts = (torch.tensor(v, dtype=torch.float64, requires_grad=True) for v in (a_np, b_np, s_np))
+    ty = torch.sigmoid(ta * tb + 1.0) * torch.tanh(ta - ts) / (tb * tb + 2.0)
+    torch.sin(ty).sum().backward()
+    for got, want, what in zip(outs[0], [ty.detach(), ta.grad, tb.grad, ts.grad], ["value", "da", "db", "ds"]):
+        assert_close(got, want.numpy(), what="fused vs float64: " + what)
+
+
+def test_fused_expression_one_launch_each_way(nd):
+    """The fused forward is one program and the fused backward one program (plus the reductions of
+    broadcast inputs): count library calls."""
+    from endia_amd import _lib as L
+    calls = []
+    orig = L.call
+
+    def spy(name, *args):
+        calls.append(name)
+        return orig(name, *args)
+
+    f = nd.fuse(lambda a, b: nd.relu(a * b) + nd.exp(-nd.abs(a)))
+    a = nd.array(np.linspace(-2, 2, 64, dtype=np.float32).reshape(4, 16), requires_grad=True)
+    b = nd.array(np.linspace(1, 3, 64, dtype=np.float32).reshape(4, 16), requires_grad=True)
+    f(a, b)  # traced and compiled
+    L.call = spy
+    try:
+        y = f(a, b)
+        fwd = [c for c in calls if c not in ("endia_hip_malloc", "endia_hip_free")]
+        assert fwd == ["endia_hip_ew_program"], fwd
+        del calls[:]
+        seed = nd.ones([4, 16])
+        y._vjp(y._args, seed, y)
+        bwd = [c for c in calls if c not in ("endia_hip_malloc", "endia_hip_free", "endia_hip_fill")]
+        assert bwd == ["endia_hip_ew_program"], bwd
+    finally:
+        L.call = orig
+    x64 = np.linspace(-2, 2, 64).reshape(4, 16)
+    w64 = np.linspace(1, 3, 64).reshape(4, 16)
+    assert_close(y.to_numpy(), np.maximum(x64 * w64, 0) + np.exp(-np.abs(x64)), what="fused value")
+
+
+def test_fused_expression_second_order(nd):
+    """Under create_graph the fused gradient is rebuilt from differentiable ops, so a Hessian-vector
+    product through a fused expression equals the one through the plain ops and float64."""
+    rng = np.random.default_rng(11)
+    x_np, v_np = rng.standard_normal((6, 8)).astype(np.float32), rng.standard_normal((6, 8)).astype(np.float32)
+
+    def expr(x):
+        return nd.sin(x) * nd.exp(x * 0.5)
+
+    res = []
+    for f in (nd.fuse(expr), expr):
+        x = nd.array(x_np, requires_grad=True)
+        nd.sum(f(x)).backward(create_graph=True)
+        gx = x.grad()
+        hv = nd.grad(outs=nd.sum(gx * nd.array(v_np)), inputs=x)[0]
+        res.append((gx.to_numpy(), hv.to_numpy()))
+    assert_close(res[0][0], res[1][0], tol=1e-5, what="gradient")
+    assert_close(res[0][1], res[1][1], tol=1e-5, what="hessian-vector product")
+    x64 = x_np.astype(np.float64)
+    e = np.exp(0.5 * x64)
+    assert_close(res[0][0], e * (np.cos(x64) + 0.5 * np.sin(x64)), what="gradient vs float64")
+    assert_close(res[0][1], v_np * e * (np.cos(x64) - 0.75 * np.sin(x64)), what="hvp vs float64")
+
+
 @pytest.mark.parametrize("op", ["add", "sub", "mul", "div"])
 def test_binary_grad(nd, golden, op):  # test_add_op.mojo:34-60, test_mul_op.mojo:34-59
     g = golden("binary")

@@ -35,6 +35,52 @@ def test_unary_fwd_and_vjp(dev, golden, op, n):
         assert_close(y[:2400], g[op].reshape(-1), what=op + " vs torch")
 
 
+MORE = {"exp": L.OP_EXP, "log": L.OP_LOG, "sigmoid": L.OP_SIGMOID, "sinh": L.OP_SINH, "cosh": L.OP_COSH, "tan": L.OP_TAN,
+        "asin": L.OP_ASIN, "acos": L.OP_ACOS, "atan": L.OP_ATAN, "reciprocal": L.OP_RECIPROCAL, "sign": L.OP_SIGN}
+
+
+def _more_src(g, op):
+    return g["xp"] if op in ("log", "reciprocal", "sign") else (g["xu"] if op in ("tan", "asin", "acos") else g["x"])
+
+
+@pytest.mark.parametrize("op", sorted(MORE))
+@pytest.mark.parametrize("n", [7, 30 * 40 * 2 + 3])
+def test_unary_more_fwd_and_vjp(dev, golden, op, n):
+    g = golden("unary_more")
+    x = np.resize(_more_src(g, op).reshape(-1), n).astype(np.float32)
+    gr = np.resize(g["x"].reshape(-1)[::-1], n).astype(np.float32)
+    dx_, dg = dev.put(x), dev.put(gr)
+    dy, dd = dev.alloc(4 * n), dev.alloc(4 * n)
+    dev.call("endia_hip_unary_fwd", MORE[op], n, dx_, dy, 0)
+    dev.call("endia_hip_unary_vjp", MORE[op], n, dx_, dg, dd, 0)
+    y, d = dev.get(dy, (n,)), dev.get(dd, (n,))
+    assert_close(y, R.unary(op, x), what=op)
+    assert_close(d, R.unary_vjp(op, x, gr), what="vjp " + op)
+    if n == 2403:
+        assert_close(y[:2400], g[op].reshape(-1), what=op + " vs torch")
+        if op != "sign":
+            assert_close(d[:2400], g["d" + op].reshape(-1) * gr[:2400], what="vjp " + op + " vs torch")
+    if op in ("exp", "sigmoid", "tan"):  # the same gradient from the stored output
+        dev.call("endia_hip_unary_vjp_from_output", MORE[op], n, dy, dg, dd)
+        assert_close(dev.get(dd, (n,)), R.unary_vjp(op, x, gr), what="vjp from output " + op)
+
+
+@pytest.mark.parametrize("op", ["sin", "cos", "tanh", "exp", "log", "sinh", "cosh", "sqrt", "reciprocal", "sign", "neg",
+                                "square"])
+def test_complex_unary_forward(dev, golden, op):
+    g = golden("unary_more")
+    z = g["z"].reshape(-1)
+    codes = dict(OPS, **MORE)
+    dz, dy = dev.put(z), dev.alloc(8 * z.size)
+    dev.call("endia_hip_unary_fwd", codes[op], z.size, dz, dy, 1)
+    y = dev.get(dy, z.shape, np.complex64)
+    assert_close(y, R.unary_complex(op, z), what="complex " + op)
+    if "c" + op in g.files:
+        assert_close(y, g["c" + op].reshape(-1), what="complex " + op + " vs torch")
+    with pytest.raises(L.EndiaHipError):
+        dev.call("endia_hip_unary_fwd", L.OP_RELU, z.size, dz, dy, 1)   # relu_op.mojo:51-52
+
+
 def test_unary_special_values(dev):
     x = np.array([0.0, -0.0, 1e-30, -1.0, 60.0, -60.0], np.float32)
     dx_, dg = dev.put(x), dev.put(np.ones(6, np.float32))
@@ -101,6 +147,111 @@ def test_binary_broadcast(dev, golden, name):
         a = rng.standard_normal(sa).astype(np.float32)
         bb = (np.abs(rng.standard_normal(sb)) + 0.5).astype(np.float32)
         assert_close(_binary(dev, code, a, bb), R.binary(name, a, bb), tol=1e-6, what="%s %s%s" % (name, sa, sb))
+
+
+def test_pow_and_comparisons(dev, golden):
+    g = golden("binary_more")
+    out = _binary(dev, L.BIN_POW, g["a"], g["b"])
+    assert_close(out, R.binary("pow", g["a"], g["b"]), tol=1e-5, what="pow")
+    assert_close(out, g["pow"], what="pow vs torch")
+    assert_close(_binary(dev, L.BIN_POW, g["an"], g["ei"]), g["pow_neg"], what="negative base, integer exponent")
+    for name, code in [("greater", L.BIN_GREATER), ("greater_equal", L.BIN_GREATER_EQUAL), ("less", L.BIN_LESS),
+                       ("less_equal", L.BIN_LESS_EQUAL), ("equal", L.BIN_EQUAL), ("not_equal", L.BIN_NOT_EQUAL)]:
+        np.testing.assert_array_equal(_binary(dev, code, g["ca"], g["cb"]), g[name], err_msg=name)
+    rng = np.random.default_rng(5)
+    za = (rng.standard_normal((6, 7)) + 1j * rng.standard_normal((6, 7))).astype(np.complex64)
+    zb = (rng.standard_normal((7,)) + 1j * rng.standard_normal((7,))).astype(np.complex64)
+    assert_close(_binary(dev, L.BIN_POW, za, zb), R.binary("pow", za, zb), tol=1e-5, what="complex pow")
+    assert_close(_binary(dev, L.BIN_POW, za, zb), za.astype(np.complex128) ** zb.astype(np.complex128), what="complex pow vs numpy")
+    with pytest.raises(L.EndiaHipError):
+        _binary(dev, L.BIN_LESS, za, zb)
+
+
+def _run_program(dev, rows, cols, inputs, modes, n_out, steps):
+    import ctypes
+    pin = (ctypes.c_void_p * max(len(inputs), 1))(*[dev.put(a) for a in inputs])
+    pmode = (ctypes.c_int32 * max(len(inputs), 1))(*modes)
+    outs = [dev.alloc(max(4 * rows * cols, 4)) for _ in range(n_out)]
+    pout = (ctypes.c_void_p * n_out)(*outs)
+    arr = (L.EwStep * len(steps))(*[L.EwStep(*s) for s in steps])
+    dev.call("endia_hip_ew_program", rows, cols, len(inputs), pin, pmode, n_out, pout, len(steps), arr)
+    return [dev.get(o, (rows, cols)) for o in outs]
+
+
+def _program_expected(rows, cols, inputs, modes, n_out, steps):
+    """The program's meaning, op by op, with the oracle's unary and binary bodies."""
+    names_u = {v: k for k, v in dict(OPS, **MORE).items()}
+    names_b = {L.BIN_ADD: "add", L.BIN_SUB: "sub", L.BIN_MUL: "mul", L.BIN_DIV: "div", L.BIN_GREATER: "greater",
+               L.BIN_POW: "pow", L.BIN_LESS: "less"}
+    full = [np.broadcast_to(a.reshape((1, -1)) if m else a.reshape(rows, cols), (rows, cols)).astype(np.float32)
+            for a, m in zip(inputs, modes)]
+    acc = np.zeros((rows, cols), np.float32)
+    slots = [np.zeros((rows, cols), np.float32) for _ in range(4)]
+    outs = [None] * n_out
+    for kind, op, sk, si, imm in steps:
+        x = full[si] if sk == L.EW_SRC_INPUT else (slots[si] if sk == L.EW_SRC_SLOT else np.full((rows, cols), imm, np.float32))
+        if kind == L.EW_LOAD:
+            acc = x.copy()
+        elif kind == L.EW_UNARY:
+            acc = R.unary(names_u[op], acc)
+        elif kind == L.EW_BINARY:
+            acc = R.binary(names_b[op], acc, x)
+        elif kind == L.EW_RBINARY:
+            acc = R.binary(names_b[op], x, acc)
+        elif kind == L.EW_SAVE:
+            slots[si] = acc.copy()
+        else:
+            outs[si] = acc.copy()
+    return outs
+
+
+@pytest.mark.parametrize("rows,cols", [(1, 1), (3, 5), (64, 48), (33, 1000), (2, 4099)])
+def test_ew_program(dev, rows, cols):
+    rng = np.random.default_rng(rows * 131 + cols)
+    a = rng.standard_normal((rows, cols)).astype(np.float32)
+    b = rng.standard_normal((rows, cols)).astype(np.float32)
+    bias = rng.standard_normal(cols).astype(np.float32)
+    scale = np.array([0.75], np.float32)
+    I, S, M = L.EW_SRC_INPUT, L.EW_SRC_SLOT, L.EW_SRC_IMM
+    steps = [
+        (L.EW_LOAD, 0, I, 0, 0.0),                  # a
+        (L.EW_BINARY, L.BIN_MUL, I, 1, 0.0),        # a*b
+        (L.EW_BINARY, L.BIN_ADD, I, 2, 0.0),        # + bias (row vector)
+        (L.EW_SAVE, 0, 0, 1, 0.0),                  # z -> slot 1
+        (L.EW_UNARY, L.OP_TANH, 0, 0, 0.0),         # tanh(z)
+        (L.EW_STORE, 0, 0, 0, 0.0),                 # out0 = tanh(z)
+        (L.EW_UNARY, L.OP_SQUARE, 0, 0, 0.0),
+        (L.EW_RBINARY, L.BIN_SUB, M, 0, 1.0),       # 1 - tanh^2
+        (L.EW_BINARY, L.BIN_MUL, I, 3, 0.0),        # * scale (one element)
+        (L.EW_SAVE, 0, 0, 3, 0.0),
+        (L.EW_LOAD, 0, S, 1, 0.0),                  # z again
+        (L.EW_UNARY, L.OP_SIGMOID, 0, 0, 0.0),
+        (L.EW_RBINARY, L.BIN_DIV, S, 3, 0.0),       # slot3 / sigmoid(z)
+        (L.EW_STORE, 0, 0, 1, 0.0),
+    ]
+    modes = [L.EW_FULL, L.EW_FULL, L.EW_ROW_VECTOR, L.EW_SCALAR]
+    got = _run_program(dev, rows, cols, [a, b, bias, scale], modes, 2, steps)
+    want = _program_expected(rows, cols, [a, b, bias, scale], modes, 2, steps)
+    for i in range(2):
+        assert_close(got[i], want[i], what="program output %d (%d x %d)" % (i, rows, cols))
+    z = a.astype(np.float64) * b + bias
+    assert_close(got[0], np.tanh(z), what="tanh(a*b+bias) vs float64")
+    assert_close(got[1], (1 - np.tanh(z) ** 2) * 0.75 * (1 + np.exp(-z)), what="second output vs float64")
+
+
+def test_ew_program_rejects_bad_programs(dev):
+    a = np.ones((2, 4), np.float32)
+    ok = [(L.EW_LOAD, 0, L.EW_SRC_INPUT, 0, 0.0), (L.EW_STORE, 0, 0, 0, 0.0)]
+    np.testing.assert_array_equal(_run_program(dev, 2, 4, [a], [L.EW_FULL], 1, ok)[0], a)
+    for bad in ([(L.EW_LOAD, 0, L.EW_SRC_INPUT, 1, 0.0), (L.EW_STORE, 0, 0, 0, 0.0)],     # input out of range
+                [(L.EW_LOAD, 0, L.EW_SRC_INPUT, 0, 0.0)],                                # nothing stored
+                [(L.EW_LOAD, 0, L.EW_SRC_INPUT, 0, 0.0), (L.EW_UNARY, 99, 0, 0, 0.0), (L.EW_STORE, 0, 0, 0, 0.0)],
+                [(L.EW_LOAD, 0, L.EW_SRC_SLOT, 7, 0.0), (L.EW_STORE, 0, 0, 0, 0.0)],
+                [(L.EW_LOAD, 0, L.EW_SRC_INPUT, 0, 0.0), (L.EW_STORE, 0, 0, 2, 0.0)]):
+        with pytest.raises(L.EndiaHipError):
+            _run_program(dev, 2, 4, [a], [L.EW_FULL], 1, bad)
+    # empty arrays are accepted and launch nothing
+    _run_program(dev, 0, 4, [np.zeros((0, 4), np.float32)], [L.EW_FULL], 1, ok)
 
 
 def test_binary_complex(dev, golden):

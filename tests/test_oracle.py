@@ -62,6 +62,54 @@ def test_unary_golden(golden, op):
     assert_close(R.unary_vjp(op, x, np.ones_like(x)), g["d" + op], what="d" + op)
 
 
+MORE_UNARY = ["exp", "log", "sigmoid", "sinh", "cosh", "tan", "asin", "acos", "atan", "reciprocal"]
+
+
+def _more_src(g, op):
+    return g["xp"] if op in ("log", "reciprocal", "sign") else (g["xu"] if op in ("tan", "asin", "acos") else g["x"])
+
+
+@pytest.mark.parametrize("op", MORE_UNARY)
+def test_unary_more_golden(golden, op):
+    g = golden("unary_more")
+    x = _more_src(g, op)
+    assert_close(R.unary(op, x), g[op], what=op)
+    assert_close(R.unary_vjp(op, x, np.ones_like(x)), g["d" + op], what="d" + op)
+
+
+def test_unary_more_special_values(golden):
+    g = golden("unary_more")
+    assert_close(R.unary("sign", g["xp"]), g["sign"], what="sign")
+    assert_close(R.unary("sign", -g["xp"]), -g["sign"], what="sign of negatives")
+    assert np.isnan(R.unary("sign", np.zeros(1, np.float32))[0])        # x / |x| at 0 (sign_op.mojo:78-79)
+    # log is the log of the modulus (log_op.mojo:111-113), so a negative input gives log|x|, not NaN
+    np.testing.assert_allclose(R.unary("log", np.array([-np.e], np.float32)), [1.0], rtol=1e-6)
+    # sign hands the gradient on unchanged (sign_op.mojo:58)
+    gr = np.arange(4, dtype=np.float32)
+    np.testing.assert_array_equal(R.unary_vjp("sign", np.ones(4, np.float32), gr), gr)
+
+
+@pytest.mark.parametrize("op", ["sin", "cos", "tanh", "exp", "log", "sinh", "cosh", "sqrt", "reciprocal", "sign"])
+def test_unary_complex_golden(golden, op):
+    g = golden("unary_more")
+    assert_close(R.unary_complex(op, g["z"]), g["c" + op], what="complex " + op)
+
+
+def test_pow_and_comparisons_golden(golden):
+    g = golden("binary_more")
+    y = R.binary("pow", g["a"], g["b"])
+    assert_close(y, g["pow"], what="pow")
+    # VJP as the reference composes it: g*b*(out/a), g*out*log(a), broadcast axis summed (pow_op.mojo:109-115)
+    gy = np.ones_like(y)
+    da = R.binary("mul", R.binary("mul", gy, g["b"]), R.binary("div", y, g["a"]))
+    db = R.reduce_add(R.binary("mul", R.binary("mul", gy, y), R.unary("log", g["a"])), [0])
+    assert_close(da, g["dpow_a"], what="dpow/da")
+    assert_close(db, g["dpow_b"], what="dpow/db")
+    assert_close(R.binary("pow", g["an"], g["ei"]), g["pow_neg"], what="negative base, integer exponent")
+    for name in ("greater", "greater_equal", "less", "less_equal", "equal", "not_equal"):
+        np.testing.assert_array_equal(R.binary(name, g["ca"], g["cb"]), g[name], err_msg=name)
+
+
 def test_unary_special_values():
     # strict > in the relu mask (greater_op.mojo:57-59); sqrt of a negative is 0, not NaN (sqrt_op.mojo:111-114)
     x = np.array([0.0, -0.0, 1e-30, -1.0], np.float32)
