@@ -184,6 +184,29 @@ def kernel_table(reps=10):
         ("tanh_fwd", lambda: L.call("endia_hip_unary_fwd", L.OP_TANH, nn, A, C, 0), 8.0 * nn, "hbm"),
         ("tanh_vjp", lambda: L.call("endia_hip_unary_vjp", L.OP_TANH, nn, A, B, C, 0), 12.0 * nn, "hbm"),
     ]
+    # fused elementwise programs: tanh(a * b + bias) in one pass (two full inputs, one output) and a
+    # two-output gradient program (three full inputs, two outputs)
+    I_, S_, M_ = L.EW_SRC_INPUT, L.EW_SRC_SLOT, L.EW_SRC_IMM
+    fwd_steps = [(L.EW_LOAD, 0, I_, 0, 0.0), (L.EW_BINARY, L.BIN_MUL, I_, 1, 0.0), (L.EW_BINARY, L.BIN_ADD, I_, 2, 0.0),
+                 (L.EW_UNARY, L.OP_TANH, 0, 0, 0.0), (L.EW_STORE, 0, 0, 0, 0.0)]
+    bwd_steps = [(L.EW_LOAD, 0, I_, 2, 0.0), (L.EW_UNARY, L.OP_SQUARE, 0, 0, 0.0), (L.EW_RBINARY, L.BIN_SUB, M_, 0, 1.0),
+                 (L.EW_BINARY, L.BIN_MUL, I_, 3, 0.0), (L.EW_SAVE, 0, 0, 0, 0.0), (L.EW_BINARY, L.BIN_MUL, I_, 1, 0.0),
+                 (L.EW_STORE, 0, 0, 0, 0.0), (L.EW_LOAD, 0, S_, 0, 0.0), (L.EW_BINARY, L.BIN_MUL, I_, 0, 0.0),
+                 (L.EW_STORE, 0, 0, 1, 0.0)]
+
+    def program(steps, ins, modes, outs):
+        arr = (L.EwStep * len(steps))(*[L.EwStep(*st) for st in steps])
+        pin = (ctypes.c_void_p * len(ins))(*ins)
+        pm = (ctypes.c_int32 * len(ins))(*modes)
+        po = (ctypes.c_void_p * len(outs))(*outs)
+        return lambda: L.call("endia_hip_ew_program", n, n, len(ins), pin, pm, len(outs), po, len(steps), arr)
+
+    F_, R_ = L.EW_FULL, L.EW_ROW_VECTOR
+    cases += [
+        ("ew_program  tanh(a*b + bias), 5 steps", program(fwd_steps, [A, B, bias], [F_, F_, R_], [C]), 12.0 * nn, "hbm"),
+        ("ew_program  gradients of it, 10 steps, 2 outputs", program(bwd_steps, [A, B, D, E], [F_, F_, F_, F_], [C, bufs[4]]),
+         20.0 * nn, "hbm"),
+    ]
     rows = []
     ms = ctypes.c_float()
     for _ in range(30):  # bring the clocks up before the first timed kernel

@@ -195,7 +195,8 @@ ENDIA_API int32_t endia_hip_unary_vjp_from_output(int32_t op, int64_t n, const f
  *        LOAD     acc = operand            UNARY    acc = op(acc)           (endia_hip_unary_op)
  *        BINARY   acc = op(acc, operand)   RBINARY  acc = op(operand, acc)  (endia_hip_binary_op)
  *        SAVE     slot[src_index] = acc    STORE    outputs[src_index][i] = acc
- *      An operand is input `src_index` (src_kind INPUT), slot `src_index` (SLOT) or `imm` (IMM).
+ *      An operand is input `src_index` (src_kind INPUT), slot `src_index` (SLOT; an earlier step must
+ *      have saved it) or `imm` (IMM).
  *      Inputs are real fp32: FULL = [rows*cols] contiguous, ROW_VECTOR = [cols] broadcast over rows,
  *      SCALAR = one element. Outputs are [rows*cols]; every output must be stored by some step. */
 typedef enum { ENDIA_EW_LOAD = 0, ENDIA_EW_UNARY = 1, ENDIA_EW_BINARY = 2, ENDIA_EW_RBINARY = 3, ENDIA_EW_SAVE = 4,
