@@ -44,6 +44,13 @@ class EwStep(ctypes.Structure):
     _fields_ = [("kind", c_int32), ("op", c_int32), ("src_kind", c_int32), ("src_index", c_int32), ("imm", c_float)]
 
 
+class PoolDesc(ctypes.Structure):
+    _fields_ = [(n, c_int64) for n in ("N", "C", "D", "H", "W")] + [
+        (n, c_int64 * 3) for n in ("kernel", "stride", "padding", "dilation")]
+
+
+POOL_MAX, POOL_AVG = 0, 1
+
 _fp = c_void_p  # device pointers travel as plain addresses
 _i64p = POINTER(c_int64)
 
@@ -90,6 +97,9 @@ SIGNATURES = {
     "endia_hip_conv2d_bwd_data": [POINTER(Conv2dDesc), _fp, _fp, _fp],
     "endia_hip_conv2d_bwd_weight": [POINTER(Conv2dDesc), _fp, _fp, _fp],
     "endia_hip_conv2d_bwd_bias": [POINTER(Conv2dDesc), _fp, _fp],
+    "endia_hip_pool_out_shape": [POINTER(PoolDesc), _i64p],
+    "endia_hip_pool_fwd": [POINTER(PoolDesc), c_int32, _fp, _fp, _fp],
+    "endia_hip_pool_bwd": [POINTER(PoolDesc), c_int32, _fp, _fp, _fp],
     "endia_hip_sgd_step": [c_int64, _fp, _fp, c_float],
     "endia_hip_sgd_momentum_step": [c_int64, _fp, _fp, _fp, c_float, c_float, c_float],
     "endia_hip_adagrad_step": [c_int64, _fp, _fp, _fp, c_float, c_float],

@@ -1,0 +1,226 @@
+// Max and average pooling over 1, 2 or 3 spatial axes of an [N, C, D, H, W] array (unused leading
+// spatial axes have extent 1), forward and backward.
+//
+// Forward follows MaxPool{1,2,3}d.__call__ and AvgPool{1,2,3}d.__call__
+// (endia/functional/spacial_ops/max_pool2d_op.mojo:88-150, avg_pool2d_op.mojo:84-140 and their 1-D / 3-D
+// siblings; output extent (in + 2*pad - dil*(k-1) - 1) / stride + 1, max_pool2d_op.mojo:57-82):
+//   window of output o = taps  o*stride - pad + k*dil,  taps outside the array are skipped;
+//   max:  the largest tap (-inf when the window is empty);
+//   avg:  sum of the taps / number of taps INSIDE the array (0 when the window is empty).
+// The reference registers no backward rule for pooling (vjp = default_vjp, max_pool2d_op.mojo:152-154);
+// the gradients here are the adjoints of those loops:
+//   max:  dx[i] = sum of dy[o] over the outputs o whose window maximum sits at i (the first tap in scan
+//         order that attains the maximum; its flat index within the (D,H,W) volume is written by the forward),
+//   avg:  dx[i] = sum over the outputs o whose window holds i of dy[o] / count[o].
+// Both directions are gathers (one lane per result element, no atomics), so results do not depend
+// on scheduling. The kernels are HBM-bound: algorithmic traffic is the input once and the output once.
+#include "common.h"
+#include "mfma_tile.h"
+
+namespace {
+
+using mfma::FastDiv;
+using mfma::fdiv;
+
+constexpr int TPB = 256;
+
+struct PoolP {
+  int D, H, W, Do, Ho, Wo;
+  int kd, kh, kw, sd, sh, sw, pd, ph, pw, dd, dh, dw;
+  FastDiv d_wo, d_ho, d_do;  // decode a flat output index
+  FastDiv d_w, d_h, d_d;     // decode a flat input index
+  FastDiv d_sd, d_sh, d_sw;  // divide by the strides (backward)
+  int64_t n_out, n_in;       // N*C*Do*Ho*Wo, N*C*D*H*W
+};
+
+inline int stream_grid(int64_t n) {
+  int64_t blocks = ceil_div64(n, TPB);
+  int64_t cap = (int64_t)endia::ctx().cu_count * 8;
+  if (cap < 256) cap = 2048;
+  return (int)(blocks > cap ? cap : (blocks < 1 ? 1 : blocks));
+}
+
+// flat index within [0, 2^32): split into (plane, z, y, x) with three magic-number divisions
+__device__ __forceinline__ void decode(uint32_t j, const FastDiv& dx, const FastDiv& dy, const FastDiv& dz, int X, int Y, int Z,
+                                       uint32_t& plane, int& z, int& y, int& x) {
+  uint32_t q = fdiv(j, dx);
+  x = (int)(j - q * (uint32_t)X);
+  uint32_t q2 = fdiv(q, dy);
+  y = (int)(q - q2 * (uint32_t)Y);
+  plane = fdiv(q2, dz);
+  z = (int)(q2 - plane * (uint32_t)Z);
+}
+
+template <bool MAX>
+__global__ __launch_bounds__(TPB) void pool_fwd_kernel(PoolP p, const float* __restrict__ x, float* __restrict__ y,
+                                                       int32_t* __restrict__ arg) {
+  const int64_t stride = (int64_t)gridDim.x * TPB;
+  const int64_t vol = (int64_t)p.D * p.H * p.W;
+  for (int64_t j = (int64_t)blockIdx.x * TPB + threadIdx.x; j < p.n_out; j += stride) {
+    uint32_t plane;
+    int oz, oy, ox;
+    decode((uint32_t)j, p.d_wo, p.d_ho, p.d_do, p.Wo, p.Ho, p.Do, plane, oz, oy, ox);
+    const float* src = x + plane * vol;
+    const int z0 = oz * p.sd - p.pd, y0 = oy * p.sh - p.ph, x0 = ox * p.sw - p.pw;
+    float best = -INFINITY, sum = 0.f;
+    int best_at = -1, count = 0;
+    for (int a = 0; a < p.kd; ++a) {
+      const int z = z0 + a * p.dd;
+      if ((unsigned)z >= (unsigned)p.D) continue;
+      for (int b = 0; b < p.kh; ++b) {
+        const int yy = y0 + b * p.dh;
+        if ((unsigned)yy >= (unsigned)p.H) continue;
+        const int row = (z * p.H + yy) * p.W;
+        for (int c = 0; c < p.kw; ++c) {
+          const int xx = x0 + c * p.dw;
+          if ((unsigned)xx >= (unsigned)p.W) continue;
+          const float v = src[row + xx];
+          if (MAX) {
+            if (best_at < 0 || v > best) { best = v; best_at = row + xx; }
+          } else {
+            sum += v;
+            ++count;
+          }
+        }
+      }
+    }
+    if (MAX) {
+      y[j] = best;
+      if (arg) arg[j] = best_at;
+    } else {
+      y[j] = count > 0 ? sum / (float)count : 0.f;
+    }
+  }
+}
+
+// number of taps of output coordinate o that fall inside [0, extent)
+__device__ __forceinline__ int taps_inside(int o, int k, int s, int pad, int dil, int extent) {
+  int n = 0;
+  for (int a = 0; a < k; ++a) n += (unsigned)(o * s - pad + a * dil) < (unsigned)extent;
+  return n;
+}
+
+template <bool MAX>
+__global__ __launch_bounds__(TPB) void pool_bwd_kernel(PoolP p, const float* __restrict__ dy, const int32_t* __restrict__ arg,
+                                                       float* __restrict__ dx) {
+  const int64_t stride = (int64_t)gridDim.x * TPB;
+  const int64_t ovol = (int64_t)p.Do * p.Ho * p.Wo;
+  for (int64_t j = (int64_t)blockIdx.x * TPB + threadIdx.x; j < p.n_in; j += stride) {
+    uint32_t plane;
+    int z, yy, xx;
+    decode((uint32_t)j, p.d_w, p.d_h, p.d_d, p.W, p.H, p.D, plane, z, yy, xx);
+    const float* g = dy + plane * ovol;
+    const int32_t* at = MAX ? arg + plane * ovol : nullptr;
+    const int self = (z * p.H + yy) * p.W + xx;
+    float acc = 0.f;
+    // outputs whose window holds this element: o*stride - pad + k*dil = coordinate, per axis
+    for (int a = 0; a < p.kd; ++a) {
+      const int tz = z + p.pd - a * p.dd;
+      if (tz < 0) continue;
+      const int oz = (int)fdiv((uint32_t)tz, p.d_sd);
+      if (oz * p.sd != tz || oz >= p.Do) continue;
+      const int cz = MAX ? 0 : taps_inside(oz, p.kd, p.sd, p.pd, p.dd, p.D);
+      for (int b = 0; b < p.kh; ++b) {
+        const int ty = yy + p.ph - b * p.dh;
+        if (ty < 0) continue;
+        const int oy = (int)fdiv((uint32_t)ty, p.d_sh);
+        if (oy * p.sh != ty || oy >= p.Ho) continue;
+        const int cy = MAX ? 0 : taps_inside(oy, p.kh, p.sh, p.ph, p.dh, p.H);
+        for (int c = 0; c < p.kw; ++c) {
+          const int tx = xx + p.pw - c * p.dw;
+          if (tx < 0) continue;
+          const int ox = (int)fdiv((uint32_t)tx, p.d_sw);
+          if (ox * p.sw != tx || ox >= p.Wo) continue;
+          const int o = (oz * p.Ho + oy) * p.Wo + ox;
+          if (MAX) {
+            if (at[o] == self) acc += g[o];
+          } else {
+            const int cx = taps_inside(ox, p.kw, p.sw, p.pw, p.dw, p.W);
+            acc += g[o] / (float)(cz * cy * cx);
+          }
+        }
+      }
+    }
+    dx[j] = acc;
+  }
+}
+
+int32_t make_params(const endia_hip_pool_desc* d, PoolP& p, const char* who) {
+  if (!d) return endia::fail(ENDIA_HIP_ERR_INVALID, "%s: null descriptor", who);
+  const int64_t in[3] = {d->D, d->H, d->W};
+  int64_t out[3];
+  if (d->N < 0 || d->C < 0) return endia::fail(ENDIA_HIP_ERR_INVALID, "%s: negative batch or channel count", who);
+  for (int i = 0; i < 3; ++i) {
+    if (in[i] < 1 || d->kernel[i] < 1 || d->stride[i] < 1 || d->padding[i] < 0 || d->dilation[i] < 1)
+      return endia::fail(ENDIA_HIP_ERR_INVALID, "%s: axis %d: extent %lld kernel %lld stride %lld padding %lld dilation %lld", who,
+                         i, (long long)in[i], (long long)d->kernel[i], (long long)d->stride[i], (long long)d->padding[i],
+                         (long long)d->dilation[i]);
+    const int64_t span = in[i] + 2 * d->padding[i] - d->dilation[i] * (d->kernel[i] - 1) - 1;
+    if (span < 0) return endia::fail(ENDIA_HIP_ERR_INVALID, "%s: axis %d: the window does not fit the padded input", who, i);
+    out[i] = span / d->stride[i] + 1;
+    if (in[i] >= (1ll << 30) || d->kernel[i] > 1024 || d->padding[i] > (1 << 20) || d->dilation[i] > (1 << 20) || d->stride[i] > (1 << 20))
+      return endia::fail(ENDIA_HIP_ERR_INVALID, "%s: axis %d: window parameters out of range", who, i);
+  }
+  p.n_in = d->N * d->C * in[0] * in[1] * in[2];
+  p.n_out = d->N * d->C * out[0] * out[1] * out[2];
+  if (p.n_in >= (1ll << 31) || p.n_out >= (1ll << 31))
+    return endia::fail(ENDIA_HIP_ERR_UNSUPPORTED, "%s: more than 2^31 elements", who);
+  p.D = (int)in[0]; p.H = (int)in[1]; p.W = (int)in[2];
+  p.Do = (int)out[0]; p.Ho = (int)out[1]; p.Wo = (int)out[2];
+  p.kd = (int)d->kernel[0]; p.kh = (int)d->kernel[1]; p.kw = (int)d->kernel[2];
+  p.sd = (int)d->stride[0]; p.sh = (int)d->stride[1]; p.sw = (int)d->stride[2];
+  p.pd = (int)d->padding[0]; p.ph = (int)d->padding[1]; p.pw = (int)d->padding[2];
+  p.dd = (int)d->dilation[0]; p.dh = (int)d->dilation[1]; p.dw = (int)d->dilation[2];
+  p.d_wo = make_fastdiv(p.Wo); p.d_ho = make_fastdiv(p.Ho); p.d_do = make_fastdiv(p.Do);
+  p.d_w = make_fastdiv(p.W); p.d_h = make_fastdiv(p.H); p.d_d = make_fastdiv(p.D);
+  p.d_sd = make_fastdiv(p.sd); p.d_sh = make_fastdiv(p.sh); p.d_sw = make_fastdiv(p.sw);
+  return ENDIA_HIP_OK;
+}
+
+}  // namespace
+
+using namespace endia;
+
+extern "C" {
+
+int32_t endia_hip_pool_out_shape(const endia_hip_pool_desc* desc, int64_t* out_dhw) {
+  PoolP p;
+  int32_t rc = make_params(desc, p, __func__);
+  if (rc) return rc;
+  ENDIA_CHECK_ARG(out_dhw, "endia_hip_pool_out_shape: null output");
+  out_dhw[0] = p.Do; out_dhw[1] = p.Ho; out_dhw[2] = p.Wo;
+  return ENDIA_HIP_OK;
+}
+
+int32_t endia_hip_pool_fwd(const endia_hip_pool_desc* desc, int32_t mode, const float* x, float* y, int32_t* argmax) {
+  ENDIA_REQUIRE_INIT();
+  PoolP p;
+  int32_t rc = make_params(desc, p, __func__);
+  if (rc) return rc;
+  ENDIA_CHECK_ARG(mode == ENDIA_POOL_MAX || mode == ENDIA_POOL_AVG, "endia_hip_pool_fwd: unknown mode %d", mode);
+  if (p.n_out == 0) return ENDIA_HIP_OK;
+  ENDIA_CHECK_ARG(x && y, "endia_hip_pool_fwd: null pointer");
+  const int grid = stream_grid(p.n_out);
+  if (mode == ENDIA_POOL_MAX) hipLaunchKernelGGL((pool_fwd_kernel<true>), dim3(grid), dim3(TPB), 0, ctx().stream, p, x, y, argmax);
+  else hipLaunchKernelGGL((pool_fwd_kernel<false>), dim3(grid), dim3(TPB), 0, ctx().stream, p, x, y, (int32_t*)nullptr);
+  ENDIA_LAUNCH_CHECK();
+  return ENDIA_HIP_OK;
+}
+
+int32_t endia_hip_pool_bwd(const endia_hip_pool_desc* desc, int32_t mode, const float* dy, const int32_t* argmax, float* dx) {
+  ENDIA_REQUIRE_INIT();
+  PoolP p;
+  int32_t rc = make_params(desc, p, __func__);
+  if (rc) return rc;
+  ENDIA_CHECK_ARG(mode == ENDIA_POOL_MAX || mode == ENDIA_POOL_AVG, "endia_hip_pool_bwd: unknown mode %d", mode);
+  if (p.n_in == 0) return ENDIA_HIP_OK;
+  ENDIA_CHECK_ARG(dy && dx, "endia_hip_pool_bwd: null pointer");
+  ENDIA_CHECK_ARG(mode != ENDIA_POOL_MAX || argmax, "endia_hip_pool_bwd: max pooling needs the argmax array of the forward");
+  const int grid = stream_grid(p.n_in);
+  if (mode == ENDIA_POOL_MAX) hipLaunchKernelGGL((pool_bwd_kernel<true>), dim3(grid), dim3(TPB), 0, ctx().stream, p, dy, argmax, dx);
+  else hipLaunchKernelGGL((pool_bwd_kernel<false>), dim3(grid), dim3(TPB), 0, ctx().stream, p, dy, argmax, dx);
+  ENDIA_LAUNCH_CHECK();
+  return ENDIA_HIP_OK;
+}
+
+}  // extern "C"

@@ -13,7 +13,7 @@ Every forward body is one or two calls into libendia_hip.so.
 import numpy as np
 
 from . import _lib as L
-from ._array import Array, _contiguous_copy, _prod, contiguous_strides
+from ._array import Array, Buffer, _contiguous_copy, _prod, contiguous_strides
 
 
 # --------------------------------------------------------------------------------------------------
@@ -793,6 +793,91 @@ def conv2d(x, kernel, bias=None, stride=1, padding=0, dilation=1, groups=1, _act
 
     args = [x, kernel] + ([bias] if bias is not None else [])
     return _register(out, args, "conv2d", vjp)
+
+
+def conv1d(x, kernel, bias=None, stride=1, padding=0, dilation=1, groups=1):
+    """[N, C, L] cross-correlation with kernel [K, C, S] (conv1d_op.mojo): the 2-D kernels on a height-1 image."""
+    if x.ndim() != 3:
+        raise ValueError("Input must be 3-dimensional (batch_size, in_channels, length) for 1D convolution!")
+    if x._shape[1] != kernel._shape[1]:
+        raise ValueError("Input channels must match kernel channels for 1D convolution!")
+    N, C, Ln = x._shape
+    K, _, S = kernel._shape
+    y = conv2d(reshape(x, [N, C, 1, Ln]), reshape(kernel, [K, C, 1, S]), bias, (1, int(stride)), (0, int(padding)),
+               (1, int(dilation)), groups)
+    return reshape(y, [N, K, y._shape[-1]])
+
+
+# --------------------------------------------------------------------------------------------------
+# pooling (endia/functional/spacial_ops/{max,avg}_pool{1,2,3}d_op.mojo)
+# --------------------------------------------------------------------------------------------------
+def _tuple_n(v, n):
+    return (int(v),) * n if np.isscalar(v) else tuple(int(e) for e in v)
+
+
+_POOL_RANK_ERR = {
+    1: "Input must be 3-dimensional (batch_size, channels, length) for 1D pooling!",
+    2: "Input must be 4-dimensional (batch_size, channels, height, width) for 2D pooling!",
+    3: "Input must be 5-dimensional (batch_size, channels, depth, height, width) for 3D pooling!",
+}
+
+
+def _pool(x, mode, nsp, kernel_size, stride, padding, dilation):
+    """Shared body of the six pooling ops. The reference has no backward rule for them (vjp = default_vjp,
+    max_pool2d_op.mojo:152-154); the VJP here is the adjoint of its forward loop."""
+    import ctypes
+    name = ("max" if mode == L.POOL_MAX else "avg") + "_pool%dd" % nsp
+    if x.ndim() != nsp + 2:
+        raise ValueError(_POOL_RANK_ERR[nsp])
+    if x.is_complex_:
+        raise ValueError("Complex numbers are not supported for %s!" % name)
+    desc = L.PoolDesc()
+    desc.N, desc.C = x._shape[0], x._shape[1]
+    desc.D, desc.H, desc.W = [1] * (3 - nsp) + list(x._shape[2:])
+    for field, v, fill in (("kernel", kernel_size, 1), ("stride", stride, 1), ("padding", padding, 0), ("dilation", dilation, 1)):
+        getattr(desc, field)[:] = [fill] * (3 - nsp) + list(_tuple_n(v, nsp))
+    o = (ctypes.c_int64 * 3)()
+    L.call("endia_hip_pool_out_shape", ctypes.byref(desc), o)
+    out_shape = list(x._shape[:2]) + list(o[3 - nsp:])
+    xs = contiguous(x)
+    out = Array.empty(out_shape)
+    arg = Buffer(4 * max(out.size(), 1)) if (mode == L.POOL_MAX and x._requires_grad) else None
+    L.call("endia_hip_pool_fwd", ctypes.byref(desc), mode, xs.data_ptr(), out.data_ptr(), arg.ptr if arg else None)
+
+    def vjp(primals, grad, out_):
+        from .autograd.functional import building_graph
+        if building_graph():
+            raise NotImplementedError("%s has no second-order rule" % name)
+        g = contiguous(grad)
+        dx = Array.empty(primals[0]._shape)
+        L.call("endia_hip_pool_bwd", ctypes.byref(desc), mode, g.data_ptr(), arg.ptr if arg else None, dx.data_ptr())
+        return [dx]
+
+    return _register(out, [x], name, vjp)
+
+
+def max_pool1d(x, kernel_size, stride=1, padding=0, dilation=1):
+    return _pool(x, L.POOL_MAX, 1, kernel_size, stride, padding, dilation)
+
+
+def max_pool2d(x, kernel_size, stride=(1, 1), padding=(0, 0), dilation=(1, 1)):
+    return _pool(x, L.POOL_MAX, 2, kernel_size, stride, padding, dilation)
+
+
+def max_pool3d(x, kernel_size, stride=(1, 1, 1), padding=(0, 0, 0), dilation=(1, 1, 1)):
+    return _pool(x, L.POOL_MAX, 3, kernel_size, stride, padding, dilation)
+
+
+def avg_pool1d(x, kernel_size, stride=1, padding=0, dilation=1):
+    return _pool(x, L.POOL_AVG, 1, kernel_size, stride, padding, dilation)
+
+
+def avg_pool2d(x, kernel_size, stride=(1, 1), padding=(0, 0), dilation=(1, 1)):
+    return _pool(x, L.POOL_AVG, 2, kernel_size, stride, padding, dilation)
+
+
+def avg_pool3d(x, kernel_size, stride=(1, 1, 1), padding=(0, 0, 0), dilation=(1, 1, 1)):
+    return _pool(x, L.POOL_AVG, 3, kernel_size, stride, padding, dilation)
 
 
 # --------------------------------------------------------------------------------------------------

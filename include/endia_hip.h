@@ -264,6 +264,27 @@ ENDIA_API int32_t endia_hip_conv2d_bwd_weight(const endia_hip_conv2d_desc* d, co
                                     float* dw);
 ENDIA_API int32_t endia_hip_conv2d_bwd_bias(const endia_hip_conv2d_desc* d, const float* dy, float* db);
 
+/* ---- pooling over 1, 2 or 3 spatial axes of a contiguous [N, C, D, H, W] array (set the unused leading
+ *      axes to extent 1 with kernel 1, stride 1, padding 0, dilation 1). Forward: MaxPool{1,2,3}d.__call__
+ *      (spacial_ops/max_pool2d_op.mojo:88-150 and siblings), AvgPool{1,2,3}d.__call__
+ *      (spacial_ops/avg_pool2d_op.mojo:84-140 and siblings); output extent per axis
+ *      (in + 2*pad - dil*(k-1) - 1) / stride + 1 (max_pool2d_op.mojo:57-82). Taps outside the array are
+ *      skipped: max over the taps inside (-inf if none), average = sum / number of taps inside (0 if none).
+ *      The reference has no backward rule for pooling (vjp = default_vjp, max_pool2d_op.mojo:152-154);
+ *      endia_hip_pool_bwd is the adjoint of the forward loop. For max pooling the forward writes, per
+ *      output, the flat (d*H + h)*W + w position of the first tap that attains the maximum into `argmax`
+ *      (may be null if no gradient is needed) and the backward reads it; average pooling ignores it. */
+typedef enum { ENDIA_POOL_MAX = 0, ENDIA_POOL_AVG = 1 } endia_hip_pool_mode;
+typedef struct endia_hip_pool_desc {
+  int64_t N, C, D, H, W;
+  int64_t kernel[3], stride[3], padding[3], dilation[3]; /* order: depth, height, width */
+} endia_hip_pool_desc;
+ENDIA_API int32_t endia_hip_pool_out_shape(const endia_hip_pool_desc* desc, int64_t* out_dhw);
+ENDIA_API int32_t endia_hip_pool_fwd(const endia_hip_pool_desc* desc, int32_t mode, const float* x, float* y,
+                           int32_t* argmax);
+ENDIA_API int32_t endia_hip_pool_bwd(const endia_hip_pool_desc* desc, int32_t mode, const float* dy,
+                           const int32_t* argmax, float* dx);
+
 /* ---- optimizers: SGD.step plain path (optim/sgd.mojo:61-62) and Adam.step (optim/adam.mojo:47-65),
  *      each as one pass over the parameter. t is Adam's fp32 step counter (starts at 1, adam.mojo:40). */
 ENDIA_API int32_t endia_hip_sgd_step(int64_t n, float* p, const float* g, float lr);

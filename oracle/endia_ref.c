@@ -520,6 +520,148 @@ void ref_conv2d_bwd(const conv_desc* d, const float* x, const float* w, const fl
         }
 }
 
+/* ---- pooling: MaxPool{1,2,3}d.__call__ / AvgPool{1,2,3}d.__call__ (spacial_ops/max_pool2d_op.mojo:88-150,
+ * avg_pool2d_op.mojo:84-140 and their 1-D / 3-D siblings) over [N, C, D, H, W]; the 1-D and 2-D ops are the
+ * cases D = 1 (and H = 1). mode 0 = max, 1 = average over the taps inside the array. ---------------- */
+typedef struct {
+  int64_t N, C, D, H, W;
+  int64_t kernel[3], stride[3], padding[3], dilation[3];
+} pool_desc;
+
+static void pool_out(const pool_desc* d, int64_t* o) {
+  const int64_t in[3] = {d->D, d->H, d->W};
+  for (int i = 0; i < 3; ++i) /* max_pool2d_op.mojo:57-82 */
+    o[i] = (in[i] + 2 * d->padding[i] - d->dilation[i] * (d->kernel[i] - 1) - 1) / d->stride[i] + 1;
+}
+
+void ref_pool_out_shape(const pool_desc* d, int64_t* o) { pool_out(d, o); }
+
+void ref_pool_fwd(const pool_desc* d, int32_t mode, const float* x, float* y) {
+  int64_t o[3];
+  pool_out(d, o);
+  for (int64_t nc = 0; nc < d->N * d->C; ++nc)
+    for (int64_t oz = 0; oz < o[0]; ++oz)
+      for (int64_t oy = 0; oy < o[1]; ++oy)
+        for (int64_t ox = 0; ox < o[2]; ++ox) {
+          int64_t z0 = oz * d->stride[0] - d->padding[0], y0 = oy * d->stride[1] - d->padding[1],
+                  x0 = ox * d->stride[2] - d->padding[2];
+          float max_val = -INFINITY, sum_val = 0.f;
+          int64_t count = 0;
+          for (int64_t kz = 0; kz < d->kernel[0]; ++kz) {
+            int64_t z = z0 + kz * d->dilation[0];
+            if (z < 0 || z >= d->D) continue;
+            for (int64_t ky = 0; ky < d->kernel[1]; ++ky) {
+              int64_t yy = y0 + ky * d->dilation[1];
+              if (yy < 0 || yy >= d->H) continue;
+              for (int64_t kx = 0; kx < d->kernel[2]; ++kx) {
+                int64_t xx = x0 + kx * d->dilation[2];
+                if (xx < 0 || xx >= d->W) continue;
+                float val = x[((nc * d->D + z) * d->H + yy) * d->W + xx];
+                max_val = max_val > val ? max_val : val; /* max(max_val, val): max_pool2d_op.mojo:137 */
+                sum_val = sum_val + val;                 /* avg_pool2d_op.mojo:129-130 */
+                ++count;
+              }
+            }
+          }
+          y[((nc * o[0] + oz) * o[1] + oy) * o[2] + ox] =
+              mode == 0 ? max_val : (count > 0 ? sum_val / (float)count : 0.f); /* avg_pool2d_op.mojo:137-140 */
+        }
+}
+
+/* Adjoint of the loop above (the reference has none: vjp = default_vjp, max_pool2d_op.mojo:152-154), in
+ * scatter form: every output hands its gradient to the first tap that attains its maximum (max), or an
+ * equal share to every tap inside the array (average). */
+void ref_pool_bwd(const pool_desc* d, int32_t mode, const float* x, const float* dy, float* dx) {
+  int64_t o[3];
+  pool_out(d, o);
+  memset(dx, 0, sizeof(float) * (size_t)(d->N * d->C * d->D * d->H * d->W));
+  for (int64_t nc = 0; nc < d->N * d->C; ++nc)
+    for (int64_t oz = 0; oz < o[0]; ++oz)
+      for (int64_t oy = 0; oy < o[1]; ++oy)
+        for (int64_t ox = 0; ox < o[2]; ++ox) {
+          int64_t z0 = oz * d->stride[0] - d->padding[0], y0 = oy * d->stride[1] - d->padding[1],
+                  x0 = ox * d->stride[2] - d->padding[2];
+          float g = dy[((nc * o[0] + oz) * o[1] + oy) * o[2] + ox];
+          int64_t count = 0, best = -1;
+          for (int pass = 0; pass < 2; ++pass)
+            for (int64_t kz = 0; kz < d->kernel[0]; ++kz) {
+              int64_t z = z0 + kz * d->dilation[0];
+              if (z < 0 || z >= d->D) continue;
+              for (int64_t ky = 0; ky < d->kernel[1]; ++ky) {
+                int64_t yy = y0 + ky * d->dilation[1];
+                if (yy < 0 || yy >= d->H) continue;
+                for (int64_t kx = 0; kx < d->kernel[2]; ++kx) {
+                  int64_t xx = x0 + kx * d->dilation[2];
+                  if (xx < 0 || xx >= d->W) continue;
+                  int64_t at = ((nc * d->D + z) * d->H + yy) * d->W + xx;
+                  if (pass == 0) {
+                    ++count;
+                    if (best < 0 || x[at] > x[best]) best = at;
+                  } else if (mode == 1) {
+                    dx[at] = dx[at] + g / (float)count;
+                  }
+                }
+              }
+            }
+          if (mode == 0 && best >= 0) dx[best] = dx[best] + g;
+        }
+}
+
+/* ---- Conv3d.__call__: spacial_ops/conv3d_op.mojo:111-259 (groups = 1); Conv1d is the case D = H = 1
+ * (spacial_ops/conv1d_op.mojo). x [N,C,D,H,W], w [K,C,T,R,S], bias [K] or null. -------------------- */
+typedef struct {
+  int64_t N, C, D, H, W, K, T, R, S;
+  int64_t stride[3], padding[3], dilation[3];
+} conv3d_desc;
+
+static void conv3d_out(const conv3d_desc* d, int64_t* o) {
+  const int64_t in[3] = {d->D, d->H, d->W}, k[3] = {d->T, d->R, d->S};
+  for (int i = 0; i < 3; ++i) o[i] = (in[i] + 2 * d->padding[i] - d->dilation[i] * (k[i] - 1) - 1) / d->stride[i] + 1;
+}
+
+void ref_conv3d_out_shape(const conv3d_desc* d, int64_t* o) { conv3d_out(d, o); }
+
+/* forward when dx, dw, db are all null; otherwise the adjoints, every (output, tap) pair scattering its term */
+void ref_conv3d(const conv3d_desc* d, const float* x, const float* w, const float* bias, float* y, const float* dy,
+                float* dx, float* dw, float* db) {
+  int64_t o[3];
+  conv3d_out(d, o);
+  int bwd = dx || dw || db;
+  if (dx) memset(dx, 0, sizeof(float) * (size_t)(d->N * d->C * d->D * d->H * d->W));
+  if (dw) memset(dw, 0, sizeof(float) * (size_t)(d->K * d->C * d->T * d->R * d->S));
+  if (db) memset(db, 0, sizeof(float) * (size_t)d->K);
+  for (int64_t n = 0; n < d->N; ++n)
+    for (int64_t k = 0; k < d->K; ++k)
+      for (int64_t oz = 0; oz < o[0]; ++oz)
+        for (int64_t oy = 0; oy < o[1]; ++oy)
+          for (int64_t ox = 0; ox < o[2]; ++ox) {
+            int64_t oi = (((n * d->K + k) * o[0] + oz) * o[1] + oy) * o[2] + ox;
+            float value = 0.f, g = bwd ? dy[oi] : 0.f;
+            if (db) db[k] = db[k] + g;
+            int64_t z0 = oz * d->stride[0] - d->padding[0], y0 = oy * d->stride[1] - d->padding[1],
+                    x0 = ox * d->stride[2] - d->padding[2];
+            for (int64_t c = 0; c < d->C; ++c)
+              for (int64_t kz = 0; kz < d->T; ++kz) {
+                int64_t z = z0 + kz * d->dilation[0];
+                if (z < 0 || z >= d->D) continue;
+                for (int64_t ky = 0; ky < d->R; ++ky) {
+                  int64_t yy = y0 + ky * d->dilation[1];
+                  if (yy < 0 || yy >= d->H) continue;
+                  for (int64_t kx = 0; kx < d->S; ++kx) {
+                    int64_t xx = x0 + kx * d->dilation[2];
+                    if (xx < 0 || xx >= d->W) continue;
+                    int64_t xi = (((n * d->C + c) * d->D + z) * d->H + yy) * d->W + xx;
+                    int64_t wi = (((k * d->C + c) * d->T + kz) * d->R + ky) * d->S + kx;
+                    if (!bwd) value = value + x[xi] * w[wi]; /* conv3d_op.mojo:196-236 */
+                    if (dx) dx[xi] = dx[xi] + g * w[wi];
+                    if (dw) dw[wi] = dw[wi] + g * x[xi];
+                  }
+                }
+              }
+            if (!bwd) y[oi] = value + (bias ? bias[k] : 0.f); /* conv3d_op.mojo:238-240 */
+          }
+}
+
 /* ---- optimizers ------------------------------------------------------------------------------
  * SGD plain path: p -= lr * g (optim/sgd.mojo:61-62). Adam: optim/adam.mojo:47-65, one fp32 Array op
  * at a time. Scalars are fp32 (adam.mojo:19-23); t starts at 1 and is incremented by the caller. */

@@ -193,6 +193,90 @@ def conv2d_bwd(x, w, dy, stride=(1, 1), padding=(0, 0), dilation=(1, 1)):
     return dx, dw, db
 
 
+class PoolDesc(ctypes.Structure):
+    _fields_ = [(n, c_int64) for n in ("N", "C", "D", "H", "W")] + [
+        (n, c_int64 * 3) for n in ("kernel", "stride", "padding", "dilation")]
+
+
+def _triple(v, n, fill):
+    v = [v] if isinstance(v, int) else list(v)
+    assert len(v) == n
+    return [fill] * (3 - n) + v
+
+
+def _pool_desc(xshape, kernel, stride, padding, dilation):
+    nsp = len(xshape) - 2
+    d = PoolDesc()
+    d.N, d.C = xshape[0], xshape[1]
+    d.D, d.H, d.W = [1] * (3 - nsp) + list(xshape[2:])
+    d.kernel[:] = _triple(kernel, nsp, 1)
+    d.stride[:] = _triple(stride, nsp, 1)
+    d.padding[:] = _triple(padding, nsp, 0)
+    d.dilation[:] = _triple(dilation, nsp, 1)
+    return d, nsp
+
+
+def pool(mode, x, kernel, stride=1, padding=0, dilation=1):
+    """max / avg pooling of [N, C, spatial...] with 1 to 3 spatial axes."""
+    x = _f32(x)
+    nsp = x.ndim - 2
+    stride, padding, dilation = ([v] * nsp if isinstance(v, int) else v for v in (stride, padding, dilation))
+    d, nsp = _pool_desc(x.shape, kernel, stride, padding, dilation)
+    o = (c_int64 * 3)()
+    lib().ref_pool_out_shape(ctypes.byref(d), o)
+    y = np.empty(tuple(x.shape[:2]) + tuple(o[3 - nsp:]), np.float32)
+    lib().ref_pool_fwd(ctypes.byref(d), c_int32(0 if mode == "max" else 1), _ptr(x), _ptr(y))
+    return y
+
+
+def pool_bwd(mode, x, dy, kernel, stride=1, padding=0, dilation=1):
+    x, dy = _f32(x), _f32(dy)
+    nsp = x.ndim - 2
+    stride, padding, dilation = ([v] * nsp if isinstance(v, int) else v for v in (stride, padding, dilation))
+    d, nsp = _pool_desc(x.shape, kernel, stride, padding, dilation)
+    dx = np.empty_like(x)
+    lib().ref_pool_bwd(ctypes.byref(d), c_int32(0 if mode == "max" else 1), _ptr(x), _ptr(dy), _ptr(dx))
+    return dx
+
+
+class Conv3dDesc(ctypes.Structure):
+    _fields_ = [(n, c_int64) for n in ("N", "C", "D", "H", "W", "K", "T", "R", "S")] + [
+        (n, c_int64 * 3) for n in ("stride", "padding", "dilation")]
+
+
+def _conv3d_desc(xshape, wshape, stride, padding, dilation):
+    nsp = len(xshape) - 2
+    d = Conv3dDesc()
+    d.N, d.C, d.K = xshape[0], xshape[1], wshape[0]
+    d.D, d.H, d.W = [1] * (3 - nsp) + list(xshape[2:])
+    d.T, d.R, d.S = [1] * (3 - nsp) + list(wshape[2:])
+    stride, padding, dilation = ([v] * nsp if isinstance(v, int) else list(v) for v in (stride, padding, dilation))
+    d.stride[:] = _triple(stride, nsp, 1)
+    d.padding[:] = _triple(padding, nsp, 0)
+    d.dilation[:] = _triple(dilation, nsp, 1)
+    o = (c_int64 * 3)()
+    lib().ref_conv3d_out_shape(ctypes.byref(d), o)
+    return d, tuple(o[3 - nsp:])
+
+
+def convnd(x, w, bias=None, stride=1, padding=0, dilation=1):
+    """conv1d / conv2d / conv3d by the rank of x ([N, C, spatial...]), via the 3-D loop."""
+    x, w = _f32(x), _f32(w)
+    d, osp = _conv3d_desc(x.shape, w.shape, stride, padding, dilation)
+    y = np.empty((x.shape[0], w.shape[0]) + osp, np.float32)
+    b = _f32(bias) if bias is not None else None
+    lib().ref_conv3d(ctypes.byref(d), _ptr(x), _ptr(w), _ptr(b) if b is not None else None, _ptr(y), None, None, None, None)
+    return y
+
+
+def convnd_bwd(x, w, dy, stride=1, padding=0, dilation=1):
+    x, w, dy = _f32(x), _f32(w), _f32(dy)
+    d, _ = _conv3d_desc(x.shape, w.shape, stride, padding, dilation)
+    dx, dw, db = np.empty_like(x), np.empty_like(w), np.empty(w.shape[0], np.float32)
+    lib().ref_conv3d(ctypes.byref(d), _ptr(x), _ptr(w), None, None, _ptr(dy), _ptr(dx), _ptr(dw), _ptr(db))
+    return dx, dw, db
+
+
 def sgd(p, g, lr):
     p = _f32(p).copy()
     g = _f32(g)

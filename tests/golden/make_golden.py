@@ -291,3 +291,50 @@ for name, fn in [("greater", torch.gt), ("greater_equal", torch.ge), ("less", to
                  ("equal", torch.eq), ("not_equal", torch.ne)]:
     d[name] = fn(tca, tcb).numpy().astype(np.float32)
 save("binary_more", **d)
+
+# ---- pooling: forward and gradient of sum(pool(x) * g) (test_max_pool2d_op.mojo, test_avg_pool2d_op.mojo and
+# their 1-D / 3-D siblings compare the forward with torch; the gradients have no reference test). Average
+# pooling divides by the taps inside the array, torch's count_include_pad=False. ------------------------
+import torch.nn.functional as TF
+
+d = {}
+POOL_CASES = [  # name, x shape, kernel, stride, padding, dilation
+    ("1d", (2, 3, 17), (3,), (2,), (1,), (1,)),
+    ("2d", (2, 3, 13, 10), (3, 2), (2, 1), (1, 1), (1, 1)),
+    ("3d", (2, 2, 7, 8, 6), (2, 3, 2), (1, 2, 2), (1, 1, 0), (1, 1, 1)),
+    ("2d_dil", (1, 2, 12, 12), (2, 3), (1, 2), (1, 1), (2, 2)),
+]
+for name, xs, k, st, pad, dil in POOL_CASES:
+    x = f32(*xs)
+    nsp = len(xs) - 2
+    mp = [TF.max_pool1d, TF.max_pool2d, TF.max_pool3d][nsp - 1]
+    ap = [TF.avg_pool1d, TF.avg_pool2d, TF.avg_pool3d][nsp - 1]
+    t = t64(x, True)
+    y = mp(t, k, st, pad, dil)
+    g = f32(*y.shape)
+    (y * t64(g)).sum().backward()
+    d.update({"x_" + name: x, "g_" + name: g, "max_" + name: y.detach().numpy(), "dmax_" + name: t.grad.numpy(),
+              "cfg_" + name: np.array([k, st, pad, dil], dtype=np.int64)})
+    if all(v == 1 for v in dil):
+        t = t64(x, True)
+        y = ap(t, k, st, pad, count_include_pad=False)
+        (y * t64(g)).sum().backward()
+        d.update({"avg_" + name: y.detach().numpy(), "davg_" + name: t.grad.numpy()})
+save("pool", **d)
+
+# ---- conv1d and conv3d with bias, stride / padding / dilation, and their gradients (test_conv1d_op.mojo,
+# test_conv3d_op.mojo compare the forward with torch; the gradients are new) ----------------------------
+d = {}
+for name, xs, ws, st, pad, dil in [("1d", (3, 4, 29), (6, 4, 5), (2,), (3,), (2,)),
+                                    ("3d", (2, 3, 6, 9, 8), (5, 3, 2, 3, 3), (1, 2, 1), (1, 1, 2), (2, 1, 1)),
+                                    ("3d_unit", (2, 4, 5, 6, 8), (3, 4, 3, 3, 3), (1, 1, 1), (1, 1, 1), (1, 1, 1))]:
+    x, w, b = f32(*xs), f32(*ws, scale=0.3), f32(ws[0])
+    tx, tw, tb = t64(x, True), t64(w, True), t64(b, True)
+    conv = TF.conv1d if len(xs) == 3 else TF.conv3d
+    y = conv(tx, tw, tb, st, pad, dil)
+    g = f32(*y.shape)
+    (y * t64(g)).sum().backward()
+    d.update({"x_" + name: x, "w_" + name: w, "b_" + name: b, "g_" + name: g, "y_" + name: y.detach().numpy(),
+              "dx_" + name: tx.grad.numpy(), "dw_" + name: tw.grad.numpy(), "db_" + name: tb.grad.numpy(),
+              "cfg_" + name: np.array([st, pad, dil], dtype=np.int64)})
+save("convnd", **d)

@@ -511,3 +511,34 @@ def test_shape_errors(nd):
         nd.relu(nd.zeros([2], is_complex=True))
     with pytest.raises(ValueError, match="4-dimensional"):
         nd.conv2d(nd.zeros([3, 3]), nd.zeros([1, 1, 1, 1]))
+
+
+@pytest.mark.parametrize("name", ["1d", "2d", "3d", "2d_dil"])
+def test_pooling_ops(nd, golden, name):  # test_max_pool2d_op.mojo / test_avg_pool2d_op.mojo and siblings, plus gradients
+    g = golden("pool")
+    k, st, pad, dil = (tuple(int(v) for v in row) for row in g["cfg_" + name])
+    nsp = len(k)
+    if nsp == 1:
+        k, st, pad, dil = k[0], st[0], pad[0], dil[0]
+    for kind in ("max", "avg"):
+        if kind + "_" + name not in g.files:
+            continue
+        x = nd.array(g["x_" + name], requires_grad=True)
+        y = getattr(nd, "%s_pool%dd" % (kind, nsp))(x, k, st, pad, dil)
+        assert_close(y.to_numpy(), g[kind + "_" + name], what=kind)
+        nd.sum(y * nd.array(g["g_" + name])).backward()
+        assert_close(x.grad().to_numpy(), g["d" + kind + "_" + name], what=kind + " grad")
+    with pytest.raises(ValueError):
+        nd.max_pool2d(nd.zeros([2, 3, 4]), (2, 2))
+
+
+def test_conv1d(nd, golden):  # test_conv1d_op.mojo, plus gradients
+    g = golden("convnd")
+    st, pad, dil = (int(row[0]) for row in g["cfg_1d"])
+    x, w, b = (nd.array(g[k + "_1d"], requires_grad=True) for k in ("x", "w", "b"))
+    y = nd.conv1d(x, w, b, st, pad, dil)
+    assert_close(y.to_numpy(), g["y_1d"], what="conv1d")
+    nd.sum(y * nd.array(g["g_1d"])).backward()
+    assert_close(x.grad().to_numpy(), g["dx_1d"], what="dx")
+    assert_close(w.grad().to_numpy(), g["dw_1d"], what="dw")
+    assert_close(b.grad().to_numpy(), g["db_1d"], what="db")

@@ -530,3 +530,69 @@ def test_pool_reuses_buffers(dev):
     dev.call("endia_hip_pool_stats", ctypes.byref(u), ctypes.byref(c), ctypes.byref(n1))
     assert q == p and n1.value == n0.value  # same buffer, no new device allocation
     assert L.lib().endia_hip_free(ctypes.c_void_p(12345)) == L.ERR_INVALID
+
+
+def _pool_desc(xshape, k, st, pad, dil):
+    nsp = len(xshape) - 2
+    d = L.PoolDesc()
+    d.N, d.C = xshape[0], xshape[1]
+    d.D, d.H, d.W = [1] * (3 - nsp) + list(xshape[2:])
+    for field, v, fill in (("kernel", k, 1), ("stride", st, 1), ("padding", pad, 0), ("dilation", dil, 1)):
+        getattr(d, field)[:] = [fill] * (3 - nsp) + list(v)
+    return d
+
+
+def _pool_run(dev, mode, x, gy, k, st, pad, dil):
+    d = _pool_desc(x.shape, k, st, pad, dil)
+    o = (ctypes.c_int64 * 3)()
+    dev.call("endia_hip_pool_out_shape", ctypes.byref(d), o)
+    oshape = tuple(x.shape[:2]) + tuple(o[3 - (x.ndim - 2):])
+    n_out = int(np.prod(oshape))
+    dx_, dy, darg, ddx = dev.put(x), dev.alloc(4 * max(n_out, 1)), dev.alloc(4 * max(n_out, 1)), dev.alloc(max(x.nbytes, 4))
+    dev.call("endia_hip_pool_fwd", ctypes.byref(d), mode, dx_, dy, darg if mode == L.POOL_MAX else None)
+    y = dev.get(dy, oshape)
+    dg = dev.put(gy if gy is not None else np.ones(oshape, np.float32))
+    dev.call("endia_hip_pool_bwd", ctypes.byref(d), mode, dg, darg if mode == L.POOL_MAX else None, ddx)
+    return y, dev.get(ddx, x.shape)
+
+
+@pytest.mark.parametrize("name", ["1d", "2d", "3d", "2d_dil"])
+def test_pool_fwd_bwd(dev, golden, name):
+    g = golden("pool")
+    k, st, pad, dil = (tuple(int(v) for v in row) for row in g["cfg_" + name])
+    x, gy = g["x_" + name], g["g_" + name]
+    for mode, mname in ((L.POOL_MAX, "max"), (L.POOL_AVG, "avg")):
+        y, dx = _pool_run(dev, mode, x, gy, k, st, pad, dil)
+        if mname == "max":
+            np.testing.assert_array_equal(y, R.pool(mname, x, k, st, pad, dil))
+        else:
+            assert_close(y, R.pool(mname, x, k, st, pad, dil), tol=1e-6, what=mname)
+        assert_close(dx, R.pool_bwd(mname, x, gy, k, st, pad, dil), tol=1e-6, what=mname + " grad")
+        if mname + "_" + name in g.files:
+            assert_close(y, g[mname + "_" + name], what=mname + " vs torch")
+            assert_close(dx, g["d" + mname + "_" + name], what=mname + " grad vs torch")
+
+
+def test_pool_edge_cases(dev):
+    # windows that lie wholly in the padding: -inf / 0 forward, nothing flows back (avg_pool2d_op.mojo:137-140)
+    z = np.ones((1, 1, 2), np.float32)
+    y, dx = _pool_run(dev, L.POOL_MAX, z, None, (1,), (1,), (2,), (1,))
+    assert y[0, 0, 0] == -np.inf and y[0, 0, 2] == 1.0
+    np.testing.assert_array_equal(dx, z)
+    y, dx = _pool_run(dev, L.POOL_AVG, z, None, (1,), (1,), (2,), (1,))
+    assert y[0, 0, 0] == 0.0
+    np.testing.assert_array_equal(dx, z)
+    # ties: the first tap in scan order takes the whole gradient
+    t = np.zeros((1, 1, 4, 4), np.float32)
+    _, dx = _pool_run(dev, L.POOL_MAX, t, None, (2, 2), (2, 2), (0, 0), (1, 1))
+    np.testing.assert_array_equal(dx[0, 0], np.array([[1, 0, 1, 0], [0, 0, 0, 0], [1, 0, 1, 0], [0, 0, 0, 0]], np.float32))
+    # argument checks
+    d = _pool_desc((1, 1, 4, 4), (5, 5), (1, 1), (0, 0), (1, 1))
+    o = (ctypes.c_int64 * 3)()
+    with pytest.raises(L.EndiaHipError):
+        dev.call("endia_hip_pool_out_shape", ctypes.byref(d), o)
+    d = _pool_desc((1, 1, 4, 4), (2, 2), (0, 1), (0, 0), (1, 1))
+    with pytest.raises(L.EndiaHipError):
+        dev.call("endia_hip_pool_out_shape", ctypes.byref(d), o)
+    # empty batch
+    _pool_run(dev, L.POOL_MAX, np.zeros((0, 3, 8, 8), np.float32), None, (2, 2), (2, 2), (0, 0), (1, 1))

@@ -302,3 +302,66 @@ def test_complex_mlp_conjugate_convention(golden):
         dW_wirtinger = R.matmul(np.conj(acts[i]).T, delta)
         assert_close(dW_wirtinger, g["dW%d" % i], what="Wirtinger dW%d" % i)
         delta = R.matmul(delta, np.conj(Ws[i]).T)
+
+
+POOL_CASES = ["1d", "2d", "3d", "2d_dil"]
+
+
+def _pool_cfg(g, name):
+    k, st, pad, dil = (tuple(int(v) for v in row) for row in g["cfg_" + name])
+    return k, st, pad, dil
+
+
+@pytest.mark.parametrize("name", POOL_CASES)
+def test_pool_golden(golden, name):  # test_max_pool2d_op.mojo, test_avg_pool2d_op.mojo and siblings: forward vs torch
+    g = golden("pool")
+    k, st, pad, dil = _pool_cfg(g, name)
+    x, gy = g["x_" + name], g["g_" + name]
+    assert_close(R.pool("max", x, k, st, pad, dil), g["max_" + name], tol=1e-7, what="max_pool" + name)
+    assert_close(R.pool_bwd("max", x, gy, k, st, pad, dil), g["dmax_" + name], tol=1e-6, what="max_pool grad " + name)
+    if "avg_" + name in g.files:
+        assert_close(R.pool("avg", x, k, st, pad, dil), g["avg_" + name], tol=1e-6, what="avg_pool" + name)
+        assert_close(R.pool_bwd("avg", x, gy, k, st, pad, dil), g["davg_" + name], tol=1e-6, what="avg_pool grad " + name)
+
+
+def test_avg_pool_dilated_brute_force():
+    """torch's average pooling has no dilation; check that case against a direct numpy restatement and the
+    adjoint identity <pool(x), g> = <x, pool_bwd(g)> (average pooling is linear)."""
+    rng = np.random.default_rng(3)
+    x = rng.standard_normal((2, 2, 9, 8)).astype(np.float32)
+    k, st, pad, dil = (2, 3), (2, 1), (1, 2), (3, 2)
+    y = R.pool("avg", x, k, st, pad, dil)
+    want = np.zeros(y.shape)
+    for oy in range(y.shape[2]):
+        for ox in range(y.shape[3]):
+            taps = [(oy * st[0] - pad[0] + a * dil[0], ox * st[1] - pad[1] + b * dil[1]) for a in range(k[0]) for b in range(k[1])]
+            taps = [(r, c) for r, c in taps if 0 <= r < 9 and 0 <= c < 8]
+            want[:, :, oy, ox] = sum(x[:, :, r, c].astype(np.float64) for r, c in taps) / len(taps) if taps else 0.0
+    assert_close(y, want, tol=1e-6, what="dilated avg_pool")
+    gy = rng.standard_normal(y.shape).astype(np.float32)
+    lhs = np.vdot(y.astype(np.float64), gy)
+    rhs = np.vdot(x.astype(np.float64), R.pool_bwd("avg", x, gy, k, st, pad, dil))
+    assert abs(lhs - rhs) <= 1e-5 * abs(lhs)
+    # an empty window (all taps outside) gives -inf for max and 0 for average (avg_pool2d_op.mojo:137-140)
+    z = np.ones((1, 1, 2), np.float32)
+    assert R.pool("max", z, 1, 1, 2)[0, 0, 0] == -np.inf and R.pool("avg", z, 1, 1, 2)[0, 0, 0] == 0.0
+
+
+@pytest.mark.parametrize("name", ["1d", "3d", "3d_unit"])
+def test_conv1d_conv3d_golden(golden, name):  # test_conv1d_op.mojo, test_conv3d_op.mojo: forward vs torch
+    g = golden("convnd")
+    st, pad, dil = (tuple(int(v) for v in row) for row in g["cfg_" + name])
+    x, w, b, gy = (g[k + "_" + name] for k in ("x", "w", "b", "g"))
+    assert_close(R.convnd(x, w, b, st, pad, dil), g["y_" + name], tol=1e-6, what="conv" + name)
+    dx, dw, db = R.convnd_bwd(x, w, gy, st, pad, dil)
+    assert_close(dx, g["dx_" + name], tol=1e-6, what="dx " + name)
+    assert_close(dw, g["dw_" + name], tol=1e-6, what="dw " + name)
+    assert_close(db, g["db_" + name], tol=1e-6, what="db " + name)
+
+
+def test_convnd_reduces_to_conv2d(golden):
+    """The 3-D loop with depth 1 is the 2-D loop: both restatements must agree exactly."""
+    g = golden("conv2d")
+    x, w, b = g["x"], g["w"], g["b"]
+    y2 = R.conv2d(x, w, b, (2, 2), (1, 1), (1, 1))
+    np.testing.assert_array_equal(R.convnd(x, w, b, (2, 2), (1, 1), (1, 1)), y2)
