@@ -261,6 +261,20 @@ def conv_table(reps=10):
         ("conv2d_bwd_weight", lambda: L.call("endia_hip_conv2d_bwd_weight", ref, x, dy, dw), flop, "mfma"),
         ("conv2d_bwd_bias", lambda: L.call("endia_hip_conv2d_bwd_bias", ref, dy, db), 4.0 * N * K * P * Q, "hbm"),
     ]
+    # pooling of the conv output y [64,128,56,56]: 2x2 stride 2 (max, with argmax; average), forward and backward.
+    # Algorithmic bytes: input once + output once (+ the int32 argmax for max pooling).
+    pd = L.PoolDesc()
+    pd.N, pd.C, pd.D, pd.H, pd.W = N, K, 1, P, Q
+    pd.kernel[:], pd.stride[:], pd.padding[:], pd.dilation[:] = [1, 2, 2], [1, 2, 2], [0, 0, 0], [1, 1, 1]
+    n_in, n_out = N * K * P * Q, N * K * (P // 2) * (Q // 2)
+    py, parg = put(np.zeros(n_out, np.float32)), put(np.zeros(n_out, np.int32))
+    pref = ctypes.byref(pd)
+    cases += [
+        ("max_pool2d 2x2/2 fwd", lambda: L.call("endia_hip_pool_fwd", pref, L.POOL_MAX, dy, py, parg), 4.0 * n_in + 8.0 * n_out, "hbm"),
+        ("max_pool2d 2x2/2 bwd", lambda: L.call("endia_hip_pool_bwd", pref, L.POOL_MAX, py, parg, y), 4.0 * n_in + 8.0 * n_out, "hbm"),
+        ("avg_pool2d 2x2/2 fwd", lambda: L.call("endia_hip_pool_fwd", pref, L.POOL_AVG, dy, py, None), 4.0 * n_in + 4.0 * n_out, "hbm"),
+        ("avg_pool2d 2x2/2 bwd", lambda: L.call("endia_hip_pool_bwd", pref, L.POOL_AVG, py, None, y), 4.0 * n_in + 4.0 * n_out, "hbm"),
+    ]
     rows = []
     ms = ctypes.c_float()
     for name, fn, work, bound in cases:

@@ -93,14 +93,25 @@ __global__ __launch_bounds__(TPB) void pool_fwd_kernel(PoolP p, const float* __r
   }
 }
 
-// number of taps of output coordinate o that fall inside [0, extent)
+// number of taps of output coordinate o that fall inside [0, extent); without padding every tap does
 __device__ __forceinline__ int taps_inside(int o, int k, int s, int pad, int dil, int extent) {
+  if (pad == 0) return k;
   int n = 0;
   for (int a = 0; a < k; ++a) n += (unsigned)(o * s - pad + a * dil) < (unsigned)extent;
   return n;
 }
 
-template <bool MAX>
+// The outputs along one axis whose window holds input coordinate i, for dilation 1: a contiguous range
+// lo..hi (empty when lo > hi), o*s - pad <= i <= o*s - pad + k - 1.
+__device__ __forceinline__ void covering(int i, int k, int pad, int n_out, const FastDiv& ds, int& lo, int& hi) {
+  const int top = i + pad, bottom = i + pad - (k - 1);
+  hi = (int)fdiv((uint32_t)top, ds);
+  if (hi > n_out - 1) hi = n_out - 1;
+  lo = bottom <= 0 ? 0 : (int)fdiv((uint32_t)(bottom + (int)ds.d - 1), ds);
+}
+
+// UNIT: every dilation is 1, so the covering outputs are ranges; otherwise each tap is tried in turn.
+template <bool MAX, bool UNIT>
 __global__ __launch_bounds__(TPB) void pool_bwd_kernel(PoolP p, const float* __restrict__ dy, const int32_t* __restrict__ arg,
                                                        float* __restrict__ dx) {
   const int64_t stride = (int64_t)gridDim.x * TPB;
@@ -113,35 +124,97 @@ __global__ __launch_bounds__(TPB) void pool_bwd_kernel(PoolP p, const float* __r
     const int32_t* at = MAX ? arg + plane * ovol : nullptr;
     const int self = (z * p.H + yy) * p.W + xx;
     float acc = 0.f;
-    // outputs whose window holds this element: o*stride - pad + k*dil = coordinate, per axis
-    for (int a = 0; a < p.kd; ++a) {
-      const int tz = z + p.pd - a * p.dd;
-      if (tz < 0) continue;
-      const int oz = (int)fdiv((uint32_t)tz, p.d_sd);
-      if (oz * p.sd != tz || oz >= p.Do) continue;
-      const int cz = MAX ? 0 : taps_inside(oz, p.kd, p.sd, p.pd, p.dd, p.D);
-      for (int b = 0; b < p.kh; ++b) {
-        const int ty = yy + p.ph - b * p.dh;
-        if (ty < 0) continue;
-        const int oy = (int)fdiv((uint32_t)ty, p.d_sh);
-        if (oy * p.sh != ty || oy >= p.Ho) continue;
-        const int cy = MAX ? 0 : taps_inside(oy, p.kh, p.sh, p.ph, p.dh, p.H);
-        for (int c = 0; c < p.kw; ++c) {
-          const int tx = xx + p.pw - c * p.dw;
-          if (tx < 0) continue;
-          const int ox = (int)fdiv((uint32_t)tx, p.d_sw);
-          if (ox * p.sw != tx || ox >= p.Wo) continue;
-          const int o = (oz * p.Ho + oy) * p.Wo + ox;
-          if (MAX) {
-            if (at[o] == self) acc += g[o];
-          } else {
-            const int cx = taps_inside(ox, p.kw, p.sw, p.pw, p.dw, p.W);
-            acc += g[o] / (float)(cz * cy * cx);
+    if (UNIT) {
+      int z_lo, z_hi, y_lo, y_hi, x_lo, x_hi;
+      covering(z, p.kd, p.pd, p.Do, p.d_sd, z_lo, z_hi);
+      covering(yy, p.kh, p.ph, p.Ho, p.d_sh, y_lo, y_hi);
+      covering(xx, p.kw, p.pw, p.Wo, p.d_sw, x_lo, x_hi);
+      for (int oz = z_lo; oz <= z_hi; ++oz) {
+        const int cz = MAX ? 0 : taps_inside(oz, p.kd, p.sd, p.pd, 1, p.D);
+        for (int oy = y_lo; oy <= y_hi; ++oy) {
+          const int cy = MAX ? 0 : taps_inside(oy, p.kh, p.sh, p.ph, 1, p.H);
+          for (int ox = x_lo; ox <= x_hi; ++ox) {
+            const int o = (oz * p.Ho + oy) * p.Wo + ox;
+            if (MAX) {
+              if (at[o] == self) acc += g[o];
+            } else {
+              acc += g[o] / (float)(cz * cy * taps_inside(ox, p.kw, p.sw, p.pw, 1, p.W));
+            }
+          }
+        }
+      }
+    } else {
+      // outputs whose window holds this element: o*stride - pad + k*dil = coordinate, per axis
+      for (int a = 0; a < p.kd; ++a) {
+        const int tz = z + p.pd - a * p.dd;
+        if (tz < 0) continue;
+        const int oz = (int)fdiv((uint32_t)tz, p.d_sd);
+        if (oz * p.sd != tz || oz >= p.Do) continue;
+        const int cz = MAX ? 0 : taps_inside(oz, p.kd, p.sd, p.pd, p.dd, p.D);
+        for (int b = 0; b < p.kh; ++b) {
+          const int ty = yy + p.ph - b * p.dh;
+          if (ty < 0) continue;
+          const int oy = (int)fdiv((uint32_t)ty, p.d_sh);
+          if (oy * p.sh != ty || oy >= p.Ho) continue;
+          const int cy = MAX ? 0 : taps_inside(oy, p.kh, p.sh, p.ph, p.dh, p.H);
+          for (int c = 0; c < p.kw; ++c) {
+            const int tx = xx + p.pw - c * p.dw;
+            if (tx < 0) continue;
+            const int ox = (int)fdiv((uint32_t)tx, p.d_sw);
+            if (ox * p.sw != tx || ox >= p.Wo) continue;
+            const int o = (oz * p.Ho + oy) * p.Wo + ox;
+            if (MAX) {
+              if (at[o] == self) acc += g[o];
+            } else {
+              acc += g[o] / (float)(cz * cy * taps_inside(ox, p.kw, p.sw, p.pw, p.dw, p.W));
+            }
           }
         }
       }
     }
     dx[j] = acc;
+  }
+}
+
+// Unit dilation, W a multiple of 4: one lane produces 4 consecutive elements of a row, so the index
+// decode and the depth / height ranges are shared by the four and the store is 16 bytes.
+template <bool MAX>
+__global__ __launch_bounds__(TPB) void pool_bwd_row4_kernel(PoolP p, FastDiv d_w4, const float* __restrict__ dy,
+                                                            const int32_t* __restrict__ arg, float* __restrict__ dx) {
+  const int64_t stride = (int64_t)gridDim.x * TPB;
+  const int64_t ovol = (int64_t)p.Do * p.Ho * p.Wo;
+  const int W4 = p.W >> 2;
+  for (int64_t j = (int64_t)blockIdx.x * TPB + threadIdx.x; j < (p.n_in >> 2); j += stride) {
+    uint32_t plane;
+    int z, yy, x4;
+    decode((uint32_t)j, d_w4, p.d_h, p.d_d, W4, p.H, p.D, plane, z, yy, x4);
+    const float* g = dy + plane * ovol;
+    const int32_t* at = MAX ? arg + plane * ovol : nullptr;
+    const int self0 = (z * p.H + yy) * p.W + x4 * 4;
+    int z_lo, z_hi, y_lo, y_hi;
+    covering(z, p.kd, p.pd, p.Do, p.d_sd, z_lo, z_hi);
+    covering(yy, p.kh, p.ph, p.Ho, p.d_sh, y_lo, y_hi);
+    int x_lo[4], x_hi[4];
+#pragma unroll
+    for (int e = 0; e < 4; ++e) covering(x4 * 4 + e, p.kw, p.pw, p.Wo, p.d_sw, x_lo[e], x_hi[e]);
+    float acc[4] = {0.f, 0.f, 0.f, 0.f};
+    for (int oz = z_lo; oz <= z_hi; ++oz) {
+      const int cz = MAX ? 0 : taps_inside(oz, p.kd, p.sd, p.pd, 1, p.D);
+      for (int oy = y_lo; oy <= y_hi; ++oy) {
+        const int czy = MAX ? 0 : cz * taps_inside(oy, p.kh, p.sh, p.ph, 1, p.H);
+        const int row = (oz * p.Ho + oy) * p.Wo;
+#pragma unroll
+        for (int e = 0; e < 4; ++e)
+          for (int ox = x_lo[e]; ox <= x_hi[e]; ++ox) {
+            if (MAX) {
+              if (at[row + ox] == self0 + e) acc[e] += g[row + ox];
+            } else {
+              acc[e] += g[row + ox] / (float)(czy * taps_inside(ox, p.kw, p.sw, p.pw, 1, p.W));
+            }
+          }
+      }
+    }
+    reinterpret_cast<float4*>(dx)[j] = make_float4(acc[0], acc[1], acc[2], acc[3]);
   }
 }
 
@@ -217,8 +290,19 @@ int32_t endia_hip_pool_bwd(const endia_hip_pool_desc* desc, int32_t mode, const 
   ENDIA_CHECK_ARG(dy && dx, "endia_hip_pool_bwd: null pointer");
   ENDIA_CHECK_ARG(mode != ENDIA_POOL_MAX || argmax, "endia_hip_pool_bwd: max pooling needs the argmax array of the forward");
   const int grid = stream_grid(p.n_in);
-  if (mode == ENDIA_POOL_MAX) hipLaunchKernelGGL((pool_bwd_kernel<true>), dim3(grid), dim3(TPB), 0, ctx().stream, p, dy, argmax, dx);
-  else hipLaunchKernelGGL((pool_bwd_kernel<false>), dim3(grid), dim3(TPB), 0, ctx().stream, p, dy, argmax, dx);
+  const bool unit = p.dd == 1 && p.dh == 1 && p.dw == 1;
+  if (unit && p.W % 4 == 0 && (reinterpret_cast<uintptr_t>(dx) & 15) == 0) {
+    const FastDiv d_w4 = make_fastdiv(p.W / 4);
+    const int g4 = stream_grid(p.n_in / 4);
+    if (mode == ENDIA_POOL_MAX) hipLaunchKernelGGL((pool_bwd_row4_kernel<true>), dim3(g4), dim3(TPB), 0, ctx().stream, p, d_w4, dy, argmax, dx);
+    else hipLaunchKernelGGL((pool_bwd_row4_kernel<false>), dim3(g4), dim3(TPB), 0, ctx().stream, p, d_w4, dy, argmax, dx);
+  } else if (mode == ENDIA_POOL_MAX) {
+    if (unit) hipLaunchKernelGGL((pool_bwd_kernel<true, true>), dim3(grid), dim3(TPB), 0, ctx().stream, p, dy, argmax, dx);
+    else hipLaunchKernelGGL((pool_bwd_kernel<true, false>), dim3(grid), dim3(TPB), 0, ctx().stream, p, dy, argmax, dx);
+  } else {
+    if (unit) hipLaunchKernelGGL((pool_bwd_kernel<false, true>), dim3(grid), dim3(TPB), 0, ctx().stream, p, dy, argmax, dx);
+    else hipLaunchKernelGGL((pool_bwd_kernel<false, false>), dim3(grid), dim3(TPB), 0, ctx().stream, p, dy, argmax, dx);
+  }
   ENDIA_LAUNCH_CHECK();
   return ENDIA_HIP_OK;
 }

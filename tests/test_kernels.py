@@ -596,3 +596,21 @@ def test_pool_edge_cases(dev):
         dev.call("endia_hip_pool_out_shape", ctypes.byref(d), o)
     # empty batch
     _pool_run(dev, L.POOL_MAX, np.zeros((0, 3, 8, 8), np.float32), None, (2, 2), (2, 2), (0, 0), (1, 1))
+
+
+@pytest.mark.parametrize("xs,k,st,pad,dil", [
+    ((2, 3, 12, 16), (3, 3), (2, 1), (1, 1), (1, 1)),        # rows of 4: the vectorised backward
+    ((2, 3, 12, 16), (2, 2), (2, 2), (0, 0), (1, 1)),        # windows that tile the input exactly
+    ((1, 2, 5, 6, 8), (2, 3, 3), (1, 2, 3), (1, 0, 1), (1, 1, 1)),
+    ((3, 2, 40), (5,), (3,), (2,), (1,)),
+    ((2, 2, 9, 12), (3, 2), (1, 2), (2, 1), (2, 3)),          # dilated: the tap-by-tap backward
+])
+def test_pool_against_oracle(dev, xs, k, st, pad, dil):
+    rng = np.random.default_rng(sum(xs))
+    x = rng.standard_normal(xs).astype(np.float32)
+    for mode, mname in ((L.POOL_MAX, "max"), (L.POOL_AVG, "avg")):
+        want = R.pool(mname, x, k, st, pad, dil)
+        gy = rng.standard_normal(want.shape).astype(np.float32)
+        y, dx = _pool_run(dev, mode, x, gy, k, st, pad, dil)
+        assert_close(y, want, tol=1e-6, what=mname)
+        assert_close(dx, R.pool_bwd(mname, x, gy, k, st, pad, dil), tol=1e-6, what=mname + " grad")
