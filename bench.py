@@ -261,6 +261,22 @@ def conv_table(reps=10):
         ("conv2d_bwd_weight", lambda: L.call("endia_hip_conv2d_bwd_weight", ref, x, dy, dw), flop, "mfma"),
         ("conv2d_bwd_bias", lambda: L.call("endia_hip_conv2d_bwd_bias", ref, dy, db), 4.0 * N * K * P * Q, "hbm"),
     ]
+    # conv3d: x [8,32,16,56,56], w [64,32,3,3,3], stride 1, pad 1: 2*N*K*C*T*R*S*O*P*Q = 44.4 GFLOP per pass
+    d3 = L.Conv3dDesc()
+    d3.N, d3.C, d3.D, d3.H, d3.W, d3.K, d3.T, d3.R, d3.S = 8, 32, 16, 56, 56, 64, 3, 3, 3
+    d3.stride[:], d3.padding[:], d3.dilation[:], d3.groups = [1, 1, 1], [1, 1, 1], [1, 1, 1], 1
+    x3 = put(rng.standard_normal((8, 32, 16, 56, 56)).astype(np.float32))
+    w3 = put((rng.standard_normal((64, 32, 3, 3, 3)) * np.sqrt(2.0 / (32 * 27))).astype(np.float32))
+    y3 = put(np.zeros((8, 64, 16, 56, 56), np.float32))
+    dx3 = put(np.zeros((8, 32, 16, 56, 56), np.float32))
+    dw3 = put(np.zeros((64, 32, 3, 3, 3), np.float32))
+    flop3 = 2.0 * 8 * 64 * 32 * 27 * 16 * 56 * 56
+    r3 = ctypes.byref(d3)
+    cases += [
+        ("conv3d_fwd", lambda: L.call("endia_hip_conv3d_fwd", r3, x3, w3, None, y3, L.OP_IDENTITY), flop3, "mfma"),
+        ("conv3d_bwd_data", lambda: L.call("endia_hip_conv3d_bwd_data", r3, y3, w3, dx3), flop3, "mfma"),
+        ("conv3d_bwd_weight", lambda: L.call("endia_hip_conv3d_bwd_weight", r3, x3, y3, dw3), flop3, "mfma"),
+    ]
     # pooling of the conv output y [64,128,56,56]: 2x2 stride 2 (max, with argmax; average), forward and backward.
     # Algorithmic bytes: input once + output once (+ the int32 argmax for max pooling).
     pd = L.PoolDesc()

@@ -44,6 +44,11 @@ class EwStep(ctypes.Structure):
     _fields_ = [("kind", c_int32), ("op", c_int32), ("src_kind", c_int32), ("src_index", c_int32), ("imm", c_float)]
 
 
+class Conv3dDesc(ctypes.Structure):
+    _fields_ = [(n, c_int64) for n in ("N", "C", "D", "H", "W", "K", "T", "R", "S")] + [
+        (n, c_int64 * 3) for n in ("stride", "padding", "dilation")] + [("groups", c_int64)]
+
+
 class PoolDesc(ctypes.Structure):
     _fields_ = [(n, c_int64) for n in ("N", "C", "D", "H", "W")] + [
         (n, c_int64 * 3) for n in ("kernel", "stride", "padding", "dilation")]
@@ -97,6 +102,11 @@ SIGNATURES = {
     "endia_hip_conv2d_bwd_data": [POINTER(Conv2dDesc), _fp, _fp, _fp],
     "endia_hip_conv2d_bwd_weight": [POINTER(Conv2dDesc), _fp, _fp, _fp],
     "endia_hip_conv2d_bwd_bias": [POINTER(Conv2dDesc), _fp, _fp],
+    "endia_hip_conv3d_out_shape": [POINTER(Conv3dDesc), _i64p],
+    "endia_hip_conv3d_fwd": [POINTER(Conv3dDesc), _fp, _fp, _fp, _fp, c_int32],
+    "endia_hip_conv3d_bwd_data": [POINTER(Conv3dDesc), _fp, _fp, _fp],
+    "endia_hip_conv3d_bwd_weight": [POINTER(Conv3dDesc), _fp, _fp, _fp],
+    "endia_hip_conv3d_bwd_bias": [POINTER(Conv3dDesc), _fp, _fp],
     "endia_hip_pool_out_shape": [POINTER(PoolDesc), _i64p],
     "endia_hip_pool_fwd": [POINTER(PoolDesc), c_int32, _fp, _fp, _fp],
     "endia_hip_pool_bwd": [POINTER(PoolDesc), c_int32, _fp, _fp, _fp],

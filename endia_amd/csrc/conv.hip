@@ -1,4 +1,7 @@
-// conv2d (NCHW, cross-correlation, groups = 1) as implicit GEMMs on the fp32 matrix cores.
+// conv1d / conv2d / conv3d (channels-first, cross-correlation, groups = 1) as implicit GEMMs on the fp32
+// matrix cores. Everything below is written for [N, C, D, H, W] with a [K, C, T, R, S] kernel; the 2-D op is
+// the case D = T = 1 (the extra index decodes cost nothing there) and the formulas in this header are
+// written for it. Conv3d.__call__ is endia/functional/spacial_ops/conv3d_op.mojo:104-259.
 //
 // Forward follows Conv2d.__call__ (endia/functional/spacial_ops/conv2d_op.mojo:88-196; output shape rule
 // conv2d_op.mojo:31-85):
@@ -33,8 +36,8 @@ constexpr int TPB = 256;
 constexpr int FAR = -(1 << 28);  // coordinate that fails every bounds test
 
 struct ConvP {
-  int N, C, H, W, K, R, S, P, Q;
-  int sh, sw, ph, pw, dh, dw;
+  int N, C, D, H, W, K, T, R, S, O, P, Q;  // O, P, Q: output depth, height, width
+  int sd, sh, sw, pd, ph, pw, dd, dh, dw;
 };
 
 enum { MODE_FWD = 0, MODE_BWD_DATA = 1 };
@@ -46,16 +49,16 @@ struct IgemmArgs {
   const float* bias;  // fwd: [K] or null
   float* out;         // fwd: y; data grad: dx
   int Mrows, Cred;    // output channels of this GEMM; channels reduced over
-  int SH, SW, OH, OW; // source and output spatial extents
-  int Kd, Kd_pad;     // Cred*R*S and its multiple-of-4 padding
-  int Ncols;          // N*OH*OW
-  int R, S, sh, sw, ph, pw, dh, dw;
-  FastDiv d_rs, d_s, d_ohw, d_ow, d_sh, d_sw;
+  int SD, SH, SW, OD, OH, OW; // source and output spatial extents
+  int Kd, Kd_pad;     // Cred*T*R*S and its multiple-of-4 padding
+  int Ncols;          // N*OD*OH*OW
+  int T, R, S, sd, sh, sw, pd, ph, pw, dd, dh, dw;
+  FastDiv d_trs, d_rs, d_s, d_ovol, d_ohw, d_ow, d_sd, d_sh, d_sw;
   int tiles_m, tiles_n, relu;
   int64_t src_bytes;
 };
 
-// B operand: rows = reduction index t = (ch, r, s), columns = output pixels j = (n, oy, ox).
+// B operand: rows = reduction index t = (ch, kz, r, s), columns = output pixels j = (n, oz, oy, ox).
 // A lane owns 4 consecutive columns for the whole kernel (decoded once) and PASSES rows per K tile.
 template <int MODE, int BN, int NT>
 struct GatherColsLoader {
@@ -63,7 +66,7 @@ struct GatherColsLoader {
   static constexpr int ROWS_PER_PASS = NT / F4_PER_ROW;
   static constexpr int PASSES = BK / ROWS_PER_PASS;
   static constexpr int LD = TileShape<false, BN>::LD;
-  int base[4], y0[4], x0[4];
+  int base[4], z0[4], y0[4], x0[4];
   int r, lds_off;
   float reg[PASSES][4];
 
@@ -75,15 +78,19 @@ struct GatherColsLoader {
     for (int e = 0; e < 4; ++e) {
       int j = n0 + c4 + e;
       if (j < a.Ncols) {
-        int n = (int)fdiv((uint32_t)j, a.d_ohw);
-        int rem = j - n * a.OH * a.OW;
+        int n = (int)fdiv((uint32_t)j, a.d_ovol);
+        int rem = j - n * a.OD * a.OH * a.OW;
+        int oz = (int)fdiv((uint32_t)rem, a.d_ohw);
+        rem -= oz * a.OH * a.OW;
         int oy = (int)fdiv((uint32_t)rem, a.d_ow);
         int ox = rem - oy * a.OW;
-        base[e] = n * a.Cred * a.SH * a.SW;
+        base[e] = n * a.Cred * a.SD * a.SH * a.SW;
+        z0[e] = MODE == MODE_FWD ? oz * a.sd - a.pd : oz + a.pd;
         y0[e] = MODE == MODE_FWD ? oy * a.sh - a.ph : oy + a.ph;
         x0[e] = MODE == MODE_FWD ? ox * a.sw - a.pw : ox + a.pw;
       } else {
         base[e] = 0;
+        z0[e] = 0;
         y0[e] = FAR;
         x0[e] = 0;
       }
@@ -94,35 +101,41 @@ struct GatherColsLoader {
 #pragma unroll
     for (int i = 0; i < PASSES; ++i) {
       int t = k0 + r + i * ROWS_PER_PASS;
-      int ch = (int)fdiv((uint32_t)t, a.d_rs);
-      int rem = t - ch * a.R * a.S;
+      int ch = (int)fdiv((uint32_t)t, a.d_trs);
+      int rem = t - ch * a.T * a.R * a.S;
+      int kz = (int)fdiv((uint32_t)rem, a.d_rs);
+      rem -= kz * a.R * a.S;
       int rr = (int)fdiv((uint32_t)rem, a.d_s);
       int ss = rem - rr * a.S;
-      int roff = ch * a.SH * a.SW;
+      int roff = ch * a.SD * a.SH * a.SW;
+      int dzv = kz * a.dd;
       int dyv = t < a.Kd ? rr * a.dh : (MODE == MODE_FWD ? FAR : -FAR);
       int dxv = ss * a.dw;
 #pragma unroll
       for (int e = 0; e < 4; ++e) {
-        int iy, ix;
+        int iz, iy, ix;
         bool ok;
         if (MODE == MODE_FWD) {
+          iz = z0[e] + dzv;
           iy = y0[e] + dyv;
           ix = x0[e] + dxv;
-          ok = (unsigned)iy < (unsigned)a.SH && (unsigned)ix < (unsigned)a.SW;
+          ok = (unsigned)iz < (unsigned)a.SD && (unsigned)iy < (unsigned)a.SH && (unsigned)ix < (unsigned)a.SW;
         } else {
-          int ty = y0[e] - dyv, tx = x0[e] - dxv;
-          if (a.sh == 1 && a.sw == 1) {
+          int tz = z0[e] - dzv, ty = y0[e] - dyv, tx = x0[e] - dxv;
+          if (a.sd == 1 && a.sh == 1 && a.sw == 1) {
+            iz = tz;
             iy = ty;
             ix = tx;
-            ok = (unsigned)iy < (unsigned)a.SH && (unsigned)ix < (unsigned)a.SW;
+            ok = (unsigned)iz < (unsigned)a.SD && (unsigned)iy < (unsigned)a.SH && (unsigned)ix < (unsigned)a.SW;
           } else {
-            ok = ty >= 0 && tx >= 0;
+            ok = tz >= 0 && ty >= 0 && tx >= 0;
+            iz = (int)fdiv((uint32_t)(ok ? tz : 0), a.d_sd);
             iy = (int)fdiv((uint32_t)(ok ? ty : 0), a.d_sh);
             ix = (int)fdiv((uint32_t)(ok ? tx : 0), a.d_sw);
-            ok = ok && iy * a.sh == ty && ix * a.sw == tx && iy < a.SH && ix < a.SW;
+            ok = ok && iz * a.sd == tz && iy * a.sh == ty && ix * a.sw == tx && iz < a.SD && iy < a.SH && ix < a.SW;
           }
         }
-        uint32_t off = ok ? (uint32_t)(base[e] + roff + iy * a.SW + ix) * 4u : OOB_OFFSET;
+        uint32_t off = ok ? (uint32_t)(base[e] + roff + (iz * a.SH + iy) * a.SW + ix) * 4u : OOB_OFFSET;
         reg[i][e] = buffer_load_f1(rs, off);
       }
     }
@@ -179,12 +192,12 @@ __global__ __launch_bounds__(WGM* WGN * 64, 3) void conv_igemm_kernel(IgemmArgs 
     }
   }
 
-  const int64_t ohw = (int64_t)a.OH * a.OW;
+  const int64_t ohw = (int64_t)a.OD * a.OH * a.OW;  // output positions per image
 #pragma unroll
   for (int fn = 0; fn < FN; ++fn) {
     int j = n0 + wn * FN * 32 + fn * 32 + l32;
     if (j >= a.Ncols) continue;
-    int n = (int)fdiv((uint32_t)j, a.d_ohw);
+    int n = (int)fdiv((uint32_t)j, a.d_ovol);
     int64_t col_off = (int64_t)n * a.Mrows * ohw + (j - (int64_t)n * ohw);
 #pragma unroll
     for (int fm = 0; fm < FM; ++fm)
@@ -208,15 +221,15 @@ struct WgradArgs {
   const float* x;
   const float* dy;
   float* part;  // [splits][K][Kd]
-  int N, C, H, W, K, R, S, P, Q, sh, sw, ph, pw, dh, dw;
+  int N, C, D, H, W, K, T, R, S, O, P, Q, sd, sh, sw, pd, ph, pw, dd, dh, dw;
   int Kd;
-  int total_j, chunk;  // N*P*Q and the slice of it one split reduces over (multiple of 32)
-  FastDiv d_pq, d_q, d_rs, d_s;
+  int total_j, chunk;  // N*O*P*Q and the slice of it one split reduces over (multiple of 32)
+  FastDiv d_opq, d_pq, d_q, d_trs, d_rs, d_s;
   int tiles_m, tiles_n;
   int64_t x_bytes, dy_bytes;
 };
 
-// dy as the A operand: rows = output channel k, 32 consecutive j = (n, p, q) per tile.
+// dy as the A operand: rows = output channel k, 32 consecutive j = (n, o, p, q) per tile.
 template <int BM, int NT>
 struct DyRowsLoader {
   static constexpr int ROWS_PER_PASS = NT / 8;
@@ -231,14 +244,14 @@ struct DyRowsLoader {
 #pragma unroll
     for (int i = 0; i < PASSES; ++i) {
       int m = m0 + r + i * ROWS_PER_PASS;
-      rowoff[i] = m < a.K ? m * a.P * a.Q : -1;
+      rowoff[i] = m < a.K ? m * a.O * a.P * a.Q : -1;
     }
   }
   __device__ __forceinline__ void load(const WgradArgs& a, int jt, int j_end) {
     __amdgpu_buffer_rsrc_t rs = make_rsrc(a.dy, a.dy_bytes);
-    const int pq_n = a.P * a.Q;
+    const int pq_n = a.O * a.P * a.Q;
     int j = jt + c4;
-    int n = (int)fdiv((uint32_t)j, a.d_pq);
+    int n = (int)fdiv((uint32_t)j, a.d_opq);
     int pq = j - n * pq_n;
     int off[4];
 #pragma unroll
@@ -261,12 +274,12 @@ struct DyRowsLoader {
   }
 };
 
-// col(x) as the B operand: rows = filter tap t = (c, r, s), 32 consecutive j per tile.
+// col(x) as the B operand: rows = filter tap t = (c, kz, r, s), 32 consecutive j per tile.
 template <int BN, int NT>
 struct TapRowsLoader {
   static constexpr int ROWS_PER_PASS = NT / 8;
   static constexpr int PASSES = BN / ROWS_PER_PASS;
-  int roff[PASSES], dyv[PASSES], dxv[PASSES];
+  int roff[PASSES], dzv[PASSES], dyv[PASSES], dxv[PASSES];
   int c4, lds_off;
   float reg[PASSES][4];
   __device__ __forceinline__ void init(const WgradArgs& a, int n0, int tid) {
@@ -276,11 +289,14 @@ struct TapRowsLoader {
 #pragma unroll
     for (int i = 0; i < PASSES; ++i) {
       int t = n0 + r + i * ROWS_PER_PASS;
-      int ch = (int)fdiv((uint32_t)t, a.d_rs);
-      int rem = t - ch * a.R * a.S;
+      int ch = (int)fdiv((uint32_t)t, a.d_trs);
+      int rem = t - ch * a.T * a.R * a.S;
+      int kz = (int)fdiv((uint32_t)rem, a.d_rs);
+      rem -= kz * a.R * a.S;
       int rr = (int)fdiv((uint32_t)rem, a.d_s);
       int ss = rem - rr * a.S;
-      roff[i] = ch * a.H * a.W;
+      roff[i] = ch * a.D * a.H * a.W;
+      dzv[i] = kz * a.dd - a.pd;
       dyv[i] = t < a.Kd ? rr * a.dh - a.ph : FAR;
       dxv[i] = ss * a.dw - a.pw;
     }
@@ -288,25 +304,28 @@ struct TapRowsLoader {
   __device__ __forceinline__ void load(const WgradArgs& a, int jt, int j_end) {
     __amdgpu_buffer_rsrc_t rs = make_rsrc(a.x, a.x_bytes);
     int j = jt + c4;
-    int n = (int)fdiv((uint32_t)j, a.d_pq);
-    int rem = j - n * a.P * a.Q;
+    int n = (int)fdiv((uint32_t)j, a.d_opq);
+    int rem = j - n * a.O * a.P * a.Q;
+    int o = (int)fdiv((uint32_t)rem, a.d_pq);
+    rem -= o * a.P * a.Q;
     int p = (int)fdiv((uint32_t)rem, a.d_q);
     int q = rem - p * a.Q;
-    int base[4], ye[4], xe[4];
+    int base[4], ze[4], ye[4], xe[4];
 #pragma unroll
     for (int e = 0; e < 4; ++e) {
-      base[e] = n * a.C * a.H * a.W;
+      base[e] = n * a.C * a.D * a.H * a.W;
+      ze[e] = o * a.sd;
       ye[e] = (j + e < j_end) ? p * a.sh : FAR;
       xe[e] = q * a.sw;
-      if (++q == a.Q) { q = 0; if (++p == a.P) { p = 0; ++n; } }
+      if (++q == a.Q) { q = 0; if (++p == a.P) { p = 0; if (++o == a.O) { o = 0; ++n; } } }
     }
 #pragma unroll
     for (int i = 0; i < PASSES; ++i)
 #pragma unroll
       for (int e = 0; e < 4; ++e) {
-        int iy = ye[e] + dyv[i], ix = xe[e] + dxv[i];
-        bool ok = (unsigned)iy < (unsigned)a.H && (unsigned)ix < (unsigned)a.W;
-        reg[i][e] = buffer_load_f1(rs, ok ? (uint32_t)(base[e] + roff[i] + iy * a.W + ix) * 4u : OOB_OFFSET);
+        int iz = ze[e] + dzv[i], iy = ye[e] + dyv[i], ix = xe[e] + dxv[i];
+        bool ok = (unsigned)iz < (unsigned)a.D && (unsigned)iy < (unsigned)a.H && (unsigned)ix < (unsigned)a.W;
+        reg[i][e] = buffer_load_f1(rs, ok ? (uint32_t)(base[e] + roff[i] + (iz * a.H + iy) * a.W + ix) * 4u : OOB_OFFSET);
       }
   }
   __device__ __forceinline__ void store(float* lds) {
@@ -381,14 +400,14 @@ __global__ __launch_bounds__(WGM* WGN * 64, 2) void conv_wgrad_kernel(WgradArgs 
 // consecutive output pixels then read four consecutive source floats: ONE 16-byte buffer load at
 // colbase(j) + table[t], and the whole gather is one integer add per load.
 struct VecArgs {
-  const float* src;   // padded source [N, Cred, Hp, Wp]
+  const float* src;   // padded source [N, Cred, Dp, Hp, Wp]
   const float* wp;    // packed weights [Mrows, Kd_pad]
   const int* table;   // [Kd_pad] byte offset of reduction index t inside an image; OOB_OFFSET for padding rows
   const float* bias;
   float* out;
-  int Mrows, OH, OW, Ncols, Kd_pad;
-  int img_floats, Wp, sh;  // floats per padded image, padded row length, stride along rows
-  FastDiv d_ohw, d_ow;
+  int Mrows, OD, OH, OW, Ncols, Kd_pad;
+  int img_floats, Wp, sh, zstep;  // floats per padded image, padded row length, stride along rows, floats per output depth step
+  FastDiv d_ovol, d_ohw, d_ow;
   int tiles_m, tiles_n, relu;
   int64_t src_bytes;
 };
@@ -420,11 +439,13 @@ __global__ __launch_bounds__(WGM* WGN * 64, 4) void conv_igemm_vec_kernel(VecArg
   {
     int j = n0 + c4;
     if (j < a.Ncols) {
-      int n = (int)fdiv((uint32_t)j, a.d_ohw);
-      int rem = j - n * a.OH * a.OW;
+      int n = (int)fdiv((uint32_t)j, a.d_ovol);
+      int rem = j - n * a.OD * a.OH * a.OW;
+      int oz = (int)fdiv((uint32_t)rem, a.d_ohw);
+      rem -= oz * a.OH * a.OW;
       int oy = (int)fdiv((uint32_t)rem, a.d_ow);
       int ox = rem - oy * a.OW;
-      colbase = (uint32_t)(n * a.img_floats + oy * a.sh * a.Wp + ox) * 4u;
+      colbase = (uint32_t)(n * a.img_floats + oz * a.zstep + oy * a.sh * a.Wp + ox) * 4u;
     }
   }
   const __amdgpu_buffer_rsrc_t rs = make_rsrc(a.src, a.src_bytes);
@@ -463,12 +484,12 @@ __global__ __launch_bounds__(WGM* WGN * 64, 4) void conv_igemm_vec_kernel(VecArg
     }
   }
 
-  const int64_t ohw = (int64_t)a.OH * a.OW;
+  const int64_t ohw = (int64_t)a.OD * a.OH * a.OW;  // output positions per image
 #pragma unroll
   for (int fn = 0; fn < FN; ++fn) {
     int j = n0 + wn * FN * 32 + fn * 32 + l32;
     if (j >= a.Ncols) continue;
-    int n = (int)fdiv((uint32_t)j, a.d_ohw);
+    int n = (int)fdiv((uint32_t)j, a.d_ovol);
     int64_t col_off = (int64_t)n * a.Mrows * ohw + (j - (int64_t)n * ohw);
 #pragma unroll
     for (int fm = 0; fm < FM; ++fm)
@@ -488,13 +509,13 @@ __global__ __launch_bounds__(WGM* WGN * 64, 4) void conv_igemm_vec_kernel(VecArg
 }
 
 struct WgradVecArgs {
-  const float* xpad;  // [N, C, Hp, Wp]
-  const float* dy;    // [N, K, P, Q], Q % 4 == 0
+  const float* xpad;  // [N, C, Dp, Hp, Wp]
+  const float* dy;    // [N, K, O, P, Q], Q % 4 == 0
   const int* table;   // [tiles_n * BN] byte offset of tap t inside a padded image; OOB_OFFSET past Kd
   float* part;
-  int K, Kd, PQ, Q, sh, Wp, img_floats;
+  int K, Kd, OPQ, PQ, Q, sh, Wp, img_floats, zstep;
   int total_j, chunk;
-  FastDiv d_pq, d_q;
+  FastDiv d_opq, d_pq, d_q;
   int tiles_m, tiles_n;
   int64_t x_bytes, dy_bytes;
 };
@@ -521,7 +542,7 @@ __global__ __launch_bounds__(WGM* WGN * 64, 4) void conv_wgrad_vec_kernel(WgradV
 #pragma unroll
   for (int i = 0; i < PA; ++i) {
     int m = m0 + r + i * ROWS_PER_PASS;
-    rowa[i] = m < a.K ? (uint32_t)(m * a.PQ) * 4u : OOB_OFFSET;
+    rowa[i] = m < a.K ? (uint32_t)(m * a.OPQ) * 4u : OOB_OFFSET;
   }
 #pragma unroll
   for (int i = 0; i < PB; ++i) rowb[i] = (uint32_t)a.table[n0 + r + i * ROWS_PER_PASS];
@@ -533,12 +554,14 @@ __global__ __launch_bounds__(WGM* WGN * 64, 4) void conv_wgrad_vec_kernel(WgradV
     int j = jt + c4;
     uint32_t ca = OOB_OFFSET, cb = OOB_OFFSET;
     if (j < j_end) {
-      int n = (int)fdiv((uint32_t)j, a.d_pq);
-      int pq = j - n * a.PQ;
+      int n = (int)fdiv((uint32_t)j, a.d_opq);
+      int opq = j - n * a.OPQ;
+      int o = (int)fdiv((uint32_t)opq, a.d_pq);
+      int pq = opq - o * a.PQ;
       int p = (int)fdiv((uint32_t)pq, a.d_q);
       int q = pq - p * a.Q;
-      ca = (uint32_t)(n * a.K * a.PQ + pq) * 4u;
-      cb = (uint32_t)(n * a.img_floats + p * a.sh * a.Wp + q) * 4u;
+      ca = (uint32_t)(n * a.K * a.OPQ + opq) * 4u;
+      cb = (uint32_t)(n * a.img_floats + o * a.zstep + p * a.sh * a.Wp + q) * 4u;
     }
 #pragma unroll
     for (int i = 0; i < PA; ++i) ra[i] = buffer_load_f4(rs_dy, ca + rowa[i]);
@@ -583,17 +606,19 @@ __global__ __launch_bounds__(WGM* WGN * 64, 4) void conv_wgrad_vec_kernel(WgradV
   }
 }
 
-// Zero-padded copy: dst[pl][y][x] = src[pl][y - py][x - px] where in range, else 0. One wave per padded row
-// (rows are short: the walk over x needs no division, and reads and writes stay contiguous).
+// Zero-padded copy: dst[pl][z][y][x] = src[pl][z - pz][y - py][x - px] where in range, else 0. One wave per
+// padded row (rows are short: the walk over x needs no division, and reads and writes stay contiguous).
 __global__ __launch_bounds__(TPB) void pad_kernel(const float* __restrict__ src, float* __restrict__ dst, int64_t rows_total,
-                                                  int H, int W, int Hp, int Wp, int py, int px) {
+                                                  int D, int H, int W, int Dp, int Hp, int Wp, int pz, int py, int px) {
   const int lane = threadIdx.x & 63;
   const int64_t waves = (int64_t)gridDim.x * (TPB / 64);
   for (int64_t row = (int64_t)blockIdx.x * (TPB / 64) + (threadIdx.x >> 6); row < rows_total; row += waves) {
-    const int64_t pl = row / Hp;
-    const int y = (int)(row - pl * Hp), sy = y - py;
-    const bool row_ok = (unsigned)sy < (unsigned)H;
-    const float* s = src + (pl * H + (row_ok ? sy : 0)) * W;
+    const int64_t slab = row / Hp;  // (plane, padded depth)
+    const int y = (int)(row - slab * Hp), sy = y - py;
+    const int64_t pl = slab / Dp;
+    const int sz = (int)(slab - pl * Dp) - pz;
+    const bool row_ok = (unsigned)sy < (unsigned)H && (unsigned)sz < (unsigned)D;
+    const float* s = src + ((pl * D + (row_ok ? sz : 0)) * H + (row_ok ? sy : 0)) * W;
     float* d = dst + row * Wp;
     for (int x = lane; x < Wp; x += 64) {
       int sx = x - px;
@@ -602,21 +627,23 @@ __global__ __launch_bounds__(TPB) void pad_kernel(const float* __restrict__ src,
   }
 }
 
-// table[t] for t = (ch, r, s): byte offset (ch*Hp + r_eff*dh)*Wp + s_eff*dw inside a padded image, where the
-// data gradient walks the taps in reverse (r_eff = R-1-r). Entries past Kd get OOB_OFFSET.
-__global__ __launch_bounds__(TPB) void tap_table_kernel(int* __restrict__ table, int n, int Kd, int R, int S, int Hp, int Wp,
-                                                        int dh, int dw, int flip) {
+// table[t] for t = (ch, kz, r, s): byte offset ((ch*Dp + kz*dd)*Hp + r*dh)*Wp + s*dw inside a padded image; the
+// data gradient walks the taps in reverse (kz -> T-1-kz, r -> R-1-r, s -> S-1-s). Entries past Kd get OOB_OFFSET.
+__global__ __launch_bounds__(TPB) void tap_table_kernel(int* __restrict__ table, int n, int Kd, int T, int R, int S, int Dp,
+                                                        int Hp, int Wp, int dd, int dh, int dw, int flip) {
   int t = blockIdx.x * TPB + threadIdx.x;
   if (t >= n) return;
   if (t >= Kd) { table[t] = (int)OOB_OFFSET; return; }
-  int ch = t / (R * S), rem = t - ch * R * S, r = rem / S, s = rem - r * S;
-  if (flip) { r = R - 1 - r; s = S - 1 - s; }
-  table[t] = ((ch * Hp + r * dh) * Wp + s * dw) * 4;
+  int ch = t / (T * R * S), rem = t - ch * T * R * S, kz = rem / (R * S);
+  rem -= kz * R * S;
+  int r = rem / S, s = rem - r * S;
+  if (flip) { kz = T - 1 - kz; r = R - 1 - r; s = S - 1 - s; }
+  table[t] = (((ch * Dp + kz * dd) * Hp + r * dh) * Wp + s * dw) * 4;
 }
 
 // ---- weight repacking -------------------------------------------------------------------------------
-// fwd:  wp[k][t]        = w[k][t]                       t = (c, r, s), rows padded to Kd_pad with zeros
-// data: wp[c][(k,r,s)]  = w[k][c][r][s]
+// fwd:  wp[k][t]          = w[k][t]                     t = (c, kz, r, s), rows padded to Kd_pad with zeros
+// data: wp[c][(k,kz,r,s)] = w[k][c][kz][r][s]            (RS below is T*R*S)
 __global__ __launch_bounds__(TPB) void pack_weights_kernel(const float* __restrict__ w, float* __restrict__ wp, int K, int C,
                                                            int RS, int Kd_pad, int transpose) {
   const int rows = transpose ? C : K;
@@ -633,27 +660,53 @@ __global__ __launch_bounds__(TPB) void pack_weights_kernel(const float* __restri
   }
 }
 
-int32_t make_params(const endia_hip_conv2d_desc* d, ConvP& p) {
-  if (!d) return endia::fail(ENDIA_HIP_ERR_INVALID, "conv2d: descriptor is null");
-  if (d->N < 0 || d->C <= 0 || d->H <= 0 || d->W <= 0 || d->K <= 0 || d->R <= 0 || d->S <= 0)
-    return endia::fail(ENDIA_HIP_ERR_INVALID, "conv2d: non-positive extent");
-  if (d->stride_h <= 0 || d->stride_w <= 0 || d->dil_h <= 0 || d->dil_w <= 0 || d->pad_h < 0 || d->pad_w < 0)
-    return endia::fail(ENDIA_HIP_ERR_INVALID, "conv2d: bad stride, dilation or padding");
-  if (d->groups != 1)
-    return endia::fail(ENDIA_HIP_ERR_UNSUPPORTED, "conv2d: groups = %lld; only groups = 1 is implemented", (long long)d->groups);
-  int64_t eh = d->H + 2 * d->pad_h - d->dil_h * (d->R - 1) - 1, ew = d->W + 2 * d->pad_w - d->dil_w * (d->S - 1) - 1;
-  if (eh < 0 || ew < 0) return endia::fail(ENDIA_HIP_ERR_INVALID, "conv2d: kernel larger than padded input");
-  int64_t P = eh / d->stride_h + 1, Q = ew / d->stride_w + 1;
+struct ConvIn {  // the descriptor fields of either entry-point family, depth first
+  int64_t N, C, K, in[3], k[3], stride[3], pad[3], dil[3], groups;
+};
+
+int32_t make_params(const char* op, const ConvIn& d, ConvP& p) {
+  if (d.N < 0 || d.C <= 0 || d.K <= 0) return endia::fail(ENDIA_HIP_ERR_INVALID, "%s: non-positive extent", op);
+  if (d.groups != 1)
+    return endia::fail(ENDIA_HIP_ERR_UNSUPPORTED, "%s: groups = %lld; only groups = 1 is implemented", op, (long long)d.groups);
+  int64_t out[3];
+  for (int i = 0; i < 3; ++i) {
+    if (d.in[i] <= 0 || d.k[i] <= 0) return endia::fail(ENDIA_HIP_ERR_INVALID, "%s: non-positive extent", op);
+    if (d.stride[i] <= 0 || d.dil[i] <= 0 || d.pad[i] < 0)
+      return endia::fail(ENDIA_HIP_ERR_INVALID, "%s: bad stride, dilation or padding", op);
+    int64_t e = d.in[i] + 2 * d.pad[i] - d.dil[i] * (d.k[i] - 1) - 1;  // conv2d_op.mojo:65-84, conv3d_op.mojo:71-101
+    if (e < 0) return endia::fail(ENDIA_HIP_ERR_INVALID, "%s: kernel larger than padded input", op);
+    out[i] = e / d.stride[i] + 1;
+    if (d.pad[i] >= (1 << 20) || d.dil[i] * d.k[i] >= (1 << 20) || d.stride[i] >= (1 << 20))
+      return endia::fail(ENDIA_HIP_ERR_UNSUPPORTED, "%s: stride, padding or dilated kernel extent of 2^20 or more", op);
+  }
   // element offsets are 32-bit with 4-byte scaling inside the gathers: every tensor must stay below 2^29 elements
   const int64_t lim = 1ll << 29;
-  if (d->N * d->C * d->H * d->W >= lim || d->N * d->K * P * Q >= lim || d->K * d->C * d->R * d->S >= lim ||
-      d->pad_h >= (1 << 20) || d->pad_w >= (1 << 20) || d->dil_h * d->R >= (1 << 20) || d->dil_w * d->S >= (1 << 20))
-    return endia::fail(ENDIA_HIP_ERR_UNSUPPORTED, "conv2d: tensor has 2^29 elements or more");
-  p.N = (int)d->N; p.C = (int)d->C; p.H = (int)d->H; p.W = (int)d->W; p.K = (int)d->K; p.R = (int)d->R; p.S = (int)d->S;
-  p.P = (int)P; p.Q = (int)Q;
-  p.sh = (int)d->stride_h; p.sw = (int)d->stride_w; p.ph = (int)d->pad_h; p.pw = (int)d->pad_w;
-  p.dh = (int)d->dil_h; p.dw = (int)d->dil_w;
+  if (d.N * d.C * d.in[0] * d.in[1] * d.in[2] >= lim || d.N * d.K * out[0] * out[1] * out[2] >= lim ||
+      d.K * d.C * d.k[0] * d.k[1] * d.k[2] >= lim)
+    return endia::fail(ENDIA_HIP_ERR_UNSUPPORTED, "%s: tensor has 2^29 elements or more", op);
+  p.N = (int)d.N; p.C = (int)d.C; p.K = (int)d.K;
+  p.D = (int)d.in[0]; p.H = (int)d.in[1]; p.W = (int)d.in[2];
+  p.T = (int)d.k[0]; p.R = (int)d.k[1]; p.S = (int)d.k[2];
+  p.O = (int)out[0]; p.P = (int)out[1]; p.Q = (int)out[2];
+  p.sd = (int)d.stride[0]; p.sh = (int)d.stride[1]; p.sw = (int)d.stride[2];
+  p.pd = (int)d.pad[0]; p.ph = (int)d.pad[1]; p.pw = (int)d.pad[2];
+  p.dd = (int)d.dil[0]; p.dh = (int)d.dil[1]; p.dw = (int)d.dil[2];
   return ENDIA_HIP_OK;
+}
+
+int32_t make_params(const endia_hip_conv2d_desc* d, ConvP& p) {
+  if (!d) return endia::fail(ENDIA_HIP_ERR_INVALID, "conv2d: descriptor is null");
+  ConvIn in = {d->N, d->C, d->K, {1, d->H, d->W}, {1, d->R, d->S}, {1, d->stride_h, d->stride_w},
+               {0, d->pad_h, d->pad_w}, {1, d->dil_h, d->dil_w}, d->groups};
+  return make_params("conv2d", in, p);
+}
+
+int32_t make_params(const endia_hip_conv3d_desc* d, ConvP& p) {
+  if (!d) return endia::fail(ENDIA_HIP_ERR_INVALID, "conv3d: descriptor is null");
+  ConvIn in = {d->N, d->C, d->K, {d->D, d->H, d->W}, {d->T, d->R, d->S},
+               {d->stride[0], d->stride[1], d->stride[2]}, {d->padding[0], d->padding[1], d->padding[2]},
+               {d->dilation[0], d->dilation[1], d->dilation[2]}, d->groups};
+  return make_params("conv3d", in, p);
 }
 
 struct PoolBuf {  // scratch from the library's pool, returned on scope exit (stream-ordered reuse)
@@ -667,25 +720,25 @@ inline int grid_for(int64_t n) {
   return (int)(b < 1 ? 1 : b);
 }
 
-// Padded copy of a [planes, H, W] tensor with (py, px) zeros on every side.
-int32_t make_padded(const float* src, int64_t planes, int H, int W, int py, int px, PoolBuf& buf) {
-  const int Hp = H + 2 * py, Wp = W + 2 * px;
-  int32_t rc = endia_hip_malloc(planes * Hp * Wp * 4, &buf.p);
+// Padded copy of a [planes, D, H, W] tensor with (pz, py, px) zeros on every side.
+int32_t make_padded(const float* src, int64_t planes, int D, int H, int W, int pz, int py, int px, PoolBuf& buf) {
+  const int Dp = D + 2 * pz, Hp = H + 2 * py, Wp = W + 2 * px;
+  int32_t rc = endia_hip_malloc(planes * Dp * Hp * Wp * 4, &buf.p);
   if (rc) return rc;
-  const int64_t rows = planes * Hp;
+  const int64_t rows = planes * Dp * Hp;
   int64_t blocks = (rows + 3) / 4, cap = (int64_t)endia::ctx().cu_count * 64;
   if (blocks > cap) blocks = cap;
   hipLaunchKernelGGL(pad_kernel, dim3((unsigned)blocks), dim3(TPB), 0, endia::ctx().stream, src,
-                     static_cast<float*>(buf.p), rows, H, W, Hp, Wp, py, px);
+                     static_cast<float*>(buf.p), rows, D, H, W, Dp, Hp, Wp, pz, py, px);
   ENDIA_LAUNCH_CHECK();
   return ENDIA_HIP_OK;
 }
 
-int32_t make_table(int n, int Kd, int R, int S, int Hp, int Wp, int dh, int dw, int flip, PoolBuf& buf) {
+int32_t make_table(int n, int Kd, const ConvP& p, int Dp, int Hp, int Wp, int flip, PoolBuf& buf) {
   int32_t rc = endia_hip_malloc((int64_t)n * 4, &buf.p);
   if (rc) return rc;
   hipLaunchKernelGGL(tap_table_kernel, dim3((n + TPB - 1) / TPB), dim3(TPB), 0, endia::ctx().stream,
-                     static_cast<int*>(buf.p), n, Kd, R, S, Hp, Wp, dh, dw, flip);
+                     static_cast<int*>(buf.p), n, Kd, p.T, p.R, p.S, Dp, Hp, Wp, p.dd, p.dh, p.dw, flip);
   ENDIA_LAUNCH_CHECK();
   return ENDIA_HIP_OK;
 }
@@ -698,7 +751,7 @@ int32_t pack_weights(const ConvP& p, const float* w, int transpose, int Kd_pad, 
   int blocks = (int)((total + TPB - 1) / TPB);
   if (blocks > 2048) blocks = 2048;
   hipLaunchKernelGGL(pack_weights_kernel, dim3(blocks), dim3(TPB), 0, endia::ctx().stream, w, static_cast<float*>(buf.p),
-                     p.K, p.C, p.R * p.S, Kd_pad, transpose);
+                     p.K, p.C, p.T * p.R * p.S, Kd_pad, transpose);
   ENDIA_LAUNCH_CHECK();
   return ENDIA_HIP_OK;
 }
@@ -706,35 +759,36 @@ int32_t pack_weights(const ConvP& p, const float* w, int transpose, int Kd_pad, 
 // Fast path of forward / data gradient (see VecArgs). Returns 1 when the shape does not qualify.
 int32_t run_igemm_vec(int mode, const ConvP& p, const float* src, const float* w, const float* bias, float* out, int relu) {
   const bool fwd = mode == MODE_FWD;
-  const int OW = fwd ? p.Q : p.W, OH = fwd ? p.P : p.H;
-  const int SH = fwd ? p.H : p.P, SW = fwd ? p.W : p.Q;
+  const int OW = fwd ? p.Q : p.W, OH = fwd ? p.P : p.H, OD = fwd ? p.O : p.D;
+  const int SD = fwd ? p.D : p.O, SH = fwd ? p.H : p.P, SW = fwd ? p.W : p.Q;
   const int Cred = fwd ? p.C : p.K, Mrows = fwd ? p.K : p.C;
-  int py, px, row_stride;
+  int pz, py, px, row_stride, depth_stride;
   if (fwd) {
     if (p.sw != 1 || OW % 4) return 1;
-    py = p.ph; px = p.pw; row_stride = p.sh;
+    pz = p.pd; py = p.ph; px = p.pw; row_stride = p.sh; depth_stride = p.sd;
   } else {  // transposed convolution with unit strides: pad by (R-1)*d - p
-    if (p.sh != 1 || p.sw != 1 || OW % 4) return 1;
-    py = (p.R - 1) * p.dh - p.ph; px = (p.S - 1) * p.dw - p.pw; row_stride = 1;
-    if (py < 0 || px < 0) return 1;
+    if (p.sd != 1 || p.sh != 1 || p.sw != 1 || OW % 4) return 1;
+    pz = (p.T - 1) * p.dd - p.pd; py = (p.R - 1) * p.dh - p.ph; px = (p.S - 1) * p.dw - p.pw;
+    row_stride = 1; depth_stride = 1;
+    if (pz < 0 || py < 0 || px < 0) return 1;
   }
-  const int Hp = SH + 2 * py, Wp = SW + 2 * px;
-  const int Kd = Cred * p.R * p.S, Kd_pad = (Kd + 31) / 32 * 32;
-  if ((int64_t)p.N * Cred * Hp * Wp >= (1ll << 29) || Kd_pad > 8192) return 1;
+  const int Dp = SD + 2 * pz, Hp = SH + 2 * py, Wp = SW + 2 * px;
+  const int Kd = Cred * p.T * p.R * p.S, Kd_pad = (Kd + 31) / 32 * 32;
+  if ((int64_t)p.N * Cred * Dp * Hp * Wp >= (1ll << 29) || Kd_pad > 8192) return 1;
   // the last reads of a row group must stay inside the padded image rows: ox + 3 + (S-1)*dw <= Wp - 1 holds because
   // OW - 1 + (S-1)*dw <= Wp - 1 by the output-size rule; nothing else to check.
   PoolBuf spad, wp, table;
-  int32_t rc = make_padded(src, (int64_t)p.N * Cred, SH, SW, py, px, spad);
+  int32_t rc = make_padded(src, (int64_t)p.N * Cred, SD, SH, SW, pz, py, px, spad);
   if (rc) return rc;
   if ((rc = pack_weights(p, w, fwd ? 0 : 1, Kd_pad, wp))) return rc;
-  if ((rc = make_table(Kd_pad, Kd, p.R, p.S, Hp, Wp, p.dh, p.dw, fwd ? 0 : 1, table))) return rc;
+  if ((rc = make_table(Kd_pad, Kd, p, Dp, Hp, Wp, fwd ? 0 : 1, table))) return rc;
   VecArgs a;
   a.src = static_cast<const float*>(spad.p); a.wp = static_cast<const float*>(wp.p);
   a.table = static_cast<const int*>(table.p); a.bias = bias; a.out = out; a.relu = relu;
-  a.Mrows = Mrows; a.OH = OH; a.OW = OW; a.Ncols = p.N * OH * OW; a.Kd_pad = Kd_pad;
-  a.img_floats = Cred * Hp * Wp; a.Wp = Wp; a.sh = row_stride;
-  a.d_ohw = make_fastdiv(OH * OW); a.d_ow = make_fastdiv(OW);
-  a.src_bytes = (int64_t)p.N * Cred * Hp * Wp * 4;
+  a.Mrows = Mrows; a.OD = OD; a.OH = OH; a.OW = OW; a.Ncols = p.N * OD * OH * OW; a.Kd_pad = Kd_pad;
+  a.img_floats = Cred * Dp * Hp * Wp; a.Wp = Wp; a.sh = row_stride; a.zstep = depth_stride * Hp * Wp;
+  a.d_ovol = make_fastdiv(OD * OH * OW); a.d_ohw = make_fastdiv(OH * OW); a.d_ow = make_fastdiv(OW);
+  a.src_bytes = (int64_t)p.N * Cred * Dp * Hp * Wp * 4;
   a.tiles_n = (a.Ncols + 127) / 128;
   hipStream_t s = endia::ctx().stream;
   const size_t dyn = (size_t)Kd_pad * 4;
@@ -746,7 +800,12 @@ int32_t run_igemm_vec(int mode, const ConvP& p, const float* src, const float* w
     double rounds = t >= cus ? ((int64_t)((t + cus - 1) / cus)) / (t / cus) : 1.0;
     return rounds * (tm * bm) / (double)Mrows;
   };
-  if (cost(128) <= cost(64) * 0.97) {
+  if (Mrows <= 32) {  // a 32-row tile wastes no MFMA rows on a thin output
+    a.tiles_m = 1;
+    dim3 grid((unsigned)a.tiles_n);
+    if (fwd) hipLaunchKernelGGL((conv_igemm_vec_kernel<1, 4, 1, 1, true>), grid, dim3(256), dyn, s, a);
+    else hipLaunchKernelGGL((conv_igemm_vec_kernel<1, 4, 1, 1, false>), grid, dim3(256), dyn, s, a);
+  } else if (cost(128) <= cost(64) * 0.97) {
     a.tiles_m = (Mrows + 127) / 128;
     dim3 grid((unsigned)(a.tiles_m * a.tiles_n));
     if (fwd) hipLaunchKernelGGL((conv_igemm_vec_kernel<2, 2, 2, 2, true>), grid, dim3(256), dyn, s, a);
@@ -772,23 +831,29 @@ int32_t run_igemm(int mode, const ConvP& p, const float* src, const float* w, co
   a.src = src; a.bias = bias; a.out = out; a.relu = relu;
   a.Mrows = fwd ? p.K : p.C;
   a.Cred = fwd ? p.C : p.K;
-  a.SH = fwd ? p.H : p.P; a.SW = fwd ? p.W : p.Q;
-  a.OH = fwd ? p.P : p.H; a.OW = fwd ? p.Q : p.W;
-  a.Kd = a.Cred * p.R * p.S;
+  a.SD = fwd ? p.D : p.O; a.SH = fwd ? p.H : p.P; a.SW = fwd ? p.W : p.Q;
+  a.OD = fwd ? p.O : p.D; a.OH = fwd ? p.P : p.H; a.OW = fwd ? p.Q : p.W;
+  a.Kd = a.Cred * p.T * p.R * p.S;
   a.Kd_pad = (a.Kd + 3) / 4 * 4;
-  a.Ncols = p.N * a.OH * a.OW;
-  a.R = p.R; a.S = p.S; a.sh = p.sh; a.sw = p.sw; a.ph = p.ph; a.pw = p.pw; a.dh = p.dh; a.dw = p.dw;
-  a.d_rs = make_fastdiv(p.R * p.S); a.d_s = make_fastdiv(p.S);
-  a.d_ohw = make_fastdiv(a.OH * a.OW); a.d_ow = make_fastdiv(a.OW);
-  a.d_sh = make_fastdiv(p.sh); a.d_sw = make_fastdiv(p.sw);
-  a.src_bytes = (int64_t)p.N * a.Cred * a.SH * a.SW * 4;
+  a.Ncols = p.N * a.OD * a.OH * a.OW;
+  a.T = p.T; a.R = p.R; a.S = p.S; a.sd = p.sd; a.sh = p.sh; a.sw = p.sw; a.pd = p.pd; a.ph = p.ph; a.pw = p.pw;
+  a.dd = p.dd; a.dh = p.dh; a.dw = p.dw;
+  a.d_trs = make_fastdiv(p.T * p.R * p.S); a.d_rs = make_fastdiv(p.R * p.S); a.d_s = make_fastdiv(p.S);
+  a.d_ovol = make_fastdiv(a.OD * a.OH * a.OW); a.d_ohw = make_fastdiv(a.OH * a.OW); a.d_ow = make_fastdiv(a.OW);
+  a.d_sd = make_fastdiv(p.sd); a.d_sh = make_fastdiv(p.sh); a.d_sw = make_fastdiv(p.sw);
+  a.src_bytes = (int64_t)p.N * a.Cred * a.SD * a.SH * a.SW * 4;
 
   PoolBuf wp;
   int32_t rc = pack_weights(p, w, fwd ? 0 : 1, a.Kd_pad, wp);
   if (rc) return rc;
   a.wp = static_cast<const float*>(wp.p);
   a.tiles_n = (a.Ncols + 127) / 128;
-  if (a.Mrows > 64) {
+  if (a.Mrows <= 32) {
+    a.tiles_m = 1;
+    dim3 grid((unsigned)a.tiles_n);
+    if (fwd) hipLaunchKernelGGL((conv_igemm_kernel<MODE_FWD, 1, 4, 1, 1>), grid, dim3(256), 0, s, a);
+    else hipLaunchKernelGGL((conv_igemm_kernel<MODE_BWD_DATA, 1, 4, 1, 1>), grid, dim3(256), 0, s, a);
+  } else if (a.Mrows > 64) {
     a.tiles_m = (a.Mrows + 127) / 128;
     dim3 grid((unsigned)(a.tiles_m * a.tiles_n));
     if (fwd) hipLaunchKernelGGL((conv_igemm_kernel<MODE_FWD, 2, 2, 2, 2>), grid, dim3(256), 0, s, a);
@@ -803,9 +868,122 @@ int32_t run_igemm(int mode, const ConvP& p, const float* src, const float* w, co
   return ENDIA_HIP_OK;
 }
 
+int32_t conv_fwd(const char* who, const ConvP& p, const float* x, const float* w, const float* bias, float* y, int32_t act) {
+  if (!(act == ENDIA_OP_IDENTITY || act == ENDIA_OP_RELU))
+    return endia::fail(ENDIA_HIP_ERR_INVALID, "%s: activation must be identity or relu", who);
+  if ((int64_t)p.N * p.K * p.O * p.P * p.Q == 0) return ENDIA_HIP_OK;
+  if (!(x && w && y)) return endia::fail(ENDIA_HIP_ERR_INVALID, "%s: null pointer", who);
+  return run_igemm(MODE_FWD, p, x, w, bias, y, act == ENDIA_OP_RELU ? 1 : 0);
+}
+
+int32_t conv_bwd_data(const char* who, const ConvP& p, const float* dy, const float* w, float* dx) {
+  int64_t total = (int64_t)p.N * p.C * p.D * p.H * p.W;
+  if (total == 0) return ENDIA_HIP_OK;
+  if (!dx) return endia::fail(ENDIA_HIP_ERR_INVALID, "%s: dx is null", who);
+  if ((int64_t)p.O * p.P * p.Q == 0) return endia_hip_fill(dx, total, 0.f);
+  if (!(dy && w)) return endia::fail(ENDIA_HIP_ERR_INVALID, "%s: null pointer", who);
+  return run_igemm(MODE_BWD_DATA, p, dy, w, nullptr, dx, 0);
+}
+
+int32_t conv_bwd_weight(const char* who, const ConvP& p, const float* x, const float* dy, float* dw) {
+  const int Kd = p.C * p.T * p.R * p.S;
+  const int64_t taps = (int64_t)p.K * Kd;
+  if (!dw) return endia::fail(ENDIA_HIP_ERR_INVALID, "%s: dw is null", who);
+  const int64_t total_j = (int64_t)p.N * p.O * p.P * p.Q;
+  if (total_j == 0) return endia_hip_fill(dw, taps, 0.f);
+  if (!(x && dy)) return endia::fail(ENDIA_HIP_ERR_INVALID, "%s: null pointer", who);
+  hipStream_t s = endia::ctx().stream;
+
+  WgradArgs a;
+  a.x = x; a.dy = dy;
+  a.N = p.N; a.C = p.C; a.D = p.D; a.H = p.H; a.W = p.W; a.K = p.K; a.T = p.T; a.R = p.R; a.S = p.S;
+  a.O = p.O; a.P = p.P; a.Q = p.Q;
+  a.sd = p.sd; a.sh = p.sh; a.sw = p.sw; a.pd = p.pd; a.ph = p.ph; a.pw = p.pw; a.dd = p.dd; a.dh = p.dh; a.dw = p.dw;
+  a.Kd = Kd;
+  a.total_j = (int)total_j;
+  a.d_opq = make_fastdiv(p.O * p.P * p.Q); a.d_pq = make_fastdiv(p.P * p.Q); a.d_q = make_fastdiv(p.Q);
+  a.d_trs = make_fastdiv(p.T * p.R * p.S); a.d_rs = make_fastdiv(p.R * p.S); a.d_s = make_fastdiv(p.S);
+  a.x_bytes = (int64_t)p.N * p.C * p.D * p.H * p.W * 4;
+  a.dy_bytes = (int64_t)p.N * p.K * p.O * p.P * p.Q * 4;
+  const int Dp = p.D + 2 * p.pd, Hp = p.H + 2 * p.ph, Wp = p.W + 2 * p.pw;
+  const bool vec = p.sw == 1 && p.Q % 4 == 0 && (int64_t)p.N * p.C * Dp * Hp * Wp < (1ll << 29) &&
+                   (reinterpret_cast<uintptr_t>(dy) & 15) == 0;
+  // 64-wide tiles over the taps when the last 128-wide tile would be at most half full
+  const int bn = (vec && Kd % 128 != 0 && Kd % 128 <= 64) ? 64 : 128;
+  // likewise 64-high tiles over the output channels
+  const int bm = (vec && p.K % 128 != 0 && p.K % 128 <= 64) ? 64 : 128;
+  a.tiles_m = (p.K + bm - 1) / bm;
+  a.tiles_n = (Kd + bn - 1) / bn;
+  // split the N*O*P*Q reduction so that about 4 work-groups per CU exist; every split reduces >= 256 columns
+  int64_t tiles = (int64_t)a.tiles_m * a.tiles_n;
+  int64_t splits = ((int64_t)endia::ctx().cu_count * 4 + tiles - 1) / tiles;
+  int64_t max_splits = (total_j + 255) / 256;
+  if (splits > max_splits) splits = max_splits;
+  if (splits > 1024) splits = 1024;
+  if (splits < 1) splits = 1;
+  int64_t chunk = ((total_j + splits - 1) / splits + 31) / 32 * 32;
+  splits = (total_j + chunk - 1) / chunk;
+  a.chunk = (int)chunk;
+
+  PoolBuf part;
+  int32_t rc;
+  if (splits > 1) {
+    rc = endia_hip_malloc(splits * taps * 4, &part.p);
+    if (rc) return rc;
+    a.part = static_cast<float*>(part.p);
+  } else {
+    a.part = dw;
+  }
+  dim3 grid((unsigned)tiles, (unsigned)splits);
+  if (vec) {
+    PoolBuf xpad, table;
+    if ((rc = make_padded(x, (int64_t)p.N * p.C, p.D, p.H, p.W, p.pd, p.ph, p.pw, xpad))) return rc;
+    if ((rc = make_table(a.tiles_n * bn, Kd, p, Dp, Hp, Wp, 0, table))) return rc;
+    WgradVecArgs v;
+    v.xpad = static_cast<const float*>(xpad.p); v.dy = dy; v.table = static_cast<const int*>(table.p); v.part = a.part;
+    v.K = p.K; v.Kd = Kd; v.OPQ = p.O * p.P * p.Q; v.PQ = p.P * p.Q; v.Q = p.Q; v.sh = p.sh; v.Wp = Wp;
+    v.img_floats = p.C * Dp * Hp * Wp; v.zstep = p.sd * Hp * Wp;
+    v.total_j = a.total_j; v.chunk = a.chunk; v.d_opq = a.d_opq; v.d_pq = a.d_pq; v.d_q = a.d_q;
+    v.tiles_m = a.tiles_m; v.tiles_n = a.tiles_n;
+    v.x_bytes = (int64_t)p.N * p.C * Dp * Hp * Wp * 4; v.dy_bytes = a.dy_bytes;
+    if (bm == 128 && bn == 128) hipLaunchKernelGGL((conv_wgrad_vec_kernel<2, 2, 2, 2>), grid, dim3(256), 0, s, v);
+    else if (bm == 128) hipLaunchKernelGGL((conv_wgrad_vec_kernel<2, 2, 2, 1>), grid, dim3(256), 0, s, v);
+    else if (bn == 128) hipLaunchKernelGGL((conv_wgrad_vec_kernel<2, 2, 1, 2>), grid, dim3(256), 0, s, v);
+    else hipLaunchKernelGGL((conv_wgrad_vec_kernel<2, 2, 1, 1>), grid, dim3(256), 0, s, v);
+  } else {
+    hipLaunchKernelGGL((conv_wgrad_kernel<2, 2, 2, 2>), grid, dim3(256), 0, s, a);
+  }
+  ENDIA_LAUNCH_CHECK();
+  if (splits > 1) return endia::col_reduce(1, splits, taps, a.part, dw, 1.f);  // partials added in split order
+  return ENDIA_HIP_OK;
+}
+
+int32_t conv_bwd_bias(const char* who, const ConvP& p, const float* dy, float* db) {
+  if (!db) return endia::fail(ENDIA_HIP_ERR_INVALID, "%s: db is null", who);
+  const int64_t PQ = (int64_t)p.O * p.P * p.Q, rows = (int64_t)p.N * p.K;
+  if (rows * PQ == 0) return endia_hip_fill(db, p.K, 0.f);
+  if (!dy) return endia::fail(ENDIA_HIP_ERR_INVALID, "%s: dy is null", who);
+  if (rows > 65535) return endia::fail(ENDIA_HIP_ERR_INVALID, "%s: N*K = %lld exceeds 65535", who, (long long)rows);
+  // [N*K, O*P*Q] -> [N*K] with wave-shuffle row sums, then [N, K] -> [K]
+  PoolBuf tmp;
+  int32_t rc = endia_hip_malloc(rows * (int64_t)sizeof(float), &tmp.p);
+  if (rc) return rc;
+  rc = endia::row_reduce(rows, PQ, dy, static_cast<float*>(tmp.p), 1.f);
+  if (!rc) rc = endia::col_reduce(1, p.N, p.K, static_cast<float*>(tmp.p), db, 1.f);
+  return rc;
+}
+
 }  // namespace
 
 using namespace endia;
+
+#define ENDIA_CONV_PARAMS(d)       \
+  ENDIA_REQUIRE_INIT();            \
+  ConvP p;                         \
+  {                                \
+    int32_t rc_ = make_params(d, p); \
+    if (rc_) return rc_;           \
+  }
 
 extern "C" {
 
@@ -821,116 +999,55 @@ int32_t endia_hip_conv2d_out_shape(const endia_hip_conv2d_desc* d, int64_t* P, i
 
 int32_t endia_hip_conv2d_fwd(const endia_hip_conv2d_desc* d, const float* x, const float* w, const float* bias, float* y,
                              int32_t act) {
-  ENDIA_REQUIRE_INIT();
-  ConvP p;
-  int32_t rc = make_params(d, p);
-  if (rc) return rc;
-  ENDIA_CHECK_ARG(act == ENDIA_OP_IDENTITY || act == ENDIA_OP_RELU, "endia_hip_conv2d_fwd: activation must be identity or relu");
-  if ((int64_t)p.N * p.K * p.P * p.Q == 0) return ENDIA_HIP_OK;
-  ENDIA_CHECK_ARG(x && w && y, "endia_hip_conv2d_fwd: null pointer");
-  return run_igemm(MODE_FWD, p, x, w, bias, y, act == ENDIA_OP_RELU ? 1 : 0);
+  ENDIA_CONV_PARAMS(d);
+  return conv_fwd(__func__, p, x, w, bias, y, act);
 }
 
 int32_t endia_hip_conv2d_bwd_data(const endia_hip_conv2d_desc* d, const float* dy, const float* w, float* dx) {
-  ENDIA_REQUIRE_INIT();
-  ConvP p;
-  int32_t rc = make_params(d, p);
-  if (rc) return rc;
-  int64_t total = (int64_t)p.N * p.C * p.H * p.W;
-  if (total == 0) return ENDIA_HIP_OK;
-  ENDIA_CHECK_ARG(dx != nullptr, "endia_hip_conv2d_bwd_data: dx is null");
-  if ((int64_t)p.P * p.Q == 0) return endia_hip_fill(dx, total, 0.f);
-  ENDIA_CHECK_ARG(dy && w, "endia_hip_conv2d_bwd_data: null pointer");
-  return run_igemm(MODE_BWD_DATA, p, dy, w, nullptr, dx, 0);
+  ENDIA_CONV_PARAMS(d);
+  return conv_bwd_data(__func__, p, dy, w, dx);
 }
 
 int32_t endia_hip_conv2d_bwd_weight(const endia_hip_conv2d_desc* d, const float* x, const float* dy, float* dw) {
-  ENDIA_REQUIRE_INIT();
-  ConvP p;
-  int32_t rc = make_params(d, p);
-  if (rc) return rc;
-  const int Kd = p.C * p.R * p.S;
-  const int64_t taps = (int64_t)p.K * Kd;
-  ENDIA_CHECK_ARG(dw != nullptr, "endia_hip_conv2d_bwd_weight: dw is null");
-  const int64_t total_j = (int64_t)p.N * p.P * p.Q;
-  if (total_j == 0) return endia_hip_fill(dw, taps, 0.f);
-  ENDIA_CHECK_ARG(x && dy, "endia_hip_conv2d_bwd_weight: null pointer");
-  hipStream_t s = ctx().stream;
-
-  WgradArgs a;
-  a.x = x; a.dy = dy;
-  a.N = p.N; a.C = p.C; a.H = p.H; a.W = p.W; a.K = p.K; a.R = p.R; a.S = p.S; a.P = p.P; a.Q = p.Q;
-  a.sh = p.sh; a.sw = p.sw; a.ph = p.ph; a.pw = p.pw; a.dh = p.dh; a.dw = p.dw;
-  a.Kd = Kd;
-  a.total_j = (int)total_j;
-  a.d_pq = make_fastdiv(p.P * p.Q); a.d_q = make_fastdiv(p.Q);
-  a.d_rs = make_fastdiv(p.R * p.S); a.d_s = make_fastdiv(p.S);
-  a.x_bytes = (int64_t)p.N * p.C * p.H * p.W * 4;
-  a.dy_bytes = (int64_t)p.N * p.K * p.P * p.Q * 4;
-  const int Hp = p.H + 2 * p.ph, Wp = p.W + 2 * p.pw;
-  const bool vec = p.sw == 1 && p.Q % 4 == 0 && (int64_t)p.N * p.C * Hp * Wp < (1ll << 29) &&
-                   (reinterpret_cast<uintptr_t>(dy) & 15) == 0;
-  // 64-wide tiles over the taps when the last 128-wide tile would be at most half full
-  const int bn = (vec && Kd % 128 != 0 && Kd % 128 <= 64) ? 64 : 128;
-  a.tiles_m = (p.K + 127) / 128;
-  a.tiles_n = (Kd + bn - 1) / bn;
-  // split the N*P*Q reduction so that about 4 work-groups per CU exist; every split reduces >= 256 columns
-  int64_t tiles = (int64_t)a.tiles_m * a.tiles_n;
-  int64_t splits = ((int64_t)ctx().cu_count * 4 + tiles - 1) / tiles;
-  int64_t max_splits = (total_j + 255) / 256;
-  if (splits > max_splits) splits = max_splits;
-  if (splits > 1024) splits = 1024;
-  if (splits < 1) splits = 1;
-  int64_t chunk = ((total_j + splits - 1) / splits + 31) / 32 * 32;
-  splits = (total_j + chunk - 1) / chunk;
-  a.chunk = (int)chunk;
-
-  PoolBuf part;
-  if (splits > 1) {
-    rc = endia_hip_malloc(splits * taps * 4, &part.p);
-    if (rc) return rc;
-    a.part = static_cast<float*>(part.p);
-  } else {
-    a.part = dw;
-  }
-  dim3 grid((unsigned)tiles, (unsigned)splits);
-  if (vec) {
-    PoolBuf xpad, table;
-    if ((rc = make_padded(x, (int64_t)p.N * p.C, p.H, p.W, p.ph, p.pw, xpad))) return rc;
-    if ((rc = make_table(a.tiles_n * bn, Kd, p.R, p.S, Hp, Wp, p.dh, p.dw, 0, table))) return rc;
-    WgradVecArgs v;
-    v.xpad = static_cast<const float*>(xpad.p); v.dy = dy; v.table = static_cast<const int*>(table.p); v.part = a.part;
-    v.K = p.K; v.Kd = Kd; v.PQ = p.P * p.Q; v.Q = p.Q; v.sh = p.sh; v.Wp = Wp; v.img_floats = p.C * Hp * Wp;
-    v.total_j = a.total_j; v.chunk = a.chunk; v.d_pq = a.d_pq; v.d_q = a.d_q;
-    v.tiles_m = a.tiles_m; v.tiles_n = a.tiles_n;
-    v.x_bytes = (int64_t)p.N * p.C * Hp * Wp * 4; v.dy_bytes = a.dy_bytes;
-    if (bn == 128) hipLaunchKernelGGL((conv_wgrad_vec_kernel<2, 2, 2, 2>), grid, dim3(256), 0, s, v);
-    else hipLaunchKernelGGL((conv_wgrad_vec_kernel<2, 2, 2, 1>), grid, dim3(256), 0, s, v);
-  } else {
-    hipLaunchKernelGGL((conv_wgrad_kernel<2, 2, 2, 2>), grid, dim3(256), 0, s, a);
-  }
-  ENDIA_LAUNCH_CHECK();
-  if (splits > 1) return col_reduce(1, splits, taps, a.part, dw, 1.f);  // partials added in split order
-  return ENDIA_HIP_OK;
+  ENDIA_CONV_PARAMS(d);
+  return conv_bwd_weight(__func__, p, x, dy, dw);
 }
 
 int32_t endia_hip_conv2d_bwd_bias(const endia_hip_conv2d_desc* d, const float* dy, float* db) {
-  ENDIA_REQUIRE_INIT();
+  ENDIA_CONV_PARAMS(d);
+  return conv_bwd_bias(__func__, p, dy, db);
+}
+
+int32_t endia_hip_conv3d_out_shape(const endia_hip_conv3d_desc* d, int64_t* out_dhw) {
   ConvP p;
   int32_t rc = make_params(d, p);
   if (rc) return rc;
-  ENDIA_CHECK_ARG(db != nullptr, "endia_hip_conv2d_bwd_bias: db is null");
-  const int64_t PQ = (int64_t)p.P * p.Q, rows = (int64_t)p.N * p.K;
-  if (rows * PQ == 0) return endia_hip_fill(db, p.K, 0.f);
-  ENDIA_CHECK_ARG(dy != nullptr, "endia_hip_conv2d_bwd_bias: dy is null");
-  ENDIA_CHECK_ARG(rows <= 65535, "endia_hip_conv2d_bwd_bias: N*K = %lld exceeds 65535", (long long)rows);
-  // [N*K, P*Q] -> [N*K] with wave-shuffle row sums, then [N, K] -> [K]
-  PoolBuf tmp;
-  rc = endia_hip_malloc(rows * (int64_t)sizeof(float), &tmp.p);
-  if (rc) return rc;
-  rc = row_reduce(rows, PQ, dy, static_cast<float*>(tmp.p), 1.f);
-  if (!rc) rc = col_reduce(1, p.N, p.K, static_cast<float*>(tmp.p), db, 1.f);
-  return rc;
+  ENDIA_CHECK_ARG(out_dhw, "endia_hip_conv3d_out_shape: null output");
+  out_dhw[0] = p.O;
+  out_dhw[1] = p.P;
+  out_dhw[2] = p.Q;
+  return ENDIA_HIP_OK;
+}
+
+int32_t endia_hip_conv3d_fwd(const endia_hip_conv3d_desc* d, const float* x, const float* w, const float* bias, float* y,
+                             int32_t act) {
+  ENDIA_CONV_PARAMS(d);
+  return conv_fwd(__func__, p, x, w, bias, y, act);
+}
+
+int32_t endia_hip_conv3d_bwd_data(const endia_hip_conv3d_desc* d, const float* dy, const float* w, float* dx) {
+  ENDIA_CONV_PARAMS(d);
+  return conv_bwd_data(__func__, p, dy, w, dx);
+}
+
+int32_t endia_hip_conv3d_bwd_weight(const endia_hip_conv3d_desc* d, const float* x, const float* dy, float* dw) {
+  ENDIA_CONV_PARAMS(d);
+  return conv_bwd_weight(__func__, p, x, dy, dw);
+}
+
+int32_t endia_hip_conv3d_bwd_bias(const endia_hip_conv3d_desc* d, const float* dy, float* db) {
+  ENDIA_CONV_PARAMS(d);
+  return conv_bwd_bias(__func__, p, dy, db);
 }
 
 }  // extern "C"

@@ -808,6 +808,50 @@ def conv1d(x, kernel, bias=None, stride=1, padding=0, dilation=1, groups=1):
     return reshape(y, [N, K, y._shape[-1]])
 
 
+def conv3d(x, kernel, bias=None, stride=(1, 1, 1), padding=(0, 0, 0), dilation=(1, 1, 1), groups=1):
+    """[N, C, D, H, W] cross-correlation with kernel [K, C, T, R, S] (conv3d_op.mojo:104-259; tuple order is
+    (depth, height, width)). The reference has no backward rule for it (conv3d_op.mojo:261-263); the VJP here
+    is the adjoint of its forward loop."""
+    import ctypes
+    if x.ndim() != 5:
+        raise ValueError("Input must be 5-dimensional (batch_size, in_channels, depth, height, width) for 3D convolution!")
+    if x._shape[1] != kernel._shape[1]:
+        raise ValueError("Input channels must match kernel channels for 3D convolution!")
+    if x.is_complex_ or kernel.is_complex_:
+        raise ValueError("Complex numbers are not supported for conv3d!")
+    desc = L.Conv3dDesc()
+    desc.N, desc.C, desc.D, desc.H, desc.W = x._shape
+    desc.K, _, desc.T, desc.R, desc.S = kernel._shape
+    desc.stride[:], desc.padding[:], desc.dilation[:] = _tuple_n(stride, 3), _tuple_n(padding, 3), _tuple_n(dilation, 3)
+    desc.groups = groups
+    o = (ctypes.c_int64 * 3)()
+    L.call("endia_hip_conv3d_out_shape", ctypes.byref(desc), o)
+    xs, ks = contiguous(x), contiguous(kernel)
+    bsrc = contiguous(bias) if bias is not None else None
+    out = Array.empty([desc.N, desc.K, o[0], o[1], o[2]])
+    L.call("endia_hip_conv3d_fwd", ctypes.byref(desc), xs.data_ptr(), ks.data_ptr(),
+           bsrc.data_ptr() if bsrc is not None else None, out.data_ptr(), L.OP_IDENTITY)
+
+    def vjp(primals, grad, out_):
+        from .autograd.functional import building_graph
+        if building_graph():
+            raise NotImplementedError("conv3d has no second-order rule")
+        g = contiguous(grad)
+        res = [None] * len(primals)
+        if primals[0]._requires_grad:
+            res[0] = Array.empty(primals[0]._shape)
+            L.call("endia_hip_conv3d_bwd_data", ctypes.byref(desc), g.data_ptr(), ks.data_ptr(), res[0].data_ptr())
+        if primals[1]._requires_grad:
+            res[1] = Array.empty(primals[1]._shape)
+            L.call("endia_hip_conv3d_bwd_weight", ctypes.byref(desc), xs.data_ptr(), g.data_ptr(), res[1].data_ptr())
+        if len(primals) > 2 and primals[2]._requires_grad:
+            res[2] = Array.empty(primals[2]._shape)
+            L.call("endia_hip_conv3d_bwd_bias", ctypes.byref(desc), g.data_ptr(), res[2].data_ptr())
+        return res
+
+    return _register(out, [x, kernel] + ([bias] if bias is not None else []), "conv3d", vjp)
+
+
 # --------------------------------------------------------------------------------------------------
 # pooling (endia/functional/spacial_ops/{max,avg}_pool{1,2,3}d_op.mojo)
 # --------------------------------------------------------------------------------------------------

@@ -264,6 +264,23 @@ ENDIA_API int32_t endia_hip_conv2d_bwd_weight(const endia_hip_conv2d_desc* d, co
                                     float* dw);
 ENDIA_API int32_t endia_hip_conv2d_bwd_bias(const endia_hip_conv2d_desc* d, const float* dy, float* db);
 
+/* ---- conv3d, [N,C,D,H,W] with kernel [K,C,T,R,S], groups = 1: Conv3d.__call__ (spacial_ops/conv3d_op.mojo:104-259),
+ *      output extents per axis (in + 2*pad - dil*(k-1) - 1) / stride + 1 (conv3d_op.mojo:71-101). Conv1d
+ *      (spacial_ops/conv1d_op.mojo) is conv2d on a height-1 image. Same kernels as conv2d, which is the case
+ *      D = T = 1; the three gradients are the adjoints of the forward loop (the reference has none:
+ *      Conv3d.vjp = default_vjp). Array order in stride / padding / dilation: depth, height, width. */
+typedef struct endia_hip_conv3d_desc {
+  int64_t N, C, D, H, W, K, T, R, S;
+  int64_t stride[3], padding[3], dilation[3];
+  int64_t groups;
+} endia_hip_conv3d_desc;
+ENDIA_API int32_t endia_hip_conv3d_out_shape(const endia_hip_conv3d_desc* desc, int64_t* out_dhw);
+ENDIA_API int32_t endia_hip_conv3d_fwd(const endia_hip_conv3d_desc* desc, const float* x, const float* w, const float* bias,
+                             float* y, int32_t act);
+ENDIA_API int32_t endia_hip_conv3d_bwd_data(const endia_hip_conv3d_desc* desc, const float* dy, const float* w, float* dx);
+ENDIA_API int32_t endia_hip_conv3d_bwd_weight(const endia_hip_conv3d_desc* desc, const float* x, const float* dy, float* dw);
+ENDIA_API int32_t endia_hip_conv3d_bwd_bias(const endia_hip_conv3d_desc* desc, const float* dy, float* db);
+
 /* ---- pooling over 1, 2 or 3 spatial axes of a contiguous [N, C, D, H, W] array (set the unused leading
  *      axes to extent 1 with kernel 1, stride 1, padding 0, dilation 1). Forward: MaxPool{1,2,3}d.__call__
  *      (spacial_ops/max_pool2d_op.mojo:88-150 and siblings), AvgPool{1,2,3}d.__call__

@@ -607,7 +607,7 @@ void ref_pool_bwd(const pool_desc* d, int32_t mode, const float* x, const float*
         }
 }
 
-/* ---- Conv3d.__call__: spacial_ops/conv3d_op.mojo:111-259 (groups = 1); Conv1d is the case D = H = 1
+/* ---- Conv3d.__call__: spacial_ops/conv3d_op.mojo:104-259 (groups = 1); Conv1d is the case D = H = 1
  * (spacial_ops/conv1d_op.mojo). x [N,C,D,H,W], w [K,C,T,R,S], bias [K] or null. -------------------- */
 typedef struct {
   int64_t N, C, D, H, W, K, T, R, S;

@@ -542,3 +542,18 @@ def test_conv1d(nd, golden):  # test_conv1d_op.mojo, plus gradients
     assert_close(x.grad().to_numpy(), g["dx_1d"], what="dx")
     assert_close(w.grad().to_numpy(), g["dw_1d"], what="dw")
     assert_close(b.grad().to_numpy(), g["db_1d"], what="db")
+
+
+@pytest.mark.parametrize("name", ["3d", "3d_unit"])
+def test_conv3d(nd, golden, name):  # test_conv3d_op.mojo, plus gradients
+    g = golden("convnd")
+    st, pad, dil = (tuple(int(v) for v in row) for row in g["cfg_" + name])
+    x, w, b = (nd.array(g[k + "_" + name], requires_grad=True) for k in ("x", "w", "b"))
+    y = nd.conv3d(x, w, b, st, pad, dil)
+    assert_close(y.to_numpy(), g["y_" + name], what="conv3d")
+    nd.sum(y * nd.array(g["g_" + name])).backward()
+    assert_close(x.grad().to_numpy(), g["dx_" + name], what="dx")
+    assert_close(w.grad().to_numpy(), g["dw_" + name], what="dw")
+    assert_close(b.grad().to_numpy(), g["db_" + name], what="db")
+    with pytest.raises(ValueError):
+        nd.conv3d(nd.zeros([1, 2, 3, 4]), w)

@@ -614,3 +614,45 @@ def test_pool_against_oracle(dev, xs, k, st, pad, dil):
         y, dx = _pool_run(dev, mode, x, gy, k, st, pad, dil)
         assert_close(y, want, tol=1e-6, what=mname)
         assert_close(dx, R.pool_bwd(mname, x, gy, k, st, pad, dil), tol=1e-6, what=mname + " grad")
+
+
+def _conv3d_desc(xs, ws, st, pad, dil):
+    d = L.Conv3dDesc()
+    d.N, d.C, d.D, d.H, d.W = xs
+    d.K, _, d.T, d.R, d.S = ws
+    d.stride[:], d.padding[:], d.dilation[:] = st, pad, dil
+    d.groups = 1
+    return d
+
+
+@pytest.mark.parametrize("xs,ws,st,pad,dil", [
+    ((2, 3, 6, 9, 8), (5, 3, 2, 3, 3), (1, 2, 1), (1, 1, 2), (2, 1, 1)),     # mixed strides and dilations: gather path
+    ((2, 4, 5, 6, 8), (3, 4, 3, 3, 3), (1, 1, 1), (1, 1, 1), (1, 1, 1)),     # all unit: padded-source path in every direction
+    ((1, 3, 7, 8, 9), (4, 3, 3, 2, 3), (2, 2, 2), (1, 0, 1), (1, 1, 1)),     # strided: gather path, data gradient with holes
+    ((2, 2, 4, 5, 12), (70, 2, 2, 2, 1), (1, 1, 1), (0, 1, 0), (1, 2, 1)),   # more than 64 output channels, width-1 kernel
+    ((1, 1, 3, 3, 3), (1, 1, 3, 3, 3), (1, 1, 1), (0, 0, 0), (1, 1, 1)),     # a single output position
+    ((2, 2, 3, 6, 8), (6, 2, 2, 2, 3), (1, 1, 1), (0, 0, 1), (1, 1, 1)),     # few taps, few channels: the 64 x 64 weight-gradient tile
+    ((1, 40, 3, 6, 8), (40, 40, 1, 3, 3), (1, 1, 1), (0, 1, 1), (1, 1, 1)),  # 33..64 channels: 64-row tiles
+])
+def test_conv3d_fwd_bwd(dev, xs, ws, st, pad, dil):
+    rng = np.random.default_rng(sum(xs) + sum(ws))
+    x = rng.standard_normal(xs).astype(np.float32)
+    w = (rng.standard_normal(ws) * 0.3).astype(np.float32)
+    b = rng.standard_normal(ws[0]).astype(np.float32)
+    want = R.convnd(x, w, b, st, pad, dil)
+    gy = rng.standard_normal(want.shape).astype(np.float32)
+    d = _conv3d_desc(xs, ws, st, pad, dil)
+    o = (ctypes.c_int64 * 3)()
+    dev.call("endia_hip_conv3d_out_shape", ctypes.byref(d), o)
+    assert tuple(o) == want.shape[2:]
+    dx_, dw_, db_, dg = dev.put(x), dev.put(w), dev.put(b), dev.put(gy)
+    dy, ddx, ddw, ddb = dev.alloc(want.nbytes), dev.alloc(x.nbytes), dev.alloc(w.nbytes), dev.alloc(b.nbytes)
+    dev.call("endia_hip_conv3d_fwd", ctypes.byref(d), dx_, dw_, db_, dy, L.OP_IDENTITY)
+    assert_close(dev.get(dy, want.shape), want, tol=1e-5, what="conv3d")
+    dev.call("endia_hip_conv3d_bwd_data", ctypes.byref(d), dg, dw_, ddx)
+    dev.call("endia_hip_conv3d_bwd_weight", ctypes.byref(d), dx_, dg, ddw)
+    dev.call("endia_hip_conv3d_bwd_bias", ctypes.byref(d), dg, ddb)
+    rdx, rdw, rdb = R.convnd_bwd(x, w, gy, st, pad, dil)
+    assert_close(dev.get(ddx, xs), rdx, tol=1e-5, what="conv3d dx")
+    assert_close(dev.get(ddw, ws), rdw, tol=1e-5, what="conv3d dw")
+    assert_close(dev.get(ddb, (ws[0],)), rdb, tol=1e-5, what="conv3d db")
