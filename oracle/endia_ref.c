@@ -11,15 +11,17 @@
  * Build: see oracle/Makefile (-O3, -ffp-contract=off so that no product-sum is fused).
  *
  * How each function is pinned (tests/test_oracle.py, no GPU needed):
- *   matmul (real, complex), binary ops + broadcast, unary ops and their VJPs, reduce_add, mse,
- *   conv2d forward, SGD, Adam and the full MLP step are compared with PyTorch float64 -- the oracle
+ *   matmul (real, complex), binary ops + broadcast (incl. pow and the comparisons), the 21 unary ops
+ *   and their VJPs, the complex unary bodies, reduce_add, mse, conv1d / conv2d / conv3d forward, max and
+ *   average pooling forward, SGD, Adam and the full MLP step are compared with PyTorch float64 -- the oracle
  *   the reference's own tests use (tests/test_endia/.../test_matmul_op.mojo:18-59 and siblings,
  *   metric endia/utils/array_conversions.mojo:63-135) -- with the doc known-answers
  *   (README.md:74-76,106-108; examples/custom_ops_examples/custom_mul.mojo:64-71) and with
- *   invariants (adjoint identities for the conv2d gradients, which the reference does not have).
+ *   invariants (adjoint identities for the convolution and pooling gradients, which the reference does
+ *   not have; torch autograd gives the same gradients).
  *   Parity unpinned by any reference test: complex matmul VJP without conjugation (pinned by
- *   reading matmul_op.mojo:278-283 only) and the conv2d gradients (absent from the reference,
- *   conv2d_op.mojo:198-200).
+ *   reading matmul_op.mojo:278-283 only), the convolution gradients (absent from the reference,
+ *   conv2d_op.mojo:198-200) and the pooling gradients (absent, max_pool2d_op.mojo:152-154).
  */
 #include <math.h>
 #include <stdint.h>

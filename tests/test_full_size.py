@@ -60,7 +60,7 @@ def test_adam_and_sgd_full_size_closed_form(dev):
 
 
 def test_wide_mlp_backward_matches_directional_derivative():
-    """BASELINE's wide configuration (batch 4096, 4096-wide layers, tanh, MSE; 4 of the 8 layers to keep the
+    """The wide benchmark configuration (batch 4096, 4096-wide layers, tanh, MSE; 4 of the 8 layers to keep the
     test short). <grad, v> from one backward pass must equal the central difference of the loss along v."""
     import endia_amd as nd
     rng = np.random.default_rng(102)
