@@ -22,7 +22,7 @@ FLAGS = [
     "--offload-arch=gfx950", "-O3", "-fPIC", "-std=c++17", "-fvisibility=hidden",
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
     "-Wno-unused-result", "-Wno-unused-command-line-argument",
-]
+] + os.environ.get("ENDIA_EXTRA_HIPCC_FLAGS", "").split()
 
 
 def sources():

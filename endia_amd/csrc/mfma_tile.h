@@ -48,39 +48,58 @@ __device__ __forceinline__ float buffer_load_f1(__amdgpu_buffer_rsrc_t rs, uint3
 // All MFMAs of one K tile. a_row / b_col: this lane's row of the A tile / column of the B tile for
 // block 0 (blocks are 32 apart); h = lane / 32.
 template <bool AK, bool BKM, int FM, int FN, int BM, int BN>
-__device__ __forceinline__ void compute_ktile(const float* __restrict__ As, const float* __restrict__ Bs, int a_row,
-                                              int b_col, int h, floatx16 (&acc)[FM][FN]) {
+__device__ __forceinline__ void load_fragments(const float* __restrict__ As, const float* __restrict__ Bs, int a_row, int b_col,
+                                               int h, int j, float (&af)[FM][4], float (&bf)[FN][4]) {
   constexpr int LDA = TileShape<AK, BM>::LD, LDB = TileShape<BKM, BN>::LD;
 #pragma unroll
-  for (int j = 0; j < BK / 8; ++j) {
-    float af[FM][4], bf[FN][4];
+  for (int f = 0; f < FM; ++f) {
+    if (AK) {
+      float4 t = *reinterpret_cast<const float4*>(&As[(a_row + 32 * f) * LDA + 8 * j + 4 * h]);
+      af[f][0] = t.x; af[f][1] = t.y; af[f][2] = t.z; af[f][3] = t.w;
+    } else {
 #pragma unroll
-    for (int f = 0; f < FM; ++f) {
-      if (AK) {
-        float4 t = *reinterpret_cast<const float4*>(&As[(a_row + 32 * f) * LDA + 8 * j + 4 * h]);
-        af[f][0] = t.x; af[f][1] = t.y; af[f][2] = t.z; af[f][3] = t.w;
-      } else {
-#pragma unroll
-        for (int i = 0; i < 4; ++i) af[f][i] = As[(8 * j + 4 * h + i) * LDA + a_row + 32 * f];
-      }
+      for (int i = 0; i < 4; ++i) af[f][i] = As[(8 * j + 4 * h + i) * LDA + a_row + 32 * f];
     }
+  }
 #pragma unroll
-    for (int f = 0; f < FN; ++f) {
-      if (BKM) {
-        float4 t = *reinterpret_cast<const float4*>(&Bs[(b_col + 32 * f) * LDB + 8 * j + 4 * h]);
-        bf[f][0] = t.x; bf[f][1] = t.y; bf[f][2] = t.z; bf[f][3] = t.w;
-      } else {
+  for (int f = 0; f < FN; ++f) {
+    if (BKM) {
+      float4 t = *reinterpret_cast<const float4*>(&Bs[(b_col + 32 * f) * LDB + 8 * j + 4 * h]);
+      bf[f][0] = t.x; bf[f][1] = t.y; bf[f][2] = t.z; bf[f][3] = t.w;
+    } else {
 #pragma unroll
-        for (int i = 0; i < 4; ++i) bf[f][i] = Bs[(8 * j + 4 * h + i) * LDB + b_col + 32 * f];
-      }
+      for (int i = 0; i < 4; ++i) bf[f][i] = Bs[(8 * j + 4 * h + i) * LDB + b_col + 32 * f];
     }
+  }
+}
+
+template <bool AK, bool BKM, int FM, int FN, int BM, int BN>
+__device__ __forceinline__ void compute_ktile(const float* __restrict__ As, const float* __restrict__ Bs, int a_row,
+                                              int b_col, int h, floatx16 (&acc)[FM][FN]) {
+  if constexpr (FM * FN == 1) {
+    // One MFMA block per wave leaves registers to spare: the fragments of all four step groups are
+    // fetched up front, so the LDS latency is paid once per K tile instead of once per group.
+    float af[4][FM][4], bf[4][FN][4];
 #pragma unroll
-    for (int i = 0; i < 4; ++i)
+    for (int j = 0; j < BK / 8; ++j) load_fragments<AK, BKM, FM, FN, BM, BN>(As, Bs, a_row, b_col, h, j, af[j], bf[j]);
 #pragma unroll
-      for (int fm = 0; fm < FM; ++fm)
+    for (int j = 0; j < BK / 8; ++j)
 #pragma unroll
-        for (int fn = 0; fn < FN; ++fn)
-          acc[fm][fn] = __builtin_amdgcn_mfma_f32_32x32x2f32(af[fm][i], bf[fn][i], acc[fm][fn], 0, 0, 0);
+      for (int i = 0; i < 4; ++i)
+        acc[0][0] = __builtin_amdgcn_mfma_f32_32x32x2f32(af[j][0][i], bf[j][0][i], acc[0][0], 0, 0, 0);
+  } else {
+#pragma unroll
+    for (int j = 0; j < BK / 8; ++j) {
+      float af[FM][4], bf[FN][4];
+      load_fragments<AK, BKM, FM, FN, BM, BN>(As, Bs, a_row, b_col, h, j, af, bf);
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int fm = 0; fm < FM; ++fm)
+#pragma unroll
+          for (int fn = 0; fn < FN; ++fn)
+            acc[fm][fn] = __builtin_amdgcn_mfma_f32_32x32x2f32(af[fm][i], bf[fn][i], acc[fm][fn], 0, 0, 0);
+    }
   }
 }
 
