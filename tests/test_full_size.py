@@ -129,3 +129,103 @@ def test_empty_inputs_are_noops(dev):
     assert nd.tanh(e).shape() == [0, 8]
     assert nd.reduce_add(e, [0]).to_numpy().tolist() == [[0.0] * 8]
     assert (e @ nd.zeros([8, 3])).shape() == [0, 3]
+
+
+def test_fused_program_full_size(dev):
+    """tanh(a * b + bias) and both of its gradients over 4096 x 4096 elements against numpy float64."""
+    import ctypes
+    rng = np.random.default_rng(102)
+    a = rng.standard_normal((N, N)).astype(np.float32)
+    b = rng.standard_normal((N, N)).astype(np.float32)
+    g = rng.standard_normal((N, N)).astype(np.float32)
+    bias = rng.standard_normal(N).astype(np.float32)
+    da, db_, dg, dbias = dev.put(a), dev.put(b), dev.put(g), dev.put(bias)
+    dy, d1, d2 = dev.alloc(a.nbytes), dev.alloc(a.nbytes), dev.alloc(a.nbytes)
+    I, S, M = L.EW_SRC_INPUT, L.EW_SRC_SLOT, L.EW_SRC_IMM
+
+    def run(ins, modes, outs, steps):
+        pin = (ctypes.c_void_p * len(ins))(*ins)
+        pm = (ctypes.c_int32 * len(ins))(*modes)
+        po = (ctypes.c_void_p * len(outs))(*outs)
+        arr = (L.EwStep * len(steps))(*[L.EwStep(*s) for s in steps])
+        dev.call("endia_hip_ew_program", N, N, len(ins), pin, pm, len(outs), po, len(steps), arr)
+
+    run([da, db_, dbias], [L.EW_FULL, L.EW_FULL, L.EW_ROW_VECTOR], [dy],
+        [(L.EW_LOAD, 0, I, 0, 0.0), (L.EW_BINARY, L.BIN_MUL, I, 1, 0.0), (L.EW_BINARY, L.BIN_ADD, I, 2, 0.0),
+         (L.EW_UNARY, L.OP_TANH, 0, 0, 0.0), (L.EW_STORE, 0, 0, 0, 0.0)])
+    z = a.astype(np.float64) * b + bias
+    y64 = np.tanh(z)
+    assert_close(dev.get(dy, (N, N)), y64, tol=1e-6, what="tanh(a*b+bias)")
+    # gradients from the stored output: t = (1 - y^2) * g; da = t * b; db = t * a
+    run([da, db_, dy, dg], [L.EW_FULL] * 4, [d1, d2],
+        [(L.EW_LOAD, 0, I, 2, 0.0), (L.EW_UNARY, L.OP_SQUARE, 0, 0, 0.0), (L.EW_RBINARY, L.BIN_SUB, M, 0, 1.0),
+         (L.EW_BINARY, L.BIN_MUL, I, 3, 0.0), (L.EW_SAVE, 0, 0, 0, 0.0), (L.EW_BINARY, L.BIN_MUL, I, 1, 0.0),
+         (L.EW_STORE, 0, 0, 0, 0.0), (L.EW_LOAD, 0, S, 0, 0.0), (L.EW_BINARY, L.BIN_MUL, I, 0, 0.0),
+         (L.EW_STORE, 0, 0, 1, 0.0)])
+    t = (1 - y64 * y64) * g
+    assert_close(dev.get(d1, (N, N)), t * b, tol=1e-5, what="d/da")
+    assert_close(dev.get(d2, (N, N)), t * a, tol=1e-5, what="d/db")
+
+
+def test_pooling_full_size_properties(dev):
+    """2x2 stride-2 pooling of a [64,128,56,56] array: forward against numpy, and size-independent properties of
+    the backward: average pooling is linear with <pool(x), g> = <x, pool_bwd(g)>; max pooling hands every output
+    gradient to exactly one input, so the sums agree and dx is zero wherever x is not its window's maximum."""
+    import ctypes
+    rng = np.random.default_rng(103)
+    shape = (64, 128, 56, 56)
+    x = rng.standard_normal(shape).astype(np.float32)
+    g = rng.standard_normal((64, 128, 28, 28)).astype(np.float32)
+    d = L.PoolDesc()
+    d.N, d.C, d.D, d.H, d.W = 64, 128, 1, 56, 56
+    d.kernel[:], d.stride[:], d.padding[:], d.dilation[:] = [1, 2, 2], [1, 2, 2], [0, 0, 0], [1, 1, 1]
+    dx_, dg = dev.put(x), dev.put(g)
+    dy, darg, ddx = dev.alloc(g.nbytes), dev.alloc(g.nbytes), dev.alloc(x.nbytes)
+    win = x.reshape(64, 128, 28, 2, 28, 2)
+    g64_ = g.astype(np.float64)
+    for mode, want in ((L.POOL_MAX, win.max(axis=(3, 5))), (L.POOL_AVG, win.astype(np.float64).mean(axis=(3, 5)))):
+        dev.call("endia_hip_pool_fwd", ctypes.byref(d), mode, dx_, dy, darg if mode == L.POOL_MAX else None)
+        y = dev.get(dy, g.shape)
+        assert_close(y, want, tol=1e-6, what="pool forward")
+        dev.call("endia_hip_pool_bwd", ctypes.byref(d), mode, dg, darg if mode == L.POOL_MAX else None, ddx)
+        dxv = dev.get(ddx, shape).astype(np.float64)
+        if mode == L.POOL_AVG:
+            lhs, rhs = np.vdot(y.astype(np.float64), g), np.vdot(x.astype(np.float64), dxv)
+            assert abs(lhs - rhs) <= 1e-6 * np.abs(y.astype(np.float64) * g).sum()
+            assert_close(dxv, np.repeat(np.repeat(g.astype(np.float64) / 4, 2, axis=2), 2, axis=3), tol=1e-6, what="avg grad")
+        else:
+            assert abs(dxv.sum() - g.astype(np.float64).sum()) <= 1e-6 * np.abs(g).sum()
+            is_max = x == np.repeat(np.repeat(want, 2, axis=2), 2, axis=3)
+            assert np.all(dxv[~is_max] == 0)
+            np.testing.assert_array_equal(dxv.reshape(64, 128, 28, 2, 28, 2).sum(axis=(3, 5)), g64_)
+
+
+def test_conv3d_full_size_properties(dev):
+    """conv3d at the benchmark shape (x [8,32,16,56,56], w [64,32,3,3,3], pad 1): adjoint identities
+    <conv(x,w), g> = <x, dX> = <w, dW>, db = sum of g, and a float64 probe of scattered output elements."""
+    import ctypes
+    rng = np.random.default_rng(104)
+    xs, ws = (8, 32, 16, 56, 56), (64, 32, 3, 3, 3)
+    x = rng.standard_normal(xs).astype(np.float32)
+    w = (rng.standard_normal(ws) * 0.05).astype(np.float32)
+    g = rng.standard_normal((8, 64, 16, 56, 56)).astype(np.float32)
+    d = L.Conv3dDesc()
+    d.N, d.C, d.D, d.H, d.W, d.K, d.T, d.R, d.S = 8, 32, 16, 56, 56, 64, 3, 3, 3
+    d.stride[:], d.padding[:], d.dilation[:], d.groups = [1, 1, 1], [1, 1, 1], [1, 1, 1], 1
+    dx_, dw_, dg = dev.put(x), dev.put(w), dev.put(g)
+    dy, ddx, ddw, ddb = dev.alloc(g.nbytes), dev.alloc(x.nbytes), dev.alloc(w.nbytes), dev.alloc(4 * 64)
+    dev.call("endia_hip_conv3d_fwd", ctypes.byref(d), dx_, dw_, None, dy, L.OP_IDENTITY)
+    dev.call("endia_hip_conv3d_bwd_data", ctypes.byref(d), dg, dw_, ddx)
+    dev.call("endia_hip_conv3d_bwd_weight", ctypes.byref(d), dx_, dg, ddw)
+    dev.call("endia_hip_conv3d_bwd_bias", ctypes.byref(d), dg, ddb)
+    y = dev.get(dy, g.shape)
+    g64 = g.astype(np.float64)
+    lhs = np.vdot(y.astype(np.float64), g64)
+    tol = 1e-5 * np.abs(y.astype(np.float64) * g64).sum()
+    assert abs(lhs - np.vdot(x.astype(np.float64), dev.get(ddx, xs))) <= tol
+    assert abs(lhs - np.vdot(w.astype(np.float64), dev.get(ddw, ws))) <= tol
+    assert_close(dev.get(ddb, (64,)), g64.sum(axis=(0, 2, 3, 4)), tol=1e-5, what="db")
+    xp = np.pad(x.astype(np.float64), ((0, 0), (0, 0), (1, 1), (1, 1), (1, 1)))
+    for n, k, z, r, c in [(0, 0, 0, 0, 0), (7, 63, 15, 55, 55), (3, 17, 8, 30, 1), (5, 40, 1, 0, 55), (2, 9, 15, 27, 28)]:
+        want = (xp[n, :, z:z + 3, r:r + 3, c:c + 3] * w[k].astype(np.float64)).sum()
+        assert abs(y[n, k, z, r, c] - want) <= 1e-4 * max(1.0, abs(want))
