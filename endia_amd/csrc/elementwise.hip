@@ -202,6 +202,31 @@ __global__ __launch_bounds__(TPB) void bin_general_kernel(BinDesc d, const float
   }
 }
 
+// 2-D op where one operand is a transposed view (element strides (1, ld)) and the other is
+// contiguous: the transposed operand goes through a 32 x 32 LDS tile so that its reads, the other
+// operand's reads and the writes all run along contiguous memory. (This is the shape of x + y.T(),
+// which a second backward pass produces whenever a weight is used through its transposed view.)
+template <int OP>
+__global__ __launch_bounds__(256) void bin_transposed_kernel(const float* __restrict__ full, const float* __restrict__ tr,
+                                                            float* __restrict__ o, int64_t rows, int64_t cols,
+                                                            int64_t ld_tr, int tr_is_lhs) {
+  __shared__ float t[32][33];
+  const int64_t c0 = (int64_t)blockIdx.x * 32, r0 = (int64_t)blockIdx.y * 32;
+  const int tx = threadIdx.x & 31, ty = threadIdx.x >> 5;
+  for (int k = ty; k < 32; k += 8) {  // tr[(r, c)] lives at c * ld_tr + r: walk r fastest
+    int64_t c = c0 + k, r = r0 + tx;
+    t[k][tx] = (c < cols && r < rows) ? tr[c * ld_tr + r] : 0.f;
+  }
+  __syncthreads();
+  for (int k = ty; k < 32; k += 8) {
+    int64_t r = r0 + k, c = c0 + tx;
+    if (r < rows && c < cols) {
+      float x = full[r * cols + c], y = t[tx][k];
+      o[r * cols + c] = tr_is_lhs ? bin_real(OP, y, x) : bin_real(OP, x, y);
+    }
+  }
+}
+
 __global__ __launch_bounds__(TPB) void axpby_kernel(int64_t n, float alpha, const float* __restrict__ a, float beta,
                                                     const float* __restrict__ b, float* __restrict__ o, int vec) {
   int64_t i = (int64_t)blockIdx.x * TPB + threadIdx.x;
@@ -412,7 +437,23 @@ int32_t endia_hip_binary(int32_t op, int32_t ndim, const int64_t* shape, const i
   };
   int am = classify(a_strides), bm = classify(b_strides);
   int rc = 0;
-  if (!is_complex && am == 0 && bm == 0 && al16(a) && al16(b) && al16(out)) {
+  // [R, C] with one operand contiguous and the other a transposed view
+  auto transposed = [&](const int64_t* st) {
+    return ndim == 2 && shape[0] > 1 && shape[1] > 1 && st[0] == 1 && st[1] >= shape[0];
+  };
+  if (!is_complex && ndim == 2 && ((am == 0 && transposed(b_strides)) || (bm == 0 && transposed(a_strides))) &&
+      ceil_div64(shape[0], 32) <= 65535) {
+    const bool tr_is_lhs = am != 0;
+    const float* full = tr_is_lhs ? b : a;
+    const float* tr = tr_is_lhs ? a : b;
+    const int64_t ld = tr_is_lhs ? a_strides[1] : b_strides[1];
+    dim3 grid((unsigned)ceil_div64(shape[1], 32), (unsigned)ceil_div64(shape[0], 32));
+    rc = dispatch_binary(op, [&](auto tag) {
+      constexpr int OP = decltype(tag)::value;
+      hipLaunchKernelGGL((bin_transposed_kernel<OP>), grid, dim3(256), 0, s, full, tr, out, shape[0], shape[1], ld,
+                         tr_is_lhs ? 1 : 0);
+    });
+  } else if (!is_complex && am == 0 && bm == 0 && al16(a) && al16(b) && al16(out)) {
     rc = dispatch_binary(op, [&](auto tag) {
       constexpr int OP = decltype(tag)::value;
       hipLaunchKernelGGL((bin_flat_kernel<OP>), dim3(stream_grid((n + 3) / 4)), dim3(TPB), 0, s, a, b, out, n);

@@ -656,3 +656,21 @@ def test_conv3d_fwd_bwd(dev, xs, ws, st, pad, dil):
     assert_close(dev.get(ddx, xs), rdx, tol=1e-5, what="conv3d dx")
     assert_close(dev.get(ddw, ws), rdw, tol=1e-5, what="conv3d dw")
     assert_close(dev.get(ddb, (ws[0],)), rdb, tol=1e-5, what="conv3d db")
+
+
+@pytest.mark.parametrize("rows,cols,ld", [(37, 50, 37), (64, 64, 64), (100, 33, 128), (2048, 96, 2048)])
+def test_binary_with_transposed_view(dev, rows, cols, ld):
+    """x op y.T() and y.T() op x, where y.T() is a stride-(1, ld) view of a [cols, ld] buffer (the case that the
+    gradient accumulation of a transposed weight view produces)."""
+    rng = np.random.default_rng(rows + cols)
+    full = rng.standard_normal((rows, cols)).astype(np.float32)
+    base = (np.abs(rng.standard_normal((cols, ld))) + 0.5).astype(np.float32)
+    view = base[:, :rows].T  # shape [rows, cols], element strides (1, ld)
+    dfull, dbase, dout = dev.put(full), dev.put(base), dev.alloc(full.nbytes)
+    shape = L.i64_array([rows, cols])
+    s_full, s_view = L.i64_array([cols, 1]), L.i64_array([1, ld])
+    for name, code in [("add", L.BIN_ADD), ("sub", L.BIN_SUB), ("div", L.BIN_DIV), ("greater", L.BIN_GREATER)]:
+        dev.call("endia_hip_binary", code, 2, shape, s_full, s_view, dfull, dbase, dout, 0)
+        np.testing.assert_array_equal(dev.get(dout, (rows, cols)), R.binary(name, full, view), err_msg=name)
+        dev.call("endia_hip_binary", code, 2, shape, s_view, s_full, dbase, dfull, dout, 0)
+        np.testing.assert_array_equal(dev.get(dout, (rows, cols)), R.binary(name, view, full), err_msg=name + " reversed")
