@@ -243,13 +243,10 @@ extern "C" int32_t endia_hip_cgemm(int32_t transA, int32_t conjA, int32_t transB
                            conjB ? -1.f : 1.f, Br, Bi, B3);
       ENDIA_LAUNCH_CHECK();
     }
-    auto mm = [&](const float* X, const float* Y, float* Z) {
-      return sgemm_impl(transA, transB, M, N, K, X, a_cols, Y, b_cols, Z, N, 1, 0, 0, 0, ENDIA_EPI_NONE, ENDIA_OP_IDENTITY,
-                        nullptr, nullptr, nullptr);
-    };
-    if ((rc = mm(Ar, Br, P0))) return rc;
-    if ((rc = mm(Ai, Bi, P1))) return rc;
-    if ((rc = mm(A3, B3, P2))) return rc;
+    // the three products are independent: one batched launch (the planes are na / nb / nc floats apart)
+    rc = sgemm_impl(transA, transB, M, N, K, Ar, a_cols, Br, b_cols, P0, N, 3, na, nb, nc, ENDIA_EPI_NONE, ENDIA_OP_IDENTITY,
+                    nullptr, nullptr, nullptr);
+    if (rc) return rc;
     hipLaunchKernelGGL(join_kernel, dim3(grid_for(M * N)), dim3(TPB), 0, s, Cb, M, N, ldc, P0, P1, P2, accumulate ? 1 : 0);
     ENDIA_LAUNCH_CHECK();
   }
