@@ -9,11 +9,16 @@
 //   3M:  T1 = Ar Br, T2 = Ai Bi, T3 = (Ar+Ai)(Br+Bi) ;  Cr = T1 - T2 ;  Ci = T3 - T1 - T2
 // 3M does 6 MNK flops instead of 8 MNK but its imaginary part is a difference of larger numbers,
 // so its rounding error is larger than 4M's.
-// 4M runs as ONE real GEMM of shape M x 2N x 2K on the real embedding of the operands,
-//   [Cr | Ci] = [Ar | Ai] . [[Br, Bi], [-Bi, Br]],
-// which is the same four products with the two sums of each output taken inside one K loop. One
-// launch with twice the reduction length and twice the tiles keeps the matrix pipe busier than four
-// launches of M x N x K (2048^3: 0.53 ms against 0.56 ms).
+// 4M runs as ONE real GEMM of shape M x 2N x 2K on the real embedding of the right operand: an
+// interleaved complex matrix IS a real matrix with twice the columns, and with
+//   E(B)[2k  , 2n..2n+1] = ( Br[k,n], Bi[k,n])       (row k of B as stored)
+//   E(B)[2k+1, 2n..2n+1] = (-Bi[k,n], Br[k,n])       (row k of i*B)
+// the real product  A_real (M x 2K) . E(B) (2K x 2N)  is C as stored, interleaved: the same four
+// products, the two sums of each output taken inside one K loop. So a non-transposed A is used in
+// place, C is written (or accumulated) in place by the GEMM epilogue, and only B is rewritten. A
+// transposed A is copied into stacked planes [Re ; Im] (2K x M) and E(B) orders its rows to match.
+// One launch with twice the reduction length and twice the tiles also keeps the matrix pipe busier
+// than four launches of M x N x K (2048^3: 0.50 ms against 0.56 ms).
 #include "common.h"
 
 namespace endia {
@@ -44,77 +49,43 @@ __global__ __launch_bounds__(TPB) void split_kernel(const float2* __restrict__ s
   }
 }
 
-// The three kernels below move PAIRS of complex elements (16 bytes in, 8 bytes per plane out); `cols` is the
-// number of complex columns and must be even for the pair form (PAIR = 2), else PAIR = 1.
-
-// Real embedding of the left operand. src: rows x cols complex (row stride ld). Not transposed (rows = M,
-// cols = K): out is M x 2K, row r = [Re row | sign*Im row]. Transposed (rows = K, cols = M): out is 2K x M,
-// the Re plane followed by the sign*Im plane. Either way the real GEMM sees op(A) as M x 2K.
-template <int PAIR>
-__global__ __launch_bounds__(TPB) void embed_a_kernel(const float* __restrict__ src, int64_t rows, int64_t cols, int64_t ld,
-                                                      float sign, int trans, float* __restrict__ out) {
-  const int64_t cp = cols / PAIR, n = rows * cp, stride = (int64_t)gridDim.x * TPB;
+// Left operand used through its transpose (src: K rows x M cols complex): out is 2K x M real, the Re plane
+// followed by the Im plane, so that the real GEMM sees op(A) as M x 2K with k order (all Re, all Im).
+__global__ __launch_bounds__(TPB) void stack_planes_kernel(const float2* __restrict__ src, int64_t rows, int64_t cols, int64_t ld,
+                                                           float* __restrict__ out) {
+  const int64_t n = rows * cols, stride = (int64_t)gridDim.x * TPB;
   for (int64_t j = (int64_t)blockIdx.x * TPB + threadIdx.x; j < n; j += stride) {
-    const int64_t r = j / cp, c = (j - r * cp) * PAIR;
-    float re[PAIR], im[PAIR];
-    if (PAIR == 2) {
-      const float4 z = *reinterpret_cast<const float4*>(src + 2 * (r * ld + c));
-      re[0] = z.x; im[0] = sign * z.y; re[PAIR - 1] = z.z; im[PAIR - 1] = sign * z.w;
-    } else {
-      const float2 z = *reinterpret_cast<const float2*>(src + 2 * (r * ld + c));
-      re[0] = z.x; im[0] = sign * z.y;
-    }
-    float* o_re = trans ? out + r * cols + c : out + r * 2 * cols + c;
-    float* o_im = trans ? out + (rows + r) * cols + c : out + r * 2 * cols + cols + c;
-#pragma unroll
-    for (int e = 0; e < PAIR; ++e) { o_re[e] = re[e]; o_im[e] = im[e]; }
+    const int64_t r = j / cols, c = j - r * cols;
+    const float2 z = src[r * ld + c];
+    out[j] = z.x;
+    out[n + j] = z.y;
   }
 }
 
-// Real embedding of the right operand. src: rows x cols complex. out is 2*rows x 2*cols (row stride 2*cols):
-//   not transposed (rows = K, cols = N):  [[Br, Bi], [-Bi, Br]]
-//   transposed     (rows = N, cols = K):  its transpose [[Br^T, -Bi^T], [Bi^T, Br^T]] in the stored orientation
-// with Bi = sign * Im.
-template <int PAIR>
-__global__ __launch_bounds__(TPB) void embed_b_kernel(const float* __restrict__ src, int64_t rows, int64_t cols, int64_t ld,
-                                                      float sign, int trans, float* __restrict__ out) {
-  const int64_t cp = cols / PAIR, n = rows * cp, stride = (int64_t)gridDim.x * TPB;
+// Real embedding E(op(B)) of the right operand, in the orientation B is stored in.
+//   src: rows x cols complex; bsign = -1 conjugates B; asign = -1 stands for a conjugated A (it negates the
+//   rows that multiply Im A). `blocked`: k order (all Re, all Im) to match stack_planes_kernel, else (Re, Im) pairs.
+//   not transposed (rows = K, cols = N): out is 2K x 2N, out[row(k,0)] = (Br, Bi) pairs, out[row(k,1)] = asign * (-Bi, Br)
+//   transposed     (rows = N, cols = K): out is 2N x 2K (the transpose of the above):
+//                  out[2n][col(k,0)] = Br, out[2n][col(k,1)] = -asign*Bi, out[2n+1][col(k,0)] = Bi, out[2n+1][col(k,1)] = asign*Br
+__global__ __launch_bounds__(TPB) void embed_b_kernel(const float2* __restrict__ src, int64_t rows, int64_t cols, int64_t ld,
+                                                      float bsign, float asign, int trans, int blocked, float* __restrict__ out) {
+  const int64_t n = rows * cols, stride = (int64_t)gridDim.x * TPB;
   const int64_t ldo = 2 * cols;
-  const float up = trans ? -sign : sign;  // sign of Im in the upper right block; the lower left takes the opposite
   for (int64_t j = (int64_t)blockIdx.x * TPB + threadIdx.x; j < n; j += stride) {
-    const int64_t r = j / cp, c = (j - r * cp) * PAIR;
-    float re[PAIR], im[PAIR];
-    if (PAIR == 2) {
-      const float4 z = *reinterpret_cast<const float4*>(src + 2 * (r * ld + c));
-      re[0] = z.x; im[0] = z.y; re[PAIR - 1] = z.z; im[PAIR - 1] = z.w;
-    } else {
-      const float2 z = *reinterpret_cast<const float2*>(src + 2 * (r * ld + c));
-      re[0] = z.x; im[0] = z.y;
-    }
-#pragma unroll
-    for (int e = 0; e < PAIR; ++e) {
-      out[r * ldo + c + e] = re[e];
-      out[r * ldo + cols + c + e] = up * im[e];
-      out[(rows + r) * ldo + c + e] = -up * im[e];
-      out[(rows + r) * ldo + cols + c + e] = re[e];
-    }
-  }
-}
-
-// [Cr | Ci] (rows x 2*cols) -> interleaved complex
-template <int PAIR>
-__global__ __launch_bounds__(TPB) void join_embedded_kernel(float* __restrict__ dst, int64_t rows, int64_t cols, int64_t ld,
-                                                            const float* __restrict__ p, int accumulate) {
-  const int64_t cp = cols / PAIR, n = rows * cp, stride = (int64_t)gridDim.x * TPB;
-  for (int64_t j = (int64_t)blockIdx.x * TPB + threadIdx.x; j < n; j += stride) {
-    const int64_t r = j / cp, c = (j - r * cp) * PAIR;
-    float* d = dst + 2 * (r * ld + c);
-#pragma unroll
-    for (int e = 0; e < PAIR; ++e) {
-      float re = p[r * 2 * cols + c + e], im = p[r * 2 * cols + cols + c + e];
-      if (accumulate) { re += d[2 * e]; im += d[2 * e + 1]; }
-      d[2 * e] = re;
-      d[2 * e + 1] = im;
+    const int64_t r = j / cols, c = j - r * cols;
+    const float2 z = src[r * ld + c];
+    const float br = z.x, bi = bsign * z.y;
+    if (!trans) {  // r = k, c = n
+      const int64_t row0 = blocked ? r : 2 * r, row1 = blocked ? rows + r : 2 * r + 1;
+      *reinterpret_cast<float2*>(out + row0 * ldo + 2 * c) = make_float2(br, bi);
+      *reinterpret_cast<float2*>(out + row1 * ldo + 2 * c) = make_float2(-asign * bi, asign * br);
+    } else {       // r = n, c = k
+      const int64_t col0 = blocked ? c : 2 * c, col1 = blocked ? cols + c : 2 * c + 1;
+      out[(2 * r) * ldo + col0] = br;
+      out[(2 * r) * ldo + col1] = -asign * bi;
+      out[(2 * r + 1) * ldo + col0] = bi;
+      out[(2 * r + 1) * ldo + col1] = asign * br;
     }
   }
 }
@@ -168,48 +139,29 @@ extern "C" int32_t endia_hip_cgemm(int32_t transA, int32_t conjA, int32_t transB
   const int three_m = algo == ENDIA_CGEMM_3M;
 
   if (!three_m) {
-    // one real GEMM on the embedded operands
-    const int64_t na = pad4(2 * M * K), nb = pad4(4 * K * N), nc = pad4(2 * M * N);
+    // one real GEMM: A as stored (or its stacked planes), the embedded B, C written in place
+    const int64_t na = transA ? pad4(2 * M * K) : 0, nb = pad4(4 * K * N);
     void* ws = nullptr;
-    int32_t rc = workspace((na + nb + nc) * (int64_t)sizeof(float), &ws);
+    int32_t rc = workspace((na + nb) * (int64_t)sizeof(float), &ws);
     if (rc) return rc;
     float* Ae = static_cast<float*>(ws);
     float* Be = Ae + na;
-    float* Ce = Be + nb;
     for (int64_t b = 0; b < batch; ++b) {
       const float2* Ab = reinterpret_cast<const float2*>(A) + b * strideA;
       const float2* Bb = reinterpret_cast<const float2*>(B) + b * strideB;
-      float2* Cb = reinterpret_cast<float2*>(C) + b * strideC;
+      float* Cb = C + 2 * b * strideC;
       if (K > 0) {
-        // pairs of complex elements need 16-byte aligned rows on the source side
-        const bool pa = a_cols % 2 == 0 && lda % 2 == 0 && (reinterpret_cast<uintptr_t>(Ab) & 15) == 0;
-        const bool pb = b_cols % 2 == 0 && ldb % 2 == 0 && (reinterpret_cast<uintptr_t>(Bb) & 15) == 0;
-        const float* Af = reinterpret_cast<const float*>(Ab);
-        const float* Bf = reinterpret_cast<const float*>(Bb);
-        if (b == 0 || strideA != 0) {  // operands that broadcast over the batch are embedded once
-          if (pa) hipLaunchKernelGGL((embed_a_kernel<2>), dim3(grid_for(M * K / 2)), dim3(TPB), 0, s, Af, a_rows, a_cols, lda,
-                                     conjA ? -1.f : 1.f, transA ? 1 : 0, Ae);
-          else hipLaunchKernelGGL((embed_a_kernel<1>), dim3(grid_for(M * K)), dim3(TPB), 0, s, Af, a_rows, a_cols, lda,
-                                  conjA ? -1.f : 1.f, transA ? 1 : 0, Ae);
-        }
-        if (b == 0 || strideB != 0) {
-          if (pb) hipLaunchKernelGGL((embed_b_kernel<2>), dim3(grid_for(K * N / 2)), dim3(TPB), 0, s, Bf, b_rows, b_cols, ldb,
-                                     conjB ? -1.f : 1.f, transB ? 1 : 0, Be);
-          else hipLaunchKernelGGL((embed_b_kernel<1>), dim3(grid_for(K * N)), dim3(TPB), 0, s, Bf, b_rows, b_cols, ldb,
-                                  conjB ? -1.f : 1.f, transB ? 1 : 0, Be);
-        }
+        if (transA && (b == 0 || strideA != 0))  // operands that broadcast over the batch are prepared once
+          hipLaunchKernelGGL(stack_planes_kernel, dim3(grid_for(M * K)), dim3(TPB), 0, s, Ab, a_rows, a_cols, lda, Ae);
+        if (b == 0 || strideB != 0)
+          hipLaunchKernelGGL(embed_b_kernel, dim3(grid_for(K * N)), dim3(TPB), 0, s, Bb, b_rows, b_cols, ldb,
+                             conjB ? -1.f : 1.f, conjA ? -1.f : 1.f, transB ? 1 : 0, transA ? 1 : 0, Be);
         ENDIA_LAUNCH_CHECK();
       }
-      rc = sgemm_impl(transA, transB, M, 2 * N, 2 * K, Ae, transA ? M : 2 * K, Be, 2 * b_cols, Ce, 2 * N, 1, 0, 0, 0,
-                      ENDIA_EPI_NONE, ENDIA_OP_IDENTITY, nullptr, nullptr, nullptr);
+      const float* Ar = transA ? Ae : reinterpret_cast<const float*>(Ab);
+      rc = sgemm_impl(transA, transB, M, 2 * N, 2 * K, Ar, transA ? M : 2 * lda, Be, 2 * b_cols, Cb, 2 * ldc, 1, 0, 0, 0,
+                      ENDIA_EPI_NONE | (accumulate ? ENDIA_GEMM_ACCUMULATE : 0), ENDIA_OP_IDENTITY, nullptr, nullptr, nullptr);
       if (rc) return rc;
-      if (N % 2 == 0)
-        hipLaunchKernelGGL((join_embedded_kernel<2>), dim3(grid_for(M * N / 2)), dim3(TPB), 0, s, reinterpret_cast<float*>(Cb), M, N,
-                           ldc, Ce, accumulate ? 1 : 0);
-      else
-        hipLaunchKernelGGL((join_embedded_kernel<1>), dim3(grid_for(M * N)), dim3(TPB), 0, s, reinterpret_cast<float*>(Cb), M, N,
-                           ldc, Ce, accumulate ? 1 : 0);
-      ENDIA_LAUNCH_CHECK();
     }
     return ENDIA_HIP_OK;
   }

@@ -163,3 +163,34 @@ def test_sgemm_large_properties(dev):
         got = C.astype(np.float64).sum()
         assert abs(got - total) <= 1e-4 * np.abs(opA).astype(np.float64).sum(0) @ np.abs(opB).astype(np.float64).sum(1)
         dev.release()
+
+
+@pytest.mark.parametrize("algo", [L.CGEMM_4M, L.CGEMM_3M])
+@pytest.mark.parametrize("M,N,K,pad", [(96, 72, 40, 0), (64, 128, 64, 4), (33, 21, 17, 3)])
+def test_cgemm_all_flag_combinations(dev, algo, M, N, K, pad):
+    """Every transpose / conjugate combination, leading dimensions larger than the rows, accumulation into C,
+    sizes that take the aligned MFMA path and sizes that take the unaligned one."""
+    rng = np.random.default_rng(M + N + K)
+
+    def cplx(*shape):
+        return (rng.standard_normal(shape) + 1j * rng.standard_normal(shape)).astype(np.complex64)
+
+    for ta in (0, 1):
+        for ca in (0, 1):
+            for tb in (0, 1):
+                for cb in (0, 1):
+                    a_shape = (K, M) if ta else (M, K)
+                    b_shape = (N, K) if tb else (K, N)
+                    Ap, Bp, Cp = cplx(a_shape[0], a_shape[1] + pad), cplx(b_shape[0], b_shape[1] + pad), cplx(M, N + pad)
+                    A, B, C0 = Ap[:, :a_shape[1]], Bp[:, :b_shape[1]], Cp[:, :N]
+                    dA, dB, dC = dev.put(Ap), dev.put(Bp), dev.put(Cp)
+                    opA = np.conj(A.T if ta else A) if ca else (A.T if ta else A)
+                    opB = np.conj(B.T if tb else B) if cb else (B.T if tb else B)
+                    want = opA.astype(np.complex128) @ opB.astype(np.complex128)
+                    dev.call("endia_hip_cgemm", ta, ca, tb, cb, M, N, K, dA, Ap.shape[1], dB, Bp.shape[1], dC, N + pad,
+                             1, 0, 0, 0, algo, 1)
+                    got = dev.get(dC, Cp.shape, np.complex64)
+                    what = "ta=%d ca=%d tb=%d cb=%d" % (ta, ca, tb, cb)
+                    assert_close(got[:, :N], want + C0, what=what)
+                    np.testing.assert_array_equal(got[:, N:], Cp[:, N:], err_msg=what + ": padding columns of C touched")
+                    dev.release()
