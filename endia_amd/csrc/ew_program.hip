@@ -239,7 +239,11 @@ extern "C" int32_t endia_hip_ew_program(int64_t rows, int64_t cols, int32_t n_in
     ENDIA_CHECK_ARG(inputs[i] != nullptr || a.n == 0, "endia_hip_ew_program: input %d is null", i);
     a.in[i] = inputs[i];
     a.mode[i] = input_modes[i];
-    if (input_modes[i] == ENDIA_EW_ROW_VECTOR) a.need_col = 1;
+    if (input_modes[i] == ENDIA_EW_ROW_VECTOR) {
+      a.need_col = 1;
+      if (cols >= (1ll << 31))
+        return fail(ENDIA_HIP_ERR_UNSUPPORTED, "endia_hip_ew_program: a row-vector input with 2^31 columns or more");
+    }
     if (input_modes[i] != ENDIA_EW_SCALAR && (reinterpret_cast<uintptr_t>(inputs[i]) & 15)) vec = false;
   }
   for (int i = 0; i < n_outputs; ++i) {

@@ -216,6 +216,34 @@ __global__ __launch_bounds__(256) void sgemm_generic_kernel(GemmArgs p, int tran
     }
 }
 
+// A product with very few outputs and a long reduction (the weight gradient of a 1-wide layer over a
+// batch: 32 outputs, K = 128) is bound by memory latency in any tiled kernel, whose K loop is a chain
+// of dependent load -> LDS -> barrier rounds. Here one 128-thread group owns one output element: every
+// thread issues all its loads at once, and the partial sums meet in a wave shuffle and an LDS add.
+__global__ __launch_bounds__(128) void sgemm_skinny_kernel(GemmArgs p, int transA, int transB) {
+  __shared__ float red[2];
+  const int out = blockIdx.x;
+  const int m = out / p.N, n = out - m * p.N;
+  const int64_t bz = blockIdx.y;
+  const float* __restrict__ A = p.A + bz * p.sA;
+  const float* __restrict__ B = p.B + bz * p.sB;
+  float acc = 0.f;
+  for (int k = threadIdx.x; k < p.K; k += 128) {
+    const float a = transA ? A[(int64_t)k * p.lda + m] : A[(int64_t)m * p.lda + k];
+    const float b = transB ? B[(int64_t)n * p.ldb + k] : B[(int64_t)k * p.ldb + n];
+    acc = fmaf(a, b, acc);
+  }
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) acc += __shfl_down(acc, off, 64);
+  if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = acc;
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    float* c = p.C + bz * p.sC + (int64_t)m * p.ldc + n;
+    const float v = red[0] + red[1];
+    *c = p.accumulate ? *c + v : v;
+  }
+}
+
 template <int EPI, int F>
 void launch_mfma(const GemmArgs& p, int transA, int transB, dim3 grid, hipStream_t s) {
   const bool ak = !transA, bk = transB != 0;
@@ -365,6 +393,9 @@ int32_t sgemm_impl(int transA, int transB, int64_t M, int64_t N, int64_t K, cons
       ENDIA_LAUNCH_CHECK();
       return col_reduce(1, splits, M * N, p.C, C_final, 1.f);  // partials added in slice order
     }
+  } else if (epi == ENDIA_EPI_NONE && M * N <= 2048 && K >= 64) {
+    p.k_split = 0;
+    hipLaunchKernelGGL(sgemm_skinny_kernel, dim3((unsigned)(M * N), (unsigned)batch), dim3(128), 0, s, p, transA, transB);
   } else {
     p.k_split = 0;
     p.tiles_m = (int)ceil_div64(M, 64);

@@ -88,6 +88,24 @@ __global__ __launch_bounds__(TPB) void sgd_kernel(int64_t n, float* __restrict__
   }
 }
 
+// Plain SGD over several parameter tensors in one launch (blockIdx.y picks the tensor). A model of many
+// small tensors is bound by launch latency, not bandwidth: the reference's sine-fit MLP has 16 of them.
+constexpr int MULTI_MAX = 32;
+struct SgdMulti {
+  float* p[MULTI_MAX];
+  const float* g[MULTI_MAX];
+  int64_t n[MULTI_MAX];
+};
+
+__global__ __launch_bounds__(TPB) void sgd_multi_kernel(SgdMulti t, float lr) {
+  const int k = blockIdx.y;
+  float* __restrict__ p = t.p[k];
+  const float* __restrict__ g = t.g[k];
+  const int64_t n = t.n[k];
+  const int64_t stride = (int64_t)gridDim.x * TPB;
+  for (int64_t j = (int64_t)blockIdx.x * TPB + threadIdx.x; j < n; j += stride) p[j] = sgd_one(p[j], g[j], lr);
+}
+
 // kind: 0 = SGD with momentum / weight decay, 1 = Adagrad, 2 = RMSprop. `s` is the state tensor (velocity or cache).
 struct OptK {
   int kind;
@@ -180,6 +198,31 @@ int32_t endia_hip_sgd_step(int64_t n, float* p, const float* g, float lr) {
   int vec = al16(p) && al16(g);
   hipLaunchKernelGGL(sgd_kernel, dim3(stream_grid(vec ? (n + 3) / 4 : n)), dim3(TPB), 0, ctx().stream, n, p, g, lr, vec);
   ENDIA_LAUNCH_CHECK();
+  return ENDIA_HIP_OK;
+}
+
+int32_t endia_hip_sgd_step_multi(int32_t count, const int64_t* n, float* const* p, const float* const* g, float lr) {
+  ENDIA_REQUIRE_INIT();
+  ENDIA_CHECK_ARG(count >= 0, "endia_hip_sgd_step_multi: negative count");
+  if (count == 0) return ENDIA_HIP_OK;
+  ENDIA_CHECK_ARG(n && p && g, "endia_hip_sgd_step_multi: null table");
+  for (int32_t first = 0; first < count; first += MULTI_MAX) {
+    const int32_t m = count - first < MULTI_MAX ? count - first : MULTI_MAX;
+    SgdMulti t = {};
+    int64_t largest = 0;
+    for (int32_t i = 0; i < m; ++i) {
+      ENDIA_CHECK_ARG(n[first + i] >= 0, "endia_hip_sgd_step_multi: tensor %d has a negative size", first + i);
+      ENDIA_CHECK_ARG(n[first + i] == 0 || (p[first + i] && g[first + i]), "endia_hip_sgd_step_multi: tensor %d has a null pointer",
+                      first + i);
+      t.p[i] = p[first + i];
+      t.g[i] = g[first + i];
+      t.n[i] = n[first + i];
+      if (t.n[i] > largest) largest = t.n[i];
+    }
+    if (largest == 0) continue;
+    hipLaunchKernelGGL(sgd_multi_kernel, dim3((unsigned)stream_grid(largest), (unsigned)m), dim3(TPB), 0, ctx().stream, t, lr);
+    ENDIA_LAUNCH_CHECK();
+  }
   return ENDIA_HIP_OK;
 }
 

@@ -216,6 +216,14 @@ int32_t col_reduce(int64_t batch, int64_t R, int64_t C, const float* x, float* o
   const int64_t col_tiles = ceil_div64(C, 256);
   if (col_tiles * 1 > 2147483647ll || batch > 65535)
     return fail(ENDIA_HIP_ERR_UNSUPPORTED, "col_reduce: extent too large");
+  // A small input (the bias gradient of a narrow layer) is one launch: the second-stage kernel applied to the
+  // input itself, 64 columns per group, the four waves taking alternate rows.
+  if (R <= 1024 && batch * R * C <= (1 << 20)) {
+    hipLaunchKernelGGL(col_reduce_final_kernel, dim3((unsigned)ceil_div64(C, 64), (unsigned)batch), dim3(TPB), 0, s, x, out, R,
+                       C, batch, scale);
+    ENDIA_LAUNCH_CHECK();
+    return ENDIA_HIP_OK;
+  }
   // enough row splits for ~4 groups per CU, at least 16 rows each
   int64_t want = (int64_t)ctx().cu_count * 4;
   int64_t S = want / (col_tiles * batch);
@@ -244,6 +252,11 @@ int32_t col_reduce(int64_t batch, int64_t R, int64_t C, const float* x, float* o
 int32_t row_reduce(int64_t R, int64_t C, const float* x, float* out, float scale) {
   hipStream_t s = ctx().stream;
   if (R > 65535) return fail(ENDIA_HIP_ERR_UNSUPPORTED, "row_reduce: more than 65535 rows");
+  if (C <= 4096 && R * C <= (1 << 20)) {  // small input: one wave per row, one launch
+    hipLaunchKernelGGL(row_reduce_final_kernel, dim3((unsigned)ceil_div64(R, 4)), dim3(TPB), 0, s, x, out, R, C, scale);
+    ENDIA_LAUNCH_CHECK();
+    return ENDIA_HIP_OK;
+  }
   int64_t want = (int64_t)ctx().cu_count * 8;
   int64_t S = want / R;
   if (S < 1) S = 1;

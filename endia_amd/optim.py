@@ -31,6 +31,18 @@ class SGD:
         self.velocity = [Array(p.shape()) for p in self.params] if self.momentum > 0 else []
 
     def step(self):
+        if self.momentum == 0 and self.weight_decay == 0 and len(self.params) > 1:
+            # plain SGD: every parameter tensor in one launch
+            import ctypes
+            grads = [_flat_grad(p) for p in self.params]
+            k = len(self.params)
+            assert all(p.is_contiguous() for p in self.params)
+            L.call("endia_hip_sgd_step_multi", k, L.i64_array([p.size() for p in self.params]),
+                   (ctypes.c_void_p * k)(*[p.data_ptr() for p in self.params]),
+                   (ctypes.c_void_p * k)(*[g.data_ptr() for g in grads]), self.lr)
+            for p in self.params:
+                p.clear_args()
+            return
         for i, p in enumerate(self.params):
             g = _flat_grad(p)
             assert p.is_contiguous()

@@ -305,6 +305,9 @@ ENDIA_API int32_t endia_hip_pool_bwd(const endia_hip_pool_desc* desc, int32_t mo
 /* ---- optimizers: SGD.step plain path (optim/sgd.mojo:61-62) and Adam.step (optim/adam.mojo:47-65),
  *      each as one pass over the parameter. t is Adam's fp32 step counter (starts at 1, adam.mojo:40). */
 ENDIA_API int32_t endia_hip_sgd_step(int64_t n, float* p, const float* g, float lr);
+/* The same update for `count` parameter tensors in one launch (n, p, g are host arrays of length count): a model
+ * of many small tensors, like the reference's sine-fit MLP, is bound by launch latency rather than bandwidth. */
+ENDIA_API int32_t endia_hip_sgd_step_multi(int32_t count, const int64_t* n, float* const* p, const float* const* g, float lr);
 /* SGD with momentum and / or weight decay (optim/sgd.mojo:42-60): vel = momentum*vel - lr*(g + wd*p); p += vel
  * (without momentum: p -= lr*(g + wd*p); vel may then be null). Adagrad (optim/adagrad.mojo:36-45):
  * cache += g*g; p -= lr*g / (sqrt(cache) + eps). RMSprop (optim/rmsprop.mojo:39-53):

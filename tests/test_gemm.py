@@ -27,7 +27,8 @@ def run_sgemm(dev, A, B, ta, tb, M, N, K, epi=L.EPI_NONE, act=L.OP_IDENTITY, bia
 
 
 SHAPES = [(128, 128, 32), (256, 384, 72), (132, 260, 100), (37, 53, 19), (4, 4, 4), (1, 1, 1), (128, 1, 32),
-          (1, 32, 128), (300, 200, 8), (64, 64, 1024), (64, 96, 8192), (128, 200, 5000), (72, 64, 2052)]
+          (1, 32, 128), (300, 200, 8), (64, 64, 1024), (64, 96, 8192), (128, 200, 5000), (72, 64, 2052),
+          (32, 1, 128), (3, 5, 1000), (40, 50, 64), (1, 1, 4096)]  # few outputs, long reduction: one work-group per output
 
 
 @pytest.mark.parametrize("ta,tb", [(0, 0), (0, 1), (1, 0), (1, 1)])
@@ -40,6 +41,20 @@ def test_sgemm_modes_vs_oracle(dev, M, N, K, ta, tb):
     opA, opB = (A.T if ta else A), (B.T if tb else B)
     assert_close(C, R.matmul(opA, opB), what="vs oracle")
     assert_close(C, opA.astype(np.float64) @ opB.astype(np.float64), what="vs float64")
+
+
+def test_sgemm_few_outputs_batched_accumulate(dev):
+    """The one-group-per-output kernel with a batch, a broadcast operand and accumulation into C."""
+    rng = np.random.default_rng(77)
+    M, N, K, batch = 4, 6, 300, 3
+    A = rng.standard_normal((batch, K, M)).astype(np.float32)   # used transposed
+    B = rng.standard_normal((K, N)).astype(np.float32)          # shared by the batch
+    C0 = rng.standard_normal((batch, M, N)).astype(np.float32)
+    dA, dB, dC = dev.put(A), dev.put(B), dev.put(C0)
+    dev.call("endia_hip_sgemm", 1, 0, M, N, K, dA, M, dB, N, dC, N, batch, K * M, 0, M * N, L.EPI_NONE | L.GEMM_ACCUMULATE,
+             L.OP_IDENTITY, None, None, None)
+    want = C0 + np.einsum("bkm,kn->bmn", A.astype(np.float64), B.astype(np.float64))
+    assert_close(dev.get(dC, (batch, M, N)), want, what="batched accumulate")
 
 
 def test_sgemm_golden(dev, golden):

@@ -674,3 +674,17 @@ def test_binary_with_transposed_view(dev, rows, cols, ld):
         np.testing.assert_array_equal(dev.get(dout, (rows, cols)), R.binary(name, full, view), err_msg=name)
         dev.call("endia_hip_binary", code, 2, shape, s_view, s_full, dbase, dfull, dout, 0)
         np.testing.assert_array_equal(dev.get(dout, (rows, cols)), R.binary(name, view, full), err_msg=name + " reversed")
+
+
+def test_sgd_step_multi(dev):
+    """Several parameter tensors in one launch: bit-identical to one launch per tensor."""
+    rng = np.random.default_rng(9)
+    sizes = [1, 32, 2048, 5, 16384, 64, 33] + [7] * 30   # more than one table of 32
+    ps = [rng.standard_normal(n).astype(np.float32) for n in sizes]
+    gs = [rng.standard_normal(n).astype(np.float32) for n in sizes]
+    dps, dgs = [dev.put(p) for p in ps], [dev.put(g) for g in gs]
+    k = len(sizes)
+    dev.call("endia_hip_sgd_step_multi", k, L.i64_array(sizes), (ctypes.c_void_p * k)(*dps), (ctypes.c_void_p * k)(*dgs), 0.125)
+    for p, g, dp, n in zip(ps, gs, dps, sizes):
+        np.testing.assert_array_equal(dev.get(dp, (n,)), R.sgd(p, g, 0.125))
+    dev.call("endia_hip_sgd_step_multi", 0, None, None, None, 0.125)
