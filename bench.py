@@ -33,7 +33,7 @@ HBM_PEAK_GBS = 8000.0
 # bias+tanh epilogue, 7 NT with the tanh' epilogue, 8 TN). It cannot be read while the benchmark runs: it comes
 # from two rocprofv3 --pmc runs (FETCH_SIZE, WRITE_SIZE in KiB per dispatch), each scaled by what the same counter
 # reads for a 64 MiB copy kernel (x1.999 and x1.000); the per-kernel table is in profiles/.
-GEMM_TRAFFIC_BYTES = int((8 * 802.7 + 7 * 1364.9 + 8 * 752.5) / 23 * 1024 * 1024)
+GEMM_TRAFFIC_BYTES = int((8 * 677.8 + 7 * 1351.0 + 8 * 745.7) / 23 * 1024 * 1024)
 
 
 def build_wide_mlp(nd, width=4096, layers=8, batch=4096, seed=2):
