@@ -347,6 +347,7 @@ int32_t sgemm_impl(int transA, int transB, int64_t M, int64_t N, int64_t K, cons
     p.tiles_m = (int)ceil_div64(M, 64 * F);
     p.tiles_n = (int)ceil_div64(N, 64 * F);
     const int64_t tiles = (int64_t)p.tiles_m * p.tiles_n;
+    ENDIA_CHECK_ARG(tiles < (1ll << 31), "sgemm: too many output tiles");
     // A long reduction with few output tiles (dW of a narrow layer over a large batch) is split along K:
     // slices write partial products that are then added in slice order.
     int64_t splits = 1;

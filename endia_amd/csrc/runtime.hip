@@ -62,12 +62,25 @@ static int64_t g_next_graph = 1, g_capture_id = 0;
 
 static void* g_ws = nullptr;
 static int64_t g_ws_bytes = 0;
+// Workspaces that were outgrown while captured steps existed: kernels recorded in those steps hold the
+// old address, so the memory stays allocated until the last captured step has been destroyed.
+static std::vector<void*> g_ws_retired;
+
+static void free_retired_workspaces() {
+  for (void* p : g_ws_retired) (void)hipFree(p);
+  g_ws_retired.clear();
+}
 
 int32_t workspace(int64_t bytes, void** out) {
   if (bytes > g_ws_bytes) {
     if (g_ctx.capturing)
       return fail(ENDIA_HIP_ERR_UNSUPPORTED, "workspace: would have to grow during capture; run the step once eagerly first");
-    if (g_ws) (void)hipFree(g_ws);
+    if (g_ws) {
+      if (g_graphs.empty())
+        (void)hipFree(g_ws);  // blocks until the queued users of the old workspace have finished
+      else
+        g_ws_retired.push_back(g_ws);
+    }
     g_ws = nullptr;
     g_ws_bytes = 0;
     int64_t want = bucket_of(bytes);
@@ -129,8 +142,16 @@ int32_t endia_hip_init(int32_t device) {
 
 int32_t endia_hip_shutdown(void) {
   if (!g_ctx.ready) return ENDIA_HIP_OK;
+  if (g_ctx.capturing) {  // abandon the unfinished capture; nothing recorded in it has run
+    hipGraph_t dropped = nullptr;
+    (void)hipStreamEndCapture(g_ctx.stream, &dropped);
+    if (dropped) (void)hipGraphDestroy(dropped);
+    (void)hipGetLastError();
+    g_ctx.capturing = false;
+  }
   (void)hipStreamSynchronize(g_ctx.stream);
   while (!g_graphs.empty()) release_graph(g_graphs.begin()->first);
+  free_retired_workspaces();
   for (auto& kv : g_pool.owned) (void)hipFree(kv.first);
   g_pool = Pool();
   if (g_ws) (void)hipFree(g_ws);
@@ -329,6 +350,7 @@ static void release_graph(int64_t id) {
   // buffers of this graph that are still held elsewhere become ordinary buffers
   for (auto& kv : g_pool.live)
     if (kv.second.graph == id) kv.second.graph = 0;
+  if (g_graphs.empty()) free_retired_workspaces();  // callers have synchronised the stream
 }
 
 int32_t endia_hip_graph_end(int64_t* handle) {
