@@ -202,6 +202,29 @@ class Array:
         from . import functional as F
         return F.reshape(self, shape)
 
+    @staticmethod
+    def _as_slices(index):
+        index = list(index) if isinstance(index, tuple) else [index]
+        return [i if isinstance(i, slice) else slice(i, i + 1 if i != -1 else None) for i in index]
+
+    def __getitem__(self, index):
+        """a[1:3, ::2] is array_slice (_array.mojo:805-809); an integer keeps its axis with length 1."""
+        from . import functional as F
+        return F.array_slice(self, self._as_slices(index))
+
+    def __setitem__(self, index, value):
+        """Write an array of the block's shape, or a scalar, through the slice view (_array.mojo:811-880)."""
+        from . import functional as F
+        sub = F.array_slice(F.detach(self), self._as_slices(index))
+        if not isinstance(value, Array):
+            value = F.full(sub.shape(), float(value))
+        if value.shape() != sub.shape() or value.is_complex_ != self.is_complex_:
+            raise ValueError("Error: Shapes do not match")
+        src = value if value.is_contiguous() else _contiguous_copy(value)
+        if src.size():
+            L.call("endia_hip_strided_scatter", sub.ndim(), L.i64_array(sub._shape), L.i64_array(sub._strides),
+                   sub._offset, src.data_ptr(), self._buf.ptr, 0, 1 if self.is_complex_ else 0)
+
     def _bin(self, other, fn, reverse=False):
         from . import functional as F
         if not isinstance(other, Array):

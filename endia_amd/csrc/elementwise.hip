@@ -283,6 +283,35 @@ __global__ __launch_bounds__(TPB) void strided_copy_kernel(CopyDesc d, const flo
   }
 }
 
+// The store side of a view: dst[offset + sum i_k * stride_k] (=, +=) src[j] for the row-major index j. With
+// ACC the view's elements may alias (overlapping windows of an as_strided view), so the add is atomic.
+template <bool CPLX, bool ACC>
+__global__ __launch_bounds__(TPB) void strided_scatter_kernel(CopyDesc d, const float* __restrict__ src,
+                                                              float* __restrict__ dst, int64_t n) {
+  int64_t i = (int64_t)blockIdx.x * TPB + threadIdx.x;
+  int64_t stride = (int64_t)gridDim.x * TPB;
+  for (int64_t j = i; j < n; j += stride) {
+    int64_t r = j, id = d.offset;
+    for (int k = d.ndim - 1; k >= 0; --k) {
+      int64_t q = r / d.shape[k];
+      id += (r - q * d.shape[k]) * d.st[k];
+      r = q;
+    }
+    if (CPLX) {
+      const float2 v = reinterpret_cast<const float2*>(src)[j];
+      if (ACC) {
+        atomicAdd(&dst[2 * id], v.x);
+        atomicAdd(&dst[2 * id + 1], v.y);
+      } else {
+        reinterpret_cast<float2*>(dst)[id] = v;
+      }
+    } else {
+      if (ACC) atomicAdd(&dst[id], src[j]);
+      else dst[id] = src[j];
+    }
+  }
+}
+
 // 2-D transpose through LDS: dst[r][c] = src[c*ld + r]; both sides coalesced.
 __global__ __launch_bounds__(256) void transpose_kernel(const float* __restrict__ src, float* __restrict__ dst,
                                                         int64_t rows, int64_t cols, int64_t ld, int64_t off) {
@@ -544,6 +573,52 @@ int32_t endia_hip_strided_copy(int32_t ndim, const int64_t* shape, const int64_t
     hipLaunchKernelGGL((strided_copy_kernel<true>), dim3(stream_grid(n)), dim3(TPB), 0, s, d, src, dst, n);
   else
     hipLaunchKernelGGL((strided_copy_kernel<false>), dim3(stream_grid(n)), dim3(TPB), 0, s, d, src, dst, n);
+  ENDIA_LAUNCH_CHECK();
+  return ENDIA_HIP_OK;
+}
+
+int32_t endia_hip_strided_scatter(int32_t ndim, const int64_t* shape, const int64_t* dst_strides, int64_t dst_offset,
+                                  const float* src, float* dst, int32_t accumulate, int32_t is_complex) {
+  ENDIA_REQUIRE_INIT();
+  ENDIA_CHECK_ARG(ndim >= 0 && ndim <= 8, "endia_hip_strided_scatter: ndim %d out of [0,8]", ndim);
+  ENDIA_CHECK_ARG(ndim == 0 || (shape && dst_strides), "endia_hip_strided_scatter: null descriptor");
+  ENDIA_CHECK_ARG(dst_offset >= 0, "endia_hip_strided_scatter: negative offset");
+  int64_t n = 1;
+  for (int i = 0; i < ndim; ++i) {
+    ENDIA_CHECK_ARG(shape[i] >= 0 && dst_strides[i] >= 0, "endia_hip_strided_scatter: negative extent or stride");
+    n *= shape[i];
+  }
+  if (n == 0) return ENDIA_HIP_OK;
+  ENDIA_CHECK_ARG(src && dst, "endia_hip_strided_scatter: null pointer");
+  if (!accumulate) {
+    // plain stores need a view whose elements are distinct: sorted by stride, every stride must step past
+    // the whole extent of the axes below it
+    int order[8], m = 0;
+    for (int i = 0; i < ndim; ++i)
+      if (shape[i] > 1) order[m++] = i;
+    for (int a = 1; a < m; ++a)
+      for (int b = a; b > 0 && dst_strides[order[b]] < dst_strides[order[b - 1]]; --b) {
+        int t = order[b]; order[b] = order[b - 1]; order[b - 1] = t;
+      }
+    int64_t span = 0;  // largest offset reachable with the axes seen so far
+    for (int a = 0; a < m; ++a) {
+      ENDIA_CHECK_ARG(dst_strides[order[a]] > span, "endia_hip_strided_scatter: the view's elements overlap; pass accumulate = 1");
+      span += (shape[order[a]] - 1) * dst_strides[order[a]];
+    }
+  }
+  CopyDesc d;
+  d.ndim = ndim;
+  d.offset = dst_offset;
+  for (int i = 0; i < 8; ++i) {
+    d.shape[i] = i < ndim ? shape[i] : 1;
+    d.st[i] = i < ndim ? dst_strides[i] : 0;
+  }
+  hipStream_t s = ctx().stream;
+  const dim3 grid(stream_grid(n)), block(TPB);
+  if (is_complex && accumulate) hipLaunchKernelGGL((strided_scatter_kernel<true, true>), grid, block, 0, s, d, src, dst, n);
+  else if (is_complex) hipLaunchKernelGGL((strided_scatter_kernel<true, false>), grid, block, 0, s, d, src, dst, n);
+  else if (accumulate) hipLaunchKernelGGL((strided_scatter_kernel<false, true>), grid, block, 0, s, d, src, dst, n);
+  else hipLaunchKernelGGL((strided_scatter_kernel<false, false>), grid, block, 0, s, d, src, dst, n);
   ENDIA_LAUNCH_CHECK();
   return ENDIA_HIP_OK;
 }

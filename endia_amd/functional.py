@@ -235,6 +235,148 @@ def reshape(x, shape):
     return _view(src, shape, contiguous_strides(shape), src._offset, [x], "reshape", vjp)
 
 
+def _dot(a, b):  # the module's own `sum` is the array op
+    t = 0
+    for u, v in zip(a, b):
+        t += u * v
+    return t
+
+
+def _norm_slices(slices, shape):
+    """Python-style (start, stop, step) per axis, step > 0, clamped to the axis; missing axes are whole."""
+    out = []
+    for i, n in enumerate(shape):
+        sl = slices[i] if i < len(slices) else slice(None)
+        if isinstance(sl, int):
+            sl = slice(sl, sl + 1 if sl != -1 else None)
+        start, stop, step = sl.indices(n)
+        if step <= 0:
+            raise ValueError("array_slice: steps must be positive")
+        out.append((start, max(stop, start), step))
+    return out
+
+
+def array_slice(x, slices):
+    """A view of a block of x: start / stop / step per leading axis (array_slice_op.mojo:41-83: stride times
+    step, offset plus start times stride). Its VJP pads the gradient back with zeros (:104-120)."""
+    if len(slices) > x.ndim():
+        raise ValueError("array_slice: %d slices for %d dimensions" % (len(slices), x.ndim()))
+    norm = _norm_slices(list(slices), x._shape)
+    shape = [(stop - start + step - 1) // step for start, stop, step in norm]
+    strides = [st * step for st, (_, _, step) in zip(x._strides, norm)]
+    offset = x._offset + _dot(x._strides, [start for start, _, _ in norm])
+    in_shape = list(x._shape)
+
+    def vjp(primals, grad, out):
+        lead = grad.ndim() - out.ndim()
+        whole = [slice(None)] * lead
+        return [pad(grad, list(grad._shape[:lead]) + in_shape, whole + [slice(a, b, c) for a, b, c in norm])]
+
+    return _view(x, shape, strides, offset, [x], "slice", vjp)
+
+
+def pad(x, target_shape, slices_in_target):
+    """x copied into the block `slices_in_target` of a zero array of `target_shape` (pad_op.mojo:35-142); the
+    VJP is the same block of the gradient (:83-101)."""
+    target_shape = list(target_shape)
+    if len(target_shape) != x.ndim():
+        raise ValueError("pad: target has %d dimensions, the array %d" % (len(target_shape), x.ndim()))
+    norm = _norm_slices(list(slices_in_target), target_shape)
+    block = [(stop - start + step - 1) // step for start, stop, step in norm]
+    if block != list(x._shape):
+        raise ValueError("Error in pad: target_shape and sliced_curr shape do not match")  # pad_op.mojo:137-140
+    out = Array(target_shape, is_complex=x.is_complex_)
+    src = contiguous(x)
+    if src.size():
+        L.call("endia_hip_strided_scatter", x.ndim(), L.i64_array(x._shape),
+               L.i64_array([st * step for st, (_, _, step) in zip(out._strides, norm)]),
+               _dot(out._strides, [start for start, _, _ in norm]), src.data_ptr(), out._buf.ptr, 0,
+               1 if x.is_complex_ else 0)
+
+    def vjp(primals, grad, o):
+        lead = grad.ndim() - o.ndim()
+        return [array_slice(grad, [slice(None)] * lead + [slice(a, b, c) for a, b, c in norm])]
+
+    return _register(out, [x], "pad", vjp)
+
+
+def _check_window(name, numel, shape, stride, storage_offset):
+    if len(shape) != len(stride) or any(s < 0 for s in shape) or any(s < 0 for s in stride) or storage_offset < 0:
+        raise ValueError("%s: shape and stride must have equal length and no negative entries" % name)
+    last = storage_offset + _dot([n - 1 for n in shape], stride) if _prod(shape) else 0
+    if last >= numel and _prod(shape):
+        raise ValueError("%s: the view reaches element %d of a buffer of %d" % (name, last, numel))
+
+
+def as_strided(x, shape, stride, storage_offset=0):
+    """A view of x's storage with the given shape, strides and offset, as torch.as_strided (as_strided_op.mojo:
+    33-160; the view is taken over the base buffer, :47-60). Windows may overlap. VJP: as_strided_inv (:67-89)."""
+    shape, stride = [int(s) for s in shape], [int(s) for s in stride]
+    base = contiguous(x)
+    _check_window("as_strided", base.size(), shape, stride, storage_offset)
+    in_shape = list(x._shape)
+
+    def vjp(primals, grad, out):
+        if grad.ndim() != len(shape):
+            raise ValueError("as_strided: batched cotangents are not supported")
+        return [as_strided_inv(grad, in_shape, shape, stride, storage_offset)]
+
+    return _view(base, shape, stride, base._offset + storage_offset, [x], "as_strided", vjp)
+
+
+def as_strided_inv(g, target_shape, shape, stride, storage_offset=0):
+    """Adjoint of as_strided: g added through an as_strided view into a zero array of target_shape
+    (as_strided_op.mojo:169-190). Where windows overlap the contributions add up. VJP: as_strided (:197-215)."""
+    shape, stride = [int(s) for s in shape], [int(s) for s in stride]
+    if list(g._shape) != shape:
+        raise ValueError("as_strided_inv: the array has shape %s, the view %s" % (g.shape(), shape))
+    out = Array(list(target_shape), is_complex=g.is_complex_)
+    _check_window("as_strided_inv", out.size(), shape, stride, storage_offset)
+    src = contiguous(g)
+    if src.size():
+        L.call("endia_hip_strided_scatter", len(shape), L.i64_array(shape), L.i64_array(stride), storage_offset,
+               src.data_ptr(), out._buf.ptr, 1, 1 if g.is_complex_ else 0)
+
+    def vjp(primals, grad, o):
+        return [as_strided(grad, shape, stride, storage_offset)]
+
+    return _register(out, [g], "as_strided_inv", vjp)
+
+
+def concat(arrays, axis=0):
+    """The arrays joined along `axis` (index_ops/concat_op.mojo:27-110; its forward allocates the result but
+    copies nothing and its VJP returns no gradients, :64-95, so the arithmetic here is numpy.concatenate's:
+    each argument is written into its block, and each gradient is that block of the cotangent)."""
+    arrays = list(arrays)
+    if not arrays:
+        raise ValueError("concat: no arrays")
+    nd = arrays[0].ndim()
+    axis = axis + nd if axis < 0 else axis
+    if not 0 <= axis < nd:
+        raise ValueError("Error: Axis out of bounds")
+    for a in arrays[1:]:
+        if a.ndim() != nd or any(a._shape[j] != arrays[0]._shape[j] for j in range(nd) if j != axis) \
+                or a.is_complex_ != arrays[0].is_complex_:
+            raise ValueError("Error: Incompatible shapes for concatenation")
+    shape = list(arrays[0]._shape)
+    shape[axis] = _dot([a._shape[axis] for a in arrays], [1] * len(arrays))
+    out = Array(shape, is_complex=arrays[0].is_complex_, _zero=False)
+    blocks, at = [], 0
+    for a in arrays:
+        blocks.append((at, at + a._shape[axis]))
+        src = contiguous(a)
+        if src.size():
+            L.call("endia_hip_strided_scatter", nd, L.i64_array(a._shape), L.i64_array(out._strides),
+                   at * out._strides[axis], src.data_ptr(), out._buf.ptr, 0, 1 if a.is_complex_ else 0)
+        at += a._shape[axis]
+
+    def vjp(primals, grad, o):
+        lead = grad.ndim() - o.ndim()
+        return [array_slice(grad, [slice(None)] * (lead + axis) + [slice(b0, b1)]) for b0, b1 in blocks]
+
+    return _register(out, arrays, "concat", vjp)
+
+
 def real_part(x):
     """real(): stride-2 fp32 view of a complex array (real_op.mojo:43-52); VJP complex(g, 0) (:74-77)."""
     if not x.is_complex_:

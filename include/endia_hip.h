@@ -148,6 +148,18 @@ ENDIA_API int32_t endia_hip_gemm_timing_end(int64_t* launches, double* total_ms,
 ENDIA_API int32_t endia_hip_strided_copy(int32_t ndim, const int64_t* shape, const int64_t* src_strides,
                                int64_t src_offset, const float* src, float* dst, int32_t is_complex);
 
+/* ---- strided scatter, the store side of a view: Pad.__call__ (view_ops/pad_op.mojo:115-142) writes its
+ *      argument through a slice view of a zeroed target (this is also the gradient of a slice,
+ *      array_slice_op.mojo:104-120), and AsStridedInv.__call__ (view_ops/as_strided_op.mojo:169-190), the
+ *      gradient of as_strided, adds it through an as_strided view of a zeroed target.
+ *      dst[dst_offset + sum i_d*stride_d] = src[i0..i_{r-1}] (+= when accumulate), src contiguous row-major
+ *      of `shape`, strides >= 0, ndim <= 8; dst is not cleared. accumulate = 0 requires a view whose
+ *      elements are distinct (checked); accumulate = 1 allows overlapping windows: the additions are
+ *      atomic and their order, hence the last bit of a sum, is not fixed. is_complex moves pairs. */
+ENDIA_API int32_t endia_hip_strided_scatter(int32_t ndim, const int64_t* shape, const int64_t* dst_strides,
+                                  int64_t dst_offset, const float* src, float* dst, int32_t accumulate,
+                                  int32_t is_complex);
+
 /* ---- fp32 GEMM: matmul_fwd (binary_ops/matmul_op.mojo:93-254) and both products of matmul_vjp
  *      (matmul_op.mojo:278-283). C[b] = opA(A[b]) . opB(B[b]), C is M x N with row stride ldc.
  *      transA = 0: A is M x K, element (m,k) at A[m*lda + k];  transA = 1: A is stored K x M, element

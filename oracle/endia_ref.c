@@ -13,7 +13,8 @@
  * How each function is pinned (tests/test_oracle.py, no GPU needed):
  *   matmul (real, complex), binary ops + broadcast (incl. pow and the comparisons), the 21 unary ops
  *   and their VJPs, the complex unary bodies, reduce_add, mse, conv1d / conv2d / conv3d forward, max and
- *   average pooling forward, SGD, Adam and the full MLP step are compared with PyTorch float64 -- the oracle
+ *   average pooling forward, the strided gather and scatter behind slice / pad / as_strided and their
+ *   gradients, SGD, Adam and the full MLP step are compared with PyTorch float64 -- the oracle
  *   the reference's own tests use (tests/test_endia/.../test_matmul_op.mojo:18-59 and siblings,
  *   metric endia/utils/array_conversions.mojo:63-135) -- with the doc known-answers
  *   (README.md:74-76,106-108; examples/custom_ops_examples/custom_mul.mojo:64-71) and with
@@ -62,6 +63,28 @@ void ref_strided_copy(int32_t ndim, const int64_t* shape, const int64_t* strides
       dst[2 * j + 1] = src[2 * is + 1];
     } else {
       dst[j] = src[is];
+    }
+  }
+}
+
+/* ---- the store side of a view. Pad.__call__ (view_ops/pad_op.mojo:115-142) stores its argument element
+ * by element through a slice view of the zero-filled result; AsStridedInv.__call__
+ * (view_ops/as_strided_op.mojo:169-190) adds it, in row-major order of the view, so that overlapping
+ * windows accumulate. dst must already hold the zero-filled target. */
+void ref_strided_scatter(int32_t ndim, const int64_t* shape, const int64_t* strides, int64_t offset,
+                         const float* src, float* dst, int32_t accumulate, int32_t is_complex) {
+  int64_t n = 1;
+  for (int i = 0; i < ndim; ++i) n *= shape[i];
+  const int w = is_complex ? 2 : 1;
+  for (int64_t j = 0; j < n; ++j) {
+    int64_t r = j, id = offset;
+    for (int k = ndim - 1; k >= 0; --k) {
+      id += (r % shape[k]) * strides[k];
+      r /= shape[k];
+    }
+    for (int c = 0; c < w; ++c) {
+      if (accumulate) dst[w * id + c] = dst[w * id + c] + src[w * j + c];
+      else dst[w * id + c] = src[w * j + c];
     }
   }
 }

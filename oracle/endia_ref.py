@@ -59,6 +59,28 @@ def _elem_strides(a, itemsize):
     return [s // itemsize for s in a.strides]
 
 
+def as_strided(x, shape, stride, offset=0):
+    """as_strided followed by contiguous(): the gather of functional/_utils.mojo:79-205 over x's storage."""
+    x = np.ascontiguousarray(x)
+    cplx = np.iscomplexobj(x)
+    x = x.astype(np.complex64 if cplx else np.float32)
+    out = np.zeros(tuple(shape), dtype=x.dtype)
+    lib().ref_strided_copy(c_int32(len(shape)), _i64(shape), _i64(stride), c_int64(offset), _ptr(x), _ptr(out),
+                           c_int32(1 if cplx else 0))
+    return out
+
+
+def strided_scatter(src, target_shape, stride, offset=0, accumulate=False):
+    """Pad.__call__ (accumulate False) / AsStridedInv.__call__ (True): src written or added through the view
+    (src.shape, stride, offset) of a zero array of target_shape."""
+    cplx = np.iscomplexobj(src)
+    src = np.ascontiguousarray(src, dtype=np.complex64 if cplx else np.float32)
+    out = np.zeros(tuple(target_shape), dtype=src.dtype)
+    lib().ref_strided_scatter(c_int32(src.ndim), _i64(src.shape), _i64(stride), c_int64(offset), _ptr(src), _ptr(out),
+                              c_int32(1 if accumulate else 0), c_int32(1 if cplx else 0))
+    return out
+
+
 def matmul(a, b):
     """matmul_fwd on 2-D or batched operands; a and b may be strided views (e.g. x.T)."""
     cplx = np.iscomplexobj(a) or np.iscomplexobj(b)

@@ -338,3 +338,36 @@ for name, xs, ws, st, pad, dil in [("1d", (3, 4, 29), (6, 4, 5), (2,), (3,), (2,
               "dx_" + name: tx.grad.numpy(), "dw_" + name: tw.grad.numpy(), "db_" + name: tb.grad.numpy(),
               "cfg_" + name: np.array([st, pad, dil], dtype=np.int64)})
 save("convnd", **d)
+
+# ---- views: as_strided with overlapping windows and its gradient (test_as_strided_op.mojo: the same two
+# cases, shapes (2,30,40) -> (1,2,40,2,2) and (30,30,2) with strides (9,30,2)), a strided slice and its
+# gradient (array_slice_op.mojo:104-120 pads the cotangent), pad and concat ---------------------------------
+d = {}
+x = f32(2, 30, 40)
+d["as_x"] = x
+d["as_y"] = torch.as_strided(t64(x), (1, 2, 40, 2, 2), (16, 8, 2, 2, 1), 0).numpy()
+x2 = np.arange(30 * 30 * 2, dtype=np.float32).reshape(30, 30, 2) * 0.01
+t = t64(x2, True)
+torch.sum(torch.sin(torch.as_strided(t, (30, 30, 2), (9, 30, 2), 0))).backward()
+d["as_x2"], d["as_dx2"] = x2, t.grad.numpy()
+x3 = f32(7, 9, 10)
+t = t64(x3, True)
+y = t[1:6:2, 2:, ::3]
+g = f32(*y.shape)
+(y * t64(g)).sum().backward()
+d.update({"sl_x": x3, "sl_y": y.detach().numpy(), "sl_g": g, "sl_dx": t.grad.numpy()})
+p = f32(3, 4)
+t = t64(p, True)
+big = torch.zeros(5, 9, dtype=torch.float64)
+big[1:4, 2:9:2] = t
+gb = f32(5, 9)
+(big * t64(gb)).sum().backward()
+d.update({"pad_x": p, "pad_y": big.detach().numpy(), "pad_g": gb, "pad_dx": t.grad.numpy()})
+c1, c2, c3 = f32(2, 3, 4), f32(2, 5, 4), f32(2, 1, 4)
+t1, t2, t3 = t64(c1, True), t64(c2, True), t64(c3, True)
+y = torch.cat([t1, t2, t3], dim=1)
+gc = f32(*y.shape)
+(y * t64(gc)).sum().backward()
+d.update({"cat_1": c1, "cat_2": c2, "cat_3": c3, "cat_y": y.detach().numpy(), "cat_g": gc, "cat_d1": t1.grad.numpy(),
+          "cat_d2": t2.grad.numpy(), "cat_d3": t3.grad.numpy()})
+save("views", **d)

@@ -557,3 +557,80 @@ def test_conv3d(nd, golden, name):  # test_conv3d_op.mojo, plus gradients
     assert_close(b.grad().to_numpy(), g["db_" + name], what="db")
     with pytest.raises(ValueError):
         nd.conv3d(nd.zeros([1, 2, 3, 4]), w)
+
+
+def test_as_strided(nd, golden):  # test_as_strided_op.mojo: the same two cases
+    g = golden("views")
+    y = nd.as_strided(nd.array(g["as_x"]), shape=[1, 2, 40, 2, 2], stride=[16, 8, 2, 2, 1], storage_offset=0)
+    np.testing.assert_array_equal(y.to_numpy(), g["as_y"])
+    arr = nd.array(g["as_x2"], requires_grad=True)
+    res = nd.sum(nd.sin(nd.as_strided(arr, shape=[30, 30, 2], stride=[9, 30, 2], storage_offset=0)))
+    res.backward()
+    assert_close(arr.grad().to_numpy(), g["as_dx2"], what="as_strided grad (overlapping windows)")
+    with pytest.raises(ValueError, match="reaches element"):
+        nd.as_strided(arr, [30, 30, 2], [90, 30, 2], 0)
+    # second order: the gradient of as_strided_inv is as_strided again (as_strided_op.mojo:197-215)
+    a = nd.array(g["as_x2"][:4, :3, 0].copy(), requires_grad=True)
+    win = nd.as_strided(a, [3, 2, 2], [3, 1, 1], 1)
+    (da,) = nd.grad([nd.sum(win * win * win)], [a], create_graph=True)
+    (dda,) = nd.grad([nd.sum(da)], [a])
+    x = g["as_x2"][:4, :3, 0].astype(np.float64).reshape(-1)
+    cnt = np.zeros(12)
+    for i in range(3):
+        for j in range(2):
+            for k in range(2):
+                cnt[1 + 3 * i + j + k] += 1
+    assert_close(da.to_numpy().reshape(-1), 3 * x * x * cnt, what="first derivative")
+    assert_close(dda.to_numpy().reshape(-1), 6 * x * cnt, what="second derivative")
+
+
+def test_slice_pad_concat(nd, golden):
+    g = golden("views")
+    x = nd.array(g["sl_x"], requires_grad=True)
+    y = x[1:6:2, 2:, ::3]
+    assert y.shape() == [3, 7, 4] and not y.is_contiguous()
+    np.testing.assert_array_equal(y.to_numpy(), g["sl_y"])
+    nd.sum(y * nd.array(g["sl_g"])).backward()
+    np.testing.assert_array_equal(x.grad().to_numpy(), g["sl_dx"])
+    np.testing.assert_array_equal(nd.array_slice(x, [slice(2, 3)]).to_numpy(), g["sl_x"][2:3])
+    np.testing.assert_array_equal(x[-1].to_numpy(), g["sl_x"][-1:])   # an integer keeps its axis
+
+    p = nd.array(g["pad_x"], requires_grad=True)
+    big = nd.pad(p, [5, 9], [slice(1, 4), slice(2, 9, 2)])
+    np.testing.assert_array_equal(big.to_numpy(), g["pad_y"])
+    nd.sum(big * nd.array(g["pad_g"])).backward()
+    np.testing.assert_array_equal(p.grad().to_numpy(), g["pad_dx"])
+    with pytest.raises(ValueError, match="do not match"):
+        nd.pad(p, [5, 9], [slice(0, 4), slice(0, 4)])
+
+    cs = [nd.array(g["cat_%d" % i], requires_grad=True) for i in (1, 2, 3)]
+    cat = nd.concat(cs, axis=1)
+    np.testing.assert_array_equal(cat.to_numpy(), g["cat_y"])
+    nd.sum(cat * nd.array(g["cat_g"])).backward()
+    for i, c in enumerate(cs):
+        np.testing.assert_array_equal(c.grad().to_numpy(), g["cat_d%d" % (i + 1)])
+    np.testing.assert_array_equal(nd.concat(cs, axis=-2).to_numpy(), g["cat_y"])
+    with pytest.raises(ValueError, match="Incompatible"):
+        nd.concat([cs[0], nd.zeros([2, 3, 5])], axis=1)
+
+    # slices compose with the other ops: a strided block feeds a matmul, gradient flows back through the view
+    a = nd.array(g["sl_x"][0], requires_grad=True)             # (9, 10)
+    w = nd.array(g["pad_x"].T.copy())                          # (4, 3)
+    out = nd.sum(a[1:8:2, 2:6] @ w)
+    out.backward()
+    want = np.zeros((9, 10), np.float32)
+    want[1:8:2, 2:6] = np.ones((4, 3), np.float32) @ g["pad_x"]
+    assert_close(a.grad().to_numpy(), want, what="grad through slice and matmul")
+
+    # __setitem__ writes through the view (array or scalar)
+    z = nd.zeros([4, 6])
+    z[1:3, ::2] = nd.array(np.arange(6, dtype=np.float32).reshape(2, 3))
+    z[3, 1:3] = 7.0
+    want = np.zeros((4, 6), np.float32)
+    want[1:3, ::2] = np.arange(6).reshape(2, 3)
+    want[3, 1:3] = 7
+    np.testing.assert_array_equal(z.to_numpy(), want)
+
+    # complex arrays move as pairs
+    zc = nd.array((g["pad_x"] + 1j * g["pad_x"][::-1]).astype(np.complex64))
+    np.testing.assert_array_equal(zc[1:, ::2].to_numpy(), (g["pad_x"] + 1j * g["pad_x"][::-1])[1:, ::2])

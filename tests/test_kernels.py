@@ -688,3 +688,40 @@ def test_sgd_step_multi(dev):
     for p, g, dp, n in zip(ps, gs, dps, sizes):
         np.testing.assert_array_equal(dev.get(dp, (n,)), R.sgd(p, g, 0.125))
     dev.call("endia_hip_sgd_step_multi", 0, None, None, None, 0.125)
+
+
+@pytest.mark.gpu
+def test_strided_scatter(dev, golden):
+    """endia_hip_strided_scatter against the oracle and the torch fixtures: slice gradient (plain stores),
+    as_strided gradient with overlapping windows (atomic adds; compared at 1e-6 because their order is free),
+    complex pairs, and the refusal of overlapping windows without accumulate."""
+    g = golden("views")
+    # slice [1:6:2, 2:, ::3] of (7, 9, 10)
+    src, dst = dev.put(g["sl_g"]), dev.put(np.zeros((7, 9, 10), np.float32))
+    dev.call("endia_hip_strided_scatter", 3, L.i64_array([3, 7, 4]), L.i64_array([180, 10, 3]), 110, src, dst, 0, 0)
+    got = dev.get(dst, (7, 9, 10))
+    np.testing.assert_array_equal(got, g["sl_dx"])
+    np.testing.assert_array_equal(got, R.strided_scatter(g["sl_g"], (7, 9, 10), (180, 10, 3), 110))
+    # gradient of sum(sin(as_strided(x, (30,30,2), (9,30,2)))): overlapping windows
+    x2 = g["as_x2"]
+    cot = np.cos(R.as_strided(x2, (30, 30, 2), (9, 30, 2)).astype(np.float64)).astype(np.float32)
+    src, dst = dev.put(cot), dev.put(np.zeros(x2.shape, np.float32))
+    dev.call("endia_hip_strided_scatter", 3, L.i64_array([30, 30, 2]), L.i64_array([9, 30, 2]), 0, src, dst, 1, 0)
+    got = dev.get(dst, x2.shape)
+    assert_close(got, g["as_dx2"], tol=1e-6, what="as_strided gradient vs torch")
+    assert_close(got, R.strided_scatter(cot, x2.shape, (9, 30, 2), 0, accumulate=True), tol=1e-6, what="vs oracle")
+    with pytest.raises(L.EndiaHipError, match="overlap"):
+        dev.call("endia_hip_strided_scatter", 3, L.i64_array([30, 30, 2]), L.i64_array([9, 30, 2]), 0, src, dst, 0, 0)
+    # complex block into a (4, 4) target, then accumulated a second time
+    rng = np.random.default_rng(5)
+    z = (rng.standard_normal((2, 3)) + 1j * rng.standard_normal((2, 3))).astype(np.complex64)
+    src, dst = dev.put(z), dev.put(np.zeros((4, 4), np.complex64))
+    dev.call("endia_hip_strided_scatter", 2, L.i64_array([2, 3]), L.i64_array([4, 1]), 5, src, dst, 0, 1)
+    dev.call("endia_hip_strided_scatter", 2, L.i64_array([2, 3]), L.i64_array([4, 1]), 5, src, dst, 1, 1)
+    want = np.zeros((4, 4), np.complex64)
+    want[1:3, 1:4] = 2 * z
+    np.testing.assert_array_equal(dev.get(dst, (4, 4), np.complex64), want)
+    # empty extents are a no-op; bad descriptors are refused
+    dev.call("endia_hip_strided_scatter", 2, L.i64_array([0, 3]), L.i64_array([4, 1]), 0, src, dst, 0, 0)
+    with pytest.raises(L.EndiaHipError):
+        dev.call("endia_hip_strided_scatter", 9, L.i64_array([1] * 9), L.i64_array([1] * 9), 0, src, dst, 0, 0)

@@ -365,3 +365,34 @@ def test_convnd_reduces_to_conv2d(golden):
     x, w, b = g["x"], g["w"], g["b"]
     y2 = R.conv2d(x, w, b, (2, 2), (1, 1), (1, 1))
     np.testing.assert_array_equal(R.convnd(x, w, b, (2, 2), (1, 1), (1, 1)), y2)
+
+
+def test_views_golden(golden):
+    """The oracle's strided gather and scatter against torch: as_strided with overlapping windows and its
+    gradient (the two cases of test_as_strided_op.mojo), a stepped slice, pad."""
+    g = golden("views")
+    assert_close(R.as_strided(g["as_x"], (1, 2, 40, 2, 2), (16, 8, 2, 2, 1)), g["as_y"], tol=0, what="as_strided")
+    x2 = g["as_x2"]
+    cot = np.cos(R.as_strided(x2, (30, 30, 2), (9, 30, 2)).astype(np.float64)).astype(np.float32)
+    assert_close(R.strided_scatter(cot, x2.shape, (9, 30, 2), 0, accumulate=True), g["as_dx2"], what="as_strided grad")
+    # slice [1:6:2, 2:, ::3] of a (7, 9, 10) array: element strides (90, 10, 1) -> (180, 10, 3), offset 90 + 20
+    assert_close(R.as_strided(g["sl_x"], (3, 7, 4), (180, 10, 3), 110), g["sl_y"], tol=0, what="slice")
+    assert_close(R.strided_scatter(g["sl_g"], (7, 9, 10), (180, 10, 3), 110), g["sl_dx"], tol=0, what="slice grad")
+    # pad: a (3, 4) block at [1:4, 2:9:2] of a (5, 9) target: strides (9, 2), offset 11
+    assert_close(R.strided_scatter(g["pad_x"], (5, 9), (9, 2), 11), g["pad_y"], tol=0, what="pad")
+    assert_close(R.as_strided(g["pad_g"], (3, 4), (9, 2), 11), g["pad_dx"], tol=0, what="pad grad")
+
+
+def test_strided_scatter_brute_force():
+    """Overlapping windows accumulate: a sliding window of 3 with stride 1 over 6 elements, by hand."""
+    src = np.arange(12, dtype=np.float32).reshape(4, 3)
+    want = np.zeros(6, np.float32)
+    for i in range(4):
+        for j in range(3):
+            want[i + j] += src[i, j]
+    np.testing.assert_array_equal(R.strided_scatter(src, (6,), (1, 1), 0, accumulate=True), want)
+    z = (np.arange(6) + 1j * np.arange(6)).astype(np.complex64).reshape(2, 3)
+    out = R.strided_scatter(z, (4, 4), (4, 1), 5)
+    want = np.zeros((4, 4), np.complex64)
+    want[1:3, 1:4] = z
+    np.testing.assert_array_equal(out, want)
