@@ -767,12 +767,13 @@ def _gemm_operand(x):
     return d
 
 
-def matmul(a, b, _conj_vjp=False):
+def matmul(a, b, _conj_vjp=False, _ca=0, _cb=0):
     """Batched matrix product with broadcast batch axes (matmul_op.mojo:36-90,309-346).
 
     VJP (matmul_op.mojo:278-283): dA = g @ B.T(), dB = A.T() @ g -- for complex operands WITHOUT
     conjugation, exactly as the reference codes it. `_conj_vjp=True` selects the Wirtinger rule
-    (g @ B^H, A^H @ g) that PyTorch uses.
+    (g @ B^H, A^H @ g) that PyTorch uses; its conjugations are flags of the complex GEMM (`_ca`, `_cb`:
+    the product is taken with conj(a), conj(b)), never materialised copies.
     """
     if a.ndim() < 2 or b.ndim() < 2:
         raise ValueError("Invalid shapes for matmul, i.e. ndim < 2")
@@ -803,7 +804,7 @@ def matmul(a, b, _conj_vjp=False):
     batch = _prod(bshape)
     if out.size():
         if a.is_complex_:
-            L.call("endia_hip_cgemm", ta, 0, tb, 0, M, N, K, A_.data_ptr(), lda, B_.data_ptr(), ldb, out.data_ptr(), N,
+            L.call("endia_hip_cgemm", ta, _ca, tb, _cb, M, N, K, A_.data_ptr(), lda, B_.data_ptr(), ldb, out.data_ptr(), N,
                    batch, sa, sb, M * N, _cgemm_algo[0], 0)
         else:
             L.call("endia_hip_sgemm", ta, tb, M, N, K, A_.data_ptr(), lda, B_.data_ptr(), ldb, out.data_ptr(), N, batch,
@@ -812,8 +813,9 @@ def matmul(a, b, _conj_vjp=False):
     def vjp(primals, grad, out_):
         p0, p1 = primals
         if _conj_vjp and p0.is_complex_:
-            lhs = matmul(grad, conj(p1).T(), True) if p0._requires_grad else None
-            rhs = matmul(conj(p0).T(), grad, True) if p1._requires_grad else None
+            # with A' = conj^ca(A), B' = conj^cb(B): dA = conj^ca(g B'^H), dB = conj^cb(A'^H g)
+            lhs = matmul(grad, p1.T(), True, _ca, _ca ^ (1 - _cb)) if p0._requires_grad else None
+            rhs = matmul(p0.T(), grad, True, _cb ^ (1 - _ca), _cb) if p1._requires_grad else None
         else:
             lhs = matmul(grad, p1.T()) if p0._requires_grad else None
             rhs = matmul(p0.T(), grad) if p1._requires_grad else None

@@ -634,3 +634,23 @@ def test_slice_pad_concat(nd, golden):
     # complex arrays move as pairs
     zc = nd.array((g["pad_x"] + 1j * g["pad_x"][::-1]).astype(np.complex64))
     np.testing.assert_array_equal(zc[1:, ::2].to_numpy(), (g["pad_x"] + 1j * g["pad_x"][::-1])[1:, ::2])
+
+
+@pytest.mark.parametrize("ca,cb", [(0, 0), (0, 1), (1, 0), (1, 1)])
+def test_complex_matmul_wirtinger_flags(nd, ca, cb):
+    """The Wirtinger rule runs its conjugations as flags of the complex GEMM. For every flag pair the product
+    conj^ca(A) conj^cb(B) and both gradients of sum(Re(P) * G) must equal torch's (complex128 autograd)."""
+    import torch
+    rng = np.random.default_rng(40 + 2 * ca + cb)
+    A = (rng.standard_normal((9, 12)) + 1j * rng.standard_normal((9, 12))).astype(np.complex64)
+    B = (rng.standard_normal((12, 7)) + 1j * rng.standard_normal((12, 7))).astype(np.complex64)
+    G = rng.standard_normal((9, 7)).astype(np.float32)
+    ta, tb = (torch.tensor(v, dtype=torch.complex128, requires_grad=True) for v in (A, B))
+    tp = (ta.conj() if ca else ta) @ (tb.conj() if cb else tb)
+    (tp.real * torch.tensor(G, dtype=torch.float64)).sum().backward()
+    a, b = nd.array(A, requires_grad=True), nd.array(B, requires_grad=True)
+    p = nd.matmul(a, b, True, ca, cb)
+    assert_close(p.to_numpy(), tp.detach().resolve_conj().numpy(), what="product")
+    nd.sum(nd.real(p) * nd.array(G)).backward()
+    assert_close(a.grad().to_numpy(), ta.grad.resolve_conj().numpy(), what="dA")
+    assert_close(b.grad().to_numpy(), tb.grad.resolve_conj().numpy(), what="dB")

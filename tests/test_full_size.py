@@ -229,3 +229,79 @@ def test_conv3d_full_size_properties(dev):
     for n, k, z, r, c in [(0, 0, 0, 0, 0), (7, 63, 15, 55, 55), (3, 17, 8, 30, 1), (5, 40, 1, 0, 55), (2, 9, 15, 27, 28)]:
         want = (xp[n, :, z:z + 3, r:r + 3, c:c + 3] * w[k].astype(np.float64)).sum()
         assert abs(y[n, k, z, r, c] - want) <= 1e-4 * max(1.0, abs(want))
+
+
+def test_hvp_full_size_symmetry_and_linearity():
+    """The second-order benchmark configuration (batch 1024, 4 layers 2048 wide, sin, loss sum(out^2)): the
+    Hessian is symmetric, so <u, H v> = <v, H u>, and H (2 v) = 2 H v. Both hold for any size, so they check
+    the double-backward path at its real shapes without a CPU reference of that size."""
+    import endia_amd as nd
+    rng = np.random.default_rng(103)
+    B, Wd, Ly = 1024, 2048, 4
+    mlp = nd.nn.MLP([Wd] * (Ly + 1), compute_backward=True, activation="sin", fused=True)
+    for i in range(Ly):
+        mlp.weights[i] = nd.array((rng.standard_normal((Wd, Wd)) / np.sqrt(Wd)).astype(np.float32), requires_grad=True)
+        mlp.biases[i] = nd.array((rng.standard_normal(Wd) / np.sqrt(Wd)).astype(np.float32), requires_grad=True)
+    x = nd.array(rng.standard_normal((B, Wd)).astype(np.float32))
+    shapes = [p.shape() for p in mlp.params()]
+    u = [rng.standard_normal(s).astype(np.float32) for s in shapes]
+    v = [rng.standard_normal(s).astype(np.float32) for s in shapes]
+
+    def hvp(vec):
+        out = mlp.forward(x)
+        loss = nd.sum(out * out)
+        loss.backward(create_graph=True)
+        s = None
+        for p, w in zip(mlp.params(), vec):
+            term = nd.sum(p.grad() * nd.array(w))
+            s = term if s is None else s + term
+        hv = nd.grad(outs=s, inputs=mlp.params())
+        loss.zero_grad()
+        return [h.to_numpy().astype(np.float64).reshape(-1) for h in hv]
+
+    def dot(a, b):
+        return float(sum(np.dot(p, q.astype(np.float64).reshape(-1)) for p, q in zip(a, b)))
+
+    Hv, Hu = hvp(v), hvp(u)
+    uHv, vHu = dot(Hv, u), dot(Hu, v)
+    assert abs(uHv - vHu) <= 1e-3 * max(abs(uHv), abs(vHu)), (uHv, vHu)
+    H2v = hvp([2 * w for w in v])
+    for a, b in zip(H2v, Hv):
+        assert_close(a, 2 * b, tol=1e-5, what="H (2 v) = 2 H v")
+    assert all(np.isfinite(h).all() for h in Hv) and dot(Hv, v) != 0.0
+
+
+@pytest.mark.parametrize("algo", ["4m", "3m"])
+def test_complex_mlp_full_size_directional_derivative(algo):
+    """The complex benchmark configuration (batch 2048, 4 complex layers 2048 wide, loss sum |out|^2). With the
+    Wirtinger rule the gradient g satisfies dL(W + eps V)/d eps = Re <g, V>, whatever the size; checked with a
+    central difference for both GEMM algorithms. (The reference's rule without conjugation is not the
+    gradient of a real loss; it is compared with the oracle's composition of the same products at small sizes.)"""
+    import endia_amd as nd
+    rng = np.random.default_rng(104)
+    n, Ly = 2048, 4
+    nd.set_complex_matmul_algorithm(algo)
+    try:
+        Wn = [((rng.standard_normal((n, n)) + 1j * rng.standard_normal((n, n))) / np.sqrt(2 * n)).astype(np.complex64)
+              for _ in range(Ly)]
+        Vn = [(rng.standard_normal((n, n)) + 1j * rng.standard_normal((n, n))).astype(np.complex64) for _ in range(Ly)]
+        z = nd.array((rng.standard_normal((n, n)) + 1j * rng.standard_normal((n, n))).astype(np.complex64))
+
+        def loss_at(eps, want_grad):
+            Ws = [nd.array(W + np.complex64(eps) * V, requires_grad=want_grad) for W, V in zip(Wn, Vn)]
+            h = z
+            for W in Ws:
+                h = nd.matmul(h, W, _conj_vjp=True)
+            loss = nd.sum(nd.square(nd.abs(h)))
+            if not want_grad:
+                return float(loss.item())
+            loss.backward()
+            return float(loss.item()), sum(float(np.vdot(W.grad().to_numpy().astype(np.complex128), V).real)
+                                           for W, V in zip(Ws, Vn))
+
+        l0, analytic = loss_at(0.0, True)
+        eps = 1e-4
+        numeric = (loss_at(eps, False) - loss_at(-eps, False)) / (2 * eps)
+        assert abs(numeric - analytic) <= 2e-2 * abs(analytic), (algo, l0, analytic, numeric)
+    finally:
+        nd.set_complex_matmul_algorithm("4m")
