@@ -313,6 +313,36 @@ def conv_table(reps=10):
     return rows
 
 
+def conv_step(nd, steps, warmup, x_grad):
+    """One training step of the convolution configuration through the public API: loss = mean(relu(conv2d(x, w,
+    b))), backward to w and b (and to x when x_grad). Algorithmic work 2*N*K*C*R*S*P*Q = 29.6 GFLOP per
+    convolution-shaped pass: forward + weight gradient (+ data gradient)."""
+    rng = np.random.default_rng(5)
+    N, C, H, W, K, R, S = 64, 64, 56, 56, 128, 3, 3
+    x = nd.array(rng.standard_normal((N, C, H, W)).astype(np.float32), requires_grad=x_grad)
+    w = nd.array((rng.standard_normal((K, C, R, S)) * np.sqrt(2.0 / (C * R * S))).astype(np.float32), requires_grad=True)
+    b = nd.array(rng.standard_normal(K).astype(np.float32), requires_grad=True)
+
+    def step():
+        loss = nd.mean(nd.conv2d(x, w, b, stride=1, padding=1, act="relu"))
+        loss.backward()
+        loss.zero_grad()
+        return loss
+
+    for _ in range(max(warmup, 3)):
+        step()
+    nd.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        step()
+    nd.synchronize()
+    dt = (time.perf_counter() - t0) / steps
+    flops = (3 if x_grad else 2) * 2.0 * N * K * C * R * S * H * W
+    return {"passes": "forward + weight gradient + bias gradient" + (" + data gradient" if x_grad else ""),
+            "ms_per_step": dt * 1e3, "steps_per_s": 1.0 / dt, "algorithmic_tflops": flops / dt / 1e12,
+            "frac_of_fp32_mfma_peak": flops / dt / 1e12 / FP32_MFMA_PEAK_TFLOPS}
+
+
 def gemm_roofline(L, elapsed_s, algorithmic_flops_total, kernel):
     """Close a gemm_timing window and price the MFMA GEMM launches inside it: achieved = algorithmic flops /
     summed HIP-event kernel time of those launches (events recorded on the library's stream)."""
@@ -467,7 +497,9 @@ def main():
     if args.workload == "conv2d":
         rows = conv_table(max(args.steps, 1))
         print(json.dumps({"metric": "conv2d fwd + VJPs, batch 64, 64->128 channels, 3x3, stride 1, pad 1, 56x56, fp32",
-                          "device": dev_name, "reps": max(args.steps, 1), "kernels": rows}))
+                          "device": dev_name, "reps": max(args.steps, 1), "kernels": rows,
+                          "train_step": [conv_step(nd, max(args.steps, 1), args.warmup, False),
+                                         conv_step(nd, max(args.steps, 1), args.warmup, True)]}))
         return
     if args.workload == "kernels":
         rows = kernel_table(max(args.steps, 1))

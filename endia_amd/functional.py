@@ -476,6 +476,8 @@ pow_to = pow
 
 
 def _comparison(op, name, a, b):
+    if _fusion is not None and _fusion.tracing(a, b):  # inside a fused expression; a plain number is an immediate
+        return _fusion.sym_binary(op, name, a, b, None)
     if a.is_complex_ or b.is_complex_:
         raise ValueError("%s is implemented for real arrays only" % name)
     return _binary(op, name, detach(a), detach(b), None)
@@ -883,9 +885,31 @@ def _pair(v):
     return (int(v), int(v)) if np.isscalar(v) else (int(v[0]), int(v[1]))
 
 
-def conv2d(x, kernel, bias=None, stride=1, padding=0, dilation=1, groups=1, _act=None):
+_relu_grad_of_scalar = [None]
+
+
+def _relu_grad_from_output(out, grad):
+    """grad * [out > 0] in one pass. A cotangent that is one value spread over the whole array (the gradient of
+    a mean or a sum: a stride-0 view) is read as a scalar, so no full-size copy of it is ever written."""
+    if grad.size() and all(st == 0 or n == 1 for st, n in zip(grad._strides, grad._shape)) and not grad.is_complex_:
+        if _relu_grad_of_scalar[0] is None:
+            _relu_grad_of_scalar[0] = _fusion.fuse(lambda o, g: mul(greater(o, 0.0), g), "relu_grad")
+        one = Array([1], _buffer=grad._buf, _strides=[1], _offset=grad._offset)
+        return _relu_grad_of_scalar[0](detach(out), one)
+    g = contiguous(grad)
+    gp = Array.empty(out._shape)
+    L.call("endia_hip_unary_vjp_from_output", L.OP_RELU, out.size(), out.data_ptr(), g.data_ptr(), gp.data_ptr())
+    return gp
+
+
+def conv2d(x, kernel, bias=None, stride=1, padding=0, dilation=1, groups=1, act=None):
     """NCHW cross-correlation (conv2d_op.mojo:88-196; tuple order is (height, width)). The reference has
-    no backward rule for it (conv2d_op.mojo:198-200); the VJP here is the adjoint of its forward loop."""
+    no backward rule for it (conv2d_op.mojo:198-200); the VJP here is the adjoint of its forward loop.
+    act="relu" (no counterpart in the reference) applies the activation in the kernel's epilogue and its
+    derivative on the way into the gradients, instead of as separate passes over the output."""
+    if act not in (None, "relu"):
+        raise ValueError("conv2d: act must be None or 'relu'")
+    _act = act
     if x.ndim() != 4:
         raise ValueError("Input must be 4-dimensional (batch_size, in_channels, height, width) for 2D convolution!")
     if x._shape[1] != kernel._shape[1]:
@@ -910,9 +934,7 @@ def conv2d(x, kernel, bias=None, stride=1, padding=0, dilation=1, groups=1, _act
         from .autograd.functional import building_graph
         if building_graph():
             raise NotImplementedError("conv2d has no second-order rule")
-        g = contiguous(grad)
-        if _act == "relu":
-            g = mul(greater(out_, zeros([out_._shape[-1]])), g)
+        g = contiguous(_relu_grad_from_output(out_, grad)) if _act == "relu" else contiguous(grad)
         res = []
         if primals[0]._requires_grad:
             dx = Array.empty(primals[0]._shape)

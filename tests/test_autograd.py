@@ -654,3 +654,35 @@ def test_complex_matmul_wirtinger_flags(nd, ca, cb):
     nd.sum(nd.real(p) * nd.array(G)).backward()
     assert_close(a.grad().to_numpy(), ta.grad.resolve_conj().numpy(), what="dA")
     assert_close(b.grad().to_numpy(), tb.grad.resolve_conj().numpy(), what="dB")
+
+
+def test_conv2d_fused_relu_step(nd, golden):
+    """conv2d(..., act="relu") under a mean loss (the convolution benchmark's step): the activation runs in the
+    kernel's epilogue, and its derivative meets the broadcast mean gradient in one pass. Same numbers as the
+    op-by-op composition and as torch; also with an ordinary full-size cotangent."""
+    import torch
+    g = golden("conv2d")
+    tx, tw, tb = (torch.tensor(g[k], dtype=torch.float64, requires_grad=True) for k in ("x", "w", "b"))
+    ty = torch.relu(torch.nn.functional.conv2d(tx, tw, tb, stride=1, padding=1))
+    ty.mean().backward()
+    x, w, b = (nd.array(g[k], requires_grad=True) for k in ("x", "w", "b"))
+    y = nd.conv2d(x, w, b, stride=1, padding=1, act="relu")
+    assert_close(y.to_numpy(), ty.detach().numpy(), what="relu(conv2d)")
+    loss = nd.mean(y)
+    loss.backward()
+    assert_close([loss.item()], [ty.mean().item()], what="loss")
+    assert_close(x.grad().to_numpy(), tx.grad.numpy(), what="dx")
+    assert_close(w.grad().to_numpy(), tw.grad.numpy(), what="dw")
+    assert_close(b.grad().to_numpy(), tb.grad.numpy(), what="db")
+    # a dense cotangent takes the other branch (one relu-gradient kernel on the stored output)
+    cot = np.random.default_rng(9).standard_normal(ty.shape).astype(np.float32)
+    for t in (tx, tw, tb):
+        t.grad = None
+    ty2 = torch.relu(torch.nn.functional.conv2d(tx, tw, tb, stride=1, padding=1))
+    (ty2 * torch.tensor(cot, dtype=torch.float64)).sum().backward()
+    x, w, b = (nd.array(g[k], requires_grad=True) for k in ("x", "w", "b"))
+    nd.sum(nd.conv2d(x, w, b, stride=1, padding=1, act="relu") * nd.array(cot)).backward()
+    assert_close(x.grad().to_numpy(), tx.grad.numpy(), what="dx (dense cotangent)")
+    assert_close(w.grad().to_numpy(), tw.grad.numpy(), what="dw (dense cotangent)")
+    with pytest.raises(ValueError, match="act"):
+        nd.conv2d(x, w, b, act="tanh")
