@@ -138,6 +138,91 @@ def cpu_baseline_sine(steps=200):
             "sample": "%d full fwd+bwd+SGD steps of the ref-order CPU restatement, 1 thread" % steps}
 
 
+def _timed(fn):
+    t0 = time.perf_counter()
+    fn()
+    return time.perf_counter() - t0
+
+
+def _extrapolate(fn, r1, r2, full):
+    """Time fn(r) on two slice heights and extend the straight line through them to `full` rows: the per-call
+    copies of the reference's matmul (contiguous LHS, transposed RHS) are then counted once, not once per slice."""
+    t1, t2 = _timed(lambda: fn(r1)), _timed(lambda: fn(r2))
+    per_row = max((t2 - t1) / (r2 - r1), 0.0)
+    return max(t1 - r1 * per_row, 0.0) + full * per_row
+
+
+def cpu_baseline_hvp(rows=96):
+    """The reference's single-threaded path for one Hessian-vector product, composed from row slices: the 31
+    products of 1024 x 2048 x 2048 (11 NN, 9 NT, 11 TN, as the tape issues them) plus the elementwise and
+    reduction passes over [1024, 2048] arrays that the double backward adds (counted on the device trace)."""
+    from oracle import endia_ref as R
+    rng = np.random.default_rng(3)
+    t_all0 = time.perf_counter()
+    B, Wd = 1024, 2048
+    X = rng.standard_normal((B, Wd)).astype(np.float32)
+    W = (rng.standard_normal((Wd, Wd)) / np.sqrt(Wd)).astype(np.float32)
+    t_nn = _extrapolate(lambda r: R.matmul(X[:r], W), rows, 2 * rows, B)
+    t_nt = _extrapolate(lambda r: R.matmul(X[:r], W.T), rows, 2 * rows, B)
+    t_tn = _extrapolate(lambda r: R.matmul(X[:, :r].T, X), rows, 2 * rows, Wd)
+    Z = X[:128]
+    t_bin = _timed(lambda: R.binary("mul", Z, Z)) * (B / 128)
+    t_un = _timed(lambda: R.unary("sin", Z)) * (B / 128)
+    t_red = _timed(lambda: R.reduce_add(Z, [0])) * (B / 128)
+    n_bin, n_un, n_red = 58, 12, 17
+    step = 11 * t_nn + 9 * t_nt + 11 * t_tn + n_bin * t_bin + n_un * t_un + n_red * t_red
+    return {"value": 1.0 / step, "unit": "HVP/s", "cores": 1, "kind": "port", "host_cores_available": os.cpu_count(),
+            "seconds_per_step": step,
+            "sample": "ref-order CPU restatement (oracle/endia_ref.c, 1 thread): %d- and 2x%d-row slices of the NN, NT and TN products "
+                      "extrapolated linearly and composed as 11 + 9 + 11 products, plus %d binary, %d unary and %d reduction passes "
+                      "over [1024, 2048] timed on 128-row slices; %.1f s of CPU work" % (rows, rows, n_bin, n_un, n_red, time.perf_counter() - t_all0)}
+
+
+def cpu_baseline_complex(rows=96):
+    """The reference's complex matmul (four real multiply-adds per element, matmul_op.mojo:201-238) on row slices
+    of the 2048^3 products, composed as the step issues them: 4 forward (NN), 3 data gradients (NT), 4 weight
+    gradients (TN)."""
+    from oracle import endia_ref as R
+    rng = np.random.default_rng(4)
+    t_all0 = time.perf_counter()
+    n = 2048
+    Z = (rng.standard_normal((n, n)) + 1j * rng.standard_normal((n, n))).astype(np.complex64)
+    t_nn = _extrapolate(lambda r: R.matmul(Z[:r], Z), rows, 2 * rows, n)
+    t_nt = _extrapolate(lambda r: R.matmul(Z[:r], Z.T), rows, 2 * rows, n)
+    t_tn = _extrapolate(lambda r: R.matmul(Z[:, :r].T, Z), rows, 2 * rows, n)
+    step = 4 * t_nn + 3 * t_nt + 4 * t_tn
+    return {"value": 1.0 / step, "unit": "steps/s", "cores": 1, "kind": "port", "host_cores_available": os.cpu_count(),
+            "seconds_per_step": step,
+            "sample": "ref-order CPU restatement (1 thread): %d- and 2x%d-row slices of the complex NN, NT and TN products of 2048^3, "
+                      "extrapolated linearly and composed as 4 + 3 + 4 products (the elementwise loss passes are under 1 %% and "
+                      "left out); %.1f s of CPU work" % (rows, rows, time.perf_counter() - t_all0)}
+
+
+def cpu_baseline_conv():
+    """The reference's 7-deep convolution loop (conv2d_op.mojo:127-196) and the brute-force adjoints of it, on four
+    images of the batch of 64, extrapolated by 16; plus the ReLU / mean passes over those images' output."""
+    from oracle import endia_ref as R
+    rng = np.random.default_rng(5)
+    t_all0 = time.perf_counter()
+    C, H, K = 64, 56, 128
+    n_img = 4
+    x = rng.standard_normal((n_img, C, H, H)).astype(np.float32)
+    w = (rng.standard_normal((K, C, 3, 3)) * np.sqrt(2.0 / (C * 9))).astype(np.float32)
+    bias = rng.standard_normal(K).astype(np.float32)
+    dy = rng.standard_normal((n_img, K, H, H)).astype(np.float32)
+    scale = 64 / n_img
+    t_fwd = _timed(lambda: R.conv2d(x, w, bias, (1, 1), (1, 1), (1, 1))) * scale
+    t_bwd = _timed(lambda: R.conv2d_bwd(x, w, dy, (1, 1), (1, 1), (1, 1))) * scale   # dx, dw and db together
+    t_ew = (_timed(lambda: R.unary("relu", dy)) + _timed(lambda: R.unary_vjp("relu", dy, dy)) +
+            _timed(lambda: R.reduce_add(dy.reshape(1, -1), [1]))) * scale
+    step = t_fwd + t_bwd + t_ew
+    return {"value": 1.0 / step, "unit": "steps/s", "cores": 1, "kind": "port", "host_cores_available": os.cpu_count(),
+            "seconds_per_step": step, "forward_seconds": t_fwd, "gradients_seconds": t_bwd,
+            "sample": "ref-order CPU restatement (1 thread): forward loop and its adjoints (dx, dw, db) on 4 of the 64 "
+                      "images, extrapolated by 16, plus relu / relu-gradient / mean passes; %.1f s of CPU work"
+                      % (time.perf_counter() - t_all0)}
+
+
 def kernel_table(reps=10):
     """Times each hot kernel alone at the wide-MLP shape with HIP events on the library's stream and
     prices it against its roofline (fp32 MFMA peak for the GEMMs, HBM peak for the rest). Algorithmic
@@ -489,17 +574,26 @@ def main():
     dev_name, cus, mhz = L.device_info()
 
     if args.workload == "hvp":
-        print(json.dumps(run_hvp(nd, args.steps, args.warmup)))
+        out = run_hvp(nd, args.steps, args.warmup)
+        if not args.no_cpu_baseline:
+            out["cpu_baseline"] = cpu_baseline_hvp()
+        print(json.dumps(out))
         return
     if args.workload.startswith("complex_mlp"):
-        print(json.dumps(run_complex(nd, args.steps, args.warmup, "3m" if args.workload.endswith("3m") else "4m")))
+        out = run_complex(nd, args.steps, args.warmup, "3m" if args.workload.endswith("3m") else "4m")
+        if not args.no_cpu_baseline:
+            out["cpu_baseline"] = cpu_baseline_complex()
+        print(json.dumps(out))
         return
     if args.workload == "conv2d":
         rows = conv_table(max(args.steps, 1))
-        print(json.dumps({"metric": "conv2d fwd + VJPs, batch 64, 64->128 channels, 3x3, stride 1, pad 1, 56x56, fp32",
-                          "device": dev_name, "reps": max(args.steps, 1), "kernels": rows,
-                          "train_step": [conv_step(nd, max(args.steps, 1), args.warmup, False),
-                                         conv_step(nd, max(args.steps, 1), args.warmup, True)]}))
+        out = {"metric": "conv2d fwd + VJPs, batch 64, 64->128 channels, 3x3, stride 1, pad 1, 56x56, fp32",
+               "device": dev_name, "reps": max(args.steps, 1), "kernels": rows,
+               "train_step": [conv_step(nd, max(args.steps, 1), args.warmup, False),
+                              conv_step(nd, max(args.steps, 1), args.warmup, True)]}
+        if not args.no_cpu_baseline:
+            out["cpu_baseline"] = cpu_baseline_conv()
+        print(json.dumps(out))
         return
     if args.workload == "kernels":
         rows = kernel_table(max(args.steps, 1))
