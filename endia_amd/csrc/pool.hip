@@ -218,6 +218,51 @@ __global__ __launch_bounds__(TPB) void pool_bwd_row4_kernel(PoolP p, FastDiv d_w
   }
 }
 
+// Windows that tile the input (stride = kernel, no padding, unit dilation; the usual 2 x 2 / 2): an input
+// element lies in at most one window, found with one division per axis, so the gradient is one select
+// (or one scale) per element. KW = kernel width in {1, 2, 4}; a lane writes 4 consecutive elements.
+template <bool MAX, int KW>
+__global__ __launch_bounds__(TPB) void pool_bwd_tiling_kernel(PoolP p, FastDiv d_w4, const float* __restrict__ dy,
+                                                              const int32_t* __restrict__ arg, float* __restrict__ dx, float taps) {
+  constexpr int NWIN = 4 / KW;  // windows met by the lane's four elements
+  const int64_t stride = (int64_t)gridDim.x * TPB;
+  const int64_t ovol = (int64_t)p.Do * p.Ho * p.Wo;
+  const int W4 = p.W >> 2;
+  for (int64_t j = (int64_t)blockIdx.x * TPB + threadIdx.x; j < (p.n_in >> 2); j += stride) {
+    uint32_t plane;
+    int z, yy, x4;
+    decode((uint32_t)j, d_w4, p.d_h, p.d_d, W4, p.H, p.D, plane, z, yy, x4);
+    const int oz = (int)fdiv((uint32_t)z, p.d_sd), oy = (int)fdiv((uint32_t)yy, p.d_sh), ox0 = x4 * NWIN;
+    float out[4] = {0.f, 0.f, 0.f, 0.f};
+    if (oz < p.Do && oy < p.Ho) {  // rows and slabs past the last whole window receive no gradient
+      const int64_t row = plane * ovol + ((int64_t)oz * p.Ho + oy) * p.Wo;
+      const int self0 = (z * p.H + yy) * p.W + x4 * 4;
+#pragma unroll
+      for (int w = 0; w < NWIN; ++w) {
+        if (ox0 + w >= p.Wo) break;
+        const float g = dy[row + ox0 + w];
+        if (MAX) {
+          const int at = arg[row + ox0 + w];
+#pragma unroll
+          for (int e = 0; e < KW; ++e) out[w * KW + e] = at == self0 + w * KW + e ? g : 0.f;
+        } else {
+#pragma unroll
+          for (int e = 0; e < KW; ++e) out[w * KW + e] = g / taps;
+        }
+      }
+    }
+    reinterpret_cast<float4*>(dx)[j] = make_float4(out[0], out[1], out[2], out[3]);
+  }
+}
+
+template <bool MAX>
+void launch_tiling(const PoolP& p, FastDiv d_w4, int grid, hipStream_t s, const float* dy, const int32_t* arg, float* dx) {
+  const float inv = (float)(p.kd * p.kh * p.kw);  // every tap of every window lies inside the array
+  if (p.kw == 1) hipLaunchKernelGGL((pool_bwd_tiling_kernel<MAX, 1>), dim3(grid), dim3(TPB), 0, s, p, d_w4, dy, arg, dx, inv);
+  else if (p.kw == 2) hipLaunchKernelGGL((pool_bwd_tiling_kernel<MAX, 2>), dim3(grid), dim3(TPB), 0, s, p, d_w4, dy, arg, dx, inv);
+  else hipLaunchKernelGGL((pool_bwd_tiling_kernel<MAX, 4>), dim3(grid), dim3(TPB), 0, s, p, d_w4, dy, arg, dx, inv);
+}
+
 int32_t make_params(const endia_hip_pool_desc* d, PoolP& p, const char* who) {
   if (!d) return endia::fail(ENDIA_HIP_ERR_INVALID, "%s: null descriptor", who);
   const int64_t in[3] = {d->D, d->H, d->W};
@@ -291,7 +336,14 @@ int32_t endia_hip_pool_bwd(const endia_hip_pool_desc* desc, int32_t mode, const 
   ENDIA_CHECK_ARG(mode != ENDIA_POOL_MAX || argmax, "endia_hip_pool_bwd: max pooling needs the argmax array of the forward");
   const int grid = stream_grid(p.n_in);
   const bool unit = p.dd == 1 && p.dh == 1 && p.dw == 1;
-  if (unit && p.W % 4 == 0 && (reinterpret_cast<uintptr_t>(dx) & 15) == 0) {
+  const bool tiling = unit && p.sd == p.kd && p.sh == p.kh && p.sw == p.kw && p.pd == 0 && p.ph == 0 && p.pw == 0 &&
+                      (p.kw == 1 || p.kw == 2 || p.kw == 4);
+  if (tiling && p.W % 4 == 0 && (reinterpret_cast<uintptr_t>(dx) & 15) == 0) {
+    const FastDiv d_w4 = make_fastdiv(p.W / 4);
+    const int g4 = stream_grid(p.n_in / 4);
+    if (mode == ENDIA_POOL_MAX) launch_tiling<true>(p, d_w4, g4, ctx().stream, dy, argmax, dx);
+    else launch_tiling<false>(p, d_w4, g4, ctx().stream, dy, argmax, dx);
+  } else if (unit && p.W % 4 == 0 && (reinterpret_cast<uintptr_t>(dx) & 15) == 0) {
     const FastDiv d_w4 = make_fastdiv(p.W / 4);
     const int g4 = stream_grid(p.n_in / 4);
     if (mode == ENDIA_POOL_MAX) hipLaunchKernelGGL((pool_bwd_row4_kernel<true>), dim3(g4), dim3(TPB), 0, ctx().stream, p, d_w4, dy, argmax, dx);

@@ -725,3 +725,28 @@ def test_strided_scatter(dev, golden):
     dev.call("endia_hip_strided_scatter", 2, L.i64_array([0, 3]), L.i64_array([4, 1]), 0, src, dst, 0, 0)
     with pytest.raises(L.EndiaHipError):
         dev.call("endia_hip_strided_scatter", 9, L.i64_array([1] * 9), L.i64_array([1] * 9), 0, src, dst, 0, 0)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("xs,k", [((3, 5, 10, 12), (2, 2)), ((2, 3, 11, 8), (3, 4)), ((2, 4, 9, 16), (2, 1)),
+                                   ((2, 2, 6, 7, 8), (2, 3, 2)), ((4, 3, 20), (4,)), ((1, 2, 5, 4), (7 - 2, 1))])
+def test_pool_bwd_tiling_windows(dev, xs, k):
+    """Windows that tile the input (stride = kernel, no padding) take a dedicated gradient kernel: the same
+    numbers as the oracle (bit for bit: one select or one division per element) and as torch, including
+    heights and depths that leave rows beyond the last whole window."""
+    import torch
+    import torch.nn.functional as TF
+    rng = np.random.default_rng(len(xs) * 100 + k[0])
+    x = rng.standard_normal(xs).astype(np.float32)
+    nsp = len(k)
+    zeros, ones = (0,) * nsp, (1,) * nsp
+    for mode, mname in ((L.POOL_MAX, "max"), (L.POOL_AVG, "avg")):
+        y, _ = _pool_run(dev, mode, x, None, k, k, zeros, ones)
+        gy = rng.standard_normal(y.shape).astype(np.float32)
+        _, dx = _pool_run(dev, mode, x, gy, k, k, zeros, ones)
+        np.testing.assert_array_equal(dx, R.pool_bwd(mname, x, gy, k, k, zeros, ones))
+        t = torch.tensor(x, dtype=torch.float64, requires_grad=True)
+        fn = {("max", 1): TF.max_pool1d, ("max", 2): TF.max_pool2d, ("max", 3): TF.max_pool3d,
+              ("avg", 1): TF.avg_pool1d, ("avg", 2): TF.avg_pool2d, ("avg", 3): TF.avg_pool3d}[(mname, nsp)]
+        (fn(t, k, k) * torch.tensor(gy, dtype=torch.float64)).sum().backward()
+        assert_close(dx, t.grad.numpy(), what=mname + " grad vs torch")
