@@ -152,33 +152,33 @@ def _extrapolate(fn, r1, r2, full):
     return max(t1 - r1 * per_row, 0.0) + full * per_row
 
 
-def cpu_baseline_hvp(rows=96):
-    """The reference's single-threaded path for one Hessian-vector product, composed from row slices: the 31
-    products of 1024 x 2048 x 2048 (11 NN, 9 NT, 11 TN, as the tape issues them) plus the elementwise and
-    reduction passes over [1024, 2048] arrays that the double backward adds (counted on the device trace)."""
+def cpu_baseline_hvp():
+    """The reference's single-threaded path for one Hessian-vector product, composed by op count: one full
+    product of each mode timed at its real shape (the tape issues 11 NN, 9 NT and 11 TN products of
+    1024 x 2048 x 2048) plus the elementwise and reduction passes over [1024, 2048] arrays that the double
+    backward adds (counted on the device trace)."""
     from oracle import endia_ref as R
     rng = np.random.default_rng(3)
     t_all0 = time.perf_counter()
     B, Wd = 1024, 2048
     X = rng.standard_normal((B, Wd)).astype(np.float32)
     W = (rng.standard_normal((Wd, Wd)) / np.sqrt(Wd)).astype(np.float32)
-    t_nn = _extrapolate(lambda r: R.matmul(X[:r], W), rows, 2 * rows, B)
-    t_nt = _extrapolate(lambda r: R.matmul(X[:r], W.T), rows, 2 * rows, B)
-    t_tn = _extrapolate(lambda r: R.matmul(X[:, :r].T, X), rows, 2 * rows, Wd)
-    Z = X[:128]
-    t_bin = _timed(lambda: R.binary("mul", Z, Z)) * (B / 128)
-    t_un = _timed(lambda: R.unary("sin", Z)) * (B / 128)
-    t_red = _timed(lambda: R.reduce_add(Z, [0])) * (B / 128)
+    t_nn = _timed(lambda: R.matmul(X, W))
+    t_nt = _timed(lambda: R.matmul(X, W.T))
+    t_tn = _timed(lambda: R.matmul(X.T, X))
+    t_bin = _timed(lambda: R.binary("mul", X, X))
+    t_un = _timed(lambda: R.unary("sin", X))
+    t_red = _timed(lambda: R.reduce_add(X, [0]))
     n_bin, n_un, n_red = 58, 12, 17
     step = 11 * t_nn + 9 * t_nt + 11 * t_tn + n_bin * t_bin + n_un * t_un + n_red * t_red
     return {"value": 1.0 / step, "unit": "HVP/s", "cores": 1, "kind": "port", "host_cores_available": os.cpu_count(),
             "seconds_per_step": step,
-            "sample": "ref-order CPU restatement (oracle/endia_ref.c, 1 thread): %d- and 2x%d-row slices of the NN, NT and TN products "
-                      "extrapolated linearly and composed as 11 + 9 + 11 products, plus %d binary, %d unary and %d reduction passes "
-                      "over [1024, 2048] timed on 128-row slices; %.1f s of CPU work" % (rows, rows, n_bin, n_un, n_red, time.perf_counter() - t_all0)}
+            "sample": "ref-order CPU restatement (oracle/endia_ref.c, 1 thread): one full 1024 x 2048 x 2048 product of each mode "
+                      "(NN, NT, TN) composed as 11 + 9 + 11 products, plus %d binary, %d unary and %d reduction passes over "
+                      "[1024, 2048], each timed once at full size; %.1f s of CPU work" % (n_bin, n_un, n_red, time.perf_counter() - t_all0)}
 
 
-def cpu_baseline_complex(rows=96):
+def cpu_baseline_complex(rows=512):
     """The reference's complex matmul (four real multiply-adds per element, matmul_op.mojo:201-238) on row slices
     of the 2048^3 products, composed as the step issues them: 4 forward (NN), 3 data gradients (NT), 4 weight
     gradients (TN)."""
@@ -199,13 +199,13 @@ def cpu_baseline_complex(rows=96):
 
 
 def cpu_baseline_conv():
-    """The reference's 7-deep convolution loop (conv2d_op.mojo:127-196) and the brute-force adjoints of it, on four
-    images of the batch of 64, extrapolated by 16; plus the ReLU / mean passes over those images' output."""
+    """The reference's 7-deep convolution loop (conv2d_op.mojo:127-196) and the brute-force adjoints of it, on 16
+    images of the batch of 64, extrapolated by 4; plus the ReLU / mean passes over those images' output."""
     from oracle import endia_ref as R
     rng = np.random.default_rng(5)
     t_all0 = time.perf_counter()
     C, H, K = 64, 56, 128
-    n_img = 4
+    n_img = 16
     x = rng.standard_normal((n_img, C, H, H)).astype(np.float32)
     w = (rng.standard_normal((K, C, 3, 3)) * np.sqrt(2.0 / (C * 9))).astype(np.float32)
     bias = rng.standard_normal(K).astype(np.float32)
@@ -218,8 +218,8 @@ def cpu_baseline_conv():
     step = t_fwd + t_bwd + t_ew
     return {"value": 1.0 / step, "unit": "steps/s", "cores": 1, "kind": "port", "host_cores_available": os.cpu_count(),
             "seconds_per_step": step, "forward_seconds": t_fwd, "gradients_seconds": t_bwd,
-            "sample": "ref-order CPU restatement (1 thread): forward loop and its adjoints (dx, dw, db) on 4 of the 64 "
-                      "images, extrapolated by 16, plus relu / relu-gradient / mean passes; %.1f s of CPU work"
+            "sample": "ref-order CPU restatement (1 thread): forward loop and its adjoints (dx, dw, db) on 16 of the 64 "
+                      "images, extrapolated by 4, plus relu / relu-gradient / mean passes; %.1f s of CPU work"
                       % (time.perf_counter() - t_all0)}
 
 
