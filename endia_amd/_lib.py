@@ -23,6 +23,7 @@ EW_MAX_INPUTS, EW_MAX_OUTPUTS, EW_MAX_SLOTS, EW_MAX_STEPS = 8, 4, 4, 48
 EPI_NONE, EPI_BIAS, EPI_BIAS_ACT, EPI_ACT_GRAD = range(4)
 ACT_FROM_OUTPUT = 0x100
 GEMM_ACCUMULATE = 0x200
+GEMM_COLSUM_B = 0x400
 CGEMM_4M, CGEMM_3M = 0, 1
 
 ERR_INVALID, ERR_NOT_INIT, ERR_RUNTIME, ERR_NOMEM, ERR_UNSUPPORTED = -1, -2, -3, -4, -5

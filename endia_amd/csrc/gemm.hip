@@ -48,6 +48,7 @@ struct GemmArgs {
   int act;        // endia_hip_unary_op
   int from_out;   // activation gradient from stored output instead of pre-activation
   int accumulate;
+  int colsum;     // also write sum_k B[k][n] to aux_out[n] (B MN-major; done by the work-groups of the first tile row)
 };
 
 __device__ __forceinline__ float act_fwd(int act, float z) {
@@ -91,8 +92,13 @@ __device__ __forceinline__ void epilogue_store(const GemmArgs& p, float* __restr
 
 // F = MFMA blocks per wave in each direction: F = 2 gives the 128 x 128 tile, F = 1 the 64 x 64 tile
 // used when the larger one would leave CUs without work.
-template <bool A_KMAJOR, bool B_KMAJOR, int EPI, int F>
+// SHORTK (64 x 64 tile only): the reduction is at most four K tiles long, which is the case of every product
+// of a small model (the reference's sine-fit MLP has K <= 128 throughout). Such launches are a handful of
+// work-groups whose time is a chain of global-load latencies, one per K tile; here the loads of all four tiles
+// are issued before anything else, so that latency is paid once.
+template <bool A_KMAJOR, bool B_KMAJOR, int EPI, int F, bool SHORTK = false>
 __global__ __launch_bounds__(NTHREADS, 4) void sgemm_mfma_kernel(GemmArgs p) {
+  static_assert(!SHORTK || F == 1, "the short-reduction variant exists for the 64 x 64 tile");
   constexpr int BM = 64 * F, BN = 64 * F;
   using LA = MatrixTileLoader<A_KMAJOR, BM, NTHREADS>;
   using LB = MatrixTileLoader<B_KMAJOR, BN, NTHREADS>;
@@ -123,6 +129,38 @@ __global__ __launch_bounds__(NTHREADS, 4) void sgemm_mfma_kernel(GemmArgs p) {
   floatx16 acc[F][F];
   zero_acc<F, F>(acc);
 
+  // Column sums of B (the bias gradient when C = A^T dY): the first tile row's groups add up their B tiles as
+  // they pass through LDS, one column per thread, k ascending.
+  float colsum = 0.f;
+  const bool do_colsum = !B_KMAJOR && EPI == ENDIA_EPI_NONE && p.colsum && tm == 0 && tid < BN;
+  auto add_colsum = [&]() {
+    if (do_colsum) {
+#pragma unroll 8
+      for (int k = 0; k < BK; ++k) colsum += Bs[k * TileShape<B_KMAJOR, BN>::LD + tid];
+    }
+  };
+
+  if constexpr (SHORTK) {
+    constexpr int DEPTH = 4;
+    float4 ra[DEPTH][LA::PASSES], rb[DEPTH][LB::PASSES];
+#pragma unroll
+    for (int t = 0; t < DEPTH; ++t) {  // tiles past the end of K load as zeros without touching memory
+      la.load_into(ra[t], K - t * BK);
+      lb.load_into(rb[t], K - t * BK);
+      la.advance();
+      lb.advance();
+    }
+#pragma unroll
+    for (int t = 0; t < DEPTH; ++t) {
+      if (t * BK >= K) break;
+      if (t) __syncthreads();
+      la.store_from(As, ra[t]);
+      lb.store_from(Bs, rb[t]);
+      __syncthreads();
+      add_colsum();
+      compute_ktile<A_KMAJOR, B_KMAJOR, F, F, BM, BN>(As, Bs, wm * 32 * F + l32, wn * 32 * F + l32, h, acc);
+    }
+  } else {
   la.load(K);
   lb.load(K);
   la.store(As);
@@ -137,6 +175,7 @@ __global__ __launch_bounds__(NTHREADS, 4) void sgemm_mfma_kernel(GemmArgs p) {
       la.load(K - k0 - BK);
       lb.load(K - k0 - BK);
     }
+    add_colsum();
     compute_ktile<A_KMAJOR, B_KMAJOR, F, F, BM, BN>(As, Bs, wm * 32 * F + l32, wn * 32 * F + l32, h, acc);
     if (more) {
       __syncthreads();
@@ -145,6 +184,9 @@ __global__ __launch_bounds__(NTHREADS, 4) void sgemm_mfma_kernel(GemmArgs p) {
       __syncthreads();
     }
   }
+  }
+
+  if (do_colsum && n0 + tid < p.N) p.aux_out[n0 + tid] = colsum;
 
 #pragma unroll
   for (int fm = 0; fm < F; ++fm)
@@ -244,22 +286,22 @@ __global__ __launch_bounds__(128) void sgemm_skinny_kernel(GemmArgs p, int trans
   }
 }
 
-template <int EPI, int F>
+template <int EPI, int F, bool SHORTK>
 void launch_mfma(const GemmArgs& p, int transA, int transB, dim3 grid, hipStream_t s) {
   const bool ak = !transA, bk = transB != 0;
-  if (ak && bk) hipLaunchKernelGGL((sgemm_mfma_kernel<true, true, EPI, F>), grid, dim3(NTHREADS), 0, s, p);
-  else if (ak && !bk) hipLaunchKernelGGL((sgemm_mfma_kernel<true, false, EPI, F>), grid, dim3(NTHREADS), 0, s, p);
-  else if (!ak && bk) hipLaunchKernelGGL((sgemm_mfma_kernel<false, true, EPI, F>), grid, dim3(NTHREADS), 0, s, p);
-  else hipLaunchKernelGGL((sgemm_mfma_kernel<false, false, EPI, F>), grid, dim3(NTHREADS), 0, s, p);
+  if (ak && bk) hipLaunchKernelGGL((sgemm_mfma_kernel<true, true, EPI, F, SHORTK>), grid, dim3(NTHREADS), 0, s, p);
+  else if (ak && !bk) hipLaunchKernelGGL((sgemm_mfma_kernel<true, false, EPI, F, SHORTK>), grid, dim3(NTHREADS), 0, s, p);
+  else if (!ak && bk) hipLaunchKernelGGL((sgemm_mfma_kernel<false, true, EPI, F, SHORTK>), grid, dim3(NTHREADS), 0, s, p);
+  else hipLaunchKernelGGL((sgemm_mfma_kernel<false, false, EPI, F, SHORTK>), grid, dim3(NTHREADS), 0, s, p);
 }
 
-template <int F>
+template <int F, bool SHORTK = false>
 void launch_mfma_epi(const GemmArgs& p, int epi, int transA, int transB, dim3 grid, hipStream_t s) {
   switch (epi) {
-    case ENDIA_EPI_NONE: launch_mfma<ENDIA_EPI_NONE, F>(p, transA, transB, grid, s); break;
-    case ENDIA_EPI_BIAS: launch_mfma<ENDIA_EPI_BIAS, F>(p, transA, transB, grid, s); break;
-    case ENDIA_EPI_BIAS_ACT: launch_mfma<ENDIA_EPI_BIAS_ACT, F>(p, transA, transB, grid, s); break;
-    default: launch_mfma<ENDIA_EPI_ACT_GRAD, F>(p, transA, transB, grid, s); break;
+    case ENDIA_EPI_NONE: launch_mfma<ENDIA_EPI_NONE, F, SHORTK>(p, transA, transB, grid, s); break;
+    case ENDIA_EPI_BIAS: launch_mfma<ENDIA_EPI_BIAS, F, SHORTK>(p, transA, transB, grid, s); break;
+    case ENDIA_EPI_BIAS_ACT: launch_mfma<ENDIA_EPI_BIAS_ACT, F, SHORTK>(p, transA, transB, grid, s); break;
+    default: launch_mfma<ENDIA_EPI_ACT_GRAD, F, SHORTK>(p, transA, transB, grid, s); break;
   }
 }
 
@@ -296,6 +338,7 @@ int32_t sgemm_impl(int transA, int transB, int64_t M, int64_t N, int64_t K, cons
                    const float* aux_in, float* aux_out) {
   const int epi = epi_flags & 0xff;
   const int accumulate = (epi_flags & ENDIA_GEMM_ACCUMULATE) ? 1 : 0;
+  const int colsum = (epi_flags & ENDIA_GEMM_COLSUM_B) ? 1 : 0;
   const int act = act_flags & 0xff;
   const int from_out = (act_flags & ENDIA_ACT_FROM_OUTPUT) ? 1 : 0;
   ENDIA_CHECK_ARG(M >= 0 && N >= 0 && K >= 0 && batch >= 0, "sgemm: negative dimension (M=%lld N=%lld K=%lld batch=%lld)",
@@ -303,11 +346,14 @@ int32_t sgemm_impl(int transA, int transB, int64_t M, int64_t N, int64_t K, cons
   ENDIA_CHECK_ARG(M < (1ll << 31) && N < (1ll << 31) && K < (1ll << 31) && batch <= 65535,
                   "sgemm: dimension too large");
   ENDIA_CHECK_ARG(epi >= ENDIA_EPI_NONE && epi <= ENDIA_EPI_ACT_GRAD, "sgemm: unknown epilogue %d", epi);
-  ENDIA_CHECK_ARG((epi_flags & ~(0xff | ENDIA_GEMM_ACCUMULATE)) == 0, "sgemm: unknown epilogue flag bits 0x%x", epi_flags);
+  ENDIA_CHECK_ARG((epi_flags & ~(0xff | ENDIA_GEMM_ACCUMULATE | ENDIA_GEMM_COLSUM_B)) == 0, "sgemm: unknown epilogue flag bits 0x%x", epi_flags);
+  ENDIA_CHECK_ARG(!colsum || (epi == ENDIA_EPI_NONE && !transB && batch == 1 && ldb == N && aux_out != nullptr),
+                  "sgemm: COLSUM_B needs the plain epilogue, transB = 0, batch = 1, ldb = N and aux_out");
   ENDIA_CHECK_ARG(act == ENDIA_OP_RELU || act == ENDIA_OP_TANH || act == ENDIA_OP_SIN || act == ENDIA_OP_IDENTITY,
                   "sgemm: activation %d is not one of relu/tanh/sin/identity", act);
   ENDIA_CHECK_ARG(!(from_out && act == ENDIA_OP_SIN), "sgemm: sin gradient needs the pre-activation, not the output");
-  if (M == 0 || N == 0 || batch == 0) return ENDIA_HIP_OK;
+  if (N == 0 || batch == 0) return ENDIA_HIP_OK;
+  if (M == 0) return colsum ? col_reduce(1, K, N, B, aux_out, 1.f) : ENDIA_HIP_OK;
   ENDIA_CHECK_ARG(C != nullptr, "sgemm: C is null");
   ENDIA_CHECK_ARG(K == 0 || (A != nullptr && B != nullptr), "sgemm: A or B is null");
   ENDIA_CHECK_ARG(lda >= (transA ? M : K) && ldb >= (transB ? K : N) && ldc >= N,
@@ -321,6 +367,7 @@ int32_t sgemm_impl(int transA, int transB, int64_t M, int64_t N, int64_t K, cons
   GemmArgs p;
   p.A = A; p.B = B; p.C = C; p.bias = bias; p.aux_in = aux_in;
   p.aux_out = (epi == ENDIA_EPI_BIAS_ACT) ? aux_out : nullptr;
+  p.colsum = 0;
   p.lda = lda; p.ldb = ldb; p.ldc = ldc; p.sA = sA; p.sB = sB; p.sC = sC;
   p.M = (int)M; p.N = (int)N; p.K = (int)K;
   p.act = act; p.from_out = from_out; p.accumulate = accumulate;
@@ -359,6 +406,13 @@ int32_t sgemm_impl(int transA, int transB, int64_t M, int64_t N, int64_t K, cons
     PoolBuf part;
     float* const C_final = C;
     p.k_split = 0;
+    // Small B: the launch below produces the column sums as well (a launch saved where launches are what a step
+    // costs). For a large B the first tile row's groups would finish last and hold up the whole launch, and the
+    // separate streaming reduction is cheaper.
+    if (colsum && splits == 1 && K * N <= (1ll << 20)) {
+      p.colsum = 1;
+      p.aux_out = aux_out;
+    }
     if (splits > 1) {
       int64_t chunk = ceil_div64(ceil_div64(K, splits), BK) * BK;
       splits = ceil_div64(K, chunk);
@@ -384,6 +438,7 @@ int32_t sgemm_impl(int transA, int transB, int64_t M, int64_t N, int64_t K, cons
       ENDIA_HIP_CALL(hipEventRecord(g_timing.start[g_timing.used], s));
     }
     if (F == 2) launch_mfma_epi<2>(p, epi, transA, transB, grid, s);
+    else if (K <= 4 * BK && splits == 1) launch_mfma_epi<1, true>(p, epi, transA, transB, grid, s);
     else launch_mfma_epi<1>(p, epi, transA, transB, grid, s);
     if (timed) {
       ENDIA_HIP_CALL(hipEventRecord(g_timing.stop[g_timing.used], s));
@@ -392,7 +447,8 @@ int32_t sgemm_impl(int transA, int transB, int64_t M, int64_t N, int64_t K, cons
     }
     if (splits > 1) {
       ENDIA_LAUNCH_CHECK();
-      return col_reduce(1, splits, M * N, p.C, C_final, 1.f);  // partials added in slice order
+      int32_t rc = col_reduce(1, splits, M * N, p.C, C_final, 1.f);  // partials added in slice order
+      if (rc || !colsum) return rc;
     }
   } else if (epi == ENDIA_EPI_NONE && M * N <= 2048 && K >= 64) {
     p.k_split = 0;
@@ -411,6 +467,7 @@ int32_t sgemm_impl(int transA, int transB, int64_t M, int64_t N, int64_t K, cons
     }
   }
   ENDIA_LAUNCH_CHECK();
+  if (colsum && !p.colsum) return col_reduce(1, K, N, B, aux_out, 1.f);  // paths that do not fuse it
   return ENDIA_HIP_OK;
 }
 

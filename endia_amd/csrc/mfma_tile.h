@@ -167,6 +167,20 @@ struct MatrixTileLoader {
       reg[i] = buffer_load_f4(rs, o);
     }
   }
+  // The same two steps with the staging registers held by the caller (several tiles in flight at once).
+  __device__ __forceinline__ void load_into(float4 (&dst)[PASSES], int k_left) {
+    __amdgpu_buffer_rsrc_t rs = make_rsrc(base, records);
+#pragma unroll
+    for (int i = 0; i < PASSES; ++i) {
+      uint32_t o = voff[i];
+      if (KMAJOR) o = (c < k_left) ? o : OOB_OFFSET;
+      dst[i] = buffer_load_f4(rs, o);
+    }
+  }
+  __device__ __forceinline__ void store_from(float* lds, const float4 (&src)[PASSES]) {
+#pragma unroll
+    for (int i = 0; i < PASSES; ++i) *reinterpret_cast<float4*>(&lds[lds_off + i * ROWS_PER_PASS * LD]) = src[i];
+  }
   __device__ __forceinline__ void advance() {
     base = reinterpret_cast<const float*>(reinterpret_cast<const char*>(base) + step);
     records -= step;

@@ -1176,15 +1176,17 @@ def _linear_node(out, x, W, b, xs, Ws, act):
             L.call("endia_hip_unary_vjp_from_output", _ACT[act], B * N, out_.data_ptr(), g.data_ptr(), gp.data_ptr())
             g = gp
         res = [None, None, None]
+        db = Array.empty([1, N]) if pb._requires_grad else None  # kept leading axis, like Expand.vjp (expand_op.mojo:121-126)
         if pW._requires_grad:
             dW = Array.empty([K, N])
+            # the weight-gradient launch also sums the columns of g: the bias gradient costs no launch of its own
             L.call("endia_hip_sgemm", 1, 0, K, N, B, xs.data_ptr(), K, g.data_ptr(), N, dW.data_ptr(), N, 1, 0, 0, 0,
-                   L.EPI_NONE, L.OP_IDENTITY, None, None, None)
+                   L.EPI_NONE | (L.GEMM_COLSUM_B if db is not None else 0), L.OP_IDENTITY, None, None,
+                   db.data_ptr() if db is not None else None)
             res[1] = dW
-        if pb._requires_grad:
-            db = Array.empty([1, N])  # kept leading axis, like Expand.vjp (expand_op.mojo:121-126)
+        elif db is not None:
             L.call("endia_hip_reduce_add", 2, L.i64_array([B, N]), 1, g.data_ptr(), db.data_ptr(), 1.0, 0)
-            res[2] = db
+        res[2] = db
         if px._requires_grad:
             dx = Array.empty([B, K])
             pm = _fused_act_of(px)

@@ -94,6 +94,9 @@ typedef enum {
 } endia_hip_epilogue;
 #define ENDIA_ACT_FROM_OUTPUT 0x100
 #define ENDIA_GEMM_ACCUMULATE 0x200 /* or'ed into `epilogue`: C += result instead of C = result */
+#define ENDIA_GEMM_COLSUM_B 0x400  /* or'ed into `epilogue` (with ENDIA_EPI_NONE, transB = 0, batch = 1, ldb = N): aux_out[n] also
+                                      receives sum_k B[k][n]. With C = A^T dY this is the bias gradient, the VJP of the broadcast
+                                      bias add (expand_op.mojo:121-126), produced by the weight-gradient launch itself */
 
 typedef enum { ENDIA_CGEMM_4M = 0, ENDIA_CGEMM_3M = 1 } endia_hip_cgemm_algo;
 
@@ -166,10 +169,10 @@ ENDIA_API int32_t endia_hip_strided_scatter(int32_t ndim, const int64_t* shape, 
  *      (m,k) at A[k*lda + m]. Same for B (K x N, or stored N x K when transB = 1). The transposed
  *      forms replace the reference's materialised .T() copies (matmul_op.mojo:111-136).
  *      batch >= 1; a batch stride of 0 broadcasts that operand (matmul_op.mojo:162-165).
- *      epilogue: endia_hip_epilogue, optionally | ENDIA_GEMM_ACCUMULATE.
+ *      epilogue: endia_hip_epilogue, optionally | ENDIA_GEMM_ACCUMULATE | ENDIA_GEMM_COLSUM_B.
  *      act: endia_hip_unary_op in {RELU,TANH,SIN,IDENTITY}, optionally | ENDIA_ACT_FROM_OUTPUT.
  *      bias: N floats (BIAS, BIAS_ACT) else null.  aux_in: M x N, row stride ldc (ACT_GRAD) else null.
- *      aux_out: M x N, row stride ldc, or null (BIAS_ACT only). */
+ *      aux_out: M x N, row stride ldc, or null (BIAS_ACT); N floats (COLSUM_B). */
 ENDIA_API int32_t endia_hip_sgemm(int32_t transA, int32_t transB, int64_t M, int64_t N, int64_t K,
                         const float* A, int64_t lda, const float* B, int64_t ldb, float* C, int64_t ldc,
                         int64_t batch, int64_t strideA, int64_t strideB, int64_t strideC,

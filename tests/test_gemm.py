@@ -28,7 +28,8 @@ def run_sgemm(dev, A, B, ta, tb, M, N, K, epi=L.EPI_NONE, act=L.OP_IDENTITY, bia
 
 SHAPES = [(128, 128, 32), (256, 384, 72), (132, 260, 100), (37, 53, 19), (4, 4, 4), (1, 1, 1), (128, 1, 32),
           (1, 32, 128), (300, 200, 8), (64, 64, 1024), (64, 96, 8192), (128, 200, 5000), (72, 64, 2052),
-          (32, 1, 128), (3, 5, 1000), (40, 50, 64), (1, 1, 4096)]  # few outputs, long reduction: one work-group per output
+          (32, 1, 128), (3, 5, 1000), (40, 50, 64), (1, 1, 4096),  # few outputs, long reduction: one work-group per output
+          (128, 128, 128), (128, 64, 96), (64, 128, 36), (132, 68, 124), (128, 32, 132)]  # reductions of 1-4 K tiles, and just past
 
 
 @pytest.mark.parametrize("ta,tb", [(0, 0), (0, 1), (1, 0), (1, 1)])
@@ -209,3 +210,24 @@ def test_cgemm_all_flag_combinations(dev, algo, M, N, K, pad):
                     assert_close(got[:, :N], want + C0, what=what)
                     np.testing.assert_array_equal(got[:, N:], Cp[:, N:], err_msg=what + ": padding columns of C touched")
                     dev.release()
+
+
+@pytest.mark.parametrize("M,N,K", [(128, 128, 128), (64, 96, 40), (256, 384, 520), (32, 1, 128), (3, 5, 1000), (128, 200, 5000),
+                                   (37, 53, 19), (64, 64, 4096)])
+def test_sgemm_colsum_b(dev, M, N, K):
+    """ENDIA_GEMM_COLSUM_B: C = A^T B as before, and aux_out[n] = sum_k B[k][n] from the same call, whichever
+    kernel the shape selects (fused in the MFMA kernels, a separate reduction on the other paths and under split-K)."""
+    rng = np.random.default_rng(M + N + K)
+    A = rng.standard_normal((K, M)).astype(np.float32)
+    B = rng.standard_normal((K, N)).astype(np.float32)
+    dA, dB = dev.put(A), dev.put(B)
+    dC, dsum = dev.put(np.full((M, N), np.nan, np.float32)), dev.put(np.full(N, np.nan, np.float32))
+    dev.call("endia_hip_sgemm", 1, 0, M, N, K, dA, M, dB, N, dC, N, 1, 0, 0, 0, L.EPI_NONE | L.GEMM_COLSUM_B, L.OP_IDENTITY,
+             None, None, dsum)
+    assert_close(dev.get(dC, (M, N)), A.astype(np.float64).T @ B.astype(np.float64), what="C")
+    assert_close(dev.get(dsum, (N,)), B.astype(np.float64).sum(0), tol=1e-5, what="column sums")
+    assert_close(dev.get(dsum, (N,)), R.reduce_add(B, [0]).reshape(-1), tol=1e-5, what="column sums vs oracle")
+    for bad in [(1, 1), (0, 0)]:   # transB = 1, or a fused epilogue, is refused
+        with pytest.raises(L.EndiaHipError):
+            dev.call("endia_hip_sgemm", 1, bad[0], M, N, K, dA, M, dB, N if not bad[0] else K, dC, N, 1, 0, 0, 0,
+                     (L.EPI_NONE if bad[0] else L.EPI_BIAS) | L.GEMM_COLSUM_B, L.OP_IDENTITY, dsum, None, dsum)

@@ -526,9 +526,10 @@ def test_pool_reuses_buffers(dev):
     dev._live.remove(p)
     dev.call("endia_hip_pool_stats", ctypes.byref(u), ctypes.byref(c), ctypes.byref(n0))
     q = dev.alloc(1 << 20)
+    assert q  # (which cached buffer of the bucket comes back is not specified)
     n1 = ctypes.c_int64()
     dev.call("endia_hip_pool_stats", ctypes.byref(u), ctypes.byref(c), ctypes.byref(n1))
-    assert q == p and n1.value == n0.value  # same buffer, no new device allocation
+    assert n1.value == n0.value  # served from the cached buffers of that size: no new device allocation
     assert L.lib().endia_hip_free(ctypes.c_void_p(12345)) == L.ERR_INVALID
 
 
