@@ -22,6 +22,19 @@ def building_graph():
     return _building_graph[0]
 
 
+_SEED = []
+
+
+def _seed_one():
+    """ones(1), the seed of a scalar output (functional.mojo:34-38). It is read, never written, so one array
+    serves every backward pass and a step spends no launch on filling it."""
+    if not _SEED:
+        seed = F.ones([1])
+        seed._is_seed = True
+        _SEED.append(seed)
+    return _SEED[0]
+
+
 def top_order(out):
     """Post-order DFS over args (general.mojo:26-32), iterative so deep graphs do not hit the
     interpreter's recursion limit."""
@@ -60,8 +73,7 @@ def jacrev(arg, create_graph=False):
         n = out.size()
         seed = F.reshape(F.eye(n), out.shape() + out.shape())
     else:
-        seed = F.ones([dims])
-        seed._is_seed = True
+        seed = _seed_one()
     out.grad_(seed)
 
     prev = _building_graph[0]

@@ -265,13 +265,14 @@ __global__ __launch_bounds__(256) void sgemm_generic_kernel(GemmArgs p, int tran
 __global__ __launch_bounds__(128) void sgemm_skinny_kernel(GemmArgs p, int transA, int transB) {
   __shared__ float red[2];
   const int out = blockIdx.x;
-  const int m = out / p.N, n = out - m * p.N;
+  const bool colsum = out >= p.M * p.N;  // the groups past the last output element sum the columns of B
+  const int m = colsum ? 0 : out / p.N, n = colsum ? out - p.M * p.N : out - m * p.N;
   const int64_t bz = blockIdx.y;
   const float* __restrict__ A = p.A + bz * p.sA;
   const float* __restrict__ B = p.B + bz * p.sB;
   float acc = 0.f;
   for (int k = threadIdx.x; k < p.K; k += 128) {
-    const float a = transA ? A[(int64_t)k * p.lda + m] : A[(int64_t)m * p.lda + k];
+    const float a = colsum ? 1.f : (transA ? A[(int64_t)k * p.lda + m] : A[(int64_t)m * p.lda + k]);
     const float b = transB ? B[(int64_t)n * p.ldb + k] : B[(int64_t)k * p.ldb + n];
     acc = fmaf(a, b, acc);
   }
@@ -280,9 +281,13 @@ __global__ __launch_bounds__(128) void sgemm_skinny_kernel(GemmArgs p, int trans
   if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = acc;
   __syncthreads();
   if (threadIdx.x == 0) {
-    float* c = p.C + bz * p.sC + (int64_t)m * p.ldc + n;
     const float v = red[0] + red[1];
-    *c = p.accumulate ? *c + v : v;
+    if (colsum) {
+      p.aux_out[n] = v;
+    } else {
+      float* c = p.C + bz * p.sC + (int64_t)m * p.ldc + n;
+      *c = p.accumulate ? *c + v : v;
+    }
   }
 }
 
@@ -452,7 +457,11 @@ int32_t sgemm_impl(int transA, int transB, int64_t M, int64_t N, int64_t K, cons
     }
   } else if (epi == ENDIA_EPI_NONE && M * N <= 2048 && K >= 64) {
     p.k_split = 0;
-    hipLaunchKernelGGL(sgemm_skinny_kernel, dim3((unsigned)(M * N), (unsigned)batch), dim3(128), 0, s, p, transA, transB);
+    if (colsum) {  // N more groups produce the column sums of B in the same launch
+      p.colsum = 1;
+      p.aux_out = aux_out;
+    }
+    hipLaunchKernelGGL(sgemm_skinny_kernel, dim3((unsigned)(M * N + (colsum ? N : 0)), (unsigned)batch), dim3(128), 0, s, p, transA, transB);
   } else {
     p.k_split = 0;
     p.tiles_m = (int)ceil_div64(M, 64);

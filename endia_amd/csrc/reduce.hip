@@ -162,7 +162,7 @@ __global__ __launch_bounds__(TPB) void generic_reduce_kernel(RedDesc d, const fl
 // One pass: dpred = 2 (p - t) / n and per-group partial sums of (p - t)^2.
 __global__ __launch_bounds__(TPB) void mse_kernel(const float* __restrict__ p, const float* __restrict__ t,
                                                   float* __restrict__ dp, float* __restrict__ part, int64_t n,
-                                                  float two_over_n, int vec) {
+                                                  float two_over_n, int vec, float part_scale) {
   __shared__ float red[4];
   int64_t i = (int64_t)blockIdx.x * TPB + threadIdx.x;
   int64_t stride = (int64_t)gridDim.x * TPB;
@@ -191,7 +191,7 @@ __global__ __launch_bounds__(TPB) void mse_kernel(const float* __restrict__ p, c
     }
   }
   float s = block_sum(acc, red);
-  if (part && threadIdx.x == 0) part[blockIdx.x] = s;
+  if (part && threadIdx.x == 0) part[blockIdx.x] = s * part_scale;
 }
 
 __global__ __launch_bounds__(TPB) void sum_partials_kernel(const float* __restrict__ part, float* __restrict__ out,
@@ -348,16 +348,20 @@ int32_t endia_hip_mse_fwd_bwd(int64_t n, const float* pred, const float* target,
   int64_t cap = (int64_t)ctx().cu_count * 8;
   if (blocks > cap) blocks = cap;
   float* part = nullptr;
-  if (loss) {
+  float part_scale = 1.f;
+  const float inv_n = 1.0f / (float)n;
+  if (loss && blocks == 1) {  // a single group: its sum is the loss, no second launch
+    part = loss;
+    part_scale = inv_n;
+  } else if (loss) {
     void* ws = nullptr;
     int32_t rc = workspace(blocks * (int64_t)sizeof(float), &ws);
     if (rc) return rc;
     part = static_cast<float*>(ws);
   }
-  const float inv_n = 1.0f / (float)n;
-  hipLaunchKernelGGL(mse_kernel, dim3((unsigned)blocks), dim3(TPB), 0, s, pred, target, dpred, part, n, 2.0f * inv_n, vec);
+  hipLaunchKernelGGL(mse_kernel, dim3((unsigned)blocks), dim3(TPB), 0, s, pred, target, dpred, part, n, 2.0f * inv_n, vec, part_scale);
   ENDIA_LAUNCH_CHECK();
-  if (loss) {
+  if (loss && blocks > 1) {
     hipLaunchKernelGGL(sum_partials_kernel, dim3(1), dim3(TPB), 0, s, part, loss, blocks, inv_n);
     ENDIA_LAUNCH_CHECK();
   }
