@@ -87,6 +87,7 @@ SIGNATURES = {
     "endia_hip_strided_scatter": [c_int32, _i64p, _i64p, c_int64, _fp, _fp, c_int32, c_int32],
     "endia_hip_sgemm": [c_int32, c_int32, c_int64, c_int64, c_int64, _fp, c_int64, _fp, c_int64, _fp, c_int64,
                         c_int64, c_int64, c_int64, c_int64, c_int32, c_int32, _fp, _fp, _fp],
+    "endia_hip_linear_bwd": [c_int64, c_int64, c_int64, _fp, _fp, _fp, c_int32, _fp, _fp, _fp, _fp],
     "endia_hip_cgemm": [c_int32, c_int32, c_int32, c_int32, c_int64, c_int64, c_int64, _fp, c_int64, _fp, c_int64,
                         _fp, c_int64, c_int64, c_int64, c_int64, c_int64, c_int32, c_int32],
     "endia_hip_unary_fwd": [c_int32, c_int64, _fp, _fp, c_int32],

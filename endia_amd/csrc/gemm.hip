@@ -96,14 +96,14 @@ __device__ __forceinline__ void epilogue_store(const GemmArgs& p, float* __restr
 // of a small model (the reference's sine-fit MLP has K <= 128 throughout). Such launches are a handful of
 // work-groups whose time is a chain of global-load latencies, one per K tile; here the loads of all four tiles
 // are issued before anything else, so that latency is paid once.
-template <bool A_KMAJOR, bool B_KMAJOR, int EPI, int F, bool SHORTK = false>
-__global__ __launch_bounds__(NTHREADS, 4) void sgemm_mfma_kernel(GemmArgs p) {
+// One work-group's tile of one product: group `block` of `nblocks`, batch entry (or K slice) bz, LDS handed in.
+template <bool A_KMAJOR, bool B_KMAJOR, int EPI, int F, bool SHORTK>
+__device__ __forceinline__ void gemm_tile(const GemmArgs& p, int block, int nblocks, int64_t bz, float* __restrict__ As,
+                                          float* __restrict__ Bs) {
   static_assert(!SHORTK || F == 1, "the short-reduction variant exists for the 64 x 64 tile");
   constexpr int BM = 64 * F, BN = 64 * F;
   using LA = MatrixTileLoader<A_KMAJOR, BM, NTHREADS>;
   using LB = MatrixTileLoader<B_KMAJOR, BN, NTHREADS>;
-  __shared__ __attribute__((aligned(16))) float As[TileShape<A_KMAJOR, BM>::FLOATS];
-  __shared__ __attribute__((aligned(16))) float Bs[TileShape<B_KMAJOR, BN>::FLOATS];
 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
@@ -112,9 +112,8 @@ __global__ __launch_bounds__(NTHREADS, 4) void sgemm_mfma_kernel(GemmArgs p) {
   const int l32 = lane & 31, h = lane >> 5;
 
   int tm, tn;
-  tile_of_block(blockIdx.x, gridDim.x, p.tiles_m, p.tiles_n, tm, tn);
+  tile_of_block(block, nblocks, p.tiles_m, p.tiles_n, tm, tn);
   const int m0 = tm * BM, n0 = tn * BN;
-  const int64_t bz = blockIdx.y;
   float* __restrict__ C = p.C + bz * p.sC;
   const float* __restrict__ aux_in = p.aux_in ? p.aux_in + bz * p.sC : nullptr;
   float* __restrict__ aux_out = p.aux_out ? p.aux_out + bz * p.sC : nullptr;
@@ -200,6 +199,26 @@ __global__ __launch_bounds__(NTHREADS, 4) void sgemm_mfma_kernel(GemmArgs p) {
         if (row < p.M) epilogue_store<EPI>(p, C, aux_in, aux_out, row, col, acc[fm][fn][v]);
       }
     }
+}
+
+template <bool A_KMAJOR, bool B_KMAJOR, int EPI, int F, bool SHORTK = false>
+__global__ __launch_bounds__(NTHREADS, 4) void sgemm_mfma_kernel(GemmArgs p) {
+  __shared__ __attribute__((aligned(16))) float As[TileShape<A_KMAJOR, 64 * F>::FLOATS];
+  __shared__ __attribute__((aligned(16))) float Bs[TileShape<B_KMAJOR, 64 * F>::FLOATS];
+  gemm_tile<A_KMAJOR, B_KMAJOR, EPI, F, SHORTK>(p, blockIdx.x, gridDim.x, blockIdx.y, As, Bs);
+}
+
+// Backward of a small dense layer in ONE launch: the first nx work-groups compute the tiles of
+// dx = (g W^T) * act'(aux) (both operands K-major, activation-gradient or plain epilogue), the others the tiles of
+// dW = x^T g (both MN-major) and, in their first tile row, db = column sums of g. Both reductions are at most four
+// K tiles long. For models of this size a step costs what its launches cost, and this halves the backward's.
+template <int EPI_X>
+__global__ __launch_bounds__(NTHREADS, 4) void linear_bwd_small_kernel(GemmArgs px, GemmArgs pw, int nx) {
+  static_assert(TileShape<true, 64>::FLOATS == TileShape<false, 64>::FLOATS, "one LDS pair serves both layouts");
+  __shared__ __attribute__((aligned(16))) float As[TileShape<true, 64>::FLOATS];
+  __shared__ __attribute__((aligned(16))) float Bs[TileShape<true, 64>::FLOATS];
+  if ((int)blockIdx.x < nx) gemm_tile<true, true, EPI_X, 1, true>(px, blockIdx.x, nx, 0, As, Bs);
+  else gemm_tile<false, false, ENDIA_EPI_NONE, 1, true>(pw, blockIdx.x - nx, gridDim.x - nx, 0, As, Bs);
 }
 
 // Fallback for operands the vector path cannot take (leading dimensions, sizes or pointers that are
@@ -480,7 +499,56 @@ int32_t sgemm_impl(int transA, int transB, int64_t M, int64_t N, int64_t K, cons
   return ENDIA_HIP_OK;
 }
 
+// dx = (g W^T) * act'(aux), dW = x^T g, db = column sums of g; see endia_hip_linear_bwd.
+int32_t linear_bwd_impl(int64_t B, int64_t K, int64_t N, const float* x, const float* W, const float* g, int act_flags,
+                        const float* aux, float* dx, float* dW, float* db) {
+  ENDIA_CHECK_ARG(B >= 0 && K >= 0 && N >= 0, "linear_bwd: negative dimension");
+  ENDIA_CHECK_ARG(g != nullptr || B * N == 0, "linear_bwd: g is null");
+  ENDIA_CHECK_ARG(!dx || W, "linear_bwd: dx needs W");
+  ENDIA_CHECK_ARG(!dW || x, "linear_bwd: dW needs x");
+  const int epi_x = aux ? ENDIA_EPI_ACT_GRAD : ENDIA_EPI_NONE;
+  const int act = act_flags & 0xff;
+  // One launch for all three when every operand takes the vector path and both reductions fit four K tiles.
+  const bool small = dx && dW && db && B > 0 && K > 0 && N > 0 && N <= 4 * BK && B <= 4 * BK && K % 4 == 0 && N % 4 == 0 &&
+                     N >= 8 && B >= 8 && aligned16(x) && aligned16(W) && aligned16(g) &&
+                     (act == ENDIA_OP_RELU || act == ENDIA_OP_TANH || act == ENDIA_OP_SIN || act == ENDIA_OP_IDENTITY) &&
+                     !((act_flags & ENDIA_ACT_FROM_OUTPUT) && act == ENDIA_OP_SIN);
+  if (small) {
+    GemmArgs px{}, pw{};
+    px.A = g; px.B = W; px.C = dx; px.aux_in = aux; px.lda = N; px.ldb = N; px.ldc = K;
+    px.M = (int)B; px.N = (int)K; px.K = (int)N;
+    px.tiles_m = (int)ceil_div64(B, 64); px.tiles_n = (int)ceil_div64(K, 64);
+    px.act = act; px.from_out = (act_flags & ENDIA_ACT_FROM_OUTPUT) ? 1 : 0;
+    pw.A = x; pw.B = g; pw.C = dW; pw.aux_out = db; pw.lda = K; pw.ldb = N; pw.ldc = N;
+    pw.M = (int)K; pw.N = (int)N; pw.K = (int)B;
+    pw.tiles_m = (int)ceil_div64(K, 64); pw.tiles_n = (int)ceil_div64(N, 64);
+    pw.act = ENDIA_OP_IDENTITY; pw.colsum = 1;
+    const int nx = px.tiles_m * px.tiles_n, nw = pw.tiles_m * pw.tiles_n;
+    hipStream_t s = ctx().stream;
+    if (aux) hipLaunchKernelGGL((linear_bwd_small_kernel<ENDIA_EPI_ACT_GRAD>), dim3((unsigned)(nx + nw)), dim3(NTHREADS), 0, s, px, pw, nx);
+    else hipLaunchKernelGGL((linear_bwd_small_kernel<ENDIA_EPI_NONE>), dim3((unsigned)(nx + nw)), dim3(NTHREADS), 0, s, px, pw, nx);
+    ENDIA_LAUNCH_CHECK();
+    return ENDIA_HIP_OK;
+  }
+  if (dW) {
+    int32_t rc = sgemm_impl(1, 0, K, N, B, x, K, g, N, dW, N, 1, 0, 0, 0, ENDIA_EPI_NONE | (db ? ENDIA_GEMM_COLSUM_B : 0),
+                            ENDIA_OP_IDENTITY, nullptr, nullptr, db);
+    if (rc) return rc;
+  } else if (db && N > 0) {
+    int32_t rc = col_reduce(1, B, N, g, db, 1.f);
+    if (rc) return rc;
+  }
+  if (dx) return sgemm_impl(0, 1, B, K, N, g, N, W, N, dx, K, 1, 0, 0, 0, epi_x, aux ? act_flags : ENDIA_OP_IDENTITY, nullptr, aux, nullptr);
+  return ENDIA_HIP_OK;
+}
+
 }  // namespace endia
+
+extern "C" int32_t endia_hip_linear_bwd(int64_t B, int64_t K, int64_t N, const float* x, const float* W, const float* g,
+                                        int32_t act, const float* aux, float* dx, float* dW, float* db) {
+  ENDIA_REQUIRE_INIT();
+  return endia::linear_bwd_impl(B, K, N, x, W, g, act, aux, dx, dW, db);
+}
 
 extern "C" int32_t endia_hip_sgemm(int32_t transA, int32_t transB, int64_t M, int64_t N, int64_t K,
                                    const float* A, int64_t lda, const float* B, int64_t ldb, float* C,

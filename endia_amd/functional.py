@@ -1175,30 +1175,22 @@ def _linear_node(out, x, W, b, xs, Ws, act):
             gp = Array.empty([B, N])
             L.call("endia_hip_unary_vjp_from_output", _ACT[act], B * N, out_.data_ptr(), g.data_ptr(), gp.data_ptr())
             g = gp
-        res = [None, None, None]
+        # endia_hip_linear_bwd: dW = x^T g, db = column sums of g, dx = (g W^T) * act'(.) of the layer below -- one
+        # launch for a small layer, the separate GEMMs (and the reduction) for a large one
         db = Array.empty([1, N]) if pb._requires_grad else None  # kept leading axis, like Expand.vjp (expand_op.mojo:121-126)
-        if pW._requires_grad:
-            dW = Array.empty([K, N])
-            # the weight-gradient launch also sums the columns of g: the bias gradient costs no launch of its own
-            L.call("endia_hip_sgemm", 1, 0, K, N, B, xs.data_ptr(), K, g.data_ptr(), N, dW.data_ptr(), N, 1, 0, 0, 0,
-                   L.EPI_NONE | (L.GEMM_COLSUM_B if db is not None else 0), L.OP_IDENTITY, None, None,
-                   db.data_ptr() if db is not None else None)
-            res[1] = dW
-        elif db is not None:
-            L.call("endia_hip_reduce_add", 2, L.i64_array([B, N]), 1, g.data_ptr(), db.data_ptr(), 1.0, 0)
-        res[2] = db
+        dW = Array.empty([K, N]) if pW._requires_grad else None
+        dx, flags, aux = None, L.OP_IDENTITY, None
         if px._requires_grad:
             dx = Array.empty([B, K])
             pm = _fused_act_of(px)
-            if pm:
+            if pm:  # px is a fused layer's output with this one consumer: its activation derivative rides along
                 flags = _ACT[pm["act"]] | (L.ACT_FROM_OUTPUT if pm["from_output"] else 0)
-                L.call("endia_hip_sgemm", 0, 1, B, K, N, g.data_ptr(), N, Ws.data_ptr(), N, dx.data_ptr(), K, 1, 0, 0, 0,
-                       L.EPI_ACT_GRAD, flags, None, contiguous(pm["aux"]).data_ptr(), None)
+                aux = contiguous(pm["aux"])
                 dx._act_applied = True
-            else:
-                L.call("endia_hip_sgemm", 0, 1, B, K, N, g.data_ptr(), N, Ws.data_ptr(), N, dx.data_ptr(), K, 1, 0, 0, 0,
-                       L.EPI_NONE, L.OP_IDENTITY, None, None, None)
-            res[0] = dx
+        L.call("endia_hip_linear_bwd", B, K, N, xs.data_ptr(), Ws.data_ptr(), g.data_ptr(), flags,
+               aux.data_ptr() if aux is not None else None, dx.data_ptr() if dx is not None else None,
+               dW.data_ptr() if dW is not None else None, db.data_ptr() if db is not None else None)
+        res = [dx, dW, db]
         return res
 
     meta = {"act": act, "aux": out, "from_output": True} if act in _ACT_FN else {"act": None}

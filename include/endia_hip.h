@@ -179,6 +179,18 @@ ENDIA_API int32_t endia_hip_sgemm(int32_t transA, int32_t transB, int64_t M, int
                         int32_t epilogue, int32_t act, const float* bias, const float* aux_in,
                         float* aux_out);
 
+/* ---- backward of one dense layer y = act(x W + b) in one call: both products of matmul_vjp
+ *      (matmul_op.mojo:278-283), the bias gradient (Expand.vjp, expand_op.mojo:121-126) and the activation
+ *      derivative of the layer BELOW on the way out (relu_op.mojo:95, tanh_op.mojo:92, sin_op.mojo:92).
+ *      x [B,K], W [K,N], g [B,N] = cotangent of x W + b (contiguous, row-major).
+ *        dx [B,K] = (g W^T) * act'(aux)   when aux [B,K] is given (act as in endia_hip_sgemm's ACT_GRAD epilogue,
+ *                                          optionally | ENDIA_ACT_FROM_OUTPUT), else g W^T
+ *        dW [K,N] = x^T g,   db [N] = sum over rows of g.        Any of dx, dW, db may be null.
+ *      When all three are wanted and the layer is small (B and N at most 128) they come from ONE launch; otherwise
+ *      the call is the corresponding endia_hip_sgemm calls. The results are those calls' results either way. */
+ENDIA_API int32_t endia_hip_linear_bwd(int64_t B, int64_t K, int64_t N, const float* x, const float* W, const float* g,
+                             int32_t act, const float* aux, float* dx, float* dW, float* db);
+
 /* ---- complex64 GEMM: the complex branch of matmul_fwd (matmul_op.mojo:201-238). Interleaved
  *      operands; lda/ldb/ldc and strides count complex elements. conjA/conjB conjugate the operand
  *      (the reference's VJP does not conjugate, matmul_op.mojo:278-283; the Wirtinger convention does).

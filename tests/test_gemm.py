@@ -231,3 +231,35 @@ def test_sgemm_colsum_b(dev, M, N, K):
         with pytest.raises(L.EndiaHipError):
             dev.call("endia_hip_sgemm", 1, bad[0], M, N, K, dA, M, dB, N if not bad[0] else K, dC, N, 1, 0, 0, 0,
                      (L.EPI_NONE if bad[0] else L.EPI_BIAS) | L.GEMM_COLSUM_B, L.OP_IDENTITY, dsum, None, dsum)
+
+
+@pytest.mark.parametrize("B,K,N", [(128, 128, 128), (128, 32, 64), (128, 64, 32), (64, 128, 96), (8, 4, 8), (128, 128, 132),
+                                   (256, 64, 64), (128, 1, 32), (128, 30, 64), (100, 36, 20)])
+@pytest.mark.parametrize("act", ["relu", "tanh", "none"])
+def test_linear_bwd(dev, B, K, N, act):
+    """endia_hip_linear_bwd against float64 for layers that take the one-launch path (B, N <= 128, aligned) and for
+    ones that do not (large, unaligned, 1-wide): dx = (g W^T) * act'(aux), dW = x^T g, db = column sums of g;
+    also with outputs left out."""
+    rng = np.random.default_rng(B * 5 + K * 3 + N + len(act))
+    x = rng.standard_normal((B, K)).astype(np.float32)
+    W = rng.standard_normal((K, N)).astype(np.float32)
+    g = rng.standard_normal((B, N)).astype(np.float32)
+    aux = np.maximum(x, 0) if act == "relu" else np.tanh(x).astype(np.float32)   # the layer below's stored OUTPUT
+    dmask = {"relu": (aux > 0).astype(np.float64), "tanh": 1 - aux.astype(np.float64) ** 2, "none": 1.0}[act]
+    want_dx = (g.astype(np.float64) @ W.astype(np.float64).T) * dmask
+    want_dW = x.astype(np.float64).T @ g.astype(np.float64)
+    want_db = g.astype(np.float64).sum(0)
+    flags = {"relu": L.OP_RELU | L.ACT_FROM_OUTPUT, "tanh": L.OP_TANH | L.ACT_FROM_OUTPUT, "none": L.OP_IDENTITY}[act]
+    dxp, dWp, dbp = (dev.put(np.full(s, np.nan, np.float32)) for s in ((B, K), (K, N), (N,)))
+    px, pW, pg, paux = dev.put(x), dev.put(W), dev.put(g), dev.put(aux)
+    dev.call("endia_hip_linear_bwd", B, K, N, px, pW, pg, flags, paux if act != "none" else None, dxp, dWp, dbp)
+    assert_close(dev.get(dxp, (B, K)), want_dx, what="dx")
+    assert_close(dev.get(dWp, (K, N)), want_dW, what="dW")
+    assert_close(dev.get(dbp, (N,)), want_db, tol=1e-5, what="db")
+    # outputs left out: only dW and db (first layer of a model), only dx
+    dW2, db2, dx2 = (dev.put(np.full(s, np.nan, np.float32)) for s in ((K, N), (N,), (B, K)))
+    dev.call("endia_hip_linear_bwd", B, K, N, px, pW, pg, L.OP_IDENTITY, None, None, dW2, db2)
+    assert_close(dev.get(dW2, (K, N)), want_dW, what="dW alone")
+    assert_close(dev.get(db2, (N,)), want_db, tol=1e-5, what="db alone")
+    dev.call("endia_hip_linear_bwd", B, K, N, px, pW, pg, flags, paux if act != "none" else None, dx2, None, None)
+    assert_close(dev.get(dx2, (B, K)), want_dx, what="dx alone")
