@@ -72,22 +72,31 @@ __device__ __forceinline__ float act_grad(int act, int from_out, float aux) {
   }
 }
 
+// bias_v = bias[col] and aux_v = aux_in[row, col], fetched by the caller (early, where registers allow)
+template <int EPI>
+__device__ __forceinline__ void epilogue_apply(const GemmArgs& p, float* __restrict__ C, float* __restrict__ aux_out,
+                                               int row, int col, float v, float bias_v, float aux_v) {
+  int64_t off = (int64_t)row * p.ldc + col;
+  if (EPI == ENDIA_EPI_BIAS) {
+    v += bias_v;
+  } else if (EPI == ENDIA_EPI_BIAS_ACT) {
+    v += bias_v;
+    if (aux_out) aux_out[off] = v;
+    v = act_fwd(p.act, v);
+  } else if (EPI == ENDIA_EPI_ACT_GRAD) {
+    v *= act_grad(p.act, p.from_out, aux_v);
+  }
+  if (p.accumulate) v += C[off];
+  C[off] = v;
+}
+
 template <int EPI>
 __device__ __forceinline__ void epilogue_store(const GemmArgs& p, float* __restrict__ C,
                                                const float* __restrict__ aux_in,
                                                float* __restrict__ aux_out, int row, int col, float v) {
-  int64_t off = (int64_t)row * p.ldc + col;
-  if (EPI == ENDIA_EPI_BIAS) {
-    v += p.bias[col];
-  } else if (EPI == ENDIA_EPI_BIAS_ACT) {
-    v += p.bias[col];
-    if (aux_out) aux_out[off] = v;
-    v = act_fwd(p.act, v);
-  } else if (EPI == ENDIA_EPI_ACT_GRAD) {
-    v *= act_grad(p.act, p.from_out, aux_in[off]);
-  }
-  if (p.accumulate) v += C[off];
-  C[off] = v;
+  const float bias_v = (EPI == ENDIA_EPI_BIAS || EPI == ENDIA_EPI_BIAS_ACT) ? p.bias[col] : 0.f;
+  const float aux_v = EPI == ENDIA_EPI_ACT_GRAD ? aux_in[(int64_t)row * p.ldc + col] : 0.f;
+  epilogue_apply<EPI>(p, C, aux_out, row, col, v, bias_v, aux_v);
 }
 
 // F = MFMA blocks per wave in each direction: F = 2 gives the 128 x 128 tile, F = 1 the 64 x 64 tile
@@ -139,6 +148,25 @@ __device__ __forceinline__ void gemm_tile(const GemmArgs& p, int block, int nblo
     }
   };
 
+  // The small tile has registers to spare: what the epilogue reads (a bias element, 16 elements of the activation
+  // operand) is requested here, behind the tile loads, instead of after the last MFMA, where it would be one more
+  // memory round trip on the critical path of a launch that is a few such round trips long.
+  constexpr bool PRE = F == 1 && EPI != ENDIA_EPI_NONE;
+  float bias_pre = 0.f, aux_pre[PRE ? 16 : 1];
+  auto prefetch_epilogue = [&]() {
+    if constexpr (PRE) {
+      const int col = n0 + wn * 32 + l32;
+      if (EPI == ENDIA_EPI_BIAS || EPI == ENDIA_EPI_BIAS_ACT) bias_pre = col < p.N ? p.bias[col] : 0.f;
+      if (EPI == ENDIA_EPI_ACT_GRAD) {
+#pragma unroll
+        for (int v = 0; v < 16; ++v) {
+          const int row = m0 + wm * 32 + acc_row(v, h);
+          aux_pre[v] = (row < p.M && col < p.N) ? aux_in[(int64_t)row * p.ldc + col] : 0.f;
+        }
+      }
+    }
+  };
+
   if constexpr (SHORTK) {
     constexpr int DEPTH = 4;
     float4 ra[DEPTH][LA::PASSES], rb[DEPTH][LB::PASSES];
@@ -149,6 +177,7 @@ __device__ __forceinline__ void gemm_tile(const GemmArgs& p, int block, int nblo
       la.advance();
       lb.advance();
     }
+    prefetch_epilogue();
 #pragma unroll
     for (int t = 0; t < DEPTH; ++t) {
       if (t * BK >= K) break;
@@ -162,6 +191,7 @@ __device__ __forceinline__ void gemm_tile(const GemmArgs& p, int block, int nblo
   } else {
   la.load(K);
   lb.load(K);
+  prefetch_epilogue();
   la.store(As);
   lb.store(Bs);
   __syncthreads();
@@ -196,7 +226,9 @@ __device__ __forceinline__ void gemm_tile(const GemmArgs& p, int block, int nblo
 #pragma unroll
       for (int v = 0; v < 16; ++v) {
         int row = m0 + wm * 32 * F + fm * 32 + acc_row(v, h);
-        if (row < p.M) epilogue_store<EPI>(p, C, aux_in, aux_out, row, col, acc[fm][fn][v]);
+        if (row >= p.M) continue;
+        if constexpr (PRE) epilogue_apply<EPI>(p, C, aux_out, row, col, acc[fm][fn][v], bias_pre, aux_pre[v]);
+        else epilogue_store<EPI>(p, C, aux_in, aux_out, row, col, acc[fm][fn][v]);
       }
     }
 }
@@ -305,9 +337,31 @@ __global__ __launch_bounds__(128) void sgemm_skinny_kernel(GemmArgs p, int trans
       p.aux_out[n] = v;
     } else {
       float* c = p.C + bz * p.sC + (int64_t)m * p.ldc + n;
-      *c = p.accumulate ? *c + v : v;
+      float r = p.bias ? v + p.bias[n] : v;          // bias: the BIAS and BIAS_ACT epilogues
+      if (p.bias && p.aux_out && !p.colsum) p.aux_out[bz * p.sC + (int64_t)m * p.ldc + n] = r;
+      r = act_fwd(p.act, r);                         // identity unless BIAS_ACT
+      *c = p.accumulate ? *c + r : r;
     }
   }
+}
+
+// A reduction of one to four terms (the 1-wide first layer of the reference's sine-fit MLP and the data gradient
+// of its 1-wide last layer are outer products): one thread per output element, every epilogue.
+template <int EPI>
+__global__ __launch_bounds__(256) void sgemm_thin_k_kernel(GemmArgs p, int transA, int transB) {
+  const int64_t bz = blockIdx.y;
+  const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (i >= (int64_t)p.M * p.N) return;
+  const int m = (int)(i / p.N), n = (int)(i - (int64_t)m * p.N);
+  const float* __restrict__ A = p.A + bz * p.sA;
+  const float* __restrict__ B = p.B + bz * p.sB;
+  float acc = 0.f;
+  for (int k = 0; k < p.K; ++k) {
+    const float a = transA ? A[(int64_t)k * p.lda + m] : A[(int64_t)m * p.lda + k];
+    const float b = transB ? B[(int64_t)n * p.ldb + k] : B[(int64_t)k * p.ldb + n];
+    acc = fmaf(a, b, acc);
+  }
+  epilogue_store<EPI>(p, p.C + bz * p.sC, p.aux_in ? p.aux_in + bz * p.sC : nullptr, p.aux_out ? p.aux_out + bz * p.sC : nullptr, m, n, acc);
 }
 
 template <int EPI, int F, bool SHORTK>
@@ -474,8 +528,19 @@ int32_t sgemm_impl(int transA, int transB, int64_t M, int64_t N, int64_t K, cons
       int32_t rc = col_reduce(1, splits, M * N, p.C, C_final, 1.f);  // partials added in slice order
       if (rc || !colsum) return rc;
     }
-  } else if (epi == ENDIA_EPI_NONE && M * N <= 2048 && K >= 64) {
+  } else if (K >= 1 && K <= 4 && M * N < (1ll << 31) * 256) {
     p.k_split = 0;
+    dim3 grid((unsigned)ceil_div64(M * N, 256), (unsigned)batch);
+    switch (epi) {
+      case ENDIA_EPI_NONE: hipLaunchKernelGGL((sgemm_thin_k_kernel<ENDIA_EPI_NONE>), grid, dim3(256), 0, s, p, transA, transB); break;
+      case ENDIA_EPI_BIAS: hipLaunchKernelGGL((sgemm_thin_k_kernel<ENDIA_EPI_BIAS>), grid, dim3(256), 0, s, p, transA, transB); break;
+      case ENDIA_EPI_BIAS_ACT: hipLaunchKernelGGL((sgemm_thin_k_kernel<ENDIA_EPI_BIAS_ACT>), grid, dim3(256), 0, s, p, transA, transB); break;
+      default: hipLaunchKernelGGL((sgemm_thin_k_kernel<ENDIA_EPI_ACT_GRAD>), grid, dim3(256), 0, s, p, transA, transB); break;
+    }
+  } else if (epi != ENDIA_EPI_ACT_GRAD && M * N <= 2048 && K >= (epi == ENDIA_EPI_NONE ? 64 : 16)) {
+    p.k_split = 0;
+    if (epi == ENDIA_EPI_NONE) p.bias = nullptr;
+    if (epi != ENDIA_EPI_BIAS_ACT) p.act = ENDIA_OP_IDENTITY;
     if (colsum) {  // N more groups produce the column sums of B in the same launch
       p.colsum = 1;
       p.aux_out = aux_out;

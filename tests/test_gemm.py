@@ -69,7 +69,8 @@ def test_sgemm_golden(dev, golden):
     assert_close(run_sgemm(dev, g["sa"], g["sg"], 1, 0, 64, 64, 64), g["dsb"], what="dB")
 
 
-@pytest.mark.parametrize("M,N,K", [(256, 256, 64), (50, 30, 7), (130, 70, 36)])
+@pytest.mark.parametrize("M,N,K", [(256, 256, 64), (50, 30, 7), (130, 70, 36),
+                                   (128, 32, 1), (128, 1, 32), (40, 50, 3), (16, 8, 100), (128, 64, 128)])  # thin K, few outputs, short K
 @pytest.mark.parametrize("act", ["relu", "tanh", "sin", "identity"])
 def test_sgemm_epilogues(dev, M, N, K, act):
     rng = np.random.default_rng(5)
