@@ -264,3 +264,51 @@ def test_linear_bwd(dev, B, K, N, act):
     assert_close(dev.get(db2, (N,)), want_db, tol=1e-5, what="db alone")
     dev.call("endia_hip_linear_bwd", B, K, N, px, pW, pg, flags, paux if act != "none" else None, dx2, None, None)
     assert_close(dev.get(dx2, (B, K)), want_dx, what="dx alone")
+
+
+def test_sgemm_random_shapes_and_flags(dev):
+    """Seeded sweep over the dispatch boundaries (tiled / short-reduction / few-outputs / thin-K / generic kernels,
+    aligned and unaligned extents, every transpose and epilogue, accumulate, column sums): 240 cases against float64."""
+    rng = np.random.default_rng(2024)
+    picks = [1, 2, 3, 4, 5, 8, 16, 31, 32, 33, 63, 64, 65, 96, 127, 128, 129, 132, 200, 256, 260]
+    for case in range(240):
+        M, N = (int(rng.choice(picks)) for _ in range(2))
+        K = int(rng.choice([0, 1, 2, 4, 5, 8, 16, 28, 32, 36, 64, 100, 128, 132, 256, 515, 1024]))
+        if case % 3 == 0:  # favour the aligned, vectorised paths
+            M, N, K = (max(4, v // 4 * 4) for v in (M, N, max(K, 4)))
+        ta, tb = int(rng.integers(2)), int(rng.integers(2))
+        epi = int(rng.choice([L.EPI_NONE, L.EPI_NONE, L.EPI_BIAS, L.EPI_BIAS_ACT, L.EPI_ACT_GRAD]))
+        act = int(rng.choice([L.OP_RELU, L.OP_TANH, L.OP_SIN, L.OP_IDENTITY]))
+        accumulate = epi == L.EPI_NONE and case % 5 == 0
+        colsum = epi == L.EPI_NONE and not tb and not accumulate and case % 2 == 0
+        A = rng.standard_normal((K, M) if ta else (M, K)).astype(np.float32)
+        B = rng.standard_normal((N, K) if tb else (K, N)).astype(np.float32)
+        bias = rng.standard_normal(N).astype(np.float32)
+        aux = rng.standard_normal((M, N)).astype(np.float32)
+        C0 = rng.standard_normal((M, N)).astype(np.float32)
+        opA = (A.T if ta else A).astype(np.float64)
+        opB = (B.T if tb else B).astype(np.float64)
+        want = opA @ opB
+        if epi in (L.EPI_BIAS, L.EPI_BIAS_ACT):
+            want = want + bias
+        if epi == L.EPI_BIAS_ACT:
+            want = {L.OP_RELU: lambda z: np.maximum(z, 0), L.OP_TANH: np.tanh, L.OP_SIN: np.sin, L.OP_IDENTITY: lambda z: z}[act](want)
+        if epi == L.EPI_ACT_GRAD:
+            a64 = aux.astype(np.float64)
+            want = want * {L.OP_RELU: (a64 > 0) * 1.0, L.OP_TANH: 1 - np.tanh(a64) ** 2, L.OP_SIN: np.cos(a64), L.OP_IDENTITY: 1.0}[act]
+        if accumulate:
+            want = want + C0
+        dA, dB, dC = dev.put(A), dev.put(B), dev.put(C0)
+        dsum = dev.put(np.full(max(N, 1), np.nan, np.float32))
+        flags = epi | (L.GEMM_ACCUMULATE if accumulate else 0) | (L.GEMM_COLSUM_B if colsum else 0)
+        dev.call("endia_hip_sgemm", ta, tb, M, N, K, dA, M if ta else max(K, 1), dB, K if tb and K else (max(K, 1) if tb else N), dC, N,
+                 1, 0, 0, 0, flags, act, dev.put(bias) if epi in (L.EPI_BIAS, L.EPI_BIAS_ACT) else None,
+                 dev.put(aux) if epi == L.EPI_ACT_GRAD else None, dsum if colsum else None)
+        what = "case %d: M=%d N=%d K=%d ta=%d tb=%d epi=%d act=%d acc=%d colsum=%d" % (case, M, N, K, ta, tb, epi, act, accumulate, colsum)
+        got = dev.get(dC, (M, N))
+        scale = max(float(np.abs(want).max()), 1e-30)
+        assert np.abs(got - want).max() <= 2e-5 * scale * max(1.0, np.sqrt(K)), what
+        if colsum:
+            s = dev.get(dsum, (N,))
+            assert np.abs(s - B.astype(np.float64).sum(0)).max() <= 2e-5 * max(1.0, np.sqrt(K)) * max(1.0, float(np.abs(B).max()) if K else 1.0), what + " (column sums)"
+        dev.release()
