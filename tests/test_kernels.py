@@ -124,7 +124,11 @@ def _binary(dev, op, a, b):
     shape = np.broadcast_shapes(a.shape, b.shape)
     isz = a.itemsize
     av, bv = np.broadcast_to(a, shape), np.broadcast_to(b, shape)
-    da, db = dev.put(a), dev.put(b)
+
+    def upload(x):  # a transposed view is uploaded as its storage (the strides above describe that memory)
+        return dev.put(x.T if x.ndim == 2 and x.flags.f_contiguous and not x.flags.c_contiguous else x)
+
+    da, db = upload(a), upload(b)
     n = int(np.prod(shape))
     do = dev.alloc(max(n * isz, 4))
     dev.call("endia_hip_binary", op, len(shape), L.i64_array(shape), L.i64_array([s // isz for s in av.strides]),
@@ -751,3 +755,55 @@ def test_pool_bwd_tiling_windows(dev, xs, k):
               ("avg", 1): TF.avg_pool1d, ("avg", 2): TF.avg_pool2d, ("avg", 3): TF.avg_pool3d}[(mname, nsp)]
         (fn(t, k, k) * torch.tensor(gy, dtype=torch.float64)).sum().backward()
         assert_close(dx, t.grad.numpy(), what=mname + " grad vs torch")
+
+
+@pytest.mark.gpu
+def test_reduce_add_random_masks(dev):
+    """Seeded sweep over shapes and axis masks (row, column, batched-column, small single-launch and general
+    paths, size-1 axes in every position): 150 cases against float64 on the scale of sum |x|."""
+    rng = np.random.default_rng(77)
+    sizes = [1, 2, 3, 4, 5, 7, 8, 16, 31, 33, 64, 100, 257]
+    for case in range(150):
+        nd_ = int(rng.integers(1, 5))
+        shape = tuple(int(rng.choice(sizes)) for _ in range(nd_))
+        if np.prod(shape) > 2_000_000:
+            continue
+        mask = int(rng.integers(0, 1 << nd_))
+        axes = tuple(i for i in range(nd_) if mask >> i & 1)
+        x = rng.standard_normal(shape).astype(np.float32)
+        oshape = tuple(1 if i in axes else s for i, s in enumerate(shape))
+        dx_, do = dev.put(x), dev.alloc(4 * int(np.prod(oshape)))
+        scale = float(rng.choice([1.0, 0.5, 1.0 / max(int(np.prod([shape[a] for a in axes])), 1)]))
+        dev.call("endia_hip_reduce_add", nd_, L.i64_array(shape), mask, dx_, do, scale, 0)
+        out = dev.get(do, oshape)
+        x64 = x.astype(np.float64)
+        want = (x64.sum(axis=axes, keepdims=True) if axes else x64) * scale
+        bound = (np.abs(x64).sum(axis=axes, keepdims=True) if axes else np.abs(x64)) * abs(scale)
+        assert np.all(np.abs(out - want) <= 1e-5 * bound + 1e-30), "case %d: shape %s axes %s" % (case, shape, axes)
+        dev.release()
+
+
+@pytest.mark.gpu
+def test_binary_random_broadcasts(dev):
+    """Seeded sweep over broadcast patterns (same shape, row vector, scalar, middle axes, transposed operand, rank
+    mismatch) for every binary op with a closed form: 200 cases against float64."""
+    rng = np.random.default_rng(78)
+    ops = [(L.BIN_ADD, np.add), (L.BIN_SUB, np.subtract), (L.BIN_MUL, np.multiply), (L.BIN_DIV, np.divide),
+           (L.BIN_GREATER, lambda a, b: (a > b) * 1.0), (L.BIN_LESS_EQUAL, lambda a, b: (a <= b) * 1.0)]
+    sizes = [1, 2, 3, 4, 5, 8, 17, 32, 33, 64, 96]
+    for case in range(200):
+        nd_ = int(rng.integers(1, 5))
+        full = [int(rng.choice(sizes)) for _ in range(nd_)]
+        sa = [s if rng.random() < 0.7 else 1 for s in full]
+        sb = [s if rng.random() < 0.7 else 1 for s in full]
+        sb = sb[int(rng.integers(0, nd_)):] if rng.random() < 0.3 else sb     # lower rank on one side
+        a = rng.standard_normal(sa).astype(np.float32)
+        b = (np.abs(rng.standard_normal(sb)) + 0.5).astype(np.float32)
+        if nd_ == 2 and rng.random() < 0.5 and len(sb) == 2:                   # a transposed view as the second operand
+            b = np.ascontiguousarray(b.T).T
+        code, fn = ops[case % len(ops)]
+        want = fn(a.astype(np.float64), b.astype(np.float64))
+        got = _binary(dev, code, a, b)
+        assert got.shape == want.shape
+        assert np.all(np.abs(got - want) <= 2e-6 * np.maximum(np.abs(want), 1.0)), "case %d: %s op %s" % (case, (sa, sb), code)
+        dev.release()
