@@ -807,3 +807,61 @@ def test_binary_random_broadcasts(dev):
         assert got.shape == want.shape
         assert np.all(np.abs(got - want) <= 2e-6 * np.maximum(np.abs(want), 1.0)), "case %d: %s op %s" % (case, (sa, sb), code)
         dev.release()
+
+
+@pytest.mark.gpu
+def test_conv_and_pool_random_configs(dev):
+    """Seeded sweep over convolution and pooling configurations (channel counts on both sides of the tile sizes,
+    strides, paddings, dilations, widths that do and do not take the vectorised paths): forward and every gradient
+    against torch float64."""
+    import torch
+    import torch.nn.functional as TF
+    rng = np.random.default_rng(79)
+    for case in range(40):
+        N, C, K = int(rng.integers(1, 4)), int(rng.choice([1, 3, 4, 8, 17, 40])), int(rng.choice([1, 4, 16, 33, 70, 130]))
+        H, W = int(rng.integers(5, 21)), int(rng.choice([5, 8, 12, 13, 16, 20]))
+        R_, S_ = int(rng.choice([1, 2, 3, 5])), int(rng.choice([1, 2, 3, 5]))
+        st = (int(rng.integers(1, 4)), int(rng.integers(1, 3)))
+        pd = (int(rng.integers(0, 3)), int(rng.integers(0, 3)))
+        dl = (int(rng.integers(1, 3)), int(rng.integers(1, 3)))
+        if H + 2 * pd[0] < dl[0] * (R_ - 1) + 1 or W + 2 * pd[1] < dl[1] * (S_ - 1) + 1:
+            continue
+        x = rng.standard_normal((N, C, H, W)).astype(np.float32)
+        w = (rng.standard_normal((K, C, R_, S_)) * 0.3).astype(np.float32)
+        b = rng.standard_normal(K).astype(np.float32)
+        tx, tw, tb = (torch.tensor(v, dtype=torch.float64, requires_grad=True) for v in (x, w, b))
+        ty = TF.conv2d(tx, tw, tb, stride=st, padding=pd, dilation=dl)
+        gy = rng.standard_normal(tuple(ty.shape)).astype(np.float32)
+        (ty * torch.tensor(gy, dtype=torch.float64)).sum().backward()
+        d = _desc(x, w, st, pd, dl)
+        dx_, dw_, db_, dg = dev.put(x), dev.put(w), dev.put(b), dev.put(gy)
+        dy, ddx, ddw, ddb = dev.alloc(gy.nbytes), dev.alloc(x.nbytes), dev.alloc(w.nbytes), dev.alloc(b.nbytes)
+        dev.call("endia_hip_conv2d_fwd", ctypes.byref(d), dx_, dw_, db_, dy, L.OP_IDENTITY)
+        dev.call("endia_hip_conv2d_bwd_data", ctypes.byref(d), dg, dw_, ddx)
+        dev.call("endia_hip_conv2d_bwd_weight", ctypes.byref(d), dx_, dg, ddw)
+        dev.call("endia_hip_conv2d_bwd_bias", ctypes.byref(d), dg, ddb)
+        what = "conv case %d: x %s w %s stride %s pad %s dil %s" % (case, x.shape, w.shape, st, pd, dl)
+        assert_close(dev.get(dy, gy.shape), ty.detach().numpy(), what=what + " fwd")
+        assert_close(dev.get(ddx, x.shape), tx.grad.numpy(), what=what + " dx")
+        assert_close(dev.get(ddw, w.shape), tw.grad.numpy(), what=what + " dw")
+        assert_close(dev.get(ddb, b.shape), tb.grad.numpy(), what=what + " db")
+        dev.release()
+    for case in range(40):
+        N, C = int(rng.integers(1, 4)), int(rng.integers(1, 6))
+        H, W = int(rng.integers(4, 19)), int(rng.choice([4, 7, 8, 12, 15, 16]))
+        k = (int(rng.integers(1, 4)), int(rng.choice([1, 2, 3, 4])))
+        st = k if case % 2 == 0 else (int(rng.integers(1, 4)), int(rng.integers(1, 4)))
+        pd = (0, 0) if case % 2 == 0 else (int(rng.integers(0, k[0] // 2 + 1)), int(rng.integers(0, k[1] // 2 + 1)))
+        if H + 2 * pd[0] < k[0] or W + 2 * pd[1] < k[1]:
+            continue
+        x = rng.standard_normal((N, C, H, W)).astype(np.float32)
+        for mode, mname in ((L.POOL_MAX, "max"), (L.POOL_AVG, "avg")):
+            t = torch.tensor(x, dtype=torch.float64, requires_grad=True)
+            ty = TF.max_pool2d(t, k, st, pd) if mname == "max" else TF.avg_pool2d(t, k, st, pd, count_include_pad=False)
+            gy = rng.standard_normal(tuple(ty.shape)).astype(np.float32)
+            (ty * torch.tensor(gy, dtype=torch.float64)).sum().backward()
+            y, dx = _pool_run(dev, mode, x, gy, k, st, pd, (1, 1))
+            what = "pool case %d %s: x %s k %s stride %s pad %s" % (case, mname, x.shape, k, st, pd)
+            assert_close(y, ty.detach().numpy(), what=what + " fwd")
+            assert_close(dx, t.grad.numpy(), what=what + " grad")
+        dev.release()
