@@ -686,3 +686,36 @@ def test_conv2d_fused_relu_step(nd, golden):
     assert_close(w.grad().to_numpy(), tw.grad.numpy(), what="dw (dense cotangent)")
     with pytest.raises(ValueError, match="act"):
         nd.conv2d(x, w, b, act="tanh")
+
+
+def test_random_mlps_vs_oracle(nd):
+    """Seeded sweep over small MLPs (widths and batches on both sides of the one-launch layer backward's limits,
+    1-wide and unaligned layers, every activation, fused and op-by-op): loss and every gradient against the CPU
+    oracle's step."""
+    from oracle import endia_ref as R
+    rng = np.random.default_rng(81)
+    widths_pool = [1, 4, 8, 30, 32, 33, 64, 100, 128, 132, 160]
+    for case in range(24):
+        depth = int(rng.integers(1, 5))
+        widths = [int(rng.choice(widths_pool)) for _ in range(depth + 1)]
+        batch = int(rng.choice([8, 20, 100, 128, 130, 256]))
+        act = ["relu", "tanh", "sin"][case % 3]
+        fused = case % 4 != 3
+        Ws = [(rng.standard_normal((widths[i], widths[i + 1])) * np.sqrt(1.0 / widths[i])).astype(np.float32) for i in range(depth)]
+        bs = [(rng.standard_normal(widths[i + 1]) * 0.1).astype(np.float32) for i in range(depth)]
+        xb = rng.standard_normal((batch, widths[0])).astype(np.float32)
+        yb = rng.standard_normal((batch, widths[-1])).astype(np.float32)
+        loss_ref, dWr, dbr = R.mlp_step(widths, act, xb, yb, [w.copy() for w in Ws], [b.copy() for b in bs])
+        mlp = nd.nn.MLP(widths, compute_backward=True, activation=act, fused=fused)
+        for i in range(depth):
+            mlp.weights[i] = nd.array(Ws[i], requires_grad=True)
+            mlp.biases[i] = nd.array(bs[i], requires_grad=True)
+        x, y = nd.array(xb), nd.array(yb)
+        loss = nd.mse(mlp.forward(x), y)
+        loss.backward()
+        what = "case %d: widths %s batch %d %s fused=%s" % (case, widths, batch, act, fused)
+        assert_close([loss.item()], [loss_ref], what=what + " loss")
+        for i in range(depth):
+            assert_close(mlp.weights[i].grad().to_numpy(), dWr[i], what=what + " dW%d" % i)
+            assert_close(mlp.biases[i].grad().to_numpy(), dbr[i], tol=2e-4, what=what + " db%d" % i)
+        loss.zero_grad()
