@@ -538,7 +538,23 @@ def _unary(op, name, x, vjp):
     out = Array.empty(x._shape, is_complex=x.is_complex_)
     if out.size():
         L.call("endia_hip_unary_fwd", op, src.size(), src.data_ptr(), out.data_ptr(), 1 if x.is_complex_ else 0)
-    return _register(out, [x], name, vjp)
+
+    def first_order_vjp(primals, grad, out_):
+        # The rule handed in is the reference's, written in differentiable ops (two to four launches); it is what a
+        # create_graph pass records. An ordinary pass computes the same g * op'(x) with the one kernel made for it.
+        from .autograd.functional import building_graph
+        p = primals[0]
+        if building_graph() or p.is_complex_ or grad.is_complex_ or op in _NO_VJP_KERNEL or grad._shape != p._shape or not p.size():
+            return vjp(primals, grad, out_)
+        g, xs_ = contiguous(grad), contiguous(p)
+        dx = Array.empty(p._shape)
+        L.call("endia_hip_unary_vjp", op, p.size(), xs_.data_ptr(), g.data_ptr(), dx.data_ptr(), 0)
+        return [dx]
+
+    return _register(out, [x], name, first_order_vjp if vjp is not None else None)
+
+
+_NO_VJP_KERNEL = (L.OP_SIGN, L.OP_IDENTITY, L.OP_ABS)
 
 
 def relu(x):
