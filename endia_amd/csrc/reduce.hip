@@ -93,7 +93,7 @@ __global__ __launch_bounds__(TPB) void col_reduce_final_kernel(const float* __re
 // ---- row reduction: x[R][C] -> out[R] (sum over C) --------------------------------------------
 // grid (S, R). Each group sums a contiguous chunk of one row; partials [R][S].
 __global__ __launch_bounds__(TPB) void row_reduce_kernel(const float* __restrict__ x, float* __restrict__ part,
-                                                         int64_t C, int64_t chunk, int vec) {
+                                                         int64_t C, int64_t chunk, int vec, float scale) {
   __shared__ float red[4];
   const int64_t r = blockIdx.y;
   const int64_t c0 = (int64_t)blockIdx.x * chunk;
@@ -113,7 +113,7 @@ __global__ __launch_bounds__(TPB) void row_reduce_kernel(const float* __restrict
     for (int64_t j = c0 + threadIdx.x; j < c1; j += TPB) acc += row[j];
   }
   float s = block_sum(acc, red);
-  if (threadIdx.x == 0) part[r * gridDim.x + blockIdx.x] = s;
+  if (threadIdx.x == 0) part[r * gridDim.x + blockIdx.x] = s * scale;
 }
 
 // stage 2: out[r] = scale * sum_s part[r][s]; one wave per row
@@ -265,11 +265,16 @@ int32_t row_reduce(int64_t R, int64_t C, const float* x, float* out, float scale
   int64_t chunk = ceil_div64(ceil_div64(C, S), 4) * 4;
   S = ceil_div64(C, chunk);
   const int vec = (C % 4 == 0) && al16(x);
+  if (S == 1) {  // one group per row: its sum is the result, no second stage
+    hipLaunchKernelGGL(row_reduce_kernel, dim3(1, (unsigned)R), dim3(TPB), 0, s, x, out, C, chunk, vec, scale);
+    ENDIA_LAUNCH_CHECK();
+    return ENDIA_HIP_OK;
+  }
   void* ws = nullptr;
   int32_t rc = workspace(R * S * (int64_t)sizeof(float), &ws);
   if (rc) return rc;
   float* part = static_cast<float*>(ws);
-  hipLaunchKernelGGL(row_reduce_kernel, dim3((unsigned)S, (unsigned)R), dim3(TPB), 0, s, x, part, C, chunk, vec);
+  hipLaunchKernelGGL(row_reduce_kernel, dim3((unsigned)S, (unsigned)R), dim3(TPB), 0, s, x, part, C, chunk, vec, 1.f);
   ENDIA_LAUNCH_CHECK();
   hipLaunchKernelGGL(row_reduce_final_kernel, dim3((unsigned)ceil_div64(R, 4)), dim3(TPB), 0, s, part, out, R, S, scale);
   ENDIA_LAUNCH_CHECK();
