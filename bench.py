@@ -49,7 +49,7 @@ def build_wide_mlp(nd, width=4096, layers=8, batch=4096, seed=2):
     return mlp, opt, x, y
 
 
-def build_sine_mlp(nd, seed=0):
+def build_sine_mlp(nd, seed=0, optimizer="sgd"):
     rng = np.random.default_rng(seed)
     widths = [1, 32, 64, 128, 128, 128, 64, 32, 1]
     mlp = nd.nn.MLP(widths, compute_backward=True, activation="relu", fused=True)
@@ -59,7 +59,9 @@ def build_sine_mlp(nd, seed=0):
         mlp.biases[i] = nd.array((rng.standard_normal(widths[i + 1]) * s).astype(np.float32), requires_grad=True)
     xb = rng.uniform(0, 1, (128, 1)).astype(np.float32)
     x, y = nd.array(xb), nd.array(np.sin(2 * np.pi * xb).astype(np.float32))
-    opt = nd.optim.SGD(mlp.params(), lr=1e-3)
+    # "adam" is what the reference's own script uses (benchmarks/mlp_benchmarks/mlp_imp.mojo:38-40); its step counter
+    # lives in device memory here so that the step can be replayed as a graph
+    opt = nd.optim.SGD(mlp.params(), lr=1e-3) if optimizer == "sgd" else nd.optim.Adam(mlp.params(), lr=1e-3, capturable=True)
     return mlp, opt, x, y
 
 
@@ -121,7 +123,7 @@ def cpu_baseline_wide(width=4096, layers=8, batch=4096, rows=None, target_second
     }
 
 
-def cpu_baseline_sine(steps=200):
+def cpu_baseline_sine(steps=200, optimizer="sgd"):
     from oracle import endia_ref as R
     rng = np.random.default_rng(0)
     widths = [1, 32, 64, 128, 128, 128, 64, 32, 1]
@@ -129,13 +131,16 @@ def cpu_baseline_sine(steps=200):
     bs = [(rng.standard_normal(widths[i + 1]) * np.sqrt(2.0 / widths[i])).astype(np.float32) for i in range(8)]
     xb = rng.uniform(0, 1, (128, 1)).astype(np.float32)
     yb = np.sin(2 * np.pi * xb).astype(np.float32)
-    R.mlp_step(widths, "relu", xb, yb, Ws, bs, opt="sgd", lr=1e-3)
+    state = None
+    if optimizer == "adam":
+        state = {k: [np.zeros_like(a) for a in (Ws if k.endswith("W") else bs)] for k in ("mW", "vW", "mb", "vb")}
+    R.mlp_step(widths, "relu", xb, yb, Ws, bs, opt=optimizer, lr=1e-3, t=1.0, state=state)
     t0 = time.perf_counter()
-    for _ in range(steps):
-        R.mlp_step(widths, "relu", xb, yb, Ws, bs, opt="sgd", lr=1e-3)
+    for i in range(steps):
+        R.mlp_step(widths, "relu", xb, yb, Ws, bs, opt=optimizer, lr=1e-3, t=float(i + 2), state=state)
     dt = time.perf_counter() - t0
     return {"value": steps / dt, "unit": "steps/s", "cores": 1, "kind": "port", "host_cores_available": os.cpu_count(),
-            "sample": "%d full fwd+bwd+SGD steps of the ref-order CPU restatement, 1 thread" % steps}
+            "sample": "%d full fwd+bwd+%s steps of the ref-order CPU restatement, 1 thread" % (steps, optimizer.upper() if optimizer == "sgd" else "Adam")}
 
 
 def _timed(fn):
@@ -563,6 +568,7 @@ def main():
     ap.add_argument("--workload", default="wide_mlp", choices=["wide_mlp", "sine_mlp", "kernels", "conv2d", "hvp", "complex_mlp", "complex_mlp_3m"])
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--eager", action="store_true", help="sine_mlp: issue every kernel from the host instead of replaying a graph")
+    ap.add_argument("--optimizer", default="sgd", choices=["sgd", "adam"], help="sine_mlp: SGD (the benchmark configuration) or Adam (the reference script's)")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build runs on ONE GPU (no collectives, no sharding); --gpus %d is not supported. "
@@ -608,12 +614,13 @@ def main():
         config = {"workload": "wide_mlp: 8 x Linear(4096->4096)+bias, tanh, MSE, Adam, batch 4096, fp32",
                   "batch": batch, "width": width, "layers": layers, "optimizer": "adam"}
     else:
-        mlp, opt, x, y = build_sine_mlp(nd)
+        mlp, opt, x, y = build_sine_mlp(nd, optimizer=args.optimizer)
         w = [1, 32, 64, 128, 128, 128, 64, 32, 1]
         kn = sum(w[i] * w[i + 1] for i in range(8))
         gemm_flops_step = 2.0 * 128 * (3 * kn - w[0] * w[1])
-        config = {"workload": "sine_mlp: widths 1-32-64-128-128-128-64-32-1, relu, MSE, SGD 1e-3, batch 128, fp32",
-                  "batch": 128, "optimizer": "sgd"}
+        config = {"workload": "sine_mlp: widths 1-32-64-128-128-128-64-32-1, relu, MSE, %s 1e-3, batch 128, fp32"
+                              % ("SGD" if args.optimizer == "sgd" else "Adam"),
+                  "batch": 128, "optimizer": args.optimizer}
 
     for _ in range(args.warmup):
         train_step(nd, mlp, opt, x, y)
@@ -638,7 +645,7 @@ def main():
     steps_per_s = args.steps / elapsed
     out = {
         "metric": "fwd+bwd train steps/s + MFMA util %, 8-layer 4096-wide fp32 MLP, batch 4096"
-                  if args.workload == "wide_mlp" else "fwd+bwd+SGD train steps/s, sine-fit MLP",
+                  if args.workload == "wide_mlp" else "fwd+bwd+%s train steps/s, sine-fit MLP" % ("SGD" if args.optimizer == "sgd" else "Adam"),
         "value": steps_per_s, "unit": "steps/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": ms_per_step, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "f32", "data": "synthetic", "config": config,
@@ -660,7 +667,7 @@ def main():
         }
         out["mfma_util_pct"] = 100.0 * achieved / FP32_MFMA_PEAK_TFLOPS
     if not args.no_cpu_baseline:
-        out["cpu_baseline"] = cpu_baseline_wide() if args.workload == "wide_mlp" else cpu_baseline_sine()
+        out["cpu_baseline"] = cpu_baseline_wide() if args.workload == "wide_mlp" else cpu_baseline_sine(optimizer=args.optimizer)
     print(json.dumps(out))
 
 

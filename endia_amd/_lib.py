@@ -115,6 +115,8 @@ SIGNATURES = {
     "endia_hip_pool_bwd": [POINTER(PoolDesc), c_int32, _fp, _fp, _fp],
     "endia_hip_sgd_step": [c_int64, _fp, _fp, c_float],
     "endia_hip_sgd_step_multi": [c_int32, _i64p, POINTER(c_void_p), POINTER(c_void_p), c_float],
+    "endia_hip_adam_step_multi": [c_int32, _i64p, POINTER(c_void_p), POINTER(c_void_p), POINTER(c_void_p), POINTER(c_void_p),
+                                  c_float, c_float, c_float, c_float, _fp],
     "endia_hip_sgd_momentum_step": [c_int64, _fp, _fp, _fp, c_float, c_float, c_float],
     "endia_hip_adagrad_step": [c_int64, _fp, _fp, _fp, c_float, c_float],
     "endia_hip_rmsprop_step": [c_int64, _fp, _fp, _fp, c_float, c_float, c_float],

@@ -106,6 +106,35 @@ __global__ __launch_bounds__(TPB) void sgd_multi_kernel(SgdMulti t, float lr) {
   for (int64_t j = (int64_t)blockIdx.x * TPB + threadIdx.x; j < n; j += stride) p[j] = sgd_one(p[j], g[j], lr);
 }
 
+// Adam over several tensors with the step counter in device memory: nothing that changes from step to step is a
+// kernel argument, so the launch can be recorded into a HIP graph and replayed. Every group computes the two bias
+// corrections from *t itself (two powf per group).
+struct AdamMulti {
+  float* p[MULTI_MAX];
+  const float* g[MULTI_MAX];
+  float* m[MULTI_MAX];
+  float* v[MULTI_MAX];
+  int64_t n[MULTI_MAX];
+};
+
+__global__ __launch_bounds__(TPB) void adam_multi_kernel(AdamMulti t, AdamK k, const float* __restrict__ step) {
+  const int i = blockIdx.y;
+  const float ts = step[0];
+  k.c1 = 1.0f - powf(k.b1, ts);
+  k.c2 = 1.0f - powf(k.b2, ts);
+  float* __restrict__ p = t.p[i];
+  const float* __restrict__ g = t.g[i];
+  float* __restrict__ m = t.m[i];
+  float* __restrict__ v = t.v[i];
+  const int64_t n = t.n[i];
+  const int64_t stride = (int64_t)gridDim.x * TPB;
+  for (int64_t j = (int64_t)blockIdx.x * TPB + threadIdx.x; j < n; j += stride) adam_one(p[j], g[j], m[j], v[j], k);
+}
+
+__global__ void counter_add_kernel(float* __restrict__ c, float delta) {
+  if (threadIdx.x == 0 && blockIdx.x == 0) c[0] = c[0] + delta;
+}
+
 // kind: 0 = SGD with momentum / weight decay, 1 = Adagrad, 2 = RMSprop. `s` is the state tensor (velocity or cache).
 struct OptK {
   int kind;
@@ -223,6 +252,38 @@ int32_t endia_hip_sgd_step_multi(int32_t count, const int64_t* n, float* const* 
     hipLaunchKernelGGL(sgd_multi_kernel, dim3((unsigned)stream_grid(largest), (unsigned)m), dim3(TPB), 0, ctx().stream, t, lr);
     ENDIA_LAUNCH_CHECK();
   }
+  return ENDIA_HIP_OK;
+}
+
+int32_t endia_hip_adam_step_multi(int32_t count, const int64_t* n, float* const* p, const float* const* g, float* const* m,
+                                  float* const* v, float lr, float beta1, float beta2, float eps, float* step) {
+  ENDIA_REQUIRE_INIT();
+  ENDIA_CHECK_ARG(count >= 0, "endia_hip_adam_step_multi: negative count");
+  ENDIA_CHECK_ARG(step != nullptr, "endia_hip_adam_step_multi: the step counter is null");
+  if (count == 0) return ENDIA_HIP_OK;
+  ENDIA_CHECK_ARG(n && p && g && m && v, "endia_hip_adam_step_multi: null table");
+  AdamK k;
+  k.lr = lr; k.b1 = beta1; k.b2 = beta2; k.eps = eps;
+  k.omb1 = 1.0f - beta1;
+  k.omb2 = 1.0f - beta2;
+  k.c1 = k.c2 = 1.f;  // set on the device from the counter
+  for (int32_t first = 0; first < count; first += MULTI_MAX) {
+    const int32_t cnt = count - first < MULTI_MAX ? count - first : MULTI_MAX;
+    AdamMulti t = {};
+    int64_t largest = 0;
+    for (int32_t i = 0; i < cnt; ++i) {
+      const int32_t j = first + i;
+      ENDIA_CHECK_ARG(n[j] >= 0, "endia_hip_adam_step_multi: tensor %d has a negative size", j);
+      ENDIA_CHECK_ARG(n[j] == 0 || (p[j] && g[j] && m[j] && v[j]), "endia_hip_adam_step_multi: tensor %d has a null pointer", j);
+      t.p[i] = p[j]; t.g[i] = g[j]; t.m[i] = m[j]; t.v[i] = v[j]; t.n[i] = n[j];
+      if (t.n[i] > largest) largest = t.n[i];
+    }
+    if (largest == 0) continue;
+    hipLaunchKernelGGL(adam_multi_kernel, dim3((unsigned)stream_grid(largest), (unsigned)cnt), dim3(TPB), 0, ctx().stream, t, k, step);
+    ENDIA_LAUNCH_CHECK();
+  }
+  hipLaunchKernelGGL(counter_add_kernel, dim3(1), dim3(64), 0, ctx().stream, step, 1.0f);  // t + 1 after all parameters (adam.mojo:65)
+  ENDIA_LAUNCH_CHECK();
   return ENDIA_HIP_OK;
 }
 

@@ -8,7 +8,7 @@ step computes.
     def step():
         loss = nd.mse(mlp.forward(x), y)
         loss.backward()
-        opt.step()          # SGD / Adagrad / RMSprop; Adam's step counter changes per step, see below
+        opt.step()          # SGD / Adagrad / RMSprop, or Adam(capturable=True); see below
         loss.zero_grad()
         return loss
 
@@ -19,8 +19,10 @@ step computes.
         captured.replay()
     print(captured.outputs.item())
 
-Scalar kernel arguments are frozen at capture time, so an optimizer whose scalars change from step
-to step (Adam's bias correction) refuses to run inside a capture.
+Scalar kernel arguments are frozen at capture time. Adam's bias correction 1 - beta^t changes every step:
+`Adam(..., capturable=True)` keeps t in device memory, where the update kernel reads it and a last tiny
+kernel adds one, so nothing in the recorded launches depends on the step number; an Adam whose counter
+lives on the host refuses to run inside a capture.
 """
 import ctypes
 

@@ -88,19 +88,50 @@ class RMSprop:
 
 
 class Adam:
-    """adam.mojo:14-65. `t` is an fp32 counter that starts at 1 and grows by one per step()."""
+    """adam.mojo:14-65. `t` is an fp32 counter that starts at 1 and grows by one per step().
 
-    def __init__(self, params, lr=0.001, beta1=0.9, beta2=0.999, eps=1e-8):
+    capturable=True (or the first step() taken while a step is being captured) keeps the counter in device memory
+    and updates every parameter tensor in one launch that reads it there, so the step can be replayed as a HIP
+    graph; the bias corrections then come from the device's powf (last-bit differences from the host's)."""
+
+    def __init__(self, params, lr=0.001, beta1=0.9, beta2=0.999, eps=1e-8, capturable=False):
         self.params = list(params)
         self.lr, self.beta1, self.beta2, self.eps = (float(np.float32(v)) for v in (lr, beta1, beta2, eps))
         self.t = 1.0
         self.m = [Array(p.shape()) for p in self.params]
         self.v = [Array(p.shape()) for p in self.params]
+        self._t_dev = None
+        if capturable:
+            self._device_counter()
+
+    def _device_counter(self):
+        if self._t_dev is None:
+            if L.capturing:
+                raise RuntimeError("Adam: take one eager step() (or pass capturable=True) before capturing, so that the "
+                                   "device step counter exists when the capture starts")
+            from . import functional as F
+            self._t_dev = F.full([1], self.t)
+        return self._t_dev
+
+    def step_count(self):
+        """The counter t that the next step() will use."""
+        return float(self._t_dev.item()) if self._t_dev is not None else self.t
 
     def step(self):
-        if L.capturing:
-            raise NotImplementedError("Adam inside a captured step: its bias correction 1 - beta^t changes every step, "
-                                      "but a captured kernel's scalar arguments are frozen")
+        if self._t_dev is not None or L.capturing:
+            import ctypes
+            t_dev = self._device_counter()
+            grads = [_flat_grad(p) for p in self.params]
+            k = len(self.params)
+            assert all(p.is_contiguous() for p in self.params)
+            vp = ctypes.c_void_p * k
+            L.call("endia_hip_adam_step_multi", k, L.i64_array([p.size() for p in self.params]),
+                   vp(*[p.data_ptr() for p in self.params]), vp(*[g.data_ptr() for g in grads]),
+                   vp(*[m.data_ptr() for m in self.m]), vp(*[v.data_ptr() for v in self.v]),
+                   self.lr, self.beta1, self.beta2, self.eps, t_dev.data_ptr())
+            for p in self.params:
+                p.clear_args()
+            return
         for p, m, v in zip(self.params, self.m, self.v):
             g = _flat_grad(p)
             assert p.is_contiguous()

@@ -335,6 +335,14 @@ ENDIA_API int32_t endia_hip_sgd_step(int64_t n, float* p, const float* g, float 
 /* The same update for `count` parameter tensors in one launch (n, p, g are host arrays of length count): a model
  * of many small tensors, like the reference's sine-fit MLP, is bound by launch latency rather than bandwidth. */
 ENDIA_API int32_t endia_hip_sgd_step_multi(int32_t count, const int64_t* n, float* const* p, const float* const* g, float lr);
+/* Adam.step for `count` tensors with the step counter t in DEVICE memory (`step`: one float, 1 before the first
+ * step): the kernels read it, compute 1 - beta^t themselves, and a last tiny kernel adds 1 to it after all
+ * parameters (adam.mojo:65). No argument changes from one step to the next, so the call can be recorded into a
+ * captured step and replayed. beta^t comes from the device's powf here and from the host's in endia_hip_adam_step:
+ * the two may differ in the last bit of the bias corrections (1e-7 relative in the update). */
+ENDIA_API int32_t endia_hip_adam_step_multi(int32_t count, const int64_t* n, float* const* p, const float* const* g,
+                                  float* const* m, float* const* v, float lr, float beta1, float beta2, float eps,
+                                  float* step);
 /* SGD with momentum and / or weight decay (optim/sgd.mojo:42-60): vel = momentum*vel - lr*(g + wd*p); p += vel
  * (without momentum: p -= lr*(g + wd*p); vel may then be null). Adagrad (optim/adagrad.mojo:36-45):
  * cache += g*g; p -= lr*g / (sqrt(cache) + eps). RMSprop (optim/rmsprop.mojo:39-53):

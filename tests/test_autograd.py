@@ -490,16 +490,65 @@ def test_captured_step_matches_eager(nd, golden):
     captured.close()
     with pytest.raises(RuntimeError):
         captured.replay()
-    # host reads and Adam are refused inside a capture, and the failed capture leaves the library usable
+    # host reads are refused inside a capture, and so is an Adam whose step counter still lives on the host; the
+    # failed captures leave the library usable
     with pytest.raises(nd._lib.EndiaHipError, match="captured"):
         nd.capture(lambda: scratch.to_numpy())
     mlp_a, _ = _load_mlp(nd, g, 8, "relu", True)
     adam = nd.optim.Adam(mlp_a.params())
     for p in mlp_a.params():
         p.grad_(nd.zeros(p.shape()))
-    with pytest.raises(NotImplementedError):
+    with pytest.raises(RuntimeError, match="capturable"):
         nd.capture(adam.step)
     assert nd.sum(nd.ones([5])).item() == 5.0
+
+
+def test_captured_adam_step(nd, golden):
+    """Adam with its step counter in device memory (capturable=True): the captured step, replayed, follows the
+    eager host-counter Adam and the oracle's Adam step for step (1e-6: the bias corrections come from the device's
+    powf), and the counter advances by one per replay."""
+    from oracle import endia_ref as R
+    g = golden("mlp_sine")
+    mlp_e, _ = _load_mlp(nd, g, 8, "relu", True)
+    mlp_c, _ = _load_mlp(nd, g, 8, "relu", True)
+    opt_e = nd.optim.Adam(mlp_e.params(), lr=1e-2)
+    opt_c = nd.optim.Adam(mlp_c.params(), lr=1e-2, capturable=True)
+    x, y = nd.array(g["x"]), nd.array(g["y"])
+
+    def make(mlp, opt):
+        def step():
+            loss = nd.mse(mlp.forward(x), y)
+            loss.backward()
+            opt.step()
+            loss.zero_grad()
+            return loss
+        return step
+
+    step_e, step_c = make(mlp_e, opt_e), make(mlp_c, opt_c)
+    step_e()
+    step_c()                                   # eager, through the device-counter path
+    assert opt_c.step_count() == 2.0
+    captured = nd.capture(step_c)
+    for it in range(5):
+        loss_e = step_e()
+        loss_c = captured.replay()
+        assert_close([loss_c.item()], [loss_e.item()], tol=1e-5, what="loss at replay %d" % it)
+        for pe, pc in zip(mlp_e.params(), mlp_c.params()):
+            assert_close(pc.to_numpy(), pe.to_numpy(), tol=2e-6, what="parameters at replay %d" % it)
+    assert opt_c.step_count() == 7.0 and opt_e.t == 7.0
+    captured.close()
+    # one tensor, three steps, against the oracle's Adam
+    rng = np.random.default_rng(12)
+    p0 = rng.standard_normal((37, 5)).astype(np.float32)
+    grads = [rng.standard_normal((37, 5)).astype(np.float32) for _ in range(3)]
+    p = nd.array(p0, requires_grad=True)
+    opt = nd.optim.Adam([p], lr=1e-2, capturable=True)
+    pr, m, v = p0.copy(), np.zeros_like(p0), np.zeros_like(p0)
+    for i, gr in enumerate(grads):
+        p.grad_(nd.array(gr))
+        opt.step()
+        pr, m, v = R.adam(pr, gr, m, v, lr=1e-2, t=float(i + 1))
+        assert_close(p.to_numpy(), pr, tol=1e-6, what="oracle step %d" % i)
 
 
 def test_shape_errors(nd):
