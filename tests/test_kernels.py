@@ -865,3 +865,32 @@ def test_conv_and_pool_random_configs(dev):
             assert_close(y, ty.detach().numpy(), what=what + " fwd")
             assert_close(dx, t.grad.numpy(), what=what + " grad")
         dev.release()
+
+
+@pytest.mark.gpu
+def test_adam_step_multi(dev):
+    """endia_hip_adam_step_multi through the C ABI: 40 tensors (two launch tables, one of them empty), three steps
+    with the counter in device memory, against the oracle's Adam (1e-6: device powf) and the counter's own value."""
+    rng = np.random.default_rng(31)
+    sizes = [1, 5, 1024, 0, 33, 4096] + [7] * 34
+    k = len(sizes)
+    P = [rng.standard_normal(n).astype(np.float32) for n in sizes]
+    M = [np.zeros(n, np.float32) for n in sizes]
+    V = [np.zeros(n, np.float32) for n in sizes]
+    dp, dm, dv = [dev.put(a) for a in P], [dev.put(a) for a in M], [dev.put(a) for a in V]
+    dt = dev.put(np.array([1.0], np.float32))
+    vp = ctypes.c_void_p * k
+    for step in range(3):
+        G = [rng.standard_normal(n).astype(np.float32) for n in sizes]
+        dg = [dev.put(a) for a in G]
+        dev.call("endia_hip_adam_step_multi", k, L.i64_array(sizes), vp(*dp), vp(*dg), vp(*dm), vp(*dv),
+                 1e-2, 0.9, 0.999, 1e-8, dt)
+        for i in range(k):
+            P[i], M[i], V[i] = R.adam(P[i], G[i], M[i], V[i], lr=1e-2, t=float(step + 1))
+        assert dev.get(dt, (1,))[0] == step + 2.0
+        for i in (0, 1, 2, 4, 5, 20, 39):
+            assert_close(dev.get(dp[i], (sizes[i],)), P[i], tol=1e-6, what="p[%d] after step %d" % (i, step))
+            assert_close(dev.get(dv[i], (sizes[i],)), V[i], tol=1e-6, what="v[%d] after step %d" % (i, step))
+    with pytest.raises(L.EndiaHipError):
+        dev.call("endia_hip_adam_step_multi", k, L.i64_array(sizes), vp(*dp), vp(*dg), vp(*dm), vp(*dv), 1e-2, 0.9, 0.999, 1e-8, None)
+    dev.call("endia_hip_adam_step_multi", 0, None, None, None, None, None, 1e-2, 0.9, 0.999, 1e-8, dt)
