@@ -606,41 +606,6 @@ __global__ __launch_bounds__(WGM* WGN * 64, 4) void conv_wgrad_vec_kernel(WgradV
   }
 }
 
-// Zero-padded copy: dst[pl][z][y][x] = src[pl][z - pz][y - py][x - px] where in range, else 0. One wave per
-// padded row (rows are short: the walk over x needs no division, and reads and writes stay contiguous).
-__global__ __launch_bounds__(TPB) void pad_kernel(const float* __restrict__ src, float* __restrict__ dst, int64_t rows_total,
-                                                  int D, int H, int W, int Dp, int Hp, int Wp, int pz, int py, int px) {
-  const int lane = threadIdx.x & 63;
-  const int64_t waves = (int64_t)gridDim.x * (TPB / 64);
-  for (int64_t row = (int64_t)blockIdx.x * (TPB / 64) + (threadIdx.x >> 6); row < rows_total; row += waves) {
-    const int64_t slab = row / Hp;  // (plane, padded depth)
-    const int y = (int)(row - slab * Hp), sy = y - py;
-    const int64_t pl = slab / Dp;
-    const int sz = (int)(slab - pl * Dp) - pz;
-    const bool row_ok = (unsigned)sy < (unsigned)H && (unsigned)sz < (unsigned)D;
-    const float* s = src + ((pl * D + (row_ok ? sz : 0)) * H + (row_ok ? sy : 0)) * W;
-    float* d = dst + row * Wp;
-    for (int x = lane; x < Wp; x += 64) {
-      int sx = x - px;
-      d[x] = (row_ok && (unsigned)sx < (unsigned)W) ? s[sx] : 0.f;
-    }
-  }
-}
-
-// table[t] for t = (ch, kz, r, s): byte offset ((ch*Dp + kz*dd)*Hp + r*dh)*Wp + s*dw inside a padded image; the
-// data gradient walks the taps in reverse (kz -> T-1-kz, r -> R-1-r, s -> S-1-s). Entries past Kd get OOB_OFFSET.
-__global__ __launch_bounds__(TPB) void tap_table_kernel(int* __restrict__ table, int n, int Kd, int T, int R, int S, int Dp,
-                                                        int Hp, int Wp, int dd, int dh, int dw, int flip) {
-  int t = blockIdx.x * TPB + threadIdx.x;
-  if (t >= n) return;
-  if (t >= Kd) { table[t] = (int)OOB_OFFSET; return; }
-  int ch = t / (T * R * S), rem = t - ch * T * R * S, kz = rem / (R * S);
-  rem -= kz * R * S;
-  int r = rem / S, s = rem - r * S;
-  if (flip) { kz = T - 1 - kz; r = R - 1 - r; s = S - 1 - s; }
-  table[t] = (((ch * Dp + kz * dd) * Hp + r * dh) * Wp + s * dw) * 4;
-}
-
 // ---- weight repacking -------------------------------------------------------------------------------
 // fwd:  wp[k][t]          = w[k][t]                     t = (c, kz, r, s), rows padded to Kd_pad with zeros
 // data: wp[c][(k,kz,r,s)] = w[k][c][kz][r][s]            (RS below is T*R*S)
@@ -657,6 +622,64 @@ __global__ __launch_bounds__(TPB) void pack_weights_kernel(const float* __restri
       else { int k = t / RS, rs = t - k * RS; v = w[((int64_t)k * C + m) * RS + rs]; }
     }
     wp[i] = v;
+  }
+}
+
+// The set-up of a vectorised call in ONE launch: the first work-groups write the tap table, the next ones repack
+// the weights (when there are any to repack), the rest make the zero-padded copy. The three are independent;
+// as three launches they cost about ten microseconds of a call that lasts three hundred.
+//   table[t], t = (ch, kz, r, s): byte offset ((ch*Dp + kz*dd)*Hp + r*dh)*Wp + s*dw inside a padded image; the data
+//     gradient walks the taps in reverse (kz -> T-1-kz, r -> R-1-r, s -> S-1-s); entries past Kd get OOB_OFFSET.
+//   padded copy: dst[pl][z][y][x] = src[pl][z - pz][y - py][x - px] where in range, else 0; one wave per padded row
+//     (rows are short: the walk over x needs no division, and reads and writes stay contiguous).
+struct PrepArgs {
+  const float* src; float* dst; int64_t rows_total; int D, H, W, Dp, Hp, Wp, pz, py, px;   // padded copy
+  int* table; int tn, Kd, T, R, S, dd, dh, dw, flip;                                        // tap table
+  const float* w; float* wp; int K, C, RS, Kd_pad, transpose;                               // weight repacking (w may be null)
+  int table_blocks, pack_blocks;
+};
+
+__global__ __launch_bounds__(TPB) void conv_prep_kernel(PrepArgs a) {
+  const int b = blockIdx.x;
+  if (b < a.table_blocks) {
+    int t = b * TPB + threadIdx.x;
+    if (t >= a.tn) return;
+    if (t >= a.Kd) { a.table[t] = (int)OOB_OFFSET; return; }
+    int ch = t / (a.T * a.R * a.S), rem = t - ch * a.T * a.R * a.S, kz = rem / (a.R * a.S);
+    rem -= kz * a.R * a.S;
+    int r = rem / a.S, s = rem - r * a.S;
+    if (a.flip) { kz = a.T - 1 - kz; r = a.R - 1 - r; s = a.S - 1 - s; }
+    a.table[t] = (((ch * a.Dp + kz * a.dd) * a.Hp + r * a.dh) * a.Wp + s * a.dw) * 4;
+  } else if (b < a.table_blocks + a.pack_blocks) {
+    const int rows = a.transpose ? a.C : a.K;
+    const int64_t total = (int64_t)rows * a.Kd_pad;
+    const int kd = (a.transpose ? a.K : a.C) * a.RS;
+    for (int64_t i = (int64_t)(b - a.table_blocks) * TPB + threadIdx.x; i < total; i += (int64_t)a.pack_blocks * TPB) {
+      int m = (int)(i / a.Kd_pad), t = (int)(i - (int64_t)m * a.Kd_pad);
+      float v = 0.f;
+      if (t < kd) {
+        if (!a.transpose) v = a.w[(int64_t)m * kd + t];
+        else { int k = t / a.RS, rs = t - k * a.RS; v = a.w[((int64_t)k * a.C + m) * a.RS + rs]; }
+      }
+      a.wp[i] = v;
+    }
+  } else {
+    const int first = a.table_blocks + a.pack_blocks;
+    const int lane = threadIdx.x & 63;
+    const int64_t waves = (int64_t)(gridDim.x - first) * (TPB / 64);
+    for (int64_t row = (int64_t)(b - first) * (TPB / 64) + (threadIdx.x >> 6); row < a.rows_total; row += waves) {
+      const int64_t slab = row / a.Hp;  // (plane, padded depth)
+      const int y = (int)(row - slab * a.Hp), sy = y - a.py;
+      const int64_t pl = slab / a.Dp;
+      const int sz = (int)(slab - pl * a.Dp) - a.pz;
+      const bool row_ok = (unsigned)sy < (unsigned)a.H && (unsigned)sz < (unsigned)a.D;
+      const float* s = a.src + ((pl * a.D + (row_ok ? sz : 0)) * a.H + (row_ok ? sy : 0)) * a.W;
+      float* d = a.dst + row * a.Wp;
+      for (int x = lane; x < a.Wp; x += 64) {
+        int sx = x - a.px;
+        d[x] = (row_ok && (unsigned)sx < (unsigned)a.W) ? s[sx] : 0.f;
+      }
+    }
   }
 }
 
@@ -720,29 +743,6 @@ inline int grid_for(int64_t n) {
   return (int)(b < 1 ? 1 : b);
 }
 
-// Padded copy of a [planes, D, H, W] tensor with (pz, py, px) zeros on every side.
-int32_t make_padded(const float* src, int64_t planes, int D, int H, int W, int pz, int py, int px, PoolBuf& buf) {
-  const int Dp = D + 2 * pz, Hp = H + 2 * py, Wp = W + 2 * px;
-  int32_t rc = endia_hip_malloc(planes * Dp * Hp * Wp * 4, &buf.p);
-  if (rc) return rc;
-  const int64_t rows = planes * Dp * Hp;
-  int64_t blocks = (rows + 3) / 4, cap = (int64_t)endia::ctx().cu_count * 64;
-  if (blocks > cap) blocks = cap;
-  hipLaunchKernelGGL(pad_kernel, dim3((unsigned)blocks), dim3(TPB), 0, endia::ctx().stream, src,
-                     static_cast<float*>(buf.p), rows, D, H, W, Dp, Hp, Wp, pz, py, px);
-  ENDIA_LAUNCH_CHECK();
-  return ENDIA_HIP_OK;
-}
-
-int32_t make_table(int n, int Kd, const ConvP& p, int Dp, int Hp, int Wp, int flip, PoolBuf& buf) {
-  int32_t rc = endia_hip_malloc((int64_t)n * 4, &buf.p);
-  if (rc) return rc;
-  hipLaunchKernelGGL(tap_table_kernel, dim3((n + TPB - 1) / TPB), dim3(TPB), 0, endia::ctx().stream,
-                     static_cast<int*>(buf.p), n, Kd, p.T, p.R, p.S, Dp, Hp, Wp, p.dd, p.dh, p.dw, flip);
-  ENDIA_LAUNCH_CHECK();
-  return ENDIA_HIP_OK;
-}
-
 int32_t pack_weights(const ConvP& p, const float* w, int transpose, int Kd_pad, PoolBuf& buf) {
   const int rows = transpose ? p.C : p.K;
   int32_t rc = endia_hip_malloc((int64_t)rows * Kd_pad * 4, &buf.p);
@@ -752,6 +752,36 @@ int32_t pack_weights(const ConvP& p, const float* w, int transpose, int Kd_pad, 
   if (blocks > 2048) blocks = 2048;
   hipLaunchKernelGGL(pack_weights_kernel, dim3(blocks), dim3(TPB), 0, endia::ctx().stream, w, static_cast<float*>(buf.p),
                      p.K, p.C, p.T * p.R * p.S, Kd_pad, transpose);
+  ENDIA_LAUNCH_CHECK();
+  return ENDIA_HIP_OK;
+}
+
+// Padded copy of src, tap table of n entries and (when w is given) repacked weights, from one launch.
+int32_t prep_vec(const ConvP& p, const float* src, int64_t planes, int SD, int SH, int SW, int pz, int py, int px, int n_table,
+                 int Kd, int flip, const float* w, int transpose, int Kd_pad, PoolBuf& spad, PoolBuf& table, PoolBuf& wp) {
+  const int Dp = SD + 2 * pz, Hp = SH + 2 * py, Wp = SW + 2 * px;
+  int32_t rc = endia_hip_malloc(planes * Dp * Hp * Wp * 4, &spad.p);
+  if (rc) return rc;
+  if ((rc = endia_hip_malloc((int64_t)n_table * 4, &table.p))) return rc;
+  PrepArgs a = {};
+  a.src = src; a.dst = static_cast<float*>(spad.p); a.rows_total = planes * Dp * Hp;
+  a.D = SD; a.H = SH; a.W = SW; a.Dp = Dp; a.Hp = Hp; a.Wp = Wp; a.pz = pz; a.py = py; a.px = px;
+  a.table = static_cast<int*>(table.p); a.tn = n_table; a.Kd = Kd; a.T = p.T; a.R = p.R; a.S = p.S;
+  a.dd = p.dd; a.dh = p.dh; a.dw = p.dw; a.flip = flip;
+  a.table_blocks = (n_table + TPB - 1) / TPB;
+  a.pack_blocks = 0;
+  if (w) {
+    const int rows = transpose ? p.C : p.K;
+    if ((rc = endia_hip_malloc((int64_t)rows * Kd_pad * 4, &wp.p))) return rc;
+    a.w = w; a.wp = static_cast<float*>(wp.p); a.K = p.K; a.C = p.C; a.RS = p.T * p.R * p.S; a.Kd_pad = Kd_pad; a.transpose = transpose;
+    int64_t pb = ((int64_t)rows * Kd_pad + TPB - 1) / TPB;
+    a.pack_blocks = (int)(pb > 2048 ? 2048 : pb);
+  }
+  int64_t pad_blocks = (a.rows_total + 3) / 4, cap = (int64_t)endia::ctx().cu_count * 64;
+  if (pad_blocks > cap) pad_blocks = cap;
+  if (pad_blocks < 1) pad_blocks = 1;
+  hipLaunchKernelGGL(conv_prep_kernel, dim3((unsigned)(a.table_blocks + a.pack_blocks + pad_blocks)), dim3(TPB), 0,
+                     endia::ctx().stream, a);
   ENDIA_LAUNCH_CHECK();
   return ENDIA_HIP_OK;
 }
@@ -778,10 +808,9 @@ int32_t run_igemm_vec(int mode, const ConvP& p, const float* src, const float* w
   // the last reads of a row group must stay inside the padded image rows: ox + 3 + (S-1)*dw <= Wp - 1 holds because
   // OW - 1 + (S-1)*dw <= Wp - 1 by the output-size rule; nothing else to check.
   PoolBuf spad, wp, table;
-  int32_t rc = make_padded(src, (int64_t)p.N * Cred, SD, SH, SW, pz, py, px, spad);
+  int32_t rc = prep_vec(p, src, (int64_t)p.N * Cred, SD, SH, SW, pz, py, px, Kd_pad, Kd, fwd ? 0 : 1, w, fwd ? 0 : 1, Kd_pad,
+                        spad, table, wp);
   if (rc) return rc;
-  if ((rc = pack_weights(p, w, fwd ? 0 : 1, Kd_pad, wp))) return rc;
-  if ((rc = make_table(Kd_pad, Kd, p, Dp, Hp, Wp, fwd ? 0 : 1, table))) return rc;
   VecArgs a;
   a.src = static_cast<const float*>(spad.p); a.wp = static_cast<const float*>(wp.p);
   a.table = static_cast<const int*>(table.p); a.bias = bias; a.out = out; a.relu = relu;
@@ -936,9 +965,10 @@ int32_t conv_bwd_weight(const char* who, const ConvP& p, const float* x, const f
   }
   dim3 grid((unsigned)tiles, (unsigned)splits);
   if (vec) {
-    PoolBuf xpad, table;
-    if ((rc = make_padded(x, (int64_t)p.N * p.C, p.D, p.H, p.W, p.pd, p.ph, p.pw, xpad))) return rc;
-    if ((rc = make_table(a.tiles_n * bn, Kd, p, Dp, Hp, Wp, 0, table))) return rc;
+    PoolBuf xpad, table, none;
+    if ((rc = prep_vec(p, x, (int64_t)p.N * p.C, p.D, p.H, p.W, p.pd, p.ph, p.pw, a.tiles_n * bn, Kd, 0, nullptr, 0, 0, xpad, table,
+                       none)))
+      return rc;
     WgradVecArgs v;
     v.xpad = static_cast<const float*>(xpad.p); v.dy = dy; v.table = static_cast<const int*>(table.p); v.part = a.part;
     v.K = p.K; v.Kd = Kd; v.OPQ = p.O * p.P * p.Q; v.PQ = p.P * p.Q; v.Q = p.Q; v.sh = p.sh; v.Wp = Wp;
