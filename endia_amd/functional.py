@@ -925,7 +925,6 @@ def conv2d(x, kernel, bias=None, stride=1, padding=0, dilation=1, groups=1, act=
     derivative on the way into the gradients, instead of as separate passes over the output."""
     if act not in (None, "relu"):
         raise ValueError("conv2d: act must be None or 'relu'")
-    _act = act
     if x.ndim() != 4:
         raise ValueError("Input must be 4-dimensional (batch_size, in_channels, height, width) for 2D convolution!")
     if x._shape[1] != kernel._shape[1]:
@@ -942,15 +941,14 @@ def conv2d(x, kernel, bias=None, stride=1, padding=0, dilation=1, groups=1, act=
     xs, ks = contiguous(x), contiguous(kernel)
     bsrc = contiguous(bias) if bias is not None else None
     out = Array.empty([N, K, P.value, Q.value])
-    act = L.OP_RELU if _act == "relu" else L.OP_IDENTITY
     L.call("endia_hip_conv2d_fwd", ctypes.byref(desc), xs.data_ptr(), ks.data_ptr(),
-           bsrc.data_ptr() if bsrc is not None else None, out.data_ptr(), act)
+           bsrc.data_ptr() if bsrc is not None else None, out.data_ptr(), L.OP_RELU if act == "relu" else L.OP_IDENTITY)
 
     def vjp(primals, grad, out_):
         from .autograd.functional import building_graph
         if building_graph():
             raise NotImplementedError("conv2d has no second-order rule")
-        g = contiguous(_relu_grad_from_output(out_, grad)) if _act == "relu" else contiguous(grad)
+        g = contiguous(_relu_grad_from_output(out_, grad)) if act == "relu" else contiguous(grad)
         res = []
         if primals[0]._requires_grad:
             dx = Array.empty(primals[0]._shape)
