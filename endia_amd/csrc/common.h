@@ -16,7 +16,12 @@ struct Context {
   hipStream_t stream = nullptr;
   int cu_count = 0;
   int clock_mhz = 0;
+  // Arrival counters of kernels whose work-groups meet in memory (the last one to arrive finishes the job).
+  // All zero between launches: the group that arrives last puts its counter back to zero.
+  unsigned* tickets = nullptr;
 };
+
+constexpr int kTicketCount = 4096;
 
 Context& ctx();
 int32_t fail(int32_t code, const char* fmt, ...);

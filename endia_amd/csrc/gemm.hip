@@ -45,6 +45,9 @@ struct GemmArgs {
   int M, N, K;
   int tiles_m, tiles_n;
   int k_split;    // > 0: grid.y indexes slices of K of this length instead of batch entries
+  int splits;     // > 0: the slices' partial sums meet in `part` and the last group of a tile to arrive finishes it
+  float* part;    // [splits][tiles][accumulator registers][256 lanes]
+  unsigned* tickets;  // one arrival counter per tile, zero between launches
   int act;        // endia_hip_unary_op
   int from_out;   // activation gradient from stored output instead of pre-activation
   int accumulate;
@@ -123,9 +126,10 @@ __device__ __forceinline__ void gemm_tile(const GemmArgs& p, int block, int nblo
   int tm, tn;
   tile_of_block(block, nblocks, p.tiles_m, p.tiles_n, tm, tn);
   const int m0 = tm * BM, n0 = tn * BN;
-  float* __restrict__ C = p.C + bz * p.sC;
-  const float* __restrict__ aux_in = p.aux_in ? p.aux_in + bz * p.sC : nullptr;
-  float* __restrict__ aux_out = p.aux_out ? p.aux_out + bz * p.sC : nullptr;
+  const int64_t cz = p.splits ? 0 : bz;  // every slice of a split reduction belongs to the one C
+  float* __restrict__ C = p.C + cz * p.sC;
+  const float* __restrict__ aux_in = p.aux_in ? p.aux_in + cz * p.sC : nullptr;
+  float* __restrict__ aux_out = p.aux_out ? p.aux_out + cz * p.sC : nullptr;
 
   // split-K: this group reduces k in [bz * k_split, bz * k_split + K) and writes slice bz of the partials
   const int K = p.k_split ? (p.K - (int)bz * p.k_split < p.k_split ? p.K - (int)bz * p.k_split : p.k_split) : p.K;
@@ -217,6 +221,47 @@ __device__ __forceinline__ void gemm_tile(const GemmArgs& p, int block, int nblo
 
   if (do_colsum && n0 + tid < p.N) p.aux_out[n0 + tid] = colsum;
 
+  // K split over gridDim.y groups per tile: every group leaves its accumulators in memory (register order, so the
+  // stores and loads are contiguous per wave) and takes a ticket; the group that draws the last ticket adds the
+  // slices in slice order, whichever group it is, so the sum does not depend on timing, and runs the epilogue.
+  // The partial sums travel as device-scope stores and loads (written through to, and read from, the level all
+  // XCDs share) rather than behind device-scope fences, which write back and invalidate a whole L2 per use: a
+  // wave's stores have completed when its counter of outstanding memory operations is zero, which the barrier
+  // ahead of the ticket waits for.
+  if (p.splits) {
+    constexpr int64_t SLICE = (int64_t)F * F * 16 * NTHREADS;
+    float* mine = p.part + (bz * nblocks + block) * SLICE + tid;
+#pragma unroll
+    for (int f = 0; f < F * F; ++f)
+#pragma unroll
+      for (int v = 0; v < 16; ++v)
+        __hip_atomic_store(mine + (f * 16 + v) * NTHREADS, acc[f / F][f % F][v], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    __builtin_amdgcn_s_waitcnt(0);
+    __syncthreads();
+    int* flag = reinterpret_cast<int*>(As);
+    if (tid == 0) {
+      const unsigned arrived = __hip_atomic_fetch_add(&p.tickets[block], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      const bool last = arrived + 1u == (unsigned)p.splits;
+      if (last) __hip_atomic_store(&p.tickets[block], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);  // for the next launch
+      flag[0] = last;
+    }
+    __syncthreads();
+    if (!flag[0]) return;
+    zero_acc<F, F>(acc);
+    for (int s = 0; s < p.splits; ++s) {
+      const float* theirs = p.part + ((int64_t)s * nblocks + block) * SLICE + tid;
+#pragma unroll
+      for (int f = 0; f < F * F; ++f) {
+        float t[16];  // sixteen loads in flight, then sixteen additions
+#pragma unroll
+        for (int v = 0; v < 16; ++v)
+          t[v] = __hip_atomic_load(theirs + (f * 16 + v) * NTHREADS, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+#pragma unroll
+        for (int v = 0; v < 16; ++v) acc[f / F][f % F][v] += t[v];
+      }
+    }
+  }
+
 #pragma unroll
   for (int fm = 0; fm < F; ++fm)
 #pragma unroll
@@ -267,9 +312,10 @@ __global__ __launch_bounds__(256) void sgemm_generic_kernel(GemmArgs p, int tran
   const int64_t bz = blockIdx.z;
   const float* __restrict__ A = p.A + bz * p.sA;
   const float* __restrict__ B = p.B + bz * p.sB;
-  float* __restrict__ C = p.C + bz * p.sC;
-  const float* __restrict__ aux_in = p.aux_in ? p.aux_in + bz * p.sC : nullptr;
-  float* __restrict__ aux_out = p.aux_out ? p.aux_out + bz * p.sC : nullptr;
+  const int64_t cz = p.splits ? 0 : bz;  // every slice of a split reduction belongs to the one C
+  float* __restrict__ C = p.C + cz * p.sC;
+  const float* __restrict__ aux_in = p.aux_in ? p.aux_in + cz * p.sC : nullptr;
+  float* __restrict__ aux_out = p.aux_out ? p.aux_out + cz * p.sC : nullptr;
   float acc[4][4] = {};
   for (int k0 = 0; k0 < p.K; k0 += TK) {
     for (int e = tid; e < T * TK; e += 256) {
@@ -442,7 +488,7 @@ int32_t sgemm_impl(int transA, int transB, int64_t M, int64_t N, int64_t K, cons
   if (epi == ENDIA_EPI_BIAS || epi == ENDIA_EPI_BIAS_ACT) ENDIA_CHECK_ARG(bias != nullptr, "sgemm: epilogue needs bias");
   if (epi == ENDIA_EPI_ACT_GRAD) ENDIA_CHECK_ARG(aux_in != nullptr, "sgemm: ACT_GRAD epilogue needs aux_in");
 
-  GemmArgs p;
+  GemmArgs p{};
   p.A = A; p.B = B; p.C = C; p.bias = bias; p.aux_in = aux_in;
   p.aux_out = (epi == ENDIA_EPI_BIAS_ACT) ? aux_out : nullptr;
   p.colsum = 0;
@@ -473,13 +519,24 @@ int32_t sgemm_impl(int transA, int transB, int64_t M, int64_t N, int64_t K, cons
     p.tiles_n = (int)ceil_div64(N, 64 * F);
     const int64_t tiles = (int64_t)p.tiles_m * p.tiles_n;
     ENDIA_CHECK_ARG(tiles < (1ll << 31), "sgemm: too many output tiles");
-    // A long reduction with few output tiles (dW of a narrow layer over a large batch) is split along K:
-    // slices write partial products that are then added in slice order.
+    // A product with fewer than two tiles per CU is split along K so that more groups are in flight (a lone group
+    // per CU spends most of its time waiting for loads). Up to 16 slices of at least 128: the slices of a tile are
+    // added, in slice order, by whichever of its groups finishes last, inside the one launch, with any epilogue.
+    // A long reduction with very few tiles (dW of a narrow layer over a large batch) wants more slices than one
+    // group should add up: its partial products are added, also in slice order, by a second, chip-wide launch.
     int64_t splits = 1;
-    if (batch == 1 && epi == ENDIA_EPI_NONE && !accumulate && ldc == N && tiles * 2 <= cus && K >= 2048) {
-      splits = (4 * cus + tiles - 1) / tiles;
-      if (splits > K / 256) splits = K / 256;
-      if (splits > 1024) splits = 1024;
+    bool meet_in_kernel = false;
+    if (batch == 1 && K >= 256) {
+      int64_t want = (4 * cus) / tiles;
+      if (want > K / 128) want = K / 128;
+      if (want > 16 && epi == ENDIA_EPI_NONE && !accumulate && ldc == N && K >= 2048) {
+        splits = (4 * cus + tiles - 1) / tiles;
+        if (splits > K / 256) splits = K / 256;
+        if (splits > 1024) splits = 1024;
+      } else if (want >= 2 && tiles <= kTicketCount) {
+        splits = want < 16 ? want : 16;
+        meet_in_kernel = true;
+      }
     }
     PoolBuf part;
     float* const C_final = C;
@@ -491,17 +548,27 @@ int32_t sgemm_impl(int transA, int transB, int64_t M, int64_t N, int64_t K, cons
       p.colsum = 1;
       p.aux_out = aux_out;
     }
+    int64_t chunk = K;
     if (splits > 1) {
-      int64_t chunk = ceil_div64(ceil_div64(K, splits), BK) * BK;
+      chunk = ceil_div64(ceil_div64(K, splits), BK) * BK;
       splits = ceil_div64(K, chunk);
-      int32_t rc = endia_hip_malloc(splits * M * N * 4, &part.p);
+    }
+    if (splits > 1) {
+      const int64_t part_floats = meet_in_kernel ? splits * tiles * (64 * F) * (64 * F) : splits * M * N;
+      int32_t rc = endia_hip_malloc(part_floats * 4, &part.p);
       if (rc) return rc;
       p.k_split = (int)chunk;
       p.sA = chunk * (transA ? lda : 1);
       p.sB = chunk * (transB ? 1 : ldb);
-      p.C = static_cast<float*>(part.p);
-      p.ldc = N;
-      p.sC = M * N;
+      if (meet_in_kernel) {
+        p.splits = (int)splits;
+        p.part = static_cast<float*>(part.p);
+        p.tickets = ctx().tickets;
+      } else {
+        p.C = static_cast<float*>(part.p);
+        p.ldc = N;
+        p.sC = M * N;
+      }
     }
     dim3 grid((unsigned)tiles, (unsigned)(splits > 1 ? splits : batch));
     const bool timed = g_timing.on && !ctx().capturing;
@@ -523,7 +590,7 @@ int32_t sgemm_impl(int transA, int transB, int64_t M, int64_t N, int64_t K, cons
       g_timing.used++;
       g_timing.flops += 2.0 * (double)M * (double)N * (double)K * (double)batch;
     }
-    if (splits > 1) {
+    if (splits > 1 && !meet_in_kernel) {
       ENDIA_LAUNCH_CHECK();
       int32_t rc = col_reduce(1, splits, M * N, p.C, C_final, 1.f);  // partials added in slice order
       if (rc || !colsum) return rc;

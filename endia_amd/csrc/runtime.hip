@@ -133,6 +133,8 @@ int32_t endia_hip_init(int32_t device) {
     }
     g_ev_made = true;
   }
+  ENDIA_HIP_CALL(hipMalloc(reinterpret_cast<void**>(&g_ctx.tickets), kTicketCount * sizeof(unsigned)));
+  ENDIA_HIP_CALL(hipMemset(g_ctx.tickets, 0, kTicketCount * sizeof(unsigned)));
   g_ctx.device = device;
   g_ctx.cu_count = prop.multiProcessorCount;
   g_ctx.clock_mhz = prop.clockRate / 1000;
@@ -157,6 +159,7 @@ int32_t endia_hip_shutdown(void) {
   if (g_ws) (void)hipFree(g_ws);
   g_ws = nullptr;
   g_ws_bytes = 0;
+  if (g_ctx.tickets) (void)hipFree(g_ctx.tickets);
   (void)hipStreamDestroy(g_ctx.stream);
   g_ctx = Context();
   return ENDIA_HIP_OK;

@@ -99,6 +99,41 @@ def test_sgemm_epilogues(dev, M, N, K, act):
                  C0 + R.matmul(A, B), what="accumulate")
 
 
+@pytest.mark.parametrize("ta,tb", [(0, 0), (0, 1), (1, 0)])
+@pytest.mark.parametrize("M,N,K", [(512, 512, 512), (256, 192, 1000), (64, 64, 4096), (128, 256, 260), (1024, 1024, 512),
+                                   (200, 136, 768)])
+def test_sgemm_reduction_split_inside_the_launch(dev, M, N, K, ta, tb):
+    """Products with few tiles per CU and K >= 256: K is cut into slices whose partial sums the last group of each
+    tile adds up. Every epilogue, accumulation and a padded C go through that path; results repeat bit for bit."""
+    rng = np.random.default_rng(M + 3 * N + 7 * K + ta + 2 * tb)
+    A = rng.standard_normal((K, M) if ta else (M, K)).astype(np.float32)
+    B = (rng.standard_normal((N, K) if tb else (K, N)) / np.sqrt(K)).astype(np.float32)
+    opA, opB = (A.T if ta else A), (B.T if tb else B)
+    ref = opA.astype(np.float64) @ opB.astype(np.float64)
+    first = run_sgemm(dev, A, B, ta, tb, M, N, K)
+    assert_close(first, R.matmul(opA, opB), what="vs oracle")
+    assert_close(first, ref, what="vs float64")
+    for _ in range(3):  # the arrival counters are back at zero after every launch, and the order of the sum is fixed
+        np.testing.assert_array_equal(run_sgemm(dev, A, B, ta, tb, M, N, K), first)
+    bias = rng.standard_normal(N).astype(np.float32)
+    aux = rng.standard_normal((M, N)).astype(np.float32)
+    C, Z = run_sgemm(dev, A, B, ta, tb, M, N, K, L.EPI_BIAS_ACT, L.OP_TANH, bias=bias, want_z=True)
+    assert_close(Z, ref + bias, what="stored pre-activation")
+    assert_close(C, np.tanh(ref + bias), what="bias + tanh")
+    assert_close(run_sgemm(dev, A, B, ta, tb, M, N, K, L.EPI_ACT_GRAD, L.OP_RELU, aux=aux), ref * (aux > 0), what="relu gradient")
+    C0 = rng.standard_normal((M, N)).astype(np.float32)
+    assert_close(run_sgemm(dev, A, B, ta, tb, M, N, K, L.EPI_NONE | L.GEMM_ACCUMULATE, C0=C0), C0 + ref, what="accumulate")
+    # C with a leading dimension larger than N: the columns past N keep their contents
+    ldc = N + 12
+    wide = rng.standard_normal((M, ldc)).astype(np.float32)
+    dA, dB, dC = dev.put(A), dev.put(B), dev.put(wide)
+    dev.call("endia_hip_sgemm", ta, tb, M, N, K, dA, A.shape[1], dB, B.shape[1], dC, ldc, 1, 0, 0, 0, L.EPI_BIAS, L.OP_IDENTITY,
+             dev.put(bias), None, None)
+    got = dev.get(dC, (M, ldc))
+    assert_close(got[:, :N], ref + bias, what="padded C")
+    np.testing.assert_array_equal(got[:, N:], wide[:, N:])
+
+
 def test_sgemm_edge_cases(dev):
     A = np.ones((4, 4), np.float32)
     # K = 0: the empty sum
