@@ -519,7 +519,7 @@ int32_t sgemm_impl(int transA, int transB, int64_t M, int64_t N, int64_t K, cons
     p.tiles_n = (int)ceil_div64(N, 64 * F);
     const int64_t tiles = (int64_t)p.tiles_m * p.tiles_n;
     ENDIA_CHECK_ARG(tiles < (1ll << 31), "sgemm: too many output tiles");
-    // A product with fewer than two tiles per CU is split along K so that more groups are in flight (a lone group
+    // A product with fewer than about three tiles per CU is split along K so that more groups are in flight (a lone group
     // per CU spends most of its time waiting for loads). Up to 16 slices of at least 128: the slices of a tile are
     // added, in slice order, by whichever of its groups finishes last, inside the one launch, with any epilogue.
     // A long reduction with very few tiles (dW of a narrow layer over a large batch) wants more slices than one
@@ -527,7 +527,7 @@ int32_t sgemm_impl(int transA, int transB, int64_t M, int64_t N, int64_t K, cons
     int64_t splits = 1;
     bool meet_in_kernel = false;
     if (batch == 1 && K >= 256) {
-      int64_t want = (4 * cus) / tiles;
+      int64_t want = (5 * cus + tiles / 2) / tiles;  // about five groups per CU in all (measured optimum 4-6)
       if (want > K / 128) want = K / 128;
       if (want > 16 && epi == ENDIA_EPI_NONE && !accumulate && ldc == N && K >= 2048) {
         splits = (4 * cus + tiles - 1) / tiles;
