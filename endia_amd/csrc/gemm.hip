@@ -22,6 +22,7 @@
 // operands use the same mapping.
 #include "common.h"
 #include "mfma_tile.h"
+#include "ticket.h"
 
 #include <stdlib.h>
 
@@ -224,29 +225,14 @@ __device__ __forceinline__ void gemm_tile(const GemmArgs& p, int block, int nblo
   // K split over gridDim.y groups per tile: every group leaves its accumulators in memory (register order, so the
   // stores and loads are contiguous per wave) and takes a ticket; the group that draws the last ticket adds the
   // slices in slice order, whichever group it is, so the sum does not depend on timing, and runs the epilogue.
-  // The partial sums travel as device-scope stores and loads (written through to, and read from, the level all
-  // XCDs share) rather than behind device-scope fences, which write back and invalidate a whole L2 per use: a
-  // wave's stores have completed when its counter of outstanding memory operations is zero, which the barrier
-  // ahead of the ticket waits for.
   if (p.splits) {
     constexpr int64_t SLICE = (int64_t)F * F * 16 * NTHREADS;
     float* mine = p.part + (bz * nblocks + block) * SLICE + tid;
 #pragma unroll
     for (int f = 0; f < F * F; ++f)
 #pragma unroll
-      for (int v = 0; v < 16; ++v)
-        __hip_atomic_store(mine + (f * 16 + v) * NTHREADS, acc[f / F][f % F][v], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    __builtin_amdgcn_s_waitcnt(0);
-    __syncthreads();
-    int* flag = reinterpret_cast<int*>(As);
-    if (tid == 0) {
-      const unsigned arrived = __hip_atomic_fetch_add(&p.tickets[block], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-      const bool last = arrived + 1u == (unsigned)p.splits;
-      if (last) __hip_atomic_store(&p.tickets[block], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);  // for the next launch
-      flag[0] = last;
-    }
-    __syncthreads();
-    if (!flag[0]) return;
+      for (int v = 0; v < 16; ++v) endia::store_shared(mine + (f * 16 + v) * NTHREADS, acc[f / F][f % F][v]);
+    if (!endia::arrive_last(&p.tickets[block], (unsigned)p.splits, reinterpret_cast<int*>(As))) return;
     zero_acc<F, F>(acc);
     for (int s = 0; s < p.splits; ++s) {
       const float* theirs = p.part + ((int64_t)s * nblocks + block) * SLICE + tid;
@@ -254,8 +240,7 @@ __device__ __forceinline__ void gemm_tile(const GemmArgs& p, int block, int nblo
       for (int f = 0; f < F * F; ++f) {
         float t[16];  // sixteen loads in flight, then sixteen additions
 #pragma unroll
-        for (int v = 0; v < 16; ++v)
-          t[v] = __hip_atomic_load(theirs + (f * 16 + v) * NTHREADS, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        for (int v = 0; v < 16; ++v) t[v] = endia::load_shared(theirs + (f * 16 + v) * NTHREADS);
 #pragma unroll
         for (int v = 0; v < 16; ++v) acc[f / F][f % F][v] += t[v];
       }
@@ -526,7 +511,7 @@ int32_t sgemm_impl(int transA, int transB, int64_t M, int64_t N, int64_t K, cons
     // group should add up: its partial products are added, also in slice order, by a second, chip-wide launch.
     int64_t splits = 1;
     bool meet_in_kernel = false;
-    if (batch == 1 && K >= 256) {
+    if (F == 1 && batch == 1 && K >= 256) {  // (the 128 x 128 tile is only chosen where there are enough tiles)
       int64_t want = (5 * cus + tiles / 2) / tiles;  // about five groups per CU in all (measured optimum 4-6)
       if (want > K / 128) want = K / 128;
       if (want > 16 && epi == ENDIA_EPI_NONE && !accumulate && ldc == N && K >= 2048) {
