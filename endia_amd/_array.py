@@ -88,6 +88,20 @@ def _prod(shape):
 class Array:
     """`Array(shape)` gives a zero-filled array like the reference's constructor (_array.mojo:198-214)."""
 
+    # autograd fields that most arrays never change live on the class; an instance stores what differs
+    _requires_grad = False
+    _grad = None
+    _args = ()
+    _vjp = None
+    _name = "arg"
+    _meta = None
+    _id = -1
+    _consumers = 0
+    _is_seed = False
+    _act_applied = False  # a gradient that already carries the producer's activation derivative
+    _offset = 0
+    is_complex_ = False
+
     def __init__(self, shape=None, requires_grad=False, is_complex=False, _buffer=None, _strides=None, _offset=0,
                  _zero=True):
         if isinstance(shape, np.ndarray):
@@ -97,29 +111,34 @@ class Array:
         shape = tuple(int(s) for s in (shape if shape is not None else (0,)))
         self._shape = shape
         self._strides = tuple(_strides) if _strides is not None else contiguous_strides(shape)
-        self._offset = int(_offset)
-        self.is_complex_ = bool(is_complex)
+        if _offset:
+            self._offset = int(_offset)
+        if is_complex:
+            self.is_complex_ = True
         if _buffer is None:
             n = _prod(shape) * (2 if is_complex else 1)
             _buffer = Buffer(4 * n)
             if _zero and n:
                 L.call("endia_hip_fill", _buffer.ptr, n, 0.0)
         self._buf = _buffer
-        self._requires_grad = bool(requires_grad)
-        self._grad = None
-        self._args = []
-        self._vjp = None
-        self._name = "arg"
-        self._meta = None
-        self._id = -1
-        self._consumers = 0
-        self._is_seed = False
-        self._act_applied = False  # a gradient that already carries the producer's activation derivative
+        if requires_grad:
+            self._requires_grad = True
 
     # ---- construction / host transfer ---------------------------------------------------------
     @staticmethod
     def empty(shape, is_complex=False):
-        return Array(shape, is_complex=is_complex, _zero=False)
+        """An array whose contents the caller is about to overwrite (no fill launch). `shape` holds ints."""
+        self = object.__new__(Array)
+        self._shape = shape = tuple(shape)
+        self._strides = contiguous_strides(shape)
+        n = 4
+        for s in shape:
+            n *= s
+        if is_complex:
+            self.is_complex_ = True
+            n *= 2
+        self._buf = Buffer(n)
+        return self
 
     @staticmethod
     def from_numpy(a, requires_grad=False):

@@ -160,9 +160,17 @@ def ensure_init(device=0):
     return lib()
 
 
+_entry = {}
+
+
 def call(name, *args):
     """Call an entry point on the initialised library and raise on a non-zero status."""
-    check(getattr(ensure_init(), name)(*args))
+    fn = _entry.get(name)
+    if fn is None:
+        fn = _entry[name] = getattr(ensure_init(), name)
+    code = fn(*args)
+    if code:
+        check(code)
 
 
 def i64_array(values):
