@@ -44,6 +44,7 @@ __global__ __launch_bounds__(TPB) void col_reduce_vec_kernel(const float* __rest
   float4 acc = make_float4(0.f, 0.f, 0.f, 0.f);
   if (c < C) {
     const float* base = x + b * R * C + c;
+#pragma unroll 8
     for (int64_t r = r0 + w; r < r1; r += 4) {
       float4 v = *reinterpret_cast<const float4*>(base + r * C);
       acc.x += v.x; acc.y += v.y; acc.z += v.z; acc.w += v.w;
@@ -83,8 +84,10 @@ __global__ __launch_bounds__(TPB) void col_reduce_final_kernel(const float* __re
   const int64_t c = (int64_t)blockIdx.x * 64 + lane;
   const int64_t b = blockIdx.y;
   float acc = 0.f;
-  if (c < C)
+  if (c < C) {
+#pragma unroll 8
     for (int64_t s = w; s < S; s += 4) acc += part[(b * S + s) * C + c];
+  }
   red[w][lane] = acc;
   __syncthreads();
   if (w == 0 && c < C) out[b * C + c] = ((red[0][lane] + red[1][lane]) + (red[2][lane] + red[3][lane])) * scale;
@@ -104,6 +107,7 @@ __global__ __launch_bounds__(TPB) void row_reduce_kernel(const float* __restrict
   if (vec) {  // chunk % 4 == 0, row base 16-byte aligned
     int64_t n4 = (c1 - c0) >> 2;
     const float4* p4 = reinterpret_cast<const float4*>(row + c0);
+#pragma unroll 4
     for (int64_t j = threadIdx.x; j < n4; j += TPB) {
       float4 v = p4[j];
       acc += (v.x + v.y) + (v.z + v.w);
@@ -227,7 +231,8 @@ int32_t col_reduce(int64_t batch, int64_t R, int64_t C, const float* x, float* o
   // enough row splits for ~4 groups per CU, at least 16 rows each
   int64_t want = (int64_t)ctx().cu_count * 4;
   int64_t S = want / (col_tiles * batch);
-  if (S > 64) S = 64;
+  const int64_t cap = col_tiles * batch * 64 < ctx().cu_count ? 256 : 64;  // a narrow input needs more row splits to fill the chip
+  if (S > cap) S = cap;
   if (S < 1) S = 1;
   int64_t max_s = ceil_div64(R, 16);
   if (S > max_s) S = max_s;
