@@ -93,6 +93,56 @@ __global__ __launch_bounds__(TPB) void pool_fwd_kernel(PoolP p, const float* __r
   }
 }
 
+// Windows that tile the input (stride = kernel, no padding, unit dilation; the usual 2 x 2 / 2), W a multiple of 4:
+// a lane reads its windows' rows 16 bytes at a time (four consecutive input elements are 4 / KW whole windows
+// along the row) and writes 4 / KW outputs. Same visiting order as pool_fwd_kernel (depth, row, column), so the
+// first maximum wins and the average adds up in the same order. KW = kernel width in {1, 2, 4}.
+template <bool MAX, int KW>
+__global__ __launch_bounds__(TPB) void pool_fwd_tiling_kernel(PoolP p, FastDiv d_w4, const float* __restrict__ x,
+                                                              float* __restrict__ y, int32_t* __restrict__ arg) {
+  constexpr int NWIN = 4 / KW;
+  const int64_t stride = (int64_t)gridDim.x * TPB;
+  const int64_t vol = (int64_t)p.D * p.H * p.W, ovol = (int64_t)p.Do * p.Ho * p.Wo;
+  const int W4 = p.W >> 2;
+  const int64_t total = (p.n_out / p.Wo) * W4;  // (plane, oz, oy) rows times groups of four input columns
+  for (int64_t j = (int64_t)blockIdx.x * TPB + threadIdx.x; j < total; j += stride) {
+    uint32_t plane;
+    int oz, oy, x4;
+    decode((uint32_t)j, d_w4, p.d_ho, p.d_do, W4, p.Ho, p.Do, plane, oz, oy, x4);
+    const float* src = x + plane * vol;
+    float best[NWIN], sum[NWIN];
+    int at[NWIN];
+#pragma unroll
+    for (int w = 0; w < NWIN; ++w) { best[w] = 0.f; sum[w] = 0.f; at[w] = -1; }
+    for (int a = 0; a < p.kd; ++a)
+      for (int b = 0; b < p.kh; ++b) {
+        const int row = ((oz * p.kd + a) * p.H + oy * p.kh + b) * p.W + x4 * 4;
+        const float4 v4 = *reinterpret_cast<const float4*>(src + row);
+        const float v[4] = {v4.x, v4.y, v4.z, v4.w};
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          const int w = e / KW;
+          if (MAX) {
+            if (at[w] < 0 || v[e] > best[w]) { best[w] = v[e]; at[w] = row + e; }
+          } else {
+            sum[w] += v[e];
+          }
+        }
+      }
+    const int64_t o = plane * ovol + ((int64_t)oz * p.Ho + oy) * p.Wo + x4 * NWIN;
+#pragma unroll
+    for (int w = 0; w < NWIN; ++w) {
+      if (x4 * NWIN + w >= p.Wo) break;
+      if (MAX) {
+        y[o + w] = best[w];
+        if (arg) arg[o + w] = at[w];
+      } else {
+        y[o + w] = sum[w] / (float)(p.kd * p.kh * KW);
+      }
+    }
+  }
+}
+
 // number of taps of output coordinate o that fall inside [0, extent); without padding every tap does
 __device__ __forceinline__ int taps_inside(int o, int k, int s, int pad, int dil, int extent) {
   if (pad == 0) return k;
@@ -319,8 +369,27 @@ int32_t endia_hip_pool_fwd(const endia_hip_pool_desc* desc, int32_t mode, const 
   if (p.n_out == 0) return ENDIA_HIP_OK;
   ENDIA_CHECK_ARG(x && y, "endia_hip_pool_fwd: null pointer");
   const int grid = stream_grid(p.n_out);
-  if (mode == ENDIA_POOL_MAX) hipLaunchKernelGGL((pool_fwd_kernel<true>), dim3(grid), dim3(TPB), 0, ctx().stream, p, x, y, argmax);
-  else hipLaunchKernelGGL((pool_fwd_kernel<false>), dim3(grid), dim3(TPB), 0, ctx().stream, p, x, y, (int32_t*)nullptr);
+  const bool tiling = p.dd == 1 && p.dh == 1 && p.dw == 1 && p.sd == p.kd && p.sh == p.kh && p.sw == p.kw && p.pd == 0 &&
+                      p.ph == 0 && p.pw == 0 && (p.kw == 1 || p.kw == 2 || p.kw == 4);
+  if (tiling && p.W % 4 == 0 && (reinterpret_cast<uintptr_t>(x) & 15) == 0) {
+    const FastDiv d_w4 = make_fastdiv(p.W / 4);
+    const int g4 = stream_grid(p.n_out / p.Wo * (p.W / 4));
+    hipStream_t s = ctx().stream;
+    int32_t* none = nullptr;
+#define ENDIA_POOL_FWD_TILING(KW)                                                                                         \
+  do {                                                                                                                    \
+    if (mode == ENDIA_POOL_MAX) hipLaunchKernelGGL((pool_fwd_tiling_kernel<true, KW>), dim3(g4), dim3(TPB), 0, s, p, d_w4, x, y, argmax); \
+    else hipLaunchKernelGGL((pool_fwd_tiling_kernel<false, KW>), dim3(g4), dim3(TPB), 0, s, p, d_w4, x, y, none);             \
+  } while (0)
+    if (p.kw == 1) ENDIA_POOL_FWD_TILING(1);
+    else if (p.kw == 2) ENDIA_POOL_FWD_TILING(2);
+    else ENDIA_POOL_FWD_TILING(4);
+#undef ENDIA_POOL_FWD_TILING
+  } else if (mode == ENDIA_POOL_MAX) {
+    hipLaunchKernelGGL((pool_fwd_kernel<true>), dim3(grid), dim3(TPB), 0, ctx().stream, p, x, y, argmax);
+  } else {
+    hipLaunchKernelGGL((pool_fwd_kernel<false>), dim3(grid), dim3(TPB), 0, ctx().stream, p, x, y, (int32_t*)nullptr);
+  }
   ENDIA_LAUNCH_CHECK();
   return ENDIA_HIP_OK;
 }
