@@ -735,7 +735,7 @@ def test_strided_scatter(dev, golden):
 @pytest.mark.gpu
 @pytest.mark.parametrize("xs,k", [((3, 5, 10, 12), (2, 2)), ((2, 3, 11, 8), (3, 4)), ((2, 4, 9, 16), (2, 1)),
                                    ((2, 2, 6, 7, 8), (2, 3, 2)), ((4, 3, 20), (4,)), ((1, 2, 5, 4), (7 - 2, 1))])
-def test_pool_bwd_tiling_windows(dev, xs, k):
+def test_pool_tiling_windows(dev, xs, k):
     """Windows that tile the input (stride = kernel, no padding) take a dedicated gradient kernel: the same
     numbers as the oracle (bit for bit: one select or one division per element) and as torch, including
     heights and depths that leave rows beyond the last whole window."""
@@ -747,6 +747,12 @@ def test_pool_bwd_tiling_windows(dev, xs, k):
     zeros, ones = (0,) * nsp, (1,) * nsp
     for mode, mname in ((L.POOL_MAX, "max"), (L.POOL_AVG, "avg")):
         y, _ = _pool_run(dev, mode, x, None, k, k, zeros, ones)
+        # the forward of such windows has its own kernel too (16-byte reads where the rows allow): the oracle's numbers,
+        # the maxima bit for bit, the averages up to the rounding of the sum
+        if mname == "max":
+            np.testing.assert_array_equal(y, R.pool(mname, x, k, k, zeros, ones))
+        else:
+            assert_close(y, R.pool(mname, x, k, k, zeros, ones), what="avg forward")
         gy = rng.standard_normal(y.shape).astype(np.float32)
         _, dx = _pool_run(dev, mode, x, gy, k, k, zeros, ones)
         np.testing.assert_array_equal(dx, R.pool_bwd(mname, x, gy, k, k, zeros, ones))
