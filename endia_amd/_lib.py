@@ -25,6 +25,7 @@ ACT_FROM_OUTPUT = 0x100
 GEMM_ACCUMULATE = 0x200
 GEMM_COLSUM_B = 0x400
 CGEMM_4M, CGEMM_3M = 0, 1
+REDUCE_MAX, REDUCE_MIN, REDUCE_MUL, REDUCE_ARGMAX, REDUCE_ARGMIN = range(5)
 
 ERR_INVALID, ERR_NOT_INIT, ERR_RUNTIME, ERR_NOMEM, ERR_UNSUPPORTED = -1, -2, -3, -4, -5
 
@@ -99,6 +100,7 @@ SIGNATURES = {
     "endia_hip_axpby": [c_int64, c_float, _fp, c_float, _fp, _fp],
     "endia_hip_complex_pack": [c_int64, _fp, _fp, _fp],
     "endia_hip_reduce_add": [c_int32, _i64p, c_uint32, _fp, _fp, c_float, c_int32],
+    "endia_hip_reduce": [c_int32, c_int32, _i64p, c_uint32, _fp, _fp],
     "endia_hip_mse_fwd_bwd": [c_int64, _fp, _fp, _fp, _fp],
     "endia_hip_conv2d_out_shape": [POINTER(Conv2dDesc), _i64p, _i64p],
     "endia_hip_conv2d_fwd": [POINTER(Conv2dDesc), _fp, _fp, _fp, _fp, c_int32],

@@ -162,6 +162,74 @@ __global__ __launch_bounds__(TPB) void generic_reduce_kernel(RedDesc d, const fl
   if (threadIdx.x == 0) out[o] = s * scale;
 }
 
+// ---- max / min / product and the positions of the extrema: one work-group per output element ----
+// Each thread walks its share of the reduced elements in ascending order, so "first" means the same in every
+// thread; threads are then combined by value, ties going to the smaller position.
+struct Extreme {
+  float v;
+  int64_t at;
+};
+
+template <int OP>
+__device__ __forceinline__ bool better(float v, float best) {
+  return (OP == ENDIA_REDUCE_MAX || OP == ENDIA_REDUCE_ARGMAX) ? v > best : v < best;
+}
+
+template <int OP>
+__device__ __forceinline__ Extreme pick(Extreme a, Extreme b) {
+  if (better<OP>(b.v, a.v)) return b;
+  if (better<OP>(a.v, b.v)) return a;
+  if (a.at < 0) return b;  // neither holds a value yet, or equal values: the smaller position
+  if (b.at < 0) return a;
+  return a.at <= b.at ? a : b;
+}
+
+template <int OP>
+__global__ __launch_bounds__(TPB) void reduce_op_kernel(RedDesc d, const float* __restrict__ x, float* __restrict__ out,
+                                                        int64_t nred) {
+  constexpr bool ARG = OP == ENDIA_REDUCE_ARGMAX || OP == ENDIA_REDUCE_ARGMIN;
+  constexpr bool MUL = OP == ENDIA_REDUCE_MUL;
+  constexpr bool UP = OP == ENDIA_REDUCE_MAX || OP == ENDIA_REDUCE_ARGMAX;
+  __shared__ float red_v[4];
+  __shared__ long long red_at[4];
+  int64_t o = blockIdx.x, rem = o, base = 0;
+  for (int k = d.nk - 1; k >= 0; --k) {
+    int64_t q = rem / d.kshape[k];
+    base += (rem - q * d.kshape[k]) * d.kstride[k];
+    rem = q;
+  }
+  Extreme e = {MUL ? 1.f : (UP ? -INFINITY : INFINITY), -1};
+  for (int64_t j = threadIdx.x; j < nred; j += TPB) {
+    int64_t r = j, off = base;
+    for (int k = d.nr - 1; k >= 0; --k) {
+      int64_t q = r / d.rshape[k];
+      off += (r - q * d.rshape[k]) * d.rstride[k];
+      r = q;
+    }
+    const float v = x[off];
+    if (MUL) e.v *= v;
+    else if (better<OP>(v, e.v)) { e.v = v; e.at = j; }
+  }
+#pragma unroll
+  for (int s = 32; s > 0; s >>= 1) {
+    Extreme other = {__shfl_down(e.v, s, 64), (int64_t)__shfl_down((long long)e.at, s, 64)};
+    if (MUL) e.v *= other.v;
+    else e = pick<OP>(e, other);
+  }
+  const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
+  if (lane == 0) { red_v[w] = e.v; red_at[w] = e.at; }
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    Extreme t = {red_v[0], (int64_t)red_at[0]};
+    for (int i = 1; i < 4; ++i) {
+      Extreme other = {red_v[i], (int64_t)red_at[i]};
+      if (MUL) t.v *= other.v;
+      else t = pick<OP>(t, other);
+    }
+    out[o] = ARG ? (float)t.at : t.v;
+  }
+}
+
 // ---- MSE ------------------------------------------------------------------------------------
 // One pass: dpred = 2 (p - t) / n and per-group partial sums of (p - t)^2.
 __global__ __launch_bounds__(TPB) void mse_kernel(const float* __restrict__ p, const float* __restrict__ t,
@@ -343,6 +411,55 @@ int32_t endia_hip_reduce_add(int32_t ndim, const int64_t* shape, uint32_t reduce
   }
   ENDIA_CHECK_ARG(nout <= 2147483647ll, "endia_hip_reduce_add: too many outputs for the general path");
   hipLaunchKernelGGL(generic_reduce_kernel, dim3((unsigned)nout), dim3(TPB), 0, ctx().stream, d, x, out, nred, scale);
+  ENDIA_LAUNCH_CHECK();
+  return ENDIA_HIP_OK;
+}
+
+int32_t endia_hip_reduce(int32_t op, int32_t ndim, const int64_t* shape, uint32_t reduce_mask, const float* x, float* out) {
+  ENDIA_REQUIRE_INIT();
+  ENDIA_CHECK_ARG(op >= ENDIA_REDUCE_MAX && op <= ENDIA_REDUCE_ARGMIN, "endia_hip_reduce: unknown op %d", op);
+  ENDIA_CHECK_ARG(ndim >= 0 && ndim <= 8, "endia_hip_reduce: ndim %d out of [0,8]", ndim);
+  ENDIA_CHECK_ARG(ndim == 0 || shape, "endia_hip_reduce: null shape");
+  ENDIA_CHECK_ARG(ndim == 8 ? true : (reduce_mask >> ndim) == 0, "endia_hip_reduce: mask 0x%x names an axis >= ndim", reduce_mask);
+  const bool arg = op == ENDIA_REDUCE_ARGMAX || op == ENDIA_REDUCE_ARGMIN;
+  ENDIA_CHECK_ARG(!arg || __builtin_popcount(reduce_mask) == 1, "endia_hip_reduce: argmax / argmin reduce exactly one axis");
+  // neighbouring axes with the same status collapse into groups, as in endia_hip_reduce_add
+  int64_t gshape[8];
+  int gred[8];
+  int ng = 0;
+  int64_t total = 1, nout = 1;
+  for (int i = 0; i < ndim; ++i) {
+    ENDIA_CHECK_ARG(shape[i] >= 0, "endia_hip_reduce: negative extent");
+    total *= shape[i];
+    const int red = (reduce_mask >> i) & 1;
+    if (!red) nout *= shape[i];
+    if (shape[i] == 1) continue;
+    if (ng && gred[ng - 1] == red) gshape[ng - 1] *= shape[i];
+    else { gshape[ng] = shape[i]; gred[ng] = red; ++ng; }
+  }
+  if (nout == 0) return ENDIA_HIP_OK;
+  ENDIA_CHECK_ARG(out != nullptr, "endia_hip_reduce: out is null");
+  const float start = op == ENDIA_REDUCE_MUL ? 1.f : (arg ? -1.f : (op == ENDIA_REDUCE_MAX ? -INFINITY : INFINITY));
+  if (total == 0) return endia_hip_fill(out, nout, start);
+  ENDIA_CHECK_ARG(x != nullptr, "endia_hip_reduce: x is null");
+  ENDIA_CHECK_ARG(nout <= 2147483647ll, "endia_hip_reduce: too many outputs");
+  RedDesc d;
+  d.nk = d.nr = 0;
+  int64_t st = 1, nred = 1, strides[8];
+  for (int g = ng - 1; g >= 0; --g) { strides[g] = st; st *= gshape[g]; }
+  for (int g = 0; g < ng; ++g) {
+    if (gred[g]) { d.rshape[d.nr] = gshape[g]; d.rstride[d.nr] = strides[g]; ++d.nr; nred *= gshape[g]; }
+    else { d.kshape[d.nk] = gshape[g]; d.kstride[d.nk] = strides[g]; ++d.nk; }
+  }
+  const dim3 grid((unsigned)nout), block(TPB);
+  hipStream_t s = ctx().stream;
+  switch (op) {
+    case ENDIA_REDUCE_MAX: hipLaunchKernelGGL((reduce_op_kernel<ENDIA_REDUCE_MAX>), grid, block, 0, s, d, x, out, nred); break;
+    case ENDIA_REDUCE_MIN: hipLaunchKernelGGL((reduce_op_kernel<ENDIA_REDUCE_MIN>), grid, block, 0, s, d, x, out, nred); break;
+    case ENDIA_REDUCE_MUL: hipLaunchKernelGGL((reduce_op_kernel<ENDIA_REDUCE_MUL>), grid, block, 0, s, d, x, out, nred); break;
+    case ENDIA_REDUCE_ARGMAX: hipLaunchKernelGGL((reduce_op_kernel<ENDIA_REDUCE_ARGMAX>), grid, block, 0, s, d, x, out, nred); break;
+    default: hipLaunchKernelGGL((reduce_op_kernel<ENDIA_REDUCE_ARGMIN>), grid, block, 0, s, d, x, out, nred); break;
+  }
   ENDIA_LAUNCH_CHECK();
   return ENDIA_HIP_OK;
 }

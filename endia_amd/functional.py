@@ -747,6 +747,79 @@ def mean(x, axes=None, keepdims=False):
     return out if keepdims else squeeze(out)
 
 
+def _reduce_other(x, axis, keepdims, op, name, cite):
+    """Shared body of reduce_max / reduce_min / reduce_mul / reduce_argmax / reduce_argmin: the reduced axes stay as
+    size 1 unless keepdims is False, in which case every size-1 axis is squeezed away, as the reference does."""
+    if x.is_complex_:
+        raise ValueError("Warning in %s:  The %s operation does not support complex numbers." % (name, name))
+    axes = sorted(set(_norm_axes([axis] if isinstance(axis, int) else list(axis), x.ndim())))
+    if x.ndim() > 8:
+        raise ValueError("more than 8 dimensions")
+    if op in (L.REDUCE_ARGMAX, L.REDUCE_ARGMIN) and len(axes) != 1:
+        raise ValueError("%s: exactly one axis (the reference's result for several axes is not a position)" % name)
+    src = contiguous(x)
+    out = Array.empty([1 if i in axes else s for i, s in enumerate(x._shape)])
+    mask = 0
+    for a in axes:
+        mask |= 1 << a
+    if out.size():
+        L.call("endia_hip_reduce", op, x.ndim(), L.i64_array(x._shape), mask, src.data_ptr(), out.data_ptr())
+
+    def vjp(primals, grad, out_):
+        raise NotImplementedError("%s has no backward rule in the reference (%s); none is provided here" % (name, cite))
+
+    out = _register(out, [x], name, vjp)
+    return out if keepdims else squeeze(out)
+
+
+def reduce_max(x, axis, keepdims=False):
+    """Maximum over `axis` (an int or a list), reduce_max_op.mojo:66-190, 228-257."""
+    return _reduce_other(x, axis, keepdims, L.REDUCE_MAX, "reduce_max", "reduce_max_op.mojo:196-198 is the default rule")
+
+
+def reduce_min(x, axis, keepdims=False):
+    """Minimum over `axis`, reduce_min_op.mojo:66-190, 228-257."""
+    return _reduce_other(x, axis, keepdims, L.REDUCE_MIN, "reduce_min", "reduce_min_op.mojo:196-198 is the default rule")
+
+
+def reduce_argmax(x, axis, keepdims=False):
+    """Position of the first maximum along one axis, as a float array (reduce_argmax_op.mojo:66-163, 218-247)."""
+    return _reduce_other(x, axis, keepdims, L.REDUCE_ARGMAX, "reduce_argmax", "reduce_argmax_op.mojo:169-171 is the default rule")
+
+
+def reduce_argmin(x, axis, keepdims=False):
+    """Position of the first minimum along one axis, as a float array (reduce_argmin_op.mojo:66-163, 218-247)."""
+    return _reduce_other(x, axis, keepdims, L.REDUCE_ARGMIN, "reduce_argmin", "reduce_argmin_op.mojo:169-171 is the default rule")
+
+
+def reduce_mul(x, axis, keepdims=False):
+    """Product over `axis` (reduce_mul_op.mojo:65-210, 288-321). The reference's backward rule for it is a placeholder
+    that hands the cotangent through unchanged (reduce_mul_op.mojo:238-255, "TODO" in its test file)."""
+    return _reduce_other(x, axis, keepdims, L.REDUCE_MUL, "reduce_mul", "reduce_mul_op.mojo:238-255 is a placeholder")
+
+
+def prod(x):
+    """Product of all elements, shape [1] (prod_op.mojo:35-62)."""
+    return squeeze(reduce_mul(x, list(range(x.ndim())), keepdims=True))
+
+
+def variance(x, axes=(0,), unbiased=True, keepdims=False):
+    """variance_op.mojo:35-79, op for op: the mean from reduce_add, the squared differences, their sum divided by
+    count - 1 (or count). Differentiable through those ops."""
+    axes = list(axes)
+    res = reduce_add(x, axes)
+    count = float(x.size() // max(res.size(), 1))
+    divisor = count - 1.0 if unbiased else count
+    diff = x - res / count
+    out = reduce_add(diff * diff, axes) / divisor
+    return out if keepdims else squeeze(out)
+
+
+def std(x, axes=(0,), unbiased=True, keepdims=False):
+    """std_op.mojo:35-65: sqrt(variance)."""
+    return sqrt(variance(x, axes, unbiased, keepdims))
+
+
 # --------------------------------------------------------------------------------------------------
 # matmul (endia/functional/binary_ops/matmul_op.mojo)
 # --------------------------------------------------------------------------------------------------

@@ -267,6 +267,24 @@ ENDIA_API int32_t endia_hip_complex_pack(int64_t n, const float* re, const float
 ENDIA_API int32_t endia_hip_reduce_add(int32_t ndim, const int64_t* shape, uint32_t reduce_mask, const float* x,
                              float* out, float scale, int32_t is_complex);
 
+/* ---- the other reductions: ReduceMax / ReduceMin / ReduceMul .__call__ (reduce_ops/reduce_max_op.mojo:66-190,
+ *      reduce_min_op.mojo:66-190, reduce_mul_op.mojo:65-210) and ReduceArgMax / ReduceArgMin .__call__
+ *      (reduce_argmax_op.mojo:66-163, reduce_argmin_op.mojo:66-163). Same layout contract as
+ *      endia_hip_reduce_add (kept axes of size 1, ndim <= 8, real arrays). The arg variants reduce exactly one
+ *      axis and write the position along it as a float (the reference's arrays hold fp32 only): the first
+ *      position whose value is strictly greater (smaller) than everything before it, -1 when no value exceeds
+ *      the starting value -inf (+inf), as the reference's loop leaves it. An empty reduction yields the
+ *      starting value: -inf, +inf, 1, -1. */
+typedef enum {
+  ENDIA_REDUCE_MAX = 0,
+  ENDIA_REDUCE_MIN = 1,
+  ENDIA_REDUCE_MUL = 2,
+  ENDIA_REDUCE_ARGMAX = 3,
+  ENDIA_REDUCE_ARGMIN = 4
+} endia_hip_reduce_op;
+ENDIA_API int32_t endia_hip_reduce(int32_t op, int32_t ndim, const int64_t* shape, uint32_t reduce_mask, const float* x,
+                         float* out);
+
 /* ---- loss: mse (loss_ops/mse_op.mojo:17-20) and its gradient 2(p-t)/n as produced by the
  *      sub/mul/sum/div VJP chain. loss is one device float; dpred may be null (forward only);
  *      loss may be null (gradient only). */

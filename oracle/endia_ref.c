@@ -455,6 +455,48 @@ void ref_reduce_add(int32_t ndim, const int64_t* shape, uint32_t mask, const flo
   }
 }
 
+/* ---- ReduceMax / ReduceMin / ReduceMul .__call__ (reduce_ops/reduce_max_op.mojo:66-190, reduce_min_op.mojo:66-190,
+ * reduce_mul_op.mojo:65-210) and ReduceArgMax / ReduceArgMin .__call__ (reduce_argmax_op.mojo:66-163,
+ * reduce_argmin_op.mojo:66-163). op: 0 max, 1 min, 2 product, 3 argmax, 4 argmin. The output starts at -inf / +inf /
+ * 1 (the arg variants at -1 beside a running extreme of -inf / +inf) and every input element is folded into its
+ * target in row-major input order; an arg variant records the element's position along the ONE reduced axis when
+ * the element is strictly beyond the running extreme (reduce_argmax_op.mojo:136-142; for one reduced axis the
+ * recorded quotient arg_max_idx // denom is that position). */
+void ref_reduce_op(int32_t op, int32_t ndim, const int64_t* shape, uint32_t mask, const float* x, float* out) {
+  int64_t n = 1, nout = 1, tstride[8], red_axis = -1;
+  for (int i = 0; i < ndim; ++i) n *= shape[i];
+  for (int i = ndim - 1; i >= 0; --i) {
+    int red = (mask >> i) & 1;
+    tstride[i] = red ? 0 : nout;
+    if (!red) nout *= shape[i];
+    else red_axis = i;
+  }
+  const int arg = op >= 3, up = (op == 0 || op == 3);
+  float* run = arg ? fresh(nout) : out;  /* the running extreme (tmp_max in the reference's arg variants) */
+  for (int64_t i = 0; i < nout; ++i) {
+    run[i] = op == 2 ? 1.f : (up ? -INFINITY : INFINITY);
+    if (arg) out[i] = -1.f;
+  }
+  for (int64_t j = 0; j < n; ++j) {
+    int64_t r = j, t = 0, pos = 0;
+    for (int k = ndim - 1; k >= 0; --k) {
+      int64_t idx = r % shape[k];
+      t += idx * tstride[k];
+      if (k == red_axis) pos = idx;
+      r /= shape[k];
+    }
+    const float v = x[j];
+    if (op == 2) {
+      run[t] = run[t] * v;
+    } else {
+      const float next = up ? (run[t] > v ? run[t] : v) : (run[t] < v ? run[t] : v);
+      if (arg && (up ? next > run[t] : next < run[t])) out[t] = (float)pos;
+      run[t] = next;
+    }
+  }
+  if (arg) free(run);
+}
+
 /* ---- mse: loss_ops/mse_op.mojo:17-20 = sum((p - t) * (p - t)) / n, and the gradient its VJP chain
  * yields: Div.vjp g/n (div_op.mojo:108-110), ReduceAdd.vjp expand (reduce_add_op.mojo:234), Mul.vjp
  * returns diff*g for both operands, which land on the same tensor and are added

@@ -173,6 +173,48 @@ def reduce_add(x, axes):
     return out
 
 
+_REDUCE_OPS = {"max": 0, "min": 1, "mul": 2, "argmax": 3, "argmin": 4}
+
+
+def reduce_op(kind, x, axes):
+    """ReduceMax / ReduceMin / ReduceMul / ReduceArgMax / ReduceArgMin over `axes`, kept as size 1; the arg variants
+    take one axis and return positions as floats."""
+    x = _f32(x)
+    axes = [ax % x.ndim for ax in ([axes] if isinstance(axes, int) else axes)]
+    if kind.startswith("arg") and len(set(axes)) != 1:
+        raise ValueError("argmax / argmin reduce one axis")
+    mask = 0
+    for ax in axes:
+        mask |= 1 << ax
+    out = np.zeros(tuple(1 if i in axes else s for i, s in enumerate(x.shape)), dtype=np.float32)
+    lib().ref_reduce_op(c_int32(_REDUCE_OPS[kind]), c_int32(x.ndim), _i64(x.shape), c_uint32(mask), _ptr(x), _ptr(out))
+    return out
+
+
+def variance(x, axes=(0,), unbiased=True, keepdims=False):
+    """variance_op.mojo:35-79 with the ops above: reduce_add, the count as a float, sub, mul, reduce_add, div."""
+    x = _f32(x)
+    axes = list(axes)
+    res = reduce_add(x, axes)
+    count = np.float32(x.size // max(res.size, 1))
+    divisor = count - np.float32(1) if unbiased else count
+    mean_res = binary("div", res, np.full((1,), count, np.float32))
+    diff = binary("sub", x, mean_res)
+    var = binary("div", reduce_add(binary("mul", diff, diff), axes), np.full((1,), divisor, np.float32))
+    return var if keepdims else _squeeze(var)
+
+
+def std(x, axes=(0,), unbiased=True, keepdims=False):
+    """std_op.mojo:35-65."""
+    return unary("sqrt", variance(x, axes, unbiased, keepdims))
+
+
+def _squeeze(a):
+    """Squeeze: every size-1 axis goes, one stays if all are (squeeze_op.mojo:31-60)."""
+    shape = [s for s in a.shape if s != 1] or [1]
+    return a.reshape(shape)
+
+
 def mse(pred, target):
     """Returns (loss, dpred) as the reference's op chain produces them."""
     pred, target = _f32(pred), _f32(target)

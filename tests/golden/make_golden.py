@@ -371,3 +371,22 @@ gc = f32(*y.shape)
 d.update({"cat_1": c1, "cat_2": c2, "cat_3": c3, "cat_y": y.detach().numpy(), "cat_g": gc, "cat_d1": t1.grad.numpy(),
           "cat_d2": t2.grad.numpy(), "cat_d3": t3.grad.numpy()})
 save("views", **d)
+
+# ---- the other reductions (test_reduce_max_op.mojo:18-34, test_reduce_min_op.mojo:18-34, test_reduce_argmax_op.mojo:18-33,
+# test_reduce_argmin_op.mojo:18-33, test_reduce_mul_op.mojo:18-33, test_std_op.mojo:18-58, test_variance_op.mojo:18-59) ------
+x = f32(2, 30, 40)
+t = t64(x)
+d = {"x": x, "max1": torch.max(t, dim=1)[0].numpy(), "min1": torch.min(t, dim=1)[0].numpy(),
+     "argmax1": torch.argmax(t, dim=1).numpy().astype(np.float64), "argmin1": torch.argmin(t, dim=1).numpy().astype(np.float64),
+     "max02": torch.amax(t, dim=(0, 2)).numpy(), "min12": torch.amin(t, dim=(1, 2)).numpy(),
+     "argmax2": torch.argmax(t, dim=2).numpy().astype(np.float64), "prod1": torch.prod(t, 1).numpy(),
+     "prod_all": torch.prod(t64(x[0, :8, :5])).numpy().reshape(1),
+     "std1": torch.std(t, [1]).numpy(), "var1": torch.var(t, [1]).numpy(), "var02_biased": torch.var(t, [0, 2], unbiased=False).numpy(),
+     "std1_keep": torch.std(t, [1], keepdim=True).numpy()}
+tg = t64(x, True)
+torch.sum(torch.std(tg, [1])).backward()
+d["dstd1"] = tg.grad.numpy()
+tg = t64(x, True)
+torch.sum(torch.var(tg, [1])).backward()
+d["dvar1"] = tg.grad.numpy()
+save("reduce_more", **d)

@@ -204,6 +204,38 @@ def test_reduce_mean_expand_grad(nd, golden):  # test_reduce_add_op / test_mean_
     assert_close(b.grad().to_numpy(), g["dexpand"], what="d expand")
 
 
+def test_other_reductions_and_their_gradients(nd, golden):
+    """reduce_max / reduce_min / reduce_argmax / reduce_argmin / reduce_mul / prod / variance / std as the reference's
+    tests call them (test_reduce_max_op.mojo:18-34 and siblings, test_std_op.mojo:18-58, test_variance_op.mojo:18-59)."""
+    g = golden("reduce_more")
+    x = nd.array(g["x"])
+    for name, fn, axis, key in (("max", nd.reduce_max, [1], "max1"), ("min", nd.reduce_min, [1], "min1"),
+                                ("argmax", nd.reduce_argmax, [1], "argmax1"), ("argmin", nd.reduce_argmin, [1], "argmin1"),
+                                ("argmax last axis", nd.reduce_argmax, 2, "argmax2"), ("max over two axes", nd.reduce_max, [0, 2], "max02")):
+        out = fn(x, axis)
+        assert out.shape() == list(g[key].shape), name
+        np.testing.assert_array_equal(out.to_numpy(), g[key], err_msg=name)
+    assert nd.reduce_max(x, [1], keepdims=True).shape() == [2, 1, 40]
+    assert_close(nd.reduce_mul(x, [1]).to_numpy(), g["prod1"], what="reduce_mul")
+    assert_close(nd.prod(nd.array(g["x"][0, :8, :5].copy())).to_numpy(), g["prod_all"], what="prod")
+    assert_close(nd.variance(x, [1]).to_numpy(), g["var1"], what="variance")
+    assert_close(nd.variance(x, [0, 2], unbiased=False).to_numpy(), g["var02_biased"], what="biased variance")
+    assert_close(nd.std(x, [1]).to_numpy(), g["std1"], what="std")
+    assert_close(nd.std(x, [1], keepdims=True).to_numpy(), g["std1_keep"], what="std, kept axis")
+    for fn, key in ((nd.std, "dstd1"), (nd.variance, "dvar1")):
+        xg = nd.array(g["x"], requires_grad=True)
+        nd.sum(fn(xg, [1])).backward()
+        assert_close(xg.grad().to_numpy(), g[key], what=key)
+    # no backward rule exists for the extrema or the product (the reference's are the default / a placeholder): refused loudly
+    xg = nd.array(g["x"], requires_grad=True)
+    with pytest.raises(NotImplementedError):
+        nd.sum(nd.reduce_max(xg, [1])).backward()
+    with pytest.raises(ValueError):
+        nd.reduce_argmax(x, [0, 1])
+    with pytest.raises(ValueError):
+        nd.reduce_max(nd.complex(x, x), [1])
+
+
 def test_permute_reshape_views(nd):
     rng = np.random.default_rng(0)
     a = rng.standard_normal((2, 3, 4)).astype(np.float32)

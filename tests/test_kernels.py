@@ -325,6 +325,55 @@ def test_reduce_golden_scale_complex_empty(dev, golden):
     np.testing.assert_array_equal(dev.get(do, (8,)), np.zeros(8, np.float32))  # empty sum
 
 
+_REDUCE_KINDS = {"max": L.REDUCE_MAX, "min": L.REDUCE_MIN, "mul": L.REDUCE_MUL, "argmax": L.REDUCE_ARGMAX, "argmin": L.REDUCE_ARGMIN}
+
+
+def _reduce_run(dev, kind, x, axes):
+    mask = 0
+    for a in axes:
+        mask |= 1 << a
+    oshape = tuple(1 if i in axes else s for i, s in enumerate(x.shape))
+    dx_, do = dev.put(x), dev.alloc(4 * max(int(np.prod(oshape)), 1))
+    dev.call("endia_hip_reduce", _REDUCE_KINDS[kind], x.ndim, L.i64_array(x.shape), mask, dx_, do)
+    return dev.get(do, oshape)
+
+
+def test_other_reductions(dev, golden):
+    """endia_hip_reduce against the golden fixture (torch float64) and the oracle: extrema and their positions bit for
+    bit, products within the tolerance (the order of the multiplications differs)."""
+    g = golden("reduce_more")
+    x = g["x"]
+    np.testing.assert_array_equal(_reduce_run(dev, "max", x, [1]).reshape(2, 40), g["max1"])
+    np.testing.assert_array_equal(_reduce_run(dev, "min", x, [1]).reshape(2, 40), g["min1"])
+    np.testing.assert_array_equal(_reduce_run(dev, "argmax", x, [1]).reshape(2, 40), g["argmax1"])
+    np.testing.assert_array_equal(_reduce_run(dev, "argmin", x, [1]).reshape(2, 40), g["argmin1"])
+    np.testing.assert_array_equal(_reduce_run(dev, "argmax", x, [2]).reshape(2, 30), g["argmax2"])
+    np.testing.assert_array_equal(_reduce_run(dev, "max", x, [0, 2]).reshape(30), g["max02"])
+    np.testing.assert_array_equal(_reduce_run(dev, "min", x, [1, 2]).reshape(2), g["min12"])
+    assert_close(_reduce_run(dev, "mul", x, [1]).reshape(2, 40), g["prod1"], what="product over axis 1")
+    assert_close(_reduce_run(dev, "mul", x[0, :8, :5].copy(), [0, 1]).reshape(1), g["prod_all"], what="product of everything")
+    rng = np.random.default_rng(5)
+    for shape, axes in (((7, 1, 33), [2]), ((300, 5), [0]), ((4, 3, 2, 5), [1, 3]), ((1000,), [0]), ((3, 1), [1]), ((2, 600, 3), [1])):
+        v = rng.standard_normal(shape).astype(np.float32)
+        v.reshape(-1)[::7] = v.reshape(-1)[0]  # repeated values: ties must go to the first position
+        for kind in ("max", "min", "mul") + (("argmax", "argmin") if len(axes) == 1 else ()):
+            got, want = _reduce_run(dev, kind, v, axes), R.reduce_op(kind, v, axes)
+            if kind == "mul":
+                assert_close(got, want, what="%s %s %s" % (kind, shape, axes))
+            else:
+                np.testing.assert_array_equal(got, want, err_msg="%s %s %s" % (kind, shape, axes))
+    # starting values: nothing exceeds -inf, so no position is recorded; an empty reduction yields the starting value
+    np.testing.assert_array_equal(_reduce_run(dev, "argmax", np.full((2, 3), -np.inf, np.float32), [1]).reshape(-1), [-1, -1])
+    do = dev.alloc(4 * 8)
+    for kind, start in (("max", -np.inf), ("min", np.inf), ("mul", 1.0), ("argmin", -1.0)):
+        dev.call("endia_hip_reduce", _REDUCE_KINDS[kind], 2, L.i64_array([0, 8]), 0b01, None, do)
+        np.testing.assert_array_equal(dev.get(do, (8,)), np.full(8, start, np.float32))
+    lib = L.lib()
+    dx_ = dev.put(x)
+    assert lib.endia_hip_reduce(L.REDUCE_ARGMAX, 3, L.i64_array([2, 30, 40]), 0b011, dx_, do) == L.ERR_INVALID
+    assert lib.endia_hip_reduce(9, 3, L.i64_array([2, 30, 40]), 0b010, dx_, do) == L.ERR_INVALID
+
+
 @pytest.mark.parametrize("n", [1, 128, 16 * 8, 100003])
 def test_mse(dev, golden, n):
     g = golden("mse")

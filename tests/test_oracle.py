@@ -159,6 +159,41 @@ def test_reduce_golden(golden):
     assert_close(R.reduce_add(v, [0]), [v.astype(np.float64).sum()], what="rank-1 sum")
 
 
+def test_other_reductions_golden_and_brute_force(golden):
+    """max / min / argmax / argmin / product / variance / std of the oracle against torch float64 (the reference's own
+    check: test_reduce_max_op.mojo:18-34 and its siblings, test_std_op.mojo:18-58, test_variance_op.mojo:18-59), against
+    plain loops on a small array, and on the cases the loops' starting values decide."""
+    g = golden("reduce_more")
+    x = g["x"]
+    np.testing.assert_array_equal(R.reduce_op("max", x, [1]).reshape(2, 40), g["max1"])
+    np.testing.assert_array_equal(R.reduce_op("min", x, [1]).reshape(2, 40), g["min1"])
+    np.testing.assert_array_equal(R.reduce_op("argmax", x, [1]).reshape(2, 40), g["argmax1"])
+    np.testing.assert_array_equal(R.reduce_op("argmin", x, [1]).reshape(2, 40), g["argmin1"])
+    np.testing.assert_array_equal(R.reduce_op("argmax", x, [2]).reshape(2, 30), g["argmax2"])
+    np.testing.assert_array_equal(R.reduce_op("max", x, [0, 2]).reshape(30), g["max02"])
+    np.testing.assert_array_equal(R.reduce_op("min", x, [1, 2]).reshape(2), g["min12"])
+    assert_close(R.reduce_op("mul", x, [1]).reshape(2, 40), g["prod1"], what="product over axis 1")
+    assert_close(R.reduce_op("mul", x[0, :8, :5], [0, 1]).reshape(1), g["prod_all"], what="product of everything")
+    assert_close(R.variance(x, [1]), g["var1"], what="variance")
+    assert_close(R.std(x, [1]), g["std1"], what="std")
+    assert_close(R.std(x, [1], keepdims=True), g["std1_keep"], what="std, kept axis")
+    assert_close(R.variance(x, [0, 2], unbiased=False), g["var02_biased"], what="biased variance over two axes")
+    # plain loops
+    small = x[1, :4, :6]
+    for j in range(6):
+        col = [float(v) for v in small[:, j]]
+        assert R.reduce_op("max", small, [0])[0, j] == max(col)
+        assert R.reduce_op("argmin", small, [0])[0, j] == col.index(min(col))
+        p = np.float32(1)
+        for v in small[:, j]:
+            p = np.float32(p * v)
+        assert R.reduce_op("mul", small, [0])[0, j] == p
+    # ties go to the first position; an axis holding only the starting value leaves -1; a size-1 axis gives 0
+    np.testing.assert_array_equal(R.reduce_op("argmax", np.array([[1, 3, 3], [2, 2, 1]], np.float32), [1]).reshape(-1), [1, 0])
+    np.testing.assert_array_equal(R.reduce_op("argmax", np.full((2, 3), -np.inf, np.float32), [1]).reshape(-1), [-1, -1])
+    np.testing.assert_array_equal(R.reduce_op("argmin", np.ones((3, 1), np.float32), [1]).reshape(-1), [0, 0, 0])
+
+
 def test_mse_golden(golden):
     g = golden("mse")
     loss, dpred = R.mse(g["pred"], g["target"])
