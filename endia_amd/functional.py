@@ -794,7 +794,7 @@ def reduce_argmin(x, axis, keepdims=False):
 
 def reduce_mul(x, axis, keepdims=False):
     """Product over `axis` (reduce_mul_op.mojo:65-210, 288-321). The reference's backward rule for it is a placeholder
-    that hands the cotangent through unchanged (reduce_mul_op.mojo:238-255, "TODO" in its test file)."""
+    that hands the cotangent through unchanged (reduce_mul_op.mojo:238-255, its test file says the rule is still to be written)."""
     return _reduce_other(x, axis, keepdims, L.REDUCE_MUL, "reduce_mul", "reduce_mul_op.mojo:238-255 is a placeholder")
 
 
