@@ -512,6 +512,13 @@ FAST_CASES = [
     ((2, 8, 7, 12), (130, 8, 3, 3), (1, 1), (1, 1), (1, 1)),
     ((2, 3, 9, 9), (4, 3, 3, 3), (1, 1), (0, 0), (1, 1)),      # output width 7: general path
     ((2, 3, 11, 13), (4, 3, 3, 3), (2, 2), (1, 1), (1, 1)),    # strided data gradient: general path
+    # 3 x 3, unit stride, padding <= 1, channels a multiple of 8, rows of 28 or more: source rows cached in LDS
+    ((3, 8, 30, 28), (40, 8, 3, 3), (1, 1), (1, 1), (1, 1)),   # tiles that straddle images; 40 of 64 tile rows used
+    ((2, 16, 20, 36), (24, 16, 3, 3), (1, 1), (0, 0), (1, 1)),  # no padding (forward only; its data gradient pads by 2)
+    ((2, 8, 9, 64), (72, 8, 3, 3), (1, 1), (1, 1), (1, 1)),    # rows longer than 59: the wider cache pitch
+    ((1, 8, 6, 44), (136, 8, 3, 3), (1, 1), (1, 1), (1, 1)),   # more than 128 output channels: 128-row tiles
+    ((2, 8, 10, 48), (16, 8, 3, 3), (1, 1), (1, 0), (1, 1)),   # padded rows, unpadded columns
+    ((5, 24, 31, 32), (8, 24, 3, 3), (1, 1), (1, 1), (1, 1)),  # three chunks of channels; data gradient over one chunk
 ]
 
 
