@@ -624,7 +624,7 @@ struct DirectArgs {
   float* out;         // [N, Mrows, OH, OW]
   int Mrows, Cred, chunks, OH, OW, SH, SW, Ncols, NOH;
   int py, px;         // zero rows / columns in front of the source (0 or 1)
-  int MR, plane;      // output rows a pixel tile can touch; floats per cached channel = 3 * MR * PITCH
+  int MR, plane;      // output rows a pixel tile can touch; floats per cached channel = 3 * MR * PITCH + 32
   int tasks;          // 16-byte pieces of source rows per chunk: 8 * 3 * MR * SW / 4
   FastDiv d_ohw, d_ow, d_oh, d_f4row;
   int tiles_m, tiles_n, relu;
@@ -652,8 +652,9 @@ __global__ __launch_bounds__(256, 2) void conv_direct3x3_kernel(DirectArgs a) {
   // the columns on either side of a cached row are never written again: zero them once (everything between them is
   // rewritten with every chunk, zeros included where a row lies outside its image)
   for (int i = tid; i < CC * 3 * a.MR; i += 256) {
-    Bc[i * PITCH + 3] = 0.f;
-    Bc[i * PITCH + 4 + a.SW] = 0.f;
+    const int cc = i / (3 * a.MR), at = cc * a.plane + (i - cc * 3 * a.MR) * PITCH;
+    Bc[at + 3] = 0.f;
+    Bc[at + 4 + a.SW] = 0.f;
   }
 
   // source rows -> cache: task u = (channel, cached row, 16-byte piece); a cached row 3g + r holds source row
@@ -1064,7 +1065,10 @@ int32_t run_direct3x3(int mode, const ConvP& p, const float* src, const float* w
   // 64 output channels per work-group up to 128 channels in all (measured faster than 128 at 128: 0.298 against 0.313 ms,
   // twice the tiles to spread over the CUs and three work-groups per CU instead of two), 128 beyond
   const int fm = Mrows > 128 ? 2 : 1, BM = 64 * fm;
-  const size_t lds = ((size_t)BM * 76 + (size_t)8 * 3 * MR * pitch) * 4;
+  // a cached channel is 3 * MR rows plus half a row of banks, so that the two half-waves of a fragment read (one
+  // channel apart) fall into opposite halves of the 64 LDS banks
+  const int plane = 3 * MR * pitch + 32;
+  const size_t lds = ((size_t)BM * 76 + (size_t)8 * plane) * 4;
   if (tasks > 2048 || lds > 64 * 1024 || (int64_t)p.N * Cred * SH * SW >= (1ll << 29)) return 1;
   DirectArgs a;
   a.tiles_m = (Mrows + BM - 1) / BM;
@@ -1079,7 +1083,7 @@ int32_t run_direct3x3(int mode, const ConvP& p, const float* src, const float* w
   ENDIA_LAUNCH_CHECK();
   a.src = src; a.wp = static_cast<const float*>(wp.p); a.bias = bias; a.out = out; a.relu = relu;
   a.Mrows = Mrows; a.Cred = Cred; a.OH = OH; a.OW = OW; a.SH = SH; a.SW = SW; a.Ncols = p.N * OH * OW; a.NOH = p.N * OH;
-  a.py = py; a.px = px; a.MR = MR; a.plane = 3 * MR * pitch; a.tasks = tasks;
+  a.py = py; a.px = px; a.MR = MR; a.plane = plane; a.tasks = tasks;
   a.d_ohw = make_fastdiv(OH * OW); a.d_ow = make_fastdiv(OW); a.d_oh = make_fastdiv(OH); a.d_f4row = make_fastdiv(SW / 4);
   a.tiles_n = (a.Ncols + 127) / 128;
   a.src_bytes = (int64_t)p.N * Cred * SH * SW * 4;
