@@ -627,23 +627,24 @@ struct DirectArgs {
   int MR, plane;      // output rows a pixel tile can touch; floats per cached channel = 3 * MR * PITCH + 32
   int tasks;          // 16-byte pieces of source rows per chunk: 8 * 3 * MR * SW / 4
   FastDiv d_ohw, d_ow, d_oh, d_f4row;
-  int tiles_m, tiles_n, relu;
+  int tiles_m, relu;
+  int full_blocks, full_tiles_n;  // tiles of 128 pixels: full_tiles_n per tile row
+  int MR_half, tasks_half;        // the same for the 64-pixel tiles behind them
   int64_t src_bytes, wp_bytes;
 };
 
-template <int FM, int PITCH, bool FWD>
-__global__ __launch_bounds__(256, 2) void conv_direct3x3_kernel(DirectArgs a) {
-  constexpr int FN = 2, BM = 64 * FM, BN = 128, CC = 8, KC = 72, LDA = KC + 4;
+// One tile: rows [tm * 64 * FM, ...) of the output channels, pixels [n0, n0 + 64 * FN). MR / tasks: the cache rows and
+// staging pieces a tile of that many pixels needs.
+template <int FM, int FN, int PITCH, bool FWD>
+__device__ __forceinline__ void direct3x3_tile(const DirectArgs& a, int tm, int n0, int MR, int tasks, float* smem) {
+  constexpr int BM = 64 * FM, CC = 8, KC = 72, LDA = KC + 4;
   constexpr int A_F4 = BM * (KC / 4), PA = (A_F4 + 255) / 256, PB = 8;
-  extern __shared__ __attribute__((aligned(16))) float smem[];
   float* As = smem;
   float* Bc = smem + BM * LDA;
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int wm = wave >> 1, wn = wave & 1, l32 = lane & 31, h = lane >> 5;
-  int tm, tn;
-  tile_of_block(blockIdx.x, gridDim.x, a.tiles_m, a.tiles_n, tm, tn);
-  const int m0 = tm * BM, n0 = tn * BN;
+  const int m0 = tm * BM;
   const int ohw = a.OH * a.OW;
   // global output row (image * OH + row) of the tile's first pixel
   const int img0 = (int)fdiv((uint32_t)n0, a.d_ohw);
@@ -651,8 +652,8 @@ __global__ __launch_bounds__(256, 2) void conv_direct3x3_kernel(DirectArgs a) {
 
   // the columns on either side of a cached row are never written again: zero them once (everything between them is
   // rewritten with every chunk, zeros included where a row lies outside its image)
-  for (int i = tid; i < CC * 3 * a.MR; i += 256) {
-    const int cc = i / (3 * a.MR), at = cc * a.plane + (i - cc * 3 * a.MR) * PITCH;
+  for (int i = tid; i < CC * 3 * MR; i += 256) {
+    const int cc = i / (3 * MR), at = cc * a.plane + (i - cc * 3 * MR) * PITCH;
     Bc[at + 3] = 0.f;
     Bc[at + 4 + a.SW] = 0.f;
   }
@@ -667,9 +668,9 @@ __global__ __launch_bounds__(256, 2) void conv_direct3x3_kernel(DirectArgs a) {
     const int u = tid + p * 256;
     goff[p] = OOB_OFFSET;
     loff[p] = -1;
-    if (u < a.tasks) {
+    if (u < tasks) {
       const int rowid = (int)fdiv((uint32_t)u, a.d_f4row), c4 = u - rowid * f4row;
-      const int cc = rowid / (3 * a.MR), rr = rowid - cc * 3 * a.MR;
+      const int cc = rowid / (3 * MR), rr = rowid - cc * 3 * MR;
       const int g = rr / 3, r = rr - 3 * g;
       const int grow = grow0 + g;
       loff[p] = cc * a.plane + rr * PITCH + 4 + 4 * c4;
@@ -718,7 +719,7 @@ __global__ __launch_bounds__(256, 2) void conv_direct3x3_kernel(DirectArgs a) {
   int pix[FN];
 #pragma unroll
   for (int fn = 0; fn < FN; ++fn) {
-    const int j = n0 + wn * 64 + fn * 32 + l32;
+    const int j = n0 + wn * 32 * FN + fn * 32 + l32;
     pix[fn] = h * a.plane;
     if (j < a.Ncols) {
       const int img = (int)fdiv((uint32_t)j, a.d_ohw), rem = j - img * ohw;
@@ -766,7 +767,7 @@ __global__ __launch_bounds__(256, 2) void conv_direct3x3_kernel(DirectArgs a) {
 
 #pragma unroll
   for (int fn = 0; fn < FN; ++fn) {
-    const int j = n0 + wn * 64 + fn * 32 + l32;
+    const int j = n0 + wn * 32 * FN + fn * 32 + l32;
     if (j >= a.Ncols) continue;
     const int img = (int)fdiv((uint32_t)j, a.d_ohw);
     const int64_t col_off = (int64_t)img * a.Mrows * ohw + (j - (int64_t)img * ohw);
@@ -784,6 +785,22 @@ __global__ __launch_bounds__(256, 2) void conv_direct3x3_kernel(DirectArgs a) {
           a.out[col_off + (int64_t)m * ohw] = val;
         }
       }
+  }
+}
+
+// Whole tiles of 128 pixels first; what is left after the last full round over the CUs is cut into tiles of 64
+// pixels, so that the CUs that get one more tile than the others get half a tile more (see run_direct3x3).
+template <int FM, int PITCH, bool FWD>
+__global__ __launch_bounds__(256, 2) void conv_direct3x3_kernel(DirectArgs a) {
+  extern __shared__ __attribute__((aligned(16))) float smem[];
+  const int b = blockIdx.x;
+  if (b < a.full_blocks) {
+    int tm, tn;
+    tile_of_block(b, a.full_blocks, a.tiles_m, a.full_tiles_n, tm, tn);
+    direct3x3_tile<FM, 2, PITCH, FWD>(a, tm, tn * 128, a.MR, a.tasks, smem);
+  } else {
+    const int hb = b - a.full_blocks, tn = hb / a.tiles_m, tm = hb - tn * a.tiles_m;
+    direct3x3_tile<FM, 1, PITCH, FWD>(a, tm, a.full_tiles_n * 128 + tn * 64, a.MR_half, a.tasks_half, smem);
   }
 }
 
@@ -1085,10 +1102,21 @@ int32_t run_direct3x3(int mode, const ConvP& p, const float* src, const float* w
   a.Mrows = Mrows; a.Cred = Cred; a.OH = OH; a.OW = OW; a.SH = SH; a.SW = SW; a.Ncols = p.N * OH * OW; a.NOH = p.N * OH;
   a.py = py; a.px = px; a.MR = MR; a.plane = plane; a.tasks = tasks;
   a.d_ohw = make_fastdiv(OH * OW); a.d_ow = make_fastdiv(OW); a.d_oh = make_fastdiv(OH); a.d_f4row = make_fastdiv(SW / 4);
-  a.tiles_n = (a.Ncols + 127) / 128;
   a.src_bytes = (int64_t)p.N * Cred * SH * SW * 4;
   a.wp_bytes = (int64_t)a.chunks * rows_pad * 72 * 4;
-  const dim3 grid((unsigned)(a.tiles_m * a.tiles_n));
+  // The busiest CU sets the time, and with t tiles on c CUs it works on ceil(t / c) of them. When the tiles beyond the
+  // last full round are few (at most one for every other CU), they are cut into 64-pixel tiles: twice as many CUs get
+  // half as much extra work. 200704 pixels, 64 channels per tile row: 1568 tiles = 6 rounds + 32 -> 6 rounds + 64 halves.
+  const int tiles_n = (a.Ncols + 127) / 128, cus = endia::ctx().cu_count;
+  const int total = a.tiles_m * tiles_n, beyond = total % cus;
+  a.full_tiles_n = tiles_n;
+  if (total > cus && beyond > 0 && beyond <= cus / 2 && cus % a.tiles_m == 0) a.full_tiles_n = (total - beyond) / a.tiles_m;
+  a.full_blocks = a.tiles_m * a.full_tiles_n;
+  const int left = a.Ncols - a.full_tiles_n * 128;  // pixels for the 64-pixel tiles
+  const int half_tiles_n = left > 0 ? (left + 63) / 64 : 0;
+  a.MR_half = (63 + OW - 1) / OW + 1;
+  a.tasks_half = 8 * 3 * a.MR_half * (SW / 4);
+  const dim3 grid((unsigned)(a.full_blocks + a.tiles_m * half_tiles_n));
 #define ENDIA_LAUNCH_DIRECT(FM, PITCH)                                                                                       \
   do {                                                                                                                       \
     if (fwd) hipLaunchKernelGGL((conv_direct3x3_kernel<FM, PITCH, true>), grid, dim3(256), lds, s, a);                         \

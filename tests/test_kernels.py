@@ -519,6 +519,7 @@ FAST_CASES = [
     ((1, 8, 6, 44), (136, 8, 3, 3), (1, 1), (1, 1), (1, 1)),   # more than 128 output channels: 128-row tiles
     ((2, 8, 10, 48), (16, 8, 3, 3), (1, 1), (1, 0), (1, 1)),   # padded rows, unpadded columns
     ((5, 24, 31, 32), (8, 24, 3, 3), (1, 1), (1, 1), (1, 1)),  # three chunks of channels; data gradient over one chunk
+    ((12, 8, 56, 56), (8, 8, 3, 3), (1, 1), (1, 1), (1, 1)),   # 294 pixel tiles on 256 CUs: the last 38 run as 76 half tiles
 ]
 
 
