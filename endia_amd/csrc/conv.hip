@@ -616,7 +616,8 @@ __global__ __launch_bounds__(WGM* WGN * 64, 4) void conv_wgrad_vec_kernel(WgradV
 // second element), and the pair is made of the SAME tap in two neighbouring channels, so the half-waves differ by
 // one cached channel, a constant folded into the lane's base address. Within a chunk, element k = 8j + 4h + i of
 // the packed weights belongs to step 4j + i = 9 * (channel pair) + 3r + s and to channel 2 * (channel pair) + h.
-// 144 MFMAs per wave between two barriers (the dense kernel has 64), two work-groups per CU.
+// The weights do not pass through LDS at all (see the tile function). 72 or 144 MFMAs per wave between two barriers
+// (the dense kernel has 64 at its large tile), three or four work-groups per CU.
 struct DirectArgs {
   const float* src;   // [N, Cred, SH, SW]
   const float* wp;    // [chunks][tiles_m * BM][72], packed as described above
@@ -637,10 +638,8 @@ struct DirectArgs {
 // staging pieces a tile of that many pixels needs.
 template <int FM, int FN, int PITCH, bool FWD>
 __device__ __forceinline__ void direct3x3_tile(const DirectArgs& a, int tm, int n0, int MR, int tasks, float* smem) {
-  constexpr int BM = 64 * FM, CC = 8, KC = 72, LDA = KC + 4;
-  constexpr int A_F4 = BM * (KC / 4), PA = (A_F4 + 255) / 256, PB = 8;
-  float* As = smem;
-  float* Bc = smem + BM * LDA;
+  constexpr int BM = 64 * FM, CC = 8, KC = 72, PB = 8;
+  float* Bc = smem;
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int wm = wave >> 1, wn = wave & 1, l32 = lane & 31, h = lane >> 5;
@@ -680,26 +679,11 @@ __device__ __forceinline__ void direct3x3_tile(const DirectArgs& a, int tm, int 
       }
     }
   }
-  // packed weights of this tile's rows: BM * 72 consecutive floats per chunk
-  uint32_t aoff[PA];
-  int alds[PA];
-#pragma unroll
-  for (int p = 0; p < PA; ++p) {
-    const int f = tid + p * 256;
-    aoff[p] = f < A_F4 ? (uint32_t)((m0 * KC + 4 * f) * 4) : OOB_OFFSET;
-    const int row = f / (KC / 4);
-    alds[p] = row * LDA + 4 * (f - row * (KC / 4));
-  }
   const __amdgpu_buffer_rsrc_t rs_src = make_rsrc(a.src, a.src_bytes);
   const __amdgpu_buffer_rsrc_t rs_w = make_rsrc(a.wp, a.wp_bytes);
   const uint32_t src_step = (uint32_t)(CC * a.SH * a.SW) * 4u, w_step = (uint32_t)(a.tiles_m * BM * KC) * 4u;
-  float4 ra[PA], rb[PB];
+  float4 rb[PB];
   auto load = [&](int chunk) {
-#pragma unroll
-    for (int p = 0; p < PA; ++p) {
-      v4i v = __builtin_amdgcn_raw_buffer_load_b128(rs_w, (int)aoff[p], (int)(chunk * w_step), 0);
-      ra[p] = *reinterpret_cast<float4*>(&v);
-    }
 #pragma unroll
     for (int p = 0; p < PB; ++p) {
       v4i v = __builtin_amdgcn_raw_buffer_load_b128(rs_src, (int)goff[p], (int)(chunk * src_step), 0);
@@ -707,9 +691,6 @@ __device__ __forceinline__ void direct3x3_tile(const DirectArgs& a, int tm, int 
     }
   };
   auto store = [&]() {
-#pragma unroll
-    for (int p = 0; p < PA; ++p)
-      if (tid + p * 256 < A_F4) *reinterpret_cast<float4*>(&As[alds[p]]) = ra[p];
 #pragma unroll
     for (int p = 0; p < PB; ++p)
       if (loff[p] >= 0) *reinterpret_cast<float4*>(&Bc[loff[p]]) = rb[p];
@@ -731,8 +712,23 @@ __device__ __forceinline__ void direct3x3_tile(const DirectArgs& a, int tm, int 
 
   floatx16 acc[FM][FN];
   zero_acc<FM, FN>(acc);
+  // The weights go from memory straight into the A fragments: every lane reads its own rows of the packed weights
+  // (group jg of a chunk is the 16 bytes at 8 * jg + 4 * h floats of the row), one group of four steps ahead of the
+  // MFMAs that use it. All work-groups read the same few hundred KiB, which stay in L2; LDS holds the row cache alone.
+  uint32_t arow[FM];
+#pragma unroll
+  for (int fm = 0; fm < FM; ++fm) arow[fm] = (uint32_t)(((m0 + a_row + 32 * fm) * KC + 4 * h) * 4);
+  float4 afn[FM];
+  auto fetch_a = [&](int chunk, int jg) {
+#pragma unroll
+    for (int fm = 0; fm < FM; ++fm) {
+      v4i v = __builtin_amdgcn_raw_buffer_load_b128(rs_w, (int)(arow[fm] + 32u * jg), (int)(chunk * w_step), 0);
+      afn[fm] = *reinterpret_cast<float4*>(&v);
+    }
+  };
   load(0);
-  __syncthreads();  // cache zeroed before the first rows land in it
+  fetch_a(0, 0);
+  __syncthreads();  // border columns zeroed before the first rows land in the cache
   store();
   __syncthreads();
   for (int chunk = 0; chunk < a.chunks; ++chunk) {
@@ -743,9 +739,11 @@ __device__ __forceinline__ void direct3x3_tile(const DirectArgs& a, int tm, int 
       float af[FM][4];
 #pragma unroll
       for (int fm = 0; fm < FM; ++fm) {
-        const float4 t = *reinterpret_cast<const float4*>(&As[(a_row + 32 * fm) * LDA + 8 * jg + 4 * h]);
+        const float4 t = afn[fm];
         af[fm][0] = t.x; af[fm][1] = t.y; af[fm][2] = t.z; af[fm][3] = t.w;
       }
+      if (jg + 1 < KC / 8) fetch_a(chunk, jg + 1);
+      else if (more) fetch_a(chunk + 1, 0);
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
         const int q = 4 * jg + i, ccp = q / 9, tap = q - 9 * ccp, r = tap / 3, sx = tap - 3 * r;
@@ -1081,11 +1079,13 @@ int32_t run_direct3x3(int mode, const ConvP& p, const float* src, const float* w
   const int tasks = 8 * 3 * MR * (SW / 4);
   // 64 output channels per work-group up to 128 channels in all (measured faster than 128 at 128: 0.298 against 0.313 ms,
   // twice the tiles to spread over the CUs and three work-groups per CU instead of two), 128 beyond
+  // 64 output channels per work-group up to 128 channels in all (twice the tiles to spread over the CUs, four work-groups
+  // per CU instead of three; measured the same speed as 128 at 128 channels), 128 beyond
   const int fm = Mrows > 128 ? 2 : 1, BM = 64 * fm;
   // a cached channel is 3 * MR rows plus half a row of banks, so that the two half-waves of a fragment read (one
   // channel apart) fall into opposite halves of the 64 LDS banks
   const int plane = 3 * MR * pitch + 32;
-  const size_t lds = ((size_t)BM * 76 + (size_t)8 * plane) * 4;
+  const size_t lds = (size_t)8 * plane * 4;
   if (tasks > 2048 || lds > 64 * 1024 || (int64_t)p.N * Cred * SH * SW >= (1ll << 29)) return 1;
   DirectArgs a;
   a.tiles_m = (Mrows + BM - 1) / BM;
