@@ -854,10 +854,11 @@ __global__ __launch_bounds__(TPB) void pack_weights_kernel(const float* __restri
 // as three launches they cost about ten microseconds of a call that lasts three hundred.
 //   table[t], t = (ch, kz, r, s): byte offset ((ch*Dp + kz*dd)*Hp + r*dh)*Wp + s*dw inside a padded image; the data
 //     gradient walks the taps in reverse (kz -> T-1-kz, r -> R-1-r, s -> S-1-s); entries past Kd get OOB_OFFSET.
-//   padded copy: dst[pl][z][y][x] = src[pl][z - pz][y - py][x - px] where in range, else 0; one wave per padded row
-//     (rows are short: the walk over x needs no division, and reads and writes stay contiguous).
+//   padded copy: dst[pl][z][y][x] = src[pl][z - pz][y - py][x - px] where in range, else 0; padded rows are a whole
+//     number of 16-byte pieces, one piece per thread (32-bit index arithmetic with precomputed divisions).
 struct PrepArgs {
   const float* src; float* dst; int64_t rows_total; int D, H, W, Dp, Hp, Wp, pz, py, px;   // padded copy
+  FastDiv d_w4, d_hp, d_dp;                                                                 // Wp / 4, Hp, Dp
   int* table; int tn, Kd, T, R, S, dd, dh, dw, flip;                                        // tap table
   const float* w; float* wp; int K, C, RS, Kd_pad, transpose;                               // weight repacking (w may be null)
   int table_blocks, pack_blocks;
@@ -888,21 +889,33 @@ __global__ __launch_bounds__(TPB) void conv_prep_kernel(PrepArgs a) {
       a.wp[i] = v;
     }
   } else {
+    // one 16-byte piece of a padded row per thread: interior pieces are one (unaligned) 16-byte load, pieces that touch
+    // the zero columns load their elements one by one
+    struct __attribute__((packed, aligned(4))) Quad { float x, y, z, w; };
     const int first = a.table_blocks + a.pack_blocks;
-    const int lane = threadIdx.x & 63;
-    const int64_t waves = (int64_t)(gridDim.x - first) * (TPB / 64);
-    for (int64_t row = (int64_t)(b - first) * (TPB / 64) + (threadIdx.x >> 6); row < a.rows_total; row += waves) {
-      const int64_t slab = row / a.Hp;  // (plane, padded depth)
-      const int y = (int)(row - slab * a.Hp), sy = y - a.py;
-      const int64_t pl = slab / a.Dp;
-      const int sz = (int)(slab - pl * a.Dp) - a.pz;
-      const bool row_ok = (unsigned)sy < (unsigned)a.H && (unsigned)sz < (unsigned)a.D;
-      const float* s = a.src + ((pl * a.D + (row_ok ? sz : 0)) * a.H + (row_ok ? sy : 0)) * a.W;
-      float* d = a.dst + row * a.Wp;
-      for (int x = lane; x < a.Wp; x += 64) {
-        int sx = x - a.px;
-        d[x] = (row_ok && (unsigned)sx < (unsigned)a.W) ? s[sx] : 0.f;
+    const int W4 = a.Wp >> 2;
+    const uint32_t total = (uint32_t)a.rows_total * (uint32_t)W4, stride = (uint32_t)(gridDim.x - first) * TPB;
+    for (uint32_t idx = (uint32_t)(b - first) * TPB + threadIdx.x; idx < total; idx += stride) {
+      const uint32_t row = fdiv(idx, a.d_w4), c4 = idx - row * (uint32_t)W4;
+      const uint32_t slab = fdiv(row, a.d_hp);  // (plane, padded depth)
+      const int sy = (int)(row - slab * (uint32_t)a.Hp) - a.py;
+      const uint32_t pl = fdiv(slab, a.d_dp);
+      const int sz = (int)(slab - pl * (uint32_t)a.Dp) - a.pz;
+      float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
+      if ((unsigned)sy < (unsigned)a.H && (unsigned)sz < (unsigned)a.D) {
+        const float* s = a.src + (((int64_t)pl * a.D + sz) * a.H + sy) * a.W;
+        const int x0 = (int)(c4 * 4) - a.px;
+        if (x0 >= 0 && x0 + 3 < a.W) {
+          const Quad q = *reinterpret_cast<const Quad*>(s + x0);
+          v = make_float4(q.x, q.y, q.z, q.w);
+        } else {
+          if ((unsigned)x0 < (unsigned)a.W) v.x = s[x0];
+          if ((unsigned)(x0 + 1) < (unsigned)a.W) v.y = s[x0 + 1];
+          if ((unsigned)(x0 + 2) < (unsigned)a.W) v.z = s[x0 + 2];
+          if ((unsigned)(x0 + 3) < (unsigned)a.W) v.w = s[x0 + 3];
+        }
       }
+      reinterpret_cast<float4*>(a.dst)[idx] = v;
     }
   }
 }
@@ -956,6 +969,10 @@ int32_t make_params(const endia_hip_conv3d_desc* d, ConvP& p) {
   return make_params("conv3d", in, p);
 }
 
+// Row length of a zero-padded copy: the padding on both sides, rounded up to whole 16-byte pieces so that the copy
+// writes aligned float4s (the extra columns are zeros that no tap reaches).
+inline int padded_row(int W, int px) { return (W + 2 * px + 3) & ~3; }
+
 struct PoolBuf {  // scratch from the library's pool, returned on scope exit (stream-ordered reuse)
   void* p = nullptr;
   ~PoolBuf() { if (p) endia_hip_free(p); }
@@ -983,13 +1000,14 @@ int32_t pack_weights(const ConvP& p, const float* w, int transpose, int Kd_pad, 
 // Padded copy of src, tap table of n entries and (when w is given) repacked weights, from one launch.
 int32_t prep_vec(const ConvP& p, const float* src, int64_t planes, int SD, int SH, int SW, int pz, int py, int px, int n_table,
                  int Kd, int flip, const float* w, int transpose, int Kd_pad, PoolBuf& spad, PoolBuf& table, PoolBuf& wp) {
-  const int Dp = SD + 2 * pz, Hp = SH + 2 * py, Wp = SW + 2 * px;
+  const int Dp = SD + 2 * pz, Hp = SH + 2 * py, Wp = padded_row(SW, px);
   int32_t rc = endia_hip_malloc(planes * Dp * Hp * Wp * 4, &spad.p);
   if (rc) return rc;
   if ((rc = endia_hip_malloc((int64_t)n_table * 4, &table.p))) return rc;
   PrepArgs a = {};
   a.src = src; a.dst = static_cast<float*>(spad.p); a.rows_total = planes * Dp * Hp;
   a.D = SD; a.H = SH; a.W = SW; a.Dp = Dp; a.Hp = Hp; a.Wp = Wp; a.pz = pz; a.py = py; a.px = px;
+  a.d_w4 = make_fastdiv(Wp / 4); a.d_hp = make_fastdiv(Hp); a.d_dp = make_fastdiv(Dp);
   a.table = static_cast<int*>(table.p); a.tn = n_table; a.Kd = Kd; a.T = p.T; a.R = p.R; a.S = p.S;
   a.dd = p.dd; a.dh = p.dh; a.dw = p.dw; a.flip = flip;
   a.table_blocks = (n_table + TPB - 1) / TPB;
@@ -1001,7 +1019,7 @@ int32_t prep_vec(const ConvP& p, const float* src, int64_t planes, int SD, int S
     int64_t pb = ((int64_t)rows * Kd_pad + TPB - 1) / TPB;
     a.pack_blocks = (int)(pb > 2048 ? 2048 : pb);
   }
-  int64_t pad_blocks = (a.rows_total + 3) / 4, cap = (int64_t)endia::ctx().cu_count * 64;
+  int64_t pad_blocks = (a.rows_total * (Wp / 4) + TPB - 1) / TPB, cap = (int64_t)endia::ctx().cu_count * 16;
   if (pad_blocks > cap) pad_blocks = cap;
   if (pad_blocks < 1) pad_blocks = 1;
   hipLaunchKernelGGL(conv_prep_kernel, dim3((unsigned)(a.table_blocks + a.pack_blocks + pad_blocks)), dim3(TPB), 0,
@@ -1026,7 +1044,7 @@ int32_t run_igemm_vec(int mode, const ConvP& p, const float* src, const float* w
     row_stride = 1; depth_stride = 1;
     if (pz < 0 || py < 0 || px < 0) return 1;
   }
-  const int Dp = SD + 2 * pz, Hp = SH + 2 * py, Wp = SW + 2 * px;
+  const int Dp = SD + 2 * pz, Hp = SH + 2 * py, Wp = padded_row(SW, px);
   const int Kd = Cred * p.T * p.R * p.S, Kd_pad = (Kd + 31) / 32 * 32;
   if ((int64_t)p.N * Cred * Dp * Hp * Wp >= (1ll << 29) || Kd_pad > 8192) return 1;
   // the last reads of a row group must stay inside the padded image rows: ox + 3 + (S-1)*dw <= Wp - 1 holds because
@@ -1225,7 +1243,7 @@ int32_t conv_bwd_weight(const char* who, const ConvP& p, const float* x, const f
   a.d_trs = make_fastdiv(p.T * p.R * p.S); a.d_rs = make_fastdiv(p.R * p.S); a.d_s = make_fastdiv(p.S);
   a.x_bytes = (int64_t)p.N * p.C * p.D * p.H * p.W * 4;
   a.dy_bytes = (int64_t)p.N * p.K * p.O * p.P * p.Q * 4;
-  const int Dp = p.D + 2 * p.pd, Hp = p.H + 2 * p.ph, Wp = p.W + 2 * p.pw;
+  const int Dp = p.D + 2 * p.pd, Hp = p.H + 2 * p.ph, Wp = padded_row(p.W, p.pw);
   const bool vec = p.sw == 1 && p.Q % 4 == 0 && (int64_t)p.N * p.C * Dp * Hp * Wp < (1ll << 29) &&
                    (reinterpret_cast<uintptr_t>(dy) & 15) == 0;
   // 64-wide tiles over the taps when the last 128-wide tile would be at most half full
