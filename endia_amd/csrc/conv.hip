@@ -997,15 +997,18 @@ int32_t pack_weights(const ConvP& p, const float* w, int transpose, int Kd_pad, 
   return ENDIA_HIP_OK;
 }
 
-// Padded copy of src, tap table of n entries and (when w is given) repacked weights, from one launch.
+// Padded copy of src (spad stays empty when the source needs none), tap table of n entries and (when w is given)
+// repacked weights, from one launch.
 int32_t prep_vec(const ConvP& p, const float* src, int64_t planes, int SD, int SH, int SW, int pz, int py, int px, int n_table,
                  int Kd, int flip, const float* w, int transpose, int Kd_pad, PoolBuf& spad, PoolBuf& table, PoolBuf& wp) {
   const int Dp = SD + 2 * pz, Hp = SH + 2 * py, Wp = padded_row(SW, px);
-  int32_t rc = endia_hip_malloc(planes * Dp * Hp * Wp * 4, &spad.p);
-  if (rc) return rc;
+  // nothing to pad (a 1 x 1 kernel, an unpadded convolution over rows of whole 16-byte pieces): the source serves as it is
+  const bool copy = pz || py || px || Wp != SW || (reinterpret_cast<uintptr_t>(src) & 15);
+  int32_t rc = ENDIA_HIP_OK;
+  if (copy && (rc = endia_hip_malloc(planes * Dp * Hp * Wp * 4, &spad.p))) return rc;
   if ((rc = endia_hip_malloc((int64_t)n_table * 4, &table.p))) return rc;
   PrepArgs a = {};
-  a.src = src; a.dst = static_cast<float*>(spad.p); a.rows_total = planes * Dp * Hp;
+  a.src = src; a.dst = static_cast<float*>(spad.p); a.rows_total = copy ? planes * Dp * Hp : 0;
   a.D = SD; a.H = SH; a.W = SW; a.Dp = Dp; a.Hp = Hp; a.Wp = Wp; a.pz = pz; a.py = py; a.px = px;
   a.d_w4 = make_fastdiv(Wp / 4); a.d_hp = make_fastdiv(Hp); a.d_dp = make_fastdiv(Dp);
   a.table = static_cast<int*>(table.p); a.tn = n_table; a.Kd = Kd; a.T = p.T; a.R = p.R; a.S = p.S;
@@ -1021,7 +1024,7 @@ int32_t prep_vec(const ConvP& p, const float* src, int64_t planes, int SD, int S
   }
   int64_t pad_blocks = (a.rows_total * (Wp / 4) + TPB - 1) / TPB, cap = (int64_t)endia::ctx().cu_count * 16;
   if (pad_blocks > cap) pad_blocks = cap;
-  if (pad_blocks < 1) pad_blocks = 1;
+  if (pad_blocks < 1 && copy) pad_blocks = 1;
   hipLaunchKernelGGL(conv_prep_kernel, dim3((unsigned)(a.table_blocks + a.pack_blocks + pad_blocks)), dim3(TPB), 0,
                      endia::ctx().stream, a);
   ENDIA_LAUNCH_CHECK();
@@ -1054,7 +1057,7 @@ int32_t run_igemm_vec(int mode, const ConvP& p, const float* src, const float* w
                         spad, table, wp);
   if (rc) return rc;
   VecArgs a;
-  a.src = static_cast<const float*>(spad.p); a.wp = static_cast<const float*>(wp.p);
+  a.src = spad.p ? static_cast<const float*>(spad.p) : src; a.wp = static_cast<const float*>(wp.p);
   a.table = static_cast<const int*>(table.p); a.bias = bias; a.out = out; a.relu = relu;
   a.Mrows = Mrows; a.OD = OD; a.OH = OH; a.OW = OW; a.Ncols = p.N * OD * OH * OW; a.Kd_pad = Kd_pad;
   a.img_floats = Cred * Dp * Hp * Wp; a.Wp = Wp; a.sh = row_stride; a.zstep = depth_stride * Hp * Wp;
@@ -1279,7 +1282,7 @@ int32_t conv_bwd_weight(const char* who, const ConvP& p, const float* x, const f
                        none)))
       return rc;
     WgradVecArgs v;
-    v.xpad = static_cast<const float*>(xpad.p); v.dy = dy; v.table = static_cast<const int*>(table.p); v.part = a.part;
+    v.xpad = xpad.p ? static_cast<const float*>(xpad.p) : x; v.dy = dy; v.table = static_cast<const int*>(table.p); v.part = a.part;
     v.K = p.K; v.Kd = Kd; v.OPQ = p.O * p.P * p.Q; v.PQ = p.P * p.Q; v.Q = p.Q; v.sh = p.sh; v.Wp = Wp;
     v.img_floats = p.C * Dp * Hp * Wp; v.zstep = p.sd * Hp * Wp;
     v.total_j = a.total_j; v.chunk = a.chunk; v.d_opq = a.d_opq; v.d_pq = a.d_pq; v.d_q = a.d_q;
