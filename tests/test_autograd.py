@@ -535,6 +535,44 @@ def test_captured_step_matches_eager(nd, golden):
     assert nd.sum(nd.ones([5])).item() == 5.0
 
 
+def test_captured_step_with_split_reductions(nd):
+    """A captured step whose products are split along K inside their launches (few tiles per CU, K >= 256): the groups
+    of a tile meet through arrival counters that the last arriver puts back to zero, so every replay must give what
+    the eager step gives, bit for bit."""
+    rng = np.random.default_rng(21)
+    x = nd.array(rng.standard_normal((256, 512)).astype(np.float32))
+    y = nd.array(rng.standard_normal((256, 512)).astype(np.float32))
+
+    def build():
+        r = np.random.default_rng(3)
+        mlp = nd.nn.MLP([512, 512, 512], compute_backward=True)
+        for prm in mlp.params():
+            prm.copy_from_numpy((r.standard_normal(prm.shape()) * 0.04).astype(np.float32))
+        return mlp, nd.optim.SGD(mlp.params(), lr=1e-2)
+
+    def make(mlp, opt):
+        def step():
+            loss = nd.mse(mlp.forward(x), y)
+            loss.backward()
+            opt.step()
+            loss.zero_grad()
+            return loss
+        return step
+
+    (mlp_e, opt_e), (mlp_c, opt_c) = build(), build()
+    step_e, step_c = make(mlp_e, opt_e), make(mlp_c, opt_c)
+    step_e()
+    step_c()
+    captured = nd.capture(step_c)
+    for it in range(4):
+        loss_e = step_e()
+        loss_c = captured.replay()
+        assert loss_c.item() == loss_e.item(), "loss at replay %d" % it
+        for pe, pc in zip(mlp_e.params(), mlp_c.params()):
+            np.testing.assert_array_equal(pc.to_numpy(), pe.to_numpy(), err_msg="parameters at replay %d" % it)
+    captured.close()
+
+
 def test_captured_adam_step(nd, golden):
     """Adam with its step counter in device memory (capturable=True): the captured step, replayed, follows the
     eager host-counter Adam and the oracle's Adam step for step (1e-6: the bias corrections come from the device's
