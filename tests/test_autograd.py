@@ -838,3 +838,76 @@ def test_random_mlps_vs_oracle(nd):
             assert_close(mlp.weights[i].grad().to_numpy(), dWr[i], what=what + " dW%d" % i)
             assert_close(mlp.biases[i].grad().to_numpy(), dbr[i], tol=2e-4, what=what + " db%d" % i)
         loss.zero_grad()
+
+
+def test_random_expression_graphs_vs_torch(nd):
+    """Seeded random graphs over three leaves: elementwise ops with broadcasting, views (permute, reshape, slices),
+    reductions and matmuls, tensors used more than once (gradient accumulation), first and second order. Value and
+    every gradient against PyTorch float64 running the same sequence of ops."""
+    import torch
+    rng = np.random.default_rng(2024)
+    unary = [("sin", nd.sin, torch.sin), ("cos", nd.cos, torch.cos), ("tanh", nd.tanh, torch.tanh),
+             ("sigmoid", nd.sigmoid, torch.sigmoid), ("square", nd.square, torch.square),
+             ("relu", nd.relu, torch.relu), ("neg", nd.neg, torch.neg)]
+    for case in range(30):
+        m, k, n = (int(rng.choice([3, 8, 17, 32])) for _ in range(3))
+        leaves_np = [rng.standard_normal((m, k)), rng.standard_normal((k, n)), rng.standard_normal((n,))]
+        leaves_np = [(0.7 * a).astype(np.float32) for a in leaves_np]
+        ours = [nd.array(a, requires_grad=True) for a in leaves_np]
+        theirs = [torch.tensor(a, dtype=torch.float64, requires_grad=True) for a in leaves_np]
+        # pool of (ours, theirs) values of shape [m, n]
+        pool = [(nd.matmul(ours[0], ours[1]) + ours[2], torch.matmul(theirs[0], theirs[1]) + theirs[2])]
+        trace = ["A@B+c"]
+        for _ in range(int(rng.integers(3, 9))):
+            kind = int(rng.integers(0, 7))
+            a, ta = pool[int(rng.integers(len(pool)))]
+            b, tb = pool[int(rng.integers(len(pool)))]
+            if kind == 0:
+                name, f, tf = unary[int(rng.integers(len(unary)))]
+                pool.append((f(a), tf(ta)))
+                trace.append(name)
+            elif kind == 1:
+                op = int(rng.integers(3))
+                pool.append(((a + b, a - b, a * b)[op], (ta + tb, ta - tb, ta * tb)[op]))
+                trace.append("+-*"[op])
+            elif kind == 2:  # division by something bounded away from zero
+                pool.append((a / (nd.square(b) + 1.5), ta / (torch.square(tb) + 1.5)))
+                trace.append("/")
+            elif kind == 3:  # row and column sums broadcast back
+                ax = int(rng.integers(2))
+                pool.append((a * nd.reduce_add(b, [ax]), ta * tb.sum(dim=ax, keepdim=True)))
+                trace.append("bcast-sum%d" % ax)
+            elif kind == 4:  # through a transposed view and back
+                pool.append((nd.permute(nd.sin(nd.permute(a, [1, 0])), [1, 0]), torch.sin(ta.T).T))
+                trace.append("T-sin-T")
+            elif kind == 5:  # a slice padded back to the full shape by its gradient only: multiply a sub-block
+                r0, c0 = int(rng.integers(0, m - 1)), int(rng.integers(0, n - 1))
+                sub, tsub = a[r0:, c0:], ta[r0:, c0:]
+                pool.append((a * nd.mean(nd.tanh(sub)), ta * torch.tanh(tsub).mean()))
+                trace.append("slice-mean")
+            else:  # another product through the leaves: (a^T a) scaled into [m, n] via A B
+                g_, tg = nd.matmul(nd.permute(a, [1, 0]), b), torch.matmul(ta.T, tb)       # [n, n]
+                pool.append((nd.matmul(a, nd.tanh(g_) * (1.0 / n)), torch.matmul(ta, torch.tanh(tg) / n)))
+                trace.append("a@tanh(a^T b)")
+        out, tout = pool[-1]
+        for extra, textra in pool[:-1][::2]:  # tie earlier nodes in, so no branch of the graph is dead
+            out, tout = out + 0.1 * extra, tout + 0.1 * textra
+        loss, tloss = nd.sum(nd.square(out)) / float(m * n), torch.square(tout).sum() / (m * n)
+        what = "case %d (%s)" % (case, " ".join(trace))
+        second = case % 3 == 0
+        if second:  # gradient of the squared gradient norm w.r.t. the first leaf, i.e. a double backward
+            loss.backward(create_graph=True)
+            tg0, = torch.autograd.grad(tloss, theirs[0], create_graph=True)
+            g0 = ours[0].grad()
+            loss.zero_grad()  # drop the first pass's stored gradients everywhere, as grad() does (functional.mojo:77-82)
+            loss2, tloss2 = nd.sum(nd.square(g0)), torch.square(tg0).sum()
+            loss2.backward()
+            tloss2.backward()
+            assert_close([loss2.item()], [tloss2.item()], tol=2e-4, what=what + " squared gradient norm")
+        else:
+            loss.backward()
+            tloss.backward()
+            assert_close([loss.item()], [tloss.item()], what=what + " value")
+        for i, (lf, tl) in enumerate(zip(ours, theirs)):
+            want = tl.grad.numpy() if tl.grad is not None else np.zeros(lf.shape())
+            assert_close(lf.grad().to_numpy().reshape(want.shape), want, tol=5e-4 if second else 1e-4, what=what + " grad of leaf %d" % i)
