@@ -37,6 +37,30 @@ def test_streaming_kernels_full_size(dev):
     assert_close(dev.get(dy, (N, N)), 2 * (x64 - g64) / (N * N), tol=1e-6, what="mse grad")
 
 
+def test_streaming_kernels_past_2_31_elements(dev):
+    """2^31 + 4096 elements (8.6 GB per array): element indices no longer fit 32 bits. Constant inputs, so the expected
+    values are known without a host copy of the arrays; the head and the tail of every result are read back."""
+    n = (1 << 31) + 4096
+    x, y = dev.alloc(4 * n), dev.alloc(4 * n)
+
+    def ends(p):
+        return np.concatenate([dev.get(p, (512,)), dev.get(p + 4 * (n - 512), (512,))])
+
+    dev.call("endia_hip_fill", x, n, 0.5)
+    dev.call("endia_hip_unary_fwd", L.OP_SQUARE, n, x, y, 0)
+    np.testing.assert_array_equal(ends(y), np.full(1024, 0.25, np.float32))
+    dev.call("endia_hip_axpby", n, 2.0, y, 1.0, x, y)            # y = 2 * 0.25 + 0.5
+    np.testing.assert_array_equal(ends(y), np.ones(1024, np.float32))
+    dev.call("endia_hip_sgd_step", n, x, y, 0.5)                 # x = 0.5 - 0.5 * 1
+    np.testing.assert_array_equal(ends(x), np.zeros(1024, np.float32))
+    one = L.i64_array([1])
+    dev.call("endia_hip_binary", L.BIN_ADD, 1, L.i64_array([n]), one, one, x, y, x, 0)   # x = 0 + 1
+    np.testing.assert_array_equal(ends(x), np.ones(1024, np.float32))
+    total = dev.alloc(4)
+    dev.call("endia_hip_reduce_add", 1, L.i64_array([n]), 1, x, total, 1.0, 0)
+    assert abs(float(dev.get(total, (1,))[0]) - n) <= 1e-6 * n
+
+
 def test_adam_and_sgd_full_size_closed_form(dev):
     rng = np.random.default_rng(101)
     p = rng.standard_normal((N, N)).astype(np.float32)
