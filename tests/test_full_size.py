@@ -61,6 +61,21 @@ def test_streaming_kernels_past_2_31_elements(dev):
     assert abs(float(dev.get(total, (1,))[0]) - n) <= 1e-6 * n
 
 
+@pytest.mark.parametrize("K", [8, 2])
+def test_gemm_output_past_2_31_elements(dev, K):
+    """C = A B with 65536 x 40000 outputs (2.6e9 elements, 10.5 GB): output offsets need 64 bits. K = 8 takes the MFMA
+    kernel, K = 2 the one-thread-per-output kernel; rows from the top, the middle and the end of C against float64."""
+    M, N = 65536, 40000
+    rng = np.random.default_rng(K)
+    A = rng.standard_normal((M, K)).astype(np.float32)
+    B = rng.standard_normal((K, N)).astype(np.float32)
+    dA, dB, dC = dev.put(A), dev.put(B), dev.alloc(4 * M * N)
+    dev.call("endia_hip_sgemm", 0, 0, M, N, K, dA, K, dB, N, dC, N, 1, 0, 0, 0, L.EPI_NONE, L.OP_IDENTITY, None, None, None)
+    for r in (0, 1, 32767, 53688, M - 2, M - 1):   # row 53688 starts past element 2^31
+        got = dev.get(dC + 4 * r * N, (N,))
+        assert_close(got, A[r].astype(np.float64) @ B.astype(np.float64), tol=1e-6, what="row %d" % r)
+
+
 def test_adam_and_sgd_full_size_closed_form(dev):
     rng = np.random.default_rng(101)
     p = rng.standard_normal((N, N)).astype(np.float32)
