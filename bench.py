@@ -29,11 +29,11 @@ sys.path.insert(0, ROOT)
 
 FP32_MFMA_PEAK_TFLOPS = 157.3
 HBM_PEAK_GBS = 8000.0
-# HBM-side bytes per 4096^3 GEMM launch, averaged over the launch mix of one training step (8 NN with the bias /
-# bias+tanh epilogue, 7 NT with the tanh' epilogue, 8 TN). It cannot be read while the benchmark runs: it comes
+# HBM-side bytes per 4096^3 GEMM launch, averaged over the launch mix of one training step (1 NN with the bias epilogue,
+# 7 NN with bias+tanh, 7 NT with the tanh' epilogue, 8 TN; MiB per launch as in the per-kernel table). It cannot be read while the benchmark runs: it comes
 # from two rocprofv3 --pmc runs (FETCH_SIZE, WRITE_SIZE in KiB per dispatch), each scaled by what the same counter
 # reads for a 64 MiB copy kernel (x1.999 and x1.000); the per-kernel table is in profiles/.
-GEMM_TRAFFIC_BYTES = int((8 * 677.8 + 7 * 1351.0 + 8 * 745.7) / 23 * 1024 * 1024)
+GEMM_TRAFFIC_BYTES = int((1 * 704.1 + 7 * 608.7 + 7 * 1342.0 + 8 * 749.6) / 23 * 1024 * 1024)
 
 
 def build_wide_mlp(nd, width=4096, layers=8, batch=4096, seed=2):
