@@ -20,10 +20,17 @@ from .functional import (  # noqa: E402,F401
     relu, reshape, seed, set_complex_matmul_algorithm, sigmoid, sign, sin, sinh, sqrt, square, squeeze, std, sub, sum, tan,
     tanh, unsqueeze, variance, zeros,
 )
+from .functional import (  # noqa: E402,F401  the rest of the initialisers (endia/functional/init_ops/init_ops.mojo)
+    eye_like, fill_, fill_like, linspace, ones_, ones_like, rand_he_normal_, rand_he_normal_like, rand_he_uniform,
+    rand_he_uniform_, rand_he_uniform_like, rand_lecun_normal, rand_lecun_normal_, rand_lecun_normal_like,
+    rand_lecun_uniform, rand_lecun_uniform_, rand_lecun_uniform_like, rand_xavier_normal, rand_xavier_normal_,
+    rand_xavier_normal_like, rand_xavier_uniform, rand_xavier_uniform_, rand_xavier_uniform_like, randn_, randn_like,
+    randu_, randu_like, zeros_, zeros_like,
+)
 from .autograd.functional import backward, grad, hessian, jacobian, value_and_grad  # noqa: E402,F401
 from . import autograd, fusion, graph, nn, optim, utils  # noqa: E402,F401
 from .fusion import fuse  # noqa: E402,F401
-from .graph import capture  # noqa: E402,F401
+from .graph import capture, jit  # noqa: E402,F401
 
 
 def synchronize():

@@ -11,7 +11,7 @@ non-JIT branch of Callable.__call__ (endia/compile/callable.mojo:100-197): repea
 backward(create_graph=True) passes, then detached copies of the results.
 """
 from .. import functional as F
-from .._array import Array
+from .._array import Array, _contiguous_copy
 
 _building_graph = [False]
 
@@ -176,10 +176,10 @@ class Callable:
                 for i in idx:
                     leaves[i].remove_grad()
             outs = nxt
-        # detach by copy (callable.mojo:165-176)
-        final = [F.array(g.to_numpy()) for g in outs]
+        # detach by copy (callable.mojo:165-176), device to device
+        final = [_contiguous_copy(g) for g in outs]
         if self.keep_outs:
-            final = [F.array(value.to_numpy())] + final
+            final = [_contiguous_copy(value)] + final
         if len(final) == 1:
             return final[0]
         return final

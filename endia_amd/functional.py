@@ -106,6 +106,151 @@ def rand_he_normal(shape, fan_in, requires_grad=False):
     return randn(shape, 0.0, float(np.sqrt(2.0 / fan_in)), requires_grad)
 
 
+def linspace(start=0.0, end=1.0, num=50, requires_grad=False):
+    """init_ops.mojo:94-107: start, then `num - 1` additions of the fp32 step (so the last value carries their rounding)."""
+    step = (np.float32(end) - np.float32(start)) / np.float32(num - 1)
+    out, value = np.empty(num, np.float32), np.float32(start)
+    for i in range(num):
+        out[i] = value
+        value = np.float32(value + step)
+    return array(out, requires_grad)
+
+
+def _overwrite(arg, values):
+    """In-place initialisers write through to the buffer of a contiguous array (zeros_ / randu_ / ... : init_ops.mojo:126-265)."""
+    arg.copy_from_numpy(np.asarray(values).reshape(arg.shape()))
+    return arg
+
+
+def fill_(arg, value):
+    """init_ops.mojo:185-193."""
+    if not arg.is_contiguous() or arg.is_complex_:
+        return _overwrite(arg, np.full(arg.shape(), value, np.complex64 if arg.is_complex_ else np.float32))
+    if arg.size():
+        L.call("endia_hip_fill", arg.data_ptr(), arg.size(), float(value))
+    return arg
+
+
+def zeros_(arg):
+    return fill_(arg, 0.0)
+
+
+def ones_(arg):
+    return fill_(arg, 1.0)
+
+
+def randu_(arg, min=0.0, max=1.0):
+    """init_ops.mojo:227-236."""
+    return _overwrite(arg, _rng.uniform(min, max, tuple(arg.shape())).astype(np.float32))
+
+
+def randn_(arg, mean=0.0, std=1.0):
+    """init_ops.mojo:255-264."""
+    return _overwrite(arg, (_rng.standard_normal(tuple(arg.shape())) * std + mean).astype(np.float32))
+
+
+def zeros_like(arg):
+    return zeros(arg.shape(), arg._requires_grad)
+
+
+def ones_like(arg):
+    return ones(arg.shape(), arg._requires_grad)
+
+
+def fill_like(arg, value):
+    return full(arg.shape(), value, arg._requires_grad)
+
+
+def eye_like(arg):
+    """init_ops.mojo:162-182: ones where the last two indices agree."""
+    shape = arg.shape()
+    block = np.eye(shape[-2], shape[-1], dtype=np.float32)
+    return array(np.broadcast_to(block, shape).copy(), arg._requires_grad)
+
+
+def randu_like(arg, min=0.0, max=1.0):
+    return randu(arg.shape(), min, max, arg._requires_grad)
+
+
+def randn_like(arg, mean=0.0, std=1.0):
+    return randn(arg.shape(), mean, std, arg._requires_grad)
+
+
+# the initialisation schemes of init_ops.mojo:285-416: a normal or uniform draw whose scale follows the fan sizes
+def rand_he_normal_(arg, fan_in=1.0):
+    return randn_(arg, 0.0, float(np.sqrt(2.0 / fan_in)))
+
+
+def rand_he_normal_like(arg, fan_in=1.0):
+    return rand_he_normal(arg.shape(), fan_in, arg._requires_grad)
+
+
+def rand_he_uniform(shape, fan_in=1.0, requires_grad=False):
+    limit = float(np.sqrt(6.0 / fan_in))
+    return randu(shape, -limit, limit, requires_grad)
+
+
+def rand_he_uniform_(arg, fan_in=1.0):
+    limit = float(np.sqrt(6.0 / fan_in))
+    return randu_(arg, -limit, limit)
+
+
+def rand_he_uniform_like(arg, fan_in=1.0):
+    return rand_he_uniform(arg.shape(), fan_in, arg._requires_grad)
+
+
+def rand_xavier_normal(shape, fan_in=1.0, fan_out=1.0, requires_grad=False):
+    return randn(shape, 0.0, float(np.sqrt(2.0 / (fan_in + fan_out))), requires_grad)
+
+
+def rand_xavier_normal_(arg, fan_in=1.0, fan_out=1.0):
+    return randn_(arg, 0.0, float(np.sqrt(2.0 / (fan_in + fan_out))))
+
+
+def rand_xavier_normal_like(arg, fan_in=1.0, fan_out=1.0):
+    return rand_xavier_normal(arg.shape(), fan_in, fan_out, arg._requires_grad)
+
+
+def rand_xavier_uniform(shape, fan_in=1.0, fan_out=1.0, requires_grad=False):
+    limit = float(np.sqrt(6.0 / (fan_in + fan_out)))
+    return randu(shape, -limit, limit, requires_grad)
+
+
+def rand_xavier_uniform_(arg, fan_in=1.0, fan_out=1.0):
+    limit = float(np.sqrt(6.0 / (fan_in + fan_out)))
+    return randu_(arg, -limit, limit)
+
+
+def rand_xavier_uniform_like(arg, fan_in=1.0, fan_out=1.0):
+    return rand_xavier_uniform(arg.shape(), fan_in, fan_out, arg._requires_grad)
+
+
+def rand_lecun_normal(shape, fan_in=1.0, requires_grad=False):
+    return randn(shape, 0.0, float(np.sqrt(1.0 / fan_in)), requires_grad)
+
+
+def rand_lecun_normal_(arg, fan_in=1.0):
+    return randn_(arg, 0.0, float(np.sqrt(1.0 / fan_in)))
+
+
+def rand_lecun_normal_like(arg, fan_in=1.0):
+    return rand_lecun_normal(arg.shape(), fan_in, arg._requires_grad)
+
+
+def rand_lecun_uniform(shape, fan_in=1.0, requires_grad=False):
+    limit = float(np.sqrt(3.0 / fan_in))
+    return randu(shape, -limit, limit, requires_grad)
+
+
+def rand_lecun_uniform_(arg, fan_in=1.0):
+    limit = float(np.sqrt(3.0 / fan_in))
+    return randu_(arg, -limit, limit)
+
+
+def rand_lecun_uniform_like(arg, fan_in=1.0):
+    return rand_lecun_uniform(arg.shape(), fan_in, arg._requires_grad)
+
+
 def complex(real, imag=None):
     """complex(real, imag): init_ops.mojo:419-433."""
     r = contiguous(real)

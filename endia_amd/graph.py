@@ -27,6 +27,7 @@ lives on the host refuses to run inside a capture.
 import ctypes
 
 from . import _lib as L
+from ._array import Array, _contiguous_copy
 
 
 class CapturedStep:
@@ -70,3 +71,74 @@ class CapturedStep:
 def capture(fn):
     """Record everything `fn()` enqueues and return a CapturedStep; `fn` must not read device data."""
     return CapturedStep(fn)
+
+
+def _leaves(tree, out):
+    """The arrays of a nest of lists/tuples, left to right."""
+    if isinstance(tree, Array):
+        out.append(tree)
+    elif isinstance(tree, (list, tuple)):
+        for t in tree:
+            _leaves(t, out)
+    elif tree is not None:
+        raise TypeError("jit: arguments and results must be arrays or lists of arrays, not %s" % type(tree).__name__)
+    return out
+
+
+def _rebuild(tree, it):
+    if isinstance(tree, Array):
+        return next(it)
+    if isinstance(tree, (list, tuple)):
+        return type(tree)(_rebuild(t, it) for t in tree)
+    return None
+
+
+class JitCallable:
+    """jit(fn): the call-compatible counterpart of the reference's caching Callable (endia/compile/callable.mojo:60-98,
+    endia/compile/functional.mojo:43-88).
+
+    The reference keeps one set of argument arrays per jitted function, copies each call's inputs into them, runs
+    the cached graph and hands back copies of the results. The same here, with a HIP graph as the cache: the first
+    call with a given list of input shapes runs `fn` once eagerly on private copies of the inputs (which sizes the
+    buffer pool), records a second run into a graph, and from then on a call is: copy the inputs in (device to
+    device), one graph launch, copy the results out. `fn` must be a pure function of its array arguments that
+    enqueues the same kernels on every call and reads no device data on the host (no item(), to_numpy() or host
+    uploads inside); one that does fails at the first call with the library's "not allowed while a step is being
+    captured" error. Inputs of another shape get a graph of their own.
+    """
+
+    def __init__(self, fn):
+        self.fn = fn
+        self._cache = {}
+
+    def __call__(self, *args):
+        if L.capturing:  # a jitted function used inside a captured step is simply part of that step
+            return self.fn(*args)
+        given = _leaves(args, [])
+        key = tuple((tuple(a._shape), a.is_complex_, a._requires_grad) for a in given)
+        entry = self._cache.get(key)
+        if entry is None:
+            held = [_contiguous_copy(a).requires_grad_(a._requires_grad) for a in given]
+            private = _rebuild(args, iter(held))
+            self.fn(*private)
+            step = CapturedStep(lambda: self.fn(*private))
+            entry = self._cache[key] = (held, step, _leaves(step.outputs, []))
+        else:
+            for mine, a in zip(entry[0], given):
+                mine._assign_from(a)
+        held, step, results = entry
+        step.replay()
+        return _rebuild(step.outputs, iter([_contiguous_copy(r) for r in results]))
+
+    def close(self):
+        for _, step, _ in self._cache.values():
+            step.close()
+        self._cache.clear()
+
+
+def jit(fn, compile_with_MAX=False):
+    """nd.jit(fn): see JitCallable. `compile_with_MAX` is accepted for call compatibility and must stay False: there
+    is no MAX engine here (endia/compile/functional.mojo:43-55)."""
+    if compile_with_MAX:
+        raise NotImplementedError("jit: compile_with_MAX=True asks for the MAX engine, which this library does not have")
+    return JitCallable(fn)

@@ -911,3 +911,90 @@ def test_random_expression_graphs_vs_torch(nd):
         for i, (lf, tl) in enumerate(zip(ours, theirs)):
             want = tl.grad.numpy() if tl.grad is not None else np.zeros(lf.shape())
             assert_close(lf.grad().to_numpy().reshape(want.shape), want, tol=5e-4 if second else 1e-4, what=what + " grad of leaf %d" % i)
+
+
+def test_initialisers(nd):
+    """The rest of init_ops.mojo: shapes, the values that are fixed (zeros/ones/eye/fill/linspace), and for the random
+    schemes the scale the fan sizes fix (he: sqrt(2/fan_in), sqrt(6/fan_in); xavier: sqrt(2/(in+out)), sqrt(6/(in+out));
+    lecun: sqrt(1/fan_in), sqrt(3/fan_in); init_ops.mojo:285-416). The draws themselves are time-seeded in the reference
+    and cannot be compared."""
+    base = nd.array(np.arange(24, dtype=np.float32).reshape(2, 3, 4), requires_grad=True)
+    for made, want in ((nd.zeros_like(base), 0.0), (nd.ones_like(base), 1.0), (nd.fill_like(base, 2.5), 2.5)):
+        assert made.shape() == [2, 3, 4] and made.requires_grad()
+        np.testing.assert_array_equal(made.to_numpy(), np.full((2, 3, 4), want, np.float32))
+    np.testing.assert_array_equal(nd.eye_like(base).to_numpy(), np.broadcast_to(np.eye(3, 4, dtype=np.float32), (2, 3, 4)))
+    np.testing.assert_array_equal(nd.linspace(0.0, 1.0, 5).to_numpy(), np.float32([0, 0.25, 0.5, 0.75, 1.0]))
+    assert_close(nd.linspace(-2.0, 7.0, 1000).to_numpy(), np.linspace(-2.0, 7.0, 1000), what="linspace")
+
+    work = nd.array(np.arange(12, dtype=np.float32).reshape(3, 4))
+    before = work.data_ptr()
+    for fn, want in ((nd.ones_, 1.0), (nd.zeros_, 0.0), (lambda a: nd.fill_(a, -3.0), -3.0)):
+        assert fn(work) is work and work.data_ptr() == before
+        np.testing.assert_array_equal(work.to_numpy(), np.full((3, 4), want, np.float32))
+    cz = nd.fill_(nd.complex(nd.ones([2, 2]), nd.ones([2, 2])), 4.0)
+    np.testing.assert_array_equal(cz.to_numpy(), np.full((2, 2), 4.0, np.complex64))
+    with pytest.raises(ValueError):
+        nd.fill_(nd.permute(work, [1, 0]), 1.0)
+
+    nd.seed(5)
+    big = nd.zeros([400, 500])
+    draw = nd.randu_(big, -2.0, 6.0).to_numpy()
+    assert draw.min() >= -2.0 and draw.max() <= 6.0 and abs(draw.mean() - 2.0) < 0.05
+    draw = nd.randn_(big, 1.0, 3.0).to_numpy()
+    assert abs(draw.mean() - 1.0) < 0.05 and abs(draw.std() - 3.0) < 0.05
+    assert nd.randu_like(big).shape() == [400, 500] and nd.randn_like(big).shape() == [400, 500]
+
+    fan_in, fan_out = 50.0, 30.0
+    normal = {"rand_he_normal": (np.sqrt(2 / fan_in), (fan_in,)), "rand_lecun_normal": (np.sqrt(1 / fan_in), (fan_in,)),
+              "rand_xavier_normal": (np.sqrt(2 / (fan_in + fan_out)), (fan_in, fan_out))}
+    uniform = {"rand_he_uniform": (np.sqrt(6 / fan_in), (fan_in,)), "rand_lecun_uniform": (np.sqrt(3 / fan_in), (fan_in,)),
+               "rand_xavier_uniform": (np.sqrt(6 / (fan_in + fan_out)), (fan_in, fan_out))}
+    for name, (scale, fans) in list(normal.items()) + list(uniform.items()):
+        for draw in (getattr(nd, name)([400, 500], *fans).to_numpy(), getattr(nd, name + "_like")(big, *fans).to_numpy(),
+                     getattr(nd, name + "_")(big, *fans).to_numpy()):
+            assert draw.shape == (400, 500) and abs(draw.mean()) < 0.02 * scale * 3
+            if name in normal:
+                assert abs(draw.std() / scale - 1.0) < 0.02, name
+            else:  # uniform on (-limit, limit): bounded, and std = limit / sqrt(3)
+                assert np.abs(draw).max() <= scale and abs(draw.std() * np.sqrt(3) / scale - 1.0) < 0.02, name
+
+
+def test_jit_follows_the_eager_callable(nd):
+    """nd.jit over a function and over value_and_grad(function) (the reference's examples/benchmarks use both:
+    endia/compile/functional.mojo:43-88): every call must return what the eager callable returns for the same inputs,
+    bit for bit, on fresh arrays, also after the inputs change and for a second input shape; results of earlier
+    calls stay what they were."""
+    rng = np.random.default_rng(77)
+
+    def foo(args):
+        h = nd.tanh(nd.matmul(args[0], args[1]) + args[2])
+        return nd.sum(h * h)
+
+    eager = nd.value_and_grad(foo)
+    fast = nd.jit(nd.value_and_grad(foo), compile_with_MAX=False)
+    plain = nd.jit(foo)
+    kept = []
+    for shape in ((16, 24, 8), (16, 24, 8), (5, 7, 3), (16, 24, 8)):
+        m, k, n = shape
+        args = [nd.array(rng.standard_normal(s).astype(np.float32)) for s in ((m, k), (k, n), (n,))]
+        want, got = eager(args), fast(args)
+        assert len(got) == 4
+        for w, g in zip(want, got):
+            np.testing.assert_array_equal(g.to_numpy(), w.to_numpy())
+        np.testing.assert_array_equal(plain(args).to_numpy(), want[0].to_numpy())
+        kept.append((got, [w.to_numpy() for w in want]))
+    for got, want in kept:  # a later call does not write into an earlier call's results
+        for g, w in zip(got, want):
+            np.testing.assert_array_equal(g.to_numpy(), w)
+    assert len(fast._cache) == 2
+
+    def reads_the_device(args):
+        return nd.sum(args[0]) * float(args[0].item())
+
+    with pytest.raises(RuntimeError, match="captured"):
+        nd.jit(reads_the_device)([nd.ones([4])])
+    nd.sum(nd.ones([4])).item()  # the library is usable after the failed capture
+    with pytest.raises(NotImplementedError):
+        nd.jit(foo, compile_with_MAX=True)
+    fast.close()
+    plain.close()
