@@ -263,6 +263,122 @@ __device__ __forceinline__ void gemm_tile(const GemmArgs& p, int block, int nblo
     }
 }
 
+// The 256 x 256 tile: one work-group per CU, one wave per SIMD, each wave 128 x 128 = 4 x 4 MFMA blocks (256 accumulator
+// registers per lane). With nobody else on the SIMD to fill a wave's stalls, the order of instructions is the
+// schedule, and whatever is not an MFMA is hidden only if it sits BETWEEN two MFMAs (the matrix pipe is busy for 64
+// cycles per instruction; what follows in program order issues meanwhile). So a K tile is 16 steps of 16 MFMAs, cut
+// into quads, and in front of every quad goes one small piece of the other work, fenced by scheduling barriers so the
+// compiler keeps it there:
+//   * LDS holds two stages; steps 0-11 read, block by block, the fragments of the next group of four steps from the
+//     current stage (one group ahead of their use), steps 12-15 the first fragments of the next tile from the other
+//     stage, behind the tile's only barrier (at step 12 everybody has written its share of that stage and has read
+//     the last of this one);
+//   * steps 0-11 also move the next tile, one 16-byte piece per lane at a time, from registers to the other stage and
+//     request the same piece of the tile after it from memory, which then has a whole K tile (~7 us) to arrive.
+// Tiles past the end of K load as zeros (descriptor bounds) into a stage nobody reads.
+template <bool A_KMAJOR, bool B_KMAJOR, int EPI>
+__device__ __forceinline__ void gemm_tile256(const GemmArgs& p, int block, int nblocks, int64_t bz, float* __restrict__ smem) {
+  constexpr int F = 4, BM = 256, BN = 256;
+  using LA = MatrixTileLoader<A_KMAJOR, BM, NTHREADS>;
+  using LB = MatrixTileLoader<B_KMAJOR, BN, NTHREADS>;
+  constexpr int SA = TileShape<A_KMAJOR, BM>::FLOATS, STAGE = SA + TileShape<B_KMAJOR, BN>::FLOATS;
+  static_assert(BK == 32 && LA::PASSES == 8 && LB::PASSES == 8, "the step plan below is written for these");
+
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int wm = wave >> 1, wn = wave & 1, l32 = lane & 31, h = lane >> 5;
+  int tm, tn;
+  tile_of_block(block, nblocks, p.tiles_m, p.tiles_n, tm, tn);
+  const int m0 = tm * BM, n0 = tn * BN;
+  float* __restrict__ C = p.C + bz * p.sC;
+  const float* __restrict__ aux_in = p.aux_in ? p.aux_in + bz * p.sC : nullptr;
+  float* __restrict__ aux_out = p.aux_out ? p.aux_out + bz * p.sC : nullptr;
+  const int K = p.K;
+  LA la;
+  LB lb;
+  la.init(p.A + bz * p.sA, p.lda, m0, p.M, K, tid);
+  lb.init(p.B + bz * p.sB, p.ldb, n0, p.N, K, tid);
+
+  floatx16 acc[F][F];
+  zero_acc<F, F>(acc);
+  const int a_row = wm * 128 + l32, b_col = wn * 128 + l32;
+
+  la.load(K);
+  lb.load(K);
+  la.store(smem);
+  lb.store(smem + SA);
+  la.advance();
+  lb.advance();
+  la.load(K - BK);
+  lb.load(K - BK);
+  __syncthreads();
+  float af[2][F][4], bf[2][F][4];
+#pragma unroll
+  for (int f = 0; f < F; ++f) {
+    load_fragment_block<A_KMAJOR, BM>(smem, a_row + 32 * f, h, 0, af[0][f]);
+    load_fragment_block<B_KMAJOR, BN>(smem + SA, b_col + 32 * f, h, 0, bf[0][f]);
+  }
+  const int T = (K + BK - 1) / BK;
+  for (int t = 0; t < T; ++t) {
+    const float* Ac = smem + (t & 1) * STAGE;
+    float* An = smem + ((t + 1) & 1) * STAGE;
+    la.advance();  // the loaders now point at tile t + 2
+    lb.advance();
+    const int k_left = K - (t + 2) * BK;
+    const __amdgpu_buffer_rsrc_t rsa = la.rsrc(), rsb = lb.rsrc();
+#pragma unroll
+    for (int s = 0; s < 16; ++s) {
+      const int j = s >> 2, i = s & 3, cur = j & 1, nxt = cur ^ 1;
+      if (s == 12) __syncthreads();
+      const float* Sf = s < 12 ? Ac : An;
+      const int jn = s < 12 ? j + 1 : 0;
+      auto quad = [&](int fm) {
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int fn = 0; fn < F; ++fn)
+          acc[fm][fn] = __builtin_amdgcn_mfma_f32_32x32x2f32(af[cur][fm][i], bf[cur][fn][i], acc[fm][fn], 0, 0, 0);
+        __builtin_amdgcn_sched_barrier(0);
+      };
+      load_fragment_block<A_KMAJOR, BM>(Sf, a_row + 32 * i, h, jn, af[nxt][i]);
+      quad(0);
+      load_fragment_block<B_KMAJOR, BN>(Sf + SA, b_col + 32 * i, h, jn, bf[nxt][i]);
+      quad(1);
+      if (s < 8) {
+        la.store_pass(An, s);
+        la.load_pass(s, k_left, rsa);
+      } else if (s < 12) {
+        lb.store_pass(An + SA, s - 4);
+        lb.load_pass(s - 4, k_left, rsb);
+      }
+      quad(2);
+      if (s < 4) {
+        lb.store_pass(An + SA, s);
+        lb.load_pass(s, k_left, rsb);
+      }
+      quad(3);
+    }
+  }
+
+#pragma unroll
+  for (int fm = 0; fm < F; ++fm)
+#pragma unroll
+    for (int fn = 0; fn < F; ++fn) {
+      const int col = n0 + wn * 128 + fn * 32 + l32;
+      if (col >= p.N) continue;
+#pragma unroll
+      for (int v = 0; v < 16; ++v) {
+        const int row = m0 + wm * 128 + fm * 32 + acc_row(v, h);
+        if (row >= p.M) continue;
+        epilogue_store<EPI>(p, C, aux_in, aux_out, row, col, acc[fm][fn][v]);
+      }
+    }
+}
+
+template <bool A_KMAJOR, bool B_KMAJOR, int EPI>
+__global__ __launch_bounds__(NTHREADS, 1) void sgemm_mfma256_kernel(GemmArgs p) {
+  extern __shared__ __attribute__((aligned(16))) float smem256[];
+  gemm_tile256<A_KMAJOR, B_KMAJOR, EPI>(p, blockIdx.x, gridDim.x, blockIdx.y, smem256);
+}
+
 template <bool A_KMAJOR, bool B_KMAJOR, int EPI, int F, bool SHORTK = false>
 __global__ __launch_bounds__(NTHREADS, 4) void sgemm_mfma_kernel(GemmArgs p) {
   __shared__ __attribute__((aligned(16))) float As[TileShape<A_KMAJOR, 64 * F>::FLOATS];
@@ -404,6 +520,19 @@ void launch_mfma(const GemmArgs& p, int transA, int transB, dim3 grid, hipStream
   else hipLaunchKernelGGL((sgemm_mfma_kernel<false, false, EPI, F, SHORTK>), grid, dim3(NTHREADS), 0, s, p);
 }
 
+template <bool AK, bool BKM, int EPI>
+int32_t launch_one256(const GemmArgs& p, dim3 grid, hipStream_t s) {
+  constexpr size_t lds = 2 * (size_t)(TileShape<AK, 256>::FLOATS + TileShape<BKM, 256>::FLOATS) * sizeof(float);
+  static bool allowed = false;  // more than 64 KiB of LDS has to be asked for, once per kernel
+  if (!allowed) {
+    ENDIA_HIP_CALL(hipFuncSetAttribute(reinterpret_cast<const void*>(&sgemm_mfma256_kernel<AK, BKM, EPI>),
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+    allowed = true;
+  }
+  hipLaunchKernelGGL((sgemm_mfma256_kernel<AK, BKM, EPI>), grid, dim3(NTHREADS), lds, s, p);
+  return ENDIA_HIP_OK;
+}
+
 template <int F, bool SHORTK = false>
 void launch_mfma_epi(const GemmArgs& p, int epi, int transA, int transB, dim3 grid, hipStream_t s) {
   switch (epi) {
@@ -436,6 +565,7 @@ struct GemmTiming {
   double flops = 0.0;
 };
 GemmTiming g_timing;
+int g_forced_tile = 0;  // endia_hip_gemm_force_tile
 }  // namespace
 
 namespace endia {
@@ -499,7 +629,16 @@ int32_t sgemm_impl(int transA, int transB, int64_t M, int64_t N, int64_t K, cons
     const double per_cu = (double)t128 / (double)cus;
     const double score128 = balance(t128) * (per_cu >= 3.0 ? 1.0 : (per_cu >= 2.0 ? 0.95 : 0.80));
     const double score64 = balance(t64) * 0.92;
-    const int F = (fits128 && score128 >= score64) ? 2 : 1;
+    int F = (fits128 && score128 >= score64) ? 2 : 1;
+    // 256 x 256 tiles, one per CU at a time: when they fill every round over the CUs (4096^2 outputs are 256 of them)
+    const int64_t t256 = ceil_div64(M, 256) * ceil_div64(N, 256) * batch;
+    const bool fits256 = (double)(ceil_div64(M, 256) * 256) * (double)(ceil_div64(N, 256) * 256) <= 1.1 * (double)M * (double)N;
+    // Built for the weight-gradient form only (A stored K x M, B stored K x N, plain or accumulating epilogue): with an
+    // operand whose K index is the contiguous one it measured no faster than the 128 x 128 tile (NN) or slower (NT).
+    const bool has256 = transA && !transB && epi == ENDIA_EPI_NONE && !colsum;
+    if (g_forced_tile == 64) F = 1;
+    else if (g_forced_tile == 128) F = 2;
+    if (has256 && (g_forced_tile == 256 || (g_forced_tile == 0 && fits256 && t256 >= cus && balance(t256) >= 0.9 && K >= 256))) F = 4;
     p.tiles_m = (int)ceil_div64(M, 64 * F);
     p.tiles_n = (int)ceil_div64(N, 64 * F);
     const int64_t tiles = (int64_t)p.tiles_m * p.tiles_n;
@@ -567,7 +706,10 @@ int32_t sgemm_impl(int transA, int transB, int64_t M, int64_t N, int64_t K, cons
       }
       ENDIA_HIP_CALL(hipEventRecord(g_timing.start[g_timing.used], s));
     }
-    if (F == 2) launch_mfma_epi<2>(p, epi, transA, transB, grid, s);
+    if (F == 4) {
+      int32_t rc = launch_one256<false, false, ENDIA_EPI_NONE>(p, grid, s);
+      if (rc) return rc;
+    } else if (F == 2) launch_mfma_epi<2>(p, epi, transA, transB, grid, s);
     else if (K <= 4 * BK && splits == 1) launch_mfma_epi<1, true>(p, epi, transA, transB, grid, s);
     else launch_mfma_epi<1>(p, epi, transA, transB, grid, s);
     if (timed) {
@@ -675,6 +817,12 @@ extern "C" int32_t endia_hip_sgemm(int32_t transA, int32_t transB, int64_t M, in
   ENDIA_REQUIRE_INIT();
   return endia::sgemm_impl(transA, transB, M, N, K, A, lda, B, ldb, C, ldc, batch, strideA, strideB,
                            strideC, epilogue, act, bias, aux_in, aux_out);
+}
+
+extern "C" int32_t endia_hip_gemm_force_tile(int32_t tile) {
+  ENDIA_CHECK_ARG(tile == 0 || tile == 64 || tile == 128 || tile == 256, "endia_hip_gemm_force_tile: tile %d is not one of 0, 64, 128, 256", tile);
+  g_forced_tile = tile;
+  return ENDIA_HIP_OK;
 }
 
 extern "C" int32_t endia_hip_gemm_timing_begin(void) {

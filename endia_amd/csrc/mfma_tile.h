@@ -73,6 +73,19 @@ __device__ __forceinline__ void load_fragments(const float* __restrict__ As, con
   }
 }
 
+// The fragment of ONE 32-row block for step group j (the four steps 4j .. 4j + 3); row: this lane's row of the tile.
+template <bool KMAJOR, int BMN>
+__device__ __forceinline__ void load_fragment_block(const float* __restrict__ S, int row, int h, int j, float (&f)[4]) {
+  constexpr int LD = TileShape<KMAJOR, BMN>::LD;
+  if (KMAJOR) {
+    float4 t = *reinterpret_cast<const float4*>(&S[row * LD + 8 * j + 4 * h]);
+    f[0] = t.x; f[1] = t.y; f[2] = t.z; f[3] = t.w;
+  } else {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) f[i] = S[(8 * j + 4 * h + i) * LD + row];
+  }
+}
+
 template <bool AK, bool BKM, int FM, int FN, int BM, int BN>
 __device__ __forceinline__ void compute_ktile(const float* __restrict__ As, const float* __restrict__ Bs, int a_row,
                                               int b_col, int h, floatx16 (&acc)[FM][FN]) {
@@ -180,6 +193,16 @@ struct MatrixTileLoader {
   __device__ __forceinline__ void store_from(float* lds, const float4 (&src)[PASSES]) {
 #pragma unroll
     for (int i = 0; i < PASSES; ++i) *reinterpret_cast<float4*>(&lds[lds_off + i * ROWS_PER_PASS * LD]) = src[i];
+  }
+  // One pass at a time, for loops that spread a tile's loads and LDS stores between their MFMAs.
+  __device__ __forceinline__ __amdgpu_buffer_rsrc_t rsrc() const { return make_rsrc(base, records); }
+  __device__ __forceinline__ void load_pass(int i, int k_left, __amdgpu_buffer_rsrc_t rs) {
+    uint32_t o = voff[i];
+    if (KMAJOR) o = (c < k_left) ? o : OOB_OFFSET;
+    reg[i] = buffer_load_f4(rs, o);
+  }
+  __device__ __forceinline__ void store_pass(float* lds, int i) {
+    *reinterpret_cast<float4*>(&lds[lds_off + i * ROWS_PER_PASS * LD]) = reg[i];
   }
   __device__ __forceinline__ void advance() {
     base = reinterpret_cast<const float*>(reinterpret_cast<const char*>(base) + step);

@@ -145,6 +145,13 @@ ENDIA_API int32_t endia_hip_graph_destroy(int64_t handle);
 ENDIA_API int32_t endia_hip_gemm_timing_begin(void);
 ENDIA_API int32_t endia_hip_gemm_timing_end(int64_t* launches, double* total_ms, double* total_flops);
 
+/* Tile choice of the fp32 matrix-core kernels behind endia_hip_sgemm (and everything built on it). No counterpart in the
+ * reference: a hook for tests and tuning. tile = 0 (the default) lets every call choose by shape; 64, 128 or 256
+ * makes every later call that runs on the matrix cores use that tile where a kernel for it exists (256 x 256: only
+ * for transA = 1, transB = 0 with the plain epilogue; other calls keep the automatic choice). Results do not depend on the tile
+ * beyond the order of the additions along K. Process-wide, not thread-safe against concurrent sgemm calls. */
+ENDIA_API int32_t endia_hip_gemm_force_tile(int32_t tile);
+
 /* ---- strided gather copy: execute_copy_raw / contiguous (functional/_utils.mojo:79-205).
  *      dst is contiguous row-major of `shape`; src element (i0..i_{r-1}) is at
  *      src[offset + sum i_d*stride_d]; stride 0 broadcasts. ndim <= 8. is_complex copies pairs. */

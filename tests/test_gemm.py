@@ -347,3 +347,45 @@ def test_sgemm_random_shapes_and_flags(dev):
             s = dev.get(dsum, (N,))
             assert np.abs(s - B.astype(np.float64).sum(0)).max() <= 2e-5 * max(1.0, np.sqrt(K)) * max(1.0, float(np.abs(B).max()) if K else 1.0), what + " (column sums)"
         dev.release()
+
+
+@pytest.mark.parametrize("M,N,K", [(256, 256, 32), (256, 512, 64), (300, 520, 70), (516, 260, 1000), (1024, 768, 4100), (260, 1028, 36),
+                                   (128, 64, 512)])
+def test_sgemm_every_tile_forced(dev, M, N, K):
+    """endia_hip_gemm_force_tile: the weight-gradient form (A stored K x M, B stored K x N) through the 64, 128 and 256
+    tiles on shapes with ragged edges in M, N and K (the 256 x 256 tile is otherwise only chosen for products that fill
+    every CU with one): every tile against the oracle and float64, plain and accumulating, a padded C, a batch; the other
+    forms keep working while 256 is forced (they have no such kernel and fall back to the automatic choice)."""
+    rng = np.random.default_rng(M + 3 * N + 7 * K)
+    A = rng.standard_normal((K, M)).astype(np.float32)
+    B = (rng.standard_normal((K, N)) / np.sqrt(K)).astype(np.float32)
+    ref = A.T.astype(np.float64) @ B.astype(np.float64)
+    want = R.matmul(np.ascontiguousarray(A.T), B)
+    C0 = rng.standard_normal((M, N)).astype(np.float32)
+    try:
+        for tile in (64, 128, 256):
+            dev.call("endia_hip_gemm_force_tile", tile)
+            got = run_sgemm(dev, A, B, 1, 0, M, N, K)
+            assert_close(got, want, what="tile %d vs oracle" % tile)
+            assert_close(got, ref, what="tile %d vs float64" % tile)
+            np.testing.assert_array_equal(run_sgemm(dev, A, B, 1, 0, M, N, K), got)
+            assert_close(run_sgemm(dev, A, B, 1, 0, M, N, K, L.EPI_NONE | L.GEMM_ACCUMULATE, C0=C0), C0 + ref, what="tile %d accumulate" % tile)
+            ldc = N + 12
+            wide = rng.standard_normal((M, ldc)).astype(np.float32)
+            dA, dB, dC = dev.put(A), dev.put(B), dev.put(wide)
+            dev.call("endia_hip_sgemm", 1, 0, M, N, K, dA, M, dB, N, dC, ldc, 1, 0, 0, 0, L.EPI_NONE, L.OP_IDENTITY, None, None, None)
+            out = dev.get(dC, (M, ldc))
+            assert_close(out[:, :N], ref, what="tile %d padded C" % tile)
+            np.testing.assert_array_equal(out[:, N:], wide[:, N:])
+        # a batch of two through the 256 tile (second entry: the operands swapped in sign), and the other forms untouched
+        A2, B2 = np.stack([A, -A]), np.stack([B, B])
+        dA, dB, dC = dev.put(A2), dev.put(B2), dev.put(np.zeros((2, M, N), np.float32))
+        dev.call("endia_hip_sgemm", 1, 0, M, N, K, dA, M, dB, N, dC, N, 2, K * M, K * N, M * N, L.EPI_NONE, L.OP_IDENTITY, None, None, None)
+        out = dev.get(dC, (2, M, N))
+        assert_close(out[0], ref, what="batch entry 0")
+        assert_close(out[1], -ref, what="batch entry 1")
+        At = np.ascontiguousarray(A.T)
+        assert_close(run_sgemm(dev, At, B, 0, 0, M, N, K), ref, what="NN while 256 is forced")
+    finally:
+        dev.call("endia_hip_gemm_force_tile", 0)
+    assert L.lib().endia_hip_gemm_force_tile(96) == L.ERR_INVALID
