@@ -635,7 +635,7 @@ int32_t sgemm_impl(int transA, int transB, int64_t M, int64_t N, int64_t K, cons
     const bool fits256 = (double)(ceil_div64(M, 256) * 256) * (double)(ceil_div64(N, 256) * 256) <= 1.1 * (double)M * (double)N;
     // Built for the weight-gradient form only (A stored K x M, B stored K x N, plain or accumulating epilogue): with an
     // operand whose K index is the contiguous one it measured no faster than the 128 x 128 tile (NN) or slower (NT).
-    const bool has256 = transA && !transB && epi == ENDIA_EPI_NONE && !colsum;
+    const bool has256 = transA && !transB && epi == ENDIA_EPI_NONE && !(colsum && K * N <= (1ll << 20));  // (column sums of a small B ride in the launch)
     if (g_forced_tile == 64) F = 1;
     else if (g_forced_tile == 128) F = 2;
     if (has256 && (g_forced_tile == 256 || (g_forced_tile == 0 && fits256 && t256 >= cus && balance(t256) >= 0.9 && K >= 256))) F = 4;

@@ -350,7 +350,7 @@ def test_sgemm_random_shapes_and_flags(dev):
 
 
 @pytest.mark.parametrize("M,N,K", [(256, 256, 32), (256, 512, 64), (300, 520, 70), (516, 260, 1000), (1024, 768, 4100), (260, 1028, 36),
-                                   (128, 64, 512)])
+                                   (128, 64, 512), (512, 1024, 1100)])
 def test_sgemm_every_tile_forced(dev, M, N, K):
     """endia_hip_gemm_force_tile: the weight-gradient form (A stored K x M, B stored K x N) through the 64, 128 and 256
     tiles on shapes with ragged edges in M, N and K (the 256 x 256 tile is otherwise only chosen for products that fill
@@ -386,6 +386,12 @@ def test_sgemm_every_tile_forced(dev, M, N, K):
         assert_close(out[1], -ref, what="batch entry 1")
         At = np.ascontiguousarray(A.T)
         assert_close(run_sgemm(dev, At, B, 0, 0, M, N, K), ref, what="NN while 256 is forced")
+        # the column sums of B from the same call (the bias gradient beside the weight gradient), small and large B
+        dC, dsum = dev.put(np.full((M, N), np.nan, np.float32)), dev.put(np.full(N, np.nan, np.float32))
+        dev.call("endia_hip_sgemm", 1, 0, M, N, K, dev.put(A), M, dev.put(B), N, dC, N, 1, 0, 0, 0, L.EPI_NONE | L.GEMM_COLSUM_B,
+                 L.OP_IDENTITY, None, None, dsum)
+        assert_close(dev.get(dC, (M, N)), ref, what="C beside the column sums")
+        assert_close(dev.get(dsum, (N,)), B.astype(np.float64).sum(0), tol=1e-5, what="column sums")
     finally:
         dev.call("endia_hip_gemm_force_tile", 0)
     assert L.lib().endia_hip_gemm_force_tile(96) == L.ERR_INVALID
