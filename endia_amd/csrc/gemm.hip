@@ -26,6 +26,7 @@
 
 #include <stdlib.h>
 
+#include <type_traits>
 #include <vector>
 
 namespace {
@@ -317,19 +318,47 @@ __device__ __forceinline__ void gemm_tile256(const GemmArgs& p, int block, int n
     load_fragment_block<A_KMAJOR, BM>(smem, a_row + 32 * f, h, 0, af[0][f]);
     load_fragment_block<B_KMAJOR, BN>(smem + SA, b_col + 32 * f, h, 0, bf[0][f]);
   }
-  const int T = (K + BK - 1) / BK;
-  for (int t = 0; t < T; ++t) {
-    const float* Ac = smem + (t & 1) * STAGE;
-    float* An = smem + ((t + 1) & 1) * STAGE;
-    la.advance();  // the loaders now point at tile t + 2
-    lb.advance();
-    const int k_left = K - (t + 2) * BK;
-    const __amdgpu_buffer_rsrc_t rsa = la.rsrc(), rsb = lb.rsrc();
+  // Loop state that changes from tile to tile lives in scalar registers: operand base pointers and the bytes left in
+  // their descriptors (32-bit: the host takes this tile only for operands below 2 GiB). A vector ALU instruction
+  // between two MFMAs of a lone wave is not hidden the way an LDS or memory instruction is (a select per load cost
+  // 4 % of the kernel), so there is none: LDS addresses are loop constants because the loop body is written out for
+  // both stages, and the K tail is handled once, when it comes, by rewriting the lanes' offsets.
+  const char* base_a = reinterpret_cast<const char*>(la.base);
+  const char* base_b = reinterpret_cast<const char*>(lb.base);
+  int rec_a = (int)(la.records < 0 ? 0 : (la.records > 0x7FFFFFF0ll ? 0x7FFFFFF0ll : la.records));
+  int rec_b = (int)(lb.records < 0 ? 0 : (lb.records > 0x7FFFFFF0ll ? 0x7FFFFFF0ll : lb.records));
+  const int step_a = (int)la.step, step_b = (int)lb.step;
+  int k_left = K - BK;  // reduction elements from the tile the loaders point at to the end
+  // Per stage and operand, the lane's LDS position for fragment reads and for staging stores, each in a register of
+  // its own (the empty asm keeps the compiler from deriving one from another with an addition inside the loop);
+  // everything else in an LDS address is a constant within reach of the instruction's 64 KiB offset field.
+  int fa_at[2], fb_at[2], sa_at[2], sb_at[2];
+#pragma unroll
+  for (int st = 0; st < 2; ++st) {
+    fa_at[st] = st * STAGE + fragment_lane_offset<A_KMAJOR, BM>(a_row, h);
+    fb_at[st] = st * STAGE + SA + fragment_lane_offset<B_KMAJOR, BN>(b_col, h);
+    sa_at[st] = st * STAGE + la.lds_off;
+    sb_at[st] = st * STAGE + SA + lb.lds_off;
+    asm volatile("" : "+v"(fa_at[st]), "+v"(fb_at[st]), "+v"(sa_at[st]), "+v"(sb_at[st]));
+  }
+  auto tile_body = [&](auto stage) {
+    constexpr int ST = decltype(stage)::value;
+    base_a += step_a;  // the tile after the next one
+    base_b += step_b;
+    rec_a = rec_a > step_a ? rec_a - step_a : 0;
+    rec_b = rec_b > step_b ? rec_b - step_b : 0;
+    k_left -= BK;
+    if (k_left < BK) {
+      la.mask_tail(k_left);
+      lb.mask_tail(k_left);
+    }
+    const __amdgpu_buffer_rsrc_t rsa = __builtin_amdgcn_make_buffer_rsrc(const_cast<char*>(base_a), 0, rec_a, 0x00020000);
+    const __amdgpu_buffer_rsrc_t rsb = __builtin_amdgcn_make_buffer_rsrc(const_cast<char*>(base_b), 0, rec_b, 0x00020000);
 #pragma unroll
     for (int s = 0; s < 16; ++s) {
       const int j = s >> 2, i = s & 3, cur = j & 1, nxt = cur ^ 1;
       if (s == 12) __syncthreads();
-      const float* Sf = s < 12 ? Ac : An;
+      const int fs = s < 12 ? ST : ST ^ 1;  // stage the fragments are read from
       const int jn = s < 12 ? j + 1 : 0;
       auto quad = [&](int fm) {
         __builtin_amdgcn_sched_barrier(0);
@@ -338,24 +367,30 @@ __device__ __forceinline__ void gemm_tile256(const GemmArgs& p, int block, int n
           acc[fm][fn] = __builtin_amdgcn_mfma_f32_32x32x2f32(af[cur][fm][i], bf[cur][fn][i], acc[fm][fn], 0, 0, 0);
         __builtin_amdgcn_sched_barrier(0);
       };
-      load_fragment_block<A_KMAJOR, BM>(Sf, a_row + 32 * i, h, jn, af[nxt][i]);
+      load_fragment_at<A_KMAJOR, BM>(smem, fa_at[fs], i, jn, af[nxt][i]);
       quad(0);
-      load_fragment_block<B_KMAJOR, BN>(Sf + SA, b_col + 32 * i, h, jn, bf[nxt][i]);
+      load_fragment_at<B_KMAJOR, BN>(smem, fb_at[fs], i, jn, bf[nxt][i]);
       quad(1);
       if (s < 8) {
-        la.store_pass(An, s);
-        la.load_pass(s, k_left, rsa);
+        la.store_pass_at(smem, sa_at[ST ^ 1], s);
+        la.load_pass(s, rsa);
       } else if (s < 12) {
-        lb.store_pass(An + SA, s - 4);
-        lb.load_pass(s - 4, k_left, rsb);
+        lb.store_pass_at(smem, sb_at[ST ^ 1], s - 4);
+        lb.load_pass(s - 4, rsb);
       }
       quad(2);
       if (s < 4) {
-        lb.store_pass(An + SA, s);
-        lb.load_pass(s, k_left, rsb);
+        lb.store_pass_at(smem, sb_at[ST ^ 1], s);
+        lb.load_pass(s, rsb);
       }
       quad(3);
     }
+  };
+  // two K tiles per trip, one per LDS stage; an odd tile count runs one more tile of zeros
+  const int T = (K + BK - 1) / BK;
+  for (int t = 0; t < T; t += 2) {
+    tile_body(std::integral_constant<int, 0>());
+    tile_body(std::integral_constant<int, 1>());
   }
 
 #pragma unroll
@@ -533,6 +568,24 @@ int32_t launch_one256(const GemmArgs& p, dim3 grid, hipStream_t s) {
   return ENDIA_HIP_OK;
 }
 
+template <int EPI>
+int32_t launch_mfma256(const GemmArgs& p, int transA, int transB, dim3 grid, hipStream_t s) {
+  const bool ak = !transA, bk = transB != 0;
+  if (ak && bk) return launch_one256<true, true, EPI>(p, grid, s);
+  if (ak && !bk) return launch_one256<true, false, EPI>(p, grid, s);
+  if (!ak && bk) return launch_one256<false, true, EPI>(p, grid, s);
+  return launch_one256<false, false, EPI>(p, grid, s);
+}
+
+int32_t launch_mfma256_epi(const GemmArgs& p, int epi, int transA, int transB, dim3 grid, hipStream_t s) {
+  switch (epi) {
+    case ENDIA_EPI_NONE: return launch_mfma256<ENDIA_EPI_NONE>(p, transA, transB, grid, s);
+    case ENDIA_EPI_BIAS: return launch_mfma256<ENDIA_EPI_BIAS>(p, transA, transB, grid, s);
+    case ENDIA_EPI_BIAS_ACT: return launch_mfma256<ENDIA_EPI_BIAS_ACT>(p, transA, transB, grid, s);
+    default: return launch_mfma256<ENDIA_EPI_ACT_GRAD>(p, transA, transB, grid, s);
+  }
+}
+
 template <int F, bool SHORTK = false>
 void launch_mfma_epi(const GemmArgs& p, int epi, int transA, int transB, dim3 grid, hipStream_t s) {
   switch (epi) {
@@ -633,9 +686,8 @@ int32_t sgemm_impl(int transA, int transB, int64_t M, int64_t N, int64_t K, cons
     // 256 x 256 tiles, one per CU at a time: when they fill every round over the CUs (4096^2 outputs are 256 of them)
     const int64_t t256 = ceil_div64(M, 256) * ceil_div64(N, 256) * batch;
     const bool fits256 = (double)(ceil_div64(M, 256) * 256) * (double)(ceil_div64(N, 256) * 256) <= 1.1 * (double)M * (double)N;
-    // Built for the weight-gradient form only (A stored K x M, B stored K x N, plain or accumulating epilogue): with an
-    // operand whose K index is the contiguous one it measured no faster than the 128 x 128 tile (NN) or slower (NT).
-    const bool has256 = transA && !transB && epi == ENDIA_EPI_NONE && !(colsum && K * N <= (1ll << 20));  // (column sums of a small B ride in the launch)
+    // (its descriptors count bytes in 32 bits; the column sums of a small B ride in the launch of the other kernels)
+    const bool has256 = !(colsum && K * N <= (1ll << 20)) && (transA ? K : M) * lda < (1ll << 29) && (transB ? N : K) * ldb < (1ll << 29);
     if (g_forced_tile == 64) F = 1;
     else if (g_forced_tile == 128) F = 2;
     if (has256 && (g_forced_tile == 256 || (g_forced_tile == 0 && fits256 && t256 >= cus && balance(t256) >= 0.9 && K >= 256))) F = 4;
@@ -707,7 +759,7 @@ int32_t sgemm_impl(int transA, int transB, int64_t M, int64_t N, int64_t K, cons
       ENDIA_HIP_CALL(hipEventRecord(g_timing.start[g_timing.used], s));
     }
     if (F == 4) {
-      int32_t rc = launch_one256<false, false, ENDIA_EPI_NONE>(p, grid, s);
+      int32_t rc = launch_mfma256_epi(p, epi, transA, transB, grid, s);
       if (rc) return rc;
     } else if (F == 2) launch_mfma_epi<2>(p, epi, transA, transB, grid, s);
     else if (K <= 4 * BK && splits == 1) launch_mfma_epi<1, true>(p, epi, transA, transB, grid, s);

@@ -86,6 +86,25 @@ __device__ __forceinline__ void load_fragment_block(const float* __restrict__ S,
   }
 }
 
+// The same with the lane's part of the address already in `at` (its row and half-wave, in floats from `S`), so that
+// block f and step group j only add constants that fit the instruction's offset field.
+template <bool KMAJOR, int BMN>
+__device__ __forceinline__ int fragment_lane_offset(int row, int h) {
+  constexpr int LD = TileShape<KMAJOR, BMN>::LD;
+  return KMAJOR ? row * LD + 4 * h : 4 * h * LD + row;
+}
+template <bool KMAJOR, int BMN>
+__device__ __forceinline__ void load_fragment_at(const float* __restrict__ S, int at, int f, int j, float (&out)[4]) {
+  constexpr int LD = TileShape<KMAJOR, BMN>::LD;
+  if (KMAJOR) {
+    float4 t = *reinterpret_cast<const float4*>(&S[at + 32 * f * LD + 8 * j]);
+    out[0] = t.x; out[1] = t.y; out[2] = t.z; out[3] = t.w;
+  } else {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) out[i] = S[at + (8 * j + i) * LD + 32 * f];
+  }
+}
+
 template <bool AK, bool BKM, int FM, int FN, int BM, int BN>
 __device__ __forceinline__ void compute_ktile(const float* __restrict__ As, const float* __restrict__ Bs, int a_row,
                                               int b_col, int h, floatx16 (&acc)[FM][FN]) {
@@ -195,14 +214,21 @@ struct MatrixTileLoader {
     for (int i = 0; i < PASSES; ++i) *reinterpret_cast<float4*>(&lds[lds_off + i * ROWS_PER_PASS * LD]) = src[i];
   }
   // One pass at a time, for loops that spread a tile's loads and LDS stores between their MFMAs.
-  __device__ __forceinline__ __amdgpu_buffer_rsrc_t rsrc() const { return make_rsrc(base, records); }
-  __device__ __forceinline__ void load_pass(int i, int k_left, __amdgpu_buffer_rsrc_t rs) {
-    uint32_t o = voff[i];
-    if (KMAJOR) o = (c < k_left) ? o : OOB_OFFSET;
-    reg[i] = buffer_load_f4(rs, o);
+  // No address arithmetic per pass: the caller has run mask_tail for a tile that reaches past the end of K.
+  __device__ __forceinline__ void load_pass(int i, __amdgpu_buffer_rsrc_t rs) { reg[i] = buffer_load_f4(rs, voff[i]); }
+  // A K-major tile that holds fewer than BK reduction elements: the pieces beyond them read as zeros from here on
+  // (every later tile lies further out). The descriptor bounds do the same for an MN-major tile.
+  __device__ __forceinline__ void mask_tail(int k_left) {
+    if (KMAJOR) {
+#pragma unroll
+      for (int i = 0; i < PASSES; ++i) voff[i] = (c < k_left) ? voff[i] : OOB_OFFSET;
+    }
   }
   __device__ __forceinline__ void store_pass(float* lds, int i) {
     *reinterpret_cast<float4*>(&lds[lds_off + i * ROWS_PER_PASS * LD]) = reg[i];
+  }
+  __device__ __forceinline__ void store_pass_at(float* lds, int at, int i) {  // at: lds_off plus the tile's place in LDS
+    *reinterpret_cast<float4*>(&lds[at + i * ROWS_PER_PASS * LD]) = reg[i];
   }
   __device__ __forceinline__ void advance() {
     base = reinterpret_cast<const float*>(reinterpret_cast<const char*>(base) + step);

@@ -350,12 +350,12 @@ def test_sgemm_random_shapes_and_flags(dev):
 
 
 @pytest.mark.parametrize("M,N,K", [(256, 256, 32), (256, 512, 64), (300, 520, 70), (516, 260, 1000), (1024, 768, 4100), (260, 1028, 36),
-                                   (128, 64, 512), (512, 1024, 1100)])
+                                   (128, 64, 512), (512, 1024, 1100), (256, 256, 31), (320, 256, 97)])
 def test_sgemm_every_tile_forced(dev, M, N, K):
     """endia_hip_gemm_force_tile: the weight-gradient form (A stored K x M, B stored K x N) through the 64, 128 and 256
     tiles on shapes with ragged edges in M, N and K (the 256 x 256 tile is otherwise only chosen for products that fill
-    every CU with one): every tile against the oracle and float64, plain and accumulating, a padded C, a batch; the other
-    forms keep working while 256 is forced (they have no such kernel and fall back to the automatic choice)."""
+    every CU with one): every tile against the oracle and float64, plain and accumulating, a padded C, a batch; all four
+    forms and every fused epilogue through the 256 tile."""
     rng = np.random.default_rng(M + 3 * N + 7 * K)
     A = rng.standard_normal((K, M)).astype(np.float32)
     B = (rng.standard_normal((K, N)) / np.sqrt(K)).astype(np.float32)
@@ -384,8 +384,22 @@ def test_sgemm_every_tile_forced(dev, M, N, K):
         out = dev.get(dC, (2, M, N))
         assert_close(out[0], ref, what="batch entry 0")
         assert_close(out[1], -ref, what="batch entry 1")
-        At = np.ascontiguousarray(A.T)
-        assert_close(run_sgemm(dev, At, B, 0, 0, M, N, K), ref, what="NN while 256 is forced")
+        # the other forms and the fused epilogues through the 256 tile (still forced)
+        At, Bt = np.ascontiguousarray(A.T), np.ascontiguousarray(B.T)
+        bias = rng.standard_normal(N).astype(np.float32)
+        aux = rng.standard_normal((M, N)).astype(np.float32)
+        for ta, tb, a, b in ((0, 0, At, B), (0, 1, At, Bt), (1, 1, A, Bt), (1, 0, A, B)):
+            if K % 4 and (not ta or tb):
+                continue  # a K-major operand needs K in whole 16-byte pieces for the matrix-core path
+            what = "form (%d, %d) on the 256 tile: " % (ta, tb)
+            assert_close(run_sgemm(dev, a, b, ta, tb, M, N, K), ref, what=what + "plain")
+            assert_close(run_sgemm(dev, a, b, ta, tb, M, N, K, L.EPI_BIAS, bias=bias), ref + bias, what=what + "bias")
+            Cz, Z = run_sgemm(dev, a, b, ta, tb, M, N, K, L.EPI_BIAS_ACT, L.OP_TANH, bias=bias, want_z=True)
+            assert_close(Z, ref + bias, what=what + "stored pre-activation")
+            assert_close(Cz, np.tanh(ref + bias), what=what + "bias + tanh")
+            assert_close(run_sgemm(dev, a, b, ta, tb, M, N, K, L.EPI_ACT_GRAD, L.OP_RELU, aux=aux), ref * (aux > 0), what=what + "relu gradient")
+            assert_close(run_sgemm(dev, a, b, ta, tb, M, N, K, L.EPI_ACT_GRAD, L.OP_TANH | L.ACT_FROM_OUTPUT, aux=np.tanh(aux)),
+                         ref * (1 - np.tanh(aux.astype(np.float64)) ** 2), what=what + "tanh gradient from the output")
         # the column sums of B from the same call (the bias gradient beside the weight gradient), small and large B
         dC, dsum = dev.put(np.full((M, N), np.nan, np.float32)), dev.put(np.full(N, np.nan, np.float32))
         dev.call("endia_hip_sgemm", 1, 0, M, N, K, dev.put(A), M, dev.put(B), N, dC, N, 1, 0, 0, 0, L.EPI_NONE | L.GEMM_COLSUM_B,
