@@ -393,19 +393,92 @@ __device__ __forceinline__ void gemm_tile256(const GemmArgs& p, int block, int n
     tile_body(std::integral_constant<int, 1>());
   }
 
+  // Epilogue. Nothing overlaps it (the CU's only tile ends here), so what it reads is requested ahead of the stores,
+  // which the compiler must assume to alias it: the bias of the lane's four columns up front, and the activation
+  // operand of the next 32 x 32 block before the current block is stored.
+  // The general form below tests bounds, accumulation and the kind of activation per element; written out for 256
+  // elements per lane with the bodies of tanh and sin inlined that is 60-70 thousand instructions, and fetching them
+  // costs more than executing them (60-90 us per launch at 4096^3). The usual cases (a tile inside the matrix, no
+  // accumulation, relu or tanh) therefore have a body of their own with everything uniform decided once.
+  float bias_v[F];
 #pragma unroll
-  for (int fm = 0; fm < F; ++fm)
-#pragma unroll
-    for (int fn = 0; fn < F; ++fn) {
+  for (int fn = 0; fn < F; ++fn) {
+    const int col = n0 + wn * 128 + fn * 32 + l32;
+    bias_v[fn] = ((EPI == ENDIA_EPI_BIAS || EPI == ENDIA_EPI_BIAS_ACT) && col < p.N) ? p.bias[col] : 0.f;
+  }
+  auto fetch_aux = [&](int blk, float (&aux)[16]) {
+    if constexpr (EPI == ENDIA_EPI_ACT_GRAD) {
+      const int fm = blk >> 2, fn = blk & 3;
       const int col = n0 + wn * 128 + fn * 32 + l32;
-      if (col >= p.N) continue;
 #pragma unroll
       for (int v = 0; v < 16; ++v) {
         const int row = m0 + wm * 128 + fm * 32 + acc_row(v, h);
-        if (row >= p.M) continue;
-        epilogue_store<EPI>(p, C, aux_in, aux_out, row, col, acc[fm][fn][v]);
+        aux[v] = (row < p.M && col < p.N) ? aux_in[(int64_t)row * p.ldc + col] : 0.f;
       }
     }
+  };
+  // ACT: ENDIA_OP_TANH or ENDIA_OP_RELU (ignored by the plain and bias epilogues); the tile lies inside C, C = result
+  auto store_inside = [&](auto act_c) {
+    constexpr int ACT = decltype(act_c)::value;
+    float* __restrict__ Ct = C + (int64_t)(m0 + wm * 128 + 4 * h) * p.ldc + (n0 + wn * 128 + l32);
+    const float* __restrict__ Xt = EPI == ENDIA_EPI_ACT_GRAD ? aux_in + (int64_t)(m0 + wm * 128 + 4 * h) * p.ldc + (n0 + wn * 128 + l32) : nullptr;
+    float cur[16] = {}, nxt[16] = {};
+    auto fetch = [&](int blk, float (&aux)[16]) {
+      if constexpr (EPI == ENDIA_EPI_ACT_GRAD) {
+        const int fm = blk >> 2, fn = blk & 3;
+#pragma unroll
+        for (int v = 0; v < 16; ++v) aux[v] = Xt[(int64_t)(fm * 32 + 8 * (v >> 2) + (v & 3)) * p.ldc + fn * 32];
+      }
+    };
+    fetch(0, cur);
+#pragma unroll
+    for (int blk = 0; blk < F * F; ++blk) {
+      const int fm = blk >> 2, fn = blk & 3;
+      if (blk + 1 < F * F) fetch(blk + 1, nxt);
+#pragma unroll
+      for (int v = 0; v < 16; ++v) {
+        float r = acc[fm][fn][v];
+        if constexpr (EPI == ENDIA_EPI_BIAS) r += bias_v[fn];
+        if constexpr (EPI == ENDIA_EPI_BIAS_ACT) {
+          r += bias_v[fn];
+          r = ACT == ENDIA_OP_TANH ? tanhf(r) : (r > 0.f ? r : 0.f);
+        }
+        if constexpr (EPI == ENDIA_EPI_ACT_GRAD) r *= ACT == ENDIA_OP_TANH ? 1.f - cur[v] * cur[v] : (cur[v] > 0.f ? 1.f : 0.f);
+        Ct[(int64_t)(fm * 32 + 8 * (v >> 2) + (v & 3)) * p.ldc + fn * 32] = r;
+      }
+#pragma unroll
+      for (int v = 0; v < 16; ++v) cur[v] = nxt[v];
+    }
+  };
+  if (m0 + BM <= p.M && n0 + BN <= p.N && !p.accumulate) {
+    if constexpr (EPI == ENDIA_EPI_NONE || EPI == ENDIA_EPI_BIAS) {
+      store_inside(std::integral_constant<int, ENDIA_OP_RELU>());
+      return;
+    } else if constexpr (EPI == ENDIA_EPI_BIAS_ACT) {
+      if (!aux_out && p.act == ENDIA_OP_TANH) { store_inside(std::integral_constant<int, ENDIA_OP_TANH>()); return; }
+      if (!aux_out && p.act == ENDIA_OP_RELU) { store_inside(std::integral_constant<int, ENDIA_OP_RELU>()); return; }
+    } else {
+      if (p.act == ENDIA_OP_TANH && p.from_out) { store_inside(std::integral_constant<int, ENDIA_OP_TANH>()); return; }
+      if (p.act == ENDIA_OP_RELU) { store_inside(std::integral_constant<int, ENDIA_OP_RELU>()); return; }
+    }
+  }
+  float aux_cur[16] = {}, aux_nxt[16] = {};
+  fetch_aux(0, aux_cur);
+#pragma unroll
+  for (int blk = 0; blk < F * F; ++blk) {
+    const int fm = blk >> 2, fn = blk & 3;
+    if (blk + 1 < F * F) fetch_aux(blk + 1, aux_nxt);
+    const int col = n0 + wn * 128 + fn * 32 + l32;
+    if (col < p.N) {
+#pragma unroll
+      for (int v = 0; v < 16; ++v) {
+        const int row = m0 + wm * 128 + fm * 32 + acc_row(v, h);
+        if (row < p.M) epilogue_apply<EPI>(p, C, aux_out, row, col, acc[fm][fn][v], bias_v[fn], aux_cur[v]);
+      }
+    }
+#pragma unroll
+    for (int v = 0; v < 16; ++v) aux_cur[v] = aux_nxt[v];
+  }
 }
 
 template <bool A_KMAJOR, bool B_KMAJOR, int EPI>
