@@ -30,10 +30,10 @@ sys.path.insert(0, ROOT)
 FP32_MFMA_PEAK_TFLOPS = 157.3
 HBM_PEAK_GBS = 8000.0
 # HBM-side bytes per 4096^3 GEMM launch, averaged over the launch mix of one training step (1 NN with the bias epilogue,
-# 7 NN with bias+tanh, 7 NT with the tanh' epilogue, 8 TN on the 256 x 256 tile; MiB per launch as in the per-kernel table). It cannot be read while the benchmark runs: it comes
+# 7 NN with bias+tanh, 7 NT with the tanh' epilogue, 8 TN, all on the 256 x 256 tile; MiB per launch as in the per-kernel table). It cannot be read while the benchmark runs: it comes
 # from two rocprofv3 --pmc runs (FETCH_SIZE, WRITE_SIZE in KiB per dispatch), each scaled by what the same counter
 # reads for a 64 MiB copy kernel (x1.999 and x1.000); the per-kernel table is in profiles/.
-GEMM_TRAFFIC_BYTES = int((1 * 701.3 + 7 * 610.2 + 7 * 1338.7 + 8 * 450.8) / 23 * 1024 * 1024)
+GEMM_TRAFFIC_BYTES = int((1 * 451.2 + 7 * 449.1 + 7 * 512.3 + 8 * 450.9) / 23 * 1024 * 1024)
 
 
 def build_wide_mlp(nd, width=4096, layers=8, batch=4096, seed=2):
@@ -657,7 +657,7 @@ def main():
         flops_per_launch = g_flops.value / launches.value
         achieved = flops_per_launch / (avg_ms * 1e-3) / 1e12
         out["roofline"] = {
-            "bound": "mfma", "kernel": "sgemm_mfma_kernel / sgemm_mfma256_kernel (fp32 v_mfma_f32_32x32x2; 128x128x32 tiles forward and data gradient, 256x256x32 weight gradient)",
+            "bound": "mfma", "kernel": "sgemm_mfma256_kernel (fp32 v_mfma_f32_32x32x2, 256x256x32 tiles, one work-group per CU)",
             "achieved": achieved, "peak": FP32_MFMA_PEAK_TFLOPS, "unit": "TFLOP/s", "frac": achieved / FP32_MFMA_PEAK_TFLOPS,
             "traffic": GEMM_TRAFFIC_BYTES if args.workload == "wide_mlp" else None,
             "traffic_source": "rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, see profiles/kernels_wide_mlp_counters.md",
