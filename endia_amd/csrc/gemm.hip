@@ -248,6 +248,39 @@ __device__ __forceinline__ void gemm_tile(const GemmArgs& p, int block, int nblo
     }
   }
 
+  // The 128 x 128 tile inside the matrix, no accumulation, relu or tanh: a body with everything uniform decided once.
+  // The general loop below tests bounds, accumulation and the kind of activation per element with the bodies of tanh
+  // and sin inlined 64 times, and fetching those instructions costs more than running them.
+  if constexpr (F == 2 && EPI != ENDIA_EPI_NONE) {
+    const bool relu = p.act == ENDIA_OP_RELU, tanh_ok = p.act == ENDIA_OP_TANH && (EPI != ENDIA_EPI_ACT_GRAD || p.from_out);
+    const bool plain_store = !p.accumulate && !p.splits && !(EPI == ENDIA_EPI_BIAS_ACT && aux_out);
+    if (m0 + BM <= p.M && n0 + BN <= p.N && plain_store && (EPI == ENDIA_EPI_BIAS || relu || tanh_ok)) {
+      const int64_t at = (int64_t)(m0 + wm * 64 + 4 * h) * p.ldc + (n0 + wn * 64 + l32);
+      float* __restrict__ Ct = C + at;
+      float bias2[F];
+#pragma unroll
+      for (int fn = 0; fn < F; ++fn) bias2[fn] = (EPI == ENDIA_EPI_BIAS || EPI == ENDIA_EPI_BIAS_ACT) ? p.bias[n0 + wn * 64 + fn * 32 + l32] : 0.f;
+#pragma unroll
+      for (int fm = 0; fm < F; ++fm)
+#pragma unroll
+        for (int fn = 0; fn < F; ++fn) {
+          float aux[16] = {};
+          if constexpr (EPI == ENDIA_EPI_ACT_GRAD) {
+#pragma unroll
+            for (int v = 0; v < 16; ++v) aux[v] = aux_in[at + (int64_t)(fm * 32 + 8 * (v >> 2) + (v & 3)) * p.ldc + fn * 32];
+          }
+#pragma unroll
+          for (int v = 0; v < 16; ++v) {
+            float r = acc[fm][fn][v] + bias2[fn];
+            if constexpr (EPI == ENDIA_EPI_BIAS_ACT) r = relu ? (r > 0.f ? r : 0.f) : tanhf(r);
+            if constexpr (EPI == ENDIA_EPI_ACT_GRAD) r *= relu ? (aux[v] > 0.f ? 1.f : 0.f) : 1.f - aux[v] * aux[v];
+            Ct[(int64_t)(fm * 32 + 8 * (v >> 2) + (v & 3)) * p.ldc + fn * 32] = r;
+          }
+        }
+      return;
+    }
+  }
+
 #pragma unroll
   for (int fm = 0; fm < F; ++fm)
 #pragma unroll

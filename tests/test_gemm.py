@@ -384,14 +384,15 @@ def test_sgemm_every_tile_forced(dev, M, N, K):
         out = dev.get(dC, (2, M, N))
         assert_close(out[0], ref, what="batch entry 0")
         assert_close(out[1], -ref, what="batch entry 1")
-        # the other forms and the fused epilogues through the 256 tile (still forced)
+        # all forms and the fused epilogues through the 128 and 256 tiles (tiles inside the matrix take bodies of their own)
         At, Bt = np.ascontiguousarray(A.T), np.ascontiguousarray(B.T)
         bias = rng.standard_normal(N).astype(np.float32)
         aux = rng.standard_normal((M, N)).astype(np.float32)
-        for ta, tb, a, b in ((0, 0, At, B), (0, 1, At, Bt), (1, 1, A, Bt), (1, 0, A, B)):
+        for tile, ta, tb, a, b in [(t,) + f for t in (128, 256) for f in ((0, 0, At, B), (0, 1, At, Bt), (1, 1, A, Bt), (1, 0, A, B))]:
             if K % 4 and (not ta or tb):
                 continue  # a K-major operand needs K in whole 16-byte pieces for the matrix-core path
-            what = "form (%d, %d) on the 256 tile: " % (ta, tb)
+            dev.call("endia_hip_gemm_force_tile", tile)
+            what = "form (%d, %d) on the %d tile: " % (ta, tb, tile)
             assert_close(run_sgemm(dev, a, b, ta, tb, M, N, K), ref, what=what + "plain")
             assert_close(run_sgemm(dev, a, b, ta, tb, M, N, K, L.EPI_BIAS, bias=bias), ref + bias, what=what + "bias")
             Cz, Z = run_sgemm(dev, a, b, ta, tb, M, N, K, L.EPI_BIAS_ACT, L.OP_TANH, bias=bias, want_z=True)
@@ -400,6 +401,7 @@ def test_sgemm_every_tile_forced(dev, M, N, K):
             assert_close(run_sgemm(dev, a, b, ta, tb, M, N, K, L.EPI_ACT_GRAD, L.OP_RELU, aux=aux), ref * (aux > 0), what=what + "relu gradient")
             assert_close(run_sgemm(dev, a, b, ta, tb, M, N, K, L.EPI_ACT_GRAD, L.OP_TANH | L.ACT_FROM_OUTPUT, aux=np.tanh(aux)),
                          ref * (1 - np.tanh(aux.astype(np.float64)) ** 2), what=what + "tanh gradient from the output")
+        dev.call("endia_hip_gemm_force_tile", 256)
         # the column sums of B from the same call (the bias gradient beside the weight gradient), small and large B
         dC, dsum = dev.put(np.full((M, N), np.nan, np.float32)), dev.put(np.full(N, np.nan, np.float32))
         dev.call("endia_hip_sgemm", 1, 0, M, N, K, dev.put(A), M, dev.put(B), N, dC, N, 1, 0, 0, 0, L.EPI_NONE | L.GEMM_COLSUM_B,
