@@ -12,7 +12,8 @@ from ctypes import POINTER, c_float, c_int32, c_int64, c_uint32, c_void_p
 import numpy as np
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
-LIB_PATH = os.path.join(_HERE, "libendia_ref.so")
+# ENDIA_REF_LIB selects another build of the same source (the sanitizer build, oracle/Makefile)
+LIB_PATH = os.environ.get("ENDIA_REF_LIB") or os.path.join(_HERE, "libendia_ref.so")
 
 OP = dict(relu=0, tanh=1, sin=2, cos=3, neg=4, square=5, sqrt=6, abs=7, identity=8, greater0=9, exp=10, log=11,
           sigmoid=12, sinh=13, cosh=14, tan=15, asin=16, acos=17, atan=18, reciprocal=19, sign=20)

@@ -594,6 +594,19 @@ def test_pool_reuses_buffers(dev):
     assert L.lib().endia_hip_free(ctypes.c_void_p(12345)) == L.ERR_INVALID
 
 
+def test_malloc_reports_out_of_memory(dev):
+    """A request beyond the device's memory is refused with ENDIA_HIP_ERR_NOMEM (after the pool has handed its cached
+    buffers back and tried once more), leaves a null pointer, and the library keeps working afterwards."""
+    p = ctypes.c_void_p(1)
+    rc = L.lib().endia_hip_malloc(1 << 46, ctypes.byref(p))
+    assert rc == L.ERR_NOMEM and not p.value
+    assert b"hipMalloc" in L.lib().endia_hip_last_error()
+    a = np.arange(1000, dtype=np.float32)
+    da, dout = dev.put(a), dev.alloc(4)
+    dev.call("endia_hip_reduce_add", 1, L.i64_array([1000]), 1, da, dout, 1.0, 0)
+    assert dev.get(dout, (1,))[0] == a.sum()
+
+
 def _pool_desc(xshape, k, st, pad, dil):
     nsp = len(xshape) - 2
     d = L.PoolDesc()
