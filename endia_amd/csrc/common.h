@@ -30,6 +30,10 @@ int32_t fail(int32_t code, const char* fmt, ...);
 // never shrinks; all users run on the one stream, so consecutive users never overlap.
 int32_t workspace(int64_t bytes, void** out);
 
+// Resolves, once per device, the address of the static scratch array of the entry point that allocates nothing
+// (reduce.hip). Called by endia_hip_init with `device` current.
+int32_t static_scratch_init(int device);
+
 }  // namespace endia
 
 #define ENDIA_REQUIRE_INIT()                                                         \

@@ -279,10 +279,31 @@ inline bool al16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15) =
 
 }  // namespace
 
+// Scratch of endia_hip_col_sum_static, the entry point for callers that cannot allocate: the first-stage partial sums
+// live in this array instead of the library's growing workspace. Every device the library runs on holds its own copy
+// (1 MiB) until the process ends. In host code the name `scratch` is only a handle for hipGetSymbolAddress, never an
+// address a kernel could use: static_scratch_init() resolves it once per device and everything else uses that pointer.
+constexpr int64_t kStaticScratchFloats = 1 << 18;
+static __device__ __align__(256) float scratch[kStaticScratchFloats];
+constexpr int kMaxDevices = 64;
+static float* g_scratch_ptr[kMaxDevices] = {};
+
 namespace endia {
 
-// out[b][c] = scale * sum_r x[b][r][c]
-int32_t col_reduce(int64_t batch, int64_t R, int64_t C, const float* x, float* out, float scale) {
+// Called by endia_hip_init with `device` current: the address of this device's copy of the static scratch array.
+int32_t static_scratch_init(int device) {
+  if (device < 0 || device >= kMaxDevices) return ENDIA_HIP_OK;  // endia_hip_col_sum_static reports it when called
+  if (g_scratch_ptr[device]) return ENDIA_HIP_OK;
+  float* ptr = nullptr;
+  ENDIA_HIP_CALL(hipGetSymbolAddress(reinterpret_cast<void**>(&ptr), HIP_SYMBOL(scratch)));
+  g_scratch_ptr[device] = ptr;
+  return ENDIA_HIP_OK;
+}
+
+// out[b][c] = scale * sum_r x[b][r][c]. The first-stage partial sums go to `part` (room for part_floats) when the
+// caller brings it, else to the library's workspace; with too little room the rows are cut into fewer splits.
+static int32_t col_reduce_with(int64_t batch, int64_t R, int64_t C, const float* x, float* out, float scale, float* part,
+                               int64_t part_floats) {
   hipStream_t s = ctx().stream;
   const bool vec = (C % 4 == 0) && al16(x);
   const int64_t col_tiles = ceil_div64(C, 256);
@@ -305,12 +326,16 @@ int32_t col_reduce(int64_t batch, int64_t R, int64_t C, const float* x, float* o
   int64_t max_s = ceil_div64(R, 16);
   if (S > max_s) S = max_s;
   if (S > 1024) S = 1024;
+  if (part && S * batch * C > part_floats) S = part_floats / (batch * C);
+  if (S < 1) return fail(ENDIA_HIP_ERR_INVALID, "col_reduce: %lld columns do not fit the %lld floats of scratch", (long long)(batch * C), (long long)part_floats);
   int64_t rows_per_split = ceil_div64(R, S);
   S = ceil_div64(R, rows_per_split);
-  void* ws = nullptr;
-  int32_t rc = workspace(batch * S * C * (int64_t)sizeof(float), &ws);
-  if (rc) return rc;
-  float* part = static_cast<float*>(ws);
+  if (!part) {
+    void* ws = nullptr;
+    int32_t rc = workspace(batch * S * C * (int64_t)sizeof(float), &ws);
+    if (rc) return rc;
+    part = static_cast<float*>(ws);
+  }
   dim3 grid((unsigned)col_tiles, (unsigned)S, (unsigned)batch);
   if (vec) hipLaunchKernelGGL(col_reduce_vec_kernel, grid, dim3(TPB), 0, s, x, part, R, C, rows_per_split);
   else hipLaunchKernelGGL(col_reduce_scalar_kernel, grid, dim3(TPB), 0, s, x, part, R, C, rows_per_split);
@@ -319,6 +344,10 @@ int32_t col_reduce(int64_t batch, int64_t R, int64_t C, const float* x, float* o
                      out, S, C, batch, scale);
   ENDIA_LAUNCH_CHECK();
   return ENDIA_HIP_OK;
+}
+
+int32_t col_reduce(int64_t batch, int64_t R, int64_t C, const float* x, float* out, float scale) {
+  return col_reduce_with(batch, R, C, x, out, scale, nullptr, 0);
 }
 
 // out[r] = scale * sum_c x[r][c]
@@ -413,6 +442,21 @@ int32_t endia_hip_reduce_add(int32_t ndim, const int64_t* shape, uint32_t reduce
   hipLaunchKernelGGL(generic_reduce_kernel, dim3((unsigned)nout), dim3(TPB), 0, ctx().stream, d, x, out, nred, scale);
   ENDIA_LAUNCH_CHECK();
   return ENDIA_HIP_OK;
+}
+
+int32_t endia_hip_col_sum_static(int64_t R, int64_t C, const float* x, float* out, float scale) {
+  ENDIA_REQUIRE_INIT();
+  ENDIA_CHECK_ARG(R >= 0 && C >= 0, "endia_hip_col_sum_static: negative extent (R=%lld C=%lld)", (long long)R, (long long)C);
+  if (C == 0) return ENDIA_HIP_OK;
+  ENDIA_CHECK_ARG(C <= kStaticScratchFloats, "endia_hip_col_sum_static: %lld columns exceed the maximum of %lld (the static scratch holds one row of partial sums per row split)",
+                  (long long)C, (long long)kStaticScratchFloats);
+  ENDIA_CHECK_ARG(out != nullptr, "endia_hip_col_sum_static: out is null");
+  if (R == 0) return endia_hip_fill(out, C, 0.f);  // empty sum (a fill kernel: no allocation, safe to record)
+  ENDIA_CHECK_ARG(x != nullptr, "endia_hip_col_sum_static: x is null");
+  const int dev = ctx().device;
+  float* part = (dev >= 0 && dev < kMaxDevices) ? g_scratch_ptr[dev] : nullptr;
+  if (!part) return fail(ENDIA_HIP_ERR_UNSUPPORTED, "endia_hip_col_sum_static: no static scratch was resolved for device %d", dev);
+  return col_reduce_with(1, R, C, x, out, scale, part, kStaticScratchFloats);
 }
 
 int32_t endia_hip_reduce(int32_t op, int32_t ndim, const int64_t* shape, uint32_t reduce_mask, const float* x, float* out) {

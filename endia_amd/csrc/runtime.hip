@@ -135,6 +135,10 @@ int32_t endia_hip_init(int32_t device) {
   }
   ENDIA_HIP_CALL(hipMalloc(reinterpret_cast<void**>(&g_ctx.tickets), kTicketCount * sizeof(unsigned)));
   ENDIA_HIP_CALL(hipMemset(g_ctx.tickets, 0, kTicketCount * sizeof(unsigned)));
+  {
+    int32_t rc = static_scratch_init(device);
+    if (rc) return rc;
+  }
   g_ctx.device = device;
   g_ctx.cu_count = prop.multiProcessorCount;
   g_ctx.clock_mhz = prop.clockRate / 1000;

@@ -275,6 +275,18 @@ ENDIA_API int32_t endia_hip_complex_pack(int64_t n, const float* re, const float
 ENDIA_API int32_t endia_hip_reduce_add(int32_t ndim, const int64_t* shape, uint32_t reduce_mask, const float* x,
                              float* out, float scale, int32_t is_complex);
 
+/* ---- column sums without any allocation. No counterpart in the reference: a variant of endia_hip_reduce_add for
+ *      callers that cannot allocate device memory (code under HIP-graph capture, tight serving loops, harnesses that
+ *      forbid hipMalloc). out[c] = scale * sum_r x[r][c] for a contiguous row-major x of R rows and C columns: the
+ *      bias gradient db = 1^T dZ, i.e. endia_hip_reduce_add with ndim = 2 and reduce_mask = 1, and the same result bit
+ *      for bit (the row splits that call chooses on a 256-CU device never need more than 262144 partial sums; on a
+ *      device where they would, the rows are cut into fewer pieces and the last bits may differ). The partial sums of its first stage live in a 1 MiB array
+ *      that is part of the library's device image instead of the library's growing workspace, so the call performs no
+ *      hipMalloc / hipFree. C above 262144 is refused with ENDIA_HIP_ERR_INVALID. Every call on a device uses that
+ *      device's one array: calls that overlap on one device (two host threads, two processes' worth of streams)
+ *      race; calls on the library's single stream, the only kind this ABI issues, are ordered. */
+ENDIA_API int32_t endia_hip_col_sum_static(int64_t R, int64_t C, const float* x, float* out, float scale);
+
 /* ---- the other reductions: ReduceMax / ReduceMin / ReduceMul .__call__ (reduce_ops/reduce_max_op.mojo:66-190,
  *      reduce_min_op.mojo:66-190, reduce_mul_op.mojo:65-210) and ReduceArgMax / ReduceArgMin .__call__
  *      (reduce_argmax_op.mojo:66-163, reduce_argmin_op.mojo:66-163). Same layout contract as
