@@ -514,7 +514,7 @@ def run_complex(nd, steps, warmup, algo):
     def step(wirtinger=False):
         h = z
         for W in Ws:
-            h = nd.matmul(h, W, _conj_vjp=wirtinger)
+            h = nd.matmul(h, W, vjp_rule="wirtinger" if wirtinger else "reference")
         loss = nd.sum(nd.square(nd.abs(h)))
         loss.backward()
         loss.zero_grad()

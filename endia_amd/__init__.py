@@ -17,7 +17,7 @@ from .functional import (  # noqa: E402,F401
     expand, eye, full, greater, greater_equal, imag, less, less_equal, linear, log, matmul, max_pool1d, max_pool2d, max_pool3d, mean, mse, mul, neg,
     not_equal, ones, pad, permute, pow, pow_to, prod, rand_he_normal, randn, randn_complex, randu, real, reciprocal, reduce_add,
     reduce_argmax, reduce_argmin, reduce_max, reduce_min, reduce_mul,
-    relu, reshape, seed, set_complex_matmul_algorithm, sigmoid, sign, sin, sinh, sqrt, square, squeeze, std, sub, sum, tan,
+    relu, reshape, seed, set_complex_matmul_algorithm, set_complex_vjp_rule, sigmoid, sign, sin, sinh, sqrt, square, squeeze, std, sub, sum, tan,
     tanh, unsqueeze, variance, zeros,
 )
 from .functional import (  # noqa: E402,F401  the rest of the initialisers (endia/functional/init_ops/init_ops.mojo)

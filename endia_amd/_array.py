@@ -99,6 +99,8 @@ class Array:
     _consumers = 0
     _is_seed = False
     _act_applied = False  # a gradient that already carries the producer's activation derivative
+    _grad_fused = None    # such a gradient on its way to this node's own VJP rule; never what grad() returns
+    _true_grad = None     # on an _act_applied gradient: a function that computes the gradient without the derivative
     _offset = 0
     is_complex_ = False
 
@@ -213,18 +215,24 @@ class Array:
         return self
 
     def has_grad(self):
-        return self._grad is not None
+        return self._grad is not None or self._grad_fused is not None
 
     def grad_(self, g):
         self._grad = g
 
     def grad(self):
         if self._grad is None:
+            if self._grad_fused is not None:
+                # A fused layer handed this node dL/dh * act'(h) for its own backward rule. The gradient a caller
+                # reads is dL/dh itself, as the reference stores it on every node: computed here, on first use.
+                self._grad = self._grad_fused._true_grad()
+                return self._grad
             return Array(self._shape, is_complex=self.is_complex_)
         return self._grad
 
     def remove_grad(self):
         self._grad = None
+        self._grad_fused = None
 
     def args(self):
         return list(self._args)

@@ -83,15 +83,19 @@ def jacrev(arg, create_graph=False):
             primals = curr._args
             if not primals or curr._vjp is None:
                 continue
-            grad = curr.grad()
+            # a gradient that already carries this node's activation derivative travels in its own slot
+            grad = curr._grad_fused if curr._grad_fused is not None else curr.grad()
             primals_grads = curr._vjp(primals, grad, curr)
             for primal, pg in zip(primals, primals_grads):
                 if not primal._requires_grad or pg is None:
                     continue
                 if primal.has_grad():
-                    if pg._act_applied or primal._grad._act_applied:
+                    if pg._act_applied or primal._grad_fused is not None:
                         raise RuntimeError("internal: a fused activation gradient met an accumulated gradient")
                     pg = F.add(pg, primal._grad)
+                if pg._act_applied:
+                    primal._grad_fused = pg
+                    continue
                 primal.grad_(pg)
                 if not create_graph:
                     pg.clear_args()
@@ -153,19 +157,24 @@ class Callable:
         self.order = order
         self.keep_outs = keep_outs
 
+    def _wanted(self, order, n):
+        chosen = self.argnums[order]
+        return list(range(n)) if chosen[0] == -1 else [i for i in range(n) if i in chosen]
+
     def __call__(self, *args):
         single = len(args) == 1 and isinstance(args[0], Array)
         arrs = list(args[0]) if (len(args) == 1 and not single) else list(args)
-        # fresh leaves, so that repeated calls never see stale graphs (callable.mojo:100-112)
+        # fresh leaves, so that repeated calls never see stale graphs; an argument takes part in the graph when ANY
+        # order differentiates with respect to it (callable.mojo:100-112)
         leaves = [F.detach(a) for a in arrs]
-        chosen = self.argnums[0]
-        idx = list(range(len(leaves))) if chosen == [-1] else chosen
-        for i in idx:
-            leaves[i].requires_grad_(True)
+        for o in range(self.order):
+            for i in self._wanted(o, len(leaves)):
+                leaves[i].requires_grad_(True)
         res = self.func(leaves[0]) if single else self.func(leaves)
         outs = [res]
-        value = res
+        per_order = [[res]]
         for o in range(self.order):
+            idx = self._wanted(o, len(leaves))  # the arguments of THIS order (callable.mojo:146-151)
             nxt = []
             last = o == self.order - 1
             for arr in outs:
@@ -173,16 +182,16 @@ class Callable:
                 arr.backward(create_graph=not last)
                 for i in idx:
                     nxt.append(leaves[i].grad())
-                for i in idx:
-                    leaves[i].remove_grad()
+                for leaf in leaves:
+                    leaf.remove_grad()
             outs = nxt
+            per_order.append(nxt)
         # detach by copy (callable.mojo:165-176), device to device
-        final = [_contiguous_copy(g) for g in outs]
-        if self.keep_outs:
-            final = [_contiguous_copy(value)] + final
-        if len(final) == 1:
-            return final[0]
-        return final
+        if not self.keep_outs:
+            final = [_contiguous_copy(g) for g in outs]
+            return final[0] if len(final) == 1 else final
+        # value_and_grad: one list per order of differentiation, [[value], [first derivatives], ...] (callable.mojo:186-195)
+        return [[_contiguous_copy(g) for g in group] for group in per_order]
 
 
 def jacobian(f, argnums=None):

@@ -1003,14 +1003,20 @@ def _gemm_operand(x):
     return d
 
 
-def matmul(a, b, _conj_vjp=False, _ca=0, _cb=0):
+def matmul(a, b, vjp_rule=None, _ca=0, _cb=0):
     """Batched matrix product with broadcast batch axes (matmul_op.mojo:36-90,309-346).
 
-    VJP (matmul_op.mojo:278-283): dA = g @ B.T(), dB = A.T() @ g -- for complex operands WITHOUT
-    conjugation, exactly as the reference codes it. `_conj_vjp=True` selects the Wirtinger rule
-    (g @ B^H, A^H @ g) that PyTorch uses; its conjugations are flags of the complex GEMM (`_ca`, `_cb`:
-    the product is taken with conj(a), conj(b)), never materialised copies.
+    VJP (matmul_op.mojo:278-283): dA = g @ B.T(), dB = A.T() @ g. For complex operands the reference codes exactly
+    that, WITHOUT conjugation: vjp_rule="reference", the default. vjp_rule="wirtinger" selects g @ B^H, A^H @ g, the
+    conjugate-Wirtinger gradient of a real loss that PyTorch returns; its conjugations are flags of the complex GEMM
+    (`_ca`, `_cb`: the product is taken with conj(a), conj(b)), never materialised copies. vjp_rule=None takes the
+    process-wide choice of set_complex_vjp_rule(). Real operands are unaffected.
     """
+    if vjp_rule is None:
+        vjp_rule = _complex_vjp_rule[0]
+    if vjp_rule not in ("reference", "wirtinger"):
+        raise ValueError("matmul: vjp_rule must be 'reference' or 'wirtinger'")
+    _conj_vjp = vjp_rule == "wirtinger"
     if a.ndim() < 2 or b.ndim() < 2:
         raise ValueError("Invalid shapes for matmul, i.e. ndim < 2")
     if a._shape[-1] != b._shape[-2]:
@@ -1050,17 +1056,26 @@ def matmul(a, b, _conj_vjp=False, _ca=0, _cb=0):
         p0, p1 = primals
         if _conj_vjp and p0.is_complex_:
             # with A' = conj^ca(A), B' = conj^cb(B): dA = conj^ca(g B'^H), dB = conj^cb(A'^H g)
-            lhs = matmul(grad, p1.T(), True, _ca, _ca ^ (1 - _cb)) if p0._requires_grad else None
-            rhs = matmul(p0.T(), grad, True, _cb ^ (1 - _ca), _cb) if p1._requires_grad else None
+            lhs = matmul(grad, p1.T(), "wirtinger", _ca, _ca ^ (1 - _cb)) if p0._requires_grad else None
+            rhs = matmul(p0.T(), grad, "wirtinger", _cb ^ (1 - _ca), _cb) if p1._requires_grad else None
         else:
-            lhs = matmul(grad, p1.T()) if p0._requires_grad else None
-            rhs = matmul(p0.T(), grad) if p1._requires_grad else None
+            lhs = matmul(grad, p1.T(), "reference") if p0._requires_grad else None
+            rhs = matmul(p0.T(), grad, "reference") if p1._requires_grad else None
         return [lhs, rhs]
 
     return _register(out, [ea, eb], "matmul", vjp)
 
 
 _cgemm_algo = [L.CGEMM_4M]
+_complex_vjp_rule = ["reference"]
+
+
+def set_complex_vjp_rule(name):
+    """The rule matmul's VJP uses for complex operands when a call does not name one: 'reference' (the reference's
+    code, no conjugation: matmul_op.mojo:278-283; the default) or 'wirtinger' (g B^H, A^H g)."""
+    if name not in ("reference", "wirtinger"):
+        raise ValueError("set_complex_vjp_rule: 'reference' or 'wirtinger'")
+    _complex_vjp_rule[0] = name
 
 
 def set_complex_matmul_algorithm(name):
@@ -1166,6 +1181,8 @@ def conv2d(x, kernel, bias=None, stride=1, padding=0, dilation=1, groups=1, act=
         from .autograd.functional import building_graph
         if building_graph():
             raise NotImplementedError("conv2d has no second-order rule")
+        if grad.ndim() != out_.ndim():
+            raise NotImplementedError("conv2d has no rule for a cotangent with leading Jacobian axes (non-scalar output)")
         g = contiguous(_relu_grad_from_output(out_, grad)) if act == "relu" else contiguous(grad)
         res = []
         if primals[0]._requires_grad:
@@ -1234,6 +1251,8 @@ def conv3d(x, kernel, bias=None, stride=(1, 1, 1), padding=(0, 0, 0), dilation=(
         from .autograd.functional import building_graph
         if building_graph():
             raise NotImplementedError("conv3d has no second-order rule")
+        if grad.ndim() != out_.ndim():
+            raise NotImplementedError("conv3d has no rule for a cotangent with leading Jacobian axes (non-scalar output)")
         g = contiguous(grad)
         res = [None] * len(primals)
         if primals[0]._requires_grad:
@@ -1290,6 +1309,8 @@ def _pool(x, mode, nsp, kernel_size, stride, padding, dilation):
         from .autograd.functional import building_graph
         if building_graph():
             raise NotImplementedError("%s has no second-order rule" % name)
+        if grad.ndim() != out_.ndim():
+            raise NotImplementedError("%s has no rule for a cotangent with leading Jacobian axes (non-scalar output)" % name)
         g = contiguous(grad)
         dx = Array.empty(primals[0]._shape)
         L.call("endia_hip_pool_bwd", ctypes.byref(desc), mode, g.data_ptr(), arg.ptr if arg else None, dx.data_ptr())
@@ -1373,7 +1394,7 @@ def _sin_of_linear_node(out, zz):
     def vjp(primals, grad, out_):
         from .autograd.functional import building_graph
         z = primals[0]
-        if building_graph():
+        if building_graph() or grad.ndim() != out_.ndim():  # (a Jacobian seed's leading axes broadcast through mul)
             return [mul(cos(z), grad)]  # sin_op.mojo:92
         if grad._act_applied:
             return [grad]
@@ -1392,16 +1413,18 @@ def _linear_node(out, x, W, b, xs, Ws, act):
     def vjp(primals, grad, out_):
         from .autograd.functional import building_graph
         px, pW, pb = primals
-        if building_graph():
+        lead = grad.ndim() - out_.ndim()  # leading axes of a Jacobian seed (autograd/functional.mojo:35-37)
+        if building_graph() or lead:
             if act == "tanh":
                 g = mul(1 - square(out_), grad)                      # tanh_op.mojo:92 with tanh(z) = out
             elif act == "relu":
                 g = mul(greater(out_, zeros([N])), grad)             # relu_op.mojo:95; out > 0 iff z > 0
             else:
                 g = grad
+            # matmul treats the leading axes as a batch; the bias gradient sums the layer's batch axis, which follows them
             return [matmul(g, pW.T()) if px._requires_grad else None,
                     matmul(px.T(), g) if pW._requires_grad else None,
-                    reduce_add(g, [0]) if pb._requires_grad else None]
+                    reduce_add(g, [lead]) if pb._requires_grad else None]
         g = contiguous(grad)
         if act in _ACT_FN and not grad._act_applied:  # relu and tanh derivatives from the stored output
             gp = Array.empty([B, N])
@@ -1419,6 +1442,8 @@ def _linear_node(out, x, W, b, xs, Ws, act):
                 flags = _ACT[pm["act"]] | (L.ACT_FROM_OUTPUT if pm["from_output"] else 0)
                 aux = contiguous(pm["aux"])
                 dx._act_applied = True
+                # what px.grad() shows is dL/dpx itself; nobody reads it in a training step, so it is made on demand
+                dx._true_grad = lambda: matmul(detach(g), detach(Ws).T())
         L.call("endia_hip_linear_bwd", B, K, N, xs.data_ptr(), Ws.data_ptr(), g.data_ptr(), flags,
                aux.data_ptr() if aux is not None else None, dx.data_ptr() if dx is not None else None,
                dW.data_ptr() if dW is not None else None, db.data_ptr() if db is not None else None)

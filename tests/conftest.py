@@ -33,12 +33,18 @@ def mean_rel(x, ref):
 RTOL = 1e-4
 
 
-def assert_close(x, ref, tol=RTOL, what=""):
+def assert_close(x, ref, tol=RTOL, what="", mean_tol=None):
+    """Both metrics: ||x - ref||_2 / ||ref||_2 <= tol, and the reference's own is_close figure (mean over the elements
+    of |x - ref| / max(|ref|, 1e-6), array_conversions.mojo:108-135) <= max(tol, 1e-4), its tests' tolerance, unless
+    the caller states another bound for it (`mean_tol`) and why."""
     x, ref = np.asarray(x), np.asarray(ref)
     assert x.size == ref.size, "%s: size %s vs %s" % (what, x.shape, ref.shape)
     x = x.reshape(ref.shape)
     e = rel_l2(x, ref)
     assert np.isfinite(e) and e <= tol, "%s: relative L2 error %.3e > %.1e" % (what, e, tol)
+    m = mean_rel(x, ref)
+    bound = max(tol, RTOL) if mean_tol is None else mean_tol
+    assert np.isfinite(m) and m <= bound, "%s: mean relative error %.3e > %.1e" % (what, m, bound)
 
 
 @pytest.fixture(scope="session")

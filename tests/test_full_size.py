@@ -330,7 +330,7 @@ def test_complex_mlp_full_size_directional_derivative(algo):
             Ws = [nd.array(W + np.complex64(eps) * V, requires_grad=want_grad) for W, V in zip(Wn, Vn)]
             h = z
             for W in Ws:
-                h = nd.matmul(h, W, _conj_vjp=True)
+                h = nd.matmul(h, W, vjp_rule="wirtinger")
             loss = nd.sum(nd.square(nd.abs(h)))
             if not want_grad:
                 return float(loss.item())

@@ -917,10 +917,13 @@ def test_conv_and_pool_random_configs(dev):
         dev.call("endia_hip_conv2d_bwd_weight", ctypes.byref(d), dx_, dg, ddw)
         dev.call("endia_hip_conv2d_bwd_bias", ctypes.byref(d), dg, ddb)
         what = "conv case %d: x %s w %s stride %s pad %s dil %s" % (case, x.shape, w.shape, st, pd, dl)
-        assert_close(dev.get(dy, gy.shape), ty.detach().numpy(), what=what + " fwd")
-        assert_close(dev.get(ddx, x.shape), tx.grad.numpy(), what=what + " dx")
-        assert_close(dev.get(ddw, w.shape), tw.grad.numpy(), what=what + " dw")
-        assert_close(dev.get(ddb, b.shape), tb.grad.numpy(), what=what + " db")
+        # Every value here is a sum of products of either sign, and some of the random tensors are tiny (a weight
+        # gradient of 40 values): one value a thousand times smaller than its neighbours carries the whole mean of the
+        # relative errors. That figure gets 1e-3 in this sweep; the relative L2 bound stays 1e-4.
+        assert_close(dev.get(dy, gy.shape), ty.detach().numpy(), what=what + " fwd", mean_tol=1e-3)
+        assert_close(dev.get(ddx, x.shape), tx.grad.numpy(), what=what + " dx", mean_tol=1e-3)
+        assert_close(dev.get(ddw, w.shape), tw.grad.numpy(), what=what + " dw", mean_tol=1e-3)
+        assert_close(dev.get(ddb, b.shape), tb.grad.numpy(), what=what + " db", mean_tol=1e-3)
         dev.release()
     for case in range(40):
         N, C = int(rng.integers(1, 4)), int(rng.integers(1, 6))
