@@ -21,6 +21,7 @@
 // k = 8j + 4h + i for half-wave h, which is what makes the 128-bit fetch possible. Both
 // operands use the same mapping.
 #include "common.h"
+#include "gemm_args.h"
 #include "mfma_tile.h"
 #include "ticket.h"
 
@@ -33,76 +34,7 @@ namespace {
 
 using namespace mfma;
 
-constexpr int NTHREADS = 256;  // four waves, 2 x 2
-
-struct GemmArgs {
-  const float* A;
-  const float* B;
-  float* C;
-  const float* bias;
-  const float* aux_in;
-  float* aux_out;
-  int64_t lda, ldb, ldc;
-  int64_t sA, sB, sC;
-  int M, N, K;
-  int tiles_m, tiles_n;
-  int k_split;    // > 0: grid.y indexes slices of K of this length instead of batch entries
-  int splits;     // > 0: the slices' partial sums meet in `part` and the last group of a tile to arrive finishes it
-  float* part;    // [splits][tiles][accumulator registers][256 lanes]
-  unsigned* tickets;  // one arrival counter per tile, zero between launches
-  int act;        // endia_hip_unary_op
-  int from_out;   // activation gradient from stored output instead of pre-activation
-  int accumulate;
-  int colsum;     // also write sum_k B[k][n] to aux_out[n] (B MN-major; done by the work-groups of the first tile row)
-};
-
-__device__ __forceinline__ float act_fwd(int act, float z) {
-  switch (act) {
-    case ENDIA_OP_RELU: return z > 0.f ? z : 0.f;
-    case ENDIA_OP_TANH: return tanhf(z);
-    case ENDIA_OP_SIN: return sinf(z);
-    default: return z;
-  }
-}
-
-__device__ __forceinline__ float act_grad(int act, int from_out, float aux) {
-  switch (act) {
-    case ENDIA_OP_RELU: return aux > 0.f ? 1.f : 0.f;
-    case ENDIA_OP_TANH: {
-      float a = from_out ? aux : tanhf(aux);
-      return 1.f - a * a;
-    }
-    case ENDIA_OP_SIN: return cosf(aux);
-    default: return 1.f;
-  }
-}
-
-// bias_v = bias[col] and aux_v = aux_in[row, col], fetched by the caller (early, where registers allow)
-template <int EPI>
-__device__ __forceinline__ void epilogue_apply(const GemmArgs& p, float* __restrict__ C, float* __restrict__ aux_out,
-                                               int row, int col, float v, float bias_v, float aux_v) {
-  int64_t off = (int64_t)row * p.ldc + col;
-  if (EPI == ENDIA_EPI_BIAS) {
-    v += bias_v;
-  } else if (EPI == ENDIA_EPI_BIAS_ACT) {
-    v += bias_v;
-    if (aux_out) aux_out[off] = v;
-    v = act_fwd(p.act, v);
-  } else if (EPI == ENDIA_EPI_ACT_GRAD) {
-    v *= act_grad(p.act, p.from_out, aux_v);
-  }
-  if (p.accumulate) v += C[off];
-  C[off] = v;
-}
-
-template <int EPI>
-__device__ __forceinline__ void epilogue_store(const GemmArgs& p, float* __restrict__ C,
-                                               const float* __restrict__ aux_in,
-                                               float* __restrict__ aux_out, int row, int col, float v) {
-  const float bias_v = (EPI == ENDIA_EPI_BIAS || EPI == ENDIA_EPI_BIAS_ACT) ? p.bias[col] : 0.f;
-  const float aux_v = EPI == ENDIA_EPI_ACT_GRAD ? aux_in[(int64_t)row * p.ldc + col] : 0.f;
-  epilogue_apply<EPI>(p, C, aux_out, row, col, v, bias_v, aux_v);
-}
+using namespace endia_gemm;  // GemmArgs, epilogue bodies, launchers of the one-wave-per-SIMD tiles (gemm_args.h)
 
 // F = MFMA blocks per wave in each direction: F = 2 gives the 128 x 128 tile, F = 1 the 64 x 64 tile
 // used when the larger one would leave CUs without work.
@@ -297,229 +229,6 @@ __device__ __forceinline__ void gemm_tile(const GemmArgs& p, int block, int nblo
     }
 }
 
-// The 256 x 256 tile: one work-group per CU, one wave per SIMD, each wave 128 x 128 = 4 x 4 MFMA blocks (256 accumulator
-// registers per lane). With nobody else on the SIMD to fill a wave's stalls, the order of instructions is the
-// schedule, and whatever is not an MFMA is hidden only if it sits BETWEEN two MFMAs (the matrix pipe is busy for 64
-// cycles per instruction; what follows in program order issues meanwhile). So a K tile is 16 steps of 16 MFMAs, cut
-// into quads, and in front of every quad goes one small piece of the other work, fenced by scheduling barriers so the
-// compiler keeps it there:
-//   * LDS holds two stages; steps 0-11 read, block by block, the fragments of the next group of four steps from the
-//     current stage (one group ahead of their use), steps 12-15 the first fragments of the next tile from the other
-//     stage, behind the tile's only barrier (at step 12 everybody has written its share of that stage and has read
-//     the last of this one);
-//   * steps 0-11 also move the next tile, one 16-byte piece per lane at a time, from registers to the other stage and
-//     request the same piece of the tile after it from memory, which then has a whole K tile (~7 us) to arrive.
-// Tiles past the end of K load as zeros (descriptor bounds) into a stage nobody reads.
-template <bool A_KMAJOR, bool B_KMAJOR, int EPI>
-__device__ __forceinline__ void gemm_tile256(const GemmArgs& p, int block, int nblocks, int64_t bz, float* __restrict__ smem) {
-  constexpr int F = 4, BM = 256, BN = 256;
-  using LA = MatrixTileLoader<A_KMAJOR, BM, NTHREADS>;
-  using LB = MatrixTileLoader<B_KMAJOR, BN, NTHREADS>;
-  constexpr int SA = TileShape<A_KMAJOR, BM>::FLOATS, STAGE = SA + TileShape<B_KMAJOR, BN>::FLOATS;
-  static_assert(BK == 32 && LA::PASSES == 8 && LB::PASSES == 8, "the step plan below is written for these");
-
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-  const int wm = wave >> 1, wn = wave & 1, l32 = lane & 31, h = lane >> 5;
-  int tm, tn;
-  tile_of_block(block, nblocks, p.tiles_m, p.tiles_n, tm, tn);
-  const int m0 = tm * BM, n0 = tn * BN;
-  float* __restrict__ C = p.C + bz * p.sC;
-  const float* __restrict__ aux_in = p.aux_in ? p.aux_in + bz * p.sC : nullptr;
-  float* __restrict__ aux_out = p.aux_out ? p.aux_out + bz * p.sC : nullptr;
-  const int K = p.K;
-  LA la;
-  LB lb;
-  la.init(p.A + bz * p.sA, p.lda, m0, p.M, K, tid);
-  lb.init(p.B + bz * p.sB, p.ldb, n0, p.N, K, tid);
-
-  floatx16 acc[F][F];
-  zero_acc<F, F>(acc);
-  const int a_row = wm * 128 + l32, b_col = wn * 128 + l32;
-
-  la.load(K);
-  lb.load(K);
-  la.store(smem);
-  lb.store(smem + SA);
-  la.advance();
-  lb.advance();
-  la.load(K - BK);
-  lb.load(K - BK);
-  __syncthreads();
-  float af[2][F][4], bf[2][F][4];
-#pragma unroll
-  for (int f = 0; f < F; ++f) {
-    load_fragment_block<A_KMAJOR, BM>(smem, a_row + 32 * f, h, 0, af[0][f]);
-    load_fragment_block<B_KMAJOR, BN>(smem + SA, b_col + 32 * f, h, 0, bf[0][f]);
-  }
-  // Loop state that changes from tile to tile lives in scalar registers: operand base pointers and the bytes left in
-  // their descriptors (32-bit: the host takes this tile only for operands below 2 GiB). A vector ALU instruction
-  // between two MFMAs of a lone wave is not hidden the way an LDS or memory instruction is (a select per load cost
-  // 4 % of the kernel), so there is none: LDS addresses are loop constants because the loop body is written out for
-  // both stages, and the K tail is handled once, when it comes, by rewriting the lanes' offsets.
-  const char* base_a = reinterpret_cast<const char*>(la.base);
-  const char* base_b = reinterpret_cast<const char*>(lb.base);
-  int rec_a = (int)(la.records < 0 ? 0 : (la.records > 0x7FFFFFF0ll ? 0x7FFFFFF0ll : la.records));
-  int rec_b = (int)(lb.records < 0 ? 0 : (lb.records > 0x7FFFFFF0ll ? 0x7FFFFFF0ll : lb.records));
-  const int step_a = (int)la.step, step_b = (int)lb.step;
-  int k_left = K - BK;  // reduction elements from the tile the loaders point at to the end
-  // Per stage and operand, the lane's LDS position for fragment reads and for staging stores, each in a register of
-  // its own (the empty asm keeps the compiler from deriving one from another with an addition inside the loop);
-  // everything else in an LDS address is a constant within reach of the instruction's 64 KiB offset field.
-  int fa_at[2], fb_at[2], sa_at[2], sb_at[2];
-#pragma unroll
-  for (int st = 0; st < 2; ++st) {
-    fa_at[st] = st * STAGE + fragment_lane_offset<A_KMAJOR, BM>(a_row, h);
-    fb_at[st] = st * STAGE + SA + fragment_lane_offset<B_KMAJOR, BN>(b_col, h);
-    sa_at[st] = st * STAGE + la.lds_off;
-    sb_at[st] = st * STAGE + SA + lb.lds_off;
-    asm volatile("" : "+v"(fa_at[st]), "+v"(fb_at[st]), "+v"(sa_at[st]), "+v"(sb_at[st]));
-  }
-  auto tile_body = [&](auto stage) {
-    constexpr int ST = decltype(stage)::value;
-    base_a += step_a;  // the tile after the next one
-    base_b += step_b;
-    rec_a = rec_a > step_a ? rec_a - step_a : 0;
-    rec_b = rec_b > step_b ? rec_b - step_b : 0;
-    k_left -= BK;
-    if (k_left < BK) {
-      la.mask_tail(k_left);
-      lb.mask_tail(k_left);
-    }
-    const __amdgpu_buffer_rsrc_t rsa = __builtin_amdgcn_make_buffer_rsrc(const_cast<char*>(base_a), 0, rec_a, 0x00020000);
-    const __amdgpu_buffer_rsrc_t rsb = __builtin_amdgcn_make_buffer_rsrc(const_cast<char*>(base_b), 0, rec_b, 0x00020000);
-#pragma unroll
-    for (int s = 0; s < 16; ++s) {
-      const int j = s >> 2, i = s & 3, cur = j & 1, nxt = cur ^ 1;
-      if (s == 12) __syncthreads();
-      const int fs = s < 12 ? ST : ST ^ 1;  // stage the fragments are read from
-      const int jn = s < 12 ? j + 1 : 0;
-      auto quad = [&](int fm) {
-        __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-        for (int fn = 0; fn < F; ++fn)
-          acc[fm][fn] = __builtin_amdgcn_mfma_f32_32x32x2f32(af[cur][fm][i], bf[cur][fn][i], acc[fm][fn], 0, 0, 0);
-        __builtin_amdgcn_sched_barrier(0);
-      };
-      load_fragment_at<A_KMAJOR, BM>(smem, fa_at[fs], i, jn, af[nxt][i]);
-      quad(0);
-      load_fragment_at<B_KMAJOR, BN>(smem, fb_at[fs], i, jn, bf[nxt][i]);
-      quad(1);
-      if (s < 8) {
-        la.store_pass_at(smem, sa_at[ST ^ 1], s);
-        la.load_pass(s, rsa);
-      } else if (s < 12) {
-        lb.store_pass_at(smem, sb_at[ST ^ 1], s - 4);
-        lb.load_pass(s - 4, rsb);
-      }
-      quad(2);
-      if (s < 4) {
-        lb.store_pass_at(smem, sb_at[ST ^ 1], s);
-        lb.load_pass(s, rsb);
-      }
-      quad(3);
-    }
-  };
-  // two K tiles per trip, one per LDS stage; an odd tile count runs one more tile of zeros
-  const int T = (K + BK - 1) / BK;
-  for (int t = 0; t < T; t += 2) {
-    tile_body(std::integral_constant<int, 0>());
-    tile_body(std::integral_constant<int, 1>());
-  }
-
-  // Epilogue. Nothing overlaps it (the CU's only tile ends here), so what it reads is requested ahead of the stores,
-  // which the compiler must assume to alias it: the bias of the lane's four columns up front, and the activation
-  // operand of the next 32 x 32 block before the current block is stored.
-  // The general form below tests bounds, accumulation and the kind of activation per element; written out for 256
-  // elements per lane with the bodies of tanh and sin inlined that is 60-70 thousand instructions, and fetching them
-  // costs more than executing them (60-90 us per launch at 4096^3). The usual cases (a tile inside the matrix, no
-  // accumulation, relu or tanh) therefore have a body of their own with everything uniform decided once.
-  float bias_v[F];
-#pragma unroll
-  for (int fn = 0; fn < F; ++fn) {
-    const int col = n0 + wn * 128 + fn * 32 + l32;
-    bias_v[fn] = ((EPI == ENDIA_EPI_BIAS || EPI == ENDIA_EPI_BIAS_ACT) && col < p.N) ? p.bias[col] : 0.f;
-  }
-  auto fetch_aux = [&](int blk, float (&aux)[16]) {
-    if constexpr (EPI == ENDIA_EPI_ACT_GRAD) {
-      const int fm = blk >> 2, fn = blk & 3;
-      const int col = n0 + wn * 128 + fn * 32 + l32;
-#pragma unroll
-      for (int v = 0; v < 16; ++v) {
-        const int row = m0 + wm * 128 + fm * 32 + acc_row(v, h);
-        aux[v] = (row < p.M && col < p.N) ? aux_in[(int64_t)row * p.ldc + col] : 0.f;
-      }
-    }
-  };
-  // ACT: ENDIA_OP_TANH or ENDIA_OP_RELU (ignored by the plain and bias epilogues); the tile lies inside C, C = result
-  auto store_inside = [&](auto act_c) {
-    constexpr int ACT = decltype(act_c)::value;
-    float* __restrict__ Ct = C + (int64_t)(m0 + wm * 128 + 4 * h) * p.ldc + (n0 + wn * 128 + l32);
-    const float* __restrict__ Xt = EPI == ENDIA_EPI_ACT_GRAD ? aux_in + (int64_t)(m0 + wm * 128 + 4 * h) * p.ldc + (n0 + wn * 128 + l32) : nullptr;
-    float cur[16] = {}, nxt[16] = {};
-    auto fetch = [&](int blk, float (&aux)[16]) {
-      if constexpr (EPI == ENDIA_EPI_ACT_GRAD) {
-        const int fm = blk >> 2, fn = blk & 3;
-#pragma unroll
-        for (int v = 0; v < 16; ++v) aux[v] = Xt[(int64_t)(fm * 32 + 8 * (v >> 2) + (v & 3)) * p.ldc + fn * 32];
-      }
-    };
-    fetch(0, cur);
-#pragma unroll
-    for (int blk = 0; blk < F * F; ++blk) {
-      const int fm = blk >> 2, fn = blk & 3;
-      if (blk + 1 < F * F) fetch(blk + 1, nxt);
-#pragma unroll
-      for (int v = 0; v < 16; ++v) {
-        float r = acc[fm][fn][v];
-        if constexpr (EPI == ENDIA_EPI_BIAS) r += bias_v[fn];
-        if constexpr (EPI == ENDIA_EPI_BIAS_ACT) {
-          r += bias_v[fn];
-          r = ACT == ENDIA_OP_TANH ? tanhf(r) : (r > 0.f ? r : 0.f);
-        }
-        if constexpr (EPI == ENDIA_EPI_ACT_GRAD) r *= ACT == ENDIA_OP_TANH ? 1.f - cur[v] * cur[v] : (cur[v] > 0.f ? 1.f : 0.f);
-        Ct[(int64_t)(fm * 32 + 8 * (v >> 2) + (v & 3)) * p.ldc + fn * 32] = r;
-      }
-#pragma unroll
-      for (int v = 0; v < 16; ++v) cur[v] = nxt[v];
-    }
-  };
-  if (m0 + BM <= p.M && n0 + BN <= p.N && !p.accumulate) {
-    if constexpr (EPI == ENDIA_EPI_NONE || EPI == ENDIA_EPI_BIAS) {
-      store_inside(std::integral_constant<int, ENDIA_OP_RELU>());
-      return;
-    } else if constexpr (EPI == ENDIA_EPI_BIAS_ACT) {
-      if (!aux_out && p.act == ENDIA_OP_TANH) { store_inside(std::integral_constant<int, ENDIA_OP_TANH>()); return; }
-      if (!aux_out && p.act == ENDIA_OP_RELU) { store_inside(std::integral_constant<int, ENDIA_OP_RELU>()); return; }
-    } else {
-      if (p.act == ENDIA_OP_TANH && p.from_out) { store_inside(std::integral_constant<int, ENDIA_OP_TANH>()); return; }
-      if (p.act == ENDIA_OP_RELU) { store_inside(std::integral_constant<int, ENDIA_OP_RELU>()); return; }
-    }
-  }
-  float aux_cur[16] = {}, aux_nxt[16] = {};
-  fetch_aux(0, aux_cur);
-#pragma unroll
-  for (int blk = 0; blk < F * F; ++blk) {
-    const int fm = blk >> 2, fn = blk & 3;
-    if (blk + 1 < F * F) fetch_aux(blk + 1, aux_nxt);
-    const int col = n0 + wn * 128 + fn * 32 + l32;
-    if (col < p.N) {
-#pragma unroll
-      for (int v = 0; v < 16; ++v) {
-        const int row = m0 + wm * 128 + fm * 32 + acc_row(v, h);
-        if (row < p.M) epilogue_apply<EPI>(p, C, aux_out, row, col, acc[fm][fn][v], bias_v[fn], aux_cur[v]);
-      }
-    }
-#pragma unroll
-    for (int v = 0; v < 16; ++v) aux_cur[v] = aux_nxt[v];
-  }
-}
-
-template <bool A_KMAJOR, bool B_KMAJOR, int EPI>
-__global__ __launch_bounds__(NTHREADS, 1) void sgemm_mfma256_kernel(GemmArgs p) {
-  extern __shared__ __attribute__((aligned(16))) float smem256[];
-  gemm_tile256<A_KMAJOR, B_KMAJOR, EPI>(p, blockIdx.x, gridDim.x, blockIdx.y, smem256);
-}
-
 template <bool A_KMAJOR, bool B_KMAJOR, int EPI, int F, bool SHORTK = false>
 __global__ __launch_bounds__(NTHREADS, 4) void sgemm_mfma_kernel(GemmArgs p) {
   __shared__ __attribute__((aligned(16))) float As[TileShape<A_KMAJOR, 64 * F>::FLOATS];
@@ -661,37 +370,6 @@ void launch_mfma(const GemmArgs& p, int transA, int transB, dim3 grid, hipStream
   else hipLaunchKernelGGL((sgemm_mfma_kernel<false, false, EPI, F, SHORTK>), grid, dim3(NTHREADS), 0, s, p);
 }
 
-template <bool AK, bool BKM, int EPI>
-int32_t launch_one256(const GemmArgs& p, dim3 grid, hipStream_t s) {
-  constexpr size_t lds = 2 * (size_t)(TileShape<AK, 256>::FLOATS + TileShape<BKM, 256>::FLOATS) * sizeof(float);
-  static bool allowed = false;  // more than 64 KiB of LDS has to be asked for, once per kernel
-  if (!allowed) {
-    ENDIA_HIP_CALL(hipFuncSetAttribute(reinterpret_cast<const void*>(&sgemm_mfma256_kernel<AK, BKM, EPI>),
-                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
-    allowed = true;
-  }
-  hipLaunchKernelGGL((sgemm_mfma256_kernel<AK, BKM, EPI>), grid, dim3(NTHREADS), lds, s, p);
-  return ENDIA_HIP_OK;
-}
-
-template <int EPI>
-int32_t launch_mfma256(const GemmArgs& p, int transA, int transB, dim3 grid, hipStream_t s) {
-  const bool ak = !transA, bk = transB != 0;
-  if (ak && bk) return launch_one256<true, true, EPI>(p, grid, s);
-  if (ak && !bk) return launch_one256<true, false, EPI>(p, grid, s);
-  if (!ak && bk) return launch_one256<false, true, EPI>(p, grid, s);
-  return launch_one256<false, false, EPI>(p, grid, s);
-}
-
-int32_t launch_mfma256_epi(const GemmArgs& p, int epi, int transA, int transB, dim3 grid, hipStream_t s) {
-  switch (epi) {
-    case ENDIA_EPI_NONE: return launch_mfma256<ENDIA_EPI_NONE>(p, transA, transB, grid, s);
-    case ENDIA_EPI_BIAS: return launch_mfma256<ENDIA_EPI_BIAS>(p, transA, transB, grid, s);
-    case ENDIA_EPI_BIAS_ACT: return launch_mfma256<ENDIA_EPI_BIAS_ACT>(p, transA, transB, grid, s);
-    default: return launch_mfma256<ENDIA_EPI_ACT_GRAD>(p, transA, transB, grid, s);
-  }
-}
-
 template <int F, bool SHORTK = false>
 void launch_mfma_epi(const GemmArgs& p, int epi, int transA, int transB, dim3 grid, hipStream_t s) {
   switch (epi) {
@@ -789,16 +467,29 @@ int32_t sgemm_impl(int transA, int transB, int64_t M, int64_t N, int64_t K, cons
     const double score128 = balance(t128) * (per_cu >= 3.0 ? 1.0 : (per_cu >= 2.0 ? 0.95 : 0.80));
     const double score64 = balance(t64) * 0.92;
     int F = (fits128 && score128 >= score64) ? 2 : 1;
-    // 256 x 256 tiles, one per CU at a time: when they fill every round over the CUs (4096^2 outputs are 256 of them)
-    const int64_t t256 = ceil_div64(M, 256) * ceil_div64(N, 256) * batch;
-    const bool fits256 = (double)(ceil_div64(M, 256) * 256) * (double)(ceil_div64(N, 256) * 256) <= 1.1 * (double)M * (double)N;
-    // (its descriptors count bytes in 32 bits; the column sums of a small B ride in the launch of the other kernels)
-    const bool has256 = !(colsum && K * N <= (1ll << 20)) && (transA ? K : M) * lda < (1ll << 29) && (transB ? N : K) * ldb < (1ll << 29);
+    // One-wave-per-SIMD tiles (gemm_lone.h), one work-group per CU at a time: 256 x 256 or 256 x 128, the larger one
+    // whose tiles fill every round over the CUs (4096^2 outputs are 256 tiles of 256 x 256, 2048 x 4096 outputs 256 of
+    // 256 x 128). Smaller tiles written the same way (128 x 128, 128 x 64) were measured and bring nothing over the
+    // shared-CU kernels below: their K tile is so short that the LDS traffic per MFMA stalls a lone wave's issue.
+    // (The descriptors count bytes in 32 bits; the column sums of a small B ride in the launch of the other kernels.)
+    const bool lone_ok = !(colsum && K * N <= (1ll << 20)) && (transA ? K : M) * lda < (1ll << 29) && (transB ? N : K) * ldb < (1ll << 29);
+    static const int lone_bm[2] = {256, 256}, lone_bn[2] = {256, 128};
+    int lone = -1;  // index into the tables above
+    if (lone_ok && g_forced_tile == 0 && K >= 256) {
+      for (int i = 0; i < 2 && lone < 0; ++i) {
+        const int64_t tm_ = ceil_div64(M, lone_bm[i]), tn_ = ceil_div64(N, lone_bn[i]), t = tm_ * tn_ * batch;
+        const bool fits = (double)(tm_ * lone_bm[i]) * (double)(tn_ * lone_bn[i]) <= 1.1 * (double)M * (double)N;
+        if (fits && t >= cus && balance(t) >= 0.9) lone = i;
+      }
+    } else if (lone_ok) {
+      lone = g_forced_tile == 256 ? 0 : g_forced_tile == 256128 ? 1 : -1;
+    }
     if (g_forced_tile == 64) F = 1;
     else if (g_forced_tile == 128) F = 2;
-    if (has256 && (g_forced_tile == 256 || (g_forced_tile == 0 && fits256 && t256 >= cus && balance(t256) >= 0.9 && K >= 256))) F = 4;
-    p.tiles_m = (int)ceil_div64(M, 64 * F);
-    p.tiles_n = (int)ceil_div64(N, 64 * F);
+    const int BM_ = lone >= 0 ? lone_bm[lone] : 64 * F, BN_ = lone >= 0 ? lone_bn[lone] : 64 * F;
+    if (lone >= 0) F = 0;  // none of the shared-CU tiles
+    p.tiles_m = (int)ceil_div64(M, BM_);
+    p.tiles_n = (int)ceil_div64(N, BN_);
     const int64_t tiles = (int64_t)p.tiles_m * p.tiles_n;
     ENDIA_CHECK_ARG(tiles < (1ll << 31), "sgemm: too many output tiles");
     // A product with fewer than about three tiles per CU is split along K so that more groups are in flight (a lone group
@@ -864,8 +555,11 @@ int32_t sgemm_impl(int transA, int transB, int64_t M, int64_t N, int64_t K, cons
       }
       ENDIA_HIP_CALL(hipEventRecord(g_timing.start[g_timing.used], s));
     }
-    if (F == 4) {
-      int32_t rc = launch_mfma256_epi(p, epi, transA, transB, grid, s);
+#ifdef ENDIA_LONE_STAMPS
+    if (lone >= 0) p.part = reinterpret_cast<float*>(ctx().tickets);  // profiling build: per-group wall-clock stamps (<= 512 groups)
+#endif
+    if (lone >= 0) {
+      int32_t rc = lone == 0 ? launch_lone_256x256(p, epi, transA, transB, grid, s) : launch_lone_256x128(p, epi, transA, transB, grid, s);
       if (rc) return rc;
     } else if (F == 2) launch_mfma_epi<2>(p, epi, transA, transB, grid, s);
     else if (K <= 4 * BK && splits == 1) launch_mfma_epi<1, true>(p, epi, transA, transB, grid, s);
@@ -978,7 +672,8 @@ extern "C" int32_t endia_hip_sgemm(int32_t transA, int32_t transB, int64_t M, in
 }
 
 extern "C" int32_t endia_hip_gemm_force_tile(int32_t tile) {
-  ENDIA_CHECK_ARG(tile == 0 || tile == 64 || tile == 128 || tile == 256, "endia_hip_gemm_force_tile: tile %d is not one of 0, 64, 128, 256", tile);
+  ENDIA_CHECK_ARG(tile == 0 || tile == 64 || tile == 128 || tile == 256 || tile == 256128,
+                  "endia_hip_gemm_force_tile: tile %d is not one of 0, 64, 128, 256, 256128", tile);
   g_forced_tile = tile;
   return ENDIA_HIP_OK;
 }
@@ -1006,3 +701,8 @@ extern "C" int32_t endia_hip_gemm_timing_end(int64_t* launches, double* total_ms
   if (total_flops) *total_flops = g_timing.flops;
   return ENDIA_HIP_OK;
 }
+
+#ifdef ENDIA_LONE_STAMPS
+// profiling build only: where the one-wave-per-SIMD kernels leave their per-group wall-clock stamps
+extern "C" __attribute__((visibility("default"))) void* endia_debug_stamps(void) { return endia::ctx().tickets; }
+#endif

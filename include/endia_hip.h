@@ -146,9 +146,9 @@ ENDIA_API int32_t endia_hip_gemm_timing_begin(void);
 ENDIA_API int32_t endia_hip_gemm_timing_end(int64_t* launches, double* total_ms, double* total_flops);
 
 /* Tile choice of the fp32 matrix-core kernels behind endia_hip_sgemm (and everything built on it). No counterpart in the
- * reference: a hook for tests and tuning. tile = 0 (the default) lets every call choose by shape; 64, 128 or 256 makes
- * every later call that runs on the matrix cores use the 64 x 64, 128 x 128 or 256 x 256 tile (all transpose forms and
- * epilogues; a call that no matrix-core kernel takes, e.g. unaligned operands, keeps its own path). Results do not
+ * reference: a hook for tests and tuning. tile = 0 (the default) lets every call choose by shape; 64, 128, 256 or 256128
+ * makes every later call that runs on the matrix cores use the 64 x 64, 128 x 128, 256 x 256 or 256 x 128 tile (all
+ * transpose forms and epilogues; a call that no matrix-core kernel takes, e.g. unaligned operands, keeps its own path). Results do not
  * depend on the tile beyond the order of the additions along K. Process-wide, not thread-safe against concurrent
  * sgemm calls. */
 ENDIA_API int32_t endia_hip_gemm_force_tile(int32_t tile);

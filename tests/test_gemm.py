@@ -352,10 +352,11 @@ def test_sgemm_random_shapes_and_flags(dev):
 @pytest.mark.parametrize("M,N,K", [(256, 256, 32), (256, 512, 64), (300, 520, 70), (516, 260, 1000), (1024, 768, 4100), (260, 1028, 36),
                                    (128, 64, 512), (512, 1024, 1100), (256, 256, 31), (320, 256, 97)])
 def test_sgemm_every_tile_forced(dev, M, N, K):
-    """endia_hip_gemm_force_tile: the weight-gradient form (A stored K x M, B stored K x N) through the 64, 128 and 256
-    tiles on shapes with ragged edges in M, N and K (the 256 x 256 tile is otherwise only chosen for products that fill
-    every CU with one): every tile against the oracle and float64, plain and accumulating, a padded C, a batch; all four
-    forms and every fused epilogue through the 256 tile."""
+    """endia_hip_gemm_force_tile: the weight-gradient form (A stored K x M, B stored K x N) through the 64, 128, 256 x 256
+    and 256 x 128 tiles on shapes with ragged edges in M, N and K (the two one-wave-per-SIMD tiles are otherwise only
+    chosen for products that fill every CU with one): every tile against the oracle and float64, plain and accumulating,
+    a padded C, a batch; all four forms and every fused epilogue (also sin with the stored pre-activation, and cos as its
+    gradient, the Hessian-vector benchmark's epilogues) through the 128, 256 x 256 and 256 x 128 tiles."""
     rng = np.random.default_rng(M + 3 * N + 7 * K)
     A = rng.standard_normal((K, M)).astype(np.float32)
     B = (rng.standard_normal((K, N)) / np.sqrt(K)).astype(np.float32)
@@ -363,7 +364,7 @@ def test_sgemm_every_tile_forced(dev, M, N, K):
     want = R.matmul(np.ascontiguousarray(A.T), B)
     C0 = rng.standard_normal((M, N)).astype(np.float32)
     try:
-        for tile in (64, 128, 256):
+        for tile in (64, 128, 256, 256128):
             dev.call("endia_hip_gemm_force_tile", tile)
             got = run_sgemm(dev, A, B, 1, 0, M, N, K)
             assert_close(got, want, what="tile %d vs oracle" % tile)
@@ -388,7 +389,7 @@ def test_sgemm_every_tile_forced(dev, M, N, K):
         At, Bt = np.ascontiguousarray(A.T), np.ascontiguousarray(B.T)
         bias = rng.standard_normal(N).astype(np.float32)
         aux = rng.standard_normal((M, N)).astype(np.float32)
-        for tile, ta, tb, a, b in [(t,) + f for t in (128, 256) for f in ((0, 0, At, B), (0, 1, At, Bt), (1, 1, A, Bt), (1, 0, A, B))]:
+        for tile, ta, tb, a, b in [(t,) + f for t in (128, 256, 256128) for f in ((0, 0, At, B), (0, 1, At, Bt), (1, 1, A, Bt), (1, 0, A, B))]:
             if K % 4 and (not ta or tb):
                 continue  # a K-major operand needs K in whole 16-byte pieces for the matrix-core path
             dev.call("endia_hip_gemm_force_tile", tile)
@@ -401,6 +402,11 @@ def test_sgemm_every_tile_forced(dev, M, N, K):
             assert_close(run_sgemm(dev, a, b, ta, tb, M, N, K, L.EPI_ACT_GRAD, L.OP_RELU, aux=aux), ref * (aux > 0), what=what + "relu gradient")
             assert_close(run_sgemm(dev, a, b, ta, tb, M, N, K, L.EPI_ACT_GRAD, L.OP_TANH | L.ACT_FROM_OUTPUT, aux=np.tanh(aux)),
                          ref * (1 - np.tanh(aux.astype(np.float64)) ** 2), what=what + "tanh gradient from the output")
+            Cs, Zs = run_sgemm(dev, a, b, ta, tb, M, N, K, L.EPI_BIAS_ACT, L.OP_SIN, bias=bias, want_z=True)
+            assert_close(Zs, ref + bias, what=what + "stored pre-activation (sin)")
+            assert_close(Cs, np.sin(ref + bias), tol=2e-4 if K > 2000 else 1e-4, what=what + "bias + sin")  # (sin of sums of size sqrt(K))
+            assert_close(run_sgemm(dev, a, b, ta, tb, M, N, K, L.EPI_ACT_GRAD, L.OP_SIN, aux=aux), ref * np.cos(aux.astype(np.float64)),
+                         what=what + "sin gradient from the pre-activation")
         dev.call("endia_hip_gemm_force_tile", 256)
         # the column sums of B from the same call (the bias gradient beside the weight gradient), small and large B
         dC, dsum = dev.put(np.full((M, N), np.nan, np.float32)), dev.put(np.full(N, np.nan, np.float32))
