@@ -41,6 +41,17 @@ def contiguous(x):
 
 
 _fusion = None  # set by endia_amd.fusion: while it traces a function, ops on its symbols build an expression
+_fused_rules = {}
+
+
+def _fused_rule(name, fn):
+    """A VJP rule written in elementwise ops, as ONE differentiable fused launch (endia_amd.fusion). Used by passes that
+    record their own graph (create_graph=True): the reference records two to four elementwise nodes per rule there
+    (e.g. cos and mul for sin_op.mojo:92), and a second-order pass then pays one launch per node and per node's rule."""
+    f = _fused_rules.get(name)
+    if f is None:
+        f = _fused_rules[name] = _fusion.fuse(fn, name)
+    return f
 
 
 def detach(x):
@@ -689,6 +700,11 @@ def _unary(op, name, x, vjp):
         # create_graph pass records. An ordinary pass computes the same g * op'(x) with the one kernel made for it.
         from .autograd.functional import building_graph
         p = primals[0]
+        if building_graph() and not (p.is_complex_ or grad.is_complex_ or op in _NO_VJP_KERNEL or grad._shape != p._shape or not p.size()):
+            try:  # the same rule, recorded as one fused node
+                return [_fused_rule("vjp_" + name, lambda x, g, o: vjp([x], g, o)[0])(p, grad, out_)]
+            except _fusion.FusionError:
+                return vjp(primals, grad, out_)
         if building_graph() or p.is_complex_ or grad.is_complex_ or op in _NO_VJP_KERNEL or grad._shape != p._shape or not p.size():
             return vjp(primals, grad, out_)
         g, xs_ = contiguous(grad), contiguous(p)
@@ -1394,6 +1410,8 @@ def _sin_of_linear_node(out, zz):
     def vjp(primals, grad, out_):
         from .autograd.functional import building_graph
         z = primals[0]
+        if building_graph() and grad._shape == z._shape:
+            return [_fused_rule("cos_mul", lambda zz_, g: mul(cos(zz_), g))(z, grad)]  # sin_op.mojo:92 as one node
         if building_graph() or grad.ndim() != out_.ndim():  # (a Jacobian seed's leading axes broadcast through mul)
             return [mul(cos(z), grad)]  # sin_op.mojo:92
         if grad._act_applied:
@@ -1415,7 +1433,11 @@ def _linear_node(out, x, W, b, xs, Ws, act):
         px, pW, pb = primals
         lead = grad.ndim() - out_.ndim()  # leading axes of a Jacobian seed (autograd/functional.mojo:35-37)
         if building_graph() or lead:
-            if act == "tanh":
+            if act == "tanh" and not lead:
+                g = _fused_rule("tanh_out_mul", lambda o, gg: mul(1 - square(o), gg))(out_, grad)
+            elif act == "relu" and not lead:
+                g = _fused_rule("relu_out_mul", lambda o, gg: mul(greater(o, 0.0), gg))(out_, grad)
+            elif act == "tanh":
                 g = mul(1 - square(out_), grad)                      # tanh_op.mojo:92 with tanh(z) = out
             elif act == "relu":
                 g = mul(greater(out_, zeros([N])), grad)             # relu_op.mojo:95; out > 0 iff z > 0

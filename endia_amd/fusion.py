@@ -256,12 +256,13 @@ def _replay(node, env, cache):
         v = _UNARY_FN[node.op](_replay(node.args[0], env, cache))
     else:
         a, b = (_replay(x, env, cache) for x in node.args)
-        if not isinstance(a, Array) and not isinstance(b, Array):
-            a = F.full([1], a)
-        if not isinstance(a, Array):
-            a = F.full([b._shape[-1]], a)
-        if not isinstance(b, Array):
-            b = F.full([a._shape[-1]], b)
+        if not isinstance(a, Sym) and not isinstance(b, Sym):  # (inside a trace, numbers become immediates)
+            if not isinstance(a, Array) and not isinstance(b, Array):
+                a = F.full([1], a)
+            if not isinstance(a, Array):
+                a = F.full([b._shape[-1]], a)
+            if not isinstance(b, Array):
+                b = F.full([a._shape[-1]], b)
         v = _BINARY_FN[node.op](a, b)
     cache[node.id] = v
     return v
@@ -354,7 +355,25 @@ class FusedElementwise:
             res = [None] * len(primals)
             if not plan.wanted:
                 return res
-            if building_graph() or plan.bwd is None:
+            if list(grad._shape) != shape and grad.size() == _prod(shape):
+                grad = F.reshape(grad, shape)  # kept axes of length 1 in front (the cotangent of a reduction's operand)
+            lead_n = max(0, len(grad._shape) - len(shape))
+            lead = lead_n > 0  # a Jacobian seed's axes in front: the op-by-op rules broadcast over them
+            if building_graph() and not lead:
+                # A pass that records its own graph: every gradient expression becomes a fused function of
+                # (inputs, cotangent, forward output, captured constants), so the recorded node is ONE launch and is
+                # itself differentiable to any order by the same tracing. Expressions that do not fit a program
+                # are replayed op by op.
+                operands = list(primals) + [grad if list(grad._shape) == shape else F.expand(grad, shape), out_] + [c for c, _ in plan.consts]
+                full = []
+                for k, gs in enumerate(plan.grads):
+                    try:
+                        full.append(_gradient_function(plan, k)(*operands))
+                    except FusionError:
+                        env = dict(enumerate(operands))
+                        f = _replay(gs, env, {})
+                        full.append(f if isinstance(f, Array) else F.full(shape, f))
+            elif plan.bwd is None or lead or building_graph():
                 env = {i: p for i, p in enumerate(primals)}
                 env[plan.n] = grad
                 env[plan.n + 1] = out_
@@ -372,16 +391,32 @@ class FusedElementwise:
                     _launch(rows, cols, bins, bmodes, full, plan.bwd)
             for i, f in zip(plan.wanted, full):
                 p = primals[i]
-                if list(f._shape) != list(p._shape):
+                own = list(f._shape)[lead_n:]  # the expression's own axes, behind those of a Jacobian seed
+                if own != list(p._shape):
                     # a broadcast input: sum over the axes it was spread along, keeping them as size 1 like
                     # the VJP of the reference's expand (expand_op.mojo:121-126)
-                    lead = len(f._shape) - len(p._shape)
-                    axes = [k for k in range(len(f._shape)) if k < lead or p._shape[k - lead] != f._shape[k]]
+                    extra = len(own) - len(p._shape)
+                    axes = [lead_n + k for k in range(len(own)) if k < extra or p._shape[k - extra] != own[k]]
                     f = F.reduce_add(f, axes)
                 res[i] = f
             return res
 
         return F._register(out, arrays, "fused:" + self.name, vjp)
+
+
+def _gradient_function(plan, k):
+    """The k-th gradient expression of a traced plan as a fused function of its operands, in the order
+    (inputs..., cotangent, forward output, constants...): operand i is what the expression calls input i."""
+    cache = plan.__dict__.setdefault("grad_fns", {})
+    fn = cache.get(k)
+    if fn is None:
+        expr = plan.grads[k]
+
+        def rebuilt(*syms):  # the forward output is an operand: no need to evaluate its expression again
+            return _replay(expr, dict(enumerate(syms)), {plan.root.id: syms[plan.n + 1]})
+
+        fn = cache[k] = FusedElementwise(rebuilt, "grad%d" % k)
+    return fn
 
 
 def _bshape(sa, sb):
