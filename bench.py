@@ -52,7 +52,8 @@ def build_wide_mlp(nd, width=4096, layers=8, batch=4096, seed=2):
 def build_sine_mlp(nd, seed=0, optimizer="sgd"):
     rng = np.random.default_rng(seed)
     widths = [1, 32, 64, 128, 128, 128, 64, 32, 1]
-    mlp = nd.nn.MLP(widths, compute_backward=True, activation="relu", fused=True)
+    # fused="model": the whole stack is one op (one launch forward, two backward); "layer" keeps one op per layer
+    mlp = nd.nn.MLP(widths, compute_backward=True, activation="relu", fused=True if os.environ.get("ENDIA_SINE_PER_LAYER") else "model")
     for i in range(8):
         s = np.sqrt(2.0 / widths[i])
         mlp.weights[i] = nd.array((rng.standard_normal((widths[i], widths[i + 1])) * s).astype(np.float32), requires_grad=True)

@@ -57,6 +57,11 @@ class PoolDesc(ctypes.Structure):
 
 
 POOL_MAX, POOL_AVG = 0, 1
+MLP_MAX_LAYERS, MLP_MAX_WIDTH = 16, 128
+
+
+class MlpDesc(ctypes.Structure):
+    _fields_ = [("layers", c_int32), ("act", c_int32), ("batch", c_int64), ("widths", c_int64 * (MLP_MAX_LAYERS + 1))]
 
 _fp = c_void_p  # device pointers travel as plain addresses
 _i64p = POINTER(c_int64)
@@ -90,6 +95,9 @@ SIGNATURES = {
     "endia_hip_sgemm": [c_int32, c_int32, c_int64, c_int64, c_int64, _fp, c_int64, _fp, c_int64, _fp, c_int64,
                         c_int64, c_int64, c_int64, c_int64, c_int32, c_int32, _fp, _fp, _fp],
     "endia_hip_linear_bwd": [c_int64, c_int64, c_int64, _fp, _fp, _fp, c_int32, _fp, _fp, _fp, _fp],
+    "endia_hip_mlp_fwd": [POINTER(MlpDesc), _fp, POINTER(c_void_p), POINTER(c_void_p), POINTER(c_void_p)],
+    "endia_hip_mlp_bwd": [POINTER(MlpDesc), _fp, POINTER(c_void_p), POINTER(c_void_p), POINTER(c_void_p), POINTER(c_void_p),
+                          POINTER(c_void_p), _fp],
     "endia_hip_cgemm": [c_int32, c_int32, c_int32, c_int32, c_int64, c_int64, c_int64, _fp, c_int64, _fp, c_int64,
                         _fp, c_int64, c_int64, c_int64, c_int64, c_int64, c_int32, c_int32],
     "endia_hip_unary_fwd": [c_int32, c_int64, _fp, _fp, c_int32],

@@ -1,0 +1,489 @@
+// A whole small dense model per launch: nn.MLP.forward (endia/nn/modules/_mlp.mojo:47-53) and its backward pass.
+//
+// The reference's own benchmark model (benchmarks/mlp_benchmarks/mlp_imp.mojo:35-75: widths 1-32-64-128-128-128-64-32-1,
+// batch 128) is eight products of a few hundred kilo-flops each. One kernel per layer makes a training step a chain of
+// ~19 dependent launches whose cost is the launches. But every row of the batch is independent through all layers, in
+// the forward pass and in the chain of cotangents alike, so for layers of at most 128 units:
+//   mlp_fwd_kernel    one work-group (8 waves) owns 16 rows and runs ALL layers back to back: activations stay in LDS,
+//                     the weights (a few tens of KiB, resident in L2) go straight from memory into the B operands of
+//                     v_mfma_f32_16x16x4_f32, the next layer's while the current layer computes;
+//   mlp_delta_kernel  the same for the cotangents delta_{l-1} = (delta_l W_l^T) * act'(h_{l-1});
+//   mlp_wgrad_kernel  dW_l = h_{l-1}^T delta_l and db_l = 1^T delta_l for ALL layers in one launch, one wave per
+//                     16 x 16 block of a gradient, rows of the batch in ascending order (results repeat bit for bit).
+// No work-group ever waits for another.
+//
+// MFMA 16x16x4: A is 16 x 4 (lane: row = lane % 16, k = lane / 16), B is 4 x 16 (lane: column = lane % 16, k = lane / 16),
+// the accumulator holds rows 4 * (lane / 16) + v, v = 0..3, of column lane % 16. A sum over k may be taken in any
+// order: "super-step" t of a reduction uses k = 16 t + 4 g + i (g = lane / 16) in its MFMA i = 0..3, so that a lane's
+// four A values are one 16-byte LDS read.
+#include "common.h"
+#include "mfma_tile.h"
+
+namespace {
+
+using mfma::buffer_load_f1;
+using mfma::buffer_load_f4;
+using mfma::make_rsrc;
+using mfma::OOB_OFFSET;
+
+typedef float floatx4 __attribute__((ext_vector_type(4)));
+
+constexpr int ROWS = 16;        // rows of the batch per work-group
+constexpr int MAXW = ENDIA_MLP_MAX_WIDTH;
+constexpr int LD = MAXW + 4;    // LDS row stride: 16 rows x 16-byte reads fall into distinct banks
+constexpr int MAXT = MAXW / 16; // super-steps of a full-width reduction
+constexpr int NW = 8;             // waves per work-group of the two row-block kernels (4 were measured slower: 22 -> 16 us for the chain of cotangents)
+constexpr int SLOTS = MAXW / 16 / NW;  // 16-column blocks per wave
+
+struct MlpArgs {
+  int layers, act, batch;
+  int width[ENDIA_MLP_MAX_LAYERS + 1];
+  const float* W[ENDIA_MLP_MAX_LAYERS];
+  const float* b[ENDIA_MLP_MAX_LAYERS];
+  float* h[ENDIA_MLP_MAX_LAYERS];      // forward: outputs; backward: the stored activations
+  float* delta[ENDIA_MLP_MAX_LAYERS];  // backward: cotangents of the pre-activations (delta[layers - 1] is the incoming one)
+  float* dW[ENDIA_MLP_MAX_LAYERS];
+  float* db[ENDIA_MLP_MAX_LAYERS];
+  const float* x;
+  float* dx;
+#ifdef ENDIA_MLP_STAMPS
+  unsigned long long* stamps;  // profiling build: wall-clock stamps of work-group 0
+#endif
+};
+#ifdef ENDIA_MLP_STAMPS
+#define MLP_STAMP(i) do { if (blockIdx.x == 0 && threadIdx.x == 0) p.stamps[i] = wall_clock64(); } while (0)
+#else
+#define MLP_STAMP(i) do { } while (0)
+#endif
+
+__device__ __forceinline__ float act_apply(int act, float z) {
+  return act == ENDIA_OP_RELU ? (z > 0.f ? z : 0.f) : (act == ENDIA_OP_TANH ? tanhf(z) : z);
+}
+// derivative from the stored OUTPUT h = act(z): relu' = [h > 0] (relu_op.mojo:95: z > 0 iff h > 0), tanh' = 1 - h^2 (tanh_op.mojo:92)
+__device__ __forceinline__ float act_slope(int act, float h) {
+  return act == ENDIA_OP_RELU ? (h > 0.f ? 1.f : 0.f) : (act == ENDIA_OP_TANH ? 1.f - h * h : 1.f);
+}
+
+// B operands of one layer for this wave: element [t][s][i] multiplies k = 16 t + 4 g + i into column 16 (wave + 4 s) + c.
+// TRANSPOSED reads W^T: the reduction runs over W's columns and the output column is W's row.
+struct WFrag {
+  float v[MAXT][SLOTS][4];
+};
+
+// Loader of one layer's B operands. Every load is a buffer load whose offset is out of range where the element does
+// not exist (it then reads as zero): no branch and no wait sits between two loads, so a layer's 16 to 64 requests per
+// lane are all in flight together, and they are issued one super-step at a time between the MFMAs of the layer that is
+// being computed. Per request the lane's offset costs at most one addition: the lane-dependent part is fixed per layer.
+// The transposed form reads four consecutive floats of a row of W per request when rows are whole 16-byte pieces.
+template <bool TRANSPOSED>
+struct WLoader {
+  __amdgpu_buffer_rsrc_t rs;
+  uint32_t voff[SLOTS], voff_tail[SLOTS];
+  int red, N, g4;
+  bool vec, any;
+  // plain: out = in[., K] W[K, N]: reduction index k < K, column n < N.  transposed: out = in[., N] W^T: reduction n < N, column k < K.
+  __device__ __forceinline__ void init(const float* __restrict__ W, int K, int N_, int wave, int c, int g) {
+    any = W != nullptr;
+    N = N_;
+    g4 = 4 * g;
+    red = TRANSPOSED ? N : K;
+    const int cols = TRANSPOSED ? K : N;
+    rs = make_rsrc(W, any ? (int64_t)K * N * 4 : 0);
+    vec = TRANSPOSED && (N & 3) == 0 && (reinterpret_cast<uintptr_t>(W) & 15) == 0;
+#pragma unroll
+    for (int s = 0; s < SLOTS; ++s) {
+      const int col = 16 * (wave + NW * s) + c;
+      // rows of the plain form past K lie past the end of the buffer; the transposed form would run into the next
+      // row of W instead, so its last, partial super-step has offsets of its own
+      voff[s] = col < cols ? (uint32_t)((TRANSPOSED ? col * N + 4 * g : 4 * g * N + col) * 4) : OOB_OFFSET;
+      voff_tail[s] = 4 * g < (N & 15) ? voff[s] : OOB_OFFSET;
+    }
+  }
+  __device__ __forceinline__ void load_step(WFrag& f, int t) const {
+    if (!any || 16 * t >= red) return;
+#pragma unroll
+    for (int s = 0; s < SLOTS; ++s) {
+      if (!TRANSPOSED) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) f.v[t][s][i] = buffer_load_f1(rs, voff[s] + (uint32_t)((16 * t + i) * N * 4));
+      } else if (vec) {
+        const float4 w = buffer_load_f4(rs, (16 * t + 16 <= N ? voff[s] : voff_tail[s]) + (uint32_t)(64 * t));
+        f.v[t][s][0] = w.x; f.v[t][s][1] = w.y; f.v[t][s][2] = w.z; f.v[t][s][3] = w.w;
+      } else {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {  // rows of W that are not whole 16-byte pieces: element by element, the tail tested per lane
+          f.v[t][s][i] = buffer_load_f1(rs, 16 * t + i + g4 < N ? voff[s] + (uint32_t)((16 * t + i) * 4) : OOB_OFFSET);
+        }
+      }
+    }
+  }
+};
+
+// acc[s] = in[16 x red] (LDS) . cur, for the wave's column blocks; between the super-steps, the requests for `nxt`
+template <bool TRANSPOSED>
+__device__ __forceinline__ void layer_mfma(const float* __restrict__ in, const WFrag& cur, int red, int cols, int wave, int c, int g,
+                                           floatx4 (&acc)[SLOTS], const WLoader<TRANSPOSED>& next, WFrag& nxt) {
+#pragma unroll
+  for (int s = 0; s < SLOTS; ++s) acc[s] = floatx4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+  for (int t = 0; t < MAXT; ++t) {
+    next.load_step(nxt, t);
+    if (16 * t < red) {
+      const float4 a = *reinterpret_cast<const float4*>(&in[c * LD + 16 * t + 4 * g]);
+      const float av[4] = {a.x, a.y, a.z, a.w};
+      // (four MFMAs in a row into the same accumulator: measured twice as fast as alternating between the column blocks)
+#pragma unroll
+      for (int s = 0; s < SLOTS; ++s)
+        if (16 * (wave + NW * s) < cols) {
+#pragma unroll
+          for (int i = 0; i < 4; ++i) acc[s] = __builtin_amdgcn_mfma_f32_16x16x4f32(av[i], cur.v[t][s][i], acc[s], 0, 0, 0);
+        }
+    }
+  }
+}
+
+// Stage 16 rows of a [batch, width] array into LDS, zero beyond the array's rows and up to the next multiple of 16
+// columns (a reduction reads whole super-steps of 16; everything else in LDS is written before it is read).
+__device__ __forceinline__ void stage_rows(float* __restrict__ dst, const float* __restrict__ src, int row0, int batch, int width, int tid) {
+  const int padded = (width + 15) & ~15;
+  for (int e = tid; e < ROWS * padded; e += 64 * NW) {
+    const int r = e / padded, k = e - r * padded;
+    dst[r * LD + k] = (row0 + r < batch && k < width) ? src[(int64_t)(row0 + r) * width + k] : 0.f;
+  }
+}
+
+// Forward layers whose rows of W are whole 16-byte pieces read W sixteen bytes per lane: a wave owns 64 consecutive
+// output columns as four MFMA blocks whose column c is output column 4 c + j (j = block), so that a lane's four B values
+// of one reduction index are four neighbouring floats of a row of W, and a request of the wave covers whole rows (1 KiB)
+// instead of sixteen floats of each of four rows. The NW waves share the two column groups of a layer and split its
+// reduction: wave w takes group w % groups and the super-steps t = w / groups (mod NW / groups); the partial sums meet
+// in LDS, where bias and activation are applied. (Other layers, e.g. a 1-wide last one, take the plan of WLoader.)
+struct VFrag {
+  float4 b[2][4];  // [u][i]: super-step t = q + parts * u, reduction index 16 t + 4 g + i
+};
+constexpr int PLD = MAXW + 4;  // row stride of the partial sums
+
+struct VPlan {
+  __amdgpu_buffer_rsrc_t rs;
+  uint32_t voff;
+  int K, N, G, q, parts;
+  bool vec;
+  __device__ __forceinline__ void init(const float* __restrict__ W, int K_, int N_, int wave, int c, int g) {
+    K = K_;
+    N = N_;
+    vec = W != nullptr && (N & 3) == 0 && (reinterpret_cast<uintptr_t>(W) & 15) == 0;
+    const int groups = (N + 63) / 64;
+    parts = NW / groups;
+    G = wave % groups;
+    q = wave / groups;
+    rs = make_rsrc(W, vec ? (int64_t)K * N * 4 : 0);
+    const int col = 64 * G + 4 * c;
+    voff = col < N ? (uint32_t)((4 * g * N + col) * 4) : OOB_OFFSET;  // rows past K lie past the end of the buffer
+  }
+  __device__ __forceinline__ void request(VFrag& f) const {
+#pragma unroll
+    for (int u = 0; u < 2; ++u) {
+      const int t = q + parts * u;
+      if (16 * t < K) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) f.b[u][i] = buffer_load_f4(rs, voff + (uint32_t)((16 * t + i) * N * 4));
+      }
+    }
+  }
+};
+
+__global__ __launch_bounds__(64 * NW, 1) void mlp_fwd_kernel(MlpArgs p) {
+  static_assert(NW == 8 && SLOTS == 1 && MAXW == 128, "the reduction split below is written for eight waves and two column groups");
+  __shared__ __attribute__((aligned(16))) float hs[2][ROWS * LD];
+  __shared__ __attribute__((aligned(16))) float part[NW * ROWS * PLD];
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, c = lane & 15, g = lane >> 4;
+  const int row0 = blockIdx.x * ROWS;
+  MLP_STAMP(0);
+  WFrag cur_s, nxt_s;
+  VFrag cur_v, nxt_v;
+  WLoader<false> loader;
+  VPlan plan, plan_next;
+  // what a thread adds when the partial sums meet: four neighbouring bias values (16-byte layers) or its block's one
+  float4 bias4_cur, bias4_nxt;
+  float bias1_cur, bias1_nxt;
+  const int er = tid >> 5, en = (tid & 31) * 4;  // the four outputs a thread finishes in a 16-byte layer: row er, columns en .. en + 3
+  auto request_layer = [&](int l, VPlan& pl, VFrag& fv, WFrag& fs, float4& b4, float& b1) {
+    pl.init(p.W[l], p.width[l], p.width[l + 1], wave, c, g);
+    const __amdgpu_buffer_rsrc_t rb = make_rsrc(p.b[l], (int64_t)p.width[l + 1] * 4);
+    if (pl.vec) {
+      pl.request(fv);
+      b4 = buffer_load_f4(rb, (uint32_t)(en * 4));  // (columns past the width read as zero and are never stored)
+    } else {
+      loader.init(p.W[l], p.width[l], p.width[l + 1], wave, c, g);
+#pragma unroll
+      for (int t = 0; t < MAXT; ++t) loader.load_step(fs, t);
+      b1 = buffer_load_f1(rb, (uint32_t)((16 * wave + c) * 4));
+    }
+  };
+  request_layer(0, plan, cur_v, cur_s, bias4_cur, bias1_cur);  // the first layer's weights travel while the input is staged
+  stage_rows(hs[0], p.x, row0, p.batch, p.width[0], tid);
+  __syncthreads();
+  MLP_STAMP(1);
+  for (int l = 0; l < p.layers; ++l) {
+    MLP_STAMP(2 + 2 * l);
+    const int K = p.width[l], N = p.width[l + 1];
+    const bool last = l + 1 == p.layers;
+    if (!last) request_layer(l + 1, plan_next, nxt_v, nxt_s, bias4_nxt, bias1_nxt);  // travels while this layer computes
+    const float* in = hs[l & 1];
+    float* out = hs[(l & 1) ^ 1];
+    if (plan.vec) {
+      floatx4 acc[4];
+#pragma unroll
+      for (int j = 0; j < 4; ++j) acc[j] = floatx4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int u = 0; u < 2; ++u) {
+        const int t = plan.q + plan.parts * u;
+        if (16 * t < K) {
+          const float4 a = *reinterpret_cast<const float4*>(&in[c * LD + 16 * t + 4 * g]);
+          const float av[4] = {a.x, a.y, a.z, a.w};
+#pragma unroll
+          for (int j = 0; j < 4; ++j)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+              const float bj = j == 0 ? cur_v.b[u][i].x : (j == 1 ? cur_v.b[u][i].y : (j == 2 ? cur_v.b[u][i].z : cur_v.b[u][i].w));
+              acc[j] = __builtin_amdgcn_mfma_f32_16x16x4f32(av[i], bj, acc[j], 0, 0, 0);
+            }
+        }
+      }
+      MLP_STAMP(3 + 2 * l);
+      if (64 * plan.G < N) {
+#pragma unroll
+        for (int v = 0; v < 4; ++v)
+          *reinterpret_cast<float4*>(&part[(plan.q * ROWS + 4 * g + v) * PLD + 64 * plan.G + 4 * c]) =
+              make_float4(acc[0][v], acc[1][v], acc[2][v], acc[3][v]);
+      }
+      __syncthreads();
+      const int npad = (N + 15) & ~15;
+      if (en < npad) {
+        float4 z = bias4_cur;
+        for (int qq = 0; qq < plan.parts; ++qq) {  // partial sums in the order of their reduction ranges
+          const float4 t4 = *reinterpret_cast<const float4*>(&part[(qq * ROWS + er) * PLD + en]);
+          z.x += t4.x; z.y += t4.y; z.z += t4.z; z.w += t4.w;
+        }
+        if (!last) {
+          z.x = act_apply(p.act, z.x); z.y = act_apply(p.act, z.y); z.z = act_apply(p.act, z.z); z.w = act_apply(p.act, z.w);
+        }
+        if (en >= N) z = make_float4(0.f, 0.f, 0.f, 0.f);  // columns past the width feed the next reduction as zeros
+        *reinterpret_cast<float4*>(&out[er * LD + en]) = z;
+        if (en < N && row0 + er < p.batch) *reinterpret_cast<float4*>(&p.h[l][(int64_t)(row0 + er) * N + en]) = z;
+      }
+    } else {
+      floatx4 acc[SLOTS];
+      WLoader<false> none;
+      none.init(nullptr, 1, 1, wave, c, g);
+      layer_mfma<false>(in, cur_s, K, N, wave, c, g, acc, none, nxt_s);
+      MLP_STAMP(3 + 2 * l);
+      const int col = 16 * wave + c;
+      if (16 * wave < N) {
+#pragma unroll
+        for (int v = 0; v < 4; ++v) {
+          const int r = 4 * g + v;
+          float z = acc[0][v] + bias1_cur;
+          if (!last) z = act_apply(p.act, z);
+          if (col >= N) z = 0.f;  // the block's columns past the layer's width feed the next reduction as zeros
+          out[r * LD + col] = z;
+          if (col < N && row0 + r < p.batch) p.h[l][(int64_t)(row0 + r) * N + col] = z;
+        }
+      }
+    }
+    __syncthreads();
+    if (!last) {  // (the requests above have had the whole layer to arrive)
+      plan = plan_next;
+      cur_v = nxt_v;
+      cur_s = nxt_s;
+      bias4_cur = bias4_nxt;
+      bias1_cur = bias1_nxt;
+    }
+  }
+}
+
+// delta[layers - 1] holds the incoming cotangent (the last layer has no activation). For l = layers - 1 .. 1:
+// delta[l - 1] = (delta[l] W_l^T) * act'(h[l - 1]); finally dx = delta[0] W_0^T when asked for.
+__global__ __launch_bounds__(64 * NW, 1) void mlp_delta_kernel(MlpArgs p) {
+  __shared__ __attribute__((aligned(16))) float ds[2][ROWS * LD];
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, c = lane & 15, g = lane >> 4;
+  const int row0 = blockIdx.x * ROWS;
+  const int L = p.layers;
+  const int first = p.dx ? 0 : 1;  // lowest layer whose W^T is applied
+  if (L - 1 < first) return;
+  WFrag cur, nxt;
+  WLoader<true> loader;
+  loader.init(p.W[L - 1], p.width[L - 1], p.width[L], wave, c, g);
+#pragma unroll
+  for (int t = 0; t < MAXT; ++t) loader.load_step(cur, t);
+  stage_rows(ds[0], p.delta[L - 1], row0, p.batch, p.width[L], tid);
+  __syncthreads();
+  int buf = 0;
+  for (int l = L - 1; l >= first; --l) {
+    const int K = p.width[l], N = p.width[l + 1];  // W_l is K x N; the product is [rows, N] . [N, K]
+    const bool more = l - 1 >= first;
+    loader.init(more ? p.W[l - 1] : nullptr, more ? p.width[l - 1] : 1, p.width[l], wave, c, g);
+    // outputs of the activation that produced this layer's input (none below the first layer)
+    float hprev[SLOTS][4];
+    const __amdgpu_buffer_rsrc_t rh = make_rsrc(l > 0 ? p.h[l - 1] : p.x, l > 0 ? (int64_t)p.batch * K * 4 : 0);
+#pragma unroll
+    for (int s = 0; s < SLOTS; ++s)
+#pragma unroll
+      for (int v = 0; v < 4; ++v) {
+        const int col = 16 * (wave + NW * s) + c, r = row0 + 4 * g + v;
+        hprev[s][v] = buffer_load_f1(rh, (l > 0 && col < K && r < p.batch) ? (uint32_t)((r * K + col) * 4) : OOB_OFFSET);
+      }
+    floatx4 acc[SLOTS];
+    layer_mfma<true>(ds[buf], cur, N, K, wave, c, g, acc, loader, nxt);
+    float* out = ds[buf ^ 1];
+    float* dst = l > 0 ? p.delta[l - 1] : p.dx;
+#pragma unroll
+    for (int s = 0; s < SLOTS; ++s) {
+      const int col = 16 * (wave + NW * s) + c;
+      if (16 * (wave + NW * s) < K) {
+#pragma unroll
+        for (int v = 0; v < 4; ++v) {
+          const int r = 4 * g + v;
+          float d = col < K ? acc[s][v] * (l > 0 ? act_slope(p.act, hprev[s][v]) : 1.f) : 0.f;
+          out[r * LD + col] = d;
+          if (col < K && row0 + r < p.batch) dst[(int64_t)(row0 + r) * K + col] = d;
+        }
+      }
+    }
+    __syncthreads();
+    buf ^= 1;
+    if (more) cur = nxt;
+  }
+}
+
+// One wave per 16 x 16 block of dW_l, plus one block row per layer for db_l (a left operand of ones).
+__global__ __launch_bounds__(256) void mlp_wgrad_kernel(MlpArgs p) {
+  const int lane = threadIdx.x & 63, c = lane & 15, g = lane >> 4;
+  int blk = blockIdx.x * 4 + (threadIdx.x >> 6);
+  int l = 0, nbk = 0, nbn = 0;
+  for (; l < p.layers; ++l) {
+    nbk = (p.width[l] + 15) / 16 + 1;
+    nbn = (p.width[l + 1] + 15) / 16;
+    if (blk < nbk * nbn) break;
+    blk -= nbk * nbn;
+  }
+  if (l == p.layers) return;
+  const int K = p.width[l], N = p.width[l + 1];
+  const int bk = blk / nbn, bn = blk - bk * nbn;
+  const bool bias_row = bk == nbk - 1;
+  const float* __restrict__ hp = l == 0 ? p.x : p.h[l - 1];  // [batch, K]
+  const float* __restrict__ dl = p.delta[l];                 // [batch, N]
+  const int m = 16 * bk + c, n = 16 * bn + c;
+  floatx4 acc = {0.f, 0.f, 0.f, 0.f};
+  const __amdgpu_buffer_rsrc_t ra = make_rsrc(hp, (int64_t)p.batch * K * 4), rb = make_rsrc(dl, (int64_t)p.batch * N * 4);
+  const uint32_t va = m < K ? (uint32_t)((4 * g * K + m) * 4) : OOB_OFFSET, vb = n < N ? (uint32_t)((4 * g * N + n) * 4) : OOB_OFFSET;
+  constexpr int WGS = 4;
+  for (int t0 = 0; t0 < p.batch; t0 += 16 * WGS) {  // WGS super-steps' loads in flight at once, no branch between them
+    float a[WGS][4], b[WGS][4];
+#pragma unroll
+    for (int t = 0; t < WGS; ++t)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const int r = t0 + 16 * t + 4 * g + i;
+        const bool in = r < p.batch;
+        // (rows past the batch lie past the end of both buffers and read as zero)
+        a[t][i] = bias_row ? (in ? 1.f : 0.f) : buffer_load_f1(ra, va + (uint32_t)((t0 + 16 * t + i) * K * 4));
+        b[t][i] = buffer_load_f1(rb, vb + (uint32_t)((t0 + 16 * t + i) * N * 4));
+      }
+#pragma unroll
+    for (int t = 0; t < WGS; ++t)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) acc = __builtin_amdgcn_mfma_f32_16x16x4f32(a[t][i], b[t][i], acc, 0, 0, 0);
+  }
+  if (n >= N) return;
+  if (bias_row) {
+    if (g == 0 && p.db[l]) p.db[l][n] = acc[0];
+  } else if (p.dW[l]) {
+#pragma unroll
+    for (int v = 0; v < 4; ++v) {
+      const int k = 16 * bk + 4 * g + v;
+      if (k < K) p.dW[l][(int64_t)k * N + n] = acc[v];
+    }
+  }
+}
+
+int32_t fill_args(MlpArgs& a, const endia_hip_mlp_desc* d, const char* who) {
+  ENDIA_CHECK_ARG(d != nullptr, "%s: null descriptor", who);
+  ENDIA_CHECK_ARG(d->layers >= 1 && d->layers <= ENDIA_MLP_MAX_LAYERS, "%s: %d layers, 1..%d supported", who, d->layers, ENDIA_MLP_MAX_LAYERS);
+  ENDIA_CHECK_ARG(d->act == ENDIA_OP_RELU || d->act == ENDIA_OP_TANH || d->act == ENDIA_OP_IDENTITY,
+                  "%s: activation %d is not relu, tanh or identity", who, d->act);
+  ENDIA_CHECK_ARG(d->batch >= 0 && d->batch <= (1 << 20), "%s: batch %lld out of range", who, (long long)d->batch);
+  for (int i = 0; i <= d->layers; ++i)
+    ENDIA_CHECK_ARG(d->widths[i] >= 1 && d->widths[i] <= ENDIA_MLP_MAX_WIDTH, "%s: width %lld of layer boundary %d is not in 1..%d", who,
+                    (long long)d->widths[i], i, ENDIA_MLP_MAX_WIDTH);
+  a = MlpArgs{};
+  a.layers = d->layers;
+  a.act = d->act;
+  a.batch = (int)d->batch;
+  for (int i = 0; i <= d->layers; ++i) a.width[i] = (int)d->widths[i];
+  return ENDIA_HIP_OK;
+}
+
+}  // namespace
+
+using namespace endia;
+
+extern "C" int32_t endia_hip_mlp_fwd(const endia_hip_mlp_desc* desc, const float* x, const float* const* W, const float* const* b,
+                                     float* const* h) {
+  ENDIA_REQUIRE_INIT();
+  MlpArgs a;
+  int32_t rc = fill_args(a, desc, "endia_hip_mlp_fwd");
+  if (rc) return rc;
+  if (a.batch == 0) return ENDIA_HIP_OK;
+  ENDIA_CHECK_ARG(x && W && b && h, "endia_hip_mlp_fwd: null argument");
+  for (int l = 0; l < a.layers; ++l) {
+    ENDIA_CHECK_ARG(W[l] && b[l] && h[l], "endia_hip_mlp_fwd: null pointer for layer %d", l);
+    a.W[l] = W[l];
+    a.b[l] = b[l];
+    a.h[l] = h[l];
+  }
+  a.x = x;
+#ifdef ENDIA_MLP_STAMPS
+  a.stamps = reinterpret_cast<unsigned long long*>(ctx().tickets);
+#endif
+  hipLaunchKernelGGL(mlp_fwd_kernel, dim3((unsigned)ceil_div64(a.batch, ROWS)), dim3(64 * NW), 0, ctx().stream, a);
+  ENDIA_LAUNCH_CHECK();
+  return ENDIA_HIP_OK;
+}
+
+extern "C" int32_t endia_hip_mlp_bwd(const endia_hip_mlp_desc* desc, const float* x, const float* const* W, const float* const* h,
+                                     float* const* delta, float* const* dW, float* const* db, float* dx) {
+  ENDIA_REQUIRE_INIT();
+  MlpArgs a;
+  int32_t rc = fill_args(a, desc, "endia_hip_mlp_bwd");
+  if (rc) return rc;
+  if (a.batch == 0) return ENDIA_HIP_OK;
+  ENDIA_CHECK_ARG(x && W && h && delta && dW && db, "endia_hip_mlp_bwd: null argument");
+  int blocks = 0;
+  for (int l = 0; l < a.layers; ++l) {
+    ENDIA_CHECK_ARG(W[l] && delta[l] && (l + 1 == a.layers || h[l]), "endia_hip_mlp_bwd: null pointer for layer %d", l);
+    a.W[l] = W[l];
+    a.h[l] = const_cast<float*>(h[l]);
+    a.delta[l] = delta[l];
+    a.dW[l] = dW[l];
+    a.db[l] = db[l];
+    blocks += ((a.width[l] + 15) / 16 + 1) * ((a.width[l + 1] + 15) / 16);
+  }
+  a.x = x;
+  a.dx = dx;
+#ifdef ENDIA_MLP_STAMPS
+  a.stamps = reinterpret_cast<unsigned long long*>(ctx().tickets) + 64;
+#endif
+  hipStream_t s = ctx().stream;
+  if (a.layers > 1 || dx) {
+    hipLaunchKernelGGL(mlp_delta_kernel, dim3((unsigned)ceil_div64(a.batch, ROWS)), dim3(64 * NW), 0, s, a);
+    ENDIA_LAUNCH_CHECK();
+  }
+  hipLaunchKernelGGL(mlp_wgrad_kernel, dim3((unsigned)((blocks + 3) / 4)), dim3(256), 0, s, a);
+  ENDIA_LAUNCH_CHECK();
+  return ENDIA_HIP_OK;
+}
+
+#ifdef ENDIA_MLP_STAMPS
+extern "C" __attribute__((visibility("default"))) void* endia_debug_mlp_stamps(void) { return endia::ctx().tickets; }
+#endif

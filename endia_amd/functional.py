@@ -1395,6 +1395,50 @@ def linear(x, W, b, act=None):
     return _linear_node(out, x, W, b, xs, Ws, act)
 
 
+def mlp_forward(x, weights, biases, act=None):
+    """The whole dense stack of nn.MLP.forward (nn/modules/_mlp.mojo:47-53) as ONE op: act after every layer but the
+    last. For small models (every width at most 128, like the reference's benchmark model) the forward pass is one
+    launch and the backward pass two (endia_hip_mlp_fwd / endia_hip_mlp_bwd); anything else, and complex operands, fall
+    back to one fused layer at a time. First order only: a pass with create_graph=True, or a non-scalar output's
+    Jacobian seed, needs the per-layer graph (`nn.MLP(fused=True)`) and is refused here."""
+    import ctypes
+    Lyr = len(weights)
+    widths = [x._shape[-1]] + [w._shape[1] for w in weights]
+    small = (x.ndim() == 2 and 1 <= Lyr <= L.MLP_MAX_LAYERS and act in (None, "identity", "relu", "tanh") and x.size() > 0
+             and not x.is_complex_ and all(1 <= n <= L.MLP_MAX_WIDTH for n in widths)
+             and all(w.ndim() == 2 and not w.is_complex_ and w._shape[0] == widths[i] for i, w in enumerate(weights))
+             and all(b.size() == widths[i + 1] and not b.is_complex_ for i, b in enumerate(biases)))
+    if not small:
+        h = x
+        for i in range(Lyr):
+            h = linear(h, weights[i], biases[i], None if i == Lyr - 1 else act)
+        return h
+    B = x._shape[0]
+    xs = contiguous(x)
+    Ws, bs_ = [contiguous(w) for w in weights], [contiguous(b) for b in biases]
+    hs = [Array.empty([B, widths[i + 1]]) for i in range(Lyr)]
+    desc = L.MlpDesc()
+    desc.layers, desc.act, desc.batch = Lyr, _ACT[act], B
+    desc.widths[:Lyr + 1] = widths
+    ptrs = lambda arrs: (ctypes.c_void_p * Lyr)(*[a.data_ptr() if a is not None else None for a in arrs])
+    L.call("endia_hip_mlp_fwd", ctypes.byref(desc), xs.data_ptr(), ptrs(Ws), ptrs(bs_), ptrs(hs))
+
+    def vjp(primals, grad, out_):
+        from .autograd.functional import building_graph
+        if building_graph() or grad.ndim() != out_.ndim():
+            raise NotImplementedError("mlp_forward is a first-order op; build the model with fused=True for higher-order or Jacobian passes")
+        deltas = [Array.empty([B, widths[i + 1]]) for i in range(Lyr - 1)] + [contiguous(grad)]
+        pW, pb = primals[1:1 + Lyr], primals[1 + Lyr:]
+        dW = [Array.empty([widths[i], widths[i + 1]]) if pW[i]._requires_grad else None for i in range(Lyr)]
+        db = [Array.empty([1, widths[i + 1]]) if pb[i]._requires_grad else None for i in range(Lyr)]  # kept axis, like Expand.vjp
+        dx = Array.empty([B, widths[0]]) if primals[0]._requires_grad else None
+        L.call("endia_hip_mlp_bwd", ctypes.byref(desc), xs.data_ptr(), ptrs(Ws), ptrs(hs), ptrs(deltas), ptrs(dW), ptrs(db),
+               dx.data_ptr() if dx is not None else None)
+        return [dx] + dW + db
+
+    return _register(hs[-1], [x] + list(weights) + list(biases), "mlp", vjp)
+
+
 def _fused_act_of(px):
     """The activation a gradient may absorb on its way to px: px is the output of a fused layer (or the
     fused sin node on top of one), nothing else consumes it and it holds no earlier gradient."""

@@ -8,7 +8,9 @@ class MLP:
     (_mlp.mojo:30-43). The reference hard-codes ReLU; `activation` also accepts "tanh", "sin" and None.
 
     `fused=True` (default) evaluates each layer as one GEMM with a bias + activation epilogue;
-    `fused=False` issues the reference's op sequence matmul -> add -> activation.
+    `fused=False` issues the reference's op sequence matmul -> add -> activation;
+    `fused="model"` evaluates the WHOLE stack as one op (functional.mlp_forward): for small models (widths up to 128,
+    relu / tanh / no activation) that is one launch forward and two backward; first-order passes only.
     """
 
     def __init__(self, hidden_dims, compute_backward=False, activation="relu", fused=True):
@@ -25,6 +27,8 @@ class MLP:
                                                 requires_grad=compute_backward))
 
     def forward(self, x):
+        if self.fused == "model":
+            return F.mlp_forward(x, self.weights, self.biases, self.activation)
         pred = x
         act_fn = {"relu": F.relu, "tanh": F.tanh, "sin": F.sin, None: None}[self.activation]
         for i in range(self.num_layers):

@@ -199,6 +199,34 @@ ENDIA_API int32_t endia_hip_sgemm(int32_t transA, int32_t transB, int64_t M, int
 ENDIA_API int32_t endia_hip_linear_bwd(int64_t B, int64_t K, int64_t N, const float* x, const float* W, const float* g,
                              int32_t act, const float* aux, float* dx, float* dW, float* db);
 
+/* ---- a whole small dense model per call: nn.MLP.forward (nn/modules/_mlp.mojo:47-53: h_l = act(h_{l-1} W_l + b_l), no
+ *      activation after the last layer) and the backward pass of that chain (matmul_vjp matmul_op.mojo:278-283,
+ *      Expand.vjp expand_op.mojo:121-126, relu_op.mojo:95 / tanh_op.mojo:92), for models whose layers are at most
+ *      ENDIA_MLP_MAX_WIDTH wide, like the reference's own benchmark model (benchmarks/mlp_benchmarks/mlp_imp.mojo:35-37).
+ *      Every row of the batch is independent through all layers, so the forward pass is ONE launch (a work-group keeps
+ *      16 rows' activations in LDS from the first layer to the last) and the backward pass two (the chain of cotangents
+ *      the same way, then every dW_l and db_l at once), instead of one to three launches per layer.
+ *      widths[0..layers]: input width, then each layer's output width. W[l] is [widths[l], widths[l+1]] row-major, b[l]
+ *      is [widths[l+1]], x is [batch, widths[0]], all contiguous. act in {RELU, TANH, IDENTITY} follows every layer but
+ *      the last.
+ *      fwd: h[l] receives layer l's output [batch, widths[l+1]] (h[layers-1] is the model's output; the others are what
+ *           the backward pass needs).
+ *      bwd: delta[layers-1] holds the cotangent of the output on entry; delta[l] for l < layers-1 are buffers
+ *           [batch, widths[l+1]] that receive the cotangents of the pre-activations. dW[l] = h[l-1]^T delta[l] (x for
+ *           l = 0), db[l] = column sums of delta[l]; entries of dW / db may be null. dx [batch, widths[0]] or null. */
+#define ENDIA_MLP_MAX_LAYERS 16
+#define ENDIA_MLP_MAX_WIDTH 128
+typedef struct endia_hip_mlp_desc {
+  int32_t layers;
+  int32_t act; /* endia_hip_unary_op */
+  int64_t batch;
+  int64_t widths[ENDIA_MLP_MAX_LAYERS + 1];
+} endia_hip_mlp_desc;
+ENDIA_API int32_t endia_hip_mlp_fwd(const endia_hip_mlp_desc* desc, const float* x, const float* const* W, const float* const* b,
+                          float* const* h);
+ENDIA_API int32_t endia_hip_mlp_bwd(const endia_hip_mlp_desc* desc, const float* x, const float* const* W, const float* const* h,
+                          float* const* delta, float* const* dW, float* const* db, float* dx);
+
 /* ---- complex64 GEMM: the complex branch of matmul_fwd (matmul_op.mojo:201-238). Interleaved
  *      operands; lda/ldb/ldc and strides count complex elements. conjA/conjB conjugate the operand
  *      (the reference's VJP does not conjugate, matmul_op.mojo:278-283; the Wirtinger convention does).

@@ -318,7 +318,7 @@ def _load_mlp(nd, g, n_layers, act, fused):
     return mlp, widths
 
 
-@pytest.mark.parametrize("fused", [True, False])
+@pytest.mark.parametrize("fused", [True, False, "model"])
 def test_mlp_sine_sgd(nd, golden, fused):
     """The reference's benchmark model (mlp_imp.mojo:25-75) for three SGD steps, against torch float64
     and against the CPU oracle's restatement of the same tape."""
@@ -349,7 +349,7 @@ def test_mlp_sine_sgd(nd, golden, fused):
         assert_close(mlp.biases[i].to_numpy(), g["b%d_after" % i], what="b%d after" % i)
 
 
-@pytest.mark.parametrize("fused", [True, False])
+@pytest.mark.parametrize("fused", [True, False, "model"])
 def test_mlp_tanh_adam(nd, golden, fused):
     g = golden("mlp_tanh_adam")
     mlp, widths = _load_mlp(nd, g, 3, "tanh", fused)
@@ -481,13 +481,14 @@ def test_conv2d_autograd(nd, golden):
     assert_close(x2.grad().to_numpy(), tx.grad.numpy(), what="dx")
 
 
-def test_captured_step_matches_eager(nd, golden):
+@pytest.mark.parametrize("fused", [True, "model"])
+def test_captured_step_matches_eager(nd, golden, fused):
     """The sine-fit MLP step recorded into a HIP graph: every replay must leave exactly the parameters the
     eager step leaves. Replays are interleaved with eager work and synchronisations."""
     g = golden("mlp_sine")
 
     def build():
-        mlp, _ = _load_mlp(nd, g, 8, "relu", True)
+        mlp, _ = _load_mlp(nd, g, 8, "relu", fused)
         opt = nd.optim.SGD(mlp.params(), lr=1e-3, momentum=0.9)
         x, y = nd.array(g["x"]), nd.array(g["y"])
 
@@ -814,12 +815,14 @@ def test_random_mlps_vs_oracle(nd):
     from oracle import endia_ref as R
     rng = np.random.default_rng(81)
     widths_pool = [1, 4, 8, 30, 32, 33, 64, 100, 128, 132, 160]
-    for case in range(24):
+    for case in range(36):
         depth = int(rng.integers(1, 5))
         widths = [int(rng.choice(widths_pool)) for _ in range(depth + 1)]
         batch = int(rng.choice([8, 20, 100, 128, 130, 256]))
         act = ["relu", "tanh", "sin"][case % 3]
-        fused = case % 4 != 3
+        # per-layer fused, op by op, and the whole model as one op (one launch forward, two backward, when every width
+        # is at most 128 and the activation is relu or tanh; the per-layer kernels otherwise)
+        fused = [True, True, "model", False, "model", True][case % 6]
         Ws = [(rng.standard_normal((widths[i], widths[i + 1])) * np.sqrt(1.0 / widths[i])).astype(np.float32) for i in range(depth)]
         bs = [(rng.standard_normal(widths[i + 1]) * 0.1).astype(np.float32) for i in range(depth)]
         xb = rng.standard_normal((batch, widths[0])).astype(np.float32)
@@ -1147,3 +1150,51 @@ def test_callable_mixed_argnums(nd):
     assert_close(nested[0][0].to_numpy(), [float(tf(at, bt))], what="value")
     assert_close(nested[1][0].to_numpy(), ga.numpy(), what="first order kept")
     assert_close(nested[2][0].to_numpy(), H[0][1].numpy(), what="second order")
+
+
+def test_whole_model_mlp_op(nd):
+    """functional.mlp_forward through the C ABI's endia_hip_mlp_fwd / endia_hip_mlp_bwd: the same numbers as the
+    per-layer path for ragged widths and batches (rows and columns that do not fill a 16 x 16 block), the input
+    gradient, a parameter that needs no gradient, two calls in a row (bit-identical), and the cases it refuses."""
+    rng = np.random.default_rng(123)
+    for widths, batch, act in [([1, 32, 64, 128, 128, 128, 64, 32, 1], 128, "relu"), ([7, 50, 3, 128, 20], 37, "tanh"),
+                               ([128, 128], 16, None), ([5, 17], 1, "relu"), ([40, 100, 100, 9], 300, "relu")]:
+        Lyr = len(widths) - 1
+        Wn = [(rng.standard_normal((widths[i], widths[i + 1])) / np.sqrt(widths[i])).astype(np.float32) for i in range(Lyr)]
+        bn = [(0.2 * rng.standard_normal(widths[i + 1])).astype(np.float32) for i in range(Lyr)]
+        xn = rng.standard_normal((batch, widths[0])).astype(np.float32)
+        gn = rng.standard_normal((batch, widths[-1])).astype(np.float32)
+
+        def run(whole):
+            x = nd.array(xn, requires_grad=True)
+            W = [nd.array(w, requires_grad=(i != 1)) for i, w in enumerate(Wn)]  # the second weight matrix is frozen
+            b = [nd.array(v, requires_grad=True) for v in bn]
+            if whole:
+                out = nd.mlp_forward(x, W, b, act)
+            else:
+                out = x
+                for i in range(Lyr):
+                    out = nd.linear(out, W[i], b[i], act if i < Lyr - 1 else None)
+            nd.sum(out * nd.array(gn)).backward()
+            grads = [x.grad().to_numpy()] + [w.grad().to_numpy() for w in W if w.has_grad()] + [v.grad().to_numpy().reshape(-1) for v in b]
+            assert not W[1].has_grad() if Lyr > 1 else True
+            return out.to_numpy(), grads
+
+        out_w, g_w = run(True)
+        out_l, g_l = run(False)
+        what = "widths %s batch %d %s: " % (widths, batch, act)
+        assert_close(out_w, out_l, tol=1e-5, what=what + "output")
+        assert len(g_w) == len(g_l)
+        for k, (a, b_) in enumerate(zip(g_w, g_l)):
+            assert_close(a, b_, tol=2e-5, mean_tol=1e-3, what=what + "gradient %d" % k)  # (mean metric: a few values sum to ~0)
+        out_2, g_2 = run(True)
+        np.testing.assert_array_equal(out_2, out_w)
+        for a, b_ in zip(g_2, g_w):
+            np.testing.assert_array_equal(a, b_)
+    # wider layers, sin, or complex operands take the per-layer kernels; second-order passes are refused
+    wide = nd.mlp_forward(nd.ones([4, 200]), [nd.ones([200, 8])], [nd.zeros([8])], "relu")
+    np.testing.assert_array_equal(wide.to_numpy(), np.full((4, 8), 200.0, np.float32))
+    x = nd.array(xn[:8, :4].copy(), requires_grad=True)
+    y = nd.sum(nd.mlp_forward(x, [nd.array(np.ones((4, 3), np.float32), requires_grad=True)], [nd.zeros([3])], "relu"))
+    with pytest.raises(NotImplementedError):
+        y.backward(create_graph=True)
