@@ -510,9 +510,11 @@ __global__ __launch_bounds__(WGM* WGN * 64, 4) void conv_igemm_vec_kernel(VecArg
 
 struct WgradVecArgs {
   const float* xpad;  // [N, C, Dp, Hp, Wp]
-  const float* dy;    // [N, K, O, P, Q], Q % 4 == 0
+  const float* dy;    // [N, K, O, P, Q], Q % 4 == 0 (GATE 1: one float, the same for every element)
+  const float* gate;  // GATE > 0: the stored output y of relu(conv + bias), same shape; dy counts where y > 0
   const int* table;   // [tiles_n * BN] byte offset of tap t inside a padded image; OOB_OFFSET past Kd
   float* part;
+  float* bias_part;   // GATE > 0, may be null: [splits][K] sums of the gated dy over each split's columns
   int K, Kd, OPQ, PQ, Q, sh, Wp, img_floats, zstep;
   int total_j, chunk;
   FastDiv d_opq, d_pq, d_q;
@@ -520,8 +522,11 @@ struct WgradVecArgs {
   int64_t x_bytes, dy_bytes;
 };
 
-template <int WGM, int WGN, int FM, int FN>
-__global__ __launch_bounds__(WGM* WGN * 64, 4) void conv_wgrad_vec_kernel(WgradVecArgs a) {
+// GATE 0: dy as it is. GATE 1 / 2: dy (1: a scalar, 2: a tensor) gated by [y > 0] as the A operand is loaded, so that
+// the gradient of the ReLU is never written out; the work-groups of the first tile column also sum the rows of
+// what they load, which is the bias gradient.
+template <int WGM, int WGN, int FM, int FN, int GATE>
+__global__ __launch_bounds__(WGM* WGN * 64, FM* FN >= 6 ? 2 : 4) void conv_wgrad_vec_kernel(WgradVecArgs a) {
   constexpr int NT = WGM * WGN * 64, BM = WGM * FM * 32, BN = WGN * FN * 32;
   constexpr int ROWS_PER_PASS = NT / 8, PA = BM / ROWS_PER_PASS, PB = BN / ROWS_PER_PASS;
   __shared__ __attribute__((aligned(16))) float As[TileShape<true, BM>::FLOATS];
@@ -546,9 +551,15 @@ __global__ __launch_bounds__(WGM* WGN * 64, 4) void conv_wgrad_vec_kernel(WgradV
   }
 #pragma unroll
   for (int i = 0; i < PB; ++i) rowb[i] = (uint32_t)a.table[n0 + r + i * ROWS_PER_PASS];
-  const __amdgpu_buffer_rsrc_t rs_dy = make_rsrc(a.dy, a.dy_bytes);
+  const __amdgpu_buffer_rsrc_t rs_dy = make_rsrc(GATE == 1 ? a.gate : a.dy, a.dy_bytes);
+  const __amdgpu_buffer_rsrc_t rs_gate = make_rsrc(a.gate, a.dy_bytes);
   const __amdgpu_buffer_rsrc_t rs_x = make_rsrc(a.xpad, a.x_bytes);
-  float4 ra[PA], rb[PB];
+  float4 ra[PA], rb[PB], rg[GATE == 2 ? PA : 1];
+  const float dy_scalar = GATE == 1 ? a.dy[0] : 0.f;
+  const bool sum_rows = GATE > 0 && a.bias_part != nullptr && tn == 0;
+  float row_sum[PA];
+#pragma unroll
+  for (int i = 0; i < PA; ++i) row_sum[i] = 0.f;
 
   auto load = [&](int jt) {
     int j = jt + c4;
@@ -565,10 +576,26 @@ __global__ __launch_bounds__(WGM* WGN * 64, 4) void conv_wgrad_vec_kernel(WgradV
     }
 #pragma unroll
     for (int i = 0; i < PA; ++i) ra[i] = buffer_load_f4(rs_dy, ca + rowa[i]);
+    if (GATE == 2) {
+#pragma unroll
+      for (int i = 0; i < PA; ++i) rg[i] = buffer_load_f4(rs_gate, ca + rowa[i]);
+    }
 #pragma unroll
     for (int i = 0; i < PB; ++i) rb[i] = buffer_load_f4(rs_x, cb + rowb[i]);
   };
   auto store = [&]() {
+    if (GATE > 0) {  // out-of-range pieces were loaded as zeros and stay zeros: 0 > 0 is false
+#pragma unroll
+      for (int i = 0; i < PA; ++i) {
+        const float4 y = GATE == 1 ? ra[i] : rg[i];
+        const float4 g = GATE == 1 ? make_float4(dy_scalar, dy_scalar, dy_scalar, dy_scalar) : ra[i];
+        ra[i] = make_float4(y.x > 0.f ? g.x : 0.f, y.y > 0.f ? g.y : 0.f, y.z > 0.f ? g.z : 0.f, y.w > 0.f ? g.w : 0.f);
+      }
+      if (sum_rows) {
+#pragma unroll
+        for (int i = 0; i < PA; ++i) row_sum[i] += (ra[i].x + ra[i].y) + (ra[i].z + ra[i].w);
+      }
+    }
 #pragma unroll
     for (int i = 0; i < PA; ++i) *reinterpret_cast<float4*>(&As[lds_off + i * ROWS_PER_PASS * LDK]) = ra[i];
 #pragma unroll
@@ -588,6 +615,18 @@ __global__ __launch_bounds__(WGM* WGN * 64, 4) void conv_wgrad_vec_kernel(WgradV
       __syncthreads();
       store();
       __syncthreads();
+    }
+  }
+
+  if (sum_rows) {  // the eight threads of a row are neighbours in a wave; fixed order of additions
+#pragma unroll
+    for (int i = 0; i < PA; ++i) {
+      float v = row_sum[i];
+      v += __shfl_xor(v, 1);
+      v += __shfl_xor(v, 2);
+      v += __shfl_xor(v, 4);
+      const int m = m0 + r + i * ROWS_PER_PASS;
+      if ((tid & 7) == 0 && m < a.K) a.bias_part[(int64_t)split * a.K + m] = v;
     }
   }
 
@@ -620,6 +659,8 @@ __global__ __launch_bounds__(WGM* WGN * 64, 4) void conv_wgrad_vec_kernel(WgradV
 // (the dense kernel has 64 at its large tile), three or four work-groups per CU.
 struct DirectArgs {
   const float* src;   // [N, Cred, SH, SW]
+  const float* gate;  // GATE 2: same shape as src, which counts where gate > 0 (GATE 1: src IS the gate and every
+  const float* gscalar;  // element that passes it is worth *gscalar)
   const float* wp;    // [chunks][tiles_m * BM][72], packed as described above
   const float* bias;
   float* out;         // [N, Mrows, OH, OW]
@@ -636,7 +677,7 @@ struct DirectArgs {
 
 // One tile: rows [tm * 64 * FM, ...) of the output channels, pixels [n0, n0 + 64 * FN). MR / tasks: the cache rows and
 // staging pieces a tile of that many pixels needs.
-template <int FM, int FN, int PITCH, bool FWD>
+template <int FM, int FN, int PITCH, bool FWD, int GATE>
 __device__ __forceinline__ void direct3x3_tile(const DirectArgs& a, int tm, int n0, int MR, int tasks, float* smem) {
   constexpr int BM = 64 * FM, CC = 8, KC = 72, PB = 8;
   float* Bc = smem;
@@ -682,18 +723,33 @@ __device__ __forceinline__ void direct3x3_tile(const DirectArgs& a, int tm, int 
   const __amdgpu_buffer_rsrc_t rs_src = make_rsrc(a.src, a.src_bytes);
   const __amdgpu_buffer_rsrc_t rs_w = make_rsrc(a.wp, a.wp_bytes);
   const uint32_t src_step = (uint32_t)(CC * a.SH * a.SW) * 4u, w_step = (uint32_t)(a.tiles_m * BM * KC) * 4u;
-  float4 rb[PB];
+  const __amdgpu_buffer_rsrc_t rs_gate = make_rsrc(GATE == 2 ? a.gate : a.src, a.src_bytes);
+  const float gs = GATE == 1 ? a.gscalar[0] : 0.f;
+  float4 rb[PB], rg[GATE == 2 ? PB : 1];
   auto load = [&](int chunk) {
 #pragma unroll
     for (int p = 0; p < PB; ++p) {
       v4i v = __builtin_amdgcn_raw_buffer_load_b128(rs_src, (int)goff[p], (int)(chunk * src_step), 0);
       rb[p] = *reinterpret_cast<float4*>(&v);
     }
+    if (GATE == 2) {
+#pragma unroll
+      for (int p = 0; p < PB; ++p) {
+        v4i v = __builtin_amdgcn_raw_buffer_load_b128(rs_gate, (int)goff[p], (int)(chunk * src_step), 0);
+        rg[p] = *reinterpret_cast<float4*>(&v);
+      }
+    }
   };
   auto store = [&]() {
 #pragma unroll
-    for (int p = 0; p < PB; ++p)
+    for (int p = 0; p < PB; ++p) {
+      if (GATE > 0) {  // rows outside the image were loaded as zeros and stay zeros
+        const float4 y = GATE == 1 ? rb[p] : rg[p];
+        const float4 g = GATE == 1 ? make_float4(gs, gs, gs, gs) : rb[p];
+        rb[p] = make_float4(y.x > 0.f ? g.x : 0.f, y.y > 0.f ? g.y : 0.f, y.z > 0.f ? g.z : 0.f, y.w > 0.f ? g.w : 0.f);
+      }
       if (loff[p] >= 0) *reinterpret_cast<float4*>(&Bc[loff[p]]) = rb[p];
+    }
   };
 
   // this lane's pixels: cache position of tap (0, 0), with the half-wave's channel folded in
@@ -797,17 +853,17 @@ __device__ __forceinline__ void direct3x3_tile(const DirectArgs& a, int tm, int 
 
 // Whole tiles of 128 pixels first; what is left after the last full round over the CUs is cut into tiles of 64
 // pixels, so that the CUs that get one more tile than the others get half a tile more (see run_direct3x3).
-template <int FM, int PITCH, bool FWD>
+template <int FM, int PITCH, bool FWD, int GATE>
 __global__ __launch_bounds__(256, 2) void conv_direct3x3_kernel(DirectArgs a) {
   extern __shared__ __attribute__((aligned(16))) float smem[];
   const int b = blockIdx.x;
   if (b < a.full_blocks) {
     int tm, tn;
     tile_of_block(b, a.full_blocks, a.tiles_m, a.full_tiles_n, tm, tn);
-    direct3x3_tile<FM, 2, PITCH, FWD>(a, tm, tn * 128, a.MR, a.tasks, smem);
+    direct3x3_tile<FM, 2, PITCH, FWD, GATE>(a, tm, tn * 128, a.MR, a.tasks, smem);
   } else {
     const int hb = b - a.full_blocks, tn = hb / a.tiles_m, tm = hb - tn * a.tiles_m;
-    direct3x3_tile<FM, 1, PITCH, FWD>(a, tm, a.full_tiles_n * 128 + tn * 64, a.MR_half, a.tasks_half, smem);
+    direct3x3_tile<FM, 1, PITCH, FWD, GATE>(a, tm, a.full_tiles_n * 128 + tn * 64, a.MR_half, a.tasks_half, smem);
   }
 }
 
@@ -1096,8 +1152,12 @@ int32_t run_igemm_vec(int mode, const ConvP& p, const float* src, const float* w
 
 // 3 x 3 kernels with unit stride and dilation and at most one zero row / column around the source
 // (conv_direct3x3_kernel). Returns 1 when the shape does not qualify.
-int32_t run_direct3x3(int mode, const ConvP& p, const float* src, const float* w, const float* bias, float* out, int relu) {
+// gate_mode 1 / 2 (data gradient only): src counts where gate > 0; 1: src is the gate itself and *gscalar the value of
+// every element that passes, 2: gate is a second tensor of src's shape.
+int32_t run_direct3x3(int mode, const ConvP& p, const float* src, const float* w, const float* bias, float* out, int relu,
+                      int gate_mode = 0, const float* gate = nullptr, const float* gscalar = nullptr) {
   const bool fwd = mode == MODE_FWD;
+  if (gate_mode == 2 && (reinterpret_cast<uintptr_t>(gate) & 15)) return 1;
   if (p.T != 1 || p.D != 1 || p.R != 3 || p.S != 3 || p.dh != 1 || p.dw != 1 || p.sh != 1 || p.sw != 1 || p.sd != 1) return 1;
   const int OH = fwd ? p.P : p.H, OW = fwd ? p.Q : p.W, SH = fwd ? p.H : p.P, SW = fwd ? p.W : p.Q;
   const int Cred = fwd ? p.C : p.K, Mrows = fwd ? p.K : p.C;
@@ -1127,6 +1187,7 @@ int32_t run_direct3x3(int mode, const ConvP& p, const float* src, const float* w
                      static_cast<float*>(wp.p), p.K, p.C, rows_pad, a.chunks, fwd ? 0 : 1);
   ENDIA_LAUNCH_CHECK();
   a.src = src; a.wp = static_cast<const float*>(wp.p); a.bias = bias; a.out = out; a.relu = relu;
+  a.gate = gate; a.gscalar = gscalar;
   a.Mrows = Mrows; a.Cred = Cred; a.OH = OH; a.OW = OW; a.SH = SH; a.SW = SW; a.Ncols = p.N * OH * OW; a.NOH = p.N * OH;
   a.py = py; a.px = px; a.MR = MR; a.plane = plane; a.tasks = tasks;
   a.d_ohw = make_fastdiv(OH * OW); a.d_ow = make_fastdiv(OW); a.d_oh = make_fastdiv(OH); a.d_f4row = make_fastdiv(SW / 4);
@@ -1147,8 +1208,10 @@ int32_t run_direct3x3(int mode, const ConvP& p, const float* src, const float* w
   const dim3 grid((unsigned)(a.full_blocks + a.tiles_m * half_tiles_n));
 #define ENDIA_LAUNCH_DIRECT(FM, PITCH)                                                                                       \
   do {                                                                                                                       \
-    if (fwd) hipLaunchKernelGGL((conv_direct3x3_kernel<FM, PITCH, true>), grid, dim3(256), lds, s, a);                         \
-    else hipLaunchKernelGGL((conv_direct3x3_kernel<FM, PITCH, false>), grid, dim3(256), lds, s, a);                            \
+    if (fwd) hipLaunchKernelGGL((conv_direct3x3_kernel<FM, PITCH, true, 0>), grid, dim3(256), lds, s, a);                      \
+    else if (gate_mode == 0) hipLaunchKernelGGL((conv_direct3x3_kernel<FM, PITCH, false, 0>), grid, dim3(256), lds, s, a);     \
+    else if (gate_mode == 1) hipLaunchKernelGGL((conv_direct3x3_kernel<FM, PITCH, false, 1>), grid, dim3(256), lds, s, a);     \
+    else hipLaunchKernelGGL((conv_direct3x3_kernel<FM, PITCH, false, 2>), grid, dim3(256), lds, s, a);                         \
   } while (0)
   if (fm == 2 && pitch == 64) ENDIA_LAUNCH_DIRECT(2, 64);
   else if (fm == 2) ENDIA_LAUNCH_DIRECT(2, 128);
@@ -1226,7 +1289,18 @@ int32_t conv_bwd_data(const char* who, const ConvP& p, const float* dy, const fl
   return run_igemm(MODE_BWD_DATA, p, dy, w, nullptr, dx, 0);
 }
 
-int32_t conv_bwd_weight(const char* who, const ConvP& p, const float* x, const float* dy, float* dw) {
+// The vectorised weight-gradient kernel serves unit stride along the row, output rows that are whole 16-byte pieces
+// and 32-bit offsets into the padded copy. `rows` is the tensor its A operand is loaded from.
+bool wgrad_vec_ok(const ConvP& p, const float* rows) {
+  const int Dp = p.D + 2 * p.pd, Hp = p.H + 2 * p.ph, Wp = padded_row(p.W, p.pw);
+  return p.sw == 1 && p.Q % 4 == 0 && (int64_t)p.N * p.C * Dp * Hp * Wp < (1ll << 29) &&
+         (reinterpret_cast<uintptr_t>(rows) & 15) == 0;
+}
+
+// gate_mode 0: the plain weight gradient. 1 / 2 (only where wgrad_vec_ok): dy (1: one float, 2: a tensor) counts
+// where gate > 0, and db (may be null) receives the sums of the gated dy over n, o, p, q.
+int32_t conv_bwd_weight(const char* who, const ConvP& p, const float* x, const float* dy, float* dw, int gate_mode = 0,
+                        const float* gate = nullptr, float* db = nullptr) {
   const int Kd = p.C * p.T * p.R * p.S;
   const int64_t taps = (int64_t)p.K * Kd;
   if (!dw) return endia::fail(ENDIA_HIP_ERR_INVALID, "%s: dw is null", who);
@@ -1247,17 +1321,20 @@ int32_t conv_bwd_weight(const char* who, const ConvP& p, const float* x, const f
   a.x_bytes = (int64_t)p.N * p.C * p.D * p.H * p.W * 4;
   a.dy_bytes = (int64_t)p.N * p.K * p.O * p.P * p.Q * 4;
   const int Dp = p.D + 2 * p.pd, Hp = p.H + 2 * p.ph, Wp = padded_row(p.W, p.pw);
-  const bool vec = p.sw == 1 && p.Q % 4 == 0 && (int64_t)p.N * p.C * Dp * Hp * Wp < (1ll << 29) &&
-                   (reinterpret_cast<uintptr_t>(dy) & 15) == 0;
+  const bool vec = wgrad_vec_ok(p, gate_mode == 1 ? gate : dy) && (gate_mode != 2 || (reinterpret_cast<uintptr_t>(gate) & 15) == 0);
+  if (gate_mode && !vec) return endia::fail(ENDIA_HIP_ERR_UNSUPPORTED, "%s: gated weight gradient outside the vectorised kernel", who);
   // 64-wide tiles over the taps when the last 128-wide tile would be at most half full
-  const int bn = (vec && Kd % 128 != 0 && Kd % 128 <= 64) ? 64 : 128;
+  int bn = (vec && Kd % 128 != 0 && Kd % 128 <= 64) ? 64 : 128;
   // likewise 64-high tiles over the output channels
   const int bm = (vec && p.K % 128 != 0 && p.K % 128 <= 64) ? 64 : 128;
+  // 192-wide tiles (six accumulator blocks a wave) where they cover the taps with no more padding than the above
+  if (vec && bm == 128 && Kd >= 192 && (Kd + 191) / 192 * 192 <= (Kd + bn - 1) / bn * bn) bn = 192;
   a.tiles_m = (p.K + bm - 1) / bm;
   a.tiles_n = (Kd + bn - 1) / bn;
-  // split the N*O*P*Q reduction so that about 4 work-groups per CU exist; every split reduces >= 256 columns
+  // split the N*O*P*Q reduction so that as many work-groups exist as the CUs hold at once (4 each, 2 of the 192-wide
+  // tile); every split reduces >= 256 columns
   int64_t tiles = (int64_t)a.tiles_m * a.tiles_n;
-  int64_t splits = ((int64_t)endia::ctx().cu_count * 4 + tiles - 1) / tiles;
+  int64_t splits = ((int64_t)endia::ctx().cu_count * (bn == 192 ? 2 : 4) + tiles - 1) / tiles;
   int64_t max_splits = (total_j + 255) / 256;
   if (splits > max_splits) splits = max_splits;
   if (splits > 1024) splits = 1024;
@@ -1266,12 +1343,17 @@ int32_t conv_bwd_weight(const char* who, const ConvP& p, const float* x, const f
   splits = (total_j + chunk - 1) / chunk;
   a.chunk = (int)chunk;
 
-  PoolBuf part;
+  PoolBuf part, bias_part;
   int32_t rc;
+  float* db_part = db;
   if (splits > 1) {
     rc = endia_hip_malloc(splits * taps * 4, &part.p);
     if (rc) return rc;
     a.part = static_cast<float*>(part.p);
+    if (db) {
+      if ((rc = endia_hip_malloc(splits * p.K * 4, &bias_part.p))) return rc;
+      db_part = static_cast<float*>(bias_part.p);
+    }
   } else {
     a.part = dw;
   }
@@ -1283,20 +1365,32 @@ int32_t conv_bwd_weight(const char* who, const ConvP& p, const float* x, const f
       return rc;
     WgradVecArgs v;
     v.xpad = xpad.p ? static_cast<const float*>(xpad.p) : x; v.dy = dy; v.table = static_cast<const int*>(table.p); v.part = a.part;
+    v.gate = gate; v.bias_part = db_part;
     v.K = p.K; v.Kd = Kd; v.OPQ = p.O * p.P * p.Q; v.PQ = p.P * p.Q; v.Q = p.Q; v.sh = p.sh; v.Wp = Wp;
     v.img_floats = p.C * Dp * Hp * Wp; v.zstep = p.sd * Hp * Wp;
     v.total_j = a.total_j; v.chunk = a.chunk; v.d_opq = a.d_opq; v.d_pq = a.d_pq; v.d_q = a.d_q;
     v.tiles_m = a.tiles_m; v.tiles_n = a.tiles_n;
     v.x_bytes = (int64_t)p.N * p.C * Dp * Hp * Wp * 4; v.dy_bytes = a.dy_bytes;
-    if (bm == 128 && bn == 128) hipLaunchKernelGGL((conv_wgrad_vec_kernel<2, 2, 2, 2>), grid, dim3(256), 0, s, v);
-    else if (bm == 128) hipLaunchKernelGGL((conv_wgrad_vec_kernel<2, 2, 2, 1>), grid, dim3(256), 0, s, v);
-    else if (bn == 128) hipLaunchKernelGGL((conv_wgrad_vec_kernel<2, 2, 1, 2>), grid, dim3(256), 0, s, v);
-    else hipLaunchKernelGGL((conv_wgrad_vec_kernel<2, 2, 1, 1>), grid, dim3(256), 0, s, v);
+#define ENDIA_WGRAD_VEC(FM_, FN_)                                                                                     \
+  do {                                                                                                                \
+    if (gate_mode == 0) hipLaunchKernelGGL((conv_wgrad_vec_kernel<2, 2, FM_, FN_, 0>), grid, dim3(256), 0, s, v);      \
+    else if (gate_mode == 1) hipLaunchKernelGGL((conv_wgrad_vec_kernel<2, 2, FM_, FN_, 1>), grid, dim3(256), 0, s, v); \
+    else hipLaunchKernelGGL((conv_wgrad_vec_kernel<2, 2, FM_, FN_, 2>), grid, dim3(256), 0, s, v);                     \
+  } while (0)
+    if (bn == 192) ENDIA_WGRAD_VEC(2, 3);
+    else if (bm == 128 && bn == 128) ENDIA_WGRAD_VEC(2, 2);
+    else if (bm == 128) ENDIA_WGRAD_VEC(2, 1);
+    else if (bn == 128) ENDIA_WGRAD_VEC(1, 2);
+    else ENDIA_WGRAD_VEC(1, 1);
+#undef ENDIA_WGRAD_VEC
   } else {
     hipLaunchKernelGGL((conv_wgrad_kernel<2, 2, 2, 2>), grid, dim3(256), 0, s, a);
   }
   ENDIA_LAUNCH_CHECK();
-  if (splits > 1) return endia::col_reduce(1, splits, taps, a.part, dw, 1.f);  // partials added in split order
+  if (splits > 1) {  // partials added in split order
+    if ((rc = endia::col_reduce(1, splits, taps, a.part, dw, 1.f))) return rc;
+    if (db) return endia::col_reduce(1, splits, p.K, db_part, db, 1.f);
+  }
   return ENDIA_HIP_OK;
 }
 
@@ -1313,6 +1407,63 @@ int32_t conv_bwd_bias(const char* who, const ConvP& p, const float* dy, float* d
   rc = endia::row_reduce(rows, PQ, dy, static_cast<float*>(tmp.p), 1.f);
   if (!rc) rc = endia::col_reduce(1, p.N, p.K, static_cast<float*>(tmp.p), db, 1.f);
   return rc;
+}
+
+__global__ __launch_bounds__(TPB) void relu_gate_kernel(const float* __restrict__ y, const float* __restrict__ dy, int dy_is_scalar,
+                                                        float* __restrict__ g, int64_t n) {
+  const float sv = dy_is_scalar ? dy[0] : 0.f;
+  for (int64_t i = (int64_t)blockIdx.x * TPB + threadIdx.x; i < n; i += (int64_t)gridDim.x * TPB)
+    g[i] = y[i] > 0.f ? (dy_is_scalar ? sv : dy[i]) : 0.f;
+}
+
+// Every gradient of y = relu(conv(x, w) + bias) from the stored y. Where the 3 x 3 row-cache kernel (dx) and the
+// vectorised weight-gradient kernel (dw, db) apply, dy * [y > 0] is formed as they load their operands and never
+// exists in memory; otherwise it is written once and the plain kernels run on it.
+int32_t conv_bwd_relu(const char* who, const ConvP& p, const float* x, const float* w, const float* y, const float* dy,
+                      int dy_is_scalar, float* dx, float* dw, float* db) {
+  const int64_t out_total = (int64_t)p.N * p.K * p.O * p.P * p.Q;
+  const int64_t x_total = (int64_t)p.N * p.C * p.D * p.H * p.W;
+  int32_t rc;
+  if (out_total == 0) {
+    if (dw && (rc = endia_hip_fill(dw, (int64_t)p.K * p.C * p.T * p.R * p.S, 0.f))) return rc;
+    if (db && (rc = endia_hip_fill(db, p.K, 0.f))) return rc;
+    if (dx && x_total && (rc = endia_hip_fill(dx, x_total, 0.f))) return rc;
+    return ENDIA_HIP_OK;
+  }
+  if (!(y && dy)) return endia::fail(ENDIA_HIP_ERR_INVALID, "%s: null pointer", who);
+  if ((dw && !x) || (dx && !w)) return endia::fail(ENDIA_HIP_ERR_INVALID, "%s: null pointer", who);
+  const int gate_mode = dy_is_scalar ? 1 : 2;
+  PoolBuf gbuf;
+  auto gated = [&](const float** g) -> int32_t {  // dy * [y > 0] in memory, made at most once
+    if (!gbuf.p) {
+      int32_t r = endia_hip_malloc(out_total * 4, &gbuf.p);
+      if (r) return r;
+      hipLaunchKernelGGL(relu_gate_kernel, dim3(grid_for(out_total)), dim3(TPB), 0, endia::ctx().stream, y, dy, dy_is_scalar,
+                         static_cast<float*>(gbuf.p), out_total);
+      ENDIA_LAUNCH_CHECK();
+    }
+    *g = static_cast<const float*>(gbuf.p);
+    return ENDIA_HIP_OK;
+  };
+  const float* g = nullptr;
+  if (dw && wgrad_vec_ok(p, dy_is_scalar ? y : dy) && (dy_is_scalar || (reinterpret_cast<uintptr_t>(y) & 15) == 0)) {
+    if ((rc = conv_bwd_weight(who, p, x, dy, dw, gate_mode, y, db))) return rc;
+  } else {
+    if (dw || db) {
+      if ((rc = gated(&g))) return rc;
+    }
+    if (dw && (rc = conv_bwd_weight(who, p, x, g, dw))) return rc;
+    if (db && (rc = conv_bwd_bias(who, p, g, db))) return rc;
+  }
+  if (dx && x_total) {
+    rc = run_direct3x3(MODE_BWD_DATA, p, dy_is_scalar ? y : dy, w, nullptr, dx, 0, gate_mode, y, dy);
+    if (rc == 1) {
+      if ((rc = gated(&g))) return rc;
+      rc = conv_bwd_data(who, p, g, w, dx);
+    }
+    if (rc) return rc;
+  }
+  return ENDIA_HIP_OK;
 }
 
 }  // namespace
@@ -1353,6 +1504,12 @@ int32_t endia_hip_conv2d_bwd_data(const endia_hip_conv2d_desc* d, const float* d
 int32_t endia_hip_conv2d_bwd_weight(const endia_hip_conv2d_desc* d, const float* x, const float* dy, float* dw) {
   ENDIA_CONV_PARAMS(d);
   return conv_bwd_weight(__func__, p, x, dy, dw);
+}
+
+int32_t endia_hip_conv2d_bwd_relu(const endia_hip_conv2d_desc* d, const float* x, const float* w, const float* y,
+                                  const float* dy, int32_t dy_is_scalar, float* dx, float* dw, float* db) {
+  ENDIA_CONV_PARAMS(d);
+  return conv_bwd_relu("conv2d_bwd_relu", p, x, w, y, dy, dy_is_scalar, dx, dw, db);
 }
 
 int32_t endia_hip_conv2d_bwd_bias(const endia_hip_conv2d_desc* d, const float* dy, float* db) {

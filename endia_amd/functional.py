@@ -1150,23 +1150,6 @@ def _pair(v):
     return (int(v), int(v)) if np.isscalar(v) else (int(v[0]), int(v[1]))
 
 
-_relu_grad_of_scalar = [None]
-
-
-def _relu_grad_from_output(out, grad):
-    """grad * [out > 0] in one pass. A cotangent that is one value spread over the whole array (the gradient of
-    a mean or a sum: a stride-0 view) is read as a scalar, so no full-size copy of it is ever written."""
-    if grad.size() and all(st == 0 or n == 1 for st, n in zip(grad._strides, grad._shape)) and not grad.is_complex_:
-        if _relu_grad_of_scalar[0] is None:
-            _relu_grad_of_scalar[0] = _fusion.fuse(lambda o, g: mul(greater(o, 0.0), g), "relu_grad")
-        one = Array([1], _buffer=grad._buf, _strides=[1], _offset=grad._offset)
-        return _relu_grad_of_scalar[0](detach(out), one)
-    g = contiguous(grad)
-    gp = Array.empty(out._shape)
-    L.call("endia_hip_unary_vjp_from_output", L.OP_RELU, out.size(), out.data_ptr(), g.data_ptr(), gp.data_ptr())
-    return gp
-
-
 def conv2d(x, kernel, bias=None, stride=1, padding=0, dilation=1, groups=1, act=None):
     """NCHW cross-correlation (conv2d_op.mojo:88-196; tuple order is (height, width)). The reference has
     no backward rule for it (conv2d_op.mojo:198-200); the VJP here is the adjoint of its forward loop.
@@ -1199,7 +1182,18 @@ def conv2d(x, kernel, bias=None, stride=1, padding=0, dilation=1, groups=1, act=
             raise NotImplementedError("conv2d has no second-order rule")
         if grad.ndim() != out_.ndim():
             raise NotImplementedError("conv2d has no rule for a cotangent with leading Jacobian axes (non-scalar output)")
-        g = contiguous(_relu_grad_from_output(out_, grad)) if act == "relu" else contiguous(grad)
+        if act == "relu":
+            # one call for all three; the ReLU's derivative is applied to the cotangent as the kernels load it. A
+            # cotangent that is one value spread over the whole array (the gradient of a mean or a sum: a stride-0
+            # view) is handed over as that one value.
+            scalar = bool(grad.size()) and all(st == 0 or n == 1 for st, n in zip(grad._strides, grad._shape))
+            g = Array([1], _buffer=grad._buf, _strides=[1], _offset=grad._offset) if scalar else contiguous(grad)
+            wanted = [p_._requires_grad for p_ in primals]
+            outs = [Array.empty(p_._shape) if w_ else None for p_, w_ in zip(primals, wanted)]
+            L.call("endia_hip_conv2d_bwd_relu", ctypes.byref(desc), xs.data_ptr(), ks.data_ptr(), out_.data_ptr(), g.data_ptr(),
+                   1 if scalar else 0, *[o.data_ptr() if o is not None else None for o in (outs + [None])[:3]])
+            return outs
+        g = contiguous(grad)
         res = []
         if primals[0]._requires_grad:
             dx = Array.empty(primals[0]._shape)

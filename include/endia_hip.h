@@ -356,6 +356,14 @@ ENDIA_API int32_t endia_hip_conv2d_bwd_data(const endia_hip_conv2d_desc* d, cons
 ENDIA_API int32_t endia_hip_conv2d_bwd_weight(const endia_hip_conv2d_desc* d, const float* x, const float* dy,
                                     float* dw);
 ENDIA_API int32_t endia_hip_conv2d_bwd_bias(const endia_hip_conv2d_desc* d, const float* dy, float* db);
+/* Every gradient of y = relu(conv(x,w)+bias) in one call, from the stored y (what endia_hip_conv2d_fwd wrote with
+ * act = RELU): the ReLU's derivative [y > 0] (relu_op.mojo:51-53) is applied to dy as the kernels load it, so
+ * dy * [y > 0] is not written to memory where the fast kernels apply (it is written once where they do not).
+ * dy_is_scalar != 0: dy points at ONE device float that stands for every element of the cotangent (the gradient
+ * of a mean or a sum). dx, dw, db may each be null; x is read only for dw, w only for dx. */
+ENDIA_API int32_t endia_hip_conv2d_bwd_relu(const endia_hip_conv2d_desc* d, const float* x, const float* w,
+                                  const float* y, const float* dy, int32_t dy_is_scalar, float* dx, float* dw,
+                                  float* db);
 
 /* ---- conv3d, [N,C,D,H,W] with kernel [K,C,T,R,S], groups = 1: Conv3d.__call__ (spacial_ops/conv3d_op.mojo:104-259),
  *      output extents per axis (in + 2*pad - dil*(k-1) - 1) / stride + 1 (conv3d_op.mojo:71-101). Conv1d

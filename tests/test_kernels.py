@@ -552,6 +552,60 @@ def test_conv2d_paths_vs_oracle(dev, xs, ws, st,pd, dl):
     assert_close(dev.get(ddw, w.shape), tw.grad.numpy(), what="dw vs torch")
 
 
+@pytest.mark.parametrize("scalar", [True, False])
+@pytest.mark.parametrize("xs,ws,st,pd,dl", FAST_CASES)
+def test_conv2d_bwd_relu_matches_separate_passes(dev, xs, ws, st, pd, dl, scalar):
+    """endia_hip_conv2d_bwd_relu (the ReLU's derivative applied as the gradient kernels load dy) against the
+    oracle's gradients of the same convolution for the cotangent dy * [y > 0] computed on the host from the
+    DEVICE's y (so that no element sits on the other side of zero), and bit for bit against the plain entry points
+    fed that cotangent for dx and dw, which run the same kernels on the same numbers. Cases cover the fused
+    kernels and the ones where the gated cotangent is written out first; scalar: dy is one device float."""
+    rng = np.random.default_rng(sum(xs) + sum(ws) + 1)
+    x = rng.standard_normal(xs).astype(np.float32)
+    w = (rng.standard_normal(ws) * 0.3).astype(np.float32)
+    b = rng.standard_normal(ws[0]).astype(np.float32)
+    d = _desc(x, w, st, pd, dl)
+    y_shape = R.conv2d(x, w, b, st, pd, dl).shape
+    dx_, dw_, db_ = dev.put(x), dev.put(w), dev.put(b)
+    dy = dev.alloc(4 * int(np.prod(y_shape)))
+    dev.call("endia_hip_conv2d_fwd", ctypes.byref(d), dx_, dw_, db_, dy, L.OP_RELU)
+    y = dev.get(dy, y_shape)
+    assert 0.2 < (y > 0).mean() < 0.8
+    if scalar:
+        gy = np.full(y_shape, 1.0 / y.size, np.float32)
+        dg = dev.put(gy.reshape(-1)[:1])
+    else:
+        gy = rng.standard_normal(y_shape).astype(np.float32)
+        dg = dev.put(gy)
+    gated = np.where(y > 0, gy, np.float32(0)).astype(np.float32)
+    dx_ref, dw_ref, _ = R.conv2d_bwd(x, w, gated, st, pd, dl)
+    # the oracle adds db up one float at a time, which drifts by 2e-4 over 37632 EQUAL terms (the scalar case, where
+    # every addition rounds the same way); the sum itself in float64 is the reference here
+    db_ref = gated.astype(np.float64).sum(axis=(0, 2, 3))
+    ddx, ddw, ddb = dev.alloc(x.nbytes), dev.alloc(w.nbytes), dev.alloc(b.nbytes)
+    dev.call("endia_hip_conv2d_bwd_relu", ctypes.byref(d), dx_, dw_, dy, dg, 1 if scalar else 0, ddx, ddw, ddb)
+    got_dx, got_dw, got_db = dev.get(ddx, x.shape), dev.get(ddw, w.shape), dev.get(ddb, b.shape)
+    assert_close(got_dx, dx_ref, what="dx")
+    assert_close(got_dw, dw_ref, what="dw")
+    assert_close(got_db, db_ref, what="db")
+    dgated, pdx, pdw = dev.put(gated), dev.alloc(x.nbytes), dev.alloc(w.nbytes)
+    dev.call("endia_hip_conv2d_bwd_data", ctypes.byref(d), dgated, dw_, pdx)
+    dev.call("endia_hip_conv2d_bwd_weight", ctypes.byref(d), dx_, dgated, pdw)
+    assert np.array_equal(got_dx, dev.get(pdx, x.shape))
+    assert np.array_equal(got_dw, dev.get(pdw, w.shape))
+    # each output on its own: the others null
+    for which in range(3):
+        outs = [dev.alloc(x.nbytes) if which == 0 else None, dev.alloc(w.nbytes) if which == 1 else None,
+                dev.alloc(b.nbytes) if which == 2 else None]
+        dev.call("endia_hip_conv2d_bwd_relu", ctypes.byref(d), dx_, dw_, dy, dg, 1 if scalar else 0, *outs)
+        if which == 0:
+            assert np.array_equal(dev.get(outs[0], x.shape), got_dx)
+        elif which == 1:
+            assert np.array_equal(dev.get(outs[1], w.shape), got_dw)
+        else:
+            assert_close(dev.get(outs[2], b.shape), db_ref, what="db alone")
+
+
 def test_conv2d_full_size_properties(dev):
     """The benchmark configuration (64 x 64 x 56 x 56 input, 128 filters 3 x 3, pad 1) is too large for the
     CPU loop; check it through the adjoint identities <conv(x,w), dy> = <x, dX> = <w, dW>, through db
