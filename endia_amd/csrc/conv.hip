@@ -653,15 +653,15 @@ __global__ __launch_bounds__(WGM* WGN * 64, FM* FN >= 6 ? 2 : 4) void conv_wgrad
 // the word at (its row + r, its column + s), an LDS read whose offset is a constant of the instruction. The
 // reduction over one chunk is 8 channels x 9 taps = 72 long; the MFMA takes it in pairs (half-wave h holds the
 // second element), and the pair is made of the SAME tap in two neighbouring channels, so the half-waves differ by
-// one cached channel, a constant folded into the lane's base address. Within a chunk, element k = 8j + 4h + i of
-// the packed weights belongs to step 4j + i = 9 * (channel pair) + 3r + s and to channel 2 * (channel pair) + h.
+// one cached channel, a constant folded into the lane's base address. Within a chunk, element (group j, row, h, i)
+// of the packed weights belongs to step 4j + i = 9 * (channel pair) + 3r + s and to channel 2 * (channel pair) + h.
 // The weights do not pass through LDS at all (see the tile function). 72 or 144 MFMAs per wave between two barriers
 // (the dense kernel has 64 at its large tile), three or four work-groups per CU.
 struct DirectArgs {
   const float* src;   // [N, Cred, SH, SW]
   const float* gate;  // GATE 2: same shape as src, which counts where gate > 0 (GATE 1: src IS the gate and every
   const float* gscalar;  // element that passes it is worth *gscalar)
-  const float* wp;    // [chunks][tiles_m * BM][72], packed as described above
+  const float* wp;    // [chunks][9 groups][tiles_m * BM][8], packed as described above
   const float* bias;
   float* out;         // [N, Mrows, OH, OW]
   int Mrows, Cred, chunks, OH, OW, SH, SW, Ncols, NOH;
@@ -769,21 +769,25 @@ __device__ __forceinline__ void direct3x3_tile(const DirectArgs& a, int tm, int 
   floatx16 acc[FM][FN];
   zero_acc<FM, FN>(acc);
   // The weights go from memory straight into the A fragments: every lane reads its own rows of the packed weights
-  // (group jg of a chunk is the 16 bytes at 8 * jg + 4 * h floats of the row), one group of four steps ahead of the
-  // MFMAs that use it. All work-groups read the same few hundred KiB, which stay in L2; LDS holds the row cache alone.
+  // (group jg of a chunk holds, for every row, the four steps of either half-wave: 32 bytes a row, 1 KiB a fragment
+  // in one piece), three groups of four steps ahead of the MFMAs that use them. All work-groups read the same few
+  // hundred KiB, which stay in L2; LDS holds the row cache alone.
+  constexpr int AD = 3;  // groups in flight; 9 groups a chunk, so a group's slot is a constant of the unrolled loop
   uint32_t arow[FM];
 #pragma unroll
-  for (int fm = 0; fm < FM; ++fm) arow[fm] = (uint32_t)(((m0 + a_row + 32 * fm) * KC + 4 * h) * 4);
-  float4 afn[FM];
+  for (int fm = 0; fm < FM; ++fm) arow[fm] = (uint32_t)(((m0 + a_row + 32 * fm) * 8 + 4 * h) * 4);
+  const uint32_t g_step = (uint32_t)(a.tiles_m * BM) * 32u;  // bytes between the groups of the packed weights
+  float4 afn[AD][FM];
   auto fetch_a = [&](int chunk, int jg) {
 #pragma unroll
     for (int fm = 0; fm < FM; ++fm) {
-      v4i v = __builtin_amdgcn_raw_buffer_load_b128(rs_w, (int)(arow[fm] + 32u * jg), (int)(chunk * w_step), 0);
-      afn[fm] = *reinterpret_cast<float4*>(&v);
+      v4i v = __builtin_amdgcn_raw_buffer_load_b128(rs_w, (int)arow[fm], (int)((chunk * (KC / 8) + jg) * g_step), 0);
+      afn[jg % AD][fm] = *reinterpret_cast<float4*>(&v);
     }
   };
   load(0);
-  fetch_a(0, 0);
+#pragma unroll
+  for (int jg = 0; jg < AD; ++jg) fetch_a(0, jg);
   __syncthreads();  // border columns zeroed before the first rows land in the cache
   store();
   __syncthreads();
@@ -795,11 +799,11 @@ __device__ __forceinline__ void direct3x3_tile(const DirectArgs& a, int tm, int 
       float af[FM][4];
 #pragma unroll
       for (int fm = 0; fm < FM; ++fm) {
-        const float4 t = afn[fm];
+        const float4 t = afn[jg % AD][fm];
         af[fm][0] = t.x; af[fm][1] = t.y; af[fm][2] = t.z; af[fm][3] = t.w;
       }
-      if (jg + 1 < KC / 8) fetch_a(chunk, jg + 1);
-      else if (more) fetch_a(chunk + 1, 0);
+      if (jg + AD < KC / 8) fetch_a(chunk, jg + AD);
+      else if (more) fetch_a(chunk + 1, jg + AD - KC / 8);
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
         const int q = 4 * jg + i, ccp = q / 9, tap = q - 9 * ccp, r = tap / 3, sx = tap - 3 * r;
@@ -874,10 +878,12 @@ __global__ __launch_bounds__(TPB) void pack_direct3x3_kernel(const float* __rest
   const int Mrows = flip ? C : K, Cred = flip ? K : C;
   const int64_t total = (int64_t)chunks * rows_pad * 72;
   for (int64_t idx = (int64_t)blockIdx.x * TPB + threadIdx.x; idx < total; idx += (int64_t)gridDim.x * TPB) {
-    const int k = (int)(idx % 72);
-    const int64_t rest = idx / 72;
-    const int m = (int)(rest % rows_pad), chunk = (int)(rest / rows_pad);
-    const int j = k >> 3, h = (k >> 2) & 1, i = k & 3, q = 4 * j + i, ccp = q / 9, tap = q - 9 * ccp, r = tap / 3, s = tap - 3 * r;
+    // [chunk][group j of four steps][row m][half-wave h][step i]: the 64 lanes of a fragment load (32 rows, both
+    // half-waves) read 1 KiB in one piece
+    const int e = (int)(idx & 7), h = e >> 2, i = e & 3;
+    const int64_t rest = idx >> 3;
+    const int m = (int)(rest % rows_pad), gj = (int)(rest / rows_pad), j = gj % 9, chunk = gj / 9;
+    const int q = 4 * j + i, ccp = q / 9, tap = q - 9 * ccp, r = tap / 3, s = tap - 3 * r;
     const int ch = chunk * 8 + 2 * ccp + h;
     float v = 0.f;
     if (m < Mrows && ch < Cred)
