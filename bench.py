@@ -466,11 +466,10 @@ def run_hvp(nd, steps, warmup):
         out = mlp.forward(x)
         loss = nd.sum(out * out)
         loss.backward(create_graph=True)
-        s = None
-        for p, v in zip(mlp.params(), vs):
-            term = nd.sum(p.grad() * v)
-            s = term if s is None else s + term
-        hv = nd.grad(outs=s, inputs=mlp.params())
+        firsts = [p.grad() for p in mlp.params()]
+        # the second reverse pass starts from the first-order gradients with v as their cotangents: the gradient of
+        # <gradients, v> without forming the eight dot products
+        hv = nd.grad(outs=firsts, inputs=mlp.params(), grad_outs=[nd.reshape(v, f.shape()) for v, f in zip(vs, firsts)])
         loss.zero_grad()
         return hv
 

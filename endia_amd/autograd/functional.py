@@ -62,12 +62,6 @@ def backward(arg, create_graph=False):
 def jacrev(arg, create_graph=False):
     out = arg
     trace = top_order(out)
-    for node in trace:
-        node._consumers = 0
-    for node in trace:
-        for a in node._args:
-            a._consumers += 1
-
     dims = out._shape[-1] if out._shape else 1
     if out.ndim() != 1 or dims != 1:
         n = out.size()
@@ -75,6 +69,41 @@ def jacrev(arg, create_graph=False):
     else:
         seed = _seed_one()
     out.grad_(seed)
+    _reverse_walk(trace, create_graph)
+
+
+class _Root:
+    """Stands above several outputs so that one post-order walk covers all of their graphs."""
+
+    def __init__(self, outs):
+        self._args, self._vjp, self._consumers = list(outs), None, 0
+
+
+def vjp_from(outs, cotangents, create_graph=False):
+    """One reverse pass from several outputs at once, each seeded with its own cotangent (same shape as the
+    output) instead of ones. No counterpart in the reference, whose grad(outs, inputs) seeds every output with
+    ones, one backward pass per output (functional.mojo:70-97); this is the cotangent argument of a VJP, and
+    it computes the gradient of sum_i <out_i, cotangent_i> without forming that sum."""
+    outs, cotangents = list(outs), list(cotangents)
+    if len(outs) != len(cotangents):
+        raise ValueError("vjp_from: %d outputs but %d cotangents" % (len(outs), len(cotangents)))
+    for o, c in zip(outs, cotangents):
+        if list(o.shape()) != list(c.shape()):
+            raise ValueError("vjp_from: cotangent of shape %s for an output of shape %s" % (c.shape(), o.shape()))
+    trace = top_order(_Root(outs))
+    for o, c in zip(outs, cotangents):
+        o.grad_(F.add(o._grad, c) if o.has_grad() else c)
+    _reverse_walk(trace, create_graph)
+
+
+def _reverse_walk(trace, create_graph):
+    """The trace in reverse: every node's VJP rule, contributions to one tensor summed with `add`
+    (functional.mojo:46-65). The outputs' gradients are already in place."""
+    for node in trace:
+        node._consumers = 0
+    for node in trace:
+        for a in node._args:
+            a._consumers += 1
 
     prev = _building_graph[0]
     _building_graph[0] = bool(create_graph)
@@ -116,11 +145,16 @@ def zero_grad_rec(out):
 remove_grad_rec = zero_grad_rec
 
 
-def grad(outs=None, inputs=None, retain_grads=True, create_graph=False, argnums=None):
+def grad(outs=None, inputs=None, retain_grads=True, create_graph=False, argnums=None, grad_outs=None):
     """Two forms, as in the reference:
 
     grad(outs=[...], inputs=[...]) -> list of gradients (functional.mojo:70-97);
     grad(f, argnums=...)           -> Callable computing the gradient of f (functional.mojo:100-128).
+
+    grad_outs (not in the reference): one cotangent per output, of the output's shape; the outputs are then
+    walked in ONE reverse pass seeded with them (vjp_from), which yields the gradient of
+    sum_i <outs[i], grad_outs[i]>: a Hessian-vector product when the outputs are first-order gradients
+    taken with create_graph=True.
     """
     if isinstance(outs, Callable):
         f = outs
@@ -134,8 +168,11 @@ def grad(outs=None, inputs=None, retain_grads=True, create_graph=False, argnums=
         remove_grad_rec(o)
     for i in inputs:
         remove_grad_rec(i)
-    for o in outs:
-        o.backward(create_graph=create_graph)
+    if grad_outs is not None:
+        vjp_from(outs, [grad_outs] if isinstance(grad_outs, Array) else grad_outs, create_graph)
+    else:
+        for o in outs:
+            o.backward(create_graph=create_graph)
     res = []
     for i in inputs:
         g = i.grad()

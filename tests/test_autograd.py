@@ -370,10 +370,12 @@ def test_mlp_tanh_adam(nd, golden, fused):
         assert_close(mlp.biases[i].to_numpy(), g["b%d_after" % i], what="b%d after Adam" % i)
 
 
+@pytest.mark.parametrize("seeded", [False, True])
 @pytest.mark.parametrize("fused", [True, False])
-def test_hvp_double_backward(nd, golden, fused):
+def test_hvp_double_backward(nd, golden, fused, seeded):
     """Hessian-vector product by create_graph=True double backward (README.md:69-71 pattern) on a sin MLP
-    with loss = sum(out^2); also <u, Hv> = <v, Hu>."""
+    with loss = sum(out^2); also <u, Hv> = <v, Hu>. seeded: the second pass starts from the first-order
+    gradients with v as their cotangents (grad_outs) instead of from the scalar sum <gradients, v>."""
     g = golden("hvp_sin")
     mlp, _ = _load_mlp(nd, g, 3, "sin", fused)
     x = nd.array(g["x"])
@@ -382,12 +384,17 @@ def test_hvp_double_backward(nd, golden, fused):
         out = mlp.forward(x)
         loss = nd.sum(out * out)
         loss.backward(create_graph=True)
-        s = None
-        for p, v in zip(mlp.params(), vs):
-            term = nd.sum(p.grad() * nd.reshape(nd.array(v), p.grad().shape()))
-            s = term if s is None else s + term
         grads = [p.grad().to_numpy() for p in mlp.params()]
-        hv = nd.grad(outs=s, inputs=mlp.params())
+        if seeded:
+            firsts = [p.grad() for p in mlp.params()]
+            hv = nd.grad(outs=firsts, inputs=mlp.params(),
+                         grad_outs=[nd.reshape(nd.array(v), f.shape()) for v, f in zip(vs, firsts)])
+        else:
+            s = None
+            for p, v in zip(mlp.params(), vs):
+                term = nd.sum(p.grad() * nd.reshape(nd.array(v), p.grad().shape()))
+                s = term if s is None else s + term
+            hv = nd.grad(outs=s, inputs=mlp.params())
         res = [h.to_numpy() for h in hv]
         loss.zero_grad()
         return float(loss.item()), grads, res

@@ -131,7 +131,8 @@ def test_hvp_every_tensor_at_full_size(nd, torch):
     bound2 = [max(1e-4, 2 * mean_rel(a.numpy().reshape(-1), r.numpy().reshape(-1))) for a, r in zip(hv_f32, hv_ref)]
     print("mean-relative bounds from the float32 CPU run: gradient %s, H v %s" % (["%.1e" % b for b in bound1], ["%.1e" % b for b in bound2]))
 
-    for fused in (True, False):
+    # fused / per-op layers; the second pass from the scalar <gradients, v> or seeded with v (grad_outs)
+    for fused, seeded in ((True, True), (True, False), (False, False)):
         mlp = nd.nn.MLP([n] * (layers + 1), compute_backward=True, activation="sin", fused=fused)
         for i in range(layers):
             mlp.weights[i] = nd.array(Ws[i], requires_grad=True)
@@ -140,15 +141,20 @@ def test_hvp_every_tensor_at_full_size(nd, torch):
         loss = nd.sum(out * out)
         loss.backward(create_graph=True)
         first = [p.grad().to_numpy() for p in mlp.params()]
-        total = None
-        for p, v in zip(mlp.params(), [v for pair in zip(vW, vb) for v in pair]):
-            term = nd.sum(p.grad() * nd.reshape(nd.array(v), p.grad().shape()))
-            total = term if total is None else total + term
-        hv = [a.to_numpy() for a in nd.grad(outs=total, inputs=mlp.params())]
+        firsts = [p.grad() for p in mlp.params()]
+        vs_dev = [nd.reshape(nd.array(v), f.shape()) for f, v in zip(firsts, [v for pair in zip(vW, vb) for v in pair])]
+        if seeded:
+            hv = [a.to_numpy() for a in nd.grad(outs=firsts, inputs=mlp.params(), grad_outs=vs_dev)]
+        else:
+            total = None
+            for f, v in zip(firsts, vs_dev):
+                term = nd.sum(f * v)
+                total = term if total is None else total + term
+            hv = [a.to_numpy() for a in nd.grad(outs=total, inputs=mlp.params())]
         assert_close([float(loss.item())], [float(tloss)], tol=1e-5, what="loss")
         loss.zero_grad()
         for i, (g1, g2, r1, r2) in enumerate(zip(first, hv, grads, hv_ref)):
-            name = "%s of layer %d (fused=%s)" % ("W" if i % 2 == 0 else "b", i // 2, fused)
+            name = "%s of layer %d (fused=%s, seeded=%s)" % ("W" if i % 2 == 0 else "b", i // 2, fused, seeded)
             assert_close(g1.reshape(-1), r1.detach().numpy().reshape(-1), what="gradient, " + name, mean_tol=bound1[i])
             assert_close(g2.reshape(-1), r2.numpy().reshape(-1), what="H v, " + name, mean_tol=bound2[i])
             print("%s: H v mean-relative %.2e (bound %.1e)" % (name, mean_rel(g2.reshape(-1), r2.numpy().reshape(-1)), bound2[i]))
