@@ -886,12 +886,29 @@ def reduce_add(x, axes, _scale=1.0):
         L.call("endia_hip_reduce_add", x.ndim(), L.i64_array(x._shape), mask, src.data_ptr(), out.data_ptr(),
                float(_scale), 1 if x.is_complex_ else 0)
     in_shape = list(x._shape)
+    scale = float(_scale)
 
     def vjp(primals, grad, out_):
         lead = grad.ndim() - out_.ndim()
+        if scale != 1.0:
+            # the seed of a scalar loss times a constant is a constant: kept per value, so that a step spends no launch on it
+            grad = _scaled_seed(scale) if grad._is_seed else grad * scale
         return [expand(grad, list(grad._shape[:lead]) + in_shape)]
 
     return _register(out, [x], "reduce_add", vjp)
+
+
+_SCALED_SEEDS = {}
+
+
+def _scaled_seed(value):
+    """full([1], value), made once per value and never written: what ones(1) * value is for every backward pass."""
+    arr = _SCALED_SEEDS.get(value)
+    if arr is None:
+        if len(_SCALED_SEEDS) > 64:
+            _SCALED_SEEDS.clear()
+        arr = _SCALED_SEEDS[value] = full([1], value)
+    return arr
 
 
 def sum(x):
@@ -902,9 +919,17 @@ def sum(x):
 def mean(x, axes=None, keepdims=False):
     """mean_op.mojo:35-65: reduce_add divided by the number of reduced elements."""
     axes = list(range(x.ndim())) if axes is None else axes
-    res = reduce_add(x, axes)
-    divisor = float(x.size() // max(res.size(), 1))
-    out = res / divisor
+    kept = 1
+    for i, n in enumerate(x._shape):
+        if i not in _norm_axes(list(axes), x.ndim()):
+            kept *= n
+    divisor = float(x.size() // max(kept, 1))
+    if x.is_complex_ or divisor == 0.0:
+        out = reduce_add(x, axes) / divisor
+    else:
+        # the division rides in the reduction's last stage as a multiplication by 1 / count (one rounding away from
+        # the reference's sum / count), and in the VJP as a constant factor
+        out = reduce_add(x, axes, _scale=1.0 / divisor)
     return out if keepdims else squeeze(out)
 
 
