@@ -351,6 +351,9 @@ def conv_table(reps=10):
         ("conv2d_bwd_data", lambda: L.call("endia_hip_conv2d_bwd_data", ref, dy, w, dx), flop, "mfma"),
         ("conv2d_bwd_weight", lambda: L.call("endia_hip_conv2d_bwd_weight", ref, x, dy, dw), flop, "mfma"),
         ("conv2d_bwd_bias", lambda: L.call("endia_hip_conv2d_bwd_bias", ref, dy, db), 4.0 * N * K * P * Q, "hbm"),
+        # all three gradients of relu(conv + bias) from the stored output, dy * [y > 0] formed in the operand loads
+        ("conv2d_bwd_relu (dx, dw, db)", lambda: L.call("endia_hip_conv2d_bwd_relu", ref, x, w, y, dy, 0, dx, dw, db), 2 * flop, "mfma"),
+        ("conv2d_bwd_relu (dw, db; scalar dy)", lambda: L.call("endia_hip_conv2d_bwd_relu", ref, x, w, y, dy, 1, None, dw, db), flop, "mfma"),
     ]
     # conv3d: x [8,32,16,56,56], w [64,32,3,3,3], stride 1, pad 1: 2*N*K*C*T*R*S*O*P*Q = 44.4 GFLOP per pass
     d3 = L.Conv3dDesc()
@@ -491,7 +494,7 @@ def run_hvp(nd, steps, warmup):
     nd.synchronize()
     elapsed = time.perf_counter() - t0
     flops = 31 * 2.0 * B * Wd * Wd
-    roof = gemm_roofline(L, elapsed, flops * steps, "sgemm_mfma_kernel, 64x64x32 tiles (1024 x 2048 x 2048 products)")
+    roof = gemm_roofline(L, elapsed, flops * steps, "sgemm_mfma_kernel<F = 1> (64x64x32 tiles, K split inside the launch): the 1024 x 2048 x 2048 products")
     return {"metric": "Hessian-vector products/s, 4 x 2048 sin MLP, batch 1024 (double backward)", "value": 1.0 / dt,
             "unit": "HVP/s", "n_gpus": 1, "ms_per_step": dt * 1e3, "higher_is_better": True, "vs_baseline": None,
             "algorithmic_gemm_tflops": flops / dt / 1e12,
@@ -521,40 +524,43 @@ def run_complex(nd, steps, warmup, algo):
         return loss
 
     from endia_amd import _lib as L
+    # `value` is taken under the Wirtinger rule (g B^H, A^H g; the conjugations are flags of the complex GEMM), which
+    # yields the gradient of the real loss that the float64 checks of this configuration compare against; the
+    # reference's coded rule (no conjugation, matmul_op.mojo:278-283) costs the same launches and is timed beside it
     for _ in range(warmup):
-        step()
+        step(True)
     nd.synchronize()
     t0 = time.perf_counter()
     for _ in range(steps):
-        step()
+        step(True)
     nd.synchronize()
     dt = (time.perf_counter() - t0) / steps
-    # the same step under the Wirtinger rule (g B^H, A^H g): the conjugations are flags of the complex GEMM
     for _ in range(warmup):
-        step(True)
+        step(False)
     nd.synchronize()
     t0 = time.perf_counter()
     for _ in range(steps):
-        step(True)
+        step(False)
     nd.synchronize()
-    dt_wirtinger = (time.perf_counter() - t0) / steps
+    dt_reference = (time.perf_counter() - t0) / steps
     L.call("endia_hip_gemm_timing_begin")  # second pass, with an event pair around every GEMM launch
     t0 = time.perf_counter()
     for _ in range(steps):
-        step()
+        step(True)
     nd.synchronize()
     elapsed = time.perf_counter() - t0
     flops = 11 * 8.0 * n * n * n  # algorithmic: 8 real flops per complex multiply-add, whichever algorithm runs
-    roof = gemm_roofline(L, elapsed, flops * steps, "sgemm_mfma_kernel, " + (
-        "three real 2048^3 products per complex product in one batched launch" if algo == "3m"
-        else "one real 2048 x 4096 x 4096 product per complex product (B embedded as a 2K x 2N real matrix)"))
+    roof = gemm_roofline(L, elapsed, flops * steps, (
+        "sgemm_mfma_kernel<F = 2> (128x128x32 tiles): three real 2048^3 products per complex product in one batched launch" if algo == "3m"
+        else "sgemm_lone_kernel<FM = 4, FN = 2> (256x128x32 tiles, one work-group per CU): one real 2048 x 4096 x 4096 product "
+             "per complex product (B embedded as a 2K x 2N real matrix)"))
     return {"metric": "fwd+bwd steps/s, complex64 MLP 4 x 2048, batch 2048, algorithm " + algo, "value": 1.0 / dt,
             "unit": "steps/s", "n_gpus": 1, "ms_per_step": dt * 1e3, "higher_is_better": True, "vs_baseline": None,
             "algorithmic_gemm_tflops": flops / dt / 1e12,
             "frac_of_fp32_mfma_peak": flops / dt / 1e12 / FP32_MFMA_PEAK_TFLOPS, "steps": steps, "warmup": warmup,
-            "gradient_rule": "reference (no conjugation, matmul_op.mojo:278-283)",
-            "wirtinger_rule": {"ms_per_step": dt_wirtinger * 1e3, "steps_per_s": 1.0 / dt_wirtinger,
-                               "algorithmic_gemm_tflops": flops / dt_wirtinger / 1e12},
+            "gradient_rule": "wirtinger (dA = g B^H, dB = A^H g)",
+            "reference_rule": {"rule": "no conjugation, matmul_op.mojo:278-283", "ms_per_step": dt_reference * 1e3,
+                               "steps_per_s": 1.0 / dt_reference, "algorithmic_gemm_tflops": flops / dt_reference / 1e12},
             "dtype": "c64 (f32 pairs)", "data": "synthetic",
             "config": {"workload": "complex_mlp: 4 x complex Linear(2048->2048), identity, loss sum|out|^2, batch 2048, " + algo},
             "roofline": roof}
@@ -630,7 +636,10 @@ def main():
     if args.workload == "sine_mlp" and not args.eager:
         # launch-latency bound: replay the step as one HIP graph (same kernels, same results)
         captured = nd.capture(lambda: train_step(nd, mlp, opt, x, y))
-        config["execution"] = "HIP graph replay of the eager step"
+        config["execution"] = "HIP graph replay of the eager step" + (
+            "" if os.environ.get("ENDIA_SINE_PER_LAYER") else
+            "; nn.MLP(fused='model'): 5 launches a step (forward of all layers, MSE, cotangents of all layers, all weight "
+            "and bias gradients, optimizer over all 16 tensors)")
     L.call("endia_hip_gemm_timing_begin")
     t0 = time.perf_counter()
     for _ in range(args.steps):
@@ -657,7 +666,7 @@ def main():
         flops_per_launch = g_flops.value / launches.value
         achieved = flops_per_launch / (avg_ms * 1e-3) / 1e12
         out["roofline"] = {
-            "bound": "mfma", "kernel": "sgemm_mfma256_kernel (fp32 v_mfma_f32_32x32x2, 256x256x32 tiles, one work-group per CU)",
+            "bound": "mfma", "kernel": "sgemm_lone_kernel<FM = 4, FN = 4> (fp32 v_mfma_f32_32x32x2, 256x256x32 tiles, one work-group per CU)",
             "achieved": achieved, "peak": FP32_MFMA_PEAK_TFLOPS, "unit": "TFLOP/s", "frac": achieved / FP32_MFMA_PEAK_TFLOPS,
             "traffic": GEMM_TRAFFIC_BYTES if args.workload == "wide_mlp" else None,
             "traffic_source": "rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, see profiles/kernels_wide_mlp_counters.md",
