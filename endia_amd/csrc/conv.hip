@@ -514,7 +514,7 @@ struct WgradVecArgs {
   const float* gate;  // GATE > 0: the stored output y of relu(conv + bias), same shape; dy counts where y > 0
   const int* table;   // [tiles_n * BN] byte offset of tap t inside a padded image; OOB_OFFSET past Kd
   float* part;
-  float* bias_part;   // GATE > 0, may be null: [splits][K] sums of the gated dy over each split's columns
+  float* bias_part;   // may be null: [splits][K] sums of the (gated) dy over each split's columns
   int K, Kd, OPQ, PQ, Q, sh, Wp, img_floats, zstep;
   int total_j, chunk;
   FastDiv d_opq, d_pq, d_q;
@@ -523,8 +523,8 @@ struct WgradVecArgs {
 };
 
 // GATE 0: dy as it is. GATE 1 / 2: dy (1: a scalar, 2: a tensor) gated by [y > 0] as the A operand is loaded, so that
-// the gradient of the ReLU is never written out; the work-groups of the first tile column also sum the rows of
-// what they load, which is the bias gradient.
+// the gradient of the ReLU is never written out. In every mode the work-groups of the first tile column can also sum
+// the rows of what they load, which is the bias gradient.
 template <int WGM, int WGN, int FM, int FN, int GATE>
 __global__ __launch_bounds__(WGM* WGN * 64, FM* FN >= 6 ? 2 : 4) void conv_wgrad_vec_kernel(WgradVecArgs a) {
   constexpr int NT = WGM * WGN * 64, BM = WGM * FM * 32, BN = WGN * FN * 32;
@@ -556,7 +556,7 @@ __global__ __launch_bounds__(WGM* WGN * 64, FM* FN >= 6 ? 2 : 4) void conv_wgrad
   const __amdgpu_buffer_rsrc_t rs_x = make_rsrc(a.xpad, a.x_bytes);
   float4 ra[PA], rb[PB], rg[GATE == 2 ? PA : 1];
   const float dy_scalar = GATE == 1 ? a.dy[0] : 0.f;
-  const bool sum_rows = GATE > 0 && a.bias_part != nullptr && tn == 0;
+  const bool sum_rows = a.bias_part != nullptr && tn == 0;
   float row_sum[PA];
 #pragma unroll
   for (int i = 0; i < PA; ++i) row_sum[i] = 0.f;
@@ -583,7 +583,8 @@ __global__ __launch_bounds__(WGM* WGN * 64, FM* FN >= 6 ? 2 : 4) void conv_wgrad
 #pragma unroll
     for (int i = 0; i < PB; ++i) rb[i] = buffer_load_f4(rs_x, cb + rowb[i]);
   };
-  auto store = [&]() {
+  // applied to the staged pieces in registers ahead of the barrier that precedes the stores
+  auto gate = [&]() {
     if (GATE > 0) {  // out-of-range pieces were loaded as zeros and stay zeros: 0 > 0 is false
 #pragma unroll
       for (int i = 0; i < PA; ++i) {
@@ -591,11 +592,13 @@ __global__ __launch_bounds__(WGM* WGN * 64, FM* FN >= 6 ? 2 : 4) void conv_wgrad
         const float4 g = GATE == 1 ? make_float4(dy_scalar, dy_scalar, dy_scalar, dy_scalar) : ra[i];
         ra[i] = make_float4(y.x > 0.f ? g.x : 0.f, y.y > 0.f ? g.y : 0.f, y.z > 0.f ? g.z : 0.f, y.w > 0.f ? g.w : 0.f);
       }
-      if (sum_rows) {
-#pragma unroll
-        for (int i = 0; i < PA; ++i) row_sum[i] += (ra[i].x + ra[i].y) + (ra[i].z + ra[i].w);
-      }
     }
+    if (sum_rows) {
+#pragma unroll
+      for (int i = 0; i < PA; ++i) row_sum[i] += (ra[i].x + ra[i].y) + (ra[i].z + ra[i].w);
+    }
+  };
+  auto store = [&]() {
 #pragma unroll
     for (int i = 0; i < PA; ++i) *reinterpret_cast<float4*>(&As[lds_off + i * ROWS_PER_PASS * LDK]) = ra[i];
 #pragma unroll
@@ -605,6 +608,7 @@ __global__ __launch_bounds__(WGM* WGN * 64, FM* FN >= 6 ? 2 : 4) void conv_wgrad
   floatx16 acc[FM][FN];
   zero_acc<FM, FN>(acc);
   load(j_begin);
+  gate();
   store();
   __syncthreads();
   for (int jt = j_begin; jt < j_end; jt += BK) {
@@ -612,6 +616,7 @@ __global__ __launch_bounds__(WGM* WGN * 64, FM* FN >= 6 ? 2 : 4) void conv_wgrad
     if (more) load(jt + BK);
     compute_ktile<true, true, FM, FN, BM, BN>(As, Bs, wm * FM * 32 + l32, wn * FN * 32 + l32, h, acc);
     if (more) {
+      gate();
       __syncthreads();
       store();
       __syncthreads();
@@ -658,9 +663,8 @@ __global__ __launch_bounds__(WGM* WGN * 64, FM* FN >= 6 ? 2 : 4) void conv_wgrad
 // The weights do not pass through LDS at all (see the tile function). 72 or 144 MFMAs per wave between two barriers
 // (the dense kernel has 64 at its large tile), three or four work-groups per CU.
 struct DirectArgs {
-  const float* src;   // [N, Cred, SH, SW]
-  const float* gate;  // GATE 2: same shape as src, which counts where gate > 0 (GATE 1: src IS the gate and every
-  const float* gscalar;  // element that passes it is worth *gscalar)
+  const float* src;      // [N, Cred, SH, SW]
+  const float* gscalar;  // GATE 1: src is the stored output y; the cotangent is *gscalar where y > 0, zero elsewhere
   const float* wp;    // [chunks][9 groups][tiles_m * BM][8], packed as described above
   const float* bias;
   float* out;         // [N, Mrows, OH, OW]
@@ -723,33 +727,29 @@ __device__ __forceinline__ void direct3x3_tile(const DirectArgs& a, int tm, int 
   const __amdgpu_buffer_rsrc_t rs_src = make_rsrc(a.src, a.src_bytes);
   const __amdgpu_buffer_rsrc_t rs_w = make_rsrc(a.wp, a.wp_bytes);
   const uint32_t src_step = (uint32_t)(CC * a.SH * a.SW) * 4u, w_step = (uint32_t)(a.tiles_m * BM * KC) * 4u;
-  const __amdgpu_buffer_rsrc_t rs_gate = make_rsrc(GATE == 2 ? a.gate : a.src, a.src_bytes);
   const float gs = GATE == 1 ? a.gscalar[0] : 0.f;
-  float4 rb[PB], rg[GATE == 2 ? PB : 1];
+  float4 rb[PB];
   auto load = [&](int chunk) {
 #pragma unroll
     for (int p = 0; p < PB; ++p) {
       v4i v = __builtin_amdgcn_raw_buffer_load_b128(rs_src, (int)goff[p], (int)(chunk * src_step), 0);
       rb[p] = *reinterpret_cast<float4*>(&v);
     }
-    if (GATE == 2) {
+  };
+  // GATE 1: what was staged is y; the cotangent is *gscalar where y > 0. Applied in registers ahead of the barrier that
+  // precedes the stores (the work-group's other waves may still be in their MFMAs then; between the two barriers
+  // nothing else runs). Rows outside the image were loaded as zeros and stay zeros.
+  auto gate = [&]() {
+    if (GATE == 1) {
 #pragma unroll
-      for (int p = 0; p < PB; ++p) {
-        v4i v = __builtin_amdgcn_raw_buffer_load_b128(rs_gate, (int)goff[p], (int)(chunk * src_step), 0);
-        rg[p] = *reinterpret_cast<float4*>(&v);
-      }
+      for (int p = 0; p < PB; ++p)
+        rb[p] = make_float4(rb[p].x > 0.f ? gs : 0.f, rb[p].y > 0.f ? gs : 0.f, rb[p].z > 0.f ? gs : 0.f, rb[p].w > 0.f ? gs : 0.f);
     }
   };
   auto store = [&]() {
 #pragma unroll
-    for (int p = 0; p < PB; ++p) {
-      if (GATE > 0) {  // rows outside the image were loaded as zeros and stay zeros
-        const float4 y = GATE == 1 ? rb[p] : rg[p];
-        const float4 g = GATE == 1 ? make_float4(gs, gs, gs, gs) : rb[p];
-        rb[p] = make_float4(y.x > 0.f ? g.x : 0.f, y.y > 0.f ? g.y : 0.f, y.z > 0.f ? g.z : 0.f, y.w > 0.f ? g.w : 0.f);
-      }
+    for (int p = 0; p < PB; ++p)
       if (loff[p] >= 0) *reinterpret_cast<float4*>(&Bc[loff[p]]) = rb[p];
-    }
   };
 
   // this lane's pixels: cache position of tap (0, 0), with the half-wave's channel folded in
@@ -788,6 +788,7 @@ __device__ __forceinline__ void direct3x3_tile(const DirectArgs& a, int tm, int 
   load(0);
 #pragma unroll
   for (int jg = 0; jg < AD; ++jg) fetch_a(0, jg);
+  gate();
   __syncthreads();  // border columns zeroed before the first rows land in the cache
   store();
   __syncthreads();
@@ -817,6 +818,7 @@ __device__ __forceinline__ void direct3x3_tile(const DirectArgs& a, int tm, int 
       }
     }
     if (more) {
+      gate();
       __syncthreads();
       store();
       __syncthreads();
@@ -1158,12 +1160,12 @@ int32_t run_igemm_vec(int mode, const ConvP& p, const float* src, const float* w
 
 // 3 x 3 kernels with unit stride and dilation and at most one zero row / column around the source
 // (conv_direct3x3_kernel). Returns 1 when the shape does not qualify.
-// gate_mode 1 / 2 (data gradient only): src counts where gate > 0; 1: src is the gate itself and *gscalar the value of
-// every element that passes, 2: gate is a second tensor of src's shape.
+// gate_mode 1 (data gradient only): src is the stored output y of relu(conv + bias) and stands for a cotangent that
+// is *gscalar where y > 0 and zero elsewhere. (A tensor cotangent gated in the staging loads was measured slower than
+// writing the gated cotangent out first: twice the loads and 151 registers, three work-groups per CU instead of four.)
 int32_t run_direct3x3(int mode, const ConvP& p, const float* src, const float* w, const float* bias, float* out, int relu,
-                      int gate_mode = 0, const float* gate = nullptr, const float* gscalar = nullptr) {
+                      int gate_mode = 0, const float* gscalar = nullptr) {
   const bool fwd = mode == MODE_FWD;
-  if (gate_mode == 2 && (reinterpret_cast<uintptr_t>(gate) & 15)) return 1;
   if (p.T != 1 || p.D != 1 || p.R != 3 || p.S != 3 || p.dh != 1 || p.dw != 1 || p.sh != 1 || p.sw != 1 || p.sd != 1) return 1;
   const int OH = fwd ? p.P : p.H, OW = fwd ? p.Q : p.W, SH = fwd ? p.H : p.P, SW = fwd ? p.W : p.Q;
   const int Cred = fwd ? p.C : p.K, Mrows = fwd ? p.K : p.C;
@@ -1193,7 +1195,7 @@ int32_t run_direct3x3(int mode, const ConvP& p, const float* src, const float* w
                      static_cast<float*>(wp.p), p.K, p.C, rows_pad, a.chunks, fwd ? 0 : 1);
   ENDIA_LAUNCH_CHECK();
   a.src = src; a.wp = static_cast<const float*>(wp.p); a.bias = bias; a.out = out; a.relu = relu;
-  a.gate = gate; a.gscalar = gscalar;
+  a.gscalar = gscalar;
   a.Mrows = Mrows; a.Cred = Cred; a.OH = OH; a.OW = OW; a.SH = SH; a.SW = SW; a.Ncols = p.N * OH * OW; a.NOH = p.N * OH;
   a.py = py; a.px = px; a.MR = MR; a.plane = plane; a.tasks = tasks;
   a.d_ohw = make_fastdiv(OH * OW); a.d_ow = make_fastdiv(OW); a.d_oh = make_fastdiv(OH); a.d_f4row = make_fastdiv(SW / 4);
@@ -1216,8 +1218,7 @@ int32_t run_direct3x3(int mode, const ConvP& p, const float* src, const float* w
   do {                                                                                                                       \
     if (fwd) hipLaunchKernelGGL((conv_direct3x3_kernel<FM, PITCH, true, 0>), grid, dim3(256), lds, s, a);                      \
     else if (gate_mode == 0) hipLaunchKernelGGL((conv_direct3x3_kernel<FM, PITCH, false, 0>), grid, dim3(256), lds, s, a);     \
-    else if (gate_mode == 1) hipLaunchKernelGGL((conv_direct3x3_kernel<FM, PITCH, false, 1>), grid, dim3(256), lds, s, a);     \
-    else hipLaunchKernelGGL((conv_direct3x3_kernel<FM, PITCH, false, 2>), grid, dim3(256), lds, s, a);                         \
+    else hipLaunchKernelGGL((conv_direct3x3_kernel<FM, PITCH, false, 1>), grid, dim3(256), lds, s, a);                         \
   } while (0)
   if (fm == 2 && pitch == 64) ENDIA_LAUNCH_DIRECT(2, 64);
   else if (fm == 2) ENDIA_LAUNCH_DIRECT(2, 128);
@@ -1304,7 +1305,7 @@ bool wgrad_vec_ok(const ConvP& p, const float* rows) {
 }
 
 // gate_mode 0: the plain weight gradient. 1 / 2 (only where wgrad_vec_ok): dy (1: one float, 2: a tensor) counts
-// where gate > 0, and db (may be null) receives the sums of the gated dy over n, o, p, q.
+// where gate > 0. db (may be null, only where wgrad_vec_ok) receives the sums of the (gated) dy over n, o, p, q.
 int32_t conv_bwd_weight(const char* who, const ConvP& p, const float* x, const float* dy, float* dw, int gate_mode = 0,
                         const float* gate = nullptr, float* db = nullptr) {
   const int Kd = p.C * p.T * p.R * p.S;
@@ -1328,7 +1329,7 @@ int32_t conv_bwd_weight(const char* who, const ConvP& p, const float* x, const f
   a.dy_bytes = (int64_t)p.N * p.K * p.O * p.P * p.Q * 4;
   const int Dp = p.D + 2 * p.pd, Hp = p.H + 2 * p.ph, Wp = padded_row(p.W, p.pw);
   const bool vec = wgrad_vec_ok(p, gate_mode == 1 ? gate : dy) && (gate_mode != 2 || (reinterpret_cast<uintptr_t>(gate) & 15) == 0);
-  if (gate_mode && !vec) return endia::fail(ENDIA_HIP_ERR_UNSUPPORTED, "%s: gated weight gradient outside the vectorised kernel", who);
+  if ((gate_mode || db) && !vec) return endia::fail(ENDIA_HIP_ERR_UNSUPPORTED, "%s: gated weight gradient outside the vectorised kernel", who);
   // 64-wide tiles over the taps when the last 128-wide tile would be at most half full
   int bn = (vec && Kd % 128 != 0 && Kd % 128 <= 64) ? 64 : 128;
   // likewise 64-high tiles over the output channels
@@ -1422,9 +1423,10 @@ __global__ __launch_bounds__(TPB) void relu_gate_kernel(const float* __restrict_
     g[i] = y[i] > 0.f ? (dy_is_scalar ? sv : dy[i]) : 0.f;
 }
 
-// Every gradient of y = relu(conv(x, w) + bias) from the stored y. Where the 3 x 3 row-cache kernel (dx) and the
-// vectorised weight-gradient kernel (dw, db) apply, dy * [y > 0] is formed as they load their operands and never
-// exists in memory; otherwise it is written once and the plain kernels run on it.
+// Every gradient of y = relu(conv(x, w) + bias) from the stored y. dy * [y > 0] is formed inside the kernels as they
+// load their operands where that is the faster way (see the policy below) and written out once, by one streaming
+// kernel, where it is not; either way the bias gradient comes out of the weight-gradient launch where that is the
+// vectorised kernel.
 int32_t conv_bwd_relu(const char* who, const ConvP& p, const float* x, const float* w, const float* y, const float* dy,
                       int dy_is_scalar, float* dx, float* dw, float* db) {
   const int64_t out_total = (int64_t)p.N * p.K * p.O * p.P * p.Q;
@@ -1438,7 +1440,6 @@ int32_t conv_bwd_relu(const char* who, const ConvP& p, const float* x, const flo
   }
   if (!(y && dy)) return endia::fail(ENDIA_HIP_ERR_INVALID, "%s: null pointer", who);
   if ((dw && !x) || (dx && !w)) return endia::fail(ENDIA_HIP_ERR_INVALID, "%s: null pointer", who);
-  const int gate_mode = dy_is_scalar ? 1 : 2;
   PoolBuf gbuf;
   auto gated = [&](const float** g) -> int32_t {  // dy * [y > 0] in memory, made at most once
     if (!gbuf.p) {
@@ -1452,22 +1453,30 @@ int32_t conv_bwd_relu(const char* who, const ConvP& p, const float* x, const flo
     return ENDIA_HIP_OK;
   };
   const float* g = nullptr;
-  if (dw && wgrad_vec_ok(p, dy_is_scalar ? y : dy) && (dy_is_scalar || (reinterpret_cast<uintptr_t>(y) & 15) == 0)) {
-    if ((rc = conv_bwd_weight(who, p, x, dy, dw, gate_mode, y, db))) return rc;
-  } else {
-    if (dw || db) {
-      if ((rc = gated(&g))) return rc;
-    }
+  // A scalar cotangent is gated inside both kernels (they read y instead of a cotangent tensor). A tensor cotangent
+  // is gated inside the weight-gradient kernel when only dw / db are wanted; with dx as well, writing the gated
+  // cotangent out once (36 us at the 56 x 56 benchmark shape) and running the plain kernels on it is the faster way.
+  const bool want_dx = dx && x_total;
+  bool dx_done = false;
+  if (want_dx && dy_is_scalar) {
+    rc = run_direct3x3(MODE_BWD_DATA, p, y, w, nullptr, dx, 0, 1, dy);
+    if (rc != 0 && rc != 1) return rc;
+    dx_done = rc == 0;
+  }
+  if (want_dx && !dx_done) {
+    if ((rc = gated(&g))) return rc;
+    if ((rc = conv_bwd_data(who, p, g, w, dx))) return rc;
+  }
+  if (dw && g) {  // the gated cotangent exists: the plain kernel on it, which also sums db where it is the vectorised one
+    const bool vec = wgrad_vec_ok(p, g);
+    if ((rc = conv_bwd_weight(who, p, x, g, dw, 0, nullptr, vec ? db : nullptr))) return rc;
+    if (db && !vec && (rc = conv_bwd_bias(who, p, g, db))) return rc;
+  } else if (dw && wgrad_vec_ok(p, dy_is_scalar ? y : dy) && (dy_is_scalar || (reinterpret_cast<uintptr_t>(y) & 15) == 0)) {
+    if ((rc = conv_bwd_weight(who, p, x, dy, dw, dy_is_scalar ? 1 : 2, y, db))) return rc;
+  } else if (dw || db) {
+    if ((rc = gated(&g))) return rc;
     if (dw && (rc = conv_bwd_weight(who, p, x, g, dw))) return rc;
     if (db && (rc = conv_bwd_bias(who, p, g, db))) return rc;
-  }
-  if (dx && x_total) {
-    rc = run_direct3x3(MODE_BWD_DATA, p, dy_is_scalar ? y : dy, w, nullptr, dx, 0, gate_mode, y, dy);
-    if (rc == 1) {
-      if ((rc = gated(&g))) return rc;
-      rc = conv_bwd_data(who, p, g, w, dx);
-    }
-    if (rc) return rc;
   }
   return ENDIA_HIP_OK;
 }

@@ -357,8 +357,9 @@ ENDIA_API int32_t endia_hip_conv2d_bwd_weight(const endia_hip_conv2d_desc* d, co
                                     float* dw);
 ENDIA_API int32_t endia_hip_conv2d_bwd_bias(const endia_hip_conv2d_desc* d, const float* dy, float* db);
 /* Every gradient of y = relu(conv(x,w)+bias) in one call, from the stored y (what endia_hip_conv2d_fwd wrote with
- * act = RELU): the ReLU's derivative [y > 0] (relu_op.mojo:51-53) is applied to dy as the kernels load it, so
- * dy * [y > 0] is not written to memory where the fast kernels apply (it is written once where they do not).
+ * act = RELU): the ReLU's derivative [y > 0] (relu_op.mojo:51-53) is applied to dy inside the gradient kernels, as
+ * they load it, where that is faster than a pass of its own (always for a scalar dy, and for the weight and bias
+ * gradients of a tensor dy), and db comes out of the weight-gradient launch.
  * dy_is_scalar != 0: dy points at ONE device float that stands for every element of the cotangent (the gradient
  * of a mean or a sum). dx, dw, db may each be null; x is read only for dw, w only for dx. */
 ENDIA_API int32_t endia_hip_conv2d_bwd_relu(const endia_hip_conv2d_desc* d, const float* x, const float* w,
