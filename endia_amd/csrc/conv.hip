@@ -1417,10 +1417,16 @@ int32_t conv_bwd_bias(const char* who, const ConvP& p, const float* dy, float* d
 }
 
 __global__ __launch_bounds__(TPB) void relu_gate_kernel(const float* __restrict__ y, const float* __restrict__ dy, int dy_is_scalar,
-                                                        float* __restrict__ g, int64_t n) {
+                                                        float* __restrict__ g, int64_t n, int vec) {
   const float sv = dy_is_scalar ? dy[0] : 0.f;
-  for (int64_t i = (int64_t)blockIdx.x * TPB + threadIdx.x; i < n; i += (int64_t)gridDim.x * TPB)
-    g[i] = y[i] > 0.f ? (dy_is_scalar ? sv : dy[i]) : 0.f;
+  const int64_t i0 = (int64_t)blockIdx.x * TPB + threadIdx.x, stride = (int64_t)gridDim.x * TPB;
+  const int64_t n4 = vec ? n >> 2 : 0;
+  for (int64_t i = i0; i < n4; i += stride) {  // 16 bytes per lane and stream
+    const float4 a = reinterpret_cast<const float4*>(y)[i];
+    const float4 d = dy_is_scalar ? make_float4(sv, sv, sv, sv) : reinterpret_cast<const float4*>(dy)[i];
+    reinterpret_cast<float4*>(g)[i] = make_float4(a.x > 0.f ? d.x : 0.f, a.y > 0.f ? d.y : 0.f, a.z > 0.f ? d.z : 0.f, a.w > 0.f ? d.w : 0.f);
+  }
+  for (int64_t i = (n4 << 2) + i0; i < n; i += stride) g[i] = y[i] > 0.f ? (dy_is_scalar ? sv : dy[i]) : 0.f;
 }
 
 // Every gradient of y = relu(conv(x, w) + bias) from the stored y. dy * [y > 0] is formed inside the kernels as they
@@ -1445,8 +1451,9 @@ int32_t conv_bwd_relu(const char* who, const ConvP& p, const float* x, const flo
     if (!gbuf.p) {
       int32_t r = endia_hip_malloc(out_total * 4, &gbuf.p);
       if (r) return r;
-      hipLaunchKernelGGL(relu_gate_kernel, dim3(grid_for(out_total)), dim3(TPB), 0, endia::ctx().stream, y, dy, dy_is_scalar,
-                         static_cast<float*>(gbuf.p), out_total);
+      const int vec = ((reinterpret_cast<uintptr_t>(y) | (dy_is_scalar ? 0 : reinterpret_cast<uintptr_t>(dy))) & 15) == 0;
+      hipLaunchKernelGGL(relu_gate_kernel, dim3(grid_for((out_total + 3) / 4)), dim3(TPB), 0, endia::ctx().stream, y, dy, dy_is_scalar,
+                         static_cast<float*>(gbuf.p), out_total, vec);
       ENDIA_LAUNCH_CHECK();
     }
     *g = static_cast<const float*>(gbuf.p);
