@@ -320,6 +320,49 @@ def kernel_table(reps=10):
     return rows
 
 
+def gemm_mid_table(reps=100, warm=600):
+    """Products with fewer than 256 tiles of 256 x 256 (the shapes of the Hessian-vector and complex configurations), each
+    form, timed per launch with a HIP-event pair around every launch (endia_hip_gemm_timing_*) after `warm` launches of
+    the same product: the core clock needs a few hundred short launches to reach its sustained value, and a probe that
+    starts from an idle chip under-reports short kernels by a fifth."""
+    from endia_amd import _lib as L
+    L.ensure_init(0)
+    rng = np.random.default_rng(0)
+
+    def put(a):
+        p = ctypes.c_void_p()
+        L.call("endia_hip_malloc", a.nbytes, ctypes.byref(p))
+        L.call("endia_hip_memcpy_h2d", p.value, a.ctypes.data, a.nbytes)
+        return p.value
+
+    rows = []
+    for (M, N, K) in ((2048, 4096, 4096), (1024, 2048, 2048), (2048, 2048, 1024), (2048, 2048, 2048)):
+        for form, (ta, tb) in (("NN", (0, 0)), ("NT", (0, 1)), ("TN", (1, 0))):
+            A = put(rng.standard_normal((K, M) if ta else (M, K)).astype(np.float32))
+            B = put(rng.standard_normal((N, K) if tb else (K, N)).astype(np.float32))
+            C = put(np.zeros((M, N), np.float32))
+            lda, ldb = (M if ta else K), (K if tb else N)
+
+            def go():
+                L.call("endia_hip_sgemm", ta, tb, M, N, K, A, lda, B, ldb, C, N, 1, 0, 0, 0, L.EPI_NONE, L.OP_IDENTITY, None, None, None)
+
+            for _ in range(warm):
+                go()
+            L.call("endia_hip_gemm_timing_begin")
+            for _ in range(reps):
+                go()
+            L.call("endia_hip_sync")
+            launches, g_ms, g_flops = ctypes.c_int64(), ctypes.c_double(), ctypes.c_double()
+            L.call("endia_hip_gemm_timing_end", ctypes.byref(launches), ctypes.byref(g_ms), ctypes.byref(g_flops))
+            us = 1e3 * g_ms.value / launches.value
+            tf = 2.0 * M * N * K / (us * 1e-6) / 1e12
+            rows.append({"kernel": "sgemm %s %d x %d x %d" % (form, M, N, K), "us": us, "bound": "mfma", "achieved": tf,
+                         "peak": FP32_MFMA_PEAK_TFLOPS, "unit": "TFLOP/s", "frac": tf / FP32_MFMA_PEAK_TFLOPS})
+            for p in (A, B, C):
+                L.call("endia_hip_free", p)
+    return rows
+
+
 def conv_table(reps=10):
     """conv2d at the benchmark configuration: x [64,64,56,56], w [128,64,3,3], stride 1, pad 1 (fp32, NCHW).
     Algorithmic flops per pass: 2*N*K*C*R*S*P*Q = 29.6 GFLOP for each of forward, data and weight gradient."""
@@ -571,7 +614,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=3)
-    ap.add_argument("--workload", default="wide_mlp", choices=["wide_mlp", "sine_mlp", "kernels", "conv2d", "hvp", "complex_mlp", "complex_mlp_3m"])
+    ap.add_argument("--workload", default="wide_mlp", choices=["wide_mlp", "sine_mlp", "kernels", "gemm_mid", "conv2d", "hvp", "complex_mlp", "complex_mlp_3m"])
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--eager", action="store_true", help="sine_mlp: issue every kernel from the host instead of replaying a graph")
     ap.add_argument("--optimizer", default="sgd", choices=["sgd", "adam"], help="sine_mlp: SGD (the benchmark configuration) or Adam (the reference script's)")
@@ -606,6 +649,10 @@ def main():
         if not args.no_cpu_baseline:
             out["cpu_baseline"] = cpu_baseline_conv()
         print(json.dumps(out))
+        return
+    if args.workload == "gemm_mid":
+        print(json.dumps({"metric": "fp32 GEMM launches of the mid-size products, sustained clock", "device": dev_name,
+                          "reps": max(args.steps, 1), "kernels": gemm_mid_table(max(args.steps, 1))}))
         return
     if args.workload == "kernels":
         rows = kernel_table(max(args.steps, 1))
