@@ -23,6 +23,9 @@ __device__ __forceinline__ float load_shared(const float* p) {
 // the `expected`-th to arrive at `ticket`; that group also puts the ticket back to zero for the next launch.
 // `flag` is one int of LDS that nobody else uses until the call returns.
 __device__ __forceinline__ bool arrive_last(unsigned* ticket, unsigned expected, int* flag) {
+  // (compiler-only fences: the relaxed accesses around this call keep their program order in the generated code; the
+  // hardware side is the wait below)
+  __atomic_signal_fence(__ATOMIC_SEQ_CST);
   __builtin_amdgcn_s_waitcnt(0);
   __syncthreads();
   if (threadIdx.x == 0) {
@@ -32,6 +35,7 @@ __device__ __forceinline__ bool arrive_last(unsigned* ticket, unsigned expected,
     *flag = last;
   }
   __syncthreads();
+  __atomic_signal_fence(__ATOMIC_SEQ_CST);
   return *flag != 0;
 }
 
