@@ -650,6 +650,230 @@ __global__ __launch_bounds__(WGM* WGN * 64, FM* FN >= 6 ? 2 : 4) void conv_wgrad
   }
 }
 
+// ---- 3 x 3 weight gradient, unit stride and dilation, padding 0 or 1: rows of x and dy cached in LDS ---------
+// dW[k][c][r][s] = sum over n, p, q of dy[n][k][p][q] * x[n][c][p + r - ph][q + s - pw]: nine products with one left
+// operand. The output channels k sit on the MFMA's rows, the input channels c on its columns and the PIXELS of an
+// output row on its reduction axis (two per step, the half-wave picks one), so that one accumulator block per tap
+// (r, s) reads its B fragment at (cached row p + r, column q + s) of the lane's channel: the shift is a constant of the
+// LDS instruction, x is cached ONCE (no padded copy in memory, no gather that writes an element nine times) and
+// nothing is tested in the loop (rows outside the image and the column on either side are zeros in the cache).
+// A work-group (4 waves, 128 output channels x 32 input channels x 9 taps, 144 accumulator registers a lane) walks
+// the output rows [p_begin, p_end) of ONE image: per row it brings in the row of dy (128 x Q) and ONE new row of x
+// (the ring keeps the last three and the one arriving), both requested a row ahead into registers. Rows are 66 words
+// apart in LDS (2 mod 64), so that the 32 lanes of a fragment (one channel each) and the two half-waves (neighbouring
+// pixels) read 64 distinct banks. 252 MFMAs per wave between two barrier pairs; two work-groups per CU.
+// Every work-group writes its partial gradient [tap][k][c] (the lanes of a store are 32 neighbouring c); the
+// partials are added in split order by the column-reduction kernels and a last small kernel turns [tap][k][c] into
+// the [k][c][tap] of the weights.
+constexpr int W3_LD = 66;                 // floats between cached rows
+constexpr int W3_BK = 128, W3_BC = 32;    // output / input channels per work-group
+constexpr int W3_SLOT = W3_BC * W3_LD;    // one ring slot: one row of every input channel
+constexpr int W3_PD = 8, W3_PX = 2;       // 16-byte pieces per thread: of a dy row (128 x 64 / 4 / 256), of an x row (32 x 64 / 4 / 256)
+
+struct Wgrad3Args {
+  const float* x;     // [N, C, H, W]
+  const float* dy;    // [N, K, P, Q] (GATE 1: one float)
+  const float* gate;  // GATE > 0: the stored output y, same shape as dy
+  float* part;        // [splits][9][K][C]
+  float* bias_part;   // [splits][K] or null
+  int C, H, W, K, P, Q, ph, pw;
+  int rows_per_wg, wgs_per_image, tiles_c;
+  int64_t x_bytes, dy_bytes;
+};
+
+template <int GATE>
+__global__ __launch_bounds__(256, 2) void conv_wgrad3x3_kernel(Wgrad3Args a) {
+  __shared__ __attribute__((aligned(16))) float Xs[4 * W3_SLOT];
+  __shared__ __attribute__((aligned(16))) float Ds[W3_BK * W3_LD];
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, l32 = lane & 31, h = lane >> 5;
+  const int tk = blockIdx.x / a.tiles_c, tc = blockIdx.x - tk * a.tiles_c;
+  const int k0 = tk * W3_BK, c0 = tc * W3_BC;
+  const int split = blockIdx.y, n = split / a.wgs_per_image;
+  const int p_begin = (split - n * a.wgs_per_image) * a.rows_per_wg;
+  const int p_end = p_begin + a.rows_per_wg < a.P ? p_begin + a.rows_per_wg : a.P;
+
+  for (int i = tid; i < 4 * W3_SLOT; i += 256) Xs[i] = 0.f;
+  for (int i = tid; i < W3_BK * W3_LD; i += 256) Ds[i] = 0.f;
+
+  // the pieces this thread stages: byte offset of the piece in row 0 (of the image / of the output) and where it goes in LDS
+  const int Q4 = a.Q >> 2, W4 = a.W >> 2;
+  uint32_t dvoff[W3_PD], xvoff[W3_PX];
+  int dl[W3_PD], xl[W3_PX];
+#pragma unroll
+  for (int j = 0; j < W3_PD; ++j) {
+    const int u = tid + 256 * j, k = u / Q4, c4 = u - k * Q4;
+    const bool in = u < W3_BK * Q4;
+    dl[j] = in ? k * W3_LD + 4 * c4 : -1;
+    dvoff[j] = in && k0 + k < a.K ? (uint32_t)(((n * a.K + k0 + k) * a.P * a.Q + 4 * c4) * 4) : OOB_OFFSET;
+  }
+#pragma unroll
+  for (int j = 0; j < W3_PX; ++j) {
+    const int u = tid + 256 * j, c = u / W4, c4 = u - c * W4;
+    const bool in = u < W3_BC * W4;
+    xl[j] = in ? c * W3_LD + 2 + 4 * c4 : -1;  // column xc of a row sits at word xc + 2: words 1 and W + 2 stay zero
+    xvoff[j] = in && c0 + c < a.C ? (uint32_t)(((n * a.C + c0 + c) * a.H * a.W + 4 * c4) * 4) : OOB_OFFSET;
+  }
+  const __amdgpu_buffer_rsrc_t rs_dy = make_rsrc(GATE == 1 ? a.gate : a.dy, a.dy_bytes);
+  const __amdgpu_buffer_rsrc_t rs_gate = make_rsrc(a.gate, a.dy_bytes);
+  const __amdgpu_buffer_rsrc_t rs_x = make_rsrc(a.x, a.x_bytes);
+  const float dy_scalar = GATE == 1 ? a.dy[0] : 0.f;
+  const bool sum_rows = a.bias_part != nullptr && tc == 0;
+
+  float4 rd[W3_PD], rg[GATE == 2 ? W3_PD : 1], rx[W3_PX];
+  float row_sum[W3_PD];
+#pragma unroll
+  for (int j = 0; j < W3_PD; ++j) row_sum[j] = 0.f;
+  auto load_dy = [&](int p) {
+    const int soff = p * a.Q * 4;
+#pragma unroll
+    for (int j = 0; j < W3_PD; ++j) {
+      v4i v = __builtin_amdgcn_raw_buffer_load_b128(rs_dy, (int)dvoff[j], soff, 0);
+      rd[j] = *reinterpret_cast<float4*>(&v);
+    }
+    if (GATE == 2) {
+#pragma unroll
+      for (int j = 0; j < W3_PD; ++j) {
+        v4i v = __builtin_amdgcn_raw_buffer_load_b128(rs_gate, (int)dvoff[j], soff, 0);
+        rg[j] = *reinterpret_cast<float4*>(&v);
+      }
+    }
+  };
+  auto load_x = [&](int xr) {  // image row xr, zeros where the image has no such row
+    const bool row_in = (unsigned)xr < (unsigned)a.H;
+    const int soff = row_in ? xr * a.W * 4 : 0;
+#pragma unroll
+    for (int j = 0; j < W3_PX; ++j) {
+      v4i v = __builtin_amdgcn_raw_buffer_load_b128(rs_x, row_in ? (int)xvoff[j] : (int)OOB_OFFSET, soff, 0);
+      rx[j] = *reinterpret_cast<float4*>(&v);
+    }
+  };
+  auto gate_dy = [&]() {  // in registers, ahead of the barrier that precedes the stores
+    if (GATE > 0) {
+#pragma unroll
+      for (int j = 0; j < W3_PD; ++j) {
+        const float4 y = GATE == 1 ? rd[j] : rg[j];
+        const float4 g = GATE == 1 ? make_float4(dy_scalar, dy_scalar, dy_scalar, dy_scalar) : rd[j];
+        rd[j] = make_float4(y.x > 0.f ? g.x : 0.f, y.y > 0.f ? g.y : 0.f, y.z > 0.f ? g.z : 0.f, y.w > 0.f ? g.w : 0.f);
+      }
+    }
+    if (sum_rows) {
+#pragma unroll
+      for (int j = 0; j < W3_PD; ++j) row_sum[j] += (rd[j].x + rd[j].y) + (rd[j].z + rd[j].w);
+    }
+  };
+  // rows are 8-byte, not 16-byte, aligned in LDS (66 words): a piece goes as two 8-byte stores
+  auto store_dy = [&]() {
+#pragma unroll
+    for (int j = 0; j < W3_PD; ++j)
+      if (dl[j] >= 0) {
+        *reinterpret_cast<float2*>(&Ds[dl[j]]) = make_float2(rd[j].x, rd[j].y);
+        *reinterpret_cast<float2*>(&Ds[dl[j] + 2]) = make_float2(rd[j].z, rd[j].w);
+      }
+  };
+  auto store_x = [&](int xr) {
+    float* slot = Xs + ((xr + 4) & 3) * W3_SLOT;
+#pragma unroll
+    for (int j = 0; j < W3_PX; ++j)
+      if (xl[j] >= 0) {
+        *reinterpret_cast<float2*>(&slot[xl[j]]) = make_float2(rx[j].x, rx[j].y);
+        *reinterpret_cast<float2*>(&slot[xl[j] + 2]) = make_float2(rx[j].z, rx[j].w);
+      }
+  };
+
+  floatx16 acc[9];
+#pragma unroll
+  for (int t = 0; t < 9; ++t)
+#pragma unroll
+    for (int v = 0; v < 16; ++v) acc[t][v] = 0.f;
+
+  if (p_begin < p_end) {
+    __syncthreads();  // the zeros are in place
+    // the three rows of x under the first output row, and its row of dy
+    for (int r = 0; r < 3; ++r) {
+      load_x(p_begin - a.ph + r);
+      store_x(p_begin - a.ph + r);
+    }
+    load_dy(p_begin);
+    gate_dy();
+    store_dy();
+    __syncthreads();
+    const int steps8 = (a.Q + 7) >> 3;  // groups of four MFMA steps = eight pixels (the cache is zero beyond Q)
+    const float* a_at = Ds + (wave * 32 + l32) * W3_LD + h;
+    const int b_lane = l32 * W3_LD + h + 2 - a.pw;
+    for (int p = p_begin; p < p_end; ++p) {
+      const bool more = p + 1 < p_end;
+      if (more) {
+        load_dy(p + 1);
+        load_x(p + 3 - a.ph);
+      }
+      const float* b_at[3];
+#pragma unroll
+      for (int r = 0; r < 3; ++r) b_at[r] = Xs + ((p - a.ph + r + 4) & 3) * W3_SLOT + b_lane;
+      // the four dy values of a group of steps are read one group ahead (the cache row is 66 words: the read past
+      // the last group stays inside it)
+      float a_cur[4], a_nxt[4];
+#pragma unroll
+      for (int i = 0; i < 4; ++i) a_cur[i] = a_at[2 * i];
+      for (int g8 = 0; g8 < steps8; ++g8) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) a_nxt[i] = a_at[8 * g8 + 8 + 2 * i];
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          const int q = 8 * g8 + 2 * i;
+#pragma unroll
+          for (int r = 0; r < 3; ++r)
+#pragma unroll
+            for (int sx = 0; sx < 3; ++sx)
+              acc[3 * r + sx] = __builtin_amdgcn_mfma_f32_32x32x2f32(a_cur[i], b_at[r][q + sx], acc[3 * r + sx], 0, 0, 0);
+        }
+#pragma unroll
+        for (int i = 0; i < 4; ++i) a_cur[i] = a_nxt[i];
+      }
+      if (more) {
+        gate_dy();
+        __syncthreads();
+        store_dy();
+        store_x(p + 3 - a.ph);
+        __syncthreads();
+      }
+    }
+  }
+
+  // partial gradient of this work-group, [tap][k][c]
+  float* out = a.part + (int64_t)split * 9 * a.K * a.C;
+  const int c = c0 + l32;
+  if (c < a.C) {
+#pragma unroll
+    for (int t = 0; t < 9; ++t)
+#pragma unroll
+      for (int v = 0; v < 16; ++v) {
+        const int k = k0 + wave * 32 + acc_row(v, h);
+        if (k < a.K) out[((int64_t)t * a.K + k) * a.C + c] = acc[t][v];
+      }
+  }
+  if (sum_rows) {  // the pieces of a row of dy belong to Q / 4 neighbouring threads: added per row in piece order
+    __syncthreads();
+#pragma unroll
+    for (int j = 0; j < W3_PD; ++j) Xs[tid + 256 * j] = row_sum[j];
+    __syncthreads();
+    if (tid < W3_BK && k0 + tid < a.K) {
+      float sum = 0.f;
+      for (int i = 0; i < Q4; ++i) sum += Xs[tid * Q4 + i];
+      a.bias_part[(int64_t)split * a.K + k0 + tid] = sum;
+    }
+  }
+}
+
+// [9][K][C] -> [K][C][9]
+__global__ __launch_bounds__(TPB) void wgrad3x3_order_kernel(const float* __restrict__ src, float* __restrict__ dw, int K, int C) {
+  const int64_t total = (int64_t)9 * K * C;
+  for (int64_t i = (int64_t)blockIdx.x * TPB + threadIdx.x; i < total; i += (int64_t)gridDim.x * TPB) {
+    const int t = (int)(i / ((int64_t)K * C));
+    const int64_t kc = i - (int64_t)t * K * C;
+    dw[kc * 9 + t] = src[i];
+  }
+}
+
 // ---- 3 x 3, unit stride and dilation, padding 0 or 1: rows of the source cached in LDS --------------------
 // The gathers above write every source element into LDS once per tap it serves (nine times for a 3 x 3 kernel).
 // Here a work-group keeps, for eight input channels at a time, the three source rows under each output row of its
@@ -1304,6 +1528,60 @@ bool wgrad_vec_ok(const ConvP& p, const float* rows) {
          (reinterpret_cast<uintptr_t>(rows) & 15) == 0;
 }
 
+// The row-cache weight gradient (conv_wgrad3x3_kernel) where it applies: 1 if it does not. Same gate modes and bias
+// sums as conv_bwd_weight below.
+int32_t run_wgrad3x3(const ConvP& p, const float* x, const float* dy, float* dw, int gate_mode, const float* gate, float* db) {
+  if (getenv("ENDIA_NO_WGRAD3X3")) return 1;
+  if (p.T != 1 || p.D != 1 || p.R != 3 || p.S != 3 || p.dh != 1 || p.dw != 1 || p.sh != 1 || p.sw != 1 || p.sd != 1) return 1;
+  if (p.ph < 0 || p.ph > 1 || p.pw < 0 || p.pw > 1 || p.W % 4 || p.Q % 4 || p.Q < 8 || p.Q > 56) return 1;
+  const float* rows = gate_mode == 1 ? gate : dy;
+  if ((reinterpret_cast<uintptr_t>(x) | reinterpret_cast<uintptr_t>(rows) | (gate_mode == 2 ? reinterpret_cast<uintptr_t>(gate) : 0)) & 15) return 1;
+  const int64_t x_bytes = (int64_t)p.N * p.C * p.H * p.W * 4, dy_bytes = (int64_t)p.N * p.K * p.P * p.Q * 4;
+  if (x_bytes >= (1ll << 31) || dy_bytes >= (1ll << 31)) return 1;
+  Wgrad3Args a;
+  const int tiles_k = (p.K + W3_BK - 1) / W3_BK;
+  a.tiles_c = (p.C + W3_BC - 1) / W3_BC;
+  // few channels would leave most of the 128 x 32 tile's MFMA rows or columns multiplying zeros: the gather kernels have smaller tiles
+  if ((double)tiles_k * W3_BK * a.tiles_c * W3_BC > 1.5 * (double)p.K * p.C && !getenv("ENDIA_FORCE_WGRAD3X3")) return 1;
+  const int64_t tiles = (int64_t)tiles_k * a.tiles_c;
+  // about two work-groups per CU in all (what a CU holds), each on a run of output rows of one image
+  int64_t per_image = (2 * (int64_t)endia::ctx().cu_count + tiles * p.N - 1) / (tiles * p.N);
+  if (per_image < 1) per_image = 1;
+  if (per_image > p.P) per_image = p.P;
+  a.rows_per_wg = (int)((p.P + per_image - 1) / per_image);
+  a.wgs_per_image = (p.P + a.rows_per_wg - 1) / a.rows_per_wg;
+  const int64_t splits = (int64_t)p.N * a.wgs_per_image;
+  if (splits > 65535 || tiles > (1ll << 30)) return 1;
+  const int64_t taps = (int64_t)9 * p.K * p.C;
+  PoolBuf part, ordered, bias_part;
+  int32_t rc;
+  if ((rc = endia_hip_malloc(splits * taps * 4, &part.p))) return rc;
+  float* db_part = db;
+  if (db && splits > 1) {
+    if ((rc = endia_hip_malloc(splits * p.K * 4, &bias_part.p))) return rc;
+    db_part = static_cast<float*>(bias_part.p);
+  }
+  a.x = x; a.dy = dy; a.gate = gate; a.part = static_cast<float*>(part.p); a.bias_part = db_part;
+  a.C = p.C; a.H = p.H; a.W = p.W; a.K = p.K; a.P = p.P; a.Q = p.Q; a.ph = p.ph; a.pw = p.pw;
+  a.x_bytes = x_bytes; a.dy_bytes = dy_bytes;
+  hipStream_t s = endia::ctx().stream;
+  const dim3 grid((unsigned)tiles, (unsigned)splits);
+  if (gate_mode == 0) hipLaunchKernelGGL((conv_wgrad3x3_kernel<0>), grid, dim3(256), 0, s, a);
+  else if (gate_mode == 1) hipLaunchKernelGGL((conv_wgrad3x3_kernel<1>), grid, dim3(256), 0, s, a);
+  else hipLaunchKernelGGL((conv_wgrad3x3_kernel<2>), grid, dim3(256), 0, s, a);
+  ENDIA_LAUNCH_CHECK();
+  const float* summed = a.part;
+  if (splits > 1) {  // partials added in split order
+    if ((rc = endia_hip_malloc(taps * 4, &ordered.p))) return rc;
+    if ((rc = endia::col_reduce(1, splits, taps, a.part, static_cast<float*>(ordered.p), 1.f))) return rc;
+    summed = static_cast<const float*>(ordered.p);
+    if (db && (rc = endia::col_reduce(1, splits, p.K, db_part, db, 1.f))) return rc;
+  }
+  hipLaunchKernelGGL(wgrad3x3_order_kernel, dim3(grid_for(taps)), dim3(TPB), 0, s, summed, dw, p.K, p.C);
+  ENDIA_LAUNCH_CHECK();
+  return ENDIA_HIP_OK;
+}
+
 // gate_mode 0: the plain weight gradient. 1 / 2 (only where wgrad_vec_ok): dy (1: one float, 2: a tensor) counts
 // where gate > 0. db (may be null, only where wgrad_vec_ok) receives the sums of the (gated) dy over n, o, p, q.
 int32_t conv_bwd_weight(const char* who, const ConvP& p, const float* x, const float* dy, float* dw, int gate_mode = 0,
@@ -1314,6 +1592,10 @@ int32_t conv_bwd_weight(const char* who, const ConvP& p, const float* x, const f
   const int64_t total_j = (int64_t)p.N * p.O * p.P * p.Q;
   if (total_j == 0) return endia_hip_fill(dw, taps, 0.f);
   if (!(x && dy)) return endia::fail(ENDIA_HIP_ERR_INVALID, "%s: null pointer", who);
+  {
+    int32_t rc3 = run_wgrad3x3(p, x, dy, dw, gate_mode, gate, db);
+    if (rc3 != 1) return rc3;
+  }
   hipStream_t s = endia::ctx().stream;
 
   WgradArgs a;

@@ -892,13 +892,22 @@ def reduce_add(x, axes, _scale=1.0):
         lead = grad.ndim() - out_.ndim()
         if scale != 1.0:
             # the seed of a scalar loss times a constant is a constant: kept per value, so that a step spends no launch on it
-            grad = _scaled_seed(scale) if grad._is_seed else grad * scale
+            grad = _scaled_seed(scale) if _holds_seed(grad) else grad * scale
         return [expand(grad, list(grad._shape[:lead]) + in_shape)]
 
     return _register(out, [x], "reduce_add", vjp)
 
 
 _SCALED_SEEDS = {}
+
+
+def _holds_seed(grad):
+    """True for the seed of a scalar output and for its views (the squeeze / reshape on top of a reduction hands
+    the seed down as a view of the same buffer)."""
+    if grad._is_seed:
+        return True
+    from .autograd.functional import _SEED
+    return bool(_SEED) and grad.size() == 1 and grad._buf is _SEED[0]._buf and grad._offset == _SEED[0]._offset
 
 
 def _scaled_seed(value):

@@ -520,6 +520,10 @@ FAST_CASES = [
     ((2, 8, 10, 48), (16, 8, 3, 3), (1, 1), (1, 0), (1, 1)),   # padded rows, unpadded columns
     ((5, 24, 31, 32), (8, 24, 3, 3), (1, 1), (1, 1), (1, 1)),  # three chunks of channels; data gradient over one chunk
     ((12, 8, 56, 56), (8, 8, 3, 3), (1, 1), (1, 1), (1, 1)),   # 294 pixel tiles on 256 CUs: the last 38 run as 76 half tiles
+    # 3 x 3, unit stride, one padded column, enough channels to fill a 128 x 32 tile: the weight gradient on cached rows of x and dy
+    ((2, 32, 12, 16), (128, 32, 3, 3), (1, 1), (1, 1), (1, 1)),
+    ((3, 60, 9, 24), (250, 60, 3, 3), (1, 1), (0, 1), (1, 1)),  # no padded rows; two tiles either way with ragged ends
+    ((5, 32, 7, 56), (120, 32, 3, 3), (1, 1), (1, 1), (1, 1)),  # the widest rows it takes; more row groups than rows per image
 ]
 
 
