@@ -668,7 +668,7 @@ __global__ __launch_bounds__(WGM* WGN * 64, FM* FN >= 6 ? 2 : 4) void conv_wgrad
 constexpr int W3_LD = 66;                 // floats between cached rows
 constexpr int W3_BK = 128, W3_BC = 32;    // output / input channels per work-group
 constexpr int W3_SLOT = W3_BC * W3_LD;    // one ring slot: one row of every input channel
-constexpr int W3_PD = 8, W3_PX = 2;       // 16-byte pieces per thread: of a dy row (128 x 64 / 4 / 256), of an x row (32 x 64 / 4 / 256)
+constexpr int W3_PD = 7, W3_PX = 2;       // 16-byte pieces per thread: of a dy row (128 x 56 / 4 / 256), of an x row (32 x 64 / 4 / 256)
 
 struct Wgrad3Args {
   const float* x;     // [N, C, H, W]
