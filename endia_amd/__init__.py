@@ -14,7 +14,7 @@ from ._array import Array, Tensor, ndarray  # noqa: E402
 from .functional import (  # noqa: E402,F401
     abs, acos, add, arange, array, array_slice, as_strided, as_strided_inv, asin, atan, avg_pool1d, avg_pool2d, avg_pool3d, complex, concat, conj, contiguous, conv1d,
     conv2d, conv3d, cos, cosh, detach, div, equal, exp,
-    expand, eye, full, greater, greater_equal, imag, less, less_equal, linear, log, matmul, mlp_forward, max_pool1d, max_pool2d, max_pool3d, mean, mse, mul, neg,
+    expand, eye, full, greater, greater_equal, imag, less, less_equal, linear, log, matmul, mlp_forward, mlp_mse_loss, max_pool1d, max_pool2d, max_pool3d, mean, mse, mul, neg,
     not_equal, ones, pad, permute, pow, pow_to, prod, rand_he_normal, randn, randn_complex, randu, real, reciprocal, reduce_add,
     reduce_argmax, reduce_argmin, reduce_max, reduce_min, reduce_mul,
     relu, reshape, seed, set_complex_matmul_algorithm, set_complex_vjp_rule, sigmoid, sign, sin, sinh, sqrt, square, squeeze, std, sub, sum, tan,

@@ -96,6 +96,7 @@ SIGNATURES = {
                         c_int64, c_int64, c_int64, c_int64, c_int32, c_int32, _fp, _fp, _fp],
     "endia_hip_linear_bwd": [c_int64, c_int64, c_int64, _fp, _fp, _fp, c_int32, _fp, _fp, _fp, _fp],
     "endia_hip_mlp_fwd": [POINTER(MlpDesc), _fp, POINTER(c_void_p), POINTER(c_void_p), POINTER(c_void_p)],
+    "endia_hip_mlp_fwd_mse": [POINTER(MlpDesc), _fp, POINTER(c_void_p), POINTER(c_void_p), _fp, POINTER(c_void_p), _fp, _fp],
     "endia_hip_mlp_bwd": [POINTER(MlpDesc), _fp, POINTER(c_void_p), POINTER(c_void_p), POINTER(c_void_p), POINTER(c_void_p),
                           POINTER(c_void_p), _fp],
     "endia_hip_cgemm": [c_int32, c_int32, c_int32, c_int32, c_int64, c_int64, c_int64, _fp, c_int64, _fp, c_int64,

@@ -18,6 +18,7 @@
 // four A values are one 16-byte LDS read.
 #include "common.h"
 #include "mfma_tile.h"
+#include "ticket.h"
 
 namespace {
 
@@ -46,6 +47,14 @@ struct MlpArgs {
   float* db[ENDIA_MLP_MAX_LAYERS];
   const float* x;
   float* dx;
+  // forward with the MSE loss on top (target != null): d loss / d output = 2 (out - target) / n goes to dpred, every
+  // work-group leaves its sum of squared differences in loss_part and the last one to arrive adds them up, in row order
+  const float* target;
+  float* dpred;
+  float* loss;
+  float* loss_part;
+  unsigned* ticket;
+  float inv_n;
 #ifdef ENDIA_MLP_STAMPS
   unsigned long long* stamps;  // profiling build: wall-clock stamps of work-group 0
 #endif
@@ -300,6 +309,37 @@ __global__ __launch_bounds__(64 * NW, 1) void mlp_fwd_kernel(MlpArgs p) {
       bias1_cur = bias1_nxt;
     }
   }
+  if (p.target) {  // mse = sum((out - target)^2) / n (mse_op.mojo:17-20) and its gradient; the outputs of these rows are still in LDS
+    __shared__ float red[NW];
+    const int L = p.layers, N = p.width[L], npad = (N + 15) & ~15;
+    const float* out = hs[L & 1];
+    const float two_over_n = 2.0f * p.inv_n;
+    float acc = 0.f;
+    for (int e = tid; e < ROWS * npad; e += 64 * NW) {
+      const int r = e / npad, col = e - r * npad;
+      if (row0 + r < p.batch && col < N) {
+        const int64_t at = (int64_t)(row0 + r) * N + col;
+        const float d = out[r * LD + col] - p.target[at];
+        acc += d * d;
+        if (p.dpred) p.dpred[at] = d * two_over_n;
+      }
+    }
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) acc += __shfl_down(acc, o);
+    if (lane == 0) red[wave] = acc;
+    __syncthreads();
+    if (tid == 0) {
+      float sum = 0.f;
+#pragma unroll
+      for (int w = 0; w < NW; ++w) sum += red[w];
+      endia::store_shared(&p.loss_part[blockIdx.x], sum);
+    }
+    if (endia::arrive_last(p.ticket, gridDim.x, reinterpret_cast<int*>(part)) && tid == 0) {
+      float sum = 0.f;
+      for (unsigned i = 0; i < gridDim.x; ++i) sum += endia::load_shared(&p.loss_part[i]);
+      p.loss[0] = sum * p.inv_n;
+    }
+  }
 }
 
 // delta[layers - 1] holds the incoming cotangent (the last layer has no activation). For l = layers - 1 .. 1:
@@ -447,6 +487,42 @@ extern "C" int32_t endia_hip_mlp_fwd(const endia_hip_mlp_desc* desc, const float
   a.stamps = reinterpret_cast<unsigned long long*>(ctx().tickets);
 #endif
   hipLaunchKernelGGL(mlp_fwd_kernel, dim3((unsigned)ceil_div64(a.batch, ROWS)), dim3(64 * NW), 0, ctx().stream, a);
+  ENDIA_LAUNCH_CHECK();
+  return ENDIA_HIP_OK;
+}
+
+extern "C" int32_t endia_hip_mlp_fwd_mse(const endia_hip_mlp_desc* desc, const float* x, const float* const* W, const float* const* b,
+                                         const float* target, float* const* h, float* dpred, float* loss) {
+  ENDIA_REQUIRE_INIT();
+  MlpArgs a;
+  int32_t rc = fill_args(a, desc, "endia_hip_mlp_fwd_mse");
+  if (rc) return rc;
+  ENDIA_CHECK_ARG(loss != nullptr, "endia_hip_mlp_fwd_mse: loss is null");
+  if (a.batch == 0) return endia_hip_fill(loss, 1, 0.f);
+  ENDIA_CHECK_ARG(x && W && b && h && target, "endia_hip_mlp_fwd_mse: null argument");
+  for (int l = 0; l < a.layers; ++l) {
+    ENDIA_CHECK_ARG(W[l] && b[l] && h[l], "endia_hip_mlp_fwd_mse: null pointer for layer %d", l);
+    a.W[l] = W[l];
+    a.b[l] = b[l];
+    a.h[l] = h[l];
+  }
+  a.x = x;
+  const int64_t groups = ceil_div64(a.batch, ROWS);
+  struct Scratch {  // partial sums from the library's pool, handed back on scope exit (reuse is stream-ordered)
+    void* p = nullptr;
+    ~Scratch() { if (p) endia_hip_free(p); }
+  } part;
+  if ((rc = endia_hip_malloc(groups * 4, &part.p))) return rc;
+  a.target = target;
+  a.dpred = dpred;
+  a.loss = loss;
+  a.loss_part = static_cast<float*>(part.p);
+  a.ticket = ctx().tickets + (kTicketCount - 1);
+  a.inv_n = 1.0f / (float)((int64_t)a.batch * a.width[a.layers]);
+#ifdef ENDIA_MLP_STAMPS
+  a.stamps = reinterpret_cast<unsigned long long*>(ctx().tickets);
+#endif
+  hipLaunchKernelGGL(mlp_fwd_kernel, dim3((unsigned)groups), dim3(64 * NW), 0, ctx().stream, a);
   ENDIA_LAUNCH_CHECK();
   return ENDIA_HIP_OK;
 }

@@ -1467,6 +1467,55 @@ def mlp_forward(x, weights, biases, act=None):
     return _register(hs[-1], [x] + list(weights) + list(biases), "mlp", vjp)
 
 
+def mlp_mse_loss(x, target, weights, biases, act=None):
+    """mse(mlp_forward(x, weights, biases, act), target) for a small model (see mlp_forward) with the loss evaluated by the
+    forward launch itself (endia_hip_mlp_fwd_mse: the outputs of a work-group's rows are still in LDS when the last
+    layer is done, so the squared differences and the loss gradient 2 (out - target) / n cost no launch of their own).
+    backward() then runs the two launches of endia_hip_mlp_bwd on that stored gradient: with the optimizer, 4 launches
+    for a training step of the reference's script (mlp_imp.mojo:56-68). Anything the fused launch does not cover (a model
+    that is not small, a target that needs a gradient, complex operands) is mse(mlp_forward(...)); a second-order pass
+    fails as it does for mlp_forward. Returns the loss, shape [1]."""
+    import ctypes
+    Lyr = len(weights)
+    widths = [x._shape[-1]] + [w._shape[1] for w in weights]
+    small = (x.ndim() == 2 and 1 <= Lyr <= L.MLP_MAX_LAYERS and act in (None, "identity", "relu", "tanh") and x.size() > 0
+             and not x.is_complex_ and not target._requires_grad and not target.is_complex_
+             and list(target._shape) == [x._shape[0], widths[-1]]
+             and all(1 <= n <= L.MLP_MAX_WIDTH for n in widths)
+             and all(w.ndim() == 2 and not w.is_complex_ and w._shape[0] == widths[i] for i, w in enumerate(weights))
+             and all(b.size() == widths[i + 1] and not b.is_complex_ for i, b in enumerate(biases)))
+    if not small:
+        return mse(mlp_forward(x, weights, biases, act), target)
+    B = x._shape[0]
+    xs, ts = contiguous(x), contiguous(target)
+    Ws, bs_ = [contiguous(w) for w in weights], [contiguous(b) for b in biases]
+    hs = [Array.empty([B, widths[i + 1]]) for i in range(Lyr)]
+    dpred = Array.empty([B, widths[-1]])
+    loss = Array.empty([1])
+    desc = L.MlpDesc()
+    desc.layers, desc.act, desc.batch = Lyr, _ACT[act], B
+    desc.widths[:Lyr + 1] = widths
+    ptrs = lambda arrs: (ctypes.c_void_p * Lyr)(*[a.data_ptr() if a is not None else None for a in arrs])
+    L.call("endia_hip_mlp_fwd_mse", ctypes.byref(desc), xs.data_ptr(), ptrs(Ws), ptrs(bs_), ts.data_ptr(), ptrs(hs), dpred.data_ptr(),
+           loss.data_ptr())
+
+    def vjp(primals, grad, out_):
+        from .autograd.functional import building_graph
+        if building_graph():
+            raise NotImplementedError("mlp_mse_loss is a first-order op; use mse(model.forward(x), target) with fused=True for higher-order passes")
+        last = dpred if _holds_seed(grad) else mul(dpred, grad)  # (a cotangent other than the seed scales the stored gradient)
+        deltas = [Array.empty([B, widths[i + 1]]) for i in range(Lyr - 1)] + [contiguous(last)]
+        pW, pb = primals[2:2 + Lyr], primals[2 + Lyr:]
+        dW = [Array.empty([widths[i], widths[i + 1]]) if pW[i]._requires_grad else None for i in range(Lyr)]
+        db = [Array.empty([1, widths[i + 1]]) if pb[i]._requires_grad else None for i in range(Lyr)]  # kept axis, like Expand.vjp
+        dx = Array.empty([B, widths[0]]) if primals[0]._requires_grad else None
+        L.call("endia_hip_mlp_bwd", ctypes.byref(desc), xs.data_ptr(), ptrs(Ws), ptrs(hs), ptrs(deltas), ptrs(dW), ptrs(db),
+               dx.data_ptr() if dx is not None else None)
+        return [dx, None] + dW + db
+
+    return _register(loss, [x, target] + list(weights) + list(biases), "mlp_mse", vjp)
+
+
 def _fused_act_of(px):
     """The activation a gradient may absorb on its way to px: px is the output of a fused layer (or the
     fused sin node on top of one), nothing else consumes it and it holds no earlier gradient."""

@@ -43,6 +43,14 @@ class MLP:
 
     __call__ = forward
 
+    def mse_loss(self, x, target):
+        """mse(self.forward(x), target). With fused="model" and a small model the forward launch evaluates the loss
+        and its gradient as well (functional.mlp_mse_loss): a training step is then forward + loss, cotangents,
+        gradients and the optimizer, four launches."""
+        if self.fused == "model":
+            return F.mlp_mse_loss(x, target, self.weights, self.biases, self.activation)
+        return F.mse(self.forward(x), target)
+
     def params(self):
         out = []
         for w, b in zip(self.weights, self.biases):

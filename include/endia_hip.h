@@ -224,6 +224,12 @@ typedef struct endia_hip_mlp_desc {
 } endia_hip_mlp_desc;
 ENDIA_API int32_t endia_hip_mlp_fwd(const endia_hip_mlp_desc* desc, const float* x, const float* const* W, const float* const* b,
                           float* const* h);
+/* endia_hip_mlp_fwd with the MSE loss of the reference's training script on top (mlp_imp.mojo:56-60: forward, then
+ * mse_op.mojo:17-20), in the same launch: loss (one device float) = mean((h[layers-1] - target)^2), and dpred
+ * [batch, widths[layers]] (may be null) = 2 (h[layers-1] - target) / n, which is what endia_hip_mlp_bwd takes as
+ * delta[layers-1]. The work-groups' partial sums are added in row order by the last one to finish. */
+ENDIA_API int32_t endia_hip_mlp_fwd_mse(const endia_hip_mlp_desc* desc, const float* x, const float* const* W,
+                              const float* const* b, const float* target, float* const* h, float* dpred, float* loss);
 ENDIA_API int32_t endia_hip_mlp_bwd(const endia_hip_mlp_desc* desc, const float* x, const float* const* W, const float* const* h,
                           float* const* delta, float* const* dW, float* const* db, float* dx);
 

@@ -1159,6 +1159,62 @@ def test_callable_mixed_argnums(nd):
     assert_close(nested[2][0].to_numpy(), H[0][1].numpy(), what="second order")
 
 
+def test_whole_model_mse_loss_op(nd):
+    """functional.mlp_mse_loss (endia_hip_mlp_fwd_mse: the forward launch also evaluates the MSE loss and its gradient; the
+    work-groups' partial sums meet at a ticket) against mse(per-layer forward) + backward: loss and every gradient for
+    ragged shapes, a frozen parameter, many row groups, the input's gradient, a cotangent other than the seed, three calls
+    in a row bit-identical (the ticket is back at zero), and what it refuses."""
+    rng = np.random.default_rng(321)
+    for widths, batch, act in [([1, 32, 64, 128, 128, 128, 64, 32, 1], 128, "relu"), ([7, 50, 3, 128, 20], 37, "tanh"),
+                               ([128, 128], 16, None), ([5, 17], 1, "relu"), ([3, 8, 2], 1000, "relu"), ([40, 100, 9], 5000, "tanh")]:
+        Lyr = len(widths) - 1
+        Wn = [(rng.standard_normal((widths[i], widths[i + 1])) / np.sqrt(widths[i])).astype(np.float32) for i in range(Lyr)]
+        bn = [(0.2 * rng.standard_normal(widths[i + 1])).astype(np.float32) for i in range(Lyr)]
+        xn = rng.standard_normal((batch, widths[0])).astype(np.float32)
+        tn = rng.standard_normal((batch, widths[-1])).astype(np.float32)
+
+        def run(whole, scale=None):
+            x, t = nd.array(xn, requires_grad=True), nd.array(tn)
+            W = [nd.array(w, requires_grad=(i != 1)) for i, w in enumerate(Wn)]  # the second weight matrix is frozen
+            b = [nd.array(v, requires_grad=True) for v in bn]
+            if whole:
+                loss = nd.mlp_mse_loss(x, t, W, b, act)
+            else:
+                out = x
+                for i in range(Lyr):
+                    out = nd.linear(out, W[i], b[i], act if i < Lyr - 1 else None)
+                loss = nd.mse(out, t)
+            (loss if scale is None else loss * scale).backward()
+            grads = [x.grad().to_numpy()] + [w.grad().to_numpy() for w in W if w.has_grad()] + [v.grad().to_numpy().reshape(-1) for v in b]
+            assert not W[1].has_grad() if Lyr > 1 else True
+            return loss.to_numpy(), grads
+
+        what = "widths %s batch %d %s: " % (widths, batch, act)
+        for scale in (None, 3.0):
+            l_w, g_w = run(True, scale)
+            l_l, g_l = run(False, scale)
+            assert_close(l_w, l_l, tol=1e-5, what=what + "loss")
+            assert len(g_w) == len(g_l)
+            for k, (a, b_) in enumerate(zip(g_w, g_l)):
+                assert_close(a, b_, tol=2e-5, mean_tol=1e-3, what=what + "gradient %d" % k)  # (mean metric: a few values sum to ~0)
+        l_w, g_w = run(True)
+        for _ in range(2):
+            l_2, g_2 = run(True)
+            np.testing.assert_array_equal(l_2, l_w)
+            for a, b_ in zip(g_2, g_w):
+                np.testing.assert_array_equal(a, b_)
+    # through the model class, and the cases the op does not cover
+    mlp = nd.nn.MLP([4, 16, 2], compute_backward=True, fused="model")
+    x, t = nd.array(xn[:8, :4].copy()), nd.array(tn[:8, :2].copy())
+    a = mlp.mse_loss(x, t)
+    b_ = nd.mse(mlp.forward(x), t)
+    assert_close(a.to_numpy(), b_.to_numpy(), tol=1e-6, what="MLP.mse_loss")
+    with pytest.raises(NotImplementedError):
+        a.backward(create_graph=True)
+    wide = nd.nn.MLP([4, 200, 2], compute_backward=True, fused="model")  # too wide for the fused launch: the per-layer route
+    assert_close(wide.mse_loss(x, t).to_numpy(), nd.mse(wide.forward(x), t).to_numpy(), tol=1e-6, what="wide model")
+
+
 def test_whole_model_mlp_op(nd):
     """functional.mlp_forward through the C ABI's endia_hip_mlp_fwd / endia_hip_mlp_bwd: the same numbers as the
     per-layer path for ragged widths and batches (rows and columns that do not fill a 16 x 16 block), the input
