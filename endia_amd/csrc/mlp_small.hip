@@ -47,6 +47,7 @@ struct MlpArgs {
   float* db[ENDIA_MLP_MAX_LAYERS];
   const float* x;
   float* dx;
+  int tile0[ENDIA_MLP_MAX_LAYERS + 1];  // weight gradients: first 32 x 32 tile of every layer in the launch's grid
   // forward with the MSE loss on top (target != null): d loss / d output = 2 (out - target) / n goes to dpred, every
   // work-group leaves its sum of squared differences in loss_part and the last one to arrive adds them up, in row order
   const float* target;
@@ -396,54 +397,377 @@ __global__ __launch_bounds__(64 * NW, 1) void mlp_delta_kernel(MlpArgs p) {
   }
 }
 
-// One wave per 16 x 16 block of dW_l, plus one block row per layer for db_l (a left operand of ones).
-__global__ __launch_bounds__(256) void mlp_wgrad_kernel(MlpArgs p) {
-  const int lane = threadIdx.x & 63, c = lane & 15, g = lane >> 4;
-  int blk = blockIdx.x * 4 + (threadIdx.x >> 6);
-  int l = 0, nbk = 0, nbn = 0;
-  for (; l < p.layers; ++l) {
-    nbk = (p.width[l] + 15) / 16 + 1;
-    nbn = (p.width[l + 1] + 15) / 16;
-    if (blk < nbk * nbn) break;
-    blk -= nbk * nbn;
+// ---- row-block kernels on v_mfma_f32_4x4x1_16b_f32 ---------------------------------------------------------------
+// The instruction computes sixteen independent 4 x 4 outer products: block B = lane / 4 takes its four A values from
+// the lanes 4 B + i (rows) and its four B values from the lanes 4 B + j (columns) and adds A[i] * B[j] to register i of
+// lane 4 B + j (checked against the hardware with distinct values in every lane). It runs at the rate of the 16 x 16 x 4
+// form (256 multiply-adds in 8 cycles) but its left operand is 4 rows, not 16, so a work-group can own FOUR rows of
+// the batch without idle MFMA rows: the reference's model at batch 128 becomes 32 work-groups instead of 8, each with a
+// quarter of the dependent chain per layer.
+//
+// A wave owns 16 output columns for the whole reduction. Its blocks are 4 column quads (cq = lane / 16) x 4 slices of
+// the reduction (kq = lane / 4 % 4): MFMA (T, e) of a layer multiplies reduction index 16 T + 4 kq + e, so that a
+// lane's four A values of one T are one 16-byte LDS read, and the four slices are added with two row rotations (DPP)
+// at the end. No partial sums pass through LDS and a layer has ONE barrier. Afterwards every lane finishes exactly one
+// output per row quad: row kq, column 16 wave + 4 cq + j (bias, activation, LDS store, global store).
+constexpr int LD4 = MAXW + 16;  // LDS row stride = 16 (mod 64): the 16-byte reads of rows i = 0..3 at 4 kq fall into distinct banks
+constexpr int MAXT4 = MAXW / 16;
+
+struct Frag4 {
+  float v[MAXT4][4];  // [T][e]
+};
+
+// v + (v rotated right by N lanes within each row of 16 lanes)
+template <int CTRL>
+__device__ __forceinline__ float row_ror_add(float v) {
+  return v + __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), CTRL, 0xf, 0xf, false));
+}
+// the sum over the four reduction slices (lanes 4 apart within a row of 16), left in all four of them
+__device__ __forceinline__ float sum_slices(float v) { return row_ror_add<0x124>(row_ror_add<0x128>(v)); }
+
+__device__ __forceinline__ float pick(const floatx4& a, int i) { return i == 0 ? a[0] : (i == 1 ? a[1] : (i == 2 ? a[2] : a[3])); }
+
+template <int RQ>
+__device__ __forceinline__ void stage_rows4(float* __restrict__ dst, const float* __restrict__ src, int row0, int batch, int width, int tid) {
+  const int padded = (width + 15) & ~15;
+  for (int e = tid; e < 4 * RQ * padded; e += 64 * NW) {
+    const int r = e / padded, k = e - r * padded;
+    dst[r * LD4 + k] = (row0 + r < batch && k < width) ? src[(int64_t)(row0 + r) * width + k] : 0.f;
   }
-  if (l == p.layers) return;
-  const int K = p.width[l], N = p.width[l + 1];
-  const int bk = blk / nbn, bn = blk - bk * nbn;
-  const bool bias_row = bk == nbk - 1;
-  const float* __restrict__ hp = l == 0 ? p.x : p.h[l - 1];  // [batch, K]
-  const float* __restrict__ dl = p.delta[l];                 // [batch, N]
-  const int m = 16 * bk + c, n = 16 * bn + c;
-  floatx4 acc = {0.f, 0.f, 0.f, 0.f};
-  const __amdgpu_buffer_rsrc_t ra = make_rsrc(hp, (int64_t)p.batch * K * 4), rb = make_rsrc(dl, (int64_t)p.batch * N * 4);
-  const uint32_t va = m < K ? (uint32_t)((4 * g * K + m) * 4) : OOB_OFFSET, vb = n < N ? (uint32_t)((4 * g * N + n) * 4) : OOB_OFFSET;
-  constexpr int WGS = 4;
-  for (int t0 = 0; t0 < p.batch; t0 += 16 * WGS) {  // WGS super-steps' loads in flight at once, no branch between them
-    float a[WGS][4], b[WGS][4];
+}
+
+// acc[rq] (register i = row 4 rq + i, lane's column) = in[4 RQ x red] (LDS) . w; the sum over the slices is taken here
+template <int RQ>
+__device__ __forceinline__ void layer_mfma4(const float* __restrict__ in, const Frag4& w, int red, int kq, int j, floatx4 (&out)[RQ]) {
+  floatx4 acc[RQ][2];  // two chains per row quad: MFMA e does not wait for MFMA e - 1
 #pragma unroll
-    for (int t = 0; t < WGS; ++t)
+  for (int rq = 0; rq < RQ; ++rq) acc[rq][0] = acc[rq][1] = floatx4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        const int r = t0 + 16 * t + 4 * g + i;
-        const bool in = r < p.batch;
-        // (rows past the batch lie past the end of both buffers and read as zero)
-        a[t][i] = bias_row ? (in ? 1.f : 0.f) : buffer_load_f1(ra, va + (uint32_t)((t0 + 16 * t + i) * K * 4));
-        b[t][i] = buffer_load_f1(rb, vb + (uint32_t)((t0 + 16 * t + i) * N * 4));
+  for (int T = 0; T < MAXT4; ++T) {
+    if (16 * T < red) {
+      float av[RQ][4];
+#pragma unroll
+      for (int rq = 0; rq < RQ; ++rq) {
+        const float4 a = *reinterpret_cast<const float4*>(&in[(4 * rq + j) * LD4 + 16 * T + 4 * kq]);
+        av[rq][0] = a.x; av[rq][1] = a.y; av[rq][2] = a.z; av[rq][3] = a.w;
       }
 #pragma unroll
-    for (int t = 0; t < WGS; ++t)
+      for (int e = 0; e < 4; ++e)
 #pragma unroll
-      for (int i = 0; i < 4; ++i) acc = __builtin_amdgcn_mfma_f32_16x16x4f32(a[t][i], b[t][i], acc, 0, 0, 0);
-  }
-  if (n >= N) return;
-  if (bias_row) {
-    if (g == 0 && p.db[l]) p.db[l][n] = acc[0];
-  } else if (p.dW[l]) {
-#pragma unroll
-    for (int v = 0; v < 4; ++v) {
-      const int k = 16 * bk + 4 * g + v;
-      if (k < K) p.dW[l][(int64_t)k * N + n] = acc[v];
+        for (int rq = 0; rq < RQ; ++rq) acc[rq][e & 1] = __builtin_amdgcn_mfma_f32_4x4x1f32(av[rq][e], w.v[T][e], acc[rq][e & 1], 0, 0, 0);
     }
+  }
+#pragma unroll
+  for (int rq = 0; rq < RQ; ++rq)
+#pragma unroll
+    for (int i = 0; i < 4; ++i) out[rq][i] = sum_slices(acc[rq][0][i] + acc[rq][1][i]);
+}
+
+// Everything a layer consumes from memory is requested one layer ahead, and a layer's outputs are stored one layer
+// later, from registers. Each layer begins by waiting for ALL outstanding memory operations: the compiler then knows
+// that the operands at hand have arrived and places no wait of its own further down (left to count the requests that
+// sit under the width tests, it waits for the NEXT layer's weights ahead of the current layer's MFMAs).
+__device__ __forceinline__ void wait_vm_all() { __builtin_amdgcn_s_waitcnt(0x0F70); }  // vmcnt(0), other counters untouched
+
+struct Pre4 {
+  Frag4 w;
+  float aux[4];  // forward: [0] = the lane's bias; backward: the stored activations at the lane's outputs, per row quad
+};
+
+// Forward pass. A request of a wave must cover whole 128-byte lines to be delivered at the CU's full rate (four times
+// the rate of 64-byte pieces, measured), and rows of W run along the OUTPUT columns. So here a wave owns sixteen rows
+// of W (reduction indices 16 wave .. 16 wave + 15) and all columns: the sixteen blocks of an MFMA are sixteen column
+// quads (lane = column within a half of 64), the left operand is the same in all blocks, and a request reads 256
+// consecutive bytes of one row. The eight waves' partial sums (4 RQ x 128 floats each) meet in LDS, where thread t
+// finishes column t % 128 of row t / 128 (+ 4 per further row quad): bias, activation, LDS, and the global store one
+// layer later.
+struct FragF {
+  float v[16][2];  // [kk][half]: W[16 wave + kk][64 half + lane]
+  float bias;
+};
+
+// The MFMAs of one wave for one layer: its sixteen reduction indices times HALVES column halves, and the partial sums
+// to LDS. Within an active wave all sixteen indices are in order: the input's columns are zero up to the next multiple
+// of 16 and rows of W past the last read as zero.
+template <int RQ, int HALVES>
+__device__ __forceinline__ void slab_mfma(const float* __restrict__ in, const FragF& w, int wave, int lane, float (*part)[MAXW]) {
+  const int j = lane & 3;
+  floatx4 acc[RQ][HALVES];
+  float a[RQ][16];
+#pragma unroll
+  for (int rq = 0; rq < RQ; ++rq) {
+#pragma unroll
+    for (int h = 0; h < HALVES; ++h) acc[rq][h] = floatx4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+      const float4 t = *reinterpret_cast<const float4*>(&in[(4 * rq + j) * LD4 + 16 * wave + 4 * q]);
+      a[rq][4 * q] = t.x; a[rq][4 * q + 1] = t.y; a[rq][4 * q + 2] = t.z; a[rq][4 * q + 3] = t.w;
+    }
+  }
+#pragma unroll
+  for (int kk = 0; kk < 16; ++kk)
+#pragma unroll
+    for (int h = 0; h < HALVES; ++h)
+#pragma unroll
+      for (int rq = 0; rq < RQ; ++rq) acc[rq][h] = __builtin_amdgcn_mfma_f32_4x4x1f32(a[rq][kk], w.v[kk][h], acc[rq][h], 0, 0, 0);
+#pragma unroll
+  for (int h = 0; h < HALVES; ++h)
+#pragma unroll
+    for (int rq = 0; rq < RQ; ++rq)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) part[4 * rq + i][64 * h + lane] = acc[rq][h][i];
+}
+
+template <int RQ>
+__global__ __launch_bounds__(64 * NW, 1) void mlp_fwd4_kernel(MlpArgs p) {
+  static_assert(NW * 16 == MAXW && 64 * NW == 4 * MAXW, "one wave per 16 reduction indices; one thread per output of a row quad");
+  constexpr int R = 4 * RQ;
+  __shared__ __attribute__((aligned(16))) float hs[2][R * LD4];
+  __shared__ float part[NW][R][MAXW];
+  __shared__ int meet;
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, j = lane & 3;
+  const int ocol = tid & (MAXW - 1), orow = tid >> 7;  // the outputs this thread finishes: column ocol of rows orow + 4 u
+  const int row0 = blockIdx.x * R;
+  auto request = [&](int l, FragF& f) {
+    const int K = p.width[l], N = p.width[l + 1];
+    const __amdgpu_buffer_rsrc_t rb = make_rsrc(p.b[l], (int64_t)N * 4);
+    f.bias = buffer_load_f1(rb, ocol < N ? (uint32_t)(ocol * 4) : OOB_OFFSET);
+    if (16 * wave >= K) return;
+    const __amdgpu_buffer_rsrc_t rs = make_rsrc(p.W[l], (int64_t)K * N * 4);  // rows past K lie past the end of the buffer
+#pragma unroll
+    for (int half = 0; half < 2; ++half)
+      if (64 * half < N) {
+        const uint32_t base = 64 * half + lane < N ? (uint32_t)((16 * wave * N + 64 * half + lane) * 4) : OOB_OFFSET;
+#pragma unroll
+        for (int kk = 0; kk < 16; ++kk) f.v[kk][half] = buffer_load_f1(rs, base + (uint32_t)(kk * N * 4));
+      }
+  };
+  float z[RQ];  // the outputs this thread finished in the last layer
+  auto store = [&](int l) {
+    const int N = p.width[l + 1];
+    if (ocol < N) {
+#pragma unroll
+      for (int u = 0; u < RQ; ++u) {
+        const int r = row0 + orow + 4 * u;
+        if (r < p.batch) p.h[l][(int64_t)r * N + ocol] = z[u];
+      }
+    }
+  };
+  auto layer = [&](int l, const FragF& cur, FragF& nxt) {
+    const int K = p.width[l], N = p.width[l + 1];
+    const bool last = l + 1 == p.layers;
+    wait_vm_all();
+    if (!last) request(l + 1, nxt);
+    if (l > 0) store(l - 1);
+    const float* in = hs[l & 1];
+    float* out = hs[(l & 1) ^ 1];
+    if (16 * wave < K) {
+      // (one straight run of MFMAs per case: a width test inside the run costs a branch and register copies per MFMA)
+      if (N > 64) slab_mfma<RQ, 2>(in, cur, wave, lane, part[wave]);
+      else slab_mfma<RQ, 1>(in, cur, wave, lane, part[wave]);
+    }
+    __syncthreads();
+    const int npad = (N + 15) & ~15, slabs = (K + 15) >> 4;
+    if (ocol < npad) {
+#pragma unroll
+      for (int u = 0; u < RQ; ++u) {
+        float pw[NW];
+#pragma unroll
+        for (int w = 0; w < NW; ++w) pw[w] = part[w][orow + 4 * u][ocol];  // (all eight reads travel together; idle waves' slots hold leftovers)
+        float v = cur.bias;
+#pragma unroll
+        for (int w = 0; w < NW; ++w) v += w < slabs ? pw[w] : 0.f;  // partial sums in the order of their reduction ranges
+        if (!last) v = act_apply(p.act, v);
+        if (ocol >= N) v = 0.f;  // columns up to the next multiple of 16 feed the next reduction as zeros
+        out[(orow + 4 * u) * LD4 + ocol] = v;
+        z[u] = v;
+      }
+    }
+    __syncthreads();
+  };
+  FragF wa, wb;
+  request(0, wa);  // the first layer's weights travel while the input is staged
+  stage_rows4<RQ>(hs[0], p.x, row0, p.batch, p.width[0], tid);
+  __syncthreads();
+  for (int l = 0; l < p.layers; l += 2) {  // (two layers per round: the operands change places without copies)
+    layer(l, wa, wb);
+    if (l + 1 < p.layers) layer(l + 1, wb, wa);
+  }
+  store(p.layers - 1);
+  if (p.target) {  // mse = sum((out - target)^2) / n (mse_op.mojo:17-20) and its gradient; the outputs of these rows are still in LDS
+    __shared__ float red[NW];
+    const int L = p.layers, N = p.width[L], npad = (N + 15) & ~15;
+    const float* out = hs[L & 1];
+    const float two_over_n = 2.0f * p.inv_n;
+    float acc = 0.f;
+    for (int e = tid; e < R * npad; e += 64 * NW) {
+      const int r = e / npad, c = e - r * npad;
+      if (row0 + r < p.batch && c < N) {
+        const int64_t at = (int64_t)(row0 + r) * N + c;
+        const float d = out[r * LD4 + c] - p.target[at];
+        acc += d * d;
+        if (p.dpred) p.dpred[at] = d * two_over_n;
+      }
+    }
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) acc += __shfl_down(acc, o);
+    if (lane == 0) red[wave] = acc;
+    __syncthreads();
+    if (tid == 0) {
+      float sum = 0.f;
+#pragma unroll
+      for (int w = 0; w < NW; ++w) sum += red[w];
+      endia::store_shared(&p.loss_part[blockIdx.x], sum);
+    }
+    if (endia::arrive_last(p.ticket, gridDim.x, &meet) && tid == 0) {
+      float sum = 0.f;
+      for (unsigned i = 0; i < gridDim.x; ++i) sum += endia::load_shared(&p.loss_part[i]);
+      p.loss[0] = sum * p.inv_n;
+    }
+  }
+}
+
+// delta[layers - 1] holds the incoming cotangent (the last layer has no activation). For l = layers - 1 .. 1:
+// delta[l - 1] = (delta[l] W_l^T) * act'(h[l - 1]); finally dx = delta[0] W_0^T when asked for.
+template <int RQ>
+__global__ __launch_bounds__(64 * NW, 1) void mlp_delta4_kernel(MlpArgs p) {
+  constexpr int R = 4 * RQ;
+  __shared__ __attribute__((aligned(16))) float ds[2][R * LD4];
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, j = lane & 3, kq = (lane >> 2) & 3, cq = lane >> 4;
+  const int col = 16 * wave + 4 * cq + j;  // the lane's output column: a row of W
+  const int row0 = blockIdx.x * R;
+  const int L = p.layers;
+  const int first = p.dx ? 0 : 1;  // lowest layer whose W^T is applied
+  if (L - 1 < first) return;
+  // B operands of layer l (W_l is K x N, the product is [rows, N] . [N, K]): element [T][e] is W[col][16 T + 4 kq + e],
+  // four neighbouring floats of a row of W: one 16-byte request where rows are whole 16-byte pieces. With them, the
+  // outputs of the activation that produced this layer's input (none below the first layer).
+  auto request = [&](int l, Pre4& f) {
+    const int K = p.width[l], N = p.width[l + 1];
+    if (16 * wave >= K) return;
+    const __amdgpu_buffer_rsrc_t rs = make_rsrc(p.W[l], (int64_t)K * N * 4);
+    const bool vec = (N & 3) == 0 && (reinterpret_cast<uintptr_t>(p.W[l]) & 15) == 0;
+    const uint32_t base = (uint32_t)((col * N + 4 * kq) * 4);
+#pragma unroll
+    for (int T = 0; T < MAXT4; ++T)
+      if (16 * T < N) {
+        if (vec) {
+          const float4 w = buffer_load_f4(rs, (col < K && 16 * T + 4 * kq < N) ? base + (uint32_t)(64 * T) : OOB_OFFSET);
+          f.w.v[T][0] = w.x; f.w.v[T][1] = w.y; f.w.v[T][2] = w.z; f.w.v[T][3] = w.w;
+        } else {
+#pragma unroll
+          for (int e = 0; e < 4; ++e)
+            f.w.v[T][e] = buffer_load_f1(rs, (col < K && 16 * T + 4 * kq + e < N) ? base + (uint32_t)((16 * T + e) * 4) : OOB_OFFSET);
+        }
+      }
+    const __amdgpu_buffer_rsrc_t rh = make_rsrc(l > 0 ? p.h[l - 1] : p.x, l > 0 ? (int64_t)p.batch * K * 4 : 0);
+#pragma unroll
+    for (int rq = 0; rq < RQ; ++rq) {
+      const int r = row0 + 4 * rq + kq;
+      f.aux[rq] = buffer_load_f1(rh, (l > 0 && col < K && r < p.batch) ? (uint32_t)((r * K + col) * 4) : OOB_OFFSET);
+    }
+  };
+  float d[RQ];  // the outputs this lane finished in the last layer
+  auto store = [&](int l) {  // outputs of layer l: delta[l - 1], or dx
+    const int K = p.width[l];
+    float* dst = l > 0 ? p.delta[l - 1] : p.dx;
+    if (col < K) {
+#pragma unroll
+      for (int rq = 0; rq < RQ; ++rq) {
+        const int r = row0 + 4 * rq + kq;
+        if (r < p.batch) dst[(int64_t)r * K + col] = d[rq];
+      }
+    }
+  };
+  int buf = 0;
+  auto layer = [&](int l, const Pre4& cur, Pre4& nxt) {
+    const int K = p.width[l], N = p.width[l + 1];
+    wait_vm_all();
+    if (l - 1 >= first) request(l - 1, nxt);
+    if (l < L - 1) store(l + 1);
+    if (16 * wave < K) {
+      floatx4 acc[RQ];
+      layer_mfma4<RQ>(ds[buf], cur.w, N, kq, j, acc);
+      float* out = ds[buf ^ 1];
+#pragma unroll
+      for (int rq = 0; rq < RQ; ++rq) {
+        d[rq] = col < K ? pick(acc[rq], kq) * (l > 0 ? act_slope(p.act, cur.aux[rq]) : 1.f) : 0.f;
+        out[(4 * rq + kq) * LD4 + col] = d[rq];
+      }
+    }
+    __syncthreads();
+    buf ^= 1;
+  };
+  Pre4 wa, wb;
+  request(L - 1, wa);
+  stage_rows4<RQ>(ds[0], p.delta[L - 1], row0, p.batch, p.width[L], tid);
+  __syncthreads();
+  int l = L - 1;
+  for (; l >= first; l -= 2) {
+    layer(l, wa, wb);
+    if (l - 1 >= first) layer(l - 1, wb, wa);
+  }
+  store(first);
+}
+
+// dW_l = h_{l-1}^T delta_l and db_l = 1^T delta_l for ALL layers in one launch: a work-group per 32 x 32 tile of a
+// gradient, v_mfma_f32_32x32x2_f32 (left operand: lane = column of h, two rows of the batch per MFMA; a request reads
+// 128 consecutive bytes of each of two rows, whole lines). The four waves take rows 32 w .. 32 w + 31 of every 128 of
+// the batch; their partial tiles meet in LDS and are added in wave order, so results repeat bit for bit. The tiles
+// with bk = 0 also sum delta's columns (db).
+constexpr int WG_PITCH = 40;  // row pitch of a partial tile: the two half-waves of a store fall into different banks
+
+__global__ __launch_bounds__(256) void mlp_wgrad_kernel(MlpArgs p) {
+  __shared__ float part[4][32 * WG_PITCH];
+  __shared__ float bsum[4][2][32];
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, c = lane & 31, h = lane >> 5;
+  int l = 0;
+  while (l + 1 < p.layers && (int)blockIdx.x >= p.tile0[l + 1]) ++l;
+  const int K = p.width[l], N = p.width[l + 1];
+  const int tn = (N + 31) >> 5, t = (int)blockIdx.x - p.tile0[l];
+  const int bk = t / tn, bn = t - bk * tn;
+  const float* __restrict__ hp = l == 0 ? p.x : p.h[l - 1];  // [batch, K]
+  const float* __restrict__ dl = p.delta[l];                 // [batch, N]
+  const int m = 32 * bk + c, n = 32 * bn + c;
+  // (rows past the batch lie past the end of both buffers and read as zero)
+  const __amdgpu_buffer_rsrc_t ra = make_rsrc(hp, (int64_t)p.batch * K * 4), rb = make_rsrc(dl, (int64_t)p.batch * N * 4);
+  const uint32_t va = m < K ? (uint32_t)((h * K + m) * 4) : OOB_OFFSET, vb = n < N ? (uint32_t)((h * N + n) * 4) : OOB_OFFSET;
+  mfma::floatx16 acc;
+#pragma unroll
+  for (int v = 0; v < 16; ++v) acc[v] = 0.f;
+  float colsum = 0.f;
+  for (int r0 = 32 * wave; r0 < p.batch; r0 += 128) {
+    float a[16], b[16];
+#pragma unroll
+    for (int s = 0; s < 16; ++s) {
+      a[s] = buffer_load_f1(ra, va + (uint32_t)((r0 + 2 * s) * K * 4));
+      b[s] = buffer_load_f1(rb, vb + (uint32_t)((r0 + 2 * s) * N * 4));
+    }
+#pragma unroll
+    for (int s = 0; s < 16; ++s) {
+      acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a[s], b[s], acc, 0, 0, 0);
+      colsum += b[s];
+    }
+  }
+#pragma unroll
+  for (int v = 0; v < 16; ++v) part[wave][mfma::acc_row(v, h) * WG_PITCH + c] = acc[v];
+  bsum[wave][h][c] = colsum;
+  __syncthreads();
+  const int ocol = tid & 31, nn = 32 * bn + ocol;
+  if (nn >= N) return;
+  if (p.dW[l]) {
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      const int row = (tid >> 5) + 8 * u, k = 32 * bk + row;
+      const float sum = ((part[0][row * WG_PITCH + ocol] + part[1][row * WG_PITCH + ocol]) + part[2][row * WG_PITCH + ocol]) + part[3][row * WG_PITCH + ocol];
+      if (k < K) p.dW[l][(int64_t)k * N + nn] = sum;
+    }
+  }
+  if (bk == 0 && tid < 32 && p.db[l]) {
+    float sum = 0.f;
+#pragma unroll
+    for (int w = 0; w < 4; ++w) sum += bsum[w][0][ocol] + bsum[w][1][ocol];
+    p.db[l][nn] = sum;
   }
 }
 
@@ -462,6 +786,34 @@ int32_t fill_args(MlpArgs& a, const endia_hip_mlp_desc* d, const char* who) {
   a.batch = (int)d->batch;
   for (int i = 0; i <= d->layers; ++i) a.width[i] = (int)d->widths[i];
   return ENDIA_HIP_OK;
+}
+
+// Four rows per work-group while that leaves the chip room (each group fetches every weight), sixteen beyond.
+constexpr int64_t kFourRowBatch = 2048;
+
+void launch_fwd(const MlpArgs& a, hipStream_t s) {
+  static const bool old_path = getenv("ENDIA_MLP_OLD") != nullptr;
+  if (old_path) {
+    hipLaunchKernelGGL(mlp_fwd_kernel, dim3((unsigned)ceil_div64(a.batch, ROWS)), dim3(64 * NW), 0, s, a);
+  } else if (a.batch <= kFourRowBatch) {
+    hipLaunchKernelGGL(mlp_fwd4_kernel<1>, dim3((unsigned)ceil_div64(a.batch, 4)), dim3(64 * NW), 0, s, a);
+  } else {
+    hipLaunchKernelGGL(mlp_fwd4_kernel<4>, dim3((unsigned)ceil_div64(a.batch, 16)), dim3(64 * NW), 0, s, a);
+  }
+}
+int64_t fwd_groups(const MlpArgs& a) {
+  static const bool old_path = getenv("ENDIA_MLP_OLD") != nullptr;
+  return ceil_div64(a.batch, (!old_path && a.batch <= kFourRowBatch) ? 4 : 16);
+}
+void launch_delta(const MlpArgs& a, hipStream_t s) {
+  static const bool old_path = getenv("ENDIA_MLP_OLD") != nullptr;
+  if (old_path) {
+    hipLaunchKernelGGL(mlp_delta_kernel, dim3((unsigned)ceil_div64(a.batch, ROWS)), dim3(64 * NW), 0, s, a);
+  } else if (a.batch <= kFourRowBatch) {
+    hipLaunchKernelGGL(mlp_delta4_kernel<1>, dim3((unsigned)ceil_div64(a.batch, 4)), dim3(64 * NW), 0, s, a);
+  } else {
+    hipLaunchKernelGGL(mlp_delta4_kernel<4>, dim3((unsigned)ceil_div64(a.batch, 16)), dim3(64 * NW), 0, s, a);
+  }
 }
 
 }  // namespace
@@ -486,7 +838,7 @@ extern "C" int32_t endia_hip_mlp_fwd(const endia_hip_mlp_desc* desc, const float
 #ifdef ENDIA_MLP_STAMPS
   a.stamps = reinterpret_cast<unsigned long long*>(ctx().tickets);
 #endif
-  hipLaunchKernelGGL(mlp_fwd_kernel, dim3((unsigned)ceil_div64(a.batch, ROWS)), dim3(64 * NW), 0, ctx().stream, a);
+  launch_fwd(a, ctx().stream);
   ENDIA_LAUNCH_CHECK();
   return ENDIA_HIP_OK;
 }
@@ -507,7 +859,7 @@ extern "C" int32_t endia_hip_mlp_fwd_mse(const endia_hip_mlp_desc* desc, const f
     a.h[l] = h[l];
   }
   a.x = x;
-  const int64_t groups = ceil_div64(a.batch, ROWS);
+  const int64_t groups = fwd_groups(a);
   struct Scratch {  // partial sums from the library's pool, handed back on scope exit (reuse is stream-ordered)
     void* p = nullptr;
     ~Scratch() { if (p) endia_hip_free(p); }
@@ -522,7 +874,7 @@ extern "C" int32_t endia_hip_mlp_fwd_mse(const endia_hip_mlp_desc* desc, const f
 #ifdef ENDIA_MLP_STAMPS
   a.stamps = reinterpret_cast<unsigned long long*>(ctx().tickets);
 #endif
-  hipLaunchKernelGGL(mlp_fwd_kernel, dim3((unsigned)groups), dim3(64 * NW), 0, ctx().stream, a);
+  launch_fwd(a, ctx().stream);
   ENDIA_LAUNCH_CHECK();
   return ENDIA_HIP_OK;
 }
@@ -543,8 +895,10 @@ extern "C" int32_t endia_hip_mlp_bwd(const endia_hip_mlp_desc* desc, const float
     a.delta[l] = delta[l];
     a.dW[l] = dW[l];
     a.db[l] = db[l];
-    blocks += ((a.width[l] + 15) / 16 + 1) * ((a.width[l + 1] + 15) / 16);
+    a.tile0[l] = blocks;
+    blocks += ((a.width[l] + 31) / 32) * ((a.width[l + 1] + 31) / 32);
   }
+  a.tile0[a.layers] = blocks;
   a.x = x;
   a.dx = dx;
 #ifdef ENDIA_MLP_STAMPS
@@ -552,10 +906,10 @@ extern "C" int32_t endia_hip_mlp_bwd(const endia_hip_mlp_desc* desc, const float
 #endif
   hipStream_t s = ctx().stream;
   if (a.layers > 1 || dx) {
-    hipLaunchKernelGGL(mlp_delta_kernel, dim3((unsigned)ceil_div64(a.batch, ROWS)), dim3(64 * NW), 0, s, a);
+    launch_delta(a, s);
     ENDIA_LAUNCH_CHECK();
   }
-  hipLaunchKernelGGL(mlp_wgrad_kernel, dim3((unsigned)((blocks + 3) / 4)), dim3(256), 0, s, a);
+  hipLaunchKernelGGL(mlp_wgrad_kernel, dim3((unsigned)blocks), dim3(256), 0, s, a);
   ENDIA_LAUNCH_CHECK();
   return ENDIA_HIP_OK;
 }
