@@ -3,14 +3,22 @@
 // The reference's own benchmark model (benchmarks/mlp_benchmarks/mlp_imp.mojo:35-75: widths 1-32-64-128-128-128-64-32-1,
 // batch 128) is eight products of a few hundred kilo-flops each. One kernel per layer makes a training step a chain of
 // ~19 dependent launches whose cost is the launches. But every row of the batch is independent through all layers, in
-// the forward pass and in the chain of cotangents alike, so for layers of at most 128 units:
-//   mlp_fwd_kernel    one work-group (8 waves) owns 16 rows and runs ALL layers back to back: activations stay in LDS,
-//                     the weights (a few tens of KiB, resident in L2) go straight from memory into the B operands of
-//                     v_mfma_f32_16x16x4_f32, the next layer's while the current layer computes;
-//   mlp_delta_kernel  the same for the cotangents delta_{l-1} = (delta_l W_l^T) * act'(h_{l-1});
-//   mlp_wgrad_kernel  dW_l = h_{l-1}^T delta_l and db_l = 1^T delta_l for ALL layers in one launch, one wave per
-//                     16 x 16 block of a gradient, rows of the batch in ascending order (results repeat bit for bit).
-// No work-group ever waits for another.
+// the forward pass and in the chain of cotangents alike, so for layers of at most 128 units a work-group owns a few
+// rows of the batch and runs ALL layers back to back: activations stay in LDS, the weights (a few tens of KiB,
+// resident in L2) go straight from memory into MFMA operands, the next layer's while the current layer computes.
+//   mlp_fwd4_kernel / mlp_delta4_kernel   FOUR rows per work-group on v_mfma_f32_4x4x1_16b_f32, for batches of up to
+//                     1024 rows (the reference's 128 rows are 32 work-groups); every weight request covers whole
+//                     128-byte lines;
+//   mlp_fwd_kernel / mlp_delta_kernel     sixteen rows per work-group on v_mfma_f32_16x16x4_f32, beyond;
+//   mlp_wgrad_kernel  dW_l = h_{l-1}^T delta_l and db_l = 1^T delta_l for ALL layers in one launch, a work-group per
+//                     32 x 32 tile of a gradient on v_mfma_f32_32x32x2_f32, a fixed order of summation (results
+//                     repeat bit for bit).
+// No work-group ever waits for another (the forward launch with the MSE loss on top meets at a ticket at its end).
+//
+// What the measurements behind these kernels say about this machine: a wave's request is delivered at 64 bytes a clock
+// when its lanes cover whole 128-byte lines and at a quarter of that when they cover 64-byte pieces of many lines;
+// a width test around a request or an MFMA makes the compiler wait for memory between requests, or copy accumulators
+// around branches, so runs of requests and of MFMAs are kept straight.
 //
 // MFMA 16x16x4: A is 16 x 4 (lane: row = lane % 16, k = lane / 16), B is 4 x 16 (lane: column = lane % 16, k = lane / 16),
 // the accumulator holds rows 4 * (lane / 16) + v, v = 0..3, of column lane % 16. A sum over k may be taken in any
@@ -29,7 +37,7 @@ using mfma::OOB_OFFSET;
 
 typedef float floatx4 __attribute__((ext_vector_type(4)));
 
-constexpr int ROWS = 16;        // rows of the batch per work-group
+constexpr int ROWS = 16;        // rows of the batch per work-group of the sixteen-row kernels
 constexpr int MAXW = ENDIA_MLP_MAX_WIDTH;
 constexpr int LD = MAXW + 4;    // LDS row stride: 16 rows x 16-byte reads fall into distinct banks
 constexpr int MAXT = MAXW / 16; // super-steps of a full-width reduction
@@ -56,15 +64,7 @@ struct MlpArgs {
   float* loss_part;
   unsigned* ticket;
   float inv_n;
-#ifdef ENDIA_MLP_STAMPS
-  unsigned long long* stamps;  // profiling build: wall-clock stamps of work-group 0
-#endif
 };
-#ifdef ENDIA_MLP_STAMPS
-#define MLP_STAMP(i) do { if (blockIdx.x == 0 && threadIdx.x == 0) p.stamps[i] = wall_clock64(); } while (0)
-#else
-#define MLP_STAMP(i) do { } while (0)
-#endif
 
 __device__ __forceinline__ float act_apply(int act, float z) {
   return act == ENDIA_OP_RELU ? (z > 0.f ? z : 0.f) : (act == ENDIA_OP_TANH ? tanhf(z) : z);
@@ -208,7 +208,6 @@ __global__ __launch_bounds__(64 * NW, 1) void mlp_fwd_kernel(MlpArgs p) {
   __shared__ __attribute__((aligned(16))) float part[NW * ROWS * PLD];
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, c = lane & 15, g = lane >> 4;
   const int row0 = blockIdx.x * ROWS;
-  MLP_STAMP(0);
   WFrag cur_s, nxt_s;
   VFrag cur_v, nxt_v;
   WLoader<false> loader;
@@ -233,9 +232,7 @@ __global__ __launch_bounds__(64 * NW, 1) void mlp_fwd_kernel(MlpArgs p) {
   request_layer(0, plan, cur_v, cur_s, bias4_cur, bias1_cur);  // the first layer's weights travel while the input is staged
   stage_rows(hs[0], p.x, row0, p.batch, p.width[0], tid);
   __syncthreads();
-  MLP_STAMP(1);
   for (int l = 0; l < p.layers; ++l) {
-    MLP_STAMP(2 + 2 * l);
     const int K = p.width[l], N = p.width[l + 1];
     const bool last = l + 1 == p.layers;
     if (!last) request_layer(l + 1, plan_next, nxt_v, nxt_s, bias4_nxt, bias1_nxt);  // travels while this layer computes
@@ -260,7 +257,6 @@ __global__ __launch_bounds__(64 * NW, 1) void mlp_fwd_kernel(MlpArgs p) {
             }
         }
       }
-      MLP_STAMP(3 + 2 * l);
       if (64 * plan.G < N) {
 #pragma unroll
         for (int v = 0; v < 4; ++v)
@@ -287,7 +283,6 @@ __global__ __launch_bounds__(64 * NW, 1) void mlp_fwd_kernel(MlpArgs p) {
       WLoader<false> none;
       none.init(nullptr, 1, 1, wave, c, g);
       layer_mfma<false>(in, cur_s, K, N, wave, c, g, acc, none, nxt_s);
-      MLP_STAMP(3 + 2 * l);
       const int col = 16 * wave + c;
       if (16 * wave < N) {
 #pragma unroll
@@ -401,66 +396,30 @@ __global__ __launch_bounds__(64 * NW, 1) void mlp_delta_kernel(MlpArgs p) {
 // The instruction computes sixteen independent 4 x 4 outer products: block B = lane / 4 takes its four A values from
 // the lanes 4 B + i (rows) and its four B values from the lanes 4 B + j (columns) and adds A[i] * B[j] to register i of
 // lane 4 B + j (checked against the hardware with distinct values in every lane). It runs at the rate of the 16 x 16 x 4
-// form (256 multiply-adds in 8 cycles) but its left operand is 4 rows, not 16, so a work-group can own FOUR rows of
-// the batch without idle MFMA rows: the reference's model at batch 128 becomes 32 work-groups instead of 8, each with a
-// quarter of the dependent chain per layer.
-//
-// A wave owns 16 output columns for the whole reduction. Its blocks are 4 column quads (cq = lane / 16) x 4 slices of
-// the reduction (kq = lane / 4 % 4): MFMA (T, e) of a layer multiplies reduction index 16 T + 4 kq + e, so that a
-// lane's four A values of one T are one 16-byte LDS read, and the four slices are added with two row rotations (DPP)
-// at the end. No partial sums pass through LDS and a layer has ONE barrier. Afterwards every lane finishes exactly one
-// output per row quad: row kq, column 16 wave + 4 cq + j (bias, activation, LDS store, global store).
-constexpr int LD4 = MAXW + 16;  // LDS row stride = 16 (mod 64): the 16-byte reads of rows i = 0..3 at 4 kq fall into distinct banks
-constexpr int MAXT4 = MAXW / 16;
-
-struct Frag4 {
-  float v[MAXT4][4];  // [T][e]
-};
+// form (256 multiply-adds in 8 cycles, measured) but its left operand is 4 rows, not 16, so a work-group can own FOUR
+// rows of the batch without idle MFMA rows: the reference's model at batch 128 becomes 32 work-groups instead of 8,
+// each with a quarter of the MFMA work per layer. What the sixteen blocks stand for differs between the two kernels:
+// it is chosen so that a wave's weight requests cover whole 128-byte lines (see each kernel).
+constexpr int LD4 = MAXW + 16;  // LDS row stride = 16 (mod 64): 16-byte reads of the rows i = 0..3 start 16 banks apart
 
 // v + (v rotated right by N lanes within each row of 16 lanes)
 template <int CTRL>
 __device__ __forceinline__ float row_ror_add(float v) {
   return v + __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), CTRL, 0xf, 0xf, false));
 }
-// the sum over the four reduction slices (lanes 4 apart within a row of 16), left in all four of them
+// the sum over four lanes 4 apart within a row of 16, left in all four of them
 __device__ __forceinline__ float sum_slices(float v) { return row_ror_add<0x124>(row_ror_add<0x128>(v)); }
 
 __device__ __forceinline__ float pick(const floatx4& a, int i) { return i == 0 ? a[0] : (i == 1 ? a[1] : (i == 2 ? a[2] : a[3])); }
 
 template <int RQ>
-__device__ __forceinline__ void stage_rows4(float* __restrict__ dst, const float* __restrict__ src, int row0, int batch, int width, int tid) {
-  const int padded = (width + 15) & ~15;
+__device__ __forceinline__ void stage_rows4(float* __restrict__ dst, const float* __restrict__ src, int row0, int batch, int width, int tid,
+                                            int pad = 16) {
+  const int padded = (width + pad - 1) & ~(pad - 1);  // zeros up to the reduction's step
   for (int e = tid; e < 4 * RQ * padded; e += 64 * NW) {
     const int r = e / padded, k = e - r * padded;
     dst[r * LD4 + k] = (row0 + r < batch && k < width) ? src[(int64_t)(row0 + r) * width + k] : 0.f;
   }
-}
-
-// acc[rq] (register i = row 4 rq + i, lane's column) = in[4 RQ x red] (LDS) . w; the sum over the slices is taken here
-template <int RQ>
-__device__ __forceinline__ void layer_mfma4(const float* __restrict__ in, const Frag4& w, int red, int kq, int j, floatx4 (&out)[RQ]) {
-  floatx4 acc[RQ][2];  // two chains per row quad: MFMA e does not wait for MFMA e - 1
-#pragma unroll
-  for (int rq = 0; rq < RQ; ++rq) acc[rq][0] = acc[rq][1] = floatx4{0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-  for (int T = 0; T < MAXT4; ++T) {
-    if (16 * T < red) {
-      float av[RQ][4];
-#pragma unroll
-      for (int rq = 0; rq < RQ; ++rq) {
-        const float4 a = *reinterpret_cast<const float4*>(&in[(4 * rq + j) * LD4 + 16 * T + 4 * kq]);
-        av[rq][0] = a.x; av[rq][1] = a.y; av[rq][2] = a.z; av[rq][3] = a.w;
-      }
-#pragma unroll
-      for (int e = 0; e < 4; ++e)
-#pragma unroll
-        for (int rq = 0; rq < RQ; ++rq) acc[rq][e & 1] = __builtin_amdgcn_mfma_f32_4x4x1f32(av[rq][e], w.v[T][e], acc[rq][e & 1], 0, 0, 0);
-    }
-  }
-#pragma unroll
-  for (int rq = 0; rq < RQ; ++rq)
-#pragma unroll
-    for (int i = 0; i < 4; ++i) out[rq][i] = sum_slices(acc[rq][0][i] + acc[rq][1][i]);
 }
 
 // Everything a layer consumes from memory is requested one layer ahead, and a layer's outputs are stored one layer
@@ -468,11 +427,6 @@ __device__ __forceinline__ void layer_mfma4(const float* __restrict__ in, const 
 // that the operands at hand have arrived and places no wait of its own further down (left to count the requests that
 // sit under the width tests, it waits for the NEXT layer's weights ahead of the current layer's MFMAs).
 __device__ __forceinline__ void wait_vm_all() { __builtin_amdgcn_s_waitcnt(0x0F70); }  // vmcnt(0), other counters untouched
-
-struct Pre4 {
-  Frag4 w;
-  float aux[4];  // forward: [0] = the lane's bias; backward: the stored activations at the lane's outputs, per row quad
-};
 
 // Forward pass. A request of a wave must cover whole 128-byte lines to be delivered at the CU's full rate (four times
 // the rate of 64-byte pieces, measured), and rows of W run along the OUTPUT columns. So here a wave owns sixteen rows
@@ -518,8 +472,8 @@ __device__ __forceinline__ void slab_mfma(const float* __restrict__ in, const Fr
       for (int i = 0; i < 4; ++i) part[4 * rq + i][64 * h + lane] = acc[rq][h][i];
 }
 
-template <int RQ>
 __global__ __launch_bounds__(64 * NW, 1) void mlp_fwd4_kernel(MlpArgs p) {
+  constexpr int RQ = 1;  // row quads per work-group (more were measured slower than the sixteen-row kernel at the batches where they would apply)
   static_assert(NW * 16 == MAXW && 64 * NW == 4 * MAXW, "one wave per 16 reduction indices; one thread per output of a row quad");
   constexpr int R = 4 * RQ;
   __shared__ __attribute__((aligned(16))) float hs[2][R * LD4];
@@ -629,78 +583,141 @@ __global__ __launch_bounds__(64 * NW, 1) void mlp_fwd4_kernel(MlpArgs p) {
 
 // delta[layers - 1] holds the incoming cotangent (the last layer has no activation). For l = layers - 1 .. 1:
 // delta[l - 1] = (delta[l] W_l^T) * act'(h[l - 1]); finally dx = delta[0] W_0^T when asked for.
-template <int RQ>
+//
+// Here the reduction runs along the rows of W, so a wave owns 16 output columns = 16 rows of W_l for the whole
+// reduction, and a lane's B operands are 16-byte pieces of one row. For a request to cover whole 128-byte lines, eight
+// lanes must sit side by side in a row of W: the sixteen blocks of an MFMA are 8 slices of the reduction (s) x 2 column
+// quads (cq), MFMA (T, e) multiplies reduction index 32 T + 4 s + e, and the wave's sixteen columns take two passes of
+// eight that share the left operand. A request then reads 128 consecutive bytes of each of eight rows. The eight
+// slices are added with two row rotations and one swap of the wave's halves; afterwards lane (cq, s, j) finishes row
+// s % 4 of column 16 wave + 8 (s / 4) + 4 cq + j.
+struct FragD {
+  float v[2][MAXW / 32][4];  // [pass][T][e]: W[16 wave + 8 pass + 4 cq + j][32 T + 4 s + e]
+  float slope[4];            // the stored activations at the lane's outputs, per row quad
+};
+
+// the sum over the eight slices: lanes 4 and 8 apart within a row of 16, and the wave's other half
+__device__ __forceinline__ float sum_slices8(float v) {
+  v = sum_slices(v);
+  typedef unsigned uint2v __attribute__((ext_vector_type(2)));
+  const unsigned u = __float_as_uint(v);
+  const uint2v r = __builtin_amdgcn_permlane32_swap(u, u, false, false);  // {[lo | lo], [hi | hi]} of the two halves
+  return __uint_as_float(r[0]) + __uint_as_float(r[1]);
+}
+
+template <int RQ, int NT>
+__device__ __forceinline__ void rows_mfma(const float* __restrict__ in, const FragD& w, int s, int j, floatx4 (&out)[RQ][2]) {
+  floatx4 acc[RQ][2];
+#pragma unroll
+  for (int rq = 0; rq < RQ; ++rq) acc[rq][0] = acc[rq][1] = floatx4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+  for (int T = 0; T < NT; ++T) {
+    float av[RQ][4];
+#pragma unroll
+    for (int rq = 0; rq < RQ; ++rq) {
+      const float4 a = *reinterpret_cast<const float4*>(&in[(4 * rq + j) * LD4 + 32 * T + 4 * s]);
+      av[rq][0] = a.x; av[rq][1] = a.y; av[rq][2] = a.z; av[rq][3] = a.w;
+    }
+#pragma unroll
+    for (int e = 0; e < 4; ++e)
+#pragma unroll
+      for (int pass = 0; pass < 2; ++pass)
+#pragma unroll
+        for (int rq = 0; rq < RQ; ++rq) acc[rq][pass] = __builtin_amdgcn_mfma_f32_4x4x1f32(av[rq][e], w.v[pass][T][e], acc[rq][pass], 0, 0, 0);
+  }
+#pragma unroll
+  for (int rq = 0; rq < RQ; ++rq)
+#pragma unroll
+    for (int pass = 0; pass < 2; ++pass)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) out[rq][pass][i] = sum_slices8(acc[rq][pass][i]);
+}
+
 __global__ __launch_bounds__(64 * NW, 1) void mlp_delta4_kernel(MlpArgs p) {
+  constexpr int RQ = 1;  // row quads per work-group, as in the forward kernel
   constexpr int R = 4 * RQ;
   __shared__ __attribute__((aligned(16))) float ds[2][R * LD4];
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, j = lane & 3, kq = (lane >> 2) & 3, cq = lane >> 4;
-  const int col = 16 * wave + 4 * cq + j;  // the lane's output column: a row of W
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, j = lane & 3, cq = (lane >> 4) & 1;
+  const int s = ((lane >> 2) & 3) | ((lane >> 5) << 2);
+  const int wrow = 4 * cq + j;                             // + 8 pass: the lane's rows of W within the wave's sixteen
+  const int ocol = 16 * wave + 8 * (s >> 2) + wrow, orow = s & 3;  // the output this lane finishes, per row quad
   const int row0 = blockIdx.x * R;
   const int L = p.layers;
   const int first = p.dx ? 0 : 1;  // lowest layer whose W^T is applied
   if (L - 1 < first) return;
-  // B operands of layer l (W_l is K x N, the product is [rows, N] . [N, K]): element [T][e] is W[col][16 T + 4 kq + e],
-  // four neighbouring floats of a row of W: one 16-byte request where rows are whole 16-byte pieces. With them, the
-  // outputs of the activation that produced this layer's input (none below the first layer).
-  auto request = [&](int l, Pre4& f) {
+  // (a wave is at work while its columns begin below the width rounded up to 32: the next reduction reads that far)
+  auto active = [&](int K) { return 16 * wave < ((K + 31) & ~31); };
+  auto request = [&](int l, FragD& f) {
     const int K = p.width[l], N = p.width[l + 1];
-    if (16 * wave >= K) return;
+    if (!active(K)) return;
     const __amdgpu_buffer_rsrc_t rs = make_rsrc(p.W[l], (int64_t)K * N * 4);
     const bool vec = (N & 3) == 0 && (reinterpret_cast<uintptr_t>(p.W[l]) & 15) == 0;
-    const uint32_t base = (uint32_t)((col * N + 4 * kq) * 4);
+    // (no width test around a request: with one, the compiler can no longer tell which registers have a request
+    // outstanding and waits for memory between any two of them; a request past the width costs next to nothing)
 #pragma unroll
-    for (int T = 0; T < MAXT4; ++T)
-      if (16 * T < N) {
+    for (int pass = 0; pass < 2; ++pass) {
+      const int c = 16 * wave + 8 * pass + wrow;
+      const uint32_t base = (uint32_t)((c * N + 4 * s) * 4);
+#pragma unroll
+      for (int T = 0; T < MAXW / 32; ++T) {
+        const int n0 = 32 * T + 4 * s;
         if (vec) {
-          const float4 w = buffer_load_f4(rs, (col < K && 16 * T + 4 * kq < N) ? base + (uint32_t)(64 * T) : OOB_OFFSET);
-          f.w.v[T][0] = w.x; f.w.v[T][1] = w.y; f.w.v[T][2] = w.z; f.w.v[T][3] = w.w;
+          const float4 w = buffer_load_f4(rs, (c < K && n0 < N) ? base + (uint32_t)(128 * T) : OOB_OFFSET);
+          f.v[pass][T][0] = w.x; f.v[pass][T][1] = w.y; f.v[pass][T][2] = w.z; f.v[pass][T][3] = w.w;
         } else {
 #pragma unroll
-          for (int e = 0; e < 4; ++e)
-            f.w.v[T][e] = buffer_load_f1(rs, (col < K && 16 * T + 4 * kq + e < N) ? base + (uint32_t)((16 * T + e) * 4) : OOB_OFFSET);
+          for (int e = 0; e < 4; ++e) f.v[pass][T][e] = buffer_load_f1(rs, (c < K && n0 + e < N) ? base + (uint32_t)((32 * T + e) * 4) : OOB_OFFSET);
         }
       }
+    }
+    // the outputs of the activation that produced this layer's input (none below the first layer)
     const __amdgpu_buffer_rsrc_t rh = make_rsrc(l > 0 ? p.h[l - 1] : p.x, l > 0 ? (int64_t)p.batch * K * 4 : 0);
 #pragma unroll
     for (int rq = 0; rq < RQ; ++rq) {
-      const int r = row0 + 4 * rq + kq;
-      f.aux[rq] = buffer_load_f1(rh, (l > 0 && col < K && r < p.batch) ? (uint32_t)((r * K + col) * 4) : OOB_OFFSET);
+      const int r = row0 + 4 * rq + orow;
+      f.slope[rq] = buffer_load_f1(rh, (l > 0 && ocol < K && r < p.batch) ? (uint32_t)((r * K + ocol) * 4) : OOB_OFFSET);
     }
   };
   float d[RQ];  // the outputs this lane finished in the last layer
   auto store = [&](int l) {  // outputs of layer l: delta[l - 1], or dx
     const int K = p.width[l];
     float* dst = l > 0 ? p.delta[l - 1] : p.dx;
-    if (col < K) {
+    if (ocol < K) {
 #pragma unroll
       for (int rq = 0; rq < RQ; ++rq) {
-        const int r = row0 + 4 * rq + kq;
-        if (r < p.batch) dst[(int64_t)r * K + col] = d[rq];
+        const int r = row0 + 4 * rq + orow;
+        if (r < p.batch) dst[(int64_t)r * K + ocol] = d[rq];
       }
     }
   };
   int buf = 0;
-  auto layer = [&](int l, const Pre4& cur, Pre4& nxt) {
+  auto layer = [&](int l, const FragD& cur, FragD& nxt) {
     const int K = p.width[l], N = p.width[l + 1];
     wait_vm_all();
     if (l - 1 >= first) request(l - 1, nxt);
     if (l < L - 1) store(l + 1);
-    if (16 * wave < K) {
-      floatx4 acc[RQ];
-      layer_mfma4<RQ>(ds[buf], cur.w, N, kq, j, acc);
+    if (active(K)) {
+      floatx4 acc[RQ][2];
+      switch ((N + 31) >> 5) {
+        case 1: rows_mfma<RQ, 1>(ds[buf], cur, s, j, acc); break;
+        case 2: rows_mfma<RQ, 2>(ds[buf], cur, s, j, acc); break;
+        case 3: rows_mfma<RQ, 3>(ds[buf], cur, s, j, acc); break;
+        default: rows_mfma<RQ, 4>(ds[buf], cur, s, j, acc); break;
+      }
       float* out = ds[buf ^ 1];
 #pragma unroll
       for (int rq = 0; rq < RQ; ++rq) {
-        d[rq] = col < K ? pick(acc[rq], kq) * (l > 0 ? act_slope(p.act, cur.aux[rq]) : 1.f) : 0.f;
-        out[(4 * rq + kq) * LD4 + col] = d[rq];
+        const float v = s < 4 ? pick(acc[rq][0], orow) : pick(acc[rq][1], orow);
+        d[rq] = ocol < K ? v * (l > 0 ? act_slope(p.act, cur.slope[rq]) : 1.f) : 0.f;  // columns past the width feed the next reduction as zeros
+        out[(4 * rq + orow) * LD4 + ocol] = d[rq];
       }
     }
     __syncthreads();
     buf ^= 1;
   };
-  Pre4 wa, wb;
+  FragD wa, wb;
   request(L - 1, wa);
-  stage_rows4<RQ>(ds[0], p.delta[L - 1], row0, p.batch, p.width[L], tid);
+  stage_rows4<RQ>(ds[0], p.delta[L - 1], row0, p.batch, p.width[L], tid, 32);
   __syncthreads();
   int l = L - 1;
   for (; l >= first; l -= 2) {
@@ -736,18 +753,30 @@ __global__ __launch_bounds__(256) void mlp_wgrad_kernel(MlpArgs p) {
 #pragma unroll
   for (int v = 0; v < 16; ++v) acc[v] = 0.f;
   float colsum = 0.f;
-  for (int r0 = 32 * wave; r0 < p.batch; r0 += 128) {
-    float a[16], b[16];
+  // two sets of operands: the next 32 rows travel while the MFMAs of the current ones run (requests past the batch
+  // read zeros, so the last one needs no test)
+  float a[2][16], b[2][16];
+  auto request = [&](int r0, float (&av)[16], float (&bv)[16]) {
 #pragma unroll
     for (int s = 0; s < 16; ++s) {
-      a[s] = buffer_load_f1(ra, va + (uint32_t)((r0 + 2 * s) * K * 4));
-      b[s] = buffer_load_f1(rb, vb + (uint32_t)((r0 + 2 * s) * N * 4));
+      av[s] = buffer_load_f1(ra, va + (uint32_t)((r0 + 2 * s) * K * 4));
+      bv[s] = buffer_load_f1(rb, vb + (uint32_t)((r0 + 2 * s) * N * 4));
     }
+  };
+  auto multiply = [&](const float (&av)[16], const float (&bv)[16]) {
 #pragma unroll
     for (int s = 0; s < 16; ++s) {
-      acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a[s], b[s], acc, 0, 0, 0);
-      colsum += b[s];
+      acc = __builtin_amdgcn_mfma_f32_32x32x2f32(av[s], bv[s], acc, 0, 0, 0);
+      colsum += bv[s];
     }
+  };
+  request(32 * wave, a[0], b[0]);
+  for (int r0 = 32 * wave; r0 < p.batch; r0 += 256) {
+    request(r0 + 128, a[1], b[1]);
+    multiply(a[0], b[0]);
+    if (r0 + 128 >= p.batch) break;
+    request(r0 + 256, a[0], b[0]);
+    multiply(a[1], b[1]);
   }
 #pragma unroll
   for (int v = 0; v < 16; ++v) part[wave][mfma::acc_row(v, h) * WG_PITCH + c] = acc[v];
@@ -788,32 +817,18 @@ int32_t fill_args(MlpArgs& a, const endia_hip_mlp_desc* d, const char* who) {
   return ENDIA_HIP_OK;
 }
 
-// Four rows per work-group while that leaves the chip room (each group fetches every weight), sixteen beyond.
-constexpr int64_t kFourRowBatch = 2048;
+// Four rows per work-group while every group still gets a CU of its own (each group fetches every weight); sixteen
+// rows on the 16 x 16 x 4 MFMA beyond (measured: 2048 rows take 127 us on the four-row kernels, 95 us on these).
+constexpr int64_t kFourRowBatch = 1024;
+int64_t fwd_groups(const MlpArgs& a) { return ceil_div64(a.batch, a.batch <= kFourRowBatch ? 4 : ROWS); }
 
 void launch_fwd(const MlpArgs& a, hipStream_t s) {
-  static const bool old_path = getenv("ENDIA_MLP_OLD") != nullptr;
-  if (old_path) {
-    hipLaunchKernelGGL(mlp_fwd_kernel, dim3((unsigned)ceil_div64(a.batch, ROWS)), dim3(64 * NW), 0, s, a);
-  } else if (a.batch <= kFourRowBatch) {
-    hipLaunchKernelGGL(mlp_fwd4_kernel<1>, dim3((unsigned)ceil_div64(a.batch, 4)), dim3(64 * NW), 0, s, a);
-  } else {
-    hipLaunchKernelGGL(mlp_fwd4_kernel<4>, dim3((unsigned)ceil_div64(a.batch, 16)), dim3(64 * NW), 0, s, a);
-  }
-}
-int64_t fwd_groups(const MlpArgs& a) {
-  static const bool old_path = getenv("ENDIA_MLP_OLD") != nullptr;
-  return ceil_div64(a.batch, (!old_path && a.batch <= kFourRowBatch) ? 4 : 16);
+  if (a.batch <= kFourRowBatch) hipLaunchKernelGGL(mlp_fwd4_kernel, dim3((unsigned)fwd_groups(a)), dim3(64 * NW), 0, s, a);
+  else hipLaunchKernelGGL(mlp_fwd_kernel, dim3((unsigned)fwd_groups(a)), dim3(64 * NW), 0, s, a);
 }
 void launch_delta(const MlpArgs& a, hipStream_t s) {
-  static const bool old_path = getenv("ENDIA_MLP_OLD") != nullptr;
-  if (old_path) {
-    hipLaunchKernelGGL(mlp_delta_kernel, dim3((unsigned)ceil_div64(a.batch, ROWS)), dim3(64 * NW), 0, s, a);
-  } else if (a.batch <= kFourRowBatch) {
-    hipLaunchKernelGGL(mlp_delta4_kernel<1>, dim3((unsigned)ceil_div64(a.batch, 4)), dim3(64 * NW), 0, s, a);
-  } else {
-    hipLaunchKernelGGL(mlp_delta4_kernel<4>, dim3((unsigned)ceil_div64(a.batch, 16)), dim3(64 * NW), 0, s, a);
-  }
+  if (a.batch <= kFourRowBatch) hipLaunchKernelGGL(mlp_delta4_kernel, dim3((unsigned)fwd_groups(a)), dim3(64 * NW), 0, s, a);
+  else hipLaunchKernelGGL(mlp_delta_kernel, dim3((unsigned)fwd_groups(a)), dim3(64 * NW), 0, s, a);
 }
 
 }  // namespace
@@ -835,9 +850,6 @@ extern "C" int32_t endia_hip_mlp_fwd(const endia_hip_mlp_desc* desc, const float
     a.h[l] = h[l];
   }
   a.x = x;
-#ifdef ENDIA_MLP_STAMPS
-  a.stamps = reinterpret_cast<unsigned long long*>(ctx().tickets);
-#endif
   launch_fwd(a, ctx().stream);
   ENDIA_LAUNCH_CHECK();
   return ENDIA_HIP_OK;
@@ -871,9 +883,6 @@ extern "C" int32_t endia_hip_mlp_fwd_mse(const endia_hip_mlp_desc* desc, const f
   a.loss_part = static_cast<float*>(part.p);
   a.ticket = ctx().tickets + (kTicketCount - 1);
   a.inv_n = 1.0f / (float)((int64_t)a.batch * a.width[a.layers]);
-#ifdef ENDIA_MLP_STAMPS
-  a.stamps = reinterpret_cast<unsigned long long*>(ctx().tickets);
-#endif
   launch_fwd(a, ctx().stream);
   ENDIA_LAUNCH_CHECK();
   return ENDIA_HIP_OK;
@@ -901,9 +910,6 @@ extern "C" int32_t endia_hip_mlp_bwd(const endia_hip_mlp_desc* desc, const float
   a.tile0[a.layers] = blocks;
   a.x = x;
   a.dx = dx;
-#ifdef ENDIA_MLP_STAMPS
-  a.stamps = reinterpret_cast<unsigned long long*>(ctx().tickets) + 64;
-#endif
   hipStream_t s = ctx().stream;
   if (a.layers > 1 || dx) {
     launch_delta(a, s);
@@ -914,6 +920,3 @@ extern "C" int32_t endia_hip_mlp_bwd(const endia_hip_mlp_desc* desc, const float
   return ENDIA_HIP_OK;
 }
 
-#ifdef ENDIA_MLP_STAMPS
-extern "C" __attribute__((visibility("default"))) void* endia_debug_mlp_stamps(void) { return endia::ctx().tickets; }
-#endif

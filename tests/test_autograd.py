@@ -1217,11 +1217,13 @@ def test_whole_model_mse_loss_op(nd):
 
 def test_whole_model_mlp_op(nd):
     """functional.mlp_forward through the C ABI's endia_hip_mlp_fwd / endia_hip_mlp_bwd: the same numbers as the
-    per-layer path for ragged widths and batches (rows and columns that do not fill a 16 x 16 block), the input
-    gradient, a parameter that needs no gradient, two calls in a row (bit-identical), and the cases it refuses."""
+    per-layer path for ragged widths and batches (rows and columns that do not fill an MFMA block), batches on both
+    sides of the switch from four to sixteen rows per work-group (1024 rows), the input gradient, a parameter that
+    needs no gradient, two calls in a row (bit-identical), and the cases it refuses."""
     rng = np.random.default_rng(123)
     for widths, batch, act in [([1, 32, 64, 128, 128, 128, 64, 32, 1], 128, "relu"), ([7, 50, 3, 128, 20], 37, "tanh"),
-                               ([128, 128], 16, None), ([5, 17], 1, "relu"), ([40, 100, 100, 9], 300, "relu")]:
+                               ([128, 128], 16, None), ([5, 17], 1, "relu"), ([40, 100, 100, 9], 300, "relu"),
+                               ([33, 128, 65, 12], 1024, "tanh"), ([33, 128, 65, 12], 1500, "relu")]:
         Lyr = len(widths) - 1
         Wn = [(rng.standard_normal((widths[i], widths[i + 1])) / np.sqrt(widths[i])).astype(np.float32) for i in range(Lyr)]
         bn = [(0.2 * rng.standard_normal(widths[i + 1])).astype(np.float32) for i in range(Lyr)]
