@@ -539,6 +539,15 @@ __global__ __launch_bounds__(64 * NW, 1) void mlp_fwd4_kernel(MlpArgs p) {
     }
     __syncthreads();
   };
+  // the targets of this thread's outputs of the last layer, asked for now and needed at the very end
+  const int NL = p.width[p.layers];
+  const bool mine = p.target != nullptr && ocol < NL;
+  float tgt[RQ];
+#pragma unroll
+  for (int u = 0; u < RQ; ++u) {
+    const int r = row0 + orow + 4 * u;
+    tgt[u] = (mine && r < p.batch) ? p.target[(int64_t)r * NL + ocol] : 0.f;
+  }
   FragF wa, wb;
   request(0, wa);  // the first layer's weights travel while the input is staged
   stage_rows4<RQ>(hs[0], p.x, row0, p.batch, p.width[0], tid);
@@ -548,19 +557,18 @@ __global__ __launch_bounds__(64 * NW, 1) void mlp_fwd4_kernel(MlpArgs p) {
     if (l + 1 < p.layers) layer(l + 1, wb, wa);
   }
   store(p.layers - 1);
-  if (p.target) {  // mse = sum((out - target)^2) / n (mse_op.mojo:17-20) and its gradient; the outputs of these rows are still in LDS
+  if (p.target) {  // mse = sum((out - target)^2) / n (mse_op.mojo:17-20) and its gradient, from the outputs still in registers
     __shared__ float red[NW];
-    const int L = p.layers, N = p.width[L], npad = (N + 15) & ~15;
-    const float* out = hs[L & 1];
-    const float two_over_n = 2.0f * p.inv_n;
     float acc = 0.f;
-    for (int e = tid; e < R * npad; e += 64 * NW) {
-      const int r = e / npad, c = e - r * npad;
-      if (row0 + r < p.batch && c < N) {
-        const int64_t at = (int64_t)(row0 + r) * N + c;
-        const float d = out[r * LD4 + c] - p.target[at];
-        acc += d * d;
-        if (p.dpred) p.dpred[at] = d * two_over_n;
+    if (mine) {
+#pragma unroll
+      for (int u = 0; u < RQ; ++u) {
+        const int r = row0 + orow + 4 * u;
+        if (r < p.batch) {
+          const float d = z[u] - tgt[u];
+          acc += d * d;
+          if (p.dpred) p.dpred[(int64_t)r * NL + ocol] = d * (2.0f * p.inv_n);
+        }
       }
     }
 #pragma unroll
@@ -573,10 +581,13 @@ __global__ __launch_bounds__(64 * NW, 1) void mlp_fwd4_kernel(MlpArgs p) {
       for (int w = 0; w < NW; ++w) sum += red[w];
       endia::store_shared(&p.loss_part[blockIdx.x], sum);
     }
-    if (endia::arrive_last(p.ticket, gridDim.x, &meet) && tid == 0) {
+    if (endia::arrive_last(p.ticket, gridDim.x, &meet) && wave == 0) {
+      // the groups' sums in a fixed order: lane i takes groups i, i + 64, .., then the lanes pairwise
       float sum = 0.f;
-      for (unsigned i = 0; i < gridDim.x; ++i) sum += endia::load_shared(&p.loss_part[i]);
-      p.loss[0] = sum * p.inv_n;
+      for (unsigned i = lane; i < gridDim.x; i += 64) sum += endia::load_shared(&p.loss_part[i]);
+#pragma unroll
+      for (int o = 32; o > 0; o >>= 1) sum += __shfl_down(sum, o);
+      if (lane == 0) p.loss[0] = sum * p.inv_n;
     }
   }
 }
@@ -660,6 +671,7 @@ __global__ __launch_bounds__(64 * NW, 1) void mlp_delta4_kernel(MlpArgs p) {
       const uint32_t base = (uint32_t)((c * N + 4 * s) * 4);
 #pragma unroll
       for (int T = 0; T < MAXW / 32; ++T) {
+        if (32 * T >= N) continue;
         const int n0 = 32 * T + 4 * s;
         if (vec) {
           const float4 w = buffer_load_f4(rs, (c < K && n0 < N) ? base + (uint32_t)(128 * T) : OOB_OFFSET);
