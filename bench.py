@@ -687,8 +687,8 @@ def main():
         captured = nd.capture(lambda: train_step(nd, mlp, opt, x, y))
         config["execution"] = "HIP graph replay of the eager step" + (
             "" if os.environ.get("ENDIA_SINE_PER_LAYER") else
-            "; nn.MLP(fused='model'): 4 launches a step (forward of all layers with the MSE loss and its gradient, cotangents of "
-            "all layers, all weight and bias gradients, optimizer over all 16 tensors)")
+            "; nn.MLP(fused='model'): 3 launches a step (forward of all layers with the MSE loss, its gradient and the cotangents "
+            "of all layers; all weight and bias gradients; optimizer over all 16 tensors)")
     L.call("endia_hip_gemm_timing_begin")
     t0 = time.perf_counter()
     for _ in range(args.steps):

@@ -99,6 +99,9 @@ SIGNATURES = {
     "endia_hip_mlp_fwd_mse": [POINTER(MlpDesc), _fp, POINTER(c_void_p), POINTER(c_void_p), _fp, POINTER(c_void_p), _fp, _fp],
     "endia_hip_mlp_bwd": [POINTER(MlpDesc), _fp, POINTER(c_void_p), POINTER(c_void_p), POINTER(c_void_p), POINTER(c_void_p),
                           POINTER(c_void_p), _fp],
+    "endia_hip_mlp_fwd_mse_delta": [POINTER(MlpDesc), _fp, POINTER(c_void_p), POINTER(c_void_p), _fp, POINTER(c_void_p),
+                                    POINTER(c_void_p), _fp, _fp],
+    "endia_hip_mlp_wgrad": [POINTER(MlpDesc), _fp, POINTER(c_void_p), POINTER(c_void_p), POINTER(c_void_p), POINTER(c_void_p)],
     "endia_hip_cgemm": [c_int32, c_int32, c_int32, c_int32, c_int64, c_int64, c_int64, _fp, c_int64, _fp, c_int64,
                         _fp, c_int64, c_int64, c_int64, c_int64, c_int64, c_int32, c_int32],
     "endia_hip_unary_fwd": [c_int32, c_int64, _fp, _fp, c_int32],

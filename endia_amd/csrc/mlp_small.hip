@@ -64,6 +64,7 @@ struct MlpArgs {
   float* loss_part;
   unsigned* ticket;
   float inv_n;
+  int chain;  // forward with the MSE loss: also run the chain of cotangents from the loss gradient (delta, dx as in the backward pass)
 };
 
 __device__ __forceinline__ float act_apply(int act, float z) {
@@ -428,170 +429,6 @@ __device__ __forceinline__ void stage_rows4(float* __restrict__ dst, const float
 // sit under the width tests, it waits for the NEXT layer's weights ahead of the current layer's MFMAs).
 __device__ __forceinline__ void wait_vm_all() { __builtin_amdgcn_s_waitcnt(0x0F70); }  // vmcnt(0), other counters untouched
 
-// Forward pass. A request of a wave must cover whole 128-byte lines to be delivered at the CU's full rate (four times
-// the rate of 64-byte pieces, measured), and rows of W run along the OUTPUT columns. So here a wave owns sixteen rows
-// of W (reduction indices 16 wave .. 16 wave + 15) and all columns: the sixteen blocks of an MFMA are sixteen column
-// quads (lane = column within a half of 64), the left operand is the same in all blocks, and a request reads 256
-// consecutive bytes of one row. The eight waves' partial sums (4 RQ x 128 floats each) meet in LDS, where thread t
-// finishes column t % 128 of row t / 128 (+ 4 per further row quad): bias, activation, LDS, and the global store one
-// layer later.
-struct FragF {
-  float v[16][2];  // [kk][half]: W[16 wave + kk][64 half + lane]
-  float bias;
-};
-
-// The MFMAs of one wave for one layer: its sixteen reduction indices times HALVES column halves, and the partial sums
-// to LDS. Within an active wave all sixteen indices are in order: the input's columns are zero up to the next multiple
-// of 16 and rows of W past the last read as zero.
-template <int RQ, int HALVES>
-__device__ __forceinline__ void slab_mfma(const float* __restrict__ in, const FragF& w, int wave, int lane, float (*part)[MAXW]) {
-  const int j = lane & 3;
-  floatx4 acc[RQ][HALVES];
-  float a[RQ][16];
-#pragma unroll
-  for (int rq = 0; rq < RQ; ++rq) {
-#pragma unroll
-    for (int h = 0; h < HALVES; ++h) acc[rq][h] = floatx4{0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-    for (int q = 0; q < 4; ++q) {
-      const float4 t = *reinterpret_cast<const float4*>(&in[(4 * rq + j) * LD4 + 16 * wave + 4 * q]);
-      a[rq][4 * q] = t.x; a[rq][4 * q + 1] = t.y; a[rq][4 * q + 2] = t.z; a[rq][4 * q + 3] = t.w;
-    }
-  }
-#pragma unroll
-  for (int kk = 0; kk < 16; ++kk)
-#pragma unroll
-    for (int h = 0; h < HALVES; ++h)
-#pragma unroll
-      for (int rq = 0; rq < RQ; ++rq) acc[rq][h] = __builtin_amdgcn_mfma_f32_4x4x1f32(a[rq][kk], w.v[kk][h], acc[rq][h], 0, 0, 0);
-#pragma unroll
-  for (int h = 0; h < HALVES; ++h)
-#pragma unroll
-    for (int rq = 0; rq < RQ; ++rq)
-#pragma unroll
-      for (int i = 0; i < 4; ++i) part[4 * rq + i][64 * h + lane] = acc[rq][h][i];
-}
-
-__global__ __launch_bounds__(64 * NW, 1) void mlp_fwd4_kernel(MlpArgs p) {
-  constexpr int RQ = 1;  // row quads per work-group (more were measured slower than the sixteen-row kernel at the batches where they would apply)
-  static_assert(NW * 16 == MAXW && 64 * NW == 4 * MAXW, "one wave per 16 reduction indices; one thread per output of a row quad");
-  constexpr int R = 4 * RQ;
-  __shared__ __attribute__((aligned(16))) float hs[2][R * LD4];
-  __shared__ float part[NW][R][MAXW];
-  __shared__ int meet;
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, j = lane & 3;
-  const int ocol = tid & (MAXW - 1), orow = tid >> 7;  // the outputs this thread finishes: column ocol of rows orow + 4 u
-  const int row0 = blockIdx.x * R;
-  auto request = [&](int l, FragF& f) {
-    const int K = p.width[l], N = p.width[l + 1];
-    const __amdgpu_buffer_rsrc_t rb = make_rsrc(p.b[l], (int64_t)N * 4);
-    f.bias = buffer_load_f1(rb, ocol < N ? (uint32_t)(ocol * 4) : OOB_OFFSET);
-    if (16 * wave >= K) return;
-    const __amdgpu_buffer_rsrc_t rs = make_rsrc(p.W[l], (int64_t)K * N * 4);  // rows past K lie past the end of the buffer
-#pragma unroll
-    for (int half = 0; half < 2; ++half)
-      if (64 * half < N) {
-        const uint32_t base = 64 * half + lane < N ? (uint32_t)((16 * wave * N + 64 * half + lane) * 4) : OOB_OFFSET;
-#pragma unroll
-        for (int kk = 0; kk < 16; ++kk) f.v[kk][half] = buffer_load_f1(rs, base + (uint32_t)(kk * N * 4));
-      }
-  };
-  float z[RQ];  // the outputs this thread finished in the last layer
-  auto store = [&](int l) {
-    const int N = p.width[l + 1];
-    if (ocol < N) {
-#pragma unroll
-      for (int u = 0; u < RQ; ++u) {
-        const int r = row0 + orow + 4 * u;
-        if (r < p.batch) p.h[l][(int64_t)r * N + ocol] = z[u];
-      }
-    }
-  };
-  auto layer = [&](int l, const FragF& cur, FragF& nxt) {
-    const int K = p.width[l], N = p.width[l + 1];
-    const bool last = l + 1 == p.layers;
-    wait_vm_all();
-    if (!last) request(l + 1, nxt);
-    if (l > 0) store(l - 1);
-    const float* in = hs[l & 1];
-    float* out = hs[(l & 1) ^ 1];
-    if (16 * wave < K) {
-      // (one straight run of MFMAs per case: a width test inside the run costs a branch and register copies per MFMA)
-      if (N > 64) slab_mfma<RQ, 2>(in, cur, wave, lane, part[wave]);
-      else slab_mfma<RQ, 1>(in, cur, wave, lane, part[wave]);
-    }
-    __syncthreads();
-    const int npad = (N + 15) & ~15, slabs = (K + 15) >> 4;
-    if (ocol < npad) {
-#pragma unroll
-      for (int u = 0; u < RQ; ++u) {
-        float pw[NW];
-#pragma unroll
-        for (int w = 0; w < NW; ++w) pw[w] = part[w][orow + 4 * u][ocol];  // (all eight reads travel together; idle waves' slots hold leftovers)
-        float v = cur.bias;
-#pragma unroll
-        for (int w = 0; w < NW; ++w) v += w < slabs ? pw[w] : 0.f;  // partial sums in the order of their reduction ranges
-        if (!last) v = act_apply(p.act, v);
-        if (ocol >= N) v = 0.f;  // columns up to the next multiple of 16 feed the next reduction as zeros
-        out[(orow + 4 * u) * LD4 + ocol] = v;
-        z[u] = v;
-      }
-    }
-    __syncthreads();
-  };
-  // the targets of this thread's outputs of the last layer, asked for now and needed at the very end
-  const int NL = p.width[p.layers];
-  const bool mine = p.target != nullptr && ocol < NL;
-  float tgt[RQ];
-#pragma unroll
-  for (int u = 0; u < RQ; ++u) {
-    const int r = row0 + orow + 4 * u;
-    tgt[u] = (mine && r < p.batch) ? p.target[(int64_t)r * NL + ocol] : 0.f;
-  }
-  FragF wa, wb;
-  request(0, wa);  // the first layer's weights travel while the input is staged
-  stage_rows4<RQ>(hs[0], p.x, row0, p.batch, p.width[0], tid);
-  __syncthreads();
-  for (int l = 0; l < p.layers; l += 2) {  // (two layers per round: the operands change places without copies)
-    layer(l, wa, wb);
-    if (l + 1 < p.layers) layer(l + 1, wb, wa);
-  }
-  store(p.layers - 1);
-  if (p.target) {  // mse = sum((out - target)^2) / n (mse_op.mojo:17-20) and its gradient, from the outputs still in registers
-    __shared__ float red[NW];
-    float acc = 0.f;
-    if (mine) {
-#pragma unroll
-      for (int u = 0; u < RQ; ++u) {
-        const int r = row0 + orow + 4 * u;
-        if (r < p.batch) {
-          const float d = z[u] - tgt[u];
-          acc += d * d;
-          if (p.dpred) p.dpred[(int64_t)r * NL + ocol] = d * (2.0f * p.inv_n);
-        }
-      }
-    }
-#pragma unroll
-    for (int o = 32; o > 0; o >>= 1) acc += __shfl_down(acc, o);
-    if (lane == 0) red[wave] = acc;
-    __syncthreads();
-    if (tid == 0) {
-      float sum = 0.f;
-#pragma unroll
-      for (int w = 0; w < NW; ++w) sum += red[w];
-      endia::store_shared(&p.loss_part[blockIdx.x], sum);
-    }
-    if (endia::arrive_last(p.ticket, gridDim.x, &meet) && wave == 0) {
-      // the groups' sums in a fixed order: lane i takes groups i, i + 64, .., then the lanes pairwise
-      float sum = 0.f;
-      for (unsigned i = lane; i < gridDim.x; i += 64) sum += endia::load_shared(&p.loss_part[i]);
-#pragma unroll
-      for (int o = 32; o > 0; o >>= 1) sum += __shfl_down(sum, o);
-      if (lane == 0) p.loss[0] = sum * p.inv_n;
-    }
-  }
-}
-
 // delta[layers - 1] holds the incoming cotangent (the last layer has no activation). For l = layers - 1 .. 1:
 // delta[l - 1] = (delta[l] W_l^T) * act'(h[l - 1]); finally dx = delta[0] W_0^T when asked for.
 //
@@ -644,18 +481,22 @@ __device__ __forceinline__ void rows_mfma(const float* __restrict__ in, const Fr
       for (int i = 0; i < 4; ++i) out[rq][pass][i] = sum_slices8(acc[rq][pass][i]);
 }
 
-__global__ __launch_bounds__(64 * NW, 1) void mlp_delta4_kernel(MlpArgs p) {
-  constexpr int RQ = 1;  // row quads per work-group, as in the forward kernel
-  constexpr int R = 4 * RQ;
-  __shared__ __attribute__((aligned(16))) float ds[2][R * LD4];
+// The chain of cotangents for the four-row kernels. `ds`: two LDS row blocks; ds[0] receives delta[layers - 1] of
+// this group's rows from stage() (zeros up to the next multiple of 32 columns), which runs after the first weights
+// have been asked for. LDS_ACTS: the stored activations come from `acts` (acts[l] = the input of layer l, LDS row
+// blocks left there by the forward pass of the same launch) instead of from memory.
+template <int RQ, bool LDS_ACTS, class Stage>
+__device__ __forceinline__ void delta_chain(const MlpArgs& p, float (*ds)[4 * RQ * LD4], const float (*acts)[4 * RQ * LD4], int row0, Stage stage) {
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, j = lane & 3, cq = (lane >> 4) & 1;
   const int s = ((lane >> 2) & 3) | ((lane >> 5) << 2);
   const int wrow = 4 * cq + j;                             // + 8 pass: the lane's rows of W within the wave's sixteen
   const int ocol = 16 * wave + 8 * (s >> 2) + wrow, orow = s & 3;  // the output this lane finishes, per row quad
-  const int row0 = blockIdx.x * R;
   const int L = p.layers;
   const int first = p.dx ? 0 : 1;  // lowest layer whose W^T is applied
-  if (L - 1 < first) return;
+  if (L - 1 < first) {
+    stage();
+    return;
+  }
   // (a wave is at work while its columns begin below the width rounded up to 32: the next reduction reads that far)
   auto active = [&](int K) { return 16 * wave < ((K + 31) & ~31); };
   auto request = [&](int l, FragD& f) {
@@ -683,11 +524,16 @@ __global__ __launch_bounds__(64 * NW, 1) void mlp_delta4_kernel(MlpArgs p) {
       }
     }
     // the outputs of the activation that produced this layer's input (none below the first layer)
-    const __amdgpu_buffer_rsrc_t rh = make_rsrc(l > 0 ? p.h[l - 1] : p.x, l > 0 ? (int64_t)p.batch * K * 4 : 0);
+    if (LDS_ACTS) {
 #pragma unroll
-    for (int rq = 0; rq < RQ; ++rq) {
-      const int r = row0 + 4 * rq + orow;
-      f.slope[rq] = buffer_load_f1(rh, (l > 0 && ocol < K && r < p.batch) ? (uint32_t)((r * K + ocol) * 4) : OOB_OFFSET);
+      for (int rq = 0; rq < RQ; ++rq) f.slope[rq] = l > 0 ? acts[l][(4 * rq + orow) * LD4 + ocol] : 1.f;
+    } else {
+      const __amdgpu_buffer_rsrc_t rh = make_rsrc(l > 0 ? p.h[l - 1] : p.x, l > 0 ? (int64_t)p.batch * K * 4 : 0);
+#pragma unroll
+      for (int rq = 0; rq < RQ; ++rq) {
+        const int r = row0 + 4 * rq + orow;
+        f.slope[rq] = buffer_load_f1(rh, (l > 0 && ocol < K && r < p.batch) ? (uint32_t)((r * K + ocol) * 4) : OOB_OFFSET);
+      }
     }
   };
   float d[RQ];  // the outputs this lane finished in the last layer
@@ -729,7 +575,7 @@ __global__ __launch_bounds__(64 * NW, 1) void mlp_delta4_kernel(MlpArgs p) {
   };
   FragD wa, wb;
   request(L - 1, wa);
-  stage_rows4<RQ>(ds[0], p.delta[L - 1], row0, p.batch, p.width[L], tid, 32);
+  stage();
   __syncthreads();
   int l = L - 1;
   for (; l >= first; l -= 2) {
@@ -737,6 +583,190 @@ __global__ __launch_bounds__(64 * NW, 1) void mlp_delta4_kernel(MlpArgs p) {
     if (l - 1 >= first) layer(l - 1, wb, wa);
   }
   store(first);
+}
+
+__global__ __launch_bounds__(64 * NW, 1) void mlp_delta4_kernel(MlpArgs p) {
+  constexpr int RQ = 1;  // row quads per work-group, as in the forward kernel
+  __shared__ __attribute__((aligned(16))) float ds[2][4 * RQ * LD4];
+  const int row0 = blockIdx.x * 4 * RQ;
+  delta_chain<RQ, false>(p, ds, nullptr, row0, [&]() { stage_rows4<RQ>(ds[0], p.delta[p.layers - 1], row0, p.batch, p.width[p.layers], threadIdx.x, 32); });
+}
+
+// Forward pass. A request of a wave must cover whole 128-byte lines to be delivered at the CU's full rate (four times
+// the rate of 64-byte pieces, measured), and rows of W run along the OUTPUT columns. So here a wave owns sixteen rows
+// of W (reduction indices 16 wave .. 16 wave + 15) and all columns: the sixteen blocks of an MFMA are sixteen column
+// quads (lane = column within a half of 64), the left operand is the same in all blocks, and a request reads 256
+// consecutive bytes of one row. The eight waves' partial sums (4 RQ x 128 floats each) meet in LDS, where thread t
+// finishes column t % 128 of row t / 128 (+ 4 per further row quad): bias, activation, LDS, and the global store one
+// layer later.
+struct FragF {
+  float v[16][2];  // [kk][half]: W[16 wave + kk][64 half + lane]
+  float bias;
+};
+
+// The MFMAs of one wave for one layer: its sixteen reduction indices times HALVES column halves, and the partial sums
+// to LDS. Within an active wave all sixteen indices are in order: the input's columns are zero up to the next multiple
+// of 16 and rows of W past the last read as zero.
+template <int RQ, int HALVES>
+__device__ __forceinline__ void slab_mfma(const float* __restrict__ in, const FragF& w, int wave, int lane, float (*part)[MAXW]) {
+  const int j = lane & 3;
+  floatx4 acc[RQ][HALVES];
+  float a[RQ][16];
+#pragma unroll
+  for (int rq = 0; rq < RQ; ++rq) {
+#pragma unroll
+    for (int h = 0; h < HALVES; ++h) acc[rq][h] = floatx4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+      const float4 t = *reinterpret_cast<const float4*>(&in[(4 * rq + j) * LD4 + 16 * wave + 4 * q]);
+      a[rq][4 * q] = t.x; a[rq][4 * q + 1] = t.y; a[rq][4 * q + 2] = t.z; a[rq][4 * q + 3] = t.w;
+    }
+  }
+#pragma unroll
+  for (int kk = 0; kk < 16; ++kk)
+#pragma unroll
+    for (int h = 0; h < HALVES; ++h)
+#pragma unroll
+      for (int rq = 0; rq < RQ; ++rq) acc[rq][h] = __builtin_amdgcn_mfma_f32_4x4x1f32(a[rq][kk], w.v[kk][h], acc[rq][h], 0, 0, 0);
+#pragma unroll
+  for (int h = 0; h < HALVES; ++h)
+#pragma unroll
+    for (int rq = 0; rq < RQ; ++rq)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) part[4 * rq + i][64 * h + lane] = acc[rq][h][i];
+}
+
+__global__ __launch_bounds__(64 * NW, 1) void mlp_fwd4_kernel(MlpArgs p) {
+  constexpr int RQ = 1;  // row quads per work-group (more were measured slower than the sixteen-row kernel at the batches where they would apply)
+  static_assert(NW * 16 == MAXW && 64 * NW == 4 * MAXW, "one wave per 16 reduction indices; one thread per output of a row quad");
+  constexpr int R = 4 * RQ;
+  // every layer's input stays in LDS: the next layer reads it, and the chain of cotangents (when this launch runs it) takes the
+  // activations' slopes from it
+  __shared__ __attribute__((aligned(16))) float acts[ENDIA_MLP_MAX_LAYERS + 1][R * LD4];
+  __shared__ __attribute__((aligned(16))) float ds[2][R * LD4];
+  __shared__ float part[NW][R][MAXW];
+  __shared__ int meet;
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, j = lane & 3;
+  const int ocol = tid & (MAXW - 1), orow = tid >> 7;  // the outputs this thread finishes: column ocol of rows orow + 4 u
+  const int row0 = blockIdx.x * R;
+  auto request = [&](int l, FragF& f) {
+    const int K = p.width[l], N = p.width[l + 1];
+    const __amdgpu_buffer_rsrc_t rb = make_rsrc(p.b[l], (int64_t)N * 4);
+    f.bias = buffer_load_f1(rb, ocol < N ? (uint32_t)(ocol * 4) : OOB_OFFSET);
+    if (16 * wave >= K) return;
+    const __amdgpu_buffer_rsrc_t rs = make_rsrc(p.W[l], (int64_t)K * N * 4);  // rows past K lie past the end of the buffer
+#pragma unroll
+    for (int half = 0; half < 2; ++half)
+      if (64 * half < N) {
+        const uint32_t base = 64 * half + lane < N ? (uint32_t)((16 * wave * N + 64 * half + lane) * 4) : OOB_OFFSET;
+#pragma unroll
+        for (int kk = 0; kk < 16; ++kk) f.v[kk][half] = buffer_load_f1(rs, base + (uint32_t)(kk * N * 4));
+      }
+  };
+  float z[RQ];  // the outputs this thread finished in the last layer
+  auto store = [&](int l) {
+    const int N = p.width[l + 1];
+    if (ocol < N) {
+#pragma unroll
+      for (int u = 0; u < RQ; ++u) {
+        const int r = row0 + orow + 4 * u;
+        if (r < p.batch) p.h[l][(int64_t)r * N + ocol] = z[u];
+      }
+    }
+  };
+  auto layer = [&](int l, const FragF& cur, FragF& nxt) {
+    const int K = p.width[l], N = p.width[l + 1];
+    const bool last = l + 1 == p.layers;
+    wait_vm_all();
+    if (!last) request(l + 1, nxt);
+    if (l > 0) store(l - 1);
+    const float* in = acts[l];
+    float* out = acts[l + 1];
+    if (16 * wave < K) {
+      // (one straight run of MFMAs per case: a width test inside the run costs a branch and register copies per MFMA)
+      if (N > 64) slab_mfma<RQ, 2>(in, cur, wave, lane, part[wave]);
+      else slab_mfma<RQ, 1>(in, cur, wave, lane, part[wave]);
+    }
+    __syncthreads();
+    const int npad = (N + 15) & ~15, slabs = (K + 15) >> 4;
+    if (ocol < npad) {
+#pragma unroll
+      for (int u = 0; u < RQ; ++u) {
+        float pw[NW];
+#pragma unroll
+        for (int w = 0; w < NW; ++w) pw[w] = part[w][orow + 4 * u][ocol];  // (all eight reads travel together; idle waves' slots hold leftovers)
+        float v = cur.bias;
+#pragma unroll
+        for (int w = 0; w < NW; ++w) v += w < slabs ? pw[w] : 0.f;  // partial sums in the order of their reduction ranges
+        if (!last) v = act_apply(p.act, v);
+        if (ocol >= N) v = 0.f;  // columns up to the next multiple of 16 feed the next reduction as zeros
+        out[(orow + 4 * u) * LD4 + ocol] = v;
+        z[u] = v;
+      }
+    }
+    __syncthreads();
+  };
+  // the targets of this thread's outputs of the last layer, asked for now and needed at the very end
+  const int NL = p.width[p.layers];
+  const bool mine = p.target != nullptr && ocol < NL;
+  float tgt[RQ];
+#pragma unroll
+  for (int u = 0; u < RQ; ++u) {
+    const int r = row0 + orow + 4 * u;
+    tgt[u] = (mine && r < p.batch) ? p.target[(int64_t)r * NL + ocol] : 0.f;
+  }
+  FragF wa, wb;
+  request(0, wa);  // the first layer's weights travel while the input is staged
+  stage_rows4<RQ>(acts[0], p.x, row0, p.batch, p.width[0], tid);
+  __syncthreads();
+  for (int l = 0; l < p.layers; l += 2) {  // (two layers per round: the operands change places without copies)
+    layer(l, wa, wb);
+    if (l + 1 < p.layers) layer(l + 1, wb, wa);
+  }
+  store(p.layers - 1);
+  if (p.target) {  // mse = sum((out - target)^2) / n (mse_op.mojo:17-20) and its gradient, from the outputs still in registers
+    __shared__ float red[NW];
+    float acc = 0.f, dp[RQ];
+#pragma unroll
+    for (int u = 0; u < RQ; ++u) {
+      const int r = row0 + orow + 4 * u;
+      dp[u] = 0.f;
+      if (mine && r < p.batch) {
+        const float d = z[u] - tgt[u];
+        acc += d * d;
+        dp[u] = d * (2.0f * p.inv_n);
+        if (p.dpred) p.dpred[(int64_t)r * NL + ocol] = dp[u];
+      }
+    }
+    if (p.chain) {
+      // the cotangents of all layers for these rows, from the loss gradient at hand: the backward pass is left with the
+      // weight gradients (rows are independent through the whole chain; nobody waits for another group)
+      delta_chain<RQ, true>(p, ds, acts, row0, [&]() {
+        if (ocol < ((NL + 31) & ~31)) {
+#pragma unroll
+          for (int u = 0; u < RQ; ++u) ds[0][(orow + 4 * u) * LD4 + ocol] = dp[u];
+        }
+      });
+    }
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) acc += __shfl_down(acc, o);
+    if (lane == 0) red[wave] = acc;
+    __syncthreads();
+    if (tid == 0) {
+      float sum = 0.f;
+#pragma unroll
+      for (int w = 0; w < NW; ++w) sum += red[w];
+      endia::store_shared(&p.loss_part[blockIdx.x], sum);
+    }
+    if (endia::arrive_last(p.ticket, gridDim.x, &meet) && wave == 0) {
+      // the groups' sums in a fixed order: lane i takes groups i, i + 64, .., then the lanes pairwise
+      float sum = 0.f;
+      for (unsigned i = lane; i < gridDim.x; i += 64) sum += endia::load_shared(&p.loss_part[i]);
+#pragma unroll
+      for (int o = 32; o > 0; o >>= 1) sum += __shfl_down(sum, o);
+      if (lane == 0) p.loss[0] = sum * p.inv_n;
+    }
+  }
 }
 
 // dW_l = h_{l-1}^T delta_l and db_l = 1^T delta_l for ALL layers in one launch: a work-group per 32 x 32 tile of a
@@ -867,20 +897,24 @@ extern "C" int32_t endia_hip_mlp_fwd(const endia_hip_mlp_desc* desc, const float
   return ENDIA_HIP_OK;
 }
 
-extern "C" int32_t endia_hip_mlp_fwd_mse(const endia_hip_mlp_desc* desc, const float* x, const float* const* W, const float* const* b,
-                                         const float* target, float* const* h, float* dpred, float* loss) {
+namespace {
+
+// The forward launch with the MSE loss on top; with `delta` also the chain of cotangents from the loss gradient.
+int32_t fwd_mse(const char* who, const endia_hip_mlp_desc* desc, const float* x, const float* const* W, const float* const* b,
+                const float* target, float* const* h, float* dpred, float* loss, float* const* delta, float* dx) {
   ENDIA_REQUIRE_INIT();
   MlpArgs a;
-  int32_t rc = fill_args(a, desc, "endia_hip_mlp_fwd_mse");
+  int32_t rc = fill_args(a, desc, who);
   if (rc) return rc;
-  ENDIA_CHECK_ARG(loss != nullptr, "endia_hip_mlp_fwd_mse: loss is null");
+  ENDIA_CHECK_ARG(loss != nullptr, "%s: loss is null", who);
   if (a.batch == 0) return endia_hip_fill(loss, 1, 0.f);
-  ENDIA_CHECK_ARG(x && W && b && h && target, "endia_hip_mlp_fwd_mse: null argument");
+  ENDIA_CHECK_ARG(x && W && b && h && target, "%s: null argument", who);
   for (int l = 0; l < a.layers; ++l) {
-    ENDIA_CHECK_ARG(W[l] && b[l] && h[l], "endia_hip_mlp_fwd_mse: null pointer for layer %d", l);
+    ENDIA_CHECK_ARG(W[l] && b[l] && h[l] && (!delta || delta[l]), "%s: null pointer for layer %d", who, l);
     a.W[l] = W[l];
     a.b[l] = b[l];
     a.h[l] = h[l];
+    if (delta) a.delta[l] = delta[l];
   }
   a.x = x;
   const int64_t groups = fwd_groups(a);
@@ -890,28 +924,51 @@ extern "C" int32_t endia_hip_mlp_fwd_mse(const endia_hip_mlp_desc* desc, const f
   } part;
   if ((rc = endia_hip_malloc(groups * 4, &part.p))) return rc;
   a.target = target;
-  a.dpred = dpred;
+  a.dpred = delta ? delta[a.layers - 1] : dpred;
   a.loss = loss;
   a.loss_part = static_cast<float*>(part.p);
   a.ticket = ctx().tickets + (kTicketCount - 1);
   a.inv_n = 1.0f / (float)((int64_t)a.batch * a.width[a.layers]);
+  a.dx = delta ? dx : nullptr;
+  // the four-row kernel runs the chain itself; beyond its batches the chain is the launch it always was
+  a.chain = delta != nullptr && a.batch <= kFourRowBatch;
   launch_fwd(a, ctx().stream);
   ENDIA_LAUNCH_CHECK();
+  if (delta && !a.chain && (a.layers > 1 || dx)) {
+    launch_delta(a, ctx().stream);
+    ENDIA_LAUNCH_CHECK();
+  }
   return ENDIA_HIP_OK;
 }
 
-extern "C" int32_t endia_hip_mlp_bwd(const endia_hip_mlp_desc* desc, const float* x, const float* const* W, const float* const* h,
-                                     float* const* delta, float* const* dW, float* const* db, float* dx) {
+}  // namespace
+
+extern "C" int32_t endia_hip_mlp_fwd_mse(const endia_hip_mlp_desc* desc, const float* x, const float* const* W, const float* const* b,
+                                         const float* target, float* const* h, float* dpred, float* loss) {
+  return fwd_mse("endia_hip_mlp_fwd_mse", desc, x, W, b, target, h, dpred, loss, nullptr, nullptr);
+}
+
+extern "C" int32_t endia_hip_mlp_fwd_mse_delta(const endia_hip_mlp_desc* desc, const float* x, const float* const* W,
+                                               const float* const* b, const float* target, float* const* h, float* const* delta,
+                                               float* loss, float* dx) {
+  ENDIA_CHECK_ARG(delta != nullptr, "endia_hip_mlp_fwd_mse_delta: delta is null");
+  return fwd_mse("endia_hip_mlp_fwd_mse_delta", desc, x, W, b, target, h, nullptr, loss, delta, dx);
+}
+
+namespace {
+
+int32_t bwd(const char* who, const endia_hip_mlp_desc* desc, const float* x, const float* const* W, const float* const* h,
+            float* const* delta, float* const* dW, float* const* db, float* dx, bool chain) {
   ENDIA_REQUIRE_INIT();
   MlpArgs a;
-  int32_t rc = fill_args(a, desc, "endia_hip_mlp_bwd");
+  int32_t rc = fill_args(a, desc, who);
   if (rc) return rc;
   if (a.batch == 0) return ENDIA_HIP_OK;
-  ENDIA_CHECK_ARG(x && W && h && delta && dW && db, "endia_hip_mlp_bwd: null argument");
+  ENDIA_CHECK_ARG(x && (W || !chain) && h && delta && dW && db, "%s: null argument", who);
   int blocks = 0;
   for (int l = 0; l < a.layers; ++l) {
-    ENDIA_CHECK_ARG(W[l] && delta[l] && (l + 1 == a.layers || h[l]), "endia_hip_mlp_bwd: null pointer for layer %d", l);
-    a.W[l] = W[l];
+    ENDIA_CHECK_ARG((!chain || W[l]) && delta[l] && (l + 1 == a.layers || h[l]), "%s: null pointer for layer %d", who, l);
+    a.W[l] = chain ? W[l] : nullptr;
     a.h[l] = const_cast<float*>(h[l]);
     a.delta[l] = delta[l];
     a.dW[l] = dW[l];
@@ -923,7 +980,7 @@ extern "C" int32_t endia_hip_mlp_bwd(const endia_hip_mlp_desc* desc, const float
   a.x = x;
   a.dx = dx;
   hipStream_t s = ctx().stream;
-  if (a.layers > 1 || dx) {
+  if (chain && (a.layers > 1 || dx)) {
     launch_delta(a, s);
     ENDIA_LAUNCH_CHECK();
   }
@@ -932,3 +989,14 @@ extern "C" int32_t endia_hip_mlp_bwd(const endia_hip_mlp_desc* desc, const float
   return ENDIA_HIP_OK;
 }
 
+}  // namespace
+
+extern "C" int32_t endia_hip_mlp_bwd(const endia_hip_mlp_desc* desc, const float* x, const float* const* W, const float* const* h,
+                                     float* const* delta, float* const* dW, float* const* db, float* dx) {
+  return bwd("endia_hip_mlp_bwd", desc, x, W, h, delta, dW, db, dx, true);
+}
+
+extern "C" int32_t endia_hip_mlp_wgrad(const endia_hip_mlp_desc* desc, const float* x, const float* const* h,
+                                       const float* const* delta, float* const* dW, float* const* db) {
+  return bwd("endia_hip_mlp_wgrad", desc, x, nullptr, h, const_cast<float* const*>(delta), dW, db, nullptr, false);
+}

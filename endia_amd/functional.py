@@ -1469,10 +1469,11 @@ def mlp_forward(x, weights, biases, act=None):
 
 def mlp_mse_loss(x, target, weights, biases, act=None):
     """mse(mlp_forward(x, weights, biases, act), target) for a small model (see mlp_forward) with the loss evaluated by the
-    forward launch itself (endia_hip_mlp_fwd_mse: the outputs of a work-group's rows are still in LDS when the last
-    layer is done, so the squared differences and the loss gradient 2 (out - target) / n cost no launch of their own).
-    backward() then runs the two launches of endia_hip_mlp_bwd on that stored gradient: with the optimizer, 4 launches
-    for a training step of the reference's script (mlp_imp.mojo:56-68). Anything the fused launch does not cover (a model
+    forward launch itself (endia_hip_mlp_fwd_mse_delta: the outputs of a work-group's rows are still on chip when the
+    last layer is done, so the squared differences, the loss gradient 2 (out - target) / n and, since every row is
+    independent through the whole chain, the cotangents of all layers cost no launch of their own). backward() then is
+    the one launch of endia_hip_mlp_wgrad: with the optimizer, 3 launches for a training step of the reference's script
+    (mlp_imp.mojo:56-68). A cotangent other than the seed runs the chain again from the scaled loss gradient. Anything the fused launch does not cover (a model
     that is not small, a target that needs a gradient, complex operands) is mse(mlp_forward(...)); a second-order pass
     fails as it does for mlp_forward. Returns the loss, shape [1]."""
     import ctypes
@@ -1490,26 +1491,39 @@ def mlp_mse_loss(x, target, weights, biases, act=None):
     xs, ts = contiguous(x), contiguous(target)
     Ws, bs_ = [contiguous(w) for w in weights], [contiguous(b) for b in biases]
     hs = [Array.empty([B, widths[i + 1]]) for i in range(Lyr)]
-    dpred = Array.empty([B, widths[-1]])
     loss = Array.empty([1])
     desc = L.MlpDesc()
     desc.layers, desc.act, desc.batch = Lyr, _ACT[act], B
     desc.widths[:Lyr + 1] = widths
     ptrs = lambda arrs: (ctypes.c_void_p * Lyr)(*[a.data_ptr() if a is not None else None for a in arrs])
-    L.call("endia_hip_mlp_fwd_mse", ctypes.byref(desc), xs.data_ptr(), ptrs(Ws), ptrs(bs_), ts.data_ptr(), ptrs(hs), dpred.data_ptr(),
-           loss.data_ptr())
+    # With something to differentiate, the forward launch goes on to the cotangents of all layers for the loss gradient
+    # (rows are independent through the whole chain), and backward() is left with the weight gradients.
+    wants = [a._requires_grad for a in [x] + list(weights) + list(biases)]
+    deltas = [Array.empty([B, widths[i + 1]]) for i in range(Lyr)]
+    dx0 = Array.empty([B, widths[0]]) if wants[0] else None
+    if any(wants):
+        L.call("endia_hip_mlp_fwd_mse_delta", ctypes.byref(desc), xs.data_ptr(), ptrs(Ws), ptrs(bs_), ts.data_ptr(), ptrs(hs), ptrs(deltas),
+               loss.data_ptr(), dx0.data_ptr() if dx0 is not None else None)
+    else:
+        L.call("endia_hip_mlp_fwd_mse", ctypes.byref(desc), xs.data_ptr(), ptrs(Ws), ptrs(bs_), ts.data_ptr(), ptrs(hs), deltas[-1].data_ptr(),
+               loss.data_ptr())
 
     def vjp(primals, grad, out_):
         from .autograd.functional import building_graph
         if building_graph():
             raise NotImplementedError("mlp_mse_loss is a first-order op; use mse(model.forward(x), target) with fused=True for higher-order passes")
-        last = dpred if _holds_seed(grad) else mul(dpred, grad)  # (a cotangent other than the seed scales the stored gradient)
-        deltas = [Array.empty([B, widths[i + 1]]) for i in range(Lyr - 1)] + [contiguous(last)]
         pW, pb = primals[2:2 + Lyr], primals[2 + Lyr:]
         dW = [Array.empty([widths[i], widths[i + 1]]) if pW[i]._requires_grad else None for i in range(Lyr)]
         db = [Array.empty([1, widths[i + 1]]) if pb[i]._requires_grad else None for i in range(Lyr)]  # kept axis, like Expand.vjp
-        dx = Array.empty([B, widths[0]]) if primals[0]._requires_grad else None
-        L.call("endia_hip_mlp_bwd", ctypes.byref(desc), xs.data_ptr(), ptrs(Ws), ptrs(hs), ptrs(deltas), ptrs(dW), ptrs(db),
+        want_dx = primals[0]._requires_grad
+        if _holds_seed(grad) and any(wants) and (dx0 is not None or not want_dx):
+            L.call("endia_hip_mlp_wgrad", ctypes.byref(desc), xs.data_ptr(), ptrs(hs), ptrs(deltas), ptrs(dW), ptrs(db))
+            return [dx0 if want_dx else None, None] + dW + db
+        # a cotangent other than the seed scales the stored loss gradient; the chain is run again from there
+        last = deltas[-1] if _holds_seed(grad) else mul(deltas[-1], grad)
+        again = [Array.empty([B, widths[i + 1]]) for i in range(Lyr - 1)] + [contiguous(last)]
+        dx = Array.empty([B, widths[0]]) if want_dx else None
+        L.call("endia_hip_mlp_bwd", ctypes.byref(desc), xs.data_ptr(), ptrs(Ws), ptrs(hs), ptrs(again), ptrs(dW), ptrs(db),
                dx.data_ptr() if dx is not None else None)
         return [dx, None] + dW + db
 

@@ -232,6 +232,18 @@ ENDIA_API int32_t endia_hip_mlp_fwd_mse(const endia_hip_mlp_desc* desc, const fl
                               const float* const* b, const float* target, float* const* h, float* dpred, float* loss);
 ENDIA_API int32_t endia_hip_mlp_bwd(const endia_hip_mlp_desc* desc, const float* x, const float* const* W, const float* const* h,
                           float* const* delta, float* const* dW, float* const* db, float* dx);
+/* The training step of mlp_imp.mojo:56-66 (forward, mse, backward) split so that the backward pass is one launch:
+ * endia_hip_mlp_fwd_mse_delta is endia_hip_mlp_fwd_mse that goes on, in the same launch for batches of up to 1024 rows,
+ * to the cotangents of ALL layers for the loss gradient 2 (h[layers-1] - target) / n (every row of the batch is
+ * independent through the whole chain): delta[l] [batch, widths[l+1]], none null, and dx [batch, widths[0]] when not
+ * null, exactly what endia_hip_mlp_bwd leaves there when its delta[layers-1] is that loss gradient.
+ * endia_hip_mlp_wgrad is the rest of endia_hip_mlp_bwd: dW[l] = h[l-1]^T delta[l] (h[-1] = x) and db[l] = the column
+ * sums of delta[l], for the layers whose pointers are not null. */
+ENDIA_API int32_t endia_hip_mlp_fwd_mse_delta(const endia_hip_mlp_desc* desc, const float* x, const float* const* W,
+                                    const float* const* b, const float* target, float* const* h, float* const* delta,
+                                    float* loss, float* dx);
+ENDIA_API int32_t endia_hip_mlp_wgrad(const endia_hip_mlp_desc* desc, const float* x, const float* const* h,
+                            const float* const* delta, float* const* dW, float* const* db);
 
 /* ---- complex64 GEMM: the complex branch of matmul_fwd (matmul_op.mojo:201-238). Interleaved
  *      operands; lda/ldb/ldc and strides count complex elements. conjA/conjB conjugate the operand
