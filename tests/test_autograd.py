@@ -1215,6 +1215,62 @@ def test_whole_model_mse_loss_op(nd):
     assert_close(wide.mse_loss(x, t).to_numpy(), nd.mse(wide.forward(x), t).to_numpy(), tol=1e-6, what="wide model")
 
 
+def test_whole_model_forward_with_cotangents_entry_points(nd):
+    """endia_hip_mlp_fwd_mse_delta + endia_hip_mlp_wgrad through the C ABI against endia_hip_mlp_fwd_mse +
+    endia_hip_mlp_bwd: the same loss, activations, cotangents of every layer, dx, dW and db, bit for bit (the chain is
+    the same arithmetic whether it runs in the forward launch or in its own), on both sides of the 1024-row switch, with
+    and without dx, with gradients that are not asked for, and twice in a row."""
+    import ctypes
+    from endia_amd import _lib as L
+    from endia_amd._array import Array
+    rng = np.random.default_rng(77)
+    act_code = {None: L.OP_IDENTITY, "relu": L.OP_RELU, "tanh": L.OP_TANH}
+    for widths, batch, act, want_dx in [([1, 32, 64, 128, 128, 128, 64, 32, 1], 128, "relu", False), ([7, 50, 3, 128, 20], 37, "tanh", True),
+                                        ([128, 128], 16, None, True), ([5, 17], 1, "relu", False), ([33, 128, 65, 12], 1024, "tanh", True),
+                                        ([33, 128, 65, 12], 1500, "relu", True), ([6, 9, 4], 3, "relu", True)]:
+        Lyr = len(widths) - 1
+        W = [nd.array((rng.standard_normal((widths[i], widths[i + 1])) / np.sqrt(widths[i])).astype(np.float32)) for i in range(Lyr)]
+        b = [nd.array((0.2 * rng.standard_normal(widths[i + 1])).astype(np.float32)) for i in range(Lyr)]
+        x = nd.array(rng.standard_normal((batch, widths[0])).astype(np.float32))
+        t = nd.array(rng.standard_normal((batch, widths[-1])).astype(np.float32))
+        desc = L.MlpDesc()
+        desc.layers, desc.act, desc.batch = Lyr, act_code[act], batch
+        desc.widths[:Lyr + 1] = widths
+        ptrs = lambda arrs: (ctypes.c_void_p * Lyr)(*[a.data_ptr() if a is not None else None for a in arrs])
+        new = lambda shape: Array.empty(list(shape))
+
+        def two_calls():
+            h = [new([batch, widths[i + 1]]) for i in range(Lyr)]
+            delta = [new([batch, widths[i + 1]]) for i in range(Lyr)]
+            dW = [new([widths[i], widths[i + 1]]) if i != 1 else None for i in range(Lyr)]  # the second dW is not asked for
+            db = [new([widths[i + 1]]) for i in range(Lyr)]
+            dx, loss = (new([batch, widths[0]]) if want_dx else None), new([1])
+            L.call("endia_hip_mlp_fwd_mse", ctypes.byref(desc), x.data_ptr(), ptrs(W), ptrs(b), t.data_ptr(), ptrs(h), delta[-1].data_ptr(), loss.data_ptr())
+            L.call("endia_hip_mlp_bwd", ctypes.byref(desc), x.data_ptr(), ptrs(W), ptrs(h), ptrs(delta), ptrs(dW), ptrs(db), dx.data_ptr() if dx else None)
+            return [loss] + h + delta + [a for a in dW if a is not None] + db + ([dx] if dx else [])
+
+        def fused():
+            h = [new([batch, widths[i + 1]]) for i in range(Lyr)]
+            delta = [new([batch, widths[i + 1]]) for i in range(Lyr)]
+            dW = [new([widths[i], widths[i + 1]]) if i != 1 else None for i in range(Lyr)]
+            db = [new([widths[i + 1]]) for i in range(Lyr)]
+            dx, loss = (new([batch, widths[0]]) if want_dx else None), new([1])
+            L.call("endia_hip_mlp_fwd_mse_delta", ctypes.byref(desc), x.data_ptr(), ptrs(W), ptrs(b), t.data_ptr(), ptrs(h), ptrs(delta), loss.data_ptr(),
+                   dx.data_ptr() if dx else None)
+            L.call("endia_hip_mlp_wgrad", ctypes.byref(desc), x.data_ptr(), ptrs(h), ptrs(delta), ptrs(dW), ptrs(db))
+            return [loss] + h + delta + [a for a in dW if a is not None] + db + ([dx] if dx else [])
+
+        ref = [a.to_numpy() for a in two_calls()]
+        for _ in range(2):
+            got = [a.to_numpy() for a in fused()]
+            assert len(got) == len(ref)
+            for k, (g, r) in enumerate(zip(got, ref)):
+                np.testing.assert_array_equal(g, r, err_msg="widths %s batch %d %s: tensor %d" % (widths, batch, act, k))
+    # arguments the entry points refuse
+    with pytest.raises(Exception):
+        L.call("endia_hip_mlp_fwd_mse_delta", ctypes.byref(desc), x.data_ptr(), ptrs(W), ptrs(b), t.data_ptr(), ptrs(W), None, x.data_ptr(), None)
+
+
 def test_whole_model_mlp_op(nd):
     """functional.mlp_forward through the C ABI's endia_hip_mlp_fwd / endia_hip_mlp_bwd: the same numbers as the
     per-layer path for ragged widths and batches (rows and columns that do not fill an MFMA block), batches on both
