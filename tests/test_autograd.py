@@ -1271,6 +1271,61 @@ def test_whole_model_forward_with_cotangents_entry_points(nd):
         L.call("endia_hip_mlp_fwd_mse_delta", ctypes.byref(desc), x.data_ptr(), ptrs(W), ptrs(b), t.data_ptr(), ptrs(W), None, x.data_ptr(), None)
 
 
+def test_whole_model_entry_points_unaligned_and_deep(nd):
+    """The whole-model entry points against float64 numpy (the chain rule written out) where the per-layer comparison
+    does not reach: weight matrices that start 4 bytes off a 16-byte boundary (the cotangent chain then reads W element
+    by element), and the deepest model the entry points take (16 layers: every LDS row block of the forward launch)."""
+    import ctypes
+    from endia_amd import _lib as L
+    from endia_amd._array import Array
+    rng = np.random.default_rng(78)
+    for widths, batch, act, off in [([12, 40, 128, 24, 8], 50, "tanh", 1), ([12, 40, 128, 24, 8], 1100, "relu", 1),
+                                    ([8] * 17, 10, "tanh", 0), ([128] * 17, 9, "relu", 0)]:
+        Lyr = len(widths) - 1
+        Wn = [(rng.standard_normal((widths[i], widths[i + 1])) / np.sqrt(widths[i])).astype(np.float32) for i in range(Lyr)]
+        bn = [(0.2 * rng.standard_normal(widths[i + 1])).astype(np.float32) for i in range(Lyr)]
+        xn = rng.standard_normal((batch, widths[0])).astype(np.float32)
+        tn = rng.standard_normal((batch, widths[-1])).astype(np.float32)
+        # weights inside larger buffers, `off` floats past their start
+        Wbuf = [nd.array(np.concatenate([np.zeros(off, np.float32), w.reshape(-1)])) for w in Wn]
+        Wp = [wb.data_ptr() + 4 * off for wb in Wbuf]
+        b = [nd.array(v) for v in bn]
+        x, t = nd.array(xn), nd.array(tn)
+        desc = L.MlpDesc()
+        desc.layers, desc.act, desc.batch = Lyr, {"relu": L.OP_RELU, "tanh": L.OP_TANH}[act], batch
+        desc.widths[:Lyr + 1] = widths
+        vp = lambda ps: (ctypes.c_void_p * Lyr)(*ps)
+        ptrs = lambda arrs: vp([a.data_ptr() for a in arrs])
+        h = [Array.empty([batch, widths[i + 1]]) for i in range(Lyr)]
+        delta = [Array.empty([batch, widths[i + 1]]) for i in range(Lyr)]
+        dW = [Array.empty([widths[i], widths[i + 1]]) for i in range(Lyr)]
+        db = [Array.empty([widths[i + 1]]) for i in range(Lyr)]
+        dx, loss = Array.empty([batch, widths[0]]), Array.empty([1])
+        L.call("endia_hip_mlp_fwd_mse_delta", ctypes.byref(desc), x.data_ptr(), vp(Wp), ptrs(b), t.data_ptr(), ptrs(h), ptrs(delta), loss.data_ptr(),
+               dx.data_ptr())
+        L.call("endia_hip_mlp_wgrad", ctypes.byref(desc), x.data_ptr(), ptrs(h), ptrs(delta), ptrs(dW), ptrs(db))
+        # float64: h_l = act(h_{l-1} W_l + b_l) (none after the last layer), loss = mean((h_L - t)^2)
+        f = (lambda z: np.maximum(z, 0)) if act == "relu" else np.tanh
+        slope = (lambda o: (o > 0).astype(np.float64)) if act == "relu" else (lambda o: 1 - o * o)
+        hs = [xn.astype(np.float64)]
+        for i in range(Lyr):
+            z = hs[-1] @ Wn[i].astype(np.float64) + bn[i]
+            hs.append(z if i == Lyr - 1 else f(z))
+        d = 2 * (hs[-1] - tn) / tn.size
+        what = "widths %s batch %d %s offset %d: " % (widths[:5], batch, act, off)
+        assert_close(loss.to_numpy(), [np.mean((hs[-1] - tn) ** 2)], tol=1e-5, what=what + "loss")
+        for i in reversed(range(Lyr)):
+            assert_close(delta[i].to_numpy(), d, tol=2e-5, mean_tol=1e-3, what=what + "delta %d" % i)
+            assert_close(dW[i].to_numpy(), hs[i].T @ d, tol=2e-5, mean_tol=1e-3, what=what + "dW %d" % i)
+            assert_close(db[i].to_numpy(), d.sum(0), tol=2e-5, mean_tol=1e-3, what=what + "db %d" % i)
+            d = d @ Wn[i].astype(np.float64).T
+            if i > 0:
+                d = d * slope(hs[i])
+        assert_close(dx.to_numpy(), d, tol=2e-5, mean_tol=1e-3, what=what + "dx")
+        for i in range(Lyr):
+            assert_close(h[i].to_numpy(), hs[i + 1], tol=1e-5, what=what + "h %d" % i)
+
+
 def test_whole_model_mlp_op(nd):
     """functional.mlp_forward through the C ABI's endia_hip_mlp_fwd / endia_hip_mlp_bwd: the same numbers as the
     per-layer path for ragged widths and batches (rows and columns that do not fill an MFMA block), batches on both
