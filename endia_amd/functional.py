@@ -1053,6 +1053,12 @@ def _gemm_operand(x):
     return d
 
 
+def _is_transposed_matrix(x):
+    """x is a real 2-D transposed view of a row-major matrix (unit ROW stride), larger than a vector."""
+    return (x.ndim() == 2 and not x.is_complex_ and x._shape[0] > 1 and x._shape[1] > 1
+            and x._strides[0] == 1 and x._strides[1] >= x._shape[0])
+
+
 def matmul(a, b, vjp_rule=None, _ca=0, _cb=0):
     """Batched matrix product with broadcast batch axes (matmul_op.mojo:36-90,309-346).
 
@@ -1109,8 +1115,15 @@ def matmul(a, b, vjp_rule=None, _ca=0, _cb=0):
             lhs = matmul(grad, p1.T(), "wirtinger", _ca, _ca ^ (1 - _cb)) if p0._requires_grad else None
             rhs = matmul(p0.T(), grad, "wirtinger", _cb ^ (1 - _ca), _cb) if p1._requires_grad else None
         else:
-            lhs = matmul(grad, p1.T(), "reference") if p0._requires_grad else None
-            rhs = matmul(p0.T(), grad, "reference") if p1._requires_grad else None
+            # A gradient is laid out like its primal: for a transposed view (x.T() of a row-major x) the same product is
+            # taken as its transpose, B g^T for (g B^T)^T, and handed on as that array's .T(). The view's own VJP then
+            # returns a ROW-MAJOR gradient for x, and what meets it there (the sum with another contribution, a fused
+            # elementwise rule) takes the flat kernels instead of the transposed ones.
+            lhs = rhs = None
+            if p0._requires_grad:
+                lhs = matmul(p1, grad.T(), "reference").T() if _is_transposed_matrix(p0) else matmul(grad, p1.T(), "reference")
+            if p1._requires_grad:
+                rhs = matmul(grad.T(), p0, "reference").T() if _is_transposed_matrix(p1) else matmul(p0.T(), grad, "reference")
         return [lhs, rhs]
 
     return _register(out, [ea, eb], "matmul", vjp)
