@@ -56,6 +56,11 @@ struct MlpArgs {
   const float* x;
   float* dx;
   int tile0[ENDIA_MLP_MAX_LAYERS + 1];  // weight gradients: first 32 x 32 tile of every layer in the launch's grid
+  // weight gradients of a large batch: the launch's grid.y slices of rows_per_slice rows leave their sums in wpart
+  // ([slice][woff[layers]] floats; layer l: dW at woff[l], db behind it), which a second launch adds up in slice order
+  float* wpart;
+  int woff[ENDIA_MLP_MAX_LAYERS + 1];
+  int rows_per_slice;
   // forward with the MSE loss on top (target != null): d loss / d output = 2 (out - target) / n goes to dpred, every
   // work-group leaves its sum of squared differences in loss_part and the last one to arrive adds them up, in row order
   const float* target;
@@ -812,11 +817,13 @@ __global__ __launch_bounds__(256) void mlp_wgrad_kernel(MlpArgs p) {
       colsum += bv[s];
     }
   };
-  request(32 * wave, a[0], b[0]);
-  for (int r0 = 32 * wave; r0 < p.batch; r0 += 256) {
+  const int begin = (int)blockIdx.y * p.rows_per_slice;  // (a multiple of 128; one slice unless the batch is large)
+  const int end = min(p.batch, begin + p.rows_per_slice);
+  request(begin + 32 * wave, a[0], b[0]);
+  for (int r0 = begin + 32 * wave; r0 < end; r0 += 256) {
     request(r0 + 128, a[1], b[1]);
     multiply(a[0], b[0]);
-    if (r0 + 128 >= p.batch) break;
+    if (r0 + 128 >= end) break;
     request(r0 + 256, a[0], b[0]);
     multiply(a[1], b[1]);
   }
@@ -826,20 +833,38 @@ __global__ __launch_bounds__(256) void mlp_wgrad_kernel(MlpArgs p) {
   __syncthreads();
   const int ocol = tid & 31, nn = 32 * bn + ocol;
   if (nn >= N) return;
-  if (p.dW[l]) {
+  // one slice: the gradients themselves; several: this slice's sums
+  float* dWl = gridDim.y > 1 ? p.wpart + (int64_t)blockIdx.y * p.woff[p.layers] + p.woff[l] : p.dW[l];
+  float* dbl = gridDim.y > 1 ? dWl + K * N : p.db[l];
+  if (dWl) {
 #pragma unroll
     for (int u = 0; u < 4; ++u) {
       const int row = (tid >> 5) + 8 * u, k = 32 * bk + row;
       const float sum = ((part[0][row * WG_PITCH + ocol] + part[1][row * WG_PITCH + ocol]) + part[2][row * WG_PITCH + ocol]) + part[3][row * WG_PITCH + ocol];
-      if (k < K) p.dW[l][(int64_t)k * N + nn] = sum;
+      if (k < K) dWl[(int64_t)k * N + nn] = sum;
     }
   }
-  if (bk == 0 && tid < 32 && p.db[l]) {
+  if (bk == 0 && tid < 32 && dbl) {
     float sum = 0.f;
 #pragma unroll
     for (int w = 0; w < 4; ++w) sum += bsum[w][0][ocol] + bsum[w][1][ocol];
-    p.db[l][nn] = sum;
+    dbl[nn] = sum;
   }
+}
+
+// The second launch of a large batch's weight gradients: every gradient element is the sum of its slices, in slice order.
+__global__ __launch_bounds__(256) void mlp_wgrad_sum_kernel(MlpArgs p, int slices) {
+  const int total = p.woff[p.layers];
+  const int e = blockIdx.x * 256 + threadIdx.x;
+  if (e >= total) return;
+  int l = 0;
+  while (l + 1 < p.layers && e >= p.woff[l + 1]) ++l;
+  const int at = e - p.woff[l], kn = p.width[l] * p.width[l + 1];
+  float* dst = at < kn ? (p.dW[l] ? p.dW[l] + at : nullptr) : (p.db[l] ? p.db[l] + (at - kn) : nullptr);
+  if (!dst) return;
+  float sum = 0.f;
+  for (int s = 0; s < slices; ++s) sum += p.wpart[(int64_t)s * total + e];
+  *dst = sum;
 }
 
 int32_t fill_args(MlpArgs& a, const endia_hip_mlp_desc* d, const char* who) {
@@ -984,8 +1009,32 @@ int32_t bwd(const char* who, const endia_hip_mlp_desc* desc, const float* x, con
     launch_delta(a, s);
     ENDIA_LAUNCH_CHECK();
   }
-  hipLaunchKernelGGL(mlp_wgrad_kernel, dim3((unsigned)blocks), dim3(256), 0, s, a);
+  // A large batch is cut into slices of at least 1024 rows, enough of them for two work-groups per CU; their sums meet in
+  // a second launch (pooled scratch, handed back on scope exit: reuse is stream-ordered).
+  int total = 0;
+  for (int l = 0; l < a.layers; ++l) {
+    a.woff[l] = total;
+    total += a.width[l] * a.width[l + 1] + a.width[l + 1];
+  }
+  a.woff[a.layers] = total;
+  int64_t slices = std::min<int64_t>(std::max<int64_t>(1, 2 * ctx().cu_count / blocks), a.batch / 1024);
+  if (slices < 1) slices = 1;
+  a.rows_per_slice = (int)(ceil_div64(ceil_div64(a.batch, slices), 128) * 128);
+  slices = ceil_div64(a.batch, a.rows_per_slice);
+  struct Scratch {
+    void* p = nullptr;
+    ~Scratch() { if (p) endia_hip_free(p); }
+  } part;
+  if (slices > 1) {
+    if ((rc = endia_hip_malloc(slices * total * 4, &part.p))) return rc;
+    a.wpart = static_cast<float*>(part.p);
+  }
+  hipLaunchKernelGGL(mlp_wgrad_kernel, dim3((unsigned)blocks, (unsigned)slices), dim3(256), 0, s, a);
   ENDIA_LAUNCH_CHECK();
+  if (slices > 1) {
+    hipLaunchKernelGGL(mlp_wgrad_sum_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, s, a, (int)slices);
+    ENDIA_LAUNCH_CHECK();
+  }
   return ENDIA_HIP_OK;
 }
 
