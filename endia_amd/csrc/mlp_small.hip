@@ -651,7 +651,7 @@ __global__ __launch_bounds__(64 * NW, 1) void mlp_fwd4_kernel(MlpArgs p) {
   __shared__ __attribute__((aligned(16))) float ds[2][R * LD4];
   __shared__ float part[NW][R][MAXW];
   __shared__ int meet;
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, j = lane & 3;
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int ocol = tid & (MAXW - 1), orow = tid >> 7;  // the outputs this thread finishes: column ocol of rows orow + 4 u
   const int row0 = blockIdx.x * R;
   auto request = [&](int l, FragF& f) {
