@@ -7,7 +7,7 @@
 // rows of the batch and runs ALL layers back to back: activations stay in LDS, the weights (a few tens of KiB,
 // resident in L2) go straight from memory into MFMA operands, the next layer's while the current layer computes.
 //   mlp_fwd4_kernel / mlp_delta4_kernel   FOUR rows per work-group on v_mfma_f32_4x4x1_16b_f32, for batches of up to
-//                     1024 rows (the reference's 128 rows are 32 work-groups); every weight request covers whole
+//                     2048 rows (the reference's 128 rows are 32 work-groups); every weight request covers whole
 //                     128-byte lines;
 //   mlp_fwd_kernel / mlp_delta_kernel     sixteen rows per work-group on v_mfma_f32_16x16x4_f32, beyond;
 //   mlp_wgrad_kernel  dW_l = h_{l-1}^T delta_l and db_l = 1^T delta_l for ALL layers in one launch, a work-group per
@@ -884,9 +884,10 @@ int32_t fill_args(MlpArgs& a, const endia_hip_mlp_desc* d, const char* who) {
   return ENDIA_HIP_OK;
 }
 
-// Four rows per work-group while every group still gets a CU of its own (each group fetches every weight); sixteen
-// rows on the 16 x 16 x 4 MFMA beyond (measured: 2048 rows take 127 us on the four-row kernels, 95 us on these).
-constexpr int64_t kFourRowBatch = 1024;
+// Four rows per work-group up to 2048 rows (two groups per CU), sixteen rows on the 16 x 16 x 4 MFMA beyond: every group
+// fetches every weight, so more groups cost more traffic. Measured, forward + backward of four 128-wide layers replayed as
+// a graph: 2048 rows 72 us on the four-row kernels against 80 us, 4096 rows 102 against 98, 8192 rows 166 against 150.
+constexpr int64_t kFourRowBatch = 2048;
 int64_t fwd_groups(const MlpArgs& a) { return ceil_div64(a.batch, a.batch <= kFourRowBatch ? 4 : ROWS); }
 
 void launch_fwd(const MlpArgs& a, hipStream_t s) {

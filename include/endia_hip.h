@@ -233,7 +233,7 @@ ENDIA_API int32_t endia_hip_mlp_fwd_mse(const endia_hip_mlp_desc* desc, const fl
 ENDIA_API int32_t endia_hip_mlp_bwd(const endia_hip_mlp_desc* desc, const float* x, const float* const* W, const float* const* h,
                           float* const* delta, float* const* dW, float* const* db, float* dx);
 /* The training step of mlp_imp.mojo:56-66 (forward, mse, backward) split so that the backward pass is one launch:
- * endia_hip_mlp_fwd_mse_delta is endia_hip_mlp_fwd_mse that goes on, in the same launch for batches of up to 1024 rows,
+ * endia_hip_mlp_fwd_mse_delta is endia_hip_mlp_fwd_mse that goes on, in the same launch for batches of up to 2048 rows,
  * to the cotangents of ALL layers for the loss gradient 2 (h[layers-1] - target) / n (every row of the batch is
  * independent through the whole chain): delta[l] [batch, widths[l+1]], none null, and dx [batch, widths[0]] when not
  * null, exactly what endia_hip_mlp_bwd leaves there when its delta[layers-1] is that loss gradient.

@@ -1218,7 +1218,7 @@ def test_whole_model_mse_loss_op(nd):
 def test_whole_model_forward_with_cotangents_entry_points(nd):
     """endia_hip_mlp_fwd_mse_delta + endia_hip_mlp_wgrad through the C ABI against endia_hip_mlp_fwd_mse +
     endia_hip_mlp_bwd: the same loss, activations, cotangents of every layer, dx, dW and db, bit for bit (the chain is
-    the same arithmetic whether it runs in the forward launch or in its own), on both sides of the 1024-row switch, with
+    the same arithmetic whether it runs in the forward launch or in its own), on both sides of the 2048-row switch, with
     and without dx, with gradients that are not asked for, and twice in a row."""
     import ctypes
     from endia_amd import _lib as L
@@ -1227,7 +1227,7 @@ def test_whole_model_forward_with_cotangents_entry_points(nd):
     act_code = {None: L.OP_IDENTITY, "relu": L.OP_RELU, "tanh": L.OP_TANH}
     for widths, batch, act, want_dx in [([1, 32, 64, 128, 128, 128, 64, 32, 1], 128, "relu", False), ([7, 50, 3, 128, 20], 37, "tanh", True),
                                         ([128, 128], 16, None, True), ([5, 17], 1, "relu", False), ([33, 128, 65, 12], 1024, "tanh", True),
-                                        ([33, 128, 65, 12], 1500, "relu", True), ([6, 9, 4], 3, "relu", True)]:
+                                        ([33, 128, 65, 12], 2048, "relu", True), ([33, 128, 65, 12], 2500, "relu", True), ([6, 9, 4], 3, "relu", True)]:
         Lyr = len(widths) - 1
         W = [nd.array((rng.standard_normal((widths[i], widths[i + 1])) / np.sqrt(widths[i])).astype(np.float32)) for i in range(Lyr)]
         b = [nd.array((0.2 * rng.standard_normal(widths[i + 1])).astype(np.float32)) for i in range(Lyr)]
@@ -1279,7 +1279,7 @@ def test_whole_model_entry_points_unaligned_and_deep(nd):
     from endia_amd import _lib as L
     from endia_amd._array import Array
     rng = np.random.default_rng(78)
-    for widths, batch, act, off in [([12, 40, 128, 24, 8], 50, "tanh", 1), ([12, 40, 128, 24, 8], 1100, "relu", 1),
+    for widths, batch, act, off in [([12, 40, 128, 24, 8], 50, "tanh", 1), ([12, 40, 128, 24, 8], 2100, "relu", 1),
                                     ([8] * 17, 10, "tanh", 0), ([128] * 17, 9, "relu", 0)]:
         Lyr = len(widths) - 1
         Wn = [(rng.standard_normal((widths[i], widths[i + 1])) / np.sqrt(widths[i])).astype(np.float32) for i in range(Lyr)]
@@ -1329,12 +1329,12 @@ def test_whole_model_entry_points_unaligned_and_deep(nd):
 def test_whole_model_mlp_op(nd):
     """functional.mlp_forward through the C ABI's endia_hip_mlp_fwd / endia_hip_mlp_bwd: the same numbers as the
     per-layer path for ragged widths and batches (rows and columns that do not fill an MFMA block), batches on both
-    sides of the switch from four to sixteen rows per work-group (1024 rows), the input gradient, a parameter that
+    sides of the switch from four to sixteen rows per work-group (2048 rows), the input gradient, a parameter that
     needs no gradient, two calls in a row (bit-identical), and the cases it refuses."""
     rng = np.random.default_rng(123)
     for widths, batch, act in [([1, 32, 64, 128, 128, 128, 64, 32, 1], 128, "relu"), ([7, 50, 3, 128, 20], 37, "tanh"),
                                ([128, 128], 16, None), ([5, 17], 1, "relu"), ([40, 100, 100, 9], 300, "relu"),
-                               ([33, 128, 65, 12], 1024, "tanh"), ([33, 128, 65, 12], 1500, "relu")]:
+                               ([33, 128, 65, 12], 2048, "tanh"), ([33, 128, 65, 12], 2500, "relu")]:
         Lyr = len(widths) - 1
         Wn = [(rng.standard_normal((widths[i], widths[i + 1])) / np.sqrt(widths[i])).astype(np.float32) for i in range(Lyr)]
         bn = [(0.2 * rng.standard_normal(widths[i + 1])).astype(np.float32) for i in range(Lyr)]
