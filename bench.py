@@ -49,11 +49,11 @@ def build_wide_mlp(nd, width=4096, layers=8, batch=4096, seed=2):
     return mlp, opt, x, y
 
 
-def build_sine_mlp(nd, seed=0, optimizer="sgd"):
+def build_sine_mlp(nd, seed=0, optimizer="sgd", per_layer=False):
     rng = np.random.default_rng(seed)
     widths = [1, 32, 64, 128, 128, 128, 64, 32, 1]
-    # fused="model": the whole stack is one op (one launch forward, two backward); "layer" keeps one op per layer
-    mlp = nd.nn.MLP(widths, compute_backward=True, activation="relu", fused=True if os.environ.get("ENDIA_SINE_PER_LAYER") else "model")
+    # fused="model": the whole stack is one op (one launch forward, two backward); per_layer keeps one op per layer
+    mlp = nd.nn.MLP(widths, compute_backward=True, activation="relu", fused=True if per_layer else "model")
     for i in range(8):
         s = np.sqrt(2.0 / widths[i])
         mlp.weights[i] = nd.array((rng.standard_normal((widths[i], widths[i + 1])) * s).astype(np.float32), requires_grad=True)
@@ -66,11 +66,11 @@ def build_sine_mlp(nd, seed=0, optimizer="sgd"):
     return mlp, opt, x, y
 
 
-def train_step(nd, mlp, opt, x, y):
-    if os.environ.get("ENDIA_SINE_SEPARATE_LOSS"):  # the reference script's call shape: forward, then mse
-        loss = nd.mse(mlp.forward(x), y)
-    else:  # the same two calls behind one method, which a whole-model MLP evaluates in its forward launch
+def train_step(nd, mlp, opt, x, y, fused_loss=False):
+    if fused_loss:  # forward and loss behind one method, which a whole-model MLP evaluates in its forward launch
         loss = mlp.mse_loss(x, y)
+    else:  # the reference script's call shape: forward, then mse (mlp_imp.mojo:56-60)
+        loss = nd.mse(mlp.forward(x), y)
     loss.backward()
     opt.step()
     loss.zero_grad()
@@ -206,14 +206,13 @@ def cpu_baseline_complex(rows=512):
                       "left out); %.1f s of CPU work" % (rows, rows, time.perf_counter() - t_all0)}
 
 
-def cpu_baseline_conv():
-    """The reference's 7-deep convolution loop (conv2d_op.mojo:127-196) and the brute-force adjoints of it, on 16
-    images of the batch of 64, extrapolated by 4; plus the ReLU / mean passes over those images' output."""
+def cpu_baseline_conv(n_img=16):
+    """The reference's 7-deep convolution loop (conv2d_op.mojo:127-196) and the brute-force adjoints of it, on n_img
+    images of the batch of 64, extrapolated; plus the ReLU / mean passes over those images' output."""
     from oracle import endia_ref as R
     rng = np.random.default_rng(5)
     t_all0 = time.perf_counter()
     C, H, K = 64, 56, 128
-    n_img = 16
     x = rng.standard_normal((n_img, C, H, H)).astype(np.float32)
     w = (rng.standard_normal((K, C, 3, 3)) * np.sqrt(2.0 / (C * 9))).astype(np.float32)
     bias = rng.standard_normal(K).astype(np.float32)
@@ -226,9 +225,9 @@ def cpu_baseline_conv():
     step = t_fwd + t_bwd + t_ew
     return {"value": 1.0 / step, "unit": "steps/s", "cores": 1, "kind": "port", "host_cores_available": os.cpu_count(),
             "seconds_per_step": step, "forward_seconds": t_fwd, "gradients_seconds": t_bwd,
-            "sample": "ref-order CPU restatement (1 thread): forward loop and its adjoints (dx, dw, db) on 16 of the 64 "
-                      "images, extrapolated by 4, plus relu / relu-gradient / mean passes; %.1f s of CPU work"
-                      % (time.perf_counter() - t_all0)}
+            "sample": "ref-order CPU restatement (1 thread): forward loop and its adjoints (dx, dw, db) on %d of the 64 "
+                      "images, extrapolated by %g, plus relu / relu-gradient / mean passes; %.1f s of CPU work"
+                      % (n_img, scale, time.perf_counter() - t_all0)}
 
 
 def kernel_table(reps=10):
@@ -365,7 +364,7 @@ def gemm_mid_table(reps=100, warm=600):
     return rows
 
 
-def conv_table(reps=10):
+def conv_table(reps=10, only=None):
     """conv2d at the benchmark configuration: x [64,64,56,56], w [128,64,3,3], stride 1, pad 1 (fp32, NCHW).
     Algorithmic flops per pass: 2*N*K*C*R*S*P*Q = 29.6 GFLOP for each of forward, data and weight gradient."""
     from endia_amd import _lib as L
@@ -430,6 +429,8 @@ def conv_table(reps=10):
         ("avg_pool2d 2x2/2 fwd", lambda: L.call("endia_hip_pool_fwd", pref, L.POOL_AVG, dy, py, None), 4.0 * n_in + 4.0 * n_out, "hbm"),
         ("avg_pool2d 2x2/2 bwd", lambda: L.call("endia_hip_pool_bwd", pref, L.POOL_AVG, py, None, y), 4.0 * n_in + 4.0 * n_out, "hbm"),
     ]
+    if only:
+        cases = [c for c in cases if c[0] in only]
     rows = []
     ms = ctypes.c_float()
     for _ in range(30):  # bring the clocks up before the first timed kernel
@@ -569,29 +570,15 @@ def run_complex(nd, steps, warmup, algo):
         return loss
 
     from endia_amd import _lib as L
-    # `value` is taken under the Wirtinger rule (g B^H, A^H g; the conjugations are flags of the complex GEMM), which
-    # yields the gradient of the real loss that the float64 checks of this configuration compare against; the
-    # reference's coded rule (no conjugation, matmul_op.mojo:278-283) costs the same launches and is timed beside it
-    for _ in range(warmup):
-        step(True)
-    nd.synchronize()
-    t0 = time.perf_counter()
-    for _ in range(steps):
-        step(True)
-    nd.synchronize()
-    dt = (time.perf_counter() - t0) / steps
-    for _ in range(warmup):
-        step(False)
-    nd.synchronize()
-    t0 = time.perf_counter()
-    for _ in range(steps):
-        step(False)
-    nd.synchronize()
-    dt_reference = (time.perf_counter() - t0) / steps
+    # `value` is taken under the library's default, the reference's coded rule (no conjugation, matmul_op.mojo:278-283);
+    # the Wirtinger rule (g B^H, A^H g: the gradient of the real loss, which the float64 checks of this configuration
+    # compare with torch's complex128 autograd) costs the same launches with other conjugation flags and is timed beside it
+    dt, _ = _time_steps(nd, lambda: step(False), steps, warmup)
+    dt_wirtinger, _ = _time_steps(nd, lambda: step(True), steps, warmup)
     L.call("endia_hip_gemm_timing_begin")  # second pass, with an event pair around every GEMM launch
     t0 = time.perf_counter()
     for _ in range(steps):
-        step(True)
+        step(False)
     nd.synchronize()
     elapsed = time.perf_counter() - t0
     flops = 11 * 8.0 * n * n * n  # algorithmic: 8 real flops per complex multiply-add, whichever algorithm runs
@@ -603,12 +590,134 @@ def run_complex(nd, steps, warmup, algo):
             "unit": "steps/s", "n_gpus": 1, "ms_per_step": dt * 1e3, "higher_is_better": True, "vs_baseline": None,
             "algorithmic_gemm_tflops": flops / dt / 1e12,
             "frac_of_fp32_mfma_peak": flops / dt / 1e12 / FP32_MFMA_PEAK_TFLOPS, "steps": steps, "warmup": warmup,
-            "gradient_rule": "wirtinger (dA = g B^H, dB = A^H g)",
-            "reference_rule": {"rule": "no conjugation, matmul_op.mojo:278-283", "ms_per_step": dt_reference * 1e3,
-                               "steps_per_s": 1.0 / dt_reference, "algorithmic_gemm_tflops": flops / dt_reference / 1e12},
+            "gradient_rule": "reference (dA = g B^T, dB = A^T g, no conjugation: matmul_op.mojo:278-283)",
+            "wirtinger_rule": {"rule": "dA = g B^H, dB = A^H g (vjp_rule='wirtinger')", "ms_per_step": dt_wirtinger * 1e3,
+                               "steps_per_s": 1.0 / dt_wirtinger, "algorithmic_gemm_tflops": flops / dt_wirtinger / 1e12},
             "dtype": "c64 (f32 pairs)", "data": "synthetic",
             "config": {"workload": "complex_mlp: 4 x complex Linear(2048->2048), identity, loss sum|out|^2, batch 2048, " + algo},
             "roofline": roof}
+
+
+def _time_steps(nd, step, steps, warmup):
+    for _ in range(warmup):
+        step()
+    nd.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        out = step()
+    nd.synchronize()
+    return (time.perf_counter() - t0) / steps, out
+
+
+def run_sine(nd, steps, warmup, optimizer="sgd", eager=False, per_layer=False):
+    """BASELINE configuration 1, the reference's own benchmark model (benchmarks/mlp_benchmarks/mlp_imp.mojo:35-75), as
+    a HIP-graph replay of the eager step. `value` is taken with the reference script's call shape, mse(mlp.forward(x),
+    y); the same step with forward and loss behind one method (MLP.mse_loss, no counterpart in the reference) is
+    timed beside it. Launch-latency bound: no roofline claim."""
+    w = [1, 32, 64, 128, 128, 128, 64, 32, 1]
+    kn = sum(w[i] * w[i + 1] for i in range(8))
+    flops = 2.0 * 128 * (3 * kn - w[0] * w[1])
+    res = {}
+    for fused_loss in (False, True):
+        mlp, opt, x, y = build_sine_mlp(nd, optimizer=optimizer, per_layer=per_layer)
+        step = lambda: train_step(nd, mlp, opt, x, y, fused_loss)
+        for _ in range(max(warmup, 3)):
+            step()
+        nd.synchronize()
+        captured = None if eager else nd.capture(step)
+        dt, loss = _time_steps(nd, captured.replay if captured else step, steps, 20)
+        res[fused_loss] = (dt, float(loss.item()))
+        if captured:
+            captured.close()
+    dt, final_loss = res[False]
+    return {"metric": "fwd+bwd+%s train steps/s, sine-fit MLP" % ("SGD" if optimizer == "sgd" else "Adam"),
+            "value": 1.0 / dt, "unit": "steps/s", "n_gpus": 1, "steps": steps, "warmup": warmup, "ms_per_step": dt * 1e3,
+            "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f32", "data": "synthetic",
+            "config": {"workload": "sine_mlp: widths 1-32-64-128-128-128-64-32-1, relu, MSE, %s 1e-3, batch 128, fp32"
+                                   % ("SGD" if optimizer == "sgd" else "Adam"), "batch": 128, "optimizer": optimizer,
+                       "execution": ("host-issued launches" if eager else "HIP graph replay of the eager step") +
+                                    ("; one fused op per layer" if per_layer else "; nn.MLP(fused='model')") +
+                                    "; loss = mse(mlp.forward(x), y) as in the reference's script"},
+            "final_loss": final_loss, "gemm_tflops_whole_step": flops / dt / 1e12,
+            "roofline": {"bound": "launch latency", "kernel": None, "achieved": None, "peak": None, "frac": None,
+                         "note": "a step is a handful of dependent launches of 4-20 us; no roofline claim"},
+            "fused_loss_call": {"call": "MLP.mse_loss(x, y): forward, loss and the cotangents of all layers in one launch",
+                                "value": 1.0 / res[True][0], "ms_per_step": res[True][0] * 1e3, "final_loss": res[True][1]}}
+
+
+def run_wide(nd, steps, warmup):
+    from endia_amd import _lib as L
+    mlp, opt, x, y = build_wide_mlp(nd)
+    width, layers, batch = 4096, 8, 4096
+    gemm_flops_step = (layers + layers + layers - 1) * 2.0 * batch * width * width
+    for _ in range(warmup):
+        train_step(nd, mlp, opt, x, y)
+    nd.synchronize()
+    L.call("endia_hip_gemm_timing_begin")
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        loss = train_step(nd, mlp, opt, x, y)
+    nd.synchronize()
+    elapsed = time.perf_counter() - t0
+    launches, g_ms, g_flops = ctypes.c_int64(), ctypes.c_double(), ctypes.c_double()
+    L.call("endia_hip_gemm_timing_end", ctypes.byref(launches), ctypes.byref(g_ms), ctypes.byref(g_flops))
+    ms_per_step = 1e3 * elapsed / steps
+    out = {
+        "metric": "fwd+bwd train steps/s + MFMA util %, 8-layer 4096-wide fp32 MLP, batch 4096",
+        "value": steps / elapsed, "unit": "steps/s", "n_gpus": 1, "steps": steps, "warmup": warmup,
+        "ms_per_step": ms_per_step, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "f32", "data": "synthetic",
+        "config": {"workload": "wide_mlp: 8 x Linear(4096->4096)+bias, tanh, MSE, Adam, batch 4096, fp32",
+                   "batch": batch, "width": width, "layers": layers, "optimizer": "adam"},
+        "final_loss": float(loss.item()),
+        "gemm_tflops_whole_step": gemm_flops_step / (ms_per_step * 1e-3) / 1e12,
+    }
+    if launches.value:
+        avg_ms = g_ms.value / launches.value
+        flops_per_launch = g_flops.value / launches.value
+        achieved = flops_per_launch / (avg_ms * 1e-3) / 1e12
+        out["roofline"] = {
+            "bound": "mfma", "kernel": "sgemm_lone_kernel<FM = 4, FN = 4> (fp32 v_mfma_f32_32x32x2, 256x256x32 tiles, one work-group per CU)",
+            "achieved": achieved, "peak": FP32_MFMA_PEAK_TFLOPS, "unit": "TFLOP/s", "frac": achieved / FP32_MFMA_PEAK_TFLOPS,
+            "traffic": GEMM_TRAFFIC_BYTES,
+            "traffic_source": "rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, see profiles/kernels_wide_mlp_counters.md",
+            "algorithmic_bytes": 3 * 4096 * 4096 * 4,
+            "launches": launches.value, "avg_launch_ms": avg_ms,
+            "flops_per_launch": flops_per_launch, "gemm_share_of_step": g_ms.value / (1e3 * elapsed),
+        }
+        out["mfma_util_pct"] = 100.0 * achieved / FP32_MFMA_PEAK_TFLOPS
+    return out
+
+
+def run_conv(nd, steps, warmup):
+    """BASELINE configuration 5 as a training step through the public API (forward with fused ReLU, mean loss, weight
+    and bias gradients; the same with the data gradient beside it). `roofline` prices the forward entry point, the
+    longest of the step's launches, timed alone with HIP events on the library's stream."""
+    rows = conv_table(max(min(steps, 10), 3), only=("conv2d_fwd (+bias, relu)", "conv2d_bwd_data", "conv2d_bwd_weight"))
+    step, with_dx = conv_step(nd, steps, warmup, False), conv_step(nd, steps, warmup, True)
+    fwd = rows[0]
+    return {"metric": "conv2d fwd + VJPs train steps/s, batch 64, 64->128 channels, 3x3, stride 1, pad 1, 56x56, fp32",
+            "value": step["steps_per_s"], "unit": "steps/s", "n_gpus": 1, "steps": steps, "warmup": warmup,
+            "ms_per_step": step["ms_per_step"], "higher_is_better": True, "vs_baseline": None, "dtype": "f32", "data": "synthetic",
+            "config": {"workload": "conv2d: x [64,64,56,56], w [128,64,3,3], stride 1, pad 1, relu, mean loss; forward + dw + db"},
+            "algorithmic_tflops": step["algorithmic_tflops"], "frac_of_fp32_mfma_peak": step["frac_of_fp32_mfma_peak"],
+            "with_data_gradient": with_dx, "entry_points": rows,
+            "roofline": {"bound": "mfma", "kernel": "conv_direct3x3_kernel (forward; weight packing included)", "achieved": fwd["achieved"],
+                         "peak": fwd["peak"], "unit": fwd["unit"], "frac": fwd["frac"], "traffic": None, "avg_launch_ms": fwd["ms"]}}
+
+
+def _brief(out):
+    """What the headline line keeps of another configuration's result."""
+    keep = ("value", "unit", "ms_per_step", "steps", "warmup", "dtype", "algorithmic_gemm_tflops", "algorithmic_tflops",
+            "frac_of_fp32_mfma_peak", "fused_loss_call", "wirtinger_rule", "with_data_gradient", "gradient_rule", "final_loss")
+    b = {"workload": out["config"]["workload"]}
+    b.update({k: out[k] for k in keep if k in out})
+    r = out.get("roofline") or {}
+    b["roofline"] = {k: r.get(k) for k in ("bound", "kernel", "achieved", "peak", "unit", "frac", "launches", "avg_launch_ms") if k in r}
+    c = out.get("cpu_baseline")
+    if c:
+        b["cpu_baseline"] = {k: c[k] for k in ("value", "unit", "cores", "kind", "sample") if k in c}
+    return b
 
 
 def main():
@@ -616,9 +725,11 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=3)
-    ap.add_argument("--workload", default="wide_mlp", choices=["wide_mlp", "sine_mlp", "kernels", "gemm_mid", "conv2d", "hvp", "complex_mlp", "complex_mlp_3m"])
+    ap.add_argument("--workload", default="wide_mlp", choices=["wide_mlp", "sine_mlp", "kernels", "gemm_mid", "conv2d", "conv2d_kernels", "hvp", "complex_mlp", "complex_mlp_3m"])
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--headline-only", action="store_true", help="wide_mlp: leave the other four configurations out of the line")
     ap.add_argument("--eager", action="store_true", help="sine_mlp: issue every kernel from the host instead of replaying a graph")
+    ap.add_argument("--per-layer", action="store_true", help="sine_mlp: one fused op per layer instead of the whole-model op")
     ap.add_argument("--optimizer", default="sgd", choices=["sgd", "adam"], help="sine_mlp: SGD (the benchmark configuration) or Adam (the reference script's)")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -629,103 +740,53 @@ def main():
     from endia_amd import _lib as L
     L.ensure_init(0)
     dev_name, cus, mhz = L.device_info()
+    cpu = not args.no_cpu_baseline
 
     if args.workload == "hvp":
         out = run_hvp(nd, args.steps, args.warmup)
-        if not args.no_cpu_baseline:
+        if cpu:
             out["cpu_baseline"] = cpu_baseline_hvp()
-        print(json.dumps(out))
-        return
-    if args.workload.startswith("complex_mlp"):
+    elif args.workload.startswith("complex_mlp"):
         out = run_complex(nd, args.steps, args.warmup, "3m" if args.workload.endswith("3m") else "4m")
-        if not args.no_cpu_baseline:
+        if cpu:
             out["cpu_baseline"] = cpu_baseline_complex()
-        print(json.dumps(out))
-        return
-    if args.workload == "conv2d":
-        rows = conv_table(max(args.steps, 1))
-        out = {"metric": "conv2d fwd + VJPs, batch 64, 64->128 channels, 3x3, stride 1, pad 1, 56x56, fp32",
-               "device": dev_name, "reps": max(args.steps, 1), "kernels": rows,
-               "train_step": [conv_step(nd, max(args.steps, 1), args.warmup, False),
-                              conv_step(nd, max(args.steps, 1), args.warmup, True)]}
-        if not args.no_cpu_baseline:
+    elif args.workload == "conv2d":
+        out = run_conv(nd, max(args.steps, 1), args.warmup)
+        if cpu:
             out["cpu_baseline"] = cpu_baseline_conv()
-        print(json.dumps(out))
-        return
-    if args.workload == "gemm_mid":
-        print(json.dumps({"metric": "fp32 GEMM launches of the mid-size products, sustained clock", "device": dev_name,
-                          "reps": max(args.steps, 1), "kernels": gemm_mid_table(max(args.steps, 1))}))
-        return
-    if args.workload == "kernels":
-        rows = kernel_table(max(args.steps, 1))
-        print(json.dumps({"metric": "per-kernel roofline at the wide-MLP shape (4096 x 4096 operands)", "device": dev_name,
-                          "reps": max(args.steps, 1), "kernels": rows}))
-        return
-
-    if args.workload == "wide_mlp":
-        mlp, opt, x, y = build_wide_mlp(nd)
-        width, layers, batch = 4096, 8, 4096
-        gemm_flops_step = (layers + layers + layers - 1) * 2.0 * batch * width * width
-        config = {"workload": "wide_mlp: 8 x Linear(4096->4096)+bias, tanh, MSE, Adam, batch 4096, fp32",
-                  "batch": batch, "width": width, "layers": layers, "optimizer": "adam"}
+    elif args.workload == "conv2d_kernels":
+        out = {"metric": "conv2d / conv3d / pooling entry points, fp32", "device": dev_name, "reps": max(args.steps, 1),
+               "kernels": conv_table(max(args.steps, 1))}
+    elif args.workload == "gemm_mid":
+        out = {"metric": "fp32 GEMM launches of the mid-size products, sustained clock", "device": dev_name,
+               "reps": max(args.steps, 1), "kernels": gemm_mid_table(max(args.steps, 1))}
+    elif args.workload == "kernels":
+        out = {"metric": "per-kernel roofline at the wide-MLP shape (4096 x 4096 operands)", "device": dev_name,
+               "reps": max(args.steps, 1), "kernels": kernel_table(max(args.steps, 1))}
+    elif args.workload == "sine_mlp":
+        out = run_sine(nd, max(args.steps, 200), args.warmup, args.optimizer, args.eager, args.per_layer)
+        if cpu:
+            out["cpu_baseline"] = cpu_baseline_sine(optimizer=args.optimizer)
     else:
-        mlp, opt, x, y = build_sine_mlp(nd, optimizer=args.optimizer)
-        w = [1, 32, 64, 128, 128, 128, 64, 32, 1]
-        kn = sum(w[i] * w[i + 1] for i in range(8))
-        gemm_flops_step = 2.0 * 128 * (3 * kn - w[0] * w[1])
-        config = {"workload": "sine_mlp: widths 1-32-64-128-128-128-64-32-1, relu, MSE, %s 1e-3, batch 128, fp32"
-                              % ("SGD" if args.optimizer == "sgd" else "Adam"),
-                  "batch": 128, "optimizer": args.optimizer}
-
-    for _ in range(args.warmup):
-        train_step(nd, mlp, opt, x, y)
-    nd.synchronize()
-
-    captured = None
-    if args.workload == "sine_mlp" and not args.eager:
-        # launch-latency bound: replay the step as one HIP graph (same kernels, same results)
-        captured = nd.capture(lambda: train_step(nd, mlp, opt, x, y))
-        config["execution"] = "HIP graph replay of the eager step" + (
-            "" if os.environ.get("ENDIA_SINE_PER_LAYER") else
-            "; nn.MLP(fused='model'): 3 launches a step (forward of all layers with the MSE loss, its gradient and the cotangents "
-            "of all layers; all weight and bias gradients; optimizer over all 16 tensors)")
-    L.call("endia_hip_gemm_timing_begin")
-    t0 = time.perf_counter()
-    for _ in range(args.steps):
-        loss = captured.replay() if captured else train_step(nd, mlp, opt, x, y)
-    nd.synchronize()
-    elapsed = time.perf_counter() - t0
-    launches, g_ms, g_flops = ctypes.c_int64(), ctypes.c_double(), ctypes.c_double()
-    L.call("endia_hip_gemm_timing_end", ctypes.byref(launches), ctypes.byref(g_ms), ctypes.byref(g_flops))
-    final_loss = float(loss.item())
-
-    ms_per_step = 1e3 * elapsed / args.steps
-    steps_per_s = args.steps / elapsed
-    out = {
-        "metric": "fwd+bwd train steps/s + MFMA util %, 8-layer 4096-wide fp32 MLP, batch 4096"
-                  if args.workload == "wide_mlp" else "fwd+bwd+%s train steps/s, sine-fit MLP" % ("SGD" if args.optimizer == "sgd" else "Adam"),
-        "value": steps_per_s, "unit": "steps/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
-        "ms_per_step": ms_per_step, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
-        "dtype": "f32", "data": "synthetic", "config": config,
-        "device": dev_name, "final_loss": final_loss,
-        "gemm_tflops_whole_step": gemm_flops_step / (ms_per_step * 1e-3) / 1e12,
-    }
-    if launches.value:
-        avg_ms = g_ms.value / launches.value
-        flops_per_launch = g_flops.value / launches.value
-        achieved = flops_per_launch / (avg_ms * 1e-3) / 1e12
-        out["roofline"] = {
-            "bound": "mfma", "kernel": "sgemm_lone_kernel<FM = 4, FN = 4> (fp32 v_mfma_f32_32x32x2, 256x256x32 tiles, one work-group per CU)",
-            "achieved": achieved, "peak": FP32_MFMA_PEAK_TFLOPS, "unit": "TFLOP/s", "frac": achieved / FP32_MFMA_PEAK_TFLOPS,
-            "traffic": GEMM_TRAFFIC_BYTES if args.workload == "wide_mlp" else None,
-            "traffic_source": "rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, see profiles/kernels_wide_mlp_counters.md",
-            "algorithmic_bytes": 3 * 4096 * 4096 * 4 if args.workload == "wide_mlp" else None,
-            "launches": launches.value, "avg_launch_ms": avg_ms,
-            "flops_per_launch": flops_per_launch, "gemm_share_of_step": g_ms.value / (1e3 * elapsed),
-        }
-        out["mfma_util_pct"] = 100.0 * achieved / FP32_MFMA_PEAK_TFLOPS
-    if not args.no_cpu_baseline:
-        out["cpu_baseline"] = cpu_baseline_wide() if args.workload == "wide_mlp" else cpu_baseline_sine(optimizer=args.optimizer)
+        out = run_wide(nd, args.steps, args.warmup)
+        out["device"] = dev_name
+        if cpu:
+            out["cpu_baseline"] = cpu_baseline_wide()
+        if not args.headline_only:
+            # the other four benchmark configurations, each bounded to a second or two of GPU time and a few seconds of
+            # CPU baseline: the same functions that `--workload sine_mlp | hvp | complex_mlp | conv2d` run alone
+            others = []
+            for name, fn, base in (
+                    ("sine_mlp", lambda: run_sine(nd, 2000, 3), lambda: cpu_baseline_sine(steps=200)),
+                    ("hvp", lambda: run_hvp(nd, 40, 5), cpu_baseline_hvp),
+                    ("complex_mlp", lambda: run_complex(nd, 20, 3, "4m"), lambda: cpu_baseline_complex(rows=256)),
+                    ("conv2d", lambda: run_conv(nd, 100, 10), lambda: cpu_baseline_conv(n_img=8))):
+                r = fn()
+                if cpu:
+                    r["cpu_baseline"] = base()
+                others.append(_brief(r))
+                nd.synchronize()
+            out["configs"] = others
     print(json.dumps(out))
 
 

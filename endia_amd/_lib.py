@@ -122,6 +122,7 @@ SIGNATURES = {
     "endia_hip_conv2d_bwd_weight": [POINTER(Conv2dDesc), _fp, _fp, _fp],
     "endia_hip_conv2d_bwd_bias": [POINTER(Conv2dDesc), _fp, _fp],
     "endia_hip_conv2d_bwd_relu": [POINTER(Conv2dDesc), _fp, _fp, _fp, _fp, c_int32, _fp, _fp, _fp],
+    "endia_hip_conv_force_path": [c_int32],
     "endia_hip_conv3d_out_shape": [POINTER(Conv3dDesc), _i64p],
     "endia_hip_conv3d_fwd": [POINTER(Conv3dDesc), _fp, _fp, _fp, _fp, c_int32],
     "endia_hip_conv3d_bwd_data": [POINTER(Conv3dDesc), _fp, _fp, _fp],

@@ -34,6 +34,7 @@ using namespace mfma;
 
 constexpr int TPB = 256;
 constexpr int FAR = -(1 << 28);  // coordinate that fails every bounds test
+int g_forced_path = 0;  // endia_hip_conv_force_path
 
 struct ConvP {
   int N, C, D, H, W, K, T, R, S, O, P, Q;  // O, P, Q: output depth, height, width
@@ -1531,7 +1532,7 @@ bool wgrad_vec_ok(const ConvP& p, const float* rows) {
 // The row-cache weight gradient (conv_wgrad3x3_kernel) where it applies: 1 if it does not. Same gate modes and bias
 // sums as conv_bwd_weight below.
 int32_t run_wgrad3x3(const ConvP& p, const float* x, const float* dy, float* dw, int gate_mode, const float* gate, float* db) {
-  if (getenv("ENDIA_NO_WGRAD3X3")) return 1;
+  if (g_forced_path == 1) return 1;
   if (p.T != 1 || p.D != 1 || p.R != 3 || p.S != 3 || p.dh != 1 || p.dw != 1 || p.sh != 1 || p.sw != 1 || p.sd != 1) return 1;
   if (p.ph < 0 || p.ph > 1 || p.pw < 0 || p.pw > 1 || p.W % 4 || p.Q % 4 || p.Q < 8 || p.Q > 56) return 1;
   const float* rows = gate_mode == 1 ? gate : dy;
@@ -1542,7 +1543,7 @@ int32_t run_wgrad3x3(const ConvP& p, const float* x, const float* dy, float* dw,
   const int tiles_k = (p.K + W3_BK - 1) / W3_BK;
   a.tiles_c = (p.C + W3_BC - 1) / W3_BC;
   // few channels would leave most of the 128 x 32 tile's MFMA rows or columns multiplying zeros: the gather kernels have smaller tiles
-  if ((double)tiles_k * W3_BK * a.tiles_c * W3_BC > 1.5 * (double)p.K * p.C && !getenv("ENDIA_FORCE_WGRAD3X3")) return 1;
+  if ((double)tiles_k * W3_BK * a.tiles_c * W3_BC > 1.5 * (double)p.K * p.C && g_forced_path != 2) return 1;
   const int64_t tiles = (int64_t)tiles_k * a.tiles_c;
   // about two work-groups per CU in all (what a CU holds), each on a run of output rows of one image
   int64_t per_image = (2 * (int64_t)endia::ctx().cu_count + tiles * p.N - 1) / (tiles * p.N);
@@ -1783,6 +1784,12 @@ using namespace endia;
   }
 
 extern "C" {
+
+int32_t endia_hip_conv_force_path(int32_t path) {
+  ENDIA_CHECK_ARG(path >= 0 && path <= 2, "endia_hip_conv_force_path: path %d is not one of 0, 1, 2", path);
+  g_forced_path = path;
+  return ENDIA_HIP_OK;
+}
 
 int32_t endia_hip_conv2d_out_shape(const endia_hip_conv2d_desc* d, int64_t* P, int64_t* Q) {
   ConvP p;

@@ -555,9 +555,6 @@ int32_t sgemm_impl(int transA, int transB, int64_t M, int64_t N, int64_t K, cons
       }
       ENDIA_HIP_CALL(hipEventRecord(g_timing.start[g_timing.used], s));
     }
-#ifdef ENDIA_LONE_STAMPS
-    if (lone >= 0) p.part = reinterpret_cast<float*>(ctx().tickets);  // profiling build: per-group wall-clock stamps (<= 512 groups)
-#endif
     if (lone >= 0) {
       int32_t rc = lone == 0 ? launch_lone_256x256(p, epi, transA, transB, grid, s) : launch_lone_256x128(p, epi, transA, transB, grid, s);
       if (rc) return rc;
@@ -702,7 +699,3 @@ extern "C" int32_t endia_hip_gemm_timing_end(int64_t* launches, double* total_ms
   return ENDIA_HIP_OK;
 }
 
-#ifdef ENDIA_LONE_STAMPS
-// profiling build only: where the one-wave-per-SIMD kernels leave their per-group wall-clock stamps
-extern "C" __attribute__((visibility("default"))) void* endia_debug_stamps(void) { return endia::ctx().tickets; }
-#endif

@@ -46,10 +46,6 @@ __device__ __forceinline__ void gemm_tile_lone(const GemmArgs& p, int block, int
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int wm = wave >> 1, wn = wave & 1, l32 = lane & 31, h = lane >> 5;
-#ifdef ENDIA_LONE_STAMPS
-  unsigned long long stamp[4];
-  stamp[0] = wall_clock64();
-#endif
   int tm, tn;
   tile_of_block(block, nblocks, p.tiles_m, p.tiles_n, tm, tn);
   const int m0 = tm * BM, n0 = tn * BN;
@@ -186,23 +182,10 @@ __device__ __forceinline__ void gemm_tile_lone(const GemmArgs& p, int block, int
   };
   // two K tiles per trip, one per LDS stage; an odd tile count runs one more tile of zeros
   const int T = (K + BK - 1) / BK;
-#ifdef ENDIA_LONE_STAMPS
-  stamp[1] = wall_clock64();
-#endif
   for (int t = 0; t < T; t += 2) {
     tile_body(std::integral_constant<int, 0>());
     tile_body(std::integral_constant<int, 1>());
   }
-#ifdef ENDIA_LONE_STAMPS
-  stamp[2] = wall_clock64();
-  struct StampOut {
-    const GemmArgs& p; int block, tid; unsigned long long (&stamp)[4];
-    __device__ ~StampOut() {
-      stamp[3] = wall_clock64();
-      if (tid == 0 && p.part) for (int i = 0; i < 4; ++i) reinterpret_cast<unsigned long long*>(p.part)[block * 4 + i] = stamp[i];
-    }
-  } stamp_out{p, block, tid, stamp};
-#endif
 
   // Epilogue. Nothing overlaps it (the CU's only tile ends here), so what it reads is requested ahead of the stores,
   // which the compiler must assume to alias it: the bias of the lane's columns up front, and the activation operand

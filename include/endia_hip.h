@@ -384,6 +384,13 @@ ENDIA_API int32_t endia_hip_conv2d_bwd_relu(const endia_hip_conv2d_desc* d, cons
                                   const float* y, const float* dy, int32_t dy_is_scalar, float* dx, float* dw,
                                   float* db);
 
+/* Kernel choice of the 3 x 3 weight gradient. No counterpart in the reference: a hook for tests and tuning, like
+ * endia_hip_gemm_force_tile. path = 0 (the default) chooses by shape; 1 keeps every weight gradient on the gather
+ * kernels; 2 runs the cached-rows kernel on every shape it can compute, also where few channels would leave most of
+ * its tile multiplying zeros. Results do not depend on the path beyond the order of the additions. Process-wide, not
+ * thread-safe against concurrent convolution calls. */
+ENDIA_API int32_t endia_hip_conv_force_path(int32_t path);
+
 /* ---- conv3d, [N,C,D,H,W] with kernel [K,C,T,R,S], groups = 1: Conv3d.__call__ (spacial_ops/conv3d_op.mojo:104-259),
  *      output extents per axis (in + 2*pad - dil*(k-1) - 1) / stride + 1 (conv3d_op.mojo:71-101). Conv1d
  *      (spacial_ops/conv1d_op.mojo) is conv2d on a height-1 image. Same kernels as conv2d, which is the case

@@ -1261,7 +1261,11 @@ def test_whole_model_forward_with_cotangents_entry_points(nd):
             return [loss] + h + delta + [a for a in dW if a is not None] + db + ([dx] if dx else [])
 
         ref = [a.to_numpy() for a in two_calls()]
-        for _ in range(2):
+        for _ in range(2):  # the loss sum meets at a ticket: the same bits on every call
+            again = [a.to_numpy() for a in two_calls()]
+            for k, (g, r) in enumerate(zip(again, ref)):
+                np.testing.assert_array_equal(g, r, err_msg="widths %s batch %d %s: tensor %d differs between runs" % (widths, batch, act, k))
+        for _ in range(3):
             got = [a.to_numpy() for a in fused()]
             assert len(got) == len(ref)
             for k, (g, r) in enumerate(zip(got, ref)):
@@ -1269,6 +1273,54 @@ def test_whole_model_forward_with_cotangents_entry_points(nd):
     # arguments the entry points refuse
     with pytest.raises(Exception):
         L.call("endia_hip_mlp_fwd_mse_delta", ctypes.byref(desc), x.data_ptr(), ptrs(W), ptrs(b), t.data_ptr(), ptrs(W), None, x.data_ptr(), None)
+
+
+def test_whole_model_large_batch_repeats_bit_for_bit(nd):
+    """65 536 rows of four 128-wide layers: the weight gradients are summed over 64 row slices by a second launch and
+    the loss over 4096 work-groups that meet at a ticket. Three runs of forward + loss + chain + gradients give the
+    same bits (fixed order of every sum), and the gradients match float64."""
+    import ctypes
+    from endia_amd import _lib as L
+    from endia_amd._array import Array
+    rng = np.random.default_rng(79)
+    widths, batch = [128] * 5, 65536
+    Lyr = 4
+    Wn = [(rng.standard_normal((128, 128)) / np.sqrt(128)).astype(np.float32) for _ in range(Lyr)]
+    bn = [(0.2 * rng.standard_normal(128)).astype(np.float32) for _ in range(Lyr)]
+    xn = rng.standard_normal((batch, 128)).astype(np.float32)
+    tn = rng.standard_normal((batch, 128)).astype(np.float32)
+    W, b, x, t = [nd.array(w) for w in Wn], [nd.array(v) for v in bn], nd.array(xn), nd.array(tn)
+    desc = L.MlpDesc()
+    desc.layers, desc.act, desc.batch = Lyr, L.OP_TANH, batch
+    desc.widths[:Lyr + 1] = widths
+    ptrs = lambda arrs: (ctypes.c_void_p * Lyr)(*[a.data_ptr() for a in arrs])
+
+    def run():
+        h = [Array.empty([batch, 128]) for _ in range(Lyr)]
+        delta = [Array.empty([batch, 128]) for _ in range(Lyr)]
+        dW, db = [Array.empty([128, 128]) for _ in range(Lyr)], [Array.empty([128]) for _ in range(Lyr)]
+        loss = Array.empty([1])
+        L.call("endia_hip_mlp_fwd_mse_delta", ctypes.byref(desc), x.data_ptr(), ptrs(W), ptrs(b), t.data_ptr(), ptrs(h), ptrs(delta),
+               loss.data_ptr(), None)
+        L.call("endia_hip_mlp_wgrad", ctypes.byref(desc), x.data_ptr(), ptrs(h), ptrs(delta), ptrs(dW), ptrs(db))
+        return [loss.to_numpy()] + [a.to_numpy() for a in dW + db]
+
+    first = run()
+    for _ in range(2):
+        for k, (g, r) in enumerate(zip(run(), first)):
+            np.testing.assert_array_equal(g, r, err_msg="tensor %d differs between runs" % k)
+    # float64 chain rule on the host
+    hs = [xn.astype(np.float64)]
+    for i in range(Lyr):
+        z = hs[-1] @ Wn[i].astype(np.float64) + bn[i]
+        hs.append(np.tanh(z) if i < Lyr - 1 else z)
+    d = 2.0 * (hs[-1] - tn) / tn.size
+    assert_close(first[0], [np.mean((hs[-1] - tn) ** 2)], tol=1e-5, what="loss")
+    for i in reversed(range(Lyr)):
+        assert_close(first[1 + i], hs[i].T @ d, what="dW%d" % i)
+        assert_close(first[1 + Lyr + i], d.sum(0), what="db%d" % i)
+        if i:
+            d = (d @ Wn[i].astype(np.float64).T) * (1.0 - hs[i] ** 2)
 
 
 def test_whole_model_entry_points_unaligned_and_deep(nd):

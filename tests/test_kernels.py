@@ -527,8 +527,19 @@ FAST_CASES = [
 ]
 
 
+@pytest.fixture
+def conv_path(dev):
+    """endia_hip_conv_force_path for one test; the default choice is restored afterwards."""
+    yield lambda path: dev.call("endia_hip_conv_force_path", path)
+    dev.call("endia_hip_conv_force_path", 0)
+
+
+@pytest.mark.parametrize("path", [0, 1, 2])
 @pytest.mark.parametrize("xs,ws,st,pd,dl", FAST_CASES)
-def test_conv2d_paths_vs_oracle(dev, xs, ws, st,pd, dl):
+def test_conv2d_paths_vs_oracle(dev, conv_path, xs, ws, st, pd, dl, path):
+    """path 0: the kernels the library chooses; 1: every weight gradient on the gather kernels; 2: the cached-rows
+    weight gradient wherever it can compute the shape, however few channels."""
+    conv_path(path)
     rng = np.random.default_rng(sum(xs) + sum(ws))
     x = rng.standard_normal(xs).astype(np.float32)
     w = (rng.standard_normal(ws) * 0.3).astype(np.float32)
