@@ -101,6 +101,8 @@ class Array:
     _act_applied = False  # a gradient that already carries the producer's activation derivative
     _grad_fused = None    # such a gradient on its way to this node's own VJP rule; never what grad() returns
     _true_grad = None     # on an _act_applied gradient: a function that computes the gradient without the derivative
+    _internal = False     # a node that a VJP rule created (the transposes and broadcasts inside a recorded backward pass)
+    _absorbed = False     # a VJP result that already includes the gradient its primal held (functional._absorb)
     _offset = 0
     is_complex_ = False
 

@@ -10,6 +10,8 @@ The functional wrappers (grad / jacobian / hessian / value_and_grad over a Pytho
 non-JIT branch of Callable.__call__ (endia/compile/callable.mojo:100-197): repeated
 backward(create_graph=True) passes, then detached copies of the results.
 """
+import sys
+
 from .. import functional as F
 from .._array import Array, _contiguous_copy
 
@@ -96,9 +98,33 @@ def vjp_from(outs, cotangents, create_graph=False):
     _reverse_walk(trace, create_graph)
 
 
+_VIEW_OPS = ("permute", "reshape", "squeeze", "unsqueeze")
+absorb_enabled = [True]  # tests switch the in-launch accumulation off to compare with the walk's own `add`
+
+
+def _offers(primals):
+    """What the primals of one VJP call already hold, for rules that can add it in their own last launch
+    (functional._absorb): id(primal) -> (gradient, exclusive). `exclusive`: no other name refers to the gradient array
+    or shares its buffer (reference counts: the gradient slot, the local below and the call's argument; the array's
+    buffer field and the call's argument), so a rule may accumulate into it in place."""
+    offers = None
+    if not absorb_enabled[0]:
+        return None
+    for p in primals:
+        g = p._grad
+        if g is None or not p._requires_grad or p._grad_fused is not None or g._is_seed:
+            continue
+        exclusive = sys.getrefcount(g) <= 3 and sys.getrefcount(g._buf) <= 2
+        if offers is None:
+            offers = {}
+        offers[id(p)] = (g, exclusive)
+    return offers
+
+
 def _reverse_walk(trace, create_graph):
     """The trace in reverse: every node's VJP rule, contributions to one tensor summed with `add`
-    (functional.mojo:46-65). The outputs' gradients are already in place."""
+    (functional.mojo:46-65), or inside the launch that computes the later contribution where its rule can
+    (functional._absorb). The outputs' gradients are already in place."""
     for node in trace:
         node._consumers = 0
     for node in trace:
@@ -114,14 +140,26 @@ def _reverse_walk(trace, create_graph):
                 continue
             # a gradient that already carries this node's activation derivative travels in its own slot
             grad = curr._grad_fused if curr._grad_fused is not None else curr.grad()
-            primals_grads = curr._vjp(primals, grad, curr)
+            F._absorb = None if create_graph else _offers(primals)
+            F._in_rule[0] = True
+            try:
+                primals_grads = curr._vjp(primals, grad, curr)
+            finally:
+                F._absorb = None
+                F._in_rule[0] = False
+            if not create_graph and curr._internal and curr._name in _VIEW_OPS:
+                # a view that an earlier pass's rule made (x.T() inside a recorded matmul rule): nobody can ask for its
+                # gradient, and letting go of it leaves the gradient it handed on as the only holder of that buffer
+                grad = None
+                curr._grad = None
             for primal, pg in zip(primals, primals_grads):
                 if not primal._requires_grad or pg is None:
                     continue
                 if primal.has_grad():
                     if pg._act_applied or primal._grad_fused is not None:
                         raise RuntimeError("internal: a fused activation gradient met an accumulated gradient")
-                    pg = F.add(pg, primal._grad)
+                    if not pg._absorbed:  # (an absorbed contribution already holds the sum)
+                        pg = F.add(pg, primal._grad)
                 if pg._act_applied:
                     primal._grad_fused = pg
                     continue

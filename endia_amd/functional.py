@@ -19,8 +19,13 @@ from ._array import Array, Buffer, _contiguous_copy, _prod, contiguous_strides
 # --------------------------------------------------------------------------------------------------
 # registration
 # --------------------------------------------------------------------------------------------------
+_in_rule = [False]  # set by the reverse walk while a VJP rule runs
+
+
 def _register(out, args, name, vjp, meta=None):
     out._name = name
+    if _in_rule[0]:
+        out._internal = True  # made by a VJP rule: no user code holds this node
     if any(a._requires_grad for a in args):
         out._requires_grad = True
         out._args = list(args)
@@ -606,6 +611,10 @@ def sub(a, b):
 
 def mul(a, b):
     def vjp(primals, grad, out):  # mul_op.mojo:125-128 (no conjugation for complex operands)
+        if primals[0] is primals[1] and primals[0]._requires_grad and not primals[0].is_complex_ and grad._shape == primals[0]._shape \
+                and (_fusion is None or not _fusion.tracing(grad, primals[0])):
+            # x * x: both contributions, x g + x g, as one launch and one node instead of two products and their sum
+            return [_fused_rule("twice_mul", lambda x_, g_: mul(add(x_, x_), g_))(primals[0], grad), None]
         return [mul(primals[1], grad) if primals[0]._requires_grad else None,
                 mul(primals[0], grad) if primals[1]._requires_grad else None]
     return _binary(L.BIN_MUL, "mul", a, b, vjp)
@@ -1016,6 +1025,32 @@ def std(x, axes=(0,), unbiased=True, keepdims=False):
 
 
 # --------------------------------------------------------------------------------------------------
+# gradients that absorb an earlier contribution
+# --------------------------------------------------------------------------------------------------
+# Where a tensor has several consumers the reverse walk adds their contributions with one `add` launch each
+# (autograd/functional.mojo:51-57). A rule whose last step is a matrix product can do that addition in the product's
+# epilogue instead. The walk offers, per VJP call, the gradient a primal already holds (`_absorb`: id(primal) ->
+# (gradient, exclusive)); a rule that uses the offer marks its result `_absorbed`, and the walk stores it as the new
+# total without adding. Two forms: the earlier gradient is a row broadcast over the rows (the cotangent of a bias
+# gradient on its way to the layer's pre-activation): it becomes the bias operand of the product's epilogue, the
+# result is a fresh array; or it is a plain array that nobody else holds (`exclusive`): the product accumulates into
+# its buffer. Never offered while a pass records its own graph, where every contribution stays a node.
+_absorb = None
+_absorbed_launches = [0]  # how many `add` launches the protocol has replaced (read by the tests)
+
+
+def _absorb_offer(primal):
+    return _absorb.get(id(primal)) if _absorb else None
+
+
+def _as_bias_row(g, rows, cols):
+    """g viewed as [rows, cols] is one row of memory repeated: its device address, else None."""
+    if g.is_complex_ or list(g._shape) != [rows, cols] or g._strides[0] != 0 or (cols > 1 and g._strides[1] != 1):
+        return None
+    return g.data_ptr()
+
+
+# --------------------------------------------------------------------------------------------------
 # matmul (endia/functional/binary_ops/matmul_op.mojo)
 # --------------------------------------------------------------------------------------------------
 def _gemm_operand(x):
@@ -1059,7 +1094,7 @@ def _is_transposed_matrix(x):
             and x._strides[0] == 1 and x._strides[1] >= x._shape[0])
 
 
-def matmul(a, b, vjp_rule=None, _ca=0, _cb=0):
+def matmul(a, b, vjp_rule=None, _ca=0, _cb=0, _into=None):
     """Batched matrix product with broadcast batch axes (matmul_op.mojo:36-90,309-346).
 
     VJP (matmul_op.mojo:278-283): dA = g @ B.T(), dB = A.T() @ g. For complex operands the reference codes exactly
@@ -1098,15 +1133,28 @@ def matmul(a, b, vjp_rule=None, _ca=0, _cb=0):
     eb = expand(b, bshape + [K, N], [-2, -1])
     A_, ta, lda, sa = _gemm_operand(ea)
     B_, tb, ldb, sb = _gemm_operand(eb)
-    out = Array.empty(out_shape, is_complex=a.is_complex_)
     batch = _prod(bshape)
+    # `_into` (an offer of the reverse walk, see _absorb above): (earlier gradient of this product's shape, exclusive)
+    epi, bias_ptr, out = L.EPI_NONE, None, None
+    if _into is not None and not a.is_complex_ and len(out_shape) == 2 and M * N * K > 0:
+        g0, exclusive = _into
+        bias_ptr = _as_bias_row(g0, M, N)
+        if bias_ptr is not None:
+            epi = L.EPI_BIAS
+        elif exclusive and list(g0._shape) == out_shape and g0.is_contiguous() and not g0.is_complex_:
+            epi, out = L.EPI_NONE | L.GEMM_ACCUMULATE, Array(out_shape, _buffer=g0._buf, _offset=g0._offset)
+    if out is None:
+        out = Array.empty(out_shape, is_complex=a.is_complex_)
+    if epi != L.EPI_NONE:
+        out._absorbed = True
+        _absorbed_launches[0] += 1
     if out.size():
         if a.is_complex_:
             L.call("endia_hip_cgemm", ta, _ca, tb, _cb, M, N, K, A_.data_ptr(), lda, B_.data_ptr(), ldb, out.data_ptr(), N,
                    batch, sa, sb, M * N, _cgemm_algo[0], 0)
         else:
             L.call("endia_hip_sgemm", ta, tb, M, N, K, A_.data_ptr(), lda, B_.data_ptr(), ldb, out.data_ptr(), N, batch,
-                   sa, sb, M * N, L.EPI_NONE, L.OP_IDENTITY, None, None, None)
+                   sa, sb, M * N, epi, L.OP_IDENTITY, bias_ptr, None, None)
 
     def vjp(primals, grad, out_):
         p0, p1 = primals
@@ -1120,13 +1168,36 @@ def matmul(a, b, vjp_rule=None, _ca=0, _cb=0):
             # returns a ROW-MAJOR gradient for x, and what meets it there (the sum with another contribution, a fused
             # elementwise rule) takes the flat kernels instead of the transposed ones.
             lhs = rhs = None
+            o0 = _absorb_offer(p0) if p0 is not p1 else None
+            o1 = _absorb_offer(p1) if p0 is not p1 else None
             if p0._requires_grad:
-                lhs = matmul(p1, grad.T(), "reference").T() if _is_transposed_matrix(p0) else matmul(grad, p1.T(), "reference")
+                if _is_transposed_matrix(p0):
+                    lhs = _keep_absorbed(matmul(p1, grad.T(), "reference", _into=_transposed_offer(o0)))
+                else:
+                    lhs = matmul(grad, p1.T(), "reference", _into=o0)
             if p1._requires_grad:
-                rhs = matmul(grad.T(), p0, "reference").T() if _is_transposed_matrix(p1) else matmul(p0.T(), grad, "reference")
+                if _is_transposed_matrix(p1):
+                    rhs = _keep_absorbed(matmul(grad.T(), p0, "reference", _into=_transposed_offer(o1)))
+                else:
+                    rhs = matmul(p0.T(), grad, "reference", _into=o1)
         return [lhs, rhs]
 
     return _register(out, [ea, eb], "matmul", vjp)
+
+
+def _transposed_offer(offer):
+    """The walk's offer for a primal that is a transposed view, as seen by the product that computes the gradient's
+    transpose: only the in-place form applies (the transpose of a row broadcast is not one)."""
+    if offer is None or not offer[1] or offer[0].ndim() != 2:
+        return None
+    return (offer[0].T(), True)
+
+
+def _keep_absorbed(prod):
+    t = prod.T()
+    if prod._absorbed:
+        t._absorbed = True
+    return t
 
 
 _cgemm_algo = [L.CGEMM_4M]
@@ -1564,6 +1635,13 @@ def _sin_of_linear_node(out, zz):
             return [mul(cos(z), grad)]  # sin_op.mojo:92
         if grad._act_applied:
             return [grad]
+        offer = _absorb_offer(z)
+        if offer is not None and offer[0]._shape == z._shape and grad._shape == z._shape and not offer[0].is_complex_:
+            # z already holds a gradient (a second-order pass reaches the pre-activation twice): one launch for both
+            gz = _fused_rule("cos_mul_add", lambda zz_, g_, e_: add(mul(cos(zz_), g_), e_))(detach(z), detach(grad), detach(offer[0]))
+            gz._absorbed = True
+            _absorbed_launches[0] += 1
+            return [gz]
         g = contiguous(grad)
         gz = Array.empty(out_._shape)
         L.call("endia_hip_unary_vjp", L.OP_SIN, n, z.data_ptr(), g.data_ptr(), gz.data_ptr(), 0)
@@ -1614,11 +1692,35 @@ def _linear_node(out, x, W, b, xs, Ws, act):
                 dx._act_applied = True
                 # what px.grad() shows is dL/dpx itself; nobody reads it in a training step, so it is made on demand
                 dx._true_grad = lambda: matmul(detach(g), detach(Ws).T())
-        L.call("endia_hip_linear_bwd", B, K, N, xs.data_ptr(), Ws.data_ptr(), g.data_ptr(), flags,
-               aux.data_ptr() if aux is not None else None, dx.data_ptr() if dx is not None else None,
-               dW.data_ptr() if dW is not None else None, db.data_ptr() if db is not None else None)
-        res = [dx, dW, db]
-        return res
+        # A weight or an input that already holds a gradient nobody else refers to (second-order passes reach both
+        # twice) takes this layer's product on top of it in the GEMM's epilogue instead of through an `add` launch.
+        def in_place(offer, shape):
+            if offer is None or not offer[1] or B * K * N == 0:
+                return None
+            g0 = offer[0]
+            if list(g0._shape) != shape or not g0.is_contiguous() or g0.is_complex_:
+                return None
+            _absorbed_launches[0] += 1
+            tot = Array(shape, _buffer=g0._buf, _offset=g0._offset)
+            tot._absorbed = True
+            return tot
+        accW = in_place(_absorb_offer(pW), [K, N]) if dW is not None and pW is not px else None
+        accX = in_place(_absorb_offer(px), [B, K]) if dx is not None and aux is None and pW is not px else None
+        if accW is not None:
+            L.call("endia_hip_sgemm", 1, 0, K, N, B, xs.data_ptr(), K, g.data_ptr(), N, accW.data_ptr(), N, 1, 0, 0, 0,
+                   L.EPI_NONE | L.GEMM_ACCUMULATE | (L.GEMM_COLSUM_B if db is not None else 0), L.OP_IDENTITY, None, None,
+                   db.data_ptr() if db is not None else None)
+        if accX is not None:
+            L.call("endia_hip_sgemm", 0, 1, B, K, N, g.data_ptr(), N, Ws.data_ptr(), N, accX.data_ptr(), K, 1, 0, 0, 0,
+                   L.EPI_NONE | L.GEMM_ACCUMULATE, L.OP_IDENTITY, None, None, None)
+        rest_dx = dx if accX is None else None
+        rest_dW = dW if accW is None else None
+        rest_db = db if accW is None else None
+        if rest_dx is not None or rest_dW is not None or rest_db is not None:
+            L.call("endia_hip_linear_bwd", B, K, N, xs.data_ptr(), Ws.data_ptr(), g.data_ptr(), flags,
+                   aux.data_ptr() if aux is not None else None, rest_dx.data_ptr() if rest_dx is not None else None,
+                   rest_dW.data_ptr() if rest_dW is not None else None, rest_db.data_ptr() if rest_db is not None else None)
+        return [accX if accX is not None else dx, accW if accW is not None else dW, db]
 
     meta = {"act": act, "aux": out, "from_output": True} if act in _ACT_FN else {"act": None}
     return _register(out, [x, W, b], "linear", vjp, meta)

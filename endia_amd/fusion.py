@@ -332,7 +332,15 @@ class FusedElementwise:
         ins, modes = [], []
         for a in arrays:
             if list(a._shape) == shape:
-                ins.append(F.contiguous(a)); modes.append(L.EW_FULL)
+                # a broadcast view of the full shape (the cotangent a reduction hands down) is read as what it is,
+                # one element or one row, instead of being copied out
+                spread = [st == 0 for n_, st in zip(a._shape, a._strides) if n_ != 1]
+                if a.size() > 1 and all(spread):
+                    ins.append(Array([1], _buffer=a._buf, _offset=a._offset)); modes.append(L.EW_SCALAR)
+                elif rows > 1 and cols > 1 and a._strides[-1] == 1 and all(spread[:-1]):
+                    ins.append(Array([cols], _buffer=a._buf, _offset=a._offset)); modes.append(L.EW_ROW_VECTOR)
+                else:
+                    ins.append(F.contiguous(a)); modes.append(L.EW_FULL)
             elif a.size() == 1:
                 ins.append(a); modes.append(L.EW_SCALAR)
             elif a.size() == cols and a._shape[-1] == cols:

@@ -417,6 +417,80 @@ def test_hvp_double_backward(nd, golden, fused, seeded):
     assert abs(uHv - vHu) <= 1e-4 * max(abs(uHv), abs(vHu))
 
 
+def test_gradient_accumulation_inside_the_product_launch(nd, golden):
+    """Where a tensor has several consumers the walk sums their contributions with `add` (autograd/functional.mojo:51-57).
+    A matmul / linear / sin rule takes the earlier gradient into its own launch instead (a bias row or an in-place
+    accumulate in the GEMM epilogue, one fused elementwise launch): the Hessian-vector product with that switched on
+    and off gives the same numbers, launches are saved, and an array that user code holds is never written."""
+    from endia_amd.autograd import functional as AF
+    from endia_amd import functional as F
+    g = golden("hvp_sin")
+    x = nd.array(g["x"])
+    vs = []
+    for i in range(3):
+        vs += [g["vW%d" % i], g["vb%d" % i]]
+
+    def hvp(fused):
+        mlp, _ = _load_mlp(nd, g, 3, "sin", fused)
+        out = mlp.forward(x)
+        loss = nd.sum(out * out)
+        loss.backward(create_graph=True)
+        firsts = [p.grad() for p in mlp.params()]
+        hv = nd.grad(outs=firsts, inputs=mlp.params(), grad_outs=[nd.reshape(nd.array(v), f.shape()) for v, f in zip(vs, firsts)])
+        res = [h.to_numpy() for h in hv]
+        loss.zero_grad()
+        return res
+
+    for fused in (True, False):
+        before = F._absorbed_launches[0]
+        with_absorb = hvp(fused)
+        saved = F._absorbed_launches[0] - before
+        AF.absorb_enabled[0] = False
+        try:
+            plain = hvp(fused)
+            assert F._absorbed_launches[0] - before == saved
+        finally:
+            AF.absorb_enabled[0] = True
+        assert saved >= (8 if fused else 4), "only %d additions were taken into product launches" % saved
+        for i in range(3):
+            assert_close(with_absorb[2 * i], g["hW%d" % i], what="HvW%d" % i)
+            assert_close(with_absorb[2 * i + 1], g["hb%d" % i], what="Hvb%d" % i)
+        for a, b in zip(with_absorb, plain):
+            assert_close(a, b, tol=2e-6, mean_tol=1e-4, what="with and without in-launch accumulation")
+
+    # a cotangent that the caller holds is an output's gradient and then meets a product's contribution: it must be
+    # read, not accumulated into
+    rng = np.random.default_rng(11)
+    a = nd.array(rng.standard_normal((6, 5)).astype(np.float32), requires_grad=True)
+    Mn = rng.standard_normal((5, 5)).astype(np.float32)
+    cn, dn = rng.standard_normal((6, 5)).astype(np.float32), rng.standard_normal((6, 5)).astype(np.float32)
+    y = a * 1.0
+    w = nd.matmul(y, nd.array(Mn))
+    c, d = nd.array(cn), nd.array(dn)
+    (ga,) = nd.grad(outs=[y, w], inputs=[a], grad_outs=[c, d])
+    np.testing.assert_array_equal(c.to_numpy(), cn)
+    np.testing.assert_array_equal(d.to_numpy(), dn)
+    assert_close(ga.to_numpy(), cn.astype(np.float64) + dn.astype(np.float64) @ Mn.T.astype(np.float64), what="two contributions")
+    # three products into one tensor: the second and third accumulate in place into the first one's result
+    a = nd.array(rng.standard_normal((6, 5)).astype(np.float32), requires_grad=True)
+    Ms = [rng.standard_normal((5, 4)).astype(np.float32) for _ in range(3)]
+    before = F._absorbed_launches[0]
+    total = None
+    for M in Ms:
+        t = nd.sum(nd.matmul(a, nd.array(M)))
+        total = t if total is None else total + t
+    total.backward()
+    assert F._absorbed_launches[0] - before == 2
+    assert_close(a.grad().to_numpy(), np.ones((6, 4)) @ np.sum([M.astype(np.float64) for M in Ms], 0).T, what="three products")
+    # matmul(a, a): both gradients go to the same tensor and nothing is offered
+    a = nd.array(rng.standard_normal((4, 4)).astype(np.float32), requires_grad=True)
+    b = nd.array(rng.standard_normal((4, 4)).astype(np.float32), requires_grad=True)
+    an, bn = a.to_numpy().astype(np.float64), b.to_numpy().astype(np.float64)
+    nd.sum(nd.matmul(a, a) + nd.matmul(a, b)).backward()
+    one = np.ones((4, 4))
+    assert_close(a.grad().to_numpy(), one @ an.T + an.T @ one + one @ bn.T, what="matmul(a, a) + matmul(a, b)")
+
+
 def test_optimizer_classes(nd, golden):
     g = golden("optim")
     makers = {
