@@ -79,6 +79,9 @@ __device__ __forceinline__ void epilogue_store(const GemmArgs& p, float* __restr
   epilogue_apply<EPI>(p, C, aux_out, row, col, v, bias_v, aux_v);
 }
 
+// Launcher of the shared-CU tiles (tile = 64 or 128) for operands read 4 bytes at a time (gemm_unaligned.hip).
+void launch_mfma_unaligned(const GemmArgs& p, int epi, int tile, bool a_vec, bool b_vec, int transA, int transB, dim3 grid, hipStream_t s);
+
 // Launchers of the one-wave-per-SIMD tiles, one translation unit per tile shape (gemm_lone_*.hip).
 // The caller checks the launch with hipGetLastError.
 int32_t launch_lone_256x256(const GemmArgs& p, int epi, int transA, int transB, dim3 grid, hipStream_t s);

@@ -154,8 +154,10 @@ __device__ __forceinline__ int acc_row(int v, int h) { return 8 * (v >> 2) + 4 *
 // `records` returns zero, which pads the M/N edge of K-major operands and the K tail of MN-major
 // operands. The other edge (K tail of a K-major operand, M/N edge of an MN-major operand) is folded
 // into the offset, which becomes OOB_OFFSET. One 32-bit offset per pass is the only per-lane address
-// state. Requires 4-float alignment of the base, the leading dimension and the contiguous extent.
-template <bool KMAJOR, int BMN, int NTHREADS>
+// state. VEC requires 4-float alignment of the base, the leading dimension and the contiguous extent. Without it
+// (any view of any matrix: the reference's matmul has no alignment rule, matmul_op.mojo:93-199) a thread reads the same
+// four elements with four 32-bit loads, each with its own bounds test, and the LDS side is unchanged.
+template <bool KMAJOR, int BMN, int NTHREADS, bool VEC = true>
 struct MatrixTileLoader {
   static constexpr int F4_PER_ROW = KMAJOR ? BK / 4 : BMN / 4;
   static constexpr int ROWS_PER_PASS = NTHREADS / F4_PER_ROW;
@@ -166,6 +168,7 @@ struct MatrixTileLoader {
   const float* base;
   int64_t records, step;
   int c, lds_off;
+  int nvalid;  // !VEC, MN-major: how many of this thread's four columns lie inside the operand
   float4 reg[PASSES];
 
   // X: the operand; mn0: first row (K-major) or column (MN-major) of the tile; MN, K: operand extents
@@ -187,27 +190,35 @@ struct MatrixTileLoader {
       for (int i = 0; i < PASSES; ++i)
         voff[i] = (c < valid) ? (uint32_t)(((int64_t)(r + i * ROWS_PER_PASS) * ld + c) * 4) : OOB_OFFSET;
     }
+    nvalid = valid - c;
     lds_off = r * LD + c;
+  }
+  // one piece of four consecutive elements; k_left as in load()
+  __device__ __forceinline__ float4 load_piece(__amdgpu_buffer_rsrc_t rs, uint32_t o, int k_left) const {
+    if constexpr (VEC) {
+      if (KMAJOR) o = (c < k_left) ? o : OOB_OFFSET;
+      return buffer_load_f4(rs, o);
+    } else {
+      float v[4];
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        const bool in = KMAJOR ? (c + e < k_left) : (e < nvalid);
+        v[e] = buffer_load_f1(rs, in ? o + 4u * e : OOB_OFFSET);
+      }
+      return make_float4(v[0], v[1], v[2], v[3]);
+    }
   }
   // k_left = K - (first k of the tile being loaded); base/records already point at that tile
   __device__ __forceinline__ void load(int k_left) {
     __amdgpu_buffer_rsrc_t rs = make_rsrc(base, records);
 #pragma unroll
-    for (int i = 0; i < PASSES; ++i) {
-      uint32_t o = voff[i];
-      if (KMAJOR) o = (c < k_left) ? o : OOB_OFFSET;
-      reg[i] = buffer_load_f4(rs, o);
-    }
+    for (int i = 0; i < PASSES; ++i) reg[i] = load_piece(rs, voff[i], k_left);
   }
   // The same two steps with the staging registers held by the caller (several tiles in flight at once).
   __device__ __forceinline__ void load_into(float4 (&dst)[PASSES], int k_left) {
     __amdgpu_buffer_rsrc_t rs = make_rsrc(base, records);
 #pragma unroll
-    for (int i = 0; i < PASSES; ++i) {
-      uint32_t o = voff[i];
-      if (KMAJOR) o = (c < k_left) ? o : OOB_OFFSET;
-      dst[i] = buffer_load_f4(rs, o);
-    }
+    for (int i = 0; i < PASSES; ++i) dst[i] = load_piece(rs, voff[i], k_left);
   }
   __device__ __forceinline__ void store_from(float* lds, const float4 (&src)[PASSES]) {
 #pragma unroll
@@ -215,7 +226,10 @@ struct MatrixTileLoader {
   }
   // One pass at a time, for loops that spread a tile's loads and LDS stores between their MFMAs.
   // No address arithmetic per pass: the caller has run mask_tail for a tile that reaches past the end of K.
-  __device__ __forceinline__ void load_pass(int i, __amdgpu_buffer_rsrc_t rs) { reg[i] = buffer_load_f4(rs, voff[i]); }
+  __device__ __forceinline__ void load_pass(int i, __amdgpu_buffer_rsrc_t rs) {
+    static_assert(VEC, "the hand-scheduled loops read 16 bytes per request");
+    reg[i] = buffer_load_f4(rs, voff[i]);
+  }
   // A K-major tile that holds fewer than BK reduction elements: the pieces beyond them read as zeros from here on
   // (every later tile lies further out). The descriptor bounds do the same for an MN-major tile.
   __device__ __forceinline__ void mask_tail(int k_left) {

@@ -44,6 +44,67 @@ def test_sgemm_modes_vs_oracle(dev, M, N, K, ta, tb):
     assert_close(C, opA.astype(np.float64) @ opB.astype(np.float64), what="vs float64")
 
 
+def _embedded(rng, rows, cols, ld, off):
+    """A rows x cols matrix inside a larger host buffer: `off` floats in front, leading dimension ld >= cols, the
+    padding filled with large values that a read past an edge would drag into the result."""
+    buf = np.full(off + rows * ld + 3, 1.0e6, np.float32)
+    view = buf[off:off + rows * ld].reshape(rows, ld)
+    view[:, :cols] = rng.standard_normal((rows, cols)).astype(np.float32)
+    return buf, view[:, :cols]
+
+
+@pytest.mark.parametrize("ta,tb", [(0, 0), (0, 1), (1, 0), (1, 1)])
+@pytest.mark.parametrize("M,N,K,pad_a,pad_b,off_a,off_b", [
+    (30 * 4, 50, 40, 1, 0, 0, 0),     # odd leading dimension of A only (the shapes of the reference's own matmul test, rows x 4)
+    (129, 131, 67, 0, 0, 0, 0),       # every extent odd, leading dimensions = extents
+    (200, 72, 96, 0, 0, 1, 3),        # aligned shapes, bases 4 and 12 bytes off a 16-byte boundary
+    (64, 64, 33, 3, 1, 2, 1),         # one tile, K one past a K tile, padded rows
+    (256, 130, 515, 2, 3, 0, 1),      # few tiles and a long reduction: K is split inside the launch
+    (1000, 10, 300, 0, 0, 0, 0),      # a classifier head: ten columns
+    (70, 300, 9, 1, 1, 1, 1),         # shortest reduction the matrix-core path takes
+])
+def test_sgemm_unaligned_operands_on_the_matrix_cores(dev, M, N, K, pad_a, pad_b, off_a, off_b, ta, tb):
+    """Operands whose base address, leading dimension or extents are not multiples of four floats (the reference's
+    matmul takes any view: matmul_op.mojo:93-199) run the MFMA tiles with 4-byte loads. All four forms, every epilogue,
+    accumulation, the bias gradient riding along, against the oracle and float64; repeated runs give the same bits."""
+    rng = np.random.default_rng(M + 3 * N + 5 * K + 7 * ta + 11 * tb)
+    ar, ac = (K, M) if ta else (M, K)
+    br, bc = (N, K) if tb else (K, N)
+    bufA, A = _embedded(rng, ar, ac, ac + pad_a, off_a)
+    bufB, B = _embedded(rng, br, bc, bc + pad_b, off_b)
+    B *= 1.0 / np.sqrt(K)
+    dA, dB = dev.put(bufA) + 4 * off_a, dev.put(bufB) + 4 * off_b
+    lda, ldb = ac + pad_a, bc + pad_b
+    opA, opB = (A.T if ta else A), (B.T if tb else B)
+    ref64 = opA.astype(np.float64) @ opB.astype(np.float64)
+    ref = R.matmul(np.ascontiguousarray(opA), np.ascontiguousarray(opB))
+
+    def run(epi=L.EPI_NONE, act=L.OP_IDENTITY, bias=None, aux=None, C0=None, aux_out=None):
+        dC = dev.put(C0) if C0 is not None else dev.alloc(M * N * 4)
+        dev.call("endia_hip_sgemm", ta, tb, M, N, K, dA, lda, dB, ldb, dC, N, 1, 0, 0, 0, epi, act,
+                 dev.put(bias) if bias is not None else None, dev.put(aux) if aux is not None else None, aux_out)
+        return dev.get(dC, (M, N))
+
+    first = run()
+    assert_close(first, ref, what="vs oracle")
+    assert_close(first, ref64, what="vs float64")
+    for _ in range(2):
+        np.testing.assert_array_equal(run(), first)
+    bias = rng.standard_normal(N).astype(np.float32)
+    aux = rng.standard_normal((M, N)).astype(np.float32)
+    assert_close(run(L.EPI_BIAS, bias=bias), ref64 + bias, what="bias")
+    dz = dev.alloc(M * N * 4)
+    assert_close(run(L.EPI_BIAS_ACT, L.OP_TANH, bias=bias, aux_out=dz), np.tanh(ref64 + bias), what="bias + tanh")
+    assert_close(dev.get(dz, (M, N)), ref64 + bias, what="stored pre-activation")
+    assert_close(run(L.EPI_ACT_GRAD, L.OP_SIN, aux=aux), ref64 * np.cos(aux.astype(np.float64)), what="sin gradient epilogue")
+    C0 = rng.standard_normal((M, N)).astype(np.float32)
+    assert_close(run(L.EPI_NONE | L.GEMM_ACCUMULATE, C0=C0), C0 + ref64, what="accumulate")
+    if not tb and pad_b == 0:  # the column sums of B (a bias gradient) from the same call
+        dsum = dev.alloc(N * 4)
+        assert_close(run(L.EPI_NONE | L.GEMM_COLSUM_B, aux_out=dsum), ref64, what="product with column sums")
+        assert_close(dev.get(dsum, (N,)), B.astype(np.float64).sum(0), what="column sums of B")
+
+
 def test_sgemm_few_outputs_batched_accumulate(dev):
     """The one-group-per-output kernel with a batch, a broadcast operand and accumulation into C."""
     rng = np.random.default_rng(77)
