@@ -380,6 +380,65 @@ def gemm_mid_table(reps=100, warm=600):
     return rows
 
 
+def gemm_grouped_table(reps=100, warm=400):
+    """endia_hip_sgemm_grouped against the same products issued one by one, at the shapes of the second-order
+    configuration: x2 / x4 of each shape and form, and the mix a step of the double-backward chain offers."""
+    from endia_amd import _lib as L
+    L.ensure_init(0)
+    rng = np.random.default_rng(0)
+
+    def put(a):
+        p = ctypes.c_void_p()
+        L.call("endia_hip_malloc", a.nbytes, ctypes.byref(p))
+        L.call("endia_hip_memcpy_h2d", p.value, a.ctypes.data, a.nbytes)
+        return p.value
+
+    def member(M, N, K, ta, tb):
+        return (ta, tb, M, N, K, put(rng.standard_normal((K, M) if ta else (M, K)).astype(np.float32)), (M if ta else K),
+                put(rng.standard_normal((N, K) if tb else (K, N)).astype(np.float32)), (K if tb else N), put(np.zeros((M, N), np.float32)))
+
+    dx, dw = (1024, 2048, 2048), (2048, 2048, 1024)
+    cases = [("4 x NN 1024 x 2048 x 2048", [member(*dx, 0, 0) for _ in range(4)]),
+             ("4 x NT 1024 x 2048 x 2048", [member(*dx, 0, 1) for _ in range(4)]),
+             ("2 x TN 2048 x 2048 x 1024", [member(*dw, 1, 0) for _ in range(2)]),
+             ("2 x NN 1024 x 2048 x 2048", [member(*dx, 0, 0) for _ in range(2)]),
+             ("NT + NN 1024 x 2048 x 2048 and 2 x TN 2048 x 2048 x 1024", [member(*dx, 0, 1), member(*dx, 0, 0), member(*dw, 1, 0), member(*dw, 1, 0)]),
+             ("NN 1024 x 2048 x 2048 and TN 2048 x 2048 x 1024", [member(*dx, 0, 0), member(*dw, 1, 0)])]
+    rows = []
+    ms = ctypes.c_float()
+    for name, members in cases:
+        descs = (L.SgemmDesc * len(members))()
+        for d, (ta, tb, M, N, K, A, lda, B, ldb, C) in zip(descs, members):
+            d.transA, d.transB, d.M, d.N, d.K, d.A, d.lda, d.B, d.ldb, d.C, d.ldc, d.epilogue, d.bias = ta, tb, M, N, K, A, lda, B, ldb, C, N, L.EPI_NONE, None
+
+        def grouped():
+            L.call("endia_hip_sgemm_grouped", len(members), descs)
+
+        def one_by_one():
+            for (ta, tb, M, N, K, A, lda, B, ldb, C) in members:
+                L.call("endia_hip_sgemm", ta, tb, M, N, K, A, lda, B, ldb, C, N, 1, 0, 0, 0, L.EPI_NONE, L.OP_IDENTITY, None, None, None)
+
+        flops = sum(2.0 * m[2] * m[3] * m[4] for m in members)
+        row = {"products": name}
+        for label, fn in (("one_by_one", one_by_one), ("grouped", grouped)):
+            for _ in range(warm // len(members)):
+                fn()
+            L.call("endia_hip_timer_start", 1)
+            for _ in range(reps):
+                fn()
+            L.call("endia_hip_timer_stop", 1)
+            L.call("endia_hip_timer_elapsed_ms", 1, ctypes.byref(ms))
+            us = 1e3 * ms.value / reps
+            row[label + "_us"] = us
+            row[label + "_tflops"] = flops / (us * 1e-6) / 1e12
+        row["frac"] = row["grouped_tflops"] / FP32_MFMA_PEAK_TFLOPS
+        rows.append(row)
+        for m in members:
+            for ptr in (m[5], m[7], m[9]):
+                L.call("endia_hip_free", ptr)
+    return rows
+
+
 def conv_table(reps=10, only=None):
     """conv2d at the benchmark configuration: x [64,64,56,56], w [128,64,3,3], stride 1, pad 1 (fp32, NCHW).
     Algorithmic flops per pass: 2*N*K*C*R*S*P*Q = 29.6 GFLOP for each of forward, data and weight gradient."""
@@ -775,7 +834,8 @@ def main():
                "kernels": conv_table(max(args.steps, 1))}
     elif args.workload == "gemm_mid":
         out = {"metric": "fp32 GEMM launches of the mid-size products, sustained clock", "device": dev_name,
-               "reps": max(args.steps, 1), "kernels": gemm_mid_table(max(args.steps, 1))}
+               "reps": max(args.steps, 1), "kernels": gemm_mid_table(max(args.steps, 1)),
+               "grouped": gemm_grouped_table(max(args.steps, 1))}
     elif args.workload == "kernels":
         out = {"metric": "per-kernel roofline at the wide-MLP shape (4096 x 4096 operands)", "device": dev_name,
                "reps": max(args.steps, 1), "kernels": kernel_table(max(args.steps, 1))}

@@ -63,6 +63,12 @@ MLP_MAX_LAYERS, MLP_MAX_WIDTH = 16, 128
 class MlpDesc(ctypes.Structure):
     _fields_ = [("layers", c_int32), ("act", c_int32), ("batch", c_int64), ("widths", c_int64 * (MLP_MAX_LAYERS + 1))]
 
+class SgemmDesc(ctypes.Structure):
+    _fields_ = [("transA", c_int32), ("transB", c_int32), ("M", c_int64), ("N", c_int64), ("K", c_int64), ("A", c_void_p),
+                ("lda", c_int64), ("B", c_void_p), ("ldb", c_int64), ("C", c_void_p), ("ldc", c_int64), ("epilogue", c_int32),
+                ("bias", c_void_p)]
+
+
 _fp = c_void_p  # device pointers travel as plain addresses
 _i64p = POINTER(c_int64)
 
@@ -94,6 +100,7 @@ SIGNATURES = {
     "endia_hip_strided_scatter": [c_int32, _i64p, _i64p, c_int64, _fp, _fp, c_int32, c_int32],
     "endia_hip_sgemm": [c_int32, c_int32, c_int64, c_int64, c_int64, _fp, c_int64, _fp, c_int64, _fp, c_int64,
                         c_int64, c_int64, c_int64, c_int64, c_int32, c_int32, _fp, _fp, _fp],
+    "endia_hip_sgemm_grouped": [c_int32, POINTER(SgemmDesc)],
     "endia_hip_linear_bwd": [c_int64, c_int64, c_int64, _fp, _fp, _fp, c_int32, _fp, _fp, _fp, _fp],
     "endia_hip_mlp_fwd": [POINTER(MlpDesc), _fp, POINTER(c_void_p), POINTER(c_void_p), POINTER(c_void_p)],
     "endia_hip_mlp_fwd_mse": [POINTER(MlpDesc), _fp, POINTER(c_void_p), POINTER(c_void_p), _fp, POINTER(c_void_p), _fp, _fp],

@@ -26,6 +26,7 @@
 
 #include <stdlib.h>
 
+#include <algorithm>
 #include <type_traits>
 #include <vector>
 
@@ -448,6 +449,153 @@ extern "C" int32_t endia_hip_sgemm(int32_t transA, int32_t transB, int64_t M, in
   ENDIA_REQUIRE_INIT();
   return endia::sgemm_impl(transA, transB, M, N, K, A, lda, B, ldb, C, ldc, batch, strideA, strideB,
                            strideC, epilogue, act, bias, aux_in, aux_out);
+}
+
+namespace endia {
+
+// endia_hip_sgemm_grouped: which members share a launch. A member that can run on the 256 x 128 one-wave-per-SIMD tile
+// is a number of equal tiles, each a number of K tiles long; a launch puts one work-group on every CU, in block order,
+// and a CU takes the next block when it is done (longest first: the caller's blocks are sorted that way). A set of
+// members is worth one launch when that schedule keeps the CUs busy: its length, priced at what a K tile of this
+// kernel takes, has to beat the members launched one by one at the rate the shared-CU tiles reach on such products.
+namespace {
+struct Member {
+  int index;        // in the caller's array
+  int64_t tiles;    // 256 x 128 tiles
+  int64_t ktiles;   // K tiles of 32 per tile
+  double alone_us;  // estimate for endia_hip_sgemm on it alone
+};
+
+// length, in K tiles, of the schedule of `set` (sorted by ktiles, descending) on `cus` CUs
+int64_t schedule_length(const std::vector<Member>& set, int64_t cus) {
+  std::vector<int64_t> busy((size_t)cus, 0);  // a heap would do; the sets are a few hundred tiles
+  int64_t longest = 0;
+  for (const Member& m : set)
+    for (int64_t t = 0; t < m.tiles; ++t) {
+      size_t at = 0;
+      for (size_t c = 1; c < busy.size(); ++c)
+        if (busy[c] < busy[at]) at = c;
+      busy[at] += m.ktiles;
+      if (busy[at] > longest) longest = busy[at];
+    }
+  return longest;
+}
+constexpr double kGroupFixedUs = 11.4, kGroupKtileUs = 3.57;  // measured: 2 x (2048 x 2048 x 1024) 125.7 us, 4 x (1024 x 2048 x 2048) 240.4 us
+constexpr double kAloneTflops = 113.0;                        // what such a product reaches alone (64 x 64 tiles, K split in the launch)
+}  // namespace
+
+int32_t sgemm_grouped_impl(int32_t count, const endia_hip_sgemm_desc* d) {
+  ENDIA_CHECK_ARG(count >= 0 && count <= 64, "sgemm_grouped: count %d out of [0, 64]", count);
+  ENDIA_CHECK_ARG(count == 0 || d != nullptr, "sgemm_grouped: null descriptors");
+  const int64_t cus = ctx().cu_count;
+  std::vector<Member> can;
+  std::vector<int> alone;
+  for (int i = 0; i < count; ++i) {
+    const endia_hip_sgemm_desc& m = d[i];
+    const int epi = m.epilogue & 0xff;
+    ENDIA_CHECK_ARG((epi == ENDIA_EPI_NONE || epi == ENDIA_EPI_BIAS) && (m.epilogue & ~(0xff | ENDIA_GEMM_ACCUMULATE)) == 0,
+                    "sgemm_grouped: member %d: epilogue 0x%x is not NONE or BIAS, optionally with ACCUMULATE", i, m.epilogue);
+    ENDIA_CHECK_ARG(m.M >= 0 && m.N >= 0 && m.K >= 0 && m.M < (1ll << 31) && m.N < (1ll << 31) && m.K < (1ll << 31),
+                    "sgemm_grouped: member %d: bad dimensions", i);
+    const bool a_ok = aligned16(m.A) && m.lda % 4 == 0 && (m.transA ? m.M % 4 == 0 : m.K % 4 == 0);
+    const bool b_ok = aligned16(m.B) && m.ldb % 4 == 0 && (m.transB ? m.K % 4 == 0 : m.N % 4 == 0);
+    const int64_t tiles = ceil_div64(m.M, 256) * ceil_div64(m.N, 128);
+    const bool fits = (double)(ceil_div64(m.M, 256) * 256) * (double)(ceil_div64(m.N, 128) * 128) <= 1.1 * (double)m.M * (double)m.N;
+    const bool lone_ok = a_ok && b_ok && m.A && m.B && m.C && (epi != ENDIA_EPI_BIAS || m.bias) && m.K >= 256 && fits && tiles < cus &&
+                         m.lda >= (m.transA ? m.M : m.K) && m.ldb >= (m.transB ? m.K : m.N) && m.ldc >= m.N &&
+                         m.lda < (1ll << 22) && m.ldb < (1ll << 22) && (m.transA ? m.K : m.M) * m.lda < (1ll << 29) &&
+                         (m.transB ? m.N : m.K) * m.ldb < (1ll << 29) && g_forced_tile == 0;
+    if (lone_ok) can.push_back({i, tiles, ceil_div64(m.K, BK), 2.0 * (double)m.M * (double)m.N * (double)m.K / (kAloneTflops * 1e6)});
+    else alone.push_back(i);
+  }
+  std::stable_sort(can.begin(), can.end(), [](const Member& a, const Member& b) { return a.ktiles > b.ktiles; });
+  std::vector<std::vector<Member>> groups;
+  std::vector<bool> used(can.size(), false);
+  for (size_t i = 0; i < can.size(); ++i) {
+    if (used[i]) continue;
+    std::vector<Member> set{can[i]};
+    used[i] = true;
+    auto gain = [&](const std::vector<Member>& v) {  // time saved over launching the members one by one
+      double sum = 0.0;
+      for (const Member& m : v) sum += m.alone_us;
+      return sum - (kGroupFixedUs + kGroupKtileUs * (double)schedule_length(v, cus));
+    };
+    double best = gain(set);
+    // grow the set with whichever remaining member improves the saving most, until nothing does
+    while ((int)set.size() < kMaxGroup) {
+      size_t pick = can.size();
+      double pick_gain = best;
+      for (size_t j = i + 1; j < can.size(); ++j) {
+        if (used[j]) continue;
+        std::vector<Member> trial = set;
+        trial.push_back(can[j]);
+        std::stable_sort(trial.begin(), trial.end(), [](const Member& a, const Member& b) { return a.ktiles > b.ktiles; });
+        const double gj = gain(trial);
+        if (gj > pick_gain + 1.0) { pick = j; pick_gain = gj; }
+      }
+      if (pick == can.size()) break;
+      set.push_back(can[pick]);
+      std::stable_sort(set.begin(), set.end(), [](const Member& a, const Member& b) { return a.ktiles > b.ktiles; });
+      used[pick] = true;
+      best = pick_gain;
+    }
+    if (set.size() >= 2 && best > 0.0) groups.push_back(set);
+    else
+      for (const Member& m : set) alone.push_back(m.index);  // (a set of one never beats its own launch)
+  }
+  hipStream_t s = ctx().stream;
+  for (const std::vector<Member>& set : groups) {
+    GroupArgs g{};
+    g.count = (int)set.size();
+    double flops = 0.0;
+    for (size_t k = 0; k < set.size(); ++k) {
+      const endia_hip_sgemm_desc& m = d[set[k].index];
+      GemmArgs& p = g.p[k];
+      p.A = m.A; p.B = m.B; p.C = m.C; p.bias = m.bias;
+      p.lda = m.lda; p.ldb = m.ldb; p.ldc = m.ldc;
+      p.M = (int)m.M; p.N = (int)m.N; p.K = (int)m.K;
+      p.tiles_m = (int)ceil_div64(m.M, 256); p.tiles_n = (int)ceil_div64(m.N, 128);
+      p.act = ENDIA_OP_IDENTITY;
+      p.accumulate = (m.epilogue & ENDIA_GEMM_ACCUMULATE) ? 1 : 0;
+      g.first[k + 1] = g.first[k] + (int)set[k].tiles;
+      g.kind[k] = (m.transA ? 2 : 0) + (m.transB ? 0 : 1) + ((m.epilogue & 0xff) == ENDIA_EPI_BIAS ? 4 : 0);
+      flops += 2.0 * (double)m.M * (double)m.N * (double)m.K;
+    }
+    const bool timed = g_timing.on && !ctx().capturing;
+    if (timed) {
+      if (g_timing.used == g_timing.start.size()) {
+        hipEvent_t a, b;
+        ENDIA_HIP_CALL(hipEventCreate(&a));
+        ENDIA_HIP_CALL(hipEventCreate(&b));
+        g_timing.start.push_back(a);
+        g_timing.stop.push_back(b);
+      }
+      ENDIA_HIP_CALL(hipEventRecord(g_timing.start[g_timing.used], s));
+    }
+    int32_t rc = launch_lone_grouped_256x128(g, s);
+    if (rc) return rc;
+    if (timed) {
+      ENDIA_HIP_CALL(hipEventRecord(g_timing.stop[g_timing.used], s));
+      g_timing.used++;
+      g_timing.flops += flops;
+    }
+    ENDIA_LAUNCH_CHECK();
+  }
+  std::sort(alone.begin(), alone.end());
+  for (int i : alone) {
+    const endia_hip_sgemm_desc& m = d[i];
+    int32_t rc = sgemm_impl(m.transA, m.transB, m.M, m.N, m.K, m.A, m.lda, m.B, m.ldb, m.C, m.ldc, 1, 0, 0, 0, m.epilogue,
+                            ENDIA_OP_IDENTITY, m.bias, nullptr, nullptr);
+    if (rc) return rc;
+  }
+  return ENDIA_HIP_OK;
+}
+
+}  // namespace endia
+
+extern "C" int32_t endia_hip_sgemm_grouped(int32_t count, const endia_hip_sgemm_desc* members) {
+  ENDIA_REQUIRE_INIT();
+  return endia::sgemm_grouped_impl(count, members);
 }
 
 extern "C" int32_t endia_hip_gemm_force_tile(int32_t tile) {

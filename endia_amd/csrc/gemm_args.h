@@ -79,6 +79,18 @@ __device__ __forceinline__ void epilogue_store(const GemmArgs& p, float* __restr
   epilogue_apply<EPI>(p, C, aux_out, row, col, v, bias_v, aux_v);
 }
 
+// Several independent products in one launch of the 256 x 128 one-wave-per-SIMD tile (gemm_lone_grouped.hip): the
+// work-groups [first[i], first[i + 1]) are the tiles of product i. kind = form (0: A and B K-major, 1: A only, 2: B
+// only, 3: neither) + 4 for the bias epilogue; accumulation is the member's own flag.
+constexpr int kMaxGroup = 8;
+struct GroupArgs {
+  int count;
+  int first[kMaxGroup + 1];
+  int kind[kMaxGroup];
+  GemmArgs p[kMaxGroup];
+};
+int32_t launch_lone_grouped_256x128(const GroupArgs& g, hipStream_t s);
+
 // Launcher of the shared-CU tiles (tile = 64 or 128) for operands read 4 bytes at a time (gemm_unaligned.hip).
 void launch_mfma_unaligned(const GemmArgs& p, int epi, int tile, bool a_vec, bool b_vec, int transA, int transB, dim3 grid, hipStream_t s);
 

@@ -145,6 +145,27 @@ ENDIA_API int32_t endia_hip_graph_destroy(int64_t handle);
 ENDIA_API int32_t endia_hip_gemm_timing_begin(void);
 ENDIA_API int32_t endia_hip_gemm_timing_end(int64_t* launches, double* total_ms, double* total_flops);
 
+/* ---- several independent fp32 products in one call. No counterpart in the reference, whose backward pass issues its
+ *      matmul VJPs one at a time (autograd/functional.mojo:46-65, matmul_op.mojo:278-283): a second-order pass holds many
+ *      products of 1024 x 2048 x 2048 that do not depend on each other, each too small to fill the chip, and members that
+ *      fit together share one launch of the 256 x 128 one-wave-per-SIMD tile (one tile per CU); the others run as
+ *      endia_hip_sgemm would run them. Results are those of endia_hip_sgemm on every member in turn (the order of the
+ *      additions along K may differ). No member's C may overlap another member's A, B or C. epilogue: ENDIA_EPI_NONE
+ *      or ENDIA_EPI_BIAS (bias[n] added), optionally | ENDIA_GEMM_ACCUMULATE. count <= 64. */
+typedef struct endia_hip_sgemm_desc {
+  int32_t transA, transB;
+  int64_t M, N, K;
+  const float* A;
+  int64_t lda;
+  const float* B;
+  int64_t ldb;
+  float* C;
+  int64_t ldc;
+  int32_t epilogue;
+  const float* bias;
+} endia_hip_sgemm_desc;
+ENDIA_API int32_t endia_hip_sgemm_grouped(int32_t count, const endia_hip_sgemm_desc* members);
+
 /* Tile choice of the fp32 matrix-core kernels behind endia_hip_sgemm (and everything built on it). No counterpart in the
  * reference: a hook for tests and tuning. tile = 0 (the default) lets every call choose by shape; 64, 128, 256 or 256128
  * makes every later call that runs on the matrix cores use the 64 x 64, 128 x 128, 256 x 256 or 256 x 128 tile (all

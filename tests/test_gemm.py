@@ -105,6 +105,82 @@ def test_sgemm_unaligned_operands_on_the_matrix_cores(dev, M, N, K, pad_a, pad_b
         assert_close(dev.get(dsum, (N,)), B.astype(np.float64).sum(0), what="column sums of B")
 
 
+def _grouped(dev, members):
+    """members: dicts with ta, tb, A, B (host arrays as stored), optional bias, C0 (accumulate). Runs them through
+    endia_hip_sgemm_grouped and returns the outputs."""
+    import ctypes
+    descs = (L.SgemmDesc * len(members))()
+    outs = []
+    for d, m in zip(descs, members):
+        A, B, ta, tb = m["A"], m["B"], m["ta"], m["tb"]
+        M, K = (A.shape[1], A.shape[0]) if ta else A.shape
+        N = B.shape[0] if tb else B.shape[1]
+        dC = dev.put(m["C0"]) if m.get("C0") is not None else dev.alloc(max(M * N * 4, 4))
+        d.transA, d.transB, d.M, d.N, d.K = ta, tb, M, N, K
+        d.A, d.lda, d.B, d.ldb, d.C, d.ldc = dev.put(A), A.shape[1], dev.put(B), B.shape[1], dC, N
+        d.epilogue = (L.EPI_BIAS if m.get("bias") is not None else L.EPI_NONE) | (L.GEMM_ACCUMULATE if m.get("C0") is not None else 0)
+        d.bias = dev.put(m["bias"]) if m.get("bias") is not None else None
+        outs.append((dC, (M, N)))
+    dev.call("endia_hip_sgemm_grouped", len(members), descs)
+    return [dev.get(p, shape) for p, shape in outs]
+
+
+def _member(rng, ta, tb, M, N, K, bias=False, acc=False):
+    m = {"ta": ta, "tb": tb, "A": rng.standard_normal((K, M) if ta else (M, K)).astype(np.float32),
+         "B": (rng.standard_normal((N, K) if tb else (K, N)) / np.sqrt(K)).astype(np.float32)}
+    if bias:
+        m["bias"] = rng.standard_normal(N).astype(np.float32)
+    if acc:
+        m["C0"] = rng.standard_normal((M, N)).astype(np.float32)
+    return m
+
+
+def _member_ref(m):
+    opA, opB = (m["A"].T if m["ta"] else m["A"]), (m["B"].T if m["tb"] else m["B"])
+    ref = opA.astype(np.float64) @ opB.astype(np.float64)
+    if m.get("bias") is not None:
+        ref = ref + m["bias"]
+    if m.get("C0") is not None:
+        ref = ref + m["C0"]
+    return ref
+
+
+@pytest.mark.parametrize("case", ["four_forms", "two_wide", "mixed_lengths", "ragged", "leftovers", "small_and_odd"])
+def test_sgemm_grouped(dev, case):
+    """endia_hip_sgemm_grouped: independent products that share one launch of the 256 x 128 tile (one tile per CU), in
+    every transpose form, with the bias epilogue and accumulation, ragged edges, members of different reduction lengths,
+    and members that no shared launch takes (they run as endia_hip_sgemm would run them). Against float64 and, bit for
+    bit, against a second run."""
+    rng = np.random.default_rng(len(case))
+    if case == "four_forms":      # 4 x 64 tiles = one per CU, all four forms, one with bias, one accumulating
+        ms = [_member(rng, 0, 0, 1024, 2048, 512, bias=True), _member(rng, 0, 1, 1024, 2048, 512), _member(rng, 1, 0, 1024, 2048, 512, acc=True),
+              _member(rng, 1, 1, 1024, 2048, 512)]
+    elif case == "two_wide":      # 2 x 128 tiles
+        ms = [_member(rng, 1, 0, 2048, 2048, 256), _member(rng, 0, 0, 2048, 2048, 256, acc=True, bias=True)]
+    elif case == "mixed_lengths":  # 2 x 64 long tiles and 2 x 128 tiles half as long: the short ones fill in behind
+        ms = [_member(rng, 1, 0, 2048, 2048, 256), _member(rng, 0, 1, 1024, 2048, 512), _member(rng, 0, 0, 2048, 2048, 256),
+              _member(rng, 0, 0, 1024, 2048, 512, bias=True)]
+    elif case == "ragged":        # extents that are not multiples of the tile or of the K tile
+        ms = [_member(rng, 0, 0, 1000, 2040, 500), _member(rng, 0, 1, 1020, 2000, 516, acc=True), _member(rng, 1, 0, 1016, 1944, 260),
+              _member(rng, 1, 1, 1024, 2048, 300, bias=True)]
+    elif case == "leftovers":     # five equal members: four share a launch, the fifth runs alone
+        ms = [_member(rng, i % 2, 0, 1024, 2048, 512, acc=(i == 4)) for i in range(5)]
+    else:                          # nothing here fits the shared launch: too small, unaligned, too short a reduction
+        ms = [_member(rng, 0, 0, 64, 64, 64), _member(rng, 0, 1, 129, 131, 67, bias=True), _member(rng, 1, 0, 1024, 2048, 128),
+              _member(rng, 0, 0, 4, 4, 4, acc=True)]
+    got = _grouped(dev, ms)
+    for k, (c, m) in enumerate(zip(got, ms)):
+        assert_close(c, _member_ref(m), what="%s member %d" % (case, k))
+    again = _grouped(dev, ms)
+    for a, b in zip(got, again):
+        np.testing.assert_array_equal(a, b)
+    with pytest.raises(L.EndiaHipError):  # an epilogue the grouped call does not take
+        ms[0]["bias"] = None
+        descs = (L.SgemmDesc * 1)()
+        descs[0].epilogue = L.EPI_ACT_GRAD
+        dev.call("endia_hip_sgemm_grouped", 1, descs)
+
+
 def test_sgemm_few_outputs_batched_accumulate(dev):
     """The one-group-per-output kernel with a batch, a broadcast operand and accumulation into C."""
     rng = np.random.default_rng(77)
