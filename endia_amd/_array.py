@@ -29,27 +29,35 @@ _CACHE_MAX_TOTAL = 256 << 20
 class Buffer:
     """One allocation from the library's pool; returned to the pool when the last view dies."""
 
-    __slots__ = ("ptr", "nbytes", "captured")
+    __slots__ = ("address", "nbytes", "captured", "pending")
 
     def __init__(self, nbytes):
         nbytes = int(nbytes)
         self.nbytes = nbytes
         self.captured = L.capturing
+        self.pending = False  # a parked product (see _lib.park_product) has yet to write this buffer
         if not L.capturing:
             held = _FREE.get(nbytes)
             if held:
-                self.ptr = held.pop()
+                self.address = held.pop()
                 _FREE_BYTES[0] -= nbytes
                 return
         p = ctypes.c_void_p()
         L.call("endia_hip_malloc", nbytes, ctypes.byref(p))
-        self.ptr = p.value or 0
+        self.address = p.value or 0
+
+    @property
+    def ptr(self):
+        """The device address, for a kernel argument or a copy: whatever is still to write this buffer is launched first."""
+        if self.pending:
+            L.flush(self)
+        return self.address
 
     def __del__(self):
-        ptr = getattr(self, "ptr", 0)
+        ptr = getattr(self, "address", 0)
         if not ptr:
             return
-        self.ptr = 0
+        self.address = 0
         try:
             if (not self.captured and not L.capturing and self.nbytes <= _CACHE_MAX_BUFFER
                     and _FREE_BYTES[0] + self.nbytes <= _CACHE_MAX_TOTAL):

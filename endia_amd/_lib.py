@@ -100,7 +100,7 @@ SIGNATURES = {
     "endia_hip_strided_scatter": [c_int32, _i64p, _i64p, c_int64, _fp, _fp, c_int32, c_int32],
     "endia_hip_sgemm": [c_int32, c_int32, c_int64, c_int64, c_int64, _fp, c_int64, _fp, c_int64, _fp, c_int64,
                         c_int64, c_int64, c_int64, c_int64, c_int32, c_int32, _fp, _fp, _fp],
-    "endia_hip_sgemm_grouped": [c_int32, POINTER(SgemmDesc)],
+    "endia_hip_sgemm_grouped": [c_int32, POINTER(SgemmDesc), c_int32, POINTER(c_int32)],
     "endia_hip_linear_bwd": [c_int64, c_int64, c_int64, _fp, _fp, _fp, c_int32, _fp, _fp, _fp, _fp],
     "endia_hip_mlp_fwd": [POINTER(MlpDesc), _fp, POINTER(c_void_p), POINTER(c_void_p), POINTER(c_void_p)],
     "endia_hip_mlp_fwd_mse": [POINTER(MlpDesc), _fp, POINTER(c_void_p), POINTER(c_void_p), _fp, POINTER(c_void_p), _fp, _fp],
@@ -188,14 +188,92 @@ def ensure_init(device=0):
 _entry = {}
 
 
-def call(name, *args):
-    """Call an entry point on the initialised library and raise on a non-zero status."""
+def _raw_call(name, *args):
     fn = _entry.get(name)
     if fn is None:
         fn = _entry[name] = getattr(ensure_init(), name)
     code = fn(*args)
     if code:
         check(code)
+
+
+# ---- products waiting for a shared launch -----------------------------------------------------------------
+# A backward pass (above all a second-order one) issues many fp32 products that do not depend on each other, each too
+# small to fill the chip. functional._sgemm parks such a product here instead of launching it; flush() hands everything
+# parked to endia_hip_sgemm_grouped, which lets the members that fit together share a launch. What keeps this invisible:
+#   * a parked product's output buffer is marked `pending`, and reading the address of a pending buffer (Buffer.ptr,
+#     the only way to it) flushes first, so nothing ever consumes a result that has not been launched;
+#   * every library call flushes first unless it is one of _WRITES_FRESH below, the entry points this package only ever
+#     calls with outputs it has just allocated: nothing parked can depend on, or be overtaken by, such a call (a parked
+#     product holds its operands' buffers, so a fresh buffer is never one of them). Everything that writes into existing
+#     memory, synchronises, copies to the host, records or replays a graph flushes;
+#   * a product that accumulates into a buffer which a parked product reads or writes flushes before it is parked.
+_WRITES_FRESH = frozenset({
+    "endia_hip_malloc", "endia_hip_free", "endia_hip_binary", "endia_hip_unary_fwd", "endia_hip_unary_vjp",
+    "endia_hip_unary_vjp_from_output", "endia_hip_ew_program", "endia_hip_reduce_add", "endia_hip_reduce",
+    "endia_hip_strided_copy", "endia_hip_mse_fwd_bwd", "endia_hip_complex_pack", "endia_hip_linear_bwd",
+    "endia_hip_conv2d_out_shape", "endia_hip_conv3d_out_shape", "endia_hip_pool_out_shape",
+})
+_parked = []          # (fields of an endia_hip_sgemm_desc, buffers kept alive, output buffer)
+MAX_PARKED = 16
+defer_products = [True]  # tests switch the parking off to compare
+flush_observer = [None]  # tests and probes: called with (descriptor fields of what was parked, index needed or -1, launched flags)
+
+
+def park_product(fields, buffers, out_buffer):
+    if len(_parked) >= MAX_PARKED:
+        flush()
+    out_buffer.pending = True
+    _parked.append((fields, buffers, out_buffer))
+
+
+def parked_uses(buffer):
+    """True when a parked product reads or writes `buffer`."""
+    for _, buffers, out in _parked:
+        if out is buffer:
+            return True
+        for b in buffers:
+            if b is buffer:
+                return True
+    return False
+
+
+def flush(need=None):
+    """Launch what is parked, in one endia_hip_sgemm_grouped call: everything, or, when `need` names the output buffer
+    somebody is about to read, that product and whichever parked products make its launch a better one (the rest stay
+    parked and may find better company later)."""
+    if not _parked:
+        return
+    items = _parked[:]
+    index = -1
+    if need is not None:
+        for i, (_, _, out) in enumerate(items):
+            if out is need:
+                index = i
+        if index < 0:
+            return
+    descs = (SgemmDesc * len(items))()
+    for d, (f, _, _) in zip(descs, items):
+        (d.transA, d.transB, d.M, d.N, d.K, d.A, d.lda, d.B, d.ldb, d.C, d.ldc, d.epilogue, d.bias) = f
+    done = (c_int32 * len(items))()
+    del _parked[:]  # (nothing below comes back here: the raw call flushes nothing)
+    try:
+        _raw_call("endia_hip_sgemm_grouped", len(items), descs, index, done)
+    finally:
+        if flush_observer[0] is not None:
+            flush_observer[0]([item[0] for item in items], index, list(done))
+        for item, flag in zip(items, done):
+            if flag or index < 0:
+                item[2].pending = False
+            else:
+                _parked.append(item)
+
+
+def call(name, *args):
+    """Call an entry point on the initialised library and raise on a non-zero status."""
+    if _parked and name not in _WRITES_FRESH and not (name == "endia_hip_sgemm" and not (args[15] & GEMM_ACCUMULATE)):
+        flush()
+    _raw_call(name, *args)
 
 
 def i64_array(values):

@@ -27,6 +27,9 @@
 #include <stdlib.h>
 
 #include <algorithm>
+#include <functional>
+#include <map>
+#include <queue>
 #include <type_traits>
 #include <vector>
 
@@ -468,15 +471,15 @@ struct Member {
 
 // length, in K tiles, of the schedule of `set` (sorted by ktiles, descending) on `cus` CUs
 int64_t schedule_length(const std::vector<Member>& set, int64_t cus) {
-  std::vector<int64_t> busy((size_t)cus, 0);  // a heap would do; the sets are a few hundred tiles
+  std::priority_queue<int64_t, std::vector<int64_t>, std::greater<int64_t>> busy;  // when each CU is free again
+  for (int64_t c = 0; c < cus; ++c) busy.push(0);
   int64_t longest = 0;
   for (const Member& m : set)
     for (int64_t t = 0; t < m.tiles; ++t) {
-      size_t at = 0;
-      for (size_t c = 1; c < busy.size(); ++c)
-        if (busy[c] < busy[at]) at = c;
-      busy[at] += m.ktiles;
-      if (busy[at] > longest) longest = busy[at];
+      const int64_t end = busy.top() + m.ktiles;
+      busy.pop();
+      busy.push(end);
+      if (end > longest) longest = end;
     }
   return longest;
 }
@@ -484,13 +487,75 @@ constexpr double kGroupFixedUs = 11.4, kGroupKtileUs = 3.57;  // measured: 2 x (
 constexpr double kAloneTflops = 113.0;                        // what such a product reaches alone (64 x 64 tiles, K split in the launch)
 }  // namespace
 
-int32_t sgemm_grouped_impl(int32_t count, const endia_hip_sgemm_desc* d) {
+// The members of `pool` (indices into `can`, none of them used) that should share a launch with can[seed]: grown one
+// member at a time by whichever keeps the CUs busiest, then cut back to the size that saves most over launching the
+// members one by one. Empty when no shared launch beats that.
+static std::vector<size_t> pick_group_uncached(const std::vector<Member>& can, size_t seed, const std::vector<bool>& used, int64_t cus);
+
+// A training loop offers the same shapes in the same order step after step: the choice is looked up by them.
+static std::vector<size_t> pick_group(const std::vector<Member>& can, size_t seed, const std::vector<bool>& used, int64_t cus) {
+  static std::map<std::vector<int64_t>, std::vector<size_t>> known;
+  std::vector<int64_t> key{(int64_t)seed, cus};
+  for (size_t j = 0; j < can.size(); ++j) {
+    key.push_back(used[j] ? -1 : can[j].tiles);
+    key.push_back(can[j].ktiles);
+  }
+  auto it = known.find(key);
+  if (it != known.end()) return it->second;
+  if (known.size() > 4096) known.clear();
+  return known[key] = pick_group_uncached(can, seed, used, cus);
+}
+
+static std::vector<size_t> pick_group_uncached(const std::vector<Member>& can, size_t seed, const std::vector<bool>& used, int64_t cus) {
+  auto by_length = [](const Member& a, const Member& b) { return a.ktiles > b.ktiles; };
+  std::vector<size_t> chosen{seed};
+  std::vector<Member> set{can[seed]};
+  auto work = [](const std::vector<Member>& v) {
+    double w = 0.0;
+    for (const Member& m : v) w += (double)m.tiles * (double)m.ktiles;
+    return w;
+  };
+  auto gain = [&](const std::vector<Member>& v) {
+    double sum = 0.0;
+    for (const Member& m : v) sum += m.alone_us;
+    return sum - (kGroupFixedUs + kGroupKtileUs * (double)schedule_length(v, cus));
+  };
+  double eff = work(set) / ((double)cus * (double)schedule_length(set, cus));
+  double best_gain = 0.0;
+  size_t best_size = 0;  // how many of `chosen` to keep
+  while ((int)set.size() < kMaxGroup) {
+    size_t pick = can.size();
+    double pick_eff = eff;
+    for (size_t j = 0; j < can.size(); ++j) {
+      if (used[j] || std::find(chosen.begin(), chosen.end(), j) != chosen.end()) continue;
+      std::vector<Member> trial = set;
+      trial.push_back(can[j]);
+      std::stable_sort(trial.begin(), trial.end(), by_length);
+      const double e = work(trial) / ((double)cus * (double)schedule_length(trial, cus));
+      if (e > pick_eff + 1e-9) { pick = j; pick_eff = e; }
+    }
+    if (pick == can.size()) break;
+    chosen.push_back(pick);
+    set.push_back(can[pick]);
+    std::stable_sort(set.begin(), set.end(), by_length);
+    eff = pick_eff;
+    const double g = gain(set);
+    if (g > best_gain + 1.0) { best_gain = g; best_size = chosen.size(); }
+  }
+  chosen.resize(best_size);
+  return chosen;
+}
+
+int32_t sgemm_grouped_impl(int32_t count, const endia_hip_sgemm_desc* d, int32_t need, int32_t* launched) {
   ENDIA_CHECK_ARG(count >= 0 && count <= 64, "sgemm_grouped: count %d out of [0, 64]", count);
   ENDIA_CHECK_ARG(count == 0 || d != nullptr, "sgemm_grouped: null descriptors");
+  ENDIA_CHECK_ARG(need >= -1 && need < count, "sgemm_grouped: need = %d with %d members", need, count);
+  ENDIA_CHECK_ARG(need < 0 || launched != nullptr, "sgemm_grouped: need >= 0 reports what it launched: launched is null");
   const int64_t cus = ctx().cu_count;
   std::vector<Member> can;
   std::vector<int> alone;
   for (int i = 0; i < count; ++i) {
+    if (launched) launched[i] = 0;
     const endia_hip_sgemm_desc& m = d[i];
     const int epi = m.epilogue & 0xff;
     ENDIA_CHECK_ARG((epi == ENDIA_EPI_NONE || epi == ENDIA_EPI_BIAS) && (m.epilogue & ~(0xff | ENDIA_GEMM_ACCUMULATE)) == 0,
@@ -506,42 +571,25 @@ int32_t sgemm_grouped_impl(int32_t count, const endia_hip_sgemm_desc* d) {
                          m.lda < (1ll << 22) && m.ldb < (1ll << 22) && (m.transA ? m.K : m.M) * m.lda < (1ll << 29) &&
                          (m.transB ? m.N : m.K) * m.ldb < (1ll << 29) && g_forced_tile == 0;
     if (lone_ok) can.push_back({i, tiles, ceil_div64(m.K, BK), 2.0 * (double)m.M * (double)m.N * (double)m.K / (kAloneTflops * 1e6)});
-    else alone.push_back(i);
+    else if (need < 0 || i == need) alone.push_back(i);
   }
-  std::stable_sort(can.begin(), can.end(), [](const Member& a, const Member& b) { return a.ktiles > b.ktiles; });
   std::vector<std::vector<Member>> groups;
   std::vector<bool> used(can.size(), false);
   for (size_t i = 0; i < can.size(); ++i) {
-    if (used[i]) continue;
-    std::vector<Member> set{can[i]};
-    used[i] = true;
-    auto gain = [&](const std::vector<Member>& v) {  // time saved over launching the members one by one
-      double sum = 0.0;
-      for (const Member& m : v) sum += m.alone_us;
-      return sum - (kGroupFixedUs + kGroupKtileUs * (double)schedule_length(v, cus));
-    };
-    double best = gain(set);
-    // grow the set with whichever remaining member improves the saving most, until nothing does
-    while ((int)set.size() < kMaxGroup) {
-      size_t pick = can.size();
-      double pick_gain = best;
-      for (size_t j = i + 1; j < can.size(); ++j) {
-        if (used[j]) continue;
-        std::vector<Member> trial = set;
-        trial.push_back(can[j]);
-        std::stable_sort(trial.begin(), trial.end(), [](const Member& a, const Member& b) { return a.ktiles > b.ktiles; });
-        const double gj = gain(trial);
-        if (gj > pick_gain + 1.0) { pick = j; pick_gain = gj; }
+    if (used[i] || (need >= 0 && can[i].index != need)) continue;
+    std::vector<size_t> chosen = pick_group(can, i, used, cus);
+    if (chosen.size() >= 2) {
+      std::vector<Member> set;
+      for (size_t c : chosen) {
+        set.push_back(can[c]);
+        used[c] = true;
       }
-      if (pick == can.size()) break;
-      set.push_back(can[pick]);
       std::stable_sort(set.begin(), set.end(), [](const Member& a, const Member& b) { return a.ktiles > b.ktiles; });
-      used[pick] = true;
-      best = pick_gain;
+      groups.push_back(set);
+    } else {
+      used[i] = true;
+      alone.push_back(can[i].index);
     }
-    if (set.size() >= 2 && best > 0.0) groups.push_back(set);
-    else
-      for (const Member& m : set) alone.push_back(m.index);  // (a set of one never beats its own launch)
   }
   hipStream_t s = ctx().stream;
   for (const std::vector<Member>& set : groups) {
@@ -550,6 +598,7 @@ int32_t sgemm_grouped_impl(int32_t count, const endia_hip_sgemm_desc* d) {
     double flops = 0.0;
     for (size_t k = 0; k < set.size(); ++k) {
       const endia_hip_sgemm_desc& m = d[set[k].index];
+      if (launched) launched[set[k].index] = 1;
       GemmArgs& p = g.p[k];
       p.A = m.A; p.B = m.B; p.C = m.C; p.bias = m.bias;
       p.lda = m.lda; p.ldb = m.ldb; p.ldc = m.ldc;
@@ -584,6 +633,7 @@ int32_t sgemm_grouped_impl(int32_t count, const endia_hip_sgemm_desc* d) {
   std::sort(alone.begin(), alone.end());
   for (int i : alone) {
     const endia_hip_sgemm_desc& m = d[i];
+    if (launched) launched[i] = 1;
     int32_t rc = sgemm_impl(m.transA, m.transB, m.M, m.N, m.K, m.A, m.lda, m.B, m.ldb, m.C, m.ldc, 1, 0, 0, 0, m.epilogue,
                             ENDIA_OP_IDENTITY, m.bias, nullptr, nullptr);
     if (rc) return rc;
@@ -593,9 +643,9 @@ int32_t sgemm_grouped_impl(int32_t count, const endia_hip_sgemm_desc* d) {
 
 }  // namespace endia
 
-extern "C" int32_t endia_hip_sgemm_grouped(int32_t count, const endia_hip_sgemm_desc* members) {
+extern "C" int32_t endia_hip_sgemm_grouped(int32_t count, const endia_hip_sgemm_desc* members, int32_t need, int32_t* launched) {
   ENDIA_REQUIRE_INIT();
-  return endia::sgemm_grouped_impl(count, members);
+  return endia::sgemm_grouped_impl(count, members, need, launched);
 }
 
 extern "C" int32_t endia_hip_gemm_force_tile(int32_t tile) {

@@ -53,9 +53,10 @@ __device__ __forceinline__ float act_grad(int act, int from_out, float aux) {
 }
 
 // bias_v = bias[col] and aux_v = aux_in[row, col], fetched by the caller (early, where registers allow)
+// old_v: what C holds at (row, col), fetched by the caller ahead of its stores when it accumulates (null: read here)
 template <int EPI>
 __device__ __forceinline__ void epilogue_apply(const GemmArgs& p, float* __restrict__ C, float* __restrict__ aux_out,
-                                               int row, int col, float v, float bias_v, float aux_v) {
+                                               int row, int col, float v, float bias_v, float aux_v, const float* old_v = nullptr) {
   int64_t off = (int64_t)row * p.ldc + col;
   if (EPI == ENDIA_EPI_BIAS) {
     v += bias_v;
@@ -66,7 +67,7 @@ __device__ __forceinline__ void epilogue_apply(const GemmArgs& p, float* __restr
   } else if (EPI == ENDIA_EPI_ACT_GRAD) {
     v *= act_grad(p.act, p.from_out, aux_v);
   }
-  if (p.accumulate) v += C[off];
+  if (p.accumulate) v += old_v ? *old_v : C[off];
   C[off] = v;
 }
 

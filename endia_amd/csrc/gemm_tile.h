@@ -194,12 +194,26 @@ __device__ __forceinline__ void gemm_tile(const GemmArgs& p, int block, int nblo
     for (int fn = 0; fn < F; ++fn) {
       int col = n0 + wn * 32 * F + fn * 32 + l32;
       if (col >= p.N) continue;
+      // accumulation: the block's sixteen old values are requested together, ahead of the stores (the compiler must
+      // assume that a store changes what a later load reads, and would wait for each in turn)
+      float old[16];
+      if (p.accumulate) {
+#pragma unroll
+        for (int v = 0; v < 16; ++v) {
+          const int row = m0 + wm * 32 * F + fm * 32 + acc_row(v, h);
+          old[v] = row < p.M ? C[(int64_t)row * p.ldc + col] : 0.f;
+        }
+      }
 #pragma unroll
       for (int v = 0; v < 16; ++v) {
         int row = m0 + wm * 32 * F + fm * 32 + acc_row(v, h);
         if (row >= p.M) continue;
-        if constexpr (PRE) epilogue_apply<EPI>(p, C, aux_out, row, col, acc[fm][fn][v], bias_pre, aux_pre[v]);
-        else epilogue_store<EPI>(p, C, aux_in, aux_out, row, col, acc[fm][fn][v]);
+        if constexpr (PRE) epilogue_apply<EPI>(p, C, aux_out, row, col, acc[fm][fn][v], bias_pre, aux_pre[v], &old[v]);
+        else {
+          const float bias_v = (EPI == ENDIA_EPI_BIAS || EPI == ENDIA_EPI_BIAS_ACT) ? p.bias[col] : 0.f;
+          const float aux_v = EPI == ENDIA_EPI_ACT_GRAD ? aux_in[(int64_t)row * p.ldc + col] : 0.f;
+          epilogue_apply<EPI>(p, C, aux_out, row, col, acc[fm][fn][v], bias_v, aux_v, &old[v]);
+        }
       }
     }
 }

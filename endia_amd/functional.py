@@ -1044,10 +1044,40 @@ def _absorb_offer(primal):
 
 
 def _as_bias_row(g, rows, cols):
-    """g viewed as [rows, cols] is one row of memory repeated: its device address, else None."""
+    """g viewed as [rows, cols] is one row of memory repeated: that row as an array of its own, else None."""
     if g.is_complex_ or list(g._shape) != [rows, cols] or g._strides[0] != 0 or (cols > 1 and g._strides[1] != 1):
         return None
-    return g.data_ptr()
+    return Array([cols], _buffer=g._buf, _offset=g._offset)
+
+
+_CUS = []
+
+
+def _sgemm(ta, tb, M, N, K, A_, lda, B_, ldb, out, epi=L.EPI_NONE, bias=None):
+    """One real, unbatched product C = op(A) op(B) (+ bias row, or on top of what C holds) into `out`, a contiguous
+    array. A product that cannot fill the chip alone (fewer 256 x 128 tiles than CUs) but is large enough to be worth a
+    one-tile-per-CU launch is parked (_lib.park_product) so that it can share a launch with the independent products
+    that a backward pass issues next to it; anything else is launched here."""
+    if not _CUS:
+        _CUS.append(L.device_info()[1])
+    tiles = -(-M // 256) * -(-N // 128)
+    parkable = (L.defer_products[0] and not L.capturing and tiles < _CUS[0] and M >= 256 and N >= 128 and K >= 256
+                and lda % 4 == 0 and ldb % 4 == 0 and (epi & 0xff) in (L.EPI_NONE, L.EPI_BIAS))
+    a_ptr, b_ptr = A_.data_ptr(), B_.data_ptr()
+    bias_ptr = bias.data_ptr() if isinstance(bias, Array) else bias
+    if not parkable or (a_ptr | b_ptr) & 15:
+        L.call("endia_hip_sgemm", ta, tb, M, N, K, a_ptr, lda, b_ptr, ldb, out.data_ptr(), N, 1, 0, 0, 0, epi, L.OP_IDENTITY,
+               bias_ptr, None, None)
+        return
+    obuf = out._buf
+    if epi & L.GEMM_ACCUMULATE:  # what is parked and writes, or reads, the buffer this product adds to goes first
+        if obuf.pending:
+            L.flush(obuf)
+        if L.parked_uses(obuf):
+            L.flush()
+    buffers = [A_._buf, B_._buf] + ([bias._buf] if isinstance(bias, Array) else [])
+    c_ptr = obuf.address + 4 * out._offset
+    L.park_product((ta, tb, M, N, K, a_ptr, lda, b_ptr, ldb, c_ptr, N, epi, bias_ptr), buffers, obuf)
 
 
 # --------------------------------------------------------------------------------------------------
@@ -1135,11 +1165,11 @@ def matmul(a, b, vjp_rule=None, _ca=0, _cb=0, _into=None):
     B_, tb, ldb, sb = _gemm_operand(eb)
     batch = _prod(bshape)
     # `_into` (an offer of the reverse walk, see _absorb above): (earlier gradient of this product's shape, exclusive)
-    epi, bias_ptr, out = L.EPI_NONE, None, None
+    epi, bias_row, out = L.EPI_NONE, None, None
     if _into is not None and not a.is_complex_ and len(out_shape) == 2 and M * N * K > 0:
         g0, exclusive = _into
-        bias_ptr = _as_bias_row(g0, M, N)
-        if bias_ptr is not None:
+        bias_row = _as_bias_row(g0, M, N)
+        if bias_row is not None:
             epi = L.EPI_BIAS
         elif exclusive and list(g0._shape) == out_shape and g0.is_contiguous() and not g0.is_complex_:
             epi, out = L.EPI_NONE | L.GEMM_ACCUMULATE, Array(out_shape, _buffer=g0._buf, _offset=g0._offset)
@@ -1152,9 +1182,11 @@ def matmul(a, b, vjp_rule=None, _ca=0, _cb=0, _into=None):
         if a.is_complex_:
             L.call("endia_hip_cgemm", ta, _ca, tb, _cb, M, N, K, A_.data_ptr(), lda, B_.data_ptr(), ldb, out.data_ptr(), N,
                    batch, sa, sb, M * N, _cgemm_algo[0], 0)
+        elif batch == 1 and K > 0:
+            _sgemm(ta, tb, M, N, K, A_, lda, B_, ldb, out, epi, bias_row)
         else:
             L.call("endia_hip_sgemm", ta, tb, M, N, K, A_.data_ptr(), lda, B_.data_ptr(), ldb, out.data_ptr(), N, batch,
-                   sa, sb, M * N, epi, L.OP_IDENTITY, bias_ptr, None, None)
+                   sa, sb, M * N, epi, L.OP_IDENTITY, None, None, None)
 
     def vjp(primals, grad, out_):
         p0, p1 = primals
@@ -1706,16 +1738,26 @@ def _linear_node(out, x, W, b, xs, Ws, act):
             return tot
         accW = in_place(_absorb_offer(pW), [K, N]) if dW is not None and pW is not px else None
         accX = in_place(_absorb_offer(px), [B, K]) if dx is not None and aux is None and pW is not px else None
-        if accW is not None:
-            L.call("endia_hip_sgemm", 1, 0, K, N, B, xs.data_ptr(), K, g.data_ptr(), N, accW.data_ptr(), N, 1, 0, 0, 0,
-                   L.EPI_NONE | L.GEMM_ACCUMULATE | (L.GEMM_COLSUM_B if db is not None else 0), L.OP_IDENTITY, None, None,
-                   db.data_ptr() if db is not None else None)
+        # (the products go through _sgemm, which may park them for a shared launch; a large layer's bias gradient is a
+        # reduction of its own either way, a small one's rides in the weight-gradient launch)
+        split = B * N > (1 << 20)
+        if accW is not None or (dW is not None and split):
+            if db is not None and split:
+                L.call("endia_hip_reduce_add", 2, L.i64_array([B, N]), 1, g.data_ptr(), db.data_ptr(), 1.0, 0)
+                _sgemm(1, 0, K, N, B, xs, K, g, N, accW if accW is not None else dW, L.EPI_NONE | (L.GEMM_ACCUMULATE if accW is not None else 0))
+            else:
+                tgt = accW if accW is not None else dW
+                L.call("endia_hip_sgemm", 1, 0, K, N, B, xs.data_ptr(), K, g.data_ptr(), N, tgt.data_ptr(), N, 1, 0, 0, 0,
+                       L.EPI_NONE | (L.GEMM_ACCUMULATE if accW is not None else 0) | (L.GEMM_COLSUM_B if db is not None else 0),
+                       L.OP_IDENTITY, None, None, db.data_ptr() if db is not None else None)
+            w_done = True
+        else:
+            w_done = False
         if accX is not None:
-            L.call("endia_hip_sgemm", 0, 1, B, K, N, g.data_ptr(), N, Ws.data_ptr(), N, accX.data_ptr(), K, 1, 0, 0, 0,
-                   L.EPI_NONE | L.GEMM_ACCUMULATE, L.OP_IDENTITY, None, None, None)
+            _sgemm(0, 1, B, K, N, g, N, Ws, N, accX, L.EPI_NONE | L.GEMM_ACCUMULATE)
         rest_dx = dx if accX is None else None
-        rest_dW = dW if accW is None else None
-        rest_db = db if accW is None else None
+        rest_dW = dW if not w_done else None
+        rest_db = db if not w_done else None
         if rest_dx is not None or rest_dW is not None or rest_db is not None:
             L.call("endia_hip_linear_bwd", B, K, N, xs.data_ptr(), Ws.data_ptr(), g.data_ptr(), flags,
                    aux.data_ptr() if aux is not None else None, rest_dx.data_ptr() if rest_dx is not None else None,

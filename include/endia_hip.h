@@ -151,7 +151,10 @@ ENDIA_API int32_t endia_hip_gemm_timing_end(int64_t* launches, double* total_ms,
  *      fit together share one launch of the 256 x 128 one-wave-per-SIMD tile (one tile per CU); the others run as
  *      endia_hip_sgemm would run them. Results are those of endia_hip_sgemm on every member in turn (the order of the
  *      additions along K may differ). No member's C may overlap another member's A, B or C. epilogue: ENDIA_EPI_NONE
- *      or ENDIA_EPI_BIAS (bias[n] added), optionally | ENDIA_GEMM_ACCUMULATE. count <= 64. */
+ *      or ENDIA_EPI_BIAS (bias[n] added), optionally | ENDIA_GEMM_ACCUMULATE. count <= 64.
+ *      need = -1 runs every member. need = i (a caller that keeps a list of products it has put off and now has to
+ *      have member i) runs member i and whichever other members make its launch a better one, and leaves the rest to
+ *      the caller. launched (may be null when need = -1) receives one flag per member: 1 = it has been run. */
 typedef struct endia_hip_sgemm_desc {
   int32_t transA, transB;
   int64_t M, N, K;
@@ -164,7 +167,7 @@ typedef struct endia_hip_sgemm_desc {
   int32_t epilogue;
   const float* bias;
 } endia_hip_sgemm_desc;
-ENDIA_API int32_t endia_hip_sgemm_grouped(int32_t count, const endia_hip_sgemm_desc* members);
+ENDIA_API int32_t endia_hip_sgemm_grouped(int32_t count, const endia_hip_sgemm_desc* members, int32_t need, int32_t* launched);
 
 /* Tile choice of the fp32 matrix-core kernels behind endia_hip_sgemm (and everything built on it). No counterpart in the
  * reference: a hook for tests and tuning. tile = 0 (the default) lets every call choose by shape; 64, 128, 256 or 256128

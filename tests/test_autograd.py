@@ -491,6 +491,66 @@ def test_gradient_accumulation_inside_the_product_launch(nd, golden):
     assert_close(a.grad().to_numpy(), one @ an.T + an.T @ one + one @ bn.T, what="matmul(a, a) + matmul(a, b)")
 
 
+def test_parked_products_share_launches(nd):
+    """Mid-size products of a backward pass are parked and launched together (functional._sgemm, _lib.park_product).
+    A two-layer sin model of 1024-wide layers, batch 512: gradient and Hessian-vector product with parking on and off
+    agree, reading any result launches what it depends on, in-place accumulation into a parked product's output keeps
+    its order, and an optimizer step sees finished gradients."""
+    from endia_amd import _lib as L
+    rng = np.random.default_rng(21)
+    Bn, Wd = 512, 1024
+    Wn = [(rng.standard_normal((Wd, Wd)) / np.sqrt(Wd)).astype(np.float32) for _ in range(2)]
+    bn = [(0.1 * rng.standard_normal(Wd)).astype(np.float32) for _ in range(2)]
+    vn = [rng.standard_normal(a.shape).astype(np.float32) for a in (Wn[0], bn[0], Wn[1], bn[1])]
+    xn = rng.standard_normal((Bn, Wd)).astype(np.float32)
+
+    def run():
+        mlp = nd.nn.MLP([Wd] * 3, compute_backward=True, activation="sin", fused=True)
+        for i in range(2):
+            mlp.weights[i], mlp.biases[i] = nd.array(Wn[i], requires_grad=True), nd.array(bn[i], requires_grad=True)
+        out = mlp.forward(nd.array(xn))
+        loss = nd.sum(out * out)
+        loss.backward(create_graph=True)
+        firsts = [p.grad() for p in mlp.params()]
+        hv = nd.grad(outs=firsts, inputs=mlp.params(), grad_outs=[nd.reshape(nd.array(v), f.shape()) for v, f in zip(vn, firsts)])
+        res = [f.to_numpy() for f in firsts] + [h.to_numpy() for h in hv]
+        loss.zero_grad()
+        return res
+
+    parked = run()
+    assert not L._parked
+    L.defer_products[0] = False
+    try:
+        plain = run()
+    finally:
+        L.defer_products[0] = True
+    for k, (a, b) in enumerate(zip(parked, plain)):
+        assert_close(a, b, tol=2e-6, mean_tol=1e-4, what="tensor %d with and without parking" % k)
+    # float64 on the host
+    import torch
+    tW = [torch.tensor(w, dtype=torch.float64, requires_grad=True) for w in Wn]
+    tb = [torch.tensor(b, dtype=torch.float64, requires_grad=True) for b in bn]
+    h = torch.sin(torch.tensor(xn, dtype=torch.float64) @ tW[0] + tb[0])
+    o = h @ tW[1] + tb[1]
+    ps = [tW[0], tb[0], tW[1], tb[1]]
+    gs = torch.autograd.grad((o * o).sum(), ps, create_graph=True)
+    hv = torch.autograd.grad(gs, ps, grad_outputs=[torch.tensor(v, dtype=torch.float64) for v in vn])
+    for k, t in enumerate(list(gs) + list(hv)):
+        assert_close(parked[k], t.detach().numpy(), what="tensor %d vs float64" % k, mean_tol=1e-3)
+    # a first-order step: the optimizer (an in-place writer) must see launched gradients
+    a = nd.array(xn[:, :512].copy())
+    W = nd.array(Wn[0][:512, :512].copy(), requires_grad=True)
+    opt = nd.optim.SGD([W], lr=0.5)
+    y = nd.matmul(a, W)                       # parked (512 x 512 x 512 is below the size that parks: run it anyway)
+    z = nd.matmul(nd.array(xn), nd.array(Wn[1]))  # 512 x 1024 x 1024: parked
+    assert L._parked
+    nd.sum(y).backward()
+    opt.step()
+    assert not L._parked
+    assert_close(W.to_numpy(), Wn[0][:512, :512] - 0.5 * (xn[:, :512].astype(np.float64).T @ np.ones((Bn, 512))), what="SGD after parked products")
+    assert_close(z.to_numpy(), xn.astype(np.float64) @ Wn[1], what="a parked product read later")
+
+
 def test_optimizer_classes(nd, golden):
     g = golden("optim")
     makers = {

@@ -121,7 +121,7 @@ def _grouped(dev, members):
         d.epilogue = (L.EPI_BIAS if m.get("bias") is not None else L.EPI_NONE) | (L.GEMM_ACCUMULATE if m.get("C0") is not None else 0)
         d.bias = dev.put(m["bias"]) if m.get("bias") is not None else None
         outs.append((dC, (M, N)))
-    dev.call("endia_hip_sgemm_grouped", len(members), descs)
+    dev.call("endia_hip_sgemm_grouped", len(members), descs, -1, None)
     return [dev.get(p, shape) for p, shape in outs]
 
 
@@ -178,7 +178,45 @@ def test_sgemm_grouped(dev, case):
         ms[0]["bias"] = None
         descs = (L.SgemmDesc * 1)()
         descs[0].epilogue = L.EPI_ACT_GRAD
-        dev.call("endia_hip_sgemm_grouped", 1, descs)
+        dev.call("endia_hip_sgemm_grouped", 1, descs, -1, None)
+
+
+def test_sgemm_grouped_runs_what_is_needed_and_its_company(dev):
+    """need = i: member i runs together with the members that make its launch a better one, the others are left to
+    the caller (their outputs untouched), and `launched` says which is which. Three products of 1024 x 2048 x 512 and
+    two of 2048 x 2048 x 256 are offered; whatever subset runs, a second call with need = -1 finishes the job."""
+    import ctypes
+    rng = np.random.default_rng(3)
+    ms = [_member(rng, 0, 0, 1024, 2048, 512), _member(rng, 1, 0, 2048, 2048, 256), _member(rng, 0, 1, 1024, 2048, 512),
+          _member(rng, 1, 0, 2048, 2048, 256), _member(rng, 0, 0, 1024, 2048, 512), _member(rng, 0, 0, 8, 8, 8)]
+    descs = (L.SgemmDesc * len(ms))()
+    outs = []
+    for d, m in zip(descs, ms):
+        A, B, ta, tb = m["A"], m["B"], m["ta"], m["tb"]
+        M, K = (A.shape[1], A.shape[0]) if ta else A.shape
+        N = B.shape[0] if tb else B.shape[1]
+        dC = dev.put(np.full((M, N), -7.0, np.float32))
+        d.transA, d.transB, d.M, d.N, d.K = ta, tb, M, N, K
+        d.A, d.lda, d.B, d.ldb, d.C, d.ldc, d.epilogue, d.bias = dev.put(A), A.shape[1], dev.put(B), B.shape[1], dC, N, L.EPI_NONE, None
+        outs.append((dC, (M, N)))
+    done = (ctypes.c_int32 * len(ms))()
+    dev.call("endia_hip_sgemm_grouped", len(ms), descs, 2, done)
+    flags = list(done)
+    assert flags[2] == 1 and flags[5] == 0, flags      # the needed member ran; the tiny one shares no launch and was not needed
+    assert sum(flags) >= 2, flags                      # and it found company
+    for k, ((p, shape), m) in enumerate(zip(outs, ms)):
+        got = dev.get(p, shape)
+        if flags[k]:
+            assert_close(got, _member_ref(m), what="member %d (launched)" % k)
+        else:
+            assert np.all(got == -7.0), "member %d was reported as not launched but its output changed" % k
+    rest = [k for k in range(len(ms)) if not flags[k]]
+    sub = (L.SgemmDesc * len(rest))(*[descs[k] for k in rest])
+    dev.call("endia_hip_sgemm_grouped", len(rest), sub, -1, None)
+    for k, ((p, shape), m) in enumerate(zip(outs, ms)):
+        assert_close(dev.get(p, shape), _member_ref(m), what="member %d" % k)
+    with pytest.raises(L.EndiaHipError):
+        dev.call("endia_hip_sgemm_grouped", len(ms), descs, len(ms), done)
 
 
 def test_sgemm_few_outputs_batched_accumulate(dev):
