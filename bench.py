@@ -36,7 +36,7 @@ HBM_PEAK_GBS = 8000.0
 GEMM_TRAFFIC_BYTES = int((1 * 451.2 + 7 * 449.1 + 7 * 512.3 + 8 * 450.9) / 23 * 1024 * 1024)
 
 
-def build_wide_mlp(nd, width=4096, layers=8, batch=4096, seed=2):
+def build_wide_mlp(nd, width=4096, layers=8, batch=4096, seed=2, fused_backward=False):
     rng = np.random.default_rng(seed)
     std = 1.0 / np.sqrt(width)
     mlp = nd.nn.MLP([width] * (layers + 1), compute_backward=True, activation="tanh", fused=True)
@@ -45,7 +45,7 @@ def build_wide_mlp(nd, width=4096, layers=8, batch=4096, seed=2):
         mlp.biases[i] = nd.array((rng.standard_normal(width) * std).astype(np.float32), requires_grad=True)
     x = nd.array(rng.standard_normal((batch, width)).astype(np.float32))
     y = nd.array(rng.standard_normal((batch, width)).astype(np.float32))
-    opt = nd.optim.Adam(mlp.params(), lr=1e-3, beta1=0.9, beta2=0.999, eps=1e-8)
+    opt = nd.optim.Adam(mlp.params(), lr=1e-3, beta1=0.9, beta2=0.999, eps=1e-8, fused_backward=fused_backward)
     return mlp, opt, x, y
 
 
@@ -726,9 +726,9 @@ def run_sine(nd, steps, warmup, optimizer="sgd", eager=False, per_layer=False):
                                 "value": 1.0 / res[True][0], "ms_per_step": res[True][0] * 1e3, "final_loss": res[True][1]}}
 
 
-def run_wide(nd, steps, warmup):
+def run_wide(nd, steps, warmup, fused_backward=False):
     from endia_amd import _lib as L
-    mlp, opt, x, y = build_wide_mlp(nd)
+    mlp, opt, x, y = build_wide_mlp(nd, fused_backward=fused_backward)
     width, layers, batch = 4096, 8, 4096
     gemm_flops_step = (layers + layers + layers - 1) * 2.0 * batch * width * width
     for _ in range(warmup):
@@ -809,6 +809,8 @@ def main():
     ap.add_argument("--workload", default="wide_mlp", choices=["wide_mlp", "sine_mlp", "kernels", "gemm_mid", "conv2d", "conv2d_kernels", "hvp", "complex_mlp", "complex_mlp_3m"])
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--headline-only", action="store_true", help="wide_mlp: leave the other four configurations out of the line")
+    ap.add_argument("--adam-in-backward", action="store_true", help="wide_mlp: optim.Adam(fused_backward=True), the update of a layer "
+                    "issued by backward() right behind that layer's gradients")
     ap.add_argument("--eager", action="store_true", help="sine_mlp: issue every kernel from the host instead of replaying a graph")
     ap.add_argument("--per-layer", action="store_true", help="sine_mlp: one fused op per layer instead of the whole-model op")
     ap.add_argument("--optimizer", default="sgd", choices=["sgd", "adam"], help="sine_mlp: SGD (the benchmark configuration) or Adam (the reference script's)")
@@ -850,7 +852,9 @@ def main():
         if cpu:
             out["cpu_baseline"] = cpu_baseline_sine(optimizer=args.optimizer)
     else:
-        out = run_wide(nd, args.steps, args.warmup)
+        out = run_wide(nd, args.steps, args.warmup, args.adam_in_backward)
+        if args.adam_in_backward:
+            out["config"]["optimizer"] = "adam, applied by backward() layer by layer (optim.Adam(fused_backward=True))"
         out["device"] = dev_name
         if cpu:
             out["cpu_baseline"] = cpu_baseline_wide()

@@ -105,10 +105,12 @@ class Array:
     _meta = None
     _id = -1
     _consumers = 0
+    _contributions_left = 0  # during a reverse walk: consumers whose VJP has not run yet
     _is_seed = False
     _act_applied = False  # a gradient that already carries the producer's activation derivative
     _grad_fused = None    # such a gradient on its way to this node's own VJP rule; never what grad() returns
     _true_grad = None     # on an _act_applied gradient: a function that computes the gradient without the derivative
+    _on_final_grad = None  # set by an optimizer with fused_backward=True: called by backward() when this leaf's gradient is complete
     _internal = False     # a node that a VJP rule created (the transposes and broadcasts inside a recorded backward pass)
     _absorbed = False     # a VJP result that already includes the gradient its primal held (functional._absorb)
     _offset = 0

@@ -130,9 +130,12 @@ def _reverse_walk(trace, create_graph):
     for node in trace:
         for a in node._args:
             a._consumers += 1
+    for node in trace:
+        node._contributions_left = node._consumers
 
     prev = _building_graph[0]
     _building_graph[0] = bool(create_graph)
+    finished = []
     try:
         for curr in reversed(trace):
             primals = curr._args
@@ -153,6 +156,9 @@ def _reverse_walk(trace, create_graph):
                 grad = None
                 curr._grad = None
             for primal, pg in zip(primals, primals_grads):
+                primal._contributions_left -= 1
+                if primal._on_final_grad is not None and primal._contributions_left == 0 and not create_graph:
+                    finished.append(primal)  # every consumer has contributed once this one is stored
                 if not primal._requires_grad or pg is None:
                     continue
                 if primal.has_grad():
@@ -166,6 +172,12 @@ def _reverse_walk(trace, create_graph):
                 primal.grad_(pg)
                 if not create_graph:
                     pg.clear_args()
+            # An optimizer built with fused_backward=True updates a parameter as soon as its gradient is complete, while
+            # the gradient still sits in the last-level cache; the walk goes on with the other layers meanwhile.
+            while finished:
+                leaf = finished.pop()
+                if leaf._grad is not None:
+                    leaf._on_final_grad(leaf)
     finally:
         _building_graph[0] = prev
 

@@ -424,15 +424,18 @@ int32_t linear_bwd_impl(int64_t B, int64_t K, int64_t N, const float* x, const f
     ENDIA_LAUNCH_CHECK();
     return ENDIA_HIP_OK;
   }
-  if (dW) {
-    int32_t rc = sgemm_impl(1, 0, K, N, B, x, K, g, N, dW, N, 1, 0, 0, 0, ENDIA_EPI_NONE | (db ? ENDIA_GEMM_COLSUM_B : 0),
-                            ENDIA_OP_IDENTITY, nullptr, nullptr, db);
-    if (rc) return rc;
-  } else if (db && N > 0) {
-    int32_t rc = col_reduce(1, B, N, g, db, 1.f);
+  // dx first: the weight gradient is then the last thing written, and an optimizer update issued right behind this call
+  // (optim.Adam(fused_backward=True)) finds it in the last-level cache
+  if (dx) {
+    int32_t rc = sgemm_impl(0, 1, B, K, N, g, N, W, N, dx, K, 1, 0, 0, 0, epi_x, aux ? act_flags : ENDIA_OP_IDENTITY, nullptr, aux, nullptr);
     if (rc) return rc;
   }
-  if (dx) return sgemm_impl(0, 1, B, K, N, g, N, W, N, dx, K, 1, 0, 0, 0, epi_x, aux ? act_flags : ENDIA_OP_IDENTITY, nullptr, aux, nullptr);
+  if (dW) {
+    return sgemm_impl(1, 0, K, N, B, x, K, g, N, dW, N, 1, 0, 0, 0, ENDIA_EPI_NONE | (db ? ENDIA_GEMM_COLSUM_B : 0),
+                      ENDIA_OP_IDENTITY, nullptr, nullptr, db);
+  } else if (db && N > 0) {
+    return col_reduce(1, B, N, g, db, 1.f);
+  }
   return ENDIA_HIP_OK;
 }
 

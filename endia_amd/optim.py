@@ -92,17 +92,41 @@ class Adam:
 
     capturable=True (or the first step() taken while a step is being captured) keeps the counter in device memory
     and updates every parameter tensor in one launch that reads it there, so the step can be replayed as a HIP
-    graph; the bias corrections then come from the device's powf (last-bit differences from the host's)."""
+    graph; the bias corrections then come from the device's powf (last-bit differences from the host's).
 
-    def __init__(self, params, lr=0.001, beta1=0.9, beta2=0.999, eps=1e-8, capturable=False):
+    fused_backward=True (no counterpart in the reference): backward() itself applies this optimizer's update to a
+    parameter the moment that parameter's gradient is complete (every consumer in the graph has contributed), while
+    the gradient is still in the last-level cache and before the walk moves on to the layers below; step() then only
+    updates what backward() did not reach and advances t. Same arithmetic, same results as step() after backward();
+    `p.grad()` stays readable. For loops that run exactly one backward() per step(): a second backward() before
+    step() would update again. Passes with create_graph=True never update. Not together with capturable."""
+
+    def __init__(self, params, lr=0.001, beta1=0.9, beta2=0.999, eps=1e-8, capturable=False, fused_backward=False):
         self.params = list(params)
         self.lr, self.beta1, self.beta2, self.eps = (float(np.float32(v)) for v in (lr, beta1, beta2, eps))
         self.t = 1.0
         self.m = [Array(p.shape()) for p in self.params]
         self.v = [Array(p.shape()) for p in self.params]
         self._t_dev = None
+        if capturable and fused_backward:
+            raise ValueError("Adam: fused_backward and capturable cannot be combined")
         if capturable:
             self._device_counter()
+        self._updated = [False] * len(self.params)
+        if fused_backward:
+            for i, p in enumerate(self.params):
+                p._on_final_grad = (lambda leaf, i=i: self._update(i))
+
+    def _update(self, i):
+        if self._updated[i] or L.capturing:
+            return
+        p = self.params[i]
+        g = _flat_grad(p)
+        assert p.is_contiguous()
+        L.call("endia_hip_adam_step", p.size(), p.data_ptr(), g.data_ptr(), self.m[i].data_ptr(), self.v[i].data_ptr(), self.lr,
+               self.beta1, self.beta2, self.eps, self.t)
+        p.clear_args()
+        self._updated[i] = True
 
     def _device_counter(self):
         if self._t_dev is None:
@@ -132,10 +156,7 @@ class Adam:
             for p in self.params:
                 p.clear_args()
             return
-        for p, m, v in zip(self.params, self.m, self.v):
-            g = _flat_grad(p)
-            assert p.is_contiguous()
-            L.call("endia_hip_adam_step", p.size(), p.data_ptr(), g.data_ptr(), m.data_ptr(), v.data_ptr(), self.lr,
-                   self.beta1, self.beta2, self.eps, self.t)
-            p.clear_args()
+        for i in range(len(self.params)):
+            self._update(i)
+        self._updated = [False] * len(self.params)
         self.t += 1.0

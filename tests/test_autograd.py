@@ -571,6 +571,59 @@ def test_optimizer_classes(nd, golden):
             assert_close(p.to_numpy(), g["%s_p%d" % (name, i + 1)], tol=2e-6, what="%s step %d" % (name, i))
 
 
+@pytest.mark.parametrize("fused", [True, False, "model"])
+def test_adam_applied_inside_backward(nd, fused):
+    """optim.Adam(fused_backward=True): backward() updates each parameter as soon as its gradient is complete. Three
+    steps give bit for bit the parameters, moments and gradients of step() after backward(), for a tanh MLP in every
+    fusion mode, with a weight shared by two layers (its update has to wait for both contributions), and a pass with
+    create_graph=True does not update anything."""
+    rng = np.random.default_rng(17)
+    widths = [12, 32, 32, 5]
+    Wn = [(rng.standard_normal((widths[i], widths[i + 1])) / np.sqrt(widths[i])).astype(np.float32) for i in range(3)]
+    bn = [(0.1 * rng.standard_normal(widths[i + 1])).astype(np.float32) for i in range(3)]
+    xn, yn = rng.standard_normal((20, 12)).astype(np.float32), rng.standard_normal((20, 5)).astype(np.float32)
+
+    def run(inside):
+        mlp = nd.nn.MLP(widths, compute_backward=True, activation="tanh", fused=fused)
+        for i in range(3):
+            mlp.weights[i], mlp.biases[i] = nd.array(Wn[i], requires_grad=True), nd.array(bn[i], requires_grad=True)
+        opt = nd.optim.Adam(mlp.params(), lr=1e-2, fused_backward=inside)
+        x, y = nd.array(xn), nd.array(yn)
+        grads = []
+        for _ in range(3):
+            loss = nd.mse(mlp.forward(x), y)
+            loss.backward()
+            grads.append([p.grad().to_numpy() for p in mlp.params()])
+            opt.step()
+            loss.zero_grad()
+        return [p.to_numpy() for p in mlp.params()], [m.to_numpy() for m in opt.m + opt.v], grads, opt.t
+
+    p1, s1, g1, t1 = run(True)
+    p0, s0, g0, t0 = run(False)
+    assert t1 == t0 == 4.0
+    for a, b in zip(p1 + s1 + sum(g1, []), p0 + s0 + sum(g0, [])):
+        np.testing.assert_array_equal(a, b)
+    if fused == "model":
+        return
+    # one weight used by two layers: updated once, after the second contribution
+    W = nd.array(Wn[1], requires_grad=True)
+    x = nd.array(rng.standard_normal((20, 32)).astype(np.float32))
+    opt = nd.optim.Adam([W], lr=1e-2, fused_backward=True)
+    ref_W = nd.array(Wn[1], requires_grad=True)
+    ref = nd.optim.Adam([ref_W], lr=1e-2)
+    for w, o in ((W, opt), (ref_W, ref)):
+        h = nd.tanh(nd.matmul(x, w))
+        nd.sum(nd.matmul(h, w)).backward()
+        o.step()
+    np.testing.assert_array_equal(W.to_numpy(), ref_W.to_numpy())
+    # a pass that records its graph leaves the parameters alone
+    before = W.to_numpy()
+    nd.sum(nd.matmul(x, W)).backward(create_graph=True)
+    np.testing.assert_array_equal(W.to_numpy(), before)
+    with pytest.raises(ValueError):
+        nd.optim.Adam([W], capturable=True, fused_backward=True)
+
+
 def test_complex_mlp_both_conventions(nd, golden):
     """Identity complex layers, loss = sum |out|^2. `vjp_rule="wirtinger"` gives the Wirtinger-conjugate
     gradients (equal to torch); the default follows the reference's coded rule without conjugation
