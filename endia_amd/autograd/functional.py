@@ -114,7 +114,7 @@ def _offers(primals):
         g = p._grad
         if g is None or not p._requires_grad or p._grad_fused is not None or g._is_seed:
             continue
-        exclusive = sys.getrefcount(g) <= 3 and sys.getrefcount(g._buf) <= 2
+        exclusive = sys.getrefcount(g) <= 3 and sys.getrefcount(g._buf) <= (3 if g._buf.pending else 2)  # (a parked product holds its output buffer)
         if offers is None:
             offers = {}
         offers[id(p)] = (g, exclusive)

@@ -1053,16 +1053,19 @@ def _as_bias_row(g, rows, cols):
 _CUS = []
 
 
+def _would_park(M, N, K):
+    """The size test of _sgemm: fewer 256 x 128 tiles than CUs, yet large enough for a one-tile-per-CU launch."""
+    if not _CUS:
+        _CUS.append(L.device_info()[1])
+    return (L.defer_products[0] and not L.capturing and -(-M // 256) * -(-N // 128) < _CUS[0] and M >= 256 and N >= 128 and K >= 256)
+
+
 def _sgemm(ta, tb, M, N, K, A_, lda, B_, ldb, out, epi=L.EPI_NONE, bias=None):
     """One real, unbatched product C = op(A) op(B) (+ bias row, or on top of what C holds) into `out`, a contiguous
     array. A product that cannot fill the chip alone (fewer 256 x 128 tiles than CUs) but is large enough to be worth a
     one-tile-per-CU launch is parked (_lib.park_product) so that it can share a launch with the independent products
     that a backward pass issues next to it; anything else is launched here."""
-    if not _CUS:
-        _CUS.append(L.device_info()[1])
-    tiles = -(-M // 256) * -(-N // 128)
-    parkable = (L.defer_products[0] and not L.capturing and tiles < _CUS[0] and M >= 256 and N >= 128 and K >= 256
-                and lda % 4 == 0 and ldb % 4 == 0 and (epi & 0xff) in (L.EPI_NONE, L.EPI_BIAS))
+    parkable = _would_park(M, N, K) and lda % 4 == 0 and ldb % 4 == 0 and (epi & 0xff) in (L.EPI_NONE, L.EPI_BIAS)
     a_ptr, b_ptr = A_.data_ptr(), B_.data_ptr()
     bias_ptr = bias.data_ptr() if isinstance(bias, Array) else bias
     if not parkable or (a_ptr | b_ptr) & 15:
@@ -1738,30 +1741,32 @@ def _linear_node(out, x, W, b, xs, Ws, act):
             return tot
         accW = in_place(_absorb_offer(pW), [K, N]) if dW is not None and pW is not px else None
         accX = in_place(_absorb_offer(px), [B, K]) if dx is not None and aux is None and pW is not px else None
-        # (the products go through _sgemm, which may park them for a shared launch; a large layer's bias gradient is a
-        # reduction of its own either way, a small one's rides in the weight-gradient launch)
+        # The data gradient first, the weight gradient last (an optimizer that updates inside backward() then finds it in
+        # the last-level cache). Products that accumulate, or that are of the size that shares launches (_would_park), go
+        # through _sgemm piece by piece; a large layer's bias gradient is a reduction of its own either way, a small one's
+        # rides in the weight-gradient launch. Everything else is one endia_hip_linear_bwd call.
         split = B * N > (1 << 20)
-        if accW is not None or (dW is not None and split):
-            if db is not None and split:
-                L.call("endia_hip_reduce_add", 2, L.i64_array([B, N]), 1, g.data_ptr(), db.data_ptr(), 1.0, 0)
-                _sgemm(1, 0, K, N, B, xs, K, g, N, accW if accW is not None else dW, L.EPI_NONE | (L.GEMM_ACCUMULATE if accW is not None else 0))
-            else:
-                tgt = accW if accW is not None else dW
-                L.call("endia_hip_sgemm", 1, 0, K, N, B, xs.data_ptr(), K, g.data_ptr(), N, tgt.data_ptr(), N, 1, 0, 0, 0,
-                       L.EPI_NONE | (L.GEMM_ACCUMULATE if accW is not None else 0) | (L.GEMM_COLSUM_B if db is not None else 0),
-                       L.OP_IDENTITY, None, None, db.data_ptr() if db is not None else None)
-            w_done = True
-        else:
-            w_done = False
+        own_W = accW is not None or (dW is not None and split and _would_park(K, N, B))
         if accX is not None:
             _sgemm(0, 1, B, K, N, g, N, Ws, N, accX, L.EPI_NONE | L.GEMM_ACCUMULATE)
-        rest_dx = dx if accX is None else None
-        rest_dW = dW if not w_done else None
-        rest_db = db if not w_done else None
-        if rest_dx is not None or rest_dW is not None or rest_db is not None:
+        lib_dx = dx if accX is None else None
+        if own_W:
+            if lib_dx is not None:
+                L.call("endia_hip_linear_bwd", B, K, N, xs.data_ptr(), Ws.data_ptr(), g.data_ptr(), flags,
+                       aux.data_ptr() if aux is not None else None, lib_dx.data_ptr(), None, None)
+            tgt = accW if accW is not None else dW
+            epi_w = L.EPI_NONE | (L.GEMM_ACCUMULATE if accW is not None else 0)
+            if db is not None and split:
+                L.call("endia_hip_reduce_add", 2, L.i64_array([B, N]), 1, g.data_ptr(), db.data_ptr(), 1.0, 0)
+                _sgemm(1, 0, K, N, B, xs, K, g, N, tgt, epi_w)
+            else:
+                L.call("endia_hip_sgemm", 1, 0, K, N, B, xs.data_ptr(), K, g.data_ptr(), N, tgt.data_ptr(), N, 1, 0, 0, 0,
+                       epi_w | (L.GEMM_COLSUM_B if db is not None else 0), L.OP_IDENTITY, None, None,
+                       db.data_ptr() if db is not None else None)
+        elif lib_dx is not None or dW is not None or db is not None:
             L.call("endia_hip_linear_bwd", B, K, N, xs.data_ptr(), Ws.data_ptr(), g.data_ptr(), flags,
-                   aux.data_ptr() if aux is not None else None, rest_dx.data_ptr() if rest_dx is not None else None,
-                   rest_dW.data_ptr() if rest_dW is not None else None, rest_db.data_ptr() if rest_db is not None else None)
+                   aux.data_ptr() if aux is not None else None, lib_dx.data_ptr() if lib_dx is not None else None,
+                   dW.data_ptr() if dW is not None else None, db.data_ptr() if db is not None else None)
         return [accX if accX is not None else dx, accW if accW is not None else dW, db]
 
     meta = {"act": act, "aux": out, "from_output": True} if act in _ACT_FN else {"act": None}
