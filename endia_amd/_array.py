@@ -29,13 +29,14 @@ _CACHE_MAX_TOTAL = 256 << 20
 class Buffer:
     """One allocation from the library's pool; returned to the pool when the last view dies."""
 
-    __slots__ = ("address", "nbytes", "captured", "pending")
+    __slots__ = ("address", "nbytes", "captured", "pending", "version")
 
     def __init__(self, nbytes):
         nbytes = int(nbytes)
         self.nbytes = nbytes
         self.captured = L.capturing
         self.pending = False  # a parked product (see _lib.park_product) has yet to write this buffer
+        self.version = 0      # counts in-place writes by user-visible updates (optimizer steps, -=, copy_from_numpy, a[...] = v)
         if not L.capturing:
             held = _FREE.get(nbytes)
             if held:
@@ -172,6 +173,7 @@ class Array:
             raise ValueError("copy_from_numpy: need a contiguous destination of the same element count")
         if a.size:
             L.call("endia_hip_memcpy_h2d", self.data_ptr(), a.ctypes.data, a.nbytes)
+        self._buf.version += 1
         return self
 
     def to_numpy(self):
@@ -238,6 +240,7 @@ class Array:
                 # A fused layer handed this node dL/dh * act'(h) for its own backward rule. The gradient a caller
                 # reads is dL/dh itself, as the reference stores it on every node: computed here, on first use.
                 self._grad = self._grad_fused._true_grad()
+                self._grad_fused._true_grad = None  # evaluated once: let go of the cotangent it held
                 return self._grad
             return Array(self._shape, is_complex=self.is_complex_)
         return self._grad
@@ -297,6 +300,7 @@ class Array:
         if src.size():
             L.call("endia_hip_strided_scatter", sub.ndim(), L.i64_array(sub._shape), L.i64_array(sub._strides),
                    sub._offset, src.data_ptr(), self._buf.ptr, 0, 1 if self.is_complex_ else 0)
+            self._buf.version += 1
 
     def _bin(self, other, fn, reverse=False):
         from . import functional as F
@@ -356,6 +360,7 @@ class Array:
         src = other if other.is_contiguous() else _contiguous_copy(other)
         assert self.is_contiguous()
         L.call("endia_hip_memcpy_d2d", self.data_ptr(), src.data_ptr(), 4 * self.size() * (2 if self.is_complex_ else 1))
+        self._buf.version += 1
 
     def __isub__(self, o):
         self._assign_from(self - o)

@@ -867,6 +867,13 @@ __global__ __launch_bounds__(256) void mlp_wgrad_sum_kernel(MlpArgs p, int slice
   *dst = sum;
 }
 
+// The kernels read and write activations, cotangents, biases and gradients 16 bytes at a time wherever a layer's width is
+// a multiple of four; only the weights have an element-by-element route. So every other array has to start on a
+// 16-byte boundary (what every allocator hands out).
+bool on_16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; }
+#define ENDIA_MLP_ALIGNED(ptr, what, l) \
+  ENDIA_CHECK_ARG(on_16(ptr), "%s: %s of layer %d is not 16-byte aligned (only the weight matrices may start anywhere)", who, what, l)
+
 int32_t fill_args(MlpArgs& a, const endia_hip_mlp_desc* d, const char* who) {
   ENDIA_CHECK_ARG(d != nullptr, "%s: null descriptor", who);
   ENDIA_CHECK_ARG(d->layers >= 1 && d->layers <= ENDIA_MLP_MAX_LAYERS, "%s: %d layers, 1..%d supported", who, d->layers, ENDIA_MLP_MAX_LAYERS);
@@ -911,8 +918,12 @@ extern "C" int32_t endia_hip_mlp_fwd(const endia_hip_mlp_desc* desc, const float
   if (rc) return rc;
   if (a.batch == 0) return ENDIA_HIP_OK;
   ENDIA_CHECK_ARG(x && W && b && h, "endia_hip_mlp_fwd: null argument");
+  const char* who = "endia_hip_mlp_fwd";
+  ENDIA_MLP_ALIGNED(x, "x", 0);
   for (int l = 0; l < a.layers; ++l) {
     ENDIA_CHECK_ARG(W[l] && b[l] && h[l], "endia_hip_mlp_fwd: null pointer for layer %d", l);
+    ENDIA_MLP_ALIGNED(b[l], "b", l);
+    ENDIA_MLP_ALIGNED(h[l], "h", l);
     a.W[l] = W[l];
     a.b[l] = b[l];
     a.h[l] = h[l];
@@ -937,11 +948,18 @@ int32_t fwd_mse(const char* who, const endia_hip_mlp_desc* desc, const float* x,
   ENDIA_CHECK_ARG(x && W && b && h && target, "%s: null argument", who);
   for (int l = 0; l < a.layers; ++l) {
     ENDIA_CHECK_ARG(W[l] && b[l] && h[l] && (!delta || delta[l]), "%s: null pointer for layer %d", who, l);
+    ENDIA_MLP_ALIGNED(b[l], "b", l);
+    ENDIA_MLP_ALIGNED(h[l], "h", l);
+    if (delta) ENDIA_MLP_ALIGNED(delta[l], "delta", l);
     a.W[l] = W[l];
     a.b[l] = b[l];
     a.h[l] = h[l];
     if (delta) a.delta[l] = delta[l];
   }
+  ENDIA_MLP_ALIGNED(x, "x", 0);
+  ENDIA_MLP_ALIGNED(target, "target", a.layers - 1);
+  ENDIA_MLP_ALIGNED(dpred, "dpred", a.layers - 1);
+  ENDIA_MLP_ALIGNED(dx, "dx", 0);
   a.x = x;
   const int64_t groups = fwd_groups(a);
   struct Scratch {  // partial sums from the library's pool, handed back on scope exit (reuse is stream-ordered)
@@ -994,6 +1012,10 @@ int32_t bwd(const char* who, const endia_hip_mlp_desc* desc, const float* x, con
   int blocks = 0;
   for (int l = 0; l < a.layers; ++l) {
     ENDIA_CHECK_ARG((!chain || W[l]) && delta[l] && (l + 1 == a.layers || h[l]), "%s: null pointer for layer %d", who, l);
+    ENDIA_MLP_ALIGNED(h[l], "h", l);
+    ENDIA_MLP_ALIGNED(delta[l], "delta", l);
+    ENDIA_MLP_ALIGNED(dW[l], "dW", l);
+    ENDIA_MLP_ALIGNED(db[l], "db", l);
     a.W[l] = chain ? W[l] : nullptr;
     a.h[l] = const_cast<float*>(h[l]);
     a.delta[l] = delta[l];
@@ -1003,6 +1025,8 @@ int32_t bwd(const char* who, const endia_hip_mlp_desc* desc, const float* x, con
     blocks += ((a.width[l] + 31) / 32) * ((a.width[l + 1] + 31) / 32);
   }
   a.tile0[a.layers] = blocks;
+  ENDIA_MLP_ALIGNED(x, "x", 0);
+  ENDIA_MLP_ALIGNED(dx, "dx", 0);
   a.x = x;
   a.dx = dx;
   hipStream_t s = ctx().stream;

@@ -300,6 +300,35 @@ int32_t static_scratch_init(int device) {
   return ENDIA_HIP_OK;
 }
 
+// How the column reduction cuts its rows: S splits of rows_per_split rows each (S = 0: one launch, no first stage;
+// S = -1: the columns do not fit `part_floats`, the room the caller has for first-stage partial sums, 0 = no limit).
+// Pure arithmetic, no device: endia_hip_col_sum_plan exposes it so that the clamp can be tested on any host.
+static void col_reduce_plan(int64_t batch, int64_t R, int64_t C, int64_t cus, int64_t part_floats, int64_t* S_out, int64_t* rows_out) {
+  const int64_t col_tiles = ceil_div64(C, 256);
+  if (R <= 1024 && batch * R * C <= (1 << 20)) {
+    *S_out = 0;
+    *rows_out = R;
+    return;
+  }
+  // enough row splits for ~4 groups per CU, at least 16 rows each
+  int64_t S = cus * 4 / (col_tiles * batch);
+  const int64_t cap = col_tiles * batch * 64 < cus ? 256 : 64;  // a narrow input needs more row splits to fill the chip
+  if (S > cap) S = cap;
+  if (S < 1) S = 1;
+  const int64_t max_s = ceil_div64(R, 16);
+  if (S > max_s) S = max_s;
+  if (S > 1024) S = 1024;
+  if (part_floats > 0 && S * batch * C > part_floats) S = part_floats / (batch * C);
+  if (S < 1) {
+    *S_out = -1;
+    *rows_out = 0;
+    return;
+  }
+  const int64_t rows_per_split = ceil_div64(R, S);
+  *S_out = ceil_div64(R, rows_per_split);
+  *rows_out = rows_per_split;
+}
+
 // out[b][c] = scale * sum_r x[b][r][c]. The first-stage partial sums go to `part` (room for part_floats) when the
 // caller brings it, else to the library's workspace; with too little room the rows are cut into fewer splits.
 static int32_t col_reduce_with(int64_t batch, int64_t R, int64_t C, const float* x, float* out, float scale, float* part,
@@ -311,25 +340,15 @@ static int32_t col_reduce_with(int64_t batch, int64_t R, int64_t C, const float*
     return fail(ENDIA_HIP_ERR_UNSUPPORTED, "col_reduce: extent too large");
   // A small input (the bias gradient of a narrow layer) is one launch: the second-stage kernel applied to the
   // input itself, 64 columns per group, the four waves taking alternate rows.
-  if (R <= 1024 && batch * R * C <= (1 << 20)) {
+  int64_t S = 0, rows_per_split = 0;
+  col_reduce_plan(batch, R, C, ctx().cu_count, part ? part_floats : 0, &S, &rows_per_split);
+  if (S == 0) {
     hipLaunchKernelGGL(col_reduce_final_kernel, dim3((unsigned)ceil_div64(C, 64), (unsigned)batch), dim3(TPB), 0, s, x, out, R,
                        C, batch, scale);
     ENDIA_LAUNCH_CHECK();
     return ENDIA_HIP_OK;
   }
-  // enough row splits for ~4 groups per CU, at least 16 rows each
-  int64_t want = (int64_t)ctx().cu_count * 4;
-  int64_t S = want / (col_tiles * batch);
-  const int64_t cap = col_tiles * batch * 64 < ctx().cu_count ? 256 : 64;  // a narrow input needs more row splits to fill the chip
-  if (S > cap) S = cap;
-  if (S < 1) S = 1;
-  int64_t max_s = ceil_div64(R, 16);
-  if (S > max_s) S = max_s;
-  if (S > 1024) S = 1024;
-  if (part && S * batch * C > part_floats) S = part_floats / (batch * C);
-  if (S < 1) return fail(ENDIA_HIP_ERR_INVALID, "col_reduce: %lld columns do not fit the %lld floats of scratch", (long long)(batch * C), (long long)part_floats);
-  int64_t rows_per_split = ceil_div64(R, S);
-  S = ceil_div64(R, rows_per_split);
+  if (S < 0) return fail(ENDIA_HIP_ERR_INVALID, "col_reduce: %lld columns do not fit the %lld floats of scratch", (long long)(batch * C), (long long)part_floats);
   if (!part) {
     void* ws = nullptr;
     int32_t rc = workspace(batch * S * C * (int64_t)sizeof(float), &ws);
@@ -388,6 +407,13 @@ int32_t row_reduce(int64_t R, int64_t C, const float* x, float* out, float scale
 using namespace endia;
 
 extern "C" {
+
+int32_t endia_hip_col_sum_plan(int64_t R, int64_t C, int64_t cu_count, int64_t scratch_floats, int64_t* splits, int64_t* rows_per_split) {
+  ENDIA_CHECK_ARG(R >= 1 && C >= 1 && cu_count >= 1 && scratch_floats >= 0 && splits && rows_per_split,
+                  "endia_hip_col_sum_plan: R, C, cu_count >= 1, scratch_floats >= 0 and non-null outputs");
+  col_reduce_plan(1, R, C, cu_count, scratch_floats, splits, rows_per_split);
+  return ENDIA_HIP_OK;
+}
 
 int32_t endia_hip_reduce_add(int32_t ndim, const int64_t* shape, uint32_t reduce_mask, const float* x, float* out,
                              float scale, int32_t is_complex) {

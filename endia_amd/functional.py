@@ -140,6 +140,7 @@ def _overwrite(arg, values):
 
 def fill_(arg, value):
     """init_ops.mojo:185-193."""
+    arg._buf.version += 1
     if not arg.is_contiguous() or arg.is_complex_:
         return _overwrite(arg, np.full(arg.shape(), value, np.complex64 if arg.is_complex_ else np.float32))
     if arg.size():
@@ -1542,6 +1543,12 @@ def linear(x, W, b, act=None):
     return _linear_node(out, x, W, b, xs, Ws, act)
 
 
+def _starts_on_16(*arrays):
+    """Views that begin on a 16-byte boundary of their (256-byte aligned) buffers, or would after the contiguous copy a
+    non-contiguous one gets: what the whole-model entry points ask of everything but the weights."""
+    return all((a._offset * 4) % 16 == 0 or not a.is_contiguous() for a in arrays)
+
+
 def mlp_forward(x, weights, biases, act=None):
     """The whole dense stack of nn.MLP.forward (nn/modules/_mlp.mojo:47-53) as ONE op: act after every layer but the
     last. For small models (every width at most 128, like the reference's benchmark model) the forward pass is one
@@ -1554,7 +1561,8 @@ def mlp_forward(x, weights, biases, act=None):
     small = (x.ndim() == 2 and 1 <= Lyr <= L.MLP_MAX_LAYERS and act in (None, "identity", "relu", "tanh") and x.size() > 0
              and not x.is_complex_ and all(1 <= n <= L.MLP_MAX_WIDTH for n in widths)
              and all(w.ndim() == 2 and not w.is_complex_ and w._shape[0] == widths[i] for i, w in enumerate(weights))
-             and all(b.size() == widths[i + 1] and not b.is_complex_ for i, b in enumerate(biases)))
+             and all(b.size() == widths[i + 1] and not b.is_complex_ for i, b in enumerate(biases))
+             and _starts_on_16(x, *biases))
     if not small:
         h = x
         for i in range(Lyr):
@@ -1603,7 +1611,8 @@ def mlp_mse_loss(x, target, weights, biases, act=None):
              and list(target._shape) == [x._shape[0], widths[-1]]
              and all(1 <= n <= L.MLP_MAX_WIDTH for n in widths)
              and all(w.ndim() == 2 and not w.is_complex_ and w._shape[0] == widths[i] for i, w in enumerate(weights))
-             and all(b.size() == widths[i + 1] and not b.is_complex_ for i, b in enumerate(biases)))
+             and all(b.size() == widths[i + 1] and not b.is_complex_ for i, b in enumerate(biases))
+             and _starts_on_16(x, target, *biases))
     if not small:
         return mse(mlp_forward(x, weights, biases, act), target)
     B = x._shape[0]
@@ -1669,7 +1678,9 @@ def _sin_of_linear_node(out, zz):
         if building_graph() or grad.ndim() != out_.ndim():  # (a Jacobian seed's leading axes broadcast through mul)
             return [mul(cos(z), grad)]  # sin_op.mojo:92
         if grad._act_applied:
-            return [grad]
+            # the layer above already multiplied by cos(z): for the pre-activation node that IS its gradient, so it is
+            # handed on as a plain array (z.grad() then shows dL/dz, not the hidden activation's dL/dh)
+            return [Array(grad._shape, _buffer=grad._buf, _strides=grad._strides, _offset=grad._offset)]
         offer = _absorb_offer(z)
         if offer is not None and offer[0]._shape == z._shape and grad._shape == z._shape and not offer[0].is_complex_:
             # z already holds a gradient (a second-order pass reaches the pre-activation twice): one launch for both
@@ -1726,7 +1737,18 @@ def _linear_node(out, x, W, b, xs, Ws, act):
                 aux = contiguous(pm["aux"])
                 dx._act_applied = True
                 # what px.grad() shows is dL/dpx itself; nobody reads it in a training step, so it is made on demand
-                dx._true_grad = lambda: matmul(detach(g), detach(Ws).T())
+                # (it multiplies by the weights as they are when it runs: asked for after an optimizer step or any
+                # other in-place write to W it would silently use the new ones, so it refuses then. It keeps this
+                # layer's cotangent alive until it has run once or zero_grad / remove_grad drops it.)
+                w_version = Ws._buf.version
+
+                def true_grad():
+                    if Ws._buf.version != w_version:
+                        raise RuntimeError("the gradient of a hidden activation of a fused layer is computed on first use and was asked for "
+                                           "after the layer's weights were updated in place: read it before optimizer.step(), or build "
+                                           "the model with fused=False")
+                    return matmul(detach(g), detach(Ws).T())
+                dx._true_grad = true_grad
         # A weight or an input that already holds a gradient nobody else refers to (second-order passes reach both
         # twice) takes this layer's product on top of it in the GEMM's epilogue instead of through an `add` launch.
         def in_place(offer, shape):

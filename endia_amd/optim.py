@@ -42,6 +42,7 @@ class SGD:
                    (ctypes.c_void_p * k)(*[g.data_ptr() for g in grads]), self.lr)
             for p in self.params:
                 p.clear_args()
+                p._buf.version += 1
             return
         for i, p in enumerate(self.params):
             g = _flat_grad(p)
@@ -53,6 +54,7 @@ class SGD:
             else:
                 L.call("endia_hip_sgd_step", p.size(), p.data_ptr(), g.data_ptr(), self.lr)
             p.clear_args()
+            p._buf.version += 1
 
 
 class Adagrad:
@@ -69,6 +71,7 @@ class Adagrad:
             assert p.is_contiguous()
             L.call("endia_hip_adagrad_step", p.size(), p.data_ptr(), g.data_ptr(), c.data_ptr(), self.lr, self.eps)
             p.clear_args()
+            p._buf.version += 1
 
 
 class RMSprop:
@@ -85,6 +88,7 @@ class RMSprop:
             assert p.is_contiguous()
             L.call("endia_hip_rmsprop_step", p.size(), p.data_ptr(), g.data_ptr(), c.data_ptr(), self.lr, self.alpha, self.eps)
             p.clear_args()
+            p._buf.version += 1
 
 
 class Adam:
@@ -126,6 +130,7 @@ class Adam:
         L.call("endia_hip_adam_step", p.size(), p.data_ptr(), g.data_ptr(), self.m[i].data_ptr(), self.v[i].data_ptr(), self.lr,
                self.beta1, self.beta2, self.eps, self.t)
         p.clear_args()
+        p._buf.version += 1
         self._updated[i] = True
 
     def _device_counter(self):
@@ -155,6 +160,7 @@ class Adam:
                    self.lr, self.beta1, self.beta2, self.eps, t_dev.data_ptr())
             for p in self.params:
                 p.clear_args()
+                p._buf.version += 1
             return
         for i in range(len(self.params)):
             self._update(i)

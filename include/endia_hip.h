@@ -232,7 +232,8 @@ ENDIA_API int32_t endia_hip_linear_bwd(int64_t B, int64_t K, int64_t N, const fl
  *      the same way, then every dW_l and db_l at once), instead of one to three launches per layer.
  *      widths[0..layers]: input width, then each layer's output width. W[l] is [widths[l], widths[l+1]] row-major, b[l]
  *      is [widths[l+1]], x is [batch, widths[0]], all contiguous. act in {RELU, TANH, IDENTITY} follows every layer but
- *      the last.
+ *      the last. A weight matrix may start at any float; every other array (x, b, h, target, delta, dW, db, dx) must
+ *      start on a 16-byte boundary (ENDIA_HIP_ERR_INVALID otherwise): they are read and written 16 bytes at a time.
  *      fwd: h[l] receives layer l's output [batch, widths[l+1]] (h[layers-1] is the model's output; the others are what
  *           the backward pass needs).
  *      bwd: delta[layers-1] holds the cotangent of the output on entry; delta[l] for l < layers-1 are buffers
@@ -356,6 +357,13 @@ ENDIA_API int32_t endia_hip_reduce_add(int32_t ndim, const int64_t* shape, uint3
  *      device's one array: calls that overlap on one device (two host threads, two processes' worth of streams)
  *      race; calls on the library's single stream, the only kind this ABI issues, are ordered. */
 ENDIA_API int32_t endia_hip_col_sum_static(int64_t R, int64_t C, const float* x, float* out, float scale);
+/* How a column sum of R rows and C columns cuts its rows on a device of cu_count CUs when scratch_floats floats are
+ * there for first-stage partial sums (0: no limit, what endia_hip_reduce_add has; 262144: endia_hip_col_sum_static).
+ * No counterpart in the reference; pure arithmetic, needs no device and no endia_hip_init. splits = 0: one launch without
+ * a first stage; -1: C does not fit the scratch; otherwise `splits` pieces of rows_per_split rows. Two calls that get
+ * the same plan add in the same order and agree bit for bit. */
+ENDIA_API int32_t endia_hip_col_sum_plan(int64_t R, int64_t C, int64_t cu_count, int64_t scratch_floats, int64_t* splits,
+                                         int64_t* rows_per_split);
 
 /* ---- the other reductions: ReduceMax / ReduceMin / ReduceMul .__call__ (reduce_ops/reduce_max_op.mojo:66-190,
  *      reduce_min_op.mojo:66-190, reduce_mul_op.mojo:65-210) and ReduceArgMax / ReduceArgMin .__call__

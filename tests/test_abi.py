@@ -105,3 +105,28 @@ def test_c_client_trains_one_step_on_the_device():
     print(res.stdout, res.stderr)
     assert res.returncode == 0, (res.returncode, res.stdout, res.stderr)
     assert "worst relative error" in res.stdout
+
+
+def test_col_sum_plan_clamps_to_the_scratch():
+    """The row splits of a column sum, a host-side computation (no device): with unlimited scratch a 4096 x 4096 input
+    on 256 CUs is cut into 64 pieces; the 262144 floats of endia_hip_col_sum_static allow exactly those 64 (which is why
+    that entry point agrees with endia_hip_reduce_add bit for bit there); less scratch, or a device with more CUs,
+    forces fewer pieces, down to refusing columns that do not fit at all; a small input needs no first stage."""
+    lib = L.lib()
+
+    def plan(R, C, cus, scratch):
+        S, rows = ctypes.c_int64(), ctypes.c_int64()
+        assert lib.endia_hip_col_sum_plan(R, C, cus, scratch, ctypes.byref(S), ctypes.byref(rows)) == 0
+        return S.value, rows.value
+
+    assert plan(4096, 4096, 256, 0) == (64, 64)
+    assert plan(4096, 4096, 256, 1 << 18) == (64, 64)
+    assert plan(4096, 4096, 256, 1 << 16) == (16, 256)        # room for 16 partial rows only
+    assert plan(4096, 4096, 1024, 0) == (64, 64) and plan(4096, 4096, 1024, 1 << 17) == (32, 128)
+    assert plan(24, 1 << 18, 256, 1 << 18) == (1, 24)
+    assert plan(24, (1 << 18) + 4, 256, 1 << 18)[0] == -1      # does not fit
+    assert plan(40, 96, 256, 1 << 18) == (0, 40)               # one launch
+    for R, C, cus, scratch in [(1500, 772, 256, 1 << 18), (100000, 64, 304, 4096), (2000, 5000, 8, 0)]:
+        S, rows = plan(R, C, cus, scratch)
+        assert S >= 1 and (S - 1) * rows < R <= S * rows and (scratch == 0 or S * C <= scratch)
+    assert lib.endia_hip_col_sum_plan(0, 4, 256, 0, None, None) == L.ERR_INVALID

@@ -1308,6 +1308,22 @@ def test_hidden_activation_gradients_of_fused_layers(nd, act):
     got = nd.grad(outs=[loss_f], inputs=hid_f)
     for g, hu in zip(got, hid_u):
         assert_close(g.to_numpy(), hu.grad().to_numpy(), what="grad(outs, inputs=[h]) (%s)" % act)
+    if act == "sin":
+        # the fused sin layer keeps its pre-activation as a node of its own: its gradient is dL/dz = dL/dh * cos(z)
+        loss_f, hid_f, _, _ = run(True)
+        loss_f.backward()
+        for hf, hu in zip(hid_f, hid_u):
+            z = hf.args()[0]
+            zu = hu.args()[0]
+            assert_close(z.grad().to_numpy(), zu.grad().to_numpy(), what="dL/dz of a fused sin layer")
+    # a hidden gradient is computed on first use with the layer's weights: after an in-place update it refuses
+    loss_f, hid_f, W_f, b_f = run(True)
+    loss_f.backward()
+    early = hid_f[1].grad().to_numpy()          # read before the step: fine, and kept
+    nd.optim.SGD(W_f + b_f, lr=0.1).step()
+    np.testing.assert_array_equal(hid_f[1].grad().to_numpy(), early)
+    with pytest.raises(RuntimeError, match="updated in place"):
+        hid_f[0].grad()
     loss_f.zero_grad()
     assert not hid_f[0].has_grad()
 
@@ -1460,6 +1476,38 @@ def test_whole_model_forward_with_cotangents_entry_points(nd):
     # arguments the entry points refuse
     with pytest.raises(Exception):
         L.call("endia_hip_mlp_fwd_mse_delta", ctypes.byref(desc), x.data_ptr(), ptrs(W), ptrs(b), t.data_ptr(), ptrs(W), None, x.data_ptr(), None)
+
+
+def test_whole_model_entry_points_want_aligned_arrays(nd):
+    """Everything but the weights is read and written 16 bytes at a time: an activation, bias or cotangent array that
+    starts 4 bytes off a 16-byte boundary is refused by the entry points, and the ops send such views down the
+    per-layer route instead."""
+    import ctypes
+    from endia_amd import _lib as L
+    from endia_amd._array import Array
+    rng = np.random.default_rng(80)
+    widths, batch = [8, 16, 4], 6
+    W = [nd.array(rng.standard_normal((widths[i], widths[i + 1])).astype(np.float32)) for i in range(2)]
+    b = [nd.array(rng.standard_normal(widths[i + 1]).astype(np.float32)) for i in range(2)]
+    x = nd.array(rng.standard_normal((batch, 8)).astype(np.float32))
+    desc = L.MlpDesc()
+    desc.layers, desc.act, desc.batch = 2, L.OP_RELU, batch
+    desc.widths[:3] = widths
+    ptrs = lambda ps: (ctypes.c_void_p * 2)(*ps)
+    big = Array.empty([batch * 16 + 4])
+    h_ok = [Array.empty([batch, 16]), Array.empty([batch, 4])]
+    L.call("endia_hip_mlp_fwd", ctypes.byref(desc), x.data_ptr(), ptrs([w.data_ptr() for w in W]), ptrs([v.data_ptr() for v in b]),
+           ptrs([h.data_ptr() for h in h_ok]))
+    with pytest.raises(L.EndiaHipError, match="16-byte"):
+        L.call("endia_hip_mlp_fwd", ctypes.byref(desc), x.data_ptr(), ptrs([w.data_ptr() for w in W]), ptrs([v.data_ptr() for v in b]),
+               ptrs([big.data_ptr() + 4, h_ok[1].data_ptr()]))
+    # the op: a bias that is a view one float into its buffer
+    raw = nd.array(np.concatenate([[0.0], b[0].to_numpy()]).astype(np.float32))
+    odd = raw[1:]
+    assert odd._offset == 1
+    got = nd.mlp_forward(x, W, [odd, b[1]], "relu").to_numpy()
+    want = nd.mlp_forward(x, W, b, "relu").to_numpy()
+    assert_close(got, want, tol=1e-6, what="bias view with an odd offset")
 
 
 def test_whole_model_large_batch_repeats_bit_for_bit(nd):

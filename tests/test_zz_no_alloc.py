@@ -14,6 +14,19 @@ from endia_amd import _lib as L
 pytestmark = pytest.mark.gpu
 
 
+def _same_plan(R, C):
+    """Bit equality with endia_hip_reduce_add holds when both cut the rows the same way, i.e. when the 262144 floats of
+    static scratch do not force fewer row splits than the unlimited workspace gets (never on a 256-CU device; the plan
+    query says so for whatever device this is, and tests/test_abi.py checks the clamp itself on the CPU)."""
+    _, cus, _ = L.device_info()
+    plans = []
+    for scratch in (0, 1 << 18):
+        S, rows = ctypes.c_int64(), ctypes.c_int64()
+        L.call("endia_hip_col_sum_plan", R, C, cus, scratch, ctypes.byref(S), ctypes.byref(rows))
+        plans.append((S.value, rows.value))
+    return plans[0] == plans[1]
+
+
 def _both(dev, x, scale=1.0):
     R, C = x.shape
     dx = dev.put(x)
@@ -34,7 +47,9 @@ def test_col_sum_static_matches_reduce_add_twice_in_a_row(dev):
     small = rng.standard_normal((1500, 772)).astype(np.float32)    # smaller, still two stages
     for x, scale in ((big, 1.0), (small, 0.5)):
         got, ref = _both(dev, x, scale)
-        assert np.array_equal(got, ref), "static-scratch column sums differ from endia_hip_reduce_add"
+        if _same_plan(*x.shape):
+            assert np.array_equal(got, ref), "static-scratch column sums differ from endia_hip_reduce_add"
+        assert_close(got, ref, tol=1e-6, what="static scratch vs reduce_add")
         assert_close(got, scale * x.astype(np.float64).sum(axis=0), what="column sums %s" % (x.shape,))
     tiny = rng.standard_normal((40, 96)).astype(np.float32)        # the single-launch path (no scratch at all)
     got, ref = _both(dev, tiny)
@@ -46,7 +61,9 @@ def test_col_sum_static_widest_input(dev):
     rng = np.random.default_rng(12)
     x = rng.standard_normal((24, 1 << 18)).astype(np.float32)
     got, ref = _both(dev, x)
-    assert np.array_equal(got, ref)
+    if _same_plan(*x.shape):
+        assert np.array_equal(got, ref)
+    assert_close(got, ref, tol=1e-6, what="static scratch vs reduce_add")
     assert_close(got, x.astype(np.float64).sum(axis=0), what="widest column sums")
 
 
