@@ -112,6 +112,7 @@ class Array:
     _grad_fused = None    # such a gradient on its way to this node's own VJP rule; never what grad() returns
     _true_grad = None     # on an _act_applied gradient: a function that computes the gradient without the derivative
     _on_final_grad = None  # set by an optimizer with fused_backward=True: called by backward() when this leaf's gradient is complete
+    _lazy_mlp = None      # on the output of functional.mlp_forward while its launch is parked: what mse() needs to fuse with it
     _internal = False     # a node that a VJP rule created (the transposes and broadcasts inside a recorded backward pass)
     _absorbed = False     # a VJP result that already includes the gradient its primal held (functional._absorb)
     _offset = 0

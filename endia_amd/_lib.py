@@ -228,9 +228,37 @@ def park_product(fields, buffers, out_buffer):
     _parked.append((fields, buffers, out_buffer))
 
 
+def park_launch(launch, out_buffers):
+    """Park any other launch whose outputs are all fresh buffers: `launch()` issues it. Besides being run by flush() it
+    can be withdrawn (withdraw_launch) by an op that computes the same outputs as part of a larger launch."""
+    if len(_parked) >= MAX_PARKED:
+        flush()
+    for b in out_buffers:
+        b.pending = True
+    item = (None, launch, list(out_buffers))
+    _parked.append(item)
+    return item
+
+
+def withdraw_launch(item):
+    """Take a parked launch back; True when it was still parked (its buffers are then no longer pending, and whoever
+    withdrew it writes them)."""
+    for i, it in enumerate(_parked):
+        if it is item:
+            del _parked[i]
+            for b in item[2]:
+                b.pending = False
+            return True
+    return False
+
+
 def parked_uses(buffer):
     """True when a parked product reads or writes `buffer`."""
-    for _, buffers, out in _parked:
+    for fields, buffers, out in _parked:
+        if fields is None:
+            if any(b is buffer for b in out):
+                return True
+            continue
         if out is buffer:
             return True
         for b in buffers:
@@ -240,30 +268,50 @@ def parked_uses(buffer):
 
 
 def flush(need=None):
-    """Launch what is parked, in one endia_hip_sgemm_grouped call: everything, or, when `need` names the output buffer
-    somebody is about to read, that product and whichever parked products make its launch a better one (the rest stay
-    parked and may find better company later)."""
+    """Launch what is parked: everything, or, when `need` names the output buffer somebody is about to read, the launch
+    that writes it; for a product that means one endia_hip_sgemm_grouped call with that product and whichever parked
+    products make its launch a better one (the rest stay parked and may find better company later)."""
     if not _parked:
         return
     items = _parked[:]
+    if need is not None:
+        for it in items:
+            if it[0] is None and any(b is need for b in it[2]):
+                _parked.remove(it)
+                for b in it[2]:
+                    b.pending = False
+                it[1]()
+                return
+    else:
+        for it in items:
+            if it[0] is None:
+                _parked.remove(it)
+                for b in it[2]:
+                    b.pending = False
+                it[1]()
+        items = _parked[:]
+        if not items:
+            return
+    products = [it for it in items if it[0] is not None]
     index = -1
     if need is not None:
-        for i, (_, _, out) in enumerate(items):
+        for i, (_, _, out) in enumerate(products):
             if out is need:
                 index = i
         if index < 0:
             return
-    descs = (SgemmDesc * len(items))()
-    for d, (f, _, _) in zip(descs, items):
+    descs = (SgemmDesc * len(products))()
+    for d, (f, _, _) in zip(descs, products):
         (d.transA, d.transB, d.M, d.N, d.K, d.A, d.lda, d.B, d.ldb, d.C, d.ldc, d.epilogue, d.bias) = f
-    done = (c_int32 * len(items))()
-    del _parked[:]  # (nothing below comes back here: the raw call flushes nothing)
+    done = (c_int32 * len(products))()
+    for it in products:
+        _parked.remove(it)  # (nothing below comes back here: the raw call flushes nothing)
     try:
-        _raw_call("endia_hip_sgemm_grouped", len(items), descs, index, done)
+        _raw_call("endia_hip_sgemm_grouped", len(products), descs, index, done)
     finally:
         if flush_observer[0] is not None:
-            flush_observer[0]([item[0] for item in items], index, list(done))
-        for item, flag in zip(items, done):
+            flush_observer[0]([item[0] for item in products], index, list(done))
+        for item, flag in zip(products, done):
             if flag or index < 0:
                 item[2].pending = False
             else:

@@ -1277,6 +1277,12 @@ def mse(pred, target):
     if pred.is_complex_ or target.is_complex_ or pred._shape != target._shape:
         diff = sub(pred, target)
         return sum(mul(diff, diff)) / float(pred.size())
+    lazy = pred._lazy_mlp
+    if lazy is not None and not target._requires_grad and _starts_on_16(target) and L.withdraw_launch(lazy[0]):
+        # pred is the output of a whole-model forward that has not been launched yet: one launch for the forward pass, the
+        # loss, its gradient and the cotangents of all layers (mlp_mse_loss), writing the same activation arrays
+        pred._lazy_mlp = None
+        return _mlp_mse_fused(lazy, pred, target)
     p, t = contiguous(pred), contiguous(target)
     loss = Array.empty([1])
     need_grad = pred._requires_grad
@@ -1576,7 +1582,20 @@ def mlp_forward(x, weights, biases, act=None):
     desc.layers, desc.act, desc.batch = Lyr, _ACT[act], B
     desc.widths[:Lyr + 1] = widths
     ptrs = lambda arrs: (ctypes.c_void_p * Lyr)(*[a.data_ptr() if a is not None else None for a in arrs])
-    L.call("endia_hip_mlp_fwd", ctypes.byref(desc), xs.data_ptr(), ptrs(Ws), ptrs(bs_), ptrs(hs))
+    # The forward launch is parked, not issued: mse() of this output (the reference script's next call, mlp_imp.mojo:56-60)
+    # withdraws it and runs the launch that evaluates the loss and the cotangents of all layers as well; anything else that
+    # reads the output, or any call that is not a pure function of fresh buffers, launches it as it is.
+    x_ptr, W_ptrs, b_ptrs = xs.data_ptr(), ptrs(Ws), ptrs(bs_)
+    h_ptrs = (ctypes.c_void_p * Lyr)(*[h._buf.address for h in hs])
+
+    def launch_forward():
+        L._raw_call("endia_hip_mlp_fwd", ctypes.byref(desc), x_ptr, W_ptrs, b_ptrs, h_ptrs)
+
+    if L.defer_products[0]:
+        ticket = L.park_launch(launch_forward, [h._buf for h in hs])
+        hs[-1]._lazy_mlp = (ticket, xs, Ws, bs_, hs, desc, widths, act, x, list(weights), list(biases))
+    else:
+        launch_forward()
 
     def vjp(primals, grad, out_):
         from .autograd.functional import building_graph
@@ -1616,13 +1635,27 @@ def mlp_mse_loss(x, target, weights, biases, act=None):
     if not small:
         return mse(mlp_forward(x, weights, biases, act), target)
     B = x._shape[0]
-    xs, ts = contiguous(x), contiguous(target)
+    xs = contiguous(x)
     Ws, bs_ = [contiguous(w) for w in weights], [contiguous(b) for b in biases]
     hs = [Array.empty([B, widths[i + 1]]) for i in range(Lyr)]
-    loss = Array.empty([1])
     desc = L.MlpDesc()
     desc.layers, desc.act, desc.batch = Lyr, _ACT[act], B
     desc.widths[:Lyr + 1] = widths
+    return _mlp_mse_launch(x, target, list(weights), list(biases), xs, Ws, bs_, hs, desc, widths, None)
+
+
+def _mlp_mse_fused(lazy, pred, target):
+    """mse(pred, target) where pred is the output of a whole-model forward whose launch was still parked (and has just
+    been withdrawn): the launch of mlp_mse_loss on the very arrays that forward pass was going to write."""
+    _, xs, Ws, bs_, hs, desc, widths, act, x, weights, biases = lazy
+    return _mlp_mse_launch(x, target, weights, biases, xs, Ws, bs_, hs, desc, widths, pred)
+
+
+def _mlp_mse_launch(x, target, weights, biases, xs, Ws, bs_, hs, desc, widths, pred):
+    import ctypes
+    Lyr, B = len(weights), x._shape[0]
+    ts = contiguous(target)
+    loss = Array.empty([1])
     ptrs = lambda arrs: (ctypes.c_void_p * Lyr)(*[a.data_ptr() if a is not None else None for a in arrs])
     # With something to differentiate, the forward launch goes on to the cotangents of all layers for the loss gradient
     # (rows are independent through the whole chain), and backward() is left with the weight gradients.
@@ -1646,6 +1679,8 @@ def mlp_mse_loss(x, target, weights, biases, act=None):
         want_dx = primals[0]._requires_grad
         if _holds_seed(grad) and any(wants) and (dx0 is not None or not want_dx):
             L.call("endia_hip_mlp_wgrad", ctypes.byref(desc), xs.data_ptr(), ptrs(hs), ptrs(deltas), ptrs(dW), ptrs(db))
+            if pred is not None and not pred.has_grad():
+                pred.grad_(deltas[-1])  # what mse's own rule would have stored on the model's output
             return [dx0 if want_dx else None, None] + dW + db
         # a cotangent other than the seed scales the stored loss gradient; the chain is run again from there
         last = deltas[-1] if _holds_seed(grad) else mul(deltas[-1], grad)

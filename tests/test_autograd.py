@@ -1418,6 +1418,76 @@ def test_whole_model_mse_loss_op(nd):
     assert_close(wide.mse_loss(x, t).to_numpy(), nd.mse(wide.forward(x), t).to_numpy(), tol=1e-6, what="wide model")
 
 
+def test_mse_of_a_whole_model_forward_is_one_launch(nd):
+    """mse(mlp.forward(x), y), the reference script's two calls (mlp_imp.mojo:56-60), on a whole-model MLP: the forward
+    launch is parked and mse() turns it into the launch that also evaluates the loss and all cotangents. Same loss,
+    gradients, output values and output gradient as the per-layer model; reading the output first, a target that needs a
+    gradient, or a second consumer of the output all still work; a captured step replays it."""
+    from endia_amd import _lib as L
+    rng = np.random.default_rng(5)
+    widths = [3, 32, 64, 2]
+    Wn = [(rng.standard_normal((widths[i], widths[i + 1])) / np.sqrt(widths[i])).astype(np.float32) for i in range(3)]
+    bn = [(0.2 * rng.standard_normal(widths[i + 1])).astype(np.float32) for i in range(3)]
+    xn, yn = rng.standard_normal((40, 3)).astype(np.float32), rng.standard_normal((40, 2)).astype(np.float32)
+
+    def model(fused):
+        mlp = nd.nn.MLP(widths, compute_backward=True, activation="relu", fused=fused)
+        for i in range(3):
+            mlp.weights[i], mlp.biases[i] = nd.array(Wn[i], requires_grad=True), nd.array(bn[i], requires_grad=True)
+        return mlp
+
+    ref = model(True)
+    out_r = ref.forward(nd.array(xn))
+    loss_r = nd.mse(out_r, nd.array(yn))
+    loss_r.backward()
+    for variant in ("plain", "read_first", "target_grad", "two_consumers"):
+        mlp = model("model")
+        x, y = nd.array(xn), nd.array(yn, requires_grad=(variant == "target_grad"))
+        calls = []
+        orig = L._raw_call
+        L._raw_call = lambda name, *a: (calls.append(name), orig(name, *a))[1]
+        try:
+            out = mlp.forward(x)
+            assert L._parked and not [c for c in calls if c.startswith("endia_hip_mlp")]
+            if variant == "read_first":
+                first = out.to_numpy()
+            loss = nd.mse(out, y)
+            if variant == "two_consumers":
+                loss = loss + nd.sum(out) * 0.0
+            loss.backward()
+        finally:
+            L._raw_call = orig
+        launches = [c for c in calls if c.startswith("endia_hip_mlp")]
+        if variant == "plain":
+            assert launches == ["endia_hip_mlp_fwd_mse_delta", "endia_hip_mlp_wgrad"], launches
+        elif variant in ("read_first", "target_grad"):
+            assert launches[0] == "endia_hip_mlp_fwd", launches
+        assert_close(loss.to_numpy(), loss_r.to_numpy(), tol=1e-6, what=variant + ": loss")
+        assert_close(out.to_numpy(), out_r.to_numpy(), tol=1e-6, what=variant + ": output")
+        for p, q in zip(mlp.params(), ref.params()):
+            assert_close(p.grad().to_numpy().reshape(-1), q.grad().to_numpy().reshape(-1), tol=2e-5, mean_tol=1e-3, what=variant + ": gradient")
+        if variant == "plain":
+            assert_close(out.grad().to_numpy(), out_r.grad().to_numpy(), tol=1e-6, what="gradient of the model's output")
+    # captured and replayed
+    mlp = model("model")
+    opt = nd.optim.SGD(mlp.params(), lr=0.05)
+    x, y = nd.array(xn), nd.array(yn)
+
+    def step():
+        loss = nd.mse(mlp.forward(x), y)
+        loss.backward()
+        opt.step()
+        loss.zero_grad()
+        return loss
+
+    eager = [float(step().item()) for _ in range(2)]
+    cap = nd.capture(step)
+    assert not L._parked
+    replayed = [float(cap.replay().item()) for _ in range(3)]
+    assert eager[1] < eager[0] and replayed[0] < eager[1] and replayed[2] < replayed[1]
+    cap.close()
+
+
 def test_whole_model_forward_with_cotangents_entry_points(nd):
     """endia_hip_mlp_fwd_mse_delta + endia_hip_mlp_wgrad through the C ABI against endia_hip_mlp_fwd_mse +
     endia_hip_mlp_bwd: the same loss, activations, cotangents of every layer, dx, dW and db, bit for bit (the chain is
