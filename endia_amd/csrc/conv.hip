@@ -898,16 +898,18 @@ struct DirectArgs {
   int MR, plane;      // output rows a pixel tile can touch; floats per cached channel = 3 * MR * PITCH + 32
   int tasks;          // 16-byte pieces of source rows per chunk: 8 * 3 * MR * SW / 4
   FastDiv d_ohw, d_ow, d_oh, d_f4row;
+  FastDiv d_tiles_m;
+  const int2* plan;               // staging plan of a 128-pixel tile (2048 entries) and of a 64-pixel tile (2048 more), see direct3x3_plan
   int tiles_m, relu;
   int full_blocks, full_tiles_n;  // tiles of 128 pixels: full_tiles_n per tile row
   int MR_half, tasks_half;        // the same for the 64-pixel tiles behind them
-  int64_t src_bytes, wp_bytes;
+  int64_t src_bytes, wp_bytes, out_bytes;
 };
 
 // One tile: rows [tm * 64 * FM, ...) of the output channels, pixels [n0, n0 + 64 * FN). MR / tasks: the cache rows and
 // staging pieces a tile of that many pixels needs.
 template <int FM, int FN, int PITCH, bool FWD, int GATE>
-__device__ __forceinline__ void direct3x3_tile(const DirectArgs& a, int tm, int n0, int MR, int tasks, float* smem) {
+__device__ __forceinline__ void direct3x3_tile(const DirectArgs& a, int tm, int n0, int MR, const int2* __restrict__ plan, float* smem) {
   constexpr int BM = 64 * FM, CC = 8, KC = 72, PB = 8;
   float* Bc = smem;
 
@@ -919,35 +921,44 @@ __device__ __forceinline__ void direct3x3_tile(const DirectArgs& a, int tm, int 
   const int img0 = (int)fdiv((uint32_t)n0, a.d_ohw);
   const int grow0 = img0 * a.OH + (int)fdiv((uint32_t)(n0 - img0 * ohw), a.d_ow);
 
+  // What a wave does outside its MFMA loop is vector-ALU work that the MFMAs of the SIMD's other waves wait for, so the
+  // set-up is kept short: which cached row and which 16-byte piece of it a thread stages (task u = tid + 256 p) is the
+  // same for every tile and comes from a table made once per call (direct3x3_plan); what depends on the tile, the
+  // source row under each cached row, is worked out by one lane per cached row and handed over through LDS.
+  int2 te[PB];
+#pragma unroll
+  for (int p = 0; p < PB; ++p) te[p] = plan[tid + p * 256];
+  int* rowbase = reinterpret_cast<int*>(smem + CC * a.plane);  // [3 * MR] byte offsets of the source rows, channel 0
+  if (tid < 3 * MR) {
+    // cached row 3g + r holds source row oy - py + r of the image that output row grow0 + g belongs to, or zeros when
+    // that row does not exist
+    const int g = (int)((uint32_t)tid * 43691u >> 17), r = tid - 3 * g, grow = grow0 + g;
+    uint32_t off = OOB_OFFSET;
+    if (grow < a.NOH) {
+      const int img = (int)fdiv((uint32_t)grow, a.d_oh), y = grow - img * a.OH - a.py + r;
+      if ((unsigned)y < (unsigned)a.SH) off = (uint32_t)((img * a.Cred * a.SH + y) * a.SW) * 4u;
+    }
+    rowbase[tid] = (int)off;
+  }
   // the columns on either side of a cached row are never written again: zero them once (everything between them is
   // rewritten with every chunk, zeros included where a row lies outside its image)
-  for (int i = tid; i < CC * 3 * MR; i += 256) {
-    const int cc = i / (3 * MR), at = cc * a.plane + (i - cc * 3 * MR) * PITCH;
-    Bc[at + 3] = 0.f;
-    Bc[at + 4 + a.SW] = 0.f;
+  if (tid < 3 * MR) {
+#pragma unroll
+    for (int cc = 0; cc < CC; ++cc) {
+      const int at = cc * a.plane + tid * PITCH;
+      Bc[at + 3] = 0.f;
+      Bc[at + 4 + a.SW] = 0.f;
+    }
   }
-
-  // source rows -> cache: task u = (channel, cached row, 16-byte piece); a cached row 3g + r holds source row
-  // oy - py + r of the image that output row grow0 + g belongs to, or zeros when that row does not exist
-  const int f4row = a.SW >> 2;
+  __syncthreads();
   uint32_t goff[PB];
   int loff[PB];
 #pragma unroll
   for (int p = 0; p < PB; ++p) {
-    const int u = tid + p * 256;
-    goff[p] = OOB_OFFSET;
-    loff[p] = -1;
-    if (u < tasks) {
-      const int rowid = (int)fdiv((uint32_t)u, a.d_f4row), c4 = u - rowid * f4row;
-      const int cc = rowid / (3 * MR), rr = rowid - cc * 3 * MR;
-      const int g = rr / 3, r = rr - 3 * g;
-      const int grow = grow0 + g;
-      loff[p] = cc * a.plane + rr * PITCH + 4 + 4 * c4;
-      if (grow < a.NOH) {
-        const int img = (int)fdiv((uint32_t)grow, a.d_oh), y = grow - img * a.OH - a.py + r;
-        if ((unsigned)y < (unsigned)a.SH) goff[p] = (uint32_t)(((img * a.Cred + cc) * a.SH + y) * a.SW + 4 * c4) * 4u;
-      }
-    }
+    const bool task = te[p].x >= 0;  // (entries past the last task are negative)
+    const uint32_t rb = (uint32_t)rowbase[(te[p].x >> 16) & 63];
+    goff[p] = (task && rb != OOB_OFFSET) ? rb + (uint32_t)te[p].y : OOB_OFFSET;
+    loff[p] = task ? (te[p].x & 0xffff) : -1;
   }
   const __amdgpu_buffer_rsrc_t rs_src = make_rsrc(a.src, a.src_bytes);
   const __amdgpu_buffer_rsrc_t rs_w = make_rsrc(a.wp, a.wp_bytes);
@@ -1022,14 +1033,6 @@ __device__ __forceinline__ void direct3x3_tile(const DirectArgs& a, int tm, int 
     if (more) load(chunk + 1);
 #pragma unroll
     for (int jg = 0; jg < KC / 8; ++jg) {  // nine groups of four steps
-      float af[FM][4];
-#pragma unroll
-      for (int fm = 0; fm < FM; ++fm) {
-        const float4 t = afn[jg % AD][fm];
-        af[fm][0] = t.x; af[fm][1] = t.y; af[fm][2] = t.z; af[fm][3] = t.w;
-      }
-      if (jg + AD < KC / 8) fetch_a(chunk, jg + AD);
-      else if (more) fetch_a(chunk + 1, jg + AD - KC / 8);
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
         const int q = 4 * jg + i, ccp = q / 9, tap = q - 9 * ccp, r = tap / 3, sx = tap - 3 * r;
@@ -1037,10 +1040,17 @@ __device__ __forceinline__ void direct3x3_tile(const DirectArgs& a, int tm, int 
 #pragma unroll
         for (int fn = 0; fn < FN; ++fn) bf[fn] = Bc[pix[fn] + 2 * ccp * a.plane + r * PITCH + sx];
 #pragma unroll
-        for (int fm = 0; fm < FM; ++fm)
+        for (int fm = 0; fm < FM; ++fm) {
+          const float4& t = afn[jg % AD][fm];
+          const float av = i == 0 ? t.x : (i == 1 ? t.y : (i == 2 ? t.z : t.w));
 #pragma unroll
-          for (int fn = 0; fn < FN; ++fn) acc[fm][fn] = __builtin_amdgcn_mfma_f32_32x32x2f32(af[fm][i], bf[fn], acc[fm][fn], 0, 0, 0);
+          for (int fn = 0; fn < FN; ++fn) acc[fm][fn] = __builtin_amdgcn_mfma_f32_32x32x2f32(av, bf[fn], acc[fm][fn], 0, 0, 0);
+        }
       }
+      // the group's slot is free once its MFMAs have been issued: the request for the group three further on goes
+      // behind them, so that the fragments are used where they arrive and never copied
+      if (jg + AD < KC / 8) fetch_a(chunk, jg + AD);
+      else if (more) fetch_a(chunk + 1, jg + AD - KC / 8);
     }
     if (more) {
       gate();
@@ -1059,6 +1069,32 @@ __device__ __forceinline__ void direct3x3_tile(const DirectArgs& a, int tm, int 
       const int m = m0 + wm * 32 * FM + fm * 32 + acc_row(v, h);
       bias_v[fm][v] = (FWD && a.bias && m < a.Mrows) ? a.bias[m] : 0.f;
     }
+  // A tile whose rows all exist, in an output of less than 2 GiB: buffer stores, one 32-bit offset per lane and pixel
+  // column, the row's part of the address a scalar of the instruction, no test per element (a pixel past the end gets
+  // an offset the descriptor rejects). What a wave does outside its MFMA loop is vector-ALU work that the SIMD's other
+  // waves' MFMAs wait for, so the fewer instructions here the better.
+  if (m0 + BM <= a.Mrows && a.out_bytes < (1ll << 31)) {
+    const __amdgpu_buffer_rsrc_t rs_out = make_rsrc(a.out, a.out_bytes);
+    const uint32_t row_bytes = (uint32_t)ohw * 4u;
+#pragma unroll
+    for (int fn = 0; fn < FN; ++fn) {
+      const int j = n0 + wn * 32 * FN + fn * 32 + l32;
+      const int img = (int)fdiv((uint32_t)j, a.d_ohw);
+      const uint32_t at = j < a.Ncols ? (uint32_t)((img * a.Mrows + m0 + wm * 32 * FM + 4 * h) * ohw + (j - img * ohw)) * 4u : OOB_OFFSET;
+#pragma unroll
+      for (int fm = 0; fm < FM; ++fm)
+#pragma unroll
+        for (int v = 0; v < 16; ++v) {
+          float val = acc[fm][fn][v];
+          if (FWD) {
+            val += bias_v[fm][v];
+            if (a.relu) val = val > 0.f ? val : 0.f;
+          }
+          __builtin_amdgcn_raw_buffer_store_b32(__float_as_int(val), rs_out, (int)at, (int)((uint32_t)(fm * 32 + 8 * (v >> 2) + (v & 3)) * row_bytes), 0);
+        }
+    }
+    return;
+  }
 #pragma unroll
   for (int fn = 0; fn < FN; ++fn) {
     const int j = n0 + wn * 32 * FN + fn * 32 + l32;
@@ -1090,21 +1126,53 @@ __global__ __launch_bounds__(256, 2) void conv_direct3x3_kernel(DirectArgs a) {
   const int b = blockIdx.x;
   if (b < a.full_blocks) {
     int tm, tn;
-    tile_of_block(b, a.full_blocks, a.tiles_m, a.full_tiles_n, tm, tn);
-    direct3x3_tile<FM, 2, PITCH, FWD, GATE>(a, tm, tn * 128, a.MR, a.tasks, smem);
+    if (a.tiles_m <= 8) {  // tile_of_block for at most one band of tile rows, without its divisions by run-time values
+      int lid = b;
+      if ((a.full_blocks & 7) == 0) lid = (b & 7) * (a.full_blocks >> 3) + (b >> 3);
+      tn = (int)fdiv((uint32_t)lid, a.d_tiles_m);
+      tm = lid - tn * a.tiles_m;
+    } else {
+      tile_of_block(b, a.full_blocks, a.tiles_m, a.full_tiles_n, tm, tn);
+    }
+    direct3x3_tile<FM, 2, PITCH, FWD, GATE>(a, tm, tn * 128, a.MR, a.plan, smem);
   } else {
-    const int hb = b - a.full_blocks, tn = hb / a.tiles_m, tm = hb - tn * a.tiles_m;
-    direct3x3_tile<FM, 1, PITCH, FWD, GATE>(a, tm, a.full_tiles_n * 128 + tn * 64, a.MR_half, a.tasks_half, smem);
+    const int hb = b - a.full_blocks, tn = (int)fdiv((uint32_t)hb, a.d_tiles_m), tm = hb - tn * a.tiles_m;
+    direct3x3_tile<FM, 1, PITCH, FWD, GATE>(a, tm, a.full_tiles_n * 128 + tn * 64, a.MR_half, a.plan + 2048, smem);
   }
+}
+
+// The staging plan of conv_direct3x3_kernel: task u (a channel of the chunk, a cached row, a 16-byte piece of that row)
+// as {LDS word of the piece | cached row << 16, byte offset of the piece from the start of its source row in channel 0
+// of its image}; entries past the last task are negative. One table for 128-pixel tiles, one for 64-pixel tiles.
+struct DirectPlanArgs {
+  int2* plan;
+  int MR, MR_half, f4row, plane, pitch, SH, SW;
+};
+constexpr int PLAN_BLOCKS = 4096 / TPB;
+__device__ __forceinline__ void direct3x3_plan(const DirectPlanArgs& d, int u) {
+  int2* __restrict__ plan = d.plan;
+  const int MR = d.MR, MR_half = d.MR_half, f4row = d.f4row, plane = d.plane, pitch = d.pitch, SH = d.SH, SW = d.SW;
+  const int mr = u < 2048 ? MR : MR_half, t = u & 2047;
+  const int rowid = t / f4row, c4 = t - rowid * f4row;
+  const int cc = rowid / (3 * mr), rr = rowid - cc * 3 * mr;
+  int2 e = make_int2(-1, 0);
+  if (t < 8 * 3 * mr * f4row) e = make_int2((cc * plane + rr * pitch + 4 + 4 * c4) | (rr << 16), (cc * SH * SW + 4 * c4) * 4);
+  plan[u] = e;
 }
 
 // Weights in the order conv_direct3x3_kernel reads them. forward: rows m = output channel, reduced channel ch = input
 // channel, tap (r, s); data gradient: rows m = input channel, reduced channel = output channel, tap (2 - r, 2 - s).
+// (The last PLAN_BLOCKS work-groups of the launch write the staging plan instead: one launch for both.)
 __global__ __launch_bounds__(TPB) void pack_direct3x3_kernel(const float* __restrict__ w, float* __restrict__ wp, int K, int C,
-                                                             int rows_pad, int chunks, int flip) {
+                                                             int rows_pad, int chunks, int flip, DirectPlanArgs plan) {
+  const int packers = (int)gridDim.x - PLAN_BLOCKS;
+  if ((int)blockIdx.x >= packers) {
+    direct3x3_plan(plan, ((int)blockIdx.x - packers) * TPB + (int)threadIdx.x);
+    return;
+  }
   const int Mrows = flip ? C : K, Cred = flip ? K : C;
   const int64_t total = (int64_t)chunks * rows_pad * 72;
-  for (int64_t idx = (int64_t)blockIdx.x * TPB + threadIdx.x; idx < total; idx += (int64_t)gridDim.x * TPB) {
+  for (int64_t idx = (int64_t)blockIdx.x * TPB + threadIdx.x; idx < total; idx += (int64_t)packers * TPB) {
     // [chunk][group j of four steps][row m][half-wave h][step i]: the 64 lanes of a fragment load (32 rows, both
     // half-waves) read 1 KiB in one piece
     const int e = (int)(idx & 7), h = e >> 2, i = e & 3;
@@ -1406,18 +1474,20 @@ int32_t run_direct3x3(int mode, const ConvP& p, const float* src, const float* w
   // a cached channel is 3 * MR rows plus half a row of banks, so that the two half-waves of a fragment read (one
   // channel apart) fall into opposite halves of the 64 LDS banks
   const int plane = 3 * MR * pitch + 32;
-  const size_t lds = (size_t)8 * plane * 4;
-  if (tasks > 2048 || lds > 64 * 1024 || (int64_t)p.N * Cred * SH * SW >= (1ll << 29)) return 1;
+  const size_t lds = (size_t)8 * plane * 4 + 64 * 4;  // the row cache and one source-row offset per cached row
+  if (tasks > 2048 || 3 * MR > 64 || lds > 64 * 1024 || (int64_t)p.N * Cred * SH * SW >= (1ll << 29)) return 1;
   DirectArgs a;
   a.tiles_m = (Mrows + BM - 1) / BM;
   a.chunks = Cred / 8;
   const int rows_pad = a.tiles_m * BM;
-  PoolBuf wp;
+  PoolBuf wp, plan;
   int32_t rc = endia_hip_malloc((int64_t)a.chunks * rows_pad * 72 * 4, &wp.p);
   if (rc) return rc;
+  if ((rc = endia_hip_malloc(4096 * sizeof(int2), &plan.p))) return rc;
   hipStream_t s = endia::ctx().stream;
-  hipLaunchKernelGGL(pack_direct3x3_kernel, dim3(grid_for((int64_t)a.chunks * rows_pad * 72)), dim3(TPB), 0, s, w,
-                     static_cast<float*>(wp.p), p.K, p.C, rows_pad, a.chunks, fwd ? 0 : 1);
+  const DirectPlanArgs plan_args{static_cast<int2*>(plan.p), MR, (63 + OW - 1) / OW + 1, SW / 4, plane, pitch, SH, SW};
+  hipLaunchKernelGGL(pack_direct3x3_kernel, dim3(grid_for((int64_t)a.chunks * rows_pad * 72) + PLAN_BLOCKS), dim3(TPB), 0, s, w,
+                     static_cast<float*>(wp.p), p.K, p.C, rows_pad, a.chunks, fwd ? 0 : 1, plan_args);
   ENDIA_LAUNCH_CHECK();
   a.src = src; a.wp = static_cast<const float*>(wp.p); a.bias = bias; a.out = out; a.relu = relu;
   a.gscalar = gscalar;
@@ -1426,6 +1496,7 @@ int32_t run_direct3x3(int mode, const ConvP& p, const float* src, const float* w
   a.d_ohw = make_fastdiv(OH * OW); a.d_ow = make_fastdiv(OW); a.d_oh = make_fastdiv(OH); a.d_f4row = make_fastdiv(SW / 4);
   a.src_bytes = (int64_t)p.N * Cred * SH * SW * 4;
   a.wp_bytes = (int64_t)a.chunks * rows_pad * 72 * 4;
+  a.out_bytes = (int64_t)p.N * Mrows * OH * OW * 4;
   // The busiest CU sets the time, and with t tiles on c CUs it works on ceil(t / c) of them. When the tiles beyond the
   // last full round are few (at most one for every other CU), they are cut into 64-pixel tiles: twice as many CUs get
   // half as much extra work. 200704 pixels, 64 channels per tile row: 1568 tiles = 6 rounds + 32 -> 6 rounds + 64 halves.
@@ -1438,6 +1509,8 @@ int32_t run_direct3x3(int mode, const ConvP& p, const float* src, const float* w
   const int half_tiles_n = left > 0 ? (left + 63) / 64 : 0;
   a.MR_half = (63 + OW - 1) / OW + 1;
   a.tasks_half = 8 * 3 * a.MR_half * (SW / 4);
+  a.d_tiles_m = make_fastdiv(a.tiles_m);
+  a.plan = static_cast<const int2*>(plan.p);
   const dim3 grid((unsigned)(a.full_blocks + a.tiles_m * half_tiles_n));
 #define ENDIA_LAUNCH_DIRECT(FM, PITCH)                                                                                       \
   do {                                                                                                                       \
