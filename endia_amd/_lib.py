@@ -121,7 +121,7 @@ SIGNATURES = {
     "endia_hip_complex_pack": [c_int64, _fp, _fp, _fp],
     "endia_hip_reduce_add": [c_int32, _i64p, c_uint32, _fp, _fp, c_float, c_int32],
     "endia_hip_col_sum_static": [c_int64, c_int64, _fp, _fp, c_float],
-    "endia_hip_col_sum_plan": [c_int64, c_int64, c_int64, c_int64, _i64p, _i64p],
+    "endia_hip_col_sum_plan": [c_int64, c_int64, c_int64, c_int64, c_int32, _i64p, _i64p],
     "endia_hip_reduce": [c_int32, c_int32, _i64p, c_uint32, _fp, _fp],
     "endia_hip_mse_fwd_bwd": [c_int64, _fp, _fp, _fp, _fp],
     "endia_hip_conv2d_out_shape": [POINTER(Conv2dDesc), _i64p, _i64p],

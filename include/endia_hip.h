@@ -359,11 +359,12 @@ ENDIA_API int32_t endia_hip_reduce_add(int32_t ndim, const int64_t* shape, uint3
 ENDIA_API int32_t endia_hip_col_sum_static(int64_t R, int64_t C, const float* x, float* out, float scale);
 /* How a column sum of R rows and C columns cuts its rows on a device of cu_count CUs when scratch_floats floats are
  * there for first-stage partial sums (0: no limit, what endia_hip_reduce_add has; 262144: endia_hip_col_sum_static).
- * No counterpart in the reference; pure arithmetic, needs no device and no endia_hip_init. splits = 0: one launch without
- * a first stage; -1: C does not fit the scratch; otherwise `splits` pieces of rows_per_split rows. Two calls that get
- * the same plan add in the same order and agree bit for bit. */
-ENDIA_API int32_t endia_hip_col_sum_plan(int64_t R, int64_t C, int64_t cu_count, int64_t scratch_floats, int64_t* splits,
-                                         int64_t* rows_per_split);
+ * aligned16: x and out start on 16-byte boundaries. No counterpart in the reference; pure arithmetic, needs no device
+ * and no endia_hip_init. splits = 0: one launch without a first stage (small inputs, and aligned inputs of up to 2^22
+ * elements and 2048 rows); -1: C does not fit the scratch; otherwise `splits` pieces of rows_per_split rows. Two calls
+ * that get the same plan add in the same order and agree bit for bit. */
+ENDIA_API int32_t endia_hip_col_sum_plan(int64_t R, int64_t C, int64_t cu_count, int64_t scratch_floats, int32_t aligned16,
+                                         int64_t* splits, int64_t* rows_per_split);
 
 /* ---- the other reductions: ReduceMax / ReduceMin / ReduceMul .__call__ (reduce_ops/reduce_max_op.mojo:66-190,
  *      reduce_min_op.mojo:66-190, reduce_mul_op.mojo:65-210) and ReduceArgMax / ReduceArgMin .__call__

@@ -114,9 +114,9 @@ def test_col_sum_plan_clamps_to_the_scratch():
     forces fewer pieces, down to refusing columns that do not fit at all; a small input needs no first stage."""
     lib = L.lib()
 
-    def plan(R, C, cus, scratch):
+    def plan(R, C, cus, scratch, aligned=1):
         S, rows = ctypes.c_int64(), ctypes.c_int64()
-        assert lib.endia_hip_col_sum_plan(R, C, cus, scratch, ctypes.byref(S), ctypes.byref(rows)) == 0
+        assert lib.endia_hip_col_sum_plan(R, C, cus, scratch, aligned, ctypes.byref(S), ctypes.byref(rows)) == 0
         return S.value, rows.value
 
     assert plan(4096, 4096, 256, 0) == (64, 64)
@@ -126,7 +126,10 @@ def test_col_sum_plan_clamps_to_the_scratch():
     assert plan(24, 1 << 18, 256, 1 << 18) == (1, 24)
     assert plan(24, (1 << 18) + 4, 256, 1 << 18)[0] == -1      # does not fit
     assert plan(40, 96, 256, 1 << 18) == (0, 40)               # one launch
-    for R, C, cus, scratch in [(1500, 772, 256, 1 << 18), (100000, 64, 304, 4096), (2000, 5000, 8, 0)]:
+    assert plan(1024, 2048, 256, 0) == (0, 1024)               # a mid-size aligned input: one launch as well
+    assert plan(1024, 2048, 256, 0, aligned=0)[0] >= 1         # ... unless it cannot be read 16 bytes at a time
+    assert plan(1024, 2050, 256, 0)[0] >= 1
+    for R, C, cus, scratch in [(5000, 772, 256, 1 << 18), (100000, 64, 304, 4096), (2000, 5000, 8, 0)]:
         S, rows = plan(R, C, cus, scratch)
         assert S >= 1 and (S - 1) * rows < R <= S * rows and (scratch == 0 or S * C <= scratch)
-    assert lib.endia_hip_col_sum_plan(0, 4, 256, 0, None, None) == L.ERR_INVALID
+    assert lib.endia_hip_col_sum_plan(0, 4, 256, 0, 1, None, None) == L.ERR_INVALID

@@ -22,7 +22,7 @@ def _same_plan(R, C):
     plans = []
     for scratch in (0, 1 << 18):
         S, rows = ctypes.c_int64(), ctypes.c_int64()
-        L.call("endia_hip_col_sum_plan", R, C, cus, scratch, ctypes.byref(S), ctypes.byref(rows))
+        L.call("endia_hip_col_sum_plan", R, C, cus, scratch, 1, ctypes.byref(S), ctypes.byref(rows))
         plans.append((S.value, rows.value))
     return plans[0] == plans[1]
 
@@ -44,16 +44,18 @@ def _both(dev, x, scale=1.0):
 def test_col_sum_static_matches_reduce_add_twice_in_a_row(dev):
     rng = np.random.default_rng(11)
     big = rng.standard_normal((4096, 4096)).astype(np.float32)      # the wide MLP's bias gradient: two stages, 64 row splits
-    small = rng.standard_normal((1500, 772)).astype(np.float32)    # smaller, still two stages
+    small = rng.standard_normal((5000, 772)).astype(np.float32)    # smaller, still two stages (more than 4096 rows)
     for x, scale in ((big, 1.0), (small, 0.5)):
         got, ref = _both(dev, x, scale)
         if _same_plan(*x.shape):
             assert np.array_equal(got, ref), "static-scratch column sums differ from endia_hip_reduce_add"
         assert_close(got, ref, tol=1e-6, what="static scratch vs reduce_add")
         assert_close(got, scale * x.astype(np.float64).sum(axis=0), what="column sums %s" % (x.shape,))
-    tiny = rng.standard_normal((40, 96)).astype(np.float32)        # the single-launch path (no scratch at all)
-    got, ref = _both(dev, tiny)
-    assert np.array_equal(got, ref)
+    for shape in ((40, 96), (1024, 2048)):                          # the single-launch paths (no scratch at all): small, mid-size
+        tiny = rng.standard_normal(shape).astype(np.float32)
+        got, ref = _both(dev, tiny)
+        assert np.array_equal(got, ref)
+        assert_close(got, tiny.astype(np.float64).sum(axis=0), what="column sums %s" % (shape,))
 
 
 def test_col_sum_static_widest_input(dev):
