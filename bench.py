@@ -826,7 +826,7 @@ def main():
     cpu = not args.no_cpu_baseline
 
     if args.workload == "hvp":
-        out = run_hvp(nd, args.steps, args.warmup)
+        out = run_hvp(nd, max(args.steps, 40) if args.steps == 20 else args.steps, args.warmup)  # (short runs measure the clock ramp)
         if cpu:
             out["cpu_baseline"] = cpu_baseline_hvp()
     elif args.workload.startswith("complex_mlp"):
@@ -834,7 +834,7 @@ def main():
         if cpu:
             out["cpu_baseline"] = cpu_baseline_complex()
     elif args.workload == "conv2d":
-        out = run_conv(nd, max(args.steps, 1), args.warmup)
+        out = run_conv(nd, 100 if args.steps == 20 else max(args.steps, 1), max(args.warmup, 10))  # (short runs measure the clock ramp)
         if cpu:
             out["cpu_baseline"] = cpu_baseline_conv()
     elif args.workload == "conv2d_kernels":

@@ -308,14 +308,17 @@ def flush(need=None):
         _parked.remove(it)  # (nothing below comes back here: the raw call flushes nothing)
     try:
         _raw_call("endia_hip_sgemm_grouped", len(products), descs, index, done)
-    finally:
-        if flush_observer[0] is not None:
-            flush_observer[0]([item[0] for item in products], index, list(done))
-        for item, flag in zip(products, done):
-            if flag or index < 0:
-                item[2].pending = False
-            else:
-                _parked.append(item)
+    except BaseException:
+        for item in products:  # a launch that failed is not tried again: the error is the caller's to see, once
+            item[2].pending = False
+        raise
+    if flush_observer[0] is not None:
+        flush_observer[0]([item[0] for item in products], index, list(done))
+    for item, flag in zip(products, done):
+        if flag or index < 0:
+            item[2].pending = False
+        else:
+            _parked.append(item)
 
 
 def call(name, *args):
