@@ -25,6 +25,7 @@
 
 namespace endia {
 int32_t col_reduce(int64_t batch, int64_t R, int64_t C, const float* x, float* out, float scale);
+int32_t col_reduce_transposed(int64_t R, int64_t C, int64_t inner, const float* x, float* out);
 int32_t row_reduce(int64_t R, int64_t C, const float* x, float* out, float scale);
 }
 
@@ -1627,7 +1628,7 @@ int32_t run_wgrad3x3(const ConvP& p, const float* x, const float* dy, float* dw,
   const int64_t splits = (int64_t)p.N * a.wgs_per_image;
   if (splits > 65535 || tiles > (1ll << 30)) return 1;
   const int64_t taps = (int64_t)9 * p.K * p.C;
-  PoolBuf part, ordered, bias_part;
+  PoolBuf part, bias_part;
   int32_t rc;
   if ((rc = endia_hip_malloc(splits * taps * 4, &part.p))) return rc;
   float* db_part = db;
@@ -1644,14 +1645,12 @@ int32_t run_wgrad3x3(const ConvP& p, const float* x, const float* dy, float* dw,
   else if (gate_mode == 1) hipLaunchKernelGGL((conv_wgrad3x3_kernel<1>), grid, dim3(256), 0, s, a);
   else hipLaunchKernelGGL((conv_wgrad3x3_kernel<2>), grid, dim3(256), 0, s, a);
   ENDIA_LAUNCH_CHECK();
-  const float* summed = a.part;
-  if (splits > 1) {  // partials added in split order
-    if ((rc = endia_hip_malloc(taps * 4, &ordered.p))) return rc;
-    if ((rc = endia::col_reduce(1, splits, taps, a.part, static_cast<float*>(ordered.p), 1.f))) return rc;
-    summed = static_cast<const float*>(ordered.p);
+  if (splits > 1) {  // partials added in split order; the last stage of the sum stores [tap][k][c] as the weights' [k][c][tap]
+    if ((rc = endia::col_reduce_transposed(splits, taps, (int64_t)p.K * p.C, a.part, dw))) return rc;
     if (db && (rc = endia::col_reduce(1, splits, p.K, db_part, db, 1.f))) return rc;
+    return ENDIA_HIP_OK;
   }
-  hipLaunchKernelGGL(wgrad3x3_order_kernel, dim3(grid_for(taps)), dim3(TPB), 0, s, summed, dw, p.K, p.C);
+  hipLaunchKernelGGL(wgrad3x3_order_kernel, dim3(grid_for(taps)), dim3(TPB), 0, s, a.part, dw, p.K, p.C);
   ENDIA_LAUNCH_CHECK();
   return ENDIA_HIP_OK;
 }

@@ -112,8 +112,10 @@ __global__ __launch_bounds__(TPB) void col_reduce_scalar_kernel(const float* __r
 
 // stage 2: out[b][c] = scale * sum_s part[b][s][c]. 64 columns per group; the four waves take
 // s = w, w+4, ... and are combined through LDS in wave order, so the result does not depend on timing.
+// inner > 0: the columns are an [C / inner][inner] array and the sums are stored transposed, as [inner][C / inner] (the
+// 3 x 3 weight gradient sums its partial products in [tap][k][c] order and stores them as the weights' [k][c][tap]).
 __global__ __launch_bounds__(TPB) void col_reduce_final_kernel(const float* __restrict__ part, float* __restrict__ out,
-                                                               int64_t S, int64_t C, int64_t batch, float scale) {
+                                                               int64_t S, int64_t C, int64_t batch, float scale, int64_t inner) {
   __shared__ float red[4][64];
   const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
   const int64_t c = (int64_t)blockIdx.x * 64 + lane;
@@ -125,7 +127,14 @@ __global__ __launch_bounds__(TPB) void col_reduce_final_kernel(const float* __re
   }
   red[w][lane] = acc;
   __syncthreads();
-  if (w == 0 && c < C) out[b * C + c] = ((red[0][lane] + red[1][lane]) + (red[2][lane] + red[3][lane])) * scale;
+  if (w == 0 && c < C) {
+    int64_t at = c;
+    if (inner > 0) {
+      const int64_t o = c / inner;
+      at = (c - o * inner) * (C / inner) + o;
+    }
+    out[b * C + at] = ((red[0][lane] + red[1][lane]) + (red[2][lane] + red[3][lane])) * scale;
+  }
 }
 
 // ---- row reduction: x[R][C] -> out[R] (sum over C) --------------------------------------------
@@ -161,8 +170,17 @@ __global__ __launch_bounds__(TPB) void row_reduce_final_kernel(const float* __re
   const int lane = threadIdx.x & 63;
   const int64_t r = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
   if (r >= R) return;
+  // (eight loads in flight: a full reduction's 2048 partial sums are 32 rounds of one dependent load each otherwise)
   float acc = 0.f;
-  for (int64_t s = lane; s < S; s += 64) acc += part[r * S + s];
+  int64_t s = lane;
+  for (; s + 7 * 64 < S; s += 8 * 64) {
+    float t[8];
+#pragma unroll
+    for (int u = 0; u < 8; ++u) t[u] = part[r * S + s + 64 * u];
+#pragma unroll
+    for (int u = 0; u < 8; ++u) acc += t[u];
+  }
+  for (; s < S; s += 64) acc += part[r * S + s];
   acc = wave_sum(acc);
   if (lane == 0) out[r] = acc * scale;
 }
@@ -371,7 +389,7 @@ static void col_reduce_plan(int64_t batch, int64_t R, int64_t C, int64_t cus, in
 // out[b][c] = scale * sum_r x[b][r][c]. The first-stage partial sums go to `part` (room for part_floats) when the
 // caller brings it, else to the library's workspace; with too little room the rows are cut into fewer splits.
 static int32_t col_reduce_with(int64_t batch, int64_t R, int64_t C, const float* x, float* out, float scale, float* part,
-                               int64_t part_floats) {
+                               int64_t part_floats, int64_t inner = 0) {
   hipStream_t s = ctx().stream;
   const bool vec = (C % 4 == 0) && al16(x);
   const int64_t col_tiles = ceil_div64(C, 256);
@@ -380,7 +398,7 @@ static int32_t col_reduce_with(int64_t batch, int64_t R, int64_t C, const float*
   // A small input (the bias gradient of a narrow layer) is one launch: the second-stage kernel applied to the
   // input itself, 64 columns per group, the four waves taking alternate rows.
   int64_t S = 0, rows_per_split = 0;
-  const bool vec_out = vec && al16(out);
+  const bool vec_out = vec && al16(out) && inner == 0;  // (the one-launch kernel for mid-size inputs stores in place)
   col_reduce_plan(batch, R, C, ctx().cu_count, part ? part_floats : 0, vec_out, &S, &rows_per_split);
   if (S == 0 && !(R <= 1024 && batch * R * C <= (1 << 20))) {
     hipLaunchKernelGGL(col_reduce_mid_kernel, dim3((unsigned)ceil_div64(C, 16)), dim3(TPB), 0, s, x, out, R, C, scale);
@@ -389,7 +407,7 @@ static int32_t col_reduce_with(int64_t batch, int64_t R, int64_t C, const float*
   }
   if (S == 0) {
     hipLaunchKernelGGL(col_reduce_final_kernel, dim3((unsigned)ceil_div64(C, 64), (unsigned)batch), dim3(TPB), 0, s, x, out, R,
-                       C, batch, scale);
+                       C, batch, scale, inner);
     ENDIA_LAUNCH_CHECK();
     return ENDIA_HIP_OK;
   }
@@ -405,13 +423,18 @@ static int32_t col_reduce_with(int64_t batch, int64_t R, int64_t C, const float*
   else hipLaunchKernelGGL(col_reduce_scalar_kernel, grid, dim3(TPB), 0, s, x, part, R, C, rows_per_split);
   ENDIA_LAUNCH_CHECK();
   hipLaunchKernelGGL(col_reduce_final_kernel, dim3((unsigned)ceil_div64(C, 64), (unsigned)batch), dim3(TPB), 0, s, part,
-                     out, S, C, batch, scale);
+                     out, S, C, batch, scale, inner);
   ENDIA_LAUNCH_CHECK();
   return ENDIA_HIP_OK;
 }
 
 int32_t col_reduce(int64_t batch, int64_t R, int64_t C, const float* x, float* out, float scale) {
   return col_reduce_with(batch, R, C, x, out, scale, nullptr, 0);
+}
+
+// The same with the sums stored transposed: column c = o * inner + i goes to out[i * (C / inner) + o]. inner divides C.
+int32_t col_reduce_transposed(int64_t R, int64_t C, int64_t inner, const float* x, float* out) {
+  return col_reduce_with(1, R, C, x, out, 1.f, nullptr, 0, inner);
 }
 
 // out[r] = scale * sum_c x[r][c]
