@@ -33,7 +33,7 @@ HBM_PEAK_GBS = 8000.0
 # 7 NN with bias+tanh, 7 NT with the tanh' epilogue, 8 TN, all on the 256 x 256 tile; MiB per launch as in the per-kernel table). It cannot be read while the benchmark runs: it comes
 # from two rocprofv3 --pmc runs (FETCH_SIZE, WRITE_SIZE in KiB per dispatch), each scaled by what the same counter
 # reads for a 64 MiB copy kernel (x1.999 and x1.000); the per-kernel table is in profiles/.
-GEMM_TRAFFIC_BYTES = int((1 * 451.2 + 7 * 449.1 + 7 * 512.3 + 8 * 450.9) / 23 * 1024 * 1024)
+GEMM_TRAFFIC_BYTES = int((1 * 456.7 + 7 * 449.1 + 7 * 512.3 + 8 * 456.4) / 23 * 1024 * 1024)
 
 
 def build_wide_mlp(nd, width=4096, layers=8, batch=4096, seed=2, fused_backward=False):
