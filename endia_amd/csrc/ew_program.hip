@@ -22,8 +22,6 @@
 namespace {
 
 constexpr int TPB = 256;
-constexpr int CH = 4;                 // float4 chunks per lane in the tiled kernel
-constexpr int TILE = 64 * 4 * CH;     // elements one wave covers per pass: 1024
 
 struct EwArgs {
   const float* in[ENDIA_EW_MAX_INPUTS];
@@ -178,27 +176,40 @@ __device__ __forceinline__ void run_program(const EwArgs& a, int64_t base, const
   }
 }
 
-// One wave per 1024-element tile, waves striding over the tiles of [begin, n). n - begin is a multiple of TILE.
+// One wave per tile of 256 * C elements, waves striding over the tiles of [begin, n). n - begin is a multiple of the
+// tile. C = 4 shares a step's decode among sixteen elements of a lane, which is what an array that fills the chip
+// many times over wants; an array of a few million elements has fewer such tiles than the chip has wave slots and is
+// bound by the latency of one wave's chain of loads, so it takes C = 2 or 1 and spreads over four times the waves.
+template <int C>
 __global__ __launch_bounds__(TPB) void ew_program_tiled_kernel(const EwArgs a) {
-  // 16 KiB per save slot that the program uses (dynamic, so a program without saved values does not
+  // 4 * C KiB per save slot that the program uses (dynamic, so a program without saved values does not
   // pay for them in occupancy)
   extern __shared__ float4 slot_mem[];
-  float4 (*slots)[CH][TPB] = reinterpret_cast<float4 (*)[CH][TPB]>(slot_mem);
+  float4 (*slots)[C][TPB] = reinterpret_cast<float4 (*)[C][TPB]>(slot_mem);
   const int lane = threadIdx.x & 63;
   const int64_t wave = (int64_t)blockIdx.x * (TPB / 64) + (threadIdx.x >> 6);
   const int64_t waves = (int64_t)gridDim.x * (TPB / 64);
-  const int64_t tiles = (a.n - a.begin) / TILE;
+  const int64_t tiles = (a.n - a.begin) / (256 * C);
   for (int64_t t = wave; t < tiles; t += waves) {
-    const int64_t base = a.begin + t * TILE + lane * 4;
-    int col[CH] = {0, 0, 0, 0};
+    const int64_t base = a.begin + t * (256 * C) + lane * 4;
+    int col[C];
+#pragma unroll
+    for (int c = 0; c < C; ++c) col[c] = 0;
     if (a.need_col) {
       const int cols = (int)a.cols;  // the host takes this path only for cols < 2^31
       int c0 = (int)(base % a.cols);
 #pragma unroll
-      for (int c = 0; c < CH; ++c) col[c] = (int)(((unsigned)c0 + 256u * c) % (unsigned)cols);
+      for (int c = 0; c < C; ++c) col[c] = (int)(((unsigned)c0 + 256u * c) % (unsigned)cols);
     }
-    run_program<CH, 4, float4>(a, base, col, slots);
+    run_program<C, 4, float4>(a, base, col, slots);
   }
+}
+
+template <int C>
+int resident_tiled_groups(size_t lds) {
+  int r = 0;
+  if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&r, ew_program_tiled_kernel<C>, TPB, lds) != hipSuccess || r < 1) r = 2;
+  return r;
 }
 
 // One element per lane over [begin, n): unaligned operands, odd row lengths and the tail of the tiled kernel.
@@ -292,29 +303,40 @@ extern "C" int32_t endia_hip_ew_program(int64_t rows, int64_t cols, int32_t n_in
   if (a.n == 0) return ENDIA_HIP_OK;
   // A grid-stride kernel wants exactly as many work-groups as fit on the chip at once: one more and
   // the extra groups run as a second round after the first has finished.
-  static int resident_scalar = 0, resident_tiled[ENDIA_EW_MAX_SLOTS + 1] = {0};
-  const size_t lds = (size_t)n_slots * CH * TPB * sizeof(float4);
+  static int resident_scalar = 0, resident_tiled[3][ENDIA_EW_MAX_SLOTS + 1] = {{0}};
   if (resident_scalar == 0) {
     if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&resident_scalar, ew_program_scalar_kernel, TPB, 0) != hipSuccess ||
         resident_scalar < 1)
       resident_scalar = 4;
   }
-  if (resident_tiled[n_slots] == 0) {
-    int r = 0;
-    if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&r, ew_program_tiled_kernel, TPB, lds) != hipSuccess || r < 1) r = 2;
-    resident_tiled[n_slots] = r;
-  }
-  const int resident[2] = {resident_scalar, resident_tiled[n_slots]};
   const int64_t cus = ctx().cu_count > 0 ? ctx().cu_count : 256;
   const int64_t total = a.n;
   vec = vec && cols < (1ll << 31) - 1024;
-  const int64_t tiled_n = vec ? total / TILE * TILE : 0;
+  // chunks per lane: the most (4, 2, 1) that still gives every wave slot of the chip a tile
+  int ci = 2;  // index into {1, 2, 4}
+  if (vec) {
+    for (; ci > 0; --ci) {
+      const size_t lds_c = (size_t)n_slots * (1 << ci) * TPB * sizeof(float4);
+      if (resident_tiled[ci][n_slots] == 0)
+        resident_tiled[ci][n_slots] = ci == 2 ? resident_tiled_groups<4>(lds_c) : resident_tiled_groups<2>(lds_c);
+      if (2 * (total / (256 << ci)) >= cus * resident_tiled[ci][n_slots] * (TPB / 64)) break;
+    }
+    if (ci == 0 && resident_tiled[0][n_slots] == 0)
+      resident_tiled[0][n_slots] = resident_tiled_groups<1>((size_t)n_slots * TPB * sizeof(float4));
+  }
+  const int chunks = 1 << ci;
+  const int64_t tile = 256 * chunks;
+  const size_t lds = (size_t)n_slots * chunks * TPB * sizeof(float4);
+  const int resident[2] = {resident_scalar, vec ? resident_tiled[ci][n_slots] : 0};
+  const int64_t tiled_n = vec ? total / tile * tile : 0;
   if (tiled_n > 0) {
     a.begin = 0;
     a.n = tiled_n;
-    int64_t blocks = ceil_div64(tiled_n / TILE, TPB / 64);
+    int64_t blocks = ceil_div64(tiled_n / tile, TPB / 64);
     if (blocks > cus * resident[1]) blocks = cus * resident[1];
-    hipLaunchKernelGGL(ew_program_tiled_kernel, dim3((unsigned)blocks), dim3(TPB), lds, ctx().stream, a);
+    if (chunks == 4) hipLaunchKernelGGL(ew_program_tiled_kernel<4>, dim3((unsigned)blocks), dim3(TPB), lds, ctx().stream, a);
+    else if (chunks == 2) hipLaunchKernelGGL(ew_program_tiled_kernel<2>, dim3((unsigned)blocks), dim3(TPB), lds, ctx().stream, a);
+    else hipLaunchKernelGGL(ew_program_tiled_kernel<1>, dim3((unsigned)blocks), dim3(TPB), lds, ctx().stream, a);
   }
   if (tiled_n < total) {
     a.begin = tiled_n;

@@ -209,7 +209,7 @@ def _program_expected(rows, cols, inputs, modes, n_out, steps):
     return outs
 
 
-@pytest.mark.parametrize("rows,cols", [(1, 1), (3, 5), (64, 48), (33, 1000), (2, 4099)])
+@pytest.mark.parametrize("rows,cols", [(1, 1), (3, 5), (64, 48), (33, 1000), (2, 4099), (1024, 2052), (2300, 2048)])  # the last two: 512- and 1024-element tiles
 def test_ew_program(dev, rows, cols):
     rng = np.random.default_rng(rows * 131 + cols)
     a = rng.standard_normal((rows, cols)).astype(np.float32)
@@ -236,11 +236,14 @@ def test_ew_program(dev, rows, cols):
     modes = [L.EW_FULL, L.EW_FULL, L.EW_ROW_VECTOR, L.EW_SCALAR]
     got = _run_program(dev, rows, cols, [a, b, bias, scale], modes, 2, steps)
     want = _program_expected(rows, cols, [a, b, bias, scale], modes, 2, steps)
+    # 1 - tanh^2 cancels for |z| > 8; among two million samples a few such entries carry the mean of the per-element
+    # relative errors, so the large shapes bound that metric by 1e-2 (the L2 bound stays, and catches a misplaced tile)
+    mean_tol = 1e-2 if rows * cols > (1 << 20) else None
     for i in range(2):
-        assert_close(got[i], want[i], what="program output %d (%d x %d)" % (i, rows, cols))
+        assert_close(got[i], want[i], what="program output %d (%d x %d)" % (i, rows, cols), mean_tol=mean_tol)
     z = a.astype(np.float64) * b + bias
     assert_close(got[0], np.tanh(z), what="tanh(a*b+bias) vs float64")
-    assert_close(got[1], (1 - np.tanh(z) ** 2) * 0.75 * (1 + np.exp(-z)), what="second output vs float64")
+    assert_close(got[1], (1 - np.tanh(z) ** 2) * 0.75 * (1 + np.exp(-z)), what="second output vs float64", mean_tol=mean_tol)
 
 
 def test_ew_program_rejects_bad_programs(dev):
