@@ -233,6 +233,14 @@ int32_t sgemm_impl(int transA, int transB, int64_t M, int64_t N, int64_t K, cons
   p.act = act; p.from_out = from_out; p.accumulate = accumulate;
   hipStream_t s = ctx().stream;
 
+  // A classifier head: a handful of output columns, a long reduction. One pass over A at memory speed (gemm_narrow.hip).
+  if (g_forced_tile == 0 && narrow_ok(transA, transB, M, N, K, batch, A, lda, B, ldb, colsum)) {
+    const int32_t rc = launch_narrow(p, epi, transB, s);
+    if (rc) return rc;
+    ENDIA_LAUNCH_CHECK();
+    return ENDIA_HIP_OK;
+  }
+
   // The vector path loads 4 floats at a time along the contiguous index of each operand.
   const bool a_ok = aligned16(A) && lda % 4 == 0 && sA % 4 == 0 && (transA ? M % 4 == 0 : K % 4 == 0);
   const bool b_ok = aligned16(B) && ldb % 4 == 0 && sB % 4 == 0 && (transB ? K % 4 == 0 : N % 4 == 0);

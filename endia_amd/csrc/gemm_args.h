@@ -95,6 +95,12 @@ int32_t launch_lone_grouped_256x128(const GroupArgs& g, hipStream_t s);
 // Launcher of the shared-CU tiles (tile = 64 or 128) for operands read 4 bytes at a time (gemm_unaligned.hip).
 void launch_mfma_unaligned(const GemmArgs& p, int epi, int tile, bool a_vec, bool b_vec, int transA, int transB, dim3 grid, hipStream_t s);
 
+// Products with at most 16 output columns and a long reduction over a row-major A (gemm_narrow.hip): whether the kernel takes
+// the product, and its launch.
+bool narrow_ok(int transA, int transB, int64_t M, int64_t N, int64_t K, int64_t batch, const float* A, int64_t lda, const float* B,
+               int64_t ldb, int colsum);
+int32_t launch_narrow(const GemmArgs& p, int epi, int transB, hipStream_t s);
+
 // Launchers of the one-wave-per-SIMD tiles, one translation unit per tile shape (gemm_lone_*.hip).
 // The caller checks the launch with hipGetLastError.
 int32_t launch_lone_256x256(const GemmArgs& p, int epi, int transA, int transB, dim3 grid, hipStream_t s);

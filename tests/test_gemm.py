@@ -105,6 +105,42 @@ def test_sgemm_unaligned_operands_on_the_matrix_cores(dev, M, N, K, pad_a, pad_b
         assert_close(dev.get(dsum, (N,)), B.astype(np.float64).sum(0), what="column sums of B")
 
 
+@pytest.mark.parametrize("tb", [0, 1])
+@pytest.mark.parametrize("M,N,K,pad_a", [(4096, 10, 4096, 0), (1000, 7, 1028, 4), (256, 16, 512, 0), (300, 1, 2052, 8), (2049, 3, 640, 0)])
+def test_sgemm_few_output_columns(dev, M, N, K, pad_a, tb):
+    """A classifier head: at most 16 output columns over a long reduction (matmul_op.mojo:93-199 takes any shape). One pass
+    over A with the reduction cut across the waves of a work-group; ragged M and K, padded rows of A, B stored either way,
+    every epilogue and accumulation, against the oracle and float64; repeated runs give the same bits."""
+    rng = np.random.default_rng(M + 3 * N + 5 * K + tb)
+    bufA, A = _embedded(rng, M, K, K + pad_a, 0)
+    B = (rng.standard_normal((N, K) if tb else (K, N)) / np.sqrt(K)).astype(np.float32)
+    dA, dB = dev.put(bufA), dev.put(B)
+    opB = B.T if tb else B
+    ref64 = A.astype(np.float64) @ opB.astype(np.float64)
+    ref = R.matmul(np.ascontiguousarray(A), np.ascontiguousarray(opB))
+
+    def run(epi=L.EPI_NONE, act=L.OP_IDENTITY, bias=None, aux=None, C0=None, aux_out=None):
+        dC = dev.put(C0) if C0 is not None else dev.alloc(M * N * 4)
+        dev.call("endia_hip_sgemm", 0, tb, M, N, K, dA, K + pad_a, dB, B.shape[1], dC, N, 1, 0, 0, 0, epi, act,
+                 dev.put(bias) if bias is not None else None, dev.put(aux) if aux is not None else None, aux_out)
+        return dev.get(dC, (M, N))
+
+    first = run()
+    assert_close(first, ref, what="vs oracle")
+    assert_close(first, ref64, what="vs float64")
+    for _ in range(2):
+        np.testing.assert_array_equal(run(), first)
+    bias = rng.standard_normal(N).astype(np.float32)
+    aux = rng.standard_normal((M, N)).astype(np.float32)
+    assert_close(run(L.EPI_BIAS, bias=bias), ref64 + bias, what="bias")
+    dz = dev.alloc(M * N * 4)
+    assert_close(run(L.EPI_BIAS_ACT, L.OP_TANH, bias=bias, aux_out=dz), np.tanh(ref64 + bias), what="bias + tanh")
+    assert_close(dev.get(dz, (M, N)), ref64 + bias, what="stored pre-activation")
+    assert_close(run(L.EPI_ACT_GRAD, L.OP_SIN, aux=aux), ref64 * np.cos(aux.astype(np.float64)), what="sin gradient epilogue")
+    C0 = rng.standard_normal((M, N)).astype(np.float32)
+    assert_close(run(L.EPI_NONE | L.GEMM_ACCUMULATE, C0=C0), C0 + ref64, what="accumulate")
+
+
 def _grouped(dev, members):
     """members: dicts with ta, tb, A, B (host arrays as stored), optional bias, C0 (accumulate). Runs them through
     endia_hip_sgemm_grouped and returns the outputs."""
