@@ -69,6 +69,10 @@ class SgemmDesc(ctypes.Structure):
                 ("bias", c_void_p)]
 
 
+class ColSumDesc(ctypes.Structure):
+    _fields_ = [("R", c_int64), ("C", c_int64), ("x", c_void_p), ("out", c_void_p), ("scale", c_float)]
+
+
 _fp = c_void_p  # device pointers travel as plain addresses
 _i64p = POINTER(c_int64)
 
@@ -122,6 +126,7 @@ SIGNATURES = {
     "endia_hip_reduce_add": [c_int32, _i64p, c_uint32, _fp, _fp, c_float, c_int32],
     "endia_hip_col_sum_static": [c_int64, c_int64, _fp, _fp, c_float],
     "endia_hip_col_sum_plan": [c_int64, c_int64, c_int64, c_int64, c_int32, _i64p, _i64p],
+    "endia_hip_col_sum_multi": [c_int32, POINTER(ColSumDesc)],
     "endia_hip_reduce": [c_int32, c_int32, _i64p, c_uint32, _fp, _fp],
     "endia_hip_mse_fwd_bwd": [c_int64, _fp, _fp, _fp, _fp],
     "endia_hip_conv2d_out_shape": [POINTER(Conv2dDesc), _i64p, _i64p],
@@ -228,6 +233,35 @@ def park_product(fields, buffers, out_buffer):
     _parked.append((fields, buffers, out_buffer))
 
 
+_parked_sums = []     # column sums nobody has asked for yet: (R, C, x address, out address, scale, input buffer, output buffer)
+MAX_PARKED_SUMS = 16
+
+
+def park_col_sum(R, C, x_ptr, out_ptr, scale, in_buffer, out_buffer):
+    """out = scale * (sum of the rows of x), put off: a bias gradient is a leaf of the backward pass, so as a rule nothing reads
+    it before the pass is over, and the sums of a pass then go out as ONE endia_hip_col_sum_multi call (a launch of its own
+    costs each of them more than its memory traffic). The input buffer is held until then; reading the output's address
+    (Buffer.ptr) launches them."""
+    if len(_parked_sums) >= MAX_PARKED_SUMS:
+        flush_col_sums()
+    out_buffer.pending = True
+    _parked_sums.append((R, C, x_ptr, out_ptr, scale, in_buffer, out_buffer))
+
+
+def flush_col_sums():
+    """Launch the column sums that were put off (the end of a reverse pass does; so does anything that reads one of them)."""
+    if not _parked_sums:
+        return
+    items = _parked_sums[:]
+    del _parked_sums[:]
+    descs = (ColSumDesc * len(items))()
+    for d, it in zip(descs, items):
+        d.R, d.C, d.x, d.out, d.scale = it[0], it[1], it[2], it[3], it[4]
+    for it in items:
+        it[6].pending = False  # (also when the call fails: the error is the caller's to see, once)
+    _raw_call("endia_hip_col_sum_multi", len(items), descs)
+
+
 def park_launch(launch, out_buffers):
     """Park any other launch whose outputs are all fresh buffers: `launch()` issues it. Besides being run by flush() it
     can be withdrawn (withdraw_launch) by an op that computes the same outputs as part of a larger launch."""
@@ -254,6 +288,9 @@ def withdraw_launch(item):
 
 def parked_uses(buffer):
     """True when a parked product reads or writes `buffer`."""
+    for it in _parked_sums:
+        if it[5] is buffer or it[6] is buffer:
+            return True
     for fields, buffers, out in _parked:
         if fields is None:
             if any(b is buffer for b in out):
@@ -271,6 +308,11 @@ def flush(need=None):
     """Launch what is parked: everything, or, when `need` names the output buffer somebody is about to read, the launch
     that writes it; for a product that means one endia_hip_sgemm_grouped call with that product and whichever parked
     products make its launch a better one (the rest stay parked and may find better company later)."""
+    if _parked_sums and (need is None or any(it[6] is need for it in _parked_sums)):
+        # (a sum's input is never pending: its address was read when the sum was put off)
+        flush_col_sums()
+        if need is not None:
+            return
     if not _parked:
         return
     items = _parked[:]
@@ -323,7 +365,7 @@ def flush(need=None):
 
 def call(name, *args):
     """Call an entry point on the initialised library and raise on a non-zero status."""
-    if _parked and name not in _WRITES_FRESH and not (name == "endia_hip_sgemm" and not (args[15] & GEMM_ACCUMULATE)):
+    if (_parked or _parked_sums) and name not in _WRITES_FRESH and not (name == "endia_hip_sgemm" and not (args[15] & GEMM_ACCUMULATE)):
         flush()
     _raw_call(name, *args)
 

@@ -12,6 +12,7 @@ backward(create_graph=True) passes, then detached copies of the results.
 """
 import sys
 
+from .. import _lib as L
 from .. import functional as F
 from .._array import Array, _contiguous_copy
 
@@ -178,6 +179,7 @@ def _reverse_walk(trace, create_graph):
                 leaf = finished.pop()
                 if leaf._grad is not None:
                     leaf._on_final_grad(leaf)
+        L.flush_col_sums()  # the pass is over: the bias gradients it put off go out as one launch
     finally:
         _building_graph[0] = prev
 

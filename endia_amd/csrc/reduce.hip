@@ -65,11 +65,11 @@ __global__ __launch_bounds__(TPB) void col_reduce_vec_kernel(const float* __rest
 // a thread adds rows lane, lane + 64, ... with sixteen 16-byte loads in flight, and the 64 partial rows meet in LDS in a
 // fixed pairwise order. Two launches (first stage over the whole chip, then the partial sums) take 9.0 us at 1024 x 2048
 // where this takes 7.4: one launch fewer per bias gradient for steps that are counted in launches.
-__global__ __launch_bounds__(TPB) void col_reduce_mid_kernel(const float* __restrict__ x, float* __restrict__ out, int64_t R, int64_t C,
-                                                             float scale) {
+__device__ __forceinline__ void col_reduce_mid_body(const float* __restrict__ x, float* __restrict__ out, int64_t R, int64_t C,
+                                                    float scale, int64_t group) {
   __shared__ float4 red[64][4];
   const int cl = threadIdx.x & 3, rl = threadIdx.x >> 2;
-  const int64_t c = ((int64_t)blockIdx.x * 4 + cl) * 4;
+  const int64_t c = (group * 4 + cl) * 4;
   float4 acc = make_float4(0.f, 0.f, 0.f, 0.f);
   if (c < C) {
     const float* base = x + c;
@@ -93,6 +93,29 @@ __global__ __launch_bounds__(TPB) void col_reduce_mid_kernel(const float* __rest
     const float4 t = red[0][cl];
     *reinterpret_cast<float4*>(out + c) = make_float4(t.x * scale, t.y * scale, t.z * scale, t.w * scale);
   }
+}
+
+__global__ __launch_bounds__(TPB) void col_reduce_mid_kernel(const float* __restrict__ x, float* __restrict__ out, int64_t R, int64_t C,
+                                                             float scale) {
+  col_reduce_mid_body(x, out, R, C, scale, blockIdx.x);
+}
+
+// Several such sums in one launch (endia_hip_col_sum_multi): the work-groups [first[m], first[m + 1]) are the column groups
+// of member m, each computed exactly as the single launch computes it.
+constexpr int kMaxSums = 16;
+struct ColSumMembers {
+  int count;
+  int first[kMaxSums + 1];
+  const float* x[kMaxSums];
+  float* out[kMaxSums];
+  int64_t R[kMaxSums], C[kMaxSums];
+  float scale[kMaxSums];
+};
+
+__global__ __launch_bounds__(TPB) void col_reduce_mid_multi_kernel(const ColSumMembers a) {
+  int m = 0;
+  while (m + 1 < a.count && (int)blockIdx.x >= a.first[m + 1]) ++m;
+  col_reduce_mid_body(a.x[m], a.out[m], a.R[m], a.C[m], a.scale[m], (int64_t)blockIdx.x - a.first[m]);
 }
 
 // scalar variant for C not a multiple of 4 or unaligned: thread per column, 256 columns per group
@@ -432,6 +455,15 @@ int32_t col_reduce(int64_t batch, int64_t R, int64_t C, const float* x, float* o
   return col_reduce_with(batch, R, C, x, out, scale, nullptr, 0);
 }
 
+// Whether col_reduce(1, R, C, x, out, ...) is the one launch of col_reduce_mid_kernel.
+bool col_reduce_is_mid(int64_t R, int64_t C, const float* x, const float* out) {
+  if (R < 1 || C < 1 || C >= (1ll << 31)) return false;
+  const bool vec = (C % 4 == 0) && al16(x) && al16(out);
+  int64_t S = 0, rows = 0;
+  col_reduce_plan(1, R, C, ctx().cu_count, 0, vec, &S, &rows);
+  return S == 0 && !(R <= 1024 && R * C <= (1 << 20));
+}
+
 // The same with the sums stored transposed: column c = o * inner + i goes to out[i * (C / inner) + o]. inner divides C.
 int32_t col_reduce_transposed(int64_t R, int64_t C, int64_t inner, const float* x, float* out) {
   return col_reduce_with(1, R, C, x, out, 1.f, nullptr, 0, inner);
@@ -537,6 +569,56 @@ int32_t endia_hip_reduce_add(int32_t ndim, const int64_t* shape, uint32_t reduce
   hipLaunchKernelGGL(generic_reduce_kernel, dim3((unsigned)nout), dim3(TPB), 0, ctx().stream, d, x, out, nred, scale);
   ENDIA_LAUNCH_CHECK();
   return ENDIA_HIP_OK;
+}
+
+int32_t endia_hip_col_sum_multi(int32_t count, const endia_hip_col_sum_desc* members) {
+  ENDIA_REQUIRE_INIT();
+  ENDIA_CHECK_ARG(count >= 0 && count <= 64 && (count == 0 || members), "endia_hip_col_sum_multi: count %d out of [0, 64] or null members", count);
+  for (int i = 0; i < count; ++i) {
+    const endia_hip_col_sum_desc& d = members[i];
+    ENDIA_CHECK_ARG(d.R >= 0 && d.C >= 0, "endia_hip_col_sum_multi: member %d has a negative extent", i);
+    ENDIA_CHECK_ARG(d.C == 0 || d.out, "endia_hip_col_sum_multi: member %d has no output", i);
+    ENDIA_CHECK_ARG(d.R == 0 || d.C == 0 || d.x, "endia_hip_col_sum_multi: member %d has no input", i);
+  }
+  // members that the single call would run as its one-launch kernel share launches, up to kMaxSums at a time; the others
+  // run as the single call runs them
+  ColSumMembers a;
+  a.count = 0;
+  a.first[0] = 0;
+  auto launch = [&]() -> int32_t {
+    if (a.count == 0) return ENDIA_HIP_OK;
+    if (a.count == 1) {
+      hipLaunchKernelGGL(col_reduce_mid_kernel, dim3((unsigned)a.first[1]), dim3(TPB), 0, ctx().stream, a.x[0], a.out[0], a.R[0], a.C[0], a.scale[0]);
+    } else {
+      hipLaunchKernelGGL(col_reduce_mid_multi_kernel, dim3((unsigned)a.first[a.count]), dim3(TPB), 0, ctx().stream, a);
+    }
+    a.count = 0;
+    ENDIA_LAUNCH_CHECK();
+    return ENDIA_HIP_OK;
+  };
+  for (int i = 0; i < count; ++i) {
+    const endia_hip_col_sum_desc& d = members[i];
+    if (d.C == 0) continue;
+    if (d.R == 0) {
+      int32_t rc = endia_hip_fill(d.out, d.C, 0.f);
+      if (rc) return rc;
+      continue;
+    }
+    if (!col_reduce_is_mid(d.R, d.C, d.x, d.out)) {
+      int32_t rc = col_reduce(1, d.R, d.C, d.x, d.out, d.scale);
+      if (rc) return rc;
+      continue;
+    }
+    const int64_t groups = ceil_div64(d.C, 16);
+    if (a.count == kMaxSums || a.first[a.count] + groups > (1 << 30)) {
+      int32_t rc = launch();
+      if (rc) return rc;
+    }
+    const int m = a.count++;
+    a.x[m] = d.x; a.out[m] = d.out; a.R[m] = d.R; a.C[m] = d.C; a.scale[m] = d.scale;
+    a.first[m + 1] = a.first[m] + (int)groups;
+  }
+  return launch();
 }
 
 int32_t endia_hip_col_sum_static(int64_t R, int64_t C, const float* x, float* out, float scale) {

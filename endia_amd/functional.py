@@ -881,6 +881,18 @@ def abs(x):
 # --------------------------------------------------------------------------------------------------
 # reductions (endia/functional/reduce_ops)
 # --------------------------------------------------------------------------------------------------
+def _col_sum_parks(src):
+    """Whether the column sum of the contiguous real [R, C] array `src` is of the size whose launches are worth sharing (the
+    two-stage reduction for a few hundred to a few thousand rows), and products are being put off at all."""
+    R_, C_ = src._shape
+    return (L.defer_products[0] and not L.capturing and 64 <= R_ <= 2048 and (1 << 20) < R_ * C_ <= (1 << 22) and C_ % 4 == 0
+            and src.data_ptr() % 16 == 0)
+
+
+def _park_col_sum(src, out, scale):
+    L.park_col_sum(src._shape[0], src._shape[1], src.data_ptr(), out._buf.address + 4 * out._offset, scale, src._buf, out._buf)
+
+
 def reduce_add(x, axes, _scale=1.0):
     """Sum over `axes`, keeping them as size 1 (reduce_add_op.mojo:57-61,65-210); VJP = expand (:234)."""
     axes = sorted(set(_norm_axes(list(axes), x.ndim())))
@@ -893,8 +905,12 @@ def reduce_add(x, axes, _scale=1.0):
     if x.ndim() > 8:
         raise ValueError("more than 8 dimensions")
     if out.size():
-        L.call("endia_hip_reduce_add", x.ndim(), L.i64_array(x._shape), mask, src.data_ptr(), out.data_ptr(),
-               float(_scale), 1 if x.is_complex_ else 0)
+        if axes == [0] and x.ndim() == 2 and not x.is_complex_ and _col_sum_parks(src):
+            # a bias gradient of a second-order pass: put off, so that the sums of the pass share one launch
+            _park_col_sum(src, out, float(_scale))
+        else:
+            L.call("endia_hip_reduce_add", x.ndim(), L.i64_array(x._shape), mask, src.data_ptr(), out.data_ptr(),
+                   float(_scale), 1 if x.is_complex_ else 0)
     in_shape = list(x._shape)
     scale = float(_scale)
 
@@ -1814,7 +1830,10 @@ def _linear_node(out, x, W, b, xs, Ws, act):
             tgt = accW if accW is not None else dW
             epi_w = L.EPI_NONE | (L.GEMM_ACCUMULATE if accW is not None else 0)
             if db is not None and split:
-                L.call("endia_hip_reduce_add", 2, L.i64_array([B, N]), 1, g.data_ptr(), db.data_ptr(), 1.0, 0)
+                if _col_sum_parks(g):
+                    _park_col_sum(g, db, 1.0)
+                else:
+                    L.call("endia_hip_reduce_add", 2, L.i64_array([B, N]), 1, g.data_ptr(), db.data_ptr(), 1.0, 0)
                 _sgemm(1, 0, K, N, B, xs, K, g, N, tgt, epi_w)
             else:
                 L.call("endia_hip_sgemm", 1, 0, K, N, B, xs.data_ptr(), K, g.data_ptr(), N, tgt.data_ptr(), N, 1, 0, 0, 0,

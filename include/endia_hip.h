@@ -357,6 +357,19 @@ ENDIA_API int32_t endia_hip_reduce_add(int32_t ndim, const int64_t* shape, uint3
  *      device's one array: calls that overlap on one device (two host threads, two processes' worth of streams)
  *      race; calls on the library's single stream, the only kind this ABI issues, are ordered. */
 ENDIA_API int32_t endia_hip_col_sum_static(int64_t R, int64_t C, const float* x, float* out, float scale);
+/* Several column sums in one call: out[c] = scale * sum_r x[r][c] for every member, each the result, bit for bit, of
+ * endia_hip_reduce_add(2, {R, C}, 1, x, out, scale, 0). No counterpart in the reference, whose reverse walk reduces one
+ * bias gradient at a time (expand_op.mojo:121-126 from autograd/functional.mojo:46-65): a second-order pass over a
+ * few 2048-wide layers leaves eight such sums of [1024, 2048] that nothing reads until the pass is over, each a
+ * launch of 7 us that is mostly launch; members of that size share one launch, the others run as the single call
+ * runs them. Members must not overlap each other's outputs. count <= 64. */
+typedef struct endia_hip_col_sum_desc {
+  int64_t R, C;
+  const float* x;
+  float* out;
+  float scale;
+} endia_hip_col_sum_desc;
+ENDIA_API int32_t endia_hip_col_sum_multi(int32_t count, const endia_hip_col_sum_desc* members);
 /* How a column sum of R rows and C columns cuts its rows on a device of cu_count CUs when scratch_floats floats are
  * there for first-stage partial sums (0: no limit, what endia_hip_reduce_add has; 262144: endia_hip_col_sum_static).
  * aligned16: x and out start on 16-byte boundaries. No counterpart in the reference; pure arithmetic, needs no device

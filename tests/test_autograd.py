@@ -551,6 +551,78 @@ def test_parked_products_share_launches(nd):
     assert_close(z.to_numpy(), xn.astype(np.float64) @ Wn[1], what="a parked product read later")
 
 
+def test_parked_column_sums_share_a_launch(nd):
+    """The bias gradients of a reverse pass over layers of a few thousand rows (functional.reduce_add and the fused layer's
+    rule put them off, _lib.park_col_sum) go out as one endia_hip_col_sum_multi call at the end of the pass. Batch 2048 into
+    two 1024-wide sin layers: first-order bias gradients are bit for bit those of a pass with the parking off, the
+    Hessian-vector product agrees, a sum that is put off outside a pass is launched by whoever reads it, and by an in-place
+    writer of its input before that writes."""
+    from endia_amd import _lib as L
+    from endia_amd import functional as F
+    rng = np.random.default_rng(23)
+    Bn, Wd = 2048, 1024
+    Wn = [(rng.standard_normal((Wd, Wd)) / np.sqrt(Wd)).astype(np.float32) for _ in range(2)]
+    bn = [(0.1 * rng.standard_normal(Wd)).astype(np.float32) for _ in range(2)]
+    vn = [rng.standard_normal(a.shape).astype(np.float32) for a in (Wn[0], bn[0], Wn[1], bn[1])]
+    xn = rng.standard_normal((Bn, Wd)).astype(np.float32)
+    seen = []
+    raw = L._raw_call
+
+    def spy(name, *args):
+        if name == "endia_hip_col_sum_multi":
+            seen.append(args[0])
+        return raw(name, *args)
+
+    def run():
+        mlp = nd.nn.MLP([Wd] * 3, compute_backward=True, activation="sin", fused=True)
+        for i in range(2):
+            mlp.weights[i], mlp.biases[i] = nd.array(Wn[i], requires_grad=True), nd.array(bn[i], requires_grad=True)
+        out = mlp.forward(nd.array(xn))
+        loss = nd.sum(out * out)
+        loss.backward(create_graph=True)
+        assert not L._parked_sums  # the end of the pass launched them
+        firsts = [p.grad() for p in mlp.params()]
+        hv = nd.grad(outs=firsts, inputs=mlp.params(), grad_outs=[nd.reshape(nd.array(v), f.shape()) for v, f in zip(vn, firsts)])
+        assert not L._parked_sums
+        res = [f.to_numpy() for f in firsts] + [h.to_numpy() for h in hv]
+        loss.zero_grad()
+        return res
+
+    L._raw_call = spy
+    try:
+        parked = run()
+        assert seen == [2, 2], "merged calls of the two passes: %r" % (seen,)
+        L.defer_products[0] = False
+        try:
+            plain = run()
+        finally:
+            L.defer_products[0] = True
+        assert seen == [2, 2]
+        np.testing.assert_array_equal(parked[1], plain[1])  # first-order bias gradients: the same kernel body either way
+        np.testing.assert_array_equal(parked[3], plain[3])
+        for k, (a, b) in enumerate(zip(parked, plain)):
+            assert_close(a, b, tol=2e-6, mean_tol=1e-4, what="tensor %d with and without parking" % k)
+        # outside a pass: the read launches it
+        x = nd.array(xn)
+        s = F.reduce_add(x, [0])
+        assert len(L._parked_sums) == 1
+        got = s.to_numpy()
+        assert not L._parked_sums and seen[-1] == 1
+        ref64 = xn.astype(np.float64).sum(axis=0, keepdims=True)
+        assert np.all(np.abs(got - ref64) <= 1e-5 * np.abs(xn).astype(np.float64).sum(axis=0, keepdims=True))
+        # an optimizer step writes the summed tensor in place: the sum of the old values goes first
+        W = nd.array(xn, requires_grad=True)
+        s = F.reduce_add(W, [0])
+        assert len(L._parked_sums) == 1
+        W.grad_(nd.array(np.ones_like(xn)))
+        nd.optim.SGD([W], lr=1.0).step()
+        assert not L._parked_sums
+        np.testing.assert_array_equal(s.to_numpy(), got)
+        np.testing.assert_array_equal(W.to_numpy(), xn - 1.0)
+    finally:
+        L._raw_call = raw
+
+
 def test_optimizer_classes(nd, golden):
     g = golden("optim")
     makers = {

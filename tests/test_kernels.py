@@ -328,6 +328,58 @@ def test_reduce_golden_scale_complex_empty(dev, golden):
     np.testing.assert_array_equal(dev.get(do, (8,)), np.zeros(8, np.float32))  # empty sum
 
 
+def test_col_sum_multi_matches_the_single_call(dev):
+    """endia_hip_col_sum_multi: every member bit for bit what endia_hip_reduce_add (ndim 2, mask 1) gives for it alone --
+    members of the size that share launches (a few hundred to a few thousand rows, aligned, C a multiple of 4), more of them
+    than one launch holds, and members the single call runs another way (few rows, many rows, C not a multiple of 4,
+    unaligned input, no rows, no columns) mixed in between."""
+    import ctypes
+    rng = np.random.default_rng(77)
+    shapes = [(1024, 2048), (7, 12), (2048, 2048), (512, 4096), (1024, 2050), (70000, 24), (0, 16), (64, 16388), (300, 0)]
+    shapes += [(1024, 1028 + 4 * i) for i in range(18)]  # more than one launch's worth of sharing members
+    descs = (L.ColSumDesc * len(shapes))()
+    want, outs = [], []
+    for i, (R_, C_) in enumerate(shapes):
+        x = rng.standard_normal((R_, C_)).astype(np.float32)
+        pad = 1 if i == 3 else 0  # one member's input starts 4 bytes off a 16-byte boundary
+        dx_ = dev.alloc(4 * (R_ * C_ + 4))
+        if x.size:
+            L.call("endia_hip_memcpy_h2d", dx_ + 4 * pad, x.ctypes.data, x.nbytes)
+        do, dm = dev.alloc(4 * max(C_, 1)), dev.alloc(4 * max(C_, 1))
+        scale = 1.0 if i % 3 else 1.0 / max(R_, 1)
+        if C_:
+            dev.call("endia_hip_fill", do, C_, 7.0)
+            dev.call("endia_hip_fill", dm, C_, 9.0)
+            dev.call("endia_hip_reduce_add", 2, L.i64_array([R_, C_]), 1, (dx_ + 4 * pad) if R_ else None, do, scale, 0)
+        want.append(dev.get(do, (C_,)) if C_ else None)
+        outs.append(dm)
+        d = descs[i]
+        d.R, d.C, d.x, d.out, d.scale = R_, C_, dx_ + 4 * pad, dm, scale
+    for _ in range(2):  # twice: the second call must not depend on anything the first left behind
+        dev.call("endia_hip_col_sum_multi", len(shapes), descs)
+        for i, (R_, C_) in enumerate(shapes):
+            if C_:
+                np.testing.assert_array_equal(dev.get(outs[i], (C_,)), want[i], err_msg="member %d %s" % (i, shapes[i]))
+    # against float64, on the scale of sum |x|, for one sharing member (the single call's own tests cover the others)
+    x = rng.standard_normal((1536, 1024)).astype(np.float32)
+    one = (L.ColSumDesc * 1)()
+    one[0].R, one[0].C, one[0].x, one[0].out, one[0].scale = 1536, 1024, dev.put(x), dev.alloc(4096), 0.5
+    dev.call("endia_hip_col_sum_multi", 1, one)
+    ref64 = 0.5 * x.astype(np.float64).sum(axis=0)
+    assert np.all(np.abs(dev.get(one[0].out, (1024,)) - ref64) <= 1e-5 * 0.5 * np.abs(x).astype(np.float64).sum(axis=0))
+    # argument errors
+    lib = L.ensure_init()
+    assert lib.endia_hip_col_sum_multi(0, None) == 0
+    assert lib.endia_hip_col_sum_multi(65, descs) == L.ERR_INVALID
+    assert lib.endia_hip_col_sum_multi(-1, descs) == L.ERR_INVALID
+    assert lib.endia_hip_col_sum_multi(1, None) == L.ERR_INVALID
+    bad = (L.ColSumDesc * 1)()
+    bad[0].R, bad[0].C, bad[0].x, bad[0].out, bad[0].scale = 4, 4, None, one[0].out, 1.0
+    assert lib.endia_hip_col_sum_multi(1, bad) == L.ERR_INVALID
+    bad[0].R, bad[0].x, bad[0].out = -1, one[0].x, one[0].out
+    assert lib.endia_hip_col_sum_multi(1, bad) == L.ERR_INVALID
+
+
 _REDUCE_KINDS = {"max": L.REDUCE_MAX, "min": L.REDUCE_MIN, "mul": L.REDUCE_MUL, "argmax": L.REDUCE_ARGMAX, "argmin": L.REDUCE_ARGMIN}
 
 
