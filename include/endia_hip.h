@@ -362,7 +362,7 @@ ENDIA_API int32_t endia_hip_col_sum_static(int64_t R, int64_t C, const float* x,
  * bias gradient at a time (expand_op.mojo:121-126 from autograd/functional.mojo:46-65): a second-order pass over a
  * few 2048-wide layers leaves eight such sums of [1024, 2048] that nothing reads until the pass is over, each a
  * launch of 7 us that is mostly launch; members of that size share one launch, the others run as the single call
- * runs them. Members must not overlap each other's outputs. count <= 64. */
+ * runs them. No member's output may be another member's output or input (members run concurrently). count <= 64. */
 typedef struct endia_hip_col_sum_desc {
   int64_t R, C;
   const float* x;
