@@ -246,6 +246,40 @@ def test_ew_program(dev, rows, cols):
     assert_close(got[1], (1 - np.tanh(z) ** 2) * 0.75 * (1 + np.exp(-z)), what="second output vs float64", mean_tol=mean_tol)
 
 
+@pytest.mark.parametrize("rows,cols", [(3, 5), (33, 1000), (1024, 2052), (2300, 2048)])
+def test_ew_program_with_sin_cos_pow(dev, rows, cols):
+    """A program with sin, cos and pow (the ops with the longest bodies, and a saved value that is read back as a right
+    operand) at every tile size."""
+    rng = np.random.default_rng(rows * 17 + cols)
+    a = rng.standard_normal((rows, cols)).astype(np.float32) * 3
+    b = rng.standard_normal((rows, cols)).astype(np.float32)
+    I, S, M = L.EW_SRC_INPUT, L.EW_SRC_SLOT, L.EW_SRC_IMM
+    steps = [
+        (L.EW_LOAD, 0, I, 1, 0.0),
+        (L.EW_UNARY, L.OP_COS, 0, 0, 0.0),
+        (L.EW_SAVE, 0, 0, 0, 0.0),                  # cos(b) -> slot 0
+        (L.EW_LOAD, 0, I, 0, 0.0),
+        (L.EW_UNARY, L.OP_SIN, 0, 0, 0.0),
+        (L.EW_BINARY, L.BIN_MUL, S, 0, 0.0),
+        (L.EW_STORE, 0, 0, 0, 0.0),                 # out0 = sin(a) * cos(b)
+        (L.EW_LOAD, 0, I, 0, 0.0),
+        (L.EW_UNARY, L.OP_ABS, 0, 0, 0.0),
+        (L.EW_BINARY, L.BIN_ADD, M, 0, 1.0),
+        (L.EW_BINARY, L.BIN_POW, I, 1, 0.0),
+        (L.EW_STORE, 0, 0, 1, 0.0),                 # out1 = (|a| + 1) ** b
+    ]
+    modes = [L.EW_FULL, L.EW_FULL]
+    got = _run_program(dev, rows, cols, [a, b], modes, 2, steps)
+    want = _program_expected(rows, cols, [a, b], modes, 2, steps)
+    a64, b64 = a.astype(np.float64), b.astype(np.float64)
+    # sin(a) cos(b) passes through zero: a handful of the two million entries carry the mean of the per-element relative errors
+    mean_tol = 1e-2 if rows * cols > (1 << 20) else None
+    assert_close(got[0], want[0], what="sin(a) cos(b) vs the oracle's op bodies", mean_tol=mean_tol)
+    assert_close(got[0], np.sin(a64) * np.cos(b64), what="sin(a) cos(b) vs float64", mean_tol=mean_tol)
+    assert_close(got[1], want[1], what="(|a| + 1) ** b vs the oracle's op bodies")
+    assert_close(got[1], (np.abs(a64) + 1) ** b64, what="(|a| + 1) ** b vs float64")
+
+
 def test_ew_program_rejects_bad_programs(dev):
     a = np.ones((2, 4), np.float32)
     ok = [(L.EW_LOAD, 0, L.EW_SRC_INPUT, 0, 0.0), (L.EW_STORE, 0, 0, 0, 0.0)]
