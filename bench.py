@@ -695,7 +695,7 @@ def _time_steps(nd, step, steps, warmup):
 
 
 def run_sine(nd, steps, warmup, optimizer="sgd", eager=False, per_layer=False):
-    """BASELINE configuration 1, the reference's own benchmark model (benchmarks/mlp_benchmarks/mlp_imp.mojo:35-75), as
+    """Benchmark configuration 1, the reference's own benchmark model (benchmarks/mlp_benchmarks/mlp_imp.mojo:35-75), as
     a HIP-graph replay of the eager step. `value` is taken with the reference script's call shape, mse(mlp.forward(x),
     y); the same step with forward and loss behind one method (MLP.mse_loss, no counterpart in the reference) is
     timed beside it. Launch-latency bound: no roofline claim."""
@@ -775,7 +775,7 @@ def run_wide(nd, steps, warmup, fused_backward=False):
 
 
 def run_conv(nd, steps, warmup):
-    """BASELINE configuration 5 as a training step through the public API (forward with fused ReLU, mean loss, weight
+    """Benchmark configuration 5 as a training step through the public API (forward with fused ReLU, mean loss, weight
     and bias gradients; the same with the data gradient beside it). `roofline` prices the forward entry point, the
     longest of the step's launches, timed alone with HIP events on the library's stream."""
     rows = conv_table(max(min(steps, 10), 3), only=("conv2d_fwd (+bias, relu)", "conv2d_bwd_data", "conv2d_bwd_weight"))
