@@ -516,10 +516,10 @@ def conv_table(reps=10, only=None):
         cases = [c for c in cases if c[0] in only]
     rows = []
     ms = ctypes.c_float()
-    for _ in range(30):  # bring the clocks up before the first timed kernel
+    for _ in range(300):  # bring the clocks up before the first timed kernel (a few dozen launches are still on the ramp)
         cases[0][1]()
     for name, fn, work, bound in cases:
-        for _ in range(3):
+        for _ in range(20):
             fn()
         L.call("endia_hip_timer_start", 0)
         for _ in range(reps):
@@ -778,7 +778,7 @@ def run_conv(nd, steps, warmup):
     """Benchmark configuration 5 as a training step through the public API (forward with fused ReLU, mean loss, weight
     and bias gradients; the same with the data gradient beside it). `roofline` prices the forward entry point, the
     longest of the step's launches, timed alone with HIP events on the library's stream."""
-    rows = conv_table(max(min(steps, 10), 3), only=("conv2d_fwd (+bias, relu)", "conv2d_bwd_data", "conv2d_bwd_weight"))
+    rows = conv_table(max(min(steps, 200), 3), only=("conv2d_fwd (+bias, relu)", "conv2d_bwd_data", "conv2d_bwd_weight"))
     step, with_dx = conv_step(nd, steps, warmup, False), conv_step(nd, steps, warmup, True)
     fwd = rows[0]
     return {"metric": "conv2d fwd + VJPs train steps/s, batch 64, 64->128 channels, 3x3, stride 1, pad 1, 56x56, fp32",
@@ -830,7 +830,8 @@ def main():
     cpu = not args.no_cpu_baseline
 
     if args.workload == "hvp":
-        out = run_hvp(nd, max(args.steps, 40) if args.steps == 20 else args.steps, args.warmup)  # (short runs measure the clock ramp)
+        # (short runs measure the clock ramp: 40 products after 3 read 2.24 ms where 200 after 20 read 2.20)
+        out = run_hvp(nd, 200 if args.steps == 20 else args.steps, max(args.warmup, 20) if args.steps == 20 else args.warmup)
         if cpu:
             out["cpu_baseline"] = cpu_baseline_hvp()
     elif args.workload.startswith("complex_mlp"):
@@ -838,7 +839,8 @@ def main():
         if cpu:
             out["cpu_baseline"] = cpu_baseline_complex()
     elif args.workload == "conv2d":
-        out = run_conv(nd, 100 if args.steps == 20 else max(args.steps, 1), max(args.warmup, 10))  # (short runs measure the clock ramp)
+        # (short runs measure the clock ramp: 100 steps of half a millisecond read 0.511 ms where 1000 read 0.503)
+        out = run_conv(nd, 1000 if args.steps == 20 else max(args.steps, 1), max(args.warmup, 50 if args.steps == 20 else 10))
         if cpu:
             out["cpu_baseline"] = cpu_baseline_conv()
     elif args.workload == "conv2d_kernels":
@@ -868,9 +870,9 @@ def main():
             others = []
             for name, fn, base in (
                     ("sine_mlp", lambda: run_sine(nd, 2000, 3), lambda: cpu_baseline_sine(steps=200)),
-                    ("hvp", lambda: run_hvp(nd, 40, 5), cpu_baseline_hvp),
+                    ("hvp", lambda: run_hvp(nd, 200, 20), cpu_baseline_hvp),
                     ("complex_mlp", lambda: run_complex(nd, 20, 3, "4m"), lambda: cpu_baseline_complex(rows=256)),
-                    ("conv2d", lambda: run_conv(nd, 100, 10), lambda: cpu_baseline_conv(n_img=8))):
+                    ("conv2d", lambda: run_conv(nd, 1000, 50), lambda: cpu_baseline_conv(n_img=8))):
                 r = fn()
                 if cpu:
                     r["cpu_baseline"] = base()
