@@ -26,6 +26,8 @@
 namespace endia {
 int32_t col_reduce(int64_t batch, int64_t R, int64_t C, const float* x, float* out, float scale);
 int32_t col_reduce_transposed(int64_t R, int64_t C, int64_t inner, const float* x, float* out);
+int32_t col_reduce_with_rider(int64_t R, int64_t C, int64_t inner, const float* x, float* out, int64_t R2, int64_t C2, const float* x2,
+                              float* out2);
 int32_t row_reduce(int64_t R, int64_t C, const float* x, float* out, float scale);
 }
 
@@ -1646,9 +1648,9 @@ int32_t run_wgrad3x3(const ConvP& p, const float* x, const float* dy, float* dw,
   else hipLaunchKernelGGL((conv_wgrad3x3_kernel<2>), grid, dim3(256), 0, s, a);
   ENDIA_LAUNCH_CHECK();
   if (splits > 1) {  // partials added in split order; the last stage of the sum stores [tap][k][c] as the weights' [k][c][tap]
-    if ((rc = endia::col_reduce_transposed(splits, taps, (int64_t)p.K * p.C, a.part, dw))) return rc;
-    if (db && (rc = endia::col_reduce(1, splits, p.K, db_part, db, 1.f))) return rc;
-    return ENDIA_HIP_OK;
+    // (the bias gradient's partial sums ride in the launch of the weight gradient's last stage)
+    if (db) return endia::col_reduce_with_rider(splits, taps, (int64_t)p.K * p.C, a.part, dw, splits, p.K, db_part, db);
+    return endia::col_reduce_transposed(splits, taps, (int64_t)p.K * p.C, a.part, dw);
   }
   hipLaunchKernelGGL(wgrad3x3_order_kernel, dim3(grid_for(taps)), dim3(TPB), 0, s, a.part, dw, p.K, p.C);
   ENDIA_LAUNCH_CHECK();
@@ -1750,8 +1752,8 @@ int32_t conv_bwd_weight(const char* who, const ConvP& p, const float* x, const f
   }
   ENDIA_LAUNCH_CHECK();
   if (splits > 1) {  // partials added in split order
+    if (db) return endia::col_reduce_with_rider(splits, taps, 0, a.part, dw, splits, p.K, db_part, db);
     if ((rc = endia::col_reduce(1, splits, taps, a.part, dw, 1.f))) return rc;
-    if (db) return endia::col_reduce(1, splits, p.K, db_part, db, 1.f);
   }
   return ENDIA_HIP_OK;
 }

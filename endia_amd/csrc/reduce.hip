@@ -137,12 +137,11 @@ __global__ __launch_bounds__(TPB) void col_reduce_scalar_kernel(const float* __r
 // s = w, w+4, ... and are combined through LDS in wave order, so the result does not depend on timing.
 // inner > 0: the columns are an [C / inner][inner] array and the sums are stored transposed, as [inner][C / inner] (the
 // 3 x 3 weight gradient sums its partial products in [tap][k][c] order and stores them as the weights' [k][c][tap]).
-__global__ __launch_bounds__(TPB) void col_reduce_final_kernel(const float* __restrict__ part, float* __restrict__ out,
-                                                               int64_t S, int64_t C, int64_t batch, float scale, int64_t inner) {
+__device__ __forceinline__ void col_reduce_final_body(const float* __restrict__ part, float* __restrict__ out, int64_t S, int64_t C,
+                                                      float scale, int64_t inner, int64_t group, int64_t b) {
   __shared__ float red[4][64];
   const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
-  const int64_t c = (int64_t)blockIdx.x * 64 + lane;
-  const int64_t b = blockIdx.y;
+  const int64_t c = group * 64 + lane;
   float acc = 0.f;
   if (c < C) {
 #pragma unroll 8
@@ -158,6 +157,25 @@ __global__ __launch_bounds__(TPB) void col_reduce_final_kernel(const float* __re
     }
     out[b * C + at] = ((red[0][lane] + red[1][lane]) + (red[2][lane] + red[3][lane])) * scale;
   }
+}
+
+__global__ __launch_bounds__(TPB) void col_reduce_final_kernel(const float* __restrict__ part, float* __restrict__ out,
+                                                               int64_t S, int64_t C, int64_t batch, float scale, int64_t inner) {
+  col_reduce_final_body(part, out, S, C, scale, inner, blockIdx.x, blockIdx.y);
+}
+
+// The last stage of one reduction and, in the work-groups behind its own, a second small reduction that needs this stage
+// only (a weight gradient's partial sums and its bias gradient's: one launch instead of two). Each as the kernel above
+// computes it.
+struct FinalJob {
+  const float* part;
+  float* out;
+  int64_t S, C, inner;
+  float scale;
+};
+__global__ __launch_bounds__(TPB) void col_reduce_final_pair_kernel(const FinalJob a, const FinalJob b, int groups_a) {
+  if ((int)blockIdx.x < groups_a) col_reduce_final_body(a.part, a.out, a.S, a.C, a.scale, a.inner, blockIdx.x, 0);
+  else col_reduce_final_body(b.part, b.out, b.S, b.C, b.scale, b.inner, (int)blockIdx.x - groups_a, 0);
 }
 
 // ---- row reduction: x[R][C] -> out[R] (sum over C) --------------------------------------------
@@ -411,9 +429,29 @@ static void col_reduce_plan(int64_t batch, int64_t R, int64_t C, int64_t cus, in
 
 // out[b][c] = scale * sum_r x[b][r][c]. The first-stage partial sums go to `part` (room for part_floats) when the
 // caller brings it, else to the library's workspace; with too little room the rows are cut into fewer splits.
+// rider: a second reduction out2[c] = sum_r x2[r][c] of at most 1024 rows and 2^20 elements (batch 1 only), whose one stage
+// shares the launch of this reduction's last stage where there is one.
+struct ColSumRider {
+  int64_t R, C;
+  const float* x;
+  float* out;
+};
 static int32_t col_reduce_with(int64_t batch, int64_t R, int64_t C, const float* x, float* out, float scale, float* part,
-                               int64_t part_floats, int64_t inner = 0) {
+                               int64_t part_floats, int64_t inner = 0, const ColSumRider* rider = nullptr) {
   hipStream_t s = ctx().stream;
+  const bool ride = rider && batch == 1 && rider->R >= 1 && rider->R <= 1024 && rider->R * rider->C <= (1 << 20) && rider->C >= 1 &&
+                    ceil_div64(C, 64) + ceil_div64(rider->C, 64) < (1ll << 31);
+  // (the last stage, alone or with the rider in its launch)
+  auto last_stage = [&](const float* from, int64_t rows) {
+    if (ride) {
+      const FinalJob a{from, out, rows, C, inner, scale}, b{rider->x, rider->out, rider->R, rider->C, 0, 1.f};
+      const int groups_a = (int)ceil_div64(C, 64);
+      hipLaunchKernelGGL(col_reduce_final_pair_kernel, dim3((unsigned)(groups_a + ceil_div64(rider->C, 64))), dim3(TPB), 0, s, a, b, groups_a);
+    } else {
+      hipLaunchKernelGGL(col_reduce_final_kernel, dim3((unsigned)ceil_div64(C, 64), (unsigned)batch), dim3(TPB), 0, s, from, out, rows,
+                         C, batch, scale, inner);
+    }
+  };
   const bool vec = (C % 4 == 0) && al16(x);
   const int64_t col_tiles = ceil_div64(C, 256);
   if (col_tiles * 1 > 2147483647ll || batch > 65535)
@@ -426,13 +464,12 @@ static int32_t col_reduce_with(int64_t batch, int64_t R, int64_t C, const float*
   if (S == 0 && !(R <= 1024 && batch * R * C <= (1 << 20))) {
     hipLaunchKernelGGL(col_reduce_mid_kernel, dim3((unsigned)ceil_div64(C, 16)), dim3(TPB), 0, s, x, out, R, C, scale);
     ENDIA_LAUNCH_CHECK();
-    return ENDIA_HIP_OK;
+    return rider ? col_reduce_with(1, rider->R, rider->C, rider->x, rider->out, 1.f, nullptr, 0) : ENDIA_HIP_OK;
   }
   if (S == 0) {
-    hipLaunchKernelGGL(col_reduce_final_kernel, dim3((unsigned)ceil_div64(C, 64), (unsigned)batch), dim3(TPB), 0, s, x, out, R,
-                       C, batch, scale, inner);
+    last_stage(x, R);
     ENDIA_LAUNCH_CHECK();
-    return ENDIA_HIP_OK;
+    return rider && !ride ? col_reduce_with(1, rider->R, rider->C, rider->x, rider->out, 1.f, nullptr, 0) : ENDIA_HIP_OK;
   }
   if (S < 0) return fail(ENDIA_HIP_ERR_INVALID, "col_reduce: %lld columns do not fit the %lld floats of scratch", (long long)(batch * C), (long long)part_floats);
   if (!part) {
@@ -445,10 +482,9 @@ static int32_t col_reduce_with(int64_t batch, int64_t R, int64_t C, const float*
   if (vec) hipLaunchKernelGGL(col_reduce_vec_kernel, grid, dim3(TPB), 0, s, x, part, R, C, rows_per_split);
   else hipLaunchKernelGGL(col_reduce_scalar_kernel, grid, dim3(TPB), 0, s, x, part, R, C, rows_per_split);
   ENDIA_LAUNCH_CHECK();
-  hipLaunchKernelGGL(col_reduce_final_kernel, dim3((unsigned)ceil_div64(C, 64), (unsigned)batch), dim3(TPB), 0, s, part,
-                     out, S, C, batch, scale, inner);
+  last_stage(part, S);
   ENDIA_LAUNCH_CHECK();
-  return ENDIA_HIP_OK;
+  return rider && !ride ? col_reduce_with(1, rider->R, rider->C, rider->x, rider->out, 1.f, nullptr, 0) : ENDIA_HIP_OK;
 }
 
 int32_t col_reduce(int64_t batch, int64_t R, int64_t C, const float* x, float* out, float scale) {
@@ -467,6 +503,14 @@ bool col_reduce_is_mid(int64_t R, int64_t C, const float* x, const float* out) {
 // The same with the sums stored transposed: column c = o * inner + i goes to out[i * (C / inner) + o]. inner divides C.
 int32_t col_reduce_transposed(int64_t R, int64_t C, int64_t inner, const float* x, float* out) {
   return col_reduce_with(1, R, C, x, out, 1.f, nullptr, 0, inner);
+}
+
+// col_reduce_transposed (inner > 0) or col_reduce (inner = 0) of x, and the plain column sums of x2 [R2][C2] into out2 as
+// col_reduce(1, R2, C2, x2, out2, 1) gives them, in the same launch where x2 is small enough to need one stage only.
+int32_t col_reduce_with_rider(int64_t R, int64_t C, int64_t inner, const float* x, float* out, int64_t R2, int64_t C2, const float* x2,
+                              float* out2) {
+  const ColSumRider rider{R2, C2, x2, out2};
+  return col_reduce_with(1, R, C, x, out, 1.f, nullptr, 0, inner, &rider);
 }
 
 // out[r] = scale * sum_c x[r][c]
