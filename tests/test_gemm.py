@@ -106,22 +106,25 @@ def test_sgemm_unaligned_operands_on_the_matrix_cores(dev, M, N, K, pad_a, pad_b
 
 
 @pytest.mark.parametrize("tb", [0, 1])
-@pytest.mark.parametrize("M,N,K,pad_a", [(4096, 10, 4096, 0), (1000, 7, 1028, 4), (256, 16, 512, 0), (300, 1, 2052, 8), (2049, 3, 640, 0)])
-def test_sgemm_few_output_columns(dev, M, N, K, pad_a, tb):
+@pytest.mark.parametrize("M,N,K,pad_a,pad_b", [(4096, 10, 4096, 0, 0), (1000, 7, 1028, 4, 0), (256, 16, 512, 0, 0), (300, 1, 2052, 8, 0),
+                                               (2049, 3, 640, 0, 0), (1000, 10, 1028, 0, 4), (520, 13, 4100, 4, 8)])
+def test_sgemm_few_output_columns(dev, M, N, K, pad_a, pad_b, tb):
     """A classifier head: at most 16 output columns over a long reduction (matmul_op.mojo:93-199 takes any shape). One pass
-    over A with the reduction cut across the waves of a work-group; ragged M and K, padded rows of A, B stored either way,
-    every epilogue and accumulation, against the oracle and float64; repeated runs give the same bits."""
+    over A with the reduction cut across the waves of a work-group; ragged M and K, padded rows of A, B stored either way
+    and, stored [K, N], both without padding (the rows of a piece fetched as one run of memory) and with it, every epilogue
+    and accumulation, against the oracle and float64; repeated runs give the same bits."""
     rng = np.random.default_rng(M + 3 * N + 5 * K + tb)
     bufA, A = _embedded(rng, M, K, K + pad_a, 0)
-    B = (rng.standard_normal((N, K) if tb else (K, N)) / np.sqrt(K)).astype(np.float32)
-    dA, dB = dev.put(bufA), dev.put(B)
+    bufB, B = _embedded(rng, N if tb else K, K if tb else N, (K if tb else N) + pad_b, 0)
+    bufB /= np.float32(np.sqrt(K))
+    dA, dB = dev.put(bufA), dev.put(bufB)
     opB = B.T if tb else B
     ref64 = A.astype(np.float64) @ opB.astype(np.float64)
     ref = R.matmul(np.ascontiguousarray(A), np.ascontiguousarray(opB))
 
     def run(epi=L.EPI_NONE, act=L.OP_IDENTITY, bias=None, aux=None, C0=None, aux_out=None):
         dC = dev.put(C0) if C0 is not None else dev.alloc(M * N * 4)
-        dev.call("endia_hip_sgemm", 0, tb, M, N, K, dA, K + pad_a, dB, B.shape[1], dC, N, 1, 0, 0, 0, epi, act,
+        dev.call("endia_hip_sgemm", 0, tb, M, N, K, dA, K + pad_a, dB, B.shape[1] + pad_b, dC, N, 1, 0, 0, 0, epi, act,
                  dev.put(bias) if bias is not None else None, dev.put(aux) if aux is not None else None, aux_out)
         return dev.get(dC, (M, N))
 
